@@ -1,0 +1,177 @@
+/* numml_hip.h -- C ABI of libnumml_hip.so: differentiable CSR kernels for
+ * AMD gfx950 (MI355X).
+ *
+ * Every entry point takes raw DEVICE pointers, sizes and the HIP stream to
+ * enqueue on, returns an nm_status and, unless its comment says otherwise,
+ * neither allocates nor synchronises.  Outputs are written in full; inputs
+ * are never modified.  Structure arrays (`indices`, `indptr`) are int64, the
+ * layout the reference's extension receives (cpp/sparse_csr_cpu.cpp:24-25);
+ * values are float or double, selected by `dt` (the reference dispatches on
+ * the same two types, AT_DISPATCH_FLOATING_TYPES, cpp/sparse_csr_cpu.cpp:22).
+ * Column indices must be ascending inside each row, without duplicates.
+ *
+ * Each group below names the reference function it stands in for; paths are
+ * relative to the reference tree (nicknytko/numml).
+ */
+#ifndef NUMML_HIP_H_
+#define NUMML_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum nm_status {
+    NM_OK = 0,
+    NM_ERR_INVALID = 1,     /* bad argument (null pointer, negative size, bad dtype) */
+    NM_ERR_HIP = 2,         /* a HIP runtime call or kernel launch failed */
+    NM_ERR_WORKSPACE = 3,   /* caller-provided workspace too small */
+    NM_ERR_UNSUPPORTED = 4  /* size beyond what the kernels index (see nm_limits) */
+} nm_status;
+
+typedef enum nm_dtype { NM_F32 = 0, NM_F64 = 1 } nm_dtype;
+
+/* hipStream_t, spelled as void* so that C callers need no HIP headers. */
+typedef void *nm_stream;
+
+/* Version of this ABI (major * 1000 + minor). */
+int nm_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char *nm_last_error(void);
+
+/* ------------------------------------------------------------------ SpMV
+ * y = A x.  Stands in for spgemv_forward (cpp/sparse_csr.hpp:32-36,
+ * cpp/sparse_csr_cpu.cpp:11-39; CUDA launch site cpp/sparse_csr_cuda.cu:42-67).
+ * x has `cols` entries, y `rows`.  Rows whose stored entries fit the
+ * workgroup's LDS tile are summed in storage order, exactly like the CPU loop.
+ */
+int nm_spgemv_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                      const void *data, const int64_t *indices, const int64_t *indptr,
+                      const void *x, void *y, nm_stream stream);
+
+/* grad_A[k] = g[row(k)] * x[col(k)];  grad_x = A^T g (grad_x is cleared here,
+ * then accumulated with hardware floating-point atomics, so its rounding is
+ * run-to-run order dependent).  Stands in for spgemv_backward
+ * (cpp/sparse_csr.hpp:38-42, cpp/sparse_csr_cpu.cpp:41-77).  Either output
+ * pointer may be NULL to skip that gradient. */
+int nm_spgemv_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                       const void *data, const int64_t *indices, const int64_t *indptr,
+                       const void *x, const void *g,
+                       void *grad_A, void *grad_x, nm_stream stream);
+
+/* ------------------------------------------------------------------ SpMM
+ * C = A B with dense row-major B (cols x n, row stride ldb elements) and
+ * C (rows x n, row stride ldc).  Stands in for spdmm_forward
+ * (cpp/sparse_csr.hpp:81-85, cpp/sparse_csr_cpu.cpp:562-602). */
+int nm_spdmm_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                     const void *data, const int64_t *indices, const int64_t *indptr,
+                     const void *B, int64_t ldb, int64_t n,
+                     void *C, int64_t ldc, nm_stream stream);
+
+/* grad_A[k] = <gC[row(k),:], B[col(k),:]>;  grad_B = A^T gC (cleared here,
+ * accumulated with atomics).  grad_B is cols x n with row stride ldgb.
+ * Stands in for spdmm_backward (cpp/sparse_csr.hpp:87-91,
+ * cpp/sparse_csr_cpu.cpp:604-650).  Either output may be NULL. */
+int nm_spdmm_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                      const void *data, const int64_t *indices, const int64_t *indptr,
+                      const void *B, int64_t ldb, const void *gC, int64_t ldg, int64_t n,
+                      void *grad_A, void *grad_B, int64_t ldgb, nm_stream stream);
+
+/* ---------------------------------------------------------------- SpGEMM
+ * C = A B, both CSR.  Stands in for spgemm_forward (cpp/sparse_csr.hpp:45-48,
+ * cpp/sparse_csr_cpu.cpp:117-216).  Two calls, because the caller must size
+ * C between them:
+ *
+ *   nm_spgemm_workspace_bytes  -> bytes of device scratch both phases need
+ *   nm_spgemm_symbolic         -> fills C_indptr (A_rows + 1 entries); the
+ *                                 caller reads nnz(C) = C_indptr[A_rows]
+ *                                 (its own device->host copy) and allocates
+ *   nm_spgemm_numeric          -> fills C_indices (ascending in each row) and
+ *                                 C_data; entries whose sum is 0 are kept,
+ *                                 as the reference keeps them.
+ *
+ * The same workspace (contents preserved) must be passed to both phases.
+ * Products of one output entry are added in the order of A's row, which is
+ * the reference's order. */
+int nm_spgemm_workspace_bytes(int64_t A_rows, int64_t B_cols, size_t *bytes);
+
+int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols,
+                       const int64_t *A_indices, const int64_t *A_indptr,
+                       const int64_t *B_indices, const int64_t *B_indptr,
+                       int64_t *C_indptr, void *workspace, size_t workspace_bytes,
+                       nm_stream stream);
+
+int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t B_cols,
+                      const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,
+                      const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
+                      const int64_t *C_indptr, int64_t *C_indices, void *C_data,
+                      void *workspace, size_t workspace_bytes, nm_stream stream);
+
+/* grad_A[(i,j)] = sum_c gC[i,c] B[j,c];  grad_B[(k,c)] = sum_i A[i,k] gC[i,c],
+ * both restricted to the stored patterns.  Stands in for spgemm_backward
+ * (cpp/sparse_csr.hpp:50-54, cpp/sparse_csr_cpu.cpp:218-307).  grad_B is
+ * cleared here and accumulated with atomics.  Either output may be NULL. */
+int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz,
+                       const void *gC, const int64_t *C_indices, const int64_t *C_indptr,
+                       const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,
+                       const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
+                       void *grad_A, void *grad_B, nm_stream stream);
+
+/* ---------------------------------------------------------------- SpTRSV
+ * Level-scheduled triangular solve.  Stands in for sptrsv_forward /
+ * sptrsv_backward (cpp/sparse_csr.hpp:94-105, cpp/sparse_csr_cpu.cpp:652-759).
+ *
+ * A plan holds the level schedule of one triangle of one sparsity pattern
+ * together with the structure of A^T, and is reused for every solve with that
+ * pattern (values may change) in either direction: x = A^{-1} b and, with
+ * `transposed` != 0, x = A^{-T} b, the system the backward solves
+ * (cpp/sparse_csr_cpu.cpp:733-738 builds A^T explicitly and flips `lower`).
+ * `lower` always describes A itself.
+ *
+ * The plan's device arrays live in caller-provided memory (`plan_mem`, which
+ * must stay allocated until nm_sptrsv_plan_destroy); `work` is scratch needed
+ * only during nm_sptrsv_analyse.  The handle itself is a small host object.
+ * nm_sptrsv_analyse synchronises the stream: it reads the level sizes back to
+ * lay out the launches.  Rows and entries are indexed with 32 bits inside a
+ * plan (NM_ERR_UNSUPPORTED beyond 2^31 - 2).
+ */
+typedef struct nm_sptrsv_plan nm_sptrsv_plan;
+
+int nm_sptrsv_plan_bytes(int64_t rows, int64_t nnz, size_t *plan_bytes, size_t *work_bytes);
+
+int nm_sptrsv_analyse(int64_t rows, int64_t nnz,
+                      const int64_t *indices, const int64_t *indptr, int lower,
+                      void *plan_mem, size_t plan_bytes, void *work, size_t work_bytes,
+                      nm_sptrsv_plan **plan, nm_stream stream);
+
+/* Number of dependency levels / of kernel launches one solve issues. */
+int64_t nm_sptrsv_plan_levels(const nm_sptrsv_plan *plan);
+int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan);
+
+void nm_sptrsv_plan_destroy(nm_sptrsv_plan *plan);
+
+/* x = T^{-1} b where T is the planned triangle of A (or its transpose).  Sums
+ * run in double for either dtype, in the walk order of the reference loop, and
+ * are rounded once at the end (cpp/sparse_csr_cpu.cpp:659-662, :722).
+ * `unit` != 0 ignores the stored diagonal.  `xwork` is device scratch of
+ * `rows` doubles, needed for NM_F32 only (NULL is fine for NM_F64).  x must
+ * not alias b. */
+int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
+                    const void *data, const int64_t *indices, const int64_t *indptr,
+                    int unit, const void *b, void *x, double *xwork, nm_stream stream);
+
+/* out[k] = alpha * a[row(k)] * b[col(k)] for every stored entry: the masked
+ * outer product behind grad_A of the solve (alpha = -1,
+ * cpp/sparse_csr_cpu.cpp:750-755) and of SpMV (alpha = 1, :60-65). */
+int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz,
+                    const int64_t *indices, const int64_t *indptr,
+                    double alpha, const void *a, const void *b, void *out,
+                    nm_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NUMML_HIP_H_ */

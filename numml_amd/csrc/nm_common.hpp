@@ -1,0 +1,90 @@
+// Shared host/device helpers of libnumml_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "numml_hip.h"
+
+namespace nm {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// Records `msg` as the calling thread's last error and returns `code`.
+int fail(int code, const char *fmt, ...);
+
+#define NM_HIP_TRY(expr)                                                          \
+    do {                                                                          \
+        hipError_t nm_e_ = (expr);                                                \
+        if (nm_e_ != hipSuccess)                                                  \
+            return ::nm::fail(NM_ERR_HIP, "%s failed: %s (%s:%d)", #expr,         \
+                              hipGetErrorString(nm_e_), __FILE__, __LINE__);      \
+    } while (0)
+
+// Checks the launch that was just enqueued.
+#define NM_LAUNCH_CHECK(name)                                                     \
+    do {                                                                          \
+        hipError_t nm_e_ = hipGetLastError();                                     \
+        if (nm_e_ != hipSuccess)                                                  \
+            return ::nm::fail(NM_ERR_HIP, "launch of %s failed: %s", name,        \
+                              hipGetErrorString(nm_e_));                          \
+    } while (0)
+
+#define NM_REQUIRE(cond, ...)                                                     \
+    do {                                                                          \
+        if (!(cond)) return ::nm::fail(NM_ERR_INVALID, __VA_ARGS__);              \
+    } while (0)
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Grid sizes are 32-bit in HIP; every launcher caps its 1-D grid below this
+// and the kernels stride.
+constexpr int64_t kMaxGrid = 1 << 30;
+
+inline hipStream_t as_stream(nm_stream s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- device helpers -------------------------------------------------------
+
+// Sum over the 64 lanes of a wavefront; every lane gets the total.
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Sum inside aligned groups of G consecutive lanes (G a power of two <= 64).
+template <int G, typename T>
+__device__ __forceinline__ T group_sum(T v) {
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Hardware floating-point atomic add without a returned value
+// (global_atomic_add_f32 / _f64).
+__device__ __forceinline__ void atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
+__device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
+
+// out[i] = v for i in [0, n): used instead of hipMemsetAsync so that callers
+// may capture these entry points into HIP graphs.
+template <typename T>
+__global__ void fill_kernel(T *__restrict__ out, int64_t n, T v) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = v;
+}
+
+template <typename T>
+inline int fill_async(T *out, int64_t n, T v, hipStream_t s) {
+    if (n <= 0) return NM_OK;
+    const int block = 256;
+    int64_t grid = ceil_div(n, (int64_t)block * 4);
+    if (grid > 65536) grid = 65536;
+    if (grid < 1) grid = 1;
+    hipLaunchKernelGGL(fill_kernel<T>, dim3((unsigned)grid), dim3(block), 0, s, out, n, v);
+    NM_LAUNCH_CHECK("fill_kernel");
+    return NM_OK;
+}
+
+}  // namespace nm

@@ -1,0 +1,578 @@
+// Hash-based CSR x CSR product (SpGEMM) and its backward for gfx950.
+//
+// Forward, two phases around the caller's allocation of C:
+//   symbolic: rows of A are binned by an upper bound on their products
+//             (sum of the lengths of the B rows they touch).  A group of lanes
+//             (8, 64 or 256, by bin) inserts the row's column indices into a
+//             hash set in LDS and counts the distinct ones; an exclusive scan
+//             of the counts is C_indptr.
+//   numeric : rows are re-binned by their exact length.  The group accumulates
+//             (column, value) pairs in an LDS hash table, walking A's row
+//             entry by entry and B's row across the lanes, so every output
+//             entry receives its products in the order of A's row -- the
+//             order of the serial SMMP loop (cpp/sparse_csr_cpu.cpp:182-212) --
+//             and then writes the table out ranked by column, so C's rows are
+//             ascending like the reference's.
+// Rows too long for an LDS table spill to a dense accumulator in global memory
+// (one slice of B_cols entries per spill workgroup).
+//
+// Backward: one lane per stored entry (i,k) of A walks row k of B, finds each
+// column in row i of C by bisection, and forms grad_A (a sum in ascending
+// column order, as the reference's merge, cpp/sparse_csr_cpu.cpp:246-278) and
+// grad_B (atomic adds) in one pass.
+//
+// Algorithmic HBM bytes of the forward (s = sizeof(value)):
+//   nnzA*(s+8) + rowsA*8 + products*(s+8) [upper; nnzB*(s+8) compulsory]
+//   + nnzC*(s+8) + rowsA*8
+#include "nm_common.hpp"
+#include "nm_scan.hpp"
+
+namespace {
+
+using nm::kWave;
+
+constexpr int32_t kEmpty = -1;
+constexpr int kBlock = 256;
+constexpr int kBins = 4;
+constexpr int kSpillGroups = 8;     // workgroups (and dense slices) of the spill path
+constexpr int kSpillBlock = 1024;
+
+// bin upper limits (inclusive); the last bin takes the rest and spills
+constexpr int32_t kSymLimit[3] = {64, 512, 8192};     // on the product bound
+constexpr int32_t kNumLimit[3] = {32, 512, 4096};     // on the exact row length
+// table sizes per bin
+constexpr int kSymTable0 = 128, kSymTable1 = 1024, kSymTable2 = 16384;
+constexpr int kNumTable0 = 64, kNumTable1 = 1024, kNumTable2 = 8192;
+
+struct Work {
+    int32_t *key;      // [rows] binning key (product bound, then exact length)
+    int32_t *perm;     // [rows] rows grouped by bin
+    int32_t *bins;     // [16]: count[0..3], offset[4..8], cursor[9..12]
+    int64_t *scan;     // scan scratch
+    int32_t *mark;     // [kSpillGroups * B_cols]
+    double *acc;       // [kSpillGroups * B_cols]
+};
+
+inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
+
+size_t work_layout(int64_t rows, int64_t B_cols, void *base, Work *w) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        void *p = base ? static_cast<char *>(base) + off : nullptr;
+        off += align_up(bytes);
+        return p;
+    };
+    int32_t *key = (int32_t *)take((rows + 1) * 4);
+    int32_t *perm = (int32_t *)take((rows + 1) * 4);
+    int32_t *bins = (int32_t *)take(16 * 4);
+    int64_t *scan = (int64_t *)take(nm::scan_scratch_bytes(rows + 1));
+    int32_t *mark = (int32_t *)take((size_t)kSpillGroups * (B_cols + 1) * 4);
+    double *acc = (double *)take((size_t)kSpillGroups * (B_cols + 1) * 8);
+    if (w) *w = Work{key, perm, bins, scan, mark, acc};
+    return off;
+}
+
+__device__ __forceinline__ uint32_t hash32(int32_t key) { return (uint32_t)key * 0x9E3779B1u; }
+
+template <int G> __device__ __forceinline__ void group_sync() {
+    if (G > kWave) __syncthreads();
+    else __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+}
+
+// Sum over a group of G lanes (G <= 64: shuffles; G == blockDim: via LDS).
+template <int G> __device__ __forceinline__ int group_total(int v, int *s_red) {
+    if (G <= kWave) return nm::group_sum<G>(v);
+    v = nm::wave_sum(v);
+    if ((threadIdx.x & (kWave - 1)) == 0) s_red[threadIdx.x / kWave] = v;
+    __syncthreads();
+    int t = 0;
+    for (int w = 0; w < G / kWave; ++w) t += s_red[w];
+    __syncthreads();
+    return t;
+}
+
+// ---- binning ---------------------------------------------------------------
+
+// key[i] = min(sum of B row lengths over A's row i, INT32_MAX); bins[b] counts.
+__global__ void product_bound_kernel(int64_t rows, const int64_t *__restrict__ A_indices,
+                                     const int64_t *__restrict__ A_indptr,
+                                     const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows; i += stride) {
+        int64_t ub = 0;
+        const int64_t e = A_indptr[i + 1];
+        for (int64_t jj = A_indptr[i]; jj < e; ++jj) {
+            const int64_t j = A_indices[jj];
+            ub += B_indptr[j + 1] - B_indptr[j];
+        }
+        key[i] = (int32_t)(ub > 0x7fffffff ? 0x7fffffff : ub);
+    }
+}
+
+// key[i] = C_indptr[i+1] - C_indptr[i]
+__global__ void row_length_kernel(int64_t rows, const int64_t *__restrict__ C_indptr,
+                                  int32_t *__restrict__ key) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows; i += stride)
+        key[i] = (int32_t)(C_indptr[i + 1] - C_indptr[i]);
+}
+
+__device__ __forceinline__ int bin_of(int32_t k, int32_t l0, int32_t l1, int32_t l2) {
+    return k <= l0 ? 0 : (k <= l1 ? 1 : (k <= l2 ? 2 : 3));
+}
+
+__global__ void bin_clear_kernel(int32_t *bins) {
+    if (threadIdx.x < 16) bins[threadIdx.x] = 0;
+}
+
+__global__ void bin_count_kernel(int64_t rows, const int32_t *__restrict__ key, int32_t l0, int32_t l1,
+                                 int32_t l2, int32_t *bins) {
+    __shared__ int s_cnt[kBins];
+    if (threadIdx.x < kBins) s_cnt[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows; i += stride)
+        atomicAdd(&s_cnt[bin_of(key[i], l0, l1, l2)], 1);
+    __syncthreads();
+    if (threadIdx.x < kBins && s_cnt[threadIdx.x]) atomicAdd(bins + threadIdx.x, s_cnt[threadIdx.x]);
+}
+
+__global__ void bin_offsets_kernel(int32_t *bins) {
+    if (threadIdx.x == 0) {
+        int32_t run = 0;
+        for (int b = 0; b < kBins; ++b) {
+            bins[4 + b] = run;
+            bins[9 + b] = run;  // cursor
+            run += bins[b];
+        }
+        bins[4 + kBins] = run;
+    }
+}
+
+// Rows are placed a workgroup at a time so that each bin keeps them in
+// near-ascending order (neighbouring rows share B rows and C lines).
+__global__ void bin_scatter_kernel(int64_t rows, const int32_t *__restrict__ key, int32_t l0, int32_t l1,
+                                   int32_t l2, int32_t *bins, int32_t *__restrict__ perm) {
+    __shared__ int s_cnt[kBins];
+    __shared__ int s_base[kBins];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x; i0 < rows; i0 += stride) {
+        if (threadIdx.x < kBins) s_cnt[threadIdx.x] = 0;
+        __syncthreads();
+        const int64_t i = i0 + threadIdx.x;
+        int b = 0, slot = 0;
+        if (i < rows) {
+            b = bin_of(key[i], l0, l1, l2);
+            slot = atomicAdd(&s_cnt[b], 1);
+        }
+        __syncthreads();
+        if (threadIdx.x < kBins) s_base[threadIdx.x] = atomicAdd(bins + 9 + threadIdx.x, s_cnt[threadIdx.x]);
+        __syncthreads();
+        if (i < rows) perm[s_base[b] + slot] = (int32_t)i;
+        __syncthreads();
+    }
+}
+
+int bin_rows(int64_t rows, const int32_t limit[3], const Work &w, hipStream_t s) {
+    int64_t grid = nm::ceil_div(rows, kBlock);
+    if (grid > 4096) grid = 4096;
+    if (grid < 1) grid = 1;
+    hipLaunchKernelGGL(bin_clear_kernel, dim3(1), dim3(64), 0, s, w.bins);
+    hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, w.key, limit[0],
+                       limit[1], limit[2], w.bins);
+    hipLaunchKernelGGL(bin_offsets_kernel, dim3(1), dim3(64), 0, s, w.bins);
+    hipLaunchKernelGGL(bin_scatter_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, w.key, limit[0],
+                       limit[1], limit[2], w.bins, w.perm);
+    NM_LAUNCH_CHECK("bin kernels");
+    return NM_OK;
+}
+
+// ---- symbolic ----------------------------------------------------------------
+
+template <int G, int TABLE>
+__global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
+    int bin, const int32_t *__restrict__ bins, const int32_t *__restrict__ perm,
+    const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
+    const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
+    int64_t *__restrict__ C_count) {
+    constexpr int GPB = kBlock / G;
+    __shared__ int32_t s_keys[GPB * TABLE];
+    __shared__ int s_red[kBlock / kWave];
+    const int gl = threadIdx.x % G, gi = threadIdx.x / G;
+    int32_t *tab = s_keys + gi * TABLE;
+    const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
+    for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
+        const int32_t idx = idx0 + gi;
+        const bool live = idx < b1;
+        for (int t = gl; t < TABLE; t += G) tab[t] = kEmpty;
+        group_sync<G>();
+        int cnt = 0;
+        int64_t row = 0;
+        if (live) {
+            row = perm[idx];
+            const int64_t je = A_indptr[row + 1];
+            for (int64_t jj = A_indptr[row]; jj < je; ++jj) {
+                const int64_t j = A_indices[jj];
+                const int64_t ke = B_indptr[j + 1];
+                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) {
+                    const int32_t key = (int32_t)B_indices[kk];
+                    uint32_t h = hash32(key) & (TABLE - 1);
+                    for (;;) {
+                        const int32_t old = atomicCAS(&tab[h], kEmpty, key);
+                        if (old == kEmpty) { ++cnt; break; }
+                        if (old == key) break;
+                        h = (h + 1) & (TABLE - 1);
+                    }
+                }
+            }
+        }
+        cnt = group_total<G>(cnt, s_red);
+        if (live && gl == 0) C_count[row] = cnt;
+        group_sync<G>();
+    }
+}
+
+// Spill path: distinct columns counted with a stamped dense marker per workgroup.
+__global__ __launch_bounds__(kSpillBlock) void symbolic_spill_kernel(
+    const int32_t *__restrict__ bins, const int32_t *__restrict__ perm, int64_t B_cols,
+    const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
+    const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr, int32_t *mark_all,
+    int64_t *__restrict__ C_count) {
+    __shared__ int s_red[kSpillBlock / kWave];
+    const int32_t b0 = bins[4 + 3], b1 = bins[5 + 3];
+    if (b0 + (int32_t)blockIdx.x >= b1) return;
+    int32_t *mark = mark_all + (size_t)blockIdx.x * (B_cols + 1);
+    for (int64_t c = threadIdx.x; c < B_cols; c += kSpillBlock) mark[c] = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    for (int32_t idx = b0 + blockIdx.x; idx < b1; idx += gridDim.x) {
+        const int64_t row = perm[idx];
+        const int32_t stamp = (int32_t)row + 1;
+        int cnt = 0;
+        const int64_t je = A_indptr[row + 1];
+        for (int64_t jj = A_indptr[row] + wave; jj < je; jj += kSpillBlock / kWave) {
+            const int64_t j = A_indices[jj];
+            const int64_t ke = B_indptr[j + 1];
+            for (int64_t kk = B_indptr[j] + lane; kk < ke; kk += kWave)
+                if (atomicExch(mark + B_indices[kk], stamp) != stamp) ++cnt;
+        }
+        cnt = nm::wave_sum(cnt);
+        if (lane == 0) s_red[wave] = cnt;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int t = 0;
+            for (int w = 0; w < kSpillBlock / kWave; ++w) t += s_red[w];
+            C_count[row] = t;
+        }
+        __syncthreads();
+    }
+}
+
+// ---- numeric -------------------------------------------------------------------
+
+template <typename T, int G, int TABLE>
+__global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
+    int bin, const int32_t *__restrict__ bins, const int32_t *__restrict__ perm,
+    const T *__restrict__ A_data, const int64_t *__restrict__ A_indices,
+    const int64_t *__restrict__ A_indptr, const T *__restrict__ B_data,
+    const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
+    const int64_t *__restrict__ C_indptr, int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
+    constexpr int GPB = kBlock / G;
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    T *s_vals = reinterpret_cast<T *>(s_raw);
+    int32_t *s_keys = reinterpret_cast<int32_t *>(s_raw + sizeof(T) * GPB * TABLE);
+    const int gl = threadIdx.x % G, gi = threadIdx.x / G;
+    int32_t *tab = s_keys + gi * TABLE;
+    T *val = s_vals + gi * TABLE;
+    const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
+    for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
+        const int32_t idx = idx0 + gi;
+        const bool live = idx < b1;
+        for (int t = gl; t < TABLE; t += G) { tab[t] = kEmpty; val[t] = T(0); }
+        group_sync<G>();
+        int64_t row = 0;
+        if (live) {
+            row = perm[idx];
+            const int64_t je = A_indptr[row + 1];
+            for (int64_t jj = A_indptr[row]; jj < je; ++jj) {
+                const int64_t j = A_indices[jj];
+                const T a = A_data[jj];
+                const int64_t ke = B_indptr[j + 1];
+                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) {
+                    const int32_t key = (int32_t)B_indices[kk];
+                    const T prod = a * B_data[kk];
+                    uint32_t h = hash32(key) & (TABLE - 1);
+                    for (;;) {
+                        const int32_t old = atomicCAS(&tab[h], kEmpty, key);
+                        if (old == kEmpty || old == key) break;
+                        h = (h + 1) & (TABLE - 1);
+                    }
+                    // the columns of one B row are distinct, so no other lane holds slot h now
+                    val[h] = val[h] + prod;
+                }
+                group_sync<G>();  // the next entry of A's row adds after this one
+            }
+        }
+        if (G > kWave) __syncthreads();
+        if (live) {
+            const int64_t base = C_indptr[row];
+            for (int t = gl; t < TABLE; t += G) {
+                const int32_t key = tab[t];
+                if (key == kEmpty) continue;
+                int rank = 0;
+                for (int u = 0; u < TABLE; ++u) rank += (uint32_t)tab[u] < (uint32_t)key;
+                C_indices[base + rank] = key;
+                C_data[base + rank] = val[t];
+            }
+        }
+        group_sync<G>();
+    }
+}
+
+// Spill path: dense accumulator slice per workgroup, emitted by a scan of the
+// touched column range (ascending by construction).
+template <typename T>
+__global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
+    const int32_t *__restrict__ bins, const int32_t *__restrict__ perm, int64_t B_cols,
+    const T *__restrict__ A_data, const int64_t *__restrict__ A_indices,
+    const int64_t *__restrict__ A_indptr, const T *__restrict__ B_data,
+    const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
+    const int64_t *__restrict__ C_indptr, int64_t *__restrict__ C_indices, T *__restrict__ C_data,
+    int32_t *mark_all, double *acc_all) {
+    __shared__ int64_t s_wave[kSpillBlock / kWave];
+    __shared__ unsigned long long s_lo, s_hi;
+    const int32_t b0 = bins[4 + 3], b1 = bins[5 + 3];
+    if (b0 + (int32_t)blockIdx.x >= b1) return;
+    int32_t *mark = mark_all + (size_t)blockIdx.x * (B_cols + 1);
+    T *acc = reinterpret_cast<T *>(acc_all + (size_t)blockIdx.x * (B_cols + 1));
+    for (int64_t c = threadIdx.x; c < B_cols; c += kSpillBlock) { mark[c] = 0; acc[c] = T(0); }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    for (int32_t idx = b0 + blockIdx.x; idx < b1; idx += gridDim.x) {
+        const int64_t row = perm[idx];
+        const int32_t stamp = -((int32_t)row + 1);
+        if (threadIdx.x == 0) { s_lo = ~0ull; s_hi = 0ull; }
+        __syncthreads();
+        unsigned long long lo = ~0ull, hi = 0ull;
+        const int64_t je = A_indptr[row + 1];
+        for (int64_t jj = A_indptr[row] + wave; jj < je; jj += kSpillBlock / kWave) {
+            const int64_t j = A_indices[jj];
+            const T a = A_data[jj];
+            const int64_t ke = B_indptr[j + 1];
+            for (int64_t kk = B_indptr[j] + lane; kk < ke; kk += kWave) {
+                const unsigned long long c = (unsigned long long)B_indices[kk];
+                nm::atomic_add(acc + c, a * B_data[kk]);
+                mark[c] = stamp;
+                lo = c < lo ? c : lo;
+                hi = c > hi ? c : hi;
+            }
+        }
+        if (lo != ~0ull) { atomicMin(&s_lo, lo); atomicMax(&s_hi, hi); }
+        __syncthreads();
+        const int64_t c_lo = (int64_t)s_lo, c_hi = (int64_t)s_hi;
+        int64_t out = C_indptr[row];
+        if (s_lo != ~0ull) {
+            for (int64_t c0 = c_lo; c0 <= c_hi; c0 += kSpillBlock) {
+                const int64_t c = c0 + threadIdx.x;
+                const bool hit = c <= c_hi && mark[c] == stamp;
+                int64_t total;
+                const int64_t pre = nm::block_exclusive_scan(hit ? 1 : 0, s_wave, total);
+                if (hit) {
+                    C_indices[out + pre] = c;
+                    C_data[out + pre] = acc[c];
+                    acc[c] = T(0);
+                }
+                out += total;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ---- backward --------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
+    int64_t A_rows, int64_t A_nnz, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
+    const int64_t *__restrict__ C_indptr, const T *__restrict__ A_data,
+    const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
+    const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
+    const int64_t *__restrict__ B_indptr, T *__restrict__ grad_A, T *__restrict__ grad_B) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t ai = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ai < A_nnz; ai += stride) {
+        int64_t lo = 0, hi = A_rows + 1;  // first p with A_indptr[p] > ai
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (A_indptr[mid] <= ai) lo = mid + 1; else hi = mid;
+        }
+        const int64_t i = lo - 1;
+        const int64_t k = A_indices[ai];
+        const T a = grad_B ? A_data[ai] : T(0);
+        const int64_t cb = C_indptr[i], ce = C_indptr[i + 1];
+        const int64_t be = B_indptr[k + 1];
+        T acc = 0;
+        int64_t from = cb;  // both rows ascend, so each search starts where the last one ended
+        for (int64_t kk = B_indptr[k]; kk < be; ++kk) {
+            const int64_t c = B_indices[kk];
+            int64_t l = from, h = ce;
+            while (l < h) {
+                const int64_t mid = (l + h) >> 1;
+                if (C_indices[mid] < c) l = mid + 1; else h = mid;
+            }
+            from = l;
+            if (l < ce && C_indices[l] == c) {
+                const T g = gC[l];
+                acc += g * B_data[kk];
+                if (grad_B) nm::atomic_add(grad_B + kk, a * g);
+            }
+        }
+        if (grad_A) grad_A[ai] = acc;
+    }
+}
+
+int check_common(int64_t A_rows, int64_t B_cols) {
+    NM_REQUIRE(A_rows >= 0 && B_cols >= 0, "negative size");
+    if (A_rows >= 0x7ffffffe || B_cols >= 0x7ffffffe)
+        return nm::fail(NM_ERR_UNSUPPORTED, "spgemm indexes rows and columns with 32 bits inside its tables");
+    return NM_OK;
+}
+
+constexpr unsigned kPersistGrid = 4096;
+
+template <typename T>
+int launch_numeric(const Work &w, int64_t B_cols, const void *A_data, const int64_t *A_indices,
+                   const int64_t *A_indptr, const void *B_data, const int64_t *B_indices,
+                   const int64_t *B_indptr, const int64_t *C_indptr, int64_t *C_indices, void *C_data,
+                   hipStream_t s) {
+    const T *Ad = (const T *)A_data, *Bd = (const T *)B_data;
+    T *Cd = (T *)C_data;
+    constexpr size_t per = sizeof(T) + sizeof(int32_t);
+    {
+        auto k = numeric_hash_kernel<T, 8, kNumTable0>;
+        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 8) * kNumTable0, s, 0, w.bins,
+                           w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
+        NM_LAUNCH_CHECK("numeric_hash_kernel<8>");
+    }
+    {
+        auto k = numeric_hash_kernel<T, 64, kNumTable1>;
+        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 64) * kNumTable1, s, 1, w.bins,
+                           w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
+        NM_LAUNCH_CHECK("numeric_hash_kernel<64>");
+    }
+    {
+        auto k = numeric_hash_kernel<T, 256, kNumTable2>;
+        const size_t lds = per * kNumTable2;
+        NM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(1024), dim3(kBlock), lds, s, 2, w.bins, w.perm, Ad, A_indices, A_indptr, Bd,
+                           B_indices, B_indptr, C_indptr, C_indices, Cd);
+        NM_LAUNCH_CHECK("numeric_hash_kernel<256>");
+    }
+    hipLaunchKernelGGL(numeric_spill_kernel<T>, dim3(kSpillGroups), dim3(kSpillBlock), 0, s, w.bins, w.perm,
+                       B_cols, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd, w.mark,
+                       w.acc);
+    NM_LAUNCH_CHECK("numeric_spill_kernel");
+    return NM_OK;
+}
+
+}  // namespace
+
+extern "C" int nm_spgemm_workspace_bytes(int64_t A_rows, int64_t B_cols, size_t *bytes) {
+    NM_REQUIRE(bytes != nullptr, "bytes is null");
+    if (int rc = check_common(A_rows, B_cols)) return rc;
+    *bytes = work_layout(A_rows, B_cols, nullptr, nullptr);
+    return NM_OK;
+}
+
+extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t *A_indices,
+                                  const int64_t *A_indptr, const int64_t *B_indices, const int64_t *B_indptr,
+                                  int64_t *C_indptr, void *workspace, size_t workspace_bytes,
+                                  nm_stream stream) {
+    if (int rc = check_common(A_rows, B_cols)) return rc;
+    NM_REQUIRE(A_cols >= 0, "negative size");
+    NM_REQUIRE(A_indptr && B_indptr && C_indptr && workspace, "null pointer argument");
+    Work w;
+    const size_t need = work_layout(A_rows, B_cols, workspace, &w);
+    if (workspace_bytes < need)
+        return nm::fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    hipStream_t s = nm::as_stream(stream);
+    if (int rc = nm::fill_async(C_indptr + A_rows, 1, (int64_t)0, s)) return rc;
+    if (A_rows == 0) return NM_OK;
+
+    int64_t grid = nm::ceil_div(A_rows, kBlock);
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(product_bound_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_indices,
+                       A_indptr, B_indptr, w.key);
+    NM_LAUNCH_CHECK("product_bound_kernel");
+    if (int rc = bin_rows(A_rows, kSymLimit, w, s)) return rc;
+
+    hipLaunchKernelGGL((symbolic_hash_kernel<8, kSymTable0>), dim3(kPersistGrid), dim3(kBlock), 0, s, 0, w.bins,
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+    NM_LAUNCH_CHECK("symbolic_hash_kernel<8>");
+    hipLaunchKernelGGL((symbolic_hash_kernel<64, kSymTable1>), dim3(kPersistGrid), dim3(kBlock), 0, s, 1, w.bins,
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+    NM_LAUNCH_CHECK("symbolic_hash_kernel<64>");
+    hipLaunchKernelGGL((symbolic_hash_kernel<256, kSymTable2>), dim3(1024), dim3(kBlock), 0, s, 2, w.bins, w.perm,
+                       A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+    NM_LAUNCH_CHECK("symbolic_hash_kernel<256>");
+    hipLaunchKernelGGL(symbolic_spill_kernel, dim3(kSpillGroups), dim3(kSpillBlock), 0, s, w.bins, w.perm, B_cols,
+                       A_indices, A_indptr, B_indices, B_indptr, w.mark, C_indptr);
+    NM_LAUNCH_CHECK("symbolic_spill_kernel");
+    // counts sit in C_indptr[0, rows), C_indptr[rows] = 0: the exclusive scan is the row pointer
+    return nm::scan_exclusive_i64(C_indptr, A_rows + 1, w.scan, s);
+}
+
+extern "C" int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t B_cols,
+                                 const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,
+                                 const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
+                                 const int64_t *C_indptr, int64_t *C_indices, void *C_data, void *workspace,
+                                 size_t workspace_bytes, nm_stream stream) {
+    if (int rc = check_common(A_rows, B_cols)) return rc;
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(A_indptr && B_indptr && C_indptr && workspace, "null pointer argument");
+    Work w;
+    const size_t need = work_layout(A_rows, B_cols, workspace, &w);
+    if (workspace_bytes < need)
+        return nm::fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    if (A_rows == 0) return NM_OK;
+    hipStream_t s = nm::as_stream(stream);
+    int64_t grid = nm::ceil_div(A_rows, kBlock);
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(row_length_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, C_indptr, w.key);
+    NM_LAUNCH_CHECK("row_length_kernel");
+    if (int rc = bin_rows(A_rows, kNumLimit, w, s)) return rc;
+    if (dt == NM_F32)
+        return launch_numeric<float>(w, B_cols, A_data, A_indices, A_indptr, B_data, B_indices, B_indptr,
+                                     C_indptr, C_indices, C_data, s);
+    return launch_numeric<double>(w, B_cols, A_data, A_indices, A_indptr, B_data, B_indices, B_indptr, C_indptr,
+                                  C_indices, C_data, s);
+}
+
+extern "C" int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, const void *gC,
+                                  const int64_t *C_indices, const int64_t *C_indptr, const void *A_data,
+                                  const int64_t *A_indices, const int64_t *A_indptr, const void *B_data,
+                                  const int64_t *B_indices, const int64_t *B_indptr, void *grad_A,
+                                  void *grad_B, nm_stream stream) {
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(A_rows >= 0 && A_nnz >= 0 && B_nnz >= 0, "negative size");
+    hipStream_t s = nm::as_stream(stream);
+    if (grad_B) {
+        int rc = dt == NM_F32 ? nm::fill_async((float *)grad_B, B_nnz, 0.0f, s)
+                              : nm::fill_async((double *)grad_B, B_nnz, 0.0, s);
+        if (rc) return rc;
+    }
+    if (A_nnz == 0 || A_rows == 0 || (!grad_A && !grad_B)) return NM_OK;
+    NM_REQUIRE(C_indptr && A_indices && A_indptr && B_indptr && A_data, "null pointer argument");
+    int64_t grid = nm::ceil_div(A_nnz, kBlock);
+    if (grid > 1 << 20) grid = 1 << 20;
+    if (dt == NM_F32)
+        hipLaunchKernelGGL(spgemm_bwd_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_nnz,
+                           (const float *)gC, C_indices, C_indptr, (const float *)A_data, A_indices, A_indptr,
+                           (const float *)B_data, B_indices, B_indptr, (float *)grad_A, (float *)grad_B);
+    else
+        hipLaunchKernelGGL(spgemm_bwd_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_nnz,
+                           (const double *)gC, C_indices, C_indptr, (const double *)A_data, A_indices, A_indptr,
+                           (const double *)B_data, B_indices, B_indptr, (double *)grad_A, (double *)grad_B);
+    NM_LAUNCH_CHECK("spgemm_bwd_kernel");
+    return NM_OK;
+}

@@ -1,0 +1,247 @@
+// CSR SpMV forward and its fused backward for gfx950.
+//
+// Work mapping ("row-block streaming"): one 256-lane workgroup owns R
+// consecutive rows.  It stages the rows' offsets in LDS and, when the block's
+// stored entries fit the LDS tile, walks them with fully coalesced loads of
+// `data` and `indices` (lane k takes entry k), leaving the per-entry results in
+// LDS; one lane per row then adds its row's slice in storage order, which is
+// the summation order of the serial CPU loop (cpp/sparse_csr_cpu.cpp:29-35),
+// so short rows reproduce it bit for bit.  Blocks whose entries do not fit
+// (long rows) switch to one wavefront per long row with a cross-lane
+// reduction, and one lane per short row.
+//
+// Algorithmic HBM bytes, s = sizeof(value):
+//   forward : nnz*(s+8) + (rows+1)*8 + cols*s + rows*s
+//   backward: nnz*(s+8) + (rows+1)*8 + rows*s + cols*s + nnz*s + cols*s
+#include "nm_common.hpp"
+
+namespace {
+
+using nm::kWave;
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+// Rows of at least this many entries get a whole wavefront on the long-row path.
+constexpr int kLongRow = 32;
+
+template <typename T> struct Tile;
+template <> struct Tile<float>  { static constexpr int R = 512; static constexpr int CAP = 4096; };
+template <> struct Tile<double> { static constexpr int R = 512; static constexpr int CAP = 4096; };
+
+// Loads the block's row offsets relative to `base` into LDS, clamped to CAP+1
+// so that they fit 32 bits whatever the block holds.
+template <int R, int CAP>
+__device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ indptr, int64_t r0, int nr,
+                                              int64_t base, int32_t *s_off) {
+    for (int t = threadIdx.x; t <= nr; t += kBlock) {
+        const int64_t d = indptr[r0 + t] - base;
+        s_off[t] = (int32_t)(d > CAP ? CAP + 1 : d);
+    }
+}
+
+template <typename T, int R, int CAP>
+__global__ __launch_bounds__(kBlock) void spmv_fwd_kernel(
+    int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
+    const int64_t *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y) {
+    __shared__ int32_t s_off[R + 1];
+    __shared__ T s_prod[CAP];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+
+    for (int64_t r0 = (int64_t)blockIdx.x * R; r0 < rows; r0 += (int64_t)gridDim.x * R) {
+        const int nr = (int)(rows - r0 < R ? rows - r0 : R);
+        const int64_t base = indptr[r0];
+        stage_offsets<R, CAP>(indptr, r0, nr, base, s_off);
+        __syncthreads();
+        const int n = s_off[nr];
+        if (n <= CAP) {
+            const T *__restrict__ d = data + base;
+            const int64_t *__restrict__ ci = indices + base;
+            int k = threadIdx.x;
+            for (; k + 3 * kBlock < n; k += 4 * kBlock) {
+                const int64_t c0 = ci[k], c1 = ci[k + kBlock], c2 = ci[k + 2 * kBlock], c3 = ci[k + 3 * kBlock];
+                const T a0 = d[k], a1 = d[k + kBlock], a2 = d[k + 2 * kBlock], a3 = d[k + 3 * kBlock];
+                const T x0 = x[c0], x1 = x[c1], x2 = x[c2], x3 = x[c3];
+                s_prod[k] = a0 * x0;
+                s_prod[k + kBlock] = a1 * x1;
+                s_prod[k + 2 * kBlock] = a2 * x2;
+                s_prod[k + 3 * kBlock] = a3 * x3;
+            }
+            for (; k < n; k += kBlock) s_prod[k] = d[k] * x[ci[k]];
+            __syncthreads();
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                const int e = s_off[t + 1];
+                T acc = 0;
+                for (int j = s_off[t]; j < e; ++j) acc += s_prod[j];
+                y[r0 + t] = acc;
+            }
+        } else {
+            // short rows: one lane each, straight from global memory
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                const int64_t b = indptr[r0 + t], e = indptr[r0 + t + 1];
+                if (e - b >= kLongRow) continue;
+                T acc = 0;
+                for (int64_t k = b; k < e; ++k) acc += data[k] * x[indices[k]];
+                y[r0 + t] = acc;
+            }
+            // long rows: one wavefront each
+            for (int t = wave; t < nr; t += kWavesPerBlock) {
+                const int64_t b = indptr[r0 + t], e = indptr[r0 + t + 1];
+                if (e - b < kLongRow) continue;
+                T acc = 0;
+                for (int64_t k = b + lane; k < e; k += kWave) acc += data[k] * x[indices[k]];
+                acc = nm::wave_sum(acc);
+                if (lane == 0) y[r0 + t] = acc;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Fused backward: out_A[k] = alpha * (a[row] * b[col]) and, when grad_x is
+// given, grad_x[col] += a[row] * data[k].  With grad_x == nullptr this is the
+// masked outer product (cpp/sparse_csr_cpu.cpp:60-65 and :750-755).
+template <typename T, int R, int CAP>
+__global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
+    int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
+    const int64_t *__restrict__ indptr, const T *__restrict__ a, const T *__restrict__ b, T alpha,
+    T *__restrict__ out_A, T *__restrict__ grad_x) {
+    __shared__ int32_t s_off[R + 1];
+    __shared__ T s_a[CAP];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+
+    for (int64_t r0 = (int64_t)blockIdx.x * R; r0 < rows; r0 += (int64_t)gridDim.x * R) {
+        const int nr = (int)(rows - r0 < R ? rows - r0 : R);
+        const int64_t base = indptr[r0];
+        stage_offsets<R, CAP>(indptr, r0, nr, base, s_off);
+        __syncthreads();
+        const int n = s_off[nr];
+        if (n <= CAP) {
+            // spread a[row] over the row's entries
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                const T av = a[r0 + t];
+                const int e = s_off[t + 1];
+                for (int j = s_off[t]; j < e; ++j) s_a[j] = av;
+            }
+            __syncthreads();
+            const int64_t *__restrict__ ci = indices + base;
+            for (int k = threadIdx.x; k < n; k += kBlock) {
+                const int64_t c = ci[k];
+                const T av = s_a[k];
+                if (out_A) out_A[base + k] = alpha * (av * b[c]);
+                if (grad_x) nm::atomic_add(grad_x + c, av * data[base + k]);
+            }
+        } else {
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                const int64_t rb = indptr[r0 + t], re = indptr[r0 + t + 1];
+                if (re - rb >= kLongRow) continue;
+                const T av = a[r0 + t];
+                for (int64_t k = rb; k < re; ++k) {
+                    const int64_t c = indices[k];
+                    if (out_A) out_A[k] = alpha * (av * b[c]);
+                    if (grad_x) nm::atomic_add(grad_x + c, av * data[k]);
+                }
+            }
+            for (int t = wave; t < nr; t += kWavesPerBlock) {
+                const int64_t rb = indptr[r0 + t], re = indptr[r0 + t + 1];
+                if (re - rb < kLongRow) continue;
+                const T av = a[r0 + t];
+                for (int64_t k = rb + lane; k < re; k += kWave) {
+                    const int64_t c = indices[k];
+                    if (out_A) out_A[k] = alpha * (av * b[c]);
+                    if (grad_x) nm::atomic_add(grad_x + c, av * data[k]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const int64_t *indices,
+              const int64_t *indptr) {
+    NM_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0, "negative size (rows=%lld cols=%lld nnz=%lld)",
+               (long long)rows, (long long)cols, (long long)nnz);
+    NM_REQUIRE(indptr != nullptr, "indptr is null");
+    NM_REQUIRE(nnz == 0 || (data != nullptr && indices != nullptr), "data/indices null with nnz > 0");
+    return NM_OK;
+}
+
+template <typename T>
+int launch_fwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *x,
+               T *y, hipStream_t s) {
+    constexpr int R = Tile<T>::R, CAP = Tile<T>::CAP;
+    int64_t grid = nm::ceil_div(rows, R);
+    if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+    hipLaunchKernelGGL((spmv_fwd_kernel<T, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, data,
+                       indices, indptr, x, y);
+    NM_LAUNCH_CHECK("spmv_fwd_kernel");
+    return NM_OK;
+}
+
+template <typename T>
+int launch_bwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *a,
+               const T *b, T alpha, T *out_A, T *grad_x, hipStream_t s) {
+    constexpr int R = Tile<T>::R, CAP = Tile<T>::CAP;
+    int64_t grid = nm::ceil_div(rows, R);
+    if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+    hipLaunchKernelGGL((spmv_bwd_kernel<T, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, data,
+                       indices, indptr, a, b, alpha, out_A, grad_x);
+    NM_LAUNCH_CHECK("spmv_bwd_kernel");
+    return NM_OK;
+}
+
+}  // namespace
+
+extern "C" int nm_spgemv_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                 const int64_t *indices, const int64_t *indptr, const void *x, void *y,
+                                 nm_stream stream) {
+    if (int rc = check_csr(rows, cols, nnz, data, indices, indptr)) return rc;
+    if (rows == 0) return NM_OK;
+    NM_REQUIRE(y != nullptr, "y is null");
+    NM_REQUIRE(cols == 0 || x != nullptr, "x is null");
+    hipStream_t s = nm::as_stream(stream);
+    switch (dt) {
+        case NM_F32:
+            return launch_fwd<float>(rows, (const float *)data, indices, indptr, (const float *)x, (float *)y, s);
+        case NM_F64:
+            return launch_fwd<double>(rows, (const double *)data, indices, indptr, (const double *)x,
+                                      (double *)y, s);
+    }
+    return nm::fail(NM_ERR_INVALID, "unknown dtype %d", (int)dt);
+}
+
+extern "C" int nm_spgemv_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                  const int64_t *indices, const int64_t *indptr, const void *x,
+                                  const void *g, void *grad_A, void *grad_x, nm_stream stream) {
+    if (int rc = check_csr(rows, cols, nnz, data, indices, indptr)) return rc;
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    hipStream_t s = nm::as_stream(stream);
+    if (grad_x) {
+        int rc = dt == NM_F32 ? nm::fill_async((float *)grad_x, cols, 0.0f, s)
+                              : nm::fill_async((double *)grad_x, cols, 0.0, s);
+        if (rc) return rc;
+    }
+    if (rows == 0 || nnz == 0 || (!grad_A && !grad_x)) return NM_OK;
+    NM_REQUIRE(g != nullptr && x != nullptr, "g or x is null");
+    if (dt == NM_F32)
+        return launch_bwd<float>(rows, (const float *)data, indices, indptr, (const float *)g,
+                                 (const float *)x, 1.0f, (float *)grad_A, (float *)grad_x, s);
+    return launch_bwd<double>(rows, (const double *)data, indices, indptr, (const double *)g,
+                              (const double *)x, 1.0, (double *)grad_A, (double *)grad_x, s);
+}
+
+extern "C" int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz, const int64_t *indices,
+                               const int64_t *indptr, double alpha, const void *a, const void *b, void *out,
+                               nm_stream stream) {
+    NM_REQUIRE(rows >= 0 && nnz >= 0 && indptr != nullptr, "bad sizes or null indptr");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    if (rows == 0 || nnz == 0) return NM_OK;
+    NM_REQUIRE(indices && a && b && out, "null pointer argument");
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F32)
+        return launch_bwd<float>(rows, nullptr, indices, indptr, (const float *)a, (const float *)b,
+                                 (float)alpha, (float *)out, nullptr, s);
+    return launch_bwd<double>(rows, nullptr, indices, indptr, (const double *)a, (const double *)b, alpha,
+                              (double *)out, nullptr, s);
+}

@@ -11,7 +11,7 @@ on every machine.
 import numpy as np
 
 __all__ = [
-    "poisson2d", "laplace3d", "poisson2d_lower", "powerlaw", "tridiag",
+    "poisson2d", "laplace3d", "poisson2d_lower", "powerlaw", "tridiag", "bidiag",
     "random_csr", "random_tri",
 ]
 
@@ -97,6 +97,18 @@ def tridiag(n, dtype=np.float64, lo=-1.0, di=2.0, up=-1.0):
     numml/tests/test_spmv.py:9-10)."""
     r = np.arange(n, dtype=np.int64)
     legs = [(-1, r > 0, lo), (0, np.ones(n, bool), di), (1, r < n - 1, up)]
+    data, indices, indptr = _stencil_csr(legs, n)
+    return data.astype(dtype), indices, indptr, (n, n)
+
+
+def bidiag(n, dtype=np.float64, lower=True, di=2.0, off=-1.0):
+    """Bidiagonal ``2I - E_-1`` (or its transpose), the reference's triangular-solve
+    timing matrix (demos/timing.py:520-558): n dependency levels of one row each."""
+    r = np.arange(n, dtype=np.int64)
+    if lower:
+        legs = [(-1, r > 0, off), (0, np.ones(n, bool), di)]
+    else:
+        legs = [(0, np.ones(n, bool), di), (1, r < n - 1, off)]
     data, indices, indptr = _stencil_csr(legs, n)
     return data.astype(dtype), indices, indptr, (n, n)
 

@@ -1,0 +1,306 @@
+"""Stand-in for the reference's extension module ``numml_torch_cpp``.
+
+Exports the eight hot-path functions with the reference's names, positional
+signatures and return conventions (cpp/sparse_csr.cpp:307-319 binds them;
+cpp/sparse_csr.hpp:32-105 declares them), implemented on the HIP kernels of
+libnumml_hip.so.  torch is used for device memory (outputs and scratch come
+from its caching allocator) and for the current stream, nothing else.
+
+Unlike the reference there is no CPU implementation behind these functions:
+tensors that are not on a HIP device raise ``RuntimeError``.
+"""
+import collections
+import ctypes
+import threading
+
+import torch
+
+from . import _lib
+
+__all__ = [
+    "spgemv_forward", "spgemv_backward", "spdmm_forward", "spdmm_backward",
+    "spgemm_forward", "spgemm_backward", "sptrsv_forward", "sptrsv_backward",
+    "clear_plan_cache",
+]
+
+
+def _dt(t):
+    if t.dtype == torch.float32:
+        return _lib.NM_F32
+    if t.dtype == torch.float64:
+        return _lib.NM_F64
+    # the reference dispatches with AT_DISPATCH_FLOATING_TYPES (cpp/sparse_csr_cpu.cpp:22)
+    raise RuntimeError(f"numml_amd: values must be float32 or float64, got {t.dtype}")
+
+
+def _need_device(*tensors):
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError(
+            "numml_amd: this backend runs on HIP devices only; got a tensor on "
+            f"'{dev}' (no CPU implementation is provided)")
+    for t in tensors[1:]:
+        if t.device != dev:
+            devs = ", ".join(str(x.device) for x in tensors)
+            raise RuntimeError(f"expected all tensors to be on the same device, but got {devs}")
+    return dev
+
+
+def _idx(t, name):
+    if t.dtype != torch.int64:
+        # the reference reads structure through accessor<int64_t, 1> (cpp/sparse_csr_cpu.cpp:24-25)
+        raise RuntimeError(f"expected scalar type Long for {name} but found {t.dtype}")
+    return t.contiguous()
+
+
+def _same_dtype(a, b, what):
+    if a.dtype != b.dtype:
+        raise RuntimeError(f"expected {what} of type {a.dtype} but found {b.dtype}")
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream(dev):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _rowmajor(M):
+    """2-D tensor with unit column stride (copied only when it is not already)."""
+    if M.dim() != 2:
+        raise RuntimeError(f"expected a 2-D tensor, got {M.dim()}-D")
+    if M.shape[1] > 1 and M.stride(1) != 1:
+        M = M.contiguous()
+    if M.shape[0] > 1 and M.stride(0) < max(M.shape[1], 1):
+        M = M.contiguous()
+    ld = M.stride(0) if M.shape[0] > 1 else max(M.shape[1], 1)
+    return M, ld
+
+
+# --------------------------------------------------------------------- SpMV
+
+def spgemv_forward(A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
+    """y = A x  (cpp/sparse_csr.hpp:32-36)."""
+    dev = _need_device(A_data, A_col_ind, A_rowptr, x)
+    _same_dtype(A_data, x, "x")
+    A_data, x = A_data.contiguous(), x.contiguous()
+    A_col_ind, A_rowptr = _idx(A_col_ind, "A_col_ind"), _idx(A_rowptr, "A_rowptr")
+    if x.dim() != 1:
+        raise RuntimeError(f"expected 1-D x, got {x.dim()}-D")
+    with torch.cuda.device(dev):
+        y = torch.empty(A_rows, dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_spgemv_forward(
+            _dt(A_data), A_rows, x.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_col_ind),
+            _ptr(A_rowptr), _ptr(x), _ptr(y), _stream(dev)), "nm_spgemv_forward")
+    return y
+
+
+def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
+    """[grad_A, grad_x]  (cpp/sparse_csr.hpp:38-42)."""
+    dev = _need_device(grad_z, A_data, A_col_ind, A_rowptr, x)
+    _same_dtype(A_data, x, "x")
+    _same_dtype(A_data, grad_z, "grad_z")
+    A_data, x, grad_z = A_data.contiguous(), x.contiguous(), grad_z.contiguous()
+    A_col_ind, A_rowptr = _idx(A_col_ind, "A_col_ind"), _idx(A_rowptr, "A_rowptr")
+    with torch.cuda.device(dev):
+        grad_A = torch.empty_like(A_data)
+        grad_x = torch.empty_like(x)
+        _lib.check(_lib.lib().nm_spgemv_backward(
+            _dt(A_data), A_rows, x.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_col_ind),
+            _ptr(A_rowptr), _ptr(x), _ptr(grad_z), _ptr(grad_A), _ptr(grad_x), _stream(dev)),
+            "nm_spgemv_backward")
+    return [grad_A, grad_x]
+
+
+# --------------------------------------------------------------------- SpMM
+
+def spdmm_forward(A_rows, A_cols, A_data, A_indices, A_indptr, B):
+    """C = A B, B dense 2-D  (cpp/sparse_csr.hpp:81-85)."""
+    dev = _need_device(A_data, A_indices, A_indptr, B)
+    _same_dtype(A_data, B, "B")
+    A_data = A_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    B, ldb = _rowmajor(B)
+    n = B.shape[1]
+    with torch.cuda.device(dev):
+        C = torch.empty((A_rows, n), dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_spdmm_forward(
+            _dt(A_data), A_rows, B.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_indices),
+            _ptr(A_indptr), _ptr(B), ldb, n, _ptr(C), max(n, 1), _stream(dev)), "nm_spdmm_forward")
+    return C
+
+
+def spdmm_backward(A_rows, A_cols, A_data, A_indices, A_indptr, B, grad_C):
+    """[grad_A, grad_B]  (cpp/sparse_csr.hpp:87-91)."""
+    dev = _need_device(A_data, A_indices, A_indptr, B, grad_C)
+    _same_dtype(A_data, B, "B")
+    _same_dtype(A_data, grad_C, "grad_C")
+    A_data = A_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    B, ldb = _rowmajor(B)
+    grad_C, ldg = _rowmajor(grad_C)
+    n = B.shape[1]
+    with torch.cuda.device(dev):
+        grad_A = torch.empty_like(A_data)
+        grad_B = torch.empty((B.shape[0], n), dtype=B.dtype, device=dev)
+        _lib.check(_lib.lib().nm_spdmm_backward(
+            _dt(A_data), A_rows, B.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_indices),
+            _ptr(A_indptr), _ptr(B), ldb, _ptr(grad_C), ldg, n, _ptr(grad_A), _ptr(grad_B),
+            max(n, 1), _stream(dev)), "nm_spdmm_backward")
+    return [grad_A, grad_B]
+
+
+# ------------------------------------------------------------------- SpGEMM
+
+def spgemm_forward(A_rows, A_cols, A_data, A_indices, A_indptr,
+                   B_rows, B_cols, B_data, B_indices, B_indptr):
+    """[C_data, C_indices, C_indptr]  (cpp/sparse_csr.hpp:45-48).
+
+    One device->host read of nnz(C) sits between the two phases; it is inherent
+    to the interface, which returns exactly-sized tensors.
+    """
+    dev = _need_device(A_data, A_indices, A_indptr, B_data, B_indices, B_indptr)
+    _same_dtype(A_data, B_data, "B_data")
+    A_data, B_data = A_data.contiguous(), B_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    B_indices, B_indptr = _idx(B_indices, "B_indices"), _idx(B_indptr, "B_indptr")
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(L.nm_spgemm_workspace_bytes(A_rows, B_cols, ctypes.byref(nbytes)),
+                   "nm_spgemm_workspace_bytes")
+        work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+        C_indptr = torch.empty(A_rows + 1, dtype=torch.int64, device=dev)
+        st = _stream(dev)
+        _lib.check(L.nm_spgemm_symbolic(
+            A_rows, A_cols, B_cols, _ptr(A_indices), _ptr(A_indptr), _ptr(B_indices), _ptr(B_indptr),
+            _ptr(C_indptr), _ptr(work), nbytes.value, st), "nm_spgemm_symbolic")
+        nnz_c = int(C_indptr[-1].item())
+        C_indices = torch.empty(nnz_c, dtype=torch.int64, device=dev)
+        C_data = torch.empty(nnz_c, dtype=A_data.dtype, device=dev)
+        _lib.check(L.nm_spgemm_numeric(
+            _dt(A_data), A_rows, A_cols, B_cols, _ptr(A_data), _ptr(A_indices), _ptr(A_indptr),
+            _ptr(B_data), _ptr(B_indices), _ptr(B_indptr), _ptr(C_indptr), _ptr(C_indices),
+            _ptr(C_data), _ptr(work), nbytes.value, st), "nm_spgemm_numeric")
+    return [C_data, C_indices, C_indptr]
+
+
+def spgemm_backward(grad_C, C_indices, C_indptr,
+                    A_rows, A_cols, A_data, A_indices, A_indptr,
+                    B_rows, B_cols, B_data, B_indices, B_indptr):
+    """[grad_A, grad_B]  (cpp/sparse_csr.hpp:50-54)."""
+    dev = _need_device(grad_C, C_indices, C_indptr, A_data, A_indices, A_indptr,
+                       B_data, B_indices, B_indptr)
+    _same_dtype(A_data, B_data, "B_data")
+    _same_dtype(A_data, grad_C, "grad_C")
+    A_data, B_data, grad_C = A_data.contiguous(), B_data.contiguous(), grad_C.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    B_indices, B_indptr = _idx(B_indices, "B_indices"), _idx(B_indptr, "B_indptr")
+    C_indices, C_indptr = _idx(C_indices, "C_indices"), _idx(C_indptr, "C_indptr")
+    with torch.cuda.device(dev):
+        grad_A = torch.empty_like(A_data)
+        grad_B = torch.empty_like(B_data)
+        _lib.check(_lib.lib().nm_spgemm_backward(
+            _dt(A_data), A_rows, A_data.shape[0], B_data.shape[0], _ptr(grad_C), _ptr(C_indices),
+            _ptr(C_indptr), _ptr(A_data), _ptr(A_indices), _ptr(A_indptr), _ptr(B_data),
+            _ptr(B_indices), _ptr(B_indptr), _ptr(grad_A), _ptr(grad_B), _stream(dev)),
+            "nm_spgemm_backward")
+    return [grad_A, grad_B]
+
+
+# ------------------------------------------------------------------- SpTRSV
+
+class _Plan:
+    """Level schedule + transposed structure of one triangular sparsity pattern."""
+
+    def __init__(self, indices, indptr, rows, lower, dev):
+        L = _lib.lib()
+        nnz = indices.shape[0]
+        pbytes, wbytes = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _lib.check(L.nm_sptrsv_plan_bytes(rows, nnz, ctypes.byref(pbytes), ctypes.byref(wbytes)),
+                   "nm_sptrsv_plan_bytes")
+        self.mem = torch.empty(max(pbytes.value, 8), dtype=torch.uint8, device=dev)
+        work = torch.empty(max(wbytes.value, 8), dtype=torch.uint8, device=dev)
+        # the tensors are kept so that their addresses cannot be reused while the plan is cached
+        self.indices, self.indptr = indices, indptr
+        handle = ctypes.c_void_p(0)
+        _lib.check(L.nm_sptrsv_analyse(
+            rows, nnz, _ptr(indices), _ptr(indptr), int(lower), _ptr(self.mem), pbytes.value,
+            _ptr(work), wbytes.value, ctypes.byref(handle), _stream(dev)), "nm_sptrsv_analyse")
+        self.handle = handle
+        self.levels = int(L.nm_sptrsv_plan_levels(handle))
+        self.launches = int(L.nm_sptrsv_plan_launches(handle))
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None):
+                _lib.lib().nm_sptrsv_plan_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+_PLAN_CACHE_SIZE = 16
+_plans = collections.OrderedDict()
+_plans_lock = threading.Lock()
+
+
+def clear_plan_cache():
+    with _plans_lock:
+        _plans.clear()
+
+
+def _plan_for(indices, indptr, rows, lower, dev):
+    """Cached plan of (structure, triangle).  Keyed on the structure tensors' storage and
+    version counters; in-place edits of the structure therefore trigger a new analysis."""
+    key = (dev.index, indices.data_ptr(), indptr.data_ptr(), indices._version, indptr._version,
+           rows, indices.shape[0], bool(lower))
+    with _plans_lock:
+        plan = _plans.get(key)
+        if plan is not None:
+            _plans.move_to_end(key)
+            return plan
+    plan = _Plan(indices, indptr, rows, lower, dev)
+    with _plans_lock:
+        _plans[key] = plan
+        while len(_plans) > _PLAN_CACHE_SIZE:
+            _plans.popitem(last=False)
+    return plan
+
+
+def _solve(plan, transposed, A_data, A_indices, A_indptr, unit, b, rows, dev):
+    x = torch.empty(rows, dtype=A_data.dtype, device=dev)
+    xwork = None if A_data.dtype == torch.float64 else torch.empty(rows, dtype=torch.float64, device=dev)
+    _lib.check(_lib.lib().nm_sptrsv_solve(
+        plan.handle, _dt(A_data), int(transposed), _ptr(A_data), _ptr(A_indices), _ptr(A_indptr),
+        int(unit), _ptr(b), _ptr(x), _ptr(xwork), _stream(dev)), "nm_sptrsv_solve")
+    return x
+
+
+def sptrsv_forward(A_rows, A_cols, A_data, A_indices, A_indptr, lower, unit, b):
+    """x = A^{-1} b for triangular A  (cpp/sparse_csr.hpp:94-98)."""
+    dev = _need_device(A_data, A_indices, A_indptr, b)
+    _same_dtype(A_data, b, "b")
+    A_data, b = A_data.contiguous(), b.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
+        return _solve(plan, False, A_data, A_indices, A_indptr, unit, b, A_rows, dev)
+
+
+def sptrsv_backward(grad_x, x, A_rows, A_cols, A_data, A_indices, A_indptr, lower, unit, b):
+    """[grad_A, grad_b]  (cpp/sparse_csr.hpp:100-105)."""
+    dev = _need_device(grad_x, x, A_data, A_indices, A_indptr)
+    _same_dtype(A_data, grad_x, "grad_x")
+    _same_dtype(A_data, x, "x")
+    A_data, grad_x, x = A_data.contiguous(), grad_x.contiguous(), x.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
+        grad_b = _solve(plan, True, A_data, A_indices, A_indptr, unit, grad_x, A_rows, dev)
+        grad_A = torch.empty_like(A_data)
+        _lib.check(_lib.lib().nm_masked_outer(
+            _dt(A_data), A_rows, A_data.shape[0], _ptr(A_indices), _ptr(A_indptr), -1.0,
+            _ptr(grad_b), _ptr(x), _ptr(grad_A), _stream(dev)), "nm_masked_outer")
+    return [grad_A, grad_b]

@@ -1,0 +1,137 @@
+"""HIP kernels (through the C ABI) against the serial oracle on small seeded inputs.
+
+Covers the shapes the reference's tests use (1-D Poisson N=16/2048,
+numml/tests/test_spmv.py:9-10) plus empty rows, empty matrices, ragged and long
+rows, both dtypes, both triangles, unit and non-unit diagonals.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as ext
+from util import assert_close, assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+
+def _matrices(dtype):
+    yield "tridiag16", G.tridiag(16, dtype)
+    yield "tridiag2048", G.tridiag(2048, dtype)
+    yield "poisson64", G.poisson2d(64, dtype, jitter_seed=3)
+    yield "random_ragged", G.random_csr(700, 300, 0.02, 5, dtype)
+    yield "one_dense_row", G.random_csr(40, 5000, 0.9, 6, dtype, empty_rows=False)
+    yield "powerlaw", G.powerlaw(3000, 3000, target_nnz=60000, max_deg=2500, seed=7, dtype=dtype)
+    yield "empty", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(6, np.int64), (5, 4))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_spmv_forward_backward(dev, dtype):
+    for name, (d, i, p, (rows, cols)) in _matrices(dtype):
+        x, g = randn(1, cols, dtype), randn(2, rows, dtype)
+        y_ref = oracle.spgemv_forward(rows, cols, d, i, p, x)
+        gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+        D, I, P, X, Gd = to_dev(dev, d, i, p, x, g)
+        y = ext.spgemv_forward(rows, cols, D, I, P, X)
+        gA, gx = ext.spgemv_backward(Gd, rows, cols, D, I, P, X)
+        assert_close(host(y), y_ref, f"{name} y")
+        assert_same(host(gA), gA_ref, f"{name} grad_A")
+        assert_close(host(gx), gx_ref, f"{name} grad_x")
+        if name in ("tridiag16", "tridiag2048", "poisson64"):
+            # short rows are summed in storage order: bit-identical to the serial loop
+            assert_same(host(y), y_ref, f"{name} y (bitwise)")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [1, 7, 64, 100])
+def test_spmm_forward_backward(dev, dtype, n):
+    for name, (d, i, p, (rows, cols)) in _matrices(dtype):
+        if name == "one_dense_row" and n > 7:
+            continue
+        B, gC = randn(1, (cols, n), dtype), randn(2, (rows, n), dtype)
+        C_ref = oracle.spdmm_forward(rows, cols, d, i, p, B)
+        gA_ref, gB_ref = oracle.spdmm_backward(rows, cols, d, i, p, B, gC)
+        D, I, P, Bd, gCd = to_dev(dev, d, i, p, B, gC)
+        C = ext.spdmm_forward(rows, cols, D, I, P, Bd)
+        gA, gB = ext.spdmm_backward(rows, cols, D, I, P, Bd, gCd)
+        assert_same(host(C), C_ref, f"{name} C")
+        assert_close(host(gA), gA_ref, f"{name} grad_A")
+        assert_close(host(gB), gB_ref, f"{name} grad_B")
+
+
+def test_spmm_strided_operand(dev):
+    d, i, p, (rows, cols) = G.random_csr(200, 150, 0.05, 11, np.float64)
+    wide = randn(3, (cols, 40), np.float64)
+    D, I, P, W = to_dev(dev, d, i, p, wide)
+    C = ext.spdmm_forward(rows, cols, D, I, P, W[:, 4:20])          # row stride 40, 16 columns
+    Ct = ext.spdmm_forward(rows, cols, D, I, P, W[:, ::2])           # column stride 2 -> copied
+    assert_same(host(C), oracle.spdmm_forward(rows, cols, d, i, p, wide[:, 4:20]), "strided rows")
+    assert_same(host(Ct), oracle.spdmm_forward(rows, cols, d, i, p, wide[:, ::2]), "strided columns")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_spgemm_forward_backward(dev, dtype):
+    cases = [
+        ("tridiag", G.tridiag(2048, dtype), G.tridiag(2048, dtype, 1.0, -2.0, 1.0)),
+        ("poisson", G.poisson2d(48, dtype, 1), G.poisson2d(48, dtype, 2)),
+        ("laplace3d", G.laplace3d(12, dtype, 0), G.laplace3d(12, dtype, 0)),
+        ("rect", G.random_csr(300, 200, 0.03, 1, dtype), G.random_csr(200, 400, 0.04, 2, dtype)),
+        ("dense_rows", G.random_csr(64, 600, 0.3, 3, dtype), G.random_csr(600, 900, 0.2, 4, dtype)),
+        ("powerlaw", G.powerlaw(2000, 2000, 30000, max_deg=1500, seed=5, dtype=dtype),
+         G.powerlaw(2000, 2000, 30000, max_deg=1500, seed=6, dtype=dtype)),
+        ("spill", G.random_csr(6, 300, 0.9, 8, dtype, empty_rows=False),
+         G.random_csr(300, 20000, 0.2, 9, dtype)),
+        ("empty", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(4, np.int64), (3, 5)),
+         G.random_csr(5, 6, 0.5, 1, dtype)),
+    ]
+    for name, (ad, ai, ap, (ar, ac)), (bd, bi, bp, (br, bc)) in cases:
+        Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(ar, ac, ad, ai, ap, br, bc, bd, bi, bp)
+        gC = randn(9, Cd_ref.shape[0], dtype)
+        gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, ar, ac, ad, ai, ap, br, bc, bd, bi, bp)
+        AD, AI, AP, BD, BI, BP, GC = to_dev(dev, ad, ai, ap, bd, bi, bp, gC)
+        Cd, Ci, Cp = ext.spgemm_forward(ar, ac, AD, AI, AP, br, bc, BD, BI, BP)
+        assert_same(host(Cp), Cp_ref, f"{name} C_indptr")
+        assert_same(host(Ci), Ci_ref, f"{name} C_indices")
+        if name in ("spill",):
+            assert_close(host(Cd), Cd_ref, f"{name} C_data")   # spilled rows add with atomics
+        else:
+            assert_same(host(Cd), Cd_ref, f"{name} C_data")
+        gA, gB = ext.spgemm_backward(GC, Ci, Cp, ar, ac, AD, AI, AP, br, bc, BD, BI, BP)
+        assert_same(host(gA), gA_ref, f"{name} grad_A")
+        assert_close(host(gB), gB_ref, f"{name} grad_B")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("lower", [True, False])
+@pytest.mark.parametrize("unit", [False, True])
+def test_sptrsv_forward_backward(dev, dtype, lower, unit):
+    ext.clear_plan_cache()
+    tri = lambda t: t if lower else _transpose(t)
+    cases = [
+        ("bidiag", G.bidiag(700, dtype, lower)),
+        ("random", G.random_tri(400, 0.02, 3, lower, dtype)),
+        ("random_wrong_side", G.random_tri(300, 0.03, 4, lower, dtype, wrong_side=0.01)),
+        ("poisson_tri", tri(G.poisson2d_lower(40, dtype, 0))),
+        ("wide_levels", G.random_tri(5000, 0.0004, 5, lower, dtype)),
+        ("diag_only", G.random_tri(50, 0.0, 6, lower, dtype)),
+    ]
+    for name, case in cases:
+        d, i, p, (n, _) = case
+        b, g = randn(1, n, dtype), randn(2, n, dtype)
+        x_ref = oracle.sptrsv_forward(n, n, d, i, p, lower, unit, b)
+        gA_ref, gb_ref = oracle.sptrsv_backward(g, x_ref, n, n, d, i, p, lower, unit)
+        D, I, P, Bv, Gv = to_dev(dev, d, i, p, b, g)
+        x = ext.sptrsv_forward(n, n, D, I, P, lower, unit, Bv)
+        assert_same(host(x), x_ref, f"{name} x")
+        gA, gb = ext.sptrsv_backward(Gv, x, n, n, D, I, P, lower, unit, Bv)
+        assert_same(host(gb), gb_ref, f"{name} grad_b")
+        assert_same(host(gA), gA_ref, f"{name} grad_A")
+
+
+def _transpose(csr):
+    d, i, p, (r, c) = csr
+    At_d, At_i, At_p, _ = oracle.csr_transpose(r, c, d, i, p)
+    return At_d, At_i, At_p, (c, r)
