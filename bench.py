@@ -1,0 +1,382 @@
+#!/usr/bin/env python3
+"""Benchmark of the differentiable CSR hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the hot path over one synthetic input (forward, then
+backward with both gradients) through the ``numml_torch_cpp`` mirror, i.e. the
+same calls autograd makes.  Inputs are resident in HBM before the timed region.
+Prints ONE JSON line.
+
+Workloads (``--workload``; the default is the one the headline metric is quoted
+on):
+
+  spmv    fp32 SpMV fwd+bwd, 2-D Poisson 2048^2 (4,194,304 rows, 20,963,328 nnz)
+  spmv64  fp64 SpMV fwd+bwd, 2-D Poisson 256^2  (the CPU-sized plumbing case)
+  spmm    fp32 SpMM fwd+bwd, power-law 1M x 1M, ~15M nnz, 64 dense columns
+  spgemm  fp64 hash SpGEMM A@A fwd+bwd, 3-D Laplacian 128^3
+  sptrsv  fp64 triangular solve fwd+bwd, tril(Poisson 1024^2), 2047 levels
+
+``value`` is algorithmic bytes per step / time per step (GB/s) for spmv/spmm,
+GFLOP/s (2 flop per scalar product, forward only counted) for spgemm and
+milliseconds per forward solve for sptrsv.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+
+def _traffic(workload):
+    """Measured HBM bytes per launch of the dominant kernel, from the committed
+    rocprofv3 counter summaries (profiles/traffic.json), or None."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(workload, {}).get("traffic_bytes")
+    except (OSError, ValueError):
+        return None
+
+
+class Workload:
+    name = ""
+    metric = "SpMV/SpMM eff. HBM GB/s (% of peak); SpGEMM GFLOP/s; tri-solve ms"
+    unit = "GB/s"
+    dtype = "f32"
+    higher_is_better = True
+
+    def setup(self, dev):
+        raise NotImplementedError
+
+    def step(self):
+        raise NotImplementedError
+
+    def dominant(self):
+        """Runs the dominant launch once (events are recorded around this call)."""
+        raise NotImplementedError
+
+    def value(self, ms_per_step):
+        return self.bytes_per_step / (ms_per_step * 1e-3) / 1e9
+
+    def cpu_baseline(self, budget_s):
+        raise NotImplementedError
+
+
+def _spmv_bytes(rows, cols, nnz, s):
+    fwd = nnz * (s + 8) + (rows + 1) * 8 + cols * s + rows * s
+    bwd = nnz * (s + 8) + (rows + 1) * 8 + rows * s + cols * s + nnz * s + cols * s
+    return fwd, bwd
+
+
+class SpMV(Workload):
+    def __init__(self, n=2048, dtype=np.float32, jitter=0, label="poisson2d_2048"):
+        self.n, self.np_dtype, self.jitter = n, dtype, jitter
+        self.name = "spmv" if dtype == np.float32 else "spmv64"
+        self.dtype = "f32" if dtype == np.float32 else "f64"
+        self.label = label
+
+    def setup(self, dev):
+        import torch
+        from numml_amd import generators as G
+        from numml_amd import numml_torch_cpp as ext
+        self.ext = ext
+        d, i, p, (rows, cols) = G.poisson2d(self.n, self.np_dtype, jitter_seed=self.jitter)
+        self.host = (d, i, p, rows, cols)
+        self.x_h = np.random.default_rng(1).standard_normal(cols).astype(self.np_dtype)
+        self.g_h = np.random.default_rng(2).standard_normal(rows).astype(self.np_dtype)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        self.D, self.I, self.P, self.X, self.Gv = t(d), t(i), t(p), t(self.x_h), t(self.g_h)
+        self.rows, self.cols, self.nnz = rows, cols, d.shape[0]
+        s = d.dtype.itemsize
+        self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s)
+        self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
+        self.dominant_bytes = self.bwd_bytes
+        self.dominant_name = "spmv_bwd_kernel (+ fill_kernel clearing grad_x)"
+        self.config = {"workload": f"spmv_fwd_bwd_{self.dtype}_{self.label}", "rows": rows,
+                       "nnz": self.nnz, "index_bytes": 8,
+                       "algorithmic_bytes_per_step": self.bytes_per_step}
+
+    def step(self):
+        y = self.ext.spgemv_forward(self.rows, self.cols, self.D, self.I, self.P, self.X)
+        gA, gx = self.ext.spgemv_backward(self.Gv, self.rows, self.cols, self.D, self.I, self.P, self.X)
+        return y, gA, gx
+
+    def dominant(self):
+        return self.ext.spgemv_backward(self.Gv, self.rows, self.cols, self.D, self.I, self.P, self.X)
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        d, i, p, rows, cols = self.host
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            oracle.spgemv_forward(rows, cols, d, i, p, self.x_h)
+            oracle.spgemv_backward(self.g_h, rows, cols, d, i, p, self.x_h)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget_s or reps >= 200:
+                break
+        return {"value": self.bytes_per_step * reps / el / 1e9, "unit": "GB/s", "cores": 1,
+                "kind": "port",
+                "sample": f"{reps} x (spgemv_forward + spgemv_backward) of the full workload, serial C oracle"}
+
+
+class SpMM(Workload):
+    name = "spmm"
+
+    def setup(self, dev):
+        import torch
+        from numml_amd import generators as G
+        from numml_amd import numml_torch_cpp as ext
+        self.ext = ext
+        rows = cols = 1_000_000
+        n = 64
+        d, i, p, _ = G.powerlaw(rows, cols, target_nnz=16_000_000, seed=0, dtype=np.float32)
+        self.host = (d, i, p, rows, cols)
+        self.B_h = np.random.default_rng(1).standard_normal((cols, n)).astype(np.float32)
+        self.g_h = np.random.default_rng(2).standard_normal((rows, n)).astype(np.float32)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        self.D, self.I, self.P, self.B, self.Gv = t(d), t(i), t(p), t(self.B_h), t(self.g_h)
+        self.rows, self.cols, self.nnz, self.n = rows, cols, d.shape[0], n
+        s, nnz = 4, self.nnz
+        self.fwd_bytes = nnz * (s + 8) + (rows + 1) * 8 + cols * n * s + rows * n * s
+        self.bwd_bytes = (nnz * (s + 8) + (rows + 1) * 8 + rows * n * s + cols * n * s + nnz * s
+                          + cols * n * s)
+        self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
+        self.dominant_bytes = self.bwd_bytes
+        self.dominant_name = "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)"
+        self.config = {"workload": "spmm_fwd_bwd_f32_powerlaw_1M_n64", "rows": rows, "nnz": nnz,
+                       "dense_cols": n, "index_bytes": 8,
+                       "algorithmic_bytes_per_step": self.bytes_per_step,
+                       "gather_bytes_fwd": nnz * n * s}
+
+    def step(self):
+        C = self.ext.spdmm_forward(self.rows, self.cols, self.D, self.I, self.P, self.B)
+        gA, gB = self.ext.spdmm_backward(self.rows, self.cols, self.D, self.I, self.P, self.B, self.Gv)
+        return C, gA, gB
+
+    def dominant(self):
+        return self.ext.spdmm_backward(self.rows, self.cols, self.D, self.I, self.P, self.B, self.Gv)
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        d, i, p, rows, cols = self.host
+        # the reference's row->column->entry loop is slow: time the first `sub` rows only
+        sub = 50_000
+        ps = p[:sub + 1]
+        nnz_s = int(ps[-1])
+        ds, is_ = d[:nnz_s], i[:nnz_s]
+        t0 = time.perf_counter()
+        oracle.spdmm_forward(sub, cols, ds, is_, ps, self.B_h)
+        oracle.spdmm_backward(sub, cols, ds, is_, ps, self.B_h, self.g_h[:sub])
+        el = time.perf_counter() - t0
+        frac = nnz_s / self.nnz
+        return {"value": self.bytes_per_step * frac / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"first {sub} rows ({nnz_s} nnz, {frac:.3%} of the entries), 1 x (forward + backward), "
+                          "scaled by entry count, serial C oracle"}
+
+
+class SpGEMM(Workload):
+    name = "spgemm"
+    unit = "GFLOP/s"
+    dtype = "f64"
+
+    def setup(self, dev):
+        import torch
+        from numml_amd import generators as G
+        from numml_amd import numml_torch_cpp as ext
+        self.ext = ext
+        n = int(os.environ.get("NM_BENCH_SPGEMM_N", "128"))
+        d, i, p, (rows, cols) = G.laplace3d(n, np.float64, jitter_seed=0)
+        self.host = (d, i, p, rows, cols)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        self.D, self.I, self.P = t(d), t(i), t(p)
+        self.rows, self.cols, self.nnz = rows, cols, d.shape[0]
+        C = ext.spgemm_forward(rows, cols, self.D, self.I, self.P, rows, cols, self.D, self.I, self.P)
+        self.nnzC = C[0].shape[0]
+        self.gC = torch.from_numpy(np.random.default_rng(1).standard_normal(self.nnzC)).to(dev)
+        self.C = C
+        lens = np.diff(p)
+        self.products = int(lens[i].sum())
+        self.flops = 2 * self.products
+        s = 8
+        self.bytes_per_step = (self.nnz * (s + 8) + rows * 8 + self.products * (s + 8)
+                               + self.nnzC * (s + 8) + rows * 8)
+        self.dominant_bytes = self.bytes_per_step
+        self.dominant_name = "spgemm forward (symbolic + numeric launches)"
+        self.config = {"workload": f"spgemm_AxA_fwd_bwd_f64_laplace3d_{n}", "rows": rows, "nnz": self.nnz,
+                       "nnz_C": self.nnzC, "products": self.products, "index_bytes": 8}
+
+    def step(self):
+        C = self.ext.spgemm_forward(self.rows, self.cols, self.D, self.I, self.P,
+                                    self.rows, self.cols, self.D, self.I, self.P)
+        g = self.ext.spgemm_backward(self.gC, C[1], C[2], self.rows, self.cols, self.D, self.I, self.P,
+                                     self.rows, self.cols, self.D, self.I, self.P)
+        return C, g
+
+    def dominant(self):
+        return self.ext.spgemm_forward(self.rows, self.cols, self.D, self.I, self.P,
+                                       self.rows, self.cols, self.D, self.I, self.P)
+
+    def value(self, ms_per_step):
+        return self.flops / (ms_per_step * 1e-3) / 1e9
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        d, i, p, rows, cols = self.host
+        t0 = time.perf_counter()
+        C = oracle.spgemm_forward(rows, cols, d, i, p, rows, cols, d, i, p)
+        gC = np.random.default_rng(1).standard_normal(C[0].shape[0])
+        oracle.spgemm_backward(gC, C[1], C[2], rows, cols, d, i, p, rows, cols, d, i, p)
+        el = time.perf_counter() - t0
+        return {"value": self.flops / el / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+                "sample": "1 x (spgemm_forward + spgemm_backward) of the full workload, serial C oracle "
+                          "(bisection instead of the reference's std::map lookup)"}
+
+
+class SpTRSV(Workload):
+    name = "sptrsv"
+    unit = "ms"
+    dtype = "f64"
+    higher_is_better = False
+
+    def setup(self, dev):
+        import torch
+        from numml_amd import generators as G
+        from numml_amd import numml_torch_cpp as ext
+        self.ext = ext
+        n = 1024
+        d, i, p, (rows, cols) = G.poisson2d_lower(n, np.float64, diag_seed=0)
+        self.host = (d, i, p, rows, cols)
+        self.b_h = np.random.default_rng(1).standard_normal(rows)
+        self.g_h = np.random.default_rng(2).standard_normal(rows)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        self.D, self.I, self.P, self.Bv, self.Gv = t(d), t(i), t(p), t(self.b_h), t(self.g_h)
+        self.rows, self.nnz = rows, d.shape[0]
+        t0 = time.perf_counter()
+        self.x = ext.sptrsv_forward(rows, rows, self.D, self.I, self.P, True, False, self.Bv)
+        torch.cuda.synchronize()
+        self.analysis_ms = (time.perf_counter() - t0) * 1e3
+        s = 8
+        self.bytes_per_step = 2 * (self.nnz * (s + 8) + (rows + 1) * 8 + 2 * rows * s) + self.nnz * s
+        self.dominant_bytes = self.nnz * (s + 8) + (rows + 1) * 8 + 2 * rows * s
+        self.dominant_name = "sptrsv_batch_kernel (forward solve)"
+        self.config = {"workload": "sptrsv_fwd_bwd_f64_tril_poisson2d_1024", "rows": rows, "nnz": self.nnz,
+                       "levels": 2 * n - 1, "analysis_plus_first_solve_ms": round(self.analysis_ms, 3)}
+
+    def step(self):
+        x = self.ext.sptrsv_forward(self.rows, self.rows, self.D, self.I, self.P, True, False, self.Bv)
+        g = self.ext.sptrsv_backward(self.Gv, x, self.rows, self.rows, self.D, self.I, self.P, True, False,
+                                     self.Bv)
+        return x, g
+
+    def dominant(self):
+        return self.ext.sptrsv_forward(self.rows, self.rows, self.D, self.I, self.P, True, False, self.Bv)
+
+    def value(self, ms_per_step):
+        return ms_per_step
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        d, i, p, rows, cols = self.host
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            x = oracle.sptrsv_forward(rows, rows, d, i, p, True, False, self.b_h)
+            oracle.sptrsv_backward(self.g_h, x, rows, rows, d, i, p, True, False)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget_s or reps >= 100:
+                break
+        return {"value": el / reps * 1e3, "unit": "ms", "cores": 1, "kind": "port",
+                "sample": f"{reps} x (sptrsv_forward + sptrsv_backward) of the full workload, serial C oracle"}
+
+
+WORKLOADS = {
+    "spmv": lambda: SpMV(2048, np.float32, 0, "poisson2d_2048"),
+    "spmv64": lambda: SpMV(256, np.float64, None, "poisson2d_256"),
+    "spmm": SpMM,
+    "spgemm": SpGEMM,
+    "sptrsv": SpTRSV,
+}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="spmv", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=10.0,
+                    help="CPU time budget of the cpu_baseline leg (0 skips it)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
+                 f"--gpus {args.gpus} is not supported, use --gpus 1")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    w = WORKLOADS[args.workload]()
+    w.setup(dev)
+
+    for _ in range(max(args.warmup, 0)):
+        w.step()
+    torch.cuda.synchronize()
+
+    # K timed steps; the dominant launch of every step is bracketed by events on the
+    # stream it runs on (torch's current stream is the one handed to the C ABI).
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        w.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # Kernel-level timing for the roofline: same launches, events around each one.
+    evs = []
+    for _ in range(args.steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        w.dominant()
+        e1.record()
+        evs.append((e0, e1))
+    torch.cuda.synchronize()
+    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+    achieved = w.dominant_bytes / (kernel_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": w.dominant_name, "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "algorithmic_bytes": int(w.dominant_bytes), "avg_ms": round(kernel_ms, 5),
+                "traffic": _traffic(w.name)}
+
+    cpu = None
+    if args.cpu_seconds > 0:
+        cpu = w.cpu_baseline(args.cpu_seconds)
+        cpu["value"] = round(cpu["value"], 4)
+        cpu["host_cores_visible"] = os.cpu_count()
+
+    value = w.value(ms_per_step)
+    out = {
+        "metric": w.metric, "value": round(value, 3), "unit": w.unit, "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": w.higher_is_better, "scaling": "weak", "vs_baseline": None,
+        "dtype": w.dtype, "data": "synthetic", "config": w.config,
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+    if w.unit == "GB/s":
+        out["pct_of_hbm_peak"] = round(100.0 * value / HBM_PEAK_GBS, 2)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
