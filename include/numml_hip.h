@@ -62,6 +62,32 @@ int nm_spgemv_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
                        const void *x, const void *g,
                        void *grad_A, void *grad_x, nm_stream stream);
 
+/* ---------------------------------------------- transposed-structure plan
+ * The pattern of A^T as 32-bit arrays (column pointers, row of each entry and
+ * its position in A's arrays, rows ascending inside a column), built once per
+ * sparsity pattern in caller-provided device memory and reused by the
+ * *_planned backward entry points below.  It is the structure (not the values)
+ * of what csr_transpose_forward returns (cpp/sparse_csr_cpu.cpp:311-367:
+ * At_indptr, At_indices, At_to_A_idx).  The build is enqueued on `stream` and
+ * does not synchronise; `work` may be released once it has run.  Sizes up to
+ * 2^31 - 2 rows, columns and entries (NM_ERR_UNSUPPORTED beyond). */
+int nm_csr_transpose_plan_bytes(int64_t rows, int64_t cols, int64_t nnz,
+                                size_t *plan_bytes, size_t *work_bytes);
+
+int nm_csr_transpose_plan_build(int64_t rows, int64_t cols, int64_t nnz,
+                                const int64_t *indices, const int64_t *indptr,
+                                void *plan_mem, size_t plan_bytes,
+                                void *work, size_t work_bytes, nm_stream stream);
+
+/* nm_spgemv_backward on a transposed-structure plan: walks A by column, so
+ * grad_x needs neither clearing nor atomics, is summed in ascending row order
+ * (the order of cpp/sparse_csr_cpu.cpp:68-73) and is identical on every run.
+ * Either output may be NULL. */
+int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                               const void *data, const void *plan_mem,
+                               const void *x, const void *g,
+                               void *grad_A, void *grad_x, nm_stream stream);
+
 /* ------------------------------------------------------------------ SpMM
  * C = A B with dense row-major B (cols x n, row stride ldb elements) and
  * C (rows x n, row stride ldc).  Stands in for spdmm_forward
@@ -79,6 +105,15 @@ int nm_spdmm_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
                       const void *data, const int64_t *indices, const int64_t *indptr,
                       const void *B, int64_t ldb, const void *gC, int64_t ldg, int64_t n,
                       void *grad_A, void *grad_B, int64_t ldgb, nm_stream stream);
+
+/* nm_spdmm_backward on a transposed-structure plan: grad_B = A^T gC is computed
+ * as a product over A's columns (no clearing, no atomics, sums in ascending
+ * row order like cpp/sparse_csr_cpu.cpp:639-646).  Either output may be NULL. */
+int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                              const void *data, const int64_t *indices, const int64_t *indptr,
+                              const void *plan_mem,
+                              const void *B, int64_t ldb, const void *gC, int64_t ldg, int64_t n,
+                              void *grad_A, void *grad_B, int64_t ldgb, nm_stream stream);
 
 /* ---------------------------------------------------------------- SpGEMM
  * C = A B, both CSR.  Stands in for spgemm_forward (cpp/sparse_csr.hpp:45-48,

@@ -15,6 +15,7 @@
 //   forward : nnz*(s+8) + (rows+1)*8 + cols*n*s + rows*n*s
 //   backward: nnz*(s+8) + (rows+1)*8 + rows*n*s + cols*n*s + nnz*s + cols*n*s
 #include "nm_common.hpp"
+#include "nm_transpose.hpp"
 
 namespace {
 
@@ -22,11 +23,14 @@ using nm::kWave;
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 
-template <typename T>
+// IDX is the structure's index type (int64 for A as delivered, int32 for the
+// transposed-structure plan); with PERM the value of entry k is data[perm[k]]
+// (A^T shares A's value array through the plan's permutation).
+template <typename T, typename IDX, bool PERM>
 __global__ __launch_bounds__(kBlock) void spdmm_fwd_kernel(
-    int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
-    const int64_t *__restrict__ indptr, const T *__restrict__ B, int64_t ldb, int64_t n,
-    T *__restrict__ C, int64_t ldc) {
+    int64_t rows, const T *__restrict__ data, const IDX *__restrict__ indices,
+    const IDX *__restrict__ indptr, const int32_t *__restrict__ perm, const T *__restrict__ B, int64_t ldb,
+    int64_t n, T *__restrict__ C, int64_t ldc) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
     const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
@@ -39,10 +43,9 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_kernel(
             T acc = 0;
             for (int64_t kb = rb; kb < re; kb += kWave) {
                 const int64_t k = kb + lane;
-                const int64_t mycol = k < re ? indices[k] : 0;
-                const T myval = k < re ? data[k] : T(0);
+                const int64_t mycol = k < re ? (int64_t)indices[k] : 0;
+                const T myval = k < re ? (PERM ? data[perm[k]] : data[k]) : T(0);
                 const int cnt = (int)(re - kb < kWave ? re - kb : kWave);
-#pragma unroll 8
                 for (int j = 0; j < cnt; ++j) {
                     const int64_t col = __shfl(mycol, j, kWave);
                     const T v = __shfl(myval, j, kWave);
@@ -128,11 +131,13 @@ extern "C" int nm_spdmm_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t
                (long long)ldb, (long long)ldc, (long long)n);
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
-        hipLaunchKernelGGL(spdmm_fwd_kernel<float>, dim3(wave_grid(rows)), dim3(kBlock), 0, s, rows,
-                           (const float *)data, indices, indptr, (const float *)B, ldb, n, (float *)C, ldc);
+        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int64_t, false>), dim3(wave_grid(rows)), dim3(kBlock), 0, s,
+                           rows, (const float *)data, indices, indptr, nullptr, (const float *)B, ldb, n,
+                           (float *)C, ldc);
     else
-        hipLaunchKernelGGL(spdmm_fwd_kernel<double>, dim3(wave_grid(rows)), dim3(kBlock), 0, s, rows,
-                           (const double *)data, indices, indptr, (const double *)B, ldb, n, (double *)C, ldc);
+        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int64_t, false>), dim3(wave_grid(rows)), dim3(kBlock), 0, s,
+                           rows, (const double *)data, indices, indptr, nullptr, (const double *)B, ldb, n,
+                           (double *)C, ldc);
     NM_LAUNCH_CHECK("spdmm_fwd_kernel");
     return NM_OK;
 }
@@ -171,5 +176,38 @@ extern "C" int nm_spdmm_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_
                            (const double *)data, indices, indptr, (const double *)B, ldb, (const double *)gC,
                            ldg, n, (double *)grad_A, (double *)grad_B, ldgb);
     NM_LAUNCH_CHECK("spdmm_bwd_kernel");
+    return NM_OK;
+}
+
+// Backward over the transposed-structure plan: grad_A by the row-major kernel
+// (dot products only), grad_B = A^T gC as a forward product on the plan, whose
+// per-entry sums run in ascending row order like the serial CPU loop
+// (cpp/sparse_csr_cpu.cpp:639-646): no atomics, no clearing, bit-reproducible.
+extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                         const int64_t *indices, const int64_t *indptr, const void *plan_mem,
+                                         const void *B, int64_t ldb, const void *gC, int64_t ldg, int64_t n,
+                                         void *grad_A, void *grad_B, int64_t ldgb, nm_stream stream) {
+    if (int rc = check_args(dt, rows, cols, nnz, data, indices, indptr, n)) return rc;
+    NM_REQUIRE(plan_mem != nullptr, "plan is null");
+    if (grad_A) {
+        if (int rc = nm_spdmm_backward(dt, rows, cols, nnz, data, indices, indptr, B, ldb, gC, ldg, n, grad_A,
+                                       nullptr, 0, stream))
+            return rc;
+    }
+    if (!grad_B || cols == 0 || n == 0) return NM_OK;
+    NM_REQUIRE(ldgb >= n && ldg >= n, "row stride smaller than the row");
+    NM_REQUIRE(gC != nullptr || nnz == 0, "gC is null");
+    nm::TPlan t;
+    nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F32)
+        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int32_t, true>), dim3(wave_grid(cols)), dim3(kBlock), 0, s, cols,
+                           (const float *)data, t.t_row, t.t_indptr, t.t_perm, (const float *)gC, ldg, n,
+                           (float *)grad_B, ldgb);
+    else
+        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int32_t, true>), dim3(wave_grid(cols)), dim3(kBlock), 0, s,
+                           cols, (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg, n,
+                           (double *)grad_B, ldgb);
+    NM_LAUNCH_CHECK("spdmm_fwd_kernel (transposed)");
     return NM_OK;
 }

@@ -14,6 +14,7 @@
 //   forward : nnz*(s+8) + (rows+1)*8 + cols*s + rows*s
 //   backward: nnz*(s+8) + (rows+1)*8 + rows*s + cols*s + nnz*s + cols*s
 #include "nm_common.hpp"
+#include "nm_transpose.hpp"
 
 namespace {
 
@@ -158,6 +159,97 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
     }
 }
 
+// Backward over the transposed-structure plan (columns of A as rows of A^T):
+// no atomics and no clearing of grad_x.  A workgroup owns R consecutive
+// columns; lane p of the entry-parallel phase reads (row, position) of the
+// p-th entry in column-major order, writes grad_A[position] = g[row] * x[col]
+// and leaves g[row] * data[position] in LDS; one lane per column then adds its
+// slice in ascending row order, the order in which the serial CPU loop
+// accumulates grad_x (cpp/sparse_csr_cpu.cpp:68-73), so grad_x matches it bit
+// for bit and is the same on every run.
+template <typename T, int R, int CAP>
+__global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
+    int64_t cols, const T *__restrict__ data, const int32_t *__restrict__ t_indptr,
+    const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm, const T *__restrict__ x,
+    const T *__restrict__ g, T *__restrict__ grad_A, T *__restrict__ grad_x) {
+    __shared__ int32_t s_off[R + 1];
+    __shared__ T s_v[CAP];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int64_t nblk = (cols + R - 1) / R;
+    // column blocks are taken from the far end first: the forward pass that precedes a
+    // backward leaves the tail of A's value array in the last-level cache
+    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
+        const int64_t c0 = (nblk - 1 - blk) * R;
+        const int nc = (int)(cols - c0 < R ? cols - c0 : R);
+        const int32_t base = t_indptr[c0];
+        for (int t = threadIdx.x; t <= nc; t += kBlock) {
+            const int32_t d = t_indptr[c0 + t] - base;
+            s_off[t] = d > CAP ? CAP + 1 : d;
+        }
+        __syncthreads();
+        const int n = s_off[nc];
+        if (n <= CAP) {
+            if (grad_A) {
+                for (int t = threadIdx.x; t < nc; t += kBlock) {
+                    const T xv = x[c0 + t];
+                    const int e = s_off[t + 1];
+                    for (int j = s_off[t]; j < e; ++j) s_v[j] = xv;
+                }
+                __syncthreads();
+            }
+            const int32_t *__restrict__ tr = t_row + base;
+            const int32_t *__restrict__ tp = t_perm + base;
+            for (int p = threadIdx.x; p < n; p += kBlock) {
+                const int32_t k = tp[p];
+                const T gr = g[tr[p]];
+                if (grad_A) grad_A[k] = gr * s_v[p];
+                if (grad_x) s_v[p] = gr * data[k];
+            }
+            if (grad_x) {
+                __syncthreads();
+                for (int t = threadIdx.x; t < nc; t += kBlock) {
+                    const int e = s_off[t + 1];
+                    T acc = 0;
+                    for (int j = s_off[t]; j < e; ++j) acc += s_v[j];
+                    grad_x[c0 + t] = acc;
+                }
+            }
+        } else {
+            for (int t = threadIdx.x; t < nc; t += kBlock) {
+                const int32_t pb = t_indptr[c0 + t], pe = t_indptr[c0 + t + 1];
+                if (pe - pb >= kLongRow) continue;
+                const T xv = x[c0 + t];
+                T acc = 0;
+                for (int32_t p = pb; p < pe; ++p) {
+                    const int32_t k = t_perm[p];
+                    const T gr = g[t_row[p]];
+                    if (grad_A) grad_A[k] = gr * xv;
+                    if (grad_x) acc += gr * data[k];
+                }
+                if (grad_x) grad_x[c0 + t] = acc;
+            }
+            for (int t = wave; t < nc; t += kWavesPerBlock) {
+                const int32_t pb = t_indptr[c0 + t], pe = t_indptr[c0 + t + 1];
+                if (pe - pb < kLongRow) continue;
+                const T xv = x[c0 + t];
+                T acc = 0;
+                for (int32_t p = pb + lane; p < pe; p += kWave) {
+                    const int32_t k = t_perm[p];
+                    const T gr = g[t_row[p]];
+                    if (grad_A) grad_A[k] = gr * xv;
+                    if (grad_x) acc += gr * data[k];
+                }
+                if (grad_x) {
+                    acc = nm::wave_sum(acc);
+                    if (lane == 0) grad_x[c0 + t] = acc;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
 int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const int64_t *indices,
               const int64_t *indptr) {
     NM_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0, "negative size (rows=%lld cols=%lld nnz=%lld)",
@@ -244,4 +336,33 @@ extern "C" int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz, const int
                                  (float)alpha, (float *)out, nullptr, s);
     return launch_bwd<double>(rows, nullptr, indices, indptr, (const double *)a, (const double *)b, alpha,
                               (double *)out, nullptr, s);
+}
+
+extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                          const void *plan_mem, const void *x, const void *g, void *grad_A,
+                                          void *grad_x, nm_stream stream) {
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0 && plan_mem != nullptr, "bad sizes or null plan");
+    if (cols == 0 || (!grad_A && !grad_x)) return NM_OK;
+    NM_REQUIRE(nnz == 0 || (data && x && g), "null pointer argument");
+    nm::TPlan t;
+    nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F32) {
+        constexpr int R = Tile<float>::R, CAP = Tile<float>::CAP;
+        int64_t grid = nm::ceil_div(cols, R);
+        if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+        hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
+                           (const float *)data, t.t_indptr, t.t_row, t.t_perm, (const float *)x, (const float *)g,
+                           (float *)grad_A, (float *)grad_x);
+    } else {
+        constexpr int R = Tile<double>::R, CAP = Tile<double>::CAP;
+        int64_t grid = nm::ceil_div(cols, R);
+        if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+        hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
+                           (const double *)data, t.t_indptr, t.t_row, t.t_perm, (const double *)x,
+                           (const double *)g, (double *)grad_A, (double *)grad_x);
+    }
+    NM_LAUNCH_CHECK("spmv_bwd_planned_kernel");
+    return NM_OK;
 }

@@ -20,8 +20,7 @@
 // Algorithmic HBM bytes of one solve (s = sizeof(value)):
 //   nnz*(s+8) + (rows+1)*8 + 2*rows*s   (+ rows*4 for the level order)
 #include "nm_common.hpp"
-
-#include <rocprim/device/device_radix_sort.hpp>
+#include "nm_transpose.hpp"
 
 #include <new>
 #include <vector>
@@ -32,7 +31,7 @@ struct nm_sptrsv_plan {
     int32_t nlevels = 0;
     // device arrays inside the caller's plan memory
     int32_t *order = nullptr, *level_ptr = nullptr;
-    int32_t *t_indptr = nullptr, *t_indices = nullptr, *t_perm = nullptr;
+    int32_t *t_indptr = nullptr, *t_row = nullptr, *t_perm = nullptr;
     struct Launch {
         int32_t l0, l1;  // levels [l0, l1)
         int32_t q0, q1;  // slots of `order` they cover
@@ -59,64 +58,38 @@ struct Carver {
     }
 };
 
-size_t plan_persistent_bytes(int64_t rows, int64_t nnz) {
-    return align_up((rows + 1) * 4) * 3 + align_up((nnz + 1) * 4) * 2 + align_up(16 * 4);
+// plan memory: [transposed-structure plan][order][level_ptr][meta]
+size_t plan_layout(int64_t rows, int64_t nnz, void *base, nm::TPlan *t, int32_t **order, int32_t **level_ptr,
+                   int32_t **meta) {
+    size_t off = nm::tplan_layout(rows, nnz, base, t);
+    auto take = [&](size_t bytes) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += align_up(bytes);
+        return (int32_t *)q;
+    };
+    int32_t *o = take((size_t)(rows + 1) * 4), *l = take((size_t)(rows + 1) * 4), *m = take(16 * 4);
+    if (order) *order = o;
+    if (level_ptr) *level_ptr = l;
+    if (meta) *meta = m;
+    return off;
 }
 
-size_t sort_temp_bytes(int64_t nnz, int bits) {
-    size_t bytes = 0;
-    rocprim::radix_sort_pairs(nullptr, bytes, (int32_t *)nullptr, (int32_t *)nullptr, (int32_t *)nullptr,
-                              (int32_t *)nullptr, (size_t)(nnz > 0 ? nnz : 1), 0u, (unsigned)bits,
-                              (hipStream_t)0);
-    return bytes;
-}
-
-inline int bits_for(int64_t n) {
-    int b = 1;
-    while (b < 32 && (int64_t(1) << b) < n) ++b;
-    return b;
+// analysis scratch: [deg][rowid][transpose scratch]
+size_t work_bytes_needed(int64_t rows, int64_t nnz) {
+    return align_up((size_t)(rows + 1) * 4) + align_up((size_t)(nnz + 1) * 4) +
+           nm::tplan_work_bytes(rows, rows, nnz);
 }
 
 // ---- analysis kernels ------------------------------------------------------
 
-// Per stored entry: its row (bisection of indptr), sort key (column) and the
-// in-degree of its row in the dependency DAG.
-__global__ void entry_prep_kernel(int64_t nnz, int64_t rows, const int64_t *__restrict__ indices,
-                                  const int64_t *__restrict__ indptr, int lower, int32_t *__restrict__ keys,
-                                  int32_t *__restrict__ vals, int32_t *__restrict__ rowid,
-                                  int32_t *__restrict__ deg) {
+// In-degree of every row in the dependency DAG: its strictly-triangular entries.
+__global__ void indegree_kernel(int64_t nnz, const int64_t *__restrict__ indices,
+                                const int32_t *__restrict__ rowid, int lower, int32_t *__restrict__ deg) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz; k += stride) {
-        int64_t lo = 0, hi = rows + 1;  // first p with indptr[p] > k
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (indptr[mid] <= k) lo = mid + 1; else hi = mid;
-        }
-        const int64_t row = lo - 1;
         const int64_t col = indices[k];
-        keys[k] = (int32_t)col;
-        vals[k] = (int32_t)k;
-        rowid[k] = (int32_t)row;
+        const int32_t row = rowid[k];
         if (lower ? col < row : col > row) atomicAdd(deg + row, 1);
-    }
-}
-
-// Rows of A^T: t_indices[p] = row of the entry sorted to p; t_indptr[c] = first
-// sorted position whose column is >= c.
-__global__ void transpose_finish_kernel(int64_t nnz, int64_t rows, const int32_t *__restrict__ keys_sorted,
-                                        const int32_t *__restrict__ t_perm,
-                                        const int32_t *__restrict__ rowid, int32_t *__restrict__ t_indices,
-                                        int32_t *__restrict__ t_indptr) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for (int64_t p = tid; p < nnz; p += stride) t_indices[p] = rowid[t_perm[p]];
-    for (int64_t c = tid; c <= rows; c += stride) {
-        int64_t lo = 0, hi = nnz;
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (keys_sorted[mid] < c) lo = mid + 1; else hi = mid;
-        }
-        t_indptr[c] = (int32_t)lo;
     }
 }
 
@@ -125,7 +98,7 @@ __global__ void transpose_finish_kernel(int64_t nnz, int64_t rows, const int32_t
 // count as dependencies and those cannot form a cycle).
 __global__ __launch_bounds__(kNarrow) void kahn_kernel(int32_t rows, int lower,
                                                        const int32_t *__restrict__ t_indptr,
-                                                       const int32_t *__restrict__ t_indices, int32_t *deg,
+                                                       const int32_t *__restrict__ t_row, int32_t *deg,
                                                        int32_t *order, int32_t *level_ptr, int32_t *meta) {
     __shared__ int s_tail;
     if (threadIdx.x == 0) s_tail = 0;
@@ -141,7 +114,7 @@ __global__ __launch_bounds__(kNarrow) void kahn_kernel(int32_t rows, int lower,
             const int32_t r = order[q];
             const int32_t pe = t_indptr[r + 1];
             for (int32_t p = t_indptr[r]; p < pe; ++p) {
-                const int32_t d = t_indices[p];
+                const int32_t d = t_row[p];
                 if (lower ? d > r : d < r)
                     if (atomicSub(deg + d, 1) == 1) order[atomicAdd(&s_tail, 1)] = d;
             }
@@ -163,7 +136,7 @@ __global__ __launch_bounds__(kNarrow) void kahn_kernel(int32_t rows, int lower,
 template <typename T> struct SolveArgs {
     const T *data;
     const int64_t *indices, *indptr;                  // A
-    const int32_t *t_indptr, *t_indices, *t_perm;     // A^T
+    const int32_t *t_indptr, *t_row, *t_perm;         // A^T
     const int32_t *order, *level_ptr;
     const T *b;
     double *xw;
@@ -179,14 +152,14 @@ __device__ __forceinline__ void solve_row(const SolveArgs<T> &a, int32_t i) {
     else    { kb = a.indptr[i];   ke = a.indptr[i + 1]; }
     if (a.ascending) {
         for (int64_t k = kb; k < ke; ++k) {
-            const int64_t j = TR ? (int64_t)a.t_indices[k] : a.indices[k];
+            const int64_t j = TR ? (int64_t)a.t_row[k] : a.indices[k];
             if (j > i) continue;
             const double v = (double)(TR ? a.data[a.t_perm[k]] : a.data[k]);
             if (j == i) diag = v; else acc += v * a.xw[j];
         }
     } else {
         for (int64_t k = ke - 1; k >= kb; --k) {
-            const int64_t j = TR ? (int64_t)a.t_indices[k] : a.indices[k];
+            const int64_t j = TR ? (int64_t)a.t_row[k] : a.indices[k];
             if (j < i) continue;
             const double v = (double)(TR ? a.data[a.t_perm[k]] : a.data[k]);
             if (j == i) diag = v; else acc += v * a.xw[j];
@@ -245,7 +218,7 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, const
     a.indices = indices;
     a.indptr = indptr;
     a.t_indptr = p->t_indptr;
-    a.t_indices = p->t_indices;
+    a.t_row = p->t_row;
     a.t_perm = p->t_perm;
     a.order = p->order;
     a.level_ptr = p->level_ptr;
@@ -262,9 +235,8 @@ extern "C" int nm_sptrsv_plan_bytes(int64_t rows, int64_t nnz, size_t *plan_byte
     NM_REQUIRE(rows >= 0 && nnz >= 0 && plan_bytes && work_bytes, "bad arguments");
     if (rows >= (int64_t(1) << 31) - 2 || nnz >= (int64_t(1) << 31) - 2)
         return nm::fail(NM_ERR_UNSUPPORTED, "sptrsv plans index rows and entries with 32 bits");
-    *plan_bytes = plan_persistent_bytes(rows, nnz);
-    *work_bytes = align_up((rows + 1) * 4) + 4 * align_up((nnz + 1) * 4) +
-                  align_up(sort_temp_bytes(nnz, bits_for(rows))) + 256;
+    *plan_bytes = plan_layout(rows, nnz, nullptr, nullptr, nullptr, nullptr, nullptr);
+    *work_bytes = work_bytes_needed(rows, nnz);
     return NM_OK;
 }
 
@@ -287,49 +259,33 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     p->rows = rows;
     p->nnz = nnz;
     p->lower = lower ? 1 : 0;
-    Carver pm(plan_mem);
-    p->order = pm.take<int32_t>(rows + 1);
-    p->level_ptr = pm.take<int32_t>(rows + 1);
-    p->t_indptr = pm.take<int32_t>(rows + 1);
-    p->t_indices = pm.take<int32_t>(nnz + 1);
-    p->t_perm = pm.take<int32_t>(nnz + 1);
-    int32_t *meta = pm.take<int32_t>(16);
+    nm::TPlan t;
+    int32_t *meta = nullptr;
+    plan_layout(rows, nnz, plan_mem, &t, &p->order, &p->level_ptr, &meta);
+    p->t_indptr = t.t_indptr;
+    p->t_row = t.t_row;
+    p->t_perm = t.t_perm;
 
     auto bail = [&](int rc) { delete p; return rc; };
     if (rows == 0) { *plan_out = p; return NM_OK; }
 
-    Carver wk(work);
-    int32_t *deg = wk.take<int32_t>(rows + 1);
-    int32_t *keys = wk.take<int32_t>(nnz + 1);
-    int32_t *keys_sorted = wk.take<int32_t>(nnz + 1);
-    int32_t *vals = wk.take<int32_t>(nnz + 1);
-    int32_t *rowid = wk.take<int32_t>(nnz + 1);
-    const int bits = bits_for(rows);
-    size_t temp_bytes = sort_temp_bytes(nnz, bits);
-    void *temp = wk.take<char>(temp_bytes);
+    char *wbase = static_cast<char *>(work);
+    int32_t *deg = reinterpret_cast<int32_t *>(wbase);
+    int32_t *rowid = reinterpret_cast<int32_t *>(wbase + align_up((size_t)(rows + 1) * 4));
+    char *twork = wbase + align_up((size_t)(rows + 1) * 4) + align_up((size_t)(nnz + 1) * 4);
+    const size_t twork_bytes = nm::tplan_work_bytes(rows, rows, nnz);
 
+    if (int rc = nm::tplan_build(rows, rows, nnz, indices, indptr, t, twork, twork_bytes, rowid, s)) return bail(rc);
     if (int rc = nm::fill_async(deg, rows + 1, (int32_t)0, s)) return bail(rc);
     if (nnz > 0) {
         int64_t grid = nm::ceil_div(nnz, kBlock);
         if (grid > 65536) grid = 65536;
-        hipLaunchKernelGGL(entry_prep_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, rows, indices,
-                           indptr, p->lower, keys, vals, rowid, deg);
-        if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "entry_prep_kernel launch failed"));
-        hipError_t e = rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, vals, p->t_perm,
-                                                 (size_t)nnz, 0u, (unsigned)bits, s);
-        if (e != hipSuccess)
-            return bail(nm::fail(NM_ERR_HIP, "radix sort failed: %s", hipGetErrorString(e)));
+        hipLaunchKernelGGL(indegree_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, indices, rowid,
+                           p->lower, deg);
+        if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "indegree_kernel launch failed"));
     }
-    {
-        int64_t grid = nm::ceil_div((nnz > rows + 1 ? nnz : rows + 1), kBlock);
-        if (grid > 65536) grid = 65536;
-        hipLaunchKernelGGL(transpose_finish_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, rows,
-                           keys_sorted, p->t_perm, rowid, p->t_indices, p->t_indptr);
-        if (hipGetLastError() != hipSuccess)
-            return bail(nm::fail(NM_ERR_HIP, "transpose_finish_kernel launch failed"));
-    }
-    hipLaunchKernelGGL(kahn_kernel, dim3(1), dim3(kNarrow), 0, s, (int32_t)rows, p->lower, p->t_indptr,
-                       p->t_indices, deg, p->order, p->level_ptr, meta);
+    hipLaunchKernelGGL(kahn_kernel, dim3(1), dim3(kNarrow), 0, s, (int32_t)rows, p->lower, p->t_indptr, p->t_row,
+                       deg, p->order, p->level_ptr, meta);
     if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "kahn_kernel launch failed"));
 
     int32_t meta_h[2] = {0, 0};

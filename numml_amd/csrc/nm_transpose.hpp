@@ -1,0 +1,49 @@
+// Transposed-structure plan: the pattern of A^T as 32-bit arrays, built once
+// per sparsity pattern and reused by every kernel that walks A by column
+// (SpMV / SpMM backward, triangular-solve analysis and transposed solve).
+//
+//   t_indptr[c]  first entry of column c in the column-major order   (cols + 1)
+//   t_row[p]     row of the p-th entry in column-major order         (nnz)
+//   t_perm[p]    its position in A's row-major arrays                 (nnz)
+//
+// Inside a column the entries keep A's row-major order (the sort is stable), so
+// rows ascend, exactly like the counting-sort transpose of the reference
+// (cpp/sparse_csr_cpu.cpp:349-361); t_perm is that function's At_to_A_idx.
+#pragma once
+
+#include "nm_common.hpp"
+
+namespace nm {
+
+struct TPlan {
+    int32_t *t_indptr;
+    int32_t *t_row;
+    int32_t *t_perm;
+};
+
+inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+// Carves the plan arrays out of `base` (nullptr: size query only); returns bytes.
+inline size_t tplan_layout(int64_t cols, int64_t nnz, void *base, TPlan *p) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += align256(bytes);
+        return q;
+    };
+    int32_t *a = (int32_t *)take((size_t)(cols + 1) * 4);
+    int32_t *b = (int32_t *)take((size_t)(nnz + 1) * 4);
+    int32_t *c = (int32_t *)take((size_t)(nnz + 1) * 4);
+    if (p) *p = TPlan{a, b, c};
+    return off;
+}
+
+// Scratch bytes tplan_build needs.
+size_t tplan_work_bytes(int64_t rows, int64_t cols, int64_t nnz);
+
+// Enqueues the build on `s`; does not synchronise.  `rowid_out`, when given,
+// receives the row of every entry in row-major order (nnz int32).
+int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices, const int64_t *indptr,
+                const TPlan &plan, void *work, size_t work_bytes, int32_t *rowid_out, hipStream_t s);
+
+}  // namespace nm

@@ -11,6 +11,7 @@ tensors that are not on a HIP device raise ``RuntimeError``.
 """
 import collections
 import ctypes
+import os
 import threading
 
 import torch
@@ -78,6 +79,73 @@ def _rowmajor(M):
     return M, ld
 
 
+# ------------------------------------------------------------ structure plans
+#
+# Everything derived from a sparsity pattern alone (the transposed structure, the
+# level schedule of a triangle) is computed once and cached.  A plan is keyed on
+# the storage and version counters of the structure tensors, and it keeps those
+# tensors alive, so an address cannot be reused by a different pattern while its
+# plan is cached; in-place edits bump the version and miss the cache.
+
+_PLAN_CACHE_SIZE = 16
+_plans = collections.OrderedDict()
+_plans_lock = threading.Lock()
+
+# "planned": backward passes walk A by column on a cached transposed structure
+#            (deterministic, no atomics);  "atomic": stateless scatter with atomics.
+BACKWARD_MODE = os.environ.get("NUMML_AMD_BACKWARD", "planned")
+
+
+def clear_plan_cache():
+    with _plans_lock:
+        _plans.clear()
+
+
+def _cached(kind, indices, indptr, extra, make):
+    key = (kind, indices.device.index, indices.data_ptr(), indptr.data_ptr(), indices._version,
+           indptr._version, indices.shape[0], indptr.shape[0]) + tuple(extra)
+    with _plans_lock:
+        plan = _plans.get(key)
+        if plan is not None:
+            _plans.move_to_end(key)
+            return plan
+    plan = make()
+    with _plans_lock:
+        _plans[key] = plan
+        while len(_plans) > _PLAN_CACHE_SIZE:
+            _plans.popitem(last=False)
+    return plan
+
+
+class _TransposePlan:
+    """Device arrays of the transposed structure (see nm_csr_transpose_plan_build)."""
+
+    def __init__(self, indices, indptr, rows, cols, dev):
+        L = _lib.lib()
+        nnz = indices.shape[0]
+        pbytes, wbytes = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _lib.check(L.nm_csr_transpose_plan_bytes(rows, cols, nnz, ctypes.byref(pbytes),
+                                                 ctypes.byref(wbytes)), "nm_csr_transpose_plan_bytes")
+        self.mem = torch.empty(max(pbytes.value, 8), dtype=torch.uint8, device=dev)
+        work = torch.empty(max(wbytes.value, 8), dtype=torch.uint8, device=dev)
+        self.indices, self.indptr = indices, indptr
+        _lib.check(L.nm_csr_transpose_plan_build(
+            rows, cols, nnz, _ptr(indices), _ptr(indptr), _ptr(self.mem), pbytes.value, _ptr(work),
+            wbytes.value, _stream(dev)), "nm_csr_transpose_plan_build")
+        self.ready = torch.cuda.Event()
+        self.ready.record(torch.cuda.current_stream(dev))
+        # `work` returns to torch's caching allocator, which hands it out again only to
+        # work enqueued later on this same stream
+
+
+def _transpose_plan(indices, indptr, rows, cols, dev):
+    plan = _cached("T", indices, indptr, (rows, cols),
+                   lambda: _TransposePlan(indices, indptr, rows, cols, dev))
+    # a plan built on another stream must have finished before this stream reads it
+    torch.cuda.current_stream(dev).wait_event(plan.ready)
+    return plan
+
+
 # --------------------------------------------------------------------- SpMV
 
 def spgemv_forward(A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
@@ -106,6 +174,12 @@ def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_x = torch.empty_like(x)
+        if BACKWARD_MODE == "planned":
+            plan = _transpose_plan(A_col_ind, A_rowptr, A_rows, x.shape[0], dev)
+            _lib.check(_lib.lib().nm_spgemv_backward_planned(
+                _dt(A_data), A_rows, x.shape[0], A_data.shape[0], _ptr(A_data), _ptr(plan.mem), _ptr(x),
+                _ptr(grad_z), _ptr(grad_A), _ptr(grad_x), _stream(dev)), "nm_spgemv_backward_planned")
+            return [grad_A, grad_x]
         _lib.check(_lib.lib().nm_spgemv_backward(
             _dt(A_data), A_rows, x.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_col_ind),
             _ptr(A_rowptr), _ptr(x), _ptr(grad_z), _ptr(grad_A), _ptr(grad_x), _stream(dev)),
@@ -144,6 +218,13 @@ def spdmm_backward(A_rows, A_cols, A_data, A_indices, A_indptr, B, grad_C):
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_B = torch.empty((B.shape[0], n), dtype=B.dtype, device=dev)
+        if BACKWARD_MODE == "planned":
+            plan = _transpose_plan(A_indices, A_indptr, A_rows, B.shape[0], dev)
+            _lib.check(_lib.lib().nm_spdmm_backward_planned(
+                _dt(A_data), A_rows, B.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_indices),
+                _ptr(A_indptr), _ptr(plan.mem), _ptr(B), ldb, _ptr(grad_C), ldg, n, _ptr(grad_A),
+                _ptr(grad_B), max(n, 1), _stream(dev)), "nm_spdmm_backward_planned")
+            return [grad_A, grad_B]
         _lib.check(_lib.lib().nm_spdmm_backward(
             _dt(A_data), A_rows, B.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_indices),
             _ptr(A_indptr), _ptr(B), ldb, _ptr(grad_C), ldg, n, _ptr(grad_A), _ptr(grad_B),
@@ -231,6 +312,7 @@ class _Plan:
         self.handle = handle
         self.levels = int(L.nm_sptrsv_plan_levels(handle))
         self.launches = int(L.nm_sptrsv_plan_launches(handle))
+        # nm_sptrsv_analyse synchronised its stream, so the plan is complete for every stream
 
     def __del__(self):
         try:
@@ -241,32 +323,9 @@ class _Plan:
             pass
 
 
-_PLAN_CACHE_SIZE = 16
-_plans = collections.OrderedDict()
-_plans_lock = threading.Lock()
-
-
-def clear_plan_cache():
-    with _plans_lock:
-        _plans.clear()
-
-
 def _plan_for(indices, indptr, rows, lower, dev):
-    """Cached plan of (structure, triangle).  Keyed on the structure tensors' storage and
-    version counters; in-place edits of the structure therefore trigger a new analysis."""
-    key = (dev.index, indices.data_ptr(), indptr.data_ptr(), indices._version, indptr._version,
-           rows, indices.shape[0], bool(lower))
-    with _plans_lock:
-        plan = _plans.get(key)
-        if plan is not None:
-            _plans.move_to_end(key)
-            return plan
-    plan = _Plan(indices, indptr, rows, lower, dev)
-    with _plans_lock:
-        _plans[key] = plan
-        while len(_plans) > _PLAN_CACHE_SIZE:
-            _plans.popitem(last=False)
-    return plan
+    return _cached("L", indices, indptr, (rows, bool(lower)),
+                   lambda: _Plan(indices, indptr, rows, lower, dev))
 
 
 def _solve(plan, transposed, A_data, A_indices, A_indptr, unit, b, rows, dev):

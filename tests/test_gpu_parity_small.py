@@ -28,8 +28,19 @@ def _matrices(dtype):
     yield "empty", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(6, np.int64), (5, 4))
 
 
+@pytest.fixture(params=["planned", "atomic"])
+def backward_mode(request):
+    old = ext.BACKWARD_MODE
+    ext.BACKWARD_MODE = request.param
+    yield request.param
+    ext.BACKWARD_MODE = old
+
+
+STENCILS = ("tridiag16", "tridiag2048", "poisson64")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_spmv_forward_backward(dev, dtype):
+def test_spmv_forward_backward(dev, dtype, backward_mode):
     for name, (d, i, p, (rows, cols)) in _matrices(dtype):
         x, g = randn(1, cols, dtype), randn(2, rows, dtype)
         y_ref = oracle.spgemv_forward(rows, cols, d, i, p, x)
@@ -40,14 +51,16 @@ def test_spmv_forward_backward(dev, dtype):
         assert_close(host(y), y_ref, f"{name} y")
         assert_same(host(gA), gA_ref, f"{name} grad_A")
         assert_close(host(gx), gx_ref, f"{name} grad_x")
-        if name in ("tridiag16", "tridiag2048", "poisson64"):
+        if name in STENCILS:
             # short rows are summed in storage order: bit-identical to the serial loop
             assert_same(host(y), y_ref, f"{name} y (bitwise)")
+            if backward_mode == "planned":   # columns are summed in ascending row order as well
+                assert_same(host(gx), gx_ref, f"{name} grad_x (bitwise)")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n", [1, 7, 64, 100])
-def test_spmm_forward_backward(dev, dtype, n):
+def test_spmm_forward_backward(dev, dtype, n, backward_mode):
     for name, (d, i, p, (rows, cols)) in _matrices(dtype):
         if name == "one_dense_row" and n > 7:
             continue
@@ -60,6 +73,8 @@ def test_spmm_forward_backward(dev, dtype, n):
         assert_same(host(C), C_ref, f"{name} C")
         assert_close(host(gA), gA_ref, f"{name} grad_A")
         assert_close(host(gB), gB_ref, f"{name} grad_B")
+        if backward_mode == "planned":
+            assert_same(host(gB), gB_ref, f"{name} grad_B (bitwise)")
 
 
 def test_spmm_strided_operand(dev):
@@ -102,6 +117,8 @@ def test_spgemm_forward_backward(dev, dtype):
         gA, gB = ext.spgemm_backward(GC, Ci, Cp, ar, ac, AD, AI, AP, br, bc, BD, BI, BP)
         assert_same(host(gA), gA_ref, f"{name} grad_A")
         assert_close(host(gB), gB_ref, f"{name} grad_B")
+        if backward_mode == "planned":
+            assert_same(host(gB), gB_ref, f"{name} grad_B (bitwise)")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
