@@ -42,6 +42,19 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // and the kernels stride.
 constexpr int64_t kMaxGrid = 1 << 30;
 
+// MI355X has 8 accelerator dies (XCDs), each with a private L2; the hardware
+// deals consecutive workgroup ids round-robin over them.  xcd_tile() turns the
+// workgroup id into a tile index such that every XCD walks one contiguous
+// eighth of the tiles, which keeps cache lines shared by neighbouring tiles
+// (halo reads, partially written lines) inside one L2.  `ntiles_padded` is
+// xcd_padded(ntiles); ids that map past `ntiles` own no tile.
+constexpr int kXcds = 8;
+__host__ __device__ inline int64_t xcd_padded(int64_t ntiles) { return (ntiles + kXcds - 1) / kXcds * kXcds; }
+__device__ __forceinline__ int64_t xcd_tile(int64_t id, int64_t ntiles_padded) {
+    const int64_t per = ntiles_padded / kXcds;
+    return (id % kXcds) * per + id / kXcds;
+}
+
 inline hipStream_t as_stream(nm_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
 // ---- device helpers -------------------------------------------------------

@@ -49,7 +49,11 @@ __global__ __launch_bounds__(kBlock) void spmv_fwd_kernel(
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
 
-    for (int64_t r0 = (int64_t)blockIdx.x * R; r0 < rows; r0 += (int64_t)gridDim.x * R) {
+    const int64_t ntiles = (rows + R - 1) / R, npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t r0 = tile * R;
         const int nr = (int)(rows - r0 < R ? rows - r0 : R);
         const int64_t base = indptr[r0];
         stage_offsets<R, CAP>(indptr, r0, nr, base, s_off);
@@ -112,7 +116,11 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
 
-    for (int64_t r0 = (int64_t)blockIdx.x * R; r0 < rows; r0 += (int64_t)gridDim.x * R) {
+    const int64_t ntiles = (rows + R - 1) / R, npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t r0 = tile * R;
         const int nr = (int)(rows - r0 < R ? rows - r0 : R);
         const int64_t base = indptr[r0];
         stage_offsets<R, CAP>(indptr, r0, nr, base, s_off);
@@ -176,11 +184,11 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
     __shared__ T s_v[CAP];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
-    const int64_t nblk = (cols + R - 1) / R;
-    // column blocks are taken from the far end first: the forward pass that precedes a
-    // backward leaves the tail of A's value array in the last-level cache
-    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
-        const int64_t c0 = (nblk - 1 - blk) * R;
+    const int64_t ntiles = (cols + R - 1) / R, npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t c0 = tile * R;
         const int nc = (int)(cols - c0 < R ? cols - c0 : R);
         const int32_t base = t_indptr[c0];
         for (int t = threadIdx.x; t <= nc; t += kBlock) {
@@ -263,7 +271,7 @@ template <typename T>
 int launch_fwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *x,
                T *y, hipStream_t s) {
     constexpr int R = Tile<T>::R, CAP = Tile<T>::CAP;
-    int64_t grid = nm::ceil_div(rows, R);
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, R));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     hipLaunchKernelGGL((spmv_fwd_kernel<T, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, data,
                        indices, indptr, x, y);
@@ -275,7 +283,7 @@ template <typename T>
 int launch_bwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *a,
                const T *b, T alpha, T *out_A, T *grad_x, hipStream_t s) {
     constexpr int R = Tile<T>::R, CAP = Tile<T>::CAP;
-    int64_t grid = nm::ceil_div(rows, R);
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, R));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     hipLaunchKernelGGL((spmv_bwd_kernel<T, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, data,
                        indices, indptr, a, b, alpha, out_A, grad_x);
@@ -350,14 +358,14 @@ extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t col
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32) {
         constexpr int R = Tile<float>::R, CAP = Tile<float>::CAP;
-        int64_t grid = nm::ceil_div(cols, R);
+        int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
         if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
         hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
                            (const float *)data, t.t_indptr, t.t_row, t.t_perm, (const float *)x, (const float *)g,
                            (float *)grad_A, (float *)grad_x);
     } else {
         constexpr int R = Tile<double>::R, CAP = Tile<double>::CAP;
-        int64_t grid = nm::ceil_div(cols, R);
+        int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
         if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
         hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
                            (const double *)data, t.t_indptr, t.t_row, t.t_perm, (const double *)x,

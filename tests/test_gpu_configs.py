@@ -1,0 +1,135 @@
+"""The five benchmark configurations at full size: HIP path against the serial
+oracle on the same seeded inputs, plus size-independent identities.
+
+Tolerance (fp32 1e-5, fp64 1e-12): |a - ref| <= rtol * |ref| + rtol * max|ref|;
+SpGEMM structure and everything summed in the oracle's order is compared bitwise.
+"""
+import numpy as np
+import pytest
+import scipy.sparse as sps
+import torch
+
+import oracle
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as ext
+from numml_amd import sparse as sp
+from util import assert_close, assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def test_cfg1_spmv_fp64_poisson256_autograd(dev):
+    d, i, p, (rows, cols) = G.poisson2d(256, np.float64)
+    x, g = randn(0, cols, np.float64), randn(1, rows, np.float64)
+    D, I, P, X, Gv = to_dev(dev, d, i, p, x, g)
+    A = sp.SparseCSRTensor((D, I, P), (rows, cols))
+    A.requires_grad = True
+    X.requires_grad_(True)
+    y = A @ X
+    y.backward(Gv)
+    gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+    assert_same(host(y), oracle.spgemv_forward(rows, cols, d, i, p, x), "y")
+    assert_same(host(A.data.grad), gA_ref, "grad_A")
+    assert_same(host(X.grad), gx_ref, "grad_x")
+    assert A.grad.shape == (rows, cols) and A.grad.nnz == d.shape[0]
+
+
+@pytest.mark.parametrize("mode", ["planned", "atomic"])
+def test_cfg2_spmv_fp32_poisson2048(dev, mode):
+    d, i, p, (rows, cols) = G.poisson2d(2048, np.float32, jitter_seed=0)
+    assert rows == 4194304 and d.shape[0] == 20963328
+    x, g = randn(1, cols, np.float32), randn(2, rows, np.float32)
+    D, I, P, X, Gv = to_dev(dev, d, i, p, x, g)
+    old, ext.BACKWARD_MODE = ext.BACKWARD_MODE, mode
+    try:
+        y = ext.spgemv_forward(rows, cols, D, I, P, X)
+        gA, gx = ext.spgemv_backward(Gv, rows, cols, D, I, P, X)
+        gA2, gx2 = ext.spgemv_backward(Gv, rows, cols, D, I, P, X)
+    finally:
+        ext.BACKWARD_MODE = old
+    gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+    assert_same(host(y), oracle.spgemv_forward(rows, cols, d, i, p, x), "y")
+    assert_same(host(gA), gA_ref, "grad_A")
+    assert_close(host(gx), gx_ref, "grad_x")
+    if mode == "planned":
+        assert_same(host(gx), gx_ref, "grad_x (bitwise)")
+        assert torch.equal(gx, gx2) and torch.equal(gA, gA2)       # run-to-run identical
+    # adjoint identity <A x, g> = <x, A^T g> in double
+    lhs = float(host(y).astype(np.float64) @ g.astype(np.float64))
+    rhs = float(host(gx).astype(np.float64) @ x.astype(np.float64))
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
+
+
+def test_cfg3_spmm_fp32_powerlaw(dev):
+    rows = cols = 1_000_000
+    n = 64
+    d, i, p, _ = G.powerlaw(rows, cols, target_nnz=16_000_000, seed=0, dtype=np.float32)
+    lens = np.diff(p)
+    assert lens.max() == 10_000 and lens.min() >= 1 and 14e6 < d.shape[0] < 17e6
+    B, gC = randn(1, (cols, n), np.float32), randn(2, (rows, n), np.float32)
+    D, I, P, Bd, Gd = to_dev(dev, d, i, p, B, gC)
+    C = ext.spdmm_forward(rows, cols, D, I, P, Bd)
+    gA, gB = ext.spdmm_backward(rows, cols, D, I, P, Bd, Gd)
+    C, gA, gB = host(C), host(gA), host(gB)
+    # oracle on the first 30k rows (its row->column->entry loop is slow): C and grad_A are row-local
+    sub = 30_000
+    nz = int(p[sub])
+    C_ref = oracle.spdmm_forward(sub, cols, d[:nz], i[:nz], p[:sub + 1], B)
+    gA_ref, _ = oracle.spdmm_backward(sub, cols, d[:nz], i[:nz], p[:sub + 1], B, gC[:sub])
+    assert_same(C[:sub], C_ref, "C (first rows)")
+    assert_close(gA[:nz], gA_ref, "grad_A (first rows)")
+    # the longest row, wherever it is
+    r = int(np.argmax(lens))
+    sl = slice(int(p[r]), int(p[r + 1]))
+    one = np.array([0, lens[r]], dtype=np.int64)
+    assert_same(C[r:r + 1], oracle.spdmm_forward(1, cols, d[sl], i[sl], one, B), "C (longest row)")
+    # grad_B = A^T gC against SciPy in double, all rows
+    At = sps.csr_matrix((d.astype(np.float64), i, p), shape=(rows, cols)).T.tocsr()
+    gB_ref = (At @ gC.astype(np.float64))
+    scale = np.abs(gB_ref).max()
+    assert np.all(np.abs(gB - gB_ref) <= 1e-5 * np.abs(gB_ref) + 1e-5 * scale)
+    # adjoint identity <A B, gC> = <B, A^T gC>
+    lhs = float(np.sum(C.astype(np.float64) * gC))
+    rhs = float(np.sum(gB.astype(np.float64) * B))
+    assert abs(lhs - rhs) <= 1e-4 * abs(lhs)
+
+
+def test_cfg4_spgemm_fp64_laplace128(dev):
+    d, i, p, (rows, cols) = G.laplace3d(128, np.float64, jitter_seed=0)
+    assert rows == 2097152 and d.shape[0] == 14581760
+    D, I, P = to_dev(dev, d, i, p)
+    A = sp.SparseCSRTensor((D, I, P), (rows, cols), clone=False)
+    A.requires_grad = True
+    C = A @ A
+    assert C.nnz == 51742208
+    Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(rows, cols, d, i, p, rows, cols, d, i, p)
+    assert_same(host(C.indptr), Cp_ref, "C_indptr")
+    assert_same(host(C.indices), Ci_ref, "C_indices")
+    assert_same(host(C.data), Cd_ref, "C_data")
+    gC = randn(1, C.nnz, np.float64)
+    C.data.backward(to_dev(dev, gC)[0])
+    gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, rows, cols, d, i, p, rows, cols, d, i, p)
+    assert_close(host(A.data.grad), gA_ref + gB_ref, "grad wrt A.values (grad_A + grad_B)")
+
+
+def test_cfg5_sptrsv_fp64_tril_poisson1024(dev):
+    ext.clear_plan_cache()
+    d, i, p, (n, _) = G.poisson2d_lower(1024, np.float64, diag_seed=0)
+    assert n == 1048576 and d.shape[0] == 3143680
+    b, g = randn(1, n, np.float64), randn(2, n, np.float64)
+    D, I, P, Bv, Gv = to_dev(dev, d, i, p, b, g)
+    L = sp.SparseCSRTensor((D, I, P), (n, n), clone=False)
+    L.requires_grad = True
+    Bv.requires_grad_(True)
+    x = L.solve_triangular(upper=False, unit=False, b=Bv)
+    x.backward(Gv)
+    x_ref = oracle.sptrsv_forward(n, n, d, i, p, True, False, b)
+    gA_ref, gb_ref = oracle.sptrsv_backward(g, x_ref, n, n, d, i, p, True, False)
+    assert_same(host(x), x_ref, "x")
+    assert_same(host(Bv.grad), gb_ref, "grad_b")
+    assert_same(host(L.data.grad), gA_ref, "grad_A")
+    plan = next(v for k, v in ext._plans.items() if k[0] == "L")
+    assert plan.levels == 2047
+    # residual of the full-size solve
+    r = sps.csr_matrix((d, i, p), shape=(n, n)) @ host(x) - b
+    assert np.linalg.norm(r) <= 1e-12 * np.linalg.norm(b) * 10
