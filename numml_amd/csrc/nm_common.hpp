@@ -55,6 +55,14 @@ __device__ __forceinline__ int64_t xcd_tile(int64_t id, int64_t ntiles_padded) {
     return (id % kXcds) * per + id / kXcds;
 }
 
+// Same dealing, but every XCD walks its eighth from the far end: a backward pass
+// that follows a forward pass then starts on the data the forward touched last,
+// which is what the memory-side cache still holds.
+__device__ __forceinline__ int64_t xcd_tile_reversed(int64_t id, int64_t ntiles_padded) {
+    const int64_t per = ntiles_padded / kXcds;
+    return (id % kXcds) * per + (per - 1 - id / kXcds);
+}
+
 inline hipStream_t as_stream(nm_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
 // ---- device helpers -------------------------------------------------------
@@ -79,6 +87,12 @@ __device__ __forceinline__ T group_sum(T v) {
 // (global_atomic_add_f32 / _f64).
 __device__ __forceinline__ void atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
 __device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
+
+// Streaming access: data that is read or written exactly once bypasses the
+// cache retention policy (nontemporal), which leaves L2 to the gathered
+// operands.  Measured on MI355X SpMV: 62 -> 54 us forward.
+template <typename T> __device__ __forceinline__ T stream_load(const T *p) { return __builtin_nontemporal_load(p); }
+template <typename T> __device__ __forceinline__ void stream_store(T *p, T v) { __builtin_nontemporal_store(v, p); }
 
 // out[i] = v for i in [0, n): used instead of hipMemsetAsync so that callers
 // may capture these entry points into HIP graphs.

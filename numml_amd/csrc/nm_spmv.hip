@@ -28,6 +28,8 @@ constexpr int kLongRow = 32;
 template <typename T> struct Tile;
 template <> struct Tile<float>  { static constexpr int R = 512; static constexpr int CAP = 4096; };
 template <> struct Tile<double> { static constexpr int R = 512; static constexpr int CAP = 4096; };
+// columns per workgroup / LDS entries of the planned backward (measured best at cfg2: 96 vs 101 us)
+constexpr int kPlannedR = 256, kPlannedCap = 2048;
 
 // Loads the block's row offsets relative to `base` into LDS, clamped to CAP+1
 // so that they fit 32 bits whatever the block holds.
@@ -64,21 +66,23 @@ __global__ __launch_bounds__(kBlock) void spmv_fwd_kernel(
             const int64_t *__restrict__ ci = indices + base;
             int k = threadIdx.x;
             for (; k + 3 * kBlock < n; k += 4 * kBlock) {
-                const int64_t c0 = ci[k], c1 = ci[k + kBlock], c2 = ci[k + 2 * kBlock], c3 = ci[k + 3 * kBlock];
-                const T a0 = d[k], a1 = d[k + kBlock], a2 = d[k + 2 * kBlock], a3 = d[k + 3 * kBlock];
+                const int64_t c0 = nm::stream_load(ci + k), c1 = nm::stream_load(ci + k + kBlock),
+                              c2 = nm::stream_load(ci + k + 2 * kBlock), c3 = nm::stream_load(ci + k + 3 * kBlock);
+                const T a0 = nm::stream_load(d + k), a1 = nm::stream_load(d + k + kBlock),
+                        a2 = nm::stream_load(d + k + 2 * kBlock), a3 = nm::stream_load(d + k + 3 * kBlock);
                 const T x0 = x[c0], x1 = x[c1], x2 = x[c2], x3 = x[c3];
                 s_prod[k] = a0 * x0;
                 s_prod[k + kBlock] = a1 * x1;
                 s_prod[k + 2 * kBlock] = a2 * x2;
                 s_prod[k + 3 * kBlock] = a3 * x3;
             }
-            for (; k < n; k += kBlock) s_prod[k] = d[k] * x[ci[k]];
+            for (; k < n; k += kBlock) s_prod[k] = nm::stream_load(d + k) * x[nm::stream_load(ci + k)];
             __syncthreads();
             for (int t = threadIdx.x; t < nr; t += kBlock) {
                 const int e = s_off[t + 1];
                 T acc = 0;
                 for (int j = s_off[t]; j < e; ++j) acc += s_prod[j];
-                y[r0 + t] = acc;
+                nm::stream_store(y + r0 + t, acc);
             }
         } else {
             // short rows: one lane each, straight from global memory
@@ -170,23 +174,30 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
 // Backward over the transposed-structure plan (columns of A as rows of A^T):
 // no atomics and no clearing of grad_x.  A workgroup owns R consecutive
 // columns; lane p of the entry-parallel phase reads (row, position) of the
-// p-th entry in column-major order, writes grad_A[position] = g[row] * x[col]
-// and leaves g[row] * data[position] in LDS; one lane per column then adds its
-// slice in ascending row order, the order in which the serial CPU loop
-// accumulates grad_x (cpp/sparse_csr_cpu.cpp:68-73), so grad_x matches it bit
-// for bit and is the same on every run.
+// p-th entry in column-major order and leaves g[row] * data[position] in LDS;
+// one lane per column then adds its slice in ascending row order, the order in
+// which the serial CPU loop accumulates grad_x (cpp/sparse_csr_cpu.cpp:68-73),
+// so grad_x matches it bit for bit and is the same on every run.
+//
+// grad_A: in general entry p = (row r, column c) sits at `position` in A's
+// arrays and grad_A[position] = g[r] * x[c] is a scattered store.  When the
+// pattern is symmetric (plan flag) the column-major entry p is the mirror of the
+// row-major entry p = (row c, column r), so the lane writes
+// grad_A[p] = g[c] * x[r] instead: a coalesced store, every entry once.
 template <typename T, int R, int CAP>
 __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
     int64_t cols, const T *__restrict__ data, const int32_t *__restrict__ t_indptr,
-    const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm, const T *__restrict__ x,
-    const T *__restrict__ g, T *__restrict__ grad_A, T *__restrict__ grad_x) {
+    const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm,
+    const int32_t *__restrict__ flags, const T *__restrict__ x, const T *__restrict__ g,
+    T *__restrict__ grad_A, T *__restrict__ grad_x) {
     __shared__ int32_t s_off[R + 1];
     __shared__ T s_v[CAP];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
+    const bool mirror = flags[0] != 0;
     const int64_t ntiles = (cols + R - 1) / R, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
-        const int64_t tile = nm::xcd_tile(id, npad);
+        const int64_t tile = nm::xcd_tile_reversed(id, npad);
         if (tile >= ntiles) continue;
         const int64_t c0 = tile * R;
         const int nc = (int)(cols - c0 < R ? cols - c0 : R);
@@ -199,19 +210,25 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
         const int n = s_off[nc];
         if (n <= CAP) {
             if (grad_A) {
+                // spread the column's own factor over its entries: g[c] (mirror) or x[c]
+                const T *__restrict__ own = mirror ? g : x;
                 for (int t = threadIdx.x; t < nc; t += kBlock) {
-                    const T xv = x[c0 + t];
+                    const T v = own[c0 + t];
                     const int e = s_off[t + 1];
-                    for (int j = s_off[t]; j < e; ++j) s_v[j] = xv;
+                    for (int j = s_off[t]; j < e; ++j) s_v[j] = v;
                 }
                 __syncthreads();
             }
             const int32_t *__restrict__ tr = t_row + base;
             const int32_t *__restrict__ tp = t_perm + base;
             for (int p = threadIdx.x; p < n; p += kBlock) {
-                const int32_t k = tp[p];
-                const T gr = g[tr[p]];
-                if (grad_A) grad_A[k] = gr * s_v[p];
+                const int32_t k = nm::stream_load(tp + p);
+                const int32_t r = nm::stream_load(tr + p);
+                const T gr = g[r];
+                if (grad_A) {
+                    if (mirror) grad_A[base + p] = s_v[p] * x[r];
+                    else grad_A[k] = gr * s_v[p];
+                }
                 if (grad_x) s_v[p] = gr * data[k];
             }
             if (grad_x) {
@@ -357,18 +374,18 @@ extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t col
     nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32) {
-        constexpr int R = Tile<float>::R, CAP = Tile<float>::CAP;
+        constexpr int R = kPlannedR, CAP = kPlannedCap;
         int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
         if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
         hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                           (const float *)data, t.t_indptr, t.t_row, t.t_perm, (const float *)x, (const float *)g,
+                           (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.flags, (const float *)x, (const float *)g,
                            (float *)grad_A, (float *)grad_x);
     } else {
-        constexpr int R = Tile<double>::R, CAP = Tile<double>::CAP;
+        constexpr int R = kPlannedR, CAP = kPlannedCap;
         int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
         if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
         hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                           (const double *)data, t.t_indptr, t.t_row, t.t_perm, (const double *)x,
+                           (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.flags, (const double *)x,
                            (const double *)g, (double *)grad_A, (double *)grad_x);
     }
     NM_LAUNCH_CHECK("spmv_bwd_planned_kernel");

@@ -55,6 +55,22 @@ __global__ void finish_kernel(int64_t nnz, int64_t cols, const int32_t *__restri
     }
 }
 
+__global__ void symmetry_init_kernel(int32_t *flags, int square) {
+    if (threadIdx.x == 0) flags[0] = square;
+}
+
+// Clears flags[0] unless A^T has exactly A's structure.
+__global__ void symmetry_check_kernel(int64_t nnz, int64_t cols, const int64_t *__restrict__ indices,
+                                      const int64_t *__restrict__ indptr, const int32_t *__restrict__ t_row,
+                                      const int32_t *__restrict__ t_indptr, int32_t *flags) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    bool same = true;
+    for (int64_t p = tid; p < nnz; p += stride) same &= (int64_t)t_row[p] == indices[p];
+    for (int64_t c = tid; c <= cols; c += stride) same &= (int64_t)t_indptr[c] == indptr[c];
+    if (!same) flags[0] = 0;
+}
+
 struct WorkT {
     int32_t *keys, *keys_sorted, *vals, *rowid;
     void *temp;
@@ -118,6 +134,12 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
     hipLaunchKernelGGL(finish_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, cols, w.keys_sorted,
                        plan.t_perm, rowid, plan.t_row, plan.t_indptr);
     NM_LAUNCH_CHECK("transpose finish_kernel");
+    hipLaunchKernelGGL(symmetry_init_kernel, dim3(1), dim3(64), 0, s, plan.flags, rows == cols ? 1 : 0);
+    if (rows == cols) {
+        hipLaunchKernelGGL(symmetry_check_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, cols, indices,
+                           indptr, plan.t_row, plan.t_indptr, plan.flags);
+    }
+    NM_LAUNCH_CHECK("symmetry check");
     return NM_OK;
 }
 

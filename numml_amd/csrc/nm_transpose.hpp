@@ -5,6 +5,8 @@
 //   t_indptr[c]  first entry of column c in the column-major order   (cols + 1)
 //   t_row[p]     row of the p-th entry in column-major order         (nnz)
 //   t_perm[p]    its position in A's row-major arrays                 (nnz)
+//   flags[0]     1 when the pattern is symmetric (A^T has A's structure, so
+//                entry p of column c is the mirror image of the row-major entry p)
 //
 // Inside a column the entries keep A's row-major order (the sort is stable), so
 // rows ascend, exactly like the counting-sort transpose of the reference
@@ -19,6 +21,7 @@ struct TPlan {
     int32_t *t_indptr;
     int32_t *t_row;
     int32_t *t_perm;
+    int32_t *flags;
 };
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
@@ -34,7 +37,8 @@ inline size_t tplan_layout(int64_t cols, int64_t nnz, void *base, TPlan *p) {
     int32_t *a = (int32_t *)take((size_t)(cols + 1) * 4);
     int32_t *b = (int32_t *)take((size_t)(nnz + 1) * 4);
     int32_t *c = (int32_t *)take((size_t)(nnz + 1) * 4);
-    if (p) *p = TPlan{a, b, c};
+    int32_t *f = (int32_t *)take(16 * 4);
+    if (p) *p = TPlan{a, b, c, f};
     return off;
 }
 
