@@ -99,9 +99,10 @@ class SpMV(Workload):
         self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s)
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
-        self.dominant_name = "spmv_bwd_kernel (+ fill_kernel clearing grad_x)"
+        self.dominant_name = ("spmv_bwd_planned_kernel" if ext.BACKWARD_MODE == "planned"
+                              else "spmv_bwd_kernel (+ fill_kernel clearing grad_x)")
         self.config = {"workload": f"spmv_fwd_bwd_{self.dtype}_{self.label}", "rows": rows,
-                       "nnz": self.nnz, "index_bytes": 8,
+                       "nnz": self.nnz, "index_bytes": 8, "backward": ext.BACKWARD_MODE,
                        "algorithmic_bytes_per_step": self.bytes_per_step}
 
     def step(self):
@@ -151,7 +152,9 @@ class SpMM(Workload):
                           + cols * n * s)
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
-        self.dominant_name = "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)"
+        self.dominant_name = ("spdmm_bwd_kernel (grad_A) + spdmm_fwd_kernel on the transposed plan (grad_B)"
+                              if ext.BACKWARD_MODE == "planned"
+                              else "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)")
         self.config = {"workload": "spmm_fwd_bwd_f32_powerlaw_1M_n64", "rows": rows, "nnz": nnz,
                        "dense_cols": n, "index_bytes": 8,
                        "algorithmic_bytes_per_step": self.bytes_per_step,

@@ -27,7 +27,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
     f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
-]
+] + os.environ.get("NM_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def _compile(src):

@@ -28,22 +28,29 @@ constexpr int kLongRow = 32;
 template <typename T> struct Tile;
 template <> struct Tile<float>  { static constexpr int R = 512; static constexpr int CAP = 4096; };
 template <> struct Tile<double> { static constexpr int R = 512; static constexpr int CAP = 4096; };
+// forward: lanes per workgroup, rows per workgroup, LDS products
+#ifndef NM_FWD_BLOCK
+#define NM_FWD_BLOCK 256
+#define NM_FWD_R 512
+#define NM_FWD_CAP 4096
+#endif
+constexpr int kFwdBlock = NM_FWD_BLOCK, kFwdR = NM_FWD_R, kFwdCap = NM_FWD_CAP;
 // columns per workgroup / LDS entries of the planned backward (measured best at cfg2: 96 vs 101 us)
 constexpr int kPlannedR = 256, kPlannedCap = 2048;
 
 // Loads the block's row offsets relative to `base` into LDS, clamped to CAP+1
 // so that they fit 32 bits whatever the block holds.
-template <int R, int CAP>
+template <int R, int CAP, int BLOCK>
 __device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ indptr, int64_t r0, int nr,
                                               int64_t base, int32_t *s_off) {
-    for (int t = threadIdx.x; t <= nr; t += kBlock) {
+    for (int t = threadIdx.x; t <= nr; t += BLOCK) {
         const int64_t d = indptr[r0 + t] - base;
         s_off[t] = (int32_t)(d > CAP ? CAP + 1 : d);
     }
 }
 
-template <typename T, int R, int CAP>
-__global__ __launch_bounds__(kBlock) void spmv_fwd_kernel(
+template <typename T, int BLOCK, int R, int CAP>
+__global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
     int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
     const int64_t *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y) {
     __shared__ int32_t s_off[R + 1];
@@ -58,27 +65,27 @@ __global__ __launch_bounds__(kBlock) void spmv_fwd_kernel(
         const int64_t r0 = tile * R;
         const int nr = (int)(rows - r0 < R ? rows - r0 : R);
         const int64_t base = indptr[r0];
-        stage_offsets<R, CAP>(indptr, r0, nr, base, s_off);
+        stage_offsets<R, CAP, BLOCK>(indptr, r0, nr, base, s_off);
         __syncthreads();
         const int n = s_off[nr];
         if (n <= CAP) {
             const T *__restrict__ d = data + base;
             const int64_t *__restrict__ ci = indices + base;
             int k = threadIdx.x;
-            for (; k + 3 * kBlock < n; k += 4 * kBlock) {
-                const int64_t c0 = nm::stream_load(ci + k), c1 = nm::stream_load(ci + k + kBlock),
-                              c2 = nm::stream_load(ci + k + 2 * kBlock), c3 = nm::stream_load(ci + k + 3 * kBlock);
-                const T a0 = nm::stream_load(d + k), a1 = nm::stream_load(d + k + kBlock),
-                        a2 = nm::stream_load(d + k + 2 * kBlock), a3 = nm::stream_load(d + k + 3 * kBlock);
+            for (; k + 3 * BLOCK < n; k += 4 * BLOCK) {
+                const int64_t c0 = nm::stream_load(ci + k), c1 = nm::stream_load(ci + k + BLOCK),
+                              c2 = nm::stream_load(ci + k + 2 * BLOCK), c3 = nm::stream_load(ci + k + 3 * BLOCK);
+                const T a0 = nm::stream_load(d + k), a1 = nm::stream_load(d + k + BLOCK),
+                        a2 = nm::stream_load(d + k + 2 * BLOCK), a3 = nm::stream_load(d + k + 3 * BLOCK);
                 const T x0 = x[c0], x1 = x[c1], x2 = x[c2], x3 = x[c3];
                 s_prod[k] = a0 * x0;
-                s_prod[k + kBlock] = a1 * x1;
-                s_prod[k + 2 * kBlock] = a2 * x2;
-                s_prod[k + 3 * kBlock] = a3 * x3;
+                s_prod[k + BLOCK] = a1 * x1;
+                s_prod[k + 2 * BLOCK] = a2 * x2;
+                s_prod[k + 3 * BLOCK] = a3 * x3;
             }
-            for (; k < n; k += kBlock) s_prod[k] = nm::stream_load(d + k) * x[nm::stream_load(ci + k)];
+            for (; k < n; k += BLOCK) s_prod[k] = nm::stream_load(d + k) * x[nm::stream_load(ci + k)];
             __syncthreads();
-            for (int t = threadIdx.x; t < nr; t += kBlock) {
+            for (int t = threadIdx.x; t < nr; t += BLOCK) {
                 const int e = s_off[t + 1];
                 T acc = 0;
                 for (int j = s_off[t]; j < e; ++j) acc += s_prod[j];
@@ -86,7 +93,7 @@ __global__ __launch_bounds__(kBlock) void spmv_fwd_kernel(
             }
         } else {
             // short rows: one lane each, straight from global memory
-            for (int t = threadIdx.x; t < nr; t += kBlock) {
+            for (int t = threadIdx.x; t < nr; t += BLOCK) {
                 const int64_t b = indptr[r0 + t], e = indptr[r0 + t + 1];
                 if (e - b >= kLongRow) continue;
                 T acc = 0;
@@ -94,7 +101,7 @@ __global__ __launch_bounds__(kBlock) void spmv_fwd_kernel(
                 y[r0 + t] = acc;
             }
             // long rows: one wavefront each
-            for (int t = wave; t < nr; t += kWavesPerBlock) {
+            for (int t = wave; t < nr; t += (BLOCK / kWave)) {
                 const int64_t b = indptr[r0 + t], e = indptr[r0 + t + 1];
                 if (e - b < kLongRow) continue;
                 T acc = 0;
@@ -127,7 +134,7 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
         const int64_t r0 = tile * R;
         const int nr = (int)(rows - r0 < R ? rows - r0 : R);
         const int64_t base = indptr[r0];
-        stage_offsets<R, CAP>(indptr, r0, nr, base, s_off);
+        stage_offsets<R, CAP, kBlock>(indptr, r0, nr, base, s_off);
         __syncthreads();
         const int n = s_off[nr];
         if (n <= CAP) {
@@ -208,7 +215,47 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
         }
         __syncthreads();
         const int n = s_off[nc];
-        if (n <= CAP) {
+        if (n <= CAP && mirror && grad_A && grad_x) {
+            // fast path: both gradients, symmetric pattern -> every global access but the
+            // gathers of g, x and data is a coalesced stream
+            for (int t = threadIdx.x; t < nc; t += kBlock) {
+                const T v = g[c0 + t];
+                const int e = s_off[t + 1];
+                for (int j = s_off[t]; j < e; ++j) s_v[j] = v;
+            }
+            __syncthreads();
+            const int32_t *__restrict__ tr = t_row + base;
+            const int32_t *__restrict__ tp = t_perm + base;
+            T *__restrict__ ga = grad_A + base;
+            int p = threadIdx.x;
+            for (; p + kBlock < n; p += 2 * kBlock) {   // two entries in flight per lane (measured best)
+                const int32_t k0 = nm::stream_load(tp + p), k1 = nm::stream_load(tp + p + kBlock);
+                const int32_t r0 = nm::stream_load(tr + p), r1 = nm::stream_load(tr + p + kBlock);
+                const T g0 = g[r0], g1 = g[r1];
+                const T x0 = x[r0], x1 = x[r1];
+                const T d0 = data[k0], d1 = data[k1];
+                ga[p] = s_v[p] * x0;
+                ga[p + kBlock] = s_v[p + kBlock] * x1;
+                s_v[p] = g0 * d0;
+                s_v[p + kBlock] = g1 * d1;
+            }
+            for (; p < n; p += kBlock) {
+                const int32_t k = nm::stream_load(tp + p);
+                const int32_t r = nm::stream_load(tr + p);
+                const T gr = g[r];
+                const T xr = x[r];
+                const T dk = data[k];
+                ga[p] = s_v[p] * xr;
+                s_v[p] = gr * dk;
+            }
+            __syncthreads();
+            for (int t = threadIdx.x; t < nc; t += kBlock) {
+                const int e = s_off[t + 1];
+                T acc = 0;
+                for (int j = s_off[t]; j < e; ++j) acc += s_v[j];
+                grad_x[c0 + t] = acc;
+            }
+        } else if (n <= CAP) {
             if (grad_A) {
                 // spread the column's own factor over its entries: g[c] (mirror) or x[c]
                 const T *__restrict__ own = mirror ? g : x;
@@ -287,10 +334,10 @@ int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const i
 template <typename T>
 int launch_fwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *x,
                T *y, hipStream_t s) {
-    constexpr int R = Tile<T>::R, CAP = Tile<T>::CAP;
+    constexpr int R = kFwdR, CAP = kFwdCap;
     int64_t grid = nm::xcd_padded(nm::ceil_div(rows, R));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-    hipLaunchKernelGGL((spmv_fwd_kernel<T, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, data,
+    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows, data,
                        indices, indptr, x, y);
     NM_LAUNCH_CHECK("spmv_fwd_kernel");
     return NM_OK;
