@@ -191,12 +191,14 @@ void nm_sptrsv_plan_destroy(nm_sptrsv_plan *plan);
 /* x = T^{-1} b where T is the planned triangle of A (or its transpose).  Sums
  * run in double for either dtype, in the walk order of the reference loop, and
  * are rounded once at the end (cpp/sparse_csr_cpu.cpp:659-662, :722).
- * `unit` != 0 ignores the stored diagonal.  `xwork` is device scratch of
- * `rows` doubles, needed for NM_F32 only (NULL is fine for NM_F64).  x must
- * not alias b. */
+ * `unit` != 0 ignores the stored diagonal.  `work` is device scratch of
+ * nm_sptrsv_solve_bytes(rows, nnz) bytes (the call's values regathered in
+ * level order and the running solution); it must not alias x or b. */
+int nm_sptrsv_solve_bytes(int64_t rows, int64_t nnz, size_t *bytes);
+
 int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
-                    const void *data, const int64_t *indices, const int64_t *indptr,
-                    int unit, const void *b, void *x, double *xwork, nm_stream stream);
+                    const void *data, int unit, const void *b, void *x,
+                    void *work, size_t work_bytes, nm_stream stream);
 
 /* out[k] = alpha * a[row(k)] * b[col(k)] for every stored entry: the masked
  * outer product behind grad_A of the solve (alpha = -1,

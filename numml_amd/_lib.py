@@ -44,8 +44,8 @@ _SIGNATURES = {
     "nm_sptrsv_plan_bytes": [_c_i64, _c_i64, ctypes.POINTER(_c_size), ctypes.POINTER(_c_size)],
     "nm_sptrsv_analyse": [_c_i64, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_size, _c_ptr, _c_size,
                           ctypes.POINTER(_c_ptr), _c_ptr],
-    "nm_sptrsv_solve": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                        _c_ptr],
+    "nm_sptrsv_solve_bytes": [_c_i64, _c_i64, ctypes.POINTER(_c_size)],
+    "nm_sptrsv_solve": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr],
     "nm_masked_outer": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_dbl, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
 

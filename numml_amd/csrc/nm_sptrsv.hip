@@ -1,40 +1,61 @@
 // Level-scheduled sparse triangular solve for gfx950.
 //
-// Analysis (once per sparsity pattern): the strictly-triangular entries of A
-// define a dependency DAG.  A Kahn sweep, run by one workgroup, peels the DAG
-// level by level and leaves the rows in level order (`order`, `level_ptr`).
-// The sweep needs each row's dependents, i.e. A^T, which is built with a stable
-// radix sort of the entries by column; the same A^T (indices + permutation
-// into A's values) is what the backward solve runs on, so one plan serves both
-// x = A^{-1} b and grad_b = A^{-T} g: the transposed solve walks the same
-// levels in reverse.
+// Analysis (once per sparsity pattern).  The strictly-triangular entries of A
+// define a dependency DAG.  The transposed-structure plan (stable radix sort by
+// column) gives every row's dependents; a Kahn sweep run by one workgroup peels
+// the DAG level by level and leaves the rows in level order: row order[q] sits
+// in "slot" q, level l owns slots [level_ptr[l], level_ptr[l+1]).  The plan
+// then stores, for both solve directions (A and A^T), a level-major packed copy
+// of the triangle: per slot the range of its dependencies, per dependency the
+// SLOT of the row it refers to and the position of its coefficient in A's
+// value array, and the position of the diagonal coefficient.  The transposed
+// solve (the backward pass) walks the same levels in reverse.
 //
-// Solve: runs of consecutive narrow levels (<= 1024 rows) are executed by a
-// single 1024-lane workgroup that separates levels with workgroup barriers;
-// a level wider than that gets a launch of its own across the chip.  Stream
-// order is the only synchronisation between launches, so no kernel ever waits
-// on another workgroup.  Each row is one lane; sums run in double and in the
-// walk direction of the serial CPU loop (cpp/sparse_csr_cpu.cpp:672-718), so
-// results match it bit for bit.
+// Solve.  The running solution lives in slot order (xs[q]), so a dependency is
+// one indexed read and consecutive levels touch neighbouring memory.  Runs of
+// consecutive narrow levels (<= 1024 rows) are executed by ONE 1024-lane
+// workgroup: levels are separated by workgroup barriers, the solutions of the
+// last ~7000 slots are kept in an LDS ring (a dependency on a recent slot costs
+// an LDS read instead of an L2 round trip).  A chip-wide pass first gathers
+// this call's coefficients, diagonal and right-hand side into level-major
+// order (as doubles), so the workgroup reads contiguous streams only, two and
+// one level ahead through a register pipeline.  A level wider than 1024 rows gets a grid launch of its own.
+// Stream order is the only synchronisation between launches: no kernel ever
+// waits on another workgroup, so nothing can hang.
+//
+// Every row is one lane; sums run in double, in the walk order of the serial
+// CPU loop (cpp/sparse_csr_cpu.cpp:672-718: ascending for a lower triangle,
+// descending for an upper one), so results match it bit for bit.
 //
 // Algorithmic HBM bytes of one solve (s = sizeof(value)):
-//   nnz*(s+8) + (rows+1)*8 + 2*rows*s   (+ rows*4 for the level order)
+//   nnz*(s+8) + (rows+1)*8 + 2*rows*s
 #include "nm_common.hpp"
+#include "nm_scan.hpp"
 #include "nm_transpose.hpp"
 
 #include <new>
 #include <vector>
+
+namespace {
+struct Packed {        // one solve direction, level-major (all int32, device)
+    int32_t *dptr;     // [rows+1] dependency range of slot q
+    int32_t *dslot;    // [nnz]    slot of the row a dependency refers to
+    int32_t *dsrc;     // [nnz]    position of its coefficient in A's data
+    int32_t *diag;     // [rows]   position of the diagonal coefficient, -1 when not stored
+};
+}  // namespace
 
 struct nm_sptrsv_plan {
     int64_t rows = 0, nnz = 0;
     int lower = 1;
     int32_t nlevels = 0;
     // device arrays inside the caller's plan memory
-    int32_t *order = nullptr, *level_ptr = nullptr;
-    int32_t *t_indptr = nullptr, *t_row = nullptr, *t_perm = nullptr;
+    int32_t *order = nullptr, *level_ptr = nullptr, *slot_of = nullptr;
+    Packed dir[2];     // [0]: A, [1]: A^T
+    int32_t max_deps[2] = {0, 0};  // longest dependency list per direction
     struct Launch {
         int32_t l0, l1;  // levels [l0, l1)
-        int32_t q0, q1;  // slots of `order` they cover
+        int32_t q0, q1;  // slots they cover
         bool wide;       // one level, many workgroups
     };
     std::vector<Launch> launches;
@@ -42,42 +63,67 @@ struct nm_sptrsv_plan {
 
 namespace {
 
-constexpr int kNarrow = 1024;  // widest level the single-workgroup kernel takes
+constexpr int kNarrow = 1024;          // widest level the single-workgroup kernel takes
 constexpr int kBlock = 256;
+constexpr int kRing = 8192;            // LDS ring of recent solutions (doubles, power of two)
+constexpr int kRingSafe = kRing - kNarrow;
+constexpr int kMaxLevels = 4096;       // levels one single-workgroup launch takes (LDS copy of their bounds)
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
 
-struct Carver {
-    char *base;
-    size_t off = 0;
-    explicit Carver(void *p) : base(static_cast<char *>(p)) {}
-    template <typename T> T *take(size_t count) {
-        T *p = reinterpret_cast<T *>(base + off);
-        off += align_up(count * sizeof(T));
-        return p;
-    }
+struct Layout {
+    nm::TPlan t;
+    int32_t *order, *level_ptr, *slot_of, *meta;
+    Packed dir[2];
 };
 
-// plan memory: [transposed-structure plan][order][level_ptr][meta]
-size_t plan_layout(int64_t rows, int64_t nnz, void *base, nm::TPlan *t, int32_t **order, int32_t **level_ptr,
-                   int32_t **meta) {
-    size_t off = nm::tplan_layout(rows, nnz, base, t);
-    auto take = [&](size_t bytes) {
+// plan memory: [transposed-structure plan][order][level_ptr][slot_of][meta][packed A][packed A^T]
+size_t plan_layout(int64_t rows, int64_t nnz, void *base, Layout *L) {
+    Layout l;
+    size_t off = nm::tplan_layout(rows, nnz, base, &l.t);
+    auto take = [&](size_t count) {
         void *q = base ? static_cast<char *>(base) + off : nullptr;
-        off += align_up(bytes);
+        off += align_up(count * 4);
         return (int32_t *)q;
     };
-    int32_t *o = take((size_t)(rows + 1) * 4), *l = take((size_t)(rows + 1) * 4), *m = take(16 * 4);
-    if (order) *order = o;
-    if (level_ptr) *level_ptr = l;
-    if (meta) *meta = m;
+    l.order = take(rows + 1);
+    l.level_ptr = take(rows + 1);
+    l.slot_of = take(rows + 1);
+    l.meta = take(16);
+    for (int d = 0; d < 2; ++d) {
+        l.dir[d].dptr = take(rows + 1);
+        l.dir[d].dslot = take(nnz + 1);
+        l.dir[d].dsrc = take(nnz + 1);
+        l.dir[d].diag = take(rows + 1);
+    }
+    if (L) *L = l;
     return off;
 }
 
-// analysis scratch: [deg][rowid][transpose scratch]
-size_t work_bytes_needed(int64_t rows, int64_t nnz) {
-    return align_up((size_t)(rows + 1) * 4) + align_up((size_t)(nnz + 1) * 4) +
-           nm::tplan_work_bytes(rows, rows, nnz);
+// analysis scratch: [deg][rowid][count64][scan scratch][transpose scratch]
+struct Scratch {
+    int32_t *deg, *rowid;
+    int64_t *count64, *scan;
+    void *twork;
+    size_t twork_bytes;
+};
+
+size_t work_layout(int64_t rows, int64_t nnz, void *base, Scratch *S) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += align_up(bytes);
+        return q;
+    };
+    Scratch s;
+    s.deg = (int32_t *)take((size_t)(rows + 1) * 4);
+    s.rowid = (int32_t *)take((size_t)(nnz + 1) * 4);
+    s.count64 = (int64_t *)take((size_t)(rows + 1) * 8);
+    s.scan = (int64_t *)take(nm::scan_scratch_bytes(rows + 1));
+    s.twork_bytes = nm::tplan_work_bytes(rows, rows, nnz);
+    s.twork = take(s.twork_bytes);
+    if (S) *S = s;
+    return off;
 }
 
 // ---- analysis kernels ------------------------------------------------------
@@ -131,102 +177,277 @@ __global__ __launch_bounds__(kNarrow) void kahn_kernel(int32_t rows, int lower,
     }
 }
 
-// ---- solve kernels -----------------------------------------------------------
-
-template <typename T> struct SolveArgs {
-    const T *data;
-    const int64_t *indices, *indptr;                  // A
-    const int32_t *t_indptr, *t_row, *t_perm;         // A^T
-    const int32_t *order, *level_ptr;
-    const T *b;
-    double *xw;
-    int unit;
-    int ascending;  // 1: lower-triangular walk (ascending), 0: upper (descending)
-};
-
-template <typename T, bool TR>
-__device__ __forceinline__ void solve_row(const SolveArgs<T> &a, int32_t i) {
-    double diag = 0., acc = 0.;
-    int64_t kb, ke;
-    if (TR) { kb = a.t_indptr[i]; ke = a.t_indptr[i + 1]; }
-    else    { kb = a.indptr[i];   ke = a.indptr[i + 1]; }
-    if (a.ascending) {
-        for (int64_t k = kb; k < ke; ++k) {
-            const int64_t j = TR ? (int64_t)a.t_row[k] : a.indices[k];
-            if (j > i) continue;
-            const double v = (double)(TR ? a.data[a.t_perm[k]] : a.data[k]);
-            if (j == i) diag = v; else acc += v * a.xw[j];
-        }
-    } else {
-        for (int64_t k = ke - 1; k >= kb; --k) {
-            const int64_t j = TR ? (int64_t)a.t_row[k] : a.indices[k];
-            if (j < i) continue;
-            const double v = (double)(TR ? a.data[a.t_perm[k]] : a.data[k]);
-            if (j == i) diag = v; else acc += v * a.xw[j];
-        }
-    }
-    double xi = (double)a.b[i] - acc;
-    if (!a.unit) xi /= diag;
-    a.xw[i] = xi;
+__global__ void slot_of_kernel(int64_t rows, const int32_t *__restrict__ order, int32_t *__restrict__ slot_of) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < rows; q += stride)
+        slot_of[order[q]] = (int32_t)q;
 }
 
-// Levels l0, l0+step, ... (l1 exclusive), each at most kNarrow rows, by one workgroup.
-template <typename T, bool TR>
-__global__ __launch_bounds__(kNarrow) void sptrsv_batch_kernel(SolveArgs<T> a, int l0, int l1, int step) {
-    for (int l = l0; l != l1; l += step) {
-        const int q = a.level_ptr[l] + (int)threadIdx.x;
-        if (q < a.level_ptr[l + 1]) solve_row<T, TR>(a, a.order[q]);
+// Walks the row in slot q in the solve's accumulation order.  TR = 0: row of A
+// (indices/indptr); TR = 1: row of A^T (t_row/t_indptr, coefficient at t_perm).
+// With `fill` == 0 it only counts the strictly-triangular entries.
+template <int TR>
+__global__ void pack_kernel(int64_t rows, int eff_lower, int fill, const int32_t *__restrict__ order,
+                            const int32_t *__restrict__ slot_of, const int64_t *__restrict__ indices,
+                            const int64_t *__restrict__ indptr, const int32_t *__restrict__ t_indptr,
+                            const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm,
+                            int64_t *__restrict__ count64, const int32_t *__restrict__ dptr,
+                            int32_t *__restrict__ dslot, int32_t *__restrict__ dsrc, int32_t *__restrict__ diag,
+                            int32_t *max_deps) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < rows; q += stride) {
+        const int64_t i = order[q];
+        const int64_t kb = TR ? (int64_t)t_indptr[i] : indptr[i];
+        const int64_t ke = TR ? (int64_t)t_indptr[i + 1] : indptr[i + 1];
+        int64_t n = 0;
+        int32_t dpos = -1;
+        int32_t out = fill ? dptr[q] : 0;
+        for (int64_t e = 0; e < ke - kb; ++e) {
+            const int64_t k = eff_lower ? kb + e : ke - 1 - e;
+            const int64_t j = TR ? (int64_t)t_row[k] : indices[k];
+            const int32_t src = TR ? t_perm[k] : (int32_t)k;
+            if (j == i) { dpos = src; continue; }
+            if (eff_lower ? j > i : j < i) continue;   // other side of the diagonal: not part of the solve
+            if (fill) { dslot[out] = slot_of[j]; dsrc[out] = src; ++out; }
+            ++n;
+        }
+        if (fill) { diag[q] = dpos; if (n > *max_deps) atomicMax(max_deps, (int32_t)(n > 0x7fffffff ? 0x7fffffff : n)); }
+        else count64[q] = n;
+    }
+}
+
+__global__ void narrow_kernel(int64_t n, const int64_t *__restrict__ in, int32_t *__restrict__ out) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = (int32_t)in[i];
+}
+
+// ---- solve kernels -----------------------------------------------------------
+
+// Per-solve scratch (doubles): [xs: rows][diag: rows][rhs: rows][coef: nnz]
+struct SolveWork {
+    double *xs;     // running solution in slot order
+    double *dg;     // diagonal coefficient of slot q (0 when not stored)
+    double *rhs;    // right-hand side of slot q
+    double *coef;   // coefficient of packed dependency `at`
+};
+
+inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork *W) {
+    size_t off = 0;
+    auto take = [&](size_t count) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += align_up(count * 8);
+        return (double *)q;
+    };
+    SolveWork w;
+    w.xs = take(rows + 1);
+    w.dg = take(rows + 1);
+    w.rhs = take(rows + 1);
+    w.coef = take(nnz + 1);
+    if (W) *W = w;
+    return off;
+}
+
+// Gathers this call's values into the plan's level-major order, converting to
+// double once: a bandwidth-bound pass over the whole chip, after which the
+// single-workgroup solve reads nothing but contiguous streams.
+template <typename T>
+__global__ void gather_values_kernel(int64_t rows, int64_t nnz, const T *__restrict__ data,
+                                     const T *__restrict__ b, const int32_t *__restrict__ order,
+                                     const int32_t *__restrict__ dptr, const int32_t *__restrict__ dsrc,
+                                     const int32_t *__restrict__ diag, double *__restrict__ coef,
+                                     double *__restrict__ dg, double *__restrict__ rhs) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = dptr[rows];
+    for (int64_t at = tid; at < total; at += stride) coef[at] = (double)data[dsrc[at]];
+    for (int64_t q = tid; q < rows; q += stride) {
+        const int32_t d = diag[q];
+        dg[q] = d >= 0 ? (double)data[d] : 0.;
+        rhs[q] = (double)b[order[q]];
+    }
+}
+
+struct SolveArgs {
+    SolveWork w;
+    const int32_t *level_ptr, *dptr, *dslot;
+    int unit;
+};
+
+// Register pipeline stages of the single-workgroup kernel.
+struct Bounds { int qb, qe; };
+struct Meta { int q; bool live; int32_t dlo, n; };
+template <int PRE> struct Vals { Meta m; int32_t ds[PRE]; double v[PRE]; double dv, bv; };
+
+// Level bounds come from an LDS copy of this launch's slice of level_ptr
+// (s_lp[i] = level_ptr[lmin + i]), so they cost no scalar-memory round trip.
+__device__ __forceinline__ Bounds load_bounds(const int32_t *s_lp, int it, int count, int l0, int step, int lmin) {
+    Bounds r{0, 0};
+    if (it < count) {
+        const int l = l0 + it * step - lmin;
+        r.qb = s_lp[l];
+        r.qe = s_lp[l + 1];
+    }
+    return r;
+}
+
+// All loads below are unconditional with clamped indices (slot 0 / entry 0 always
+// exist), so a stage is straight-line code and the hardware wait counters stay exact.
+__device__ __forceinline__ Meta load_meta(const SolveArgs &a, const Bounds &b) {
+    Meta m;
+    m.q = b.qb + (int)threadIdx.x;
+    m.live = m.q < b.qe;
+    const int qs = m.live ? m.q : 0;
+    m.dlo = a.dptr[qs];
+    m.n = a.dptr[qs + 1] - m.dlo;
+    return m;
+}
+
+template <int PRE> __device__ __forceinline__ Vals<PRE> load_vals(const SolveArgs &a, const Meta &m) {
+    Vals<PRE> v;
+    v.m = m;
+#pragma unroll
+    for (int e = 0; e < PRE; ++e) {
+        const int32_t at = (m.live && e < m.n) ? m.dlo + e : 0;
+        v.ds[e] = a.dslot[at];
+        v.v[e] = a.w.coef[at];
+    }
+    const int qs = m.live ? m.q : 0;
+    v.dv = a.w.dg[qs];
+    v.bv = a.w.rhs[qs];
+    return v;
+}
+
+// Levels l0, l0+step, ... (`count` <= kMaxLevels of them, each at most kNarrow
+// rows) by one workgroup; [qlo, qhi) are the slots this launch solves (only
+// those can be found in the ring).
+template <int PRE>
+__global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l0, int count, int step, int qlo,
+                                                              int qhi) {
+    __shared__ double ring[kRing];
+    __shared__ int32_t s_lp[kMaxLevels + 1];
+    const int lmin = step > 0 ? l0 : l0 - (count - 1);
+    for (int i = threadIdx.x; i <= count; i += kNarrow) s_lp[i] = a.level_ptr[lmin + i];
+    __syncthreads();
+
+    Bounds p0 = load_bounds(s_lp, 0, count, l0, step, lmin);
+    Meta p1 = load_meta(a, p0);
+    p0 = load_bounds(s_lp, 1, count, l0, step, lmin);
+    Vals<PRE> p2 = load_vals<PRE>(a, p1);
+    p1 = load_meta(a, p0);
+    p0 = load_bounds(s_lp, 2, count, l0, step, lmin);
+
+    for (int it = 0; it < count; ++it) {
+        const Vals<PRE> cur = p2;
+        // advance the pipeline: what is issued here is consumed one and two levels later
+        p2 = load_vals<PRE>(a, p1);
+        p1 = load_meta(a, p0);
+        p0 = load_bounds(s_lp, it + 3, count, l0, step, lmin);
+
+        const int q = cur.m.q;
+        const int n = cur.m.live ? cur.m.n : 0;
+        // fast path: no global memory access at all -- every dependency from the LDS ring
+        double acc = 0.;
+        bool in_ring = n <= PRE;
+#pragma unroll
+        for (int e = 0; e < PRE; ++e) {
+            const int32_t ds = cur.ds[e];
+            const int dist = ds > q ? ds - q : q - ds;
+            const bool hit = ds >= qlo && ds < qhi && dist < kRingSafe;
+            const double xj = ring[ds & (kRing - 1)];
+            if (e < n) {
+                in_ring = in_ring && hit;
+                acc += cur.v[e] * xj;
+            }
+        }
+        if (!in_ring) {
+            // slow path (a dependency older than the ring, or a row longer than the
+            // pipeline holds): redo the whole sum in the same order from global memory
+            acc = 0.;
+            for (int e = 0; e < n; ++e) {
+                const int32_t at = cur.m.dlo + e;
+                const int32_t ds = e < PRE ? cur.ds[e] : a.dslot[at];
+                const double v = e < PRE ? cur.v[e] : a.w.coef[at];
+                acc += v * a.w.xs[ds];
+            }
+        }
+        if (cur.m.live) {
+            double xi = cur.bv - acc;
+            if (!a.unit) xi /= cur.dv;
+            ring[q & (kRing - 1)] = xi;
+            a.w.xs[q] = xi;
+        }
         __syncthreads();
     }
 }
 
-// One wide level: slots [q0, q1) of `order`, one lane per row.
-template <typename T, bool TR>
-__global__ __launch_bounds__(kBlock) void sptrsv_level_kernel(SolveArgs<T> a, int q0, int q1) {
+// One wide level: slots [q0, q1), one lane per row.
+__global__ __launch_bounds__(kBlock) void sptrsv_level_kernel(SolveArgs a, int q0, int q1) {
     const int q = q0 + (int)(blockIdx.x * blockDim.x + threadIdx.x);
-    if (q < q1) solve_row<T, TR>(a, a.order[q]);
+    if (q >= q1) return;
+    const int32_t dlo = a.dptr[q], dhi = a.dptr[q + 1];
+    double acc = 0.;
+    for (int32_t at = dlo; at < dhi; ++at) acc += a.w.coef[at] * a.w.xs[a.dslot[at]];
+    double xi = a.w.rhs[q] - acc;
+    if (!a.unit) xi /= a.w.dg[q];
+    a.w.xs[q] = xi;
 }
 
-__global__ void round_kernel(int64_t n, const double *__restrict__ xw, float *__restrict__ x) {
+// x[order[q]] = xs[q], rounded once to the value type (cpp/sparse_csr_cpu.cpp:722).
+template <typename T>
+__global__ void unslot_kernel(int64_t n, const int32_t *__restrict__ order, const double *__restrict__ xs,
+                              T *__restrict__ x) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) x[i] = (float)xw[i];
-}
-
-template <typename T, bool TR>
-int run_solve(const nm_sptrsv_plan *p, SolveArgs<T> a, hipStream_t s) {
-    const int n = (int)p->launches.size();
-    for (int li = 0; li < n; ++li) {
-        const auto &L = p->launches[TR ? n - 1 - li : li];
-        if (L.wide) {
-            const unsigned grid = (unsigned)nm::ceil_div(L.q1 - L.q0, kBlock);
-            hipLaunchKernelGGL((sptrsv_level_kernel<T, TR>), dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
-            NM_LAUNCH_CHECK("sptrsv_level_kernel");
-        } else {
-            const int l0 = TR ? L.l1 - 1 : L.l0, l1 = TR ? L.l0 - 1 : L.l1, step = TR ? -1 : 1;
-            hipLaunchKernelGGL((sptrsv_batch_kernel<T, TR>), dim3(1), dim3(kNarrow), 0, s, a, l0, l1, step);
-            NM_LAUNCH_CHECK("sptrsv_batch_kernel");
-        }
-    }
-    return NM_OK;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += stride) x[order[q]] = (T)xs[q];
 }
 
 template <typename T>
-int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, const int64_t *indices,
-                const int64_t *indptr, int unit, const void *b, double *xw, hipStream_t s) {
-    SolveArgs<T> a;
-    a.data = (const T *)data;
-    a.indices = indices;
-    a.indptr = indptr;
-    a.t_indptr = p->t_indptr;
-    a.t_row = p->t_row;
-    a.t_perm = p->t_perm;
-    a.order = p->order;
+int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int unit, const void *b, void *x,
+                void *work, hipStream_t s) {
+    const Packed &P = p->dir[transposed ? 1 : 0];
+    SolveArgs a;
+    solve_work_layout(p->rows, p->nnz, work, &a.w);
     a.level_ptr = p->level_ptr;
-    a.b = (const T *)b;
-    a.xw = xw;
+    a.dptr = P.dptr;
+    a.dslot = P.dslot;
     a.unit = unit;
-    a.ascending = transposed ? !p->lower : p->lower;
-    return transposed ? run_solve<T, true>(p, a, s) : run_solve<T, false>(p, a, s);
+    {
+        int64_t m = p->nnz > p->rows ? p->nnz : p->rows;
+        int64_t grid = nm::ceil_div(m, kBlock);
+        if (grid > 65536) grid = 65536;
+        // with nnz == 0 nothing reads `data`: any valid pointer will do
+        const T *dat = p->nnz > 0 ? (const T *)data : (const T *)b;
+        hipLaunchKernelGGL(gather_values_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, p->rows, p->nnz, dat,
+                           (const T *)b, p->order, P.dptr, P.dsrc, P.diag, a.w.coef, a.w.dg, a.w.rhs);
+        NM_LAUNCH_CHECK("gather_values_kernel");
+    }
+    const int n = (int)p->launches.size();
+    for (int li = 0; li < n; ++li) {
+        const auto &L = p->launches[transposed ? n - 1 - li : li];
+        if (L.wide) {
+            const unsigned grid = (unsigned)nm::ceil_div(L.q1 - L.q0, kBlock);
+            hipLaunchKernelGGL(sptrsv_level_kernel, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
+            NM_LAUNCH_CHECK("sptrsv_level_kernel");
+        } else {
+            const int count = L.l1 - L.l0;
+            const int l0 = transposed ? L.l1 - 1 : L.l0, step = transposed ? -1 : 1;
+            // dependencies per row fetched ahead through registers: the smallest pipeline that
+            // holds this direction's longest row (longer rows take the slow path)
+            const int maxdep = p->max_deps[transposed ? 1 : 0];
+            if (maxdep <= 2)
+                hipLaunchKernelGGL(sptrsv_ring_kernel<2>, dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+            else if (maxdep <= 4)
+                hipLaunchKernelGGL(sptrsv_ring_kernel<4>, dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+            else
+                hipLaunchKernelGGL(sptrsv_ring_kernel<8>, dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+            NM_LAUNCH_CHECK("sptrsv_ring_kernel");
+        }
+    }
+    int64_t grid = nm::ceil_div(p->rows, kBlock);
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(unslot_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, p->rows, p->order, a.w.xs,
+                       (T *)x);
+    NM_LAUNCH_CHECK("unslot_kernel");
+    return NM_OK;
 }
 
 }  // namespace
@@ -235,8 +456,8 @@ extern "C" int nm_sptrsv_plan_bytes(int64_t rows, int64_t nnz, size_t *plan_byte
     NM_REQUIRE(rows >= 0 && nnz >= 0 && plan_bytes && work_bytes, "bad arguments");
     if (rows >= (int64_t(1) << 31) - 2 || nnz >= (int64_t(1) << 31) - 2)
         return nm::fail(NM_ERR_UNSUPPORTED, "sptrsv plans index rows and entries with 32 bits");
-    *plan_bytes = plan_layout(rows, nnz, nullptr, nullptr, nullptr, nullptr, nullptr);
-    *work_bytes = work_bytes_needed(rows, nnz);
+    *plan_bytes = plan_layout(rows, nnz, nullptr, nullptr);
+    *work_bytes = work_layout(rows, nnz, nullptr, nullptr);
     return NM_OK;
 }
 
@@ -259,49 +480,81 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     p->rows = rows;
     p->nnz = nnz;
     p->lower = lower ? 1 : 0;
-    nm::TPlan t;
-    int32_t *meta = nullptr;
-    plan_layout(rows, nnz, plan_mem, &t, &p->order, &p->level_ptr, &meta);
-    p->t_indptr = t.t_indptr;
-    p->t_row = t.t_row;
-    p->t_perm = t.t_perm;
+    Layout L;
+    plan_layout(rows, nnz, plan_mem, &L);
+    p->order = L.order;
+    p->level_ptr = L.level_ptr;
+    p->slot_of = L.slot_of;
+    p->dir[0] = L.dir[0];
+    p->dir[1] = L.dir[1];
 
     auto bail = [&](int rc) { delete p; return rc; };
     if (rows == 0) { *plan_out = p; return NM_OK; }
+    Scratch W;
+    work_layout(rows, nnz, work, &W);
 
-    char *wbase = static_cast<char *>(work);
-    int32_t *deg = reinterpret_cast<int32_t *>(wbase);
-    int32_t *rowid = reinterpret_cast<int32_t *>(wbase + align_up((size_t)(rows + 1) * 4));
-    char *twork = wbase + align_up((size_t)(rows + 1) * 4) + align_up((size_t)(nnz + 1) * 4);
-    const size_t twork_bytes = nm::tplan_work_bytes(rows, rows, nnz);
-
-    if (int rc = nm::tplan_build(rows, rows, nnz, indices, indptr, t, twork, twork_bytes, rowid, s)) return bail(rc);
-    if (int rc = nm::fill_async(deg, rows + 1, (int32_t)0, s)) return bail(rc);
+    if (int rc = nm::tplan_build(rows, rows, nnz, indices, indptr, L.t, W.twork, W.twork_bytes, W.rowid, s))
+        return bail(rc);
+    if (int rc = nm::fill_async(W.deg, rows + 1, (int32_t)0, s)) return bail(rc);
+    int64_t egrid = nm::ceil_div(nnz > 0 ? nnz : 1, kBlock), rgrid = nm::ceil_div(rows, kBlock);
+    if (egrid > 65536) egrid = 65536;
+    if (rgrid > 65536) rgrid = 65536;
     if (nnz > 0) {
-        int64_t grid = nm::ceil_div(nnz, kBlock);
-        if (grid > 65536) grid = 65536;
-        hipLaunchKernelGGL(indegree_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, indices, rowid,
-                           p->lower, deg);
+        hipLaunchKernelGGL(indegree_kernel, dim3((unsigned)egrid), dim3(kBlock), 0, s, nnz, indices, W.rowid,
+                           p->lower, W.deg);
         if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "indegree_kernel launch failed"));
     }
-    hipLaunchKernelGGL(kahn_kernel, dim3(1), dim3(kNarrow), 0, s, (int32_t)rows, p->lower, p->t_indptr, p->t_row,
-                       deg, p->order, p->level_ptr, meta);
+    if (int rc = nm::fill_async(L.meta, 16, (int32_t)0, s)) return bail(rc);
+    hipLaunchKernelGGL(kahn_kernel, dim3(1), dim3(kNarrow), 0, s, (int32_t)rows, p->lower, L.t.t_indptr, L.t.t_row,
+                       W.deg, p->order, p->level_ptr, L.meta);
     if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "kahn_kernel launch failed"));
+    hipLaunchKernelGGL(slot_of_kernel, dim3((unsigned)rgrid), dim3(kBlock), 0, s, rows, p->order, p->slot_of);
 
-    int32_t meta_h[2] = {0, 0};
-    if (hipMemcpyAsync(meta_h, meta, sizeof(meta_h), hipMemcpyDeviceToHost, s) != hipSuccess ||
+    // level-major packed triangles for both directions: count, scan, fill
+    for (int d = 0; d < 2; ++d) {
+        const int eff_lower = d == 0 ? p->lower : !p->lower;
+        const Packed &P = p->dir[d];
+        for (int fill = 0; fill < 2; ++fill) {
+            if (d == 0)
+                hipLaunchKernelGGL(pack_kernel<0>, dim3((unsigned)rgrid), dim3(kBlock), 0, s, rows, eff_lower, fill,
+                                   p->order, p->slot_of, indices, indptr, L.t.t_indptr, L.t.t_row, L.t.t_perm,
+                                   W.count64, P.dptr, P.dslot, P.dsrc, P.diag, L.meta + 2 + d);
+            else
+                hipLaunchKernelGGL(pack_kernel<1>, dim3((unsigned)rgrid), dim3(kBlock), 0, s, rows, eff_lower, fill,
+                                   p->order, p->slot_of, indices, indptr, L.t.t_indptr, L.t.t_row, L.t.t_perm,
+                                   W.count64, P.dptr, P.dslot, P.dsrc, P.diag, L.meta + 2 + d);
+            if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "pack_kernel launch failed"));
+            if (fill == 0) {
+                if (int rc = nm::fill_async(W.count64 + rows, 1, (int64_t)0, s)) return bail(rc);
+                if (int rc = nm::scan_exclusive_i64(W.count64, rows + 1, W.scan, s)) return bail(rc);
+                hipLaunchKernelGGL(narrow_kernel, dim3((unsigned)rgrid), dim3(kBlock), 0, s, rows + 1, W.count64,
+                                   P.dptr);
+            }
+        }
+    }
+
+    int32_t meta_h[4] = {0, 0, 0, 0};
+    if (hipMemcpyAsync(meta_h, L.meta, sizeof(meta_h), hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess)
         return bail(nm::fail(NM_ERR_HIP, "reading the level count back failed: %s",
                              hipGetErrorString(hipGetLastError())));
     if (meta_h[1] != (int32_t)rows)
         return bail(nm::fail(NM_ERR_INVALID, "level analysis placed %d of %lld rows", meta_h[1], (long long)rows));
     p->nlevels = meta_h[0];
+    p->max_deps[0] = meta_h[2];
+    p->max_deps[1] = meta_h[3];
     std::vector<int32_t> lp((size_t)p->nlevels + 1);
     if (hipMemcpyAsync(lp.data(), p->level_ptr, lp.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess)
         return bail(nm::fail(NM_ERR_HIP, "reading the level sizes back failed"));
 
-    // consecutive narrow levels share one single-workgroup launch
+    // consecutive narrow levels share one single-workgroup launch (at most kMaxLevels each)
+    auto push_narrow = [&](int32_t a0, int32_t a1) {
+        for (int32_t c0 = a0; c0 < a1; c0 += kMaxLevels) {
+            const int32_t c1 = c0 + kMaxLevels < a1 ? c0 + kMaxLevels : a1;
+            p->launches.push_back({c0, c1, lp[c0], lp[c1], false});
+        }
+    };
     int32_t run0 = -1;
     for (int32_t l = 0; l < p->nlevels; ++l) {
         const bool wide = lp[l + 1] - lp[l] > kNarrow;
@@ -309,10 +562,10 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             if (run0 < 0) run0 = l;
             continue;
         }
-        if (run0 >= 0) { p->launches.push_back({run0, l, lp[run0], lp[l], false}); run0 = -1; }
+        if (run0 >= 0) { push_narrow(run0, l); run0 = -1; }
         p->launches.push_back({l, l + 1, lp[l], lp[l + 1], true});
     }
-    if (run0 >= 0) p->launches.push_back({run0, p->nlevels, lp[run0], lp[p->nlevels], false});
+    if (run0 >= 0) push_narrow(run0, p->nlevels);
     *plan_out = p;
     return NM_OK;
 }
@@ -325,21 +578,23 @@ extern "C" int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan) {
 
 extern "C" void nm_sptrsv_plan_destroy(nm_sptrsv_plan *plan) { delete plan; }
 
+extern "C" int nm_sptrsv_solve_bytes(int64_t rows, int64_t nnz, size_t *bytes) {
+    NM_REQUIRE(rows >= 0 && nnz >= 0 && bytes, "bad arguments");
+    *bytes = solve_work_layout(rows, nnz, nullptr, nullptr);
+    return NM_OK;
+}
+
 extern "C" int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed, const void *data,
-                               const int64_t *indices, const int64_t *indptr, int unit, const void *b, void *x,
-                               double *xwork, nm_stream stream) {
+                               int unit, const void *b, void *x, void *work, size_t work_bytes,
+                               nm_stream stream) {
     NM_REQUIRE(plan != nullptr, "plan is null");
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
     if (plan->rows == 0) return NM_OK;
-    NM_REQUIRE(indptr && b && x && (plan->nnz == 0 || (data && indices)), "null pointer argument");
-    NM_REQUIRE(dt == NM_F64 || xwork != nullptr, "xwork is required for NM_F32");
+    NM_REQUIRE(b && x && work && (plan->nnz == 0 || data), "null pointer argument");
+    const size_t need = solve_work_layout(plan->rows, plan->nnz, nullptr, nullptr);
+    if (work_bytes < need)
+        return nm::fail(NM_ERR_WORKSPACE, "solve workspace of %zu bytes, %zu needed", work_bytes, need);
     hipStream_t s = nm::as_stream(stream);
-    if (dt == NM_F64)  // x itself holds the running solution
-        return solve_typed<double>(plan, transposed, data, indices, indptr, unit, b, (double *)x, s);
-    if (int rc = solve_typed<float>(plan, transposed, data, indices, indptr, unit, b, xwork, s)) return rc;
-    int64_t grid = nm::ceil_div(plan->rows, kBlock);
-    if (grid > 65536) grid = 65536;
-    hipLaunchKernelGGL(round_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, plan->rows, xwork, (float *)x);
-    NM_LAUNCH_CHECK("round_kernel");
-    return NM_OK;
+    if (dt == NM_F64) return solve_typed<double>(plan, transposed, data, unit, b, x, work, s);
+    return solve_typed<float>(plan, transposed, data, unit, b, x, work, s);
 }

@@ -329,11 +329,14 @@ def _plan_for(indices, indptr, rows, lower, dev):
 
 
 def _solve(plan, transposed, A_data, A_indices, A_indptr, unit, b, rows, dev):
+    L = _lib.lib()
     x = torch.empty(rows, dtype=A_data.dtype, device=dev)
-    xwork = None if A_data.dtype == torch.float64 else torch.empty(rows, dtype=torch.float64, device=dev)
-    _lib.check(_lib.lib().nm_sptrsv_solve(
-        plan.handle, _dt(A_data), int(transposed), _ptr(A_data), _ptr(A_indices), _ptr(A_indptr),
-        int(unit), _ptr(b), _ptr(x), _ptr(xwork), _stream(dev)), "nm_sptrsv_solve")
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(L.nm_sptrsv_solve_bytes(rows, A_data.shape[0], ctypes.byref(nbytes)), "nm_sptrsv_solve_bytes")
+    work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+    _lib.check(L.nm_sptrsv_solve(
+        plan.handle, _dt(A_data), int(transposed), _ptr(A_data), int(unit), _ptr(b), _ptr(x), _ptr(work),
+        nbytes.value, _stream(dev)), "nm_sptrsv_solve")
     return x
 
 
