@@ -23,84 +23,159 @@ using nm::kWave;
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 
+constexpr int kFwdWaves = 8;                 // wavefronts (= rows) per forward workgroup
+constexpr int kFwdBlock = kFwdWaves * kWave;
+constexpr int kSplitRow = 512;               // rows longer than this are shared by the workgroup's wavefronts
+
+// acc += sum over entries [kb, ke) of value * B[col, c], terms added in storage
+// order.  Entries are fetched 64 at a time (one coalesced load each for column
+// and value) and broadcast lane by lane; gathers of B go out eight (then four)
+// at a time so that a wavefront keeps several 256-byte requests in flight.
 // IDX is the structure's index type (int64 for A as delivered, int32 for the
 // transposed-structure plan); with PERM the value of entry k is data[perm[k]]
 // (A^T shares A's value array through the plan's permutation).
 template <typename T, typename IDX, bool PERM>
-__global__ __launch_bounds__(kBlock) void spdmm_fwd_kernel(
+__device__ __forceinline__ T row_times_dense(T acc, int64_t kb0, int64_t ke0, const T *__restrict__ data,
+                                             const IDX *__restrict__ indices, const int32_t *__restrict__ perm,
+                                             const T *__restrict__ Bc, int64_t ldb, int lane) {
+    for (int64_t kb = kb0; kb < ke0; kb += kWave) {
+        const int64_t k = kb + lane;
+        const int64_t mycol = k < ke0 ? (int64_t)indices[k] : 0;
+        const T myval = k < ke0 ? (PERM ? data[perm[k]] : data[k]) : T(0);
+        const int cnt = (int)(ke0 - kb < kWave ? ke0 - kb : kWave);
+        int j = 0;
+        for (; j + 8 <= cnt; j += 8) {
+            T bv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) bv[u] = Bc[__shfl(mycol, j + u, kWave) * ldb];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += __shfl(myval, j + u, kWave) * bv[u];
+        }
+        for (; j < cnt; j += 4) {
+            T bv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) bv[u] = Bc[__shfl(mycol, j + u < cnt ? j + u : j, kWave) * ldb];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (j + u < cnt) acc += __shfl(myval, j + u, kWave) * bv[u];
+        }
+    }
+    return acc;
+}
+
+// C = A B (or, on the plan, A^T B).  A workgroup of eight wavefronts owns eight
+// consecutive rows: one wavefront per row, lane = dense column.  A row longer
+// than kSplitRow is shared instead: every wavefront sums a contiguous eighth
+// of it and the partial sums are added in wavefront order (deterministic, but
+// not the serial order, so such rows match the CPU loop to rounding only).
+template <typename T, typename IDX, bool PERM>
+__global__ __launch_bounds__(kFwdBlock) void spdmm_fwd_kernel(
     int64_t rows, const T *__restrict__ data, const IDX *__restrict__ indices,
     const IDX *__restrict__ indptr, const int32_t *__restrict__ perm, const T *__restrict__ B, int64_t ldb,
     int64_t n, T *__restrict__ C, int64_t ldc) {
+    __shared__ T s_part[kFwdWaves][kWave];
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
-    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
-    for (int64_t row = wave0; row < rows; row += nwaves) {
-        const int64_t rb = indptr[row], re = indptr[row + 1];
+    const int wave = threadIdx.x / kWave;
+    const int64_t nblk = (rows + kFwdWaves - 1) / kFwdWaves;
+    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
+        const int64_t r0 = blk * kFwdWaves;
+        const int nr = (int)(rows - r0 < kFwdWaves ? rows - r0 : kFwdWaves);
         for (int64_t c0 = 0; c0 < n; c0 += kWave) {
             const int64_t c = c0 + lane;
             const bool live = c < n;
             const T *__restrict__ Bc = B + (live ? c : 0);
-            T acc = 0;
-            for (int64_t kb = rb; kb < re; kb += kWave) {
-                const int64_t k = kb + lane;
-                const int64_t mycol = k < re ? (int64_t)indices[k] : 0;
-                const T myval = k < re ? (PERM ? data[perm[k]] : data[k]) : T(0);
-                const int cnt = (int)(re - kb < kWave ? re - kb : kWave);
-                for (int j = 0; j < cnt; ++j) {
-                    const int64_t col = __shfl(mycol, j, kWave);
-                    const T v = __shfl(myval, j, kWave);
-                    const T bv = live ? Bc[col * ldb] : T(0);
-                    acc += v * bv;
+            if (wave < nr) {
+                const int64_t row = r0 + wave;
+                const int64_t rb = indptr[row], re = indptr[row + 1];
+                if (re - rb <= kSplitRow) {
+                    const T acc = row_times_dense<T, IDX, PERM>(T(0), rb, re, data, indices, perm, Bc, ldb, lane);
+                    if (live) C[row * ldc + c] = acc;
                 }
             }
-            if (live) C[row * ldc + c] = acc;
+            for (int t = 0; t < nr; ++t) {   // shared long rows (uniform over the workgroup)
+                const int64_t row = r0 + t;
+                const int64_t rb = indptr[row], re = indptr[row + 1];
+                if (re - rb <= kSplitRow) continue;
+                int64_t chunk = (re - rb + kFwdWaves - 1) / kFwdWaves;
+                chunk = (chunk + kWave - 1) / kWave * kWave;
+                const int64_t kb = rb + wave * chunk;
+                const int64_t ke = kb + chunk < re ? kb + chunk : re;
+                T acc = T(0);
+                if (kb < re) acc = row_times_dense<T, IDX, PERM>(acc, kb, ke, data, indices, perm, Bc, ldb, lane);
+                s_part[wave][lane] = acc;
+                __syncthreads();
+                if (wave == 0) {
+                    T sum = s_part[0][lane];
+                    for (int w = 1; w < kFwdWaves; ++w) sum += s_part[w][lane];
+                    if (live) C[row * ldc + c] = sum;
+                }
+                __syncthreads();
+            }
         }
     }
 }
 
+// grad_A[k] = <gC[row(k),:], B[col(k),:]> (SDDMM) and, when grad_B is given, the
+// atomic scatter grad_B[col,:] += data[k] * gC[row,:].  Entry-balanced: a
+// wavefront owns 64 consecutive stored entries whatever rows they belong to
+// (every entry costs the same), finds its first row by bisection and walks on;
+// gathers go out four at a time.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
-    int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
+    int64_t rows, int64_t nnz, const T *__restrict__ data, const int64_t *__restrict__ indices,
     const int64_t *__restrict__ indptr, const T *__restrict__ B, int64_t ldb,
     const T *__restrict__ gC, int64_t ldg, int64_t n, T *__restrict__ grad_A,
     T *__restrict__ grad_B, int64_t ldgb) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
     const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
-    for (int64_t row = wave0; row < rows; row += nwaves) {
-        const int64_t rb = indptr[row], re = indptr[row + 1];
-        if (rb == re) continue;
-        const T *__restrict__ g = gC + row * ldg;
-        const T g0 = lane < n ? g[lane] : T(0);  // the whole row of gC when n <= 64
-        for (int64_t kb = rb; kb < re; kb += kWave) {
-            const int64_t k = kb + lane;
-            const int64_t mycol = k < re ? indices[k] : 0;
-            const T myval = (grad_B && k < re) ? data[k] : T(0);
-            const int cnt = (int)(re - kb < kWave ? re - kb : kWave);
-            T mydot = 0;
-            for (int j = 0; j < cnt; ++j) {
-                const int64_t col = __shfl(mycol, j, kWave);
-                const T v = __shfl(myval, j, kWave);
-                T part = 0;
-                if (n <= kWave) {
-                    if (lane < n) {
-                        if (grad_A) part = g0 * B[col * ldb + lane];
-                        if (grad_B) nm::atomic_add(grad_B + col * ldgb + lane, v * g0);
-                    }
-                } else {
-                    for (int64_t c = lane; c < n; c += kWave) {
-                        const T gv = g[c];
-                        if (grad_A) part += gv * B[col * ldb + c];
-                        if (grad_B) nm::atomic_add(grad_B + col * ldgb + c, v * gv);
-                    }
+    const int64_t nchunks = (nnz + kWave - 1) / kWave;
+    for (int64_t ch = wave0; ch < nchunks; ch += nwaves) {
+        const int64_t kb = ch * kWave;
+        const int cnt = (int)(nnz - kb < kWave ? nnz - kb : kWave);
+        const int64_t k = kb + lane;
+        const int64_t mycol = lane < cnt ? indices[k] : 0;
+        const T myval = (grad_B && lane < cnt) ? data[k] : T(0);
+        // row of the chunk's first entry: last r with indptr[r] <= kb
+        int64_t lo = 0, hi = rows + 1;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (indptr[mid] <= kb) lo = mid + 1; else hi = mid;
+        }
+        int64_t row = lo - 1;
+        int64_t row_end = indptr[row + 1];
+        T mydot = 0;
+        for (int j0 = 0; j0 < cnt; j0 += 4) {
+            int64_t col[4], rw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = j0 + u < cnt ? j0 + u : cnt - 1;
+                while (kb + j >= row_end) { ++row; row_end = indptr[row + 1]; }
+                rw[u] = row;
+                col[u] = __shfl(mycol, j, kWave);
+            }
+            for (int64_t c0 = 0; c0 < n; c0 += kWave) {
+                const int64_t c = c0 + lane;
+                const bool live = c < n;
+                T bv[4], gv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    gv[u] = live ? gC[rw[u] * ldg + c] : T(0);
+                    bv[u] = (live && grad_A) ? B[col[u] * ldb + c] : T(0);
                 }
-                if (grad_A) {
-                    part = nm::wave_sum(part);
-                    if (lane == j) mydot = part;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (j0 + u >= cnt) break;
+                    const T av = __shfl(myval, j0 + u, kWave);   // all lanes take part in the broadcast
+                    if (grad_B && live) nm::atomic_add(grad_B + col[u] * ldgb + c, av * gv[u]);
+                    if (grad_A) {
+                        const T part = nm::wave_sum(gv[u] * bv[u]);
+                        if (lane == j0 + u) mydot += part;
+                    }
                 }
             }
-            if (grad_A && k < re) grad_A[k] = mydot;
         }
+        if (grad_A && lane < cnt) grad_A[k] = mydot;
     }
 }
 
@@ -113,8 +188,8 @@ int check_args(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void 
     return NM_OK;
 }
 
-inline unsigned wave_grid(int64_t rows) {
-    int64_t grid = nm::ceil_div(rows, kWavesPerBlock);
+inline unsigned wave_grid(int64_t units, int per_block) {
+    int64_t grid = nm::ceil_div(units, per_block);
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     return (unsigned)(grid < 1 ? 1 : grid);
 }
@@ -131,11 +206,11 @@ extern "C" int nm_spdmm_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t
                (long long)ldb, (long long)ldc, (long long)n);
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
-        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int64_t, false>), dim3(wave_grid(rows)), dim3(kBlock), 0, s,
+        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int64_t, false>), dim3(wave_grid(rows, kFwdWaves)), dim3(kFwdBlock), 0, s,
                            rows, (const float *)data, indices, indptr, nullptr, (const float *)B, ldb, n,
                            (float *)C, ldc);
     else
-        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int64_t, false>), dim3(wave_grid(rows)), dim3(kBlock), 0, s,
+        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int64_t, false>), dim3(wave_grid(rows, kFwdWaves)), dim3(kFwdBlock), 0, s,
                            rows, (const double *)data, indices, indptr, nullptr, (const double *)B, ldb, n,
                            (double *)C, ldc);
     NM_LAUNCH_CHECK("spdmm_fwd_kernel");
@@ -168,12 +243,12 @@ extern "C" int nm_spdmm_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_
     NM_REQUIRE(B != nullptr && gC != nullptr, "B or gC is null");
     NM_REQUIRE(ldb >= n && ldg >= n, "row stride smaller than the row");
     if (dt == NM_F32)
-        hipLaunchKernelGGL(spdmm_bwd_kernel<float>, dim3(wave_grid(rows)), dim3(kBlock), 0, s, rows,
-                           (const float *)data, indices, indptr, (const float *)B, ldb, (const float *)gC,
+        hipLaunchKernelGGL(spdmm_bwd_kernel<float>, dim3(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock)),
+                           dim3(kBlock), 0, s, rows, nnz, (const float *)data, indices, indptr, (const float *)B, ldb, (const float *)gC,
                            ldg, n, (float *)grad_A, (float *)grad_B, ldgb);
     else
-        hipLaunchKernelGGL(spdmm_bwd_kernel<double>, dim3(wave_grid(rows)), dim3(kBlock), 0, s, rows,
-                           (const double *)data, indices, indptr, (const double *)B, ldb, (const double *)gC,
+        hipLaunchKernelGGL(spdmm_bwd_kernel<double>, dim3(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock)),
+                           dim3(kBlock), 0, s, rows, nnz, (const double *)data, indices, indptr, (const double *)B, ldb, (const double *)gC,
                            ldg, n, (double *)grad_A, (double *)grad_B, ldgb);
     NM_LAUNCH_CHECK("spdmm_bwd_kernel");
     return NM_OK;
@@ -201,12 +276,13 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
     nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
-        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int32_t, true>), dim3(wave_grid(cols)), dim3(kBlock), 0, s, cols,
+        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int32_t, true>), dim3(wave_grid(cols, kFwdWaves)),
+                           dim3(kFwdBlock), 0, s, cols,
                            (const float *)data, t.t_row, t.t_indptr, t.t_perm, (const float *)gC, ldg, n,
                            (float *)grad_B, ldgb);
     else
-        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int32_t, true>), dim3(wave_grid(cols)), dim3(kBlock), 0, s,
-                           cols, (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg, n,
+        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int32_t, true>), dim3(wave_grid(cols, kFwdWaves)),
+                           dim3(kFwdBlock), 0, s, cols, (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg, n,
                            (double *)grad_B, ldgb);
     NM_LAUNCH_CHECK("spdmm_fwd_kernel (transposed)");
     return NM_OK;

@@ -76,13 +76,15 @@ def test_cfg3_spmm_fp32_powerlaw(dev):
     nz = int(p[sub])
     C_ref = oracle.spdmm_forward(sub, cols, d[:nz], i[:nz], p[:sub + 1], B)
     gA_ref, _ = oracle.spdmm_backward(sub, cols, d[:nz], i[:nz], p[:sub + 1], B, gC[:sub])
-    assert_same(C[:sub], C_ref, "C (first rows)")
+    short = lens[:sub] <= 512          # summed in storage order: bitwise; longer rows: to rounding
+    assert_same(C[:sub][short], C_ref[short], "C (first rows, short)")
+    assert_close(C[:sub], C_ref, "C (first rows)")
     assert_close(gA[:nz], gA_ref, "grad_A (first rows)")
     # the longest row, wherever it is
     r = int(np.argmax(lens))
     sl = slice(int(p[r]), int(p[r + 1]))
     one = np.array([0, lens[r]], dtype=np.int64)
-    assert_same(C[r:r + 1], oracle.spdmm_forward(1, cols, d[sl], i[sl], one, B), "C (longest row)")
+    assert_close(C[r:r + 1], oracle.spdmm_forward(1, cols, d[sl], i[sl], one, B), "C (longest row)")
     # grad_B = A^T gC against SciPy in double, all rows
     At = sps.csr_matrix((d.astype(np.float64), i, p), shape=(rows, cols)).T.tocsr()
     gB_ref = (At @ gC.astype(np.float64))

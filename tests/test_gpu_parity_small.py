@@ -70,10 +70,15 @@ def test_spmm_forward_backward(dev, dtype, n, backward_mode):
         D, I, P, Bd, gCd = to_dev(dev, d, i, p, B, gC)
         C = ext.spdmm_forward(rows, cols, D, I, P, Bd)
         gA, gB = ext.spdmm_backward(rows, cols, D, I, P, Bd, gCd)
-        assert_same(host(C), C_ref, f"{name} C")
+        # rows up to 512 entries are summed in storage order (bitwise); longer rows are shared
+        # by eight wavefronts and match to rounding
+        if int(np.diff(p).max(initial=0)) <= 512:
+            assert_same(host(C), C_ref, f"{name} C")
+        else:
+            assert_close(host(C), C_ref, f"{name} C")
         assert_close(host(gA), gA_ref, f"{name} grad_A")
         assert_close(host(gB), gB_ref, f"{name} grad_B")
-        if backward_mode == "planned":
+        if backward_mode == "planned" and int(np.bincount(i, minlength=1).max()) <= 512:
             assert_same(host(gB), gB_ref, f"{name} grad_B (bitwise)")
 
 
@@ -117,7 +122,7 @@ def test_spgemm_forward_backward(dev, dtype):
         gA, gB = ext.spgemm_backward(GC, Ci, Cp, ar, ac, AD, AI, AP, br, bc, BD, BI, BP)
         assert_same(host(gA), gA_ref, f"{name} grad_A")
         assert_close(host(gB), gB_ref, f"{name} grad_B")
-        if backward_mode == "planned":
+        if backward_mode == "planned" and int(np.bincount(i, minlength=1).max()) <= 512:
             assert_same(host(gB), gB_ref, f"{name} grad_B (bitwise)")
 
 
