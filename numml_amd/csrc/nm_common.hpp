@@ -67,12 +67,49 @@ inline hipStream_t as_stream(nm_stream s) { return reinterpret_cast<hipStream_t>
 
 // ---- device helpers -------------------------------------------------------
 
-// Sum over the 64 lanes of a wavefront; every lane gets the total.
+// Data-parallel-primitive move: every lane reads the lane selected by CTRL
+// (a DPP control word) without going through LDS; lanes in rows masked off by
+// ROW_MASK receive 0.
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ double dpp_move(double v) {
+    const long long bits = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)(bits & 0xffffffffll), CTRL, ROW_MASK, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(bits >> 32), CTRL, ROW_MASK, 0xf, false);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ int dpp_move(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+
+__device__ __forceinline__ float read_lane(float v, int l) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
+__device__ __forceinline__ double read_lane(double v, int l) {
+    const long long bits = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_readlane((int)(bits & 0xffffffffll), l);
+    const int hi = __builtin_amdgcn_readlane((int)(bits >> 32), l);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+__device__ __forceinline__ int read_lane(int v, int l) { return __builtin_amdgcn_readlane(v, l); }
+
+// Sum over the 64 lanes of a wavefront with DPP adds (no LDS traffic); every
+// lane gets the total.  Steps: swap within pairs, within quads, rotate the
+// 16-lane row by 4 and 8 (row totals everywhere), then carry lane 15 into rows
+// 1 and 3 and lane 31 into rows 2 and 3; lane 63 then holds the sum.
 template <typename T>
 __device__ __forceinline__ T wave_sum(T v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    v += dpp_move<0xB1>(v);         // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);         // quad_perm [2,3,0,1]
+    v += dpp_move<0x124>(v);        // row_ror 4
+    v += dpp_move<0x128>(v);        // row_ror 8
+    v += dpp_move<0x142, 0xa>(v);   // row_bcast 15 -> rows 1, 3
+    v += dpp_move<0x143, 0xc>(v);   // row_bcast 31 -> rows 2, 3
+    return read_lane(v, kWave - 1);
 }
 
 // Sum inside aligned groups of G consecutive lanes (G a power of two <= 64).

@@ -25,6 +25,7 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 
 constexpr int kFwdWaves = 8;                 // wavefronts (= rows) per forward workgroup
 constexpr int kFwdBlock = kFwdWaves * kWave;
+constexpr int kBatch = 8;                    // gathers a wavefront keeps in flight in the backward
 constexpr int kSplitRow = 512;               // rows longer than this are shared by the workgroup's wavefronts
 
 // acc += sum over entries [kb, ke) of value * B[col, c], terms added in storage
@@ -119,13 +120,13 @@ __global__ __launch_bounds__(kFwdBlock) void spdmm_fwd_kernel(
 // atomic scatter grad_B[col,:] += data[k] * gC[row,:].  Entry-balanced: a
 // wavefront owns 64 consecutive stored entries whatever rows they belong to
 // (every entry costs the same), finds its first row by bisection and walks on;
-// gathers go out four at a time.
+// gathers go out eight at a time and the dot products are reduced with DPP adds.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
     int64_t rows, int64_t nnz, const T *__restrict__ data, const int64_t *__restrict__ indices,
     const int64_t *__restrict__ indptr, const T *__restrict__ B, int64_t ldb,
     const T *__restrict__ gC, int64_t ldg, int64_t n, T *__restrict__ grad_A,
-    T *__restrict__ grad_B, int64_t ldgb) {
+    T *__restrict__ grad_B, int64_t ldgb, const int32_t *__restrict__ chunk_row) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
     const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
@@ -136,19 +137,24 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
         const int64_t k = kb + lane;
         const int64_t mycol = lane < cnt ? indices[k] : 0;
         const T myval = (grad_B && lane < cnt) ? data[k] : T(0);
-        // row of the chunk's first entry: last r with indptr[r] <= kb
-        int64_t lo = 0, hi = rows + 1;
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (indptr[mid] <= kb) lo = mid + 1; else hi = mid;
+        // row of the chunk's first entry: from the plan, else the last r with indptr[r] <= kb
+        int64_t row;
+        if (chunk_row) {
+            row = chunk_row[ch];
+        } else {
+            int64_t lo = 0, hi = rows + 1;
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) >> 1;
+                if (indptr[mid] <= kb) lo = mid + 1; else hi = mid;
+            }
+            row = lo - 1;
         }
-        int64_t row = lo - 1;
         int64_t row_end = indptr[row + 1];
         T mydot = 0;
-        for (int j0 = 0; j0 < cnt; j0 += 4) {
-            int64_t col[4], rw[4];
+        for (int j0 = 0; j0 < cnt; j0 += kBatch) {
+            int64_t col[kBatch], rw[kBatch];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kBatch; ++u) {
                 const int j = j0 + u < cnt ? j0 + u : cnt - 1;
                 while (kb + j >= row_end) { ++row; row_end = indptr[row + 1]; }
                 rw[u] = row;
@@ -157,14 +163,14 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
             for (int64_t c0 = 0; c0 < n; c0 += kWave) {
                 const int64_t c = c0 + lane;
                 const bool live = c < n;
-                T bv[4], gv[4];
+                T bv[kBatch], gv[kBatch];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < kBatch; ++u) {
                     gv[u] = live ? gC[rw[u] * ldg + c] : T(0);
                     bv[u] = (live && grad_A) ? B[col[u] * ldb + c] : T(0);
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < kBatch; ++u) {
                     if (j0 + u >= cnt) break;
                     const T av = __shfl(myval, j0 + u, kWave);   // all lanes take part in the broadcast
                     if (grad_B && live) nm::atomic_add(grad_B + col[u] * ldgb + c, av * gv[u]);
@@ -217,10 +223,10 @@ extern "C" int nm_spdmm_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t
     return NM_OK;
 }
 
-extern "C" int nm_spdmm_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
-                                 const int64_t *indices, const int64_t *indptr, const void *B, int64_t ldb,
-                                 const void *gC, int64_t ldg, int64_t n, void *grad_A, void *grad_B,
-                                 int64_t ldgb, nm_stream stream) {
+namespace {
+int backward_impl(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data, const int64_t *indices,
+                  const int64_t *indptr, const void *B, int64_t ldb, const void *gC, int64_t ldg, int64_t n,
+                  void *grad_A, void *grad_B, int64_t ldgb, const int32_t *chunk_row, nm_stream stream) {
     if (int rc = check_args(dt, rows, cols, nnz, data, indices, indptr, n)) return rc;
     hipStream_t s = nm::as_stream(stream);
     if (grad_B && cols > 0 && n > 0) {
@@ -245,13 +251,22 @@ extern "C" int nm_spdmm_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_
     if (dt == NM_F32)
         hipLaunchKernelGGL(spdmm_bwd_kernel<float>, dim3(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock)),
                            dim3(kBlock), 0, s, rows, nnz, (const float *)data, indices, indptr, (const float *)B, ldb, (const float *)gC,
-                           ldg, n, (float *)grad_A, (float *)grad_B, ldgb);
+                           ldg, n, (float *)grad_A, (float *)grad_B, ldgb, chunk_row);
     else
         hipLaunchKernelGGL(spdmm_bwd_kernel<double>, dim3(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock)),
                            dim3(kBlock), 0, s, rows, nnz, (const double *)data, indices, indptr, (const double *)B, ldb, (const double *)gC,
-                           ldg, n, (double *)grad_A, (double *)grad_B, ldgb);
+                           ldg, n, (double *)grad_A, (double *)grad_B, ldgb, chunk_row);
     NM_LAUNCH_CHECK("spdmm_bwd_kernel");
     return NM_OK;
+}
+}  // namespace
+
+extern "C" int nm_spdmm_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                 const int64_t *indices, const int64_t *indptr, const void *B, int64_t ldb,
+                                 const void *gC, int64_t ldg, int64_t n, void *grad_A, void *grad_B,
+                                 int64_t ldgb, nm_stream stream) {
+    return backward_impl(dt, rows, cols, nnz, data, indices, indptr, B, ldb, gC, ldg, n, grad_A, grad_B, ldgb,
+                         nullptr, stream);
 }
 
 // Backward over the transposed-structure plan: grad_A by the row-major kernel
@@ -264,16 +279,16 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
                                          void *grad_A, void *grad_B, int64_t ldgb, nm_stream stream) {
     if (int rc = check_args(dt, rows, cols, nnz, data, indices, indptr, n)) return rc;
     NM_REQUIRE(plan_mem != nullptr, "plan is null");
+    nm::TPlan t;
+    nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
     if (grad_A) {
-        if (int rc = nm_spdmm_backward(dt, rows, cols, nnz, data, indices, indptr, B, ldb, gC, ldg, n, grad_A,
-                                       nullptr, 0, stream))
+        if (int rc = backward_impl(dt, rows, cols, nnz, data, indices, indptr, B, ldb, gC, ldg, n, grad_A, nullptr, 0,
+                                   t.chunk_row, stream))
             return rc;
     }
     if (!grad_B || cols == 0 || n == 0) return NM_OK;
     NM_REQUIRE(ldgb >= n && ldg >= n, "row stride smaller than the row");
     NM_REQUIRE(gC != nullptr || nnz == 0, "gC is null");
-    nm::TPlan t;
-    nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
         hipLaunchKernelGGL((spdmm_fwd_kernel<float, int32_t, true>), dim3(wave_grid(cols, kFwdWaves)),

@@ -41,10 +41,12 @@ __global__ void entry_keys_kernel(int64_t nnz, int64_t rows, const int64_t *__re
 
 __global__ void finish_kernel(int64_t nnz, int64_t cols, const int32_t *__restrict__ keys_sorted,
                               const int32_t *__restrict__ t_perm, const int32_t *__restrict__ rowid,
-                              int32_t *__restrict__ t_row, int32_t *__restrict__ t_indptr) {
+                              int32_t *__restrict__ t_row, int32_t *__restrict__ t_indptr,
+                              int32_t *__restrict__ chunk_row) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     for (int64_t p = tid; p < nnz; p += stride) t_row[p] = rowid[t_perm[p]];
+    for (int64_t h = tid; h * 64 < nnz; h += stride) chunk_row[h] = rowid[h * 64];
     for (int64_t c = tid; c <= cols; c += stride) {
         int64_t lo = 0, hi = nnz;  // first sorted position whose column is >= c
         while (lo < hi) {
@@ -132,7 +134,7 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
     int64_t grid = ceil_div(m, kBlock);
     if (grid > 65536) grid = 65536;
     hipLaunchKernelGGL(finish_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, cols, w.keys_sorted,
-                       plan.t_perm, rowid, plan.t_row, plan.t_indptr);
+                       plan.t_perm, rowid, plan.t_row, plan.t_indptr, plan.chunk_row);
     NM_LAUNCH_CHECK("transpose finish_kernel");
     hipLaunchKernelGGL(symmetry_init_kernel, dim3(1), dim3(64), 0, s, plan.flags, rows == cols ? 1 : 0);
     if (rows == cols) {

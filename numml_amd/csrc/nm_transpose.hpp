@@ -5,6 +5,8 @@
 //   t_indptr[c]  first entry of column c in the column-major order   (cols + 1)
 //   t_row[p]     row of the p-th entry in column-major order         (nnz)
 //   t_perm[p]    its position in A's row-major arrays                 (nnz)
+//   chunk_row[h] row of entry 64*h of A's ROW-major arrays (entry-balanced kernels
+//                start their walk there instead of bisecting indptr)  (ceil(nnz/64)+1)
 //   flags[0]     1 when the pattern is symmetric (A^T has A's structure, so
 //                entry p of column c is the mirror image of the row-major entry p)
 //
@@ -21,6 +23,7 @@ struct TPlan {
     int32_t *t_indptr;
     int32_t *t_row;
     int32_t *t_perm;
+    int32_t *chunk_row;
     int32_t *flags;
 };
 
@@ -37,8 +40,9 @@ inline size_t tplan_layout(int64_t cols, int64_t nnz, void *base, TPlan *p) {
     int32_t *a = (int32_t *)take((size_t)(cols + 1) * 4);
     int32_t *b = (int32_t *)take((size_t)(nnz + 1) * 4);
     int32_t *c = (int32_t *)take((size_t)(nnz + 1) * 4);
+    int32_t *h = (int32_t *)take((size_t)((nnz + 63) / 64 + 1) * 4);
     int32_t *f = (int32_t *)take(16 * 4);
-    if (p) *p = TPlan{a, b, c, f};
+    if (p) *p = TPlan{a, b, c, h, f};
     return off;
 }
 
