@@ -16,10 +16,11 @@
 // Rows too long for an LDS table spill to a dense accumulator in global memory
 // (one slice of B_cols entries per spill workgroup).
 //
-// Backward: one lane per stored entry (i,k) of A walks row k of B, finds each
-// column in row i of C by bisection, and forms grad_A (a sum in ascending
-// column order, as the reference's merge, cpp/sparse_csr_cpu.cpp:246-278) and
-// grad_B (atomic adds) in one pass.
+// Backward: eight lanes per row i of A; for each entry (i,k) the lanes share row
+// k of B, find its columns in row i of C (staged in LDS) by bisection, and form
+// grad_A (a sum in ascending column order, as the reference's merge,
+// cpp/sparse_csr_cpu.cpp:246-278) and grad_B (atomic adds, one cache line per
+// entry of A) in one pass.
 //
 // Algorithmic HBM bytes of the forward (s = sizeof(value)):
 //   nnzA*(s+8) + rowsA*8 + products*(s+8) [upper; nnzB*(s+8) compulsory]
@@ -391,42 +392,97 @@ __global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
 
 // ---- backward --------------------------------------------------------------------
 
+// Backward.  A group of 8 lanes owns one row i of A.  Row i of C (column
+// indices and upstream gradient) is staged in LDS when it has at most
+// kBwdStage entries, so the per-product lookups are LDS bisections; longer
+// rows are searched in global memory.  The group takes the row's entries
+// (i,k) one at a time and spreads row k of B over its lanes, so the eight
+// atomic updates of grad_B it issues land in one cache line (the L2 atomic
+// units are bound by lines touched, not by lanes).  The products
+// gC[i,c] * B[k,c] are then added lane by lane in ascending column order --
+// the order of the reference's merge -- which keeps grad_A bit-identical.
+constexpr int kBwdG = 8;
+constexpr int kBwdStage = 64;
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
-    int64_t A_rows, int64_t A_nnz, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
+    int64_t A_rows, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
     const int64_t *__restrict__ C_indptr, const T *__restrict__ A_data,
     const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
     const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
     const int64_t *__restrict__ B_indptr, T *__restrict__ grad_A, T *__restrict__ grad_B) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t ai = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ai < A_nnz; ai += stride) {
-        int64_t lo = 0, hi = A_rows + 1;  // first p with A_indptr[p] > ai
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (A_indptr[mid] <= ai) lo = mid + 1; else hi = mid;
-        }
-        const int64_t i = lo - 1;
-        const int64_t k = A_indices[ai];
-        const T a = grad_B ? A_data[ai] : T(0);
-        const int64_t cb = C_indptr[i], ce = C_indptr[i + 1];
-        const int64_t be = B_indptr[k + 1];
-        T acc = 0;
-        int64_t from = cb;  // both rows ascend, so each search starts where the last one ended
-        for (int64_t kk = B_indptr[k]; kk < be; ++kk) {
-            const int64_t c = B_indices[kk];
-            int64_t l = from, h = ce;
-            while (l < h) {
-                const int64_t mid = (l + h) >> 1;
-                if (C_indices[mid] < c) l = mid + 1; else h = mid;
+    constexpr int G = kBwdG, GPB = kBlock / G;
+    __shared__ int32_t s_ci[GPB * kBwdStage];
+    __shared__ T s_g[GPB * kBwdStage];
+    const int gl = threadIdx.x % G, gi = threadIdx.x / G;
+    const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);   // first lane of the group inside its wavefront
+    int32_t *ci = s_ci + gi * kBwdStage;
+    T *cg = s_g + gi * kBwdStage;
+    for (int64_t i0 = (int64_t)blockIdx.x * GPB; i0 < A_rows; i0 += (int64_t)gridDim.x * GPB) {
+        const int64_t i = i0 + gi;
+        const bool live = i < A_rows;
+        const int64_t cb = live ? C_indptr[i] : 0, ce = live ? C_indptr[i + 1] : 0;
+        const int clen = (int)(ce - cb < 0x7fffffff ? ce - cb : 0x7fffffff);
+        const bool staged = clen <= kBwdStage;
+        if (staged)
+            for (int t = gl; t < clen; t += G) {
+                ci[t] = (int32_t)C_indices[cb + t];
+                cg[t] = gC[cb + t];
             }
-            from = l;
-            if (l < ce && C_indices[l] == c) {
-                const T g = gC[l];
-                acc += g * B_data[kk];
-                if (grad_B) nm::atomic_add(grad_B + kk, a * g);
+        group_sync<G>();
+        const int64_t ab = live ? A_indptr[i] : 0, ae = live ? A_indptr[i + 1] : 0;
+        for (int64_t a0 = ab; a0 < ae; a0 += G) {
+            // each lane fetches one entry of A's row and the bounds of the B row it names
+            const int64_t my_ai = a0 + gl;
+            const bool mine = my_ai < ae;
+            const int64_t my_k = mine ? A_indices[my_ai] : 0;
+            const T my_a = (mine && grad_B) ? A_data[my_ai] : T(0);
+            const int64_t my_bb = mine ? B_indptr[my_k] : 0, my_be = mine ? B_indptr[my_k + 1] : 0;
+            const int nb = (int)(ae - a0 < G ? ae - a0 : G);
+            T my_acc = 0;
+            for (int e = 0; e < nb; ++e) {
+                const int64_t bb = __shfl(my_bb, gbase + e, kWave), be = __shfl(my_be, gbase + e, kWave);
+                const T a = __shfl(my_a, gbase + e, kWave);
+                T acc = 0;
+                for (int64_t kk0 = bb; kk0 < be; kk0 += G) {
+                    const int64_t kk = kk0 + gl;
+                    const bool have = kk < be;
+                    const int64_t c = have ? B_indices[kk] : -1;
+                    const T bval = have ? B_data[kk] : T(0);
+                    bool hit = false;
+                    T g = 0;
+                    if (staged) {
+                        int l = 0, h = clen;
+                        while (l < h) {
+                            const int mid = (l + h) >> 1;
+                            if ((int64_t)ci[mid] < c) l = mid + 1; else h = mid;
+                        }
+                        hit = have && l < clen && (int64_t)ci[l] == c;
+                        if (hit) g = cg[l];
+                    } else {
+                        int64_t l = cb, h = ce;
+                        while (l < h) {
+                            const int64_t mid = (l + h) >> 1;
+                            if (C_indices[mid] < c) l = mid + 1; else h = mid;
+                        }
+                        hit = have && l < ce && C_indices[l] == c;
+                        if (hit) g = gC[l];
+                    }
+                    if (hit && grad_B) nm::atomic_add(grad_B + kk, a * g);
+                    const T prod = g * bval;
+                    // ordered sum over the group's lanes = ascending column
+                    const int cnt = (int)(be - kk0 < G ? be - kk0 : G);
+                    for (int l2 = 0; l2 < cnt; ++l2) {
+                        const T pl = __shfl(prod, gbase + l2, kWave);
+                        const int hl = __shfl((int)hit, gbase + l2, kWave);
+                        if (hl) acc += pl;
+                    }
+                }
+                if (gl == e) my_acc = acc;
             }
+            if (mine && grad_A) grad_A[my_ai] = my_acc;
         }
-        if (grad_A) grad_A[ai] = acc;
+        group_sync<G>();
     }
 }
 
@@ -563,14 +619,14 @@ extern "C" int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, in
     }
     if (A_nnz == 0 || A_rows == 0 || (!grad_A && !grad_B)) return NM_OK;
     NM_REQUIRE(C_indptr && A_indices && A_indptr && B_indptr && A_data, "null pointer argument");
-    int64_t grid = nm::ceil_div(A_nnz, kBlock);
+    int64_t grid = nm::ceil_div(A_rows, kBlock / kBwdG);
     if (grid > 1 << 20) grid = 1 << 20;
     if (dt == NM_F32)
-        hipLaunchKernelGGL(spgemm_bwd_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_nnz,
+        hipLaunchKernelGGL(spgemm_bwd_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            (const float *)gC, C_indices, C_indptr, (const float *)A_data, A_indices, A_indptr,
                            (const float *)B_data, B_indices, B_indptr, (float *)grad_A, (float *)grad_B);
     else
-        hipLaunchKernelGGL(spgemm_bwd_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_nnz,
+        hipLaunchKernelGGL(spgemm_bwd_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            (const double *)gC, C_indices, C_indptr, (const double *)A_data, A_indices, A_indptr,
                            (const double *)B_data, B_indices, B_indptr, (double *)grad_A, (double *)grad_B);
     NM_LAUNCH_CHECK("spgemm_bwd_kernel");
