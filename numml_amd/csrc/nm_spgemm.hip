@@ -37,6 +37,8 @@ constexpr int kBlock = 256;
 constexpr int kBins = 4;
 constexpr int kSpillGroups = 8;     // workgroups (and dense slices) of the spill path
 constexpr int kSpillBlock = 1024;
+constexpr int kTablePad = 4;         // entries between the hash tables of neighbouring groups (16 bytes)
+constexpr int kAhead = 8;            // B rows whose first columns a group requests before inserting any
 
 // bin upper limits (inclusive); the last bin takes the rest and spills
 constexpr int32_t kSymLimit[3] = {64, 512, 8192};     // on the product bound
@@ -126,14 +128,25 @@ __global__ void bin_clear_kernel(int32_t *bins) {
     if (threadIdx.x < 16) bins[threadIdx.x] = 0;
 }
 
-__global__ void bin_count_kernel(int64_t rows, const int32_t *__restrict__ key, int32_t l0, int32_t l1,
-                                 int32_t l2, int32_t *bins) {
+// Rows per bin.  Each wavefront counts with ballots (one population count per
+// bin) instead of 64 colliding LDS atomics.
+__global__ __launch_bounds__(kBlock) void bin_count_kernel(int64_t rows, const int32_t *__restrict__ key,
+                                                           int32_t l0, int32_t l1, int32_t l2, int32_t *bins) {
     __shared__ int s_cnt[kBins];
     if (threadIdx.x < kBins) s_cnt[threadIdx.x] = 0;
     __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1);
+    int mine[kBins] = {0, 0, 0, 0};
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows; i += stride)
-        atomicAdd(&s_cnt[bin_of(key[i], l0, l1, l2)], 1);
+    for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x; i0 < rows; i0 += stride) {
+        const int64_t i = i0 + threadIdx.x;
+        const int b = i < rows ? bin_of(key[i], l0, l1, l2) : -1;
+#pragma unroll
+        for (int q = 0; q < kBins; ++q) mine[q] += __popcll(__ballot(b == q));
+    }
+    if (lane == 0)
+        for (int q = 0; q < kBins; ++q)
+            if (mine[q]) atomicAdd(&s_cnt[q], mine[q]);
     __syncthreads();
     if (threadIdx.x < kBins && s_cnt[threadIdx.x]) atomicAdd(bins + threadIdx.x, s_cnt[threadIdx.x]);
 }
@@ -150,26 +163,39 @@ __global__ void bin_offsets_kernel(int32_t *bins) {
     }
 }
 
-// Rows are placed a workgroup at a time so that each bin keeps them in
-// near-ascending order (neighbouring rows share B rows and C lines).
-__global__ void bin_scatter_kernel(int64_t rows, const int32_t *__restrict__ key, int32_t l0, int32_t l1,
-                                   int32_t l2, int32_t *bins, int32_t *__restrict__ perm) {
-    __shared__ int s_cnt[kBins];
+// Rows are placed a workgroup at a time, wavefront by wavefront and lane by lane,
+// so that each bin keeps them in ascending order inside a workgroup's slice
+// (neighbouring rows share B rows and C lines).
+__global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const int32_t *__restrict__ key,
+                                                             int32_t l0, int32_t l1, int32_t l2, int32_t *bins,
+                                                             int32_t *__restrict__ perm) {
+    constexpr int kWaves = kBlock / kWave;
+    __shared__ int s_wave[kWaves][kBins];   // rows of bin q in wavefront w
     __shared__ int s_base[kBins];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x; i0 < rows; i0 += stride) {
-        if (threadIdx.x < kBins) s_cnt[threadIdx.x] = 0;
-        __syncthreads();
         const int64_t i = i0 + threadIdx.x;
-        int b = 0, slot = 0;
-        if (i < rows) {
-            b = bin_of(key[i], l0, l1, l2);
-            slot = atomicAdd(&s_cnt[b], 1);
+        const int b = i < rows ? bin_of(key[i], l0, l1, l2) : -1;
+        int before = 0;   // rows of my bin in lower lanes of my wavefront
+#pragma unroll
+        for (int q = 0; q < kBins; ++q) {
+            const unsigned long long m = __ballot(b == q);
+            if (b == q) before = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) s_wave[wave][q] = __popcll(m);
         }
         __syncthreads();
-        if (threadIdx.x < kBins) s_base[threadIdx.x] = atomicAdd(bins + 9 + threadIdx.x, s_cnt[threadIdx.x]);
+        if (threadIdx.x < kBins) {
+            int total = 0;
+            for (int w = 0; w < kWaves; ++w) total += s_wave[w][threadIdx.x];
+            s_base[threadIdx.x] = total ? atomicAdd(bins + 9 + threadIdx.x, total) : 0;
+        }
         __syncthreads();
-        if (i < rows) perm[s_base[b] + slot] = (int32_t)i;
+        if (b >= 0) {
+            int off = s_base[b] + before;
+            for (int w = 0; w < wave; ++w) off += s_wave[w][b];
+            perm[off] = (int32_t)i;
+        }
         __syncthreads();
     }
 }
@@ -197,10 +223,13 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
     const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
     int64_t *__restrict__ C_count) {
     constexpr int GPB = kBlock / G;
-    __shared__ int32_t s_keys[GPB * TABLE];
+    // the tables of the groups that share a wavefront start kTablePad entries apart in
+    // bank space; without the pad they would all map slot t to the same LDS bank
+    constexpr int STRIDE = TABLE + (GPB > 1 ? kTablePad : 0);
+    __shared__ __align__(16) int32_t s_keys[GPB * STRIDE];
     __shared__ int s_red[kBlock / kWave];
     const int gl = threadIdx.x % G, gi = threadIdx.x / G;
-    int32_t *tab = s_keys + gi * TABLE;
+    int32_t *tab = s_keys + gi * STRIDE;
     const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
     for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
         const int32_t idx = idx0 + gi;
@@ -209,22 +238,54 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
         group_sync<G>();
         int cnt = 0;
         int64_t row = 0;
-        if (live) {
+        auto insert = [&](int32_t key) {
+            uint32_t h = hash32(key) & (TABLE - 1);
+            for (;;) {
+                const int32_t old = atomicCAS(&tab[h], kEmpty, key);
+                if (old == kEmpty) { ++cnt; break; }
+                if (old == key) break;
+                h = (h + 1) & (TABLE - 1);
+            }
+        };
+        if (G <= kWave) {
+            // Latency-lean walk: each lane fetches one entry of A's row together with the
+            // bounds of the B row it names; the first G columns of up to kAhead B rows are
+            // then requested back to back before any of them is inserted.
+            const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
+            row = live ? perm[idx] : 0;
+            const int64_t ab = live ? A_indptr[row] : 0, ae = live ? A_indptr[row + 1] : 0;
+            for (int64_t a0 = ab; a0 < ae; a0 += G) {
+                const int64_t my_ai = a0 + gl;
+                const bool mine = my_ai < ae;
+                const int64_t my_j = mine ? A_indices[my_ai] : 0;
+                const int64_t my_bb = mine ? B_indptr[my_j] : 0, my_be = mine ? B_indptr[my_j + 1] : 0;
+                const int nb = (int)(ae - a0 < G ? ae - a0 : G);
+                for (int e0 = 0; e0 < nb; e0 += kAhead) {
+                    int32_t pk[kAhead];
+                    int64_t bbs[kAhead], bes[kAhead];
+#pragma unroll
+                    for (int u = 0; u < kAhead; ++u) {
+                        const int src = gbase + (e0 + u < nb ? e0 + u : e0);
+                        bbs[u] = __shfl(my_bb, src, kWave);
+                        bes[u] = __shfl(my_be, src, kWave);
+                        const int64_t kk = bbs[u] + gl;
+                        pk[u] = (e0 + u < nb && kk < bes[u]) ? (int32_t)B_indices[kk] : kEmpty;
+                    }
+#pragma unroll
+                    for (int u = 0; u < kAhead; ++u) {
+                        if (e0 + u >= nb) break;
+                        if (pk[u] != kEmpty) insert(pk[u]);
+                        for (int64_t kk = bbs[u] + G + gl; kk < bes[u]; kk += G) insert((int32_t)B_indices[kk]);
+                    }
+                }
+            }
+        } else if (live) {
             row = perm[idx];
             const int64_t je = A_indptr[row + 1];
             for (int64_t jj = A_indptr[row]; jj < je; ++jj) {
                 const int64_t j = A_indices[jj];
                 const int64_t ke = B_indptr[j + 1];
-                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) {
-                    const int32_t key = (int32_t)B_indices[kk];
-                    uint32_t h = hash32(key) & (TABLE - 1);
-                    for (;;) {
-                        const int32_t old = atomicCAS(&tab[h], kEmpty, key);
-                        if (old == kEmpty) { ++cnt; break; }
-                        if (old == key) break;
-                        h = (h + 1) & (TABLE - 1);
-                    }
-                }
+                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) insert((int32_t)B_indices[kk]);
             }
         }
         cnt = group_total<G>(cnt, s_red);
@@ -279,12 +340,13 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
     const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
     const int64_t *__restrict__ C_indptr, int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
     constexpr int GPB = kBlock / G;
+    constexpr int STRIDE = TABLE + (GPB > 1 ? kTablePad : 0);   // see symbolic_hash_kernel
     extern __shared__ __align__(16) unsigned char s_raw[];
     T *s_vals = reinterpret_cast<T *>(s_raw);
-    int32_t *s_keys = reinterpret_cast<int32_t *>(s_raw + sizeof(T) * GPB * TABLE);
+    int32_t *s_keys = reinterpret_cast<int32_t *>(s_raw + sizeof(T) * GPB * STRIDE);
     const int gl = threadIdx.x % G, gi = threadIdx.x / G;
-    int32_t *tab = s_keys + gi * TABLE;
-    T *val = s_vals + gi * TABLE;
+    int32_t *tab = s_keys + gi * STRIDE;
+    T *val = s_vals + gi * STRIDE;
     const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
     for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
         const int32_t idx = idx0 + gi;
@@ -292,25 +354,63 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
         for (int t = gl; t < TABLE; t += G) { tab[t] = kEmpty; val[t] = T(0); }
         group_sync<G>();
         int64_t row = 0;
-        if (live) {
+        auto add = [&](int32_t key, T prod) {
+            uint32_t h = hash32(key) & (TABLE - 1);
+            for (;;) {
+                const int32_t old = atomicCAS(&tab[h], kEmpty, key);
+                if (old == kEmpty || old == key) break;
+                h = (h + 1) & (TABLE - 1);
+            }
+            // the columns of one B row are distinct, so no other lane holds slot h now
+            val[h] = val[h] + prod;
+        };
+        if (G <= kWave) {
+            // Same latency-lean walk as the symbolic phase; entries of A's row are still
+            // applied one after the other, so every output entry gets its products in
+            // the order of A's row.
+            const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
+            row = live ? perm[idx] : 0;
+            const int64_t ab = live ? A_indptr[row] : 0, ae = live ? A_indptr[row + 1] : 0;
+            for (int64_t a0 = ab; a0 < ae; a0 += G) {
+                const int64_t my_ai = a0 + gl;
+                const bool mine = my_ai < ae;
+                const int64_t my_j = mine ? A_indices[my_ai] : 0;
+                const T my_a = mine ? A_data[my_ai] : T(0);
+                const int64_t my_bb = mine ? B_indptr[my_j] : 0, my_be = mine ? B_indptr[my_j + 1] : 0;
+                const int nb = (int)(ae - a0 < G ? ae - a0 : G);
+                for (int e0 = 0; e0 < nb; e0 += kAhead) {
+                    int32_t pk[kAhead];
+                    T pv[kAhead], as[kAhead];
+                    int64_t bbs[kAhead], bes[kAhead];
+#pragma unroll
+                    for (int u = 0; u < kAhead; ++u) {
+                        const int src = gbase + (e0 + u < nb ? e0 + u : e0);
+                        bbs[u] = __shfl(my_bb, src, kWave);
+                        bes[u] = __shfl(my_be, src, kWave);
+                        as[u] = __shfl(my_a, src, kWave);
+                        const int64_t kk = bbs[u] + gl;
+                        const bool ok = e0 + u < nb && kk < bes[u];
+                        pk[u] = ok ? (int32_t)B_indices[kk] : kEmpty;
+                        pv[u] = ok ? B_data[kk] : T(0);
+                    }
+#pragma unroll
+                    for (int u = 0; u < kAhead; ++u) {
+                        if (e0 + u >= nb) break;
+                        if (pk[u] != kEmpty) add(pk[u], as[u] * pv[u]);
+                        for (int64_t kk = bbs[u] + G + gl; kk < bes[u]; kk += G)
+                            add((int32_t)B_indices[kk], as[u] * B_data[kk]);
+                        group_sync<G>();  // the next entry of A's row adds after this one
+                    }
+                }
+            }
+        } else if (live) {
             row = perm[idx];
             const int64_t je = A_indptr[row + 1];
             for (int64_t jj = A_indptr[row]; jj < je; ++jj) {
                 const int64_t j = A_indices[jj];
                 const T a = A_data[jj];
                 const int64_t ke = B_indptr[j + 1];
-                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) {
-                    const int32_t key = (int32_t)B_indices[kk];
-                    const T prod = a * B_data[kk];
-                    uint32_t h = hash32(key) & (TABLE - 1);
-                    for (;;) {
-                        const int32_t old = atomicCAS(&tab[h], kEmpty, key);
-                        if (old == kEmpty || old == key) break;
-                        h = (h + 1) & (TABLE - 1);
-                    }
-                    // the columns of one B row are distinct, so no other lane holds slot h now
-                    val[h] = val[h] + prod;
-                }
+                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) add((int32_t)B_indices[kk], a * B_data[kk]);
                 group_sync<G>();  // the next entry of A's row adds after this one
             }
         }
@@ -320,8 +420,15 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
             for (int t = gl; t < TABLE; t += G) {
                 const int32_t key = tab[t];
                 if (key == kEmpty) continue;
+                // rank = number of stored columns below this one; empty slots (0xffffffff) never
+                // count.  Four keys per LDS read.
                 int rank = 0;
-                for (int u = 0; u < TABLE; ++u) rank += (uint32_t)tab[u] < (uint32_t)key;
+                const uint4 *tab4 = reinterpret_cast<const uint4 *>(tab);
+                for (int u = 0; u < TABLE / 4; ++u) {
+                    const uint4 q = tab4[u];
+                    rank += (q.x < (uint32_t)key) + (q.y < (uint32_t)key) + (q.z < (uint32_t)key) +
+                            (q.w < (uint32_t)key);
+                }
                 C_indices[base + rank] = key;
                 C_data[base + rank] = val[t];
             }
@@ -505,13 +612,13 @@ int launch_numeric(const Work &w, int64_t B_cols, const void *A_data, const int6
     constexpr size_t per = sizeof(T) + sizeof(int32_t);
     {
         auto k = numeric_hash_kernel<T, 8, kNumTable0>;
-        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 8) * kNumTable0, s, 0, w.bins,
+        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 8) * (kNumTable0 + kTablePad), s, 0, w.bins,
                            w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
         NM_LAUNCH_CHECK("numeric_hash_kernel<8>");
     }
     {
         auto k = numeric_hash_kernel<T, 64, kNumTable1>;
-        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 64) * kNumTable1, s, 1, w.bins,
+        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 64) * (kNumTable1 + kTablePad), s, 1, w.bins,
                            w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
         NM_LAUNCH_CHECK("numeric_hash_kernel<64>");
     }
