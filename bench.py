@@ -16,6 +16,7 @@ on):
   spmm    fp32 SpMM fwd+bwd, power-law 1M x 1M, ~15M nnz, 64 dense columns
   spgemm  fp64 hash SpGEMM A@A fwd+bwd, 3-D Laplacian 128^3
   sptrsv  fp64 triangular solve fwd+bwd, tril(Poisson 1024^2), 2047 levels
+  copy    256 MiB device copy (counter calibration / practical bandwidth ceiling)
 
 ``value`` is algorithmic bytes per step / time per step (GB/s) for spmv/spmm,
 GFLOP/s (2 flop per scalar product, forward only counted) for spgemm and
@@ -301,12 +302,38 @@ class SpTRSV(Workload):
                 "sample": f"{reps} x (sptrsv_forward + sptrsv_backward) of the full workload, serial C oracle"}
 
 
+class Copy(Workload):
+    """Plain device copy of a known size: the calibration run for the rocprofv3
+    FETCH_SIZE / WRITE_SIZE counters and the practical HBM ceiling of this part."""
+    name = "copy"
+
+    def setup(self, dev):
+        import torch
+        n = 64 * 1024 * 1024
+        self.src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
+        self.dst = torch.empty_like(self.src)
+        self.bytes_per_step = 2 * n * 4
+        self.dominant_bytes = self.bytes_per_step
+        self.dominant_name = "torch elementwise copy kernel, 256 MiB read + 256 MiB written"
+        self.config = {"workload": "device_copy_256MiB", "bytes_read": n * 4, "bytes_written": n * 4}
+
+    def step(self):
+        self.dst.copy_(self.src)
+
+    def dominant(self):
+        self.dst.copy_(self.src)
+
+    def cpu_baseline(self, budget_s):
+        return {"value": 0.0, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "not applicable"}
+
+
 WORKLOADS = {
     "spmv": lambda: SpMV(2048, np.float32, 0, "poisson2d_2048"),
     "spmv64": lambda: SpMV(256, np.float64, None, "poisson2d_256"),
     "spmm": SpMM,
     "spgemm": SpGEMM,
     "sptrsv": SpTRSV,
+    "copy": Copy,
 }
 
 
