@@ -347,18 +347,23 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
     const int gl = threadIdx.x % G, gi = threadIdx.x / G;
     int32_t *tab = s_keys + gi * STRIDE;
     T *val = s_vals + gi * STRIDE;
+    // compacted (column, slot) lists used to order the row on the way out
+    constexpr int CSTRIDE = TABLE / 2 + 4;
+    int32_t *ck = s_keys + GPB * STRIDE + gi * 2 * CSTRIDE;
+    int32_t *cs = ck + CSTRIDE;
     const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
     for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
         const int32_t idx = idx0 + gi;
         const bool live = idx < b1;
-        for (int t = gl; t < TABLE; t += G) { tab[t] = kEmpty; val[t] = T(0); }
+        for (int t = gl; t < TABLE; t += G) tab[t] = kEmpty;   // values are written by the first insert
         group_sync<G>();
         int64_t row = 0;
         auto add = [&](int32_t key, T prod) {
             uint32_t h = hash32(key) & (TABLE - 1);
             for (;;) {
                 const int32_t old = atomicCAS(&tab[h], kEmpty, key);
-                if (old == kEmpty || old == key) break;
+                if (old == kEmpty) { val[h] = prod; return; }   // 0 + prod == prod exactly
+                if (old == key) break;
                 h = (h + 1) & (TABLE - 1);
             }
             // the columns of one B row are distinct, so no other lane holds slot h now
@@ -415,22 +420,57 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
             }
         }
         if (G > kWave) __syncthreads();
-        if (live) {
-            const int64_t base = C_indptr[row];
+        // Output in ascending column order: the occupied slots are compacted into a dense
+        // list, then every entry is ranked against that list only (its rank is its position
+        // in the row).  Rows fill at most half of their table, so this is a fraction of the
+        // compares a rank over the whole table would take.
+        {
+            int mine = 0;
+            for (int t = gl; t < TABLE; t += G) mine += tab[t] != kEmpty;
+            int incl = mine, c;
+            if (G <= kWave) {
+                const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
+#pragma unroll
+                for (int off = 1; off < G; off <<= 1) {
+                    const int up = __shfl_up(incl, off, kWave);
+                    if (gl >= off) incl += up;
+                }
+                c = __shfl(incl, gbase + G - 1, kWave);
+            } else {
+                // one row per workgroup: scan through LDS (ck doubles as scratch before it is filled)
+                int *scr = reinterpret_cast<int *>(cs);
+                scr[gl] = mine;
+                __syncthreads();
+                incl = 0;
+                c = 0;
+                for (int l2 = 0; l2 < G; ++l2) {
+                    const int v = scr[l2];
+                    if (l2 <= gl) incl += v;
+                    c += v;
+                }
+                __syncthreads();
+            }
+            int pos = incl - mine;
             for (int t = gl; t < TABLE; t += G) {
                 const int32_t key = tab[t];
-                if (key == kEmpty) continue;
-                // rank = number of stored columns below this one; empty slots (0xffffffff) never
-                // count.  Four keys per LDS read.
-                int rank = 0;
-                const uint4 *tab4 = reinterpret_cast<const uint4 *>(tab);
-                for (int u = 0; u < TABLE / 4; ++u) {
-                    const uint4 q = tab4[u];
-                    rank += (q.x < (uint32_t)key) + (q.y < (uint32_t)key) + (q.z < (uint32_t)key) +
-                            (q.w < (uint32_t)key);
+                if (key != kEmpty) { ck[pos] = key; cs[pos] = t; ++pos; }
+            }
+            if (gl < 4) ck[c + gl] = kEmpty;   // pad the list to a multiple of four keys
+            group_sync<G>();
+            if (live) {
+                const int64_t base = C_indptr[row];
+                const uint4 *ck4 = reinterpret_cast<const uint4 *>(ck);
+                const int quads = (c + 3) >> 2;
+                for (int e = gl; e < c; e += G) {
+                    const uint32_t key = (uint32_t)ck[e];
+                    int rank = 0;
+                    for (int u = 0; u < quads; ++u) {   // four keys per LDS read; the pad never counts
+                        const uint4 q = ck4[u];
+                        rank += (q.x < key) + (q.y < key) + (q.z < key) + (q.w < key);
+                    }
+                    C_indices[base + rank] = (int64_t)key;
+                    C_data[base + rank] = val[cs[e]];
                 }
-                C_indices[base + rank] = key;
-                C_data[base + rank] = val[t];
             }
         }
         group_sync<G>();
@@ -612,19 +652,19 @@ int launch_numeric(const Work &w, int64_t B_cols, const void *A_data, const int6
     constexpr size_t per = sizeof(T) + sizeof(int32_t);
     {
         auto k = numeric_hash_kernel<T, 8, kNumTable0>;
-        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 8) * (kNumTable0 + kTablePad), s, 0, w.bins,
+        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), (kBlock / 8) * (per * (kNumTable0 + kTablePad) + 4 * (kNumTable0 + 8)), s, 0, w.bins,
                            w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
         NM_LAUNCH_CHECK("numeric_hash_kernel<8>");
     }
     {
         auto k = numeric_hash_kernel<T, 64, kNumTable1>;
-        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), per * (kBlock / 64) * (kNumTable1 + kTablePad), s, 1, w.bins,
+        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), (kBlock / 64) * (per * (kNumTable1 + kTablePad) + 4 * (kNumTable1 + 8)), s, 1, w.bins,
                            w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
         NM_LAUNCH_CHECK("numeric_hash_kernel<64>");
     }
     {
         auto k = numeric_hash_kernel<T, 256, kNumTable2>;
-        const size_t lds = per * kNumTable2;
+        const size_t lds = per * kNumTable2 + 4 * (kNumTable2 + 8);
         NM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(k, dim3(1024), dim3(kBlock), lds, s, 2, w.bins, w.perm, Ad, A_indices, A_indptr, Bd,
