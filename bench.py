@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 A step is one pass of the hot path over one synthetic input (forward, then
-backward with both gradients) through the ``numml_torch_cpp`` mirror, i.e. the
+backward with both gradients) through the ``numml_torch_cpp`` functions, i.e. the
 same calls autograd makes.  Inputs are resident in HBM before the timed region.
 Prints ONE JSON line.
 
@@ -87,7 +87,8 @@ class SpMV(Workload):
     def setup(self, dev):
         import torch
         from numml_amd import generators as G
-        from numml_amd import numml_torch_cpp as ext
+        from numml_amd import _binding
+        ext = _binding.ops
         self.ext = ext
         d, i, p, (rows, cols) = G.poisson2d(self.n, self.np_dtype, jitter_seed=self.jitter)
         self.host = (d, i, p, rows, cols)
@@ -100,10 +101,11 @@ class SpMV(Workload):
         self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s)
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
-        self.dominant_name = ("spmv_bwd_planned_kernel" if ext.BACKWARD_MODE == "planned"
+        self.dominant_name = ("spmv_bwd_planned_kernel" if _binding.backward_mode() == "planned"
                               else "spmv_bwd_kernel (+ fill_kernel clearing grad_x)")
         self.config = {"workload": f"spmv_fwd_bwd_{self.dtype}_{self.label}", "rows": rows,
-                       "nnz": self.nnz, "index_bytes": 8, "backward": ext.BACKWARD_MODE,
+                       "nnz": self.nnz, "index_bytes": 8, "backward": _binding.backward_mode(),
+                       "binding": _binding.name,
                        "algorithmic_bytes_per_step": self.bytes_per_step}
 
     def step(self):
@@ -136,7 +138,8 @@ class SpMM(Workload):
     def setup(self, dev):
         import torch
         from numml_amd import generators as G
-        from numml_amd import numml_torch_cpp as ext
+        from numml_amd import _binding
+        ext = _binding.ops
         self.ext = ext
         rows = cols = 1_000_000
         n = 64
@@ -154,7 +157,7 @@ class SpMM(Workload):
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
         self.dominant_name = ("spdmm_bwd_kernel (grad_A) + spdmm_fwd_kernel on the transposed plan (grad_B)"
-                              if ext.BACKWARD_MODE == "planned"
+                              if _binding.backward_mode() == "planned"
                               else "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)")
         self.config = {"workload": "spmm_fwd_bwd_f32_powerlaw_1M_n64", "rows": rows, "nnz": nnz,
                        "dense_cols": n, "index_bytes": 8,
@@ -195,7 +198,8 @@ class SpGEMM(Workload):
     def setup(self, dev):
         import torch
         from numml_amd import generators as G
-        from numml_amd import numml_torch_cpp as ext
+        from numml_amd import _binding
+        ext = _binding.ops
         self.ext = ext
         n = int(os.environ.get("NM_BENCH_SPGEMM_N", "128"))
         d, i, p, (rows, cols) = G.laplace3d(n, np.float64, jitter_seed=0)
@@ -254,7 +258,8 @@ class SpTRSV(Workload):
     def setup(self, dev):
         import torch
         from numml_amd import generators as G
-        from numml_amd import numml_torch_cpp as ext
+        from numml_amd import _binding
+        ext = _binding.ops
         self.ext = ext
         n = 1024
         d, i, p, (rows, cols) = G.poisson2d_lower(n, np.float64, diag_seed=0)

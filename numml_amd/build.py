@@ -1,9 +1,15 @@
-"""Builds libnumml_hip.so (the C-ABI HIP library) in-tree with hipcc for gfx950.
+"""Builds the native parts in-tree.
 
-    python -m numml_amd.build          # compile every csrc/*.hip and link
+    python -m numml_amd.build          # both of the below
 
-Objects and the library land in numml_amd/lib/.  hipcc cross-compiles, so this
-runs on machines without a GPU.
+* libnumml_hip.so: every csrc/*.hip compiled with hipcc for gfx950 and linked
+  (the C ABI of include/numml_hip.h).  hipcc cross-compiles, so this runs on
+  machines without a GPU.
+* numml_torch_cpp<ext>.so: csrc/torch_binding.cpp, the pybind11 torch extension
+  that exports the reference module's hot-path functions on top of the C ABI
+  (host-only C++, compiled with g++ against the installed torch).
+
+Objects and libraries land in numml_amd/lib/.
 """
 import concurrent.futures
 import glob
@@ -58,5 +64,35 @@ def build(verbose=True):
     return LIB
 
 
+def build_extension(verbose=True):
+    """Compile csrc/torch_binding.cpp into numml_amd/lib/numml_torch_cpp<ext>.so."""
+    import sysconfig
+
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    ext = sysconfig.get_config_var("EXT_SUFFIX")
+    out = os.path.join(LIBDIR, "numml_torch_cpp" + ext)
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cmd = [
+        os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-w", "-fvisibility=hidden",
+        "-Wl,-Bsymbolic",
+        "-DTORCH_EXTENSION_NAME=numml_torch_cpp", "-DTORCH_API_INCLUDE_EXTENSION_H",
+        f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+        f"-I{os.path.join(tdir, 'include')}", f"-I{os.path.join(tdir, 'include', 'torch', 'csrc', 'api', 'include')}",
+        f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include", f"-I{os.path.join(ROOT, 'include')}",
+        os.path.join(CSRC, "torch_binding.cpp"), "-o", out,
+        f"-L{os.path.join(tdir, 'lib')}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
+        "-ltorch_python", f"-L{LIBDIR}", "-lnumml_hip",
+        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{os.path.join(tdir, 'lib')}",
+    ]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building the torch extension failed:\n{r.stderr[-4000:]}")
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build()
+    build_extension()

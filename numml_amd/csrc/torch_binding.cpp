@@ -1,0 +1,465 @@
+// numml_torch_cpp: the reference's extension module, re-implemented on the
+// C ABI of libnumml_hip.so.
+//
+// Exports the eight hot-path functions that cpp/sparse_csr.cpp:307-319 binds
+// (spgemv / spdmm / spgemm / sptrsv, _forward and _backward) with the argument
+// lists of cpp/sparse_csr.hpp:32-105, so `import numml_torch_cpp` in the
+// reference's Python layer (numml/sparse/_csr.py:2, numml/sparse/linalg.py:2)
+// resolves to HIP kernels for this path.  torch is used for device memory
+// (outputs and scratch come from its caching allocator) and for the current
+// stream; all arithmetic happens behind numml_hip.h.
+//
+// There is no CPU implementation here: tensors that are not on a HIP device
+// raise, as does any nm_status other than NM_OK.
+//
+// Host-only translation unit (compiled with g++); it needs no device code.
+#include <torch/extension.h>
+
+#include <ATen/hip/HIPContext.h>
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <atomic>
+#include <cstdlib>
+#include <list>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "numml_hip.h"
+
+namespace {
+
+using torch::Tensor;
+
+nm_dtype dtype_of(const Tensor &t) {
+    if (t.scalar_type() == torch::kFloat32) return NM_F32;
+    if (t.scalar_type() == torch::kFloat64) return NM_F64;
+    // the reference dispatches with AT_DISPATCH_FLOATING_TYPES (cpp/sparse_csr_cpu.cpp:22)
+    TORCH_CHECK(false, "numml_amd: values must be float32 or float64, got ", t.scalar_type());
+}
+
+void check(int status, const char *what) {
+    TORCH_CHECK(status == NM_OK, what, " failed with status ", status, ": ", nm_last_error());
+}
+
+c10::Device need_device(std::initializer_list<const Tensor *> ts) {
+    const c10::Device dev = (*ts.begin())->device();
+    TORCH_CHECK(dev.is_cuda(), "numml_amd: this backend runs on HIP devices only; got a tensor on '", dev,
+                "' (no CPU implementation is provided)");
+    for (const Tensor *t : ts)
+        TORCH_CHECK(t->device() == dev, "expected all tensors to be on the same device, but got ", dev, " and ",
+                    t->device());
+    return dev;
+}
+
+Tensor index_tensor(const Tensor &t, const char *name) {
+    // the reference reads structure through accessor<int64_t, 1> (cpp/sparse_csr_cpu.cpp:24-25)
+    TORCH_CHECK(t.scalar_type() == torch::kInt64, "expected scalar type Long for ", name, " but found ",
+                t.scalar_type());
+    return t.contiguous();
+}
+
+void same_dtype(const Tensor &a, const Tensor &b, const char *what) {
+    TORCH_CHECK(a.scalar_type() == b.scalar_type(), "expected ", what, " of type ", a.scalar_type(),
+                " but found ", b.scalar_type());
+}
+
+nm_stream current_stream(const c10::Device &dev) {
+    return reinterpret_cast<nm_stream>(c10::hip::getCurrentHIPStream(dev.index()).stream());
+}
+
+// 2-D tensor with unit column stride (copied only when it is not already); returns its row stride.
+Tensor row_major(const Tensor &M, int64_t *ld) {
+    TORCH_CHECK(M.dim() == 2, "expected a 2-D tensor, got ", M.dim(), "-D");
+    Tensor R = M;
+    if (R.size(1) > 1 && R.stride(1) != 1) R = R.contiguous();
+    if (R.size(0) > 1 && R.stride(0) < std::max<int64_t>(R.size(1), 1)) R = R.contiguous();
+    *ld = R.size(0) > 1 ? R.stride(0) : std::max<int64_t>(R.size(1), 1);
+    return R;
+}
+
+Tensor scratch(size_t bytes, const c10::Device &dev) {
+    return torch::empty({(int64_t)std::max<size_t>(bytes, 8)},
+                        torch::TensorOptions().dtype(torch::kUInt8).device(dev));
+}
+
+// "planned" (default): backward passes walk A by column on a cached transposed
+// structure (deterministic, no atomics); "atomic": stateless scatter with atomics.
+// NUMML_AMD_BACKWARD sets the initial value, set_backward_mode() changes it.
+std::atomic<bool> g_planned{[] {
+    const char *e = std::getenv("NUMML_AMD_BACKWARD");
+    return !(e && std::string(e) == "atomic");
+}()};
+
+bool planned_backward() { return g_planned.load(std::memory_order_relaxed); }
+
+// ---- structure plans -----------------------------------------------------------
+//
+// Everything derived from a sparsity pattern alone is computed once and cached,
+// keyed on the storage and version counters of the structure tensors.  A plan
+// keeps those tensors alive, so an address cannot be reused by another pattern
+// while the plan is cached; in-place edits bump the version and miss the cache.
+
+struct Plan {
+    char kind;  // 'T' transposed structure, 'L' level schedule
+    int device;
+    const void *idx_ptr, *ptr_ptr;
+    uint32_t idx_version, ptr_version;
+    int64_t nnz, nptr, a, b;
+    Tensor indices, indptr, mem;
+    nm_sptrsv_plan *handle = nullptr;
+    ~Plan() {
+        if (handle) nm_sptrsv_plan_destroy(handle);
+    }
+};
+
+constexpr size_t kPlanCacheSize = 16;
+std::mutex g_plans_mutex;
+std::list<std::shared_ptr<Plan>> g_plans;  // most recently used first
+
+template <typename Make>
+std::shared_ptr<Plan> cached(char kind, const Tensor &indices, const Tensor &indptr, int64_t a, int64_t b,
+                             Make make) {
+    const int device = indices.device().index();
+    const uint32_t vi = indices._version(), vp = indptr._version();
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        for (auto it = g_plans.begin(); it != g_plans.end(); ++it) {
+            Plan &p = **it;
+            if (p.kind == kind && p.device == device && p.idx_ptr == indices.data_ptr() &&
+                p.ptr_ptr == indptr.data_ptr() && p.idx_version == vi && p.ptr_version == vp &&
+                p.nnz == indices.numel() && p.nptr == indptr.numel() && p.a == a && p.b == b) {
+                auto hit = *it;
+                g_plans.erase(it);
+                g_plans.push_front(hit);
+                return hit;
+            }
+        }
+    }
+    auto plan = std::make_shared<Plan>();
+    plan->kind = kind;
+    plan->device = device;
+    plan->idx_ptr = indices.data_ptr();
+    plan->ptr_ptr = indptr.data_ptr();
+    plan->idx_version = vi;
+    plan->ptr_version = vp;
+    plan->nnz = indices.numel();
+    plan->nptr = indptr.numel();
+    plan->a = a;
+    plan->b = b;
+    plan->indices = indices;
+    plan->indptr = indptr;
+    make(*plan);
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    g_plans.push_front(plan);
+    while (g_plans.size() > kPlanCacheSize) g_plans.pop_back();
+    return plan;
+}
+
+std::shared_ptr<Plan> transpose_plan(const Tensor &indices, const Tensor &indptr, int64_t rows, int64_t cols,
+                                     const c10::Device &dev) {
+    return cached('T', indices, indptr, rows, cols, [&](Plan &p) {
+        size_t pbytes = 0, wbytes = 0;
+        check(nm_csr_transpose_plan_bytes(rows, cols, p.nnz, &pbytes, &wbytes), "nm_csr_transpose_plan_bytes");
+        p.mem = scratch(pbytes, dev);
+        Tensor work = scratch(wbytes, dev);
+        auto stream = c10::hip::getCurrentHIPStream(dev.index());
+        check(nm_csr_transpose_plan_build(rows, cols, p.nnz, indices.data_ptr<int64_t>(),
+                                          indptr.data_ptr<int64_t>(), p.mem.data_ptr(), pbytes, work.data_ptr(),
+                                          wbytes, reinterpret_cast<nm_stream>(stream.stream())),
+              "nm_csr_transpose_plan_build");
+        // one-time: the plan is complete for every stream once this returns
+        stream.synchronize();
+    });
+}
+
+std::shared_ptr<Plan> level_plan(const Tensor &indices, const Tensor &indptr, int64_t rows, bool lower,
+                                 const c10::Device &dev) {
+    return cached('L', indices, indptr, rows, lower ? 1 : 0, [&](Plan &p) {
+        size_t pbytes = 0, wbytes = 0;
+        check(nm_sptrsv_plan_bytes(rows, p.nnz, &pbytes, &wbytes), "nm_sptrsv_plan_bytes");
+        p.mem = scratch(pbytes, dev);
+        Tensor work = scratch(wbytes, dev);
+        check(nm_sptrsv_analyse(rows, p.nnz, indices.data_ptr<int64_t>(), indptr.data_ptr<int64_t>(),
+                                lower ? 1 : 0, p.mem.data_ptr(), pbytes, work.data_ptr(), wbytes, &p.handle,
+                                current_stream(dev)),
+              "nm_sptrsv_analyse");  // synchronises its stream
+    });
+}
+
+Tensor solve(const Plan &plan, bool transposed, const Tensor &A_data, bool unit, const Tensor &b, int64_t rows,
+             const c10::Device &dev) {
+    Tensor x = torch::empty({rows}, A_data.options());
+    size_t bytes = 0;
+    check(nm_sptrsv_solve_bytes(rows, A_data.numel(), &bytes), "nm_sptrsv_solve_bytes");
+    Tensor work = scratch(bytes, dev);
+    check(nm_sptrsv_solve(plan.handle, dtype_of(A_data), transposed ? 1 : 0, A_data.data_ptr(), unit ? 1 : 0,
+                          b.data_ptr(), x.data_ptr(), work.data_ptr(), bytes, current_stream(dev)),
+          "nm_sptrsv_solve");
+    return x;
+}
+
+// The exported functions below stay inside this unnamed namespace: they have the
+// same names and signatures as the reference's (cpp/sparse_csr.hpp:32-105), and
+// with external linkage a process that also loads the reference's extension could
+// bind one module's Python entries to the other module's functions.
+
+// ---------------------------------------------------------------------------- SpMV
+
+Tensor spgemv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_col_ind, Tensor A_rowptr, Tensor x) {
+    const auto dev = need_device({&A_data, &A_col_ind, &A_rowptr, &x});
+    same_dtype(A_data, x, "x");
+    TORCH_CHECK(x.dim() == 1, "expected 1-D x, got ", x.dim(), "-D");
+    A_data = A_data.contiguous();
+    x = x.contiguous();
+    A_col_ind = index_tensor(A_col_ind, "A_col_ind");
+    A_rowptr = index_tensor(A_rowptr, "A_rowptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor y = torch::empty({A_rows}, A_data.options());
+    check(nm_spgemv_forward(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
+                            A_col_ind.data_ptr<int64_t>(), A_rowptr.data_ptr<int64_t>(), x.data_ptr(),
+                            y.data_ptr(), current_stream(dev)),
+          "nm_spgemv_forward");
+    return y;
+}
+
+std::vector<Tensor> spgemv_backward(Tensor grad_z, int A_rows, int A_cols, Tensor A_data, Tensor A_col_ind,
+                                    Tensor A_rowptr, Tensor x) {
+    const auto dev = need_device({&grad_z, &A_data, &A_col_ind, &A_rowptr, &x});
+    same_dtype(A_data, x, "x");
+    same_dtype(A_data, grad_z, "grad_z");
+    A_data = A_data.contiguous();
+    x = x.contiguous();
+    grad_z = grad_z.contiguous();
+    A_col_ind = index_tensor(A_col_ind, "A_col_ind");
+    A_rowptr = index_tensor(A_rowptr, "A_rowptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty_like(A_data), grad_x = torch::empty_like(x);
+    if (planned_backward()) {
+        auto plan = transpose_plan(A_col_ind, A_rowptr, A_rows, x.size(0), dev);
+        check(nm_spgemv_backward_planned(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
+                                         plan->mem.data_ptr(), x.data_ptr(), grad_z.data_ptr(),
+                                         grad_A.data_ptr(), grad_x.data_ptr(), current_stream(dev)),
+              "nm_spgemv_backward_planned");
+    } else {
+        check(nm_spgemv_backward(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
+                                 A_col_ind.data_ptr<int64_t>(), A_rowptr.data_ptr<int64_t>(), x.data_ptr(),
+                                 grad_z.data_ptr(), grad_A.data_ptr(), grad_x.data_ptr(), current_stream(dev)),
+              "nm_spgemv_backward");
+    }
+    return {grad_A, grad_x};
+}
+
+// ---------------------------------------------------------------------------- SpMM
+
+Tensor spdmm_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr, Tensor B) {
+    // cpp/sparse_csr.cpp:125-128 checks the same thing with the same wording
+    TORCH_CHECK((A_data.device() == A_indices.device() && A_indices.device() == A_indptr.device() &&
+                 A_indptr.device() == B.device()),
+                "expected A and B to be on same device, but got A on (", A_data.device(), ", ",
+                A_indices.device(), ", ", A_indptr.device(), ") and B on ", B.device());
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B});
+    same_dtype(A_data, B, "B");
+    A_data = A_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    int64_t ldb = 1;
+    B = row_major(B, &ldb);
+    const int64_t n = B.size(1);
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor C = torch::empty({A_rows, n}, A_data.options());
+    check(nm_spdmm_forward(dtype_of(A_data), A_rows, B.size(0), A_data.numel(), A_data.data_ptr(),
+                           A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B.data_ptr(), ldb, n,
+                           C.data_ptr(), std::max<int64_t>(n, 1), current_stream(dev)),
+          "nm_spdmm_forward");
+    return C;
+}
+
+std::vector<Tensor> spdmm_backward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr,
+                                   Tensor B, Tensor grad_C) {
+    TORCH_CHECK((A_data.device() == A_indices.device() && A_indices.device() == A_indptr.device() &&
+                 A_indptr.device() == B.device()),
+                "expected A and B to be on same device, but got A on (", A_data.device(), ", ",
+                A_indices.device(), ", ", A_indptr.device(), ") and B on ", B.device());
+    TORCH_CHECK(B.device() == grad_C.device(), "expected B and grad_C to be on same device, but got B on ",
+                B.device(), " and grad_C on ", grad_C.device());
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B, &grad_C});
+    same_dtype(A_data, B, "B");
+    same_dtype(A_data, grad_C, "grad_C");
+    A_data = A_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    int64_t ldb = 1, ldg = 1;
+    B = row_major(B, &ldb);
+    grad_C = row_major(grad_C, &ldg);
+    const int64_t n = B.size(1);
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty_like(A_data);
+    Tensor grad_B = torch::empty({B.size(0), n}, B.options());
+    if (planned_backward()) {
+        auto plan = transpose_plan(A_indices, A_indptr, A_rows, B.size(0), dev);
+        check(nm_spdmm_backward_planned(dtype_of(A_data), A_rows, B.size(0), A_data.numel(), A_data.data_ptr(),
+                                        A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                        plan->mem.data_ptr(), B.data_ptr(), ldb, grad_C.data_ptr(), ldg, n,
+                                        grad_A.data_ptr(), grad_B.data_ptr(), std::max<int64_t>(n, 1),
+                                        current_stream(dev)),
+              "nm_spdmm_backward_planned");
+    } else {
+        check(nm_spdmm_backward(dtype_of(A_data), A_rows, B.size(0), A_data.numel(), A_data.data_ptr(),
+                                A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B.data_ptr(), ldb,
+                                grad_C.data_ptr(), ldg, n, grad_A.data_ptr(), grad_B.data_ptr(),
+                                std::max<int64_t>(n, 1), current_stream(dev)),
+              "nm_spdmm_backward");
+    }
+    return {grad_A, grad_B};
+}
+
+// -------------------------------------------------------------------------- SpGEMM
+
+std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr,
+                                   int B_rows, int B_cols, Tensor B_data, Tensor B_indices, Tensor B_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B_data, &B_indices, &B_indptr});
+    same_dtype(A_data, B_data, "B_data");
+    A_data = A_data.contiguous();
+    B_data = B_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    B_indices = index_tensor(B_indices, "B_indices");
+    B_indptr = index_tensor(B_indptr, "B_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    size_t bytes = 0;
+    check(nm_spgemm_workspace_bytes(A_rows, B_cols, &bytes), "nm_spgemm_workspace_bytes");
+    Tensor work = scratch(bytes, dev);
+    const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
+    Tensor C_indptr = torch::empty({(int64_t)A_rows + 1}, iopt);
+    nm_stream st = current_stream(dev);
+    check(nm_spgemm_symbolic(A_rows, A_cols, B_cols, A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                             B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                             C_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, st),
+          "nm_spgemm_symbolic");
+    // the one device->host read the interface makes inherent: C is returned exactly sized
+    const int64_t nnz_c = C_indptr[A_rows].item<int64_t>();
+    Tensor C_indices = torch::empty({nnz_c}, iopt);
+    Tensor C_data = torch::empty({nnz_c}, A_data.options());
+    check(nm_spgemm_numeric(dtype_of(A_data), A_rows, A_cols, B_cols, A_data.data_ptr(),
+                            A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
+                            B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                            C_indptr.data_ptr<int64_t>(), C_indices.data_ptr<int64_t>(), C_data.data_ptr(),
+                            work.data_ptr(), bytes, st),
+          "nm_spgemm_numeric");
+    return {C_data, C_indices, C_indptr};
+}
+
+std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_indptr, int A_rows, int A_cols,
+                                    Tensor A_data, Tensor A_indices, Tensor A_indptr, int B_rows, int B_cols,
+                                    Tensor B_data, Tensor B_indices, Tensor B_indptr) {
+    const auto dev = need_device({&grad_C, &C_indices, &C_indptr, &A_data, &A_indices, &A_indptr, &B_data,
+                                  &B_indices, &B_indptr});
+    same_dtype(A_data, B_data, "B_data");
+    same_dtype(A_data, grad_C, "grad_C");
+    A_data = A_data.contiguous();
+    B_data = B_data.contiguous();
+    grad_C = grad_C.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    B_indices = index_tensor(B_indices, "B_indices");
+    B_indptr = index_tensor(B_indptr, "B_indptr");
+    C_indices = index_tensor(C_indices, "C_indices");
+    C_indptr = index_tensor(C_indptr, "C_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty_like(A_data), grad_B = torch::empty_like(B_data);
+    check(nm_spgemm_backward(dtype_of(A_data), A_rows, A_data.numel(), B_data.numel(), grad_C.data_ptr(),
+                             C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(), A_data.data_ptr(),
+                             A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
+                             B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(), grad_A.data_ptr(),
+                             grad_B.data_ptr(), current_stream(dev)),
+          "nm_spgemm_backward");
+    return {grad_A, grad_B};
+}
+
+// -------------------------------------------------------------------------- SpTRSV
+
+Tensor sptrsv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr, bool lower,
+                      bool unit, Tensor b) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr, &b});
+    same_dtype(A_data, b, "b");
+    A_data = A_data.contiguous();
+    b = b.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    auto plan = level_plan(A_indices, A_indptr, A_rows, lower, dev);
+    return solve(*plan, false, A_data, unit, b, A_rows, dev);
+}
+
+std::vector<Tensor> sptrsv_backward(Tensor grad_x, Tensor x, int A_rows, int A_cols, Tensor A_data,
+                                    Tensor A_indices, Tensor A_indptr, bool lower, bool unit, Tensor b) {
+    const auto dev = need_device({&grad_x, &x, &A_data, &A_indices, &A_indptr});
+    same_dtype(A_data, grad_x, "grad_x");
+    same_dtype(A_data, x, "x");
+    A_data = A_data.contiguous();
+    grad_x = grad_x.contiguous();
+    x = x.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    auto plan = level_plan(A_indices, A_indptr, A_rows, lower, dev);
+    Tensor grad_b = solve(*plan, true, A_data, unit, grad_x, A_rows, dev);
+    Tensor grad_A = torch::empty_like(A_data);
+    check(nm_masked_outer(dtype_of(A_data), A_rows, A_data.numel(), A_indices.data_ptr<int64_t>(),
+                          A_indptr.data_ptr<int64_t>(), -1.0, grad_b.data_ptr(), x.data_ptr(), grad_A.data_ptr(),
+                          current_stream(dev)),
+          "nm_masked_outer");
+    return {grad_A, grad_b};
+}
+
+// (dependency levels, kernel launches per solve) of the cached or newly built level
+// schedule of a triangular pattern; no counterpart in the reference (diagnostics).
+std::tuple<int64_t, int64_t> sptrsv_schedule(int A_rows, Tensor A_indices, Tensor A_indptr, bool lower) {
+    const auto dev = need_device({&A_indices, &A_indptr});
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    auto plan = level_plan(A_indices, A_indptr, A_rows, lower, dev);
+    return {nm_sptrsv_plan_levels(plan->handle), nm_sptrsv_plan_launches(plan->handle)};
+}
+
+void clear_plan_cache() {
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    g_plans.clear();
+}
+
+int64_t plan_cache_size() {
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    return (int64_t)g_plans.size();
+}
+
+void set_backward_mode(const std::string &mode) {
+    TORCH_CHECK(mode == "planned" || mode == "atomic", "backward mode must be 'planned' or 'atomic', got '", mode,
+                "'");
+    g_planned.store(mode == "planned", std::memory_order_relaxed);
+}
+
+std::string backward_mode() { return planned_backward() ? "planned" : "atomic"; }
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.doc() = "numml_torch_cpp on AMD gfx950: differentiable CSR SpMV / SpMM / SpGEMM / SpTRSV";
+    m.def("spgemv_forward", &spgemv_forward, "SPGEMV forward");
+    m.def("spgemv_backward", &spgemv_backward, "SPGEMV backward");
+    m.def("spgemm_forward", &spgemm_forward, "SPGEMM forward");
+    m.def("spgemm_backward", &spgemm_backward, "SPGEMM backward");
+    m.def("spdmm_forward", &spdmm_forward, "Sparse times dense matrix forward");
+    m.def("spdmm_backward", &spdmm_backward, "Sparse times dense matrix backward");
+    m.def("sptrsv_forward", &sptrsv_forward, "Sparse triangular solve forward");
+    m.def("sptrsv_backward", &sptrsv_backward, "Sparse triangular solve backward");
+    m.def("sptrsv_schedule", &sptrsv_schedule, "(levels, launches per solve) of a triangular pattern");
+    m.def("clear_plan_cache", &clear_plan_cache, "Drop every cached structure plan");
+    m.def("plan_cache_size", &plan_cache_size, "Number of cached structure plans");
+    m.def("set_backward_mode", &set_backward_mode, "'planned' (cached transposed structure) or 'atomic'");
+    m.def("backward_mode", &backward_mode, "Current backward mode");
+}

@@ -21,7 +21,7 @@ from . import _lib
 __all__ = [
     "spgemv_forward", "spgemv_backward", "spdmm_forward", "spdmm_backward",
     "spgemm_forward", "spgemm_backward", "sptrsv_forward", "sptrsv_backward",
-    "clear_plan_cache",
+    "clear_plan_cache", "plan_cache_size", "sptrsv_schedule",
 ]
 
 
@@ -326,6 +326,22 @@ class _Plan:
 def _plan_for(indices, indptr, rows, lower, dev):
     return _cached("L", indices, indptr, (rows, bool(lower)),
                    lambda: _Plan(indices, indptr, rows, lower, dev))
+
+
+def sptrsv_schedule(A_rows, A_indices, A_indptr, lower):
+    """(dependency levels, kernel launches per solve) of the level schedule of a
+    triangular pattern, built or taken from the cache; diagnostics, no counterpart
+    in the reference."""
+    dev = _need_device(A_indices, A_indptr)
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
+    return plan.levels, plan.launches
+
+
+def plan_cache_size():
+    with _plans_lock:
+        return len(_plans)
 
 
 def _solve(plan, transposed, A_data, A_indices, A_indptr, unit, b, rows, dev):

@@ -17,7 +17,7 @@ CSR / COO / dense / SciPy, device and dtype moves, ``to_dense`` and
 import numpy as np
 import torch
 
-from .. import numml_torch_cpp as _ext
+from .._binding import ops as _ext
 
 __all__ = ["SparseCSRTensor", "coo_to_csr", "eye", "spgemv", "spgemm", "spdmm"]
 

@@ -21,11 +21,11 @@ def load():
     global _mod
     if _mod is not None:
         return _mod
-    hits = sorted(glob.glob(os.path.join(_HERE, "_ref", "numml_torch_cpp*.so")))
+    hits = sorted(glob.glob(os.path.join(_HERE, "_ref", "numml_ref_cpu*.so")))
     if not hits:
         return None
     import torch  # noqa: F401  (libtorch must be loaded before the extension)
-    spec = importlib.util.spec_from_file_location("numml_torch_cpp", hits[0])
+    spec = importlib.util.spec_from_file_location("numml_ref_cpu", hits[0])
     mod = importlib.util.module_from_spec(spec)
     try:
         spec.loader.exec_module(mod)
@@ -40,7 +40,7 @@ def available():
 
 
 def call(name, *args):
-    """Call ``numml_torch_cpp.<name>`` with NumPy arrays; returns NumPy array(s)."""
+    """Call the reference build's ``<name>`` with NumPy arrays; returns NumPy array(s)."""
     import torch
     mod = load()
     if mod is None:

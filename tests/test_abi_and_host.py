@@ -87,6 +87,22 @@ def test_cpu_tensors_are_refused_not_computed():
         A @ x
 
 
+def test_compiled_extension_exports_the_reference_module():
+    import numml_amd
+    cpp = numml_amd.load_compiled()
+    for name in ("spgemv_forward", "spgemv_backward", "spgemm_forward", "spgemm_backward", "spdmm_forward",
+                 "spdmm_backward", "sptrsv_forward", "sptrsv_backward"):     # cpp/sparse_csr.cpp:307-319
+        assert callable(getattr(cpp, name)), name
+    d, i, p = torch.ones(3), torch.tensor([0, 1, 2]), torch.tensor([0, 1, 2, 3])
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        cpp.spgemv_forward(3, 3, d, i, p, torch.ones(3))
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        cpp.spgemm_forward(3, 3, d, i, p, 3, 3, d, i, p)
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        cpp.sptrsv_backward(d, d, 3, 3, d, i, p, True, False, d)
+    assert cpp.backward_mode() in ("planned", "atomic") and cpp.plan_cache_size() == 0
+
+
 def test_function_level_errors_match_the_reference():
     d, i, p = torch.ones(3), torch.tensor([0, 1, 2]), torch.tensor([0, 1, 2, 3])
     A = sp.SparseCSRTensor((d, i, p), (3, 3))

@@ -1,0 +1,172 @@
+"""The compiled ``numml_torch_cpp`` extension (csrc/torch_binding.cpp) on a HIP device.
+
+It is the module the reference's Python layer imports (numml/sparse/_csr.py:2);
+here every one of its eight functions is checked against the CPU oracle on
+seeded inputs and, bit for bit, against the ctypes binding of the same C ABI.
+Tolerance: util.RTOL (1e-5 for float32, 1e-12 for float64); structure is exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+import numml_amd
+import oracle
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as mirror
+from util import assert_close, assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+
+@pytest.fixture(scope="module")
+def cpp():
+    return numml_amd.load_compiled()
+
+
+@pytest.fixture(params=["planned", "atomic"])
+def mode(request, cpp):
+    old_cpp, old_mirror = cpp.backward_mode(), mirror.BACKWARD_MODE
+    cpp.set_backward_mode(request.param)
+    mirror.BACKWARD_MODE = request.param
+    yield request.param
+    cpp.set_backward_mode(old_cpp)
+    mirror.BACKWARD_MODE = old_mirror
+
+
+def test_exports_the_reference_functions(cpp):
+    for name in ("spgemv_forward", "spgemv_backward", "spgemm_forward", "spgemm_backward", "spdmm_forward",
+                 "spdmm_backward", "sptrsv_forward", "sptrsv_backward"):     # cpp/sparse_csr.cpp:307-319
+        assert callable(getattr(cpp, name)), name
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_spgemv(dev, cpp, dtype, mode):
+    for seed, (rows, cols, density) in enumerate([(1, 1, 1.0), (37, 53, 0.2), (700, 650, 0.02), (64, 64, 0.0)]):
+        d, i, p, _ = G.random_csr(rows, cols, density, seed, dtype, empty_rows=rows > 1)
+        x, g = randn(seed + 10, cols, dtype), randn(seed + 20, rows, dtype)
+        D, I, P, X, Gz = to_dev(dev, d, i, p, x, g)
+        y = cpp.spgemv_forward(rows, cols, D, I, P, X)
+        assert_close(host(y), oracle.spgemv_forward(rows, cols, d, i, p, x), "y")
+        assert_same(host(y), host(mirror.spgemv_forward(rows, cols, D, I, P, X)), "y vs ctypes binding")
+        gA, gx = cpp.spgemv_backward(Gz, rows, cols, D, I, P, X)
+        gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+        assert_same(host(gA), gA_ref, "grad_A")
+        assert_close(host(gx), gx_ref, "grad_x")
+        mA, mx = mirror.spgemv_backward(Gz, rows, cols, D, I, P, X)
+        assert_same(host(gA), host(mA), "grad_A vs ctypes binding")
+        if mode == "planned":
+            assert_same(host(gx), host(mx), "grad_x vs ctypes binding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [1, 7, 64])
+def test_spdmm(dev, cpp, dtype, n, mode):
+    rows, cols = 300, 280
+    d, i, p, _ = G.random_csr(rows, cols, 0.05, 3, dtype)
+    B, gC = randn(4, (cols, n), dtype), randn(5, (rows, n), dtype)
+    D, I, P, Bt, Gt = to_dev(dev, d, i, p, B, gC)
+    C = cpp.spdmm_forward(rows, cols, D, I, P, Bt)
+    assert_same(host(C), oracle.spdmm_forward(rows, cols, d, i, p, B), "C")     # short rows: storage-order sums
+    gA, gB = cpp.spdmm_backward(rows, cols, D, I, P, Bt, Gt)
+    gA_ref, gB_ref = oracle.spdmm_backward(rows, cols, d, i, p, B, gC)
+    assert_close(host(gA), gA_ref, "grad_A")
+    assert_close(host(gB), gB_ref, "grad_B")
+    mA, mB = mirror.spdmm_backward(rows, cols, D, I, P, Bt, Gt)
+    assert_same(host(gA), host(mA), "grad_A vs ctypes binding")
+    if mode == "planned":
+        assert_same(host(gB), host(mB), "grad_B vs ctypes binding")
+    # a column-major B and a row-sliced grad_C take the strided/copy paths
+    Bf = Bt.t().contiguous().t()
+    Gs = torch.cat([Gt, Gt], dim=1)[:, :n]
+    assert_same(host(cpp.spdmm_forward(rows, cols, D, I, P, Bf)), host(C), "C from column-major B")
+    sA, sB = cpp.spdmm_backward(rows, cols, D, I, P, Bf, Gs)
+    assert_same(host(sA), host(gA), "grad_A from strided operands")
+    if mode == "planned":
+        assert_same(host(sB), host(gB), "grad_B from strided operands")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_spgemm(dev, cpp, dtype):
+    for seed, (m, k, n, da, db) in enumerate([(40, 50, 45, 0.15, 0.15), (500, 400, 450, 0.03, 0.03), (8, 8, 8, 0.0, 0.3)]):
+        ad, ai, ap, _ = G.random_csr(m, k, da, seed, dtype)
+        bd, bi, bp, _ = G.random_csr(k, n, db, seed + 50, dtype)
+        AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+        Cd, Ci, Cp = cpp.spgemm_forward(m, k, AD, AI, AP, k, n, BD, BI, BP)
+        rd, ri, rp = oracle.spgemm_forward(m, k, ad, ai, ap, k, n, bd, bi, bp)
+        assert_same(host(Cp), rp, "C_indptr")
+        assert_same(host(Ci), ri, "C_indices")
+        assert_same(host(Cd), rd, "C_data")
+        g = randn(seed + 7, rd.shape[0], dtype)
+        Gc, = to_dev(dev, g)
+        gA, gB = cpp.spgemm_backward(Gc, Ci, Cp, m, k, AD, AI, AP, k, n, BD, BI, BP)
+        gA_ref, gB_ref = oracle.spgemm_backward(g, ri, rp, m, k, ad, ai, ap, k, n, bd, bi, bp)
+        assert_same(host(gA), gA_ref, "grad_A")
+        assert_close(host(gB), gB_ref, "grad_B")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("lower", [True, False])
+@pytest.mark.parametrize("unit", [False, True])
+def test_sptrsv(dev, cpp, dtype, lower, unit):
+    n = 400
+    d, i, p, _ = G.random_tri(n, 0.02, 11, lower, dtype)
+    b, g = randn(12, n, dtype), randn(13, n, dtype)
+    D, I, P, Bt, Gt = to_dev(dev, d, i, p, b, g)
+    x = cpp.sptrsv_forward(n, n, D, I, P, lower, unit, Bt)
+    x_ref = oracle.sptrsv_forward(n, n, d, i, p, lower, unit, b)
+    assert_close(host(x), x_ref, "x")
+    assert_same(host(x), host(mirror.sptrsv_forward(n, n, D, I, P, lower, unit, Bt)), "x vs ctypes binding")
+    gA, gb = cpp.sptrsv_backward(Gt, x, n, n, D, I, P, lower, unit, Bt)
+    gA_ref, gb_ref = oracle.sptrsv_backward(g, host(x), n, n, d, i, p, lower, unit)
+    assert_close(host(gb), gb_ref, "grad_b")
+    assert_close(host(gA), gA_ref, "grad_A")
+
+
+def test_plan_cache_and_errors(dev, cpp):
+    d, i, p, (n, _) = G.poisson2d_lower(20, np.float64)
+    D, I, P = to_dev(dev, d, i, p)
+    b = to_dev(dev, randn(1, n, np.float64))[0]
+    cpp.clear_plan_cache()
+    assert cpp.plan_cache_size() == 0
+    cpp.sptrsv_forward(n, n, D, I, P, True, False, b)
+    cpp.sptrsv_forward(n, n, D, I, P, True, False, b)
+    assert cpp.plan_cache_size() == 1
+    cpp.sptrsv_backward(b, b, n, n, D, I, P, True, False, b)        # the transposed solve shares the plan
+    assert cpp.plan_cache_size() == 1
+    cpp.set_backward_mode("planned")
+    cpp.spgemv_backward(b, n, n, D, I, P, b)
+    assert cpp.plan_cache_size() == 2
+    # an in-place edit of the structure must not reuse the stale schedule
+    d2, i2, p2, _ = G.bidiag(n, np.float64)
+    D2, I2, P2 = to_dev(dev, d2, i2, p2)
+    I3 = I2.clone()
+    x_a = cpp.sptrsv_forward(n, n, D2, I3, P2, True, False, b)
+    I3[1] = 1                                                       # (1,0) -> (1,1): row 1 loses its dependency
+    x_b = cpp.sptrsv_forward(n, n, D2, I3, P2, True, False, b)
+    assert_same(host(x_b), oracle.sptrsv_forward(n, n, d2, host(I3), p2, True, False, host(b)), "after edit")
+    assert not torch.equal(x_a, x_b)
+    cpp.clear_plan_cache()
+
+    with pytest.raises(RuntimeError, match="Long"):
+        cpp.spgemv_forward(n, n, D, I.int(), P, b)
+    with pytest.raises(RuntimeError, match="HIP devices only|same device"):
+        cpp.spdmm_forward(n, n, D, I, P, torch.ones(n, 2, dtype=torch.float64))
+    with pytest.raises(RuntimeError, match="float32 or float64"):
+        cpp.spgemv_forward(n, n, D.half(), I, P, b.half())
+    with pytest.raises(RuntimeError, match="planned"):
+        cpp.set_backward_mode("fastest")
+
+
+def test_install_registers_the_reference_module_name(cpp):
+    import sys
+    saved = sys.modules.pop("numml_torch_cpp", None)
+    try:
+        numml_amd.install()
+        import numml_torch_cpp
+        assert numml_torch_cpp is cpp
+    finally:
+        sys.modules.pop("numml_torch_cpp", None)
+        if saved is not None:
+            sys.modules["numml_torch_cpp"] = saved
