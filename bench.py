@@ -16,6 +16,7 @@ on):
   spmm    fp32 SpMM fwd+bwd, power-law 1M x 1M, ~15M nnz, 64 dense columns
   spgemm  fp64 hash SpGEMM A@A fwd+bwd, 3-D Laplacian 128^3
   sptrsv  fp64 triangular solve fwd+bwd, tril(Poisson 1024^2), 2047 levels
+  transpose  fp32 explicit CSR transpose + its backward on the spmv matrix
   copy    256 MiB device copy (counter calibration / practical bandwidth ceiling)
 
 ``value`` is algorithmic bytes per step / time per step (GB/s) for spmv/spmm,
@@ -307,6 +308,61 @@ class SpTRSV(Workload):
                 "sample": f"{reps} x (sptrsv_forward + sptrsv_backward) of the full workload, serial C oracle"}
 
 
+class Transpose(Workload):
+    """Explicit CSR transpose and its backward on the SpMV matrix.  The sort that
+    builds the transposed structure runs once per sparsity pattern (reported as
+    ``plan_build_ms``); a step is what every later call costs."""
+    name = "transpose"
+
+    def setup(self, dev):
+        import torch
+        from numml_amd import generators as G
+        from numml_amd import _binding
+        self.ext = _binding.ops
+        d, i, p, (rows, cols) = G.poisson2d(2048, np.float32, jitter_seed=0)
+        self.host = (d, i, p, rows, cols)
+        self.g_h = np.random.default_rng(2).standard_normal(d.shape[0]).astype(np.float32)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        self.D, self.I, self.P, self.Gv = t(d), t(i), t(p), t(self.g_h)
+        self.rows, self.cols, nnz = rows, cols, d.shape[0]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = self.ext.csr_transpose_forward(rows, cols, self.D, self.I, self.P)   # builds and caches the plan
+        torch.cuda.synchronize()
+        first_ms = (time.perf_counter() - t0) * 1e3
+        self.perm = out[3]
+        s = 4
+        fwd = nnz * 8 + (cols + 1) * 4 + nnz * s + nnz * (s + 16) + (cols + 1) * 8
+        bwd = nnz * (s + 8) + nnz * s
+        self.bytes_per_step = fwd + bwd
+        self.dominant_bytes = fwd
+        self.dominant_name = "transpose_expand_kernel"
+        self.config = {"workload": "csr_transpose_fwd_bwd_f32_poisson2d_2048", "rows": rows, "nnz": nnz,
+                       "binding": _binding.name, "first_call_ms_incl_plan_build": round(first_ms, 3),
+                       "algorithmic_bytes_per_step": self.bytes_per_step}
+
+    def step(self):
+        out = self.ext.csr_transpose_forward(self.rows, self.cols, self.D, self.I, self.P)
+        return self.ext.csr_transpose_backward(self.Gv, out[3])
+
+    def dominant(self):
+        return self.ext.csr_transpose_forward(self.rows, self.cols, self.D, self.I, self.P)
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        d, i, p, rows, cols = self.host
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            T = oracle.csr_transpose(rows, cols, d, i, p)
+            oracle.csr_transpose_backward(self.g_h, T[3])
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget_s or reps >= 50:
+                break
+        return {"value": self.bytes_per_step * reps / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} x (csr_transpose + csr_transpose_backward) of the full workload, serial C oracle"}
+
+
 class Copy(Workload):
     """Plain device copy of a known size: the calibration run for the rocprofv3
     FETCH_SIZE / WRITE_SIZE counters and the practical HBM ceiling of this part."""
@@ -338,6 +394,7 @@ WORKLOADS = {
     "spmm": SpMM,
     "spgemm": SpGEMM,
     "sptrsv": SpTRSV,
+    "transpose": Transpose,
     "copy": Copy,
 }
 

@@ -79,6 +79,22 @@ int nm_csr_transpose_plan_build(int64_t rows, int64_t cols, int64_t nnz,
                                 void *plan_mem, size_t plan_bytes,
                                 void *work, size_t work_bytes, nm_stream stream);
 
+/* The explicit transpose.  Stands in for csr_transpose_forward
+ * (cpp/sparse_csr.hpp:57-61, cpp/sparse_csr_cpu.cpp:311-367): widens a built
+ * transposed-structure plan of A's pattern to At_indptr (cols + 1), At_indices
+ * and At_to_A_idx (nnz each, int64) and gathers At_data[p] = data[At_to_A_idx[p]].
+ * Rows ascend inside every row of A^T, entries with equal coordinates keep A's
+ * storage order: the arrays equal the reference's bit for bit. */
+int nm_csr_transpose_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                             const void *data, const void *plan_mem,
+                             void *At_data, int64_t *At_indices, int64_t *At_indptr,
+                             int64_t *At_to_A_idx, nm_stream stream);
+
+/* grad_A[At_to_A_idx[p]] = grad_At[p].  Stands in for csr_transpose_backward
+ * (cpp/sparse_csr.hpp:63-65, cpp/sparse_csr_cpu.cpp:369-385). */
+int nm_csr_transpose_backward(nm_dtype dt, int64_t nnz, const void *grad_At,
+                              const int64_t *At_to_A_idx, void *grad_A, nm_stream stream);
+
 /* nm_spgemv_backward on a transposed-structure plan: walks A by column, so
  * grad_x needs neither clearing nor atomics, is summed in ascending row order
  * (the order of cpp/sparse_csr_cpu.cpp:68-73) and is identical on every run.

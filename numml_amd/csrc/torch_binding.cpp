@@ -253,6 +253,42 @@ std::vector<Tensor> spgemv_backward(Tensor grad_z, int A_rows, int A_cols, Tenso
     return {grad_A, grad_x};
 }
 
+// ----------------------------------------------------------------------- transpose
+
+std::vector<Tensor> csr_transpose_forward(int A_rows, int A_columns, Tensor A_data, Tensor A_indices,
+                                          Tensor A_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr});
+    A_data = A_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    const int64_t nnz = A_data.numel();
+    auto plan = transpose_plan(A_indices, A_indptr, A_rows, A_columns, dev);
+    const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
+    Tensor At_data = torch::empty_like(A_data);
+    Tensor At_indices = torch::empty({nnz}, iopt);
+    Tensor At_indptr = torch::empty({(int64_t)A_columns + 1}, iopt);
+    Tensor At_to_A = torch::empty({nnz}, iopt);
+    check(nm_csr_transpose_forward(dtype_of(A_data), A_rows, A_columns, nnz, A_data.data_ptr(),
+                                   plan->mem.data_ptr(), At_data.data_ptr(), At_indices.data_ptr<int64_t>(),
+                                   At_indptr.data_ptr<int64_t>(), At_to_A.data_ptr<int64_t>(),
+                                   current_stream(dev)),
+          "nm_csr_transpose_forward");
+    return {At_data, At_indices, At_indptr, At_to_A};
+}
+
+Tensor csr_transpose_backward(Tensor grad_At, Tensor At_to_A_idx) {
+    const auto dev = need_device({&grad_At, &At_to_A_idx});
+    grad_At = grad_At.contiguous();
+    At_to_A_idx = index_tensor(At_to_A_idx, "At_to_A_idx");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty_like(grad_At);
+    check(nm_csr_transpose_backward(dtype_of(grad_At), grad_At.numel(), grad_At.data_ptr(),
+                                    At_to_A_idx.data_ptr<int64_t>(), grad_A.data_ptr(), current_stream(dev)),
+          "nm_csr_transpose_backward");
+    return grad_A;
+}
+
 // ---------------------------------------------------------------------------- SpMM
 
 Tensor spdmm_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr, Tensor B) {
@@ -457,6 +493,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("spdmm_backward", &spdmm_backward, "Sparse times dense matrix backward");
     m.def("sptrsv_forward", &sptrsv_forward, "Sparse triangular solve forward");
     m.def("sptrsv_backward", &sptrsv_backward, "Sparse triangular solve backward");
+    m.def("csr_transpose_forward", &csr_transpose_forward, "CSR Transpose forward");
+    m.def("csr_transpose_backward", &csr_transpose_backward, "CSR Transpose backward");
     m.def("sptrsv_schedule", &sptrsv_schedule, "(levels, launches per solve) of a triangular pattern");
     m.def("clear_plan_cache", &clear_plan_cache, "Drop every cached structure plan");
     m.def("plan_cache_size", &plan_cache_size, "Number of cached structure plans");

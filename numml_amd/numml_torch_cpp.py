@@ -21,6 +21,7 @@ from . import _lib
 __all__ = [
     "spgemv_forward", "spgemv_backward", "spdmm_forward", "spdmm_backward",
     "spgemm_forward", "spgemm_backward", "sptrsv_forward", "sptrsv_backward",
+    "csr_transpose_forward", "csr_transpose_backward",
     "clear_plan_cache", "plan_cache_size", "sptrsv_schedule",
 ]
 
@@ -188,6 +189,38 @@ def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
 
 
 # --------------------------------------------------------------------- SpMM
+
+def csr_transpose_forward(A_rows, A_columns, A_data, A_indices, A_indptr):
+    """[At_data, At_indices, At_indptr, At_to_A_idx]  (cpp/sparse_csr.hpp:57-61)."""
+    dev = _need_device(A_data, A_indices, A_indptr)
+    A_data = A_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    nnz = A_data.shape[0]
+    with torch.cuda.device(dev):
+        plan = _transpose_plan(A_indices, A_indptr, A_rows, A_columns, dev)
+        At_data = torch.empty_like(A_data)
+        At_indices = torch.empty(nnz, dtype=torch.int64, device=dev)
+        At_indptr = torch.empty(A_columns + 1, dtype=torch.int64, device=dev)
+        At_to_A = torch.empty(nnz, dtype=torch.int64, device=dev)
+        _lib.check(_lib.lib().nm_csr_transpose_forward(
+            _dt(A_data), A_rows, A_columns, nnz, _ptr(A_data), _ptr(plan.mem), _ptr(At_data),
+            _ptr(At_indices), _ptr(At_indptr), _ptr(At_to_A), _stream(dev)), "nm_csr_transpose_forward")
+    return [At_data, At_indices, At_indptr, At_to_A]
+
+
+def csr_transpose_backward(grad_At, At_to_A_idx):
+    """grad_A with grad_A[At_to_A_idx[p]] = grad_At[p]  (cpp/sparse_csr.hpp:63-65)."""
+    dev = _need_device(grad_At, At_to_A_idx)
+    _dt(grad_At)
+    grad_At = grad_At.contiguous()
+    At_to_A_idx = _idx(At_to_A_idx, "At_to_A_idx")
+    with torch.cuda.device(dev):
+        grad_A = torch.empty_like(grad_At)
+        _lib.check(_lib.lib().nm_csr_transpose_backward(
+            _dt(grad_At), grad_At.shape[0], _ptr(grad_At), _ptr(At_to_A_idx), _ptr(grad_A), _stream(dev)),
+            "nm_csr_transpose_backward")
+    return grad_A
+
 
 def spdmm_forward(A_rows, A_cols, A_data, A_indices, A_indptr, B):
     """C = A B, B dense 2-D  (cpp/sparse_csr.hpp:81-85)."""

@@ -19,7 +19,7 @@ import torch
 
 from .._binding import ops as _ext
 
-__all__ = ["SparseCSRTensor", "coo_to_csr", "eye", "spgemv", "spgemm", "spdmm"]
+__all__ = ["SparseCSRTensor", "coo_to_csr", "eye", "diag", "spgemv", "spgemm", "spdmm", "sptranspose"]
 
 
 def _type_error(kind_a, a, kind_b, b):
@@ -97,6 +97,25 @@ class spgemm(torch.autograd.Function):
             ctx.A_shape[0], ctx.A_shape[1], A_data, A_indices, A_indptr,
             ctx.B_shape[0], ctx.B_shape[1], B_data, B_indices, B_indptr)
         return None, grad_A, None, None, None, grad_B, None, None
+
+
+class sptranspose(torch.autograd.Function):
+    """A^T as a new CSR triple; returns ``(At_shape, At_data, At_indices, At_indptr)``.
+    The gradient of At's values goes back through the saved permutation
+    (numml/sparse/_csr.py:333-354)."""
+
+    @staticmethod
+    def forward(ctx, A_shape, A_data, A_indices, A_indptr):
+        At_data, At_indices, At_indptr, At_to_A_idx = _ext.csr_transpose_forward(
+            A_shape[0], A_shape[1], A_data, A_indices, A_indptr)
+        ctx.save_for_backward(At_to_A_idx)
+        ctx.mark_non_differentiable(At_indices, At_indptr)
+        return tuple(A_shape[::-1]), At_data, At_indices, At_indptr
+
+    @staticmethod
+    def backward(ctx, _g_shape, grad_At_data, _g_indices, _g_indptr):
+        (At_to_A_idx,) = ctx.saved_tensors
+        return None, _ext.csr_transpose_backward(grad_At_data, At_to_A_idx), None, None
 
 
 def coo_to_csr(values, row_ind, col_ind, shape, sort=True):
@@ -228,6 +247,25 @@ class SparseCSRTensor(object):
         raise RuntimeError(f"invalid tensor found for sparse multiply: mode {x.ndim} tensor found.  "
                            f"Trying to multiply {self.shape} sparse matrix by {x.shape} tensor.")
 
+    def transpose(self):
+        """A^T, computed eagerly as a new CSR matrix (numml/sparse/_csr.py:1074-1087)."""
+        At_shape, At_data, At_indices, At_indptr = sptranspose.apply(
+            self.shape, self.data, self.indices, self.indptr)
+        return SparseCSRTensor((At_data, At_indices, At_indptr), At_shape)
+
+    def hermitian(self):
+        At_shape, At_data, At_indices, At_indptr = sptranspose.apply(
+            self.shape, self.data.conj(), self.indices, self.indptr)
+        return SparseCSRTensor((At_data, At_indices, At_indptr), At_shape)
+
+    @property
+    def T(self):
+        return self.transpose()
+
+    @property
+    def H(self):
+        return self.hermitian()
+
     def __mul__(self, s):
         if isinstance(s, (int, float)) or (isinstance(s, torch.Tensor) and s.ndim == 0):
             return SparseCSRTensor((self.data * s, self.indices, self.indptr), self.shape)
@@ -321,6 +359,9 @@ class SparseCSRTensor(object):
 
 def eye(N, k=0, dtype=torch.float32, device=None):
     """Ones on the k-th diagonal of an N x N matrix (numml/sparse/_csr.py:467-486)."""
+    if abs(k) >= N:
+        raise RuntimeError("Specified bandwidth for eye() is larger than matrix size.  "
+                           f"Got k={abs(k)}, N={N}.")
     n = max(N - abs(k), 0)
     rows = torch.arange(n, dtype=torch.int64) + max(-k, 0)
     cols = rows + k
@@ -330,3 +371,12 @@ def eye(N, k=0, dtype=torch.float32, device=None):
     indptr[1:] = torch.cumsum(counts, 0)
     out = SparseCSRTensor((torch.ones(n, dtype=dtype), cols, indptr), (N, N), clone=False)
     return out if device is None else out.to(device)
+
+
+def diag(x, k=0):
+    """Square matrix with the vector x on its k-th diagonal (numml/sparse/_csr.py:489-508);
+    gradients flow back to x through the stored values."""
+    n = len(x)
+    N = n + abs(k)
+    rows = torch.arange(n, dtype=torch.int64, device=x.device) + max(-k, 0)
+    return SparseCSRTensor((x, (rows, rows + k)), shape=(N, N))

@@ -161,6 +161,15 @@ def csr_transpose(rows, cols, data, indices, indptr):
     return At_data, At_indices, At_indptr, At_to_A
 
 
+def csr_transpose_backward(grad_At, At_to_A_idx):
+    """csr_transpose_backward_cpu, cpp/sparse_csr_cpu.cpp:369-385:
+    grad_A[At_to_A_idx[i]] = grad_At[i]."""
+    grad_At, At_to_A_idx = _vals(grad_At), _idx(At_to_A_idx)
+    grad_A = np.empty_like(grad_At)
+    grad_A[At_to_A_idx] = grad_At
+    return grad_A
+
+
 def sptrsv_forward(rows, cols, data, indices, indptr, lower, unit, b):
     """sptrsv_forward_cpu, cpp/sparse_csr_cpu.cpp:652-723."""
     data, indices, indptr = _vals(data), _idx(indices), _idx(indptr)

@@ -124,8 +124,16 @@ def test_ref_products(dtype, seed):
     for a, b in zip(oracle.spgemm_backward(gCs, C1[1], C1[2], r, k, ad, ai, ap, k, c, bd, bi, bp),
                     ref.call("spgemm_backward", gCs, C1[1], C1[2], r, k, ad, ai, ap, k, c, bd, bi, bp)):
         same(a, b, "spgemm backward")
-    for a, b in zip(oracle.csr_transpose(r, k, ad, ai, ap), ref.call("csr_transpose_forward", r, k, ad, ai, ap)):
+    T1 = oracle.csr_transpose(r, k, ad, ai, ap)
+    for a, b in zip(T1, ref.call("csr_transpose_forward", r, k, ad, ai, ap)):
         same(a, b, "transpose")
+    gT = rng.standard_normal(ad.shape[0]).astype(dtype)
+    same(oracle.csr_transpose_backward(gT, T1[3]), ref.call("csr_transpose_backward", gT, T1[3]),
+         "transpose backward")
+    # the transpose of the transpose is the matrix itself; its permutation undoes the first
+    T2 = oracle.csr_transpose(k, r, T1[0], T1[1], T1[2])
+    same(T2[0], ad, "(A^T)^T data"), same(T2[1], ai, "(A^T)^T indices"), same(T2[2], ap, "(A^T)^T indptr")
+    same(T1[3][T2[3]], np.arange(ad.shape[0]), "permutations compose to the identity")
 
 
 @needs_ref
