@@ -15,6 +15,11 @@
 //             ascending like the reference's.
 // Rows too long for an LDS table spill to a dense accumulator in global memory
 // (one slice of B_cols entries per spill workgroup).
+// Short rows take a merge path instead of hashing: when a row of A and every row
+// of B it names have at most 8 entries (stencil and aggregation operators), eight
+// lanes each hold one B row, sorted as stored, and the group repeatedly emits the
+// smallest head column; the lanes whose head equals it contribute their product,
+// summed in lane order = the order of A's row.  These rows never enter the bins.
 //
 // Backward: eight lanes per row i of A; for each entry (i,k) the lanes share row
 // k of B, find its columns in row i of C (staged in LDS) by bisection, and form
@@ -46,6 +51,10 @@ constexpr int32_t kNumLimit[3] = {32, 512, 4096};     // on the exact row length
 // table sizes per bin
 constexpr int kSymTable0 = 128, kSymTable1 = 1024, kSymTable2 = 16384;
 constexpr int kNumTable0 = 64, kNumTable1 = 1024, kNumTable2 = 8192;
+
+constexpr int kMergeCap = 8;                  // longest A row and B row of the merge path
+constexpr int32_t kColEnd = 0x7fffffff;       // past-the-end column of a staged B row
+constexpr int32_t kMergedKey = -1;            // binning key of a row the merge path has taken
 
 struct Work {
     int32_t *key;      // [rows] binning key (product bound, then exact length)
@@ -96,32 +105,262 @@ template <int G> __device__ __forceinline__ int group_total(int v, int *s_red) {
 
 // ---- binning ---------------------------------------------------------------
 
-// key[i] = min(sum of B row lengths over A's row i, INT32_MAX); bins[b] counts.
-__global__ void product_bound_kernel(int64_t rows, const int64_t *__restrict__ A_indices,
-                                     const int64_t *__restrict__ A_indptr,
-                                     const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows; i += stride) {
-        int64_t ub = 0;
-        const int64_t e = A_indptr[i + 1];
-        for (int64_t jj = A_indptr[i]; jj < e; ++jj) {
-            const int64_t j = A_indices[jj];
-            ub += B_indptr[j + 1] - B_indptr[j];
+// ---- merge path (short rows) ---------------------------------------------------
+//
+// Lane layout: a merge group is the 8 lanes of equal parity in a 16-lane DPP row,
+// so a wavefront holds 8 groups.  Neighbours inside a group are two lanes apart:
+// rotations by 2, 4 and 8 inside the DPP row reduce over the group, and a shift by
+// 2 feeds lane k the value of lane k-1 of its group with a hardware zero for k = 0.
+
+__device__ __forceinline__ int merge_lane() { return (threadIdx.x & 15) >> 1; }
+__device__ __forceinline__ int merge_group() { return ((threadIdx.x & 63) >> 4) * 2 + (threadIdx.x & 1); }
+
+__device__ __forceinline__ int32_t merge_min(int32_t v) {
+    v = min(v, nm::dpp_move<0x122>(v));   // row_ror 2
+    v = min(v, nm::dpp_move<0x124>(v));   // row_ror 4
+    v = min(v, nm::dpp_move<0x128>(v));   // row_ror 8
+    return v;
+}
+__device__ __forceinline__ int32_t merge_max(int32_t v) {
+    v = max(v, nm::dpp_move<0x122>(v));
+    v = max(v, nm::dpp_move<0x124>(v));
+    v = max(v, nm::dpp_move<0x128>(v));
+    return v;
+}
+__device__ __forceinline__ int32_t merge_sum(int32_t v) {
+    v += nm::dpp_move<0x122>(v);
+    v += nm::dpp_move<0x124>(v);
+    v += nm::dpp_move<0x128>(v);
+    return v;
+}
+
+// True when some merge group of the wavefront has three or more of its lanes set
+// in `lanes` (a ballot).  Scalar work: the two parities are separated, which
+// leaves each group's bits at the even positions of a 16-bit field; the lowest
+// set bit of every field is cleared twice (bit 15, free, stops the borrow) and
+// anything left means three.
+__device__ __forceinline__ bool merge_three_hits(unsigned long long lanes) {
+    constexpr unsigned long long kEven = 0x5555555555555555ull, kLow = 0x0001000100010001ull,
+                                 kTop = 0x8000800080008000ull;
+    unsigned long long e = lanes & kEven, o = (lanes >> 1) & kEven;
+    e &= (e | kTop) - kLow;
+    o &= (o | kTop) - kLow;
+    e &= (e | kTop) - kLow;
+    o &= (o | kTop) - kLow;
+    return (e | o) != 0;
+}
+
+constexpr int kMergeRows = kBlock / 8;   // rows of A per workgroup pass
+constexpr int kMergeStride = kBlock + 1; // slot stride of the staged B rows (odd: slots of one lane fall in different banks)
+
+// Staging of the B rows of a wavefront into LDS.  Every lane owns one B row
+// (start `bb`, `len` <= kMergeCap entries, 0 when it has none).  Loading them
+// lane by lane would touch ~30 cache lines per instruction and use 8 bytes of
+// each; instead the wavefront loads one LEG at a time: in pass u the eight lanes
+// of sub-wavefront g read the eight entries of the row owned by lane u of group
+// g, so an instruction reads eight contiguous 64-byte pieces -- and for banded
+// matrices, where neighbouring rows of A name neighbouring rows of B, one
+// contiguous span.  Entry k of the row owned by thread t lands in slot
+// [k * kMergeStride + t]; slot kMergeCap is the end marker.
+//
+// The loads are unconditional: a lane with nothing to fetch reads `safe` (8 valid
+// bytes) and discards the result.  Predicated loads would sit in their own
+// branches, each followed by the wait for its data, i.e. one memory round trip
+// per leg instead of one for all of them.
+template <typename T, bool VALUES>
+__device__ __forceinline__ void merge_stage(int64_t bb, int len, const int64_t *__restrict__ B_indices,
+                                            const T *__restrict__ B_data, const int64_t *__restrict__ safe,
+                                            int64_t *s_bb, int32_t *s_len, int32_t *s_col, T *s_val) {
+    s_bb[threadIdx.x] = bb;
+    s_len[threadIdx.x] = len;
+    s_col[kMergeCap * kMergeStride + threadIdx.x] = kColEnd;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    const int lane = threadIdx.x & 63, g = lane >> 3, k = lane & 7;
+    const int first = (threadIdx.x & ~63) + (g >> 1) * 16 + (g & 1);   // lane 0 of merge group g
+    int64_t col[kMergeCap];
+    T val[kMergeCap];
+    bool have[kMergeCap];
+#pragma unroll
+    for (int u = 0; u < kMergeCap; ++u) {
+        const int owner = first + 2 * u;
+        const int64_t obb = s_bb[owner];
+        have[u] = k < s_len[owner];
+        col[u] = *(have[u] ? B_indices + obb + k : safe);
+        if (VALUES) val[u] = *(have[u] ? B_data + obb + k : reinterpret_cast<const T *>(safe));
+    }
+#pragma unroll
+    for (int u = 0; u < kMergeCap; ++u) {
+        const int owner = first + 2 * u;
+        s_col[k * kMergeStride + owner] = have[u] ? (int32_t)col[u] : kColEnd;
+        if (VALUES) s_val[k * kMergeStride + owner] = have[u] ? val[u] : T(0);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+}
+
+// First kernel of the symbolic phase, over all rows in their natural order.  Eight
+// lanes per row gather the lengths of the B rows it names.  Rows that qualify for
+// the merge path are counted here (key = kMergedKey); for the others key[i] is the
+// product bound min(sum of B row lengths, 2^31 - 8) that the hash path bins on.
+__global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
+    int64_t rows, int64_t nbatch_padded, const int64_t *__restrict__ A_indices,
+    const int64_t *__restrict__ A_indptr, const int64_t *__restrict__ B_indices,
+    const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key, int64_t *__restrict__ C_count) {
+    __shared__ int32_t s_col[(kMergeCap + 1) * kMergeStride];
+    __shared__ int64_t s_bb[kBlock];
+    __shared__ int32_t s_len[kBlock];
+    const int gl = merge_lane();
+    const int64_t batch = nm::xcd_tile(blockIdx.x, nbatch_padded);
+    const int64_t row = batch * kMergeRows + (threadIdx.x >> 6) * 8 + merge_group();
+    const bool live = row < rows;
+    const int64_t ab = live ? A_indptr[row] : 0, ae = live ? A_indptr[row + 1] : 0;
+    int64_t ub = 0, my_bb = 0;
+    int32_t mx = 0, my_len = 0;
+    for (int64_t a = ab + gl; a < ae; a += 8) {
+        const int64_t j = A_indices[a];
+        const int64_t bb = B_indptr[j], len = B_indptr[j + 1] - bb;
+        ub += len;
+        const int32_t l32 = (int32_t)(len > kMergeCap + 1 ? kMergeCap + 1 : len);
+        mx = max(mx, l32);
+        if (a - ab < 8) {
+            my_bb = bb;
+            my_len = l32;
         }
-        key[i] = (int32_t)(ub > 0x7fffffff ? 0x7fffffff : ub);
+    }
+    const int32_t ubc = merge_sum((int32_t)(ub > 0x0fffffff ? 0x0fffffff : ub));
+    const bool merge = live && (ae - ab) <= kMergeCap && merge_max(mx) <= kMergeCap;
+    if (live && !merge && gl == 0) key[row] = ubc;
+    merge_stage<float, false>(my_bb, merge ? my_len : 0, B_indices, nullptr, A_indptr, s_bb, s_len, s_col, nullptr);
+    const int32_t *pc = s_col + threadIdx.x;
+    int32_t cur = *pc;
+    int cnt = 0, it = 0;
+    for (;;) {
+        const int32_t m = merge_min(cur);
+        const bool open = m != kColEnd;
+        if (__ballot(open) == 0) break;
+        ++it;
+        if (open) cnt = it;   // an open group emits one column per pass
+        if (cur == m && open) {
+            pc += kMergeStride;
+            cur = *pc;
+        }
+    }
+    if (merge && gl == 0) {
+        C_count[row] = cnt;
+        key[row] = kMergedKey;
     }
 }
 
-// key[i] = C_indptr[i+1] - C_indptr[i]
+// Numeric counterpart: rows marked kMergedKey are produced here, in natural order.
+// The B rows are staged in LDS (columns and values); each pass emits the smallest head column and the sum of the
+// matching products, accumulated from +0.0 in lane order, which is the order in
+// which the serial loop adds them (cpp/sparse_csr_cpu.cpp:193-200).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void numeric_front_kernel(
+    int64_t rows, int64_t nbatch_padded, const int32_t *__restrict__ key, const T *__restrict__ A_data,
+    const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr, const T *__restrict__ B_data,
+    const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
+    const int64_t *__restrict__ C_indptr, int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
+    __shared__ int32_t s_col[(kMergeCap + 1) * kMergeStride];
+    __shared__ T s_val[kMergeCap * kMergeStride];
+    __shared__ int64_t s_bb[kBlock];
+    __shared__ int32_t s_len[kBlock];
+    const int gl = merge_lane();
+    const int64_t batch = nm::xcd_tile(blockIdx.x, nbatch_padded);
+    const int64_t row = batch * kMergeRows + (threadIdx.x >> 6) * 8 + merge_group();
+    // the row's bounds are requested together with its key: one memory round trip instead of two
+    const bool live = row < rows;
+    const int32_t my_key = live ? key[row] : 0;
+    const int64_t ab0 = live ? A_indptr[row] : 0, ae0 = live ? A_indptr[row + 1] : 0;
+    const int64_t out0 = live ? C_indptr[row] : 0;
+    const bool merge = live && my_key == kMergedKey;
+    if (__ballot(merge) == 0) return;   // wavefront-uniform; no workgroup barrier below
+    const int64_t ab = merge ? ab0 : 0, ae = merge ? ae0 : 0;
+    const bool mine = ab + gl < ae;
+    const T av_raw = *(mine ? A_data + ab + gl : reinterpret_cast<const T *>(A_indptr));
+    const int64_t j = mine ? *(A_indices + ab + gl) : 0;
+    const T av = mine ? av_raw : T(0);
+    const int64_t *bp = mine ? B_indptr + j : A_indptr;   // A_indptr: any two readable entries
+    const int64_t bb = bp[0];
+    const int my_len = mine ? (int)(bp[1] - bb) : 0;
+    merge_stage<T, true>(bb, my_len, B_indices, B_data, A_indptr, s_bb, s_len, s_col, s_val);
+    // lanes that take part in the ordered sum: the longest row of A in this wavefront
+    int steps = 1;
+#pragma unroll
+    for (int q = kMergeCap; q > 1; --q)
+        if (steps == 1 && __ballot((ae - ab) >= q) != 0) steps = q;
+    // Emitted entries pass through a ring of 8 per group so that the group writes
+    // them 8 at a time (one 64-byte piece per array) instead of lane by lane.
+    // The ring reuses the exchange arrays of merge_stage, which are dead by now; a
+    // wavefront's ring entries and its exchange entries are the same 64 slots.
+    static_assert(sizeof(T) <= sizeof(int64_t), "ring values alias s_bb");
+    int32_t *s_oc = s_len;
+    T *s_ov = reinterpret_cast<T *>(s_bb);
+    const int ring = ((threadIdx.x >> 6) * 8 + merge_group()) * 8;
+    int emitted = 0;   // entries of this row produced so far
+    auto flush = [&](int base) {
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        const int e = base + gl;
+        if (e < emitted) {
+            C_indices[out0 + e] = (int64_t)s_oc[ring + gl];
+            C_data[out0 + e] = s_ov[ring + gl];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    };
+    const int32_t *pc = s_col + threadIdx.x;   // this lane's head column / value slots
+    const T *pv = s_val + threadIdx.x;
+    int32_t cur = *pc;
+    T curv = av * *pv;
+    int it = 0;
+    for (;;) {
+        const int32_t m = merge_min(cur);
+        const bool open = m != kColEnd;
+        if (__ballot(open) == 0) break;
+        const bool hit = cur == m && open;
+        const T x = hit ? curv : T(0);
+        T t;
+        if (__ballot(merge_sum(hit ? 1 : 0) > 2) == 0) {
+            // at most two products per entry anywhere in the wavefront: a sum of two
+            // terms (and exact zeros) does not depend on the order of the additions
+            t = x + nm::dpp_move_zero<0x122>(x);
+            t += nm::dpp_move_zero<0x124>(t);
+            t += nm::dpp_move_zero<0x128>(t);
+        } else {
+            t = T(0);
+#pragma unroll
+            for (int q = 0; q < kMergeCap; ++q) {
+                if (q >= steps) break;
+                t = x + nm::dpp_move_zero<0x112>(t);   // row_shr 2: previous lane of the group, 0 for the first
+            }
+        }
+        // every group that is still open has emitted exactly `it` entries so far
+        if (gl == steps - 1 && open) {
+            s_oc[ring + (it & 7)] = m;
+            s_ov[ring + (it & 7)] = t;
+        }
+        ++it;
+        if (open) emitted = it;
+        if ((it & 7) == 0) flush(it - 8);
+        if (hit) {
+            pc += kMergeStride;
+            pv += kMergeStride;
+            cur = *pc;
+            curv = av * (cur != kColEnd ? *pv : T(0));   // no value slot behind the end marker
+        }
+    }
+    if (it & 7) flush(it & ~7);
+}
+
+// key[i] = C_indptr[i+1] - C_indptr[i], except for rows the merge path has taken
 __global__ void row_length_kernel(int64_t rows, const int64_t *__restrict__ C_indptr,
                                   int32_t *__restrict__ key) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows; i += stride)
-        key[i] = (int32_t)(C_indptr[i + 1] - C_indptr[i]);
+        if (key[i] != kMergedKey) key[i] = (int32_t)(C_indptr[i + 1] - C_indptr[i]);
 }
 
+// negative keys (rows taken by the merge path) belong to no bin
 __device__ __forceinline__ int bin_of(int32_t k, int32_t l0, int32_t l1, int32_t l2) {
-    return k <= l0 ? 0 : (k <= l1 ? 1 : (k <= l2 ? 2 : 3));
+    return k < 0 ? -1 : (k <= l0 ? 0 : (k <= l1 ? 1 : (k <= l2 ? 2 : 3)));
 }
 
 __global__ void bin_clear_kernel(int32_t *bins) {
@@ -702,11 +941,10 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     if (int rc = nm::fill_async(C_indptr + A_rows, 1, (int64_t)0, s)) return rc;
     if (A_rows == 0) return NM_OK;
 
-    int64_t grid = nm::ceil_div(A_rows, kBlock);
-    if (grid > 65536) grid = 65536;
-    hipLaunchKernelGGL(product_bound_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_indices,
-                       A_indptr, B_indptr, w.key);
-    NM_LAUNCH_CHECK("product_bound_kernel");
+    const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
+    hipLaunchKernelGGL(symbolic_front_kernel, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
+                       A_indices, A_indptr, B_indices, B_indptr, w.key, C_indptr);
+    NM_LAUNCH_CHECK("symbolic_front_kernel");
     if (int rc = bin_rows(A_rows, kSymLimit, w, s)) return rc;
 
     hipLaunchKernelGGL((symbolic_hash_kernel<8, kSymTable0>), dim3(kPersistGrid), dim3(kBlock), 0, s, 0, w.bins,
@@ -744,6 +982,16 @@ extern "C" int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, in
     hipLaunchKernelGGL(row_length_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, C_indptr, w.key);
     NM_LAUNCH_CHECK("row_length_kernel");
     if (int rc = bin_rows(A_rows, kNumLimit, w, s)) return rc;
+    const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
+    if (dt == NM_F32)
+        hipLaunchKernelGGL(numeric_front_kernel<float>, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
+                           w.key, (const float *)A_data, A_indices, A_indptr, (const float *)B_data, B_indices,
+                           B_indptr, C_indptr, C_indices, (float *)C_data);
+    else
+        hipLaunchKernelGGL(numeric_front_kernel<double>, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
+                           w.key, (const double *)A_data, A_indices, A_indptr, (const double *)B_data, B_indices,
+                           B_indptr, C_indptr, C_indices, (double *)C_data);
+    NM_LAUNCH_CHECK("numeric_front_kernel");
     if (dt == NM_F32)
         return launch_numeric<float>(w, B_cols, A_data, A_indices, A_indptr, B_data, B_indices, B_indptr,
                                      C_indptr, C_indices, C_data, s);
