@@ -16,6 +16,7 @@ on):
   spmm    fp32 SpMM fwd+bwd, power-law 1M x 1M, ~15M nnz, 64 dense columns
   spgemm  fp64 hash SpGEMM A@A fwd+bwd, 3-D Laplacian 128^3
   sptrsv  fp64 triangular solve fwd+bwd, tril(Poisson 1024^2), 2047 levels
+  lincomb    fp32 A - B (splincomb) + its backward, both on the spmv matrix pattern
   transpose  fp32 explicit CSR transpose + its backward on the spmv matrix
   copy    256 MiB device copy (counter calibration / practical bandwidth ceiling)
 
@@ -363,6 +364,58 @@ class Transpose(Workload):
                 "sample": f"{reps} x (csr_transpose + csr_transpose_backward) of the full workload, serial C oracle"}
 
 
+class Lincomb(Workload):
+    """C = A - B with its backward, both operands the SpMV matrix pattern (so nnz(C) = nnz)."""
+    name = "lincomb"
+
+    def setup(self, dev):
+        import torch
+        from numml_amd import generators as G
+        from numml_amd import _binding
+        self.ext = _binding.ops
+        d, i, p, (rows, cols) = G.poisson2d(2048, np.float32, jitter_seed=0)
+        d2 = G.poisson2d(2048, np.float32, jitter_seed=1)[0]
+        self.host = (d, d2, i, p, rows, cols)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        self.D, self.D2, self.I, self.P = t(d), t(d2), t(i), t(p)
+        self.one, self.mone = torch.tensor(1.0), torch.tensor(-1.0)
+        self.rows, self.cols, nnz = rows, cols, d.shape[0]
+        self.g_h = np.random.default_rng(2).standard_normal(nnz).astype(np.float32)
+        self.Gv = t(self.g_h)
+        s, ptr = 4, (rows + 1) * 8
+        sym = 2 * (nnz * 8 + ptr) + ptr                       # both patterns in, row pointer out
+        num = 2 * (nnz * (s + 8) + ptr) + ptr + nnz * (s + 8)   # both matrices in, C out
+        bwd = 3 * (nnz * 8 + ptr) + nnz * s + 2 * nnz * s       # three patterns and grad_C in, two gradients out
+        self.bytes_per_step = sym + num + bwd
+        self.dominant_bytes = sym + num
+        self.dominant_name = "lincomb_kernel (count pass, scan, fill pass)"
+        self.config = {"workload": "splincomb_fwd_bwd_f32_poisson2d_2048", "rows": rows, "nnz": nnz,
+                       "binding": _binding.name, "algorithmic_bytes_per_step": self.bytes_per_step}
+
+    def step(self):
+        C = self.dominant()
+        return self.ext.splincomb_backward(self.rows, self.cols, self.one, self.D, self.I, self.P, self.mone,
+                                           self.D2, self.I, self.P, self.Gv, C[1], C[2])
+
+    def dominant(self):
+        return self.ext.splincomb_forward(self.rows, self.cols, self.one, self.D, self.I, self.P, self.mone,
+                                          self.D2, self.I, self.P)
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        d, d2, i, p, rows, cols = self.host
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            C = oracle.splincomb_forward(rows, cols, 1.0, d, i, p, -1.0, d2, i, p)
+            oracle.splincomb_backward(rows, cols, 1.0, d, i, p, -1.0, d2, i, p, self.g_h, C[1], C[2])
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget_s or reps >= 50:
+                break
+        return {"value": self.bytes_per_step * reps / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} x (splincomb_forward + splincomb_backward) of the full workload, serial C oracle"}
+
+
 class Copy(Workload):
     """Plain device copy of a known size: the calibration run for the rocprofv3
     FETCH_SIZE / WRITE_SIZE counters and the practical HBM ceiling of this part."""
@@ -395,6 +448,7 @@ WORKLOADS = {
     "spgemm": SpGEMM,
     "sptrsv": SpTRSV,
     "transpose": Transpose,
+    "lincomb": Lincomb,
     "copy": Copy,
 }
 

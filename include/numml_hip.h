@@ -224,6 +224,71 @@ int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz,
                     double alpha, const void *a, const void *b, void *out,
                     nm_stream stream);
 
+/* ------------------------------------------------- linear combination
+ * C = alpha A + beta B for two matrices of one shape; a column stored by either
+ * operand is stored by C (also when the sum is 0), columns ascending.  Stands in
+ * for splincomb_forward (cpp/sparse_csr.hpp:67-72, cpp/sparse_csr_cpu.cpp:387-481),
+ * in two calls like the product: _symbolic fills C_indptr (rows + 1), the caller
+ * reads nnz(C) = C_indptr[rows] and allocates, _numeric fills C_indices and
+ * C_data.  `workspace` holds nm_splincomb_workspace_bytes(rows) bytes.  alpha
+ * and beta are rounded to the value type before use, as the reference does
+ * (alpha.item<scalar_t>()). */
+int nm_splincomb_workspace_bytes(int64_t rows, size_t *bytes);
+
+int nm_splincomb_symbolic(int64_t rows,
+                          const int64_t *A_indices, const int64_t *A_indptr,
+                          const int64_t *B_indices, const int64_t *B_indptr,
+                          int64_t *C_indptr, void *workspace, size_t workspace_bytes,
+                          nm_stream stream);
+
+int nm_splincomb_numeric(nm_dtype dt, int64_t rows,
+                         double alpha, const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,
+                         double beta, const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
+                         const int64_t *C_indptr, int64_t *C_indices, void *C_data,
+                         nm_stream stream);
+
+/* grad_A[k] = alpha * grad_C at A's coordinate, grad_B likewise with beta.  Stands
+ * in for splincomb_backward (cpp/sparse_csr.hpp:74-79,
+ * cpp/sparse_csr_cpu.cpp:483-560).  Either output may be NULL. */
+int nm_splincomb_backward(nm_dtype dt, int64_t rows,
+                          double alpha, const int64_t *A_indices, const int64_t *A_indptr,
+                          double beta, const int64_t *B_indices, const int64_t *B_indptr,
+                          const void *grad_C, const int64_t *C_indices, const int64_t *C_indptr,
+                          void *grad_A, void *grad_B, nm_stream stream);
+
+/* ------------------------------------------ dense copy, row sums, diagonal
+ * dense[i, j] = data[k] on a zero background (row stride ld >= cols); stands in for
+ * csr_to_dense_forward (cpp/sparse_csr_cpu.cpp:1052-1076).  The backward gathers
+ * grad_A[k] = grad_dense[i, j] (csr_to_dense_backward, :1078-1104). */
+int nm_csr_to_dense_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                            const void *data, const int64_t *indices, const int64_t *indptr,
+                            void *dense, int64_t ld, nm_stream stream);
+
+int nm_csr_to_dense_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                             const void *grad_dense, int64_t ld,
+                             const int64_t *indices, const int64_t *indptr,
+                             void *grad_A, nm_stream stream);
+
+/* x[i] = sum of the stored values of row i, added in storage order for rows that
+ * fit the workgroup's LDS tile (csr_row_sum_forward, cpp/sparse_csr_cpu.cpp:1106-1131);
+ * backward grad_A[k] = g[row(k)] (csr_row_sum_backward, :1133-1156). */
+int nm_csr_row_sum_forward(nm_dtype dt, int64_t rows, int64_t nnz,
+                           const void *data, const int64_t *indptr, void *x, nm_stream stream);
+
+int nm_csr_row_sum_backward(nm_dtype dt, int64_t rows, int64_t nnz,
+                            const int64_t *indptr, const void *g, void *grad_A, nm_stream stream);
+
+/* x[i] = stored entry (i, i) or 0 (csr_extract_diagonal_forward,
+ * cpp/sparse_csr_cpu.cpp:1158-1186; x has `rows` entries); backward grad_A = 0
+ * except g[i] on the diagonal entries (csr_extract_diagonal_backward, :1188-1213). */
+int nm_csr_extract_diagonal_forward(nm_dtype dt, int64_t rows, int64_t nnz,
+                                    const void *data, const int64_t *indices, const int64_t *indptr,
+                                    void *x, nm_stream stream);
+
+int nm_csr_extract_diagonal_backward(nm_dtype dt, int64_t rows, int64_t nnz,
+                                     const int64_t *indices, const int64_t *indptr,
+                                     const void *g, void *grad_A, nm_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -49,6 +49,18 @@ _SIGNATURES = {
     "nm_csr_transpose_forward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                  _c_ptr],
     "nm_csr_transpose_backward": [_c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_splincomb_workspace_bytes": [_c_i64, ctypes.POINTER(_c_size)],
+    "nm_splincomb_symbolic": [_c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr],
+    "nm_splincomb_numeric": [_c_int, _c_i64, _c_dbl, _c_ptr, _c_ptr, _c_ptr, _c_dbl, _c_ptr, _c_ptr, _c_ptr,
+                             _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_splincomb_backward": [_c_int, _c_i64, _c_dbl, _c_ptr, _c_ptr, _c_dbl, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                              _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_csr_to_dense_forward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
+    "nm_csr_to_dense_backward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_csr_row_sum_forward": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_csr_row_sum_backward": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_csr_extract_diagonal_forward": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_csr_extract_diagonal_backward": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_masked_outer": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_dbl, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
 

@@ -36,7 +36,7 @@ int fail(int code, const char *fmt, ...);
         if (!(cond)) return ::nm::fail(NM_ERR_INVALID, __VA_ARGS__);              \
     } while (0)
 
-inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Grid sizes are 32-bit in HIP; every launcher caps its 1-D grid below this
 // and the kernels stride.

@@ -49,7 +49,10 @@ __device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ indptr
     }
 }
 
-template <typename T, int BLOCK, int R, int CAP>
+// UNIT: x is taken as all ones and not read, which makes y the row sums
+// (cpp/sparse_csr_cpu.cpp:1121-1127); a * 1 == a exactly, so the summation is
+// the same storage-order sum.
+template <typename T, int BLOCK, int R, int CAP, bool UNIT = false>
 __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
     int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
     const int64_t *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y) {
@@ -73,17 +76,21 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
             const int64_t *__restrict__ ci = indices + base;
             int k = threadIdx.x;
             for (; k + 3 * BLOCK < n; k += 4 * BLOCK) {
-                const int64_t c0 = nm::stream_load(ci + k), c1 = nm::stream_load(ci + k + BLOCK),
-                              c2 = nm::stream_load(ci + k + 2 * BLOCK), c3 = nm::stream_load(ci + k + 3 * BLOCK);
                 const T a0 = nm::stream_load(d + k), a1 = nm::stream_load(d + k + BLOCK),
                         a2 = nm::stream_load(d + k + 2 * BLOCK), a3 = nm::stream_load(d + k + 3 * BLOCK);
-                const T x0 = x[c0], x1 = x[c1], x2 = x[c2], x3 = x[c3];
+                T x0 = T(1), x1 = T(1), x2 = T(1), x3 = T(1);
+                if (!UNIT) {
+                    const int64_t c0 = nm::stream_load(ci + k), c1 = nm::stream_load(ci + k + BLOCK),
+                                  c2 = nm::stream_load(ci + k + 2 * BLOCK), c3 = nm::stream_load(ci + k + 3 * BLOCK);
+                    x0 = x[c0], x1 = x[c1], x2 = x[c2], x3 = x[c3];
+                }
                 s_prod[k] = a0 * x0;
                 s_prod[k + BLOCK] = a1 * x1;
                 s_prod[k + 2 * BLOCK] = a2 * x2;
                 s_prod[k + 3 * BLOCK] = a3 * x3;
             }
-            for (; k < n; k += BLOCK) s_prod[k] = nm::stream_load(d + k) * x[nm::stream_load(ci + k)];
+            for (; k < n; k += BLOCK)
+                s_prod[k] = nm::stream_load(d + k) * (UNIT ? T(1) : x[nm::stream_load(ci + k)]);
             __syncthreads();
             for (int t = threadIdx.x; t < nr; t += BLOCK) {
                 const int e = s_off[t + 1];
@@ -97,7 +104,7 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
                 const int64_t b = indptr[r0 + t], e = indptr[r0 + t + 1];
                 if (e - b >= kLongRow) continue;
                 T acc = 0;
-                for (int64_t k = b; k < e; ++k) acc += data[k] * x[indices[k]];
+                for (int64_t k = b; k < e; ++k) acc += data[k] * (UNIT ? T(1) : x[indices[k]]);
                 y[r0 + t] = acc;
             }
             // long rows: one wavefront each
@@ -105,7 +112,7 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
                 const int64_t b = indptr[r0 + t], e = indptr[r0 + t + 1];
                 if (e - b < kLongRow) continue;
                 T acc = 0;
-                for (int64_t k = b + lane; k < e; k += kWave) acc += data[k] * x[indices[k]];
+                for (int64_t k = b + lane; k < e; k += kWave) acc += data[k] * (UNIT ? T(1) : x[indices[k]]);
                 acc = nm::wave_sum(acc);
                 if (lane == 0) y[r0 + t] = acc;
             }
@@ -344,6 +351,17 @@ int launch_fwd(int64_t rows, const T *data, const int64_t *indices, const int64_
 }
 
 template <typename T>
+int launch_row_sum(int64_t rows, const T *data, const int64_t *indptr, T *y, hipStream_t s) {
+    constexpr int R = kFwdR, CAP = kFwdCap;
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, R));
+    if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, true>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows,
+                       data, (const int64_t *)nullptr, indptr, (const T *)nullptr, y);
+    NM_LAUNCH_CHECK("spmv_fwd_kernel<unit>");
+    return NM_OK;
+}
+
+template <typename T>
 int launch_bwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *a,
                const T *b, T alpha, T *out_A, T *grad_x, hipStream_t s) {
     constexpr int R = Tile<T>::R, CAP = Tile<T>::CAP;
@@ -373,6 +391,17 @@ extern "C" int nm_spgemv_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_
                                       (double *)y, s);
     }
     return nm::fail(NM_ERR_INVALID, "unknown dtype %d", (int)dt);
+}
+
+extern "C" int nm_csr_row_sum_forward(nm_dtype dt, int64_t rows, int64_t nnz, const void *data,
+                                      const int64_t *indptr, void *x, nm_stream stream) {
+    NM_REQUIRE(rows >= 0 && nnz >= 0, "negative size");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    if (rows == 0) return NM_OK;
+    NM_REQUIRE(indptr && x && (nnz == 0 || data), "null pointer argument");
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F32) return launch_row_sum<float>(rows, (const float *)data, indptr, (float *)x, s);
+    return launch_row_sum<double>(rows, (const double *)data, indptr, (double *)x, s);
 }
 
 extern "C" int nm_spgemv_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,

@@ -1,7 +1,9 @@
-// Structure-changing CSR operations next to the products: the explicit
-// transpose (csr_transpose_forward / _backward of the reference,
-// cpp/sparse_csr_cpu.cpp:311-385).  All of it is streaming integer and copy
-// work, bound by HBM bandwidth.
+// CSR operations next to the products, all streaming integer and copy work bound
+// by HBM bandwidth:
+//   explicit transpose            cpp/sparse_csr_cpu.cpp:311-385
+//   linear combination aA + bB    cpp/sparse_csr_cpu.cpp:387-560
+//   to dense, row sums, diagonal  cpp/sparse_csr_cpu.cpp:1050-1213
+#include "nm_scan.hpp"
 #include "nm_transpose.hpp"
 
 namespace {
@@ -38,6 +40,170 @@ __global__ void transpose_scatter_kernel(int64_t nnz, const T *__restrict__ grad
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < nnz; p += stride)
         grad_A[nm::stream_load(At_to_A + p)] = nm::stream_load(grad_At + p);
+}
+
+// ---- entry-parallel maps over a CSR matrix ---------------------------------------
+//
+// A workgroup owns a tile of kTileRows rows.  Row offsets are staged in LDS, one
+// lane per row spreads the row number over the row's entries, and the entries are
+// then processed lane = entry, so the CSR arrays stream through coalesced while
+// every entry knows its row.  Tiles with more than kTileCap entries (long rows)
+// are walked one row per wavefront instead.
+
+constexpr int kTileRows = 256, kTileCap = 4096;
+
+enum MapOp { kToDense, kFromDense, kDiagBack, kRowSpread };
+
+template <typename T, int OP>
+__device__ __forceinline__ void map_entry(int64_t row, int64_t k, const int64_t *__restrict__ indices,
+                                          const T *__restrict__ src, T *__restrict__ dst, int64_t ld) {
+    if (OP == kToDense) dst[row * ld + indices[k]] = src[k];               // A_d[i][j] = data[k]
+    if (OP == kFromDense) dst[k] = src[row * ld + indices[k]];             // grad_A[k] = grad_Ad[i][j]
+    if (OP == kDiagBack) dst[k] = indices[k] == row ? src[row] : T(0);     // grad_A[k] = g[i] on the diagonal
+    if (OP == kRowSpread) dst[k] = src[row];                               // grad_A[k] = g[i]
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kBlock) void entry_map_kernel(int64_t rows, const int64_t *__restrict__ indices,
+                                                           const int64_t *__restrict__ indptr,
+                                                           const T *__restrict__ src, T *__restrict__ dst,
+                                                           int64_t ld) {
+    __shared__ int32_t s_off[kTileRows + 1];
+    __shared__ uint8_t s_row[kTileCap];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t ntiles = nm::ceil_div(rows, kTileRows), npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t r0 = tile * kTileRows;
+        const int nr = (int)(rows - r0 < kTileRows ? rows - r0 : kTileRows);
+        const int64_t base = indptr[r0];
+        for (int t = threadIdx.x; t <= nr; t += kBlock) {
+            const int64_t d = indptr[r0 + t] - base;
+            s_off[t] = (int32_t)(d > kTileCap ? kTileCap + 1 : d);
+        }
+        __syncthreads();
+        const int n = s_off[nr];
+        if (n <= kTileCap) {
+            for (int t = threadIdx.x; t < nr; t += kBlock)
+                for (int j = s_off[t]; j < s_off[t + 1]; ++j) s_row[j] = (uint8_t)t;
+            __syncthreads();
+            for (int k = threadIdx.x; k < n; k += kBlock)
+                map_entry<T, OP>(r0 + s_row[k], base + k, indices, src, dst, ld);
+        } else {
+            for (int t = wave; t < nr; t += kBlock / 64) {
+                const int64_t e = indptr[r0 + t + 1];
+                for (int64_t k = indptr[r0 + t] + lane; k < e; k += 64)
+                    map_entry<T, OP>(r0 + t, k, indices, src, dst, ld);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// x[i] = the stored entry (i, i), 0 when row i has none (cpp/sparse_csr_cpu.cpp:1170-1186).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void diagonal_kernel(int64_t rows, const T *__restrict__ data,
+                                                          const int64_t *__restrict__ indices,
+                                                          const int64_t *__restrict__ indptr, T *__restrict__ x) {
+    __shared__ int32_t s_off[kTileRows + 1];
+    __shared__ uint8_t s_row[kTileCap];
+    __shared__ T s_x[kTileRows];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t ntiles = nm::ceil_div(rows, kTileRows), npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t r0 = tile * kTileRows;
+        const int nr = (int)(rows - r0 < kTileRows ? rows - r0 : kTileRows);
+        const int64_t base = indptr[r0];
+        for (int t = threadIdx.x; t <= nr; t += kBlock) {
+            const int64_t d = indptr[r0 + t] - base;
+            s_off[t] = (int32_t)(d > kTileCap ? kTileCap + 1 : d);
+        }
+        for (int t = threadIdx.x; t < nr; t += kBlock) s_x[t] = T(0);
+        __syncthreads();
+        const int n = s_off[nr];
+        if (n <= kTileCap) {
+            for (int t = threadIdx.x; t < nr; t += kBlock)
+                for (int j = s_off[t]; j < s_off[t + 1]; ++j) s_row[j] = (uint8_t)t;
+            __syncthreads();
+            for (int k = threadIdx.x; k < n; k += kBlock)
+                if (indices[base + k] == r0 + s_row[k]) s_x[s_row[k]] = data[base + k];
+        } else {
+            for (int t = wave; t < nr; t += kBlock / 64) {
+                const int64_t e = indptr[r0 + t + 1];
+                for (int64_t k = indptr[r0 + t] + lane; k < e; k += 64)
+                    if (indices[k] == r0 + t) s_x[t] = data[k];
+            }
+        }
+        __syncthreads();
+        for (int t = threadIdx.x; t < nr; t += kBlock) x[r0 + t] = s_x[t];
+        __syncthreads();
+    }
+}
+
+// ---- linear combination --------------------------------------------------------------
+//
+// One lane merges one row of A with the same row of B (cpp/sparse_csr_cpu.cpp:428-468).
+// COUNT: only the length of the merged row is produced.
+
+template <typename T, bool COUNT>
+__global__ void lincomb_kernel(int64_t rows, T alpha, const T *__restrict__ A_data,
+                               const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr, T beta,
+                               const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
+                               const int64_t *__restrict__ B_indptr, int64_t *__restrict__ C_indptr,
+                               int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; row < rows; row += stride) {
+        int64_t iA = A_indptr[row], iB = B_indptr[row];
+        const int64_t eA = A_indptr[row + 1], eB = B_indptr[row + 1];
+        int64_t out = COUNT ? 0 : C_indptr[row];
+        while (iA < eA && iB < eB) {
+            const int64_t cA = A_indices[iA], cB = B_indices[iB];
+            if (!COUNT) {
+                C_indices[out] = cA < cB ? cA : cB;
+                C_data[out] = cA < cB ? alpha * A_data[iA]
+                                      : (cA > cB ? beta * B_data[iB] : alpha * A_data[iA] + beta * B_data[iB]);
+            }
+            iA += cA <= cB;
+            iB += cB <= cA;
+            ++out;
+        }
+        if (COUNT) {
+            out += (eA - iA) + (eB - iB);
+            C_indptr[row] = out;
+        } else {
+            for (; iA < eA; ++iA, ++out) {
+                C_indices[out] = A_indices[iA];
+                C_data[out] = alpha * A_data[iA];
+            }
+            for (; iB < eB; ++iB, ++out) {
+                C_indices[out] = B_indices[iB];
+                C_data[out] = beta * B_data[iB];
+            }
+        }
+    }
+}
+
+// grad_X[k] = coef * grad_C at the same coordinate: row of X merged with row of C
+// (cpp/sparse_csr_cpu.cpp:505-552).  Every column of X is present in C.
+template <typename T>
+__global__ void lincomb_back_kernel(int64_t rows, T coef, const int64_t *__restrict__ X_indices,
+                                    const int64_t *__restrict__ X_indptr, const T *__restrict__ gC,
+                                    const int64_t *__restrict__ C_indices, const int64_t *__restrict__ C_indptr,
+                                    T *__restrict__ grad_X) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; row < rows; row += stride) {
+        int64_t iX = X_indptr[row], iC = C_indptr[row];
+        const int64_t eX = X_indptr[row + 1], eC = C_indptr[row + 1];
+        while (iX < eX && iC < eC) {
+            const int64_t cX = X_indices[iX], cC = C_indices[iC];
+            if (cX == cC) grad_X[iX] = gC[iC] * coef;
+            iX += cX <= cC;
+            iC += cC <= cX;
+        }
+    }
 }
 
 inline unsigned grid_for(int64_t n) {
@@ -85,5 +251,167 @@ extern "C" int nm_csr_transpose_backward(nm_dtype dt, int64_t nnz, const void *g
         hipLaunchKernelGGL(transpose_scatter_kernel<double>, dim3(grid_for(nnz)), dim3(kBlock), 0, s, nnz,
                            (const double *)grad_At, At_to_A_idx, (double *)grad_A);
     NM_LAUNCH_CHECK("transpose_scatter_kernel");
+    return NM_OK;
+}
+
+// ---- C ABI of the maps -------------------------------------------------------------
+
+namespace {
+
+template <typename T, int OP>
+int launch_map(int64_t rows, const int64_t *indices, const int64_t *indptr, const void *src, void *dst, int64_t ld,
+               hipStream_t s) {
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, kTileRows));
+    if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+    hipLaunchKernelGGL((entry_map_kernel<T, OP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, indices, indptr,
+                       (const T *)src, (T *)dst, ld);
+    NM_LAUNCH_CHECK("entry_map_kernel");
+    return NM_OK;
+}
+
+template <int OP>
+int map_entry_point(nm_dtype dt, int64_t rows, int64_t nnz, const int64_t *indices, const int64_t *indptr,
+                    const void *src, void *dst, int64_t ld, nm_stream stream) {
+    NM_REQUIRE(rows >= 0 && nnz >= 0, "negative size");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "bad dtype %d", (int)dt);
+    if (rows == 0 || nnz == 0) return NM_OK;
+    NM_REQUIRE(indptr && src && dst && (OP == kRowSpread || indices), "null pointer argument");
+    if (dt == NM_F32) return launch_map<float, OP>(rows, indices, indptr, src, dst, ld, nm::as_stream(stream));
+    return launch_map<double, OP>(rows, indices, indptr, src, dst, ld, nm::as_stream(stream));
+}
+
+}  // namespace
+
+extern "C" int nm_csr_to_dense_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                       const int64_t *indices, const int64_t *indptr, void *dense, int64_t ld,
+                                       nm_stream stream) {
+    NM_REQUIRE(rows >= 0 && cols >= 0 && ld >= cols, "bad dense shape");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "bad dtype %d", (int)dt);
+    NM_REQUIRE(rows == 0 || cols == 0 || dense, "null pointer argument");
+    hipStream_t s = nm::as_stream(stream);
+    if (ld == cols) {
+        const int rc = dt == NM_F32 ? nm::fill_async((float *)dense, rows * cols, 0.0f, s)
+                                    : nm::fill_async((double *)dense, rows * cols, 0.0, s);
+        if (rc) return rc;
+    } else {
+        for (int64_t r = 0; r < rows; ++r) {   // strided output: row by row (rare)
+            const int rc = dt == NM_F32 ? nm::fill_async((float *)dense + r * ld, cols, 0.0f, s)
+                                        : nm::fill_async((double *)dense + r * ld, cols, 0.0, s);
+            if (rc) return rc;
+        }
+    }
+    return map_entry_point<kToDense>(dt, rows, nnz, indices, indptr, data, dense, ld, stream);
+}
+
+extern "C" int nm_csr_to_dense_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *grad_dense,
+                                        int64_t ld, const int64_t *indices, const int64_t *indptr, void *grad_A,
+                                        nm_stream stream) {
+    NM_REQUIRE(cols >= 0 && ld >= cols, "bad dense shape");
+    return map_entry_point<kFromDense>(dt, rows, nnz, indices, indptr, grad_dense, grad_A, ld, stream);
+}
+
+extern "C" int nm_csr_row_sum_backward(nm_dtype dt, int64_t rows, int64_t nnz, const int64_t *indptr, const void *g,
+                                       void *grad_A, nm_stream stream) {
+    return map_entry_point<kRowSpread>(dt, rows, nnz, nullptr, indptr, g, grad_A, 0, stream);
+}
+
+extern "C" int nm_csr_extract_diagonal_backward(nm_dtype dt, int64_t rows, int64_t nnz, const int64_t *indices,
+                                                const int64_t *indptr, const void *g, void *grad_A,
+                                                nm_stream stream) {
+    return map_entry_point<kDiagBack>(dt, rows, nnz, indices, indptr, g, grad_A, 0, stream);
+}
+
+extern "C" int nm_csr_extract_diagonal_forward(nm_dtype dt, int64_t rows, int64_t nnz, const void *data,
+                                               const int64_t *indices, const int64_t *indptr, void *x,
+                                               nm_stream stream) {
+    NM_REQUIRE(rows >= 0 && nnz >= 0, "negative size");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "bad dtype %d", (int)dt);
+    if (rows == 0) return NM_OK;
+    NM_REQUIRE(indptr && x && (nnz == 0 || (data && indices)), "null pointer argument");
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, kTileRows));
+    if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F32)
+        hipLaunchKernelGGL(diagonal_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, rows,
+                           (const float *)data, indices, indptr, (float *)x);
+    else
+        hipLaunchKernelGGL(diagonal_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, rows,
+                           (const double *)data, indices, indptr, (double *)x);
+    NM_LAUNCH_CHECK("diagonal_kernel");
+    return NM_OK;
+}
+
+// ---- C ABI of the linear combination ---------------------------------------------
+
+extern "C" int nm_splincomb_workspace_bytes(int64_t rows, size_t *bytes) {
+    NM_REQUIRE(bytes && rows >= 0, "bad argument");
+    *bytes = nm::scan_scratch_bytes(rows + 1);
+    return NM_OK;
+}
+
+extern "C" int nm_splincomb_symbolic(int64_t rows, const int64_t *A_indices, const int64_t *A_indptr,
+                                     const int64_t *B_indices, const int64_t *B_indptr, int64_t *C_indptr,
+                                     void *workspace, size_t workspace_bytes, nm_stream stream) {
+    NM_REQUIRE(rows >= 0, "negative size");
+    NM_REQUIRE(A_indptr && B_indptr && C_indptr && workspace, "null pointer argument");
+    if (workspace_bytes < nm::scan_scratch_bytes(rows + 1))
+        return nm::fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace_bytes,
+                        nm::scan_scratch_bytes(rows + 1));
+    hipStream_t s = nm::as_stream(stream);
+    if (int rc = nm::fill_async(C_indptr + rows, 1, (int64_t)0, s)) return rc;
+    if (rows == 0) return NM_OK;
+    hipLaunchKernelGGL((lincomb_kernel<float, true>), dim3(grid_for(rows * 4)), dim3(kBlock), 0, s, rows, 0.0f,
+                       (const float *)nullptr, A_indices, A_indptr, 0.0f, (const float *)nullptr, B_indices,
+                       B_indptr, C_indptr, (int64_t *)nullptr, (float *)nullptr);
+    NM_LAUNCH_CHECK("lincomb_kernel<count>");
+    return nm::scan_exclusive_i64(C_indptr, rows + 1, (int64_t *)workspace, s);
+}
+
+extern "C" int nm_splincomb_numeric(nm_dtype dt, int64_t rows, double alpha, const void *A_data,
+                                    const int64_t *A_indices, const int64_t *A_indptr, double beta,
+                                    const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
+                                    const int64_t *C_indptr, int64_t *C_indices, void *C_data, nm_stream stream) {
+    NM_REQUIRE(rows >= 0, "negative size");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "bad dtype %d", (int)dt);
+    if (rows == 0) return NM_OK;
+    NM_REQUIRE(A_indptr && B_indptr && C_indptr, "null pointer argument");
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F32)
+        hipLaunchKernelGGL((lincomb_kernel<float, false>), dim3(grid_for(rows * 4)), dim3(kBlock), 0, s, rows,
+                           (float)alpha, (const float *)A_data, A_indices, A_indptr, (float)beta,
+                           (const float *)B_data, B_indices, B_indptr, const_cast<int64_t *>(C_indptr), C_indices,
+                           (float *)C_data);
+    else
+        hipLaunchKernelGGL((lincomb_kernel<double, false>), dim3(grid_for(rows * 4)), dim3(kBlock), 0, s, rows, alpha,
+                           (const double *)A_data, A_indices, A_indptr, beta, (const double *)B_data, B_indices,
+                           B_indptr, const_cast<int64_t *>(C_indptr), C_indices, (double *)C_data);
+    NM_LAUNCH_CHECK("lincomb_kernel");
+    return NM_OK;
+}
+
+extern "C" int nm_splincomb_backward(nm_dtype dt, int64_t rows, double alpha, const int64_t *A_indices,
+                                     const int64_t *A_indptr, double beta, const int64_t *B_indices,
+                                     const int64_t *B_indptr, const void *grad_C, const int64_t *C_indices,
+                                     const int64_t *C_indptr, void *grad_A, void *grad_B, nm_stream stream) {
+    NM_REQUIRE(rows >= 0, "negative size");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "bad dtype %d", (int)dt);
+    if (rows == 0) return NM_OK;
+    NM_REQUIRE(C_indptr, "null pointer argument");
+    hipStream_t s = nm::as_stream(stream);
+    const unsigned grid = grid_for(rows * 4);
+    for (int side = 0; side < 2; ++side) {
+        void *out = side == 0 ? grad_A : grad_B;
+        if (!out) continue;
+        const int64_t *ind = side == 0 ? A_indices : B_indices, *ptr = side == 0 ? A_indptr : B_indptr;
+        const double coef = side == 0 ? alpha : beta;
+        NM_REQUIRE(ptr != nullptr, "null pointer argument");
+        if (dt == NM_F32)
+            hipLaunchKernelGGL(lincomb_back_kernel<float>, dim3(grid), dim3(kBlock), 0, s, rows, (float)coef, ind,
+                               ptr, (const float *)grad_C, C_indices, C_indptr, (float *)out);
+        else
+            hipLaunchKernelGGL(lincomb_back_kernel<double>, dim3(grid), dim3(kBlock), 0, s, rows, coef, ind, ptr,
+                               (const double *)grad_C, C_indices, C_indptr, (double *)out);
+        NM_LAUNCH_CHECK("lincomb_back_kernel");
+    }
     return NM_OK;
 }

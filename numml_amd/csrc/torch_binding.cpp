@@ -289,6 +289,162 @@ Tensor csr_transpose_backward(Tensor grad_At, Tensor At_to_A_idx) {
     return grad_A;
 }
 
+// ------------------------------------------------------------- linear combination
+
+std::vector<Tensor> splincomb_forward(int rows, int cols, Tensor alpha, Tensor A_data, Tensor A_indices,
+                                      Tensor A_indptr, Tensor beta, Tensor B_data, Tensor B_indices,
+                                      Tensor B_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B_data, &B_indices, &B_indptr});
+    same_dtype(A_data, B_data, "B_data");
+    A_data = A_data.contiguous();
+    B_data = B_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    B_indices = index_tensor(B_indices, "B_indices");
+    B_indptr = index_tensor(B_indptr, "B_indptr");
+    // the reference reads both scalars on the host as well (alpha.item<scalar_t>(),
+    // cpp/sparse_csr_cpu.cpp:413-414); they usually are host tensors already
+    const double a = alpha.item<double>(), b = beta.item<double>();
+    c10::hip::HIPGuard guard(dev.index());
+    size_t bytes = 0;
+    check(nm_splincomb_workspace_bytes(rows, &bytes), "nm_splincomb_workspace_bytes");
+    Tensor work = scratch(bytes, dev);
+    const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
+    Tensor C_indptr = torch::empty({(int64_t)rows + 1}, iopt);
+    nm_stream st = current_stream(dev);
+    check(nm_splincomb_symbolic(rows, A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                                C_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, st),
+          "nm_splincomb_symbolic");
+    const int64_t nnz_c = C_indptr[rows].item<int64_t>();   // C is returned exactly sized
+    Tensor C_indices = torch::empty({nnz_c}, iopt);
+    Tensor C_data = torch::empty({nnz_c}, A_data.options());
+    check(nm_splincomb_numeric(dtype_of(A_data), rows, a, A_data.data_ptr(), A_indices.data_ptr<int64_t>(),
+                               A_indptr.data_ptr<int64_t>(), b, B_data.data_ptr(), B_indices.data_ptr<int64_t>(),
+                               B_indptr.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(),
+                               C_indices.data_ptr<int64_t>(), C_data.data_ptr(), st),
+          "nm_splincomb_numeric");
+    return {C_data, C_indices, C_indptr};
+}
+
+std::vector<Tensor> splincomb_backward(int rows, int cols, Tensor alpha, Tensor A_data, Tensor A_indices,
+                                       Tensor A_indptr, Tensor beta, Tensor B_data, Tensor B_indices,
+                                       Tensor B_indptr, Tensor grad_C_data, Tensor C_indices, Tensor C_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B_data, &B_indices, &B_indptr, &grad_C_data,
+                                  &C_indices, &C_indptr});
+    same_dtype(A_data, B_data, "B_data");
+    same_dtype(A_data, grad_C_data, "grad_C_data");
+    grad_C_data = grad_C_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    B_indices = index_tensor(B_indices, "B_indices");
+    B_indptr = index_tensor(B_indptr, "B_indptr");
+    C_indices = index_tensor(C_indices, "C_indices");
+    C_indptr = index_tensor(C_indptr, "C_indptr");
+    const double a = alpha.item<double>(), b = beta.item<double>();
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty_like(A_data, at::MemoryFormat::Contiguous);
+    Tensor grad_B = torch::empty_like(B_data, at::MemoryFormat::Contiguous);
+    check(nm_splincomb_backward(dtype_of(A_data), rows, a, A_indices.data_ptr<int64_t>(),
+                                A_indptr.data_ptr<int64_t>(), b, B_indices.data_ptr<int64_t>(),
+                                B_indptr.data_ptr<int64_t>(), grad_C_data.data_ptr(), C_indices.data_ptr<int64_t>(),
+                                C_indptr.data_ptr<int64_t>(), grad_A.data_ptr(), grad_B.data_ptr(),
+                                current_stream(dev)),
+          "nm_splincomb_backward");
+    return {grad_A, grad_B};
+}
+
+// ------------------------------------------------- dense copy, row sums, diagonal
+
+Tensor csr_to_dense_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr});
+    A_data = A_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor A_d = torch::empty({A_rows, A_cols}, A_data.options());
+    check(nm_csr_to_dense_forward(dtype_of(A_data), A_rows, A_cols, A_data.numel(), A_data.data_ptr(),
+                                  A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), A_d.data_ptr(),
+                                  A_cols, current_stream(dev)),
+          "nm_csr_to_dense_forward");
+    return A_d;
+}
+
+Tensor csr_to_dense_backward(Tensor grad_Ad, int A_rows, int A_cols, Tensor A_data, Tensor A_indices,
+                             Tensor A_indptr) {
+    const auto dev = need_device({&grad_Ad, &A_data, &A_indices, &A_indptr});
+    same_dtype(A_data, grad_Ad, "grad_Ad");
+    TORCH_CHECK(grad_Ad.dim() == 2 && grad_Ad.size(0) == A_rows && grad_Ad.size(1) == A_cols,
+                "expected a ", A_rows, " x ", A_cols, " gradient, got ", grad_Ad.sizes());
+    int64_t ld = 1;
+    grad_Ad = row_major(grad_Ad, &ld);
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty({A_data.numel()}, A_data.options());
+    check(nm_csr_to_dense_backward(dtype_of(A_data), A_rows, A_cols, A_data.numel(), grad_Ad.data_ptr(),
+                                   std::max<int64_t>(ld, A_cols), A_indices.data_ptr<int64_t>(),
+                                   A_indptr.data_ptr<int64_t>(), grad_A.data_ptr(), current_stream(dev)),
+          "nm_csr_to_dense_backward");
+    return grad_A;
+}
+
+Tensor csr_row_sum_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr});
+    A_data = A_data.contiguous();
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor x = torch::empty({A_rows}, A_data.options());
+    check(nm_csr_row_sum_forward(dtype_of(A_data), A_rows, A_data.numel(), A_data.data_ptr(),
+                                 A_indptr.data_ptr<int64_t>(), x.data_ptr(), current_stream(dev)),
+          "nm_csr_row_sum_forward");
+    return x;
+}
+
+Tensor csr_row_sum_backward(Tensor grad_x, int A_rows, int A_cols, Tensor A_data, Tensor A_indices,
+                            Tensor A_indptr) {
+    const auto dev = need_device({&grad_x, &A_data, &A_indices, &A_indptr});
+    same_dtype(A_data, grad_x, "grad_x");
+    grad_x = grad_x.contiguous();
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty({A_data.numel()}, A_data.options());
+    check(nm_csr_row_sum_backward(dtype_of(A_data), A_rows, A_data.numel(), A_indptr.data_ptr<int64_t>(),
+                                  grad_x.data_ptr(), grad_A.data_ptr(), current_stream(dev)),
+          "nm_csr_row_sum_backward");
+    return grad_A;
+}
+
+Tensor csr_extract_diagonal_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr});
+    A_data = A_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor x = torch::empty({A_rows}, A_data.options());
+    check(nm_csr_extract_diagonal_forward(dtype_of(A_data), A_rows, A_data.numel(), A_data.data_ptr(),
+                                          A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                          x.data_ptr(), current_stream(dev)),
+          "nm_csr_extract_diagonal_forward");
+    return x;
+}
+
+Tensor csr_extract_diagonal_backward(Tensor grad_x, int A_rows, int A_cols, Tensor A_data, Tensor A_indices,
+                                     Tensor A_indptr) {
+    const auto dev = need_device({&grad_x, &A_data, &A_indices, &A_indptr});
+    same_dtype(A_data, grad_x, "grad_x");
+    grad_x = grad_x.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    Tensor grad_A = torch::empty({A_data.numel()}, A_data.options());
+    check(nm_csr_extract_diagonal_backward(dtype_of(A_data), A_rows, A_data.numel(),
+                                           A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                           grad_x.data_ptr(), grad_A.data_ptr(), current_stream(dev)),
+          "nm_csr_extract_diagonal_backward");
+    return grad_A;
+}
+
 // ---------------------------------------------------------------------------- SpMM
 
 Tensor spdmm_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr, Tensor B) {
@@ -495,6 +651,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sptrsv_backward", &sptrsv_backward, "Sparse triangular solve backward");
     m.def("csr_transpose_forward", &csr_transpose_forward, "CSR Transpose forward");
     m.def("csr_transpose_backward", &csr_transpose_backward, "CSR Transpose backward");
+    m.def("splincomb_forward", &splincomb_forward, "Sparse linear combination forward");
+    m.def("splincomb_backward", &splincomb_backward, "Sparse linear combination backward");
+    m.def("csr_to_dense_forward", &csr_to_dense_forward, "CSR to dense forward");
+    m.def("csr_to_dense_backward", &csr_to_dense_backward, "CSR to dense backward");
+    m.def("csr_row_sum_forward", &csr_row_sum_forward, "CSR row sum forward");
+    m.def("csr_row_sum_backward", &csr_row_sum_backward, "CSR row sum backward");
+    m.def("csr_extract_diagonal_forward", &csr_extract_diagonal_forward, "CSR extract diagonal forward");
+    m.def("csr_extract_diagonal_backward", &csr_extract_diagonal_backward, "CSR extract diagonal backward");
     m.def("sptrsv_schedule", &sptrsv_schedule, "(levels, launches per solve) of a triangular pattern");
     m.def("clear_plan_cache", &clear_plan_cache, "Drop every cached structure plan");
     m.def("plan_cache_size", &plan_cache_size, "Number of cached structure plans");

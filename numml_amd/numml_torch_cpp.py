@@ -21,7 +21,9 @@ from . import _lib
 __all__ = [
     "spgemv_forward", "spgemv_backward", "spdmm_forward", "spdmm_backward",
     "spgemm_forward", "spgemm_backward", "sptrsv_forward", "sptrsv_backward",
-    "csr_transpose_forward", "csr_transpose_backward",
+    "csr_transpose_forward", "csr_transpose_backward", "splincomb_forward", "splincomb_backward",
+    "csr_to_dense_forward", "csr_to_dense_backward", "csr_row_sum_forward", "csr_row_sum_backward",
+    "csr_extract_diagonal_forward", "csr_extract_diagonal_backward",
     "clear_plan_cache", "plan_cache_size", "sptrsv_schedule",
 ]
 
@@ -219,6 +221,138 @@ def csr_transpose_backward(grad_At, At_to_A_idx):
         _lib.check(_lib.lib().nm_csr_transpose_backward(
             _dt(grad_At), grad_At.shape[0], _ptr(grad_At), _ptr(At_to_A_idx), _ptr(grad_A), _stream(dev)),
             "nm_csr_transpose_backward")
+    return grad_A
+
+
+def _scalar(v):
+    return float(v.item()) if isinstance(v, torch.Tensor) else float(v)
+
+
+def splincomb_forward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr):
+    """[C_data, C_indices, C_indptr] of alpha A + beta B  (cpp/sparse_csr.hpp:67-72)."""
+    dev = _need_device(A_data, A_indices, A_indptr, B_data, B_indices, B_indptr)
+    _same_dtype(A_data, B_data, "B_data")
+    A_data, B_data = A_data.contiguous(), B_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    B_indices, B_indptr = _idx(B_indices, "B_indices"), _idx(B_indptr, "B_indptr")
+    a, b = _scalar(alpha), _scalar(beta)
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(L.nm_splincomb_workspace_bytes(rows, ctypes.byref(nbytes)), "nm_splincomb_workspace_bytes")
+        work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+        C_indptr = torch.empty(rows + 1, dtype=torch.int64, device=dev)
+        _lib.check(L.nm_splincomb_symbolic(rows, _ptr(A_indices), _ptr(A_indptr), _ptr(B_indices), _ptr(B_indptr),
+                                           _ptr(C_indptr), _ptr(work), nbytes.value, _stream(dev)),
+                   "nm_splincomb_symbolic")
+        nnz_c = int(C_indptr[rows].item())
+        C_indices = torch.empty(nnz_c, dtype=torch.int64, device=dev)
+        C_data = torch.empty(nnz_c, dtype=A_data.dtype, device=dev)
+        _lib.check(L.nm_splincomb_numeric(_dt(A_data), rows, a, _ptr(A_data), _ptr(A_indices), _ptr(A_indptr), b,
+                                          _ptr(B_data), _ptr(B_indices), _ptr(B_indptr), _ptr(C_indptr),
+                                          _ptr(C_indices), _ptr(C_data), _stream(dev)), "nm_splincomb_numeric")
+    return [C_data, C_indices, C_indptr]
+
+
+def splincomb_backward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr,
+                       grad_C_data, C_indices, C_indptr):
+    """[grad_A, grad_B]  (cpp/sparse_csr.hpp:74-79)."""
+    dev = _need_device(A_data, A_indices, A_indptr, B_data, B_indices, B_indptr, grad_C_data, C_indices, C_indptr)
+    _same_dtype(A_data, B_data, "B_data")
+    _same_dtype(A_data, grad_C_data, "grad_C_data")
+    grad_C_data = grad_C_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    B_indices, B_indptr = _idx(B_indices, "B_indices"), _idx(B_indptr, "B_indptr")
+    C_indices, C_indptr = _idx(C_indices, "C_indices"), _idx(C_indptr, "C_indptr")
+    a, b = _scalar(alpha), _scalar(beta)
+    with torch.cuda.device(dev):
+        grad_A = torch.empty(A_data.shape[0], dtype=A_data.dtype, device=dev)
+        grad_B = torch.empty(B_data.shape[0], dtype=B_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_splincomb_backward(
+            _dt(A_data), rows, a, _ptr(A_indices), _ptr(A_indptr), b, _ptr(B_indices), _ptr(B_indptr),
+            _ptr(grad_C_data), _ptr(C_indices), _ptr(C_indptr), _ptr(grad_A), _ptr(grad_B), _stream(dev)),
+            "nm_splincomb_backward")
+    return [grad_A, grad_B]
+
+
+def csr_to_dense_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
+    """Dense A_rows x A_cols copy  (cpp/sparse_csr.hpp:122-126)."""
+    dev = _need_device(A_data, A_indices, A_indptr)
+    A_data = A_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        A_d = torch.empty((A_rows, A_cols), dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_csr_to_dense_forward(
+            _dt(A_data), A_rows, A_cols, A_data.shape[0], _ptr(A_data), _ptr(A_indices), _ptr(A_indptr), _ptr(A_d),
+            A_cols, _stream(dev)), "nm_csr_to_dense_forward")
+    return A_d
+
+
+def csr_to_dense_backward(grad_Ad, A_rows, A_cols, A_data, A_indices, A_indptr):
+    """grad_A[k] = grad_Ad[row(k), col(k)]  (cpp/sparse_csr.hpp:128-133)."""
+    dev = _need_device(grad_Ad, A_data, A_indices, A_indptr)
+    _same_dtype(A_data, grad_Ad, "grad_Ad")
+    if grad_Ad.ndim != 2 or tuple(grad_Ad.shape) != (A_rows, A_cols):
+        raise RuntimeError(f"expected a {A_rows} x {A_cols} gradient, got {tuple(grad_Ad.shape)}")
+    grad_Ad, ld = _rowmajor(grad_Ad)
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        grad_A = torch.empty(A_data.shape[0], dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_csr_to_dense_backward(
+            _dt(A_data), A_rows, A_cols, A_data.shape[0], _ptr(grad_Ad), max(ld, A_cols), _ptr(A_indices),
+            _ptr(A_indptr), _ptr(grad_A), _stream(dev)), "nm_csr_to_dense_backward")
+    return grad_A
+
+
+def csr_row_sum_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
+    """x[i] = sum of row i  (cpp/sparse_csr.hpp:136-140)."""
+    dev = _need_device(A_data, A_indices, A_indptr)
+    A_data, A_indptr = A_data.contiguous(), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        x = torch.empty(A_rows, dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_csr_row_sum_forward(_dt(A_data), A_rows, A_data.shape[0], _ptr(A_data),
+                                                     _ptr(A_indptr), _ptr(x), _stream(dev)),
+                   "nm_csr_row_sum_forward")
+    return x
+
+
+def csr_row_sum_backward(grad_x, A_rows, A_cols, A_data, A_indices, A_indptr):
+    """grad_A[k] = grad_x[row(k)]  (cpp/sparse_csr.hpp:142-147)."""
+    dev = _need_device(grad_x, A_data, A_indices, A_indptr)
+    _same_dtype(A_data, grad_x, "grad_x")
+    grad_x, A_indptr = grad_x.contiguous(), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        grad_A = torch.empty(A_data.shape[0], dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_csr_row_sum_backward(_dt(A_data), A_rows, A_data.shape[0], _ptr(A_indptr),
+                                                      _ptr(grad_x), _ptr(grad_A), _stream(dev)),
+                   "nm_csr_row_sum_backward")
+    return grad_A
+
+
+def csr_extract_diagonal_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
+    """x[i] = stored entry (i, i) or 0  (cpp/sparse_csr.hpp:150-154)."""
+    dev = _need_device(A_data, A_indices, A_indptr)
+    A_data = A_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        x = torch.empty(A_rows, dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_csr_extract_diagonal_forward(
+            _dt(A_data), A_rows, A_data.shape[0], _ptr(A_data), _ptr(A_indices), _ptr(A_indptr), _ptr(x),
+            _stream(dev)), "nm_csr_extract_diagonal_forward")
+    return x
+
+
+def csr_extract_diagonal_backward(grad_x, A_rows, A_cols, A_data, A_indices, A_indptr):
+    """grad_A = 0 except grad_x[i] on the diagonal entries  (cpp/sparse_csr.hpp:156-161)."""
+    dev = _need_device(grad_x, A_data, A_indices, A_indptr)
+    _same_dtype(A_data, grad_x, "grad_x")
+    grad_x = grad_x.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        grad_A = torch.empty(A_data.shape[0], dtype=A_data.dtype, device=dev)
+        _lib.check(_lib.lib().nm_csr_extract_diagonal_backward(
+            _dt(A_data), A_rows, A_data.shape[0], _ptr(A_indices), _ptr(A_indptr), _ptr(grad_x), _ptr(grad_A),
+            _stream(dev)), "nm_csr_extract_diagonal_backward")
     return grad_A
 
 

@@ -19,7 +19,8 @@ import torch
 
 from .._binding import ops as _ext
 
-__all__ = ["SparseCSRTensor", "coo_to_csr", "eye", "diag", "spgemv", "spgemm", "spdmm", "sptranspose"]
+__all__ = ["SparseCSRTensor", "coo_to_csr", "eye", "diag", "spgemv", "spgemm", "spdmm", "sptranspose",
+           "splincomb", "sptodense", "sprowsum", "spdiag"]
 
 
 def _type_error(kind_a, a, kind_b, b):
@@ -116,6 +117,66 @@ class sptranspose(torch.autograd.Function):
     def backward(ctx, _g_shape, grad_At_data, _g_indices, _g_indptr):
         (At_to_A_idx,) = ctx.saved_tensors
         return None, _ext.csr_transpose_backward(grad_At_data, At_to_A_idx), None, None
+
+
+class splincomb(torch.autograd.Function):
+    """C = alpha A + beta B; returns ``(C_data, C_indices, C_indptr)``.  The scalars
+    get sum(A.data) and sum(B.data) as their gradients, as in the reference
+    (numml/sparse/_csr.py:187-231)."""
+
+    @staticmethod
+    def forward(ctx, shape, alpha, A_data, A_col_ind, A_rowptr, beta, B_data, B_col_ind, B_rowptr):
+        if A_data.type() != B_data.type():
+            raise _type_error("Matrices", A_data, "", B_data)
+        C_data, C_col_ind, C_rowptr = _ext.splincomb_forward(
+            shape[0], shape[1], alpha, A_data, A_col_ind, A_rowptr, beta, B_data, B_col_ind, B_rowptr)
+        ctx.save_for_backward(alpha, A_data, A_col_ind, A_rowptr, beta, B_data, B_col_ind, B_rowptr,
+                              C_col_ind, C_rowptr)
+        ctx.shape = shape
+        ctx.mark_non_differentiable(C_col_ind, C_rowptr)
+        return C_data, C_col_ind, C_rowptr
+
+    @staticmethod
+    def backward(ctx, grad_C_data, _g_col_ind, _g_rowptr):
+        (alpha, A_data, A_col_ind, A_rowptr, beta, B_data, B_col_ind, B_rowptr,
+         C_col_ind, C_rowptr) = ctx.saved_tensors
+        grad_A, grad_B = _ext.splincomb_backward(
+            ctx.shape[0], ctx.shape[1], alpha, A_data, A_col_ind, A_rowptr, beta, B_data, B_col_ind, B_rowptr,
+            grad_C_data, C_col_ind, C_rowptr)
+        return (None, torch.sum(A_data).to(alpha.device), grad_A, None, None,
+                torch.sum(B_data).to(beta.device), grad_B, None, None)
+
+
+def _reduction(forward_name, backward_name, doc):
+    """Function of ``(A_shape, A_data, A_indices, A_indptr)`` returning one dense tensor."""
+
+    class _Fn(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, A_shape, A_data, A_indices, A_indptr):
+            ctx.save_for_backward(A_data, A_indices, A_indptr)
+            ctx.A_shape = A_shape
+            return getattr(_ext, forward_name)(A_shape[0], A_shape[1], A_data, A_indices, A_indptr)
+
+        @staticmethod
+        def backward(ctx, grad):
+            A_data, A_indices, A_indptr = ctx.saved_tensors
+            grad_A = getattr(_ext, backward_name)(grad, ctx.A_shape[0], ctx.A_shape[1], A_data, A_indices,
+                                                  A_indptr)
+            return None, grad_A, None, None
+
+    _Fn.__doc__ = doc
+    return _Fn
+
+
+sptodense = _reduction("csr_to_dense_forward", "csr_to_dense_backward",
+                       "Dense copy of a CSR matrix (numml/sparse/_csr.py:390-413).")
+sptodense.__name__ = sptodense.__qualname__ = "sptodense"
+sprowsum = _reduction("csr_row_sum_forward", "csr_row_sum_backward",
+                      "Row sums of a CSR matrix (numml/sparse/_csr.py:416-438).")
+sprowsum.__name__ = sprowsum.__qualname__ = "sprowsum"
+spdiag = _reduction("csr_extract_diagonal_forward", "csr_extract_diagonal_backward",
+                    "Diagonal of a CSR matrix (numml/sparse/_csr.py:441-463).")
+spdiag.__name__ = spdiag.__qualname__ = "spdiag"
 
 
 def coo_to_csr(values, row_ind, col_ind, shape, sort=True):
@@ -266,15 +327,73 @@ class SparseCSRTensor(object):
     def H(self):
         return self.hermitian()
 
+    # ---- entrywise arithmetic (numml/sparse/_csr.py:840-932) ---------------------
+    @staticmethod
+    def _isscalar(x):
+        return isinstance(x, (int, float)) or (isinstance(x, torch.Tensor) and x.ndim == 0)
+
+    def _lincomb(self, othr, beta, what):
+        if self.shape != othr.shape:
+            raise RuntimeError(f"Incompatible shapes for entrywise {what}, got {self.shape} and "
+                               f"{othr.shape}, respectively.")
+        C = splincomb.apply(self.shape, torch.tensor(1.), self.data, self.indices, self.indptr,
+                            torch.tensor(beta), othr.data, othr.indices, othr.indptr)
+        return SparseCSRTensor(C, self.shape)
+
+    def __add__(self, othr):
+        if SparseCSRTensor._isscalar(othr):
+            return SparseCSRTensor((self.data + othr, self.indices, self.indptr), self.shape)
+        if isinstance(othr, SparseCSRTensor):
+            return self._lincomb(othr, 1., "addition")
+        raise RuntimeError(f"Unknown type for sparse tensor addition: {type(othr)}.")
+
+    def __sub__(self, othr):
+        if SparseCSRTensor._isscalar(othr):
+            # the reference adds the scalar here as well (numml/sparse/_csr.py:898-899)
+            return SparseCSRTensor((self.data + othr, self.indices, self.indptr), self.shape)
+        if isinstance(othr, SparseCSRTensor):
+            return self._lincomb(othr, -1., "subtraction")
+        raise RuntimeError(f"Unknown type for sparse tensor addition: {type(othr)}.")
+
     def __mul__(self, s):
-        if isinstance(s, (int, float)) or (isinstance(s, torch.Tensor) and s.ndim == 0):
+        if SparseCSRTensor._isscalar(s):
             return SparseCSRTensor((self.data * s, self.indices, self.indptr), self.shape)
-        raise RuntimeError(f"unsupported multiplication by {type(s)}")
+        if isinstance(s, torch.Tensor) and len(torch.squeeze(s).shape) == 2:
+            raise RuntimeError("Element-wise hadamard product not implemented")
+        raise RuntimeError(f"Unknown type for multiplication: {type(s)}.")
 
     __rmul__ = __mul__
 
+    def __rtruediv__(self, other):
+        if SparseCSRTensor._isscalar(other):
+            return SparseCSRTensor((other / self.data, self.indices, self.indptr), self.shape)
+        raise RuntimeError(f"Unknown type for right-division: {type(other)}.")
+
     def __neg__(self):
-        return self * -1.0
+        return SparseCSRTensor((-self.data, self.indices, self.indptr), self.shape)
+
+    def __pow__(self, p):
+        return SparseCSRTensor((self.data ** p, self.indices, self.indptr), self.shape)
+
+    def abs(self):
+        return SparseCSRTensor((torch.abs(self.data), self.indices, self.indptr), self.shape)
+
+    __abs__ = abs
+
+    # ---- reductions ----------------------------------------------------------------
+    def sum(self):
+        return self.data.sum()
+
+    def row_sum(self):
+        """x[i] = sum of the stored entries of row i (numml/sparse/_csr.py:852-861)."""
+        return sprowsum.apply(self.shape, self.data, self.indices, self.indptr)
+
+    def diagonal(self):
+        """Stored diagonal entries, 0 where a row has none (numml/sparse/_csr.py:1016-1027)."""
+        return spdiag.apply(self.shape, self.data, self.indices, self.indptr)
+
+    def trace(self):
+        return self.diagonal().sum()
 
     # ---- conversions ----------------------------------------------------------
     def row_indices(self):
@@ -283,9 +402,13 @@ class SparseCSRTensor(object):
             torch.arange(self.shape[0], device=self.indptr.device), counts)
 
     def to_dense(self):
-        """Dense copy (built with torch indexing; differentiable with respect to the values)."""
-        out = torch.zeros(self.shape, dtype=self.data.dtype, device=self.data.device)
-        return out.index_put((self.row_indices(), self.indices), self.data, accumulate=True)
+        """Dense copy; gradients flow to and from the stored entries
+        (numml/sparse/_csr.py:740-751)."""
+        return sptodense.apply(self.shape, self.data, self.indices, self.indptr)
+
+    def to_coo(self):
+        """(values, rows, cols) of the stored entries."""
+        return self.data, self.row_indices(), self.indices
 
     def to_scipy_csr(self):
         import scipy.sparse as sp

@@ -170,6 +170,92 @@ def csr_transpose_backward(grad_At, At_to_A_idx):
     return grad_A
 
 
+def splincomb_forward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr):
+    """splincomb_forward_cpu, cpp/sparse_csr_cpu.cpp:387-481 -> (C_data, C_indices, C_indptr).
+    alpha and beta are converted to the value type first (alpha.item<scalar_t>(), :413-414)."""
+    A_data, A_indices, A_indptr = _vals(A_data), _idx(A_indices), _idx(A_indptr)
+    B_data, B_indices, B_indptr = _vals(B_data, A_data.dtype), _idx(B_indices), _idx(B_indptr)
+    ct = ctypes.c_float if A_data.dtype == np.float32 else ctypes.c_double
+    fn = _fn("or_splincomb_forward", A_data.dtype)
+    C_indptr = np.zeros(rows + 1, dtype=np.int64)
+    fn(_i64(rows), ct(alpha), _p(A_data), _p(A_indices), _p(A_indptr), ct(beta), _p(B_data), _p(B_indices),
+       _p(B_indptr), _p(C_indptr), None, None)
+    counts = C_indptr[:rows].copy()
+    C_indptr[0] = 0
+    np.cumsum(counts, out=C_indptr[1:])
+    nnz = int(C_indptr[rows])
+    C_indices = np.empty(nnz, dtype=np.int64)
+    C_data = np.empty(nnz, dtype=A_data.dtype)
+    fn(_i64(rows), ct(alpha), _p(A_data), _p(A_indices), _p(A_indptr), ct(beta), _p(B_data), _p(B_indices),
+       _p(B_indptr), _p(C_indptr), _p(C_indices), _p(C_data))
+    return C_data, C_indices, C_indptr
+
+
+def splincomb_backward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr,
+                       gC, C_indices, C_indptr):
+    """splincomb_backward_cpu, cpp/sparse_csr_cpu.cpp:483-560 -> (grad_A, grad_B).  Every column of
+    A and of B is present in C, so every entry of both gradients is written."""
+    A_data, B_data = _vals(A_data), _vals(B_data)
+    gC = _vals(gC, A_data.dtype)
+    ct = ctypes.c_float if A_data.dtype == np.float32 else ctypes.c_double
+    fn = _fn("or_splincomb_backward_one", A_data.dtype)
+    C_indices, C_indptr = _idx(C_indices), _idx(C_indptr)
+    grad_A, grad_B = np.zeros_like(A_data), np.zeros_like(B_data)
+    for coef, ind, ptr, out in ((alpha, A_indices, A_indptr, grad_A), (beta, B_indices, B_indptr, grad_B)):
+        ind, ptr = _idx(ind), _idx(ptr)
+        fn(_i64(rows), ct(coef), _p(ind), _p(ptr), _p(gC), _p(C_indices), _p(C_indptr), _p(out))
+    return grad_A, grad_B
+
+
+def csr_to_dense_forward(rows, cols, data, indices, indptr):
+    """csr_to_dense_forward_cpu, cpp/sparse_csr_cpu.cpp:1052-1076: zeros, then A_d[i, j] = data[k]
+    in storage order (a later duplicate would overwrite an earlier one)."""
+    data, indices, indptr = _vals(data), _idx(indices), _idx(indptr)
+    out = np.zeros((rows, cols), dtype=data.dtype)
+    r = np.repeat(np.arange(rows), np.diff(indptr))
+    out[r, indices] = data
+    return out
+
+
+def csr_to_dense_backward(grad_Ad, rows, cols, data, indices, indptr):
+    """csr_to_dense_backward_cpu, cpp/sparse_csr_cpu.cpp:1078-1104: grad_A[k] = grad_Ad[i, j]."""
+    indices, indptr = _idx(indices), _idx(indptr)
+    r = np.repeat(np.arange(rows), np.diff(indptr))
+    return np.ascontiguousarray(np.asarray(grad_Ad)[r, indices])
+
+
+def csr_row_sum_forward(rows, cols, data, indices, indptr):
+    """csr_row_sum_forward_cpu, cpp/sparse_csr_cpu.cpp:1106-1131."""
+    data, indptr = _vals(data), _idx(indptr)
+    x = np.empty(rows, dtype=data.dtype)
+    _fn("or_row_sum", data.dtype)(_i64(rows), _p(data), _p(indptr), _p(x))
+    return x
+
+
+def csr_row_sum_backward(g, rows, cols, data, indices, indptr):
+    """csr_row_sum_backward_cpu, cpp/sparse_csr_cpu.cpp:1133-1156: grad_A[k] = g[row(k)]."""
+    indptr = _idx(indptr)
+    return np.repeat(np.asarray(g), np.diff(indptr))
+
+
+def csr_extract_diagonal_forward(rows, cols, data, indices, indptr):
+    """csr_extract_diagonal_forward_cpu, cpp/sparse_csr_cpu.cpp:1158-1186."""
+    data, indices, indptr = _vals(data), _idx(indices), _idx(indptr)
+    x = np.empty(rows, dtype=data.dtype)
+    _fn("or_diagonal", data.dtype)(_i64(rows), _p(data), _p(indices), _p(indptr), _p(x))
+    return x
+
+
+def csr_extract_diagonal_backward(g, rows, cols, data, indices, indptr):
+    """csr_extract_diagonal_backward_cpu, cpp/sparse_csr_cpu.cpp:1188-1213."""
+    data, indices, indptr = _vals(data), _idx(indices), _idx(indptr)
+    g = _vals(g, data.dtype)
+    grad_A = np.empty_like(data)
+    _fn("or_diagonal_backward", data.dtype)(_i64(rows), _i64(data.shape[0]), _p(g), _p(indices), _p(indptr),
+                                            _p(grad_A))
+    return grad_A
+
+
 def sptrsv_forward(rows, cols, data, indices, indptr, lower, unit, b):
     """sptrsv_forward_cpu, cpp/sparse_csr_cpu.cpp:652-723."""
     data, indices, indptr = _vals(data), _idx(indices), _idx(indptr)

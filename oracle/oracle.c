@@ -10,6 +10,11 @@
  *   or_csr_transpose             :311-367
  *   or_spdmm_forward/backward    :562-650
  *   or_sptrsv_forward/backward   :652-759
+ *   or_splincomb_forward/backward_one :387-560
+ *   or_row_sum, or_diagonal(_backward) :1106-1213
+ * (csr_to_dense_forward/backward, :1050-1104, and csr_transpose_backward,
+ * :369-385, are plain index assignments and are restated with NumPy indexing in
+ * oracle/__init__.py.)
  *
  * How each is pinned (tests/test_oracle.py): against the reference's own CPU
  * sources compiled in place (oracle/_ref, when the reference tree is present),

@@ -1,0 +1,121 @@
+"""Linear combination, dense copy, row sums and diagonal on a HIP device.
+
+Compared with the CPU oracle (cpp/sparse_csr_cpu.cpp:387-560, 1050-1213), through
+both bindings and through the ``SparseCSRTensor`` surface with gradients.
+Structure and copied values are exact; the linear combination is two products
+and one sum per entry in the value type, also exact; row sums are bitwise for
+rows summed in storage order and within util.RTOL (1e-5 / 1e-12) for rows long
+enough to be reduced by a wavefront.
+"""
+import numpy as np
+import pytest
+import torch
+
+import numml_amd
+import oracle
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as mirror
+from numml_amd import sparse as sp
+from util import assert_close, assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+
+@pytest.fixture(params=["compiled", "ctypes"])
+def ext(request):
+    return numml_amd.load_compiled() if request.param == "compiled" else mirror
+
+
+def _pairs(dtype):
+    yield "stencils", G.poisson2d(30, dtype, 1), G.poisson2d(30, dtype, 2)                   # same pattern
+    yield "tri_vs_id", G.tridiag(500, dtype), (np.ones(500, dtype), np.arange(500), np.arange(501), (500, 500))
+    yield "random", G.random_csr(300, 260, 0.05, 1, dtype), G.random_csr(300, 260, 0.08, 2, dtype)
+    yield "disjointish", G.random_csr(64, 900, 0.01, 3, dtype), G.random_csr(64, 900, 0.3, 4, dtype)
+    yield "powerlaw", (G.powerlaw(3000, 3000, 40000, max_deg=2500, seed=5, dtype=dtype),
+                       G.powerlaw(3000, 3000, 30000, max_deg=2500, seed=6, dtype=dtype))[0], \
+        G.powerlaw(3000, 3000, 30000, max_deg=2500, seed=6, dtype=dtype)
+    yield "empty_a", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(8, np.int64), (7, 5)), \
+        G.random_csr(7, 5, 0.4, 7, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_splincomb_forward_backward(dev, ext, dtype):
+    for name, (ad, ai, ap, (r, c)), (bd, bi, bp, _) in _pairs(dtype):
+        ai, ap, bi, bp = (np.asarray(v, np.int64) for v in (ai, ap, bi, bp))
+        for alpha, beta in ((1.0, 1.0), (1.0, -1.0), (0.75, -2.5)):
+            Cd_ref, Ci_ref, Cp_ref = oracle.splincomb_forward(r, c, alpha, ad, ai, ap, beta, bd, bi, bp)
+            AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+            Cd, Ci, Cp = ext.splincomb_forward(r, c, torch.tensor(alpha), AD, AI, AP, torch.tensor(beta), BD, BI, BP)
+            assert_same(host(Cp), Cp_ref, f"{name} C_indptr")
+            assert_same(host(Ci), Ci_ref, f"{name} C_indices")
+            assert_same(host(Cd), Cd_ref, f"{name} C_data")
+            g = randn(3, Cd_ref.shape[0], dtype)
+            gA, gB = ext.splincomb_backward(r, c, torch.tensor(alpha), AD, AI, AP, torch.tensor(beta), BD, BI, BP,
+                                            to_dev(dev, g)[0], Ci, Cp)
+            gA_ref, gB_ref = oracle.splincomb_backward(r, c, alpha, ad, ai, ap, beta, bd, bi, bp, g, Ci_ref, Cp_ref)
+            assert_same(host(gA), gA_ref, f"{name} grad_A")
+            assert_same(host(gB), gB_ref, f"{name} grad_B")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_dense_rowsum_diagonal(dev, ext, dtype):
+    cases = [("poisson", G.poisson2d(24, dtype, 1)), ("random", G.random_csr(130, 170, 0.07, 2, dtype)),
+             ("tall", G.random_csr(400, 9, 0.3, 3, dtype)), ("one_dense_row", G.random_csr(3, 6000, 0.9, 4, dtype, empty_rows=False)),
+             ("powerlaw", G.powerlaw(2500, 2500, 30000, max_deg=2000, seed=5, dtype=dtype)),
+             ("empty", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(5, np.int64), (4, 4)))]
+    for name, (d, i, p, (r, c)) in cases:
+        D, I, P = to_dev(dev, d, i, p)
+        if r * c <= 4_000_000:
+            Ad = ext.csr_to_dense_forward(r, c, D, I, P)
+            assert_same(host(Ad), oracle.csr_to_dense_forward(r, c, d, i, p), f"{name} dense")
+            gD = randn(1, (r, c), dtype)
+            assert_same(host(ext.csr_to_dense_backward(to_dev(dev, gD)[0], r, c, D, I, P)),
+                        oracle.csr_to_dense_backward(gD, r, c, d, i, p), f"{name} dense backward")
+            wide = to_dev(dev, np.concatenate([gD, gD], axis=1))[0][:, :c]          # row stride 2c
+            assert_same(host(ext.csr_to_dense_backward(wide, r, c, D, I, P)),
+                        oracle.csr_to_dense_backward(gD, r, c, d, i, p), f"{name} dense backward, strided")
+        rs = ext.csr_row_sum_forward(r, c, D, I, P)
+        rs_ref = oracle.csr_row_sum_forward(r, c, d, i, p)
+        if int(np.diff(p).max(initial=0)) <= 512:
+            assert_same(host(rs), rs_ref, f"{name} row sums")
+        else:
+            assert_close(host(rs), rs_ref, f"{name} row sums")
+        g = randn(2, r, dtype)
+        Gv = to_dev(dev, g)[0]
+        assert_same(host(ext.csr_row_sum_backward(Gv, r, c, D, I, P)), oracle.csr_row_sum_backward(g, r, c, d, i, p),
+                    f"{name} row sum backward")
+        if r <= c:                                                     # x has one entry per row
+            assert_same(host(ext.csr_extract_diagonal_forward(r, c, D, I, P)),
+                        oracle.csr_extract_diagonal_forward(r, c, d, i, p), f"{name} diagonal")
+            assert_same(host(ext.csr_extract_diagonal_backward(Gv, r, c, D, I, P)),
+                        oracle.csr_extract_diagonal_backward(g, r, c, d, i, p), f"{name} diagonal backward")
+
+
+def test_operators_and_gradients(dev):
+    ad, ai, ap, (n, _) = G.poisson2d(12, np.float64, 1)
+    bd, bi, bp, _ = G.tridiag(n, np.float64)
+    A = sp.SparseCSRTensor(tuple(to_dev(dev, ad, ai, ap)), (n, n))
+    B = sp.SparseCSRTensor(tuple(to_dev(dev, bd, bi, bp)), (n, n))
+    A.requires_grad = True
+    B.requires_grad = True
+    Ad, Bd = A.to_dense().detach(), B.to_dense().detach()
+    assert torch.equal((A + B).to_dense(), Ad + Bd)                       # numml/tests/test_splincomb.py pattern
+    assert torch.equal((A - B).to_dense(), Ad - Bd)
+    Z = A - A
+    assert Z.nnz == A.nnz and not bool(Z.data.any())                     # explicit zeros are kept
+    assert torch.equal((2.0 * A).to_dense(), 2.0 * Ad) and torch.equal((-A).to_dense(), -Ad)
+    assert torch.equal(abs(-A).data, A.data.abs()) and torch.equal((A ** 2).data, A.data ** 2)
+    # loss through +, row_sum, diagonal and to_dense
+    w = to_dev(dev, randn(1, n, np.float64))[0]
+    loss = ((A - B).row_sum() * w).sum() + (A + B).diagonal().sum() + (A.to_dense() ** 2).sum() + A.trace()
+    loss.backward()
+    rows_a = A.row_indices()
+    rows_b = B.row_indices()
+    gA = w[rows_a] + (A.indices == rows_a) * 2.0 + 2 * A.data.detach()
+    gB = -w[rows_b] + (B.indices == rows_b) * 1.0
+    assert torch.allclose(A.data.grad, gA, atol=1e-12) and torch.allclose(B.data.grad, gB, atol=1e-12)
+    with pytest.raises(RuntimeError, match="Incompatible shapes"):
+        A + sp.eye(3, dtype=torch.float64, device=dev)
+    assert torch.equal(A.sum(), A.data.sum())

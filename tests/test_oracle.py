@@ -273,3 +273,85 @@ def test_generators_match_the_stated_sizes():
     for row in range(0, r, 97):
         assert np.all(np.diff(i[p[row]:p[row + 1]]) > 0)
     np.testing.assert_allclose(np.add.reduceat(d.astype(np.float64), p[:-1]), 1.0, rtol=1e-5)
+
+
+# ------------------------------------------------- entrywise / reduction operations
+
+def _pair(dtype, seed):
+    """Two matrices of one shape with overlapping patterns (some rows empty in either)."""
+    rng = np.random.default_rng(300 + seed)
+    r, c = (int(v) for v in rng.integers(1, 70, 2))
+    A = G.random_csr(r, c, float(rng.uniform(0.05, 0.4)), 20 * seed, dtype)
+    B = G.random_csr(r, c, float(rng.uniform(0.05, 0.4)), 20 * seed + 1, dtype)
+    return r, c, A[:3], B[:3]
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_ref_lincomb_and_reductions(dtype, seed):
+    r, c, (ad, ai, ap), (bd, bi, bp) = _pair(dtype, seed)
+    alpha, beta = np.array(0.75, dtype), np.array(-1.5, dtype)
+    C1 = oracle.splincomb_forward(r, c, float(alpha), ad, ai, ap, float(beta), bd, bi, bp)
+    C2 = ref.call("splincomb_forward", r, c, alpha, ad, ai, ap, beta, bd, bi, bp)
+    for a, b, what in zip(C1, C2, ("C_data", "C_indices", "C_indptr")):
+        same(a, b, f"splincomb {what}")
+    gC = np.random.default_rng(seed).standard_normal(C1[0].shape[0]).astype(dtype)
+    for a, b in zip(oracle.splincomb_backward(r, c, float(alpha), ad, ai, ap, float(beta), bd, bi, bp, gC, C1[1], C1[2]),
+                    ref.call("splincomb_backward", r, c, alpha, ad, ai, ap, beta, bd, bi, bp, gC, C1[1], C1[2])):
+        same(a, b, "splincomb backward")
+    same(oracle.csr_to_dense_forward(r, c, ad, ai, ap), ref.call("csr_to_dense_forward", r, c, ad, ai, ap), "to_dense")
+    gD = np.random.default_rng(seed + 1).standard_normal((r, c)).astype(dtype)
+    same(oracle.csr_to_dense_backward(gD, r, c, ad, ai, ap),
+         ref.call("csr_to_dense_backward", gD, r, c, ad, ai, ap), "to_dense backward")
+    same(oracle.csr_row_sum_forward(r, c, ad, ai, ap), ref.call("csr_row_sum_forward", r, c, ad, ai, ap), "row_sum")
+    g = np.random.default_rng(seed + 2).standard_normal(r).astype(dtype)
+    same(oracle.csr_row_sum_backward(g, r, c, ad, ai, ap),
+         ref.call("csr_row_sum_backward", g, r, c, ad, ai, ap), "row_sum backward")
+    n = min(r, c)                                   # the diagonal ops index x by row: square part only
+    sq = sp.csr_matrix((ad, ai, ap), shape=(r, c))[:n, :n].tocsr()
+    sq.sort_indices()
+    sd, si, sp_ = sq.data.astype(dtype), sq.indices.astype(np.int64), sq.indptr.astype(np.int64)
+    same(oracle.csr_extract_diagonal_forward(n, n, sd, si, sp_),
+         ref.call("csr_extract_diagonal_forward", n, n, sd, si, sp_), "diagonal")
+    same(oracle.csr_extract_diagonal_backward(g[:n], n, n, sd, si, sp_),
+         ref.call("csr_extract_diagonal_backward", g[:n], n, n, sd, si, sp_), "diagonal backward")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_math_lincomb_and_reductions(dtype):
+    r, c, (ad, ai, ap), (bd, bi, bp) = _pair(dtype, 5)
+    Ad = sp.csr_matrix((ad, ai, ap), shape=(r, c)).toarray()
+    Bd = sp.csr_matrix((bd, bi, bp), shape=(r, c)).toarray()
+    Cd, Ci, Cp = oracle.splincomb_forward(r, c, 2.0, ad, ai, ap, -3.0, bd, bi, bp)
+    # structure: union of the patterns (SciPy sum of the all-ones matrices has no cancellation)
+    U = sp.csr_matrix((np.ones_like(ad), ai, ap), shape=(r, c)) + sp.csr_matrix((np.ones_like(bd), bi, bp), shape=(r, c))
+    U.sort_indices()
+    assert np.array_equal(Cp, U.indptr) and np.array_equal(Ci, U.indices)
+    assert np.array_equal(sp.csr_matrix((Cd, Ci, Cp), shape=(r, c)).toarray(), (dtype(2.0) * Ad + dtype(-3.0) * Bd))
+    # A - A keeps explicit zeros on A's pattern
+    Zd, Zi, Zp = oracle.splincomb_forward(r, c, 1.0, ad, ai, ap, -1.0, ad, ai, ap)
+    assert np.array_equal(Zi, ai) and np.array_equal(Zp, ap) and not Zd.any()
+    # gradients: d(sum(w . C))/dA[k] = alpha * w at A's column, same for B with beta
+    w = np.random.default_rng(1).standard_normal(Cd.shape[0]).astype(dtype)
+    gA, gB = oracle.splincomb_backward(r, c, 2.0, ad, ai, ap, -3.0, bd, bi, bp, w, Ci, Cp)
+    W = sp.csr_matrix((w, Ci, Cp), shape=(r, c)).toarray()
+    rows_a, rows_b = np.repeat(np.arange(r), np.diff(ap)), np.repeat(np.arange(r), np.diff(bp))
+    assert np.array_equal(gA, W[rows_a, ai] * dtype(2.0)) and np.array_equal(gB, W[rows_b, bi] * dtype(-3.0))
+    # dense round trip, row sums, diagonal
+    assert np.array_equal(oracle.csr_to_dense_forward(r, c, ad, ai, ap), Ad)
+    assert np.array_equal(oracle.csr_to_dense_backward(Ad, r, c, ad, ai, ap), ad)
+    rs = oracle.csr_row_sum_forward(r, c, ad, ai, ap)
+    assert np.allclose(rs, Ad.sum(axis=1), rtol=1e-5 if dtype == np.float32 else 1e-12, atol=1e-6)
+    g = np.random.default_rng(2).standard_normal(r).astype(dtype)
+    assert np.array_equal(oracle.csr_row_sum_backward(g, r, c, ad, ai, ap), g[rows_a])
+    n = min(r, c)
+    td, ti, tp, _ = G.poisson2d(6, dtype, 3)
+    assert np.array_equal(oracle.csr_extract_diagonal_forward(36, 36, td, ti, tp),
+                          sp.csr_matrix((td, ti, tp), shape=(36, 36)).diagonal())
+    gd = oracle.csr_extract_diagonal_backward(g[:1].repeat(36), 36, 36, td, ti, tp)
+    on_diag = ti == np.repeat(np.arange(36), np.diff(tp))
+    assert np.array_equal(gd, np.where(on_diag, g[0], 0).astype(dtype))
+    sd, si, sp_, _ = G.random_csr(9, 9, 0.3, 1, dtype)       # some rows without a stored diagonal
+    assert np.array_equal(oracle.csr_extract_diagonal_forward(9, 9, sd, si, sp_),
+                          sp.csr_matrix((sd, si, sp_), shape=(9, 9)).diagonal())
