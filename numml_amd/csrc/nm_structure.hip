@@ -145,65 +145,214 @@ __global__ __launch_bounds__(kBlock) void diagonal_kernel(int64_t rows, const T 
 
 // ---- linear combination --------------------------------------------------------------
 //
-// One lane merges one row of A with the same row of B (cpp/sparse_csr_cpu.cpp:428-468).
-// COUNT: only the length of the merged row is produced.
+// C = alpha A + beta B (cpp/sparse_csr_cpu.cpp:428-468).  A workgroup owns a tile
+// of kLcRows rows.  The column indices of both operands' tile are staged in LDS
+// with coalesced loads; one lane per row then merges its two sorted lists there
+// (the walk is a chain of dependent reads, which LDS serves in ~100 cycles where
+// global memory would take a round trip each) and leaves, for every output entry,
+// which entry of A and/or of B feeds it.  The output is finally produced lane =
+// output entry: values are fetched and C is written through coalesced accesses.
+// Tiles with more than kLcCap entries in either operand fall back to one lane per
+// row straight from global memory.
 
+constexpr int kLcRows = 256, kLcCap = 2304;
+constexpr uint32_t kLcNone = 0xffff;
+
+struct LcTile {
+    int32_t offA[kLcRows + 1], offB[kLcRows + 1], offC[kLcRows + 1];
+    int32_t colA[kLcCap], colB[kLcCap];
+    uint32_t src[2 * kLcCap];   // per output entry: local index in A (low half) and in B (high half)
+};
+
+__device__ __forceinline__ void lc_stage_offsets(const int64_t *__restrict__ indptr, int64_t r0, int nr, int32_t *off) {
+    const int64_t base = indptr[r0];
+    for (int t = threadIdx.x; t <= nr; t += kBlock) {
+        const int64_t d = indptr[r0 + t] - base;
+        off[t] = (int32_t)(d > kLcCap ? kLcCap + 1 : d);
+    }
+}
+
+// Merge of one row from global memory (fallback); COUNT: length only.
 template <typename T, bool COUNT>
-__global__ void lincomb_kernel(int64_t rows, T alpha, const T *__restrict__ A_data,
-                               const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr, T beta,
-                               const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
-                               const int64_t *__restrict__ B_indptr, int64_t *__restrict__ C_indptr,
-                               int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; row < rows; row += stride) {
-        int64_t iA = A_indptr[row], iB = B_indptr[row];
-        const int64_t eA = A_indptr[row + 1], eB = B_indptr[row + 1];
-        int64_t out = COUNT ? 0 : C_indptr[row];
-        while (iA < eA && iB < eB) {
-            const int64_t cA = A_indices[iA], cB = B_indices[iB];
-            if (!COUNT) {
-                C_indices[out] = cA < cB ? cA : cB;
-                C_data[out] = cA < cB ? alpha * A_data[iA]
-                                      : (cA > cB ? beta * B_data[iB] : alpha * A_data[iA] + beta * B_data[iB]);
-            }
-            iA += cA <= cB;
-            iB += cB <= cA;
-            ++out;
+__device__ __forceinline__ void lc_row_global(int64_t row, T alpha, const T *__restrict__ A_data,
+                                              const int64_t *__restrict__ A_indices,
+                                              const int64_t *__restrict__ A_indptr, T beta,
+                                              const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
+                                              const int64_t *__restrict__ B_indptr, int64_t *__restrict__ C_indptr,
+                                              int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
+    int64_t iA = A_indptr[row], iB = B_indptr[row];
+    const int64_t eA = A_indptr[row + 1], eB = B_indptr[row + 1];
+    int64_t out = COUNT ? 0 : C_indptr[row];
+    while (iA < eA && iB < eB) {
+        const int64_t cA = A_indices[iA], cB = B_indices[iB];
+        if (!COUNT) {
+            C_indices[out] = cA < cB ? cA : cB;
+            C_data[out] = cA < cB ? alpha * A_data[iA]
+                                  : (cA > cB ? beta * B_data[iB] : alpha * A_data[iA] + beta * B_data[iB]);
         }
-        if (COUNT) {
-            out += (eA - iA) + (eB - iB);
-            C_indptr[row] = out;
-        } else {
-            for (; iA < eA; ++iA, ++out) {
-                C_indices[out] = A_indices[iA];
-                C_data[out] = alpha * A_data[iA];
-            }
-            for (; iB < eB; ++iB, ++out) {
-                C_indices[out] = B_indices[iB];
-                C_data[out] = beta * B_data[iB];
-            }
+        iA += cA <= cB;
+        iB += cB <= cA;
+        ++out;
+    }
+    if (COUNT) {
+        C_indptr[row] = out + (eA - iA) + (eB - iB);
+    } else {
+        for (; iA < eA; ++iA, ++out) {
+            C_indices[out] = A_indices[iA];
+            C_data[out] = alpha * A_data[iA];
+        }
+        for (; iB < eB; ++iB, ++out) {
+            C_indices[out] = B_indices[iB];
+            C_data[out] = beta * B_data[iB];
         }
     }
 }
 
-// grad_X[k] = coef * grad_C at the same coordinate: row of X merged with row of C
-// (cpp/sparse_csr_cpu.cpp:505-552).  Every column of X is present in C.
-template <typename T>
-__global__ void lincomb_back_kernel(int64_t rows, T coef, const int64_t *__restrict__ X_indices,
-                                    const int64_t *__restrict__ X_indptr, const T *__restrict__ gC,
-                                    const int64_t *__restrict__ C_indices, const int64_t *__restrict__ C_indptr,
-                                    T *__restrict__ grad_X) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; row < rows; row += stride) {
-        int64_t iX = X_indptr[row], iC = C_indptr[row];
-        const int64_t eX = X_indptr[row + 1], eC = C_indptr[row + 1];
-        while (iX < eX && iC < eC) {
-            const int64_t cX = X_indices[iX], cC = C_indices[iC];
-            if (cX == cC) grad_X[iX] = gC[iC] * coef;
-            iX += cX <= cC;
-            iC += cC <= cX;
+template <typename T, bool COUNT>
+__global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, const T *__restrict__ A_data,
+                                                         const int64_t *__restrict__ A_indices,
+                                                         const int64_t *__restrict__ A_indptr, T beta,
+                                                         const T *__restrict__ B_data,
+                                                         const int64_t *__restrict__ B_indices,
+                                                         const int64_t *__restrict__ B_indptr,
+                                                         int64_t *__restrict__ C_indptr,
+                                                         int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
+    __shared__ LcTile s;
+    const int64_t ntiles = nm::ceil_div(rows, kLcRows), npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t r0 = tile * kLcRows;
+        const int nr = (int)(rows - r0 < kLcRows ? rows - r0 : kLcRows);
+        const int64_t baseA = A_indptr[r0], baseB = B_indptr[r0];
+        lc_stage_offsets(A_indptr, r0, nr, s.offA);
+        lc_stage_offsets(B_indptr, r0, nr, s.offB);
+        __syncthreads();
+        const int nA = s.offA[nr], nB = s.offB[nr];
+        if (nA <= kLcCap && nB <= kLcCap) {
+            for (int k = threadIdx.x; k < nA; k += kBlock) s.colA[k] = (int32_t)nm::stream_load(A_indices + baseA + k);
+            for (int k = threadIdx.x; k < nB; k += kBlock) s.colB[k] = (int32_t)nm::stream_load(B_indices + baseB + k);
+            const int64_t baseC = COUNT ? 0 : C_indptr[r0];
+            if (!COUNT)
+                for (int t = threadIdx.x; t <= nr; t += kBlock) s.offC[t] = (int32_t)(C_indptr[r0 + t] - baseC);
+            __syncthreads();
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                int iA = s.offA[t], iB = s.offB[t];
+                const int eA = s.offA[t + 1], eB = s.offB[t + 1];
+                int out = COUNT ? 0 : s.offC[t];
+                while (iA < eA && iB < eB) {
+                    const int32_t cA = s.colA[iA], cB = s.colB[iB];
+                    if (!COUNT) s.src[out] = (cA <= cB ? (uint32_t)iA : kLcNone) | ((cB <= cA ? (uint32_t)iB : kLcNone) << 16);
+                    iA += cA <= cB;
+                    iB += cB <= cA;
+                    ++out;
+                }
+                if (COUNT) {
+                    C_indptr[r0 + t] = out + (eA - iA) + (eB - iB);
+                } else {
+                    for (; iA < eA; ++iA, ++out) s.src[out] = (uint32_t)iA | (kLcNone << 16);
+                    for (; iB < eB; ++iB, ++out) s.src[out] = kLcNone | ((uint32_t)iB << 16);
+                }
+            }
+            if (!COUNT) {
+                __syncthreads();
+                const int nC = s.offC[nr];
+                for (int o = threadIdx.x; o < nC; o += kBlock) {
+                    const uint32_t sr = s.src[o];
+                    const uint32_t ia = sr & 0xffff, ib = sr >> 16;
+                    T v;
+                    int32_t c;
+                    if (ib == kLcNone) {
+                        c = s.colA[ia];
+                        v = alpha * A_data[baseA + ia];
+                    } else if (ia == kLcNone) {
+                        c = s.colB[ib];
+                        v = beta * B_data[baseB + ib];
+                    } else {
+                        c = s.colA[ia];
+                        v = alpha * A_data[baseA + ia] + beta * B_data[baseB + ib];
+                    }
+                    nm::stream_store(C_indices + baseC + o, (int64_t)c);
+                    nm::stream_store(C_data + baseC + o, v);
+                }
+            }
+        } else {
+            for (int t = threadIdx.x; t < nr; t += kBlock)
+                lc_row_global<T, COUNT>(r0 + t, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr,
+                                        C_indptr, C_indices, C_data);
         }
+        __syncthreads();
     }
+}
+
+// grad_X[k] = coef * grad_C at the same coordinate (cpp/sparse_csr_cpu.cpp:505-552).
+// Every column of X is present in C.  Same tiling: columns of X and of C staged in
+// LDS, one lane per row merges them and notes the matching entry of C for every
+// entry of X, then lane = entry of X gathers and scales.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lincomb_back_kernel(int64_t rows, T coef,
+                                                              const int64_t *__restrict__ X_indices,
+                                                              const int64_t *__restrict__ X_indptr,
+                                                              const T *__restrict__ gC,
+                                                              const int64_t *__restrict__ C_indices,
+                                                              const int64_t *__restrict__ C_indptr,
+                                                              T *__restrict__ grad_X) {
+    __shared__ int32_t s_offX[kLcRows + 1], s_offC[kLcRows + 1];
+    __shared__ int32_t s_colX[kLcCap], s_colC[2 * kLcCap], s_match[kLcCap];
+    const int64_t ntiles = nm::ceil_div(rows, kLcRows), npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t r0 = tile * kLcRows;
+        const int nr = (int)(rows - r0 < kLcRows ? rows - r0 : kLcRows);
+        const int64_t baseX = X_indptr[r0], baseC = C_indptr[r0];
+        lc_stage_offsets(X_indptr, r0, nr, s_offX);
+        for (int t = threadIdx.x; t <= nr; t += kBlock) {
+            const int64_t d = C_indptr[r0 + t] - baseC;
+            s_offC[t] = (int32_t)(d > 2 * kLcCap ? 2 * kLcCap + 1 : d);
+        }
+        __syncthreads();
+        const int nX = s_offX[nr], nC = s_offC[nr];
+        if (nX <= kLcCap && nC <= 2 * kLcCap) {
+            for (int k = threadIdx.x; k < nX; k += kBlock) s_colX[k] = (int32_t)nm::stream_load(X_indices + baseX + k);
+            for (int k = threadIdx.x; k < nC; k += kBlock) s_colC[k] = (int32_t)nm::stream_load(C_indices + baseC + k);
+            __syncthreads();
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                int iX = s_offX[t], iC = s_offC[t];
+                const int eX = s_offX[t + 1], eC = s_offC[t + 1];
+                while (iX < eX && iC < eC) {
+                    const int32_t cX = s_colX[iX], cC = s_colC[iC];
+                    if (cX == cC) s_match[iX] = iC;
+                    iX += cX <= cC;
+                    iC += cC <= cX;
+                }
+                for (; iX < eX; ++iX) s_match[iX] = -1;   // not reached for valid input (C holds every column of X)
+            }
+            __syncthreads();
+            for (int k = threadIdx.x; k < nX; k += kBlock) {
+                const int m = s_match[k];
+                if (m >= 0) nm::stream_store(grad_X + baseX + k, gC[baseC + m] * coef);
+            }
+        } else {
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                int64_t iX = X_indptr[r0 + t], iC = C_indptr[r0 + t];
+                const int64_t eX = X_indptr[r0 + t + 1], eC = C_indptr[r0 + t + 1];
+                while (iX < eX && iC < eC) {
+                    const int64_t cX = X_indices[iX], cC = C_indices[iC];
+                    if (cX == cC) grad_X[iX] = gC[iC] * coef;
+                    iX += cX <= cC;
+                    iC += cC <= cX;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+inline unsigned lc_grid(int64_t rows) {
+    int64_t g = nm::xcd_padded(nm::ceil_div(rows, kLcRows));
+    if (g > nm::kMaxGrid) g = nm::kMaxGrid;
+    return (unsigned)g;
 }
 
 inline unsigned grid_for(int64_t n) {
@@ -360,7 +509,7 @@ extern "C" int nm_splincomb_symbolic(int64_t rows, const int64_t *A_indices, con
     hipStream_t s = nm::as_stream(stream);
     if (int rc = nm::fill_async(C_indptr + rows, 1, (int64_t)0, s)) return rc;
     if (rows == 0) return NM_OK;
-    hipLaunchKernelGGL((lincomb_kernel<float, true>), dim3(grid_for(rows * 4)), dim3(kBlock), 0, s, rows, 0.0f,
+    hipLaunchKernelGGL((lincomb_kernel<float, true>), dim3(lc_grid(rows)), dim3(kBlock), 0, s, rows, 0.0f,
                        (const float *)nullptr, A_indices, A_indptr, 0.0f, (const float *)nullptr, B_indices,
                        B_indptr, C_indptr, (int64_t *)nullptr, (float *)nullptr);
     NM_LAUNCH_CHECK("lincomb_kernel<count>");
@@ -377,12 +526,12 @@ extern "C" int nm_splincomb_numeric(nm_dtype dt, int64_t rows, double alpha, con
     NM_REQUIRE(A_indptr && B_indptr && C_indptr, "null pointer argument");
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
-        hipLaunchKernelGGL((lincomb_kernel<float, false>), dim3(grid_for(rows * 4)), dim3(kBlock), 0, s, rows,
+        hipLaunchKernelGGL((lincomb_kernel<float, false>), dim3(lc_grid(rows)), dim3(kBlock), 0, s, rows,
                            (float)alpha, (const float *)A_data, A_indices, A_indptr, (float)beta,
                            (const float *)B_data, B_indices, B_indptr, const_cast<int64_t *>(C_indptr), C_indices,
                            (float *)C_data);
     else
-        hipLaunchKernelGGL((lincomb_kernel<double, false>), dim3(grid_for(rows * 4)), dim3(kBlock), 0, s, rows, alpha,
+        hipLaunchKernelGGL((lincomb_kernel<double, false>), dim3(lc_grid(rows)), dim3(kBlock), 0, s, rows, alpha,
                            (const double *)A_data, A_indices, A_indptr, beta, (const double *)B_data, B_indices,
                            B_indptr, const_cast<int64_t *>(C_indptr), C_indices, (double *)C_data);
     NM_LAUNCH_CHECK("lincomb_kernel");
@@ -398,7 +547,7 @@ extern "C" int nm_splincomb_backward(nm_dtype dt, int64_t rows, double alpha, co
     if (rows == 0) return NM_OK;
     NM_REQUIRE(C_indptr, "null pointer argument");
     hipStream_t s = nm::as_stream(stream);
-    const unsigned grid = grid_for(rows * 4);
+    const unsigned grid = lc_grid(rows);
     for (int side = 0; side < 2; ++side) {
         void *out = side == 0 ? grad_A : grad_B;
         if (!out) continue;
