@@ -396,10 +396,39 @@ class SparseCSRTensor(object):
         return self.diagonal().sum()
 
     # ---- conversions ----------------------------------------------------------
+    @property
     def row_indices(self):
+        """Row of every stored entry (numml/sparse/_csr.py:1002-1014)."""
         counts = self.indptr[1:] - self.indptr[:-1]
         return torch.repeat_interleave(
             torch.arange(self.shape[0], device=self.indptr.device), counts)
+
+    @property
+    def diagonal_idx(self):
+        """Position of the stored diagonal entry of each row, -1 where a row has none
+        (numml/sparse/_csr.py:985-1000)."""
+        n = min(self.shape)
+        idx = torch.full((n,), -1, dtype=torch.int64, device=self.indices.device)
+        rows = self.row_indices
+        hit = (self.indices == rows) & (rows < n)
+        idx[rows[hit]] = torch.nonzero(hit).flatten()
+        return idx
+
+    def _band(self, keep):
+        rows = self.row_indices
+        counts = torch.bincount(rows[keep], minlength=self.shape[0])
+        indptr = torch.zeros(self.shape[0] + 1, dtype=torch.int64, device=self.indptr.device)
+        indptr[1:] = torch.cumsum(counts, 0)
+        # indexing keeps the gradient path to the selected entries; the others get zero
+        return SparseCSRTensor((self.data[keep], self.indices[keep], indptr), self.shape)
+
+    def tril(self, k=0):
+        """Entries with column <= row + k (numml/sparse/_csr.py:234-280, 1063-1065)."""
+        return self._band(self.indices <= self.row_indices + k)
+
+    def triu(self, k=0):
+        """Entries with column >= row + k (numml/sparse/_csr.py:283-330, 1067-1069)."""
+        return self._band(self.indices >= self.row_indices + k)
 
     def to_dense(self):
         """Dense copy; gradients flow to and from the stored entries
@@ -408,7 +437,7 @@ class SparseCSRTensor(object):
 
     def to_coo(self):
         """(values, rows, cols) of the stored entries."""
-        return self.data, self.row_indices(), self.indices
+        return self.data, self.row_indices, self.indices
 
     def to_scipy_csr(self):
         import scipy.sparse as sp

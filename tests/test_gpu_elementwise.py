@@ -111,11 +111,35 @@ def test_operators_and_gradients(dev):
     w = to_dev(dev, randn(1, n, np.float64))[0]
     loss = ((A - B).row_sum() * w).sum() + (A + B).diagonal().sum() + (A.to_dense() ** 2).sum() + A.trace()
     loss.backward()
-    rows_a = A.row_indices()
-    rows_b = B.row_indices()
+    rows_a = A.row_indices
+    rows_b = B.row_indices
     gA = w[rows_a] + (A.indices == rows_a) * 2.0 + 2 * A.data.detach()
     gB = -w[rows_b] + (B.indices == rows_b) * 1.0
     assert torch.allclose(A.data.grad, gA, atol=1e-12) and torch.allclose(B.data.grad, gB, atol=1e-12)
     with pytest.raises(RuntimeError, match="Incompatible shapes"):
         A + sp.eye(3, dtype=torch.float64, device=dev)
     assert torch.equal(A.sum(), A.data.sum())
+
+
+def test_triangles_and_diagonal_index(dev):
+    import scipy.sparse as sps
+    d, i, p, (n, _) = G.poisson2d(9, np.float64, 2)
+    A = sp.SparseCSRTensor(tuple(to_dev(dev, d, i, p)), (n, n))
+    A.requires_grad = True
+    S = sps.csr_matrix((d, i, p), shape=(n, n))
+    for k in (-1, 0, 2):
+        for mine, theirs in ((A.tril(k), sps.tril(S, k).tocsr()), (A.triu(k), sps.triu(S, k).tocsr())):
+            theirs.sort_indices()
+            assert_same(host(mine.indptr), theirs.indptr.astype(np.int64), "indptr")
+            assert_same(host(mine.indices), theirs.indices.astype(np.int64), "indices")
+            assert_same(host(mine.data), theirs.data, "data")
+    # a solve with the lower triangle, differentiated back to A: entries above the diagonal get zero
+    b = to_dev(dev, randn(1, n, np.float64))[0]
+    x = A.tril().solve_triangular(upper=False, unit=False, b=b)
+    x.sum().backward()
+    upper = A.indices > A.row_indices
+    assert not bool(A.data.grad[upper].any()) and bool(A.data.grad[~upper].any())
+    rows = np.repeat(np.arange(n), np.diff(p))
+    want = np.full(n, -1, np.int64)
+    want[rows[i == rows]] = np.nonzero(i == rows)[0]
+    assert_same(host(A.diagonal_idx), want, "diagonal_idx")
