@@ -184,3 +184,17 @@ def random_tri(n, density, seed, lower=True, dtype=np.float64, diag=True,
     indptr = np.zeros(n + 1, dtype=np.int64)
     np.cumsum(np.bincount(r, minlength=n), out=indptr[1:])
     return vals.astype(dtype), c.astype(np.int64), indptr, (n, n)
+
+
+def ragged_csr(rows, cols, max_len, seed, dtype=np.float64, min_len=0):
+    """Rows of independently drawn lengths in [min_len, max_len] (uniform), columns drawn
+    without replacement and sorted, N(0,1) values: mixes empty, short and longer rows."""
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(min_len, min(max_len, cols) + 1, rows)
+    indptr = np.zeros(rows + 1, dtype=np.int64)
+    np.cumsum(lens, out=indptr[1:])
+    indices = np.empty(indptr[-1], dtype=np.int64)
+    for r in range(rows):
+        indices[indptr[r]:indptr[r + 1]] = np.sort(rng.choice(cols, lens[r], replace=False))
+    data = rng.standard_normal(indptr[-1]).astype(dtype)
+    return data, indices, indptr, (rows, cols)

@@ -125,6 +125,32 @@ def test_spgemm_forward_backward(dev, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_spgemm_mixed_short_and_long_rows(dev, dtype):
+    """Rows that take the merge path (A row and its B rows of at most 8 entries) next to
+    rows that do not, inside the same wavefront: lengths 0..8, exactly 8, 9 and longer."""
+    cases = [
+        ("all_le_8", G.ragged_csr(700, 500, 8, 1, dtype), G.ragged_csr(500, 600, 8, 2, dtype)),
+        ("a_le_10_b_le_10", G.ragged_csr(1000, 400, 10, 3, dtype), G.ragged_csr(400, 450, 10, 4, dtype)),
+        ("full_8", G.ragged_csr(300, 300, 8, 5, dtype, min_len=8), G.ragged_csr(300, 64, 8, 6, dtype, min_len=8)),
+        ("b_long", G.ragged_csr(257, 100, 4, 7, dtype), G.ragged_csr(100, 3000, 40, 8, dtype)),
+        ("narrow_b", G.ragged_csr(513, 90, 8, 9, dtype), G.ragged_csr(90, 3, 3, 10, dtype)),
+        ("one_row", G.ragged_csr(1, 20, 8, 11, dtype, min_len=5), G.ragged_csr(20, 30, 8, 12, dtype)),
+    ]
+    for name, (ad, ai, ap, (ar, ac)), (bd, bi, bp, (br, bc)) in cases:
+        Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(ar, ac, ad, ai, ap, br, bc, bd, bi, bp)
+        gC = randn(9, Cd_ref.shape[0], dtype)
+        gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, ar, ac, ad, ai, ap, br, bc, bd, bi, bp)
+        AD, AI, AP, BD, BI, BP, GC = to_dev(dev, ad, ai, ap, bd, bi, bp, gC)
+        Cd, Ci, Cp = ext.spgemm_forward(ar, ac, AD, AI, AP, br, bc, BD, BI, BP)
+        assert_same(host(Cp), Cp_ref, f"{name} C_indptr")
+        assert_same(host(Ci), Ci_ref, f"{name} C_indices")
+        assert_same(host(Cd), Cd_ref, f"{name} C_data")
+        gA, gB = ext.spgemm_backward(GC, Ci, Cp, ar, ac, AD, AI, AP, br, bc, BD, BI, BP)
+        assert_same(host(gA), gA_ref, f"{name} grad_A")
+        assert_close(host(gB), gB_ref, f"{name} grad_B")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("lower", [True, False])
 @pytest.mark.parametrize("unit", [False, True])
 def test_sptrsv_forward_backward(dev, dtype, lower, unit):
