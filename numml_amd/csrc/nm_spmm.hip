@@ -149,36 +149,96 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
             }
             row = lo - 1;
         }
-        int64_t row_end = indptr[row + 1];
+        // The ends of the next 64 rows sit one per lane, so that stepping over a row
+        // boundary is a lane read and not a dependent global load (which would put a
+        // memory round trip between two batches of gathers every few entries).
+        int64_t ends_row = row;   // lane l holds indptr[ends_row + 1 + l]
+        auto load_ends = [&](int64_t first) {
+            const int64_t r = first + 1 + lane;
+            return indptr[r <= rows ? r : rows];
+        };
+        int64_t my_end = load_ends(ends_row);
+        auto end_of = [&](int64_t r) {
+            const int l = __builtin_amdgcn_readfirstlane((int)(r - ends_row));
+            const long long lo = __builtin_amdgcn_readlane((int)(my_end & 0xffffffffll), l);
+            const long long hi = __builtin_amdgcn_readlane((int)(my_end >> 32), l);
+            return (int64_t)((hi << 32) | (lo & 0xffffffffll));
+        };
+        int64_t row_end = end_of(row);
         T mydot = 0;
-        for (int j0 = 0; j0 < cnt; j0 += kBatch) {
-            int64_t col[kBatch], rw[kBatch];
+        // rows and columns of the entries [j0, j0 + kBatch) of the chunk
+        auto locate = [&](int j0, int64_t (&col)[kBatch], int64_t (&rw)[kBatch]) {
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 const int j = j0 + u < cnt ? j0 + u : cnt - 1;
-                while (kb + j >= row_end) { ++row; row_end = indptr[row + 1]; }
+                while (kb + j >= row_end) {
+                    ++row;
+                    if (row - ends_row >= kWave) {   // more than 64 rows inside one chunk: empty rows
+                        ends_row = row;
+                        my_end = load_ends(ends_row);
+                    }
+                    row_end = end_of(row);
+                }
                 rw[u] = row;
                 col[u] = __shfl(mycol, j, kWave);
             }
-            for (int64_t c0 = 0; c0 < n; c0 += kWave) {
-                const int64_t c = c0 + lane;
-                const bool live = c < n;
-                T bv[kBatch], gv[kBatch];
+        };
+        auto fetch = [&](const int64_t (&col)[kBatch], const int64_t (&rw)[kBatch], int64_t c, bool live,
+                         T (&gv)[kBatch], T (&bv)[kBatch]) {
 #pragma unroll
-                for (int u = 0; u < kBatch; ++u) {
-                    gv[u] = live ? gC[rw[u] * ldg + c] : T(0);
-                    bv[u] = (live && grad_A) ? B[col[u] * ldb + c] : T(0);
-                }
+            for (int u = 0; u < kBatch; ++u) {
+                gv[u] = gC[rw[u] * ldg + (live ? c : 0)];
+                bv[u] = grad_A ? B[col[u] * ldb + (live ? c : 0)] : T(0);
+            }
+        };
+        // Sums over the wavefront of kBatch (= 8) lane-wise products at once.  Three
+        // folding steps halve the number of vectors while pairing lanes 1, 2 and 4 apart,
+        // after which lane l holds the partial sum of vector l & 7 over its group of 8
+        // lanes; three more steps add the eight groups.  27 instructions instead of
+        // 8 full reductions; the result for vector u is in every lane with (l & 7) == u.
+        auto reduce8 = [&](const T (&p)[kBatch]) {
+            static_assert(kBatch == 8, "reduce8 folds eight vectors");
+            const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
+            T q[4], r[2];
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+                q[m] = (b0 ? p[2 * m + 1] : p[2 * m]) + nm::dpp_move<0xB1>(b0 ? p[2 * m] : p[2 * m + 1]);
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+                r[m] = (b1 ? q[2 * m + 1] : q[2 * m]) + nm::dpp_move<0x4E>(b1 ? q[2 * m] : q[2 * m + 1]);
+            T t = (b2 ? r[1] : r[0]) + __shfl_xor(b2 ? r[0] : r[1], 4, kWave);
+            t += nm::dpp_move<0x128>(t);          // row_ror 8: the other group of the 16-lane row
+            t += __shfl_xor(t, 16, kWave);
+            t += __shfl_xor(t, 32, kWave);
+            return t;
+        };
+        auto consume = [&](int j0, const int64_t (&col)[kBatch], int64_t c, bool live, const T (&gv)[kBatch],
+                           const T (&bv)[kBatch]) {
+            if (grad_B) {
 #pragma unroll
                 for (int u = 0; u < kBatch; ++u) {
                     if (j0 + u >= cnt) break;
                     const T av = __shfl(myval, j0 + u, kWave);   // all lanes take part in the broadcast
-                    if (grad_B && live) nm::atomic_add(grad_B + col[u] * ldgb + c, av * gv[u]);
-                    if (grad_A) {
-                        const T part = nm::wave_sum(gv[u] * bv[u]);
-                        if (lane == j0 + u) mydot += part;
-                    }
+                    if (live) nm::atomic_add(grad_B + col[u] * ldgb + c, av * gv[u]);
                 }
+            }
+            if (grad_A) {
+                T p[kBatch];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) p[u] = live ? gv[u] * bv[u] : T(0);
+                const T t = reduce8(p);
+                if ((lane >> 3) == (j0 >> 3)) mydot += t;   // lane j0 + u takes vector u
+            }
+        };
+        for (int j0 = 0; j0 < cnt; j0 += kBatch) {
+            int64_t col[kBatch], rw[kBatch];
+            locate(j0, col, rw);
+            for (int64_t c0 = 0; c0 < n; c0 += kWave) {
+                const int64_t c = c0 + lane;
+                const bool live = c < n;
+                T bv[kBatch], gv[kBatch];
+                fetch(col, rw, c, live, gv, bv);
+                consume(j0, col, c, live, gv, bv);
             }
         }
         if (grad_A && lane < cnt) grad_A[k] = mydot;
