@@ -320,7 +320,12 @@ template <int PRE> __device__ __forceinline__ Vals<PRE> load_vals(const SolveArg
 // Levels l0, l0+step, ... (`count` <= kMaxLevels of them, each at most kNarrow
 // rows) by one workgroup; [qlo, qhi) are the slots this launch solves (only
 // those can be found in the ring).
-template <int PRE>
+// Global loads reach the registers through two stages, each issued DEPTH levels
+// before it is needed: the slot's dependency range (`Meta`), then the dependencies
+// themselves (`Vals`, whose addresses come from the range).  A level takes a few
+// hundred cycles once its operands are in registers but a global load takes one to
+// two thousand, so with DEPTH = 1 every level waited for memory.
+template <int PRE, int DEPTH>
 __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l0, int count, int step, int qlo,
                                                               int qhi) {
     __shared__ double ring[kRing];
@@ -329,54 +334,62 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
     for (int i = threadIdx.x; i <= count; i += kNarrow) s_lp[i] = a.level_ptr[lmin + i];
     __syncthreads();
 
-    Bounds p0 = load_bounds(s_lp, 0, count, l0, step, lmin);
-    Meta p1 = load_meta(a, p0);
-    p0 = load_bounds(s_lp, 1, count, l0, step, lmin);
-    Vals<PRE> p2 = load_vals<PRE>(a, p1);
-    p1 = load_meta(a, p0);
-    p0 = load_bounds(s_lp, 2, count, l0, step, lmin);
-
-    for (int it = 0; it < count; ++it) {
-        const Vals<PRE> cur = p2;
-        // advance the pipeline: what is issued here is consumed one and two levels later
-        p2 = load_vals<PRE>(a, p1);
-        p1 = load_meta(a, p0);
-        p0 = load_bounds(s_lp, it + 3, count, l0, step, lmin);
-
-        const int q = cur.m.q;
-        const int n = cur.m.live ? cur.m.n : 0;
-        // fast path: no global memory access at all -- every dependency from the LDS ring
-        double acc = 0.;
-        bool in_ring = n <= PRE;
+    Meta qm[DEPTH];          // ranges of levels it + DEPTH .. it + 2 DEPTH - 1
+    Vals<PRE> qv[DEPTH];     // operands of levels it .. it + DEPTH - 1
 #pragma unroll
-        for (int e = 0; e < PRE; ++e) {
-            const int32_t ds = cur.ds[e];
-            const int dist = ds > q ? ds - q : q - ds;
-            const bool hit = ds >= qlo && ds < qhi && dist < kRingSafe;
-            const double xj = ring[ds & (kRing - 1)];
-            if (e < n) {
-                in_ring = in_ring && hit;
-                acc += cur.v[e] * xj;
+    for (int d = 0; d < DEPTH; ++d) qm[d] = load_meta(a, load_bounds(s_lp, d, count, l0, step, lmin));
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) qv[d] = load_vals<PRE>(a, qm[d]);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) qm[d] = load_meta(a, load_bounds(s_lp, DEPTH + d, count, l0, step, lmin));
+
+    // The level loop is unrolled DEPTH times so that stage d always lives in the same
+    // registers: a stage is consumed and then refilled in place.  (Rotating the stages
+    // through register copies made every level wait for the loads it had just issued.)
+    for (int it0 = 0; it0 < count; it0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int it = it0 + d;
+            if (it >= count) break;   // uniform over the workgroup
+            const Vals<PRE> cur = qv[d];
+            qv[d] = load_vals<PRE>(a, qm[d]);
+            qm[d] = load_meta(a, load_bounds(s_lp, it + 2 * DEPTH, count, l0, step, lmin));
+
+            const int q = cur.m.q;
+            const int n = cur.m.live ? cur.m.n : 0;
+            // fast path: no global memory access at all -- every dependency from the LDS ring
+            double acc = 0.;
+            bool in_ring = n <= PRE;
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) {
+                const int32_t ds = cur.ds[e];
+                const int dist = ds > q ? ds - q : q - ds;
+                const bool hit = ds >= qlo && ds < qhi && dist < kRingSafe;
+                const double xj = ring[ds & (kRing - 1)];
+                if (e < n) {
+                    in_ring = in_ring && hit;
+                    acc += cur.v[e] * xj;
+                }
             }
-        }
-        if (!in_ring) {
-            // slow path (a dependency older than the ring, or a row longer than the
-            // pipeline holds): redo the whole sum in the same order from global memory
-            acc = 0.;
-            for (int e = 0; e < n; ++e) {
-                const int32_t at = cur.m.dlo + e;
-                const int32_t ds = e < PRE ? cur.ds[e] : a.dslot[at];
-                const double v = e < PRE ? cur.v[e] : a.w.coef[at];
-                acc += v * a.w.xs[ds];
+            if (!in_ring) {
+                // slow path (a dependency older than the ring, or a row longer than the
+                // pipeline holds): redo the whole sum in the same order from global memory
+                acc = 0.;
+                for (int e = 0; e < n; ++e) {
+                    const int32_t at = cur.m.dlo + e;
+                    const int32_t ds = e < PRE ? cur.ds[e] : a.dslot[at];
+                    const double v = e < PRE ? cur.v[e] : a.w.coef[at];
+                    acc += v * a.w.xs[ds];
+                }
             }
+            if (cur.m.live) {
+                double xi = cur.bv - acc;
+                if (!a.unit) xi /= cur.dv;
+                ring[q & (kRing - 1)] = xi;
+                a.w.xs[q] = xi;
+            }
+            __syncthreads();
         }
-        if (cur.m.live) {
-            double xi = cur.bv - acc;
-            if (!a.unit) xi /= cur.dv;
-            ring[q & (kRing - 1)] = xi;
-            a.w.xs[q] = xi;
-        }
-        __syncthreads();
     }
 }
 
@@ -434,11 +447,11 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
             // holds this direction's longest row (longer rows take the slow path)
             const int maxdep = p->max_deps[transposed ? 1 : 0];
             if (maxdep <= 2)
-                hipLaunchKernelGGL(sptrsv_ring_kernel<2>, dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ring_kernel<2, 4>), dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
             else if (maxdep <= 4)
-                hipLaunchKernelGGL(sptrsv_ring_kernel<4>, dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ring_kernel<4, 3>), dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
             else
-                hipLaunchKernelGGL(sptrsv_ring_kernel<8>, dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ring_kernel<8, 2>), dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
             NM_LAUNCH_CHECK("sptrsv_ring_kernel");
         }
     }
