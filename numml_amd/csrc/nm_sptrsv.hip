@@ -57,6 +57,7 @@ struct nm_sptrsv_plan {
         int32_t l0, l1;  // levels [l0, l1)
         int32_t q0, q1;  // slots they cover
         bool wide;       // one level, many workgroups
+        int32_t block;   // lanes of the single-workgroup launch (narrow runs)
     };
     std::vector<Launch> launches;
 };
@@ -331,7 +332,7 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
     __shared__ double ring[kRing];
     __shared__ int32_t s_lp[kMaxLevels + 1];
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
-    for (int i = threadIdx.x; i <= count; i += kNarrow) s_lp[i] = a.level_ptr[lmin + i];
+    for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
     __syncthreads();
 
     Meta qm[DEPTH];          // ranges of levels it + DEPTH .. it + 2 DEPTH - 1
@@ -447,11 +448,11 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
             // holds this direction's longest row (longer rows take the slow path)
             const int maxdep = p->max_deps[transposed ? 1 : 0];
             if (maxdep <= 2)
-                hipLaunchKernelGGL((sptrsv_ring_kernel<2, 4>), dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ring_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             else if (maxdep <= 4)
-                hipLaunchKernelGGL((sptrsv_ring_kernel<4, 3>), dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ring_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             else
-                hipLaunchKernelGGL((sptrsv_ring_kernel<8, 2>), dim3(1), dim3(kNarrow), 0, s, a, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ring_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             NM_LAUNCH_CHECK("sptrsv_ring_kernel");
         }
     }
@@ -561,12 +562,48 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         hipStreamSynchronize(s) != hipSuccess)
         return bail(nm::fail(NM_ERR_HIP, "reading the level sizes back failed"));
 
-    // consecutive narrow levels share one single-workgroup launch (at most kMaxLevels each)
+    // Consecutive narrow levels share one single-workgroup launch (at most kMaxLevels
+    // each).  The workgroup runs on one CU, where every wavefront -- also one without a
+    // row in the current level -- costs issue slots on the level's critical path
+    // (measured: 0.36 us per level with one wavefront, 0.78 us with sixteen), so a run
+    // is cut into segments by level width and each segment is launched with the
+    // smallest power-of-two workgroup (64 .. kNarrow lanes) that holds its widest level.
+    auto lanes_for = [&](int32_t l) {
+        const int32_t w = lp[l + 1] - lp[l];
+        int32_t b = 64;
+        while (b < w) b *= 2;
+        return b;
+    };
+    constexpr int32_t kMinSegment = 32;   // levels; shorter segments are not worth a launch
     auto push_narrow = [&](int32_t a0, int32_t a1) {
-        for (int32_t c0 = a0; c0 < a1; c0 += kMaxLevels) {
-            const int32_t c1 = c0 + kMaxLevels < a1 ? c0 + kMaxLevels : a1;
-            p->launches.push_back({c0, c1, lp[c0], lp[c1], false});
+        int32_t s0 = a0, block = lanes_for(a0);
+        auto flush = [&](int32_t end) {
+            for (int32_t c0 = s0; c0 < end; c0 += kMaxLevels) {
+                const int32_t c1 = c0 + kMaxLevels < end ? c0 + kMaxLevels : end;
+                p->launches.push_back({c0, c1, lp[c0], lp[c1], false, block});
+            }
+        };
+        for (int32_t l = a0 + 1; l < a1; ++l) {
+            const int32_t b = lanes_for(l);
+            if (b > block) {
+                // wider than the segment allows: widen a young segment, else start a new one
+                if (l - s0 < kMinSegment) { block = b; continue; }
+                flush(l);
+                s0 = l;
+                block = b;
+            } else if (b < block && l - s0 >= kMinSegment) {
+                // narrower: worth a new segment only if it stays narrower for a while
+                int32_t widest = b;
+                const int32_t look = l + kMinSegment < a1 ? l + kMinSegment : a1;
+                for (int32_t m = l; m < look; ++m) widest = widest > lanes_for(m) ? widest : lanes_for(m);
+                if (widest < block && look - l >= kMinSegment) {
+                    flush(l);
+                    s0 = l;
+                    block = widest;
+                }
+            }
         }
+        flush(a1);
     };
     int32_t run0 = -1;
     for (int32_t l = 0; l < p->nlevels; ++l) {
@@ -576,7 +613,7 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             continue;
         }
         if (run0 >= 0) { push_narrow(run0, l); run0 = -1; }
-        p->launches.push_back({l, l + 1, lp[l], lp[l + 1], true});
+        p->launches.push_back({l, l + 1, lp[l], lp[l + 1], true, kBlock});
     }
     if (run0 >= 0) push_narrow(run0, p->nlevels);
     *plan_out = p;
