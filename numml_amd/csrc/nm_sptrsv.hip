@@ -42,7 +42,10 @@ struct Packed {        // one solve direction, level-major (all int32, device)
     int32_t *dslot;    // [nnz]    slot of the row a dependency refers to
     int32_t *dsrc;     // [nnz]    position of its coefficient in A's data
     int32_t *diag;     // [rows]   position of the diagonal coefficient, -1 when not stored
+    int32_t *ell_ds;   // [ell_capacity] fixed-width copy of dslot: `pre` slots per row, -1 padded
 };
+// Entries of the fixed-width (ELLPACK) arrays; the layout is used when rows * pre fits.
+inline int64_t ell_capacity(int64_t rows, int64_t nnz) { return 2 * nnz + 2 * rows + 8; }
 }  // namespace
 
 struct nm_sptrsv_plan {
@@ -53,6 +56,7 @@ struct nm_sptrsv_plan {
     int32_t *order = nullptr, *level_ptr = nullptr, *slot_of = nullptr;
     Packed dir[2];     // [0]: A, [1]: A^T
     int32_t max_deps[2] = {0, 0};  // longest dependency list per direction
+    int32_t ell_pre[2] = {0, 0};   // width of the fixed-width layout per direction (2, 4, 8; 0 = not used)
     struct Launch {
         int32_t l0, l1;  // levels [l0, l1)
         int32_t q0, q1;  // slots they cover
@@ -96,6 +100,7 @@ size_t plan_layout(int64_t rows, int64_t nnz, void *base, Layout *L) {
         l.dir[d].dslot = take(nnz + 1);
         l.dir[d].dsrc = take(nnz + 1);
         l.dir[d].diag = take(rows + 1);
+        l.dir[d].ell_ds = take(ell_capacity(rows, nnz));
     }
     if (L) *L = l;
     return off;
@@ -230,6 +235,8 @@ struct SolveWork {
     double *dg;     // diagonal coefficient of slot q (0 when not stored)
     double *rhs;    // right-hand side of slot q
     double *coef;   // coefficient of packed dependency `at`
+    double *ell_coef;  // fixed-width copy of coef (0 padded), `pre` per slot
+    double *rb;        // (right-hand side, diagonal) pairs per slot
 };
 
 inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork *W) {
@@ -244,6 +251,8 @@ inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork
     w.dg = take(rows + 1);
     w.rhs = take(rows + 1);
     w.coef = take(nnz + 1);
+    w.ell_coef = take(ell_capacity(rows, nnz));
+    w.rb = take(2 * rows + 2);
     if (W) *W = w;
     return off;
 }
@@ -394,6 +403,136 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
     }
 }
 
+// ---- fixed-width (ELLPACK) variant of the single-workgroup kernel -----------------
+//
+// When no row has more than 8 dependencies, the packed triangle is also kept with a
+// fixed number PRE of dependency slots per row (-1 / 0.0 padded).  Every address a
+// level needs is then a multiple of its slot number: one vector load each for the
+// PRE dependency slots, the PRE coefficients and the (rhs, diagonal) pair, no
+// dependency-range stage in front of them, and a third of the address arithmetic --
+// which matters because the workgroup's wavefronts share one CU and the level time
+// is the time to issue their instructions.
+
+__global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict__ dptr,
+                                const int32_t *__restrict__ dslot, int32_t *__restrict__ ell_ds) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows * pre; i += stride) {
+        const int64_t q = i / pre;
+        const int e = (int)(i - q * pre);
+        const int32_t lo = dptr[q], n = dptr[q + 1] - lo;
+        ell_ds[i] = e < n ? dslot[lo + e] : -1;
+    }
+}
+
+template <typename T>
+__global__ void gather_ell_kernel(int64_t rows, int pre, const T *__restrict__ data, const T *__restrict__ b,
+                                  const int32_t *__restrict__ order, const int32_t *__restrict__ dptr,
+                                  const int32_t *__restrict__ dsrc, const int32_t *__restrict__ diag,
+                                  double *__restrict__ ell_coef, double *__restrict__ rb) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (int64_t i = tid; i < rows * pre; i += stride) {
+        const int64_t q = i / pre;
+        const int e = (int)(i - q * pre);
+        const int32_t lo = dptr[q], n = dptr[q + 1] - lo;
+        ell_coef[i] = e < n ? (double)data[dsrc[lo + e]] : 0.;
+    }
+    for (int64_t q = tid; q < rows; q += stride) {
+        const int32_t d = diag[q];
+        rb[2 * q] = (double)b[order[q]];
+        rb[2 * q + 1] = d >= 0 ? (double)data[d] : 0.;
+    }
+}
+
+struct EllArgs {
+    const int32_t *level_ptr, *ell_ds;
+    const double *ell_coef, *rb;
+    double *xs;
+    int unit;
+};
+
+template <int PRE> struct EllVals {
+    int q;
+    bool live;
+    int32_t ds[PRE];
+    double v[PRE];
+    double bv, dv;
+};
+
+template <int PRE> __device__ __forceinline__ EllVals<PRE> load_ell(const EllArgs &a, const Bounds &b) {
+    typedef int32_t IV __attribute__((ext_vector_type(PRE)));
+    typedef double DV __attribute__((ext_vector_type(PRE)));
+    typedef double D2 __attribute__((ext_vector_type(2)));
+    EllVals<PRE> v;
+    v.q = b.qb + (int)threadIdx.x;
+    v.live = v.q < b.qe;
+    const unsigned qs = v.live ? (unsigned)v.q : 0u;   // unconditional loads: slot 0 always exists
+    const IV dsv = reinterpret_cast<const IV *>(a.ell_ds)[qs];
+    const DV cv = reinterpret_cast<const DV *>(a.ell_coef)[qs];
+    const D2 r = reinterpret_cast<const D2 *>(a.rb)[qs];
+#pragma unroll
+    for (int e = 0; e < PRE; ++e) {
+        v.ds[e] = dsv[e];
+        v.v[e] = cv[e];
+    }
+    v.bv = r[0];
+    v.dv = r[1];
+    return v;
+}
+
+template <int PRE, int DEPTH>
+__global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step, int qlo,
+                                                             int qhi) {
+    __shared__ double ring[kRing];
+    __shared__ int32_t s_lp[kMaxLevels + 1];
+    const int lmin = step > 0 ? l0 : l0 - (count - 1);
+    for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
+    __syncthreads();
+
+    EllVals<PRE> qv[DEPTH];   // operands of levels it .. it + DEPTH - 1, each refilled in place
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, load_bounds(s_lp, d, count, l0, step, lmin));
+
+    for (int it0 = 0; it0 < count; it0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int it = it0 + d;
+            if (it >= count) break;   // uniform over the workgroup
+            const EllVals<PRE> cur = qv[d];
+            qv[d] = load_ell<PRE>(a, load_bounds(s_lp, it + DEPTH, count, l0, step, lmin));
+
+            const int q = cur.q;
+            double acc = 0.;
+            bool in_ring = true;
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) {
+                const int32_t ds = cur.ds[e];
+                const int dist = ds > q ? ds - q : q - ds;
+                const bool hit = ds >= qlo && ds < qhi && dist < kRingSafe;
+                const double xj = ring[ds & (kRing - 1)];
+                if (cur.live && ds >= 0) {
+                    in_ring = in_ring && hit;
+                    acc += cur.v[e] * xj;
+                }
+            }
+            if (!in_ring) {
+                // a dependency older than the ring: redo the sum in the same order from global memory
+                acc = 0.;
+#pragma unroll
+                for (int e = 0; e < PRE; ++e)
+                    if (cur.ds[e] >= 0) acc += cur.v[e] * a.xs[cur.ds[e]];
+            }
+            if (cur.live) {
+                double xi = cur.bv - acc;
+                if (!a.unit) xi /= cur.dv;
+                ring[q & (kRing - 1)] = xi;
+                a.xs[q] = xi;
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // One wide level: slots [q0, q1), one lane per row.
 __global__ __launch_bounds__(kBlock) void sptrsv_level_kernel(SolveArgs a, int q0, int q1) {
     const int q = q0 + (int)(blockIdx.x * blockDim.x + threadIdx.x);
@@ -424,7 +563,9 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     a.dptr = P.dptr;
     a.dslot = P.dslot;
     a.unit = unit;
-    {
+    bool any_wide = false;
+    for (const auto &L : p->launches) any_wide = any_wide || L.wide;
+    if (any_wide || p->ell_pre[transposed ? 1 : 0] == 0) {   // the range-based arrays have readers
         int64_t m = p->nnz > p->rows ? p->nnz : p->rows;
         int64_t grid = nm::ceil_div(m, kBlock);
         if (grid > 65536) grid = 65536;
@@ -433,6 +574,17 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
         hipLaunchKernelGGL(gather_values_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, p->rows, p->nnz, dat,
                            (const T *)b, p->order, P.dptr, P.dsrc, P.diag, a.w.coef, a.w.dg, a.w.rhs);
         NM_LAUNCH_CHECK("gather_values_kernel");
+    }
+    const int dirn = transposed ? 1 : 0;
+    const int pre = p->ell_pre[dirn];
+    EllArgs ea{p->level_ptr, P.ell_ds, a.w.ell_coef, a.w.rb, a.w.xs, unit};
+    if (pre > 0) {
+        int64_t grid = nm::ceil_div(p->rows * pre, kBlock);
+        if (grid > 65536) grid = 65536;
+        const T *dat = p->nnz > 0 ? (const T *)data : (const T *)b;
+        hipLaunchKernelGGL(gather_ell_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, p->rows, pre, dat,
+                           (const T *)b, p->order, P.dptr, P.dsrc, P.diag, a.w.ell_coef, a.w.rb);
+        NM_LAUNCH_CHECK("gather_ell_kernel");
     }
     const int n = (int)p->launches.size();
     for (int li = 0; li < n; ++li) {
@@ -447,7 +599,13 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
             // dependencies per row fetched ahead through registers: the smallest pipeline that
             // holds this direction's longest row (longer rows take the slow path)
             const int maxdep = p->max_deps[transposed ? 1 : 0];
-            if (maxdep <= 2)
+            if (pre == 2)
+                hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step, L.q0, L.q1);
+            else if (pre == 4)
+                hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step, L.q0, L.q1);
+            else if (pre == 8)
+                hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step, L.q0, L.q1);
+            else if (maxdep <= 2)
                 hipLaunchKernelGGL((sptrsv_ring_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             else if (maxdep <= 4)
                 hipLaunchKernelGGL((sptrsv_ring_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
@@ -557,6 +715,18 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     p->nlevels = meta_h[0];
     p->max_deps[0] = meta_h[2];
     p->max_deps[1] = meta_h[3];
+    for (int d = 0; d < 2; ++d) {
+        const int32_t md = p->max_deps[d];
+        const int pre = md <= 2 ? 2 : (md <= 4 ? 4 : (md <= 8 ? 8 : 0));
+        if (pre > 0 && rows * pre <= ell_capacity(rows, nnz)) {
+            p->ell_pre[d] = pre;
+            int64_t grid = nm::ceil_div(rows * pre, kBlock);
+            if (grid > 65536) grid = 65536;
+            hipLaunchKernelGGL(ell_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, pre, p->dir[d].dptr,
+                               p->dir[d].dslot, p->dir[d].ell_ds);
+            if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
+        }
+    }
     std::vector<int32_t> lp((size_t)p->nlevels + 1);
     if (hipMemcpyAsync(lp.data(), p->level_ptr, lp.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess)
@@ -616,6 +786,8 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         p->launches.push_back({l, l + 1, lp[l], lp[l + 1], true, kBlock});
     }
     if (run0 >= 0) push_narrow(run0, p->nlevels);
+    if (hipStreamSynchronize(s) != hipSuccess)   // the fixed-width copies were enqueued after the read-back
+        return bail(nm::fail(NM_ERR_HIP, "waiting for the plan to complete failed"));
     *plan_out = p;
     return NM_OK;
 }
