@@ -78,7 +78,7 @@ inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
 
 struct Layout {
     nm::TPlan t;
-    int32_t *order, *level_ptr, *slot_of, *meta;
+    int32_t *order, *level_ptr, *slot_of, *meta, *level_launch;
     Packed dir[2];
 };
 
@@ -95,6 +95,7 @@ size_t plan_layout(int64_t rows, int64_t nnz, void *base, Layout *L) {
     l.level_ptr = take(rows + 1);
     l.slot_of = take(rows + 1);
     l.meta = take(16);
+    l.level_launch = take(rows + 1);
     for (int d = 0; d < 2; ++d) {
         l.dir[d].dptr = take(rows + 1);
         l.dir[d].dslot = take(nnz + 1);
@@ -413,14 +414,38 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
 // which matters because the workgroup's wavefronts share one CU and the level time
 // is the time to issue their instructions.
 
+// Bit 30 of an entry marks a dependency the LDS ring of its launch cannot serve: the
+// row it refers to was solved by another launch, or too many slots ago.  Deciding that
+// here, once, keeps a dozen compare instructions per dependency out of every level.
+constexpr int32_t kEllFar = 1 << 30;
+
+__device__ __forceinline__ int32_t level_of_slot(const int32_t *__restrict__ level_ptr, int32_t nlevels, int32_t q) {
+    int32_t lo = 0, hi = nlevels;   // last l with level_ptr[l] <= q
+    while (hi - lo > 1) {
+        const int32_t mid = (lo + hi) >> 1;
+        if (level_ptr[mid] <= q) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict__ dptr,
-                                const int32_t *__restrict__ dslot, int32_t *__restrict__ ell_ds) {
+                                const int32_t *__restrict__ dslot, const int32_t *__restrict__ level_ptr,
+                                int32_t nlevels, const int32_t *__restrict__ level_launch,
+                                int32_t *__restrict__ ell_ds) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows * pre; i += stride) {
         const int64_t q = i / pre;
         const int e = (int)(i - q * pre);
         const int32_t lo = dptr[q], n = dptr[q + 1] - lo;
-        ell_ds[i] = e < n ? dslot[lo + e] : -1;
+        int32_t out = -1;
+        if (e < n) {
+            const int32_t ds = dslot[lo + e];
+            const int32_t dist = ds > (int32_t)q ? ds - (int32_t)q : (int32_t)q - ds;
+            const bool same = level_launch[level_of_slot(level_ptr, nlevels, (int32_t)q)] ==
+                              level_launch[level_of_slot(level_ptr, nlevels, ds)];
+            out = ds | ((same && dist < kRingSafe) ? 0 : kEllFar);
+        }
+        ell_ds[i] = out;
     }
 }
 
@@ -481,8 +506,7 @@ template <int PRE> __device__ __forceinline__ EllVals<PRE> load_ell(const EllArg
 }
 
 template <int PRE, int DEPTH>
-__global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step, int qlo,
-                                                             int qhi) {
+__global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step) {
     __shared__ double ring[kRing];
     __shared__ int32_t s_lp[kMaxLevels + 1];
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
@@ -506,21 +530,19 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
             bool in_ring = true;
 #pragma unroll
             for (int e = 0; e < PRE; ++e) {
-                const int32_t ds = cur.ds[e];
-                const int dist = ds > q ? ds - q : q - ds;
-                const bool hit = ds >= qlo && ds < qhi && dist < kRingSafe;
-                const double xj = ring[ds & (kRing - 1)];
-                if (cur.live && ds >= 0) {
-                    in_ring = in_ring && hit;
+                const int32_t raw = cur.ds[e];   // -1: no dependency; bit 30: not in this launch's ring
+                const double xj = ring[raw & (kRing - 1)];
+                if (cur.live && raw >= 0) {
+                    in_ring = in_ring && !(raw & kEllFar);
                     acc += cur.v[e] * xj;
                 }
             }
             if (!in_ring) {
-                // a dependency older than the ring: redo the sum in the same order from global memory
+                // a dependency the ring does not hold: redo the sum in the same order from global memory
                 acc = 0.;
 #pragma unroll
                 for (int e = 0; e < PRE; ++e)
-                    if (cur.ds[e] >= 0) acc += cur.v[e] * a.xs[cur.ds[e]];
+                    if (cur.ds[e] >= 0) acc += cur.v[e] * a.xs[cur.ds[e] & (kEllFar - 1)];
             }
             if (cur.live) {
                 double xi = cur.bv - acc;
@@ -600,11 +622,11 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
             // holds this direction's longest row (longer rows take the slow path)
             const int maxdep = p->max_deps[transposed ? 1 : 0];
             if (pre == 2)
-                hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
             else if (pre == 4)
-                hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
             else if (pre == 8)
-                hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step, L.q0, L.q1);
+                hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
             else if (maxdep <= 2)
                 hipLaunchKernelGGL((sptrsv_ring_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             else if (maxdep <= 4)
@@ -715,18 +737,6 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     p->nlevels = meta_h[0];
     p->max_deps[0] = meta_h[2];
     p->max_deps[1] = meta_h[3];
-    for (int d = 0; d < 2; ++d) {
-        const int32_t md = p->max_deps[d];
-        const int pre = md <= 2 ? 2 : (md <= 4 ? 4 : (md <= 8 ? 8 : 0));
-        if (pre > 0 && rows * pre <= ell_capacity(rows, nnz)) {
-            p->ell_pre[d] = pre;
-            int64_t grid = nm::ceil_div(rows * pre, kBlock);
-            if (grid > 65536) grid = 65536;
-            hipLaunchKernelGGL(ell_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, pre, p->dir[d].dptr,
-                               p->dir[d].dslot, p->dir[d].ell_ds);
-            if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
-        }
-    }
     std::vector<int32_t> lp((size_t)p->nlevels + 1);
     if (hipMemcpyAsync(lp.data(), p->level_ptr, lp.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess)
@@ -786,7 +796,27 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         p->launches.push_back({l, l + 1, lp[l], lp[l + 1], true, kBlock});
     }
     if (run0 >= 0) push_narrow(run0, p->nlevels);
-    if (hipStreamSynchronize(s) != hipSuccess)   // the fixed-width copies were enqueued after the read-back
+    // fixed-width copies of the packed triangles, with the ring-reach mark per dependency
+    std::vector<int32_t> level_launch((size_t)p->nlevels + 1, -1);
+    for (size_t li = 0; li < p->launches.size(); ++li)
+        for (int32_t l = p->launches[li].l0; l < p->launches[li].l1; ++l)
+            level_launch[l] = p->launches[li].wide ? -1 - (int32_t)li : (int32_t)li;
+    if (hipMemcpyAsync(L.level_launch, level_launch.data(), level_launch.size() * 4, hipMemcpyHostToDevice, s) !=
+        hipSuccess)
+        return bail(nm::fail(NM_ERR_HIP, "uploading the launch table failed"));
+    for (int d = 0; d < 2; ++d) {
+        const int32_t md = p->max_deps[d];
+        const int pre = md <= 2 ? 2 : (md <= 4 ? 4 : (md <= 8 ? 8 : 0));
+        if (pre > 0 && rows < kEllFar && rows * pre <= ell_capacity(rows, nnz)) {
+            p->ell_pre[d] = pre;
+            int64_t grid = nm::ceil_div(rows * pre, kBlock);
+            if (grid > 65536) grid = 65536;
+            hipLaunchKernelGGL(ell_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, pre, p->dir[d].dptr,
+                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, p->dir[d].ell_ds);
+            if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
+        }
+    }
+    if (hipStreamSynchronize(s) != hipSuccess)   // also keeps `level_launch` alive until its copy is done
         return bail(nm::fail(NM_ERR_HIP, "waiting for the plan to complete failed"));
     *plan_out = p;
     return NM_OK;
