@@ -69,7 +69,9 @@ __device__ __forceinline__ T row_times_dense(T acc, int64_t kb0, int64_t ke0, co
 // than kSplitRow is shared instead: every wavefront sums a contiguous eighth
 // of it and the partial sums are added in wavefront order (deterministic, but
 // not the serial order, so such rows match the CPU loop to rounding only).
-template <typename T, typename IDX, bool PERM>
+// LONG_ONLY: only rows longer than kSplitRow are computed (the flat kernel below
+// has done the others).
+template <typename T, typename IDX, bool PERM, bool LONG_ONLY = false>
 __global__ __launch_bounds__(kFwdBlock) void spdmm_fwd_kernel(
     int64_t rows, const T *__restrict__ data, const IDX *__restrict__ indices,
     const IDX *__restrict__ indptr, const int32_t *__restrict__ perm, const T *__restrict__ B, int64_t ldb,
@@ -85,7 +87,7 @@ __global__ __launch_bounds__(kFwdBlock) void spdmm_fwd_kernel(
             const int64_t c = c0 + lane;
             const bool live = c < n;
             const T *__restrict__ Bc = B + (live ? c : 0);
-            if (wave < nr) {
+            if (!LONG_ONLY && wave < nr) {
                 const int64_t row = r0 + wave;
                 const int64_t rb = indptr[row], re = indptr[row + 1];
                 if (re - rb <= kSplitRow) {
@@ -113,6 +115,135 @@ __global__ __launch_bounds__(kFwdBlock) void spdmm_fwd_kernel(
                 __syncthreads();
             }
         }
+    }
+}
+
+// Forward for rows of ordinary length, several rows per wavefront.  A wavefront owns
+// kFlatRows consecutive rows and walks their entries as one range: 64 entries per
+// coalesced load whatever the row lengths (a 15-entry row per load would leave 3/4 of
+// the lanes idle and cost a memory round trip per row), the next 64 requested while
+// the current ones are used, gathers of B eight at a time.  Lane = dense column; the
+// running sum is stored and restarted at every row boundary, so each row is still
+// added in storage order.  Rows longer than kSplitRow are skipped (their entries are
+// jumped over) and left to spdmm_fwd_kernel<..., LONG_ONLY>.
+constexpr int kFlatRows = 8;
+constexpr int kScoutRows = 64;   // rows a scout workgroup inspects for long ones
+
+template <typename T, typename IDX, bool PERM>
+__global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
+    int64_t rows, const T *__restrict__ data, const IDX *__restrict__ indices,
+    const IDX *__restrict__ indptr, const int32_t *__restrict__ perm, const T *__restrict__ B, int64_t ldb,
+    int64_t n, T *__restrict__ C, int64_t ldc) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    // The first `long_blocks` workgroups look for long rows, kScoutRows rows each, and
+    // share every one they find among their wavefronts (contiguous parts, partial sums added
+    // in wavefront order: deterministic, equal to the serial sum to rounding).  They come
+    // first in the grid so that this latency-bound work overlaps with the flat walk.
+    const int64_t long_blocks = (rows + kScoutRows - 1) / kScoutRows;
+    if ((int64_t)blockIdx.x < long_blocks) {
+        __shared__ T s_part[kWavesPerBlock][kWave];
+        __shared__ int s_long[kScoutRows];
+        __shared__ int s_nlong;
+        const int64_t g0 = (int64_t)blockIdx.x * kScoutRows;
+        if (threadIdx.x == 0) s_nlong = 0;
+        __syncthreads();
+        for (int t = threadIdx.x; t < kScoutRows && g0 + t < rows; t += kBlock)
+            if (indptr[g0 + t + 1] - indptr[g0 + t] > kSplitRow) s_long[atomicAdd(&s_nlong, 1)] = t;
+        __syncthreads();
+        const int nl = s_nlong;
+        for (int li = 0; li < nl; ++li) {   // uniform over the workgroup; the order of the list does not matter
+            const int64_t row = g0 + s_long[li];
+            const int64_t rb = indptr[row], re = indptr[row + 1];
+            int64_t chunk = (re - rb + kWavesPerBlock - 1) / kWavesPerBlock;
+            chunk = (chunk + kWave - 1) / kWave * kWave;
+            const int64_t kb = rb + wave * chunk;
+            const int64_t ke = kb + chunk < re ? kb + chunk : re;
+            for (int64_t c0 = 0; c0 < n; c0 += kWave) {
+                const int64_t c = c0 + lane;
+                const bool live = c < n;
+                T acc = T(0);
+                if (kb < re)
+                    acc = row_times_dense<T, IDX, PERM>(acc, kb, ke, data, indices, perm, B + (live ? c : 0), ldb, lane);
+                s_part[wave][lane] = acc;
+                __syncthreads();
+                if (wave == 0 && live) {
+                    T sum = s_part[0][lane];
+                    for (int w = 1; w < kWavesPerBlock; ++w) sum += s_part[w][lane];
+                    C[row * ldc + c] = sum;
+                }
+                __syncthreads();
+            }
+        }
+        return;
+    }
+    const int64_t r0 = (((int64_t)blockIdx.x - long_blocks) * kWavesPerBlock + wave) * kFlatRows;
+    if (r0 >= rows) return;
+    const int nr = (int)(rows - r0 < kFlatRows ? rows - r0 : kFlatRows);
+    // lane l holds indptr[r0 + l], l <= nr
+    const int64_t my_ptr = (int64_t)indptr[r0 + (lane <= nr ? lane : nr)];
+    auto ptr_of = [&](int l) {
+        const long long lo = __builtin_amdgcn_readlane((int)(my_ptr & 0xffffffffll), l);
+        const long long hi = __builtin_amdgcn_readlane((int)(my_ptr >> 32), l);
+        return (int64_t)((hi << 32) | (lo & 0xffffffffll));
+    };
+    const int64_t begin = ptr_of(0), end = ptr_of(nr);
+    for (int64_t c0 = 0; c0 < n; c0 += kWave) {
+        const int64_t c = c0 + lane;
+        const bool live = c < n;
+        const T *__restrict__ Bc = B + (live ? c : 0);
+        int r = 0;                         // current row (relative), its end, whether it is computed here
+        int64_t row_end = ptr_of(1);
+        bool mine = row_end - begin <= kSplitRow;
+        T acc = T(0);
+        auto next_row = [&]() {
+            if (mine && live) C[(r0 + r) * ldc + c] = acc;
+            acc = T(0);
+            ++r;
+            const int64_t rb = row_end;
+            row_end = ptr_of(r + 1 <= nr ? r + 1 : nr);
+            mine = row_end - rb <= kSplitRow;
+        };
+        int64_t kb = begin;
+        auto fetch = [&](int64_t at, int64_t &col, T &val) {
+            const int64_t k = at + lane < end ? at + lane : (end > begin ? end - 1 : 0);
+            col = end > begin ? (int64_t)indices[k] : 0;
+            val = end > begin ? (PERM ? data[perm[k]] : data[k]) : T(0);
+        };
+        int64_t mycol, nextcol;
+        T myval, nextval;
+        fetch(kb, mycol, myval);
+        while (kb < end) {
+            // a long row is not computed here: jump over what is left of it
+            while (r < nr && kb >= row_end) next_row();
+            if (!mine) {
+                kb = row_end;
+                if (kb >= end) break;
+                next_row();
+                fetch(kb, mycol, myval);
+                continue;
+            }
+            const int cnt = (int)(end - kb < kWave ? end - kb : kWave);
+            fetch(kb + kWave, nextcol, nextval);   // in flight while this chunk is used
+            for (int j0 = 0; j0 < cnt; j0 += kBatch) {
+                T bv[kBatch];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u)
+                    bv[u] = Bc[__shfl(mycol, j0 + u < cnt ? j0 + u : cnt - 1, kWave) * ldb];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    if (j0 + u >= cnt) break;
+                    const int64_t k = kb + j0 + u;
+                    while (k >= row_end) next_row();
+                    const T av = __shfl(myval, j0 + u, kWave);
+                    if (mine) acc += av * bv[u];
+                }
+            }
+            kb += cnt;
+            mycol = nextcol;
+            myval = nextval;
+        }
+        while (r < nr) next_row();   // the last row, and empty rows at the end
     }
 }
 
@@ -254,6 +385,12 @@ int check_args(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void 
     return NM_OK;
 }
 
+// workgroups of the flat forward kernel: the long-row scouts first, then the flat walkers
+inline unsigned flat_grid_for(int64_t rows) {
+    const int64_t g = nm::ceil_div(rows, kScoutRows) + nm::ceil_div(rows, (int64_t)kWavesPerBlock * kFlatRows);
+    return (unsigned)(g < 1 ? 1 : g);
+}
+
 inline unsigned wave_grid(int64_t units, int per_block) {
     int64_t grid = nm::ceil_div(units, per_block);
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
@@ -271,14 +408,14 @@ extern "C" int nm_spdmm_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t
     NM_REQUIRE(ldb >= n && ldc >= n, "row stride smaller than the row (ldb=%lld ldc=%lld n=%lld)",
                (long long)ldb, (long long)ldc, (long long)n);
     hipStream_t s = nm::as_stream(stream);
+    const unsigned flat_grid = flat_grid_for(rows);
     if (dt == NM_F32)
-        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int64_t, false>), dim3(wave_grid(rows, kFwdWaves)), dim3(kFwdBlock), 0, s,
-                           rows, (const float *)data, indices, indptr, nullptr, (const float *)B, ldb, n,
-                           (float *)C, ldc);
+        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<float, int64_t, false>), dim3(flat_grid), dim3(kBlock), 0, s, rows,
+                           (const float *)data, indices, indptr, nullptr, (const float *)B, ldb, n, (float *)C, ldc);
     else
-        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int64_t, false>), dim3(wave_grid(rows, kFwdWaves)), dim3(kFwdBlock), 0, s,
-                           rows, (const double *)data, indices, indptr, nullptr, (const double *)B, ldb, n,
-                           (double *)C, ldc);
+        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<double, int64_t, false>), dim3(flat_grid), dim3(kBlock), 0, s, rows,
+                           (const double *)data, indices, indptr, nullptr, (const double *)B, ldb, n, (double *)C,
+                           ldc);
     NM_LAUNCH_CHECK("spdmm_fwd_kernel");
     return NM_OK;
 }
@@ -350,14 +487,14 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
     NM_REQUIRE(ldgb >= n && ldg >= n, "row stride smaller than the row");
     NM_REQUIRE(gC != nullptr || nnz == 0, "gC is null");
     hipStream_t s = nm::as_stream(stream);
+    const unsigned flat_grid = flat_grid_for(cols);
     if (dt == NM_F32)
-        hipLaunchKernelGGL((spdmm_fwd_kernel<float, int32_t, true>), dim3(wave_grid(cols, kFwdWaves)),
-                           dim3(kFwdBlock), 0, s, cols,
+        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<float, int32_t, true>), dim3(flat_grid), dim3(kBlock), 0, s, cols,
                            (const float *)data, t.t_row, t.t_indptr, t.t_perm, (const float *)gC, ldg, n,
                            (float *)grad_B, ldgb);
     else
-        hipLaunchKernelGGL((spdmm_fwd_kernel<double, int32_t, true>), dim3(wave_grid(cols, kFwdWaves)),
-                           dim3(kFwdBlock), 0, s, cols, (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg, n,
+        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<double, int32_t, true>), dim3(flat_grid), dim3(kBlock), 0, s, cols,
+                           (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg, n,
                            (double *)grad_B, ldgb);
     NM_LAUNCH_CHECK("spdmm_fwd_kernel (transposed)");
     return NM_OK;
