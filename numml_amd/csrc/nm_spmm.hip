@@ -1,11 +1,14 @@
 // CSR x dense (SpMM) forward and backward for gfx950.
 //
-// Forward: one wavefront per row of A, lane = output column (a 64-column fp32
-// row of B is one 256-byte line, so every gather is a single coalesced
-// request).  The wavefront reads 64 (column, value) pairs of the row with one
-// coalesced load each and broadcasts them lane by lane; every lane adds its
-// column's terms in storage order, the order of the serial CPU loop
-// (cpp/sparse_csr_cpu.cpp:586-598), so C matches it bit for bit.
+// Forward: lane = output column (a 64-column fp32 row of B is one 256-byte
+// line, so every gather is a single coalesced request).  A wavefront owns a few
+// consecutive rows of A and walks their entries as one range, 64 (column,
+// value) pairs per coalesced load, broadcasting them lane by lane; every lane
+// adds its column's terms in storage order and restarts at row boundaries --
+// the order of the serial CPU loop (cpp/sparse_csr_cpu.cpp:586-598), so C
+// matches it bit for bit.  Rows longer than kSplitRow are shared by the
+// wavefronts of a workgroup instead (partial sums added in wavefront order:
+// deterministic, equal to rounding).
 //
 // Backward: the same mapping computes, per stored entry, the dot product of
 // gC[row,:] and B[col,:] (cross-lane reduction) and scatters
@@ -23,8 +26,6 @@ using nm::kWave;
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 
-constexpr int kFwdWaves = 8;                 // wavefronts (= rows) per forward workgroup
-constexpr int kFwdBlock = kFwdWaves * kWave;
 constexpr int kBatch = 8;                    // gathers a wavefront keeps in flight in the backward
 constexpr int kSplitRow = 512;               // rows longer than this are shared by the workgroup's wavefronts
 
@@ -64,68 +65,15 @@ __device__ __forceinline__ T row_times_dense(T acc, int64_t kb0, int64_t ke0, co
     return acc;
 }
 
-// C = A B (or, on the plan, A^T B).  A workgroup of eight wavefronts owns eight
-// consecutive rows: one wavefront per row, lane = dense column.  A row longer
-// than kSplitRow is shared instead: every wavefront sums a contiguous eighth
-// of it and the partial sums are added in wavefront order (deterministic, but
-// not the serial order, so such rows match the CPU loop to rounding only).
-// LONG_ONLY: only rows longer than kSplitRow are computed (the flat kernel below
-// has done the others).
-template <typename T, typename IDX, bool PERM, bool LONG_ONLY = false>
-__global__ __launch_bounds__(kFwdBlock) void spdmm_fwd_kernel(
-    int64_t rows, const T *__restrict__ data, const IDX *__restrict__ indices,
-    const IDX *__restrict__ indptr, const int32_t *__restrict__ perm, const T *__restrict__ B, int64_t ldb,
-    int64_t n, T *__restrict__ C, int64_t ldc) {
-    __shared__ T s_part[kFwdWaves][kWave];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
-    const int64_t nblk = (rows + kFwdWaves - 1) / kFwdWaves;
-    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
-        const int64_t r0 = blk * kFwdWaves;
-        const int nr = (int)(rows - r0 < kFwdWaves ? rows - r0 : kFwdWaves);
-        for (int64_t c0 = 0; c0 < n; c0 += kWave) {
-            const int64_t c = c0 + lane;
-            const bool live = c < n;
-            const T *__restrict__ Bc = B + (live ? c : 0);
-            if (!LONG_ONLY && wave < nr) {
-                const int64_t row = r0 + wave;
-                const int64_t rb = indptr[row], re = indptr[row + 1];
-                if (re - rb <= kSplitRow) {
-                    const T acc = row_times_dense<T, IDX, PERM>(T(0), rb, re, data, indices, perm, Bc, ldb, lane);
-                    if (live) C[row * ldc + c] = acc;
-                }
-            }
-            for (int t = 0; t < nr; ++t) {   // shared long rows (uniform over the workgroup)
-                const int64_t row = r0 + t;
-                const int64_t rb = indptr[row], re = indptr[row + 1];
-                if (re - rb <= kSplitRow) continue;
-                int64_t chunk = (re - rb + kFwdWaves - 1) / kFwdWaves;
-                chunk = (chunk + kWave - 1) / kWave * kWave;
-                const int64_t kb = rb + wave * chunk;
-                const int64_t ke = kb + chunk < re ? kb + chunk : re;
-                T acc = T(0);
-                if (kb < re) acc = row_times_dense<T, IDX, PERM>(acc, kb, ke, data, indices, perm, Bc, ldb, lane);
-                s_part[wave][lane] = acc;
-                __syncthreads();
-                if (wave == 0) {
-                    T sum = s_part[0][lane];
-                    for (int w = 1; w < kFwdWaves; ++w) sum += s_part[w][lane];
-                    if (live) C[row * ldc + c] = sum;
-                }
-                __syncthreads();
-            }
-        }
-    }
-}
-
-// Forward for rows of ordinary length, several rows per wavefront.  A wavefront owns
+// C = A B (or, on the plan, A^T B).  A wavefront of a "walker" workgroup owns
 // kFlatRows consecutive rows and walks their entries as one range: 64 entries per
 // coalesced load whatever the row lengths (a 15-entry row per load would leave 3/4 of
 // the lanes idle and cost a memory round trip per row), the next 64 requested while
 // the current ones are used, gathers of B eight at a time.  Lane = dense column; the
 // running sum is stored and restarted at every row boundary, so each row is still
-// added in storage order.  Rows longer than kSplitRow are skipped (their entries are
-// jumped over) and left to spdmm_fwd_kernel<..., LONG_ONLY>.
+// added in storage order.  Rows longer than kSplitRow are skipped by the walkers
+// (their entries are jumped over) and computed by the "scout" workgroups at the head
+// of the grid.
 constexpr int kFlatRows = 8;
 constexpr int kScoutRows = 64;   // rows a scout workgroup inspects for long ones
 
