@@ -256,6 +256,41 @@ def csr_extract_diagonal_backward(g, rows, cols, data, indices, indptr):
     return grad_A
 
 
+def splu(rows, cols, data, indices, indptr):
+    """splu_cpu, cpp/sparse_csr_cpu.cpp:777-1016 -> (M_data, M_indices, M_indptr, Mt_data, Mt_indices,
+    Mt_indptr): L + U without pivoting on the filled pattern (unit diagonal of L not stored) and its
+    transpose.  The matrix must be square with a stored diagonal."""
+    data, indices, indptr = _vals(data), _idx(indices), _idx(indptr)
+    assert rows == cols
+    stamp, queue = np.zeros(rows, np.int64), np.zeros(rows + 1, np.int64)
+    keep = np.zeros(cols + 1, np.uint8)
+    As_indptr = np.zeros(rows + 1, np.int64)
+    _fn("or_splu_symbolic", data.dtype)(_i64(rows), _i64(cols), _p(indices), _p(indptr), _p(As_indptr), _p(stamp),
+                                        _p(queue), _p(keep))
+    nnz = int(As_indptr[rows])
+    As_indices, As_data = np.empty(nnz, np.int64), np.empty(nnz, data.dtype)
+    Mt_indptr, Mt_indices, Mt_data = np.empty(cols + 1, np.int64), np.empty(nnz, np.int64), np.empty(nnz, data.dtype)
+    perm, cursor = np.empty(nnz, np.int64), np.empty(max(rows, cols, 1), np.int64)
+    _fn("or_splu_numeric", data.dtype)(_i64(rows), _i64(cols), _p(data), _p(indices), _p(indptr), _p(As_indptr),
+                                       _p(As_indices), _p(As_data), _p(Mt_indptr), _p(Mt_indices), _p(Mt_data),
+                                       _p(perm), _p(stamp), _p(queue), _p(keep), _p(cursor))
+    M_data, M_indices, M_indptr, _ = csr_transpose(cols, rows, Mt_data, Mt_indices, Mt_indptr)
+    return M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr
+
+
+def spsolve_backward(grad_x, x, rows, cols, Mt_data, Mt_indices, Mt_indptr, A_data, A_indices, A_indptr):
+    """spsolve_backward_cpu, cpp/sparse_csr_cpu.cpp:1018-1048 -> (grad_A, grad_b):
+    grad_b = A^-T grad_x by two solves with M^T (lower, stored diagonal; then upper, unit), and
+    grad_A[k] = -(grad_b[row] * x[col])."""
+    y = sptrsv_forward(rows, cols, Mt_data, Mt_indices, Mt_indptr, True, False, grad_x)
+    grad_b = sptrsv_forward(rows, cols, Mt_data, Mt_indices, Mt_indptr, False, True, y)
+    A_indices, A_indptr = _idx(A_indices), _idx(A_indptr)
+    r = np.repeat(np.arange(rows), np.diff(A_indptr))
+    x = np.asarray(x)
+    grad_A = (-(grad_b[r] * x[A_indices])).astype(np.asarray(A_data).dtype)
+    return grad_A, grad_b
+
+
 def sptrsv_forward(rows, cols, data, indices, indptr, lower, unit, b):
     """sptrsv_forward_cpu, cpp/sparse_csr_cpu.cpp:652-723."""
     data, indices, indptr = _vals(data), _idx(indices), _idx(indptr)

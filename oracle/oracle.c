@@ -12,6 +12,7 @@
  *   or_sptrsv_forward/backward   :652-759
  *   or_splincomb_forward/backward_one :387-560
  *   or_row_sum, or_diagonal(_backward) :1106-1213
+ *   or_splu_symbolic/numeric     :777-1016 (fill2 symbolic phase + left-looking numeric phase)
  * (csr_to_dense_forward/backward, :1050-1104, and csr_transpose_backward,
  * :369-385, are plain index assignments and are restated with NumPy indexing in
  * oracle/__init__.py.)

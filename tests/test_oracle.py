@@ -355,3 +355,57 @@ def test_math_lincomb_and_reductions(dtype):
     sd, si, sp_, _ = G.random_csr(9, 9, 0.3, 1, dtype)       # some rows without a stored diagonal
     assert np.array_equal(oracle.csr_extract_diagonal_forward(9, 9, sd, si, sp_),
                           sp.csr_matrix((sd, si, sp_), shape=(9, 9)).diagonal())
+
+
+# ------------------------------------------------------------------ sparse LU
+
+def _lu_cases(dtype):
+    yield "tridiag", G.tridiag(12, dtype)
+    yield "poisson6", G.poisson2d(6, dtype, 1)
+    rng = np.random.default_rng(5)
+    n = 40
+    m = sp.random(n, n, 0.08, random_state=3, format="csr", dtype=np.float64) + sp.eye(n) * 4.0
+    m = m.tocsr()
+    m.sort_indices()
+    yield "random_diag_dominant", (m.data.astype(dtype), m.indices.astype(np.int64), m.indptr.astype(np.int64), (n, n))
+    a = sp.random(25, 25, 0.1, random_state=7, format="csr", dtype=np.float64)
+    a = (a + a.T + sp.eye(25) * 6.0).tocsr()
+    a.sort_indices()
+    yield "symmetric_pattern", (a.data.astype(dtype), a.indices.astype(np.int64), a.indptr.astype(np.int64), (25, 25))
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_ref_splu_and_spsolve_backward(dtype):
+    for name, (d, i, p, (n, _)) in _lu_cases(dtype):
+        mine = oracle.splu(n, n, d, i, p)
+        theirs = ref.call("splu", n, n, d, i, p)
+        for a, b, what in zip(mine, theirs, ("M_data", "M_indices", "M_indptr", "Mt_data", "Mt_indices", "Mt_indptr")):
+            same(a, b, f"{name} splu {what}")
+        rng = np.random.default_rng(1)
+        gx, x = rng.standard_normal(n).astype(dtype), rng.standard_normal(n).astype(dtype)
+        for a, b in zip(oracle.spsolve_backward(gx, x, n, n, mine[3], mine[4], mine[5], d, i, p),
+                        ref.call("spsolve_backward", gx, x, n, n, mine[3], mine[4], mine[5], d, i, p)):
+            same(a, b, f"{name} spsolve_backward")
+
+
+def test_math_splu_factors_reproduce_the_matrix():
+    for name, (d, i, p, (n, _)) in _lu_cases(np.float64):
+        Md, Mi, Mp, Td, Ti, Tp = oracle.splu(n, n, d, i, p)
+        M = sp.csr_matrix((Md, Mi, Mp), shape=(n, n)).toarray()
+        L, U = np.tril(M, -1) + np.eye(n), np.triu(M)
+        A = sp.csr_matrix((d, i, p), shape=(n, n)).toarray()
+        assert np.allclose(L @ U, A, atol=1e-10), name
+        assert np.array_equal(sp.csr_matrix((Td, Ti, Tp), shape=(n, n)).toarray(), M.T), name
+        # the filled pattern contains A's and is what symbolic elimination of the pattern gives
+        pat = (A != 0)
+        for k in range(n):
+            rows_k = np.nonzero(pat[k + 1:, k])[0] + k + 1
+            cols_k = np.nonzero(pat[k, k + 1:])[0] + k + 1
+            pat[np.ix_(rows_k, cols_k)] = True
+        assert np.array_equal(sp.csr_matrix((np.ones_like(Md), Mi, Mp), shape=(n, n)).toarray() != 0, pat), name
+        # a solve through the factors
+        b = np.random.default_rng(2).standard_normal(n)
+        y = oracle.sptrsv_forward(n, n, Md, Mi, Mp, True, True, b)
+        x = oracle.sptrsv_forward(n, n, Md, Mi, Mp, False, False, y)
+        assert np.allclose(A @ x, b, atol=1e-9), name
