@@ -224,6 +224,34 @@ int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz,
                     double alpha, const void *a, const void *b, void *out,
                     nm_stream stream);
 
+/* ------------------------------------------------------------ sparse LU
+ * M = L + U of a square matrix with a stored diagonal, without pivoting, on the
+ * filled pattern (the unit diagonal of L is not stored); replaces splu_cpu /
+ * splu_cuda (cpp/sparse_csr.hpp:107-111, cpp/sparse_csr_cpu.cpp:777-1016).
+ * Pattern and factors equal the reference's CPU result bit for bit.
+ *
+ *   nm_splu_symbolic_bytes  scratch for the two pattern passes
+ *   nm_splu_symbolic        As_indptr[rows + 1] of the filled pattern (the
+ *                           caller reads As_indptr[rows] to size the next call)
+ *   nm_splu_fill            As_indices (ascending per row) and As_data: A's
+ *                           value where A stores the column, 0 at the fill
+ *   nm_splu_numeric         in-place factorisation of the TRANSPOSE of that
+ *                           matrix (rows of Mt = columns of M), ordered by the
+ *                           levels of an nm_sptrsv_analyse plan of Mt's pattern
+ *                           taken as a lower-triangular solve
+ * The caller transposes As -> Mt before, and Mt -> M after, the numeric phase. */
+int nm_splu_symbolic_bytes(int64_t rows, size_t *bytes);
+int nm_splu_symbolic(int64_t rows, const int64_t *A_indices,
+                     const int64_t *A_indptr, int64_t *As_indptr,
+                     void *workspace, size_t workspace_bytes, nm_stream stream);
+int nm_splu_fill(nm_dtype dt, int64_t rows, const void *A_data,
+                 const int64_t *A_indices, const int64_t *A_indptr,
+                 const int64_t *As_indptr, int64_t *As_indices, void *As_data,
+                 void *workspace, size_t workspace_bytes, nm_stream stream);
+int nm_splu_numeric(const nm_sptrsv_plan *plan, nm_dtype dt, void *Mt_data,
+                    const int64_t *Mt_indices, const int64_t *Mt_indptr,
+                    nm_stream stream);
+
 /* ------------------------------------------------- linear combination
  * C = alpha A + beta B for two matrices of one shape; a column stored by either
  * operand is stored by C (also when the sum is 0), columns ascending.  Stands in

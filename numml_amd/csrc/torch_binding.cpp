@@ -610,6 +610,89 @@ std::vector<Tensor> sptrsv_backward(Tensor grad_x, Tensor x, int A_rows, int A_c
 
 // (dependency levels, kernel launches per solve) of the cached or newly built level
 // schedule of a triangular pattern; no counterpart in the reference (diagnostics).
+// ------------------------------------------------------------------------ sparse LU
+
+// [M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]  (cpp/sparse_csr.hpp:107-111)
+std::vector<Tensor> splu(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    const auto dev = need_device({&A_data, &A_indices, &A_indptr});
+    TORCH_CHECK(A_rows == A_cols, "Expected square matrix for LU factorization, got ", A_rows, " x ", A_cols, ".");
+    A_data = A_data.contiguous();
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    const int64_t rows = A_rows;
+    const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
+    const nm_stream stream = current_stream(dev);
+
+    // pattern with fill: count, then write
+    size_t bytes = 0;
+    check(nm_splu_symbolic_bytes(rows, &bytes), "nm_splu_symbolic_bytes");
+    Tensor work = scratch(bytes, dev);
+    Tensor M_indptr = torch::empty({rows + 1}, iopt);
+    check(nm_splu_symbolic(rows, A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                           M_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, stream),
+          "nm_splu_symbolic");
+    const int64_t nnz = M_indptr[rows].item<int64_t>();
+    Tensor M_indices = torch::empty({nnz}, iopt);
+    Tensor As_data = torch::empty({nnz}, A_data.options());
+    check(nm_splu_fill(dtype_of(A_data), rows, A_data.data_ptr(), A_indices.data_ptr<int64_t>(),
+                       A_indptr.data_ptr<int64_t>(), M_indptr.data_ptr<int64_t>(), M_indices.data_ptr<int64_t>(),
+                       As_data.data_ptr(), work.data_ptr(), bytes, stream),
+          "nm_splu_fill");
+
+    // the factorisation runs by column: on the rows of the transpose
+    auto tplan = transpose_plan(M_indices, M_indptr, rows, rows, dev);
+    Tensor Mt_data = torch::empty_like(As_data);
+    Tensor Mt_indices = torch::empty({nnz}, iopt);
+    Tensor Mt_indptr = torch::empty({rows + 1}, iopt);
+    Tensor Mt_to_M = torch::empty({nnz}, iopt);
+    check(nm_csr_transpose_forward(dtype_of(A_data), rows, rows, nnz, As_data.data_ptr(), tplan->mem.data_ptr(),
+                                   Mt_data.data_ptr(), Mt_indices.data_ptr<int64_t>(),
+                                   Mt_indptr.data_ptr<int64_t>(), Mt_to_M.data_ptr<int64_t>(), stream),
+          "nm_csr_transpose_forward");
+    auto levels = level_plan(Mt_indices, Mt_indptr, rows, true, dev);
+    check(nm_splu_numeric(levels->handle, dtype_of(A_data), Mt_data.data_ptr(), Mt_indices.data_ptr<int64_t>(),
+                          Mt_indptr.data_ptr<int64_t>(), stream),
+          "nm_splu_numeric");
+    Tensor M_data = torch::empty_like(Mt_data);
+    check(nm_csr_transpose_backward(dtype_of(A_data), nnz, Mt_data.data_ptr(), Mt_to_M.data_ptr<int64_t>(),
+                                    M_data.data_ptr(), stream),
+          "nm_csr_transpose_backward");
+    return {M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr};
+}
+
+// [grad_A, grad_b]  (cpp/sparse_csr.hpp:113-118, cpp/sparse_csr_cpu.cpp:1018-1048): grad_b = A^-T grad_x
+// by two solves with M^T, grad_A = -(grad_b x^T) on A's pattern.
+std::vector<Tensor> spsolve_backward(Tensor grad_x, Tensor x, int A_rows, int A_cols, Tensor Mt_data,
+                                     Tensor Mt_indices, Tensor Mt_indptr, Tensor A_data, Tensor A_indices,
+                                     Tensor A_indptr) {
+    const auto dev = need_device({&grad_x, &x, &Mt_data, &Mt_indices, &Mt_indptr, &A_data, &A_indices, &A_indptr});
+    same_dtype(A_data, grad_x, "grad_x");
+    same_dtype(A_data, x, "x");
+    same_dtype(A_data, Mt_data, "Mt_data");
+    Mt_data = Mt_data.contiguous();
+    A_data = A_data.contiguous();
+    grad_x = grad_x.contiguous();
+    x = x.contiguous();
+    Mt_indices = index_tensor(Mt_indices, "Mt_indices");
+    Mt_indptr = index_tensor(Mt_indptr, "Mt_indptr");
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    auto lower = level_plan(Mt_indices, Mt_indptr, A_rows, true, dev);
+    Tensor y = solve(*lower, false, Mt_data, false, grad_x, A_rows, dev);
+    auto upper = level_plan(Mt_indices, Mt_indptr, A_rows, false, dev);
+    Tensor grad_b = solve(*upper, false, Mt_data, true, y, A_rows, dev);
+    Tensor grad_A = torch::empty_like(A_data);
+    check(nm_masked_outer(dtype_of(A_data), A_rows, A_data.numel(), A_indices.data_ptr<int64_t>(),
+                          A_indptr.data_ptr<int64_t>(), -1.0, grad_b.data_ptr(), x.data_ptr(), grad_A.data_ptr(),
+                          current_stream(dev)),
+          "nm_masked_outer");
+    return {grad_A, grad_b};
+}
+
+// ------------------------------------------------------------------------ diagnostics
+
 std::tuple<int64_t, int64_t> sptrsv_schedule(int A_rows, Tensor A_indices, Tensor A_indptr, bool lower) {
     const auto dev = need_device({&A_indices, &A_indptr});
     A_indices = index_tensor(A_indices, "A_indices");
@@ -649,6 +732,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("spdmm_backward", &spdmm_backward, "Sparse times dense matrix backward");
     m.def("sptrsv_forward", &sptrsv_forward, "Sparse triangular solve forward");
     m.def("sptrsv_backward", &sptrsv_backward, "Sparse triangular solve backward");
+    m.def("splu", &splu, "Sparse LU decomposition");
+    m.def("spsolve_backward", &spsolve_backward, "Sparse LU solve backward");
     m.def("csr_transpose_forward", &csr_transpose_forward, "CSR Transpose forward");
     m.def("csr_transpose_backward", &csr_transpose_backward, "CSR Transpose backward");
     m.def("splincomb_forward", &splincomb_forward, "Sparse linear combination forward");

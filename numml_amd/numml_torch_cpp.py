@@ -495,6 +495,61 @@ def _plan_for(indices, indptr, rows, lower, dev):
                    lambda: _Plan(indices, indptr, rows, lower, dev))
 
 
+def splu(A_rows, A_cols, A_data, A_indices, A_indptr):
+    """[M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]: L + U without pivoting on the
+    filled pattern, and its transpose  (cpp/sparse_csr.hpp:107-111)."""
+    dev = _need_device(A_data, A_indices, A_indptr)
+    if A_rows != A_cols:
+        raise RuntimeError(f"Expected square matrix for LU factorization, got {A_rows} x {A_cols}.")
+    A_data = A_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    L = _lib.lib()
+    rows = A_rows
+    with torch.cuda.device(dev):
+        stream = _stream(dev)
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(L.nm_splu_symbolic_bytes(rows, ctypes.byref(nbytes)), "nm_splu_symbolic_bytes")
+        work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+        M_indptr = torch.empty(rows + 1, dtype=torch.int64, device=dev)
+        _lib.check(L.nm_splu_symbolic(rows, _ptr(A_indices), _ptr(A_indptr), _ptr(M_indptr), _ptr(work),
+                                      nbytes.value, stream), "nm_splu_symbolic")
+        nnz = int(M_indptr[rows].item())
+        M_indices = torch.empty(nnz, dtype=torch.int64, device=dev)
+        As_data = torch.empty(nnz, dtype=A_data.dtype, device=dev)
+        _lib.check(L.nm_splu_fill(_dt(A_data), rows, _ptr(A_data), _ptr(A_indices), _ptr(A_indptr),
+                                  _ptr(M_indptr), _ptr(M_indices), _ptr(As_data), _ptr(work), nbytes.value,
+                                  stream), "nm_splu_fill")
+        # the factorisation runs by column: on the rows of the transpose
+        Mt_data, Mt_indices, Mt_indptr, Mt_to_M = csr_transpose_forward(rows, rows, As_data, M_indices, M_indptr)
+        plan = _plan_for(Mt_indices, Mt_indptr, rows, True, dev)
+        _lib.check(L.nm_splu_numeric(plan.handle, _dt(A_data), _ptr(Mt_data), _ptr(Mt_indices), _ptr(Mt_indptr),
+                                     stream), "nm_splu_numeric")
+        M_data = csr_transpose_backward(Mt_data, Mt_to_M)
+    return [M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]
+
+
+def spsolve_backward(grad_x, x, A_rows, A_cols, Mt_data, Mt_indices, Mt_indptr, A_data, A_indices, A_indptr):
+    """[grad_A, grad_b]: grad_b = A^-T grad_x by two solves with M^T, grad_A = -(grad_b x^T) on A's
+    pattern  (cpp/sparse_csr.hpp:113-118, cpp/sparse_csr_cpu.cpp:1018-1048)."""
+    dev = _need_device(grad_x, x, Mt_data, Mt_indices, Mt_indptr, A_data, A_indices, A_indptr)
+    _same_dtype(A_data, grad_x, "grad_x")
+    _same_dtype(A_data, x, "x")
+    _same_dtype(A_data, Mt_data, "Mt_data")
+    Mt_data, A_data, grad_x, x = Mt_data.contiguous(), A_data.contiguous(), grad_x.contiguous(), x.contiguous()
+    Mt_indices, Mt_indptr = _idx(Mt_indices, "Mt_indices"), _idx(Mt_indptr, "Mt_indptr")
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        lower = _plan_for(Mt_indices, Mt_indptr, A_rows, True, dev)
+        y = _solve(lower, False, Mt_data, Mt_indices, Mt_indptr, False, grad_x, A_rows, dev)
+        upper = _plan_for(Mt_indices, Mt_indptr, A_rows, False, dev)
+        grad_b = _solve(upper, False, Mt_data, Mt_indices, Mt_indptr, True, y, A_rows, dev)
+        grad_A = torch.empty_like(A_data)
+        _lib.check(_lib.lib().nm_masked_outer(
+            _dt(A_data), A_rows, A_data.shape[0], _ptr(A_indices), _ptr(A_indptr), -1.0,
+            _ptr(grad_b), _ptr(x), _ptr(grad_A), _stream(dev)), "nm_masked_outer")
+    return [grad_A, grad_b]
+
+
 def sptrsv_schedule(A_rows, A_indices, A_indptr, lower):
     """(dependency levels, kernel launches per solve) of the level schedule of a
     triangular pattern, built or taken from the cache; diagnostics, no counterpart

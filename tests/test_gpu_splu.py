@@ -1,0 +1,135 @@
+"""Sparse LU without pivoting and the direct solve on top of it (splu, spsolve_backward and
+the ``linalg.splu / splu_solve / spsolve`` surface) on a HIP device.
+
+The pattern with fill is integer work and the factors are computed in the reference's
+operation order, so both are compared bit for bit with the CPU oracle
+(cpp/sparse_csr_cpu.cpp:777-1016).  The solves go through the triangular solve, which
+accumulates in double: fp32 1e-5 / fp64 1e-12 relative, as for that solve.
+"""
+import numpy as np
+import pytest
+import scipy.sparse as sps
+import scipy.sparse.linalg as spla
+import torch
+
+import numml_amd
+import oracle
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as mirror
+from numml_amd import sparse as sp
+from numml_amd.sparse import linalg
+from util import assert_close, assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("M_data", "M_indices", "M_indptr", "Mt_data", "Mt_indices", "Mt_indptr")
+
+
+def _from_scipy(m, dtype):
+    m = m.tocsr()
+    m.sort_indices()
+    return m.data.astype(dtype), m.indices.astype(np.int64), m.indptr.astype(np.int64), m.shape
+
+
+def _cases(dtype):
+    yield "one", (np.full(1, 3, dtype), np.zeros(1, np.int64), np.array([0, 1], np.int64), (1, 1))
+    yield "diagonal", _from_scipy(sps.diags(np.arange(1, 8, dtype=np.float64)), dtype)
+    yield "tridiag12", G.tridiag(12, dtype)
+    yield "tridiag700", G.tridiag(700, dtype)
+    yield "poisson6", G.poisson2d(6, dtype, 1)
+    yield "poisson24", G.poisson2d(24, dtype, 1)
+    yield "random40", _from_scipy(sps.random(40, 40, 0.08, random_state=3, dtype=np.float64) + sps.eye(40) * 4.0, dtype)
+    a = sps.random(25, 25, 0.1, random_state=7, dtype=np.float64)
+    yield "symmetric25", _from_scipy(a + a.T + sps.eye(25) * 6.0, dtype)
+    # unsymmetric pattern, rows longer than a wavefront, an arrow that fills the matrix
+    b = sps.random(300, 300, 0.02, random_state=11, dtype=np.float64) + sps.eye(300) * 9.0
+    yield "random300", _from_scipy(b, dtype)
+    arrow = sps.lil_matrix((90, 90))
+    arrow.setdiag(5.0)
+    arrow[0, :] = 1.0
+    arrow[:, 0] = 1.0
+    arrow[0, 0] = 90.0
+    yield "arrow90", _from_scipy(arrow, dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("binding", ["compiled", "ctypes"])
+def test_splu_matches_the_oracle_bit_for_bit(dev, dtype, binding):
+    ext = numml_amd.load_compiled() if binding == "compiled" else mirror
+    for name, (d, i, p, (n, _)) in _cases(dtype):
+        print("case", name, dtype.__name__, binding, flush=True)
+        out = ext.splu(n, n, *to_dev(dev, d, i, p))
+        want = oracle.splu(n, n, d, i, p)
+        for got, ref, what in zip(out, want, NAMES):
+            assert_same(host(got), ref, f"{name} {what}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_spsolve_backward_matches_the_oracle(dev, dtype):
+    ext = numml_amd.load_compiled()
+    for name, (d, i, p, (n, _)) in _cases(dtype):
+        print("case", name, dtype.__name__, flush=True)
+        M = oracle.splu(n, n, d, i, p)
+        gx, x = randn(1, n, dtype), randn(2, n, dtype)
+        want = oracle.spsolve_backward(gx, x, n, n, M[3], M[4], M[5], d, i, p)
+        got = ext.spsolve_backward(*to_dev(dev, gx, x), n, n, *to_dev(dev, M[3], M[4], M[5], d, i, p))
+        assert_close(host(got[1]), want[1], f"{name} grad_b")
+        assert_close(host(got[0]), want[0], f"{name} grad_A")
+
+
+def test_poisson_factors_reproduce_the_matrix_and_solve(dev):
+    # 64 x 64 grid in natural ordering: the band fills (about half a million entries)
+    d, i, p, (n, _) = G.poisson2d(64, np.float64, 1)
+    A = sp.SparseCSRTensor(tuple(to_dev(dev, d, i, p)), (n, n))
+    LU = linalg.splu(A)
+    want = oracle.splu(n, n, d, i, p)
+    assert_same(host(LU.indptr), want[2], "M_indptr")
+    assert_same(host(LU.indices), want[1], "M_indices")
+    assert_same(host(LU.data), want[0], "M_data")
+    M = sps.csr_matrix((host(LU.data), host(LU.indices), host(LU.indptr)), shape=(n, n))
+    Lf = sps.tril(M, -1) + sps.eye(n)
+    Uf = sps.triu(M)
+    As = sps.csr_matrix((d, i, p), shape=(n, n))
+    assert abs(Lf @ Uf - As).max() < 1e-11
+    b = randn(3, n, np.float64)
+    x = linalg.splu_solve(LU, to_dev(dev, b)[0])
+    xs = spla.spsolve(As.tocsc(), b)
+    assert np.allclose(host(x), xs, rtol=1e-9, atol=1e-9 * np.abs(xs).max())
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_spsolve_gradients_against_dense_autograd(dev, dtype):
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    tol = 2e-4 if dtype == np.float32 else 1e-10
+    for name, (d, i, p, (n, _)) in _cases(dtype):
+        if name in ("tridiag700",):
+            continue
+        D, I, P = to_dev(dev, d, i, p)
+        A = sp.SparseCSRTensor((D.clone(), I, P), (n, n))
+        A.requires_grad = True
+        b = to_dev(dev, randn(4, n, dtype))[0].requires_grad_(True)
+        w = to_dev(dev, randn(5, n, dtype))[0]
+        x = linalg.spsolve(A, b)
+        (x * w).sum().backward()
+        # dense check in double on the host
+        Ad = torch.tensor(sps.csr_matrix((d, i, p), shape=(n, n)).toarray(), dtype=torch.float64, requires_grad=True)
+        bd = torch.tensor(host(b.detach()), dtype=torch.float64, requires_grad=True)
+        xd = torch.linalg.solve(Ad, bd)
+        (xd * torch.tensor(host(w), dtype=torch.float64)).sum().backward()
+        scale = float(xd.detach().abs().max())
+        assert np.allclose(host(x.detach()), xd.detach().numpy(), rtol=tol, atol=tol * scale), name
+        assert x.dtype == tdt
+        assert np.allclose(host(b.grad), bd.grad.numpy(), rtol=tol, atol=tol * float(bd.grad.abs().max())), name
+        rows = np.repeat(np.arange(n), np.diff(p))
+        gA = Ad.grad.numpy()[rows, i]
+        assert np.allclose(host(A.grad.data), gA, rtol=tol, atol=tol * float(np.abs(gA).max())), name
+
+
+def test_errors(dev):
+    d, i, p, _ = G.random_csr(5, 7, 0.5, 1, np.float64)
+    with pytest.raises(RuntimeError, match="square"):
+        numml_amd.load_compiled().splu(5, 7, *to_dev(dev, d, i, p))
+    with pytest.raises(RuntimeError, match="square"):
+        mirror.splu(5, 7, *to_dev(dev, d, i, p))
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        mirror.splu(5, 5, torch.ones(5), torch.arange(5), torch.arange(6))
