@@ -416,6 +416,69 @@ class Lincomb(Workload):
                 "sample": f"{reps} x (splincomb_forward + splincomb_backward) of the full workload, serial C oracle"}
 
 
+class SpSolve(Workload):
+    """x = A^-1 b by LU without pivoting (pattern with fill, numeric factors, two triangular
+    solves) and its backward, on the 2-D Poisson matrix in natural ordering, where the band
+    fills in."""
+    name = "spsolve"
+    unit = "ms"
+    dtype = "f64"
+    higher_is_better = False
+
+    def setup(self, dev):
+        import torch
+        from numml_amd import generators as G
+        from numml_amd import _binding
+        self.ext = _binding.ops
+        n = int(os.environ.get("NM_BENCH_SPSOLVE_N", "64"))
+        d, i, p, (rows, cols) = G.poisson2d(n, np.float64, jitter_seed=0)
+        self.host = (d, i, p, rows, cols)
+        self.b_h = np.random.default_rng(1).standard_normal(rows)
+        self.g_h = np.random.default_rng(2).standard_normal(rows)
+        t = lambda a: torch.from_numpy(a).to(dev)
+        self.D, self.I, self.P, self.Bv, self.Gv = t(d), t(i), t(p), t(self.b_h), t(self.g_h)
+        self.rows, self.nnz = rows, d.shape[0]
+        M = self.ext.splu(rows, rows, self.D, self.I, self.P)
+        self.nnzM = M[0].shape[0]
+        s = 8
+        # factor: A in, M and M^T out; four solves over M; grad_A out
+        self.dominant_bytes = self.nnz * (s + 8) + 2 * self.nnzM * (s + 8) + 3 * (rows + 1) * 8
+        self.bytes_per_step = self.dominant_bytes + 4 * (self.nnzM * (s + 8) + (rows + 1) * 8 + 2 * rows * s) \
+            + self.nnz * s
+        self.dominant_name = "splu: lu_rows_kernel (count, fill), transpose, lu_numeric_kernel per level run"
+        self.config = {"workload": f"spsolve_fwd_bwd_f64_poisson2d_{n}", "rows": rows, "nnz": self.nnz,
+                       "nnz_LU": self.nnzM, "binding": _binding.name}
+
+    def step(self):
+        r = self.rows
+        M = self.ext.splu(r, r, self.D, self.I, self.P)
+        y = self.ext.sptrsv_forward(r, r, M[0], M[1], M[2], True, True, self.Bv)
+        x = self.ext.sptrsv_forward(r, r, M[0], M[1], M[2], False, False, y)
+        return self.ext.spsolve_backward(self.Gv, x, r, r, M[3], M[4], M[5], self.D, self.I, self.P)
+
+    def dominant(self):
+        return self.ext.splu(self.rows, self.rows, self.D, self.I, self.P)
+
+    def value(self, ms_per_step):
+        return ms_per_step
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        d, i, p, rows, cols = self.host
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            M = oracle.splu(rows, rows, d, i, p)
+            y = oracle.sptrsv_forward(rows, rows, M[0], M[1], M[2], True, True, self.b_h)
+            x = oracle.sptrsv_forward(rows, rows, M[0], M[1], M[2], False, False, y)
+            oracle.spsolve_backward(self.g_h, x, rows, rows, M[3], M[4], M[5], d, i, p)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget_s or reps >= 20:
+                break
+        return {"value": el / reps * 1e3, "unit": "ms", "cores": 1, "kind": "port",
+                "sample": f"{reps} x (splu + two solves + spsolve_backward) of the full workload, serial C oracle"}
+
+
 class Copy(Workload):
     """Plain device copy of a known size: the calibration run for the rocprofv3
     FETCH_SIZE / WRITE_SIZE counters and the practical HBM ceiling of this part."""
@@ -447,6 +510,7 @@ WORKLOADS = {
     "spmm": SpMM,
     "spgemm": SpGEMM,
     "sptrsv": SpTRSV,
+    "spsolve": SpSolve,
     "transpose": Transpose,
     "lincomb": Lincomb,
     "copy": Copy,

@@ -235,10 +235,15 @@ int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz,
  *                           caller reads As_indptr[rows] to size the next call)
  *   nm_splu_fill            As_indices (ascending per row) and As_data: A's
  *                           value where A stores the column, 0 at the fill
+ *   nm_splu_values          As_data alone, for a pattern from an earlier
+ *                           nm_splu_fill of a matrix with A's structure
  *   nm_splu_numeric         in-place factorisation of the TRANSPOSE of that
- *                           matrix (rows of Mt = columns of M), ordered by the
- *                           levels of an nm_sptrsv_analyse plan of Mt's pattern
- *                           taken as a lower-triangular solve
+ *                           matrix (rows of Mt = columns of M).  Columns are
+ *                           taken in ascending order by wavefronts that wait
+ *                           on a flag per column they depend on; poll_limit
+ *                           bounds the polls of one flag (0 = default), and
+ *                           when it is exceeded every wavefront leaves and the
+ *                           call returns NM_ERR_HIP.  Synchronises the stream.
  * The caller transposes As -> Mt before, and Mt -> M after, the numeric phase. */
 int nm_splu_symbolic_bytes(int64_t rows, size_t *bytes);
 int nm_splu_symbolic(int64_t rows, const int64_t *A_indices,
@@ -248,8 +253,14 @@ int nm_splu_fill(nm_dtype dt, int64_t rows, const void *A_data,
                  const int64_t *A_indices, const int64_t *A_indptr,
                  const int64_t *As_indptr, int64_t *As_indices, void *As_data,
                  void *workspace, size_t workspace_bytes, nm_stream stream);
-int nm_splu_numeric(const nm_sptrsv_plan *plan, nm_dtype dt, void *Mt_data,
+int nm_splu_values(nm_dtype dt, int64_t rows, const void *A_data,
+                   const int64_t *A_indices, const int64_t *A_indptr,
+                   const int64_t *As_indptr, const int64_t *As_indices,
+                   void *As_data, nm_stream stream);
+int nm_splu_numeric_bytes(int64_t cols, size_t *bytes);
+int nm_splu_numeric(nm_dtype dt, int64_t cols, void *Mt_data,
                     const int64_t *Mt_indices, const int64_t *Mt_indptr,
+                    void *workspace, size_t workspace_bytes, int64_t poll_limit,
                     nm_stream stream);
 
 /* ------------------------------------------------- linear combination

@@ -64,7 +64,9 @@ _SIGNATURES = {
     "nm_splu_symbolic_bytes": [_c_i64, ctypes.POINTER(_c_size)],
     "nm_splu_symbolic": [_c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr],
     "nm_splu_fill": [_c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr],
-    "nm_splu_numeric": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_splu_values": [_c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_splu_numeric_bytes": [_c_i64, ctypes.POINTER(_c_size)],
+    "nm_splu_numeric": [_c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_i64, _c_ptr],
     "nm_masked_outer": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_dbl, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
 

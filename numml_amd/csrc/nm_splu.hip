@@ -15,6 +15,20 @@
 //
 // The work per row is that of the serial algorithm (the reference spends O(rows)
 // per row as well): this is meant for the moderate sizes a direct solve is used at.
+//
+// Numeric phase (cpp/sparse_csr_cpu.cpp:956-1000): left-looking column LU on the rows of
+// M^T (= columns of M).  For the entries (i, k), i < k, of column k in ascending i, every
+// later entry (j, k) takes  M_jk -= M_ji * M_ik  where column i stores row j; then the
+// entries below the diagonal are divided by it.  Per entry the operations come in the
+// serial order, so the factors equal the reference's bit for bit.
+// Column k needs the finished columns i of its entries above the diagonal, and nothing
+// else: wavefronts take columns in ascending order from a ticket counter, keep the column
+// in LDS, and before using column i wait for its flag.  A wavefront only ever waits for a
+// column with a smaller ticket, which a running wavefront holds, so the grid always makes
+// progress whatever part of it is resident; a bounded number of polls backs that up, after
+// which every wavefront leaves and the call reports an error.  Early pivots of a column
+// overlap with the tail of the columns before it, which is where a banded factor, whose
+// columns form one long dependency chain, gets its parallelism from.
 #include "nm_common.hpp"
 #include "nm_scan.hpp"
 
@@ -150,6 +164,157 @@ __global__ __launch_bounds__(kBlock) void lu_rows_kernel(int64_t rows, const T *
     }
 }
 
+// Values on a known filled pattern: one wavefront per row, a lane per entry of the row.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lu_values_kernel(int64_t rows, const T *__restrict__ A_data,
+                                                           const int64_t *__restrict__ A_indices,
+                                                           const int64_t *__restrict__ A_indptr,
+                                                           const int64_t *__restrict__ As_indptr,
+                                                           const int64_t *__restrict__ As_indices,
+                                                           T *__restrict__ As_data) {
+    const int lane = threadIdx.x & 63;
+    const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6; i < rows; i += nwaves) {
+        const int64_t ab = A_indptr[i], ae = A_indptr[i + 1], pe = As_indptr[i + 1];
+        for (int64_t p = As_indptr[i] + lane; p < pe; p += 64) {
+            const int64_t j = As_indices[p];
+            int64_t lo = ab, hi = ae;
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) >> 1;
+                if (A_indices[mid] < j) lo = mid + 1; else hi = mid;
+            }
+            As_data[p] = (lo < ae && A_indices[lo] == j) ? A_data[lo] : T(0);
+        }
+    }
+}
+
+constexpr int kLuCap = 1024;              // entries of a column kept in LDS, per wavefront
+constexpr int kLuWavesPerBlock = kBlock / 64;
+constexpr int64_t kLuSpinLimit = 1 << 24;  // polls of one dependency flag before giving up
+
+struct LuFlow {
+    int64_t *done;   // [cols] 0 = pending, else 1 + position of the column's first entry below the diagonal
+    int32_t *ctl;    // [0] next ticket, [1] failure
+};
+
+size_t flow_layout(int64_t cols, void *base, LuFlow *F) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += align_up(bytes);
+        return q;
+    };
+    LuFlow f;
+    f.ctl = (int32_t *)take(64);
+    f.done = (int64_t *)take((size_t)(cols > 0 ? cols : 1) * 8);
+    if (F) *F = f;
+    return off;
+}
+
+// The column of a wavefront: in LDS (rows as 32-bit, values) or, when it is too long, in
+// place in global memory, where the lanes hand values on through volatile accesses.
+template <typename T, bool IN_LDS>
+struct OwnColumn {
+    int32_t *s_rows;
+    T *s_vals;
+    const int64_t *g_rows;
+    volatile T *g_vals;
+    __device__ __forceinline__ int64_t row(int64_t e) const { return IN_LDS ? (int64_t)s_rows[e] : g_rows[e]; }
+    __device__ __forceinline__ T val(int64_t e) const { return IN_LDS ? s_vals[e] : g_vals[e]; }
+    __device__ __forceinline__ void set(int64_t e, T v) const {
+        if (IN_LDS) s_vals[e] = v; else g_vals[e] = v;
+    }
+};
+
+// Returns false when a dependency did not arrive within the poll limit (or another wavefront failed).
+template <typename T, bool IN_LDS>
+__device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T, IN_LDS> &own,
+                          const int64_t *__restrict__ indices, const int64_t *__restrict__ indptr, T *values,
+                          int64_t *done, int32_t *ctl, int64_t spin_limit, int lane) {
+    if (IN_LDS) {
+        for (int64_t e = lane; e < len; e += 64) {
+            own.s_rows[e] = (int32_t)indices[pb + e];
+            own.s_vals[e] = values[pb + e];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+    int64_t e = 0;
+    for (; e < len; ++e) {
+        const int64_t i = own.row(e);
+        if (i >= k) break;
+        // column i: wait for it, then its entries below the diagonal are [ls, ie)
+        int64_t flag = 0, polls = 0;
+        for (;;) {
+            flag = __hip_atomic_load(done + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (flag != 0) break;
+            if (++polls > spin_limit || __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+                return false;
+            __builtin_amdgcn_s_sleep(4);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // the loads below stay after the flag
+        const int64_t ls = flag - 1, ie = indptr[i + 1];
+        const T m_ik = own.val(e);
+        for (int64_t t0 = ls; t0 < ie; t0 += 64) {
+            const int64_t t = t0 + lane;
+            if (t < ie) {
+                const int64_t j = indices[t];
+                const T m_ji = __hip_atomic_load(values + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                int64_t lo = e + 1, hi = len;   // row j among the later entries of this column
+                while (lo < hi) {
+                    const int64_t mid = (lo + hi) >> 1;
+                    if (own.row(mid) < j) lo = mid + 1; else hi = mid;
+                }
+                if (lo < len && own.row(lo) == j) {
+                    const T prod = m_ji * m_ik;
+                    own.set(lo, own.val(lo) - prod);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+    int64_t below = e;   // first entry below the diagonal
+    if (e < len && own.row(e) == k) {
+        below = e + 1;
+        const T d = own.val(e);
+        for (int64_t q = below + lane; q < len; q += 64) own.set(q, own.val(q) / d);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+    if (IN_LDS)
+        for (int64_t q = lane; q < len; q += 64) values[pb + q] = own.s_vals[q];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    if (lane == 0) __hip_atomic_store(done + k, pb + below + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lu_flow_kernel(int64_t cols, const int64_t *__restrict__ indices,
+                                                         const int64_t *__restrict__ indptr, T *values,
+                                                         int64_t *done, int32_t *ctl, int64_t spin_limit) {
+    __shared__ int32_t s_rows[kLuWavesPerBlock][kLuCap];
+    __shared__ T s_vals[kLuWavesPerBlock][kLuCap];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (;;) {
+        int32_t ticket = 0;
+        if (lane == 0) ticket = atomicAdd(ctl, 1);
+        const int64_t k = __builtin_amdgcn_readfirstlane(ticket);
+        if (k >= cols) break;
+        if (__hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+        const int64_t pb = indptr[k], len = indptr[k + 1] - pb;
+        bool ok;
+        if (len <= kLuCap) {
+            const OwnColumn<T, true> own{s_rows[w], s_vals[w], nullptr, nullptr};
+            ok = lu_column<T, true>(k, pb, len, own, indices, indptr, values, done, ctl, spin_limit, lane);
+        } else {
+            const OwnColumn<T, false> own{nullptr, nullptr, indices + pb, values + pb};
+            ok = lu_column<T, false>(k, pb, len, own, indices, indptr, values, done, ctl, spin_limit, lane);
+        }
+        if (!ok) {
+            if (lane == 0) atomicExch(ctl + 1, 1);
+            break;
+        }
+    }
+}
+
 int check_rows(int64_t rows) {
     NM_REQUIRE(rows >= 0, "negative size");
     if (rows >= (int64_t(1) << 31) - 2)
@@ -213,5 +378,67 @@ extern "C" int nm_splu_fill(nm_dtype dt, int64_t rows, const void *A_data, const
                            (const double *)A_data, A_indices, A_indptr, const_cast<int64_t *>(As_indptr), As_indices,
                            (double *)As_data, S.stamp, S.queue, S.keep);
     NM_LAUNCH_CHECK("lu_rows_kernel<fill>");
+    return NM_OK;
+}
+
+extern "C" int nm_splu_values(nm_dtype dt, int64_t rows, const void *A_data, const int64_t *A_indices,
+                              const int64_t *A_indptr, const int64_t *As_indptr, const int64_t *As_indices,
+                              void *As_data, nm_stream stream) {
+    if (int rc = check_rows(rows)) return rc;
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    if (rows == 0) return NM_OK;
+    NM_REQUIRE(A_indptr && As_indptr, "null pointer argument");
+    hipStream_t s = nm::as_stream(stream);
+    int64_t grid = nm::ceil_div(rows * 64, kBlock);
+    if (grid > 65536) grid = 65536;
+    if (dt == NM_F32)
+        hipLaunchKernelGGL(lu_values_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, rows,
+                           (const float *)A_data, A_indices, A_indptr, As_indptr, As_indices, (float *)As_data);
+    else
+        hipLaunchKernelGGL(lu_values_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, rows,
+                           (const double *)A_data, A_indices, A_indptr, As_indptr, As_indices, (double *)As_data);
+    NM_LAUNCH_CHECK("lu_values_kernel");
+    return NM_OK;
+}
+
+extern "C" int nm_splu_numeric_bytes(int64_t cols, size_t *bytes) {
+    NM_REQUIRE(bytes != nullptr, "bytes is null");
+    if (int rc = check_rows(cols)) return rc;
+    *bytes = flow_layout(cols, nullptr, nullptr);
+    return NM_OK;
+}
+
+extern "C" int nm_splu_numeric(nm_dtype dt, int64_t cols, void *Mt_data, const int64_t *Mt_indices,
+                               const int64_t *Mt_indptr, void *workspace, size_t workspace_bytes,
+                               int64_t poll_limit, nm_stream stream) {
+    if (int rc = check_rows(cols)) return rc;
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    if (cols == 0) return NM_OK;
+    NM_REQUIRE(Mt_indptr && workspace, "null pointer argument");
+    LuFlow F;
+    const size_t need = flow_layout(cols, workspace, &F);
+    if (workspace_bytes < need)
+        return nm::fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    hipStream_t s = nm::as_stream(stream);
+    if (int rc = nm::fill_async(F.ctl, 16, (int32_t)0, s)) return rc;
+    if (int rc = nm::fill_async(F.done, cols, (int64_t)0, s)) return rc;
+    int64_t grid = nm::ceil_div(cols, kLuWavesPerBlock);
+    if (grid > 1024) grid = 1024;
+    const int64_t limit = poll_limit > 0 ? poll_limit : kLuSpinLimit;
+    if (dt == NM_F32)
+        hipLaunchKernelGGL(lu_flow_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, Mt_indices,
+                           Mt_indptr, (float *)Mt_data, F.done, F.ctl, limit);
+    else
+        hipLaunchKernelGGL(lu_flow_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, Mt_indices,
+                           Mt_indptr, (double *)Mt_data, F.done, F.ctl, limit);
+    NM_LAUNCH_CHECK("lu_flow_kernel");
+    int32_t ctl_h[2] = {0, 0};
+    if (hipMemcpyAsync(ctl_h, F.ctl, sizeof(ctl_h), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess)
+        return nm::fail(NM_ERR_HIP, "reading the factorisation status back failed: %s",
+                        hipGetErrorString(hipGetLastError()));
+    if (ctl_h[1] != 0)
+        return nm::fail(NM_ERR_HIP, "a column waited more than %lld polls for one it depends on",
+                        (long long)limit);
     return NM_OK;
 }

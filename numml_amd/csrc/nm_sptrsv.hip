@@ -163,10 +163,14 @@ __global__ __launch_bounds__(kNarrow) void kahn_kernel(int32_t rows, int lower,
     if (threadIdx.x == 0) level_ptr[0] = 0;
     while (head < tail) {
         if (threadIdx.x == 0) level_ptr[nlev + 1] = tail;
-        for (int q = head + threadIdx.x; q < tail; q += kNarrow) {
+        // a narrow level spreads the dependants of each row over g lanes
+        int g = 1;
+        while (g < 64 && (tail - head) * g * 2 <= kNarrow) g *= 2;
+        const int sub = threadIdx.x & (g - 1);
+        for (int q = head + threadIdx.x / g; q < tail; q += kNarrow / g) {
             const int32_t r = order[q];
             const int32_t pe = t_indptr[r + 1];
-            for (int32_t p = t_indptr[r]; p < pe; ++p) {
+            for (int32_t p = t_indptr[r] + sub; p < pe; p += g) {
                 const int32_t d = t_row[p];
                 if (lower ? d > r : d < r)
                     if (atomicSub(deg + d, 1) == 1) order[atomicAdd(&s_tail, 1)] = d;
@@ -829,94 +833,6 @@ extern "C" int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan) {
 }
 
 extern "C" void nm_sptrsv_plan_destroy(nm_sptrsv_plan *plan) { delete plan; }
-
-// ---- sparse LU, numeric phase ------------------------------------------------
-//
-// Left-looking column LU on the rows of M^T (= columns of M = L + U), following
-// cpp/sparse_csr_cpu.cpp:956-1000: for the entries (i, k), i < k, of column k in ascending
-// i, every later entry (j, k) takes  M_jk -= M_ji * M_ik  where column i stores row j; then
-// the entries below the diagonal are divided by it.  Column k needs the finished columns i
-// of its entries above the diagonal: exactly the dependencies of a lower-triangular solve
-// with M^T, so the plan's levels order the columns, and the columns of a level are
-// independent.  One wavefront takes a column; its pivots are serial, the updates of one
-// pivot go over the lanes.  Operation order per entry is the serial one, so the factors
-// equal the reference's bit for bit.  Values are read and written with volatile
-// operations: lanes of a wavefront, and the levels of a single-workgroup launch, hand
-// them on through memory.
-template <typename T>
-__global__ __launch_bounds__(kNarrow) void lu_numeric_kernel(const int32_t *__restrict__ order,
-                                                             const int32_t *__restrict__ level_ptr, int32_t l0,
-                                                             int32_t l1, const int64_t *__restrict__ indices,
-                                                             const int64_t *__restrict__ indptr, T *values) {
-    volatile T *data = values;
-    const int lane = threadIdx.x & 63;
-    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
-    for (int32_t l = l0; l < l1; ++l) {
-        const int32_t qe = level_ptr[l + 1];
-        for (int64_t q = level_ptr[l] + wave; q < qe; q += nwaves) {
-            const int64_t k = order[q];
-            const int64_t pe = indptr[k + 1];
-            int64_t diag = -1;
-            for (int64_t p = indptr[k]; p < pe; ++p) {
-                const int64_t i = indices[p];
-                if (i >= k) {
-                    if (i == k) diag = p;
-                    break;
-                }
-                const T m_ik = data[p];
-                const int64_t ib = indptr[i], ie = indptr[i + 1];
-                for (int64_t e = p + 1 + lane; e < pe; e += 64) {
-                    const int64_t j = indices[e];
-                    int64_t lo = ib, hi = ie;
-                    while (lo < hi) {
-                        const int64_t mid = (lo + hi) >> 1;
-                        if (indices[mid] < j) lo = mid + 1; else hi = mid;
-                    }
-                    if (lo < ie && indices[lo] == j) {
-                        const T prod = data[lo] * m_ik;
-                        data[e] = data[e] - prod;
-                    }
-                }
-                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-            }
-            if (diag >= 0) {
-                const T d = data[diag];
-                for (int64_t e = diag + 1 + lane; e < pe; e += 64) data[e] = data[e] / d;
-            }
-        }
-        if (l + 1 < l1) {   // only single-workgroup launches span levels
-            __threadfence();
-            __syncthreads();
-        }
-    }
-}
-
-extern "C" int nm_splu_numeric(const nm_sptrsv_plan *plan, nm_dtype dt, void *Mt_data, const int64_t *Mt_indices,
-                               const int64_t *Mt_indptr, nm_stream stream) {
-    NM_REQUIRE(plan != nullptr, "plan is null");
-    NM_REQUIRE(plan->lower == 1, "the plan must order M^T as a lower-triangular solve");
-    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
-    if (plan->rows == 0 || plan->nnz == 0) return NM_OK;
-    NM_REQUIRE(Mt_data && Mt_indices && Mt_indptr, "null pointer argument");
-    hipStream_t s = nm::as_stream(stream);
-    for (const nm_sptrsv_plan::Launch &L : plan->launches) {
-        unsigned grid = 1, block = kNarrow;
-        if (L.wide) {
-            block = kBlock;
-            int64_t g = nm::ceil_div((int64_t)(L.q1 - L.q0) * 64, kBlock);
-            grid = (unsigned)(g > 65536 ? 65536 : g);
-        }
-        if (dt == NM_F32)
-            hipLaunchKernelGGL(lu_numeric_kernel<float>, dim3(grid), dim3(block), 0, s, plan->order, plan->level_ptr,
-                               L.l0, L.l1, Mt_indices, Mt_indptr, (float *)Mt_data);
-        else
-            hipLaunchKernelGGL(lu_numeric_kernel<double>, dim3(grid), dim3(block), 0, s, plan->order,
-                               plan->level_ptr, L.l0, L.l1, Mt_indices, Mt_indptr, (double *)Mt_data);
-        NM_LAUNCH_CHECK("lu_numeric_kernel");
-    }
-    return NM_OK;
-}
 
 extern "C" int nm_sptrsv_solve_bytes(int64_t rows, int64_t nnz, size_t *bytes) {
     NM_REQUIRE(rows >= 0 && nnz >= 0 && bytes, "bad arguments");

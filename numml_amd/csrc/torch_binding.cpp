@@ -104,12 +104,14 @@ bool planned_backward() { return g_planned.load(std::memory_order_relaxed); }
 // while the plan is cached; in-place edits bump the version and miss the cache.
 
 struct Plan {
-    char kind;  // 'T' transposed structure, 'L' level schedule
+    char kind;  // 'T' transposed structure, 'L' level schedule, 'U' filled pattern of the LU factors
     int device;
     const void *idx_ptr, *ptr_ptr;
     uint32_t idx_version, ptr_version;
     int64_t nnz, nptr, a, b;
     Tensor indices, indptr, mem;
+    std::vector<Tensor> derived;             // 'U': structure tensors handed out to callers
+    std::vector<uint32_t> derived_versions;  //      and their version counters when built
     nm_sptrsv_plan *handle = nullptr;
     ~Plan() {
         if (handle) nm_sptrsv_plan_destroy(handle);
@@ -612,6 +614,56 @@ std::vector<Tensor> sptrsv_backward(Tensor grad_x, Tensor x, int A_rows, int A_c
 // schedule of a triangular pattern; no counterpart in the reference (diagnostics).
 // ------------------------------------------------------------------------ sparse LU
 
+// The filled pattern of the factors, its transpose and the map between them depend on A's
+// structure alone: they are computed once per pattern and the same index tensors are handed
+// out by every later call, so that the solves that follow find their level schedules cached.
+std::shared_ptr<Plan> lu_pattern(const Tensor &A_indices, const Tensor &A_indptr, int64_t rows,
+                                 const c10::Device &dev) {
+    for (int attempt = 0;; ++attempt) {
+        auto plan = cached('U', A_indices, A_indptr, rows, rows, [&](Plan &p) {
+            const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
+            const nm_stream stream = current_stream(dev);
+            size_t bytes = 0;
+            check(nm_splu_symbolic_bytes(rows, &bytes), "nm_splu_symbolic_bytes");
+            Tensor work = scratch(bytes, dev);
+            Tensor M_indptr = torch::empty({rows + 1}, iopt);
+            check(nm_splu_symbolic(rows, A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                   M_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, stream),
+                  "nm_splu_symbolic");
+            const int64_t nnz = M_indptr[rows].item<int64_t>();
+            Tensor M_indices = torch::empty({nnz}, iopt);
+            Tensor zeros = torch::zeros({std::max<int64_t>(A_indices.numel(), 1)},
+                                        torch::TensorOptions().dtype(torch::kFloat32).device(dev));
+            Tensor As_data = torch::empty({nnz}, zeros.options());
+            check(nm_splu_fill(NM_F32, rows, zeros.data_ptr(), A_indices.data_ptr<int64_t>(),
+                               A_indptr.data_ptr<int64_t>(), M_indptr.data_ptr<int64_t>(),
+                               M_indices.data_ptr<int64_t>(), As_data.data_ptr(), work.data_ptr(), bytes, stream),
+                  "nm_splu_fill");
+            auto tplan = transpose_plan(M_indices, M_indptr, rows, rows, dev);
+            Tensor Mt_data = torch::empty_like(As_data);
+            Tensor Mt_indices = torch::empty({nnz}, iopt);
+            Tensor Mt_indptr = torch::empty({rows + 1}, iopt);
+            Tensor Mt_to_M = torch::empty({nnz}, iopt);
+            check(nm_csr_transpose_forward(NM_F32, rows, rows, nnz, As_data.data_ptr(), tplan->mem.data_ptr(),
+                                           Mt_data.data_ptr(), Mt_indices.data_ptr<int64_t>(),
+                                           Mt_indptr.data_ptr<int64_t>(), Mt_to_M.data_ptr<int64_t>(), stream),
+                  "nm_csr_transpose_forward");
+            p.derived = {M_indices, M_indptr, Mt_indices, Mt_indptr, Mt_to_M};
+            for (const Tensor &t : p.derived) p.derived_versions.push_back(t._version());
+            c10::hip::getCurrentHIPStream(dev.index()).synchronize();   // complete for every stream
+        });
+        bool intact = true;   // a caller may have edited the tensors it was handed
+        for (size_t i = 0; i < plan->derived.size(); ++i)
+            intact = intact && plan->derived[i]._version() == plan->derived_versions[i];
+        if (intact || attempt > 0) {
+            TORCH_CHECK(intact, "the cached factor pattern was modified in place");
+            return plan;
+        }
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        g_plans.remove(plan);
+    }
+}
+
 // [M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]  (cpp/sparse_csr.hpp:107-111)
 std::vector<Tensor> splu(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
     const auto dev = need_device({&A_data, &A_indices, &A_indptr});
@@ -621,42 +673,37 @@ std::vector<Tensor> splu(int A_rows, int A_cols, Tensor A_data, Tensor A_indices
     A_indptr = index_tensor(A_indptr, "A_indptr");
     c10::hip::HIPGuard guard(dev.index());
     const int64_t rows = A_rows;
-    const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
     const nm_stream stream = current_stream(dev);
+    const nm_dtype dt = dtype_of(A_data);
 
-    // pattern with fill: count, then write
-    size_t bytes = 0;
-    check(nm_splu_symbolic_bytes(rows, &bytes), "nm_splu_symbolic_bytes");
-    Tensor work = scratch(bytes, dev);
-    Tensor M_indptr = torch::empty({rows + 1}, iopt);
-    check(nm_splu_symbolic(rows, A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
-                           M_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, stream),
-          "nm_splu_symbolic");
-    const int64_t nnz = M_indptr[rows].item<int64_t>();
-    Tensor M_indices = torch::empty({nnz}, iopt);
+    auto pattern = lu_pattern(A_indices, A_indptr, rows, dev);
+    const Tensor &M_indices = pattern->derived[0], &M_indptr = pattern->derived[1];
+    const Tensor &Mt_indices = pattern->derived[2], &Mt_indptr = pattern->derived[3];
+    const Tensor &Mt_to_M = pattern->derived[4];
+    const int64_t nnz = M_indices.numel();
+
+    // A's values on the filled pattern, moved to the transpose: the factorisation runs by column
     Tensor As_data = torch::empty({nnz}, A_data.options());
-    check(nm_splu_fill(dtype_of(A_data), rows, A_data.data_ptr(), A_indices.data_ptr<int64_t>(),
-                       A_indptr.data_ptr<int64_t>(), M_indptr.data_ptr<int64_t>(), M_indices.data_ptr<int64_t>(),
-                       As_data.data_ptr(), work.data_ptr(), bytes, stream),
-          "nm_splu_fill");
-
-    // the factorisation runs by column: on the rows of the transpose
+    check(nm_splu_values(dt, rows, A_data.data_ptr(), A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                         M_indptr.data_ptr<int64_t>(), M_indices.data_ptr<int64_t>(), As_data.data_ptr(), stream),
+          "nm_splu_values");
     auto tplan = transpose_plan(M_indices, M_indptr, rows, rows, dev);
+    const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
     Tensor Mt_data = torch::empty_like(As_data);
-    Tensor Mt_indices = torch::empty({nnz}, iopt);
-    Tensor Mt_indptr = torch::empty({rows + 1}, iopt);
-    Tensor Mt_to_M = torch::empty({nnz}, iopt);
-    check(nm_csr_transpose_forward(dtype_of(A_data), rows, rows, nnz, As_data.data_ptr(), tplan->mem.data_ptr(),
-                                   Mt_data.data_ptr(), Mt_indices.data_ptr<int64_t>(),
-                                   Mt_indptr.data_ptr<int64_t>(), Mt_to_M.data_ptr<int64_t>(), stream),
+    Tensor idx_scratch = torch::empty({2 * nnz + rows + 1}, iopt);   // the structure is already known
+    int64_t *is = idx_scratch.data_ptr<int64_t>();
+    check(nm_csr_transpose_forward(dt, rows, rows, nnz, As_data.data_ptr(), tplan->mem.data_ptr(),
+                                   Mt_data.data_ptr(), is, is + nnz, is + nnz + rows + 1, stream),
           "nm_csr_transpose_forward");
-    auto levels = level_plan(Mt_indices, Mt_indptr, rows, true, dev);
-    check(nm_splu_numeric(levels->handle, dtype_of(A_data), Mt_data.data_ptr(), Mt_indices.data_ptr<int64_t>(),
-                          Mt_indptr.data_ptr<int64_t>(), stream),
+    size_t bytes = 0;
+    check(nm_splu_numeric_bytes(rows, &bytes), "nm_splu_numeric_bytes");
+    Tensor work = scratch(bytes, dev);
+    check(nm_splu_numeric(dt, rows, Mt_data.data_ptr(), Mt_indices.data_ptr<int64_t>(),
+                          Mt_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, 0, stream),
           "nm_splu_numeric");
     Tensor M_data = torch::empty_like(Mt_data);
-    check(nm_csr_transpose_backward(dtype_of(A_data), nnz, Mt_data.data_ptr(), Mt_to_M.data_ptr<int64_t>(),
-                                    M_data.data_ptr(), stream),
+    check(nm_csr_transpose_backward(dt, nnz, Mt_data.data_ptr(), Mt_to_M.data_ptr<int64_t>(), M_data.data_ptr(),
+                                    stream),
           "nm_csr_transpose_backward");
     return {M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr};
 }

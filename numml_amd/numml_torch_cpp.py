@@ -495,6 +495,48 @@ def _plan_for(indices, indptr, rows, lower, dev):
                    lambda: _Plan(indices, indptr, rows, lower, dev))
 
 
+class _LUPattern:
+    """Filled pattern of the LU factors of one sparsity pattern, its transpose and the map
+    between them.  Every splu call on that pattern hands out these same index tensors, so the
+    solves that follow find their level schedules cached."""
+
+    def __init__(self, A_indices, A_indptr, rows, dev):
+        L = _lib.lib()
+        stream = _stream(dev)
+        self.indices, self.indptr = A_indices, A_indptr
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(L.nm_splu_symbolic_bytes(rows, ctypes.byref(nbytes)), "nm_splu_symbolic_bytes")
+        work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+        M_indptr = torch.empty(rows + 1, dtype=torch.int64, device=dev)
+        _lib.check(L.nm_splu_symbolic(rows, _ptr(A_indices), _ptr(A_indptr), _ptr(M_indptr), _ptr(work),
+                                      nbytes.value, stream), "nm_splu_symbolic")
+        nnz = int(M_indptr[rows].item())
+        M_indices = torch.empty(nnz, dtype=torch.int64, device=dev)
+        zeros = torch.zeros(max(A_indices.shape[0], 1), dtype=torch.float32, device=dev)
+        As_data = torch.empty(nnz, dtype=torch.float32, device=dev)
+        _lib.check(L.nm_splu_fill(_dt(zeros), rows, _ptr(zeros), _ptr(A_indices), _ptr(A_indptr),
+                                  _ptr(M_indptr), _ptr(M_indices), _ptr(As_data), _ptr(work), nbytes.value,
+                                  stream), "nm_splu_fill")
+        _, Mt_indices, Mt_indptr, Mt_to_M = csr_transpose_forward(rows, rows, As_data, M_indices, M_indptr)
+        self.derived = (M_indices, M_indptr, Mt_indices, Mt_indptr, Mt_to_M)
+        self.versions = tuple(t._version for t in self.derived)
+        torch.cuda.current_stream(dev).synchronize()    # complete for every stream
+
+    def intact(self):
+        return tuple(t._version for t in self.derived) == self.versions
+
+
+def _lu_pattern(A_indices, A_indptr, rows, dev):
+    make = lambda: _LUPattern(A_indices, A_indptr, rows, dev)
+    plan = _cached("U", A_indices, A_indptr, (rows,), make)
+    if not plan.intact():      # a caller edited the tensors it was handed: build them again
+        with _plans_lock:
+            for key in [k for k, v in _plans.items() if v is plan]:
+                del _plans[key]
+        plan = _cached("U", A_indices, A_indptr, (rows,), make)
+    return plan
+
+
 def splu(A_rows, A_cols, A_data, A_indices, A_indptr):
     """[M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]: L + U without pivoting on the
     filled pattern, and its transpose  (cpp/sparse_csr.hpp:107-111)."""
@@ -507,23 +549,18 @@ def splu(A_rows, A_cols, A_data, A_indices, A_indptr):
     rows = A_rows
     with torch.cuda.device(dev):
         stream = _stream(dev)
-        nbytes = ctypes.c_size_t(0)
-        _lib.check(L.nm_splu_symbolic_bytes(rows, ctypes.byref(nbytes)), "nm_splu_symbolic_bytes")
-        work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
-        M_indptr = torch.empty(rows + 1, dtype=torch.int64, device=dev)
-        _lib.check(L.nm_splu_symbolic(rows, _ptr(A_indices), _ptr(A_indptr), _ptr(M_indptr), _ptr(work),
-                                      nbytes.value, stream), "nm_splu_symbolic")
-        nnz = int(M_indptr[rows].item())
-        M_indices = torch.empty(nnz, dtype=torch.int64, device=dev)
+        M_indices, M_indptr, Mt_indices, Mt_indptr, Mt_to_M = _lu_pattern(A_indices, A_indptr, rows, dev).derived
+        nnz = M_indices.shape[0]
+        # A's values on the filled pattern, moved to the transpose: the factorisation runs by column
         As_data = torch.empty(nnz, dtype=A_data.dtype, device=dev)
-        _lib.check(L.nm_splu_fill(_dt(A_data), rows, _ptr(A_data), _ptr(A_indices), _ptr(A_indptr),
-                                  _ptr(M_indptr), _ptr(M_indices), _ptr(As_data), _ptr(work), nbytes.value,
-                                  stream), "nm_splu_fill")
-        # the factorisation runs by column: on the rows of the transpose
-        Mt_data, Mt_indices, Mt_indptr, Mt_to_M = csr_transpose_forward(rows, rows, As_data, M_indices, M_indptr)
-        plan = _plan_for(Mt_indices, Mt_indptr, rows, True, dev)
-        _lib.check(L.nm_splu_numeric(plan.handle, _dt(A_data), _ptr(Mt_data), _ptr(Mt_indices), _ptr(Mt_indptr),
-                                     stream), "nm_splu_numeric")
+        _lib.check(L.nm_splu_values(_dt(A_data), rows, _ptr(A_data), _ptr(A_indices), _ptr(A_indptr),
+                                    _ptr(M_indptr), _ptr(M_indices), _ptr(As_data), stream), "nm_splu_values")
+        Mt_data = csr_transpose_forward(rows, rows, As_data, M_indices, M_indptr)[0]
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(L.nm_splu_numeric_bytes(rows, ctypes.byref(nbytes)), "nm_splu_numeric_bytes")
+        work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+        _lib.check(L.nm_splu_numeric(_dt(A_data), rows, _ptr(Mt_data), _ptr(Mt_indices), _ptr(Mt_indptr),
+                                     _ptr(work), nbytes.value, 0, stream), "nm_splu_numeric")
         M_data = csr_transpose_backward(Mt_data, Mt_to_M)
     return [M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]
 

@@ -133,3 +133,48 @@ def test_errors(dev):
         mirror.splu(5, 7, *to_dev(dev, d, i, p))
     with pytest.raises(RuntimeError, match="HIP devices only"):
         mirror.splu(5, 5, torch.ones(5), torch.arange(5), torch.arange(6))
+
+
+def test_pattern_is_computed_once_per_structure(dev):
+    d, i, p, (n, _) = G.poisson2d(12, np.float64, 1)
+    D, I, P = to_dev(dev, d, i, p)
+    for ext in (numml_amd.load_compiled(), mirror):
+        ext.clear_plan_cache()
+        a = ext.splu(n, n, D, I, P)
+        b = ext.splu(n, n, D * 2.0, I, P)
+        for k in (1, 2, 4, 5):                       # the index tensors are shared between the calls
+            assert a[k].data_ptr() == b[k].data_ptr()
+        assert_same(host(b[0]), oracle.splu(n, n, d * 2.0, i, p)[0], "values follow the new data")
+        a[1][0] = a[1][0]                            # an in-place edit invalidates the cached pattern
+        c = ext.splu(n, n, D, I, P)
+        assert c[1].data_ptr() != a[1].data_ptr()
+        assert_same(host(c[0]), host(a[0]), "rebuilt")
+
+
+def test_numeric_phase_gives_up_instead_of_waiting_forever(dev):
+    # a poll limit of 1 on a matrix whose columns form one dependency chain: the kernel must
+    # leave and the call report it (or, if every dependency happened to be ready, succeed)
+    import ctypes
+    from numml_amd import _lib
+    L = _lib.lib()
+    d, i, p, (n, _) = G.tridiag(700, np.float64)
+    M = mirror.splu(n, n, *to_dev(dev, d, i, p))
+    want = host(M[3])
+    As = sps.csr_matrix((d, i, p), shape=(n, n)).T.tocsr()      # A^T on its own pattern: tridiagonal has no fill
+    As.sort_indices()
+    Td, Ti, Tp = to_dev(dev, As.data, As.indices.astype(np.int64), As.indptr.astype(np.int64))
+    nbytes = ctypes.c_size_t(0)
+    assert L.nm_splu_numeric_bytes(n, ctypes.byref(nbytes)) == 0
+    work = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    rc = L.nm_splu_numeric(1, n, Td.data_ptr(), Ti.data_ptr(), Tp.data_ptr(), work.data_ptr(), nbytes.value, 1,
+                           stream)
+    if rc != 0:
+        assert b"polls" in L.nm_last_error()
+    else:
+        assert_same(host(Td), want, "factors")
+    # the device is fine afterwards
+    Td2 = to_dev(dev, As.data)[0]
+    assert L.nm_splu_numeric(1, n, Td2.data_ptr(), Ti.data_ptr(), Tp.data_ptr(), work.data_ptr(), nbytes.value, 0,
+                             stream) == 0
+    assert_same(host(Td2), want, "factors after the failed call")
