@@ -62,6 +62,8 @@ struct nm_sptrsv_plan {
         int32_t q0, q1;  // slots they cover
         bool wide;       // one level, many workgroups
         int32_t block;   // lanes of the single-workgroup launch (narrow runs)
+        int32_t width = 0;          // rows of its widest level
+        int32_t group[2] = {0, 0};  // per direction: lanes that share a row (0: one lane per row)
     };
     std::vector<Launch> launches;
 };
@@ -408,6 +410,122 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
     }
 }
 
+// ---- long rows: several lanes per row ---------------------------------------------
+//
+// The kernels above give a row to one lane, which walks its dependencies one after the
+// other: right for the handful of entries a row of a sparse triangle usually has, but the
+// factors of a direct solve have rows of dozens to hundreds of entries in levels of one or
+// a few rows, and the level then lasts as long as that serial walk.  Here G lanes share a
+// row: each multiplies every G-th dependency, the partial sums are added across the group
+// (in double, so the rounding differs from the serial order by a few units in the last
+// place of a double), and the group's first lane finishes the row.  The first G
+// dependencies of a row come through the same two-stage register pipeline as above.
+struct GVals { Meta m; int32_t ds; double v, dv, bv; };
+
+template <int G> __device__ __forceinline__ Meta load_gmeta(const SolveArgs &a, const Bounds &b) {
+    Meta m;
+    m.q = b.qb + (int)threadIdx.x / G;
+    m.live = m.q < b.qe;
+    const int qs = m.live ? m.q : 0;
+    m.dlo = a.dptr[qs];
+    m.n = a.dptr[qs + 1] - m.dlo;
+    return m;
+}
+
+template <int G> __device__ __forceinline__ GVals load_gvals(const SolveArgs &a, const Meta &m) {
+    GVals v;
+    v.m = m;
+    const int sub = (int)threadIdx.x & (G - 1);
+    const int32_t at = (m.live && sub < m.n) ? m.dlo + sub : 0;
+    v.ds = a.dslot[at];
+    v.v = a.w.coef[at];
+    const int qs = m.live ? m.q : 0;
+    v.dv = a.w.dg[qs];
+    v.bv = a.w.rhs[qs];
+    return v;
+}
+
+template <int G> __device__ __forceinline__ double group_total(double v) {
+    if (G == 64) return nm::wave_sum(v);
+    v += nm::dpp_move<0xB1>(v);    // quad_perm [1,0,3,2]
+    v += nm::dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]
+    v += nm::dpp_move<0x124>(v);   // row_ror 4
+    v += nm::dpp_move<0x128>(v);   // row_ror 8: every lane of the 16-lane row holds the row's sum
+    return v;
+}
+
+template <int G, int DEPTH>
+__global__ __launch_bounds__(kNarrow) void sptrsv_group_kernel(SolveArgs a, int l0, int count, int step, int qlo,
+                                                               int qhi) {
+    static_assert(G == 16 || G == 64, "group sums are written for a DPP row or a wavefront");
+    __shared__ double ring[kRing];
+    __shared__ int32_t s_lp[kMaxLevels + 1];
+    const int lmin = step > 0 ? l0 : l0 - (count - 1);
+    for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
+    __syncthreads();
+    const int sub = (int)threadIdx.x & (G - 1), ngroups = (int)blockDim.x / G;
+
+    // x of slot ds as seen from slot q: the ring holds what this launch solved recently
+    auto solved = [&](int32_t ds, int q) {
+        const int dist = ds > q ? ds - q : q - ds;
+        return (ds >= qlo && ds < qhi && dist < kRingSafe) ? ring[ds & (kRing - 1)] : a.w.xs[ds];
+    };
+
+    Meta qm[DEPTH];
+    GVals qv[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) qm[d] = load_gmeta<G>(a, load_bounds(s_lp, d, count, l0, step, lmin));
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) qv[d] = load_gvals<G>(a, qm[d]);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) qm[d] = load_gmeta<G>(a, load_bounds(s_lp, DEPTH + d, count, l0, step, lmin));
+
+    for (int it0 = 0; it0 < count; it0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int it = it0 + d;
+            if (it >= count) break;   // uniform over the workgroup
+            const GVals cur = qv[d];
+            qv[d] = load_gvals<G>(a, qm[d]);
+            qm[d] = load_gmeta<G>(a, load_bounds(s_lp, it + 2 * DEPTH, count, l0, step, lmin));
+            const int qe = s_lp[l0 + it * step - lmin + 1];
+
+            // this group's first row of the level: operands already in registers
+            {
+                const int q = cur.m.q, n = cur.m.live ? cur.m.n : 0;
+                double acc = sub < n ? cur.v * solved(cur.ds, q) : 0.;
+                for (int e = sub + G; e < n; e += G) {
+                    const int32_t at = cur.m.dlo + e;
+                    acc += a.w.coef[at] * solved(a.dslot[at], q);
+                }
+                acc = group_total<G>(acc);
+                if (cur.m.live && sub == 0) {
+                    double xi = cur.bv - acc;
+                    if (!a.unit) xi /= cur.dv;
+                    ring[q & (kRing - 1)] = xi;
+                    a.w.xs[q] = xi;
+                }
+            }
+            // a level with more rows than groups: the rest straight from memory
+            for (int q0 = cur.m.q + ngroups; q0 - (int)threadIdx.x / G < qe; q0 += ngroups) {
+                const bool live = q0 < qe;
+                const int q = live ? q0 : 0;
+                const int32_t dlo = a.dptr[q], n = live ? a.dptr[q + 1] - dlo : 0;
+                double acc = 0.;
+                for (int e = sub; e < n; e += G) acc += a.w.coef[dlo + e] * solved(a.dslot[dlo + e], q);
+                acc = group_total<G>(acc);
+                if (live && sub == 0) {
+                    double xi = a.w.rhs[q] - acc;
+                    if (!a.unit) xi /= a.w.dg[q];
+                    ring[q & (kRing - 1)] = xi;
+                    a.w.xs[q] = xi;
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // ---- fixed-width (ELLPACK) variant of the single-workgroup kernel -----------------
 //
 // When no row has more than 8 dependencies, the packed triangle is also kept with a
@@ -631,7 +749,17 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
                 hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
             else if (pre == 8)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
-            else if (maxdep <= 2)
+            else if (L.group[dirn] > 0) {
+                // several lanes per row: as many groups as the widest level has rows, within one workgroup
+                const int G = L.group[dirn];
+                int groups = 1;
+                while (groups < L.width && groups * G < kNarrow) groups *= 2;
+                const int lanes = groups * G < 64 ? 64 : groups * G;
+                if (G == 64)
+                    hipLaunchKernelGGL((sptrsv_group_kernel<64, 2>), dim3(1), dim3(lanes), 0, s, a, l0, count, step, L.q0, L.q1);
+                else
+                    hipLaunchKernelGGL((sptrsv_group_kernel<16, 2>), dim3(1), dim3(lanes), 0, s, a, l0, count, step, L.q0, L.q1);
+            } else if (maxdep <= 2)
                 hipLaunchKernelGGL((sptrsv_ring_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             else if (maxdep <= 4)
                 hipLaunchKernelGGL((sptrsv_ring_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
@@ -800,6 +928,26 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         p->launches.push_back({l, l + 1, lp[l], lp[l + 1], true, kBlock});
     }
     if (run0 >= 0) push_narrow(run0, p->nlevels);
+    // Rows long enough to be shared by several lanes: decided per launch and direction from the
+    // mean number of dependencies of its rows, where no fixed-width layout serves the direction.
+    for (auto &L : p->launches) {
+        L.width = 0;
+        for (int32_t l = L.l0; l < L.l1; ++l) L.width = L.width > lp[l + 1] - lp[l] ? L.width : lp[l + 1] - lp[l];
+    }
+    for (int d = 0; d < 2; ++d) {
+        if (p->max_deps[d] <= 8) continue;
+        std::vector<int32_t> dptr_h((size_t)rows + 1);
+        if (hipMemcpyAsync(dptr_h.data(), p->dir[d].dptr, dptr_h.size() * 4, hipMemcpyDeviceToHost, s) !=
+                hipSuccess ||
+            hipStreamSynchronize(s) != hipSuccess)
+            return bail(nm::fail(NM_ERR_HIP, "reading the dependency counts back failed"));
+        for (auto &L : p->launches) {
+            if (L.wide || L.q1 <= L.q0) continue;
+            const double mean = double(dptr_h[L.q1] - dptr_h[L.q0]) / double(L.q1 - L.q0);
+            if (mean >= 40. && L.width <= 16) L.group[d] = 64;
+            else if (mean >= 12. && L.width <= 256) L.group[d] = 16;
+        }
+    }
     // fixed-width copies of the packed triangles, with the ring-reach mark per dependency
     std::vector<int32_t> level_launch((size_t)p->nlevels + 1, -1);
     for (size_t li = 0; li < p->launches.size(); ++li)
