@@ -193,7 +193,8 @@ constexpr int kLuWavesPerBlock = kBlock / 64;
 constexpr int64_t kLuSpinLimit = 1 << 24;  // polls of one dependency flag before giving up
 
 struct LuFlow {
-    int64_t *done;   // [cols] 0 = pending, else 1 + position of the column's first entry below the diagonal
+    int64_t *below;  // [cols] position of the column's first entry below the diagonal
+    int32_t *done;   // [cols] 0 = pending, 1 = the column holds its final values
     int32_t *ctl;    // [0] next ticket, [1] failure
 };
 
@@ -206,7 +207,8 @@ size_t flow_layout(int64_t cols, void *base, LuFlow *F) {
     };
     LuFlow f;
     f.ctl = (int32_t *)take(64);
-    f.done = (int64_t *)take((size_t)(cols > 0 ? cols : 1) * 8);
+    f.done = (int32_t *)take((size_t)(cols > 0 ? cols : 1) * 4);
+    f.below = (int64_t *)take((size_t)(cols > 0 ? cols : 1) * 8);
     if (F) *F = f;
     return off;
 }
@@ -226,11 +228,29 @@ struct OwnColumn {
     }
 };
 
+// below[k] = position of the first entry of column k with a row index > k.
+__global__ void lu_below_kernel(int64_t cols, const int64_t *__restrict__ indices,
+                                const int64_t *__restrict__ indptr, int64_t *__restrict__ below) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < cols; k += stride) {
+        int64_t lo = indptr[k], hi = indptr[k + 1];
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (indices[mid] <= k) lo = mid + 1; else hi = mid;
+        }
+        below[k] = lo;
+    }
+}
+
 // Returns false when a dependency did not arrive within the poll limit (or another wavefront failed).
+// Everything about a pivot that the structure alone decides -- which entries of column i lie below
+// its diagonal and where their rows sit in this column -- is looked up before the wait for column i,
+// so that what follows the arrival of the flag is one load, one multiply and one subtraction.
 template <typename T, bool IN_LDS>
 __device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T, IN_LDS> &own,
-                          const int64_t *__restrict__ indices, const int64_t *__restrict__ indptr, T *values,
-                          int64_t *done, int32_t *ctl, int64_t spin_limit, int lane) {
+                          const int64_t *__restrict__ indices, const int64_t *__restrict__ indptr,
+                          const int64_t *__restrict__ below_of, T *values, int32_t *done, int32_t *ctl,
+                          int64_t spin_limit, int lane) {
     if (IN_LDS) {
         for (int64_t e = lane; e < len; e += 64) {
             own.s_rows[e] = (int32_t)indices[pb + e];
@@ -238,58 +258,63 @@ __device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T,
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
+    // position in this column of row j, searched among the entries after e; -1 when not stored
+    auto find = [&](int64_t e, int64_t j) {
+        int64_t lo = e + 1, hi = len;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (own.row(mid) < j) lo = mid + 1; else hi = mid;
+        }
+        return (lo < len && own.row(lo) == j) ? lo : (int64_t)-1;
+    };
     int64_t e = 0;
     for (; e < len; ++e) {
         const int64_t i = own.row(e);
         if (i >= k) break;
-        // column i: wait for it, then its entries below the diagonal are [ls, ie)
-        int64_t flag = 0, polls = 0;
-        for (;;) {
-            flag = __hip_atomic_load(done + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (flag != 0) break;
+        const int64_t ls = below_of[i], ie = indptr[i + 1];
+        const int64_t t_first = ls + lane;                       // this lane's entry of column i, first round
+        const int64_t at_first = t_first < ie ? find(e, indices[t_first]) : (int64_t)-1;
+        int64_t polls = 0;
+        while (__hip_atomic_load(done + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
             if (++polls > spin_limit || __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
                 return false;
-            __builtin_amdgcn_s_sleep(4);
+            __builtin_amdgcn_s_sleep(1);
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // the loads below stay after the flag
-        const int64_t ls = flag - 1, ie = indptr[i + 1];
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // the value loads below stay after the flag
         const T m_ik = own.val(e);
-        for (int64_t t0 = ls; t0 < ie; t0 += 64) {
+        if (at_first >= 0) {
+            const T m_ji = __hip_atomic_load(values + t_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const T prod = m_ji * m_ik;
+            own.set(at_first, own.val(at_first) - prod);
+        }
+        for (int64_t t0 = ls + 64; t0 < ie; t0 += 64) {          // columns with more than 64 entries below
             const int64_t t = t0 + lane;
-            if (t < ie) {
-                const int64_t j = indices[t];
+            const int64_t at = t < ie ? find(e, indices[t]) : (int64_t)-1;
+            if (at >= 0) {
                 const T m_ji = __hip_atomic_load(values + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                int64_t lo = e + 1, hi = len;   // row j among the later entries of this column
-                while (lo < hi) {
-                    const int64_t mid = (lo + hi) >> 1;
-                    if (own.row(mid) < j) lo = mid + 1; else hi = mid;
-                }
-                if (lo < len && own.row(lo) == j) {
-                    const T prod = m_ji * m_ik;
-                    own.set(lo, own.val(lo) - prod);
-                }
+                const T prod = m_ji * m_ik;
+                own.set(at, own.val(at) - prod);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
-    int64_t below = e;   // first entry below the diagonal
     if (e < len && own.row(e) == k) {
-        below = e + 1;
         const T d = own.val(e);
-        for (int64_t q = below + lane; q < len; q += 64) own.set(q, own.val(q) / d);
+        for (int64_t q = e + 1 + lane; q < len; q += 64) own.set(q, own.val(q) / d);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
     if (IN_LDS)
         for (int64_t q = lane; q < len; q += 64) values[pb + q] = own.s_vals[q];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    if (lane == 0) __hip_atomic_store(done + k, pb + below + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(done + k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return true;
 }
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void lu_flow_kernel(int64_t cols, const int64_t *__restrict__ indices,
-                                                         const int64_t *__restrict__ indptr, T *values,
-                                                         int64_t *done, int32_t *ctl, int64_t spin_limit) {
+                                                         const int64_t *__restrict__ indptr,
+                                                         const int64_t *__restrict__ below, T *values,
+                                                         int32_t *done, int32_t *ctl, int64_t spin_limit) {
     __shared__ int32_t s_rows[kLuWavesPerBlock][kLuCap];
     __shared__ T s_vals[kLuWavesPerBlock][kLuCap];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -303,10 +328,10 @@ __global__ __launch_bounds__(kBlock) void lu_flow_kernel(int64_t cols, const int
         bool ok;
         if (len <= kLuCap) {
             const OwnColumn<T, true> own{s_rows[w], s_vals[w], nullptr, nullptr};
-            ok = lu_column<T, true>(k, pb, len, own, indices, indptr, values, done, ctl, spin_limit, lane);
+            ok = lu_column<T, true>(k, pb, len, own, indices, indptr, below, values, done, ctl, spin_limit, lane);
         } else {
             const OwnColumn<T, false> own{nullptr, nullptr, indices + pb, values + pb};
-            ok = lu_column<T, false>(k, pb, len, own, indices, indptr, values, done, ctl, spin_limit, lane);
+            ok = lu_column<T, false>(k, pb, len, own, indices, indptr, below, values, done, ctl, spin_limit, lane);
         }
         if (!ok) {
             if (lane == 0) atomicExch(ctl + 1, 1);
@@ -421,16 +446,22 @@ extern "C" int nm_splu_numeric(nm_dtype dt, int64_t cols, void *Mt_data, const i
         return nm::fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace_bytes, need);
     hipStream_t s = nm::as_stream(stream);
     if (int rc = nm::fill_async(F.ctl, 16, (int32_t)0, s)) return rc;
-    if (int rc = nm::fill_async(F.done, cols, (int64_t)0, s)) return rc;
+    if (int rc = nm::fill_async(F.done, cols, (int32_t)0, s)) return rc;
+    {
+        int64_t g = nm::ceil_div(cols, kBlock);
+        hipLaunchKernelGGL(lu_below_kernel, dim3((unsigned)(g > 65536 ? 65536 : g)), dim3(kBlock), 0, s, cols,
+                           Mt_indices, Mt_indptr, F.below);
+        NM_LAUNCH_CHECK("lu_below_kernel");
+    }
     int64_t grid = nm::ceil_div(cols, kLuWavesPerBlock);
     if (grid > 1024) grid = 1024;
     const int64_t limit = poll_limit > 0 ? poll_limit : kLuSpinLimit;
     if (dt == NM_F32)
         hipLaunchKernelGGL(lu_flow_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, Mt_indices,
-                           Mt_indptr, (float *)Mt_data, F.done, F.ctl, limit);
+                           Mt_indptr, F.below, (float *)Mt_data, F.done, F.ctl, limit);
     else
         hipLaunchKernelGGL(lu_flow_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, Mt_indices,
-                           Mt_indptr, (double *)Mt_data, F.done, F.ctl, limit);
+                           Mt_indptr, F.below, (double *)Mt_data, F.done, F.ctl, limit);
     NM_LAUNCH_CHECK("lu_flow_kernel");
     int32_t ctl_h[2] = {0, 0};
     if (hipMemcpyAsync(ctl_h, F.ctl, sizeof(ctl_h), hipMemcpyDeviceToHost, s) != hipSuccess ||
