@@ -16,13 +16,14 @@ on):
   spmm    fp32 SpMM fwd+bwd, power-law 1M x 1M, ~15M nnz, 64 dense columns
   spgemm  fp64 hash SpGEMM A@A fwd+bwd, 3-D Laplacian 128^3
   sptrsv  fp64 triangular solve fwd+bwd, tril(Poisson 1024^2), 2047 levels
+  spsolve fp64 direct solve fwd+bwd (LU without pivoting + four triangular solves), Poisson 64^2
   lincomb    fp32 A - B (splincomb) + its backward, both on the spmv matrix pattern
   transpose  fp32 explicit CSR transpose + its backward on the spmv matrix
   copy    256 MiB device copy (counter calibration / practical bandwidth ceiling)
 
 ``value`` is algorithmic bytes per step / time per step (GB/s) for spmv/spmm,
 GFLOP/s (2 flop per scalar product, forward only counted) for spgemm and
-milliseconds per forward solve for sptrsv.
+milliseconds per step for sptrsv and spsolve.
 """
 import argparse
 import json
@@ -158,7 +159,7 @@ class SpMM(Workload):
                           + cols * n * s)
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
-        self.dominant_name = ("spdmm_bwd_kernel (grad_A) + spdmm_fwd_kernel on the transposed plan (grad_B)"
+        self.dominant_name = ("spdmm_bwd_kernel (grad_A) + spdmm_fwd_flat_kernel on the transposed plan (grad_B)"
                               if _binding.backward_mode() == "planned"
                               else "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)")
         self.config = {"workload": "spmm_fwd_bwd_f32_powerlaw_1M_n64", "rows": rows, "nnz": nnz,
@@ -445,7 +446,7 @@ class SpSolve(Workload):
         self.dominant_bytes = self.nnz * (s + 8) + 2 * self.nnzM * (s + 8) + 3 * (rows + 1) * 8
         self.bytes_per_step = self.dominant_bytes + 4 * (self.nnzM * (s + 8) + (rows + 1) * 8 + 2 * rows * s) \
             + self.nnz * s
-        self.dominant_name = "splu: lu_rows_kernel (count, fill), transpose, lu_numeric_kernel per level run"
+        self.dominant_name = "splu on a cached pattern: lu_values_kernel, transpose_expand_kernel, lu_flow_kernel, transpose_scatter_kernel"
         self.config = {"workload": f"spsolve_fwd_bwd_f64_poisson2d_{n}", "rows": rows, "nnz": self.nnz,
                        "nnz_LU": self.nnzM, "binding": _binding.name}
 
