@@ -66,6 +66,9 @@ def test_mirror_has_the_reference_signatures():
         "sptrsv_forward": ["A_rows", "A_cols", "A_data", "A_indices", "A_indptr", "lower", "unit", "b"],
         "sptrsv_backward": ["grad_x", "x", "A_rows", "A_cols", "A_data", "A_indices", "A_indptr",
                             "lower", "unit", "b"],
+        "splu": ["A_rows", "A_cols", "A_data", "A_indices", "A_indptr"],                   # :107-111
+        "spsolve_backward": ["grad_x", "x", "A_rows", "A_cols", "Mt_data", "Mt_indices", "Mt_indptr",
+                             "A_data", "A_indices", "A_indptr"],                            # :113-118
     }
     for name, params in want.items():
         assert list(inspect.signature(getattr(ext, name)).parameters) == params, name
@@ -90,9 +93,13 @@ def test_cpu_tensors_are_refused_not_computed():
 def test_compiled_extension_exports_the_reference_module():
     import numml_amd
     cpp = numml_amd.load_compiled()
-    for name in ("spgemv_forward", "spgemv_backward", "spgemm_forward", "spgemm_backward", "spdmm_forward",
-                 "spdmm_backward", "sptrsv_forward", "sptrsv_backward"):     # cpp/sparse_csr.cpp:307-319
+    names = [f"{op}_{d}" for op in ("spgemv", "spgemm", "csr_transpose", "splincomb", "spdmm", "sptrsv",
+                                    "csr_to_dense", "csr_row_sum", "csr_extract_diagonal")
+             for d in ("forward", "backward")] + ["splu", "spsolve_backward"]      # cpp/sparse_csr.cpp:307-319
+    assert len(names) == 20
+    for name in names:
         assert callable(getattr(cpp, name)), name
+        assert callable(getattr(ext, name)), name
     d, i, p = torch.ones(3), torch.tensor([0, 1, 2]), torch.tensor([0, 1, 2, 3])
     with pytest.raises(RuntimeError, match="HIP devices only"):
         cpp.spgemv_forward(3, 3, d, i, p, torch.ones(3))
