@@ -436,13 +436,30 @@ class SparseCSRTensor(object):
         return sptodense.apply(self.shape, self.data, self.indices, self.indptr)
 
     def to_coo(self):
-        """(values, rows, cols) of the stored entries."""
-        return self.data, self.row_indices, self.indices
+        """torch's sparse COO tensor of the stored entries; gradients on the values carry over
+        (numml/sparse/_csr.py:753-769)."""
+        return torch.sparse_coo_tensor(torch.stack((self.row_indices, self.indices)), self.data, self.shape,
+                                       device=self.device)
+
+    def tocoo(self):
+        """SciPy COO matrix (numml/sparse/_csr.py:771-788); gradient information is dropped."""
+        import scipy.sparse as sp
+        return sp.coo_matrix((self.data.detach().cpu().numpy(),
+                              (self.row_indices.cpu().numpy().astype("int32"),
+                               self.indices.cpu().numpy().astype("int32"))), shape=self.shape)
 
     def to_scipy_csr(self):
         import scipy.sparse as sp
         return sp.csr_matrix((self.data.detach().cpu().numpy(), self.indices.cpu().numpy(),
                               self.indptr.cpu().numpy()), shape=self.shape)
+
+    tocsr = to_scipy_csr
+
+    def conjugate(self):
+        """Element-wise complex conjugation (numml/sparse/_csr.py:1041-1061)."""
+        return SparseCSRTensor((self.data.conj(), self.indices, self.indptr), self.shape)
+
+    conj = conjugate
 
     def to(self, device):
         return SparseCSRTensor((self.data.to(device), self.indices.to(device),
@@ -523,6 +540,24 @@ def eye(N, k=0, dtype=torch.float32, device=None):
     indptr[1:] = torch.cumsum(counts, 0)
     out = SparseCSRTensor((torch.ones(n, dtype=dtype), cols, indptr), (N, N), clone=False)
     return out if device is None else out.to(device)
+
+
+def spouter(x, y):
+    """x y^T on the pattern of the nonzeros of x times the nonzeros of y
+    (numml/sparse/_csr.py:511-538)."""
+    x_nz = torch.nonzero(x).flatten()
+    y_nz = torch.nonzero(y).flatten()
+    row, col = torch.meshgrid(x_nz, y_nz, indexing="ij")
+    row, col = row.flatten(), col.flatten()
+    return SparseCSRTensor((x[row] * y[col], (row, col)), shape=(len(x), len(y)))
+
+
+def unpack_csr(A):
+    return A.data, A.indices, A.indptr, A.shape
+
+
+def repack_csr(A_data, A_indices, A_indptr, A_shape):
+    return SparseCSRTensor((A_data, A_indices, A_indptr), A_shape, clone=False)
 
 
 def diag(x, k=0):
