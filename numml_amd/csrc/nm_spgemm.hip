@@ -134,22 +134,6 @@ __device__ __forceinline__ int32_t merge_sum(int32_t v) {
     return v;
 }
 
-// True when some merge group of the wavefront has three or more of its lanes set
-// in `lanes` (a ballot).  Scalar work: the two parities are separated, which
-// leaves each group's bits at the even positions of a 16-bit field; the lowest
-// set bit of every field is cleared twice (bit 15, free, stops the borrow) and
-// anything left means three.
-__device__ __forceinline__ bool merge_three_hits(unsigned long long lanes) {
-    constexpr unsigned long long kEven = 0x5555555555555555ull, kLow = 0x0001000100010001ull,
-                                 kTop = 0x8000800080008000ull;
-    unsigned long long e = lanes & kEven, o = (lanes >> 1) & kEven;
-    e &= (e | kTop) - kLow;
-    o &= (o | kTop) - kLow;
-    e &= (e | kTop) - kLow;
-    o &= (o | kTop) - kLow;
-    return (e | o) != 0;
-}
-
 constexpr int kMergeRows = kBlock / 8;   // rows of A per workgroup pass
 constexpr int kMergeStride = kBlock + 1; // slot stride of the staged B rows (odd: slots of one lane fall in different banks)
 
