@@ -200,7 +200,8 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
 // wavefront owns 64 consecutive stored entries whatever rows they belong to
 // (every entry costs the same), finds its first row by bisection and walks on;
 // gathers go out eight at a time and the dot products are reduced with DPP adds.
-template <typename T>
+// FAST: grad_A only and n <= 64 (one column tile), which allows the pipelined loop below.
+template <typename T, bool FAST>
 __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
     int64_t rows, int64_t nnz, const T *__restrict__ data, const int64_t *__restrict__ indices,
     const int64_t *__restrict__ indptr, const T *__restrict__ B, int64_t ldb,
@@ -259,15 +260,22 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
                     row_end = end_of(row);
                 }
                 rw[u] = row;
-                col[u] = __shfl(mycol, j, kWave);
+                // a scalar read, so that the row addresses below are scalar too and the gathers
+                // share one vector register of column offsets
+                const int js = __builtin_amdgcn_readfirstlane(j);
+                const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(mycol & 0xffffffffll), js);
+                const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(mycol >> 32), js);
+                col[u] = (int64_t)(((unsigned long long)hi << 32) | lo);
             }
         };
         auto fetch = [&](const int64_t (&col)[kBatch], const int64_t (&rw)[kBatch], int64_t c, bool live,
                          T (&gv)[kBatch], T (&bv)[kBatch]) {
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
-                gv[u] = gC[rw[u] * ldg + (live ? c : 0)];
-                bv[u] = grad_A ? B[col[u] * ldb + (live ? c : 0)] : T(0);
+                const T *__restrict__ grow = gC + rw[u] * ldg;
+                const T *__restrict__ brow = B + col[u] * ldb;
+                gv[u] = grow[live ? c : 0];
+                bv[u] = grad_A ? brow[live ? c : 0] : T(0);
             }
         };
         // Sums over the wavefront of kBatch (= 8) lane-wise products at once.  Three
@@ -297,7 +305,7 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
 #pragma unroll
                 for (int u = 0; u < kBatch; ++u) {
                     if (j0 + u >= cnt) break;
-                    const T av = __shfl(myval, j0 + u, kWave);   // all lanes take part in the broadcast
+                    const T av = nm::read_lane(myval, __builtin_amdgcn_readfirstlane(j0 + u));
                     if (live) nm::atomic_add(grad_B + col[u] * ldgb + c, av * gv[u]);
                 }
             }
@@ -309,15 +317,47 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
                 if ((lane >> 3) == (j0 >> 3)) mydot += t;   // lane j0 + u takes vector u
             }
         };
-        for (int j0 = 0; j0 < cnt; j0 += kBatch) {
-            int64_t col[kBatch], rw[kBatch];
-            locate(j0, col, rw);
-            for (int64_t c0 = 0; c0 < n; c0 += kWave) {
-                const int64_t c = c0 + lane;
-                const bool live = c < n;
-                T bv[kBatch], gv[kBatch];
-                fetch(col, rw, c, live, gv, bv);
-                consume(j0, col, c, live, gv, bv);
+        if (FAST) {
+            // grad_A alone, at most 64 dense columns: one column tile per batch, so a batch is
+            // just its 16 operand vectors.  Two batches are kept in flight: the gathers of the
+            // next batch are issued before the current one is reduced.  The two stages
+            // alternate in place (copying a stage whose loads are still in flight would wait
+            // for them), and the scalar rows and columns of a batch die with its address
+            // arithmetic, which keeps them out of vector registers.
+            const bool live = lane < n;
+            auto issue = [&](int j0, T (&gv)[kBatch], T (&bv)[kBatch]) {
+                int64_t col[kBatch], rw[kBatch];
+                locate(j0, col, rw);
+                fetch(col, rw, lane, live, gv, bv);
+            };
+            auto finish = [&](int j0, const T (&gv)[kBatch], const T (&bv)[kBatch]) {
+                T p[kBatch];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) p[u] = live ? gv[u] * bv[u] : T(0);
+                const T t = reduce8(p);
+                if ((lane >> 3) == (j0 >> 3)) mydot += t;
+            };
+            T gva[kBatch], bva[kBatch], gvb[kBatch], bvb[kBatch];
+            issue(0, gva, bva);
+            for (int j0 = 0;; j0 += 2 * kBatch) {
+                if (j0 + kBatch < cnt) issue(j0 + kBatch, gvb, bvb);
+                finish(j0, gva, bva);
+                if (j0 + kBatch >= cnt) break;
+                if (j0 + 2 * kBatch < cnt) issue(j0 + 2 * kBatch, gva, bva);
+                finish(j0 + kBatch, gvb, bvb);
+                if (j0 + 2 * kBatch >= cnt) break;
+            }
+        } else {
+            for (int j0 = 0; j0 < cnt; j0 += kBatch) {
+                int64_t col[kBatch], rw[kBatch];
+                locate(j0, col, rw);
+                for (int64_t c0 = 0; c0 < n; c0 += kWave) {
+                    const int64_t c = c0 + lane;
+                    const bool live = c < n;
+                    T bv[kBatch], gv[kBatch];
+                    fetch(col, rw, c, live, gv, bv);
+                    consume(j0, col, c, live, gv, bv);
+                }
             }
         }
         if (grad_A && lane < cnt) grad_A[k] = mydot;
@@ -393,14 +433,17 @@ int backward_impl(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const vo
     if (rows == 0 || nnz == 0 || n == 0 || (!grad_A && !grad_B)) return NM_OK;
     NM_REQUIRE(B != nullptr && gC != nullptr, "B or gC is null");
     NM_REQUIRE(ldb >= n && ldg >= n, "row stride smaller than the row");
-    if (dt == NM_F32)
-        hipLaunchKernelGGL(spdmm_bwd_kernel<float>, dim3(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock)),
-                           dim3(kBlock), 0, s, rows, nnz, (const float *)data, indices, indptr, (const float *)B, ldb, (const float *)gC,
-                           ldg, n, (float *)grad_A, (float *)grad_B, ldgb, chunk_row);
-    else
-        hipLaunchKernelGGL(spdmm_bwd_kernel<double>, dim3(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock)),
-                           dim3(kBlock), 0, s, rows, nnz, (const double *)data, indices, indptr, (const double *)B, ldb, (const double *)gC,
-                           ldg, n, (double *)grad_A, (double *)grad_B, ldgb, chunk_row);
+    const dim3 grid(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock));
+    const bool fast = grad_A && !grad_B && n <= kWave;
+#define NM_SDDMM(T, FAST)                                                                                         \
+    hipLaunchKernelGGL((spdmm_bwd_kernel<T, FAST>), grid, dim3(kBlock), 0, s, rows, nnz, (const T *)data, indices, \
+                       indptr, (const T *)B, ldb, (const T *)gC, ldg, n, (T *)grad_A, (T *)grad_B, ldgb, chunk_row)
+    if (dt == NM_F32) {
+        if (fast) NM_SDDMM(float, true); else NM_SDDMM(float, false);
+    } else {
+        if (fast) NM_SDDMM(double, true); else NM_SDDMM(double, false);
+    }
+#undef NM_SDDMM
     NM_LAUNCH_CHECK("spdmm_bwd_kernel");
     return NM_OK;
 }
