@@ -83,7 +83,10 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
     const IDX *__restrict__ indptr, const int32_t *__restrict__ perm, const T *__restrict__ B, int64_t ldb,
     int64_t n, T *__restrict__ C, int64_t ldc) {
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    // (the wavefront index is the same in every lane: telling the compiler so keeps everything
+    // derived from it -- row ranges, loop bounds, addresses -- in scalar registers and the
+    // control flow free of execution-mask bookkeeping)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     // The first `long_blocks` workgroups look for long rows, kScoutRows rows each, and
     // share every one they find among their wavefronts (contiguous parts, partial sums added
     // in wavefront order: deterministic, equal to the serial sum to rounding).  They come
@@ -136,22 +139,37 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
         return (int64_t)((hi << 32) | (lo & 0xffffffffll));
     };
     const int64_t begin = ptr_of(0), end = ptr_of(nr);
+    // The wavefronts of a workgroup share one CU, which issues about one scalar and one
+    // vector instruction per cycle: with ~35 instructions per entry (64-bit row addresses on
+    // the scalar unit, a row-end comparison and two bounds checks per entry) this walk was
+    // bound by instruction issue, not by its gathers.  So everything that can be done once
+    // per 64 entries is done there, by the lanes: the byte offset of each entry's row of B,
+    // and a mask of the entries that end a row.  Per entry that leaves two lane reads and
+    // one scalar add for the address, one lane read and one multiply-add for the term, and
+    // a bit test for the row boundary.
+    const int64_t row_bytes = ldb * (int64_t)sizeof(T);
     for (int64_t c0 = 0; c0 < n; c0 += kWave) {
         const int64_t c = c0 + lane;
         const bool live = c < n;
-        const T *__restrict__ Bc = B + (live ? c : 0);
-        int r = 0;                         // current row (relative), its end, whether it is computed here
-        int64_t row_end = ptr_of(1);
-        bool mine = row_end - begin <= kSplitRow;
+        const char *__restrict__ Bc = reinterpret_cast<const char *>(B + (live ? c : 0));
+        int r = 0;   // current row (relative), its range, whether it is computed here
+        int64_t row_begin = begin, row_end = ptr_of(1);
+        bool mine = row_end - row_begin <= kSplitRow;
         T acc = T(0);
         auto next_row = [&]() {
             if (mine && live) C[(r0 + r) * ldc + c] = acc;
             acc = T(0);
             ++r;
-            const int64_t rb = row_end;
+            row_begin = row_end;
             row_end = ptr_of(r + 1 <= nr ? r + 1 : nr);
-            mine = row_end - rb <= kSplitRow;
+            mine = row_end - row_begin <= kSplitRow;
         };
+        // leaves the current row and the empty rows after it (stored as zeros)
+        auto close_row = [&]() {
+            next_row();
+            while (r < nr && row_end == row_begin) next_row();
+        };
+        while (r < nr && row_end == row_begin) next_row();   // empty rows at the head
         int64_t kb = begin;
         auto fetch = [&](int64_t at, int64_t &col, T &val) {
             const int64_t k = at + lane < end ? at + lane : (end > begin ? end - 1 : 0);
@@ -161,37 +179,60 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
         int64_t mycol, nextcol;
         T myval, nextval;
         fetch(kb, mycol, myval);
-        while (kb < end) {
-            // a long row is not computed here: jump over what is left of it
-            while (r < nr && kb >= row_end) next_row();
-            if (!mine) {
+        while (kb < end) {   // entry kb belongs to row r
+            if (!mine) {     // a long row is not computed here: jump over what is left of it
                 kb = row_end;
+                close_row();
                 if (kb >= end) break;
-                next_row();
                 fetch(kb, mycol, myval);
                 continue;
             }
             const int cnt = (int)(end - kb < kWave ? end - kb : kWave);
             fetch(kb + kWave, nextcol, nextval);   // in flight while this chunk is used
-            for (int j0 = 0; j0 < cnt; j0 += kBatch) {
-                T bv[kBatch];
-#pragma unroll
-                for (int u = 0; u < kBatch; ++u)
-                    bv[u] = Bc[__shfl(mycol, j0 + u < cnt ? j0 + u : cnt - 1, kWave) * ldb];
+            // per lane, once per chunk: where my entry's row of B starts, and whether my entry is
+            // the last of its row (its row = number of row starts at or before it)
+            const int64_t k = kb + lane;
+            const int64_t myoff = mycol * row_bytes;
+            int rid = 0;
+            for (int l = 1; l < nr; ++l) rid += k >= ptr_of(l) ? 1 : 0;
+            const int64_t my_row_end = __shfl(my_ptr, rid + 1, kWave);
+            const unsigned long long ends = __ballot(lane < cnt && k + 1 == my_row_end);
+            // Two batches of gathers are in flight: the next batch is requested before the
+            // current one is added up (stages alternate in place, no copies of pending loads).
+            auto gather = [&](int j0, T (&bv)[kBatch]) {
 #pragma unroll
                 for (int u = 0; u < kBatch; ++u) {
-                    if (j0 + u >= cnt) break;
-                    const int64_t k = kb + j0 + u;
-                    while (k >= row_end) next_row();
-                    const T av = __shfl(myval, j0 + u, kWave);
-                    if (mine) acc += av * bv[u];
+                    const int j = __builtin_amdgcn_readfirstlane(j0 + u < cnt ? j0 + u : cnt - 1);
+                    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(myoff & 0xffffffffll), j);
+                    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(myoff >> 32), j);
+                    bv[u] = *reinterpret_cast<const T *>(Bc + (int64_t)(((unsigned long long)hi << 32) | lo));
                 }
+            };
+            auto add_up = [&](int j0, const T (&bv)[kBatch]) {
+                const int m = cnt - j0 < kBatch ? cnt - j0 : kBatch;   // entries of this batch
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    if (u >= m) break;
+                    const int j = __builtin_amdgcn_readfirstlane(j0 + u);
+                    acc += nm::read_lane(myval, j) * bv[u];
+                    if ((ends >> j) & 1ull) close_row();
+                }
+            };
+            T bva[kBatch], bvb[kBatch];
+            gather(0, bva);
+            for (int j0 = 0;; j0 += 2 * kBatch) {
+                if (j0 + kBatch < cnt) gather(j0 + kBatch, bvb);
+                add_up(j0, bva);
+                if (j0 + kBatch >= cnt) break;
+                if (j0 + 2 * kBatch < cnt) gather(j0 + 2 * kBatch, bva);
+                add_up(j0 + kBatch, bvb);
+                if (j0 + 2 * kBatch >= cnt) break;
             }
             kb += cnt;
             mycol = nextcol;
             myval = nextval;
         }
-        while (r < nr) next_row();   // the last row, and empty rows at the end
+        while (r < nr) next_row();   // rows of a wavefront whose entries ran out before them
     }
 }
 
@@ -208,7 +249,7 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
     const T *__restrict__ gC, int64_t ldg, int64_t n, T *__restrict__ grad_A,
     T *__restrict__ grad_B, int64_t ldgb, const int32_t *__restrict__ chunk_row) {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+    const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
     const int64_t nchunks = (nnz + kWave - 1) / kWave;
     for (int64_t ch = wave0; ch < nchunks; ch += nwaves) {
