@@ -19,7 +19,7 @@ inline size_t scan_scratch_bytes(int64_t n) {
 // workgroup total in `total`.  `s_wave` holds one slot per wavefront.
 __device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t *s_wave, int64_t &total) {
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int nwaves = blockDim.x / kWave;
     int64_t inc = v;
 #pragma unroll

@@ -395,7 +395,7 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
     constexpr int kWaves = kBlock / kWave;
     __shared__ int s_wave[kWaves][kBins];   // rows of bin q in wavefront w
     __shared__ int s_base[kBins];
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x; i0 < rows; i0 += stride) {
         const int64_t i = i0 + threadIdx.x;
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
     constexpr int STRIDE = TABLE + (GPB > 1 ? kTablePad : 0);
     __shared__ __align__(16) int32_t s_keys[GPB * STRIDE];
     __shared__ int s_red[kBlock / kWave];
-    const int gl = threadIdx.x % G, gi = threadIdx.x / G;
+    const int gl = threadIdx.x % G, gi = G >= kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x / G) : threadIdx.x / G;
     int32_t *tab = s_keys + gi * STRIDE;
     const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
     for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
@@ -529,7 +529,7 @@ __global__ __launch_bounds__(kSpillBlock) void symbolic_spill_kernel(
     int32_t *mark = mark_all + (size_t)blockIdx.x * (B_cols + 1);
     for (int64_t c = threadIdx.x; c < B_cols; c += kSpillBlock) mark[c] = 0;
     __syncthreads();
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     for (int32_t idx = b0 + blockIdx.x; idx < b1; idx += gridDim.x) {
         const int64_t row = perm[idx];
         const int32_t stamp = (int32_t)row + 1;
@@ -567,7 +567,7 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
     extern __shared__ __align__(16) unsigned char s_raw[];
     T *s_vals = reinterpret_cast<T *>(s_raw);
     int32_t *s_keys = reinterpret_cast<int32_t *>(s_raw + sizeof(T) * GPB * STRIDE);
-    const int gl = threadIdx.x % G, gi = threadIdx.x / G;
+    const int gl = threadIdx.x % G, gi = G >= kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x / G) : threadIdx.x / G;
     int32_t *tab = s_keys + gi * STRIDE;
     T *val = s_vals + gi * STRIDE;
     // compacted (column, slot) lists used to order the row on the way out
@@ -718,7 +718,7 @@ __global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
     T *acc = reinterpret_cast<T *>(acc_all + (size_t)blockIdx.x * (B_cols + 1));
     for (int64_t c = threadIdx.x; c < B_cols; c += kSpillBlock) { mark[c] = 0; acc[c] = T(0); }
     __syncthreads();
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     for (int32_t idx = b0 + blockIdx.x; idx < b1; idx += gridDim.x) {
         const int64_t row = perm[idx];
         const int32_t stamp = -((int32_t)row + 1);
@@ -784,7 +784,7 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
     constexpr int G = kBwdG, GPB = kBlock / G;
     __shared__ int32_t s_ci[GPB * kBwdStage];
     __shared__ T s_g[GPB * kBwdStage];
-    const int gl = threadIdx.x % G, gi = threadIdx.x / G;
+    const int gl = threadIdx.x % G, gi = G >= kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x / G) : threadIdx.x / G;
     const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);   // first lane of the group inside its wavefront
     int32_t *ci = s_ci + gi * kBwdStage;
     T *cg = s_g + gi * kBwdStage;

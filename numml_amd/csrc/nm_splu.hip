@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void lu_rows_kernel(int64_t rows, const T *
                                                          int64_t *__restrict__ As_indices, T *__restrict__ As_data,
                                                          int32_t *stamp_all, int32_t *queue_all, uint8_t *keep_all) {
     const int lane = threadIdx.x & 63;
-    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
     volatile int32_t *stamp = stamp_all + wave * rows;
     volatile int32_t *queue = queue_all + wave * rows;
@@ -174,7 +174,8 @@ __global__ __launch_bounds__(kBlock) void lu_values_kernel(int64_t rows, const T
                                                            T *__restrict__ As_data) {
     const int lane = threadIdx.x & 63;
     const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
-    for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6; i < rows; i += nwaves) {
+    for (int64_t i = (int64_t)blockIdx.x * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+         i < rows; i += nwaves) {
         const int64_t ab = A_indptr[i], ae = A_indptr[i + 1], pe = As_indptr[i + 1];
         for (int64_t p = As_indptr[i] + lane; p < pe; p += 64) {
             const int64_t j = As_indices[p];
@@ -317,7 +318,7 @@ __global__ __launch_bounds__(kBlock) void lu_flow_kernel(int64_t cols, const int
                                                          int32_t *done, int32_t *ctl, int64_t spin_limit) {
     __shared__ int32_t s_rows[kLuWavesPerBlock][kLuCap];
     __shared__ T s_vals[kLuWavesPerBlock][kLuCap];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     for (;;) {
         int32_t ticket = 0;
         if (lane == 0) ticket = atomicAdd(ctl, 1);

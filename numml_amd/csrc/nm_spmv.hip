@@ -59,7 +59,7 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
     __shared__ int32_t s_off[R + 1];
     __shared__ T s_prod[CAP];
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
 
     const int64_t ntiles = (rows + R - 1) / R, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
     __shared__ int32_t s_off[R + 1];
     __shared__ T s_a[CAP];
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
 
     const int64_t ntiles = (rows + R - 1) / R, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
     __shared__ int32_t s_off[R + 1];
     __shared__ T s_v[CAP];
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const bool mirror = flags[0] != 0;
     const int64_t ntiles = (cols + R - 1) / R, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {

@@ -424,7 +424,7 @@ struct GVals { Meta m; int32_t ds; double v, dv, bv; };
 
 template <int G> __device__ __forceinline__ Meta load_gmeta(const SolveArgs &a, const Bounds &b) {
     Meta m;
-    m.q = b.qb + (int)threadIdx.x / G;
+    m.q = b.qb + (G == 64 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x / G) : (int)threadIdx.x / G);
     m.live = m.q < b.qe;
     const int qs = m.live ? m.q : 0;
     m.dlo = a.dptr[qs];

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kBlock) void entry_map_kernel(int64_t rows, const i
                                                            int64_t ld) {
     __shared__ int32_t s_off[kTileRows + 1];
     __shared__ uint8_t s_row[kTileCap];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t ntiles = nm::ceil_div(rows, kTileRows), npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t tile = nm::xcd_tile(id, npad);
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kBlock) void diagonal_kernel(int64_t rows, const T 
     __shared__ int32_t s_off[kTileRows + 1];
     __shared__ uint8_t s_row[kTileCap];
     __shared__ T s_x[kTileRows];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t ntiles = nm::ceil_div(rows, kTileRows), npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t tile = nm::xcd_tile(id, npad);
