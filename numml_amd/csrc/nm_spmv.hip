@@ -234,26 +234,44 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
             const int32_t *__restrict__ tr = t_row + base;
             const int32_t *__restrict__ tp = t_perm + base;
             T *__restrict__ ga = grad_A + base;
-            int p = threadIdx.x;
-            for (; p + kBlock < n; p += 2 * kBlock) {   // two entries in flight per lane (measured best)
-                const int32_t k0 = nm::stream_load(tp + p), k1 = nm::stream_load(tp + p + kBlock);
-                const int32_t r0 = nm::stream_load(tr + p), r1 = nm::stream_load(tr + p + kBlock);
-                const T g0 = g[r0], g1 = g[r1];
-                const T x0 = x[r0], x1 = x[r1];
-                const T d0 = data[k0], d1 = data[k1];
-                ga[p] = s_v[p] * x0;
-                ga[p + kBlock] = s_v[p + kBlock] * x1;
-                s_v[p] = g0 * d0;
-                s_v[p + kBlock] = g1 * d1;
-            }
-            for (; p < n; p += kBlock) {
-                const int32_t k = nm::stream_load(tp + p);
-                const int32_t r = nm::stream_load(tr + p);
-                const T gr = g[r];
-                const T xr = x[r];
-                const T dk = data[k];
-                ga[p] = s_v[p] * xr;
-                s_v[p] = gr * dk;
+            // K entries in flight per lane: all their plan loads, then all their gathers, then
+            // the stores -- two memory round trips per K entries.  Loads are unconditional on a
+            // clamped position (a predicated load would sit in its own branch with its own wait).
+            // Measured on the 2048 x 2048 Poisson matrix (5 entries per lane and tile), kernel time:
+            // K = 2: 103 us, 4: 95 us, 5: 90 us, 6: 86 us, 8: 91 us.
+            constexpr int K = 6;
+            for (int p0 = threadIdx.x; p0 < n; p0 += K * kBlock) {
+                int32_t kk[K], rr[K];
+                T gg[K], xx[K], dd[K];
+#pragma unroll
+                for (int u = 0; u < K; ++u) {
+                    const int pc = p0 + u * kBlock < n ? p0 + u * kBlock : n - 1;
+                    kk[u] = nm::stream_load(tp + pc);
+                    rr[u] = nm::stream_load(tr + pc);
+                }
+#pragma unroll
+                for (int u = 0; u < K; ++u) {
+                    gg[u] = g[rr[u]];
+                    xx[u] = x[rr[u]];
+                    dd[u] = data[kk[u]];
+                }
+                if (p0 + (K - 1) * kBlock < n) {
+#pragma unroll
+                    for (int u = 0; u < K; ++u) {
+                        const int p = p0 + u * kBlock;
+                        ga[p] = s_v[p] * xx[u];
+                        s_v[p] = gg[u] * dd[u];
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < K; ++u) {
+                        const int p = p0 + u * kBlock;
+                        if (p < n) {
+                            ga[p] = s_v[p] * xx[u];
+                            s_v[p] = gg[u] * dd[u];
+                        }
+                    }
+                }
             }
             __syncthreads();
             for (int t = threadIdx.x; t < nc; t += kBlock) {
