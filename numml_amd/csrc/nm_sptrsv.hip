@@ -375,6 +375,11 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
             const int q = cur.m.q;
             const int n = cur.m.live ? cur.m.n : 0;
             // fast path: no global memory access at all -- every dependency from the LDS ring
+            // ring reads first, together and unconditionally; whether a term counts is a select
+            // afterwards (a read inside `if (e < n)` sits in its own branch with its own wait)
+            double xj[PRE];
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) xj[e] = ring[cur.ds[e] & (kRing - 1)];
             double acc = 0.;
             bool in_ring = n <= PRE;
 #pragma unroll
@@ -382,11 +387,9 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
                 const int32_t ds = cur.ds[e];
                 const int dist = ds > q ? ds - q : q - ds;
                 const bool hit = ds >= qlo && ds < qhi && dist < kRingSafe;
-                const double xj = ring[ds & (kRing - 1)];
-                if (e < n) {
-                    in_ring = in_ring && hit;
-                    acc += cur.v[e] * xj;
-                }
+                const double term = cur.v[e] * xj[e];
+                acc += e < n ? term : 0.;        // + 0.0 leaves the sum as it is
+                in_ring = in_ring && (hit || e >= n);
             }
             if (!in_ring) {
                 // slow path (a dependency older than the ring, or a row longer than the
@@ -638,6 +641,9 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
     EllVals<PRE> qv[DEPTH];   // operands of levels it .. it + DEPTH - 1, each refilled in place
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, load_bounds(s_lp, d, count, l0, step, lmin));
+    // The bounds of the level whose operands are requested next are read from LDS one level
+    // early, before the barrier, so that the request does not start with an LDS round trip.
+    Bounds ahead = load_bounds(s_lp, DEPTH, count, l0, step, lmin);
 
     for (int it0 = 0; it0 < count; it0 += DEPTH) {
 #pragma unroll
@@ -645,19 +651,25 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
             const int it = it0 + d;
             if (it >= count) break;   // uniform over the workgroup
             const EllVals<PRE> cur = qv[d];
-            qv[d] = load_ell<PRE>(a, load_bounds(s_lp, it + DEPTH, count, l0, step, lmin));
+            qv[d] = load_ell<PRE>(a, ahead);
 
             const int q = cur.q;
+            // All ring reads go out together and unconditionally; whether a term counts is a
+            // select afterwards.  (Reads inside `if (dependency present)` each sat in a branch of
+            // their own with the wait for the LDS behind them: PRE serial LDS round trips.)
+            double xj[PRE];
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) xj[e] = ring[cur.ds[e] & (kRing - 1)];
+            ahead = load_bounds(s_lp, it + DEPTH + 1, count, l0, step, lmin);
             double acc = 0.;
             bool in_ring = true;
 #pragma unroll
             for (int e = 0; e < PRE; ++e) {
                 const int32_t raw = cur.ds[e];   // -1: no dependency; bit 30: not in this launch's ring
-                const double xj = ring[raw & (kRing - 1)];
-                if (cur.live && raw >= 0) {
-                    in_ring = in_ring && !(raw & kEllFar);
-                    acc += cur.v[e] * xj;
-                }
+                const bool use = cur.live && raw >= 0;
+                const double term = cur.v[e] * xj[e];
+                acc += use ? term : 0.;          // + 0.0 leaves the sum as it is
+                in_ring = in_ring && !(use && (raw & kEllFar));
             }
             if (!in_ring) {
                 // a dependency the ring does not hold: redo the sum in the same order from global memory
