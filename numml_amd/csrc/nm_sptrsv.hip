@@ -44,8 +44,12 @@ struct Packed {        // one solve direction, level-major (all int32, device)
     int32_t *diag;     // [rows]   position of the diagonal coefficient, -1 when not stored
     int32_t *ell_ds;   // [ell_capacity] fixed-width copy of dslot: `pre` slots per row, -1 padded
 };
-// Entries of the fixed-width (ELLPACK) arrays; the layout is used when rows * pre fits.
-inline int64_t ell_capacity(int64_t rows, int64_t nnz) { return 2 * nnz + 2 * rows + 8; }
+// Entries of the fixed-width (ELLPACK) arrays; the layout is used when (rows + kEllPad) * pre
+// fits.  kEllPad slots of padding follow the last row in every array the fixed-width kernel
+// reads or writes by slot: its lanes load the operands of slots qb .. qb + lanes - 1 whatever
+// the level's width, so the slots behind a level's end must be readable.
+constexpr int64_t kEllPad = 1024;   // == kNarrow, the widest single-workgroup launch
+inline int64_t ell_capacity(int64_t rows, int64_t nnz) { return 2 * nnz + 2 * rows + 8 + 8 * kEllPad; }
 }  // namespace
 
 struct nm_sptrsv_plan {
@@ -254,12 +258,12 @@ inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork
         return (double *)q;
     };
     SolveWork w;
-    w.xs = take(rows + 1);
+    w.xs = take(rows + 1 + kEllPad);
     w.dg = take(rows + 1);
     w.rhs = take(rows + 1);
     w.coef = take(nnz + 1);
     w.ell_coef = take(ell_capacity(rows, nnz));
-    w.rb = take(2 * rows + 2);
+    w.rb = take(2 * (rows + kEllPad) + 2);
     if (W) *W = w;
     return off;
 }
@@ -539,10 +543,15 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_group_kernel(SolveArgs a, int 
 // which matters because the workgroup's wavefronts share one CU and the level time
 // is the time to issue their instructions.
 
-// Bit 30 of an entry marks a dependency the LDS ring of its launch cannot serve: the
-// row it refers to was solved by another launch, or too many slots ago.  Deciding that
-// here, once, keeps a dozen compare instructions per dependency out of every level.
-constexpr int32_t kEllFar = 1 << 30;
+// An entry of the fixed-width dependency array is what the level needs and nothing else: the
+// BYTE offset of the dependency's solution in the LDS ring (bits 0..16), and bit 20 when the
+// ring of this launch cannot serve it (the row was solved by another launch, or too many slots
+// ago; the rare slow path then finds the slot in the range-based arrays).  An absent dependency
+// points at ring entry kRing, which holds 0.0 for ever, and its coefficient is 0.0: it adds
+// +0.0 to the sum, so the level needs no "is there a dependency" test at all.  Deciding all
+// this once, at plan time, keeps a dozen instructions per dependency out of every level.
+constexpr int32_t kEllFar = 1 << 20;
+constexpr int32_t kEllOffsetMask = (1 << 17) - 1;
 
 __device__ __forceinline__ int32_t level_of_slot(const int32_t *__restrict__ level_ptr, int32_t nlevels, int32_t q) {
     int32_t lo = 0, hi = nlevels;   // last l with level_ptr[l] <= q
@@ -558,17 +567,18 @@ __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict
                                 int32_t nlevels, const int32_t *__restrict__ level_launch,
                                 int32_t *__restrict__ ell_ds) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < rows * pre; i += stride) {
+    // the padding slots behind the last row get "absent" entries: lanes that read them must find a valid offset
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (rows + kEllPad) * pre; i += stride) {
         const int64_t q = i / pre;
         const int e = (int)(i - q * pre);
-        const int32_t lo = dptr[q], n = dptr[q + 1] - lo;
-        int32_t out = -1;
+        const int32_t lo = q < rows ? dptr[q] : 0, n = q < rows ? dptr[q + 1] - lo : 0;
+        int32_t out = kRing * 8;   // absent: the ring entry that is always 0.0
         if (e < n) {
             const int32_t ds = dslot[lo + e];
             const int32_t dist = ds > (int32_t)q ? ds - (int32_t)q : (int32_t)q - ds;
             const bool same = level_launch[level_of_slot(level_ptr, nlevels, (int32_t)q)] ==
                               level_launch[level_of_slot(level_ptr, nlevels, ds)];
-            out = ds | ((same && dist < kRingSafe) ? 0 : kEllFar);
+            out = ((ds & (kRing - 1)) * 8) | ((same && dist < kRingSafe) ? 0 : kEllFar);
         }
         ell_ds[i] = out;
     }
@@ -595,31 +605,45 @@ __global__ void gather_ell_kernel(int64_t rows, int pre, const T *__restrict__ d
 }
 
 struct EllArgs {
-    const int32_t *level_ptr, *ell_ds;
+    const int32_t *level_ptr, *ell_ds, *dptr, *dslot;
     const double *ell_coef, *rb;
     double *xs;
     int unit;
 };
 
+// Operands of the slot qb + lane of a level.  qb is a scalar, so each of the three loads is
+// `scalar base + the lane's constant byte offset`: no vector address arithmetic per level.
+// Lanes beyond the level's end load the slots that follow it (readable: see kEllPad) and
+// compute a value that is never stored.
 template <int PRE> struct EllVals {
-    int q;
-    bool live;
+    int qb, qe;
     int32_t ds[PRE];
     double v[PRE];
     double bv, dv;
 };
+
+__device__ __forceinline__ Bounds load_bounds_uniform(const int32_t *s_lp, int it, int count, int l0, int step,
+                                                      int lmin) {
+    const Bounds b = load_bounds(s_lp, it, count, l0, step, lmin);
+    return Bounds{__builtin_amdgcn_readfirstlane(b.qb), __builtin_amdgcn_readfirstlane(b.qe)};
+}
 
 template <int PRE> __device__ __forceinline__ EllVals<PRE> load_ell(const EllArgs &a, const Bounds &b) {
     typedef int32_t IV __attribute__((ext_vector_type(PRE)));
     typedef double DV __attribute__((ext_vector_type(PRE)));
     typedef double D2 __attribute__((ext_vector_type(2)));
     EllVals<PRE> v;
-    v.q = b.qb + (int)threadIdx.x;
-    v.live = v.q < b.qe;
-    const unsigned qs = v.live ? (unsigned)v.q : 0u;   // unconditional loads: slot 0 always exists
-    const IV dsv = reinterpret_cast<const IV *>(a.ell_ds)[qs];
-    const DV cv = reinterpret_cast<const DV *>(a.ell_coef)[qs];
-    const D2 r = reinterpret_cast<const D2 *>(a.rb)[qs];
+    v.qb = b.qb;
+    v.qe = b.qe;
+    const uint32_t lane_ds = threadIdx.x * (uint32_t)(sizeof(int32_t) * PRE);
+    const uint32_t lane_cf = threadIdx.x * (uint32_t)(sizeof(double) * PRE);
+    const uint32_t lane_rb = threadIdx.x * (uint32_t)(sizeof(double) * 2);
+    const char *pd = reinterpret_cast<const char *>(a.ell_ds) + (int64_t)b.qb * (int64_t)(sizeof(int32_t) * PRE);
+    const char *pc = reinterpret_cast<const char *>(a.ell_coef) + (int64_t)b.qb * (int64_t)(sizeof(double) * PRE);
+    const char *pr = reinterpret_cast<const char *>(a.rb) + (int64_t)b.qb * (int64_t)(sizeof(double) * 2);
+    const IV dsv = *reinterpret_cast<const IV *>(pd + lane_ds);
+    const DV cv = *reinterpret_cast<const DV *>(pc + lane_cf);
+    const D2 r = *reinterpret_cast<const D2 *>(pr + lane_rb);
 #pragma unroll
     for (int e = 0; e < PRE; ++e) {
         v.ds[e] = dsv[e];
@@ -630,20 +654,27 @@ template <int PRE> __device__ __forceinline__ EllVals<PRE> load_ell(const EllArg
     return v;
 }
 
+// The workgroup lives on one CU and a level lasts as long as it takes to issue every
+// wavefront's instructions for it (four wavefronts per SIMD at 1024 rows, ~4 cycles per vector
+// instruction), so the level body is kept to what cannot be decided earlier: the ring reads
+// (offsets precomputed), the sum, the division, and the two stores.
 template <int PRE, int DEPTH>
 __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step) {
-    __shared__ double ring[kRing];
+    __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
     __shared__ int32_t s_lp[kMaxLevels + 1];
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
     for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
+    if (threadIdx.x == 0) ring[kRing] = 0.;
     __syncthreads();
+    const char *ring_bytes = reinterpret_cast<const char *>(ring);
+    const uint32_t lane8 = threadIdx.x * 8u;
 
     EllVals<PRE> qv[DEPTH];   // operands of levels it .. it + DEPTH - 1, each refilled in place
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, load_bounds(s_lp, d, count, l0, step, lmin));
+    for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, load_bounds_uniform(s_lp, d, count, l0, step, lmin));
     // The bounds of the level whose operands are requested next are read from LDS one level
     // early, before the barrier, so that the request does not start with an LDS round trip.
-    Bounds ahead = load_bounds(s_lp, DEPTH, count, l0, step, lmin);
+    Bounds ahead = load_bounds_uniform(s_lp, DEPTH, count, l0, step, lmin);
 
     for (int it0 = 0; it0 < count; it0 += DEPTH) {
 #pragma unroll
@@ -653,36 +684,34 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
             const EllVals<PRE> cur = qv[d];
             qv[d] = load_ell<PRE>(a, ahead);
 
-            const int q = cur.q;
-            // All ring reads go out together and unconditionally; whether a term counts is a
-            // select afterwards.  (Reads inside `if (dependency present)` each sat in a branch of
-            // their own with the wait for the LDS behind them: PRE serial LDS round trips.)
+            // all ring reads go out together, unconditionally
             double xj[PRE];
-#pragma unroll
-            for (int e = 0; e < PRE; ++e) xj[e] = ring[cur.ds[e] & (kRing - 1)];
-            ahead = load_bounds(s_lp, it + DEPTH + 1, count, l0, step, lmin);
-            double acc = 0.;
-            bool in_ring = true;
+            int32_t any = 0;
 #pragma unroll
             for (int e = 0; e < PRE; ++e) {
-                const int32_t raw = cur.ds[e];   // -1: no dependency; bit 30: not in this launch's ring
-                const bool use = cur.live && raw >= 0;
-                const double term = cur.v[e] * xj[e];
-                acc += use ? term : 0.;          // + 0.0 leaves the sum as it is
-                in_ring = in_ring && !(use && (raw & kEllFar));
+                xj[e] = *reinterpret_cast<const double *>(ring_bytes + (cur.ds[e] & kEllOffsetMask));
+                any |= cur.ds[e];
             }
-            if (!in_ring) {
+            ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
+            double acc = 0.;
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
+            const bool live = (int)threadIdx.x < cur.qe - cur.qb;
+            if ((any & kEllFar) && live) {
                 // a dependency the ring does not hold: redo the sum in the same order from global memory
+                const int q = cur.qb + (int)threadIdx.x;
+                const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
                 acc = 0.;
 #pragma unroll
                 for (int e = 0; e < PRE; ++e)
-                    if (cur.ds[e] >= 0) acc += cur.v[e] * a.xs[cur.ds[e] & (kEllFar - 1)];
+                    if (e < n) acc += cur.v[e] * a.xs[a.dslot[dlo + e]];
             }
-            if (cur.live) {
-                double xi = cur.bv - acc;
-                if (!a.unit) xi /= cur.dv;
-                ring[q & (kRing - 1)] = xi;
-                a.xs[q] = xi;
+            double xi = cur.bv - acc;
+            if (!a.unit) xi /= cur.dv;
+            if (live) {
+                const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
+                *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
+                *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
             }
             __syncthreads();
         }
@@ -733,7 +762,7 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     }
     const int dirn = transposed ? 1 : 0;
     const int pre = p->ell_pre[dirn];
-    EllArgs ea{p->level_ptr, P.ell_ds, a.w.ell_coef, a.w.rb, a.w.xs, unit};
+    EllArgs ea{p->level_ptr, P.ell_ds, P.dptr, P.dslot, a.w.ell_coef, a.w.rb, a.w.xs, unit};
     if (pre > 0) {
         int64_t grid = nm::ceil_div(p->rows * pre, kBlock);
         if (grid > 65536) grid = 65536;
@@ -971,7 +1000,7 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     for (int d = 0; d < 2; ++d) {
         const int32_t md = p->max_deps[d];
         const int pre = md <= 2 ? 2 : (md <= 4 ? 4 : (md <= 8 ? 8 : 0));
-        if (pre > 0 && rows < kEllFar && rows * pre <= ell_capacity(rows, nnz)) {
+        if (pre > 0 && rows < (1 << 30) && (rows + kEllPad) * pre <= ell_capacity(rows, nnz)) {
             p->ell_pre[d] = pre;
             int64_t grid = nm::ceil_div(rows * pre, kBlock);
             if (grid > 65536) grid = 65536;
