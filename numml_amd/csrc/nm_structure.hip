@@ -158,6 +158,21 @@ __global__ __launch_bounds__(kBlock) void diagonal_kernel(int64_t rows, const T 
 constexpr int kLcRows = 256, kLcCap = 2304;
 constexpr uint32_t kLcNone = 0xffff;
 
+// dst[k] = (int32) src[k] for k < n, by the whole workgroup.  K loads per lane are requested
+// before the first is stored (a plain loop waits for every load it has just issued), on
+// clamped positions so that no load is predicated.
+template <int K>
+__device__ __forceinline__ void lc_stage_cols(int32_t *dst, const int64_t *__restrict__ src, int n) {
+    for (int k0 = threadIdx.x; k0 < n; k0 += K * kBlock) {
+        int64_t v[K];
+#pragma unroll
+        for (int u = 0; u < K; ++u) v[u] = nm::stream_load(src + (k0 + u * kBlock < n ? k0 + u * kBlock : n - 1));
+#pragma unroll
+        for (int u = 0; u < K; ++u)
+            if (k0 + u * kBlock < n) dst[k0 + u * kBlock] = (int32_t)v[u];
+    }
+}
+
 struct LcTile {
     int32_t offA[kLcRows + 1], offB[kLcRows + 1], offC[kLcRows + 1];
     int32_t colA[kLcCap], colB[kLcCap];
@@ -230,8 +245,8 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
         __syncthreads();
         const int nA = s.offA[nr], nB = s.offB[nr];
         if (nA <= kLcCap && nB <= kLcCap) {
-            for (int k = threadIdx.x; k < nA; k += kBlock) s.colA[k] = (int32_t)nm::stream_load(A_indices + baseA + k);
-            for (int k = threadIdx.x; k < nB; k += kBlock) s.colB[k] = (int32_t)nm::stream_load(B_indices + baseB + k);
+            lc_stage_cols<5>(s.colA, A_indices + baseA, nA);
+            lc_stage_cols<5>(s.colB, B_indices + baseB, nB);
             const int64_t baseC = COUNT ? 0 : C_indptr[r0];
             if (!COUNT)
                 for (int t = threadIdx.x; t <= nr; t += kBlock) s.offC[t] = (int32_t)(C_indptr[r0 + t] - baseC);
@@ -257,23 +272,33 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
             if (!COUNT) {
                 __syncthreads();
                 const int nC = s.offC[nr];
-                for (int o = threadIdx.x; o < nC; o += kBlock) {
-                    const uint32_t sr = s.src[o];
-                    const uint32_t ia = sr & 0xffff, ib = sr >> 16;
-                    T v;
-                    int32_t c;
-                    if (ib == kLcNone) {
-                        c = s.colA[ia];
-                        v = alpha * A_data[baseA + ia];
-                    } else if (ia == kLcNone) {
-                        c = s.colB[ib];
-                        v = beta * B_data[baseB + ib];
-                    } else {
-                        c = s.colA[ia];
-                        v = alpha * A_data[baseA + ia] + beta * B_data[baseB + ib];
+                // K output entries per lane: their operand values are requested together and
+                // unconditionally (an operand that is absent reads entry 0 of a tile that has one
+                // and is dropped by the select), then combined and stored.
+                constexpr int K = 5;
+                const T *__restrict__ Ad = nA > 0 ? A_data + baseA : B_data + baseB;
+                const T *__restrict__ Bd = nB > 0 ? B_data + baseB : A_data + baseA;
+                for (int o0 = threadIdx.x; o0 < nC; o0 += K * kBlock) {
+                    uint32_t ia[K], ib[K];
+                    T va[K], vb[K];
+#pragma unroll
+                    for (int u = 0; u < K; ++u) {
+                        const uint32_t sr = s.src[o0 + u * kBlock < nC ? o0 + u * kBlock : nC - 1];
+                        ia[u] = sr & 0xffff;
+                        ib[u] = sr >> 16;
+                        va[u] = Ad[ia[u] == kLcNone ? 0u : ia[u]];
+                        vb[u] = Bd[ib[u] == kLcNone ? 0u : ib[u]];
                     }
-                    nm::stream_store(C_indices + baseC + o, (int64_t)c);
-                    nm::stream_store(C_data + baseC + o, v);
+#pragma unroll
+                    for (int u = 0; u < K; ++u) {
+                        const int o = o0 + u * kBlock;
+                        if (o >= nC) break;
+                        const T pa = alpha * va[u], pb = beta * vb[u];
+                        const T v = ib[u] == kLcNone ? pa : (ia[u] == kLcNone ? pb : pa + pb);
+                        const int32_t c = ia[u] == kLcNone ? s.colB[ib[u]] : s.colA[ia[u]];
+                        nm::stream_store(C_indices + baseC + o, (int64_t)c);
+                        nm::stream_store(C_data + baseC + o, v);
+                    }
                 }
             }
         } else {
@@ -287,8 +312,8 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
 
 // grad_X[k] = coef * grad_C at the same coordinate (cpp/sparse_csr_cpu.cpp:505-552).
 // Every column of X is present in C.  Same tiling: columns of X and of C staged in
-// LDS, one lane per row merges them and notes the matching entry of C for every
-// entry of X, then lane = entry of X gathers and scales.
+// LDS, one lane per row marks the row of its entries of X, then lane = entry of X
+// finds its column in the row of C by bisection in LDS, gathers and scales.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void lincomb_back_kernel(int64_t rows, T coef,
                                                               const int64_t *__restrict__ X_indices,
@@ -314,24 +339,41 @@ __global__ __launch_bounds__(kBlock) void lincomb_back_kernel(int64_t rows, T co
         __syncthreads();
         const int nX = s_offX[nr], nC = s_offC[nr];
         if (nX <= kLcCap && nC <= 2 * kLcCap) {
-            for (int k = threadIdx.x; k < nX; k += kBlock) s_colX[k] = (int32_t)nm::stream_load(X_indices + baseX + k);
-            for (int k = threadIdx.x; k < nC; k += kBlock) s_colC[k] = (int32_t)nm::stream_load(C_indices + baseC + k);
+            lc_stage_cols<5>(s_colX, X_indices + baseX, nX);
+            lc_stage_cols<5>(s_colC, C_indices + baseC, nC);
             __syncthreads();
+            // row of every entry of X: one lane per row marks its entries
             for (int t = threadIdx.x; t < nr; t += kBlock) {
-                int iX = s_offX[t], iC = s_offC[t];
-                const int eX = s_offX[t + 1], eC = s_offC[t + 1];
-                while (iX < eX && iC < eC) {
-                    const int32_t cX = s_colX[iX], cC = s_colC[iC];
-                    if (cX == cC) s_match[iX] = iC;
-                    iX += cX <= cC;
-                    iC += cC <= cX;
-                }
-                for (; iX < eX; ++iX) s_match[iX] = -1;   // not reached for valid input (C holds every column of X)
+                const int eX = s_offX[t + 1];
+                for (int k = s_offX[t]; k < eX; ++k) s_match[k] = t;
             }
             __syncthreads();
-            for (int k = threadIdx.x; k < nX; k += kBlock) {
-                const int m = s_match[k];
-                if (m >= 0) nm::stream_store(grad_X + baseX + k, gC[baseC + m] * coef);
+            // lane = entry of X: bisection for its column in the same row of C; K entries per
+            // lane so that K independent searches and then K gathers are in flight
+            constexpr int K = 5;
+            for (int k0 = threadIdx.x; k0 < nX; k0 += K * kBlock) {
+                int at[K];
+                bool found[K];
+#pragma unroll
+                for (int u = 0; u < K; ++u) {
+                    const int k = k0 + u * kBlock < nX ? k0 + u * kBlock : nX - 1;
+                    const int t = s_match[k];
+                    const int32_t cX = s_colX[k];
+                    int lo = s_offC[t], hi = s_offC[t + 1];
+                    const int end = hi;
+                    while (lo < hi) {
+                        const int mid = (lo + hi) >> 1;
+                        if (s_colC[mid] < cX) lo = mid + 1; else hi = mid;
+                    }
+                    found[u] = lo < end && s_colC[lo] == cX;   // always, for valid input
+                    at[u] = found[u] ? lo : 0;
+                }
+                T gv[K];
+#pragma unroll
+                for (int u = 0; u < K; ++u) gv[u] = nC > 0 ? gC[baseC + at[u]] : T(0);
+#pragma unroll
+                for (int u = 0; u < K; ++u)
+                    if (k0 + u * kBlock < nX && found[u]) nm::stream_store(grad_X + baseX + k0 + u * kBlock, gv[u] * coef);
             }
         } else {
             for (int t = threadIdx.x; t < nr; t += kBlock) {
