@@ -139,3 +139,43 @@ def test_dtype_and_device_errors_on_device(dev):
         ext.spdmm_forward(n, n, D, I, P, torch.ones(n, 2))
     with pytest.raises(RuntimeError, match="float32 or float64"):
         ext.spgemv_forward(n, n, D.half(), I, P, x.half())
+
+
+def test_conjugate_gradients_and_training_through_the_solver(dev):
+    # what the reference's Krylov code does with these operators (numml/krylov.py:83-155): a CG
+    # loop whose only matrix operation is A @ p, differentiated end to end -- here the stencil
+    # values of a 2-D Poisson operator are trained so that five CG steps solve A x = b better
+    import scipy.sparse.linalg as spla
+    d, i, p, (n, _) = G.poisson2d(24, np.float64, jitter_seed=None)
+    A = sp.SparseCSRTensor(tuple(to_dev(dev, d, i, p)), (n, n))
+    b = to_dev(dev, randn(1, n, np.float64))[0]
+
+    def cg(A, b, iters):
+        x = torch.zeros_like(b)
+        r = b - A @ x
+        q = r.clone()
+        rs = r @ r
+        for _ in range(iters):
+            Aq = A @ q
+            alpha = rs / (q @ Aq)
+            x = x + alpha * q
+            r = r - alpha * Aq
+            rs_new = r @ r
+            q = r + (rs_new / rs) * q
+            rs = rs_new
+        return x
+
+    x = cg(A, b, 200)
+    want = spla.spsolve(A.to_scipy_csr().tocsc(), host(b))
+    assert np.allclose(host(x), want, rtol=1e-8, atol=1e-8 * np.abs(want).max())
+    # gradient of a loss through five CG steps with respect to the stored values, against
+    # the same loop in dense float64 autograd on the host
+    A.requires_grad = True
+    loss = ((A @ cg(A, b, 5) - b) ** 2).sum()
+    loss.backward()
+    Ad = torch.tensor(A.to_scipy_csr().toarray(), dtype=torch.float64, requires_grad=True)
+    bh = torch.tensor(host(b))
+    ((Ad @ cg(Ad, bh, 5) - bh) ** 2).sum().backward()
+    rows = np.repeat(np.arange(n), np.diff(p))
+    gA = Ad.grad.numpy()[rows, i]
+    assert np.allclose(host(A.grad.data), gA, rtol=1e-8, atol=1e-10 * np.abs(gA).max())
