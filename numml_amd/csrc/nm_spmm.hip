@@ -3,8 +3,10 @@
 // Forward: lane = output column (a 64-column fp32 row of B is one 256-byte
 // line, so every gather is a single coalesced request).  A wavefront owns a few
 // consecutive rows of A and walks their entries as one range, 64 (column,
-// value) pairs per coalesced load, broadcasting them lane by lane; every lane
-// adds its column's terms in storage order and restarts at row boundaries --
+// value) pairs per coalesced load, read back entry by entry into scalar
+// registers (so that a gather is a scalar row address plus one shared vector
+// of lane offsets); every lane adds its column's terms in storage order and
+// restarts at row boundaries --
 // the order of the serial CPU loop (cpp/sparse_csr_cpu.cpp:586-598), so C
 // matches it bit for bit.  Rows longer than kSplitRow are shared by the
 // wavefronts of a workgroup instead (partial sums added in wavefront order:
@@ -445,7 +447,7 @@ extern "C" int nm_spdmm_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t
         hipLaunchKernelGGL((spdmm_fwd_flat_kernel<double, int64_t, false>), dim3(flat_grid), dim3(kBlock), 0, s, rows,
                            (const double *)data, indices, indptr, nullptr, (const double *)B, ldb, n, (double *)C,
                            ldc);
-    NM_LAUNCH_CHECK("spdmm_fwd_kernel");
+    NM_LAUNCH_CHECK("spdmm_fwd_flat_kernel");
     return NM_OK;
 }
 
@@ -528,6 +530,6 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
         hipLaunchKernelGGL((spdmm_fwd_flat_kernel<double, int32_t, true>), dim3(flat_grid), dim3(kBlock), 0, s, cols,
                            (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg, n,
                            (double *)grad_B, ldgb);
-    NM_LAUNCH_CHECK("spdmm_fwd_kernel (transposed)");
+    NM_LAUNCH_CHECK("spdmm_fwd_flat_kernel (transposed)");
     return NM_OK;
 }

@@ -23,9 +23,12 @@
 // Stream order is the only synchronisation between launches: no kernel ever
 // waits on another workgroup, so nothing can hang.
 //
-// Every row is one lane; sums run in double, in the walk order of the serial
+// A row is one lane; sums run in double, in the walk order of the serial
 // CPU loop (cpp/sparse_csr_cpu.cpp:672-718: ascending for a lower triangle,
-// descending for an upper one), so results match it bit for bit.
+// descending for an upper one), so results match it bit for bit.  The exception
+// are launches whose rows average a dozen dependencies or more (the factors of a
+// direct solve): there 16 or 64 lanes share a row and add their partial sums
+// across the group, which differs from the serial order by rounding in double.
 //
 // Algorithmic HBM bytes of one solve (s = sizeof(value)):
 //   nnz*(s+8) + (rows+1)*8 + 2*rows*s
@@ -42,7 +45,7 @@ struct Packed {        // one solve direction, level-major (all int32, device)
     int32_t *dslot;    // [nnz]    slot of the row a dependency refers to
     int32_t *dsrc;     // [nnz]    position of its coefficient in A's data
     int32_t *diag;     // [rows]   position of the diagonal coefficient, -1 when not stored
-    int32_t *ell_ds;   // [ell_capacity] fixed-width copy of dslot: `pre` slots per row, -1 padded
+    int32_t *ell_ds;   // [ell_capacity] fixed-width dependency entries, `pre` per row (ring byte offset | far bit)
 };
 // Entries of the fixed-width (ELLPACK) arrays; the layout is used when (rows + kEllPad) * pre
 // fits.  kEllPad slots of padding follow the last row in every array the fixed-width kernel
