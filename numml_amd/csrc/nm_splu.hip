@@ -95,6 +95,7 @@ __global__ __launch_bounds__(kBlock) void lu_rows_kernel(int64_t rows, const T *
         if (lane == 0) stamp[i] = mark;
         for (int64_t k = A_indptr[i] + lane; k < A_indptr[i + 1]; k += 64) {
             const int64_t u = A_indices[k];
+            if (u < 0 || u >= rows) continue;   // not a column of a square matrix: ignored rather than written
             stamp[u] = mark;
             keep[u] = 1;
         }
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(kBlock) void lu_rows_kernel(int64_t rows, const T *
                         bool fresh = false;
                         if (k < ke) {
                             w = A_indices[k];
-                            fresh = stamp[w] != mark;   // columns of a row are distinct: no two lanes share w
+                            fresh = w >= 0 && w < rows && stamp[w] != mark;   // columns of a row are distinct: no two lanes share w
                         }
                         if (fresh) {
                             stamp[w] = mark;

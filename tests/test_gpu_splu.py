@@ -50,6 +50,15 @@ def _cases(dtype):
     arrow[:, 0] = 1.0
     arrow[0, 0] = 90.0
     yield "arrow90", _from_scipy(arrow, dtype)
+    # the arrow the other way round (dense LAST row and column) does not fill, but its last column has
+    # more entries than a wavefront keeps in LDS and its last row more than a wavefront has lanes
+    n = 1300
+    back = sps.lil_matrix((n, n))
+    back.setdiag(4.0 + np.arange(n) % 3)
+    back[n - 1, :] = 0.5
+    back[:, n - 1] = -0.25
+    back[n - 1, n - 1] = 3.0 * n
+    yield "back_arrow1300", _from_scipy(back, dtype)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
@@ -102,7 +111,7 @@ def test_spsolve_gradients_against_dense_autograd(dev, dtype):
     tdt = torch.float32 if dtype == np.float32 else torch.float64
     tol = 2e-4 if dtype == np.float32 else 1e-10
     for name, (d, i, p, (n, _)) in _cases(dtype):
-        if name in ("tridiag700",):
+        if name in ("tridiag700", "back_arrow1300"):
             continue
         D, I, P = to_dev(dev, d, i, p)
         A = sp.SparseCSRTensor((D.clone(), I, P), (n, n))
