@@ -45,7 +45,18 @@ struct LuScratch {
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
 
-inline int lu_waves(int64_t rows) { return (int)(rows < kLuWaves ? (rows > 0 ? rows : 1) : kLuWaves); }
+// Wavefronts that share the rows: at most kLuWaves, at most one per row, and few enough that
+// their scratch (9 bytes per row each) stays within kLuScratchBytes.
+constexpr int64_t kLuScratchBytes = int64_t(1) << 30;
+inline int lu_waves(int64_t rows) {
+    if (rows < 1) return 1;
+    int64_t w = rows < kLuWaves ? rows : kLuWaves;
+    const int64_t fit = kLuScratchBytes / (9 * rows);
+    // (a launch is whole workgroups of four wavefronts: fewer wavefronts than rows must be a
+    //  multiple of four, or the last workgroup's extra wavefronts would take rows without scratch)
+    if (w > fit) w = (fit < 64 ? 64 : fit) / 4 * 4;
+    return (int)w;
+}
 
 size_t lu_layout(int64_t rows, void *base, LuScratch *S) {
     size_t off = 0;

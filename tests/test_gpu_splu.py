@@ -187,3 +187,33 @@ def test_numeric_phase_gives_up_instead_of_waiting_forever(dev):
     assert L.nm_splu_numeric(1, n, Td2.data_ptr(), Ti.data_ptr(), Tp.data_ptr(), work.data_ptr(), nbytes.value, 0,
                              stream) == 0
     assert_same(host(Td2), want, "factors after the failed call")
+
+
+def test_pattern_scratch_is_bounded(dev):
+    # the pattern pass gives every wavefront 9 bytes of scratch per row; the number of wavefronts
+    # is cut so that the total stays near 1 GiB (the walk itself costs O(rows) per row for a chain
+    # like this one, as in the reference, so the size here is moderate)
+    import ctypes
+    from numml_amd import _lib
+    nbytes = ctypes.c_size_t(0)
+    assert _lib.lib().nm_splu_symbolic_bytes(400_000, ctypes.byref(nbytes)) == 0
+    assert nbytes.value < 1.2 * 2 ** 30
+    n = 30_000
+    assert _lib.lib().nm_splu_symbolic_bytes(n, ctypes.byref(nbytes)) == 0
+    assert nbytes.value < 1.2 * 2 ** 30       # 4096 wavefronts would need 1.1 GB: one step under the cut
+    d, i, p, _ = G.tridiag(n, np.float64)
+    print("case tridiag", n, flush=True)
+    M = numml_amd.load_compiled().splu(n, n, *to_dev(dev, d, i, p))
+    assert_same(host(M[1]), i, "no fill")
+    assert_same(host(M[2]), p, "no fill")
+    # u_0 = 2, l_k = -1 / u_{k-1}, u_k = 2 - l_k * (-1)
+    u = np.empty(n)
+    lo = np.empty(n)
+    u[0] = 2.0
+    for k in range(1, n):
+        lo[k] = -1.0 / u[k - 1]
+        u[k] = 2.0 - lo[k] * -1.0
+    got = host(M[0])
+    diag_pos = p[:-1] + (np.arange(n) > 0)
+    assert np.array_equal(got[diag_pos], u)
+    assert np.array_equal(got[p[1:-1]], lo[1:])
