@@ -542,8 +542,8 @@ WORKLOADS = {
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="spmv", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=10.0,
                     help="CPU time budget of the cpu_baseline leg (0 skips it)")
