@@ -181,3 +181,27 @@ def _transpose(csr):
     d, i, p, (r, c) = csr
     At_d, At_i, At_p, _ = oracle.csr_transpose(r, c, d, i, p)
     return At_d, At_i, At_p, (c, r)
+
+
+def test_fp32_long_rows_against_a_double_evaluation(dev):
+    # Long rows are summed by many lanes and reduced, i.e. in another order than the serial loop.
+    # Both results are compared with the same products accumulated in double: the device's error
+    # must not exceed four times the serial loop's, plus the fp32 tolerance of the parity rule.
+    import scipy.sparse as sps
+    rtol = 1e-5
+    for name, (d, i, p, (rows, cols)) in (
+            ("powerlaw", G.powerlaw(4000, 20000, target_nnz=400_000, max_deg=9000, seed=3, dtype=np.float32)),
+            ("one_long_row", G.ragged_csr(3, 200_000, 150_000, 4, np.float32, min_len=100_000))):
+        x = randn(1, cols, np.float32)
+        B = randn(2, (cols, 8), np.float32)
+        A64 = sps.csr_matrix((d.astype(np.float64), i, p), shape=(rows, cols))
+        D, I, P, X, Bd = to_dev(dev, d, i, p, x, B)
+        for what, got, cpu, exact in (
+                ("spmv", host(ext.spgemv_forward(rows, cols, D, I, P, X)), oracle.spgemv_forward(rows, cols, d, i, p, x),
+                 A64 @ x.astype(np.float64)),
+                ("spmm", host(ext.spdmm_forward(rows, cols, D, I, P, Bd)), oracle.spdmm_forward(rows, cols, d, i, p, B),
+                 A64 @ B.astype(np.float64))):
+            err_gpu = np.abs(got.astype(np.float64) - exact)
+            err_cpu = np.abs(cpu.astype(np.float64) - exact)
+            bound = 4 * err_cpu + rtol * np.abs(exact).max()
+            assert np.all(err_gpu <= bound), f"{name} {what}: worst excess {float((err_gpu - bound).max()):.3e}"
