@@ -4,6 +4,8 @@ boundary, empty rows at either end, rows just over the long-row limits, dense wi
 not a multiple of a wavefront, triangles whose rows are long or short) are hit by construction
 rather than by luck of a hand-picked case.  Every case prints its name first.
 """
+import os
+
 import numpy as np
 import pytest
 import scipy.sparse as sps
@@ -15,7 +17,7 @@ from util import assert_close, assert_same, host, randn, to_dev
 
 pytestmark = pytest.mark.gpu
 
-SEEDS = list(range(24))
+SEEDS = list(range(int(os.environ.get("NM_SWEEP_SEEDS", "24"))))   # more seeds for a longer soak
 
 
 def _draw(seed, dtype, square=False):
