@@ -79,6 +79,51 @@ __device__ __forceinline__ T row_times_dense(T acc, int64_t kb0, int64_t ke0, co
 constexpr int kFlatRows = 8;
 constexpr int kScoutRows = 64;   // rows a scout workgroup inspects for long ones
 
+// The work of a "scout" workgroup (the first ceil(rows / kScoutRows) of the grid): look for
+// long rows among kScoutRows rows and share every one found among the workgroup's
+// wavefronts (contiguous parts, partial sums added in wavefront order: deterministic, equal
+// to the serial sum to rounding).  Lane = dense column.
+template <typename T, typename IDX, bool PERM>
+__device__ __forceinline__ void scout_long_rows(int64_t rows, const T *__restrict__ data,
+                                                const IDX *__restrict__ indices, const IDX *__restrict__ indptr,
+                                                const int32_t *__restrict__ perm, const T *__restrict__ B,
+                                                int64_t ldb, int64_t n, T *__restrict__ C, int64_t ldc, int lane,
+                                                int wave) {
+    __shared__ T s_part[kWavesPerBlock][kWave];
+    __shared__ int s_long[kScoutRows];
+    __shared__ int s_nlong;
+    const int64_t g0 = (int64_t)blockIdx.x * kScoutRows;
+    if (threadIdx.x == 0) s_nlong = 0;
+    __syncthreads();
+    for (int t = threadIdx.x; t < kScoutRows && g0 + t < rows; t += kBlock)
+        if (indptr[g0 + t + 1] - indptr[g0 + t] > kSplitRow) s_long[atomicAdd(&s_nlong, 1)] = t;
+    __syncthreads();
+    const int nl = s_nlong;
+    for (int li = 0; li < nl; ++li) {   // uniform over the workgroup; the order of the list does not matter
+        const int64_t row = g0 + s_long[li];
+        const int64_t rb = indptr[row], re = indptr[row + 1];
+        int64_t chunk = (re - rb + kWavesPerBlock - 1) / kWavesPerBlock;
+        chunk = (chunk + kWave - 1) / kWave * kWave;
+        const int64_t kb = rb + wave * chunk;
+        const int64_t ke = kb + chunk < re ? kb + chunk : re;
+        for (int64_t c0 = 0; c0 < n; c0 += kWave) {
+            const int64_t c = c0 + lane;
+            const bool live = c < n;
+            T acc = T(0);
+            if (kb < re)
+                acc = row_times_dense<T, IDX, PERM>(acc, kb, ke, data, indices, perm, B + (live ? c : 0), ldb, lane);
+            s_part[wave][lane] = acc;
+            __syncthreads();
+            if (wave == 0 && live) {
+                T sum = s_part[0][lane];
+                for (int w = 1; w < kWavesPerBlock; ++w) sum += s_part[w][lane];
+                C[row * ldc + c] = sum;
+            }
+            __syncthreads();
+        }
+    }
+}
+
 template <typename T, typename IDX, bool PERM>
 __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
     int64_t rows, const T *__restrict__ data, const IDX *__restrict__ indices,
@@ -95,39 +140,7 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
     // first in the grid so that this latency-bound work overlaps with the flat walk.
     const int64_t long_blocks = (rows + kScoutRows - 1) / kScoutRows;
     if ((int64_t)blockIdx.x < long_blocks) {
-        __shared__ T s_part[kWavesPerBlock][kWave];
-        __shared__ int s_long[kScoutRows];
-        __shared__ int s_nlong;
-        const int64_t g0 = (int64_t)blockIdx.x * kScoutRows;
-        if (threadIdx.x == 0) s_nlong = 0;
-        __syncthreads();
-        for (int t = threadIdx.x; t < kScoutRows && g0 + t < rows; t += kBlock)
-            if (indptr[g0 + t + 1] - indptr[g0 + t] > kSplitRow) s_long[atomicAdd(&s_nlong, 1)] = t;
-        __syncthreads();
-        const int nl = s_nlong;
-        for (int li = 0; li < nl; ++li) {   // uniform over the workgroup; the order of the list does not matter
-            const int64_t row = g0 + s_long[li];
-            const int64_t rb = indptr[row], re = indptr[row + 1];
-            int64_t chunk = (re - rb + kWavesPerBlock - 1) / kWavesPerBlock;
-            chunk = (chunk + kWave - 1) / kWave * kWave;
-            const int64_t kb = rb + wave * chunk;
-            const int64_t ke = kb + chunk < re ? kb + chunk : re;
-            for (int64_t c0 = 0; c0 < n; c0 += kWave) {
-                const int64_t c = c0 + lane;
-                const bool live = c < n;
-                T acc = T(0);
-                if (kb < re)
-                    acc = row_times_dense<T, IDX, PERM>(acc, kb, ke, data, indices, perm, B + (live ? c : 0), ldb, lane);
-                s_part[wave][lane] = acc;
-                __syncthreads();
-                if (wave == 0 && live) {
-                    T sum = s_part[0][lane];
-                    for (int w = 1; w < kWavesPerBlock; ++w) sum += s_part[w][lane];
-                    C[row * ldc + c] = sum;
-                }
-                __syncthreads();
-            }
-        }
+        scout_long_rows<T, IDX, PERM>(rows, data, indices, indptr, perm, B, ldb, n, C, ldc, lane, wave);
         return;
     }
     const int64_t r0 = (((int64_t)blockIdx.x - long_blocks) * kWavesPerBlock + wave) * kFlatRows;
@@ -407,6 +420,113 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
     }
 }
 
+// ---- narrow dense operands (n <= 32) -----------------------------------------------
+//
+// With lane = dense column, a 16-column operand leaves three quarters of every gather and
+// every multiply idle, and the kernels above take as long for n = 8 as for n = 64 (their time
+// is instruction issue and latency per ENTRY).  In the dot products of the backward a wavefront
+// therefore works on 64 / W entries per instruction, W = n rounded up to 8, 16 or 32: lane =
+// (entry slot, column); 1.03 -> 0.73 ms for the whole backward at n = 16 on the 1M x 1M
+// power-law matrix.  (The same mapping for the forward product, with the products of a chunk
+// staged in LDS and added per row in storage order, measured no faster than the wide kernel:
+// 0.41-0.77 ms against 0.51 ms, and was dropped.)
+
+// Sum over aligned groups of W lanes; every lane of the group gets it.
+template <int W, typename T> __device__ __forceinline__ T narrow_sum(T v) {
+    v += nm::dpp_move<0xB1>(v);                  // quad_perm [1,0,3,2]
+    v += nm::dpp_move<0x4E>(v);                  // quad_perm [2,3,0,1]
+    if (W == 8) v += nm::dpp_move<0x141>(v);     // row_half_mirror: the other quad of the 8
+    if (W >= 16) {
+        v += nm::dpp_move<0x124>(v);             // row_ror 4
+        v += nm::dpp_move<0x128>(v);             // row_ror 8
+    }
+    if (W == 32) v += __shfl_xor(v, 16, kWave);
+    return v;
+}
+
+// grad_A[k] = <gC[row(k), :], B[col(k), :]> for n <= W.  Entry-balanced like the wide kernel:
+// a wavefront owns 64 consecutive entries; every lane first finds the row of "its" entry by a
+// bisection over the ends of the next 64 rows (held one per lane), then the wavefront takes
+// 64 / W entries per step, four steps' gathers in flight.
+template <typename T, int W>
+__global__ __launch_bounds__(kBlock) void sddmm_narrow_kernel(
+    int64_t rows, int64_t nnz, const int64_t *__restrict__ indices, const int64_t *__restrict__ indptr,
+    const T *__restrict__ B, int64_t ldb, const T *__restrict__ gC, int64_t ldg, int n, T *__restrict__ grad_A,
+    const int32_t *__restrict__ chunk_row) {
+    constexpr int GPW = kWave / W;   // entries per step
+    constexpr int U = 4;             // steps per batch
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    const int64_t nchunks = (nnz + kWave - 1) / kWave;
+    const int slot = lane / W, c = lane % W;
+    const bool col_live = c < n;
+    const int cs = col_live ? c : 0;
+    for (int64_t ch = wave0; ch < nchunks; ch += nwaves) {
+        const int64_t kb = ch * kWave;
+        const int cnt = (int)(nnz - kb < kWave ? nnz - kb : kWave);
+        const int64_t k = kb + (lane < cnt ? lane : cnt - 1);
+        const int64_t mycol = indices[k];
+        int64_t row0;   // row of the chunk's first entry
+        if (chunk_row) {
+            row0 = chunk_row[ch];
+        } else {
+            int64_t lo = 0, hi = rows + 1;
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) >> 1;
+                if (indptr[mid] <= kb) lo = mid + 1; else hi = mid;
+            }
+            row0 = lo - 1;
+        }
+        // my entry's row: row0 + number of row ends at or before it
+        const int64_t er = row0 + 1 + lane;
+        const int64_t my_end = indptr[er <= rows ? er : rows];
+        int lo = 0, hi = kWave;
+#pragma unroll
+        for (int step = 0; step < 7; ++step) {   // 65 possible answers: seven halvings
+            const int mid = (lo + hi) >> 1;      // == 64 only once lo == hi == 64: the read is ignored then
+            const int64_t e = __shfl(my_end, mid & (kWave - 1), kWave);
+            if (lo < hi) {
+                if (e <= k) lo = mid + 1; else hi = mid;
+            }
+        }
+        int64_t myrow = row0 + lo;
+        if (lo == kWave) {   // more than 64 rows end inside this chunk (empty rows): look the row up
+            int64_t l2 = myrow, h2 = rows + 1;
+            while (l2 < h2) {
+                const int64_t mid = (l2 + h2) >> 1;
+                if (indptr[mid] <= k) l2 = mid + 1; else h2 = mid;
+            }
+            myrow = l2 - 1;
+        }
+        for (int j0 = 0; j0 < cnt; j0 += U * GPW) {
+            T gv[U], bv[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int j = j0 + u * GPW + slot;
+                const int js = j < cnt ? j : cnt - 1;
+                const int64_t col = __shfl(mycol, js, kWave), rw = __shfl(myrow, js, kWave);
+                gv[u] = gC[rw * ldg + cs];
+                bv[u] = B[col * ldb + cs];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int j = j0 + u * GPW + slot;
+                const T dot = narrow_sum<W>(col_live ? gv[u] * bv[u] : T(0));
+                if (c == 0 && j < cnt) grad_A[kb + j] = dot;
+            }
+        }
+    }
+}
+
+// Launches the forward product (A as delivered, or A^T through the plan).
+template <typename T, typename IDX, bool PERM>
+void launch_product(unsigned grid, hipStream_t s, int64_t rows, const T *data, const IDX *indices, const IDX *indptr,
+                    const int32_t *perm, const T *B, int64_t ldb, int64_t n, T *C, int64_t ldc) {
+    hipLaunchKernelGGL((spdmm_fwd_flat_kernel<T, IDX, PERM>), dim3(grid), dim3(kBlock), 0, s, rows, data, indices,
+                       indptr, perm, B, ldb, n, C, ldc);
+}
+
 int check_args(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
                const int64_t *indices, const int64_t *indptr, int64_t n) {
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
@@ -441,12 +561,11 @@ extern "C" int nm_spdmm_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t
     hipStream_t s = nm::as_stream(stream);
     const unsigned flat_grid = flat_grid_for(rows);
     if (dt == NM_F32)
-        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<float, int64_t, false>), dim3(flat_grid), dim3(kBlock), 0, s, rows,
-                           (const float *)data, indices, indptr, nullptr, (const float *)B, ldb, n, (float *)C, ldc);
+        launch_product<float, int64_t, false>(flat_grid, s, rows, (const float *)data, indices, indptr, nullptr,
+                                              (const float *)B, ldb, n, (float *)C, ldc);
     else
-        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<double, int64_t, false>), dim3(flat_grid), dim3(kBlock), 0, s, rows,
-                           (const double *)data, indices, indptr, nullptr, (const double *)B, ldb, n, (double *)C,
-                           ldc);
+        launch_product<double, int64_t, false>(flat_grid, s, rows, (const double *)data, indices, indptr, nullptr,
+                                               (const double *)B, ldb, n, (double *)C, ldc);
     NM_LAUNCH_CHECK("spdmm_fwd_flat_kernel");
     return NM_OK;
 }
@@ -477,6 +596,19 @@ int backward_impl(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const vo
     NM_REQUIRE(B != nullptr && gC != nullptr, "B or gC is null");
     NM_REQUIRE(ldb >= n && ldg >= n, "row stride smaller than the row");
     const dim3 grid(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock));
+    if (grad_A && !grad_B && n <= 32) {
+#define NM_NARROW(T, W)                                                                                          \
+    hipLaunchKernelGGL((sddmm_narrow_kernel<T, W>), grid, dim3(kBlock), 0, s, rows, nnz, indices, indptr,          \
+                       (const T *)B, ldb, (const T *)gC, ldg, (int)n, (T *)grad_A, chunk_row)
+        if (dt == NM_F32) {
+            if (n <= 8) NM_NARROW(float, 8); else if (n <= 16) NM_NARROW(float, 16); else NM_NARROW(float, 32);
+        } else {
+            if (n <= 8) NM_NARROW(double, 8); else if (n <= 16) NM_NARROW(double, 16); else NM_NARROW(double, 32);
+        }
+#undef NM_NARROW
+        NM_LAUNCH_CHECK("sddmm_narrow_kernel");
+        return NM_OK;
+    }
     const bool fast = grad_A && !grad_B && n <= kWave;
 #define NM_SDDMM(T, FAST)                                                                                         \
     hipLaunchKernelGGL((spdmm_bwd_kernel<T, FAST>), grid, dim3(kBlock), 0, s, rows, nnz, (const T *)data, indices, \
@@ -523,13 +655,11 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
     hipStream_t s = nm::as_stream(stream);
     const unsigned flat_grid = flat_grid_for(cols);
     if (dt == NM_F32)
-        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<float, int32_t, true>), dim3(flat_grid), dim3(kBlock), 0, s, cols,
-                           (const float *)data, t.t_row, t.t_indptr, t.t_perm, (const float *)gC, ldg, n,
-                           (float *)grad_B, ldgb);
+        launch_product<float, int32_t, true>(flat_grid, s, cols, (const float *)data, t.t_row, t.t_indptr, t.t_perm,
+                                             (const float *)gC, ldg, n, (float *)grad_B, ldgb);
     else
-        hipLaunchKernelGGL((spdmm_fwd_flat_kernel<double, int32_t, true>), dim3(flat_grid), dim3(kBlock), 0, s, cols,
-                           (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg, n,
-                           (double *)grad_B, ldgb);
+        launch_product<double, int32_t, true>(flat_grid, s, cols, (const double *)data, t.t_row, t.t_indptr,
+                                              t.t_perm, (const double *)gC, ldg, n, (double *)grad_B, ldgb);
     NM_LAUNCH_CHECK("spdmm_fwd_flat_kernel (transposed)");
     return NM_OK;
 }

@@ -58,7 +58,7 @@ def test_products(dev, seed, dtype):
     assert_same(host(gA), gA_ref, "spmv grad_A")
     assert_close(host(gx), gx_ref, "spmv grad_x")
     # SpMM at widths around the wavefront size
-    for n in (1, 7, 64, 65, 130)[seed % 2::2]:
+    for n in (1, 7, 16, 20, 32, 64, 65, 130)[seed % 2::2]:
         B, gC = randn(seed + 2, (cols, n), dtype), randn(seed + 3, (rows, n), dtype)
         Bd, gCd = to_dev(dev, B, gC)
         assert_close(host(ext.spdmm_forward(rows, cols, D, I, P, Bd)), oracle.spdmm_forward(rows, cols, d, i, p, B),
