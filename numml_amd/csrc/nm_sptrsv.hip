@@ -349,9 +349,11 @@ template <int PRE> __device__ __forceinline__ Vals<PRE> load_vals(const SolveArg
 // themselves (`Vals`, whose addresses come from the range).  A level takes a few
 // hundred cycles once its operands are in registers but a global load takes one to
 // two thousand, so with DEPTH = 1 every level waited for memory.
-template <int PRE, int DEPTH>
-__global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l0, int count, int step, int qlo,
-                                                              int qhi) {
+// MAXT: the largest workgroup the instantiation is launched with (512 leaves a wavefront twice the
+// registers of 1024, which the 16-deep pipeline needs to stay out of scratch memory).
+template <int PRE, int DEPTH, int MAXT = kNarrow>
+__global__ __launch_bounds__(MAXT) void sptrsv_ring_kernel(SolveArgs a, int l0, int count, int step, int qlo,
+                                                           int qhi) {
     __shared__ double ring[kRing];
     __shared__ int32_t s_lp[kMaxLevels + 1];
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
@@ -400,13 +402,18 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ring_kernel(SolveArgs a, int l
             }
             if (!in_ring) {
                 // slow path (a dependency older than the ring, or a row longer than the
-                // pipeline holds): redo the whole sum in the same order from global memory
+                // pipeline holds): redo the whole sum in the same order from global memory.
+                // The solutions of the first PRE dependencies are requested together (their
+                // slots are in registers; unused ones name a valid slot), the rest one by one.
+                double xg[PRE];
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) xg[e] = a.w.xs[cur.ds[e]];
                 acc = 0.;
-                for (int e = 0; e < n; ++e) {
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) acc += e < n ? cur.v[e] * xg[e] : 0.;
+                for (int e = PRE; e < n; ++e) {
                     const int32_t at = cur.m.dlo + e;
-                    const int32_t ds = e < PRE ? cur.ds[e] : a.dslot[at];
-                    const double v = e < PRE ? cur.v[e] : a.w.coef[at];
-                    acc += v * a.w.xs[ds];
+                    acc += a.w.coef[at] * a.w.xs[a.dslot[at]];
                 }
             }
             if (cur.m.live) {
@@ -702,12 +709,19 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
             const bool live = (int)threadIdx.x < cur.qe - cur.qb;
             if ((any & kEllFar) && live) {
                 // a dependency the ring does not hold: redo the sum in the same order from global memory
+                // (slots and then solutions are requested together; entries past the row's own
+                //  name a valid slot and are not added)
                 const int q = cur.qb + (int)threadIdx.x;
                 const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
+                int32_t sl[PRE];
+                double xg[PRE];
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
                 acc = 0.;
 #pragma unroll
-                for (int e = 0; e < PRE; ++e)
-                    if (e < n) acc += cur.v[e] * a.xs[a.dslot[dlo + e]];
+                for (int e = 0; e < PRE; ++e) acc += e < n ? cur.v[e] * xg[e] : 0.;
             }
             double xi = cur.bv - acc;
             if (!a.unit) xi /= cur.dv;
@@ -807,8 +821,14 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
                 hipLaunchKernelGGL((sptrsv_ring_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             else if (maxdep <= 4)
                 hipLaunchKernelGGL((sptrsv_ring_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
-            else
+            else if (maxdep <= 8)
                 hipLaunchKernelGGL((sptrsv_ring_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
+            else
+                // up to 16 dependencies through the register pipeline; longer rows take the slow path
+                if (L.block <= 512)
+                    hipLaunchKernelGGL((sptrsv_ring_kernel<16, 1, 512>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
+                else
+                    hipLaunchKernelGGL((sptrsv_ring_kernel<16, 1>), dim3(1), dim3(L.block), 0, s, a, l0, count, step, L.q0, L.q1);
             NM_LAUNCH_CHECK("sptrsv_ring_kernel");
         }
     }
