@@ -40,7 +40,13 @@ using nm::kWave;
 constexpr int32_t kEmpty = -1;
 constexpr int kBlock = 256;
 constexpr int kBins = 4;
-constexpr int kSpillGroups = 8;     // workgroups (and dense slices) of the spill path
+// Workgroups (and dense accumulator slices of B_cols entries each) of the spill path: as many as
+// fit a fixed budget of scratch, between 8 and 64.
+constexpr int64_t kSpillBudgetBytes = int64_t(192) << 20;
+inline int spill_groups(int64_t B_cols) {
+    const int64_t g = kSpillBudgetBytes / (12 * (B_cols + 1));
+    return (int)(g < 8 ? 8 : (g > 64 ? 64 : g));
+}
 constexpr int kSpillBlock = 1024;
 constexpr int kTablePad = 4;         // entries between the hash tables of neighbouring groups (16 bytes)
 constexpr int kAhead = 8;            // B rows whose first columns a group requests before inserting any
@@ -61,8 +67,8 @@ struct Work {
     int32_t *perm;     // [rows] rows grouped by bin
     int32_t *bins;     // [16]: count[0..3], offset[4..8], cursor[9..12]
     int64_t *scan;     // scan scratch
-    int32_t *mark;     // [kSpillGroups * B_cols]
-    double *acc;       // [kSpillGroups * B_cols]
+    int32_t *mark;     // [spill_groups(B_cols) * B_cols]
+    double *acc;       // [spill_groups(B_cols) * B_cols]
 };
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
@@ -78,8 +84,8 @@ size_t work_layout(int64_t rows, int64_t B_cols, void *base, Work *w) {
     int32_t *perm = (int32_t *)take((rows + 1) * 4);
     int32_t *bins = (int32_t *)take(16 * 4);
     int64_t *scan = (int64_t *)take(nm::scan_scratch_bytes(rows + 1));
-    int32_t *mark = (int32_t *)take((size_t)kSpillGroups * (B_cols + 1) * 4);
-    double *acc = (double *)take((size_t)kSpillGroups * (B_cols + 1) * 8);
+    int32_t *mark = (int32_t *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 4);
+    double *acc = (double *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 8);
     if (w) *w = Work{key, perm, bins, scan, mark, acc};
     return off;
 }
@@ -470,19 +476,23 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
                 h = (h + 1) & (TABLE - 1);
             }
         };
-        if (G <= kWave) {
+        {
             // Latency-lean walk: each lane fetches one entry of A's row together with the
-            // bounds of the B row it names; the first G columns of up to kAhead B rows are
-            // then requested back to back before any of them is inserted.
-            const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
+            // bounds of the B row it names; the first S columns of up to kAhead B rows are
+            // then requested back to back before any of them is inserted.  A group wider than
+            // a wavefront gives each of its wavefronts its own 64 entries of A's row (the
+            // order of insertion does not matter for the count).
+            constexpr int S = G < kWave ? G : kWave;
+            const int sl = gl & (S - 1), sub = G > kWave ? __builtin_amdgcn_readfirstlane(gl / S) : 0;
+            const int gbase = (threadIdx.x & (kWave - 1)) & ~(S - 1);
             row = live ? perm[idx] : 0;
             const int64_t ab = live ? A_indptr[row] : 0, ae = live ? A_indptr[row + 1] : 0;
-            for (int64_t a0 = ab; a0 < ae; a0 += G) {
-                const int64_t my_ai = a0 + gl;
+            for (int64_t a0 = ab + sub * S; a0 < ae; a0 += G) {
+                const int64_t my_ai = a0 + sl;
                 const bool mine = my_ai < ae;
                 const int64_t my_j = mine ? A_indices[my_ai] : 0;
                 const int64_t my_bb = mine ? B_indptr[my_j] : 0, my_be = mine ? B_indptr[my_j + 1] : 0;
-                const int nb = (int)(ae - a0 < G ? ae - a0 : G);
+                const int nb = (int)(ae - a0 < S ? ae - a0 : S);
                 for (int e0 = 0; e0 < nb; e0 += kAhead) {
                     int32_t pk[kAhead];
                     int64_t bbs[kAhead], bes[kAhead];
@@ -491,24 +501,16 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
                         const int src = gbase + (e0 + u < nb ? e0 + u : e0);
                         bbs[u] = __shfl(my_bb, src, kWave);
                         bes[u] = __shfl(my_be, src, kWave);
-                        const int64_t kk = bbs[u] + gl;
+                        const int64_t kk = bbs[u] + sl;
                         pk[u] = (e0 + u < nb && kk < bes[u]) ? (int32_t)B_indices[kk] : kEmpty;
                     }
 #pragma unroll
                     for (int u = 0; u < kAhead; ++u) {
                         if (e0 + u >= nb) break;
                         if (pk[u] != kEmpty) insert(pk[u]);
-                        for (int64_t kk = bbs[u] + G + gl; kk < bes[u]; kk += G) insert((int32_t)B_indices[kk]);
+                        for (int64_t kk = bbs[u] + S + sl; kk < bes[u]; kk += S) insert((int32_t)B_indices[kk]);
                     }
                 }
-            }
-        } else if (live) {
-            row = perm[idx];
-            const int64_t je = A_indptr[row + 1];
-            for (int64_t jj = A_indptr[row]; jj < je; ++jj) {
-                const int64_t j = A_indices[jj];
-                const int64_t ke = B_indptr[j + 1];
-                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) insert((int32_t)B_indices[kk]);
             }
         }
         cnt = group_total<G>(cnt, s_red);
@@ -632,47 +634,113 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
                 }
             }
         } else if (live) {
+            // One row per workgroup.  Every lane fetches one entry of A's row and the bounds of
+            // the B row it names into LDS (the compaction lists are free until the row is
+            // complete); the entries are then applied in order, the first G columns of kAhead
+            // B rows being requested before the first of them is added.
+            static_assert(G <= kWave || 2 * CSTRIDE * 4 >= G * (16 + (int)sizeof(T)), "staging area");
+            int64_t *s_bb = reinterpret_cast<int64_t *>(ck), *s_be = s_bb + G;
+            T *s_a = reinterpret_cast<T *>(s_be + G);
             row = perm[idx];
-            const int64_t je = A_indptr[row + 1];
-            for (int64_t jj = A_indptr[row]; jj < je; ++jj) {
-                const int64_t j = A_indices[jj];
-                const T a = A_data[jj];
-                const int64_t ke = B_indptr[j + 1];
-                for (int64_t kk = B_indptr[j] + gl; kk < ke; kk += G) add((int32_t)B_indices[kk], a * B_data[kk]);
-                group_sync<G>();  // the next entry of A's row adds after this one
+            const int64_t ab = A_indptr[row], ae = A_indptr[row + 1];
+            for (int64_t a0 = ab; a0 < ae; a0 += G) {
+                const int64_t my_ai = a0 + gl < ae ? a0 + gl : ab;
+                const int64_t my_j = A_indices[my_ai];
+                s_a[gl] = A_data[my_ai];
+                s_bb[gl] = B_indptr[my_j];
+                s_be[gl] = B_indptr[my_j + 1];
+                __syncthreads();
+                const int nb = (int)(ae - a0 < G ? ae - a0 : G);
+                for (int e0 = 0; e0 < nb; e0 += kAhead) {
+                    int32_t pk[kAhead];
+                    T pv[kAhead], as[kAhead];
+                    int64_t bbs[kAhead], bes[kAhead];
+#pragma unroll
+                    for (int u = 0; u < kAhead; ++u) {
+                        const int src = e0 + u < nb ? e0 + u : e0;
+                        bbs[u] = s_bb[src];
+                        bes[u] = s_be[src];
+                        as[u] = s_a[src];
+                        const int64_t kk = bbs[u] + gl;
+                        const bool ok = e0 + u < nb && kk < bes[u];
+                        pk[u] = ok ? (int32_t)B_indices[kk] : kEmpty;
+                        pv[u] = ok ? B_data[kk] : T(0);
+                    }
+#pragma unroll
+                    for (int u = 0; u < kAhead; ++u) {
+                        if (e0 + u >= nb) break;
+                        if (pk[u] != kEmpty) add(pk[u], as[u] * pv[u]);
+                        for (int64_t kk = bbs[u] + G + gl; kk < bes[u]; kk += G)
+                            add((int32_t)B_indices[kk], as[u] * B_data[kk]);
+                        __syncthreads();  // the next entry of A's row adds after this one
+                    }
+                }
             }
         }
         if (G > kWave) __syncthreads();
-        // Output in ascending column order: the occupied slots are compacted into a dense
-        // list, then every entry is ranked against that list only (its rank is its position
-        // in the row).  Rows fill at most half of their table, so this is a fraction of the
-        // compares a rank over the whole table would take.
-        {
+        // Output in ascending column order.
+        if constexpr (G > kWave) {
+            // One row per workgroup, up to TABLE / 2 entries: the occupied slots are compacted
+            // into a list of (column, slot) words, the list is padded to a power of two and
+            // sorted by a bitonic network in LDS, and the row is written out in order.  (Ranking
+            // every entry against the whole list, as the narrow groups do, grows with the square
+            // of the row and took most of this kernel's time on rows of thousands of entries.)
+            unsigned long long *list = reinterpret_cast<unsigned long long *>(ck);
+            int *scr = reinterpret_cast<int *>(cs);
             int mine = 0;
             for (int t = gl; t < TABLE; t += G) mine += tab[t] != kEmpty;
-            int incl = mine, c;
-            if (G <= kWave) {
-                const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
-#pragma unroll
-                for (int off = 1; off < G; off <<= 1) {
-                    const int up = __shfl_up(incl, off, kWave);
-                    if (gl >= off) incl += up;
-                }
-                c = __shfl(incl, gbase + G - 1, kWave);
-            } else {
-                // one row per workgroup: scan through LDS (ck doubles as scratch before it is filled)
-                int *scr = reinterpret_cast<int *>(cs);
-                scr[gl] = mine;
-                __syncthreads();
-                incl = 0;
-                c = 0;
-                for (int l2 = 0; l2 < G; ++l2) {
-                    const int v = scr[l2];
-                    if (l2 <= gl) incl += v;
-                    c += v;
-                }
-                __syncthreads();
+            scr[gl] = mine;
+            __syncthreads();
+            int pos = 0, c = 0;
+            for (int l2 = 0; l2 < G; ++l2) {
+                const int v = scr[l2];
+                if (l2 < gl) pos += v;
+                c += v;
             }
+            __syncthreads();
+            for (int t = gl; t < TABLE; t += G) {
+                const int32_t key = tab[t];
+                if (key != kEmpty) list[pos++] = ((unsigned long long)(uint32_t)key << 32) | (uint32_t)t;
+            }
+            int P = 2 * kWave;
+            while (P < c) P <<= 1;
+            for (int t = c + gl; t < P; t += G) list[t] = ~0ull;
+            __syncthreads();
+            for (int k = 2; k <= P; k <<= 1) {
+                for (int j = k >> 1; j > 0; j >>= 1) {
+                    for (int t = gl; t < P / 2; t += G) {
+                        const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1)), l = i | j;
+                        const unsigned long long x = list[i], y = list[l];
+                        if ((x > y) == ((i & k) == 0)) { list[i] = y; list[l] = x; }
+                    }
+                    // a wavefront's pairs stay inside its own 128 words while j <= 64
+                    if (j > kWave) __syncthreads(); else group_sync<kWave>();
+                }
+                if (k >= 2 * kWave) __syncthreads();
+            }
+            if (live) {
+                const int64_t base = C_indptr[row];
+                for (int e = gl; e < c; e += G) {
+                    const unsigned long long w = list[e];
+                    C_indices[base + e] = (int64_t)(w >> 32);
+                    C_data[base + e] = val[(uint32_t)w];
+                }
+            }
+        } else {
+            // The occupied slots are compacted into a dense list, then every entry is ranked
+            // against that list only (its rank is its position in the row).  Rows fill at most
+            // half of their table, so this is a fraction of the compares a rank over the whole
+            // table would take.
+            const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
+            int mine = 0;
+            for (int t = gl; t < TABLE; t += G) mine += tab[t] != kEmpty;
+            int incl = mine;
+#pragma unroll
+            for (int off = 1; off < G; off <<= 1) {
+                const int up = __shfl_up(incl, off, kWave);
+                if (gl >= off) incl += up;
+            }
+            const int c = __shfl(incl, gbase + G - 1, kWave);
             int pos = incl - mine;
             for (int t = gl; t < TABLE; t += G) {
                 const int32_t key = tab[t];
@@ -743,17 +811,34 @@ __global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
         const int64_t c_lo = (int64_t)s_lo, c_hi = (int64_t)s_hi;
         int64_t out = C_indptr[row];
         if (s_lo != ~0ull) {
-            for (int64_t c0 = c_lo; c0 <= c_hi; c0 += kSpillBlock) {
-                const int64_t c = c0 + threadIdx.x;
-                const bool hit = c <= c_hi && mark[c] == stamp;
-                int64_t total;
-                const int64_t pre = nm::block_exclusive_scan(hit ? 1 : 0, s_wave, total);
+            // Every wavefront takes a contiguous segment of the touched column range: it counts its
+            // hits, the counts are summed over the wavefronts before it, and it then emits its
+            // segment in order.  (A workgroup-wide scan per 1024 columns cost two barriers each.)
+            constexpr int kWaves = kSpillBlock / kWave;
+            const int64_t span = c_hi - c_lo + 1;
+            const int64_t seg = ((span + kWaves - 1) / kWaves + kWave - 1) / kWave * kWave;
+            const int64_t sb = c_lo + wave * seg;
+            const int64_t se = sb + seg < c_hi + 1 ? sb + seg : c_hi + 1;
+            int64_t cnt = 0;
+            for (int64_t c0 = sb; c0 < se; c0 += kWave) {
+                const int64_t c = c0 + lane;
+                cnt += __popcll(__ballot(c < se && mark[c] == stamp));
+            }
+            if (lane == 0) s_wave[wave] = cnt;
+            __syncthreads();
+            for (int w = 0; w < wave; ++w) out += s_wave[w];
+            const unsigned long long below = (1ull << lane) - 1ull;
+            for (int64_t c0 = sb; c0 < se; c0 += kWave) {
+                const int64_t c = c0 + lane;
+                const bool hit = c < se && mark[c] == stamp;
+                const unsigned long long m = __ballot(hit);
                 if (hit) {
-                    C_indices[out + pre] = c;
-                    C_data[out + pre] = acc[c];
+                    const int64_t at = out + __popcll(m & below);
+                    C_indices[at] = c;
+                    C_data[at] = acc[c];
                     acc[c] = T(0);
                 }
-                out += total;
+                out += __popcll(m);
             }
         }
         __syncthreads();
@@ -771,8 +856,23 @@ __global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
 // units are bound by lines touched, not by lanes).  The products
 // gC[i,c] * B[k,c] are then added lane by lane in ascending column order --
 // the order of the reference's merge -- which keeps grad_A bit-identical.
+//
+// Rows of C longer than kBwdLong go to a second kernel in which a whole
+// workgroup owns the row: its 32 groups share out the entries of A's row, whole
+// wavefronts take the entries whose row of B is long, and the row of C is staged
+// in LDS -- columns and gradient up to kBwdLongCap entries; columns only beyond
+// that (every stride-th column past kBwdHugeCap entries: the last steps of the
+// search then read global memory).
+// Left to one group of eight lanes, a row with thousands of products and a
+// global-memory search per product set the time of the whole launch.
 constexpr int kBwdG = 8;
 constexpr int kBwdStage = 64;
+constexpr int kBwdLong = 256;
+constexpr int kBwdLongCap = 2048;     // rows up to this long: columns and gradient in LDS
+constexpr int kBwdHugeCap = 14336;    // longer rows: columns only
+constexpr int kBwdLongChunk = 256;   // rows a workgroup of the long-row kernel looks through at a time
+constexpr int kBwdWide = 64;         // rows of B longer than this are walked by a whole wavefront ...
+constexpr int kBwdWideCap = 1024;    // ... up to this many per row of A (the rest stay with their group)
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
@@ -800,7 +900,8 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
                 cg[t] = gC[cb + t];
             }
         group_sync<G>();
-        const int64_t ab = live ? A_indptr[i] : 0, ae = live ? A_indptr[i + 1] : 0;
+        const bool here = live && clen <= kBwdLong;   // longer rows are left to spgemm_bwd_long_kernel
+        const int64_t ab = here ? A_indptr[i] : 0, ae = here ? A_indptr[i + 1] : 0;
         for (int64_t a0 = ab; a0 < ae; a0 += G) {
             // each lane fetches one entry of A's row and the bounds of the B row it names
             const int64_t my_ai = a0 + gl;
@@ -856,6 +957,135 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
     }
 }
 
+template <typename T, int CAP, bool STAGE_G>
+__global__ __launch_bounds__(kBlock) void spgemm_bwd_long_kernel(
+    int64_t A_rows, int64_t longer_than, int64_t up_to, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
+    const int64_t *__restrict__ C_indptr, const T *__restrict__ A_data,
+    const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
+    const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
+    const int64_t *__restrict__ B_indptr, T *__restrict__ grad_A, T *__restrict__ grad_B) {
+    constexpr int G = kBwdG, GROUPS = kBlock / G;
+    __shared__ T cg[STAGE_G ? CAP : 1];
+    __shared__ int32_t ci[CAP];
+    __shared__ int s_long[kBwdLongChunk];
+    __shared__ int s_wide[kBwdWideCap];
+    __shared__ int s_n, s_nw;
+    const int gl = threadIdx.x % G, gi = threadIdx.x / G;
+    const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    for (int64_t r0 = (int64_t)blockIdx.x * kBwdLongChunk; r0 < A_rows; r0 += (int64_t)gridDim.x * kBwdLongChunk) {
+        // the long rows among this chunk of rows (mostly there are none)
+        const int64_t r = r0 + threadIdx.x;
+        bool is_long = false;
+        if (threadIdx.x < kBwdLongChunk && r < A_rows) {
+            const int64_t len = C_indptr[r + 1] - C_indptr[r];
+            is_long = len > longer_than && len <= up_to;
+        }
+        if (!__syncthreads_or(is_long)) continue;
+        if (threadIdx.x == 0) s_n = 0;
+        __syncthreads();
+        if (is_long) s_long[atomicAdd(&s_n, 1)] = threadIdx.x;
+        __syncthreads();
+        const int n = s_n;
+        for (int q = 0; q < n; ++q) {
+            const int64_t i = r0 + s_long[q];
+            const int64_t cb = C_indptr[i], ce = C_indptr[i + 1], clen = ce - cb;
+            const int64_t stride = (clen + CAP - 1) / CAP;
+            const int ns = (int)((clen + stride - 1) / stride);
+            const bool whole = stride == 1;
+            for (int t = threadIdx.x; t < ns; t += kBlock) {
+                ci[t] = (int32_t)C_indices[cb + t * stride];
+                if (STAGE_G) cg[t] = gC[cb + t];   // STAGE_G kernels only get rows of at most CAP entries
+            }
+            if (threadIdx.x == 0) s_nw = 0;
+            __syncthreads();
+            // One entry (i,k) of A: W lanes (lane wl of them, the first being lane wbase of the
+            // wavefront) walk row k of B; returns sum_c gC[i,c] * B[k,c] added in ascending c.
+            auto entry = [&](auto width, int wl, int wbase, int64_t bb, int64_t be, T a) -> T {
+                constexpr int W = decltype(width)::value;
+                T acc = 0;
+                for (int64_t kk0 = bb; kk0 < be; kk0 += W) {
+                    const int64_t kk = kk0 + wl;
+                    const bool have = kk < be;
+                    const int64_t c = have ? B_indices[kk] : -1;
+                    const T bval = have ? B_data[kk] : T(0);
+                    int l = 0, h = ns;
+                    while (l < h) {
+                        const int mid = (l + h) >> 1;
+                        if ((int64_t)ci[mid] < c) l = mid + 1; else h = mid;
+                    }
+                    bool hit;
+                    T g = 0;
+                    if (whole) {
+                        hit = have && l < ns && (int64_t)ci[l] == c;
+                        if (hit) g = STAGE_G ? cg[l] : gC[cb + l];
+                    } else {
+                        // sample l is the first one not below c: the column, if present, sits
+                        // after sample l - 1 and no later than sample l
+                        int64_t lo = l == 0 ? 0 : (int64_t)(l - 1) * stride + 1;
+                        int64_t hi = (int64_t)l * stride < clen ? (int64_t)l * stride : clen;
+                        if (!have) hi = lo;
+                        while (lo < hi) {
+                            const int64_t mid = (lo + hi) >> 1;
+                            if (C_indices[cb + mid] < c) lo = mid + 1; else hi = mid;
+                        }
+                        hit = have && lo < clen && C_indices[cb + lo] == c;
+                        if (hit) g = gC[cb + lo];
+                    }
+                    if (hit && grad_B) nm::atomic_add(grad_B + kk, a * g);
+                    const T prod = hit ? g * bval : T(0);
+                    // ordered sum over the lanes = ascending column
+                    const int cnt = (int)(be - kk0 < W ? be - kk0 : W);
+                    for (int l2 = 0; l2 < cnt; ++l2) {
+                        const T pl = __shfl(prod, wbase + l2, kWave);
+                        const int hl = __shfl((int)hit, wbase + l2, kWave);
+                        if (hl) acc += pl;
+                    }
+                }
+                return acc;
+            };
+            const int64_t ab = A_indptr[i], ae = A_indptr[i + 1];
+            // entries of A's row per group and pass: as few as keeps all groups busy
+            const int64_t even = (ae - ab + GROUPS - 1) / GROUPS;
+            const int per = (int)(even < 1 ? 1 : (even > G ? G : even));
+            for (int64_t a0 = ab + gi * per; a0 < ae; a0 += GROUPS * per) {
+                const int64_t my_ai = a0 + gl;
+                const bool mine = gl < per && my_ai < ae;
+                const int64_t my_k = mine ? A_indices[my_ai] : 0;
+                const T my_a = (mine && grad_B) ? A_data[my_ai] : T(0);
+                const int64_t my_bb = mine ? B_indptr[my_k] : 0, my_be = mine ? B_indptr[my_k + 1] : 0;
+                // entries whose row of B is long are set aside for a whole wavefront
+                bool later = false;
+                if (mine && my_be - my_bb > kBwdWide) {
+                    const int slot = atomicAdd(&s_nw, 1);
+                    later = slot < kBwdWideCap;
+                    if (later) s_wide[slot] = (int)(my_ai - ab);
+                }
+                const int nb = (int)(ae - a0 < per ? ae - a0 : per);
+                T my_acc = 0;
+                for (int e = 0; e < nb; ++e) {
+                    if (__shfl((int)later, gbase + e, kWave)) continue;
+                    const int64_t bb = __shfl(my_bb, gbase + e, kWave), be = __shfl(my_be, gbase + e, kWave);
+                    const T a = __shfl(my_a, gbase + e, kWave);
+                    const T acc = entry(std::integral_constant<int, G>{}, gl, gbase, bb, be, a);
+                    if (gl == e) my_acc = acc;
+                }
+                if (mine && !later && grad_A) grad_A[my_ai] = my_acc;
+            }
+            __syncthreads();
+            const int nw = s_nw < kBwdWideCap ? s_nw : kBwdWideCap;
+            for (int d = wave; d < nw; d += kBlock / kWave) {
+                const int64_t ai = ab + s_wide[d];
+                const int64_t k = A_indices[ai];
+                const T a = grad_B ? A_data[ai] : T(0);
+                const T acc = entry(std::integral_constant<int, kWave>{}, lane, 0, B_indptr[k], B_indptr[k + 1], a);
+                if (lane == 0 && grad_A) grad_A[ai] = acc;
+            }
+            __syncthreads();
+        }
+    }
+}
+
 int check_common(int64_t A_rows, int64_t B_cols) {
     NM_REQUIRE(A_rows >= 0 && B_cols >= 0, "negative size");
     if (A_rows >= 0x7ffffffe || B_cols >= 0x7ffffffe)
@@ -894,7 +1124,7 @@ int launch_numeric(const Work &w, int64_t B_cols, const void *A_data, const int6
                            B_indices, B_indptr, C_indptr, C_indices, Cd);
         NM_LAUNCH_CHECK("numeric_hash_kernel<256>");
     }
-    hipLaunchKernelGGL(numeric_spill_kernel<T>, dim3(kSpillGroups), dim3(kSpillBlock), 0, s, w.bins, w.perm,
+    hipLaunchKernelGGL(numeric_spill_kernel<T>, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm,
                        B_cols, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd, w.mark,
                        w.acc);
     NM_LAUNCH_CHECK("numeric_spill_kernel");
@@ -940,7 +1170,7 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     hipLaunchKernelGGL((symbolic_hash_kernel<256, kSymTable2>), dim3(1024), dim3(kBlock), 0, s, 2, w.bins, w.perm,
                        A_indices, A_indptr, B_indices, B_indptr, C_indptr);
     NM_LAUNCH_CHECK("symbolic_hash_kernel<256>");
-    hipLaunchKernelGGL(symbolic_spill_kernel, dim3(kSpillGroups), dim3(kSpillBlock), 0, s, w.bins, w.perm, B_cols,
+    hipLaunchKernelGGL(symbolic_spill_kernel, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm, B_cols,
                        A_indices, A_indptr, B_indices, B_indptr, w.mark, C_indptr);
     NM_LAUNCH_CHECK("symbolic_spill_kernel");
     // counts sit in C_indptr[0, rows), C_indptr[rows] = 0: the exclusive scan is the row pointer
@@ -1009,5 +1239,23 @@ extern "C" int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, in
                            (const double *)gC, C_indices, C_indptr, (const double *)A_data, A_indices, A_indptr,
                            (const double *)B_data, B_indices, B_indptr, (double *)grad_A, (double *)grad_B);
     NM_LAUNCH_CHECK("spgemm_bwd_kernel");
+    grid = nm::ceil_div(A_rows, kBwdLongChunk);
+    if (grid > 1024) grid = 1024;
+    const int64_t none = INT64_MAX;
+#define NM_BWD_LONG(T)                                                                                          \
+    do {                                                                                                        \
+        hipLaunchKernelGGL((spgemm_bwd_long_kernel<T, kBwdLongCap, true>), dim3((unsigned)grid), dim3(kBlock),  \
+                           0, s, A_rows, (int64_t)kBwdLong, (int64_t)kBwdLongCap, (const T *)gC, C_indices,     \
+                           C_indptr, (const T *)A_data, A_indices, A_indptr, (const T *)B_data, B_indices,      \
+                           B_indptr, (T *)grad_A, (T *)grad_B);                                                 \
+        hipLaunchKernelGGL((spgemm_bwd_long_kernel<T, kBwdHugeCap, false>), dim3((unsigned)grid), dim3(kBlock), \
+                           0, s, A_rows, (int64_t)kBwdLongCap, none, (const T *)gC, C_indices, C_indptr,        \
+                           (const T *)A_data, A_indices, A_indptr, (const T *)B_data, B_indices, B_indptr,      \
+                           (T *)grad_A, (T *)grad_B);                                                           \
+    } while (0)
+    if (dt == NM_F32) NM_BWD_LONG(float);
+    else NM_BWD_LONG(double);
+#undef NM_BWD_LONG
+    NM_LAUNCH_CHECK("spgemm_bwd_long_kernel");
     return NM_OK;
 }
