@@ -152,10 +152,13 @@ __global__ __launch_bounds__(kBlock) void diagonal_kernel(int64_t rows, const T 
 // global memory would take a round trip each) and leaves, for every output entry,
 // which entry of A and/or of B feeds it.  The output is finally produced lane =
 // output entry: values are fetched and C is written through coalesced accesses.
-// Tiles with more than kLcCap entries in either operand fall back to one lane per
-// row straight from global memory.
+// A tile whose rows hold more than kLcCap entries of either operand is worked off in
+// runs of consecutive rows that do fit; a single row that does not is merged by the
+// whole workgroup from global memory (every entry finds its place in the output by a
+// bisection of the other operand's row and a count of the shared columns before it).
 
 constexpr int kLcRows = 256, kLcCap = 2304;
+constexpr int32_t kLcHuge = 1 << 30;   // tiles with this many entries: one lane per row from global memory
 constexpr uint32_t kLcNone = 0xffff;
 
 // dst[k] = (int32) src[k] for k < n, by the whole workgroup.  K loads per lane are requested
@@ -183,7 +186,7 @@ __device__ __forceinline__ void lc_stage_offsets(const int64_t *__restrict__ ind
     const int64_t base = indptr[r0];
     for (int t = threadIdx.x; t <= nr; t += kBlock) {
         const int64_t d = indptr[r0 + t] - base;
-        off[t] = (int32_t)(d > kLcCap ? kLcCap + 1 : d);
+        off[t] = (int32_t)(d > kLcHuge ? kLcHuge : d);
     }
 }
 
@@ -223,6 +226,82 @@ __device__ __forceinline__ void lc_row_global(int64_t row, T alpha, const T *__r
     }
 }
 
+// End of the run of rows that starts at row s0 of the tile and fits the LDS arrays:
+// the largest e in [s0, nr] with at most capA (capB) entries of the first (second)
+// operand in rows [s0, e).  e == s0 when row s0 alone is too long.
+__device__ __forceinline__ int lc_run_end(const int32_t *offA, const int32_t *offB, int s0, int nr, int capA,
+                                          int capB) {
+    auto fits = [&](int e) { return offA[e] - offA[s0] <= capA && offB[e] - offB[s0] <= capB; };
+    if (fits(nr)) return nr;
+    int lo = s0, hi = nr;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (fits(mid)) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// One long row merged by the whole workgroup from global memory.  Output position of
+// an entry = entries of its own row before it + entries of the other row below its
+// column - columns both rows hold below it.
+template <typename T, bool COUNT>
+__device__ __forceinline__ void lc_long_row(int64_t row, T alpha, const T *__restrict__ A_data,
+                                            const int64_t *__restrict__ A_indices,
+                                            const int64_t *__restrict__ A_indptr, T beta,
+                                            const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
+                                            const int64_t *__restrict__ B_indptr, int64_t *__restrict__ C_indptr,
+                                            int64_t *__restrict__ C_indices, T *__restrict__ C_data,
+                                            int64_t *s_scan) {
+    const int64_t a0 = A_indptr[row], m = A_indptr[row + 1] - a0;
+    const int64_t b0 = B_indptr[row], n = B_indptr[row + 1] - b0;
+    const int64_t out0 = COUNT ? 0 : C_indptr[row];
+    int64_t shared = 0;
+    for (int64_t p0 = 0; p0 < m; p0 += kBlock) {
+        const int64_t p = p0 + threadIdx.x;
+        const bool have = p < m;
+        const int64_t cA = have ? A_indices[a0 + p] : 0;
+        int64_t lo = 0, hi = have ? n : 0;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (B_indices[b0 + mid] < cA) lo = mid + 1; else hi = mid;
+        }
+        const bool both = have && lo < n && B_indices[b0 + lo] == cA;
+        int64_t total;
+        const int64_t before = nm::block_exclusive_scan(both ? 1 : 0, s_scan, total);
+        if (!COUNT && have) {
+            const int64_t o = out0 + p + lo - (shared + before);
+            const T pa = alpha * A_data[a0 + p];
+            C_indices[o] = cA;
+            C_data[o] = both ? pa + beta * B_data[b0 + lo] : pa;
+        }
+        shared += total;
+    }
+    if (COUNT) {
+        if (threadIdx.x == 0) C_indptr[row] = m + n - shared;
+        return;
+    }
+    shared = 0;
+    for (int64_t q0 = 0; q0 < n; q0 += kBlock) {
+        const int64_t q = q0 + threadIdx.x;
+        const bool have = q < n;
+        const int64_t cB = have ? B_indices[b0 + q] : 0;
+        int64_t lo = 0, hi = have ? m : 0;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (A_indices[a0 + mid] < cB) lo = mid + 1; else hi = mid;
+        }
+        const bool both = have && lo < m && A_indices[a0 + lo] == cB;
+        int64_t total;
+        const int64_t before = nm::block_exclusive_scan(both ? 1 : 0, s_scan, total);
+        if (have && !both) {
+            const int64_t o = out0 + q + lo - (shared + before);
+            C_indices[o] = cB;
+            C_data[o] = beta * B_data[b0 + q];
+        }
+        shared += total;
+    }
+}
+
 template <typename T, bool COUNT>
 __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, const T *__restrict__ A_data,
                                                          const int64_t *__restrict__ A_indices,
@@ -233,6 +312,7 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
                                                          int64_t *__restrict__ C_indptr,
                                                          int64_t *__restrict__ C_indices, T *__restrict__ C_data) {
     __shared__ LcTile s;
+    __shared__ int64_t s_scan[kBlock / nm::kWave];
     const int64_t ntiles = nm::ceil_div(rows, kLcRows), npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t tile = nm::xcd_tile(id, npad);
@@ -243,17 +323,29 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
         lc_stage_offsets(A_indptr, r0, nr, s.offA);
         lc_stage_offsets(B_indptr, r0, nr, s.offB);
         __syncthreads();
-        const int nA = s.offA[nr], nB = s.offB[nr];
-        if (nA <= kLcCap && nB <= kLcCap) {
-            lc_stage_cols<5>(s.colA, A_indices + baseA, nA);
-            lc_stage_cols<5>(s.colB, B_indices + baseB, nB);
-            const int64_t baseC = COUNT ? 0 : C_indptr[r0];
-            if (!COUNT)
-                for (int t = threadIdx.x; t <= nr; t += kBlock) s.offC[t] = (int32_t)(C_indptr[r0 + t] - baseC);
+        if (s.offA[nr] >= kLcHuge || s.offB[nr] >= kLcHuge) {
+            for (int t = threadIdx.x; t < nr; t += kBlock)
+                lc_row_global<T, COUNT>(r0 + t, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr,
+                                        C_indptr, C_indices, C_data);
             __syncthreads();
-            for (int t = threadIdx.x; t < nr; t += kBlock) {
-                int iA = s.offA[t], iB = s.offB[t];
-                const int eA = s.offA[t + 1], eB = s.offB[t + 1];
+            continue;
+        }
+        // rows [s0, e0) of the tile through LDS; WHOLE: the whole tile (s0 == 0), the common
+        // case, compiled without the run's offsets
+        auto run = [&](auto whole, const int s0, const int e0) {
+            constexpr bool WHOLE = decltype(whole)::value;
+            const int n = e0 - s0, a0 = WHOLE ? 0 : s.offA[s0], b0 = WHOLE ? 0 : s.offB[s0];
+            const int nA = s.offA[e0] - a0, nB = s.offB[e0] - b0;
+            const int64_t rs = r0 + s0, gA = baseA + a0, gB = baseB + b0;
+            lc_stage_cols<5>(s.colA, A_indices + gA, nA);
+            lc_stage_cols<5>(s.colB, B_indices + gB, nB);
+            const int64_t gC = COUNT ? 0 : C_indptr[rs];
+            if (!COUNT)
+                for (int t = threadIdx.x; t <= n; t += kBlock) s.offC[t] = (int32_t)(C_indptr[rs + t] - gC);
+            __syncthreads();
+            for (int t = threadIdx.x; t < n; t += kBlock) {
+                int iA = s.offA[s0 + t] - a0, iB = s.offB[s0 + t] - b0;
+                const int eA = s.offA[s0 + t + 1] - a0, eB = s.offB[s0 + t + 1] - b0;
                 int out = COUNT ? 0 : s.offC[t];
                 while (iA < eA && iB < eB) {
                     const int32_t cA = s.colA[iA], cB = s.colB[iB];
@@ -263,7 +355,7 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
                     ++out;
                 }
                 if (COUNT) {
-                    C_indptr[r0 + t] = out + (eA - iA) + (eB - iB);
+                    C_indptr[rs + t] = out + (eA - iA) + (eB - iB);
                 } else {
                     for (; iA < eA; ++iA, ++out) s.src[out] = (uint32_t)iA | (kLcNone << 16);
                     for (; iB < eB; ++iB, ++out) s.src[out] = kLcNone | ((uint32_t)iB << 16);
@@ -271,13 +363,13 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
             }
             if (!COUNT) {
                 __syncthreads();
-                const int nC = s.offC[nr];
+                const int nC = s.offC[n];
                 // K output entries per lane: their operand values are requested together and
-                // unconditionally (an operand that is absent reads entry 0 of a tile that has one
+                // unconditionally (an operand that is absent reads entry 0 of a run that has one
                 // and is dropped by the select), then combined and stored.
                 constexpr int K = 5;
-                const T *__restrict__ Ad = nA > 0 ? A_data + baseA : B_data + baseB;
-                const T *__restrict__ Bd = nB > 0 ? B_data + baseB : A_data + baseA;
+                const T *__restrict__ Ad = nA > 0 ? A_data + gA : B_data + gB;
+                const T *__restrict__ Bd = nB > 0 ? B_data + gB : A_data + gA;
                 for (int o0 = threadIdx.x; o0 < nC; o0 += K * kBlock) {
                     uint32_t ia[K], ib[K];
                     T va[K], vb[K];
@@ -296,24 +388,36 @@ __global__ __launch_bounds__(kBlock) void lincomb_kernel(int64_t rows, T alpha, 
                         const T pa = alpha * va[u], pb = beta * vb[u];
                         const T v = ib[u] == kLcNone ? pa : (ia[u] == kLcNone ? pb : pa + pb);
                         const int32_t c = ia[u] == kLcNone ? s.colB[ib[u]] : s.colA[ia[u]];
-                        nm::stream_store(C_indices + baseC + o, (int64_t)c);
-                        nm::stream_store(C_data + baseC + o, v);
+                        nm::stream_store(C_indices + gC + o, (int64_t)c);
+                        nm::stream_store(C_data + gC + o, v);
                     }
                 }
             }
-        } else {
-            for (int t = threadIdx.x; t < nr; t += kBlock)
-                lc_row_global<T, COUNT>(r0 + t, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr,
-                                        C_indptr, C_indices, C_data);
+            __syncthreads();
+        };
+        if (lc_run_end(s.offA, s.offB, 0, nr, kLcCap, kLcCap) == nr) {
+            run(std::true_type{}, 0, nr);
+            continue;
         }
-        __syncthreads();
+        for (int s0 = 0; s0 < nr;) {
+            const int e0 = lc_run_end(s.offA, s.offB, s0, nr, kLcCap, kLcCap);
+            if (e0 == s0) {
+                lc_long_row<T, COUNT>(r0 + s0, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr,
+                                      C_indptr, C_indices, C_data, s_scan);
+                s0 += 1;
+                continue;
+            }
+            run(std::false_type{}, s0, e0);
+            s0 = e0;
+        }
     }
 }
 
 // grad_X[k] = coef * grad_C at the same coordinate (cpp/sparse_csr_cpu.cpp:505-552).
-// Every column of X is present in C.  Same tiling: columns of X and of C staged in
-// LDS, one lane per row marks the row of its entries of X, then lane = entry of X
-// finds its column in the row of C by bisection in LDS, gathers and scales.
+// Every column of X is present in C.  Same tiling and the same runs of rows: columns
+// of X and of C staged in LDS, one lane per row marks the row of its entries of X, then
+// lane = entry of X finds its column in the row of C by bisection in LDS, gathers and
+// scales.  A row too long for LDS is searched in global memory by the whole workgroup.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void lincomb_back_kernel(int64_t rows, T coef,
                                                               const int64_t *__restrict__ X_indices,
@@ -332,20 +436,51 @@ __global__ __launch_bounds__(kBlock) void lincomb_back_kernel(int64_t rows, T co
         const int nr = (int)(rows - r0 < kLcRows ? rows - r0 : kLcRows);
         const int64_t baseX = X_indptr[r0], baseC = C_indptr[r0];
         lc_stage_offsets(X_indptr, r0, nr, s_offX);
-        for (int t = threadIdx.x; t <= nr; t += kBlock) {
-            const int64_t d = C_indptr[r0 + t] - baseC;
-            s_offC[t] = (int32_t)(d > 2 * kLcCap ? 2 * kLcCap + 1 : d);
-        }
+        lc_stage_offsets(C_indptr, r0, nr, s_offC);
         __syncthreads();
-        const int nX = s_offX[nr], nC = s_offC[nr];
-        if (nX <= kLcCap && nC <= 2 * kLcCap) {
-            lc_stage_cols<5>(s_colX, X_indices + baseX, nX);
-            lc_stage_cols<5>(s_colC, C_indices + baseC, nC);
+        if (s_offX[nr] >= kLcHuge || s_offC[nr] >= kLcHuge) {
+            for (int t = threadIdx.x; t < nr; t += kBlock) {
+                int64_t iX = X_indptr[r0 + t], iC = C_indptr[r0 + t];
+                const int64_t eX = X_indptr[r0 + t + 1], eC = C_indptr[r0 + t + 1];
+                while (iX < eX && iC < eC) {
+                    const int64_t cX = X_indices[iX], cC = C_indices[iC];
+                    if (cX == cC) grad_X[iX] = gC[iC] * coef;
+                    iX += cX <= cC;
+                    iC += cC <= cX;
+                }
+            }
+            __syncthreads();
+            continue;
+        }
+        for (int s0 = 0; s0 < nr;) {
+            const int e0 = lc_run_end(s_offX, s_offC, s0, nr, kLcCap, 2 * kLcCap);
+            if (e0 == s0) {
+                // one long row: every entry of X searches the row of C in global memory
+                const int64_t x0 = baseX + s_offX[s0], m = s_offX[s0 + 1] - s_offX[s0];
+                const int64_t c0 = baseC + s_offC[s0], n = s_offC[s0 + 1] - s_offC[s0];
+                for (int64_t k = threadIdx.x; k < m; k += kBlock) {
+                    const int64_t cX = X_indices[x0 + k];
+                    int64_t lo = 0, hi = n;
+                    while (lo < hi) {
+                        const int64_t mid = (lo + hi) >> 1;
+                        if (C_indices[c0 + mid] < cX) lo = mid + 1; else hi = mid;
+                    }
+                    if (lo < n && C_indices[c0 + lo] == cX) grad_X[x0 + k] = gC[c0 + lo] * coef;
+                }
+                s0 += 1;
+                continue;
+            }
+            // rows [s0, e0) of the tile through LDS
+            const int xo = s_offX[s0], co = s_offC[s0];
+            const int nX = s_offX[e0] - xo, nC = s_offC[e0] - co;
+            const int64_t gX = baseX + xo, gCb = baseC + co;
+            lc_stage_cols<5>(s_colX, X_indices + gX, nX);
+            lc_stage_cols<5>(s_colC, C_indices + gCb, nC);
             __syncthreads();
             // row of every entry of X: one lane per row marks its entries
-            for (int t = threadIdx.x; t < nr; t += kBlock) {
-                const int eX = s_offX[t + 1];
-                for (int k = s_offX[t]; k < eX; ++k) s_match[k] = t;
+            for (int t = s0 + threadIdx.x; t < e0; t += kBlock) {
+                const int eX = s_offX[t + 1] - xo;
+                for (int k = s_offX[t] - xo; k < eX; ++k) s_match[k] = t;
             }
             __syncthreads();
             // lane = entry of X: bisection for its column in the same row of C; K entries per
@@ -359,7 +494,7 @@ __global__ __launch_bounds__(kBlock) void lincomb_back_kernel(int64_t rows, T co
                     const int k = k0 + u * kBlock < nX ? k0 + u * kBlock : nX - 1;
                     const int t = s_match[k];
                     const int32_t cX = s_colX[k];
-                    int lo = s_offC[t], hi = s_offC[t + 1];
+                    int lo = s_offC[t] - co, hi = s_offC[t + 1] - co;
                     const int end = hi;
                     while (lo < hi) {
                         const int mid = (lo + hi) >> 1;
@@ -370,24 +505,14 @@ __global__ __launch_bounds__(kBlock) void lincomb_back_kernel(int64_t rows, T co
                 }
                 T gv[K];
 #pragma unroll
-                for (int u = 0; u < K; ++u) gv[u] = nC > 0 ? gC[baseC + at[u]] : T(0);
+                for (int u = 0; u < K; ++u) gv[u] = nC > 0 ? gC[gCb + at[u]] : T(0);
 #pragma unroll
                 for (int u = 0; u < K; ++u)
-                    if (k0 + u * kBlock < nX && found[u]) nm::stream_store(grad_X + baseX + k0 + u * kBlock, gv[u] * coef);
+                    if (k0 + u * kBlock < nX && found[u]) nm::stream_store(grad_X + gX + k0 + u * kBlock, gv[u] * coef);
             }
-        } else {
-            for (int t = threadIdx.x; t < nr; t += kBlock) {
-                int64_t iX = X_indptr[r0 + t], iC = C_indptr[r0 + t];
-                const int64_t eX = X_indptr[r0 + t + 1], eC = C_indptr[r0 + t + 1];
-                while (iX < eX && iC < eC) {
-                    const int64_t cX = X_indices[iX], cC = C_indices[iC];
-                    if (cX == cC) grad_X[iX] = gC[iC] * coef;
-                    iX += cX <= cC;
-                    iC += cC <= cX;
-                }
-            }
+            __syncthreads();
+            s0 = e0;
         }
-        __syncthreads();
     }
 }
 

@@ -36,6 +36,14 @@ def _pairs(dtype):
     yield "powerlaw", (G.powerlaw(3000, 3000, 40000, max_deg=2500, seed=5, dtype=dtype),
                        G.powerlaw(3000, 3000, 30000, max_deg=2500, seed=6, dtype=dtype))[0], \
         G.powerlaw(3000, 3000, 30000, max_deg=2500, seed=6, dtype=dtype)
+    # rows of ~40 entries: a tile of 256 rows does not fit LDS and is worked off in runs of rows
+    yield "runs_of_rows", G.random_csr(700, 400, 0.1, 8, dtype), G.random_csr(700, 400, 0.12, 9, dtype)
+    # rows too long for LDS in both operands, in one operand only, and next to short rows
+    yield "long_both", G.random_csr(5, 20000, 0.3, 10, dtype, empty_rows=False), G.random_csr(5, 20000, 0.25, 11, dtype)
+    yield "long_a_only", G.random_csr(3, 10000, 0.5, 12, dtype), G.random_csr(3, 10000, 0.001, 13, dtype)
+    yield "long_b_only", G.random_csr(3, 10000, 0.001, 14, dtype), G.random_csr(3, 10000, 0.5, 15, dtype)
+    yield "long_and_short", G.powerlaw(3000, 12000, 60000, max_deg=8000, seed=16, dtype=dtype), \
+        G.powerlaw(3000, 12000, 50000, max_deg=8000, seed=17, dtype=dtype)
     yield "empty_a", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(8, np.int64), (7, 5)), \
         G.random_csr(7, 5, 0.4, 7, dtype)
 
