@@ -13,6 +13,8 @@
 // Algorithmic HBM bytes, s = sizeof(value):
 //   forward : nnz*(s+8) + (rows+1)*8 + cols*s + rows*s
 //   backward: nnz*(s+8) + (rows+1)*8 + rows*s + cols*s + nnz*s + cols*s
+#include <type_traits>
+
 #include "nm_common.hpp"
 #include "nm_transpose.hpp"
 
@@ -38,15 +40,32 @@ constexpr int kFwdBlock = NM_FWD_BLOCK, kFwdR = NM_FWD_R, kFwdCap = NM_FWD_CAP;
 // columns per workgroup / LDS entries of the planned backward (measured best at cfg2: 96 vs 101 us)
 constexpr int kPlannedR = 256, kPlannedCap = 2048;
 
-// Loads the block's row offsets relative to `base` into LDS, clamped to CAP+1
+// A block of rows with this many entries or more is walked straight from global memory.
+constexpr int32_t kHuge = 1 << 30;
+
+// Loads the block's row offsets relative to `base` into LDS, clamped to kHuge
 // so that they fit 32 bits whatever the block holds.
 template <int R, int CAP, int BLOCK>
 __device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ indptr, int64_t r0, int nr,
                                               int64_t base, int32_t *s_off) {
     for (int t = threadIdx.x; t <= nr; t += BLOCK) {
         const int64_t d = indptr[r0 + t] - base;
-        s_off[t] = (int32_t)(d > CAP ? CAP + 1 : d);
+        s_off[t] = (int32_t)(d > kHuge ? kHuge : d);
     }
+}
+
+// End of the run of rows that starts at row s0 of the block and fits the LDS tile: the
+// largest e in [s0, nr] with at most cap entries in rows [s0, e); e == s0 when row s0
+// alone is longer.
+__device__ __forceinline__ int run_end(const int32_t *s_off, int s0, int nr, int cap) {
+    const int32_t limit = s_off[s0] + cap;
+    if (s_off[nr] <= limit) return nr;
+    int lo = s0, hi = nr;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_off[mid] <= limit) lo = mid; else hi = mid;
+    }
+    return lo;
 }
 
 // UNIT: x is taken as all ones and not read, which makes y the row sums
@@ -104,6 +123,78 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
                 T acc = 0;
                 for (int j = s_off[t]; j < e; ++j) acc += s_prod[j];
                 nm::stream_store(y + r0 + t, acc);
+            }
+        } else if (n < kHuge) {
+            // The block's entries do not fit the tile: runs of consecutive rows that do are taken
+            // one after the other.  Rows shorter than kLongRow are added by one lane in storage
+            // order as above; longer ones by a wavefront, lane l adding entries l, l + 64, ...
+            // of the row before the lanes are summed.
+            auto products = [&](int64_t first, int cnt) {   // s_prod[j] = data * x of entry first + j
+                const T *__restrict__ d = data + first;
+                const int64_t *__restrict__ ci = indices + first;
+                constexpr int K = 5;
+                for (int k0 = threadIdx.x; k0 < cnt; k0 += K * BLOCK) {
+                    T aa[K], xx[K];
+                    int64_t cc[K];
+#pragma unroll
+                    for (int u = 0; u < K; ++u) {
+                        const int kc = k0 + u * BLOCK < cnt ? k0 + u * BLOCK : cnt - 1;
+                        aa[u] = nm::stream_load(d + kc);
+                        if (!UNIT) cc[u] = nm::stream_load(ci + kc);
+                    }
+#pragma unroll
+                    for (int u = 0; u < K; ++u) xx[u] = UNIT ? T(1) : x[cc[u]];
+#pragma unroll
+                    for (int u = 0; u < K; ++u)
+                        if (k0 + u * BLOCK < cnt) s_prod[k0 + u * BLOCK] = aa[u] * xx[u];
+                }
+            };
+            for (int s0 = 0; s0 < nr;) {
+                const int e0 = run_end(s_off, s0, nr, CAP);
+                if (e0 == s0) {
+                    // a row longer than the tile, CAP entries at a time; wavefront 0 keeps the
+                    // lanes' partial sums (CAP is a multiple of 64: entry k stays with lane k % 64)
+                    const int64_t first = base + s_off[s0];
+                    const int len = s_off[s0 + 1] - s_off[s0];
+                    T acc = 0;
+                    for (int c0 = 0; c0 < len; c0 += CAP) {
+                        const int cnt = len - c0 < CAP ? len - c0 : CAP;
+                        products(first + c0, cnt);
+                        __syncthreads();
+                        if (wave == 0)
+                            for (int j = lane; j < cnt; j += kWave) acc += s_prod[j];
+                        __syncthreads();
+                    }
+                    if (wave == 0) {
+                        acc = nm::wave_sum(acc);
+                        if (lane == 0) y[r0 + s0] = acc;
+                    }
+                    s0 += 1;
+                    continue;
+                }
+                const int o0 = s_off[s0];
+                products(base + o0, s_off[e0] - o0);
+                __syncthreads();
+                for (int tb = s0; tb < e0; tb += BLOCK) {
+                    const int t = tb + threadIdx.x;
+                    const int b = t < e0 ? s_off[t] - o0 : 0, e = t < e0 ? s_off[t + 1] - o0 : 0;
+                    const bool wide = e - b >= kLongRow;
+                    if (t < e0 && !wide) {
+                        T acc = 0;
+                        for (int j = b; j < e; ++j) acc += s_prod[j];
+                        nm::stream_store(y + r0 + t, acc);
+                    }
+                    for (unsigned long long todo = __ballot(wide); todo; todo &= todo - 1) {
+                        const int src = __builtin_ctzll(todo);
+                        const int wb = __shfl(b, src, kWave), we = __shfl(e, src, kWave);
+                        T acc = 0;
+                        for (int j = wb + lane; j < we; j += kWave) acc += s_prod[j];
+                        acc = nm::wave_sum(acc);
+                        if (lane == 0) y[r0 + tb + wave * kWave + src] = acc;
+                    }
+                }
+                __syncthreads();
+                s0 = e0;
             }
         } else {
             // short rows: one lane each, straight from global memory
@@ -166,6 +257,51 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
                 if (out_A) out_A[base + k] = alpha * (av * b[c]);
                 if (grad_x) nm::atomic_add(grad_x + c, av * data[base + k]);
             }
+        } else if (n < kHuge) {
+            // runs of consecutive rows that fit the tile, one after the other
+            for (int s0 = 0; s0 < nr;) {
+                const int e0 = run_end(s_off, s0, nr, CAP);
+                if (e0 == s0) {
+                    // a row longer than the tile: lane = entry, straight from global memory
+                    const int64_t rb = base + s_off[s0];
+                    const int len = s_off[s0 + 1] - s_off[s0];
+                    const T av = a[r0 + s0];
+                    for (int k = threadIdx.x; k < len; k += kBlock) {
+                        const int64_t c = indices[rb + k];
+                        if (out_A) out_A[rb + k] = alpha * (av * b[c]);
+                        if (grad_x) nm::atomic_add(grad_x + c, av * data[rb + k]);
+                    }
+                    s0 += 1;
+                    continue;
+                }
+                const int o0 = s_off[s0], cnt = s_off[e0] - o0;
+                // spread a[row] over the row's entries: one lane per short row, a wavefront per
+                // row of kLongRow entries or more
+                for (int tb = s0; tb < e0; tb += kBlock) {
+                    const int t = tb + threadIdx.x;
+                    const int jb = t < e0 ? s_off[t] - o0 : 0, je = t < e0 ? s_off[t + 1] - o0 : 0;
+                    const T av = t < e0 ? a[r0 + t] : T(0);
+                    const bool wide = je - jb >= kLongRow;
+                    if (!wide)
+                        for (int j = jb; j < je; ++j) s_a[j] = av;
+                    for (unsigned long long todo = __ballot(wide); todo; todo &= todo - 1) {
+                        const int src = __builtin_ctzll(todo);
+                        const int wb = __shfl(jb, src, kWave), we = __shfl(je, src, kWave);
+                        const T wv = __shfl(av, src, kWave);
+                        for (int j = wb + lane; j < we; j += kWave) s_a[j] = wv;
+                    }
+                }
+                __syncthreads();
+                const int64_t first = base + o0;
+                for (int k = threadIdx.x; k < cnt; k += kBlock) {
+                    const int64_t c = indices[first + k];
+                    const T av = s_a[k];
+                    if (out_A) out_A[first + k] = alpha * (av * b[c]);
+                    if (grad_x) nm::atomic_add(grad_x + c, av * data[first + k]);
+                }
+                __syncthreads();
+                s0 = e0;
+            }
         } else {
             for (int t = threadIdx.x; t < nr; t += kBlock) {
                 const int64_t rb = indptr[r0 + t], re = indptr[r0 + t + 1];
@@ -206,7 +342,7 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
 // row-major entry p = (row c, column r), so the lane writes
 // grad_A[p] = g[c] * x[r] instead: a coalesced store, every entry once.
 template <typename T, int R, int CAP>
-__global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 8 : 7))) void spmv_bwd_planned_kernel(
     int64_t cols, const T *__restrict__ data, const int32_t *__restrict__ t_indptr,
     const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm,
     const int32_t *__restrict__ flags, const T *__restrict__ x, const T *__restrict__ g,
@@ -225,34 +361,76 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
         const int32_t base = t_indptr[c0];
         for (int t = threadIdx.x; t <= nc; t += kBlock) {
             const int32_t d = t_indptr[c0 + t] - base;
-            s_off[t] = d > CAP ? CAP + 1 : d;
+            s_off[t] = d > kHuge ? kHuge : d;
         }
         __syncthreads();
         const int n = s_off[nc];
-        if (n <= CAP && mirror && grad_A && grad_x) {
-            // fast path: both gradients, symmetric pattern -> every global access but the
-            // gathers of g, x and data is a coalesced stream
-            for (int t = threadIdx.x; t < nc; t += kBlock) {
-                const T v = g[c0 + t];
-                const int e = s_off[t + 1];
-                for (int j = s_off[t]; j < e; ++j) s_v[j] = v;
+        const bool fused = mirror && grad_A && grad_x;
+
+        // s_v[j] = own[column] for the entries j of columns [s0, e0); o0 = offset of column s0.
+        // WHOLE (the tile fits): one lane per column.  Otherwise columns of kLongRow entries
+        // or more are spread by a wavefront.
+        auto spread = [&](auto whole, const T *__restrict__ own, const int s0, const int e0, const int o0) {
+            constexpr bool WHOLE = decltype(whole)::value;
+            for (int tb = s0; tb < e0; tb += kBlock) {
+                const int t = tb + threadIdx.x;
+                const int jb = t < e0 ? s_off[t] - o0 : 0, je = t < e0 ? s_off[t + 1] - o0 : 0;
+                const T v = t < e0 ? own[c0 + t] : T(0);
+                const bool wide = !WHOLE && je - jb >= kLongRow;
+                if (!wide)
+                    for (int j = jb; j < je; ++j) s_v[j] = v;
+                if (!WHOLE)
+                    for (unsigned long long todo = __ballot(wide); todo; todo &= todo - 1) {
+                        const int src = __builtin_ctzll(todo);
+                        const int wb = __shfl(jb, src, kWave), we = __shfl(je, src, kWave);
+                        const T wv = __shfl(v, src, kWave);
+                        for (int j = wb + lane; j < we; j += kWave) s_v[j] = wv;
+                    }
             }
-            __syncthreads();
-            const int32_t *__restrict__ tr = t_row + base;
-            const int32_t *__restrict__ tp = t_perm + base;
-            T *__restrict__ ga = grad_A + base;
+        };
+        // grad_x[column] = sum of the column's slice of s_v: in storage order by one lane, or
+        // (not WHOLE, kLongRow entries or more) lane l of a wavefront adds entries l, l + 64, ...
+        auto sums = [&](auto whole, const int s0, const int e0, const int o0) {
+            constexpr bool WHOLE = decltype(whole)::value;
+            for (int tb = s0; tb < e0; tb += kBlock) {
+                const int t = tb + threadIdx.x;
+                const int jb = t < e0 ? s_off[t] - o0 : 0, je = t < e0 ? s_off[t + 1] - o0 : 0;
+                const bool wide = !WHOLE && je - jb >= kLongRow;
+                if (t < e0 && !wide) {
+                    T acc = 0;
+                    for (int j = jb; j < je; ++j) acc += s_v[j];
+                    grad_x[c0 + t] = acc;
+                }
+                if (!WHOLE)
+                    for (unsigned long long todo = __ballot(wide); todo; todo &= todo - 1) {
+                        const int src = __builtin_ctzll(todo);
+                        const int wb = __shfl(jb, src, kWave), we = __shfl(je, src, kWave);
+                        T acc = 0;
+                        for (int j = wb + lane; j < we; j += kWave) acc += s_v[j];
+                        acc = nm::wave_sum(acc);
+                        if (lane == 0) grad_x[c0 + tb + wave * kWave + src] = acc;
+                    }
+            }
+        };
+        // Entries first .. first + cnt of the plan, lane = entry, s_v holding the own factor of
+        // each: both gradients of a symmetric pattern -> every global access but the gathers of
+        // g, x and data is a coalesced stream.
+        auto entries_fused = [&](const int32_t first, const int cnt) {
+            const int32_t *__restrict__ tr = t_row + first;
+            const int32_t *__restrict__ tp = t_perm + first;
+            T *__restrict__ ga = grad_A + first;
             // K entries in flight per lane: all their plan loads, then all their gathers, then
             // the stores -- two memory round trips per K entries.  Loads are unconditional on a
             // clamped position (a predicated load would sit in its own branch with its own wait).
             // Measured on the 2048 x 2048 Poisson matrix (5 entries per lane and tile), kernel time:
             // K = 2: 103 us, 4: 95 us, 5: 90 us, 6: 86 us, 8: 91 us.
             constexpr int K = 6;
-            for (int p0 = threadIdx.x; p0 < n; p0 += K * kBlock) {
+            for (int p0 = threadIdx.x; p0 < cnt; p0 += K * kBlock) {
                 int32_t kk[K], rr[K];
                 T gg[K], xx[K], dd[K];
 #pragma unroll
                 for (int u = 0; u < K; ++u) {
-                    const int pc = p0 + u * kBlock < n ? p0 + u * kBlock : n - 1;
+                    const int pc = p0 + u * kBlock < cnt ? p0 + u * kBlock : cnt - 1;
                     kk[u] = nm::stream_load(tp + pc);
                     rr[u] = nm::stream_load(tr + pc);
                 }
@@ -262,7 +440,7 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
                     xx[u] = x[rr[u]];
                     dd[u] = data[kk[u]];
                 }
-                if (p0 + (K - 1) * kBlock < n) {
+                if (p0 + (K - 1) * kBlock < cnt) {
 #pragma unroll
                     for (int u = 0; u < K; ++u) {
                         const int p = p0 + u * kBlock;
@@ -273,51 +451,85 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
 #pragma unroll
                     for (int u = 0; u < K; ++u) {
                         const int p = p0 + u * kBlock;
-                        if (p < n) {
+                        if (p < cnt) {
                             ga[p] = s_v[p] * xx[u];
                             s_v[p] = gg[u] * dd[u];
                         }
                     }
                 }
             }
-            __syncthreads();
-            for (int t = threadIdx.x; t < nc; t += kBlock) {
-                const int e = s_off[t + 1];
-                T acc = 0;
-                for (int j = s_off[t]; j < e; ++j) acc += s_v[j];
-                grad_x[c0 + t] = acc;
-            }
-        } else if (n <= CAP) {
-            if (grad_A) {
-                // spread the column's own factor over its entries: g[c] (mirror) or x[c]
-                const T *__restrict__ own = mirror ? g : x;
-                for (int t = threadIdx.x; t < nc; t += kBlock) {
-                    const T v = own[c0 + t];
-                    const int e = s_off[t + 1];
-                    for (int j = s_off[t]; j < e; ++j) s_v[j] = v;
-                }
-                __syncthreads();
-            }
-            const int32_t *__restrict__ tr = t_row + base;
-            const int32_t *__restrict__ tp = t_perm + base;
-            for (int p = threadIdx.x; p < n; p += kBlock) {
+        };
+        // The same for one gradient only or a pattern that is not symmetric.
+        auto entries_any = [&](const int32_t first, const int cnt) {
+            const int32_t *__restrict__ tr = t_row + first;
+            const int32_t *__restrict__ tp = t_perm + first;
+            for (int p = threadIdx.x; p < cnt; p += kBlock) {
                 const int32_t k = nm::stream_load(tp + p);
                 const int32_t r = nm::stream_load(tr + p);
                 const T gr = g[r];
                 if (grad_A) {
-                    if (mirror) grad_A[base + p] = s_v[p] * x[r];
+                    if (mirror) grad_A[first + p] = s_v[p] * x[r];
                     else grad_A[k] = gr * s_v[p];
                 }
                 if (grad_x) s_v[p] = gr * data[k];
             }
+        };
+        // columns [s0, e0) through LDS
+        auto run = [&](auto whole, const int s0, const int e0) {
+            constexpr bool WHOLE = decltype(whole)::value;
+            const int o0 = WHOLE ? 0 : s_off[s0];
+            const int cnt = s_off[e0] - o0;
+            if (fused) {
+                spread(whole, g, s0, e0, o0);
+                __syncthreads();
+                entries_fused(base + o0, cnt);
+            } else {
+                if (grad_A) {
+                    spread(whole, mirror ? g : x, s0, e0, o0);
+                    __syncthreads();
+                }
+                entries_any(base + o0, cnt);
+            }
             if (grad_x) {
                 __syncthreads();
-                for (int t = threadIdx.x; t < nc; t += kBlock) {
-                    const int e = s_off[t + 1];
-                    T acc = 0;
-                    for (int j = s_off[t]; j < e; ++j) acc += s_v[j];
-                    grad_x[c0 + t] = acc;
+                sums(whole, s0, e0, o0);
+            }
+        };
+
+        if (n <= CAP) {
+            run(std::true_type{}, 0, nc);
+        } else if (n < kHuge) {
+            for (int s0 = 0; s0 < nc;) {
+                const int e0 = run_end(s_off, s0, nc, CAP);
+                if (e0 > s0) {
+                    run(std::false_type{}, s0, e0);
+                    __syncthreads();
+                    s0 = e0;
+                    continue;
                 }
+                // a column longer than the tile, CAP entries at a time; wavefront 0 keeps the
+                // lanes' partial sums (CAP is a multiple of 64: entry p stays with lane p % 64)
+                const int32_t first = base + s_off[s0];
+                const int len = s_off[s0 + 1] - s_off[s0];
+                const T own = grad_A ? (mirror ? g : x)[c0 + s0] : T(0);
+                T acc = 0;
+                for (int q0 = 0; q0 < len; q0 += CAP) {
+                    const int cnt = len - q0 < CAP ? len - q0 : CAP;
+                    if (grad_A) {
+                        for (int j = threadIdx.x; j < cnt; j += kBlock) s_v[j] = own;
+                        __syncthreads();
+                    }
+                    if (fused) entries_fused(first + q0, cnt); else entries_any(first + q0, cnt);
+                    __syncthreads();
+                    if (grad_x && wave == 0)
+                        for (int j = lane; j < cnt; j += kWave) acc += s_v[j];
+                    __syncthreads();
+                }
+                if (grad_x && wave == 0) {
+                    acc = nm::wave_sum(acc);
+                    if (lane == 0) grad_x[c0 + s0] = acc;
+                }
+                s0 += 1;
             }
         } else {
             for (int t = threadIdx.x; t < nc; t += kBlock) {

@@ -44,13 +44,15 @@ __global__ void transpose_scatter_kernel(int64_t nnz, const T *__restrict__ grad
 
 // ---- entry-parallel maps over a CSR matrix ---------------------------------------
 //
-// A workgroup owns a tile of kTileRows rows.  Row offsets are staged in LDS, one
-// lane per row spreads the row number over the row's entries, and the entries are
-// then processed lane = entry, so the CSR arrays stream through coalesced while
-// every entry knows its row.  Tiles with more than kTileCap entries (long rows)
-// are walked one row per wavefront instead.
+// A workgroup owns a tile of kTileRows rows.  Row offsets are staged in LDS, the
+// row number is spread over the row's entries (by one lane for a short row, by a
+// wavefront for a row of kTileWide entries or more), and the entries are then
+// processed lane = entry, so the CSR arrays stream through coalesced while every
+// entry knows its row.  A tile with more than kTileCap entries is taken in runs of
+// consecutive rows that fit; a single row longer than that needs no LDS at all.
 
-constexpr int kTileRows = 256, kTileCap = 4096;
+constexpr int kTileRows = 256, kTileCap = 4096, kTileWide = 32;
+constexpr int32_t kTileHuge = 1 << 30;   // tiles with this many entries: one row per wavefront from global memory
 
 enum MapOp { kToDense, kFromDense, kDiagBack, kRowSpread };
 
@@ -61,6 +63,62 @@ __device__ __forceinline__ void map_entry(int64_t row, int64_t k, const int64_t 
     if (OP == kFromDense) dst[k] = src[row * ld + indices[k]];             // grad_A[k] = grad_Ad[i][j]
     if (OP == kDiagBack) dst[k] = indices[k] == row ? src[row] : T(0);     // grad_A[k] = g[i] on the diagonal
     if (OP == kRowSpread) dst[k] = src[row];                               // grad_A[k] = g[i]
+}
+
+__device__ __forceinline__ void tile_stage_offsets(const int64_t *__restrict__ indptr, int64_t r0, int nr,
+                                                   int32_t *s_off) {
+    const int64_t base = indptr[r0];
+    for (int t = threadIdx.x; t <= nr; t += kBlock) {
+        const int64_t d = indptr[r0 + t] - base;
+        s_off[t] = (int32_t)(d > kTileHuge ? kTileHuge : d);
+    }
+}
+
+// Calls f(row within the tile, position in the CSR arrays) for every entry of the tile's
+// rows, lane = entry.  Whole workgroup; s_off holds the staged offsets (fewer than
+// kTileHuge entries), s_row is scratch for kTileCap entries.
+template <typename F>
+__device__ __forceinline__ void tile_entries(const int32_t *s_off, uint8_t *s_row, int nr, int64_t base, F f) {
+    const int lane = threadIdx.x & 63;
+    for (int s0 = 0; s0 < nr;) {
+        // rows [s0, e0): the longest run with at most kTileCap entries
+        int e0 = nr;
+        const int32_t limit = s_off[s0] + kTileCap;
+        if (s_off[nr] > limit) {
+            int lo = s0, hi = nr;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (s_off[mid] <= limit) lo = mid; else hi = mid;
+            }
+            e0 = lo;
+        }
+        if (e0 == s0) {
+            const int64_t first = base + s_off[s0];
+            const int len = s_off[s0 + 1] - s_off[s0];
+            for (int k = threadIdx.x; k < len; k += kBlock) f(s0, first + k);
+            s0 += 1;
+            continue;
+        }
+        const int o0 = s_off[s0], cnt = s_off[e0] - o0;
+        for (int tb = s0; tb < e0; tb += kBlock) {
+            const int t = tb + threadIdx.x;
+            const int jb = t < e0 ? s_off[t] - o0 : 0, je = t < e0 ? s_off[t + 1] - o0 : 0;
+            const bool wide = je - jb >= kTileWide;
+            if (!wide)
+                for (int j = jb; j < je; ++j) s_row[j] = (uint8_t)t;
+            for (unsigned long long todo = __ballot(wide); todo; todo &= todo - 1) {
+                const int src = __builtin_ctzll(todo);
+                const int wb = __shfl(jb, src, 64), we = __shfl(je, src, 64);
+                const uint8_t row = (uint8_t)__shfl(t, src, 64);
+                for (int j = wb + lane; j < we; j += 64) s_row[j] = row;
+            }
+        }
+        __syncthreads();
+        const int64_t first = base + o0;
+        for (int k = threadIdx.x; k < cnt; k += kBlock) f((int)s_row[k], first + k);
+        __syncthreads();
+        s0 = e0;
+    }
 }
 
 template <typename T, int OP>
@@ -78,18 +136,11 @@ __global__ __launch_bounds__(kBlock) void entry_map_kernel(int64_t rows, const i
         const int64_t r0 = tile * kTileRows;
         const int nr = (int)(rows - r0 < kTileRows ? rows - r0 : kTileRows);
         const int64_t base = indptr[r0];
-        for (int t = threadIdx.x; t <= nr; t += kBlock) {
-            const int64_t d = indptr[r0 + t] - base;
-            s_off[t] = (int32_t)(d > kTileCap ? kTileCap + 1 : d);
-        }
+        tile_stage_offsets(indptr, r0, nr, s_off);
         __syncthreads();
-        const int n = s_off[nr];
-        if (n <= kTileCap) {
-            for (int t = threadIdx.x; t < nr; t += kBlock)
-                for (int j = s_off[t]; j < s_off[t + 1]; ++j) s_row[j] = (uint8_t)t;
-            __syncthreads();
-            for (int k = threadIdx.x; k < n; k += kBlock)
-                map_entry<T, OP>(r0 + s_row[k], base + k, indices, src, dst, ld);
+        if (s_off[nr] < kTileHuge) {
+            tile_entries(s_off, s_row, nr, base,
+                         [&](int t, int64_t k) { map_entry<T, OP>(r0 + t, k, indices, src, dst, ld); });
         } else {
             for (int t = wave; t < nr; t += kBlock / 64) {
                 const int64_t e = indptr[r0 + t + 1];
@@ -117,19 +168,13 @@ __global__ __launch_bounds__(kBlock) void diagonal_kernel(int64_t rows, const T 
         const int64_t r0 = tile * kTileRows;
         const int nr = (int)(rows - r0 < kTileRows ? rows - r0 : kTileRows);
         const int64_t base = indptr[r0];
-        for (int t = threadIdx.x; t <= nr; t += kBlock) {
-            const int64_t d = indptr[r0 + t] - base;
-            s_off[t] = (int32_t)(d > kTileCap ? kTileCap + 1 : d);
-        }
+        tile_stage_offsets(indptr, r0, nr, s_off);
         for (int t = threadIdx.x; t < nr; t += kBlock) s_x[t] = T(0);
         __syncthreads();
-        const int n = s_off[nr];
-        if (n <= kTileCap) {
-            for (int t = threadIdx.x; t < nr; t += kBlock)
-                for (int j = s_off[t]; j < s_off[t + 1]; ++j) s_row[j] = (uint8_t)t;
-            __syncthreads();
-            for (int k = threadIdx.x; k < n; k += kBlock)
-                if (indices[base + k] == r0 + s_row[k]) s_x[s_row[k]] = data[base + k];
+        if (s_off[nr] < kTileHuge) {
+            tile_entries(s_off, s_row, nr, base, [&](int t, int64_t k) {
+                if (indices[k] == r0 + t) s_x[t] = data[k];
+            });
         } else {
             for (int t = wave; t < nr; t += kBlock / 64) {
                 const int64_t e = indptr[r0 + t + 1];
