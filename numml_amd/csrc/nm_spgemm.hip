@@ -39,7 +39,8 @@ using nm::kWave;
 
 constexpr int32_t kEmpty = -1;
 constexpr int kBlock = 256;
-constexpr int kBins = 4;
+constexpr int kBins = 7;
+constexpr int kBinStart = 8, kBinCursor = 16, kBinInts = 24;   // layout of the bins array, see Work
 // Workgroups (and dense accumulator slices of B_cols entries each) of the spill path: as many as
 // fit a fixed budget of scratch, between 8 and 64.
 constexpr int64_t kSpillBudgetBytes = int64_t(192) << 20;
@@ -52,11 +53,16 @@ constexpr int kTablePad = 4;         // entries between the hash tables of neigh
 constexpr int kAhead = 8;            // B rows whose first columns a group requests before inserting any
 
 // bin upper limits (inclusive); the last bin takes the rest and spills
-constexpr int32_t kSymLimit[3] = {64, 512, 8192};     // on the product bound
-constexpr int32_t kNumLimit[3] = {32, 512, 4096};     // on the exact row length
-// table sizes per bin
-constexpr int kSymTable0 = 128, kSymTable1 = 1024, kSymTable2 = 16384;
-constexpr int kNumTable0 = 64, kNumTable1 = 1024, kNumTable2 = 8192;
+constexpr int32_t kSymLimit[6] = {64, 128, 256, 512, 1024, 8192};     // on the product bound
+constexpr int32_t kNumLimit[6] = {32, 64, 128, 256, 512, 4096};       // on the exact row length
+// lanes per row and table sizes per bin.  The kernels wait on memory (A's row, the bounds of its B
+// rows, the B rows: a chain of round trips per row) and LDS decides how many rows a CU has in
+// flight, so rows get the smallest table that holds them at half load.
+constexpr int kGroup0 = 8, kGroup1 = 16, kGroup2 = 16, kGroup3 = 64, kGroup4 = 64, kGroup5 = 256;
+constexpr int kSymTable0 = 128, kSymTable1 = 256, kSymTable2 = 512, kSymTable3 = 1024, kSymTable4 = 2048,
+              kSymTable5 = 16384;
+constexpr int kNumTable0 = 64, kNumTable1 = 128, kNumTable2 = 256, kNumTable3 = 512, kNumTable4 = 1024,
+              kNumTable5 = 8192;
 
 constexpr int kMergeCap = 8;                  // longest A row and B row of the merge path
 constexpr int32_t kColEnd = 0x7fffffff;       // past-the-end column of a staged B row
@@ -65,7 +71,7 @@ constexpr int32_t kMergedKey = -1;            // binning key of a row the merge 
 struct Work {
     int32_t *key;      // [rows] binning key (product bound, then exact length)
     int32_t *perm;     // [rows] rows grouped by bin
-    int32_t *bins;     // [16]: count[0..3], offset[4..8], cursor[9..12]
+    int32_t *bins;     // [kBinInts]: rows per bin [0, kBins), first row of bin b at kBinStart + b (end at + b + 1), cursor at kBinCursor + b
     int64_t *scan;     // scan scratch
     int32_t *mark;     // [spill_groups(B_cols) * B_cols]
     double *acc;       // [spill_groups(B_cols) * B_cols]
@@ -82,7 +88,7 @@ size_t work_layout(int64_t rows, int64_t B_cols, void *base, Work *w) {
     };
     int32_t *key = (int32_t *)take((rows + 1) * 4);
     int32_t *perm = (int32_t *)take((rows + 1) * 4);
-    int32_t *bins = (int32_t *)take(16 * 4);
+    int32_t *bins = (int32_t *)take(kBinInts * 4);
     int64_t *scan = (int64_t *)take(nm::scan_scratch_bytes(rows + 1));
     int32_t *mark = (int32_t *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 4);
     double *acc = (double *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 8);
@@ -90,7 +96,14 @@ size_t work_layout(int64_t rows, int64_t B_cols, void *base, Work *w) {
     return off;
 }
 
-__device__ __forceinline__ uint32_t hash32(int32_t key) { return (uint32_t)key * 0x9E3779B1u; }
+// First slot of a key in a table of TABLE slots (a power of two): the HIGH bits of a
+// multiplicative hash.  The low bits of key * odd depend on the low bits of the key alone,
+// so columns a multiple of the table size apart -- the neighbours of a grid point in the
+// next row or plane -- would all start their probes in the same slot.
+template <int TABLE> __device__ __forceinline__ uint32_t first_slot(int32_t key) {
+    static_assert(TABLE >= 2 && (TABLE & (TABLE - 1)) == 0, "table size");
+    return ((uint32_t)key * 0x9E3779B1u) >> (32 - __builtin_ctz(TABLE));
+}
 
 template <int G> __device__ __forceinline__ void group_sync() {
     if (G > kWave) __syncthreads();
@@ -349,27 +362,32 @@ __global__ void row_length_kernel(int64_t rows, const int64_t *__restrict__ C_in
 }
 
 // negative keys (rows taken by the merge path) belong to no bin
-__device__ __forceinline__ int bin_of(int32_t k, int32_t l0, int32_t l1, int32_t l2) {
-    return k < 0 ? -1 : (k <= l0 ? 0 : (k <= l1 ? 1 : (k <= l2 ? 2 : 3)));
+struct BinLimits { int32_t l[kBins - 1]; };
+__device__ __forceinline__ int bin_of(int32_t k, const BinLimits &lim) {
+    if (k < 0) return -1;
+    int b = 0;
+#pragma unroll
+    for (int q = 0; q < kBins - 1; ++q) b += k > lim.l[q];
+    return b;
 }
 
 __global__ void bin_clear_kernel(int32_t *bins) {
-    if (threadIdx.x < 16) bins[threadIdx.x] = 0;
+    if (threadIdx.x < kBinInts) bins[threadIdx.x] = 0;
 }
 
 // Rows per bin.  Each wavefront counts with ballots (one population count per
 // bin) instead of 64 colliding LDS atomics.
 __global__ __launch_bounds__(kBlock) void bin_count_kernel(int64_t rows, const int32_t *__restrict__ key,
-                                                           int32_t l0, int32_t l1, int32_t l2, int32_t *bins) {
+                                                           BinLimits lim, int32_t *bins) {
     __shared__ int s_cnt[kBins];
     if (threadIdx.x < kBins) s_cnt[threadIdx.x] = 0;
     __syncthreads();
     const int lane = threadIdx.x & (kWave - 1);
-    int mine[kBins] = {0, 0, 0, 0};
+    int mine[kBins] = {};
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x; i0 < rows; i0 += stride) {
         const int64_t i = i0 + threadIdx.x;
-        const int b = i < rows ? bin_of(key[i], l0, l1, l2) : -1;
+        const int b = i < rows ? bin_of(key[i], lim) : -1;
 #pragma unroll
         for (int q = 0; q < kBins; ++q) mine[q] += __popcll(__ballot(b == q));
     }
@@ -384,11 +402,11 @@ __global__ void bin_offsets_kernel(int32_t *bins) {
     if (threadIdx.x == 0) {
         int32_t run = 0;
         for (int b = 0; b < kBins; ++b) {
-            bins[4 + b] = run;
-            bins[9 + b] = run;  // cursor
+            bins[kBinStart + b] = run;
+            bins[kBinCursor + b] = run;
             run += bins[b];
         }
-        bins[4 + kBins] = run;
+        bins[kBinStart + kBins] = run;
     }
 }
 
@@ -396,7 +414,7 @@ __global__ void bin_offsets_kernel(int32_t *bins) {
 // so that each bin keeps them in ascending order inside a workgroup's slice
 // (neighbouring rows share B rows and C lines).
 __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const int32_t *__restrict__ key,
-                                                             int32_t l0, int32_t l1, int32_t l2, int32_t *bins,
+                                                             BinLimits lim, int32_t *bins,
                                                              int32_t *__restrict__ perm) {
     constexpr int kWaves = kBlock / kWave;
     __shared__ int s_wave[kWaves][kBins];   // rows of bin q in wavefront w
@@ -405,7 +423,7 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x; i0 < rows; i0 += stride) {
         const int64_t i = i0 + threadIdx.x;
-        const int b = i < rows ? bin_of(key[i], l0, l1, l2) : -1;
+        const int b = i < rows ? bin_of(key[i], lim) : -1;
         int before = 0;   // rows of my bin in lower lanes of my wavefront
 #pragma unroll
         for (int q = 0; q < kBins; ++q) {
@@ -417,7 +435,7 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
         if (threadIdx.x < kBins) {
             int total = 0;
             for (int w = 0; w < kWaves; ++w) total += s_wave[w][threadIdx.x];
-            s_base[threadIdx.x] = total ? atomicAdd(bins + 9 + threadIdx.x, total) : 0;
+            s_base[threadIdx.x] = total ? atomicAdd(bins + kBinCursor + threadIdx.x, total) : 0;
         }
         __syncthreads();
         if (b >= 0) {
@@ -429,16 +447,17 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
     }
 }
 
-int bin_rows(int64_t rows, const int32_t limit[3], const Work &w, hipStream_t s) {
+int bin_rows(int64_t rows, const int32_t limit[kBins - 1], const Work &w, hipStream_t s) {
+    BinLimits lim;
+    for (int q = 0; q < kBins - 1; ++q) lim.l[q] = limit[q];
     int64_t grid = nm::ceil_div(rows, kBlock);
     if (grid > 4096) grid = 4096;
     if (grid < 1) grid = 1;
     hipLaunchKernelGGL(bin_clear_kernel, dim3(1), dim3(64), 0, s, w.bins);
-    hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, w.key, limit[0],
-                       limit[1], limit[2], w.bins);
+    hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, w.key, lim, w.bins);
     hipLaunchKernelGGL(bin_offsets_kernel, dim3(1), dim3(64), 0, s, w.bins);
-    hipLaunchKernelGGL(bin_scatter_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, w.key, limit[0],
-                       limit[1], limit[2], w.bins, w.perm);
+    hipLaunchKernelGGL(bin_scatter_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, w.key, lim, w.bins,
+                       w.perm);
     NM_LAUNCH_CHECK("bin kernels");
     return NM_OK;
 }
@@ -459,7 +478,7 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
     __shared__ int s_red[kBlock / kWave];
     const int gl = threadIdx.x % G, gi = G >= kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x / G) : threadIdx.x / G;
     int32_t *tab = s_keys + gi * STRIDE;
-    const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
+    const int32_t b0 = bins[kBinStart + bin], b1 = bins[kBinStart + bin + 1];
     for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
         const int32_t idx = idx0 + gi;
         const bool live = idx < b1;
@@ -468,7 +487,7 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
         int cnt = 0;
         int64_t row = 0;
         auto insert = [&](int32_t key) {
-            uint32_t h = hash32(key) & (TABLE - 1);
+            uint32_t h = first_slot<TABLE>(key);
             for (;;) {
                 const int32_t old = atomicCAS(&tab[h], kEmpty, key);
                 if (old == kEmpty) { ++cnt; break; }
@@ -526,7 +545,7 @@ __global__ __launch_bounds__(kSpillBlock) void symbolic_spill_kernel(
     const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr, int32_t *mark_all,
     int64_t *__restrict__ C_count) {
     __shared__ int s_red[kSpillBlock / kWave];
-    const int32_t b0 = bins[4 + 3], b1 = bins[5 + 3];
+    const int32_t b0 = bins[kBinStart + kBins - 1], b1 = bins[kBinStart + kBins];
     if (b0 + (int32_t)blockIdx.x >= b1) return;
     int32_t *mark = mark_all + (size_t)blockIdx.x * (B_cols + 1);
     for (int64_t c = threadIdx.x; c < B_cols; c += kSpillBlock) mark[c] = 0;
@@ -576,7 +595,7 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
     constexpr int CSTRIDE = TABLE / 2 + 4;
     int32_t *ck = s_keys + GPB * STRIDE + gi * 2 * CSTRIDE;
     int32_t *cs = ck + CSTRIDE;
-    const int32_t b0 = bins[4 + bin], b1 = bins[5 + bin];
+    const int32_t b0 = bins[kBinStart + bin], b1 = bins[kBinStart + bin + 1];
     for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
         const int32_t idx = idx0 + gi;
         const bool live = idx < b1;
@@ -584,7 +603,7 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
         group_sync<G>();
         int64_t row = 0;
         auto add = [&](int32_t key, T prod) {
-            uint32_t h = hash32(key) & (TABLE - 1);
+            uint32_t h = first_slot<TABLE>(key);
             for (;;) {
                 const int32_t old = atomicCAS(&tab[h], kEmpty, key);
                 if (old == kEmpty) { val[h] = prod; return; }   // 0 + prod == prod exactly
@@ -780,7 +799,7 @@ __global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
     int32_t *mark_all, double *acc_all) {
     __shared__ int64_t s_wave[kSpillBlock / kWave];
     __shared__ unsigned long long s_lo, s_hi;
-    const int32_t b0 = bins[4 + 3], b1 = bins[5 + 3];
+    const int32_t b0 = bins[kBinStart + kBins - 1], b1 = bins[kBinStart + kBins];
     if (b0 + (int32_t)blockIdx.x >= b1) return;
     int32_t *mark = mark_all + (size_t)blockIdx.x * (B_cols + 1);
     T *acc = reinterpret_cast<T *>(acc_all + (size_t)blockIdx.x * (B_cols + 1));
@@ -848,16 +867,15 @@ __global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
 // ---- backward --------------------------------------------------------------------
 
 // Backward.  A group of 8 lanes owns one row i of A.  Row i of C (column
-// indices and upstream gradient) is staged in LDS when it has at most
-// kBwdStage entries, so the per-product lookups are LDS bisections; longer
-// rows are searched in global memory.  The group takes the row's entries
+// indices and upstream gradient, at most kBwdStage entries) is staged in LDS,
+// so the per-product lookups are LDS bisections.  The group takes the row's entries
 // (i,k) one at a time and spreads row k of B over its lanes, so the eight
 // atomic updates of grad_B it issues land in one cache line (the L2 atomic
 // units are bound by lines touched, not by lanes).  The products
 // gC[i,c] * B[k,c] are then added lane by lane in ascending column order --
 // the order of the reference's merge -- which keeps grad_A bit-identical.
 //
-// Rows of C longer than kBwdLong go to a second kernel in which a whole
+// Rows of C longer than kBwdStage go to a second kernel in which a whole
 // workgroup owns the row: its 32 groups share out the entries of A's row, whole
 // wavefronts take the entries whose row of B is long, and the row of C is staged
 // in LDS -- columns and gradient up to kBwdLongCap entries; columns only beyond
@@ -867,7 +885,7 @@ __global__ __launch_bounds__(kSpillBlock) void numeric_spill_kernel(
 // global-memory search per product set the time of the whole launch.
 constexpr int kBwdG = 8;
 constexpr int kBwdStage = 64;
-constexpr int kBwdLong = 256;
+constexpr int kBwdLong = kBwdStage;
 constexpr int kBwdLongCap = 2048;     // rows up to this long: columns and gradient in LDS
 constexpr int kBwdHugeCap = 14336;    // longer rows: columns only
 constexpr int kBwdLongChunk = 256;   // rows a workgroup of the long-row kernel looks through at a time
@@ -893,14 +911,13 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
         const bool live = i < A_rows;
         const int64_t cb = live ? C_indptr[i] : 0, ce = live ? C_indptr[i + 1] : 0;
         const int clen = (int)(ce - cb < 0x7fffffff ? ce - cb : 0x7fffffff);
-        const bool staged = clen <= kBwdStage;
-        if (staged)
+        const bool here = live && clen <= kBwdStage;   // longer rows are left to spgemm_bwd_long_kernel
+        if (here)
             for (int t = gl; t < clen; t += G) {
                 ci[t] = (int32_t)C_indices[cb + t];
                 cg[t] = gC[cb + t];
             }
         group_sync<G>();
-        const bool here = live && clen <= kBwdLong;   // longer rows are left to spgemm_bwd_long_kernel
         const int64_t ab = here ? A_indptr[i] : 0, ae = here ? A_indptr[i + 1] : 0;
         for (int64_t a0 = ab; a0 < ae; a0 += G) {
             // each lane fetches one entry of A's row and the bounds of the B row it names
@@ -920,25 +937,13 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
                     const bool have = kk < be;
                     const int64_t c = have ? B_indices[kk] : -1;
                     const T bval = have ? B_data[kk] : T(0);
-                    bool hit = false;
-                    T g = 0;
-                    if (staged) {
-                        int l = 0, h = clen;
-                        while (l < h) {
-                            const int mid = (l + h) >> 1;
-                            if ((int64_t)ci[mid] < c) l = mid + 1; else h = mid;
-                        }
-                        hit = have && l < clen && (int64_t)ci[l] == c;
-                        if (hit) g = cg[l];
-                    } else {
-                        int64_t l = cb, h = ce;
-                        while (l < h) {
-                            const int64_t mid = (l + h) >> 1;
-                            if (C_indices[mid] < c) l = mid + 1; else h = mid;
-                        }
-                        hit = have && l < ce && C_indices[l] == c;
-                        if (hit) g = gC[l];
+                    int l = 0, h = clen;
+                    while (l < h) {
+                        const int mid = (l + h) >> 1;
+                        if ((int64_t)ci[mid] < c) l = mid + 1; else h = mid;
                     }
+                    const bool hit = have && l < clen && (int64_t)ci[l] == c;
+                    const T g = hit ? cg[l] : T(0);
                     if (hit && grad_B) nm::atomic_add(grad_B + kk, a * g);
                     const T prod = g * bval;
                     // ordered sum over the group's lanes = ascending column
@@ -1103,27 +1108,26 @@ int launch_numeric(const Work &w, int64_t B_cols, const void *A_data, const int6
     const T *Ad = (const T *)A_data, *Bd = (const T *)B_data;
     T *Cd = (T *)C_data;
     constexpr size_t per = sizeof(T) + sizeof(int32_t);
-    {
-        auto k = numeric_hash_kernel<T, 8, kNumTable0>;
-        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), (kBlock / 8) * (per * (kNumTable0 + kTablePad) + 4 * (kNumTable0 + 8)), s, 0, w.bins,
-                           w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
-        NM_LAUNCH_CHECK("numeric_hash_kernel<8>");
-    }
-    {
-        auto k = numeric_hash_kernel<T, 64, kNumTable1>;
-        hipLaunchKernelGGL(k, dim3(kPersistGrid), dim3(kBlock), (kBlock / 64) * (per * (kNumTable1 + kTablePad) + 4 * (kNumTable1 + 8)), s, 1, w.bins,
-                           w.perm, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd);
-        NM_LAUNCH_CHECK("numeric_hash_kernel<64>");
-    }
-    {
-        auto k = numeric_hash_kernel<T, 256, kNumTable2>;
-        const size_t lds = per * kNumTable2 + 4 * (kNumTable2 + 8);
-        NM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        hipLaunchKernelGGL(k, dim3(1024), dim3(kBlock), lds, s, 2, w.bins, w.perm, Ad, A_indices, A_indptr, Bd,
+    auto hashed = [&](auto group, auto table, int bin, unsigned grid) -> int {
+        constexpr int G = decltype(group)::value, TABLE = decltype(table)::value;
+        auto k = numeric_hash_kernel<T, G, TABLE>;
+        // tables (values + keys), padded apart when groups share a workgroup, and the two compaction lists
+        const size_t lds = (kBlock / G) * (per * (TABLE + (G < kBlock ? kTablePad : 0)) + 4 * (TABLE + 8));
+        if (lds > 64 * 1024)
+            NM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(grid), dim3(kBlock), lds, s, bin, w.bins, w.perm, Ad, A_indices, A_indptr, Bd,
                            B_indices, B_indptr, C_indptr, C_indices, Cd);
-        NM_LAUNCH_CHECK("numeric_hash_kernel<256>");
-    }
+        NM_LAUNCH_CHECK("numeric_hash_kernel");
+        return NM_OK;
+    };
+    using std::integral_constant;
+    if (int rc = hashed(integral_constant<int, kGroup0>{}, integral_constant<int, kNumTable0>{}, 0, kPersistGrid)) return rc;
+    if (int rc = hashed(integral_constant<int, kGroup1>{}, integral_constant<int, kNumTable1>{}, 1, kPersistGrid)) return rc;
+    if (int rc = hashed(integral_constant<int, kGroup2>{}, integral_constant<int, kNumTable2>{}, 2, kPersistGrid)) return rc;
+    if (int rc = hashed(integral_constant<int, kGroup3>{}, integral_constant<int, kNumTable3>{}, 3, kPersistGrid)) return rc;
+    if (int rc = hashed(integral_constant<int, kGroup4>{}, integral_constant<int, kNumTable4>{}, 4, kPersistGrid)) return rc;
+    if (int rc = hashed(integral_constant<int, kGroup5>{}, integral_constant<int, kNumTable5>{}, 5, 1024)) return rc;
     hipLaunchKernelGGL(numeric_spill_kernel<T>, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm,
                        B_cols, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd, w.mark,
                        w.acc);
@@ -1161,15 +1165,19 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     NM_LAUNCH_CHECK("symbolic_front_kernel");
     if (int rc = bin_rows(A_rows, kSymLimit, w, s)) return rc;
 
-    hipLaunchKernelGGL((symbolic_hash_kernel<8, kSymTable0>), dim3(kPersistGrid), dim3(kBlock), 0, s, 0, w.bins,
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup0, kSymTable0>), dim3(kPersistGrid), dim3(kBlock), 0, s, 0, w.bins,
                        w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
-    NM_LAUNCH_CHECK("symbolic_hash_kernel<8>");
-    hipLaunchKernelGGL((symbolic_hash_kernel<64, kSymTable1>), dim3(kPersistGrid), dim3(kBlock), 0, s, 1, w.bins,
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup1, kSymTable1>), dim3(kPersistGrid), dim3(kBlock), 0, s, 1, w.bins,
                        w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
-    NM_LAUNCH_CHECK("symbolic_hash_kernel<64>");
-    hipLaunchKernelGGL((symbolic_hash_kernel<256, kSymTable2>), dim3(1024), dim3(kBlock), 0, s, 2, w.bins, w.perm,
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup2, kSymTable2>), dim3(kPersistGrid), dim3(kBlock), 0, s, 2, w.bins,
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup3, kSymTable3>), dim3(kPersistGrid), dim3(kBlock), 0, s, 3, w.bins,
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup4, kSymTable4>), dim3(kPersistGrid), dim3(kBlock), 0, s, 4, w.bins,
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup5, kSymTable5>), dim3(1024), dim3(kBlock), 0, s, 5, w.bins, w.perm,
                        A_indices, A_indptr, B_indices, B_indptr, C_indptr);
-    NM_LAUNCH_CHECK("symbolic_hash_kernel<256>");
+    NM_LAUNCH_CHECK("symbolic_hash_kernel");
     hipLaunchKernelGGL(symbolic_spill_kernel, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm, B_cols,
                        A_indices, A_indptr, B_indices, B_indptr, w.mark, C_indptr);
     NM_LAUNCH_CHECK("symbolic_spill_kernel");
