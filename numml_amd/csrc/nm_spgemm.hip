@@ -488,12 +488,12 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
         int64_t row = 0;
         auto insert = [&](int32_t key) {
             uint32_t h = first_slot<TABLE>(key);
-            for (;;) {
-                const int32_t old = atomicCAS(&tab[h], kEmpty, key);
-                if (old == kEmpty) { ++cnt; break; }
-                if (old == key) break;
+            int32_t old = atomicCAS(&tab[h], kEmpty, key);
+            while (old != kEmpty && old != key) {   // one exit test: the common case probes once
                 h = (h + 1) & (TABLE - 1);
+                old = atomicCAS(&tab[h], kEmpty, key);
             }
+            cnt += old == kEmpty;
         };
         {
             // Latency-lean walk: each lane fetches one entry of A's row together with the
@@ -604,14 +604,16 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
         int64_t row = 0;
         auto add = [&](int32_t key, T prod) {
             uint32_t h = first_slot<TABLE>(key);
-            for (;;) {
-                const int32_t old = atomicCAS(&tab[h], kEmpty, key);
-                if (old == kEmpty) { val[h] = prod; return; }   // 0 + prod == prod exactly
-                if (old == key) break;
+            int32_t old = atomicCAS(&tab[h], kEmpty, key);
+            while (old != kEmpty && old != key) {   // one exit test: the common case probes once
                 h = (h + 1) & (TABLE - 1);
+                old = atomicCAS(&tab[h], kEmpty, key);
             }
-            // the columns of one B row are distinct, so no other lane holds slot h now
-            val[h] = val[h] + prod;
+            // The columns of one B row are distinct, so no other lane holds slot h now.  A slot
+            // claimed just now holds no value yet: its first product is stored as it is
+            // (0 + prod), the read of the slot is dropped by the select.
+            const T cur = val[h];
+            val[h] = old == kEmpty ? prod : cur + prod;
         };
         if (G <= kWave) {
             // Same latency-lean walk as the symbolic phase; entries of A's row are still
