@@ -110,6 +110,12 @@ def test_spgemm_forward_backward(dev, dtype):
         ("empty", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(4, np.int64), (3, 5)),
          G.random_csr(5, 6, 0.5, 1, dtype)),
     ]
+    # rows of 25 and of 125 entries: the 16-lane bins of the hash path, columns that differ by
+    # multiples of the grid's row and plane size, rows of C too long for the 8-lane backward
+    a7 = G.laplace3d(16, dtype, 0)
+    n3 = a7[3][0]
+    a25 = oracle.spgemm_forward(n3, n3, *a7[:3], n3, n3, *a7[:3]) + ((n3, n3),)
+    cases += [("stencil_25x7", a25, a7), ("stencil_7x25", a7, a25), ("stencil_25x25", a25, a25)]
     for name, (ad, ai, ap, (ar, ac)), (bd, bi, bp, (br, bc)) in cases:
         Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(ar, ac, ad, ai, ap, br, bc, bd, bi, bp)
         gC = randn(9, Cd_ref.shape[0], dtype)
