@@ -81,9 +81,9 @@ def _spmv_bytes(rows, cols, nnz, s):
 
 
 class SpMV(Workload):
-    def __init__(self, n=2048, dtype=np.float32, jitter=0, label="poisson2d_2048"):
-        self.n, self.np_dtype, self.jitter = n, dtype, jitter
-        self.name = "spmv" if dtype == np.float32 else "spmv64"
+    def __init__(self, n=2048, dtype=np.float32, jitter=0, label="poisson2d_2048", squared3d=False):
+        self.n, self.np_dtype, self.jitter, self.squared3d = n, dtype, jitter, squared3d
+        self.name = "spmv_rows25" if squared3d else ("spmv" if dtype == np.float32 else "spmv64")
         self.dtype = "f32" if dtype == np.float32 else "f64"
         self.label = label
 
@@ -93,7 +93,13 @@ class SpMV(Workload):
         from numml_amd import _binding
         ext = _binding.ops
         self.ext = ext
-        d, i, p, (rows, cols) = G.poisson2d(self.n, self.np_dtype, jitter_seed=self.jitter)
+        if self.squared3d:
+            # A @ A of the 3D 7-point matrix (25 entries per row), computed by the library itself
+            d, i, p, (rows, cols) = G.laplace3d(self.n, self.np_dtype, jitter_seed=self.jitter)
+            A = tuple(torch.from_numpy(v).to(dev) for v in (d, i, p))
+            d, i, p = (v.cpu().numpy() for v in ext.spgemm_forward(rows, cols, *A, rows, cols, *A))
+        else:
+            d, i, p, (rows, cols) = G.poisson2d(self.n, self.np_dtype, jitter_seed=self.jitter)
         self.host = (d, i, p, rows, cols)
         self.x_h = np.random.default_rng(1).standard_normal(cols).astype(self.np_dtype)
         self.g_h = np.random.default_rng(2).standard_normal(rows).astype(self.np_dtype)
@@ -208,9 +214,16 @@ class SpMM(Workload):
 
 
 class SpGEMM(Workload):
+    """C = L @ R forward + backward.  left="A": L = R = the 3D 7-point matrix (every row takes the
+    merge path); left="AA": L = A @ A (25 entries per row, computed by the library itself at
+    set-up), i.e. the hash path with its 16-lane groups."""
     name = "spgemm"
     unit = "GFLOP/s"
     dtype = "f64"
+
+    def __init__(self, left="A"):
+        self.left = left
+        self.name = "spgemm" if left == "A" else "spgemm_hash"
 
     def setup(self, dev):
         import torch
@@ -220,46 +233,51 @@ class SpGEMM(Workload):
         self.ext = ext
         n = int(os.environ.get("NM_BENCH_SPGEMM_N", "128"))
         d, i, p, (rows, cols) = G.laplace3d(n, np.float64, jitter_seed=0)
-        self.host = (d, i, p, rows, cols)
         t = lambda a: torch.from_numpy(a).to(dev)
-        self.D, self.I, self.P = t(d), t(i), t(p)
-        self.rows, self.cols, self.nnz = rows, cols, d.shape[0]
-        C = ext.spgemm_forward(rows, cols, self.D, self.I, self.P, rows, cols, self.D, self.I, self.P)
+        R = (t(d), t(i), t(p))
+        self.hostR = (d, i, p)
+        if self.left == "AA":
+            L = tuple(ext.spgemm_forward(rows, cols, *R, rows, cols, *R))
+            self.hostL = tuple(v.cpu().numpy() for v in L)
+        else:
+            L, self.hostL = R, self.hostR
+        self.L, self.R = L, R
+        self.rows, self.cols, self.nnz = rows, cols, int(L[0].shape[0])
+        C = ext.spgemm_forward(rows, cols, *L, rows, cols, *R)
         self.nnzC = C[0].shape[0]
         self.gC = torch.from_numpy(np.random.default_rng(1).standard_normal(self.nnzC)).to(dev)
         self.C = C
         lens = np.diff(p)
-        self.products = int(lens[i].sum())
+        self.products = int(lens[self.hostL[1]].sum())
         self.flops = 2 * self.products
         s = 8
         self.bytes_per_step = (self.nnz * (s + 8) + rows * 8 + self.products * (s + 8)
                                + self.nnzC * (s + 8) + rows * 8)
         self.dominant_bytes = self.bytes_per_step
         self.dominant_name = "spgemm forward (symbolic + numeric launches)"
-        self.config = {"workload": f"spgemm_AxA_fwd_bwd_f64_laplace3d_{n}", "rows": rows, "nnz": self.nnz,
+        self.config = {"workload": f"spgemm_{self.left}xA_fwd_bwd_f64_laplace3d_{n}", "rows": rows,
+                       "nnz_left": self.nnz, "nnz_right": int(d.shape[0]),
                        "nnz_C": self.nnzC, "products": self.products, "index_bytes": 8}
 
     def step(self):
-        C = self.ext.spgemm_forward(self.rows, self.cols, self.D, self.I, self.P,
-                                    self.rows, self.cols, self.D, self.I, self.P)
-        g = self.ext.spgemm_backward(self.gC, C[1], C[2], self.rows, self.cols, self.D, self.I, self.P,
-                                     self.rows, self.cols, self.D, self.I, self.P)
+        C = self.ext.spgemm_forward(self.rows, self.cols, *self.L, self.rows, self.cols, *self.R)
+        g = self.ext.spgemm_backward(self.gC, C[1], C[2], self.rows, self.cols, *self.L,
+                                     self.rows, self.cols, *self.R)
         return C, g
 
     def dominant(self):
-        return self.ext.spgemm_forward(self.rows, self.cols, self.D, self.I, self.P,
-                                       self.rows, self.cols, self.D, self.I, self.P)
+        return self.ext.spgemm_forward(self.rows, self.cols, *self.L, self.rows, self.cols, *self.R)
 
     def value(self, ms_per_step):
         return self.flops / (ms_per_step * 1e-3) / 1e9
 
     def cpu_baseline(self, budget_s):
         import oracle
-        d, i, p, rows, cols = self.host
+        rows, cols = self.rows, self.cols
         t0 = time.perf_counter()
-        C = oracle.spgemm_forward(rows, cols, d, i, p, rows, cols, d, i, p)
+        C = oracle.spgemm_forward(rows, cols, *self.hostL, rows, cols, *self.hostR)
         gC = np.random.default_rng(1).standard_normal(C[0].shape[0])
-        oracle.spgemm_backward(gC, C[1], C[2], rows, cols, d, i, p, rows, cols, d, i, p)
+        oracle.spgemm_backward(gC, C[1], C[2], rows, cols, *self.hostL, rows, cols, *self.hostR)
         el = time.perf_counter() - t0
         return {"value": self.flops / el / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
                 "sample": "1 x (spgemm_forward + spgemm_backward) of the full workload, serial C oracle "
@@ -531,6 +549,9 @@ WORKLOADS = {
     "spmv64": lambda: SpMV(256, np.float64, None, "poisson2d_256"),
     "spmm": SpMM,
     "spgemm": SpGEMM,
+    # off the reference's configurations: rows of 25 entries instead of 5-7
+    "spgemm_hash": lambda: SpGEMM("AA"),
+    "spmv_rows25": lambda: SpMV(128, np.float32, 0, "laplace3d_128_squared", squared3d=True),
     "sptrsv": SpTRSV,
     "spsolve": SpSolve,
     "transpose": Transpose,

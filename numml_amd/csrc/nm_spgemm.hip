@@ -293,11 +293,15 @@ __global__ __launch_bounds__(kBlock) void numeric_front_kernel(
         if (steps == 1 && __ballot((ae - ab) >= q) != 0) steps = q;
     // Emitted entries pass through a ring of 8 per group so that the group writes
     // them 8 at a time (one 64-byte piece per array) instead of lane by lane.
-    // The ring reuses the exchange arrays of merge_stage, which are dead by now; a
-    // wavefront's ring entries and its exchange entries are the same 64 slots.
+    // The ring reuses the exchange arrays of merge_stage, which are dead by now FOR THIS
+    // WAVEFRONT: its ring entries and its exchange entries must be the same 64 slots, because
+    // another wavefront of the workgroup may still be reading its own exchange entries (there
+    // is no workgroup barrier).  A value therefore takes a whole 8-byte slot of s_bb whatever
+    // T is (packed floats would put the ring of wavefront w over the exchange entries of
+    // wavefront w / 2, which then read a wrong row start).
     static_assert(sizeof(T) <= sizeof(int64_t), "ring values alias s_bb");
     int32_t *s_oc = s_len;
-    T *s_ov = reinterpret_cast<T *>(s_bb);
+    auto s_ov = [&](int slot) -> T & { return *reinterpret_cast<T *>(s_bb + slot); };
     const int ring = ((threadIdx.x >> 6) * 8 + merge_group()) * 8;
     int emitted = 0;   // entries of this row produced so far
     auto flush = [&](int base) {
@@ -305,7 +309,7 @@ __global__ __launch_bounds__(kBlock) void numeric_front_kernel(
         const int e = base + gl;
         if (e < emitted) {
             C_indices[out0 + e] = (int64_t)s_oc[ring + gl];
-            C_data[out0 + e] = s_ov[ring + gl];
+            C_data[out0 + e] = s_ov(ring + gl);
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     };
@@ -338,7 +342,7 @@ __global__ __launch_bounds__(kBlock) void numeric_front_kernel(
         // every group that is still open has emitted exactly `it` entries so far
         if (gl == steps - 1 && open) {
             s_oc[ring + (it & 7)] = m;
-            s_ov[ring + (it & 7)] = t;
+            s_ov(ring + (it & 7)) = t;
         }
         ++it;
         if (open) emitted = it;

@@ -134,6 +134,21 @@ def test_spgemm_forward_backward(dev, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_spgemm_merge_path_over_many_workgroups(dev, dtype):
+    """A stencil product large enough for thousands of workgroups whose wavefronts run out of
+    step: the merge path's wavefronts share LDS arrays without a workgroup barrier, so each must
+    keep to its own slots whatever the value type (fp32 rings once overlapped a neighbour's)."""
+    d, i, p, (r, c) = G.laplace3d(40, dtype, 0)
+    Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(r, c, d, i, p, r, c, d, i, p)
+    D, I, P = to_dev(dev, d, i, p)
+    for _ in range(3):
+        Cd, Ci, Cp = ext.spgemm_forward(r, c, D, I, P, r, c, D, I, P)
+        assert_same(host(Cp), Cp_ref, "C_indptr")
+        assert_same(host(Ci), Ci_ref, "C_indices")
+        assert_same(host(Cd), Cd_ref, "C_data")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_spgemm_mixed_short_and_long_rows(dev, dtype):
     """Rows that take the merge path (A row and its B rows of at most 8 entries) next to
     rows that do not, inside the same wavefront: lengths 0..8, exactly 8, 9 and longer."""
