@@ -136,3 +136,66 @@ def test_cfg5_sptrsv_fp64_tril_poisson1024(dev):
     # residual of the full-size solve
     r = sps.csr_matrix((d, i, p), shape=(n, n)) @ host(x) - b
     assert np.linalg.norm(r) <= 1e-12 * np.linalg.norm(b) * 10
+
+
+# ---- the same matrices in the other value type ---------------------------------------
+# Lane and LDS layouts depend on the width of a value; the small-case tests cover both widths
+# but only a few workgroups, these run the full grids.
+
+def test_cfg2_matrix_in_fp64(dev):
+    d, i, p, (rows, cols) = G.poisson2d(2048, np.float64, jitter_seed=0)
+    x, g = randn(1, cols, np.float64), randn(2, rows, np.float64)
+    D, I, P, X, Gv = to_dev(dev, d, i, p, x, g)
+    y = ext.spgemv_forward(rows, cols, D, I, P, X)
+    gA, gx = ext.spgemv_backward(Gv, rows, cols, D, I, P, X)
+    gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+    assert_same(host(y), oracle.spgemv_forward(rows, cols, d, i, p, x), "y")
+    assert_same(host(gA), gA_ref, "grad_A")
+    assert_same(host(gx), gx_ref, "grad_x")
+
+
+def test_cfg3_matrix_in_fp64_narrow_operand(dev):
+    rows = cols = 1_000_000
+    n = 16
+    d, i, p, _ = G.powerlaw(rows, cols, target_nnz=16_000_000, seed=0, dtype=np.float64)
+    B, gC = randn(1, (cols, n), np.float64), randn(2, (rows, n), np.float64)
+    D, I, P, Bd, Gd = to_dev(dev, d, i, p, B, gC)
+    C = host(ext.spdmm_forward(rows, cols, D, I, P, Bd))
+    gA, gB = (host(v) for v in ext.spdmm_backward(rows, cols, D, I, P, Bd, Gd))
+    A = sps.csr_matrix((d, i, p), shape=(rows, cols))
+    C_ref, gB_ref = A @ B, A.T.tocsr() @ gC
+    for got, want, what in ((C, C_ref, "C"), (gB, gB_ref, "grad_B")):
+        assert np.all(np.abs(got - want) <= 1e-12 * np.abs(want) + 1e-12 * np.abs(want).max()), what
+    # grad_A[k] = <gC[row(k)], B[col(k)]> on a sample of entries
+    k = np.random.default_rng(3).integers(0, d.shape[0], 200_000)
+    r = np.searchsorted(p, k, side="right") - 1
+    want = np.einsum("kn,kn->k", gC[r], B[i[k]])
+    assert np.all(np.abs(gA[k] - want) <= 1e-12 * np.abs(want) + 1e-12 * np.abs(want).max()), "grad_A"
+
+
+def test_cfg4_matrix_in_fp32(dev):
+    d, i, p, (rows, cols) = G.laplace3d(128, np.float32, jitter_seed=0)
+    D, I, P = to_dev(dev, d, i, p)
+    Cd, Ci, Cp = ext.spgemm_forward(rows, cols, D, I, P, rows, cols, D, I, P)
+    Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(rows, cols, d, i, p, rows, cols, d, i, p)
+    assert_same(host(Cp), Cp_ref, "C_indptr")
+    assert_same(host(Ci), Ci_ref, "C_indices")
+    assert_same(host(Cd), Cd_ref, "C_data")
+    gC = randn(1, Cd_ref.shape[0], np.float32)
+    gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], Ci, Cp, rows, cols, D, I, P, rows, cols, D, I, P)
+    gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, rows, cols, d, i, p, rows, cols, d, i, p)
+    assert_same(host(gA), gA_ref, "grad_A")
+    assert_close(host(gB), gB_ref, "grad_B")
+
+
+def test_cfg5_matrix_in_fp32(dev):
+    d, i, p, (n, _) = G.poisson2d_lower(1024, np.float32, diag_seed=0)
+    b, g = randn(1, n, np.float32), randn(2, n, np.float32)
+    D, I, P, Bv, Gv = to_dev(dev, d, i, p, b, g)
+    x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
+    gA, gb = ext.sptrsv_backward(Gv, x, n, n, D, I, P, True, False, Bv)
+    x_ref = oracle.sptrsv_forward(n, n, d, i, p, True, False, b)
+    gA_ref, gb_ref = oracle.sptrsv_backward(g, x_ref, n, n, d, i, p, True, False)
+    assert_same(host(x), x_ref, "x")
+    assert_same(host(gb), gb_ref, "grad_b")
+    assert_same(host(gA), gA_ref, "grad_A")
