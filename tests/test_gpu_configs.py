@@ -199,3 +199,30 @@ def test_cfg5_matrix_in_fp32(dev):
     assert_same(host(x), x_ref, "x")
     assert_same(host(gb), gb_ref, "grad_b")
     assert_same(host(gA), gA_ref, "grad_A")
+
+
+def test_structure_ops_on_the_cfg2_matrix_in_fp64(dev):
+    """Transpose, linear combination, row sums, diagonal and their backwards over the full grid."""
+    d, i, p, (rows, cols) = G.poisson2d(2048, np.float64, jitter_seed=0)
+    e, j, q, _ = G.poisson2d(2048, np.float64, jitter_seed=1)
+    g = randn(3, rows, np.float64)
+    D, I, P, E, J, Q, Gv = to_dev(dev, d, i, p, e, j, q, g)
+    At = ext.csr_transpose_forward(rows, cols, D, I, P)
+    for got, want, what in zip(At, oracle.csr_transpose(rows, cols, d, i, p), ("At_data", "At_indices", "At_indptr", "At_to_A")):
+        assert_same(host(got), want, what)
+    one, half = torch.tensor(1.0, dtype=torch.float64), torch.tensor(-0.5, dtype=torch.float64)
+    S = ext.splincomb_forward(rows, cols, one, D, I, P, half, E, J, Q)
+    S_ref = oracle.splincomb_forward(rows, cols, 1.0, d, i, p, -0.5, e, j, q)
+    for got, want, what in zip(S, S_ref, ("C_data", "C_indices", "C_indptr")):
+        assert_same(host(got), want, what)
+    gS = randn(4, S_ref[0].shape[0], np.float64)
+    gs = ext.splincomb_backward(rows, cols, one, D, I, P, half, E, J, Q, to_dev(dev, gS)[0], S[1], S[2])
+    for got, want, what in zip(gs, oracle.splincomb_backward(rows, cols, 1.0, d, i, p, -0.5, e, j, q, gS, S_ref[1], S_ref[2]),
+                               ("grad_A", "grad_B")):
+        assert_same(host(got), want, what)
+    A = sps.csr_matrix((d, i, p), shape=(rows, cols))
+    assert_same(host(ext.csr_row_sum_forward(rows, cols, D, I, P)), oracle.csr_row_sum_forward(rows, cols, d, i, p), "row sums")
+    assert_same(host(ext.csr_extract_diagonal_forward(rows, cols, D, I, P)), A.diagonal(), "diagonal")
+    assert_same(host(ext.csr_row_sum_backward(Gv, rows, cols, D, I, P)), np.repeat(g, np.diff(p)), "row sums backward")
+    want = np.where(i == np.repeat(np.arange(rows), np.diff(p)), np.repeat(g, np.diff(p)), 0.0)
+    assert_same(host(ext.csr_extract_diagonal_backward(Gv, rows, cols, D, I, P)), want, "diagonal backward")
