@@ -78,6 +78,7 @@ struct nm_sptrsv_plan {
 namespace {
 
 constexpr int kNarrow = 1024;          // widest level the single-workgroup kernel takes
+constexpr int kWideRows = 128, kWideEntries = 4096;   // a level with both gets a grid launch as well
 constexpr int kBlock = 256;
 constexpr int kRing = 8192;            // LDS ring of recent solutions (doubles, power of two)
 constexpr int kRingSafe = kRing - kNarrow;
@@ -747,6 +748,42 @@ __global__ __launch_bounds__(kBlock) void sptrsv_level_kernel(SolveArgs a, int q
     a.w.xs[q] = xi;
 }
 
+// One level with many entries: slots [q0, q1), G lanes per row.  Lane s of a group takes
+// dependencies s, s + G, ... of its row, so coefficients, slots and solved values are each one
+// request for the whole row instead of a chain of requests in one lane.  The products are
+// added in storage order, like the serial loop (cpp/sparse_csr_cpu.cpp:706-720): the running
+// sum is handed from lane to lane (lane k is right after G - 1 shifts), chunk after chunk.
+template <int G>
+__global__ __launch_bounds__(kBlock) void sptrsv_level_group_kernel(SolveArgs a, int q0, int q1) {
+    static_assert(G == 4 || G == 8 || G == 16, "a group lies inside one 16-lane DPP row");
+    const int sub = (int)threadIdx.x & (G - 1);
+    const int q = q0 + (int)((blockIdx.x * blockDim.x + threadIdx.x) / G);
+    const bool live = q < q1;
+    const int qs = live ? q : q0;
+    const int32_t dlo = a.dptr[qs];
+    const int32_t n = live ? a.dptr[qs + 1] - dlo : 0;
+    double carry = 0.;
+    for (int32_t e0 = 0; __any(e0 < n); e0 += G) {
+        const bool have = e0 + sub < n;
+        const int32_t at = have ? dlo + e0 + sub : 0;   // 0: a readable position (this kernel runs where rows have entries)
+        const double c = a.w.coef[at];
+        const double xv = a.w.xs[a.dslot[at]];
+        const double term = have ? c * xv : 0.;
+        double r = 0.;
+#pragma unroll
+        for (int step = 0; step < G; ++step) {
+            const double prev = nm::dpp_move<0x111>(r);   // row_shr 1
+            r = (sub == 0 ? carry : prev) + term;
+        }
+        carry = __shfl(r, ((int)threadIdx.x & 63) | (G - 1), 64);   // the group's last lane
+    }
+    if (live && sub == 0) {
+        double xi = a.w.rhs[q] - carry;
+        if (!a.unit) xi /= a.w.dg[q];
+        a.w.xs[q] = xi;
+    }
+}
+
 // x[order[q]] = xs[q], rounded once to the value type (cpp/sparse_csr_cpu.cpp:722).
 template <typename T>
 __global__ void unslot_kernel(int64_t n, const int32_t *__restrict__ order, const double *__restrict__ xs,
@@ -792,8 +829,16 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     for (int li = 0; li < n; ++li) {
         const auto &L = p->launches[transposed ? n - 1 - li : li];
         if (L.wide) {
-            const unsigned grid = (unsigned)nm::ceil_div(L.q1 - L.q0, kBlock);
-            hipLaunchKernelGGL(sptrsv_level_kernel, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
+            const int G = L.group[dirn] > 0 ? L.group[dirn] : 1;
+            const unsigned grid = (unsigned)nm::ceil_div((int64_t)(L.q1 - L.q0) * G, kBlock);
+            if (G == 16)
+                hipLaunchKernelGGL(sptrsv_level_group_kernel<16>, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
+            else if (G == 8)
+                hipLaunchKernelGGL(sptrsv_level_group_kernel<8>, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
+            else if (G == 4)
+                hipLaunchKernelGGL(sptrsv_level_group_kernel<4>, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
+            else
+                hipLaunchKernelGGL(sptrsv_level_kernel, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
             NM_LAUNCH_CHECK("sptrsv_level_kernel");
         } else {
             const int count = L.l1 - L.l0;
@@ -981,9 +1026,23 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         }
         flush(a1);
     };
+    // dependency ranges of both directions: a level is also given a launch of its own when it
+    // has enough entries to be worth the chip (one CU takes ~10 us over a level of a few
+    // thousand entries, a grid launch 3-4 us)
+    std::vector<int32_t> dptr_h[2];
+    for (int d = 0; d < 2; ++d) {
+        dptr_h[d].resize((size_t)rows + 1);
+        if (hipMemcpyAsync(dptr_h[d].data(), p->dir[d].dptr, dptr_h[d].size() * 4, hipMemcpyDeviceToHost, s) !=
+                hipSuccess ||
+            hipStreamSynchronize(s) != hipSuccess)
+            return bail(nm::fail(NM_ERR_HIP, "reading the dependency counts back failed"));
+    }
+    auto level_entries = [&](int d, int32_t l) { return dptr_h[d][lp[l + 1]] - dptr_h[d][lp[l]]; };
     int32_t run0 = -1;
     for (int32_t l = 0; l < p->nlevels; ++l) {
-        const bool wide = lp[l + 1] - lp[l] > kNarrow;
+        const int32_t width = lp[l + 1] - lp[l];
+        const int32_t entries = level_entries(0, l) > level_entries(1, l) ? level_entries(0, l) : level_entries(1, l);
+        const bool wide = width > kNarrow || (width >= kWideRows && entries >= kWideEntries);
         if (!wide) {
             if (run0 < 0) run0 = l;
             continue;
@@ -999,15 +1058,15 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         for (int32_t l = L.l0; l < L.l1; ++l) L.width = L.width > lp[l + 1] - lp[l] ? L.width : lp[l + 1] - lp[l];
     }
     for (int d = 0; d < 2; ++d) {
-        if (p->max_deps[d] <= 8) continue;
-        std::vector<int32_t> dptr_h((size_t)rows + 1);
-        if (hipMemcpyAsync(dptr_h.data(), p->dir[d].dptr, dptr_h.size() * 4, hipMemcpyDeviceToHost, s) !=
-                hipSuccess ||
-            hipStreamSynchronize(s) != hipSuccess)
-            return bail(nm::fail(NM_ERR_HIP, "reading the dependency counts back failed"));
         for (auto &L : p->launches) {
-            if (L.wide || L.q1 <= L.q0) continue;
-            const double mean = double(dptr_h[L.q1] - dptr_h[L.q0]) / double(L.q1 - L.q0);
+            if (L.q1 <= L.q0) continue;
+            const double mean = double(dptr_h[d][L.q1] - dptr_h[d][L.q0]) / double(L.q1 - L.q0);
+            if (L.wide) {
+                // a level of its own: lanes per row by its mean row length
+                L.group[d] = mean >= 10. ? 16 : (mean >= 5. ? 8 : (mean >= 2.5 ? 4 : 0));
+                continue;
+            }
+            if (p->max_deps[d] <= 8) continue;
             if (mean >= 40. && L.width <= 16) L.group[d] = 64;
             else if (mean >= 12. && L.width <= 256) L.group[d] = 16;
         }

@@ -6,6 +6,7 @@ rows, both dtypes, both triangles, unit and non-unit diagonals.
 """
 import numpy as np
 import pytest
+import scipy.sparse as sps
 import torch
 
 import oracle
@@ -199,6 +200,29 @@ def test_sptrsv_forward_backward(dev, dtype, lower, unit):
         gA, gb = ext.sptrsv_backward(Gv, x, n, n, D, I, P, lower, unit, Bv)
         assert_same(host(gb), gb_ref, f"{name} grad_b")
         assert_same(host(gA), gA_ref, f"{name} grad_A")
+    # 13 dependencies per row and levels of hundreds of rows (triangle of A @ A, 3D 7-point A):
+    # the levels with thousands of entries get grid launches with 16 lanes per row, which add in
+    # storage order; the small levels at both ends share rows among lanes and match to rounding
+    a7 = G.laplace3d(56, dtype, 0)
+    n = a7[3][0]
+    Cd, Ci, Cp = oracle.spgemm_forward(n, n, *a7[:3], n, n, *a7[:3])
+    M = sps.csr_matrix((Cd, Ci, Cp), shape=(n, n))
+    # off-diagonal row sums below one, so that the unit-diagonal solve stays bounded
+    M = (sps.tril(M, -1) if lower else sps.triu(M, 1)) * 0.01 + sps.diags(np.full(n, 1.25, dtype))
+    M = M.tocsr().astype(dtype)
+    M.sort_indices()
+    d, i, p = M.data, M.indices.astype(np.int64), M.indptr.astype(np.int64)
+    b, g = randn(1, n, dtype), randn(2, n, dtype)
+    x_ref = oracle.sptrsv_forward(n, n, d, i, p, lower, unit, b)
+    gA_ref, gb_ref = oracle.sptrsv_backward(g, x_ref, n, n, d, i, p, lower, unit)
+    D, I, P, Bv, Gv = to_dev(dev, d, i, p, b, g)
+    levels, launches = ext.sptrsv_schedule(n, I, P, lower)
+    assert launches > 20, "levels with thousands of entries are expected to get launches of their own"
+    x = ext.sptrsv_forward(n, n, D, I, P, lower, unit, Bv)
+    assert_close(host(x), x_ref, "stencil triangle x")
+    gA, gb = ext.sptrsv_backward(Gv, x, n, n, D, I, P, lower, unit, Bv)
+    assert_close(host(gb), gb_ref, "stencil triangle grad_b")
+    assert_close(host(gA), gA_ref, "stencil triangle grad_A")
 
 
 def _transpose(csr):
