@@ -145,3 +145,101 @@ def test_triangular_and_direct_solves(dev, seed, dtype):
     out = ext.splu(m, m, *to_dev(dev, d, i, p))
     for got, want, what in zip(out, oracle.splu(m, m, d, i, p), ("M_data", "M_indices", "M_indptr", "Mt_data", "Mt_indices", "Mt_indptr")):
         assert_same(host(got), want, what)
+
+
+# ---- the same comparisons over grids of thousands of workgroups ----------------------
+# Wavefronts of a workgroup that share LDS without a barrier, and workgroups that meet in
+# global memory, only get out of step on inputs of this size.
+
+def _big(seed, dtype, rows, cols, lens):
+    """CSR with the given row lengths, distinct sorted uniform columns, N(0,1) values."""
+    rng = np.random.default_rng(5000 + seed)
+    lens = np.minimum(lens, cols).astype(np.int64)
+    indptr = np.zeros(rows + 1, dtype=np.int64)
+    np.cumsum(lens, out=indptr[1:])
+    row_of = np.repeat(np.arange(rows, dtype=np.int64), lens)
+    key = row_of * cols + rng.integers(0, cols, row_of.shape[0], dtype=np.int64)
+    key.sort()
+    while True:
+        dup = np.flatnonzero(key[1:] == key[:-1]) + 1
+        if dup.size == 0:
+            break
+        key[dup] = row_of[dup] * cols + rng.integers(0, cols, dup.size, dtype=np.int64)
+        key.sort()
+    return rng.standard_normal(key.shape[0]).astype(dtype), key - row_of * cols, indptr, (rows, cols)
+
+
+def _big_draw(seed, dtype):
+    rng = np.random.default_rng(4000 + seed)
+    rows, cols = int(rng.integers(60_000, 220_000)), int(rng.integers(40_000, 200_000))
+    kind = seed % 3
+    if kind == 0:      # 0-12 entries per row, many empty rows
+        lens = rng.integers(0, 13, rows) * (rng.random(rows) < 0.8)
+    elif kind == 1:    # 15-40 entries per row: blocks of rows that do not fit the LDS tiles
+        lens = rng.integers(15, 41, rows)
+    else:              # short rows with a heavy tail up to thousands of entries
+        lens = np.clip(rng.zipf(1.9, rows), 1, 6000)
+    return _big(seed, dtype, rows, cols, lens)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("seed", range(6))
+def test_many_workgroups(dev, seed, dtype):
+    import torch
+    ext = numml_amd.load_compiled()
+    d, i, p, (rows, cols) = _big_draw(seed, dtype)
+    print(f"case seed={seed} {dtype.__name__} {rows}x{cols} nnz={d.shape[0]} longest row {np.diff(p).max()}", flush=True)
+    D, I, P = to_dev(dev, d, i, p)
+    x, g = randn(seed, cols, dtype), randn(seed + 1, rows, dtype)
+    X, Gv = to_dev(dev, x, g)
+    assert_close(host(ext.spgemv_forward(rows, cols, D, I, P, X)), oracle.spgemv_forward(rows, cols, d, i, p, x), "y")
+    gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+    for mode in ("planned", "atomic"):
+        ext.set_backward_mode(mode)
+        try:
+            gA, gx = ext.spgemv_backward(Gv, rows, cols, D, I, P, X)
+        finally:
+            ext.set_backward_mode("planned")
+        assert_same(host(gA), gA_ref, f"spmv grad_A ({mode})")
+        assert_close(host(gx), gx_ref, f"spmv grad_x ({mode})")
+    n = (4, 16, 33, 64, 7, 100)[seed]
+    B, gC = randn(seed + 2, (cols, n), dtype), randn(seed + 3, (rows, n), dtype)
+    Bd, gCd = to_dev(dev, B, gC)
+    assert_close(host(ext.spdmm_forward(rows, cols, D, I, P, Bd)), oracle.spdmm_forward(rows, cols, d, i, p, B), f"C n={n}")
+    gA, gB = ext.spdmm_backward(rows, cols, D, I, P, Bd, gCd)
+    gA_ref, gB_ref = oracle.spdmm_backward(rows, cols, d, i, p, B, gC)
+    assert_close(host(gA), gA_ref, f"spmm grad_A n={n}")
+    assert_close(host(gB), gB_ref, f"spmm grad_B n={n}")
+    out = ext.csr_transpose_forward(rows, cols, D, I, P)
+    for got, want, what in zip(out, oracle.csr_transpose(rows, cols, d, i, p), ("At_data", "At_indices", "At_indptr", "map")):
+        assert_same(host(got), want, what)
+    assert_close(host(ext.csr_row_sum_forward(rows, cols, D, I, P)), oracle.csr_row_sum_forward(rows, cols, d, i, p), "row sums")
+    assert_same(host(ext.csr_extract_diagonal_forward(rows, cols, D, I, P)),
+                oracle.csr_extract_diagonal_forward(rows, cols, d, i, p), "diagonal")
+    # linear combination with a second pattern of the same shape
+    e, j, q, _ = _big(seed + 100, dtype, rows, cols, np.random.default_rng(seed).integers(0, 9, rows))
+    al, be = torch.tensor(1.5), torch.tensor(-0.25)
+    E = to_dev(dev, e, j, q)
+    S = ext.splincomb_forward(rows, cols, al, D, I, P, be, *E)
+    S_ref = oracle.splincomb_forward(rows, cols, 1.5, d, i, p, -0.25, e, j, q)
+    for got, want, what in zip(S, S_ref, ("S_data", "S_indices", "S_indptr")):
+        assert_same(host(got), want, what)
+    gS = randn(seed + 5, S_ref[0].shape[0], dtype)
+    gs = ext.splincomb_backward(rows, cols, al, D, I, P, be, *E, to_dev(dev, gS)[0], S[1], S[2])
+    for got, want, what in zip(gs, oracle.splincomb_backward(rows, cols, 1.5, d, i, p, -0.25, e, j, q, gS, S_ref[1], S_ref[2]),
+                               ("grad_A", "grad_B")):
+        assert_same(host(got), want, f"lincomb {what}")
+    # product with a thin second operand
+    m = int(np.random.default_rng(seed).integers(2_000, 50_000))
+    d2, i2, p2, _ = _big(seed + 200, dtype, cols, m, np.random.default_rng(seed + 1).integers(0, 7, cols))
+    B2 = to_dev(dev, d2, i2, p2)
+    C = ext.spgemm_forward(rows, cols, D, I, P, cols, m, *B2)
+    C_ref = oracle.spgemm_forward(rows, cols, d, i, p, cols, m, d2, i2, p2)
+    assert_same(host(C[2]), C_ref[2], "C_indptr")
+    assert_same(host(C[1]), C_ref[1], "C_indices")
+    assert_close(host(C[0]), C_ref[0], "C_data")
+    gCs = randn(seed + 4, C_ref[0].shape[0], dtype)
+    gA, gB = ext.spgemm_backward(to_dev(dev, gCs)[0], C[1], C[2], rows, cols, D, I, P, cols, m, *B2)
+    gA_ref, gB_ref = oracle.spgemm_backward(gCs, C_ref[1], C_ref[2], rows, cols, d, i, p, cols, m, d2, i2, p2)
+    assert_close(host(gA), gA_ref, "spgemm grad_A")
+    assert_close(host(gB), gB_ref, "spgemm grad_B")
