@@ -137,12 +137,21 @@ int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
  * C between them:
  *
  *   nm_spgemm_workspace_bytes  -> bytes of device scratch both phases need
- *   nm_spgemm_symbolic         -> fills C_indptr (A_rows + 1 entries); the
- *                                 caller reads nnz(C) = C_indptr[A_rows]
- *                                 (its own device->host copy) and allocates
+ *   nm_spgemm_symbolic         -> fills C_indptr (A_rows + 1 entries)
+ *   nm_spgemm_symbolic_result  -> waits for the stream and hands the host
+ *                                 nnz(C) = C_indptr[A_rows], with which the
+ *                                 caller allocates, and the number of rows
+ *                                 the hash path took (the reference's own
+ *                                 read of the last row pointer,
+ *                                 cpp/sparse_csr_cpu.cpp:166, is this
+ *                                 synchronisation point); a caller may read
+ *                                 C_indptr[A_rows] itself instead
  *   nm_spgemm_numeric          -> fills C_indices (ascending in each row) and
  *                                 C_data; entries whose sum is 0 are kept,
- *                                 as the reference keeps them.
+ *                                 as the reference keeps them.  hash_rows is
+ *                                 the figure nm_spgemm_symbolic_result gave,
+ *                                 or -1 when it was not asked: with 0 the
+ *                                 launches of the hash path are left out.
  *
  * The same workspace (contents preserved) must be passed to both phases.
  * Products of one output entry are added in the order of A's row, which is
@@ -155,11 +164,16 @@ int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols,
                        int64_t *C_indptr, void *workspace, size_t workspace_bytes,
                        nm_stream stream);
 
+int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const void *workspace,
+                              size_t workspace_bytes, int64_t *nnz_C, int64_t *hash_rows,
+                              nm_stream stream);
+
 int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t B_cols,
                       const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,
                       const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
                       const int64_t *C_indptr, int64_t *C_indices, void *C_data,
-                      void *workspace, size_t workspace_bytes, nm_stream stream);
+                      void *workspace, size_t workspace_bytes, int64_t hash_rows,
+                      nm_stream stream);
 
 /* grad_A[(i,j)] = sum_c gC[i,c] B[j,c];  grad_B[(k,c)] = sum_i A[i,k] gC[i,c],
  * both restricted to the stored patterns.  Stands in for spgemm_backward

@@ -1,5 +1,5 @@
 // In-place exclusive prefix sum of an int64 device array (three launches:
-// per-block sums, scan of the sums by one workgroup, apply).
+// per-block sums, scan of the sums by one workgroup, apply; one launch for short arrays).
 #pragma once
 
 #include "nm_common.hpp"
@@ -88,9 +88,40 @@ static __global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(int64_t *
     }
 }
 
+// The whole scan by one workgroup, for arrays short enough that three launches would cost more
+// than the work: 8 consecutive items per lane and pass.
+constexpr int kScanSmall = 8192;
+static __global__ __launch_bounds__(1024) void scan_small_kernel(int64_t *a, int64_t n) {
+    __shared__ int64_t s_wave[1024 / kWave];
+    int64_t carry = 0;
+    for (int64_t c0 = 0; c0 < n; c0 += 1024 * kScanItems) {
+        const int64_t base = c0 + (int64_t)threadIdx.x * kScanItems;
+        int64_t item[kScanItems];
+        int64_t v = 0;
+#pragma unroll
+        for (int i = 0; i < kScanItems; ++i) {
+            item[i] = base + i < n ? a[base + i] : 0;
+            v += item[i];
+        }
+        int64_t total;
+        int64_t run = carry + block_exclusive_scan(v, s_wave, total);
+#pragma unroll
+        for (int i = 0; i < kScanItems; ++i) {
+            if (base + i < n) a[base + i] = run;
+            run += item[i];
+        }
+        carry += total;
+    }
+}
+
 // a[i] <- sum of a[0, i) for i in [0, n).  `scratch` holds scan_scratch_bytes(n).
 inline int scan_exclusive_i64(int64_t *a, int64_t n, int64_t *scratch, hipStream_t s) {
     if (n <= 0) return NM_OK;
+    if (n <= kScanSmall) {
+        hipLaunchKernelGGL(scan_small_kernel, dim3(1), dim3(1024), 0, s, a, n);
+        NM_LAUNCH_CHECK("scan_small_kernel");
+        return NM_OK;
+    }
     const int64_t tiles = ceil_div(n, kScanTile);
     if (tiles > kMaxGrid) return fail(NM_ERR_UNSUPPORTED, "scan of %lld items is too long", (long long)n);
     hipLaunchKernelGGL(scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(kScanBlock), 0, s, a, n, scratch);

@@ -75,6 +75,7 @@ struct Work {
     int64_t *scan;     // scan scratch
     int32_t *mark;     // [spill_groups(B_cols) * B_cols]
     double *acc;       // [spill_groups(B_cols) * B_cols]
+    int64_t *summary;  // [2]: nnz(C) and the number of rows on the hash path, for the host
 };
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
@@ -92,7 +93,8 @@ size_t work_layout(int64_t rows, int64_t B_cols, void *base, Work *w) {
     int64_t *scan = (int64_t *)take(nm::scan_scratch_bytes(rows + 1));
     int32_t *mark = (int32_t *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 4);
     double *acc = (double *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 8);
-    if (w) *w = Work{key, perm, bins, scan, mark, acc};
+    int64_t *summary = (int64_t *)take(2 * 8);
+    if (w) *w = Work{key, perm, bins, scan, mark, acc, summary};
     return off;
 }
 
@@ -212,6 +214,7 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     __shared__ int64_t s_bb[kBlock];
     __shared__ int32_t s_len[kBlock];
     const int gl = merge_lane();
+    if (blockIdx.x == 0 && threadIdx.x == 0) C_count[rows] = 0;   // the scan's last entry: nnz(C)
     const int64_t batch = nm::xcd_tile(blockIdx.x, nbatch_padded);
     const int64_t row = batch * kMergeRows + (threadIdx.x >> 6) * 8 + merge_group();
     const bool live = row < rows;
@@ -451,9 +454,95 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
     }
 }
 
+// What the host needs between the phases, in one place: nnz(C) and the rows the hash path took.
+__global__ void summary_kernel(const int64_t *__restrict__ nnz_c, const int32_t *__restrict__ bins,
+                               int64_t *__restrict__ summary) {
+    if (threadIdx.x == 0) {
+        summary[0] = *nnz_c;
+        summary[1] = bins[kBinStart + kBins];
+    }
+}
+
+// host_pinned[0..1] = summary, then host_pinned[2] = ticket: the host polls the ticket.
+__global__ void summary_out_kernel(const int64_t *__restrict__ summary, volatile int64_t *host_pinned,
+                                   int64_t ticket) {
+    if (threadIdx.x == 0) {
+        host_pinned[0] = summary[0];
+        host_pinned[1] = summary[1];
+        __threadfence_system();
+        host_pinned[2] = ticket;
+    }
+}
+
+// The four binning steps by one workgroup, for so few rows that the launches cost more than the
+// work: count, offsets, then rows placed in ascending order inside each bin (ballots, as in the
+// grid-wide kernels).
+constexpr int kBinSmallRows = 4096;
+__global__ __launch_bounds__(1024) void bin_small_kernel(int64_t rows, const int32_t *__restrict__ key,
+                                                         BinLimits lim, int32_t *bins,
+                                                         int32_t *__restrict__ perm) {
+    constexpr int kWaves = 1024 / kWave;
+    __shared__ int s_cnt[kWaves][kBins];
+    __shared__ int s_start[kBins + 1], s_run[kBins];
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // rows per bin
+    int mine[kBins] = {};
+    for (int64_t i0 = 0; i0 < rows; i0 += 1024) {
+        const int64_t i = i0 + threadIdx.x;
+        const int b = i < rows ? bin_of(key[i], lim) : -1;
+#pragma unroll
+        for (int q = 0; q < kBins; ++q) mine[q] += __popcll(__ballot(b == q));
+    }
+    if (lane == 0)
+        for (int q = 0; q < kBins; ++q) s_cnt[wave][q] = mine[q];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int q = 0; q < kBins; ++q) {
+            s_start[q] = run;
+            s_run[q] = run;
+            for (int w = 0; w < kWaves; ++w) run += s_cnt[w][q];
+        }
+        s_start[kBins] = run;
+    }
+    __syncthreads();
+    // rows placed chunk by chunk, wavefront by wavefront, lane by lane: ascending inside each bin
+    for (int64_t i0 = 0; i0 < rows; i0 += 1024) {
+        const int64_t i = i0 + threadIdx.x;
+        const int b = i < rows ? bin_of(key[i], lim) : -1;
+        int before = 0;
+#pragma unroll
+        for (int q = 0; q < kBins; ++q) {
+            const unsigned long long m = __ballot(b == q);
+            if (b == q) before = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) s_cnt[wave][q] = __popcll(m);
+        }
+        __syncthreads();
+        if (b >= 0) {
+            int off = s_run[b] + before;
+            for (int w = 0; w < wave; ++w) off += s_cnt[w][b];
+            perm[off] = (int32_t)i;
+        }
+        __syncthreads();
+        if (threadIdx.x < kBins) {
+            int t = 0;
+            for (int w = 0; w < kWaves; ++w) t += s_cnt[w][threadIdx.x];
+            s_run[threadIdx.x] += t;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x <= kBins) bins[kBinStart + threadIdx.x] = s_start[threadIdx.x];
+    if (threadIdx.x < kBins) bins[threadIdx.x] = s_start[threadIdx.x + 1] - s_start[threadIdx.x];
+}
+
 int bin_rows(int64_t rows, const int32_t limit[kBins - 1], const Work &w, hipStream_t s) {
     BinLimits lim;
     for (int q = 0; q < kBins - 1; ++q) lim.l[q] = limit[q];
+    if (rows <= kBinSmallRows) {
+        hipLaunchKernelGGL(bin_small_kernel, dim3(1), dim3(1024), 0, s, rows, w.key, lim, w.bins, w.perm);
+        NM_LAUNCH_CHECK("bin_small_kernel");
+        return NM_OK;
+    }
     int64_t grid = nm::ceil_div(rows, kBlock);
     if (grid > 4096) grid = 4096;
     if (grid < 1) grid = 1;
@@ -1162,8 +1251,7 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     if (workspace_bytes < need)
         return nm::fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace_bytes, need);
     hipStream_t s = nm::as_stream(stream);
-    if (int rc = nm::fill_async(C_indptr + A_rows, 1, (int64_t)0, s)) return rc;
-    if (A_rows == 0) return NM_OK;
+    if (A_rows == 0) return nm::fill_async(C_indptr, 1, (int64_t)0, s);
 
     const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
     hipLaunchKernelGGL(symbolic_front_kernel, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
@@ -1188,14 +1276,58 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
                        A_indices, A_indptr, B_indices, B_indptr, w.mark, C_indptr);
     NM_LAUNCH_CHECK("symbolic_spill_kernel");
     // counts sit in C_indptr[0, rows), C_indptr[rows] = 0: the exclusive scan is the row pointer
-    return nm::scan_exclusive_i64(C_indptr, A_rows + 1, w.scan, s);
+    if (int rc = nm::scan_exclusive_i64(C_indptr, A_rows + 1, w.scan, s)) return rc;
+    hipLaunchKernelGGL(summary_kernel, dim3(1), dim3(64), 0, s, C_indptr + A_rows, w.bins, w.summary);
+    NM_LAUNCH_CHECK("summary_kernel");
+    return NM_OK;
+}
+
+extern "C" int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const void *workspace,
+                                         size_t workspace_bytes, int64_t *nnz_C, int64_t *hash_rows,
+                                         nm_stream stream) {
+    if (int rc = check_common(A_rows, B_cols)) return rc;
+    NM_REQUIRE(workspace && nnz_C && hash_rows, "null pointer argument");
+    Work w;
+    const size_t need = work_layout(A_rows, B_cols, const_cast<void *>(workspace), &w);
+    if (workspace_bytes < need)
+        return nm::fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    *nnz_C = 0;
+    *hash_rows = 0;
+    if (A_rows == 0) return NM_OK;
+    hipStream_t s = nm::as_stream(stream);
+    // a pinned landing place per host thread, kept for the life of the process: a copy into
+    // pageable memory goes through the runtime's staging path and takes several times as long
+    // The two numbers are written straight into pinned host memory by a one-lane kernel, followed
+    // by a ticket the host polls for: waking up from hipStreamSynchronize, or a copy-engine
+    // transfer of 16 bytes, takes ~30 us, several times what the kernels of a small product take
+    // together.  One landing place per host thread, kept for the life of the process.
+    static thread_local volatile int64_t *both = nullptr;
+    static thread_local int64_t ticket = 0;
+    if (!both) {
+        void *mem = nullptr;
+        NM_HIP_TRY(hipHostMalloc(&mem, 3 * sizeof(int64_t), hipHostMallocDefault));
+        both = (volatile int64_t *)mem;
+        both[2] = 0;
+    }
+    ++ticket;
+    hipLaunchKernelGGL(summary_out_kernel, dim3(1), dim3(64), 0, s, w.summary, both, ticket);
+    NM_LAUNCH_CHECK("summary_out_kernel");
+    bool arrived = false;
+    for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = both[2] == ticket;
+    if (!arrived) {   // a long queue ahead of the kernel: wait the ordinary way
+        NM_HIP_TRY(hipStreamSynchronize(s));
+        NM_REQUIRE(both[2] == ticket, "the symbolic phase's result did not arrive");
+    }
+    *nnz_C = both[0];
+    *hash_rows = both[1];
+    return NM_OK;
 }
 
 extern "C" int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t B_cols,
                                  const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,
                                  const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
                                  const int64_t *C_indptr, int64_t *C_indices, void *C_data, void *workspace,
-                                 size_t workspace_bytes, nm_stream stream) {
+                                 size_t workspace_bytes, int64_t hash_rows, nm_stream stream) {
     if (int rc = check_common(A_rows, B_cols)) return rc;
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
     NM_REQUIRE(A_indptr && B_indptr && C_indptr && workspace, "null pointer argument");
@@ -1207,9 +1339,14 @@ extern "C" int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, in
     hipStream_t s = nm::as_stream(stream);
     int64_t grid = nm::ceil_div(A_rows, kBlock);
     if (grid > 65536) grid = 65536;
-    hipLaunchKernelGGL(row_length_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, C_indptr, w.key);
-    NM_LAUNCH_CHECK("row_length_kernel");
-    if (int rc = bin_rows(A_rows, kNumLimit, w, s)) return rc;
+    // hash_rows == 0 (from nm_spgemm_symbolic_result): every row is one of the merge path's and
+    // the binning and the hash launches, a dozen launches that would find nothing to do, are left out
+    const bool hashed = hash_rows != 0;
+    if (hashed) {
+        hipLaunchKernelGGL(row_length_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, C_indptr, w.key);
+        NM_LAUNCH_CHECK("row_length_kernel");
+        if (int rc = bin_rows(A_rows, kNumLimit, w, s)) return rc;
+    }
     const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
     if (dt == NM_F32)
         hipLaunchKernelGGL(numeric_front_kernel<float>, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
@@ -1220,6 +1357,7 @@ extern "C" int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, in
                            w.key, (const double *)A_data, A_indices, A_indptr, (const double *)B_data, B_indices,
                            B_indptr, C_indptr, C_indices, (double *)C_data);
     NM_LAUNCH_CHECK("numeric_front_kernel");
+    if (!hashed) return NM_OK;
     if (dt == NM_F32)
         return launch_numeric<float>(w, B_cols, A_data, A_indices, A_indptr, B_data, B_indices, B_indptr,
                                      C_indptr, C_indices, C_data, s);

@@ -535,14 +535,16 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
                              C_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, st),
           "nm_spgemm_symbolic");
     // the one device->host read the interface makes inherent: C is returned exactly sized
-    const int64_t nnz_c = C_indptr[A_rows].item<int64_t>();
+    int64_t nnz_c = 0, hash_rows = 0;
+    check(nm_spgemm_symbolic_result(A_rows, B_cols, work.data_ptr(), bytes, &nnz_c, &hash_rows, st),
+          "nm_spgemm_symbolic_result");
     Tensor C_indices = torch::empty({nnz_c}, iopt);
     Tensor C_data = torch::empty({nnz_c}, A_data.options());
     check(nm_spgemm_numeric(dtype_of(A_data), A_rows, A_cols, B_cols, A_data.data_ptr(),
                             A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
                             B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
                             C_indptr.data_ptr<int64_t>(), C_indices.data_ptr<int64_t>(), C_data.data_ptr(),
-                            work.data_ptr(), bytes, st),
+                            work.data_ptr(), bytes, hash_rows, st),
           "nm_spgemm_numeric");
     return {C_data, C_indices, C_indptr};
 }

@@ -424,13 +424,15 @@ def spgemm_forward(A_rows, A_cols, A_data, A_indices, A_indptr,
         _lib.check(L.nm_spgemm_symbolic(
             A_rows, A_cols, B_cols, _ptr(A_indices), _ptr(A_indptr), _ptr(B_indices), _ptr(B_indptr),
             _ptr(C_indptr), _ptr(work), nbytes.value, st), "nm_spgemm_symbolic")
-        nnz_c = int(C_indptr[-1].item())
-        C_indices = torch.empty(nnz_c, dtype=torch.int64, device=dev)
-        C_data = torch.empty(nnz_c, dtype=A_data.dtype, device=dev)
+        nnz_c, hash_rows = ctypes.c_int64(0), ctypes.c_int64(0)
+        _lib.check(L.nm_spgemm_symbolic_result(A_rows, B_cols, _ptr(work), nbytes.value, ctypes.byref(nnz_c),
+                                               ctypes.byref(hash_rows), st), "nm_spgemm_symbolic_result")
+        C_indices = torch.empty(nnz_c.value, dtype=torch.int64, device=dev)
+        C_data = torch.empty(nnz_c.value, dtype=A_data.dtype, device=dev)
         _lib.check(L.nm_spgemm_numeric(
             _dt(A_data), A_rows, A_cols, B_cols, _ptr(A_data), _ptr(A_indices), _ptr(A_indptr),
             _ptr(B_data), _ptr(B_indices), _ptr(B_indptr), _ptr(C_indptr), _ptr(C_indices),
-            _ptr(C_data), _ptr(work), nbytes.value, st), "nm_spgemm_numeric")
+            _ptr(C_data), _ptr(work), nbytes.value, hash_rows.value, st), "nm_spgemm_numeric")
     return [C_data, C_indices, C_indptr]
 
 
