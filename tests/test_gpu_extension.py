@@ -170,3 +170,35 @@ def test_install_registers_the_reference_module_name(cpp):
         sys.modules.pop("numml_torch_cpp", None)
         if saved is not None:
             sys.modules["numml_torch_cpp"] = saved
+
+
+@pytest.mark.parametrize("hint", ["given", "unknown"])
+def test_spgemm_through_the_c_abi_with_and_without_the_hash_row_count(dev, hint):
+    """The numeric phase takes the number of hash-path rows that nm_spgemm_symbolic_result reports
+    (0 lets it leave the hash launches out), or -1 from a caller that read nnz(C) itself."""
+    import ctypes
+    from numml_amd import _lib
+    L = _lib.lib()
+    for name, (d, i, p, (r, c)) in (("stencil: no row on the hash path", G.poisson2d(40, np.float64, 1)),
+                                    ("random: rows on both paths", G.random_csr(500, 500, 0.03, 2, np.float64))):
+        D, I, P = to_dev(dev, d, i, p)
+        ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+        st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(L.nm_spgemm_workspace_bytes(r, c, ctypes.byref(nbytes)), "bytes")
+        work = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+        Cp = torch.empty(r + 1, dtype=torch.int64, device=dev)
+        _lib.check(L.nm_spgemm_symbolic(r, c, c, ptr(I), ptr(P), ptr(I), ptr(P), ptr(Cp), ptr(work), nbytes.value, st), "symbolic")
+        nnz_c, hash_rows = ctypes.c_int64(-7), ctypes.c_int64(-7)
+        _lib.check(L.nm_spgemm_symbolic_result(r, c, ptr(work), nbytes.value, ctypes.byref(nnz_c), ctypes.byref(hash_rows), st),
+                   "result")
+        Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(r, c, d, i, p, r, c, d, i, p)
+        assert nnz_c.value == Cd_ref.shape[0] == int(Cp[-1].item()), name
+        assert (hash_rows.value == 0) == name.startswith("stencil"), (name, hash_rows.value)
+        Ci = torch.empty(nnz_c.value, dtype=torch.int64, device=dev)
+        Cd = torch.empty(nnz_c.value, dtype=torch.float64, device=dev)
+        _lib.check(L.nm_spgemm_numeric(1, r, c, c, ptr(D), ptr(I), ptr(P), ptr(D), ptr(I), ptr(P), ptr(Cp), ptr(Ci), ptr(Cd),
+                                       ptr(work), nbytes.value, hash_rows.value if hint == "given" else -1, st), "numeric")
+        assert_same(host(Cp), Cp_ref, f"{name} C_indptr")
+        assert_same(host(Ci), Ci_ref, f"{name} C_indices")
+        assert_same(host(Cd), Cd_ref, f"{name} C_data")
