@@ -39,8 +39,8 @@ using nm::kWave;
 
 constexpr int32_t kEmpty = -1;
 constexpr int kBlock = 256;
-constexpr int kBins = 7;
-constexpr int kBinStart = 8, kBinCursor = 16, kBinInts = 24;   // layout of the bins array, see Work
+constexpr int kBins = 8;
+constexpr int kBinStart = 8, kBinCursor = 20, kBinInts = 32;   // layout of the bins array, see Work
 // Workgroups (and dense accumulator slices of B_cols entries each) of the spill path: as many as
 // fit a fixed budget of scratch, between 8 and 64.
 constexpr int64_t kSpillBudgetBytes = int64_t(192) << 20;
@@ -53,16 +53,16 @@ constexpr int kTablePad = 4;         // entries between the hash tables of neigh
 constexpr int kAhead = 8;            // B rows whose first columns a group requests before inserting any
 
 // bin upper limits (inclusive); the last bin takes the rest and spills
-constexpr int32_t kSymLimit[6] = {64, 128, 256, 512, 1024, 8192};     // on the product bound
-constexpr int32_t kNumLimit[6] = {32, 64, 128, 256, 512, 4096};       // on the exact row length
+constexpr int32_t kSymLimit[7] = {64, 128, 256, 512, 1024, 2048, 8192};     // on the product bound
+constexpr int32_t kNumLimit[7] = {32, 64, 128, 256, 512, 1024, 4096};       // on the exact row length
 // lanes per row and table sizes per bin.  The kernels wait on memory (A's row, the bounds of its B
 // rows, the B rows: a chain of round trips per row) and LDS decides how many rows a CU has in
 // flight, so rows get the smallest table that holds them at half load.
-constexpr int kGroup0 = 8, kGroup1 = 16, kGroup2 = 16, kGroup3 = 64, kGroup4 = 64, kGroup5 = 256;
+constexpr int kGroup0 = 8, kGroup1 = 16, kGroup2 = 16, kGroup3 = 64, kGroup4 = 64, kGroup5 = 256, kGroup6 = 256;
 constexpr int kSymTable0 = 128, kSymTable1 = 256, kSymTable2 = 512, kSymTable3 = 1024, kSymTable4 = 2048,
-              kSymTable5 = 16384;
+              kSymTable5 = 4096, kSymTable6 = 16384;
 constexpr int kNumTable0 = 64, kNumTable1 = 128, kNumTable2 = 256, kNumTable3 = 512, kNumTable4 = 1024,
-              kNumTable5 = 8192;
+              kNumTable5 = 2048, kNumTable6 = 8192;
 
 constexpr int kMergeCap = 8;                  // longest A row and B row of the merge path
 constexpr int32_t kColEnd = 0x7fffffff;       // past-the-end column of a staged B row
@@ -983,7 +983,7 @@ constexpr int kBwdStage = 64;
 constexpr int kBwdLong = kBwdStage;
 constexpr int kBwdLongCap = 2048;     // rows up to this long: columns and gradient in LDS
 constexpr int kBwdHugeCap = 14336;    // longer rows: columns only
-constexpr int kBwdLongChunk = 256;   // rows a workgroup of the long-row kernel looks through at a time
+constexpr int kBwdLongChunk = 256;   // rows a workgroup of the long-row kernel looks through at a time, at most
 constexpr int kBwdWide = 64;         // rows of B longer than this are walked by a whole wavefront ...
 constexpr int kBwdWideCap = 1024;    // ... up to this many per row of A (the rest stay with their group)
 
@@ -1059,7 +1059,7 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
 
 template <typename T, int CAP, bool STAGE_G>
 __global__ __launch_bounds__(kBlock) void spgemm_bwd_long_kernel(
-    int64_t A_rows, int64_t longer_than, int64_t up_to, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
+    int64_t A_rows, int chunk, int64_t longer_than, int64_t up_to, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
     const int64_t *__restrict__ C_indptr, const T *__restrict__ A_data,
     const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
     const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
@@ -1073,11 +1073,11 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_long_kernel(
     const int gl = threadIdx.x % G, gi = threadIdx.x / G;
     const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
     const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    for (int64_t r0 = (int64_t)blockIdx.x * kBwdLongChunk; r0 < A_rows; r0 += (int64_t)gridDim.x * kBwdLongChunk) {
+    for (int64_t r0 = (int64_t)blockIdx.x * chunk; r0 < A_rows; r0 += (int64_t)gridDim.x * chunk) {
         // the long rows among this chunk of rows (mostly there are none)
         const int64_t r = r0 + threadIdx.x;
         bool is_long = false;
-        if (threadIdx.x < kBwdLongChunk && r < A_rows) {
+        if ((int)threadIdx.x < chunk && r < A_rows) {
             const int64_t len = C_indptr[r + 1] - C_indptr[r];
             is_long = len > longer_than && len <= up_to;
         }
@@ -1222,7 +1222,8 @@ int launch_numeric(const Work &w, int64_t B_cols, const void *A_data, const int6
     if (int rc = hashed(integral_constant<int, kGroup2>{}, integral_constant<int, kNumTable2>{}, 2, kPersistGrid)) return rc;
     if (int rc = hashed(integral_constant<int, kGroup3>{}, integral_constant<int, kNumTable3>{}, 3, kPersistGrid)) return rc;
     if (int rc = hashed(integral_constant<int, kGroup4>{}, integral_constant<int, kNumTable4>{}, 4, kPersistGrid)) return rc;
-    if (int rc = hashed(integral_constant<int, kGroup5>{}, integral_constant<int, kNumTable5>{}, 5, 1024)) return rc;
+    if (int rc = hashed(integral_constant<int, kGroup5>{}, integral_constant<int, kNumTable5>{}, 5, kPersistGrid)) return rc;
+    if (int rc = hashed(integral_constant<int, kGroup6>{}, integral_constant<int, kNumTable6>{}, 6, 1024)) return rc;
     hipLaunchKernelGGL(numeric_spill_kernel<T>, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm,
                        B_cols, Ad, A_indices, A_indptr, Bd, B_indices, B_indptr, C_indptr, C_indices, Cd, w.mark,
                        w.acc);
@@ -1269,7 +1270,9 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
                        w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup4, kSymTable4>), dim3(kPersistGrid), dim3(kBlock), 0, s, 4, w.bins,
                        w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
-    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup5, kSymTable5>), dim3(1024), dim3(kBlock), 0, s, 5, w.bins, w.perm,
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup5, kSymTable5>), dim3(kPersistGrid), dim3(kBlock), 0, s, 5, w.bins,
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+    hipLaunchKernelGGL((symbolic_hash_kernel<kGroup6, kSymTable6>), dim3(1024), dim3(kBlock), 0, s, 6, w.bins, w.perm,
                        A_indices, A_indptr, B_indices, B_indptr, C_indptr);
     NM_LAUNCH_CHECK("symbolic_hash_kernel");
     hipLaunchKernelGGL(symbolic_spill_kernel, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm, B_cols,
@@ -1391,17 +1394,22 @@ extern "C" int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, in
                            (const double *)gC, C_indices, C_indptr, (const double *)A_data, A_indices, A_indptr,
                            (const double *)B_data, B_indices, B_indptr, (double *)grad_A, (double *)grad_B);
     NM_LAUNCH_CHECK("spgemm_bwd_kernel");
-    grid = nm::ceil_div(A_rows, kBwdLongChunk);
-    if (grid > 1024) grid = 1024;
+    // A workgroup works off the long rows of its chunk one after the other, so a chunk is sized
+    // for at least ~4096 of them over the matrix (8 rows or more; 256 at the sizes where the pass
+    // over the row lengths is itself worth keeping short).
+    int chunk = kBwdLongChunk;
+    while (chunk > 8 && A_rows / chunk < 4096) chunk /= 2;
+    grid = nm::ceil_div(A_rows, chunk);
+    if (grid > 4096) grid = 4096;
     const int64_t none = INT64_MAX;
 #define NM_BWD_LONG(T)                                                                                          \
     do {                                                                                                        \
         hipLaunchKernelGGL((spgemm_bwd_long_kernel<T, kBwdLongCap, true>), dim3((unsigned)grid), dim3(kBlock),  \
-                           0, s, A_rows, (int64_t)kBwdLong, (int64_t)kBwdLongCap, (const T *)gC, C_indices,     \
+                           0, s, A_rows, chunk, (int64_t)kBwdLong, (int64_t)kBwdLongCap, (const T *)gC, C_indices,\
                            C_indptr, (const T *)A_data, A_indices, A_indptr, (const T *)B_data, B_indices,      \
                            B_indptr, (T *)grad_A, (T *)grad_B);                                                 \
         hipLaunchKernelGGL((spgemm_bwd_long_kernel<T, kBwdHugeCap, false>), dim3((unsigned)grid), dim3(kBlock), \
-                           0, s, A_rows, (int64_t)kBwdLongCap, none, (const T *)gC, C_indices, C_indptr,        \
+                           0, s, A_rows, chunk, (int64_t)kBwdLongCap, none, (const T *)gC, C_indices, C_indptr, \
                            (const T *)A_data, A_indices, A_indptr, (const T *)B_data, B_indices, B_indptr,      \
                            (T *)grad_A, (T *)grad_B);                                                           \
     } while (0)
