@@ -54,6 +54,15 @@ __device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ indptr
     }
 }
 
+// Rows (or columns) a workgroup takes at a time: the compiled maximum `most` where rows are
+// short, fewer where they are long, so that a block holds about `cap` entries -- a matrix with
+// few, long rows would otherwise be cut into fewer blocks than the chip has CUs.
+inline int block_rows(int64_t rows, int64_t nnz, int most, int cap) {
+    const int64_t mean = rows > 0 ? (nnz + rows - 1) / rows : 1;
+    const int64_t r = cap / (mean > 0 ? mean : 1);
+    return (int)(r > most ? most : (r < 8 ? 8 : r));
+}
+
 // End of the run of rows that starts at row s0 of the block and fits the LDS tile: the
 // largest e in [s0, nr] with at most cap entries in rows [s0, e); e == s0 when row s0
 // alone is longer.
@@ -73,19 +82,21 @@ __device__ __forceinline__ int run_end(const int32_t *s_off, int s0, int nr, int
 // the same storage-order sum.
 template <typename T, int BLOCK, int R, int CAP, bool UNIT = false>
 __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
-    int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
+    int64_t rows, int rt, const T *__restrict__ data, const int64_t *__restrict__ indices,
     const int64_t *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y) {
+    // rt <= R: rows per block of this launch (block_rows)
     __shared__ int32_t s_off[R + 1];
     __shared__ T s_prod[CAP];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
 
-    const int64_t ntiles = (rows + R - 1) / R, npad = nm::xcd_padded(ntiles);
+    const int64_t ntiles = (rows + rt - 1) / rt, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t tile = nm::xcd_tile(id, npad);
         if (tile >= ntiles) continue;
-        const int64_t r0 = tile * R;
-        const int nr = (int)(rows - r0 < R ? rows - r0 : R);
+        const int64_t r0 = tile * rt;
+        int nr = (int)(rows - r0 < rt ? rows - r0 : rt);
+        nr = nr < R ? nr : R;   // rt <= R
         const int64_t base = indptr[r0];
         stage_offsets<R, CAP, BLOCK>(indptr, r0, nr, base, s_off);
         __syncthreads();
@@ -224,7 +235,7 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
 // masked outer product (cpp/sparse_csr_cpu.cpp:60-65 and :750-755).
 template <typename T, int R, int CAP>
 __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
-    int64_t rows, const T *__restrict__ data, const int64_t *__restrict__ indices,
+    int64_t rows, int rt, const T *__restrict__ data, const int64_t *__restrict__ indices,
     const int64_t *__restrict__ indptr, const T *__restrict__ a, const T *__restrict__ b, T alpha,
     T *__restrict__ out_A, T *__restrict__ grad_x) {
     __shared__ int32_t s_off[R + 1];
@@ -232,12 +243,13 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
 
-    const int64_t ntiles = (rows + R - 1) / R, npad = nm::xcd_padded(ntiles);
+    const int64_t ntiles = (rows + rt - 1) / rt, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t tile = nm::xcd_tile(id, npad);
         if (tile >= ntiles) continue;
-        const int64_t r0 = tile * R;
-        const int nr = (int)(rows - r0 < R ? rows - r0 : R);
+        const int64_t r0 = tile * rt;
+        int nr = (int)(rows - r0 < rt ? rows - r0 : rt);
+        nr = nr < R ? nr : R;   // rt <= R
         const int64_t base = indptr[r0];
         stage_offsets<R, CAP, kBlock>(indptr, r0, nr, base, s_off);
         __syncthreads();
@@ -576,35 +588,38 @@ int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const i
 }
 
 template <typename T>
-int launch_fwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *x,
+int launch_fwd(int64_t rows, int64_t nnz, const T *data, const int64_t *indices, const int64_t *indptr, const T *x,
                T *y, hipStream_t s) {
     constexpr int R = kFwdR, CAP = kFwdCap;
-    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, R));
+    const int rt = block_rows(rows, nnz, R, CAP);
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows, data,
-                       indices, indptr, x, y);
+    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows, rt,
+                       data, indices, indptr, x, y);
     NM_LAUNCH_CHECK("spmv_fwd_kernel");
     return NM_OK;
 }
 
 template <typename T>
-int launch_row_sum(int64_t rows, const T *data, const int64_t *indptr, T *y, hipStream_t s) {
+int launch_row_sum(int64_t rows, int64_t nnz, const T *data, const int64_t *indptr, T *y, hipStream_t s) {
     constexpr int R = kFwdR, CAP = kFwdCap;
-    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, R));
+    const int rt = block_rows(rows, nnz, R, CAP);
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, true>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows,
-                       data, (const int64_t *)nullptr, indptr, (const T *)nullptr, y);
+                       rt, data, (const int64_t *)nullptr, indptr, (const T *)nullptr, y);
     NM_LAUNCH_CHECK("spmv_fwd_kernel<unit>");
     return NM_OK;
 }
 
 template <typename T>
-int launch_bwd(int64_t rows, const T *data, const int64_t *indices, const int64_t *indptr, const T *a,
+int launch_bwd(int64_t rows, int64_t nnz, const T *data, const int64_t *indices, const int64_t *indptr, const T *a,
                const T *b, T alpha, T *out_A, T *grad_x, hipStream_t s) {
     constexpr int R = Tile<T>::R, CAP = Tile<T>::CAP;
-    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, R));
+    const int rt = block_rows(rows, nnz, R, CAP);
+    int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-    hipLaunchKernelGGL((spmv_bwd_kernel<T, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, data,
+    hipLaunchKernelGGL((spmv_bwd_kernel<T, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, rows, rt, data,
                        indices, indptr, a, b, alpha, out_A, grad_x);
     NM_LAUNCH_CHECK("spmv_bwd_kernel");
     return NM_OK;
@@ -622,9 +637,9 @@ extern "C" int nm_spgemv_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_
     hipStream_t s = nm::as_stream(stream);
     switch (dt) {
         case NM_F32:
-            return launch_fwd<float>(rows, (const float *)data, indices, indptr, (const float *)x, (float *)y, s);
+            return launch_fwd<float>(rows, nnz, (const float *)data, indices, indptr, (const float *)x, (float *)y, s);
         case NM_F64:
-            return launch_fwd<double>(rows, (const double *)data, indices, indptr, (const double *)x,
+            return launch_fwd<double>(rows, nnz, (const double *)data, indices, indptr, (const double *)x,
                                       (double *)y, s);
     }
     return nm::fail(NM_ERR_INVALID, "unknown dtype %d", (int)dt);
@@ -637,8 +652,8 @@ extern "C" int nm_csr_row_sum_forward(nm_dtype dt, int64_t rows, int64_t nnz, co
     if (rows == 0) return NM_OK;
     NM_REQUIRE(indptr && x && (nnz == 0 || data), "null pointer argument");
     hipStream_t s = nm::as_stream(stream);
-    if (dt == NM_F32) return launch_row_sum<float>(rows, (const float *)data, indptr, (float *)x, s);
-    return launch_row_sum<double>(rows, (const double *)data, indptr, (double *)x, s);
+    if (dt == NM_F32) return launch_row_sum<float>(rows, nnz, (const float *)data, indptr, (float *)x, s);
+    return launch_row_sum<double>(rows, nnz, (const double *)data, indptr, (double *)x, s);
 }
 
 extern "C" int nm_spgemv_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
@@ -655,9 +670,9 @@ extern "C" int nm_spgemv_backward(nm_dtype dt, int64_t rows, int64_t cols, int64
     if (rows == 0 || nnz == 0 || (!grad_A && !grad_x)) return NM_OK;
     NM_REQUIRE(g != nullptr && x != nullptr, "g or x is null");
     if (dt == NM_F32)
-        return launch_bwd<float>(rows, (const float *)data, indices, indptr, (const float *)g,
+        return launch_bwd<float>(rows, nnz, (const float *)data, indices, indptr, (const float *)g,
                                  (const float *)x, 1.0f, (float *)grad_A, (float *)grad_x, s);
-    return launch_bwd<double>(rows, (const double *)data, indices, indptr, (const double *)g,
+    return launch_bwd<double>(rows, nnz, (const double *)data, indices, indptr, (const double *)g,
                               (const double *)x, 1.0, (double *)grad_A, (double *)grad_x, s);
 }
 
@@ -670,9 +685,9 @@ extern "C" int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz, const int
     NM_REQUIRE(indices && a && b && out, "null pointer argument");
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
-        return launch_bwd<float>(rows, nullptr, indices, indptr, (const float *)a, (const float *)b,
+        return launch_bwd<float>(rows, nnz, nullptr, indices, indptr, (const float *)a, (const float *)b,
                                  (float)alpha, (float *)out, nullptr, s);
-    return launch_bwd<double>(rows, nullptr, indices, indptr, (const double *)a, (const double *)b, alpha,
+    return launch_bwd<double>(rows, nnz, nullptr, indices, indptr, (const double *)a, (const double *)b, alpha,
                               (double *)out, nullptr, s);
 }
 
