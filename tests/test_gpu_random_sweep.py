@@ -183,7 +183,8 @@ def _big_draw(seed, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("NM_SWEEP_BIG_FIRST", "0")),
+                                         int(os.environ.get("NM_SWEEP_BIG_FIRST", "0")) + int(os.environ.get("NM_SWEEP_BIG", "6"))))
 def test_many_workgroups(dev, seed, dtype):
     import torch
     ext = numml_amd.load_compiled()
@@ -202,7 +203,7 @@ def test_many_workgroups(dev, seed, dtype):
             ext.set_backward_mode("planned")
         assert_same(host(gA), gA_ref, f"spmv grad_A ({mode})")
         assert_close(host(gx), gx_ref, f"spmv grad_x ({mode})")
-    n = (4, 16, 33, 64, 7, 100)[seed]
+    n = (4, 16, 33, 64, 7, 100)[seed % 6]
     B, gC = randn(seed + 2, (cols, n), dtype), randn(seed + 3, (rows, n), dtype)
     Bd, gCd = to_dev(dev, B, gC)
     assert_close(host(ext.spdmm_forward(rows, cols, D, I, P, Bd)), oracle.spdmm_forward(rows, cols, d, i, p, B), f"C n={n}")
