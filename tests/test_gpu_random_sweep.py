@@ -244,3 +244,42 @@ def test_many_workgroups(dev, seed, dtype):
     gA_ref, gB_ref = oracle.spgemm_backward(gCs, C_ref[1], C_ref[2], rows, cols, d, i, p, cols, m, d2, i2, p2)
     assert_close(host(gA), gA_ref, "spgemm grad_A")
     assert_close(host(gB), gB_ref, "spgemm grad_B")
+
+
+def _big_triangle(seed, dtype, n, deps, window, lower):
+    """Triangular CSR: row i holds `deps` entries (fewer near the corner) among the `window` rows
+    before it (after it for an upper triangle), N(0, 0.1) values, and a diagonal in [2, 3)."""
+    rng = np.random.default_rng(7000 + seed)
+    lens = np.minimum(np.arange(n), deps).astype(np.int64)
+    row_of = np.repeat(np.arange(n, dtype=np.int64), lens)
+    reach = np.minimum(row_of, window)
+    off = 1 + (rng.random(row_of.shape[0]) * reach).astype(np.int64)
+    key = np.unique(row_of * (window + 1) + np.minimum(off, reach))          # duplicates dropped
+    r, c = key // (window + 1), key // (window + 1) - key % (window + 1)
+    r, c = np.concatenate([r, np.arange(n)]), np.concatenate([c, np.arange(n)])
+    v = np.concatenate([rng.standard_normal(key.shape[0]) * 0.1, 2.0 + rng.random(n)])
+    M = sps.csr_matrix((v, (r, c)), shape=(n, n))
+    if not lower:
+        M = M.T.tocsr()
+    M.sort_indices()
+    return M.data.astype(dtype), M.indices.astype(np.int64), M.indptr.astype(np.int64)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("lower", [True, False])
+@pytest.mark.parametrize("deps,window", [(3, 400), (6, 3000), (14, 1500)])
+def test_triangular_solves_over_thousands_of_levels(dev, dtype, lower, deps, window):
+    ext = numml_amd.load_compiled()
+    n = 150_000
+    d, i, p = _big_triangle(deps, dtype, n, deps, window, lower)
+    print(f"case {dtype.__name__} n={n} nnz={d.shape[0]} lower={lower} deps={deps} window={window}", flush=True)
+    b, g = randn(deps, n, dtype), randn(deps + 1, n, dtype)
+    D, I, P, Bv, Gv = to_dev(dev, d, i, p, b, g)
+    for unit in (False, True):
+        x_ref = oracle.sptrsv_forward(n, n, d, i, p, lower, unit, b)
+        x = ext.sptrsv_forward(n, n, D, I, P, lower, unit, Bv)
+        assert_close(host(x), x_ref, f"x unit={unit}")
+        gA, gb = ext.sptrsv_backward(Gv, x, n, n, D, I, P, lower, unit, Bv)
+        gA_ref, gb_ref = oracle.sptrsv_backward(g, host(x), n, n, d, i, p, lower, unit)
+        assert_close(host(gb), gb_ref, f"grad_b unit={unit}")
+        assert_close(host(gA), gA_ref, f"grad_A unit={unit}")
