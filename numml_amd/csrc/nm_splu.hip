@@ -22,11 +22,13 @@
 // entries below the diagonal are divided by it.  Per entry the operations come in the
 // serial order, so the factors equal the reference's bit for bit.
 // Column k needs the finished columns i of its entries above the diagonal, and nothing
-// else: wavefronts take columns in ascending order from a ticket counter, keep the column
-// in LDS, and before using column i wait for its flag.  A wavefront only ever waits for a
-// column with a smaller ticket, which a running wavefront holds, so the grid always makes
-// progress whatever part of it is resident; a bounded number of polls backs that up, after
-// which every wavefront leaves and the call reports an error.  Early pivots of a column
+// else: workgroups take batches of consecutive columns in ascending order from a ticket
+// counter, one column per wavefront, keep the columns in LDS, and before using column i wait
+// for its flag -- a flag and values in LDS when column i belongs to the same batch, in global
+// memory otherwise.  A wavefront only ever waits for a column with a smaller number, which a
+// running wavefront holds, so the grid always makes progress whatever part of it is resident;
+// a bounded number of polls backs that up, after which every wavefront leaves and the call
+// reports an error.  Early pivots of a column
 // overlap with the tail of the columns before it, which is where a banded factor, whose
 // columns form one long dependency chain, gets its parallelism from.
 #include "nm_common.hpp"
@@ -201,8 +203,12 @@ __global__ __launch_bounds__(kBlock) void lu_values_kernel(int64_t rows, const T
     }
 }
 
+#ifndef NM_LU_WAVES
+#define NM_LU_WAVES 8
+#endif
 constexpr int kLuCap = 1024;              // entries of a column kept in LDS, per wavefront
-constexpr int kLuWavesPerBlock = kBlock / 64;
+constexpr int kLuWavesPerBlock = NM_LU_WAVES;   // columns of a batch = wavefronts of a workgroup of the numeric phase
+constexpr int kLuFlowBlock = kLuWavesPerBlock * 64;
 constexpr int64_t kLuSpinLimit = 1 << 24;  // polls of one dependency flag before giving up
 
 struct LuFlow {
@@ -259,8 +265,21 @@ __global__ void lu_below_kernel(int64_t cols, const int64_t *__restrict__ indice
 // Everything about a pivot that the structure alone decides -- which entries of column i lie below
 // its diagonal and where their rows sit in this column -- is looked up before the wait for column i,
 // so that what follows the arrival of the flag is one load, one multiply and one subtraction.
+// The columns of one batch [base, base + kLuWavesPerBlock) are worked on by the wavefronts of one
+// workgroup: a column of the batch that sits in LDS is read there, behind an LDS flag, by the
+// later columns of the batch, which spares them the round trip through global memory that the
+// flag and the values of a column of another workgroup cost.
+template <typename T>
+struct LuBatch {
+    int64_t base;                 // first column of the batch
+    const int64_t *pb;            // [kLuWavesPerBlock] LDS: start of each column in the CSR arrays
+    T (*vals)[kLuCap];            // LDS values of the batch's columns
+    volatile int32_t *ready;      // [kLuWavesPerBlock] LDS: 0 pending, 1 final values in LDS, 2 final values in global memory only
+};
+
 template <typename T, bool IN_LDS>
 __device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T, IN_LDS> &own,
+                          const LuBatch<T> &batch,
                           const int64_t *__restrict__ indices, const int64_t *__restrict__ indptr,
                           const int64_t *__restrict__ below_of, T *values, int32_t *done, int32_t *ctl,
                           int64_t spin_limit, int lane) {
@@ -280,32 +299,69 @@ __device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T,
         }
         return (lo < len && own.row(lo) == j) ? lo : (int64_t)-1;
     };
-    int64_t e = 0;
-    for (; e < len; ++e) {
+    // What the structure alone says about pivot e: the column i it names, where the entries of
+    // column i below its diagonal start and end, this lane's entry of them and the place of
+    // that entry's row in this column.  Looked up one pivot ahead: the two dependent loads it
+    // takes would otherwise stand between the arrival of a flag and the update it allows.
+    struct Look {
+        int64_t i, ls, ie, t_first, at_first;
+    };
+    auto look = [&](int64_t e) {
+        Look L{-1, 0, 0, 0, -1};
+        if (e >= len) return L;
         const int64_t i = own.row(e);
-        if (i >= k) break;
-        const int64_t ls = below_of[i], ie = indptr[i + 1];
-        const int64_t t_first = ls + lane;                       // this lane's entry of column i, first round
-        const int64_t at_first = t_first < ie ? find(e, indices[t_first]) : (int64_t)-1;
+        if (i >= k) return L;
+        L.i = i;
+        L.ls = below_of[i];
+        L.ie = indptr[i + 1];
+        L.t_first = L.ls + lane;
+        L.at_first = L.t_first < L.ie ? find(e, indices[L.t_first]) : (int64_t)-1;
+        return L;
+    };
+    int64_t e = 0;
+    Look next = look(0);
+    for (; next.i >= 0; ++e) {
+        const Look cur = next;
+        next = look(e + 1);
+        const int64_t i = cur.i, ls = cur.ls, ie = cur.ie, t_first = cur.t_first, at_first = cur.at_first;
         int64_t polls = 0;
-        while (__hip_atomic_load(done + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
-            if (++polls > spin_limit || __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
-                return false;
-            __builtin_amdgcn_s_sleep(1);
+        bool in_lds = false;   // column i is one of this batch's and its final values are in LDS
+        if (i >= batch.base) {
+            const int wi = (int)(i - batch.base);
+            int32_t state;
+            while ((state = batch.ready[wi]) == 0) {
+                if (++polls > spin_limit ||
+                    ((polls & 1023) == 0 && __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))
+                    return false;
+                __builtin_amdgcn_s_sleep(1);
+            }
+            in_lds = state == 1;
+        } else {
+            while (__hip_atomic_load(done + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+                if (++polls > spin_limit || __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+                    return false;
+                __builtin_amdgcn_s_sleep(1);
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // the value loads below stay after the flag
         const T m_ik = own.val(e);
+        // entry t of the CSR arrays, which belongs to column i
+        auto other = [&](int64_t t) -> T {
+            if (in_lds) {
+                const int wi = (int)(i - batch.base);
+                return batch.vals[wi][t - batch.pb[wi]];
+            }
+            return __hip_atomic_load(values + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        };
         if (at_first >= 0) {
-            const T m_ji = __hip_atomic_load(values + t_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const T prod = m_ji * m_ik;
+            const T prod = other(t_first) * m_ik;
             own.set(at_first, own.val(at_first) - prod);
         }
         for (int64_t t0 = ls + 64; t0 < ie; t0 += 64) {          // columns with more than 64 entries below
             const int64_t t = t0 + lane;
             const int64_t at = t < ie ? find(e, indices[t]) : (int64_t)-1;
             if (at >= 0) {
-                const T m_ji = __hip_atomic_load(values + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const T prod = m_ji * m_ik;
+                const T prod = other(t) * m_ik;
                 own.set(at, own.val(at) - prod);
             }
         }
@@ -316,40 +372,62 @@ __device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T,
         for (int64_t q = e + 1 + lane; q < len; q += 64) own.set(q, own.val(q) / d);
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
-    if (IN_LDS)
+    // the later columns of the batch first: they read this one in LDS
+    if (IN_LDS) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0) batch.ready[k - batch.base] = 1;
         for (int64_t q = lane; q < len; q += 64) values[pb + q] = own.s_vals[q];
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    if (lane == 0) __hip_atomic_store(done + k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) {
+        __hip_atomic_store(done + k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!IN_LDS) batch.ready[k - batch.base] = 2;
+    }
     return true;
 }
 
 template <typename T>
-__global__ __launch_bounds__(kBlock) void lu_flow_kernel(int64_t cols, const int64_t *__restrict__ indices,
+__global__ __launch_bounds__(kLuFlowBlock) void lu_flow_kernel(int64_t cols, const int64_t *__restrict__ indices,
                                                          const int64_t *__restrict__ indptr,
                                                          const int64_t *__restrict__ below, T *values,
                                                          int32_t *done, int32_t *ctl, int64_t spin_limit) {
-    __shared__ int32_t s_rows[kLuWavesPerBlock][kLuCap];
-    __shared__ T s_vals[kLuWavesPerBlock][kLuCap];
+    // dynamic LDS: the batch's columns, values first (8-byte aligned), then rows
+    extern __shared__ __align__(16) unsigned char s_columns[];
+    T (*s_vals)[kLuCap] = reinterpret_cast<T (*)[kLuCap]>(s_columns);
+    int32_t (*s_rows)[kLuCap] =
+        reinterpret_cast<int32_t (*)[kLuCap]>(s_columns + sizeof(T) * kLuWavesPerBlock * kLuCap);
+    __shared__ int64_t s_pb[kLuWavesPerBlock];
+    __shared__ int32_t s_ready[kLuWavesPerBlock];
+    __shared__ int32_t s_ticket, s_abort;
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     for (;;) {
-        int32_t ticket = 0;
-        if (lane == 0) ticket = atomicAdd(ctl, 1);
-        const int64_t k = __builtin_amdgcn_readfirstlane(ticket);
-        if (k >= cols) break;
-        if (__hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-        const int64_t pb = indptr[k], len = indptr[k + 1] - pb;
-        bool ok;
-        if (len <= kLuCap) {
-            const OwnColumn<T, true> own{s_rows[w], s_vals[w], nullptr, nullptr};
-            ok = lu_column<T, true>(k, pb, len, own, indices, indptr, below, values, done, ctl, spin_limit, lane);
-        } else {
-            const OwnColumn<T, false> own{nullptr, nullptr, indices + pb, values + pb};
-            ok = lu_column<T, false>(k, pb, len, own, indices, indptr, below, values, done, ctl, spin_limit, lane);
+        // one ticket per workgroup and batch of consecutive columns, one column per wavefront
+        if (threadIdx.x == 0) {
+            s_ticket = atomicAdd(ctl, kLuWavesPerBlock);
+            s_abort = __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (!ok) {
-            if (lane == 0) atomicExch(ctl + 1, 1);
-            break;
+        if (threadIdx.x < kLuWavesPerBlock) s_ready[threadIdx.x] = 0;
+        __syncthreads();
+        const int64_t base = s_ticket;
+        if (base >= cols || s_abort != 0) break;   // the same decision in every wavefront
+        const int64_t k = base + w;
+        if (k < cols) {
+            const int64_t pb = indptr[k], len = indptr[k + 1] - pb;
+            if (lane == 0) s_pb[w] = pb;
+            const LuBatch<T> batch{base, s_pb, s_vals, s_ready};
+            bool ok;
+            if (len <= kLuCap) {
+                const OwnColumn<T, true> own{s_rows[w], s_vals[w], nullptr, nullptr};
+                ok = lu_column<T, true>(k, pb, len, own, batch, indices, indptr, below, values, done, ctl, spin_limit,
+                                        lane);
+            } else {
+                const OwnColumn<T, false> own{nullptr, nullptr, indices + pb, values + pb};
+                ok = lu_column<T, false>(k, pb, len, own, batch, indices, indptr, below, values, done, ctl, spin_limit,
+                                         lane);
+            }
+            if (!ok && lane == 0) atomicExch(ctl + 1, 1);
         }
+        __syncthreads();   // the batch's columns in LDS have no readers left
     }
 }
 
@@ -469,11 +547,17 @@ extern "C" int nm_splu_numeric(nm_dtype dt, int64_t cols, void *Mt_data, const i
     int64_t grid = nm::ceil_div(cols, kLuWavesPerBlock);
     if (grid > 1024) grid = 1024;
     const int64_t limit = poll_limit > 0 ? poll_limit : kLuSpinLimit;
+    const size_t lds = (size_t)kLuWavesPerBlock * kLuCap * ((dt == NM_F32 ? 4 : 8) + 4);
+    if (lds > 64 * 1024) {
+        const void *fn = dt == NM_F32 ? reinterpret_cast<const void *>(lu_flow_kernel<float>)
+                                      : reinterpret_cast<const void *>(lu_flow_kernel<double>);
+        NM_HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    }
     if (dt == NM_F32)
-        hipLaunchKernelGGL(lu_flow_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, Mt_indices,
+        hipLaunchKernelGGL(lu_flow_kernel<float>, dim3((unsigned)grid), dim3(kLuFlowBlock), lds, s, cols, Mt_indices,
                            Mt_indptr, F.below, (float *)Mt_data, F.done, F.ctl, limit);
     else
-        hipLaunchKernelGGL(lu_flow_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, Mt_indices,
+        hipLaunchKernelGGL(lu_flow_kernel<double>, dim3((unsigned)grid), dim3(kLuFlowBlock), lds, s, cols, Mt_indices,
                            Mt_indptr, F.below, (double *)Mt_data, F.done, F.ctl, limit);
     NM_LAUNCH_CHECK("lu_flow_kernel");
     int32_t ctl_h[2] = {0, 0};
