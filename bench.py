@@ -1,12 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the differentiable CSR hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras]
 
 A step is one pass of the hot path over one synthetic input (forward, then
 backward with both gradients) through the ``numml_torch_cpp`` functions, i.e. the
 same calls autograd makes.  Inputs are resident in HBM before the timed region.
 Prints ONE JSON line.
+
+The headline fields of that line belong to ``--workload`` (default ``spmv``, the
+configuration the metric is quoted on).  With the default workload the line also
+carries a ``workloads`` object: the other configurations the metric names
+(``spmm``, ``spgemm``, ``sptrsv`` and the CPU-sized ``spmv64``), each measured the
+same way in the same process with its own ``value`` / ``ms_per_step`` /
+``roofline`` / ``cpu_baseline`` (fewer steps and a shorter CPU leg; ``--no-extras``
+leaves them out).
 
 Workloads (``--workload``; the default is the one the headline metric is quoted
 on):
@@ -20,6 +28,9 @@ on):
   lincomb    fp32 A - B (splincomb) + its backward, both on the spmv matrix pattern
   transpose  fp32 explicit CSR transpose + its backward on the spmv matrix
   copy    256 MiB device copy (counter calibration / practical bandwidth ceiling)
+  ref_timing  the shapes the reference's own timing script uses (demos/timing.py:177-217,
+          264-348, 520-558): tridiagonal SpMV N = 32 768, tridiagonal SpSpMM and SpDMM
+          N = 16 384, bidiagonal SpTRSV N = 32 768, through the Python surface, us per call
 
 ``value`` is algorithmic bytes per step / time per step (GB/s) for spmv/spmm,
 GFLOP/s (2 flop per scalar product, forward only counted) for spgemm and
@@ -39,13 +50,29 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
 
+def _source_sha(files):
+    """sha256 (first 16 hex digits) over the named kernel sources, in the given order."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(ROOT, "numml_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def _traffic(workload):
     """Measured HBM bytes per launch of the dominant kernel, from the committed
-    rocprofv3 counter summaries (profiles/traffic.json), or None."""
+    rocprofv3 counter summaries (profiles/traffic.json; a separate counter run, not
+    this one), or None.  An entry records the hash of the kernel sources it was
+    measured on; when those have changed since, the figure is stale and None is
+    reported instead."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(workload, {}).get("traffic_bytes")
+            entry = json.load(f).get(workload, {})
+        if "sources" in entry and _source_sha(entry["sources"]) != entry.get("sources_sha16"):
+            return None
+        return entry.get("traffic_bytes")
     except (OSError, ValueError):
         return None
 
@@ -112,18 +139,48 @@ class SpMV(Workload):
         self.dominant_bytes = self.bwd_bytes
         self.dominant_name = ("spmv_bwd_planned_kernel" if _binding.backward_mode() == "planned"
                               else "spmv_bwd_kernel (+ fill_kernel clearing grad_x)")
-        # structure analysis is timed apart from the steps: the first backward builds (and caches) the
-        # transposed-structure plan of this sparsity pattern
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        ext.spgemv_backward(self.Gv, rows, cols, self.D, self.I, self.P, self.X)
-        torch.cuda.synchronize()
-        first_bwd_ms = (time.perf_counter() - t0) * 1e3
+        # Structure analysis is timed apart from the steps.  The first backward calls on a new
+        # sparsity pattern are timed one by one: the transposed-structure plan of the default
+        # backward is built (and cached) during one of them.
+        firsts = []
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ext.spgemv_backward(self.Gv, rows, cols, self.D, self.I, self.P, self.X)
+            torch.cuda.synchronize()
+            firsts.append(round((time.perf_counter() - t0) * 1e3, 3))
+        self.first_backward_ms = firsts
         self.config = {"workload": f"spmv_fwd_bwd_{self.dtype}_{self.label}", "rows": rows,
-                       "first_backward_ms_incl_plan_build": round(first_bwd_ms, 3),
+                       "first_three_backward_calls_ms": firsts,
                        "nnz": self.nnz, "index_bytes": 8, "backward": _binding.backward_mode(),
                        "binding": _binding.name,
                        "algorithmic_bytes_per_step": self.bytes_per_step}
+
+    def after(self, rec, steps):
+        """The same step without a plan (stateless backward with atomics), the cost of building
+        the plan, and the number of steps after which building it has paid off."""
+        import torch
+        from numml_amd import _binding
+        if _binding.backward_mode() != "planned":
+            return
+        _binding.set_backward_mode("atomic")
+        try:
+            for _ in range(3):
+                self.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                self.step()
+            torch.cuda.synchronize()
+            stateless = (time.perf_counter() - t0) / steps * 1e3
+        finally:
+            _binding.set_backward_mode("planned")
+        build = max(self.first_backward_ms) - rec["roofline"]["avg_ms"]
+        gain = stateless - rec["ms_per_step"]
+        rec["config"]["stateless_ms_per_step"] = round(stateless, 5)
+        rec["config"]["plan_build_ms"] = round(build, 3)
+        rec["config"]["plan_break_even_steps"] = int(np.ceil(build / gain)) if gain > 0 else None
+        rec["config"]["amortised_ms_per_step_over_100_steps"] = round(rec["ms_per_step"] + build / 100, 5)
 
     def step(self):
         y = self.ext.spgemv_forward(self.rows, self.cols, self.D, self.I, self.P, self.X)
@@ -199,7 +256,7 @@ class SpMM(Workload):
         import oracle
         d, i, p, rows, cols = self.host
         # the reference's row->column->entry loop is slow: time the first `sub` rows only
-        sub = 50_000
+        sub = max(1000, int(5000 * budget_s))
         ps = p[:sub + 1]
         nnz_s = int(ps[-1])
         ds, is_ = d[:nnz_s], i[:nnz_s]
@@ -251,13 +308,21 @@ class SpGEMM(Workload):
         self.products = int(lens[self.hostL[1]].sum())
         self.flops = 2 * self.products
         s = 8
-        self.bytes_per_step = (self.nnz * (s + 8) + rows * 8 + self.products * (s + 8)
-                               + self.nnzC * (s + 8) + rows * 8)
+        nnzR = int(d.shape[0])
+        # Compulsory traffic of the forward: both operands and the result once, the two row
+        # pointer arrays.  The gather-inclusive figure (every referenced row of the right operand
+        # read again for every product) is an upper bound and is reported apart; most of those
+        # reads are served by the caches.
+        self.bytes_per_step = self.nnz * (s + 8) + nnzR * (s + 8) + self.nnzC * (s + 8) + 2 * rows * 8
         self.dominant_bytes = self.bytes_per_step
-        self.dominant_name = "spgemm forward (symbolic + numeric launches)"
+        self.dominant_name = "spgemm forward (symbolic + numeric launches, host read of nnz(C) included)"
         self.config = {"workload": f"spgemm_{self.left}xA_fwd_bwd_f64_laplace3d_{n}", "rows": rows,
-                       "nnz_left": self.nnz, "nnz_right": int(d.shape[0]),
-                       "nnz_C": self.nnzC, "products": self.products, "index_bytes": 8}
+                       "nnz_left": self.nnz, "nnz_right": nnzR,
+                       "nnz_C": self.nnzC, "products": self.products, "index_bytes": 8,
+                       "forward_compulsory_bytes": self.bytes_per_step,
+                       "forward_gather_inclusive_bytes": (self.nnz * (s + 8) + rows * 8
+                                                          + self.products * (s + 8)
+                                                          + self.nnzC * (s + 8) + rows * 8)}
 
     def step(self):
         C = self.ext.spgemm_forward(self.rows, self.cols, *self.L, self.rows, self.cols, *self.R)
@@ -560,45 +625,138 @@ WORKLOADS = {
 }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="spmv", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-seconds", type=float, default=10.0,
-                    help="CPU time budget of the cpu_baseline leg (0 skips it)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
-                 f"--gpus {args.gpus} is not supported, use --gpus 1")
-
+def ref_timing(dev, cpu_seconds):
+    """The reference's own timing protocol (demos/timing.py): the same matrices, sizes and
+    iteration counts, through the Python surface (`A @ x`, `.sum().backward()`), `it` calls
+    between two synchronisations (time_op, demos/timing.py:21-28); us per call, the C oracle
+    on one core beside it.  fp32 (torch's default dtype, as in the reference's script)."""
     import torch
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no HIP device visible")
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
+    import oracle
+    from numml_amd import generators as G
+    from numml_amd import sparse as sp
 
-    w = WORKLOADS[args.workload]()
+    def time_op(f, it):
+        f()                                   # the reference warms its GPU paths up as well (:184, :272)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(it):
+            f()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / it * 1e6
+
+    def cpu_op(f, it):
+        t0 = time.perf_counter()
+        n = 0
+        while n < it and (n == 0 or time.perf_counter() - t0 < cpu_seconds / 8):
+            f()
+            n += 1
+        return (time.perf_counter() - t0) / n * 1e6
+
+    def csr(gen):
+        d, i, p, shape = gen
+        A = sp.SparseCSRTensor((torch.from_numpy(d), torch.from_numpy(i), torch.from_numpy(p)), shape).to(dev)
+        return A, (d, i, p)
+
+    f32 = np.float32
+    rows = []
+
+    def add(name, n, it, gpu_us, cpu_us):
+        rows.append({"name": name, "n": n, "iterations": it, "gpu_us_per_call": round(gpu_us, 2),
+                     "cpu_oracle_us_per_call": round(cpu_us, 2)})
+
+    # SpMV, tridiagonal, N = 32 768, 1000 iterations (demos/timing.py:177-217)
+    N = 32_768
+    A, (d, i, p) = csr(G.tridiag(N, f32))
+    x_h = np.random.default_rng(0).random(N).astype(f32)
+    x = torch.from_numpy(x_h).to(dev)
+    ones = np.ones(N, f32)
+    add("SpMV Forward", N, 1000, time_op(lambda: A @ x, 1000),
+        cpu_op(lambda: oracle.spgemv_forward(N, N, d, i, p, x_h), 1000))
+    A.requires_grad = True
+    x.requires_grad_(True)
+    add("SpMV Backward", N, 1000, time_op(lambda: (A @ x).sum().backward(), 1000),
+        cpu_op(lambda: (oracle.spgemv_forward(N, N, d, i, p, x_h),
+                        oracle.spgemv_backward(ones, N, N, d, i, p, x_h)), 1000))
+
+    # SpSpMM and SpDMM, tridiagonal A, B = -A, N = 16 384, 2 iterations (:264-348)
+    N = 16_384
+    A, (d, i, p) = csr(G.tridiag(N, f32))
+    B, (db, ib, pb) = csr(G.tridiag(N, f32, lo=1.0, di=-2.0, up=1.0))
+    Bd = B.to_dense()
+    add("SpSpMM Forward", N, 2, time_op(lambda: A @ B, 2),
+        cpu_op(lambda: oracle.spgemm_forward(N, N, d, i, p, N, N, db, ib, pb), 2))
+    A.requires_grad = True
+    B.requires_grad = True
+    Cd, Ci, Cp = oracle.spgemm_forward(N, N, d, i, p, N, N, db, ib, pb)
+    gC = np.ones(Cd.shape[0], f32)
+    add("SpSpMM Backward", N, 2, time_op(lambda: (A @ B).sum().backward(), 2),
+        cpu_op(lambda: (oracle.spgemm_forward(N, N, d, i, p, N, N, db, ib, pb),
+                        oracle.spgemm_backward(gC, Ci, Cp, N, N, d, i, p, N, N, db, ib, pb)), 2))
+    A, _ = csr(G.tridiag(N, f32))
+    Bd_h = Bd.cpu().numpy()
+    # the oracle's dense product walks row -> column -> entry like the reference's CPU loop
+    # (cpp/sparse_csr_cpu.cpp:586-598); 512 of the 16 384 rows are timed and scaled
+    sub = 512
+    ps = p[:sub + 1]
+    nz = int(ps[-1])
+    scale = N / sub
+    add("SpDMM Forward", N, 2, time_op(lambda: A @ Bd, 2),
+        scale * cpu_op(lambda: oracle.spdmm_forward(sub, N, d[:nz], i[:nz], ps, Bd_h), 1))
+    A.requires_grad = True
+    Bd.requires_grad_(True)
+    gCd = np.ones((sub, N), f32)
+    add("SpDMM Backward", N, 2, time_op(lambda: (A @ Bd).sum().backward(), 2),
+        scale * cpu_op(lambda: (oracle.spdmm_forward(sub, N, d[:nz], i[:nz], ps, Bd_h),
+                                oracle.spdmm_backward(sub, N, d[:nz], i[:nz], ps, Bd_h, gCd)), 1))
+    del Bd, Bd_h, gCd
+
+    # SpTRSV, bidiagonal 2 I - E_{-1}, N = 32 768, 20 / 10 iterations (:520-558)
+    N = 32_768
+    L, (d, i, p) = csr(G.bidiag(N, f32))
+    b_h = np.ones(N, f32)
+    b = torch.from_numpy(b_h).to(dev)
+    add("SpTRSV Forward", N, 20, time_op(lambda: L.solve_triangular(upper=False, unit=False, b=b), 20),
+        cpu_op(lambda: oracle.sptrsv_forward(N, N, d, i, p, True, False, b_h), 20))
+    L.requires_grad = True
+    xs = oracle.sptrsv_forward(N, N, d, i, p, True, False, b_h)
+    add("SpTRSV Backward", N, 10,
+        time_op(lambda: L.solve_triangular(upper=False, unit=False, b=b).sum().backward(), 10),
+        cpu_op(lambda: (oracle.sptrsv_forward(N, N, d, i, p, True, False, b_h),
+                        oracle.sptrsv_backward(b_h, xs, N, N, d, i, p, True, False)), 10))
+    return {"metric": "reference timing protocol (demos/timing.py), us per call", "unit": "us", "n_gpus": 1,
+            "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "ref_timing", "protocol": "time_op: `iterations` calls between two device "
+                       "synchronisations, through numml_amd.sparse (autograd included)"},
+            "cpu_baseline": {"kind": "port", "cores": 1, "unit": "us",
+                             "sample": "the same calls on the serial C oracle (arithmetic only, no autograd)"},
+            "rows": rows}
+
+
+# The other configurations the metric names, measured beside the headline in the default run.
+EXTRAS = ("spmm", "spgemm", "sptrsv", "spmv64")
+
+
+def measure(w, dev, steps, warmup, cpu_seconds):
+    """One record: W warm-up steps, K timed steps, the dominant launch bracketed by events K
+    times, then the CPU leg."""
+    import torch
     w.setup(dev)
-
-    for _ in range(max(args.warmup, 0)):
+    for _ in range(max(warmup, 0)):
         w.step()
     torch.cuda.synchronize()
 
-    # K timed steps; the dominant launch of every step is bracketed by events on the
-    # stream it runs on (torch's current stream is the one handed to the C ABI).
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         w.step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
+    ms_per_step = elapsed / steps * 1e3
 
-    # Kernel-level timing for the roofline: same launches, events around each one.
+    # Kernel-level timing for the roofline: the same launches, events around each one on the
+    # stream they run on (torch's current stream is the one handed to the C ABI).
     evs = []
-    for _ in range(args.steps):
+    for _ in range(steps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         w.dominant()
@@ -613,21 +771,66 @@ def main():
                 "traffic": _traffic(w.name)}
 
     cpu = None
-    if args.cpu_seconds > 0:
-        cpu = w.cpu_baseline(args.cpu_seconds)
+    if cpu_seconds > 0:
+        cpu = w.cpu_baseline(cpu_seconds)
         cpu["value"] = round(cpu["value"], 4)
         cpu["host_cores_visible"] = os.cpu_count()
 
     value = w.value(ms_per_step)
-    out = {
+    rec = {
         "metric": w.metric, "value": round(value, 3), "unit": w.unit, "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": w.higher_is_better, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic", "config": w.config,
         "roofline": roofline, "cpu_baseline": cpu,
     }
     if w.unit == "GB/s":
-        out["pct_of_hbm_peak"] = round(100.0 * value / HBM_PEAK_GBS, 2)
+        rec["pct_of_hbm_peak"] = round(100.0 * value / HBM_PEAK_GBS, 2)
+    if hasattr(w, "after"):
+        w.after(rec, steps)
+    return rec
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="spmv", choices=sorted(WORKLOADS) + ["ref_timing"])
+    ap.add_argument("--cpu-seconds", type=float, default=10.0,
+                    help="CPU time budget of the cpu_baseline leg (0 skips it)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="with the default workload: leave out the `workloads` block")
+    ap.add_argument("--extra-steps", type=int, default=20, help="timed steps of each extra workload")
+    ap.add_argument("--extra-cpu-seconds", type=float, default=5.0,
+                    help="CPU time budget of each extra workload's cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
+                 f"--gpus {args.gpus} is not supported, use --gpus 1")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    if args.workload == "ref_timing":
+        print(json.dumps(ref_timing(dev, args.cpu_seconds)))
+        return
+
+    out = measure(WORKLOADS[args.workload](), dev, args.steps, args.warmup, args.cpu_seconds)
+    if args.workload == "spmv" and not args.no_extras:
+        from numml_amd import _binding
+        keep = ("value", "unit", "ms_per_step", "steps", "warmup", "higher_is_better", "dtype", "config",
+                "roofline", "cpu_baseline", "pct_of_hbm_peak")
+        out["workloads"] = {}
+        for name in EXTRAS:
+            _binding.ops.clear_plan_cache()
+            torch.cuda.empty_cache()
+            rec = measure(WORKLOADS[name](), dev, args.extra_steps, min(args.warmup, 3),
+                          min(args.cpu_seconds, args.extra_cpu_seconds))
+            out["workloads"][name] = {k: rec[k] for k in keep if k in rec}
     print(json.dumps(out))
 
 

@@ -138,14 +138,26 @@ int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
  *
  *   nm_spgemm_workspace_bytes  -> bytes of device scratch both phases need
  *   nm_spgemm_symbolic         -> fills C_indptr (A_rows + 1 entries)
- *   nm_spgemm_symbolic_result  -> waits for the stream and hands the host
- *                                 nnz(C) = C_indptr[A_rows], with which the
- *                                 caller allocates, and the number of rows
+ *   nm_spgemm_symbolic_result  -> waits for the symbolic phase and hands the
+ *                                 host nnz(C) = C_indptr[A_rows], with which
+ *                                 the caller allocates, and the number of rows
  *                                 the hash path took (the reference's own
  *                                 read of the last row pointer,
  *                                 cpp/sparse_csr_cpu.cpp:166, is this
  *                                 synchronisation point); a caller may read
- *                                 C_indptr[A_rows] itself instead
+ *                                 C_indptr[A_rows] itself instead.
+ *                                 host_landing: 24 bytes of pinned host memory
+ *                                 the device can write (hipHostMalloc with
+ *                                 hipHostMallocCoherent, or a pinned torch
+ *                                 tensor), zeroed once by the caller when it is
+ *                                 allocated and from then on left to this
+ *                                 call, which has a one-lane kernel write the
+ *                                 two numbers and a ticket there and polls the
+ *                                 ticket (a few us instead of the ~30 us of a
+ *                                 stream wait).  One landing place serves one
+ *                                 call at a time (one per host thread).  NULL:
+ *                                 a plain copy and hipStreamSynchronize.  The
+ *                                 library itself allocates nothing here.
  *   nm_spgemm_numeric          -> fills C_indices (ascending in each row) and
  *                                 C_data; entries whose sum is 0 are kept,
  *                                 as the reference keeps them.  hash_rows is
@@ -166,7 +178,7 @@ int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols,
 
 int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const void *workspace,
                               size_t workspace_bytes, int64_t *nnz_C, int64_t *hash_rows,
-                              nm_stream stream);
+                              void *host_landing, nm_stream stream);
 
 int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t B_cols,
                       const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,

@@ -62,6 +62,16 @@ def backward_mode():
     return ops.backward_mode() if name == "compiled" else ops.BACKWARD_MODE
 
 
+def set_backward_mode(mode):
+    """Switch the selected binding between the 'planned' and the 'atomic' backward."""
+    if mode not in ("planned", "atomic"):
+        raise ValueError(f"backward mode must be 'planned' or 'atomic', got {mode!r}")
+    if name == "compiled":
+        ops.set_backward_mode(mode)
+    else:
+        ops.BACKWARD_MODE = mode
+
+
 def install(module_name="numml_torch_cpp"):
     """Register the compiled extension under the reference's module name.
 

@@ -302,7 +302,11 @@ __global__ __launch_bounds__(kBlock) void numeric_front_kernel(
     // is no workgroup barrier).  A value therefore takes a whole 8-byte slot of s_bb whatever
     // T is (packed floats would put the ring of wavefront w over the exchange entries of
     // wavefront w / 2, which then read a wrong row start).
-    static_assert(sizeof(T) <= sizeof(int64_t), "ring values alias s_bb");
+    static_assert(sizeof(T) <= sizeof(s_bb[0]), "a ring value must fit one exchange slot of s_bb");
+    static_assert(sizeof(s_bb) / sizeof(s_bb[0]) == kBlock && sizeof(s_len) / sizeof(s_len[0]) == kBlock,
+                  "one exchange slot per lane: wavefront w owns slots [64 w, 64 w + 64)");
+    static_assert(8 /* groups per wavefront */ * 8 /* ring entries per group */ == nm::kWave,
+                  "the ring of a wavefront must cover exactly that wavefront's own exchange slots");
     int32_t *s_oc = s_len;
     auto s_ov = [&](int slot) -> T & { return *reinterpret_cast<T *>(s_bb + slot); };
     const int ring = ((threadIdx.x >> 6) * 8 + merge_group()) * 8;
@@ -1287,7 +1291,7 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
 
 extern "C" int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const void *workspace,
                                          size_t workspace_bytes, int64_t *nnz_C, int64_t *hash_rows,
-                                         nm_stream stream) {
+                                         void *host_landing, nm_stream stream) {
     if (int rc = check_common(A_rows, B_cols)) return rc;
     NM_REQUIRE(workspace && nnz_C && hash_rows, "null pointer argument");
     Work w;
@@ -1298,26 +1302,26 @@ extern "C" int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const v
     *hash_rows = 0;
     if (A_rows == 0) return NM_OK;
     hipStream_t s = nm::as_stream(stream);
-    // a pinned landing place per host thread, kept for the life of the process: a copy into
-    // pageable memory goes through the runtime's staging path and takes several times as long
-    // The two numbers are written straight into pinned host memory by a one-lane kernel, followed
-    // by a ticket the host polls for: waking up from hipStreamSynchronize, or a copy-engine
-    // transfer of 16 bytes, takes ~30 us, several times what the kernels of a small product take
-    // together.  One landing place per host thread, kept for the life of the process.
-    static thread_local volatile int64_t *both = nullptr;
-    static thread_local int64_t ticket = 0;
-    if (!both) {
-        void *mem = nullptr;
-        NM_HIP_TRY(hipHostMalloc(&mem, 3 * sizeof(int64_t), hipHostMallocDefault));
-        both = (volatile int64_t *)mem;
-        both[2] = 0;
+    if (!host_landing) {
+        // no landing place from the caller: an ordinary copy and a wait for the stream
+        int64_t both[2] = {0, 0};
+        NM_HIP_TRY(hipMemcpyAsync(both, w.summary, sizeof(both), hipMemcpyDeviceToHost, s));
+        NM_HIP_TRY(hipStreamSynchronize(s));
+        *nnz_C = both[0];
+        *hash_rows = both[1];
+        return NM_OK;
     }
-    ++ticket;
+    // The two numbers are written straight into the caller's pinned host memory by a one-lane
+    // kernel, followed by a ticket the host polls for: waking up from hipStreamSynchronize, or a
+    // copy-engine transfer of 16 bytes, takes ~30 us, several times what the kernels of a small
+    // product take together.  The ticket is one more than the last one this landing place saw.
+    volatile int64_t *both = (volatile int64_t *)host_landing;
+    const int64_t ticket = both[2] + 1;
     hipLaunchKernelGGL(summary_out_kernel, dim3(1), dim3(64), 0, s, w.summary, both, ticket);
     NM_LAUNCH_CHECK("summary_out_kernel");
     bool arrived = false;
     for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = both[2] == ticket;
-    if (!arrived) {   // a long queue ahead of the kernel: wait the ordinary way
+    if (!arrived) {   // a long queue ahead of the kernel, or memory the host sees late: wait the ordinary way
         NM_HIP_TRY(hipStreamSynchronize(s));
         NM_REQUIRE(both[2] == ticket, "the symbolic phase's result did not arrive");
     }

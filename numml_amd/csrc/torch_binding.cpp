@@ -86,6 +86,42 @@ Tensor scratch(size_t bytes, const c10::Device &dev) {
                         torch::TensorOptions().dtype(torch::kUInt8).device(dev));
 }
 
+// ---- argument shapes ------------------------------------------------------------
+//
+// Host-side checks of everything a kernel would index with: they look at tensor
+// metadata only and run before anything is launched (a wrong length would otherwise
+// become an out-of-bounds access on the device).  The reference's accessors do not
+// check these either; its CPU loops merely fail more benignly.
+
+void check_csr(const char *who, int64_t rows, int64_t cols, const Tensor &data, const Tensor &indices,
+               const Tensor &indptr) {
+    TORCH_CHECK(rows >= 0 && cols >= 0, who, ": negative shape ", rows, " x ", cols);
+    TORCH_CHECK(indptr.dim() == 1 && indptr.numel() == rows + 1, who, ": expected ", rows + 1,
+                " row pointers for ", rows, " rows, got a tensor of shape ", indptr.sizes());
+    TORCH_CHECK(data.dim() == 1 && indices.dim() == 1 && data.numel() == indices.numel(), who,
+                ": values and column indices must be 1-D and of equal length, got ", data.sizes(), " and ",
+                indices.sizes());
+}
+
+void check_vector(const char *who, const char *name, const Tensor &t, int64_t n) {
+    TORCH_CHECK(t.dim() == 1 && t.numel() == n, who, ": expected ", name, " with ", n, " entries, got shape ",
+                t.sizes());
+}
+
+void check_matrix(const char *who, const char *name, const Tensor &t, int64_t rows, int64_t cols) {
+    TORCH_CHECK(t.dim() == 2 && t.size(0) == rows && (cols < 0 || t.size(1) == cols), who, ": expected ", name,
+                " of shape ", rows, " x ", cols < 0 ? std::string("n") : std::to_string(cols), ", got ",
+                t.sizes());
+}
+
+// 24 bytes of pinned host memory per host thread (from torch's pinned-memory allocator, which
+// also takes it back): where nm_spgemm_symbolic_result has the device drop nnz(C).
+void *host_landing() {
+    thread_local Tensor landing =
+        torch::zeros({3}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+    return landing.data_ptr();
+}
+
 // "planned" (default): backward passes walk A by column on a cached transposed
 // structure (deterministic, no atomics); "atomic": stateless scatter with atomics.
 // NUMML_AMD_BACKWARD sets the initial value, set_backward_mode() changes it.
@@ -212,6 +248,8 @@ Tensor solve(const Plan &plan, bool transposed, const Tensor &A_data, bool unit,
 // ---------------------------------------------------------------------------- SpMV
 
 Tensor spgemv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_col_ind, Tensor A_rowptr, Tensor x) {
+    check_csr("spgemv_forward", A_rows, A_cols, A_data, A_col_ind, A_rowptr);
+    check_vector("spgemv_forward", "x", x, A_cols);
     const auto dev = need_device({&A_data, &A_col_ind, &A_rowptr, &x});
     same_dtype(A_data, x, "x");
     TORCH_CHECK(x.dim() == 1, "expected 1-D x, got ", x.dim(), "-D");
@@ -230,6 +268,9 @@ Tensor spgemv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_col_ind, T
 
 std::vector<Tensor> spgemv_backward(Tensor grad_z, int A_rows, int A_cols, Tensor A_data, Tensor A_col_ind,
                                     Tensor A_rowptr, Tensor x) {
+    check_csr("spgemv_backward", A_rows, A_cols, A_data, A_col_ind, A_rowptr);
+    check_vector("spgemv_backward", "x", x, A_cols);
+    check_vector("spgemv_backward", "grad_z", grad_z, A_rows);
     const auto dev = need_device({&grad_z, &A_data, &A_col_ind, &A_rowptr, &x});
     same_dtype(A_data, x, "x");
     same_dtype(A_data, grad_z, "grad_z");
@@ -259,6 +300,7 @@ std::vector<Tensor> spgemv_backward(Tensor grad_z, int A_rows, int A_cols, Tenso
 
 std::vector<Tensor> csr_transpose_forward(int A_rows, int A_columns, Tensor A_data, Tensor A_indices,
                                           Tensor A_indptr) {
+    check_csr("csr_transpose_forward", A_rows, A_columns, A_data, A_indices, A_indptr);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr});
     A_data = A_data.contiguous();
     A_indices = index_tensor(A_indices, "A_indices");
@@ -280,6 +322,8 @@ std::vector<Tensor> csr_transpose_forward(int A_rows, int A_columns, Tensor A_da
 }
 
 Tensor csr_transpose_backward(Tensor grad_At, Tensor At_to_A_idx) {
+    check_vector("csr_transpose_backward", "At_to_A_idx", At_to_A_idx, grad_At.numel());
+    TORCH_CHECK(grad_At.dim() == 1, "csr_transpose_backward: expected 1-D grad_At, got shape ", grad_At.sizes());
     const auto dev = need_device({&grad_At, &At_to_A_idx});
     grad_At = grad_At.contiguous();
     At_to_A_idx = index_tensor(At_to_A_idx, "At_to_A_idx");
@@ -296,6 +340,8 @@ Tensor csr_transpose_backward(Tensor grad_At, Tensor At_to_A_idx) {
 std::vector<Tensor> splincomb_forward(int rows, int cols, Tensor alpha, Tensor A_data, Tensor A_indices,
                                       Tensor A_indptr, Tensor beta, Tensor B_data, Tensor B_indices,
                                       Tensor B_indptr) {
+    check_csr("splincomb_forward", rows, cols, A_data, A_indices, A_indptr);
+    check_csr("splincomb_forward", rows, cols, B_data, B_indices, B_indptr);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B_data, &B_indices, &B_indptr});
     same_dtype(A_data, B_data, "B_data");
     A_data = A_data.contiguous();
@@ -332,6 +378,9 @@ std::vector<Tensor> splincomb_forward(int rows, int cols, Tensor alpha, Tensor A
 std::vector<Tensor> splincomb_backward(int rows, int cols, Tensor alpha, Tensor A_data, Tensor A_indices,
                                        Tensor A_indptr, Tensor beta, Tensor B_data, Tensor B_indices,
                                        Tensor B_indptr, Tensor grad_C_data, Tensor C_indices, Tensor C_indptr) {
+    check_csr("splincomb_backward", rows, cols, A_data, A_indices, A_indptr);
+    check_csr("splincomb_backward", rows, cols, B_data, B_indices, B_indptr);
+    check_csr("splincomb_backward", rows, cols, grad_C_data, C_indices, C_indptr);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B_data, &B_indices, &B_indptr, &grad_C_data,
                                   &C_indices, &C_indptr});
     same_dtype(A_data, B_data, "B_data");
@@ -359,6 +408,7 @@ std::vector<Tensor> splincomb_backward(int rows, int cols, Tensor alpha, Tensor 
 // ------------------------------------------------- dense copy, row sums, diagonal
 
 Tensor csr_to_dense_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    check_csr("csr_to_dense_forward", A_rows, A_cols, A_data, A_indices, A_indptr);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr});
     A_data = A_data.contiguous();
     A_indices = index_tensor(A_indices, "A_indices");
@@ -374,6 +424,7 @@ Tensor csr_to_dense_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indi
 
 Tensor csr_to_dense_backward(Tensor grad_Ad, int A_rows, int A_cols, Tensor A_data, Tensor A_indices,
                              Tensor A_indptr) {
+    check_csr("csr_to_dense_backward", A_rows, A_cols, A_data, A_indices, A_indptr);
     const auto dev = need_device({&grad_Ad, &A_data, &A_indices, &A_indptr});
     same_dtype(A_data, grad_Ad, "grad_Ad");
     TORCH_CHECK(grad_Ad.dim() == 2 && grad_Ad.size(0) == A_rows && grad_Ad.size(1) == A_cols,
@@ -392,6 +443,7 @@ Tensor csr_to_dense_backward(Tensor grad_Ad, int A_rows, int A_cols, Tensor A_da
 }
 
 Tensor csr_row_sum_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    check_csr("csr_row_sum_forward", A_rows, A_cols, A_data, A_indices, A_indptr);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr});
     A_data = A_data.contiguous();
     A_indptr = index_tensor(A_indptr, "A_indptr");
@@ -405,6 +457,8 @@ Tensor csr_row_sum_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indic
 
 Tensor csr_row_sum_backward(Tensor grad_x, int A_rows, int A_cols, Tensor A_data, Tensor A_indices,
                             Tensor A_indptr) {
+    check_csr("csr_row_sum_backward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    check_vector("csr_row_sum_backward", "grad_x", grad_x, A_rows);
     const auto dev = need_device({&grad_x, &A_data, &A_indices, &A_indptr});
     same_dtype(A_data, grad_x, "grad_x");
     grad_x = grad_x.contiguous();
@@ -418,6 +472,7 @@ Tensor csr_row_sum_backward(Tensor grad_x, int A_rows, int A_cols, Tensor A_data
 }
 
 Tensor csr_extract_diagonal_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    check_csr("csr_extract_diagonal_forward", A_rows, A_cols, A_data, A_indices, A_indptr);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr});
     A_data = A_data.contiguous();
     A_indices = index_tensor(A_indices, "A_indices");
@@ -433,6 +488,8 @@ Tensor csr_extract_diagonal_forward(int A_rows, int A_cols, Tensor A_data, Tenso
 
 Tensor csr_extract_diagonal_backward(Tensor grad_x, int A_rows, int A_cols, Tensor A_data, Tensor A_indices,
                                      Tensor A_indptr) {
+    check_csr("csr_extract_diagonal_backward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    check_vector("csr_extract_diagonal_backward", "grad_x", grad_x, A_rows);
     const auto dev = need_device({&grad_x, &A_data, &A_indices, &A_indptr});
     same_dtype(A_data, grad_x, "grad_x");
     grad_x = grad_x.contiguous();
@@ -450,6 +507,8 @@ Tensor csr_extract_diagonal_backward(Tensor grad_x, int A_rows, int A_cols, Tens
 // ---------------------------------------------------------------------------- SpMM
 
 Tensor spdmm_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr, Tensor B) {
+    check_csr("spdmm_forward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    check_matrix("spdmm_forward", "B", B, A_cols, -1);
     // cpp/sparse_csr.cpp:125-128 checks the same thing with the same wording
     TORCH_CHECK((A_data.device() == A_indices.device() && A_indices.device() == A_indptr.device() &&
                  A_indptr.device() == B.device()),
@@ -474,6 +533,9 @@ Tensor spdmm_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Te
 
 std::vector<Tensor> spdmm_backward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr,
                                    Tensor B, Tensor grad_C) {
+    check_csr("spdmm_backward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    check_matrix("spdmm_backward", "B", B, A_cols, -1);
+    check_matrix("spdmm_backward", "grad_C", grad_C, A_rows, B.size(1));
     TORCH_CHECK((A_data.device() == A_indices.device() && A_indices.device() == A_indptr.device() &&
                  A_indptr.device() == B.device()),
                 "expected A and B to be on same device, but got A on (", A_data.device(), ", ",
@@ -515,6 +577,9 @@ std::vector<Tensor> spdmm_backward(int A_rows, int A_cols, Tensor A_data, Tensor
 
 std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr,
                                    int B_rows, int B_cols, Tensor B_data, Tensor B_indices, Tensor B_indptr) {
+    check_csr("spgemm_forward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    check_csr("spgemm_forward", B_rows, B_cols, B_data, B_indices, B_indptr);
+    TORCH_CHECK(A_cols == B_rows, "spgemm_forward: A has ", A_cols, " columns but B has ", B_rows, " rows");
     const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B_data, &B_indices, &B_indptr});
     same_dtype(A_data, B_data, "B_data");
     A_data = A_data.contiguous();
@@ -536,7 +601,8 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
           "nm_spgemm_symbolic");
     // the one device->host read the interface makes inherent: C is returned exactly sized
     int64_t nnz_c = 0, hash_rows = 0;
-    check(nm_spgemm_symbolic_result(A_rows, B_cols, work.data_ptr(), bytes, &nnz_c, &hash_rows, st),
+    check(nm_spgemm_symbolic_result(A_rows, B_cols, work.data_ptr(), bytes, &nnz_c, &hash_rows, host_landing(),
+                                    st),
           "nm_spgemm_symbolic_result");
     Tensor C_indices = torch::empty({nnz_c}, iopt);
     Tensor C_data = torch::empty({nnz_c}, A_data.options());
@@ -552,6 +618,10 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
 std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_indptr, int A_rows, int A_cols,
                                     Tensor A_data, Tensor A_indices, Tensor A_indptr, int B_rows, int B_cols,
                                     Tensor B_data, Tensor B_indices, Tensor B_indptr) {
+    check_csr("spgemm_backward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    check_csr("spgemm_backward", B_rows, B_cols, B_data, B_indices, B_indptr);
+    check_csr("spgemm_backward", A_rows, B_cols, grad_C, C_indices, C_indptr);
+    TORCH_CHECK(A_cols == B_rows, "spgemm_backward: A has ", A_cols, " columns but B has ", B_rows, " rows");
     const auto dev = need_device({&grad_C, &C_indices, &C_indptr, &A_data, &A_indices, &A_indptr, &B_data,
                                   &B_indices, &B_indptr});
     same_dtype(A_data, B_data, "B_data");
@@ -580,6 +650,9 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
 
 Tensor sptrsv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr, bool lower,
                       bool unit, Tensor b) {
+    check_csr("sptrsv_forward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    TORCH_CHECK(A_rows == A_cols, "sptrsv_forward: expected a square matrix, got ", A_rows, " x ", A_cols);
+    check_vector("sptrsv_forward", "b", b, A_rows);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr, &b});
     same_dtype(A_data, b, "b");
     A_data = A_data.contiguous();
@@ -593,6 +666,10 @@ Tensor sptrsv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, T
 
 std::vector<Tensor> sptrsv_backward(Tensor grad_x, Tensor x, int A_rows, int A_cols, Tensor A_data,
                                     Tensor A_indices, Tensor A_indptr, bool lower, bool unit, Tensor b) {
+    check_csr("sptrsv_backward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    TORCH_CHECK(A_rows == A_cols, "sptrsv_backward: expected a square matrix, got ", A_rows, " x ", A_cols);
+    check_vector("sptrsv_backward", "grad_x", grad_x, A_rows);
+    check_vector("sptrsv_backward", "x", x, A_rows);
     const auto dev = need_device({&grad_x, &x, &A_data, &A_indices, &A_indptr});
     same_dtype(A_data, grad_x, "grad_x");
     same_dtype(A_data, x, "x");
@@ -668,6 +745,7 @@ std::shared_ptr<Plan> lu_pattern(const Tensor &A_indices, const Tensor &A_indptr
 
 // [M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]  (cpp/sparse_csr.hpp:107-111)
 std::vector<Tensor> splu(int A_rows, int A_cols, Tensor A_data, Tensor A_indices, Tensor A_indptr) {
+    check_csr("splu", A_rows, A_cols, A_data, A_indices, A_indptr);
     const auto dev = need_device({&A_data, &A_indices, &A_indptr});
     TORCH_CHECK(A_rows == A_cols, "Expected square matrix for LU factorization, got ", A_rows, " x ", A_cols, ".");
     A_data = A_data.contiguous();
@@ -715,6 +793,11 @@ std::vector<Tensor> splu(int A_rows, int A_cols, Tensor A_data, Tensor A_indices
 std::vector<Tensor> spsolve_backward(Tensor grad_x, Tensor x, int A_rows, int A_cols, Tensor Mt_data,
                                      Tensor Mt_indices, Tensor Mt_indptr, Tensor A_data, Tensor A_indices,
                                      Tensor A_indptr) {
+    check_csr("spsolve_backward", A_rows, A_cols, A_data, A_indices, A_indptr);
+    check_csr("spsolve_backward", A_rows, A_cols, Mt_data, Mt_indices, Mt_indptr);
+    TORCH_CHECK(A_rows == A_cols, "spsolve_backward: expected a square matrix, got ", A_rows, " x ", A_cols);
+    check_vector("spsolve_backward", "grad_x", grad_x, A_rows);
+    check_vector("spsolve_backward", "x", x, A_rows);
     const auto dev = need_device({&grad_x, &x, &Mt_data, &Mt_indices, &Mt_indptr, &A_data, &A_indices, &A_indptr});
     same_dtype(A_data, grad_x, "grad_x");
     same_dtype(A_data, x, "x");
@@ -743,6 +826,8 @@ std::vector<Tensor> spsolve_backward(Tensor grad_x, Tensor x, int A_rows, int A_
 // ------------------------------------------------------------------------ diagnostics
 
 std::tuple<int64_t, int64_t> sptrsv_schedule(int A_rows, Tensor A_indices, Tensor A_indptr, bool lower) {
+    TORCH_CHECK(A_indptr.dim() == 1 && A_indptr.numel() == (int64_t)A_rows + 1 && A_indices.dim() == 1,
+                "sptrsv_schedule: expected ", A_rows + 1, " row pointers, got shape ", A_indptr.sizes());
     const auto dev = need_device({&A_indices, &A_indptr});
     A_indices = index_tensor(A_indices, "A_indices");
     A_indptr = index_tensor(A_indptr, "A_indptr");

@@ -82,6 +82,37 @@ def _rowmajor(M):
     return M, ld
 
 
+# Host-side checks of everything a kernel would index with; they look at tensor metadata
+# only and run before anything is launched (a wrong length would otherwise become an
+# out-of-bounds access on the device).
+
+def _check_csr(who, rows, cols, data, indices, indptr):
+    if rows < 0 or cols < 0:
+        raise RuntimeError(f"{who}: negative shape {rows} x {cols}")
+    if indptr.dim() != 1 or indptr.shape[0] != rows + 1:
+        raise RuntimeError(f"{who}: expected {rows + 1} row pointers for {rows} rows, got a tensor of shape "
+                           f"{list(indptr.shape)}")
+    if data.dim() != 1 or indices.dim() != 1 or data.shape[0] != indices.shape[0]:
+        raise RuntimeError(f"{who}: values and column indices must be 1-D and of equal length, got "
+                           f"{list(data.shape)} and {list(indices.shape)}")
+
+
+def _check_vector(who, name, t, n):
+    if t.dim() != 1 or t.shape[0] != n:
+        raise RuntimeError(f"{who}: expected {name} with {n} entries, got shape {list(t.shape)}")
+
+
+def _check_matrix(who, name, t, rows, cols=None):
+    if t.dim() != 2 or t.shape[0] != rows or (cols is not None and t.shape[1] != cols):
+        raise RuntimeError(f"{who}: expected {name} of shape {rows} x {'n' if cols is None else cols}, got "
+                           f"{list(t.shape)}")
+
+
+def _square(who, rows, cols):
+    if rows != cols:
+        raise RuntimeError(f"{who}: expected a square matrix, got {rows} x {cols}")
+
+
 # ------------------------------------------------------------ structure plans
 #
 # Everything derived from a sparsity pattern alone (the transposed structure, the
@@ -153,6 +184,8 @@ def _transpose_plan(indices, indptr, rows, cols, dev):
 
 def spgemv_forward(A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
     """y = A x  (cpp/sparse_csr.hpp:32-36)."""
+    _check_csr("spgemv_forward", A_rows, A_cols, A_data, A_col_ind, A_rowptr)
+    _check_vector("spgemv_forward", "x", x, A_cols)
     dev = _need_device(A_data, A_col_ind, A_rowptr, x)
     _same_dtype(A_data, x, "x")
     A_data, x = A_data.contiguous(), x.contiguous()
@@ -169,6 +202,9 @@ def spgemv_forward(A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
 
 def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
     """[grad_A, grad_x]  (cpp/sparse_csr.hpp:38-42)."""
+    _check_csr("spgemv_backward", A_rows, A_cols, A_data, A_col_ind, A_rowptr)
+    _check_vector("spgemv_backward", "x", x, A_cols)
+    _check_vector("spgemv_backward", "grad_z", grad_z, A_rows)
     dev = _need_device(grad_z, A_data, A_col_ind, A_rowptr, x)
     _same_dtype(A_data, x, "x")
     _same_dtype(A_data, grad_z, "grad_z")
@@ -194,6 +230,7 @@ def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
 
 def csr_transpose_forward(A_rows, A_columns, A_data, A_indices, A_indptr):
     """[At_data, At_indices, At_indptr, At_to_A_idx]  (cpp/sparse_csr.hpp:57-61)."""
+    _check_csr("csr_transpose_forward", A_rows, A_columns, A_data, A_indices, A_indptr)
     dev = _need_device(A_data, A_indices, A_indptr)
     A_data = A_data.contiguous()
     A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
@@ -212,6 +249,9 @@ def csr_transpose_forward(A_rows, A_columns, A_data, A_indices, A_indptr):
 
 def csr_transpose_backward(grad_At, At_to_A_idx):
     """grad_A with grad_A[At_to_A_idx[p]] = grad_At[p]  (cpp/sparse_csr.hpp:63-65)."""
+    _check_vector("csr_transpose_backward", "At_to_A_idx", At_to_A_idx, grad_At.numel())
+    if grad_At.dim() != 1:
+        raise RuntimeError(f"csr_transpose_backward: expected 1-D grad_At, got shape {list(grad_At.shape)}")
     dev = _need_device(grad_At, At_to_A_idx)
     _dt(grad_At)
     grad_At = grad_At.contiguous()
@@ -230,6 +270,8 @@ def _scalar(v):
 
 def splincomb_forward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr):
     """[C_data, C_indices, C_indptr] of alpha A + beta B  (cpp/sparse_csr.hpp:67-72)."""
+    _check_csr("splincomb_forward", rows, cols, A_data, A_indices, A_indptr)
+    _check_csr("splincomb_forward", rows, cols, B_data, B_indices, B_indptr)
     dev = _need_device(A_data, A_indices, A_indptr, B_data, B_indices, B_indptr)
     _same_dtype(A_data, B_data, "B_data")
     A_data, B_data = A_data.contiguous(), B_data.contiguous()
@@ -257,6 +299,9 @@ def splincomb_forward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_da
 def splincomb_backward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_data, B_indices, B_indptr,
                        grad_C_data, C_indices, C_indptr):
     """[grad_A, grad_B]  (cpp/sparse_csr.hpp:74-79)."""
+    _check_csr("splincomb_backward", rows, cols, A_data, A_indices, A_indptr)
+    _check_csr("splincomb_backward", rows, cols, B_data, B_indices, B_indptr)
+    _check_csr("splincomb_backward", rows, cols, grad_C_data, C_indices, C_indptr)
     dev = _need_device(A_data, A_indices, A_indptr, B_data, B_indices, B_indptr, grad_C_data, C_indices, C_indptr)
     _same_dtype(A_data, B_data, "B_data")
     _same_dtype(A_data, grad_C_data, "grad_C_data")
@@ -277,6 +322,7 @@ def splincomb_backward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_d
 
 def csr_to_dense_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
     """Dense A_rows x A_cols copy  (cpp/sparse_csr.hpp:122-126)."""
+    _check_csr("csr_to_dense_forward", A_rows, A_cols, A_data, A_indices, A_indptr)
     dev = _need_device(A_data, A_indices, A_indptr)
     A_data = A_data.contiguous()
     A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
@@ -290,6 +336,7 @@ def csr_to_dense_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
 
 def csr_to_dense_backward(grad_Ad, A_rows, A_cols, A_data, A_indices, A_indptr):
     """grad_A[k] = grad_Ad[row(k), col(k)]  (cpp/sparse_csr.hpp:128-133)."""
+    _check_csr("csr_to_dense_backward", A_rows, A_cols, A_data, A_indices, A_indptr)
     dev = _need_device(grad_Ad, A_data, A_indices, A_indptr)
     _same_dtype(A_data, grad_Ad, "grad_Ad")
     if grad_Ad.ndim != 2 or tuple(grad_Ad.shape) != (A_rows, A_cols):
@@ -306,6 +353,7 @@ def csr_to_dense_backward(grad_Ad, A_rows, A_cols, A_data, A_indices, A_indptr):
 
 def csr_row_sum_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
     """x[i] = sum of row i  (cpp/sparse_csr.hpp:136-140)."""
+    _check_csr("csr_row_sum_forward", A_rows, A_cols, A_data, A_indices, A_indptr)
     dev = _need_device(A_data, A_indices, A_indptr)
     A_data, A_indptr = A_data.contiguous(), _idx(A_indptr, "A_indptr")
     with torch.cuda.device(dev):
@@ -318,6 +366,8 @@ def csr_row_sum_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
 
 def csr_row_sum_backward(grad_x, A_rows, A_cols, A_data, A_indices, A_indptr):
     """grad_A[k] = grad_x[row(k)]  (cpp/sparse_csr.hpp:142-147)."""
+    _check_csr("csr_row_sum_backward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_vector("csr_row_sum_backward", "grad_x", grad_x, A_rows)
     dev = _need_device(grad_x, A_data, A_indices, A_indptr)
     _same_dtype(A_data, grad_x, "grad_x")
     grad_x, A_indptr = grad_x.contiguous(), _idx(A_indptr, "A_indptr")
@@ -331,6 +381,7 @@ def csr_row_sum_backward(grad_x, A_rows, A_cols, A_data, A_indices, A_indptr):
 
 def csr_extract_diagonal_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
     """x[i] = stored entry (i, i) or 0  (cpp/sparse_csr.hpp:150-154)."""
+    _check_csr("csr_extract_diagonal_forward", A_rows, A_cols, A_data, A_indices, A_indptr)
     dev = _need_device(A_data, A_indices, A_indptr)
     A_data = A_data.contiguous()
     A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
@@ -344,6 +395,8 @@ def csr_extract_diagonal_forward(A_rows, A_cols, A_data, A_indices, A_indptr):
 
 def csr_extract_diagonal_backward(grad_x, A_rows, A_cols, A_data, A_indices, A_indptr):
     """grad_A = 0 except grad_x[i] on the diagonal entries  (cpp/sparse_csr.hpp:156-161)."""
+    _check_csr("csr_extract_diagonal_backward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_vector("csr_extract_diagonal_backward", "grad_x", grad_x, A_rows)
     dev = _need_device(grad_x, A_data, A_indices, A_indptr)
     _same_dtype(A_data, grad_x, "grad_x")
     grad_x = grad_x.contiguous()
@@ -358,6 +411,8 @@ def csr_extract_diagonal_backward(grad_x, A_rows, A_cols, A_data, A_indices, A_i
 
 def spdmm_forward(A_rows, A_cols, A_data, A_indices, A_indptr, B):
     """C = A B, B dense 2-D  (cpp/sparse_csr.hpp:81-85)."""
+    _check_csr("spdmm_forward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_matrix("spdmm_forward", "B", B, A_cols)
     dev = _need_device(A_data, A_indices, A_indptr, B)
     _same_dtype(A_data, B, "B")
     A_data = A_data.contiguous()
@@ -374,6 +429,9 @@ def spdmm_forward(A_rows, A_cols, A_data, A_indices, A_indptr, B):
 
 def spdmm_backward(A_rows, A_cols, A_data, A_indices, A_indptr, B, grad_C):
     """[grad_A, grad_B]  (cpp/sparse_csr.hpp:87-91)."""
+    _check_csr("spdmm_backward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_matrix("spdmm_backward", "B", B, A_cols)
+    _check_matrix("spdmm_backward", "grad_C", grad_C, A_rows, B.shape[1])
     dev = _need_device(A_data, A_indices, A_indptr, B, grad_C)
     _same_dtype(A_data, B, "B")
     _same_dtype(A_data, grad_C, "grad_C")
@@ -401,6 +459,18 @@ def spdmm_backward(A_rows, A_cols, A_data, A_indices, A_indptr, B, grad_C):
 
 # ------------------------------------------------------------------- SpGEMM
 
+_landing = threading.local()
+
+
+def _host_landing():
+    """24 bytes of pinned host memory per host thread: where nm_spgemm_symbolic_result has the
+    device drop nnz(C) (torch's pinned-memory allocator owns it)."""
+    t = getattr(_landing, "t", None)
+    if t is None:
+        t = _landing.t = torch.zeros(3, dtype=torch.int64).pin_memory()
+    return t
+
+
 def spgemm_forward(A_rows, A_cols, A_data, A_indices, A_indptr,
                    B_rows, B_cols, B_data, B_indices, B_indptr):
     """[C_data, C_indices, C_indptr]  (cpp/sparse_csr.hpp:45-48).
@@ -408,6 +478,10 @@ def spgemm_forward(A_rows, A_cols, A_data, A_indices, A_indptr,
     One device->host read of nnz(C) sits between the two phases; it is inherent
     to the interface, which returns exactly-sized tensors.
     """
+    _check_csr("spgemm_forward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_csr("spgemm_forward", B_rows, B_cols, B_data, B_indices, B_indptr)
+    if A_cols != B_rows:
+        raise RuntimeError(f"spgemm_forward: A has {A_cols} columns but B has {B_rows} rows")
     dev = _need_device(A_data, A_indices, A_indptr, B_data, B_indices, B_indptr)
     _same_dtype(A_data, B_data, "B_data")
     A_data, B_data = A_data.contiguous(), B_data.contiguous()
@@ -426,7 +500,8 @@ def spgemm_forward(A_rows, A_cols, A_data, A_indices, A_indptr,
             _ptr(C_indptr), _ptr(work), nbytes.value, st), "nm_spgemm_symbolic")
         nnz_c, hash_rows = ctypes.c_int64(0), ctypes.c_int64(0)
         _lib.check(L.nm_spgemm_symbolic_result(A_rows, B_cols, _ptr(work), nbytes.value, ctypes.byref(nnz_c),
-                                               ctypes.byref(hash_rows), st), "nm_spgemm_symbolic_result")
+                                               ctypes.byref(hash_rows), _ptr(_host_landing()), st),
+                   "nm_spgemm_symbolic_result")
         C_indices = torch.empty(nnz_c.value, dtype=torch.int64, device=dev)
         C_data = torch.empty(nnz_c.value, dtype=A_data.dtype, device=dev)
         _lib.check(L.nm_spgemm_numeric(
@@ -440,6 +515,11 @@ def spgemm_backward(grad_C, C_indices, C_indptr,
                     A_rows, A_cols, A_data, A_indices, A_indptr,
                     B_rows, B_cols, B_data, B_indices, B_indptr):
     """[grad_A, grad_B]  (cpp/sparse_csr.hpp:50-54)."""
+    _check_csr("spgemm_backward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_csr("spgemm_backward", B_rows, B_cols, B_data, B_indices, B_indptr)
+    _check_csr("spgemm_backward", A_rows, B_cols, grad_C, C_indices, C_indptr)
+    if A_cols != B_rows:
+        raise RuntimeError(f"spgemm_backward: A has {A_cols} columns but B has {B_rows} rows")
     dev = _need_device(grad_C, C_indices, C_indptr, A_data, A_indices, A_indptr,
                        B_data, B_indices, B_indptr)
     _same_dtype(A_data, B_data, "B_data")
@@ -542,6 +622,7 @@ def _lu_pattern(A_indices, A_indptr, rows, dev):
 def splu(A_rows, A_cols, A_data, A_indices, A_indptr):
     """[M_data, M_indices, M_indptr, Mt_data, Mt_indices, Mt_indptr]: L + U without pivoting on the
     filled pattern, and its transpose  (cpp/sparse_csr.hpp:107-111)."""
+    _check_csr("splu", A_rows, A_cols, A_data, A_indices, A_indptr)
     dev = _need_device(A_data, A_indices, A_indptr)
     if A_rows != A_cols:
         raise RuntimeError(f"Expected square matrix for LU factorization, got {A_rows} x {A_cols}.")
@@ -570,6 +651,11 @@ def splu(A_rows, A_cols, A_data, A_indices, A_indptr):
 def spsolve_backward(grad_x, x, A_rows, A_cols, Mt_data, Mt_indices, Mt_indptr, A_data, A_indices, A_indptr):
     """[grad_A, grad_b]: grad_b = A^-T grad_x by two solves with M^T, grad_A = -(grad_b x^T) on A's
     pattern  (cpp/sparse_csr.hpp:113-118, cpp/sparse_csr_cpu.cpp:1018-1048)."""
+    _check_csr("spsolve_backward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_csr("spsolve_backward", A_rows, A_cols, Mt_data, Mt_indices, Mt_indptr)
+    _square("spsolve_backward", A_rows, A_cols)
+    _check_vector("spsolve_backward", "grad_x", grad_x, A_rows)
+    _check_vector("spsolve_backward", "x", x, A_rows)
     dev = _need_device(grad_x, x, Mt_data, Mt_indices, Mt_indptr, A_data, A_indices, A_indptr)
     _same_dtype(A_data, grad_x, "grad_x")
     _same_dtype(A_data, x, "x")
@@ -593,6 +679,8 @@ def sptrsv_schedule(A_rows, A_indices, A_indptr, lower):
     """(dependency levels, kernel launches per solve) of the level schedule of a
     triangular pattern, built or taken from the cache; diagnostics, no counterpart
     in the reference."""
+    if A_indptr.dim() != 1 or A_indptr.shape[0] != A_rows + 1 or A_indices.dim() != 1:
+        raise RuntimeError(f"sptrsv_schedule: expected {A_rows + 1} row pointers, got shape {list(A_indptr.shape)}")
     dev = _need_device(A_indices, A_indptr)
     A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
     with torch.cuda.device(dev):
@@ -619,6 +707,9 @@ def _solve(plan, transposed, A_data, A_indices, A_indptr, unit, b, rows, dev):
 
 def sptrsv_forward(A_rows, A_cols, A_data, A_indices, A_indptr, lower, unit, b):
     """x = A^{-1} b for triangular A  (cpp/sparse_csr.hpp:94-98)."""
+    _check_csr("sptrsv_forward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _square("sptrsv_forward", A_rows, A_cols)
+    _check_vector("sptrsv_forward", "b", b, A_rows)
     dev = _need_device(A_data, A_indices, A_indptr, b)
     _same_dtype(A_data, b, "b")
     A_data, b = A_data.contiguous(), b.contiguous()
@@ -630,6 +721,10 @@ def sptrsv_forward(A_rows, A_cols, A_data, A_indices, A_indptr, lower, unit, b):
 
 def sptrsv_backward(grad_x, x, A_rows, A_cols, A_data, A_indices, A_indptr, lower, unit, b):
     """[grad_A, grad_b]  (cpp/sparse_csr.hpp:100-105)."""
+    _check_csr("sptrsv_backward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _square("sptrsv_backward", A_rows, A_cols)
+    _check_vector("sptrsv_backward", "grad_x", grad_x, A_rows)
+    _check_vector("sptrsv_backward", "x", x, A_rows)
     dev = _need_device(grad_x, x, A_data, A_indices, A_indptr)
     _same_dtype(A_data, grad_x, "grad_x")
     _same_dtype(A_data, x, "x")

@@ -35,6 +35,12 @@ def load():
     return _mod
 
 
+def built():
+    """True when the compiled reference is present; looks at the file system only (does
+    not load the library, so test collection stays free of it)."""
+    return bool(glob.glob(os.path.join(_HERE, "_ref", "numml_ref_cpu*.so")))
+
+
 def available():
     return load() is not None
 

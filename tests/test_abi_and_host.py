@@ -172,3 +172,68 @@ def test_product_path_does_not_touch_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
                 assert "liboracle" not in text, f
+
+
+def test_integration_snippet_runs():
+    # the "keep the reference's CPU path" block of INTEGRATION.md, executed as written against a
+    # stand-in for the reference's compiled module
+    import sys
+    import types
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = re.search(r"```python\n(import numml_torch_cpp as ref_ext.*?)```", text, flags=re.S).group(1)
+    stub = types.ModuleType("numml_torch_cpp")
+    calls = []
+    for name in ("spgemv", "spdmm", "spgemm", "sptrsv"):
+        for d in ("forward", "backward"):
+            setattr(stub, f"{name}_{d}", lambda *a, _n=f"{name}_{d}": calls.append(_n) or "cpu")
+    saved = sys.modules.get("numml_torch_cpp")
+    sys.modules["numml_torch_cpp"] = stub
+    try:
+        exec(compile(block, "INTEGRATION.md", "exec"), {})
+        d, i, p = torch.ones(3), torch.tensor([0, 1, 2]), torch.tensor([0, 1, 2, 3])
+        assert stub.spgemv_forward(3, 3, d, i, p, torch.ones(3)) == "cpu"      # CPU tensors -> the reference
+        assert stub.sptrsv_forward(3, 3, d, i, p, True, False, torch.ones(3)) == "cpu"
+        assert calls == ["spgemv_forward", "sptrsv_forward"]
+    finally:
+        if saved is None:
+            del sys.modules["numml_torch_cpp"]
+        else:
+            sys.modules["numml_torch_cpp"] = saved
+
+
+@pytest.mark.parametrize("binding", ["ctypes", "compiled"])
+def test_mismatched_sizes_raise_before_anything_is_launched(binding):
+    # every length a kernel would index with is checked on the host; CPU tensors suffice to see it,
+    # because the shape checks come before the device check
+    m = ext if binding == "ctypes" else numml_amd.load_compiled()
+    d, i, p = torch.ones(3), torch.tensor([0, 1, 2]), torch.tensor([0, 1, 2, 3])
+    x, X = torch.ones(3), torch.ones(3, 2)
+    bad = [
+        (m.spgemv_forward, (3, 3, d, i, p[:3], x), "row pointers"),
+        (m.spgemv_forward, (3, 3, d, i[:2], p, x), "equal length"),
+        (m.spgemv_forward, (3, 3, d, i, p, torch.ones(4)), "x with 3 entries"),
+        (m.spgemv_forward, (3, 4, d, i, p, x), "x with 4 entries"),
+        (m.spgemv_backward, (torch.ones(2), 3, 3, d, i, p, x), "grad_z with 3 entries"),
+        (m.spdmm_forward, (3, 3, d, i, p, torch.ones(4, 2)), "B of shape 3 x n"),
+        (m.spdmm_backward, (3, 3, d, i, p, X, torch.ones(3, 3)), "grad_C of shape 3 x 2"),
+        (m.spgemm_forward, (3, 3, d, i, p, 4, 3, d, i, torch.tensor([0, 1, 2, 3, 3])), "columns but B has"),
+        (m.spgemm_forward, (3, 3, d, i, p, 3, 3, d, i, p[:2]), "row pointers"),
+        (m.spgemm_backward, (torch.ones(2), i, p, 3, 3, d, i, p, 3, 3, d, i, p), "equal length"),
+        (m.sptrsv_forward, (3, 3, d, i, p, True, False, torch.ones(2)), "b with 3 entries"),
+        (m.sptrsv_forward, (3, 4, d, i, p, True, False, x), "square"),
+        (m.sptrsv_backward, (x, torch.ones(5), 3, 3, d, i, p, True, False, x), "x with 3 entries"),
+        (m.csr_transpose_forward, (3, 3, d, i, p[:1]), "row pointers"),
+        (m.csr_transpose_backward, (d, i[:2]), "At_to_A_idx with 3 entries"),
+        (m.splincomb_forward, (3, 3, torch.tensor(1.0), d, i, p, torch.tensor(1.0), d, i, p[:3]), "row pointers"),
+        (m.csr_to_dense_forward, (2, 3, d, i, p), "row pointers"),
+        (m.csr_row_sum_backward, (torch.ones(4), 3, 3, d, i, p), "grad_x with 3 entries"),
+        (m.csr_extract_diagonal_forward, (3, 3, d[:2], i, p), "equal length"),
+        (m.splu, (3, 3, d, i, p[:2]), "row pointers"),
+        (m.spsolve_backward, (x, x, 3, 3, d, i, p, d, i[:1], p), "equal length"),
+    ]
+    for fn, args, msg in bad:
+        with pytest.raises(RuntimeError, match=msg):
+            fn(*args)
+    # well-formed CPU tensors get past the shape checks and are refused for their device
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        m.spgemv_forward(3, 3, d, i, p, x)

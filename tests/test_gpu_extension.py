@@ -190,8 +190,10 @@ def test_spgemm_through_the_c_abi_with_and_without_the_hash_row_count(dev, hint)
         Cp = torch.empty(r + 1, dtype=torch.int64, device=dev)
         _lib.check(L.nm_spgemm_symbolic(r, c, c, ptr(I), ptr(P), ptr(I), ptr(P), ptr(Cp), ptr(work), nbytes.value, st), "symbolic")
         nnz_c, hash_rows = ctypes.c_int64(-7), ctypes.c_int64(-7)
-        _lib.check(L.nm_spgemm_symbolic_result(r, c, ptr(work), nbytes.value, ctypes.byref(nnz_c), ctypes.byref(hash_rows), st),
-                   "result")
+        # with a pinned landing place for the device to write into (hint "given"), and without one
+        landing = torch.zeros(3, dtype=torch.int64).pin_memory() if hint == "given" else None
+        _lib.check(L.nm_spgemm_symbolic_result(r, c, ptr(work), nbytes.value, ctypes.byref(nnz_c), ctypes.byref(hash_rows),
+                                               ptr(landing) if landing is not None else None, st), "result")
         Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(r, c, d, i, p, r, c, d, i, p)
         assert nnz_c.value == Cd_ref.shape[0] == int(Cp[-1].item()), name
         assert (hash_rows.value == 0) == name.startswith("stencil"), (name, hash_rows.value)

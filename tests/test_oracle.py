@@ -94,7 +94,7 @@ def test_golden_explicit_zero_is_kept():
 
 # ------------------------------------------------------------- compiled reference
 
-needs_ref = pytest.mark.skipif(not ref.available(), reason="oracle/_ref not built (needs the reference tree)")
+needs_ref = pytest.mark.skipif(not ref.built(), reason="oracle/_ref not built (needs the reference tree)")
 
 
 @needs_ref
