@@ -242,6 +242,27 @@ int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
                     const void *data, int unit, const void *b, void *x,
                     void *work, size_t work_bytes, nm_stream stream);
 
+/* nm_sptrsv_solve without the `work` argument, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  It has no counterpart in the reference.  The scratch
+ * of the solve lives in a 64 MiB device array built into the library, one copy
+ * per GPU, held until the process ends; the call allocates nothing, neither
+ * through HIP nor through any other library, and does not synchronise.  A plan
+ * whose nm_sptrsv_solve_bytes(rows, nnz) exceeds nm_sptrsv_solve_static_capacity
+ * (roughly 7 * rows + 3 * nnz doubles, e.g. 500 000 rows with three entries per
+ * row) is rejected with NM_ERR_UNSUPPORTED.  Every call on one GPU uses that
+ * GPU's one array: calls that overlap on the same GPU (two streams, two threads)
+ * race and must be serialised by the caller.  Results are bit-identical to
+ * nm_sptrsv_solve.  The device must be current on the calling thread.
+ * nm_sptrsv_solve_static_capacity also performs the one-time address look-up of
+ * the array for the current device, so a caller may call it before it starts a
+ * capture. */
+int nm_sptrsv_solve_static_capacity(size_t *bytes);
+
+int nm_sptrsv_solve_static(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
+                           const void *data, int unit, const void *b, void *x,
+                           nm_stream stream);
+
 /* out[k] = alpha * a[row(k)] * b[col(k)] for every stored entry: the masked
  * outer product behind grad_A of the solve (alpha = -1,
  * cpp/sparse_csr_cpu.cpp:750-755) and of SpMV (alpha = 1, :60-65). */

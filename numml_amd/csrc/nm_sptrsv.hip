@@ -36,6 +36,7 @@
 #include "nm_scan.hpp"
 #include "nm_transpose.hpp"
 
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -1121,6 +1122,68 @@ extern "C" int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int tran
     const size_t need = solve_work_layout(plan->rows, plan->nnz, nullptr, nullptr);
     if (work_bytes < need)
         return nm::fail(NM_ERR_WORKSPACE, "solve workspace of %zu bytes, %zu needed", work_bytes, need);
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F64) return solve_typed<double>(plan, transposed, data, unit, b, x, work, s);
+    return solve_typed<float>(plan, transposed, data, unit, b, x, work, s);
+}
+
+// ---- the solve for callers that cannot allocate ---------------------------------
+//
+// Same launches as nm_sptrsv_solve, with the per-call scratch (level-major copies of
+// the coefficients, diagonal, right-hand side and the running solution) in a
+// file-scope device array instead of caller memory.  Every GPU the library runs on
+// holds its own copy of the array at its own address until the process ends; the
+// array's name is only a host-side handle, so the device address is looked up once
+// per device and that pointer is what the kernels receive.
+namespace {
+
+constexpr size_t kStaticSolveBytes = size_t(64) << 20;   // 64 MiB per GPU
+static __device__ __align__(256) unsigned char scratch[kStaticSolveBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+void *g_static_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on first use).
+int static_scratch(void **out) {
+    int dev = -1;
+    NM_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return nm::fail(NM_ERR_UNSUPPORTED, "device index %d", dev);
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        void *ptr = nullptr;
+        NM_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return nm::fail(NM_ERR_HIP, "hipGetSymbolAddress returned a null address");
+        g_static_ptr[dev] = ptr;
+    }
+    *out = g_static_ptr[dev];
+    return NM_OK;
+}
+
+}  // namespace
+
+extern "C" int nm_sptrsv_solve_static_capacity(size_t *bytes) {
+    NM_REQUIRE(bytes != nullptr, "bytes is null");
+    void *ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    *bytes = kStaticSolveBytes;
+    return NM_OK;
+}
+
+extern "C" int nm_sptrsv_solve_static(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed, const void *data,
+                                      int unit, const void *b, void *x, nm_stream stream) {
+    NM_REQUIRE(plan != nullptr, "plan is null");
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    if (plan->rows == 0) return NM_OK;
+    NM_REQUIRE(b && x && (plan->nnz == 0 || data), "null pointer argument");
+    const size_t need = solve_work_layout(plan->rows, plan->nnz, nullptr, nullptr);
+    if (need > kStaticSolveBytes)
+        return nm::fail(NM_ERR_UNSUPPORTED,
+                        "a solve with %lld rows and %lld entries needs %zu bytes of scratch; the built-in "
+                        "buffer of nm_sptrsv_solve_static holds %zu (use nm_sptrsv_solve with caller memory)",
+                        (long long)plan->rows, (long long)plan->nnz, need, kStaticSolveBytes);
+    void *work = nullptr;
+    if (int rc = static_scratch(&work)) return rc;
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F64) return solve_typed<double>(plan, transposed, data, unit, b, x, work, s);
     return solve_typed<float>(plan, transposed, data, unit, b, x, work, s);
