@@ -101,8 +101,13 @@ class Workload:
         raise NotImplementedError
 
 
-def _spmv_bytes(rows, cols, nnz, s):
-    fwd = nnz * (s + 8) + (rows + 1) * 8 + cols * s + rows * s
+def _spmv_bytes(rows, cols, nnz, s, i_fwd=8):
+    """Algorithmic bytes of one forward and one backward.  i_fwd: index bytes the forward reads
+    per entry and per row pointer (8 as the interface delivers them, 4 when the kernel reads
+    the 32-bit copies a transposed-structure plan holds).  The planned backward reads two
+    int32 per entry (row and position in the plan), i.e. the same 8 index bytes per entry as
+    the int64 row-major formula, and 4-byte column pointers."""
+    fwd = nnz * (s + i_fwd) + (rows + 1) * i_fwd + cols * s + rows * s
     bwd = nnz * (s + 8) + (rows + 1) * 8 + rows * s + cols * s + nnz * s + cols * s
     return fwd, bwd
 
@@ -134,10 +139,13 @@ class SpMV(Workload):
         self.D, self.I, self.P, self.X, self.Gv = t(d), t(i), t(p), t(self.x_h), t(self.g_h)
         self.rows, self.cols, self.nnz = rows, cols, d.shape[0]
         s = d.dtype.itemsize
-        self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s)
+        # with a plan in the cache (every step after the second backward) the forward reads the
+        # plan's 32-bit structure
+        planned = _binding.backward_mode() != "atomic" and _binding.name == "compiled"
+        self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s, 4 if planned else 8)
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
-        self.dominant_name = ("spmv_bwd_planned_kernel" if _binding.backward_mode() == "planned"
+        self.dominant_name = ("spmv_bwd_planned_kernel" if _binding.backward_mode() != "atomic"
                               else "spmv_bwd_kernel (+ fill_kernel clearing grad_x)")
         # Structure analysis is timed apart from the steps.  The first backward calls on a new
         # sparsity pattern are timed one by one: the transposed-structure plan of the default
@@ -152,7 +160,10 @@ class SpMV(Workload):
         self.first_backward_ms = firsts
         self.config = {"workload": f"spmv_fwd_bwd_{self.dtype}_{self.label}", "rows": rows,
                        "first_three_backward_calls_ms": firsts,
-                       "nnz": self.nnz, "index_bytes": 8, "backward": _binding.backward_mode(),
+                       "nnz": self.nnz, "index_bytes_forward": 4 if planned else 8,
+                       "index_bytes_backward": 8, "backward": _binding.backward_mode(),
+                       "forward_bytes": self.fwd_bytes, "backward_bytes": self.bwd_bytes,
+                       "bytes_per_step_with_int64_forward": sum(_spmv_bytes(rows, cols, self.nnz, s, 8)),
                        "binding": _binding.name,
                        "algorithmic_bytes_per_step": self.bytes_per_step}
 
@@ -161,9 +172,11 @@ class SpMV(Workload):
         the plan, and the number of steps after which building it has paid off."""
         import torch
         from numml_amd import _binding
-        if _binding.backward_mode() != "planned":
+        mode = _binding.backward_mode()
+        if mode == "atomic":
             return
         _binding.set_backward_mode("atomic")
+        self.ext.clear_plan_cache()     # the forward, too, is to run without a plan
         try:
             for _ in range(3):
                 self.step()
@@ -174,10 +187,12 @@ class SpMV(Workload):
             torch.cuda.synchronize()
             stateless = (time.perf_counter() - t0) / steps * 1e3
         finally:
-            _binding.set_backward_mode("planned")
+            _binding.set_backward_mode(mode)
         build = max(self.first_backward_ms) - rec["roofline"]["avg_ms"]
         gain = stateless - rec["ms_per_step"]
         rec["config"]["stateless_ms_per_step"] = round(stateless, 5)
+        rec["config"]["stateless_GBps_int64_structure"] = round(
+            rec["config"]["bytes_per_step_with_int64_forward"] / (stateless * 1e-3) / 1e9, 1)
         rec["config"]["plan_build_ms"] = round(build, 3)
         rec["config"]["plan_break_even_steps"] = int(np.ceil(build / gain)) if gain > 0 else None
         rec["config"]["amortised_ms_per_step_over_100_steps"] = round(rec["ms_per_step"] + build / 100, 5)
@@ -231,15 +246,17 @@ class SpMM(Workload):
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
         self.dominant_name = ("spdmm_bwd_kernel (grad_A) + spdmm_fwd_flat_kernel on the transposed plan (grad_B)"
-                              if _binding.backward_mode() == "planned"
+                              if _binding.backward_mode() != "atomic"
                               else "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)")
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        ext.spdmm_backward(rows, cols, self.D, self.I, self.P, self.B, self.Gv)
-        torch.cuda.synchronize()
-        first_bwd_ms = (time.perf_counter() - t0) * 1e3
+        firsts = []          # the plan of the default backward is built during one of these
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ext.spdmm_backward(rows, cols, self.D, self.I, self.P, self.B, self.Gv)
+            torch.cuda.synchronize()
+            firsts.append(round((time.perf_counter() - t0) * 1e3, 3))
         self.config = {"workload": "spmm_fwd_bwd_f32_powerlaw_1M_n64", "rows": rows, "nnz": nnz,
-                       "first_backward_ms_incl_plan_build": round(first_bwd_ms, 3),
+                       "first_three_backward_calls_ms": firsts, "backward": _binding.backward_mode(),
                        "dense_cols": n, "index_bytes": 8,
                        "algorithmic_bytes_per_step": self.bytes_per_step,
                        "gather_bytes_fwd": nnz * n * s}

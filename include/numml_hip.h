@@ -62,9 +62,27 @@ int nm_spgemv_backward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
                        const void *x, const void *g,
                        void *grad_A, void *grad_x, nm_stream stream);
 
+/* -------------------------------------------------- content key of a pattern
+ * A 128-bit key of (indices, indptr), equal for equal patterns whatever memory
+ * they live in: a caller that caches per-pattern analysis (the plans below) uses
+ * it to recognise a pattern that arrives in fresh tensors, as every product
+ * C = A B of the reference's interface does (cpp/sparse_csr.hpp:45-48 returns new
+ * index tensors on each call).  No counterpart in the reference, which keeps no
+ * per-pattern state.  One pass over both arrays; `work` holds
+ * nm_structure_hash_bytes bytes of device scratch.  The call waits for the key:
+ * with `host_landing` (32 bytes of pinned host memory the device can write,
+ * zeroed once when allocated) a kernel drops it there and the host polls, with
+ * NULL it is copied back after a hipStreamSynchronize. */
+int nm_structure_hash_bytes(size_t *bytes);
+
+int nm_structure_hash(int64_t nnz, int64_t nptr, const int64_t *indices, const int64_t *indptr,
+                      void *work, size_t work_bytes, void *host_landing, uint64_t *key,
+                      nm_stream stream);
+
 /* ---------------------------------------------- transposed-structure plan
  * The pattern of A^T as 32-bit arrays (column pointers, row of each entry and
- * its position in A's arrays, rows ascending inside a column), built once per
+ * its position in A's arrays, rows ascending inside a column) together with
+ * 32-bit copies of A's own column indices and row pointers, built once per
  * sparsity pattern in caller-provided device memory and reused by the
  * *_planned backward entry points below.  It is the structure (not the values)
  * of what csr_transpose_forward returns (cpp/sparse_csr_cpu.cpp:311-367:
@@ -94,6 +112,14 @@ int nm_csr_transpose_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_t nn
  * (cpp/sparse_csr.hpp:63-65, cpp/sparse_csr_cpu.cpp:369-385). */
 int nm_csr_transpose_backward(nm_dtype dt, int64_t nnz, const void *grad_At,
                               const int64_t *At_to_A_idx, void *grad_A, nm_stream stream);
+
+/* nm_spgemv_forward for a pattern whose transposed-structure plan has been
+ * built: the kernel reads the plan's 32-bit copies of A's column indices and
+ * row pointers instead of the int64 arrays (4 instead of 8 index bytes per
+ * entry); same sums in the same order, so y is bit-identical. */
+int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                              const void *data, const void *plan_mem,
+                              const void *x, void *y, nm_stream stream);
 
 /* nm_spgemv_backward on a transposed-structure plan: walks A by column, so
  * grad_x needs neither clearing nor atomics, is summed in ascending row order

@@ -58,14 +58,15 @@ ops, name = _select()
 
 
 def backward_mode():
-    """'planned' or 'atomic': how the selected binding computes SpMV/SpMM gradients."""
+    """'planned', 'eager' or 'atomic': how the selected binding computes SpMV/SpMM gradients."""
     return ops.backward_mode() if name == "compiled" else ops.BACKWARD_MODE
 
 
 def set_backward_mode(mode):
-    """Switch the selected binding between the 'planned' and the 'atomic' backward."""
-    if mode not in ("planned", "atomic"):
-        raise ValueError(f"backward mode must be 'planned' or 'atomic', got {mode!r}")
+    """Switch the selected binding's SpMV/SpMM backward: 'planned' (transposed-structure plan from
+    the second sighting of a pattern on), 'eager' (from the first) or 'atomic' (stateless)."""
+    if mode not in ("planned", "eager", "atomic"):
+        raise ValueError(f"backward mode must be 'planned', 'eager' or 'atomic', got {mode!r}")
     if name == "compiled":
         ops.set_backward_mode(mode)
     else:

@@ -23,9 +23,13 @@ _SIGNATURES = {
     "nm_spgemv_forward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_spgemv_backward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                            _c_ptr, _c_ptr, _c_ptr],
+    "nm_structure_hash_bytes": [ctypes.POINTER(_c_size)],
+    "nm_structure_hash": [_c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr, ctypes.POINTER(ctypes.c_uint64),
+                          _c_ptr],
     "nm_csr_transpose_plan_bytes": [_c_i64, _c_i64, _c_i64, ctypes.POINTER(_c_size), ctypes.POINTER(_c_size)],
     "nm_csr_transpose_plan_build": [_c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr, _c_size,
                                     _c_ptr],
+    "nm_spgemv_forward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_spgemv_backward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                    _c_ptr, _c_ptr],
     "nm_spdmm_backward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64,

@@ -643,7 +643,7 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
     if (int rc = check_args(dt, rows, cols, nnz, data, indices, indptr, n)) return rc;
     NM_REQUIRE(plan_mem != nullptr, "plan is null");
     nm::TPlan t;
-    nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
+    nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
     if (grad_A) {
         if (int rc = backward_impl(dt, rows, cols, nnz, data, indices, indptr, B, ldb, gC, ldg, n, grad_A, nullptr, 0,
                                    t.chunk_row, stream))

@@ -45,11 +45,11 @@ constexpr int32_t kHuge = 1 << 30;
 
 // Loads the block's row offsets relative to `base` into LDS, clamped to kHuge
 // so that they fit 32 bits whatever the block holds.
-template <int R, int CAP, int BLOCK>
-__device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ indptr, int64_t r0, int nr,
+template <int R, int CAP, int BLOCK, typename IDX = int64_t>
+__device__ __forceinline__ void stage_offsets(const IDX *__restrict__ indptr, int64_t r0, int nr,
                                               int64_t base, int32_t *s_off) {
     for (int t = threadIdx.x; t <= nr; t += BLOCK) {
-        const int64_t d = indptr[r0 + t] - base;
+        const int64_t d = (int64_t)indptr[r0 + t] - base;
         s_off[t] = (int32_t)(d > kHuge ? kHuge : d);
     }
 }
@@ -80,10 +80,13 @@ __device__ __forceinline__ int run_end(const int32_t *s_off, int s0, int nr, int
 // UNIT: x is taken as all ones and not read, which makes y the row sums
 // (cpp/sparse_csr_cpu.cpp:1121-1127); a * 1 == a exactly, so the summation is
 // the same storage-order sum.
-template <typename T, int BLOCK, int R, int CAP, bool UNIT = false>
+//
+// IDX: int64_t for the structure arrays as the interface delivers them, int32_t for the
+// 32-bit copies a transposed-structure plan of the same pattern holds.
+template <typename T, int BLOCK, int R, int CAP, bool UNIT = false, typename IDX = int64_t>
 __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
-    int64_t rows, int rt, const T *__restrict__ data, const int64_t *__restrict__ indices,
-    const int64_t *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y) {
+    int64_t rows, int rt, const T *__restrict__ data, const IDX *__restrict__ indices,
+    const IDX *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y) {
     // rt <= R: rows per block of this launch (block_rows)
     __shared__ int32_t s_off[R + 1];
     __shared__ T s_prod[CAP];
@@ -98,19 +101,19 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
         int nr = (int)(rows - r0 < rt ? rows - r0 : rt);
         nr = nr < R ? nr : R;   // rt <= R
         const int64_t base = indptr[r0];
-        stage_offsets<R, CAP, BLOCK>(indptr, r0, nr, base, s_off);
+        stage_offsets<R, CAP, BLOCK, IDX>(indptr, r0, nr, base, s_off);
         __syncthreads();
         const int n = s_off[nr];
         if (n <= CAP) {
             const T *__restrict__ d = data + base;
-            const int64_t *__restrict__ ci = indices + base;
+            const IDX *__restrict__ ci = indices + base;
             // K entries in flight per lane: all their streams, then all their gathers of x.
             // Loads are unconditional on a clamped position (a predicated load would sit in
             // its own branch with its own wait).
             constexpr int K = 5;   // 4, 5 and 10 measure the same on the 2048 x 2048 Poisson matrix
             for (int k0 = threadIdx.x; k0 < n; k0 += K * BLOCK) {
                 T aa[K], xx[K];
-                int64_t cc[K];
+                IDX cc[K];
 #pragma unroll
                 for (int u = 0; u < K; ++u) {
                     const int kc = k0 + u * BLOCK < n ? k0 + u * BLOCK : n - 1;
@@ -142,11 +145,11 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
             // of the row before the lanes are summed.
             auto products = [&](int64_t first, int cnt) {   // s_prod[j] = data * x of entry first + j
                 const T *__restrict__ d = data + first;
-                const int64_t *__restrict__ ci = indices + first;
+                const IDX *__restrict__ ci = indices + first;
                 constexpr int K = 5;
                 for (int k0 = threadIdx.x; k0 < cnt; k0 += K * BLOCK) {
                     T aa[K], xx[K];
-                    int64_t cc[K];
+                    IDX cc[K];
 #pragma unroll
                     for (int u = 0; u < K; ++u) {
                         const int kc = k0 + u * BLOCK < cnt ? k0 + u * BLOCK : cnt - 1;
@@ -587,15 +590,15 @@ int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const i
     return NM_OK;
 }
 
-template <typename T>
-int launch_fwd(int64_t rows, int64_t nnz, const T *data, const int64_t *indices, const int64_t *indptr, const T *x,
+template <typename T, typename IDX>
+int launch_fwd(int64_t rows, int64_t nnz, const T *data, const IDX *indices, const IDX *indptr, const T *x,
                T *y, hipStream_t s) {
     constexpr int R = kFwdR, CAP = kFwdCap;
     const int rt = block_rows(rows, nnz, R, CAP);
     int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows, rt,
-                       data, indices, indptr, x, y);
+    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, false, IDX>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s,
+                       rows, rt, data, indices, indptr, x, y);
     NM_LAUNCH_CHECK("spmv_fwd_kernel");
     return NM_OK;
 }
@@ -637,12 +640,30 @@ extern "C" int nm_spgemv_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_
     hipStream_t s = nm::as_stream(stream);
     switch (dt) {
         case NM_F32:
-            return launch_fwd<float>(rows, nnz, (const float *)data, indices, indptr, (const float *)x, (float *)y, s);
+            return launch_fwd<float, int64_t>(rows, nnz, (const float *)data, indices, indptr, (const float *)x,
+                                              (float *)y, s);
         case NM_F64:
-            return launch_fwd<double>(rows, nnz, (const double *)data, indices, indptr, (const double *)x,
-                                      (double *)y, s);
+            return launch_fwd<double, int64_t>(rows, nnz, (const double *)data, indices, indptr, (const double *)x,
+                                               (double *)y, s);
     }
     return nm::fail(NM_ERR_INVALID, "unknown dtype %d", (int)dt);
+}
+
+extern "C" int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                         const void *plan_mem, const void *x, void *y, nm_stream stream) {
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0 && plan_mem != nullptr, "bad sizes or null plan");
+    if (rows == 0) return NM_OK;
+    NM_REQUIRE(y != nullptr && (nnz == 0 || data != nullptr), "null pointer argument");
+    NM_REQUIRE(cols == 0 || x != nullptr, "x is null");
+    nm::TPlan t;
+    nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
+    hipStream_t s = nm::as_stream(stream);
+    if (dt == NM_F32)
+        return launch_fwd<float, int32_t>(rows, nnz, (const float *)data, t.c_idx32, t.c_ptr32, (const float *)x,
+                                          (float *)y, s);
+    return launch_fwd<double, int32_t>(rows, nnz, (const double *)data, t.c_idx32, t.c_ptr32, (const double *)x,
+                                       (double *)y, s);
 }
 
 extern "C" int nm_csr_row_sum_forward(nm_dtype dt, int64_t rows, int64_t nnz, const void *data,
@@ -699,7 +720,7 @@ extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t col
     if (cols == 0 || (!grad_A && !grad_x)) return NM_OK;
     NM_REQUIRE(nnz == 0 || (data && x && g), "null pointer argument");
     nm::TPlan t;
-    nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &t);
+    nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32) {
         constexpr int R = kPlannedR, CAP = kPlannedCap;

@@ -96,7 +96,7 @@ struct Layout {
 // plan memory: [transposed-structure plan][order][level_ptr][slot_of][meta][packed A][packed A^T]
 size_t plan_layout(int64_t rows, int64_t nnz, void *base, Layout *L) {
     Layout l;
-    size_t off = nm::tplan_layout(rows, nnz, base, &l.t);
+    size_t off = nm::tplan_layout(rows, rows, nnz, base, &l.t);
     auto take = [&](size_t count) {
         void *q = base ? static_cast<char *>(base) + off : nullptr;
         off += align_up(count * 4);

@@ -583,7 +583,7 @@ extern "C" int nm_csr_transpose_forward(nm_dtype dt, int64_t rows, int64_t cols,
     NM_REQUIRE(plan_mem && At_indptr, "null pointer argument");
     NM_REQUIRE(nnz == 0 || (data && At_data && At_indices && At_to_A_idx), "null pointer argument");
     nm::TPlan plan;
-    nm::tplan_layout(cols, nnz, const_cast<void *>(plan_mem), &plan);
+    nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &plan);
     hipStream_t s = nm::as_stream(stream);
     const unsigned grid = grid_for(nnz > cols + 1 ? nnz : cols + 1);
     if (dt == NM_F32)

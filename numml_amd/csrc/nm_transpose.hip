@@ -1,82 +1,48 @@
 // Builder of the transposed-structure plan (see nm_transpose.hpp) and its C ABI.
+//
+// A counting sort by column that keeps A's storage order inside every column,
+// which is what the reference's transpose does serially
+// (cpp/sparse_csr_cpu.cpp:334-361), in five device-driven steps and without a
+// general-purpose sort:
+//
+//   1. count    row tiles stream A's entries once: one atomic add per entry into
+//               a per-column counter, and the by-products every later kernel
+//               wants in 32 bits (row of each entry, column of each entry, row
+//               pointers, the row of every 64th entry);
+//   2. scan     exclusive prefix sum of the counters = column pointers;
+//   3. scatter  every entry draws a slot in its column from a per-column cursor
+//               (atomic add with return) and leaves its own position there.  The
+//               slots of a column are now filled, but in the order the hardware
+//               happened to serve the atomics;
+//   4. order    column tiles put each column's positions into ascending order.
+//               A position in A's row-major arrays grows with the row (and, for
+//               duplicate coordinates, with the storage order), so ascending
+//               positions ARE the stable order.  A column is ranked by counting
+//               in LDS (entry j goes to slot #{keys < key j}); a column too long
+//               for LDS is ranked piece by piece and the sorted pieces are merged
+//               pairwise by the workgroup through a scratch copy;
+//   5. flags    symmetric-pattern check against A itself.
+//
+// Nothing here depends on a host read, so the build is fully asynchronous.
 #include "nm_transpose.hpp"
 
-#include <rocprim/device/device_radix_sort.hpp>
+#include "nm_scan.hpp"
 
 namespace {
 
+using nm::kWave;
+
 constexpr int kBlock = 256;
-
-inline int bits_for(int64_t n) {
-    int b = 1;
-    while (b < 32 && (int64_t(1) << b) < n) ++b;
-    return b;
-}
-
-size_t sort_temp_bytes(int64_t nnz, int bits) {
-    size_t bytes = 0;
-    (void)rocprim::radix_sort_pairs(nullptr, bytes, (int32_t *)nullptr, (int32_t *)nullptr,
-                                    (int32_t *)nullptr, (int32_t *)nullptr, (size_t)(nnz > 0 ? nnz : 1), 0u,
-                                    (unsigned)bits, (hipStream_t)0);
-    return bytes;
-}
-
-// Per stored entry: sort key (column), payload (its own position) and its row,
-// found by bisection of indptr so that rows of any length cost the same.
-__global__ void entry_keys_kernel(int64_t nnz, int64_t rows, const int64_t *__restrict__ indices,
-                                  const int64_t *__restrict__ indptr, int32_t *__restrict__ keys,
-                                  int32_t *__restrict__ vals, int32_t *__restrict__ rowid) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz; k += stride) {
-        int64_t lo = 0, hi = rows + 1;  // first p with indptr[p] > k
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (indptr[mid] <= k) lo = mid + 1; else hi = mid;
-        }
-        keys[k] = (int32_t)indices[k];
-        vals[k] = (int32_t)k;
-        rowid[k] = (int32_t)(lo - 1);
-    }
-}
-
-__global__ void finish_kernel(int64_t nnz, int64_t cols, const int32_t *__restrict__ keys_sorted,
-                              const int32_t *__restrict__ t_perm, const int32_t *__restrict__ rowid,
-                              int32_t *__restrict__ t_row, int32_t *__restrict__ t_indptr,
-                              int32_t *__restrict__ chunk_row) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for (int64_t p = tid; p < nnz; p += stride) t_row[p] = rowid[t_perm[p]];
-    for (int64_t h = tid; h * 64 < nnz; h += stride) chunk_row[h] = rowid[h * 64];
-    for (int64_t c = tid; c <= cols; c += stride) {
-        int64_t lo = 0, hi = nnz;  // first sorted position whose column is >= c
-        while (lo < hi) {
-            const int64_t mid = (lo + hi) >> 1;
-            if (keys_sorted[mid] < c) lo = mid + 1; else hi = mid;
-        }
-        t_indptr[c] = (int32_t)lo;
-    }
-}
-
-__global__ void symmetry_init_kernel(int32_t *flags, int square) {
-    if (threadIdx.x == 0) flags[0] = square;
-}
-
-// Clears flags[0] unless A^T has exactly A's structure.
-__global__ void symmetry_check_kernel(int64_t nnz, int64_t cols, const int64_t *__restrict__ indices,
-                                      const int64_t *__restrict__ indptr, const int32_t *__restrict__ t_row,
-                                      const int32_t *__restrict__ t_indptr, int32_t *flags) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    bool same = true;
-    for (int64_t p = tid; p < nnz; p += stride) same &= (int64_t)t_row[p] == indices[p];
-    for (int64_t c = tid; c <= cols; c += stride) same &= (int64_t)t_indptr[c] == indptr[c];
-    if (!same) flags[0] = 0;
-}
+constexpr int kRows = 512;      // rows (columns) a workgroup stages offsets for
+constexpr int kCap = 4096;      // LDS keys of the ordering kernel
+constexpr int kSlice = 16;      // consecutive outputs one lane produces in a merge pass
 
 struct WorkT {
-    int32_t *keys, *keys_sorted, *vals, *rowid;
-    void *temp;
-    size_t temp_bytes;
+    int64_t *count;        // [cols + 1] per-column counters, then column pointers
+    int64_t *scan;         // scratch of the prefix sum
+    int32_t *cursor;       // [cols + 1] next free slot of every column
+    int32_t *rowid;        // [nnz] row of every entry (row-major order)
+    int32_t *tmp;          // [nnz] second copy of a long column during its merge passes
 };
 
 size_t work_layout(int64_t cols, int64_t nnz, void *base, WorkT *w) {
@@ -87,14 +53,219 @@ size_t work_layout(int64_t cols, int64_t nnz, void *base, WorkT *w) {
         return q;
     };
     WorkT t;
-    t.keys = (int32_t *)take((size_t)(nnz + 1) * 4);
-    t.keys_sorted = (int32_t *)take((size_t)(nnz + 1) * 4);
-    t.vals = (int32_t *)take((size_t)(nnz + 1) * 4);
+    t.count = (int64_t *)take((size_t)(cols + 2) * 8);
+    t.scan = (int64_t *)take(nm::scan_scratch_bytes(cols + 1));
+    t.cursor = (int32_t *)take((size_t)(cols + 2) * 4);
     t.rowid = (int32_t *)take((size_t)(nnz + 1) * 4);
-    t.temp_bytes = sort_temp_bytes(nnz, bits_for(cols));
-    t.temp = take(t.temp_bytes + 256);
+    t.tmp = (int32_t *)take((size_t)(nnz + 1) * 4);
     if (w) *w = t;
     return off;
+}
+
+// Rows a workgroup takes at a time: kRows where rows are short, fewer where they are long,
+// so that a tile holds a few thousand entries and the grid stays wide.
+inline int tile_rows(int64_t rows, int64_t nnz) {
+    const int64_t mean = rows > 0 ? (nnz + rows - 1) / rows : 1;
+    const int64_t r = kCap / (mean > 0 ? mean : 1);
+    return (int)(r > kRows ? kRows : (r < 8 ? 8 : r));
+}
+
+// Step 1.  A workgroup owns `rt` consecutive rows; lane = entry.  The row of an entry is found
+// by bisection over the tile's offsets in LDS, so rows of any length cost the same.
+__global__ __launch_bounds__(kBlock) void tp_count_kernel(
+    int64_t rows, int rt, const int64_t *__restrict__ indices, const int64_t *__restrict__ indptr,
+    unsigned long long *__restrict__ count, int32_t *__restrict__ rowid, int32_t *__restrict__ col32,
+    int32_t *__restrict__ ptr32, int32_t *__restrict__ chunk_row) {
+    __shared__ int32_t s_off[kRows + 1];
+    const int64_t ntiles = (rows + rt - 1) / rt, npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t r0 = tile * rt;
+        const int nr = (int)(rows - r0 < rt ? rows - r0 : rt);
+        const int64_t base = indptr[r0];
+        for (int t = threadIdx.x; t <= nr; t += kBlock) {
+            const int64_t p = indptr[r0 + t];
+            s_off[t] = (int32_t)(p - base);        // nnz < 2^31 for plans
+            ptr32[r0 + t] = (int32_t)p;
+        }
+        __syncthreads();
+        const int n = s_off[nr];
+        for (int j = threadIdx.x; j < n; j += kBlock) {
+            int lo = 0, hi = nr;                   // last t with s_off[t] <= j
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (s_off[mid] <= j) lo = mid; else hi = mid;
+            }
+            const int64_t k = base + j;
+            const int64_t c = nm::stream_load(indices + k);
+            atomicAdd(count + c, 1ull);
+            const int32_t r = (int32_t)(r0 + lo);
+            rowid[k] = r;
+            col32[k] = (int32_t)c;
+            if ((k & 63) == 0) chunk_row[k >> 6] = r;
+        }
+        __syncthreads();
+    }
+}
+
+// Column pointers and the scatter cursors from the scanned counters.
+__global__ void tp_pointers_kernel(int64_t cols, const int64_t *__restrict__ count,
+                                   int32_t *__restrict__ t_indptr, int32_t *__restrict__ cursor) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c <= cols; c += stride) {
+        const int32_t p = (int32_t)count[c];
+        t_indptr[c] = p;
+        cursor[c] = p;
+    }
+}
+
+// Step 3.
+__global__ void tp_scatter_kernel(int64_t nnz, const int32_t *__restrict__ col32, int32_t *__restrict__ cursor,
+                                  int32_t *__restrict__ t_perm) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < nnz; k += stride) {
+        const int32_t pos = atomicAdd(cursor + col32[k], 1);
+        t_perm[pos] = (int32_t)k;
+    }
+}
+
+// End of the run of columns that starts at column s0 of the tile and fits the LDS keys.
+__device__ __forceinline__ int run_end(const int32_t *s_off, int s0, int nc, int cap) {
+    const int32_t limit = s_off[s0] + cap;
+    if (s_off[nc] <= limit) return nc;
+    int lo = s0, hi = nc;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_off[mid] <= limit) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// One merge pass of the workgroup over a long column: sorted runs of `width` keys in `src`
+// become sorted runs of 2 * width keys in `dst`.  Every lane produces kSlice consecutive
+// outputs of one pair of runs: it finds where they start in the two runs by bisection along
+// the diagonal (keys are distinct) and merges serially from there.
+__device__ void merge_pass(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int len, int width) {
+    const int nslices = (len + kSlice - 1) / kSlice;
+    for (int sl = threadIdx.x; sl < nslices; sl += kBlock) {
+        const int o0 = sl * kSlice;                         // first output of the slice
+        const int pair0 = o0 / (2 * width) * (2 * width);   // start of its pair of runs
+        const int na = min(width, len - pair0), nb = max(0, min(width, len - pair0 - width));
+        const int32_t *a = src + pair0, *b = src + pair0 + na;
+        const int d = o0 - pair0;                           // outputs of this pair before the slice
+        int lo = max(0, d - nb), hi = min(d, na);           // i = keys taken from a, d - i from b
+        while (lo < hi) {
+            const int i = (lo + hi) >> 1;
+            if (a[i] < b[d - i - 1]) lo = i + 1; else hi = i;
+        }
+        int i = lo, j = d - lo;
+        const int end = min(kSlice, pair0 + na + nb - o0);
+        for (int u = 0; u < end; ++u) {
+            const bool from_a = j >= nb || (i < na && a[i] < b[j]);
+            dst[o0 + u] = from_a ? a[i] : b[j];
+            i += from_a;
+            j += !from_a;
+        }
+    }
+}
+
+// Step 4.  A workgroup owns `ct` consecutive columns.
+__global__ __launch_bounds__(kBlock) void tp_order_kernel(
+    int64_t cols, int ct, const int32_t *__restrict__ t_indptr, int32_t *__restrict__ t_perm,
+    const int32_t *__restrict__ rowid, int32_t *__restrict__ t_row, int32_t *__restrict__ tmp) {
+    __shared__ int32_t s_off[kRows + 1];
+    __shared__ int32_t s_key[kCap];
+    const int64_t ntiles = (cols + ct - 1) / ct, npad = nm::xcd_padded(ntiles);
+    for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
+        const int64_t tile = nm::xcd_tile(id, npad);
+        if (tile >= ntiles) continue;
+        const int64_t c0 = tile * ct;
+        const int nc = (int)(cols - c0 < ct ? cols - c0 : ct);
+        const int32_t base = t_indptr[c0];
+        for (int t = threadIdx.x; t <= nc; t += kBlock) s_off[t] = t_indptr[c0 + t] - base;
+        __syncthreads();
+
+        // columns [s0, e0) fit the LDS keys: stage, rank every key inside its column, write out
+        auto ranked = [&](const int s0, const int e0) {
+            const int o0 = s_off[s0], cnt = s_off[e0] - o0;
+            const int32_t first = base + o0;
+            for (int j = threadIdx.x; j < cnt; j += kBlock) s_key[j] = t_perm[first + j];
+            __syncthreads();
+            for (int j = threadIdx.x; j < cnt; j += kBlock) {
+                int lo = s0, hi = e0;                       // column of key j
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (s_off[mid] - o0 <= j) lo = mid; else hi = mid;
+                }
+                const int b = s_off[lo] - o0, e = s_off[lo + 1] - o0;
+                const int32_t key = s_key[j];
+                int rank = 0;
+                for (int q = b; q < e; ++q) rank += s_key[q] < key;
+                t_perm[first + b + rank] = key;
+                t_row[first + b + rank] = rowid[key];
+            }
+            __syncthreads();
+        };
+
+        for (int s0 = 0; s0 < nc;) {
+            const int e0 = run_end(s_off, s0, nc, kCap);
+            if (e0 > s0) {
+                ranked(s0, e0);
+                s0 = e0;
+                continue;
+            }
+            // One column longer than the LDS keys.  Pieces of kCap keys are ranked in LDS and
+            // written to `tmp` as sorted runs; merge passes then go back and forth between
+            // `tmp` and the plan until one run is left.
+            const int32_t first = base + s_off[s0];
+            const int len = s_off[s0 + 1] - s_off[s0];
+            int32_t *col = t_perm + first, *alt = tmp + first;
+            for (int q0 = 0; q0 < len; q0 += kCap) {
+                const int cnt = len - q0 < kCap ? len - q0 : kCap;
+                for (int j = threadIdx.x; j < cnt; j += kBlock) s_key[j] = col[q0 + j];
+                __syncthreads();
+                for (int j = threadIdx.x; j < cnt; j += kBlock) {
+                    const int32_t key = s_key[j];
+                    int rank = 0;
+                    for (int q = 0; q < cnt; ++q) rank += s_key[q] < key;
+                    alt[q0 + rank] = key;
+                }
+                __syncthreads();
+            }
+            int32_t *src = alt, *dst = col;
+            for (int width = kCap; width < len; width *= 2) {
+                merge_pass(src, dst, len, width);
+                __syncthreads();
+                int32_t *sw = src; src = dst; dst = sw;
+            }
+            // `src` holds the ordered column
+            for (int j = threadIdx.x; j < len; j += kBlock) {
+                const int32_t key = src[j];
+                if (src != col) col[j] = key;
+                t_row[first + j] = rowid[key];
+            }
+            __syncthreads();
+            s0 += 1;
+        }
+        __syncthreads();
+    }
+}
+
+__global__ void symmetry_init_kernel(int32_t *flags, int square) {
+    if (threadIdx.x == 0) flags[0] = square;
+}
+
+// Clears flags[0] unless A^T has exactly A's structure.
+__global__ void symmetry_check_kernel(int64_t nnz, int64_t cols, const int32_t *__restrict__ col32,
+                                      const int32_t *__restrict__ ptr32, const int32_t *__restrict__ t_row,
+                                      const int32_t *__restrict__ t_indptr, int32_t *flags) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    bool same = true;
+    for (int64_t p = tid; p < nnz; p += stride) same &= t_row[p] == col32[p];
+    for (int64_t c = tid; c <= cols; c += stride) same &= t_indptr[c] == ptr32[c];
+    if (!same) flags[0] = 0;
 }
 
 int check_sizes(int64_t rows, int64_t cols, int64_t nnz) {
@@ -119,27 +290,45 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
     const size_t need = work_layout(cols, nnz, work, &w);
     if (work_bytes < need) return fail(NM_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", work_bytes, need);
     int32_t *rowid = rowid_out ? rowid_out : w.rowid;
+    if (int rc = fill_async(w.count, cols + 1, (int64_t)0, s)) return rc;
+    if (rows > 0) {
+        const int rt = tile_rows(rows, nnz);
+        int64_t grid = xcd_padded(ceil_div(rows, rt));
+        if (grid > 65536) grid = 65536;
+        hipLaunchKernelGGL(tp_count_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, rt, indices, indptr,
+                           (unsigned long long *)w.count, rowid, plan.c_idx32, plan.c_ptr32, plan.chunk_row);
+        NM_LAUNCH_CHECK("tp_count_kernel");
+    } else {
+        if (int rc = fill_async(plan.c_ptr32, (int64_t)1, (int32_t)0, s)) return rc;
+    }
+    if (int rc = scan_exclusive_i64(w.count, cols + 1, w.scan, s)) return rc;
+    {
+        int64_t grid = ceil_div(cols + 1, kBlock);
+        if (grid > 65536) grid = 65536;
+        hipLaunchKernelGGL(tp_pointers_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, w.count,
+                           plan.t_indptr, w.cursor);
+        NM_LAUNCH_CHECK("tp_pointers_kernel");
+    }
     if (nnz > 0) {
         int64_t grid = ceil_div(nnz, kBlock);
         if (grid > 65536) grid = 65536;
-        hipLaunchKernelGGL(entry_keys_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, rows, indices,
-                           indptr, w.keys, w.vals, rowid);
-        NM_LAUNCH_CHECK("entry_keys_kernel");
-        size_t tb = w.temp_bytes;
-        hipError_t e = rocprim::radix_sort_pairs(w.temp, tb, w.keys, w.keys_sorted, w.vals, plan.t_perm,
-                                                 (size_t)nnz, 0u, (unsigned)bits_for(cols), s);
-        if (e != hipSuccess) return fail(NM_ERR_HIP, "radix sort failed: %s", hipGetErrorString(e));
+        hipLaunchKernelGGL(tp_scatter_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, plan.c_idx32, w.cursor,
+                           plan.t_perm);
+        NM_LAUNCH_CHECK("tp_scatter_kernel");
+        const int ct = tile_rows(cols, nnz);
+        grid = xcd_padded(ceil_div(cols, ct));
+        if (grid > 65536) grid = 65536;
+        hipLaunchKernelGGL(tp_order_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, ct, plan.t_indptr,
+                           plan.t_perm, rowid, plan.t_row, w.tmp);
+        NM_LAUNCH_CHECK("tp_order_kernel");
     }
-    int64_t m = nnz > cols + 1 ? nnz : cols + 1;
-    int64_t grid = ceil_div(m, kBlock);
-    if (grid > 65536) grid = 65536;
-    hipLaunchKernelGGL(finish_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, cols, w.keys_sorted,
-                       plan.t_perm, rowid, plan.t_row, plan.t_indptr, plan.chunk_row);
-    NM_LAUNCH_CHECK("transpose finish_kernel");
     hipLaunchKernelGGL(symmetry_init_kernel, dim3(1), dim3(64), 0, s, plan.flags, rows == cols ? 1 : 0);
     if (rows == cols) {
-        hipLaunchKernelGGL(symmetry_check_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, cols, indices,
-                           indptr, plan.t_row, plan.t_indptr, plan.flags);
+        int64_t m = nnz > cols + 1 ? nnz : cols + 1;
+        int64_t grid = ceil_div(m, kBlock);
+        if (grid > 65536) grid = 65536;
+        hipLaunchKernelGGL(symmetry_check_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nnz, cols, plan.c_idx32,
+                           plan.c_ptr32, plan.t_row, plan.t_indptr, plan.flags);
     }
     NM_LAUNCH_CHECK("symmetry check");
     return NM_OK;
@@ -151,7 +340,7 @@ extern "C" int nm_csr_transpose_plan_bytes(int64_t rows, int64_t cols, int64_t n
                                            size_t *work_bytes) {
     NM_REQUIRE(plan_bytes && work_bytes, "null size pointer");
     if (int rc = check_sizes(rows, cols, nnz)) return rc;
-    *plan_bytes = nm::tplan_layout(cols, nnz, nullptr, nullptr);
+    *plan_bytes = nm::tplan_layout(rows, cols, nnz, nullptr, nullptr);
     *work_bytes = nm::tplan_work_bytes(rows, cols, nnz);
     return NM_OK;
 }
@@ -162,7 +351,7 @@ extern "C" int nm_csr_transpose_plan_build(int64_t rows, int64_t cols, int64_t n
     if (int rc = check_sizes(rows, cols, nnz)) return rc;
     NM_REQUIRE(indptr && plan_mem && work && (nnz == 0 || indices), "null pointer argument");
     nm::TPlan plan;
-    const size_t need = nm::tplan_layout(cols, nnz, plan_mem, &plan);
+    const size_t need = nm::tplan_layout(rows, cols, nnz, plan_mem, &plan);
     if (plan_bytes < need)
         return nm::fail(NM_ERR_WORKSPACE, "plan memory of %zu bytes, %zu needed", plan_bytes, need);
     return nm::tplan_build(rows, cols, nnz, indices, indptr, plan, work, work_bytes, nullptr,

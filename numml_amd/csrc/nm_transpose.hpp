@@ -9,6 +9,10 @@
 //                start their walk there instead of bisecting indptr)  (ceil(nnz/64)+1)
 //   flags[0]     1 when the pattern is symmetric (A^T has A's structure, so
 //                entry p of column c is the mirror image of the row-major entry p)
+//   c_idx32[k]   column of the k-th entry of A's ROW-major arrays, in 32 bits   (nnz)
+//   c_ptr32[i]   row pointers of A in 32 bits                                   (rows + 1)
+//                (kernels that find a plan read these instead of the int64
+//                arrays the interface delivers: half the index traffic)
 //
 // Inside a column the entries keep A's row-major order (the sort is stable), so
 // rows ascend, exactly like the counting-sort transpose of the reference
@@ -25,12 +29,14 @@ struct TPlan {
     int32_t *t_perm;
     int32_t *chunk_row;
     int32_t *flags;
+    int32_t *c_idx32;
+    int32_t *c_ptr32;
 };
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
 // Carves the plan arrays out of `base` (nullptr: size query only); returns bytes.
-inline size_t tplan_layout(int64_t cols, int64_t nnz, void *base, TPlan *p) {
+inline size_t tplan_layout(int64_t rows, int64_t cols, int64_t nnz, void *base, TPlan *p) {
     size_t off = 0;
     auto take = [&](size_t bytes) {
         void *q = base ? static_cast<char *>(base) + off : nullptr;
@@ -42,7 +48,9 @@ inline size_t tplan_layout(int64_t cols, int64_t nnz, void *base, TPlan *p) {
     int32_t *c = (int32_t *)take((size_t)(nnz + 1) * 4);
     int32_t *h = (int32_t *)take((size_t)((nnz + 63) / 64 + 1) * 4);
     int32_t *f = (int32_t *)take(16 * 4);
-    if (p) *p = TPlan{a, b, c, h, f};
+    int32_t *ci = (int32_t *)take((size_t)(nnz + 1) * 4);
+    int32_t *cp = (int32_t *)take((size_t)(rows + 2) * 4);
+    if (p) *p = TPlan{a, b, c, h, f, ci, cp};
     return off;
 }
 

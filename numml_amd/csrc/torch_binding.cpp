@@ -16,6 +16,9 @@
 #include <torch/extension.h>
 
 #include <ATen/hip/HIPContext.h>
+#include <ATen/hip/HIPEvent.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPCachingAllocator.h>
 #include <c10/hip/HIPGuard.h>
 #include <c10/hip/HIPStream.h>
 
@@ -114,114 +117,281 @@ void check_matrix(const char *who, const char *name, const Tensor &t, int64_t ro
                 t.sizes());
 }
 
-// 24 bytes of pinned host memory per host thread (from torch's pinned-memory allocator, which
-// also takes it back): where nm_spgemm_symbolic_result has the device drop nnz(C).
-void *host_landing() {
-    thread_local Tensor landing =
-        torch::zeros({3}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
-    return landing.data_ptr();
-}
-
-// "planned" (default): backward passes walk A by column on a cached transposed
-// structure (deterministic, no atomics); "atomic": stateless scatter with atomics.
+// How SpMV / SpMM backward compute grad_x / grad_B:
+//   "planned" (default)  on a cached transposed-structure plan (deterministic, no atomics) from
+//                        the SECOND time a sparsity pattern is seen; the first sighting runs the
+//                        stateless kernels, so a pattern that is used once never pays for a plan;
+//   "eager"              the plan is built at the first sighting (deterministic from the first call);
+//   "atomic"             always the stateless scatter with atomics.
 // NUMML_AMD_BACKWARD sets the initial value, set_backward_mode() changes it.
-std::atomic<bool> g_planned{[] {
+enum Mode : int { kAtomic = 0, kPlanned = 1, kEager = 2 };
+std::atomic<int> g_mode{[] {
     const char *e = std::getenv("NUMML_AMD_BACKWARD");
-    return !(e && std::string(e) == "atomic");
+    const std::string v = e ? e : "";
+    return v == "atomic" ? (int)kAtomic : v == "eager" ? (int)kEager : (int)kPlanned;
 }()};
 
-bool planned_backward() { return g_planned.load(std::memory_order_relaxed); }
+int backward_mode_now() { return g_mode.load(std::memory_order_relaxed); }
 
 // ---- structure plans -----------------------------------------------------------
 //
-// Everything derived from a sparsity pattern alone is computed once and cached,
-// keyed on the storage and version counters of the structure tensors.  A plan
-// keeps those tensors alive, so an address cannot be reused by another pattern
-// while the plan is cached; in-place edits bump the version and miss the cache.
+// Everything derived from a sparsity pattern alone (the transposed structure, the level
+// schedule of a triangle, the filled pattern of LU factors) is computed once and cached under a
+// 128-bit key of the pattern's CONTENT (nm_structure_hash), so that a pattern arriving in fresh
+// tensors -- a clone, the product A @ B computed again -- finds its plans.  Computing the key
+// costs one pass over the structure and a wait for the stream, so it is done once per pair of
+// tensors: an alias table maps the identity of (indices, indptr) -- tensor objects, storage
+// addresses, version counters -- to the key it was given.  The table holds weak references
+// only: a tensor that has died cannot be mistaken for a new one at the same address, and no
+// caller memory is kept alive.  (An edit that goes around the version counter, such as a write
+// through `.data`, is not seen: the plan of the old pattern would be used.)
+//
+// The cache is bounded by the bytes of device memory its plans hold (NUMML_AMD_PLAN_CACHE_MB,
+// default 4096), least recently used first out.
+
+struct Key {
+    uint64_t h0 = 0, h1 = 0;
+    int64_t nnz = 0, nptr = 0;
+    int device = -1;
+    bool operator==(const Key &o) const {
+        return h0 == o.h0 && h1 == o.h1 && nnz == o.nnz && nptr == o.nptr && device == o.device;
+    }
+};
+
+using WeakImpl = c10::weak_intrusive_ptr<c10::TensorImpl, c10::UndefinedTensorImpl>;
+
+struct Alias {
+    const c10::TensorImpl *idx_impl, *ptr_impl;
+    WeakImpl idx_weak, ptr_weak;
+    const void *idx_ptr, *ptr_ptr;
+    uint32_t idx_version, ptr_version;
+    Key key;
+};
 
 struct Plan {
     char kind;  // 'T' transposed structure, 'L' level schedule, 'U' filled pattern of the LU factors
-    int device;
-    const void *idx_ptr, *ptr_ptr;
-    uint32_t idx_version, ptr_version;
-    int64_t nnz, nptr, a, b;
-    Tensor indices, indptr, mem;
+    Key key;
+    int64_t a, b;
+    Tensor mem;
+    size_t bytes = 0;
     std::vector<Tensor> derived;             // 'U': structure tensors handed out to callers
     std::vector<uint32_t> derived_versions;  //      and their version counters when built
     nm_sptrsv_plan *handle = nullptr;
+    // the stream the plan was built on and the event that marks its completion there
+    c10::StreamId build_stream = 0;
+    std::unique_ptr<at::cuda::CUDAEvent> ready;
     ~Plan() {
         if (handle) nm_sptrsv_plan_destroy(handle);
     }
 };
 
-constexpr size_t kPlanCacheSize = 16;
+struct Sighting {
+    char kind;
+    Key key;
+    int64_t a, b;
+};
+
+constexpr size_t kAliasTableSize = 64, kSightingTableSize = 256;
 std::mutex g_plans_mutex;
 std::list<std::shared_ptr<Plan>> g_plans;  // most recently used first
+std::list<Alias> g_aliases;                // most recently used first
+std::list<Sighting> g_sightings;
+size_t g_plan_bytes = 0;
+std::atomic<size_t> g_plan_bytes_limit{[] {
+    const char *e = std::getenv("NUMML_AMD_PLAN_CACHE_MB");
+    const long long mb = e ? std::atoll(e) : 4096;
+    return (size_t)(mb > 0 ? mb : 0) << 20;
+}()};
+std::atomic<int64_t> g_plans_built{0}, g_keys_computed{0};
 
-template <typename Make>
-std::shared_ptr<Plan> cached(char kind, const Tensor &indices, const Tensor &indptr, int64_t a, int64_t b,
-                             Make make) {
-    const int device = indices.device().index();
-    const uint32_t vi = indices._version(), vp = indptr._version();
+// 32 bytes of pinned host memory per host thread (from torch's pinned-memory allocator, which
+// also takes it back): where nm_spgemm_symbolic_result and nm_structure_hash have the device
+// drop their results.
+void *host_landing() {
+    thread_local Tensor landing =
+        torch::zeros({4}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+    return landing.data_ptr();
+}
+
+bool alias_matches(const Alias &al, const Tensor &indices, const Tensor &indptr) {
+    return al.idx_impl == indices.unsafeGetTensorImpl() && al.ptr_impl == indptr.unsafeGetTensorImpl() &&
+           al.idx_ptr == indices.data_ptr() && al.ptr_ptr == indptr.data_ptr() &&
+           al.idx_version == indices._version() && al.ptr_version == indptr._version() &&
+           al.key.nnz == indices.numel() && al.key.nptr == indptr.numel() &&
+           al.key.device == indices.device().index() && !al.idx_weak.expired() && !al.ptr_weak.expired();
+}
+
+// The content key of (indices, indptr): from the alias table, or computed (waits for the stream).
+// With `compute` false a pair of tensors that has not been seen yields false instead.
+bool structure_key(const Tensor &indices, const Tensor &indptr, bool compute, Key *out) {
     {
         std::lock_guard<std::mutex> lock(g_plans_mutex);
-        for (auto it = g_plans.begin(); it != g_plans.end(); ++it) {
-            Plan &p = **it;
-            if (p.kind == kind && p.device == device && p.idx_ptr == indices.data_ptr() &&
-                p.ptr_ptr == indptr.data_ptr() && p.idx_version == vi && p.ptr_version == vp &&
-                p.nnz == indices.numel() && p.nptr == indptr.numel() && p.a == a && p.b == b) {
-                auto hit = *it;
-                g_plans.erase(it);
-                g_plans.push_front(hit);
-                return hit;
+        for (auto it = g_aliases.begin(); it != g_aliases.end(); ++it) {
+            if (alias_matches(*it, indices, indptr)) {
+                *out = it->key;
+                if (it != g_aliases.begin()) g_aliases.splice(g_aliases.begin(), g_aliases, it);
+                return true;
+            }
+        }
+    }
+    if (!compute) return false;
+    const c10::Device dev = indices.device();
+    size_t bytes = 0;
+    check(nm_structure_hash_bytes(&bytes), "nm_structure_hash_bytes");
+    Tensor work = scratch(bytes, dev);
+    uint64_t h[2] = {0, 0};
+    check(nm_structure_hash(indices.numel(), indptr.numel(), indices.data_ptr<int64_t>(),
+                            indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, host_landing(), h,
+                            current_stream(dev)),
+          "nm_structure_hash");
+    g_keys_computed.fetch_add(1, std::memory_order_relaxed);
+    Alias al{indices.unsafeGetTensorImpl(),
+             indptr.unsafeGetTensorImpl(),
+             WeakImpl(indices.getIntrusivePtr()),
+             WeakImpl(indptr.getIntrusivePtr()),
+             indices.data_ptr(),
+             indptr.data_ptr(),
+             indices._version(),
+             indptr._version(),
+             Key{h[0], h[1], indices.numel(), indptr.numel(), dev.index()}};
+    *out = al.key;
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    // entries of tensors that have died, or that describe these very tensors at an older version
+    g_aliases.remove_if([&](const Alias &o) {
+        return o.idx_weak.expired() || o.ptr_weak.expired() ||
+               (o.idx_impl == al.idx_impl && o.ptr_impl == al.ptr_impl);
+    });
+    g_aliases.push_front(std::move(al));
+    while (g_aliases.size() > kAliasTableSize) g_aliases.pop_back();
+    return true;
+}
+
+// Makes `plan` usable on the current stream: work enqueued there from now on runs after the
+// build, and the allocator is told that this stream reads the plan's memory.
+void join_plan(const Plan &plan, const c10::Device &dev) {
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev.index());
+    if (!plan.ready || stream.id() == plan.build_stream) return;
+    plan.ready->block(stream);
+    if (plan.mem.defined())
+        c10::hip::HIPCachingAllocator::recordStream(plan.mem.storage().data_ptr(), stream.hip_stream());
+}
+
+std::shared_ptr<Plan> find_plan_locked(char kind, const Key &key, int64_t a, int64_t b) {
+    for (auto it = g_plans.begin(); it != g_plans.end(); ++it) {
+        Plan &p = **it;
+        if (p.kind == kind && p.key == key && p.a == a && p.b == b) {
+            if (it != g_plans.begin()) g_plans.splice(g_plans.begin(), g_plans, it);
+            return g_plans.front();
+        }
+    }
+    return nullptr;
+}
+
+// The cached plan of this kind for the pattern, or nullptr; never computes a key and never
+// builds (what a forward pass may look at without paying for anything).
+std::shared_ptr<Plan> peek_plan(char kind, const Tensor &indices, const Tensor &indptr, int64_t a, int64_t b,
+                                const c10::Device &dev) {
+    Key key;
+    if (!structure_key(indices, indptr, false, &key)) return nullptr;
+    std::shared_ptr<Plan> plan;
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        plan = find_plan_locked(kind, key, a, b);
+    }
+    if (plan) join_plan(*plan, dev);
+    return plan;
+}
+
+// The plan of this kind for the pattern.  `second_sighting`: a pattern seen for the first time
+// is only noted and nullptr is returned (the caller then runs its stateless kernels); the plan
+// is built when the pattern shows up again.
+template <typename Make>
+std::shared_ptr<Plan> cached(char kind, const Tensor &indices, const Tensor &indptr, int64_t a, int64_t b,
+                             bool second_sighting, const c10::Device &dev, Make make) {
+    Key key;
+    structure_key(indices, indptr, true, &key);
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        if (auto hit = find_plan_locked(kind, key, a, b)) {
+            join_plan(*hit, dev);
+            return hit;
+        }
+        if (second_sighting) {
+            bool seen = false;
+            for (auto it = g_sightings.begin(); it != g_sightings.end(); ++it)
+                if (it->kind == kind && it->key == key && it->a == a && it->b == b) {
+                    g_sightings.erase(it);
+                    seen = true;
+                    break;
+                }
+            if (!seen) {
+                g_sightings.push_front(Sighting{kind, key, a, b});
+                while (g_sightings.size() > kSightingTableSize) g_sightings.pop_back();
+                return nullptr;
             }
         }
     }
     auto plan = std::make_shared<Plan>();
     plan->kind = kind;
-    plan->device = device;
-    plan->idx_ptr = indices.data_ptr();
-    plan->ptr_ptr = indptr.data_ptr();
-    plan->idx_version = vi;
-    plan->ptr_version = vp;
-    plan->nnz = indices.numel();
-    plan->nptr = indptr.numel();
+    plan->key = key;
     plan->a = a;
     plan->b = b;
-    plan->indices = indices;
-    plan->indptr = indptr;
     make(*plan);
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev.index());
+    plan->build_stream = stream.id();
+    plan->ready = std::make_unique<at::cuda::CUDAEvent>();
+    plan->ready->record(stream);
+    plan->bytes = plan->mem.defined() ? (size_t)plan->mem.nbytes() : 0;
+    for (const Tensor &t : plan->derived) plan->bytes += (size_t)t.nbytes();
+    g_plans_built.fetch_add(1, std::memory_order_relaxed);
     std::lock_guard<std::mutex> lock(g_plans_mutex);
     g_plans.push_front(plan);
-    while (g_plans.size() > kPlanCacheSize) g_plans.pop_back();
+    g_plan_bytes += plan->bytes;
+    const size_t limit = g_plan_bytes_limit.load(std::memory_order_relaxed);
+    while (g_plans.size() > 1 && g_plan_bytes > limit) {
+        g_plan_bytes -= g_plans.back()->bytes;
+        g_plans.pop_back();
+    }
     return plan;
 }
 
+// `second_sighting` as above; csr_transpose_forward and the LU code need the plan at once.
 std::shared_ptr<Plan> transpose_plan(const Tensor &indices, const Tensor &indptr, int64_t rows, int64_t cols,
-                                     const c10::Device &dev) {
-    return cached('T', indices, indptr, rows, cols, [&](Plan &p) {
+                                     const c10::Device &dev, bool second_sighting = false) {
+    return cached('T', indices, indptr, rows, cols, second_sighting, dev, [&](Plan &p) {
+        const int64_t nnz = indices.numel();
         size_t pbytes = 0, wbytes = 0;
-        check(nm_csr_transpose_plan_bytes(rows, cols, p.nnz, &pbytes, &wbytes), "nm_csr_transpose_plan_bytes");
+        check(nm_csr_transpose_plan_bytes(rows, cols, nnz, &pbytes, &wbytes), "nm_csr_transpose_plan_bytes");
         p.mem = scratch(pbytes, dev);
         Tensor work = scratch(wbytes, dev);
-        auto stream = c10::hip::getCurrentHIPStream(dev.index());
-        check(nm_csr_transpose_plan_build(rows, cols, p.nnz, indices.data_ptr<int64_t>(),
+        // enqueued on the current stream, nothing waits: the plan's event orders other streams
+        // behind the build, and `work` goes back to the allocator, which hands it out again
+        // only to work enqueued later on this same stream
+        check(nm_csr_transpose_plan_build(rows, cols, nnz, indices.data_ptr<int64_t>(),
                                           indptr.data_ptr<int64_t>(), p.mem.data_ptr(), pbytes, work.data_ptr(),
-                                          wbytes, reinterpret_cast<nm_stream>(stream.stream())),
+                                          wbytes, current_stream(dev)),
               "nm_csr_transpose_plan_build");
-        // one-time: the plan is complete for every stream once this returns
-        stream.synchronize();
     });
+}
+
+// The transposed-structure plan a backward pass should use under the current mode, or nullptr
+// for the stateless kernels.
+std::shared_ptr<Plan> backward_plan(const Tensor &indices, const Tensor &indptr, int64_t rows, int64_t cols,
+                                    const c10::Device &dev) {
+    const int mode = backward_mode_now();
+    if (mode == kAtomic) return nullptr;
+    return transpose_plan(indices, indptr, rows, cols, dev, mode == kPlanned);
 }
 
 std::shared_ptr<Plan> level_plan(const Tensor &indices, const Tensor &indptr, int64_t rows, bool lower,
                                  const c10::Device &dev) {
-    return cached('L', indices, indptr, rows, lower ? 1 : 0, [&](Plan &p) {
+    return cached('L', indices, indptr, rows, lower ? 1 : 0, false, dev, [&](Plan &p) {
+        const int64_t nnz = indices.numel();
         size_t pbytes = 0, wbytes = 0;
-        check(nm_sptrsv_plan_bytes(rows, p.nnz, &pbytes, &wbytes), "nm_sptrsv_plan_bytes");
+        check(nm_sptrsv_plan_bytes(rows, nnz, &pbytes, &wbytes), "nm_sptrsv_plan_bytes");
         p.mem = scratch(pbytes, dev);
         Tensor work = scratch(wbytes, dev);
-        check(nm_sptrsv_analyse(rows, p.nnz, indices.data_ptr<int64_t>(), indptr.data_ptr<int64_t>(),
+        check(nm_sptrsv_analyse(rows, nnz, indices.data_ptr<int64_t>(), indptr.data_ptr<int64_t>(),
                                 lower ? 1 : 0, p.mem.data_ptr(), pbytes, work.data_ptr(), wbytes, &p.handle,
                                 current_stream(dev)),
               "nm_sptrsv_analyse");  // synchronises its stream
@@ -259,6 +429,14 @@ Tensor spgemv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_col_ind, T
     A_rowptr = index_tensor(A_rowptr, "A_rowptr");
     c10::hip::HIPGuard guard(dev.index());
     Tensor y = torch::empty({A_rows}, A_data.options());
+    // a pattern whose transposed-structure plan exists is read through the plan's 32-bit
+    // copies of the structure (half the index bytes); looking for it costs no device work
+    if (auto plan = peek_plan('T', A_col_ind, A_rowptr, A_rows, x.size(0), dev)) {
+        check(nm_spgemv_forward_planned(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
+                                        plan->mem.data_ptr(), x.data_ptr(), y.data_ptr(), current_stream(dev)),
+              "nm_spgemv_forward_planned");
+        return y;
+    }
     check(nm_spgemv_forward(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
                             A_col_ind.data_ptr<int64_t>(), A_rowptr.data_ptr<int64_t>(), x.data_ptr(),
                             y.data_ptr(), current_stream(dev)),
@@ -281,8 +459,7 @@ std::vector<Tensor> spgemv_backward(Tensor grad_z, int A_rows, int A_cols, Tenso
     A_rowptr = index_tensor(A_rowptr, "A_rowptr");
     c10::hip::HIPGuard guard(dev.index());
     Tensor grad_A = torch::empty_like(A_data), grad_x = torch::empty_like(x);
-    if (planned_backward()) {
-        auto plan = transpose_plan(A_col_ind, A_rowptr, A_rows, x.size(0), dev);
+    if (auto plan = backward_plan(A_col_ind, A_rowptr, A_rows, x.size(0), dev)) {
         check(nm_spgemv_backward_planned(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
                                          plan->mem.data_ptr(), x.data_ptr(), grad_z.data_ptr(),
                                          grad_A.data_ptr(), grad_x.data_ptr(), current_stream(dev)),
@@ -555,8 +732,7 @@ std::vector<Tensor> spdmm_backward(int A_rows, int A_cols, Tensor A_data, Tensor
     c10::hip::HIPGuard guard(dev.index());
     Tensor grad_A = torch::empty_like(A_data);
     Tensor grad_B = torch::empty({B.size(0), n}, B.options());
-    if (planned_backward()) {
-        auto plan = transpose_plan(A_indices, A_indptr, A_rows, B.size(0), dev);
+    if (auto plan = backward_plan(A_indices, A_indptr, A_rows, B.size(0), dev)) {
         check(nm_spdmm_backward_planned(dtype_of(A_data), A_rows, B.size(0), A_data.numel(), A_data.data_ptr(),
                                         A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
                                         plan->mem.data_ptr(), B.data_ptr(), ldb, grad_C.data_ptr(), ldg, n,
@@ -699,7 +875,7 @@ std::vector<Tensor> sptrsv_backward(Tensor grad_x, Tensor x, int A_rows, int A_c
 std::shared_ptr<Plan> lu_pattern(const Tensor &A_indices, const Tensor &A_indptr, int64_t rows,
                                  const c10::Device &dev) {
     for (int attempt = 0;; ++attempt) {
-        auto plan = cached('U', A_indices, A_indptr, rows, rows, [&](Plan &p) {
+        auto plan = cached('U', A_indices, A_indptr, rows, rows, false, dev, [&](Plan &p) {
             const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
             const nm_stream stream = current_stream(dev);
             size_t bytes = 0;
@@ -729,7 +905,6 @@ std::shared_ptr<Plan> lu_pattern(const Tensor &A_indices, const Tensor &A_indptr
                   "nm_csr_transpose_forward");
             p.derived = {M_indices, M_indptr, Mt_indices, Mt_indptr, Mt_to_M};
             for (const Tensor &t : p.derived) p.derived_versions.push_back(t._version());
-            c10::hip::getCurrentHIPStream(dev.index()).synchronize();   // complete for every stream
         });
         bool intact = true;   // a caller may have edited the tensors it was handed
         for (size_t i = 0; i < plan->derived.size(); ++i)
@@ -739,7 +914,9 @@ std::shared_ptr<Plan> lu_pattern(const Tensor &A_indices, const Tensor &A_indptr
             return plan;
         }
         std::lock_guard<std::mutex> lock(g_plans_mutex);
+        const size_t before = g_plans.size();
         g_plans.remove(plan);
+        if (g_plans.size() != before) g_plan_bytes -= plan->bytes;
     }
 }
 
@@ -839,6 +1016,9 @@ std::tuple<int64_t, int64_t> sptrsv_schedule(int A_rows, Tensor A_indices, Tenso
 void clear_plan_cache() {
     std::lock_guard<std::mutex> lock(g_plans_mutex);
     g_plans.clear();
+    g_aliases.clear();
+    g_sightings.clear();
+    g_plan_bytes = 0;
 }
 
 int64_t plan_cache_size() {
@@ -846,13 +1026,31 @@ int64_t plan_cache_size() {
     return (int64_t)g_plans.size();
 }
 
-void set_backward_mode(const std::string &mode) {
-    TORCH_CHECK(mode == "planned" || mode == "atomic", "backward mode must be 'planned' or 'atomic', got '", mode,
-                "'");
-    g_planned.store(mode == "planned", std::memory_order_relaxed);
+int64_t plan_cache_bytes() {
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    return (int64_t)g_plan_bytes;
 }
 
-std::string backward_mode() { return planned_backward() ? "planned" : "atomic"; }
+void set_plan_cache_limit(int64_t bytes) {
+    TORCH_CHECK(bytes >= 0, "the plan cache limit must not be negative");
+    g_plan_bytes_limit.store((size_t)bytes, std::memory_order_relaxed);
+}
+
+// (plans built, structure keys computed) since the module was loaded
+std::tuple<int64_t, int64_t> plan_cache_stats() {
+    return {g_plans_built.load(std::memory_order_relaxed), g_keys_computed.load(std::memory_order_relaxed)};
+}
+
+void set_backward_mode(const std::string &mode) {
+    TORCH_CHECK(mode == "planned" || mode == "eager" || mode == "atomic",
+                "backward mode must be 'planned', 'eager' or 'atomic', got '", mode, "'");
+    g_mode.store(mode == "atomic" ? kAtomic : mode == "eager" ? kEager : kPlanned, std::memory_order_relaxed);
+}
+
+std::string backward_mode() {
+    const int m = backward_mode_now();
+    return m == kAtomic ? "atomic" : m == kEager ? "eager" : "planned";
+}
 
 }  // namespace
 
@@ -881,6 +1079,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sptrsv_schedule", &sptrsv_schedule, "(levels, launches per solve) of a triangular pattern");
     m.def("clear_plan_cache", &clear_plan_cache, "Drop every cached structure plan");
     m.def("plan_cache_size", &plan_cache_size, "Number of cached structure plans");
-    m.def("set_backward_mode", &set_backward_mode, "'planned' (cached transposed structure) or 'atomic'");
+    m.def("plan_cache_bytes", &plan_cache_bytes, "Device memory held by the cached structure plans");
+    m.def("set_plan_cache_limit", &set_plan_cache_limit, "Bound of plan_cache_bytes (least recently used plans go first)");
+    m.def("plan_cache_stats", &plan_cache_stats, "(plans built, structure keys computed) since the module was loaded");
+    m.def("set_backward_mode", &set_backward_mode,
+          "'planned' (cached transposed structure from the second sighting of a pattern), 'eager' (from the first) "
+          "or 'atomic' (never)");
     m.def("backward_mode", &backward_mode, "Current backward mode");
 }

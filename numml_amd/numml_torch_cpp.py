@@ -115,17 +115,18 @@ def _square(who, rows, cols):
 
 # ------------------------------------------------------------ structure plans
 #
-# Everything derived from a sparsity pattern alone (the transposed structure, the
-# level schedule of a triangle) is computed once and cached.  A plan is keyed on
-# the storage and version counters of the structure tensors, and it keeps those
-# tensors alive, so an address cannot be reused by a different pattern while its
-# plan is cached; in-place edits bump the version and miss the cache.
+# This module is the thin way to the C ABI (tests call the library through it); the plan
+# POLICY of the package -- content keys, building a plan at the second sighting of a pattern,
+# the byte-bounded cache -- lives in one place only, the compiled binding
+# (csrc/torch_binding.cpp).  Here a plan is built the first time a pair of structure tensors is
+# seen and kept under their identity (storage address and version counter; the plan keeps the
+# tensors alive so that the address cannot be reused), at most _PLAN_CACHE_SIZE of them.
 
 _PLAN_CACHE_SIZE = 16
 _plans = collections.OrderedDict()
 _plans_lock = threading.Lock()
 
-# "planned": backward passes walk A by column on a cached transposed structure
+# "planned" / "eager": backward passes walk A by column on a transposed-structure plan
 #            (deterministic, no atomics);  "atomic": stateless scatter with atomics.
 BACKWARD_MODE = os.environ.get("NUMML_AMD_BACKWARD", "planned")
 
@@ -213,7 +214,7 @@ def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_x = torch.empty_like(x)
-        if BACKWARD_MODE == "planned":
+        if BACKWARD_MODE != "atomic":
             plan = _transpose_plan(A_col_ind, A_rowptr, A_rows, x.shape[0], dev)
             _lib.check(_lib.lib().nm_spgemv_backward_planned(
                 _dt(A_data), A_rows, x.shape[0], A_data.shape[0], _ptr(A_data), _ptr(plan.mem), _ptr(x),
@@ -443,7 +444,7 @@ def spdmm_backward(A_rows, A_cols, A_data, A_indices, A_indptr, B, grad_C):
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_B = torch.empty((B.shape[0], n), dtype=B.dtype, device=dev)
-        if BACKWARD_MODE == "planned":
+        if BACKWARD_MODE != "atomic":
             plan = _transpose_plan(A_indices, A_indptr, A_rows, B.shape[0], dev)
             _lib.check(_lib.lib().nm_spdmm_backward_planned(
                 _dt(A_data), A_rows, B.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_indices),

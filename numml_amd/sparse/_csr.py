@@ -275,8 +275,9 @@ class SparseCSRTensor(object):
         C_shape, C_data, C_indices, C_indptr = spgemm.apply(
             self.shape, self.data, self.indices, self.indptr,
             othr.shape, othr.data, othr.indices, othr.indptr)
-        # the reference re-wraps with clone=True, a differentiable copy (numml/sparse/_csr.py:685)
-        return SparseCSRTensor((C_data, C_indices, C_indptr), C_shape)
+        # The reference re-wraps with clone=True (numml/sparse/_csr.py:685); the three tensors are
+        # fresh outputs of the product, so they are adopted as they are (no copy of C).
+        return SparseCSRTensor((C_data, C_indices, C_indptr), C_shape, clone=False)
 
     def solve_triangular(self, upper, unit, b):
         from . import linalg
@@ -312,12 +313,12 @@ class SparseCSRTensor(object):
         """A^T, computed eagerly as a new CSR matrix (numml/sparse/_csr.py:1074-1087)."""
         At_shape, At_data, At_indices, At_indptr = sptranspose.apply(
             self.shape, self.data, self.indices, self.indptr)
-        return SparseCSRTensor((At_data, At_indices, At_indptr), At_shape)
+        return SparseCSRTensor((At_data, At_indices, At_indptr), At_shape, clone=False)
 
     def hermitian(self):
         At_shape, At_data, At_indices, At_indptr = sptranspose.apply(
             self.shape, self.data.conj(), self.indices, self.indptr)
-        return SparseCSRTensor((At_data, At_indices, At_indptr), At_shape)
+        return SparseCSRTensor((At_data, At_indices, At_indptr), At_shape, clone=False)
 
     @property
     def T(self):
@@ -338,11 +339,11 @@ class SparseCSRTensor(object):
                                f"{othr.shape}, respectively.")
         C = splincomb.apply(self.shape, torch.tensor(1.), self.data, self.indices, self.indptr,
                             torch.tensor(beta), othr.data, othr.indices, othr.indptr)
-        return SparseCSRTensor(C, self.shape)
+        return SparseCSRTensor(C, self.shape, clone=False)
 
     def __add__(self, othr):
         if SparseCSRTensor._isscalar(othr):
-            return SparseCSRTensor((self.data + othr, self.indices, self.indptr), self.shape)
+            return SparseCSRTensor((self.data + othr, self.indices, self.indptr), self.shape, clone=False)
         if isinstance(othr, SparseCSRTensor):
             return self._lincomb(othr, 1., "addition")
         raise RuntimeError(f"Unknown type for sparse tensor addition: {type(othr)}.")
@@ -350,14 +351,14 @@ class SparseCSRTensor(object):
     def __sub__(self, othr):
         if SparseCSRTensor._isscalar(othr):
             # the reference adds the scalar here as well (numml/sparse/_csr.py:898-899)
-            return SparseCSRTensor((self.data + othr, self.indices, self.indptr), self.shape)
+            return SparseCSRTensor((self.data + othr, self.indices, self.indptr), self.shape, clone=False)
         if isinstance(othr, SparseCSRTensor):
             return self._lincomb(othr, -1., "subtraction")
         raise RuntimeError(f"Unknown type for sparse tensor addition: {type(othr)}.")
 
     def __mul__(self, s):
         if SparseCSRTensor._isscalar(s):
-            return SparseCSRTensor((self.data * s, self.indices, self.indptr), self.shape)
+            return SparseCSRTensor((self.data * s, self.indices, self.indptr), self.shape, clone=False)
         if isinstance(s, torch.Tensor) and len(torch.squeeze(s).shape) == 2:
             raise RuntimeError("Element-wise hadamard product not implemented")
         raise RuntimeError(f"Unknown type for multiplication: {type(s)}.")
@@ -366,17 +367,17 @@ class SparseCSRTensor(object):
 
     def __rtruediv__(self, other):
         if SparseCSRTensor._isscalar(other):
-            return SparseCSRTensor((other / self.data, self.indices, self.indptr), self.shape)
+            return SparseCSRTensor((other / self.data, self.indices, self.indptr), self.shape, clone=False)
         raise RuntimeError(f"Unknown type for right-division: {type(other)}.")
 
     def __neg__(self):
-        return SparseCSRTensor((-self.data, self.indices, self.indptr), self.shape)
+        return SparseCSRTensor((-self.data, self.indices, self.indptr), self.shape, clone=False)
 
     def __pow__(self, p):
-        return SparseCSRTensor((self.data ** p, self.indices, self.indptr), self.shape)
+        return SparseCSRTensor((self.data ** p, self.indices, self.indptr), self.shape, clone=False)
 
     def abs(self):
-        return SparseCSRTensor((torch.abs(self.data), self.indices, self.indptr), self.shape)
+        return SparseCSRTensor((torch.abs(self.data), self.indices, self.indptr), self.shape, clone=False)
 
     __abs__ = abs
 
@@ -457,7 +458,7 @@ class SparseCSRTensor(object):
 
     def conjugate(self):
         """Element-wise complex conjugation (numml/sparse/_csr.py:1041-1061)."""
-        return SparseCSRTensor((self.data.conj(), self.indices, self.indptr), self.shape)
+        return SparseCSRTensor((torch.clone(self.data.conj()), self.indices, self.indptr), self.shape, clone=False)
 
     conj = conjugate
 
@@ -501,7 +502,7 @@ class SparseCSRTensor(object):
 
     @property
     def grad(self):
-        return SparseCSRTensor((self.data.grad, self.indices, self.indptr), self.shape)
+        return SparseCSRTensor((self.data.grad, self.indices, self.indptr), self.shape, clone=False)
 
     @property
     def grad_fn(self):

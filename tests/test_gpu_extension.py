@@ -25,7 +25,7 @@ def cpp():
     return numml_amd.load_compiled()
 
 
-@pytest.fixture(params=["planned", "atomic"])
+@pytest.fixture(params=["eager", "atomic"])
 def mode(request, cpp):
     old_cpp, old_mirror = cpp.backward_mode(), mirror.BACKWARD_MODE
     cpp.set_backward_mode(request.param)
@@ -56,7 +56,7 @@ def test_spgemv(dev, cpp, dtype, mode):
         assert_close(host(gx), gx_ref, "grad_x")
         mA, mx = mirror.spgemv_backward(Gz, rows, cols, D, I, P, X)
         assert_same(host(gA), host(mA), "grad_A vs ctypes binding")
-        if mode == "planned":
+        if mode == "eager":
             assert_same(host(gx), host(mx), "grad_x vs ctypes binding")
 
 
@@ -75,7 +75,7 @@ def test_spdmm(dev, cpp, dtype, n, mode):
     assert_close(host(gB), gB_ref, "grad_B")
     mA, mB = mirror.spdmm_backward(rows, cols, D, I, P, Bt, Gt)
     assert_same(host(gA), host(mA), "grad_A vs ctypes binding")
-    if mode == "planned":
+    if mode == "eager":
         assert_same(host(gB), host(mB), "grad_B vs ctypes binding")
     # a column-major B and a row-sliced grad_C take the strided/copy paths
     Bf = Bt.t().contiguous().t()
@@ -83,7 +83,7 @@ def test_spdmm(dev, cpp, dtype, n, mode):
     assert_same(host(cpp.spdmm_forward(rows, cols, D, I, P, Bf)), host(C), "C from column-major B")
     sA, sB = cpp.spdmm_backward(rows, cols, D, I, P, Bf, Gs)
     assert_same(host(sA), host(gA), "grad_A from strided operands")
-    if mode == "planned":
+    if mode == "eager":
         assert_same(host(sB), host(gB), "grad_B from strided operands")
 
 
@@ -135,7 +135,7 @@ def test_plan_cache_and_errors(dev, cpp):
     assert cpp.plan_cache_size() == 1
     cpp.sptrsv_backward(b, b, n, n, D, I, P, True, False, b)        # the transposed solve shares the plan
     assert cpp.plan_cache_size() == 1
-    cpp.set_backward_mode("planned")
+    cpp.set_backward_mode("eager")
     cpp.spgemv_backward(b, n, n, D, I, P, b)
     assert cpp.plan_cache_size() == 2
     # an in-place edit of the structure must not reuse the stale schedule
@@ -157,6 +157,79 @@ def test_plan_cache_and_errors(dev, cpp):
         cpp.spgemv_forward(n, n, D.half(), I, P, b.half())
     with pytest.raises(RuntimeError, match="planned"):
         cpp.set_backward_mode("fastest")
+
+
+def test_plan_policy_second_sighting_content_key_and_byte_bound(dev, cpp):
+    """Default mode: the first backward on a new pattern runs statelessly and builds nothing, the
+    second builds the plan; the plan is found again through fresh tensors with the same content;
+    the cache is bounded by bytes."""
+    d, i, p, (rows, cols) = G.poisson2d(96, np.float64, 3)
+    D, I, P = to_dev(dev, d, i, p)
+    x, g = randn(4, cols, np.float64), randn(5, rows, np.float64)
+    X, Gv = to_dev(dev, x, g)
+    gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+    cpp.clear_plan_cache()
+    cpp.set_backward_mode("planned")
+    built0, keys0 = cpp.plan_cache_stats()
+    gA, gx = cpp.spgemv_backward(Gv, rows, cols, D, I, P, X)             # first sighting: stateless
+    assert cpp.plan_cache_size() == 0 and cpp.plan_cache_stats()[0] == built0
+    assert_same(host(gA), gA_ref, "grad_A (stateless)")
+    assert_close(host(gx), gx_ref, "grad_x (stateless)")
+    gA, gx = cpp.spgemv_backward(Gv, rows, cols, D, I, P, X)             # second sighting: plan built
+    assert cpp.plan_cache_size() == 1 and cpp.plan_cache_stats()[0] == built0 + 1
+    assert_same(host(gx), gx_ref, "grad_x (planned, bitwise)")
+    assert cpp.plan_cache_stats()[1] == keys0 + 1                         # one key for the one pair of tensors
+    y_plain = oracle.spgemv_forward(rows, cols, d, i, p, x)
+    assert_same(host(cpp.spgemv_forward(rows, cols, D, I, P, X)), y_plain, "y through the plan's 32-bit structure")
+    # the same pattern in fresh tensors: a key is computed, the plan is found, nothing is built
+    I2, P2 = I.clone(), P.clone()
+    gA, gx = cpp.spgemv_backward(Gv, rows, cols, D, I2, P2, X)
+    assert cpp.plan_cache_size() == 1 and cpp.plan_cache_stats() == (built0 + 1, keys0 + 2)
+    assert_same(host(gx), gx_ref, "grad_x (plan found through the content key)")
+    # a different pattern of the same sizes is not mistaken for it
+    I3 = I.clone()
+    I3[2] = I[2].item() + 1                      # row 0 holds columns (0, 1, 96): the last one moves to 97
+    cpp.spgemv_backward(Gv, rows, cols, D, I3, P, X)
+    assert cpp.plan_cache_size() == 1 and cpp.plan_cache_stats()[0] == built0 + 1   # first sighting of another pattern
+    # byte bound: with a limit below one plan only the most recent plan stays
+    one = cpp.plan_cache_bytes()
+    assert one > 0
+    cpp.set_plan_cache_limit(one // 2)
+    cpp.set_backward_mode("eager")
+    d4, i4, p4, (r4, c4) = G.poisson2d(64, np.float64, 1)
+    D4, I4, P4 = to_dev(dev, d4, i4, p4)
+    cpp.spgemv_backward(to_dev(dev, randn(1, r4, np.float64))[0], r4, c4, D4, I4, P4, to_dev(dev, randn(2, c4, np.float64))[0])
+    assert cpp.plan_cache_size() == 1 and cpp.plan_cache_bytes() < one
+    cpp.set_plan_cache_limit(4096 << 20)
+    cpp.clear_plan_cache()
+
+
+def test_loop_of_fresh_products_builds_one_plan_per_pattern(dev, cpp):
+    """C = A @ A computed anew in every iteration arrives in new structure tensors each time; the
+    backward of C @ x must find C's plan again instead of building one per iteration."""
+    import time
+    from numml_amd import sparse as sp
+    d, i, p, (rows, cols) = G.poisson2d(256, np.float32, 0)
+    D, I, P = to_dev(dev, d, i, p)
+    A = sp.SparseCSRTensor((D, I, P), (rows, cols), clone=False)
+    A.requires_grad = True
+    X = to_dev(dev, randn(1, cols, np.float32))[0]
+    cpp.clear_plan_cache()
+    cpp.set_backward_mode("planned")
+    built0 = cpp.plan_cache_stats()[0]
+    times = []
+    for it in range(10):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        C = A @ A
+        (C @ X).sum().backward()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    # C's pattern for the SpMV backward, and at most A's own for the product's backward
+    assert cpp.plan_cache_stats()[0] - built0 <= 2 and cpp.plan_cache_size() <= 2
+    steady = sorted(times[3:])[len(times[3:]) // 2]
+    assert max(times[3:]) <= 2.0 * steady, times
+    cpp.clear_plan_cache()
 
 
 def test_install_registers_the_reference_module_name(cpp):

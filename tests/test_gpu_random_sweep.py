@@ -195,12 +195,12 @@ def test_many_workgroups(dev, seed, dtype):
     X, Gv = to_dev(dev, x, g)
     assert_close(host(ext.spgemv_forward(rows, cols, D, I, P, X)), oracle.spgemv_forward(rows, cols, d, i, p, x), "y")
     gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
-    for mode in ("planned", "atomic"):
+    for mode in ("eager", "atomic"):
         ext.set_backward_mode(mode)
         try:
             gA, gx = ext.spgemv_backward(Gv, rows, cols, D, I, P, X)
         finally:
-            ext.set_backward_mode("planned")
+            ext.set_backward_mode("eager")
         assert_same(host(gA), gA_ref, f"spmv grad_A ({mode})")
         assert_close(host(gx), gx_ref, f"spmv grad_x ({mode})")
     n = (4, 16, 33, 64, 7, 100)[seed % 6]

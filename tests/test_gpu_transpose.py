@@ -18,6 +18,32 @@ from util import assert_close, assert_same, host, randn, to_dev
 pytestmark = pytest.mark.gpu
 
 
+def _with_dense_columns(dtype):
+    """30 000 rows; column 7 is stored in every row and column 400 in two rows of three (columns far
+    longer than what the ordering kernel keeps in LDS, so their pieces are merged through memory),
+    the rest random."""
+    rows, cols = 30_000, 900
+    rng = np.random.default_rng(11)
+    r = np.concatenate([np.arange(rows), np.arange(rows)[np.arange(rows) % 3 != 0],
+                        rng.integers(0, rows, 40_000)])
+    c = np.concatenate([np.full(rows, 7), np.full(int((np.arange(rows) % 3 != 0).sum()), 400),
+                        rng.integers(0, cols, 40_000)])
+    rc = np.unique(np.stack([r, c], 1), axis=0)            # sorted by row, then column; no duplicates
+    indptr = np.zeros(rows + 1, np.int64)
+    np.cumsum(np.bincount(rc[:, 0], minlength=rows), out=indptr[1:])
+    data = rng.standard_normal(rc.shape[0]).astype(dtype)
+    return data, rc[:, 1].astype(np.int64), indptr, (rows, cols)
+
+
+def _with_duplicates(dtype):
+    """Stored entries with equal coordinates (the container keeps them, numml/sparse/_csr.py:78-99):
+    the transpose must keep their storage order."""
+    indptr = np.array([0, 3, 3, 7, 9], np.int64)
+    indices = np.array([1, 1, 4, 0, 2, 2, 2, 1, 1], np.int64)
+    data = np.arange(1, 10).astype(dtype)
+    return data, indices, indptr, (4, 5)
+
+
 def _cases(dtype):
     yield "tridiag16", G.tridiag(16, dtype)
     yield "poisson40", G.poisson2d(40, dtype, 1)
@@ -25,6 +51,8 @@ def _cases(dtype):
     yield "rect_tall", G.random_csr(300, 19, 0.2, 2, dtype)
     yield "empty_rows_cols", G.random_csr(120, 130, 0.01, 3, dtype)
     yield "powerlaw", G.powerlaw(3000, 2500, 40000, max_deg=1200, seed=4, dtype=dtype)
+    yield "dense_columns", _with_dense_columns(dtype)
+    yield "duplicates", _with_duplicates(dtype)
     yield "no_entries", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(6, np.int64), (5, 7))
     yield "one", (np.ones(1, dtype), np.zeros(1, np.int64), np.array([0, 1], np.int64), (1, 1))
 
