@@ -223,6 +223,23 @@ int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz
                        const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
                        void *grad_A, void *grad_B, nm_stream stream);
 
+/* nm_spgemm_backward on the transposed-structure plan of A's pattern
+ * (nm_csr_transpose_plan_build with A's rows, columns and entries): work is
+ * shared out by row of B, the entries of A that meet a row come from the plan
+ * in ascending row order, and both gradients are summed in registers in the
+ * order of the reference's loops (cpp/sparse_csr_cpu.cpp:261-274 ascending
+ * column for grad_A, :291-303 ascending row for grad_B): no atomics, no
+ * clearing, identical on every run and bit-identical to the CPU result, except
+ * for rows of B whose (row length) x (length of A's column) exceeds 4096: those
+ * get a whole workgroup and grad_B is added across its lanes in tree order,
+ * which differs by rounding only.  Either output may be NULL. */
+int nm_spgemm_backward_planned(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t A_nnz,
+                               int64_t B_nnz, int64_t C_nnz,
+                               const void *gC, const int64_t *C_indices, const int64_t *C_indptr,
+                               const void *A_data, const void *A_plan_mem,
+                               const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
+                               void *grad_A, void *grad_B, nm_stream stream);
+
 /* ---------------------------------------------------------------- SpTRSV
  * Level-scheduled triangular solve.  Stands in for sptrsv_forward /
  * sptrsv_backward (cpp/sparse_csr.hpp:94-105, cpp/sparse_csr_cpu.cpp:652-759).

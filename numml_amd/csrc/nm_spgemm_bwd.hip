@@ -12,16 +12,19 @@
 //
 //   grad_B[k, c_j] += A[i, k] * g_j      accumulates in lane j's register: products
 //                                        arrive with i ascending, the order of :291-303;
-//   grad_A[i, k]    = sum_j g_j * B[k, c_j]  is added across the lanes in lane order =
+//   grad_A[i, k]    = sum_j g_j * B[k, c_j]  the terms of the batch's entries change places
+//                                        through LDS so that lane e holds the eight terms
+//                                        of entry e, and adds them in lane order =
 //                                        ascending c, the order of the merge in :261-274
-//                                        (lanes without a hit add +0.0, which changes
-//                                        nothing).
+//                                        (a column C does not store adds +0.0, which
+//                                        changes nothing).
 //
 // Every stored entry of A lies in exactly one column and every entry of B in
 // exactly one row, so each gradient entry is written once, by one lane.
 //
 // Rows of B with more than 8 entries take several passes over the column of A
-// (grad_A is then completed pass by pass); rows whose work is far beyond a group's
+// (a pass continues grad_A's sum where the pass before it stopped, so the order
+// stays the serial one); rows whose work is far beyond a group's
 // (long row of B times long column of A) are left to a second kernel that gives a
 // whole workgroup to the row and adds across lanes in tree order (equal to the
 // serial order up to rounding).
@@ -36,6 +39,7 @@ constexpr int kBlock = 256;
 constexpr int G = 8;                 // lanes per row of B
 constexpr int kGroups = kBlock / G;  // rows of B per workgroup pass
 constexpr int kStage = 256;          // staged column indices of C per group
+constexpr int kFast = 32;            // rows of C up to this long: 8 of them staged side by side
 // a row of B is "heavy" when (entries of the row) x (entries of A's column) exceeds this:
 // 64 passes of a group
 constexpr int64_t kHeavy = 64 * G * G;
@@ -44,20 +48,6 @@ __device__ __forceinline__ void group_fence() { __builtin_amdgcn_fence(__ATOMIC_
 
 template <typename T> __device__ __forceinline__ T shfl_t(T v, int src) { return __shfl(v, src, kWave); }
 
-// Sum over the 8 lanes of a group in lane order: lane 7 of the group ends up with
-// ((v0 + v1) + v2) + ... + v7.  row_shr:1 hands every lane its left neighbour's running sum
-// (lane 0 of a group takes nothing: the neighbour belongs to another group).
-template <typename T>
-__device__ __forceinline__ T ordered_group_sum(T v, int gl) {
-    T run = v;
-#pragma unroll
-    for (int s = 1; s < G; ++s) {
-        const T left = nm::dpp_move_zero<0x111>(run);   // row_shr:1
-        if (gl == s) run = left + v;
-    }
-    return run;
-}
-
 template <typename T>
 __global__ __launch_bounds__(kBlock) void spgemm_bwd_planned_kernel(
     int64_t B_rows, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
@@ -65,10 +55,14 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_planned_kernel(
     const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm, const T *__restrict__ B_data,
     const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr, T *__restrict__ grad_A,
     T *__restrict__ grad_B) {
-    __shared__ int32_t s_c[kGroups * kStage];
+    __shared__ __align__(16) int32_t s_c[kGroups * kStage];
+    __shared__ int4 s_rec[kGroups * G];
+    __shared__ T s_a[kGroups * G];
     const int gl = threadIdx.x % G, gi = threadIdx.x / G;
     const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);   // first lane of the group in its wavefront
     int32_t *st = s_c + gi * kStage;
+    int4 *rec = s_rec + gi * G;
+    T *ra = s_a + gi * G;
     const int64_t npass = nm::ceil_div(B_rows, (int64_t)kGroups), npad = nm::xcd_padded(npass);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t pass = nm::xcd_tile(id, npad);
@@ -103,53 +97,159 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_planned_kernel(
                 int mx = clen;
 #pragma unroll
                 for (int off = 1; off < G; off <<= 1) mx = max(mx, __shfl_xor(mx, off, kWave));
-                int slot = 32;
-                while (slot < mx && slot < kStage) slot <<= 1;
-                const int per = kStage / slot;        // 8, 4, 2 or 1 rows at a time
+                int slot = 32, sh = 5;
+                while (slot < mx && slot < kStage) slot <<= 1, ++sh;
+                const int per = kStage >> sh;         // 8, 4, 2 or 1 rows at a time
                 T totalA = 0;                         // lane e keeps the sum of entry e of the batch
+                // a later pass over a long row of B goes on from what the passes before it left
+                const T prevA = (mine && grad_A && jb != bb) ? grad_A[apos] : T(0);
+                if (mx <= kFast) {
+                    // The common case: every row of C of the batch has at most 32 entries.
+                    // (start, length, A's value) of the 8 rows change hands through LDS once, so that
+                    // nothing below needs a cross-lane move.
+                    group_fence();
+                    rec[gl] = make_int4((int)(cb & 0xffffffffll), (int)(cb >> 32), clen, 0);
+                    ra[gl] = a;
+                    group_fence();
+                    int64_t cbs[G];
+                    int lens[G];
+#pragma unroll
+                    for (int e8 = 0; e8 < G; ++e8) {
+                        const int4 r = rec[e8];
+                        cbs[e8] = ((int64_t)r.y << 32) | (uint32_t)r.x;
+                        lens[e8] = r.z;
+                    }
+                    // stage the column indices, 32 slots per row, unused slots = +infinity: 16 loads
+                    // in flight per lane, twice
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        int32_t got[16];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+#pragma unroll
+                            for (int ch = 0; ch < 4; ++ch) {
+                                const int e8 = half * 4 + r, t = ch * G + gl;
+                                const bool ok = t < lens[e8];
+                                const int32_t v = (int32_t) * (ok ? C_indices + cbs[e8] + t : B_indptr);
+                                got[r * 4 + ch] = ok ? v : 0x7fffffff;
+                            }
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+#pragma unroll
+                            for (int ch = 0; ch < 4; ++ch) st[(half * 4 + r) * kFast + ch * G + gl] = got[r * 4 + ch];
+                    }
+                    group_fence();
+                    // the column's place in each row: five halving steps without a branch, all rows at once
+                    int pos[G];
+#pragma unroll
+                    for (int e8 = 0; e8 < G; ++e8) pos[e8] = 0;
+#pragma unroll
+                    for (int step = kFast / 2; step > 0; step >>= 1)
+#pragma unroll
+                        for (int e8 = 0; e8 < G; ++e8)
+                            if (st[e8 * kFast + pos[e8] + step - 1] < c) pos[e8] += step;
+                    unsigned hits = 0;
+#pragma unroll
+                    for (int e8 = 0; e8 < G; ++e8) hits |= (have && st[e8 * kFast + pos[e8]] == c ? 1u : 0u) << e8;
+                    T g[G];
+#pragma unroll
+                    for (int e8 = 0; e8 < G; ++e8) g[e8] = gC[(hits >> e8) & 1u ? cbs[e8] + pos[e8] : 0];
+                    group_fence();
+                    T *tr = reinterpret_cast<T *>(st);
+#pragma unroll
+                    for (int e8 = 0; e8 < G; ++e8) {
+                        const bool hit = (hits >> e8) & 1u;
+                        accB += hit ? ra[e8] * g[e8] : T(0);
+                        tr[e8 * G + gl] = hit ? g[e8] * bval : T(0);
+                    }
+                    group_fence();
+                    T run = prevA;
+#pragma unroll
+                    for (int j = 0; j < G; ++j) run += tr[gl * G + j];
+                    totalA = run;
+                } else
                 for (int e0 = 0; e0 < nb; e0 += per) {
-                    const int e1 = e0 + per < nb ? e0 + per : nb;
+                    const int ne = nb - e0 < per ? nb - e0 : per;   // rows of C of this sub-batch
+                    // 1. stage their column indices, slot entries apart: 8 consecutive entries of one
+                    //    row per group instruction, 8 such loads in flight per lane (unconditional on a
+                    //    clamped position, stored afterwards)
                     group_fence();
-                    for (int e = e0; e < e1; ++e) {
-                        const int64_t cbe = shfl_t(cb, gbase + e);
-                        const int len = shfl_t(clen, gbase + e);
-                        if (len <= kStage)
-                            for (int t = gl; t < len; t += G) st[(e - e0) * slot + t] = (int32_t)C_indices[cbe + t];
-                    }
-                    group_fence();
-                    for (int e = e0; e < e1; ++e) {
-                        const int64_t cbe = shfl_t(cb, gbase + e);
-                        const int len = shfl_t(clen, gbase + e);
-                        const T ae = shfl_t(a, gbase + e);
-                        int l = 0, h = len;
-                        bool hit;
-                        if (len <= kStage) {
-                            const int32_t *row = st + (e - e0) * slot;
-                            while (l < h) {
-                                const int mid = (l + h) >> 1;
-                                if (row[mid] < c) l = mid + 1; else h = mid;
-                            }
-                            hit = have && l < len && row[l] == c;
-                        } else {
-                            // a row of C too long to stage: bisection in memory
-                            while (l < h) {
-                                const int mid = (l + h) >> 1;
-                                if (C_indices[cbe + mid] < c64) l = mid + 1; else h = mid;
-                            }
-                            hit = have && l < len && C_indices[cbe + l] == c64;
+                    const int nu = (ne << sh) / G;
+                    for (int u0 = 0; u0 < nu; u0 += 8) {
+                        int32_t got[8];
+#pragma unroll
+                        for (int uu = 0; uu < 8; ++uu) {
+                            const int f = (u0 + uu) * G;                 // flat staged position of lane 0
+                            const int er = f >> sh;                      // row of the sub-batch (group-uniform)
+                            const int t = (f & (slot - 1)) + gl;
+                            const int src = gbase + e0 + (er < ne ? er : 0);
+                            const int64_t cbe = shfl_t(cb, src);
+                            const int len = shfl_t(clen, src);
+                            const bool ok = er < ne && t < len && len <= kStage;
+                            got[uu] = (int32_t) * (ok ? C_indices + cbe + t : B_indptr);
                         }
-                        const T g_raw = gC[cbe + (hit ? l : 0)];   // cbe + 0 is readable whenever nnz(C) > 0
-                        const T g = hit ? g_raw : T(0);
-                        accB += ae * g;
-                        const T sum = ordered_group_sum(g * bval, gl);
-                        const T tot = shfl_t(sum, gbase + G - 1);
-                        if (gl == e) totalA = tot;
+#pragma unroll
+                        for (int uu = 0; uu < 8; ++uu)
+                            if (u0 + uu < nu) st[(u0 + uu) * G + gl] = got[uu];
+                    }
+                    group_fence();
+                    // 2. every lane finds its column in each staged row; then the gradients of C at
+                    //    those places are requested together
+                    int pos[8];
+                    unsigned hits = 0;
+#pragma unroll
+                    for (int e8 = 0; e8 < 8; ++e8) {
+                        pos[e8] = 0;
+                        if (e8 < ne) {
+                            const int64_t cbe = shfl_t(cb, gbase + e0 + e8);
+                            const int len = shfl_t(clen, gbase + e0 + e8);
+                            int l = 0, h = len;
+                            bool hit;
+                            if (len <= kStage) {
+                                const int32_t *row = st + (e8 << sh);
+                                while (l < h) {
+                                    const int mid = (l + h) >> 1;
+                                    if (row[mid] < c) l = mid + 1; else h = mid;
+                                }
+                                hit = have && l < len && row[l] == c;
+                            } else {
+                                // a row of C too long to stage: bisection in memory
+                                while (l < h) {
+                                    const int mid = (l + h) >> 1;
+                                    if (C_indices[cbe + mid] < c64) l = mid + 1; else h = mid;
+                                }
+                                hit = have && l < len && C_indices[cbe + l] == c64;
+                            }
+                            pos[e8] = l;
+                            hits |= (hit ? 1u : 0u) << e8;
+                        }
+                    }
+                    T g[8];
+#pragma unroll
+                    for (int e8 = 0; e8 < 8; ++e8) {
+                        const int64_t cbe = shfl_t(cb, gbase + e0 + (e8 < ne ? e8 : 0));
+                        g[e8] = gC[(hits >> e8) & 1u ? cbe + pos[e8] : 0];   // entry 0 is readable: nnz(C) > 0
+                    }
+                    // 3. grad_B: this lane's column, rows of C in the plan's order.  grad_A: the terms of
+                    //    entry e go to lane e through LDS, which adds them in lane order = ascending column
+                    group_fence();
+                    T *tr = reinterpret_cast<T *>(st);
+#pragma unroll
+                    for (int e8 = 0; e8 < 8; ++e8) {
+                        const bool hit = (hits >> e8) & 1u;
+                        const T ae = shfl_t(a, gbase + e0 + (e8 < ne ? e8 : 0));
+                        accB += hit ? ae * g[e8] : T(0);
+                        if (e8 < ne) tr[e8 * G + gl] = hit ? g[e8] * bval : T(0);
+                    }
+                    group_fence();
+                    if (gl >= e0 && gl < e0 + ne) {
+                        T run = prevA;
+#pragma unroll
+                        for (int j = 0; j < G; ++j) run += tr[(gl - e0) * G + j];
+                        totalA = run;
                     }
                 }
-                if (mine && grad_A) {
-                    if (jb == bb) grad_A[apos] = totalA;
-                    else grad_A[apos] += totalA;       // a later pass over a long row of B
-                }
+                if (mine && grad_A) grad_A[apos] = totalA;
             }
             if (have && grad_B) grad_B[my_j] = accB;
             jb += G;

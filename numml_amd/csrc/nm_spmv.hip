@@ -33,12 +33,30 @@ template <> struct Tile<double> { static constexpr int R = 512; static constexpr
 // forward: lanes per workgroup, rows per workgroup, LDS products
 #ifndef NM_FWD_BLOCK
 #define NM_FWD_BLOCK 256
+#endif
+#ifndef NM_FWD_R
 #define NM_FWD_R 512
 #define NM_FWD_CAP 4096
 #endif
 constexpr int kFwdBlock = NM_FWD_BLOCK, kFwdR = NM_FWD_R, kFwdCap = NM_FWD_CAP;
+// entries a lane of the forward keeps in flight when it reads 32-bit structure
+#ifndef NM_FWD32_K
+#define NM_FWD32_K 5
+#endif
+// 1: the forward on 32-bit structure loads 4 consecutive entries per lane and request
+#ifndef NM_FWD32_VEC
+#define NM_FWD32_VEC 0
+#endif
+// entries a lane of the planned backward keeps in flight
+#ifndef NM_BWD_K
+#define NM_BWD_K 6
+#endif
 // columns per workgroup / LDS entries of the planned backward (measured best at cfg2: 96 vs 101 us)
-constexpr int kPlannedR = 256, kPlannedCap = 2048;
+#ifndef NM_PLANNED_R
+#define NM_PLANNED_R 256
+#define NM_PLANNED_CAP 2048
+#endif
+constexpr int kPlannedR = NM_PLANNED_R, kPlannedCap = NM_PLANNED_CAP;
 
 // A block of rows with this many entries or more is walked straight from global memory.
 constexpr int32_t kHuge = 1 << 30;
@@ -104,13 +122,52 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
         stage_offsets<R, CAP, BLOCK, IDX>(indptr, r0, nr, base, s_off);
         __syncthreads();
         const int n = s_off[nr];
-        if (n <= CAP) {
+        if (NM_FWD32_VEC && sizeof(IDX) == 4 && !UNIT && n <= CAP) {
+            // 32-bit structure: a lane takes 4 consecutive entries per request (16-byte loads of
+            // values and columns, aligned to 4 bytes only: a tile starts wherever its first row
+            // does), two requests in flight
+            typedef T TV __attribute__((ext_vector_type(4), aligned(sizeof(T))));
+            typedef IDX IV __attribute__((ext_vector_type(4), aligned(sizeof(IDX))));
+            const T *__restrict__ d = data + base;
+            const IDX *__restrict__ ci = indices + base;
+            const int n4 = n & ~3;
+            constexpr int U = 2;
+            for (int k0 = threadIdx.x * 4; k0 < n4; k0 += U * 4 * BLOCK) {
+                TV aa[U];
+                IV cc[U];
+                T xx[U][4];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int kc = k0 + u * 4 * BLOCK < n4 ? k0 + u * 4 * BLOCK : n4 - 4;
+                    aa[u] = __builtin_nontemporal_load(reinterpret_cast<const TV *>(d + kc));
+                    cc[u] = __builtin_nontemporal_load(reinterpret_cast<const IV *>(ci + kc));
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) xx[u][q] = x[cc[u][q]];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (k0 + u * 4 * BLOCK < n4) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) s_prod[k0 + u * 4 * BLOCK + q] = aa[u][q] * xx[u][q];
+                    }
+            }
+            for (int k = n4 + threadIdx.x; k < n; k += BLOCK) s_prod[k] = d[k] * x[ci[k]];
+            __syncthreads();
+            for (int t = threadIdx.x; t < nr; t += BLOCK) {
+                const int e = s_off[t + 1];
+                T acc = 0;
+                for (int j = s_off[t]; j < e; ++j) acc += s_prod[j];
+                nm::stream_store(y + r0 + t, acc);
+            }
+        } else if (n <= CAP) {
             const T *__restrict__ d = data + base;
             const IDX *__restrict__ ci = indices + base;
             // K entries in flight per lane: all their streams, then all their gathers of x.
             // Loads are unconditional on a clamped position (a predicated load would sit in
             // its own branch with its own wait).
-            constexpr int K = 5;   // 4, 5 and 10 measure the same on the 2048 x 2048 Poisson matrix
+            constexpr int K = sizeof(IDX) == 4 ? NM_FWD32_K : 5;   // int64: 4, 5 and 10 measure the same on the 2048 x 2048 Poisson matrix
             for (int k0 = threadIdx.x; k0 < n; k0 += K * BLOCK) {
                 T aa[K], xx[K];
                 IDX cc[K];
@@ -439,7 +496,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
             // clamped position (a predicated load would sit in its own branch with its own wait).
             // Measured on the 2048 x 2048 Poisson matrix (5 entries per lane and tile), kernel time:
             // K = 2: 103 us, 4: 95 us, 5: 90 us, 6: 86 us, 8: 91 us.
-            constexpr int K = 6;
+            constexpr int K = NM_BWD_K;
             for (int p0 = threadIdx.x; p0 < cnt; p0 += K * kBlock) {
                 int32_t kk[K], rr[K];
                 T gg[K], xx[K], dd[K];

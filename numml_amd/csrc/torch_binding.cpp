@@ -813,6 +813,16 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
     C_indptr = index_tensor(C_indptr, "C_indptr");
     c10::hip::HIPGuard guard(dev.index());
     Tensor grad_A = torch::empty_like(A_data), grad_B = torch::empty_like(B_data);
+    if (auto plan = backward_plan(A_indices, A_indptr, A_rows, A_cols, dev)) {
+        check(nm_spgemm_backward_planned(dtype_of(A_data), A_rows, A_cols, A_data.numel(), B_data.numel(),
+                                         grad_C.numel(), grad_C.data_ptr(), C_indices.data_ptr<int64_t>(),
+                                         C_indptr.data_ptr<int64_t>(), A_data.data_ptr(), plan->mem.data_ptr(),
+                                         B_data.data_ptr(), B_indices.data_ptr<int64_t>(),
+                                         B_indptr.data_ptr<int64_t>(), grad_A.data_ptr(), grad_B.data_ptr(),
+                                         current_stream(dev)),
+              "nm_spgemm_backward_planned");
+        return {grad_A, grad_B};
+    }
     check(nm_spgemm_backward(dtype_of(A_data), A_rows, A_data.numel(), B_data.numel(), grad_C.data_ptr(),
                              C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(), A_data.data_ptr(),
                              A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),

@@ -532,6 +532,13 @@ def spgemm_backward(grad_C, C_indices, C_indptr,
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_B = torch.empty_like(B_data)
+        if BACKWARD_MODE != "atomic":
+            plan = _transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev)
+            _lib.check(_lib.lib().nm_spgemm_backward_planned(
+                _dt(A_data), A_rows, A_cols, A_data.shape[0], B_data.shape[0], grad_C.shape[0], _ptr(grad_C),
+                _ptr(C_indices), _ptr(C_indptr), _ptr(A_data), _ptr(plan.mem), _ptr(B_data), _ptr(B_indices),
+                _ptr(B_indptr), _ptr(grad_A), _ptr(grad_B), _stream(dev)), "nm_spgemm_backward_planned")
+            return [grad_A, grad_B]
         _lib.check(_lib.lib().nm_spgemm_backward(
             _dt(A_data), A_rows, A_data.shape[0], B_data.shape[0], _ptr(grad_C), _ptr(C_indices),
             _ptr(C_indptr), _ptr(A_data), _ptr(A_indices), _ptr(A_indptr), _ptr(B_data),

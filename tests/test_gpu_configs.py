@@ -118,7 +118,16 @@ def test_cfg4_spgemm_fp64_laplace128(dev):
     gC = randn(1, C.nnz, np.float64)
     C.data.backward(to_dev(dev, gC)[0])
     gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, rows, cols, d, i, p, rows, cols, d, i, p)
-    assert_close(host(A.data.grad), gA_ref + gB_ref, "grad wrt A.values (grad_A + grad_B)")
+    # both gradients are summed in the serial order on the plan; autograd adds the two
+    assert_same(host(A.data.grad), gA_ref + gB_ref, "grad wrt A.values (grad_A + grad_B)")
+    # ... and separately, through the binding
+    gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], C.indices, C.indptr, rows, cols, D, I, P, rows, cols, D, I, P)
+    assert_same(host(gA), gA_ref, "grad_A")
+    assert_same(host(gB), gB_ref, "grad_B")
+    _binding.set_backward_mode("atomic")      # the stateless kernels: grad_B by atomics, tolerance
+    gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], C.indices, C.indptr, rows, cols, D, I, P, rows, cols, D, I, P)
+    assert_same(host(gA), gA_ref, "grad_A (stateless)")
+    assert_close(host(gB), gB_ref, "grad_B (stateless)")
 
 
 def test_cfg5_sptrsv_fp64_tril_poisson1024(dev):
@@ -192,7 +201,7 @@ def test_cfg4_matrix_in_fp32(dev):
     gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], Ci, Cp, rows, cols, D, I, P, rows, cols, D, I, P)
     gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, rows, cols, d, i, p, rows, cols, d, i, p)
     assert_same(host(gA), gA_ref, "grad_A")
-    assert_close(host(gB), gB_ref, "grad_B")
+    assert_same(host(gB), gB_ref, "grad_B")
 
 
 def test_cfg5_matrix_in_fp32(dev):

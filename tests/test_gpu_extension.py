@@ -103,7 +103,12 @@ def test_spgemm(dev, cpp, dtype):
         gA, gB = cpp.spgemm_backward(Gc, Ci, Cp, m, k, AD, AI, AP, k, n, BD, BI, BP)
         gA_ref, gB_ref = oracle.spgemm_backward(g, ri, rp, m, k, ad, ai, ap, k, n, bd, bi, bp)
         assert_same(host(gA), gA_ref, "grad_A")
-        assert_close(host(gB), gB_ref, "grad_B")
+        assert_same(host(gB), gB_ref, "grad_B")     # on the plan: the serial order, no atomics
+        cpp.set_backward_mode("atomic")
+        gA, gB = cpp.spgemm_backward(Gc, Ci, Cp, m, k, AD, AI, AP, k, n, BD, BI, BP)
+        cpp.set_backward_mode("eager")
+        assert_same(host(gA), gA_ref, "grad_A (stateless)")
+        assert_close(host(gB), gB_ref, "grad_B (stateless)")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
