@@ -44,8 +44,20 @@ constexpr int kFwdBlock = NM_FWD_BLOCK, kFwdR = NM_FWD_R, kFwdCap = NM_FWD_CAP;
 #define NM_FWD32_K 5
 #endif
 // 1: the forward on 32-bit structure loads 4 consecutive entries per lane and request
+// (2048 x 2048 Poisson matrix, fp32: 47.6 -> 44.3 us; the same change in the planned backward made
+// it slower, 83 -> 87 us and more, so NM_BWD_VEC stays 0)
 #ifndef NM_FWD32_VEC
-#define NM_FWD32_VEC 0
+#define NM_FWD32_VEC 1
+#endif
+// 1: the planned backward loads 4 consecutive entries per lane and request, NM_BWD_VEC_U requests in flight
+#ifndef NM_BWD_VEC
+#define NM_BWD_VEC 0
+#endif
+#ifndef NM_BWD_VEC_U
+#define NM_BWD_VEC_U 2
+#endif
+#ifndef NM_FWD32_VEC_U
+#define NM_FWD32_VEC_U 2
 #endif
 // entries a lane of the planned backward keeps in flight
 #ifndef NM_BWD_K
@@ -131,7 +143,7 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
             const T *__restrict__ d = data + base;
             const IDX *__restrict__ ci = indices + base;
             const int n4 = n & ~3;
-            constexpr int U = 2;
+            constexpr int U = NM_FWD32_VEC_U;
             for (int k0 = threadIdx.x * 4; k0 < n4; k0 += U * 4 * BLOCK) {
                 TV aa[U];
                 IV cc[U];
@@ -420,7 +432,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
     const int32_t *__restrict__ flags, const T *__restrict__ x, const T *__restrict__ g,
     T *__restrict__ grad_A, T *__restrict__ grad_x) {
     __shared__ int32_t s_off[R + 1];
-    __shared__ T s_v[CAP];
+    __shared__ __align__(16) T s_v[CAP];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const bool mirror = flags[0] != 0;
@@ -496,6 +508,51 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
             // clamped position (a predicated load would sit in its own branch with its own wait).
             // Measured on the 2048 x 2048 Poisson matrix (5 entries per lane and tile), kernel time:
             // K = 2: 103 us, 4: 95 us, 5: 90 us, 6: 86 us, 8: 91 us.
+            if (NM_BWD_VEC) {
+                // a lane takes 4 consecutive entries per request: 16-byte loads of the two plan
+                // streams and one 16-byte store of grad_A (aligned to 4 bytes only), U requests in flight
+                typedef int32_t I4 __attribute__((ext_vector_type(4), aligned(4)));
+                typedef T T4 __attribute__((ext_vector_type(4), aligned(sizeof(T))));
+                constexpr int U = NM_BWD_VEC_U;
+                const int c4 = cnt & ~3;
+                for (int p0 = threadIdx.x * 4; p0 < c4; p0 += U * 4 * kBlock) {
+                    I4 kk[U], rr[U];
+                    T gg[U][4], xx[U][4], dd[U][4];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int pc = p0 + u * 4 * kBlock < c4 ? p0 + u * 4 * kBlock : c4 - 4;
+                        kk[u] = __builtin_nontemporal_load(reinterpret_cast<const I4 *>(tp + pc));
+                        rr[u] = __builtin_nontemporal_load(reinterpret_cast<const I4 *>(tr + pc));
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            gg[u][q] = g[rr[u][q]];
+                            xx[u][q] = x[rr[u][q]];
+                            dd[u][q] = data[kk[u][q]];
+                        }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int p = p0 + u * 4 * kBlock;
+                        if (p < c4) {
+                            T4 out;
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                out[q] = s_v[p + q] * xx[u][q];
+                                s_v[p + q] = gg[u][q] * dd[u][q];
+                            }
+                            *reinterpret_cast<T4 *>(ga + p) = out;
+                        }
+                    }
+                }
+                for (int p = c4 + threadIdx.x; p < cnt; p += kBlock) {
+                    const int32_t k = tp[p], r = tr[p];
+                    ga[p] = s_v[p] * x[r];
+                    s_v[p] = g[r] * data[k];
+                }
+                return;
+            }
             constexpr int K = NM_BWD_K;
             for (int p0 = threadIdx.x; p0 < cnt; p0 += K * kBlock) {
                 int32_t kk[K], rr[K];
