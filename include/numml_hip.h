@@ -285,6 +285,20 @@ int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
                     const void *data, int unit, const void *b, void *x,
                     void *work, size_t work_bytes, nm_stream stream);
 
+/* How the single-workgroup kernels of the solve keep their wavefronts in step
+ * (no counterpart in the reference).  By default every wavefront meets at a
+ * workgroup barrier after every level.  With `signalling` = 1, where no row of
+ * a triangle depends on a row more than one wavefront away inside the level
+ * before it (stencil and banded matrices), a wavefront instead publishes the
+ * levels it has finished in LDS and waits only for its neighbours.  (Measured
+ * slower than the barrier on MI355X, hence off by default; results are the same
+ * bits.)  All wavefronts of a workgroup are resident and only wait for lower
+ * levels, so the waits end; `poll_limit` bounds the polls of one wait all the
+ * same (0: the default of 2^22; negative: give up at once, for tests): when it
+ * is exceeded every wavefront of the launch leaves and x comes back as NaN
+ * throughout.  Process-wide; takes effect with the next solve. */
+int nm_sptrsv_configure(int64_t poll_limit, int signalling);
+
 /* nm_sptrsv_solve without the `work` argument, for callers that cannot allocate
  * device memory (code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc).  It has no counterpart in the reference.  The scratch
@@ -331,9 +345,11 @@ int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz,
  *                           matrix (rows of Mt = columns of M).  Columns are
  *                           taken in ascending order by wavefronts that wait
  *                           on a flag per column they depend on; poll_limit
- *                           bounds the polls of one flag (0 = default), and
- *                           when it is exceeded every wavefront leaves and the
- *                           call returns NM_ERR_HIP.  Synchronises the stream.
+ *                           bounds the polls of one flag during which no
+ *                           column anywhere finishes (0 = default), and when
+ *                           it is exceeded every wavefront leaves and the call
+ *                           returns NM_ERR_HIP; Mt_data is then left partly
+ *                           factorised (undefined).  Synchronises the stream.
  * The caller transposes As -> Mt before, and Mt -> M after, the numeric phase. */
 int nm_splu_symbolic_bytes(int64_t rows, size_t *bytes);
 int nm_splu_symbolic(int64_t rows, const int64_t *A_indices,

@@ -209,12 +209,12 @@ __global__ __launch_bounds__(kBlock) void lu_values_kernel(int64_t rows, const T
 constexpr int kLuCap = 1024;              // entries of a column kept in LDS, per wavefront
 constexpr int kLuWavesPerBlock = NM_LU_WAVES;   // columns of a batch = wavefronts of a workgroup of the numeric phase
 constexpr int kLuFlowBlock = kLuWavesPerBlock * 64;
-constexpr int64_t kLuSpinLimit = 1 << 24;  // polls of one dependency flag before giving up
+constexpr int64_t kLuSpinLimit = 1 << 24;  // polls of one dependency flag, without any column finishing, before giving up
 
 struct LuFlow {
     int64_t *below;  // [cols] position of the column's first entry below the diagonal
     int32_t *done;   // [cols] 0 = pending, 1 = the column holds its final values
-    int32_t *ctl;    // [0] next ticket, [1] failure
+    int32_t *ctl;    // [0] next ticket, [1] failure, [2] columns finished
 };
 
 size_t flow_layout(int64_t cols, void *base, LuFlow *F) {
@@ -324,22 +324,36 @@ __device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T,
         const Look cur = next;
         next = look(e + 1);
         const int64_t i = cur.i, ls = cur.ls, ie = cur.ie, t_first = cur.t_first, at_first = cur.at_first;
+        // The limit bounds polls WITHOUT PROGRESS: every 256 polls the wavefront looks at the failure
+        // word and at the count of finished columns, and starts counting afresh when that count has
+        // moved.  A wavefront that legitimately waits behind a chain of thousands of slow columns
+        // is thus never cut off, while a grid in which nothing finishes any more is.
         int64_t polls = 0;
+        int32_t seen_done = -1;
+        auto still_hopeful = [&]() -> bool {   // false: give up
+            if (++polls > spin_limit) return false;
+            if ((polls & 255) == 0) {
+                if (__hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
+                const int32_t now = __hip_atomic_load(ctl + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (now != seen_done) {
+                    seen_done = now;
+                    polls = 0;
+                }
+            }
+            return true;
+        };
         bool in_lds = false;   // column i is one of this batch's and its final values are in LDS
         if (i >= batch.base) {
             const int wi = (int)(i - batch.base);
             int32_t state;
             while ((state = batch.ready[wi]) == 0) {
-                if (++polls > spin_limit ||
-                    ((polls & 1023) == 0 && __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))
-                    return false;
+                if (!still_hopeful()) return false;
                 __builtin_amdgcn_s_sleep(1);
             }
             in_lds = state == 1;
         } else {
             while (__hip_atomic_load(done + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
-                if (++polls > spin_limit || __hip_atomic_load(ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
-                    return false;
+                if (!still_hopeful()) return false;
                 __builtin_amdgcn_s_sleep(1);
             }
         }
@@ -381,6 +395,7 @@ __device__ bool lu_column(int64_t k, int64_t pb, int64_t len, const OwnColumn<T,
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     if (lane == 0) {
         __hip_atomic_store(done + k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        atomicAdd(ctl + 2, 1);   // columns finished so far: what a waiting wavefront watches for progress
         if (!IN_LDS) batch.ready[k - batch.base] = 2;
     }
     return true;

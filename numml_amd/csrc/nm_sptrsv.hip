@@ -36,6 +36,8 @@
 #include "nm_scan.hpp"
 #include "nm_transpose.hpp"
 
+#include <atomic>
+#include <cstdlib>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -65,6 +67,7 @@ struct nm_sptrsv_plan {
     Packed dir[2];     // [0]: A, [1]: A^T
     int32_t max_deps[2] = {0, 0};  // longest dependency list per direction
     int32_t ell_pre[2] = {0, 0};   // width of the fixed-width layout per direction (2, 4, 8; 0 = not used)
+    int32_t reach[2] = {0, 0};     // per direction: largest wavefront distance between a row and a dependency
     struct Launch {
         int32_t l0, l1;  // levels [l0, l1)
         int32_t q0, q1;  // slots they cover
@@ -82,10 +85,28 @@ constexpr int kNarrow = 1024;          // widest level the single-workgroup kern
 constexpr int kWideRows = 128, kWideEntries = 4096;   // a level with both gets a grid launch as well
 constexpr int kBlock = 256;
 constexpr int kRing = 8192;            // LDS ring of recent solutions (doubles, power of two)
-constexpr int kRingSafe = kRing - kNarrow;
+// Levels a wavefront of the signalling kernel may run ahead of the slowest one of its
+// workgroup; the ring must keep what the slowest still reads while the fastest writes.
+constexpr int kSkew = 2;
+constexpr int kRingSafe = kRing - (kSkew + 1) * kNarrow;
+// Largest distance, in wavefronts, between a row and the rows it depends on (both counted from
+// the start of their level) for which wavefronts signal each other instead of meeting at a
+// workgroup barrier after every level.
+constexpr int kSigReach = 1;
 constexpr int kMaxLevels = 4096;       // levels one single-workgroup launch takes (LDS copy of their bounds)
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
+
+// Polls a wavefront of the signalling kernel makes at one level before it gives up (a poll is
+// ~100 cycles; a level takes a few hundred), and the switch between signalling and barriers.
+std::atomic<int64_t> g_sig_poll_limit{int64_t(1) << 22};
+// Off by default: on the 1024 x 1024 Poisson triangle (2047 levels, up to 16 wavefronts) a solve
+// takes 0.97 ms with a barrier per level and 1.30 ms with signals -- the two dependent LDS round
+// trips of a poll cost more than the barrier's wait for the slowest wavefront saves.
+std::atomic<bool> g_sig_enabled{[] {
+    const char *e = std::getenv("NUMML_AMD_SPTRSV_SIGNALLING");   // "1": neighbours signal
+    return e && e[0] == '1';
+}()};
 
 struct Layout {
     nm::TPlan t;
@@ -253,6 +274,7 @@ struct SolveWork {
     double *coef;   // coefficient of packed dependency `at`
     double *ell_coef;  // fixed-width copy of coef (0 padded), `pre` per slot
     double *rb;        // (right-hand side, diagonal) pairs per slot
+    int32_t *status;   // [2]: nonzero when a kernel of this solve gave up waiting
 };
 
 inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork *W) {
@@ -269,6 +291,7 @@ inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork
     w.coef = take(nnz + 1);
     w.ell_coef = take(ell_capacity(rows, nnz));
     w.rb = take(2 * (rows + kEllPad) + 2);
+    w.status = (int32_t *)take(2);
     if (W) *W = w;
     return off;
 }
@@ -577,7 +600,7 @@ __device__ __forceinline__ int32_t level_of_slot(const int32_t *__restrict__ lev
 __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict__ dptr,
                                 const int32_t *__restrict__ dslot, const int32_t *__restrict__ level_ptr,
                                 int32_t nlevels, const int32_t *__restrict__ level_launch,
-                                int32_t *__restrict__ ell_ds) {
+                                int32_t *__restrict__ ell_ds, int32_t *__restrict__ reach) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     // the padding slots behind the last row get "absent" entries: lanes that read them must find a valid offset
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (rows + kEllPad) * pre; i += stride) {
@@ -588,9 +611,16 @@ __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict
         if (e < n) {
             const int32_t ds = dslot[lo + e];
             const int32_t dist = ds > (int32_t)q ? ds - (int32_t)q : (int32_t)q - ds;
-            const bool same = level_launch[level_of_slot(level_ptr, nlevels, (int32_t)q)] ==
-                              level_launch[level_of_slot(level_ptr, nlevels, ds)];
-            out = ((ds & (kRing - 1)) * 8) | ((same && dist < kRingSafe) ? 0 : kEllFar);
+            const int32_t lq = level_of_slot(level_ptr, nlevels, (int32_t)q), ld = level_of_slot(level_ptr, nlevels, ds);
+            const bool same = level_launch[lq] == level_launch[ld];
+            const bool near = same && dist < kRingSafe;
+            out = ((ds & (kRing - 1)) * 8) | (near ? 0 : kEllFar);
+            if (near) {
+                // wavefront of the row and of the row it waits for, each inside its own level
+                const int32_t wq = ((int32_t)q - level_ptr[lq]) >> 6, wd = (ds - level_ptr[ld]) >> 6;
+                const int32_t far = wq > wd ? wq - wd : wd - wq;
+                if (far > *reach) atomicMax(reach, far);
+            }
         }
         ell_ds[i] = out;
     }
@@ -600,9 +630,11 @@ template <typename T>
 __global__ void gather_ell_kernel(int64_t rows, int pre, const T *__restrict__ data, const T *__restrict__ b,
                                   const int32_t *__restrict__ order, const int32_t *__restrict__ dptr,
                                   const int32_t *__restrict__ dsrc, const int32_t *__restrict__ diag,
-                                  double *__restrict__ ell_coef, double *__restrict__ rb) {
+                                  double *__restrict__ ell_coef, double *__restrict__ rb,
+                                  int32_t *__restrict__ status) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid == 0) status[0] = 0;   // first kernel of the solve
     for (int64_t i = tid; i < rows * pre; i += stride) {
         const int64_t q = i / pre;
         const int e = (int)(i - q * pre);
@@ -670,14 +702,33 @@ template <int PRE> __device__ __forceinline__ EllVals<PRE> load_ell(const EllArg
 // wavefront's instructions for it (four wavefronts per SIMD at 1024 rows, ~4 cycles per vector
 // instruction), so the level body is kept to what cannot be decided earlier: the ring reads
 // (offsets precomputed), the sum, the division, and the two stores.
-template <int PRE, int DEPTH>
-__global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step) {
+//
+// SIG: instead of a workgroup barrier after every level, a wavefront publishes the number of
+// levels it has finished and, before a level, waits until the wavefronts it can depend on (those
+// at most kSigReach away: the plan has checked that no row looks further) have finished the level
+// before, and until no wavefront is more than kSkew levels behind (the ring keeps what such a
+// straggler still reads).  A wavefront that has the rows of a level ready early goes on to the
+// next one while the others finish, so the workgroup is no longer as slow as its slowest
+// wavefront at every single level.  All wavefronts of the workgroup are resident and a
+// wavefront only ever waits for lower levels, so the waits end; as a backstop a wavefront
+// that has polled `poll_limit` times without success raises a flag that makes every wavefront
+// leave, and the solve's status word tells the last kernel of the solve to hand out NaN.
+template <int PRE, int DEPTH, bool SIG = false>
+__global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step,
+                                                             int64_t poll_limit = 0, int32_t *status = nullptr) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
     __shared__ int32_t s_lp[kMaxLevels + 1];
+    __shared__ int32_t s_done[kNarrow / 64];   // SIG: levels each wavefront has finished
+    __shared__ int32_t s_abort;
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
     for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
     if (threadIdx.x == 0) ring[kRing] = 0.;
+    if (SIG && threadIdx.x < kNarrow / 64) s_done[threadIdx.x] = 0;
+    if (SIG && threadIdx.x == 0) s_abort = poll_limit < 0 ? 1 : 0;   // a negative limit: give up at once (tests)
     __syncthreads();
+    const int sig_lane = threadIdx.x & 63, sig_wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sig_waves = blockDim.x >> 6;
+    bool gave_up = SIG && poll_limit < 0;
     const char *ring_bytes = reinterpret_cast<const char *>(ring);
     const uint32_t lane8 = threadIdx.x * 8u;
 
@@ -693,6 +744,28 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
         for (int d = 0; d < DEPTH; ++d) {
             const int it = it0 + d;
             if (it >= count) break;   // uniform over the workgroup
+            if (SIG && gave_up) break;
+            if (SIG) {
+                // lane w looks at wavefront w's count of finished levels
+                int64_t polls = 0;
+                for (;;) {
+                    // (relaxed atomic accesses of the LDS words themselves: a pointer to them would be
+                    // taken for a pointer to any memory, and its loads would wait for the global ones)
+                    const int32_t mine_done =
+                        __hip_atomic_load(&s_done[sig_lane & (kNarrow / 64 - 1)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    const int32_t seen = sig_lane < sig_waves ? mine_done : 0x7fffffff;
+                    const bool near = sig_lane + kSigReach >= sig_wave && sig_lane <= sig_wave + kSigReach;
+                    if (__ballot(seen >= (near ? it : it - kSkew)) == ~0ull) break;
+                    if (__hip_atomic_load(&s_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0 ||
+                        ++polls > poll_limit) {
+                        __hip_atomic_store(&s_abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        gave_up = true;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                if (gave_up) break;
+            }
             const EllVals<PRE> cur = qv[d];
             qv[d] = load_ell<PRE>(a, ahead);
 
@@ -732,9 +805,19 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
                 *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
                 *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
             }
-            __syncthreads();
+            if (SIG) {
+                // the ring write above is in LDS before the count moves (one wavefront's LDS
+                // accesses are served in the order it issued them)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                if (sig_lane == 0)
+                    __hip_atomic_store(&s_done[sig_wave], it + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else {
+                __syncthreads();
+            }
         }
+        if (SIG && gave_up) break;
     }
+    if (SIG && gave_up && sig_lane == 0 && status) status[0] = 1;
 }
 
 // One wide level: slots [q0, q1), one lane per row.
@@ -786,11 +869,15 @@ __global__ __launch_bounds__(kBlock) void sptrsv_level_group_kernel(SolveArgs a,
 }
 
 // x[order[q]] = xs[q], rounded once to the value type (cpp/sparse_csr_cpu.cpp:722).
+// `status` (may be null): nonzero when a kernel of this solve gave up waiting; x is then NaN throughout.
 template <typename T>
 __global__ void unslot_kernel(int64_t n, const int32_t *__restrict__ order, const double *__restrict__ xs,
-                              T *__restrict__ x) {
+                              T *__restrict__ x, const int32_t *__restrict__ status) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += stride) x[order[q]] = (T)xs[q];
+    const bool failed = status != nullptr && status[0] != 0;
+    const double nan = __longlong_as_double(0x7ff8000000000000ll);
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += stride)
+        x[order[q]] = (T)(failed ? nan : xs[q]);
 }
 
 template <typename T>
@@ -823,7 +910,7 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
         if (grid > 65536) grid = 65536;
         const T *dat = p->nnz > 0 ? (const T *)data : (const T *)b;
         hipLaunchKernelGGL(gather_ell_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, p->rows, pre, dat,
-                           (const T *)b, p->order, P.dptr, P.dsrc, P.diag, a.w.ell_coef, a.w.rb);
+                           (const T *)b, p->order, P.dptr, P.dsrc, P.diag, a.w.ell_coef, a.w.rb, a.w.status);
         NM_LAUNCH_CHECK("gather_ell_kernel");
     }
     const int n = (int)p->launches.size();
@@ -847,12 +934,28 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
             // dependencies per row fetched ahead through registers: the smallest pipeline that
             // holds this direction's longest row (longer rows take the slow path)
             const int maxdep = p->max_deps[transposed ? 1 : 0];
-            if (pre == 2)
-                hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
+            // wavefronts signal each other where no row looks further than kSigReach wavefronts away
+            // (and there is more than one wavefront); else they meet at a barrier after every level
+            const bool sig = pre > 0 && L.block > 64 && p->reach[dirn] <= kSigReach && g_sig_enabled.load();
+            const int64_t limit = g_sig_poll_limit.load();
+            if (pre == 2 && sig)
+                hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4, true>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
+                                   limit, a.w.status);
+            else if (pre == 4 && sig)
+                hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3, true>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
+                                   limit, a.w.status);
+            else if (pre == 8 && sig)
+                hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2, true>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
+                                   limit, a.w.status);
+            else if (pre == 2)
+                hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
+                                   (int64_t)0, (int32_t *)nullptr);
             else if (pre == 4)
-                hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
+                hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
+                                   (int64_t)0, (int32_t *)nullptr);
             else if (pre == 8)
-                hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step);
+                hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
+                                   (int64_t)0, (int32_t *)nullptr);
             else if (L.group[dirn] > 0) {
                 // several lanes per row: as many groups as the widest level has rows, within one workgroup
                 const int G = L.group[dirn];
@@ -881,7 +984,7 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     int64_t grid = nm::ceil_div(p->rows, kBlock);
     if (grid > 65536) grid = 65536;
     hipLaunchKernelGGL(unslot_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, p->rows, p->order, a.w.xs,
-                       (T *)x);
+                       (T *)x, pre > 0 ? a.w.status : (const int32_t *)nullptr);
     NM_LAUNCH_CHECK("unslot_kernel");
     return NM_OK;
 }
@@ -944,6 +1047,13 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     hipLaunchKernelGGL(kahn_kernel, dim3(1), dim3(kNarrow), 0, s, (int32_t)rows, p->lower, L.t.t_indptr, L.t.t_row,
                        W.deg, p->order, p->level_ptr, L.meta);
     if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "kahn_kernel launch failed"));
+    // The sweep appends the rows of a level in the order its atomics were served.  Rows ascending
+    // inside every level make the schedule the same on every run and keep a row's dependencies
+    // in the wavefronts next to its own, which is what lets wavefronts signal their neighbours
+    // instead of meeting at a barrier (W.count64 is not in use yet and holds 2 * rows int32).
+    if (int rc = nm::segments_sort_i32(L.meta, rows, rows, p->level_ptr, p->order,
+                                       reinterpret_cast<int32_t *>(W.count64), s))
+        return bail(rc);
     hipLaunchKernelGGL(slot_of_kernel, dim3((unsigned)rgrid), dim3(kBlock), 0, s, rows, p->order, p->slot_of);
 
     // level-major packed triangles for both directions: count, scan, fill
@@ -1088,12 +1198,17 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             int64_t grid = nm::ceil_div(rows * pre, kBlock);
             if (grid > 65536) grid = 65536;
             hipLaunchKernelGGL(ell_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, pre, p->dir[d].dptr,
-                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, p->dir[d].ell_ds);
+                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, p->dir[d].ell_ds,
+                               L.meta + 4 + d);
             if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
         }
     }
-    if (hipStreamSynchronize(s) != hipSuccess)   // also keeps `level_launch` alive until its copy is done
+    int32_t reach_h[2] = {0, 0};
+    if (hipMemcpyAsync(reach_h, L.meta + 4, sizeof(reach_h), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess)   // also keeps `level_launch` alive until its copy is done
         return bail(nm::fail(NM_ERR_HIP, "waiting for the plan to complete failed"));
+    p->reach[0] = reach_h[0];
+    p->reach[1] = reach_h[1];
     *plan_out = p;
     return NM_OK;
 }
@@ -1187,4 +1302,16 @@ extern "C" int nm_sptrsv_solve_static(const nm_sptrsv_plan *plan, nm_dtype dt, i
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F64) return solve_typed<double>(plan, transposed, data, unit, b, x, work, s);
     return solve_typed<float>(plan, transposed, data, unit, b, x, work, s);
+}
+
+// Test and diagnostics hooks of the triangular solve's single-workgroup kernels.
+//   poll_limit   polls one wavefront makes at one level before every wavefront of the launch
+//                leaves and the solve hands out NaN (0 restores the default, a negative value
+//                makes the kernels give up at once);
+//   signalling   0 (default): wavefronts meet at a workgroup barrier after every level;
+//                1: neighbours signal, where no row depends on a row more than one wavefront away.
+extern "C" int nm_sptrsv_configure(int64_t poll_limit, int signalling) {
+    g_sig_poll_limit.store(poll_limit == 0 ? int64_t(1) << 22 : poll_limit);
+    g_sig_enabled.store(signalling != 0);
+    return NM_OK;
 }

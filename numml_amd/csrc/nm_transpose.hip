@@ -170,12 +170,16 @@ __device__ void merge_pass(const int32_t *__restrict__ src, int32_t *__restrict_
     }
 }
 
-// Step 4.  A workgroup owns `ct` consecutive columns.
+// Step 4.  A workgroup owns `ct` consecutive columns.  `cols_dev`, when given, holds the number of
+// columns on the device (a caller that does not know it on the host yet); rowid / t_row may be null
+// (keys are then only put in order).
 __global__ __launch_bounds__(kBlock) void tp_order_kernel(
-    int64_t cols, int ct, const int32_t *__restrict__ t_indptr, int32_t *__restrict__ t_perm,
-    const int32_t *__restrict__ rowid, int32_t *__restrict__ t_row, int32_t *__restrict__ tmp) {
+    int64_t cols, const int32_t *__restrict__ cols_dev, int ct, const int32_t *__restrict__ t_indptr,
+    int32_t *__restrict__ t_perm, const int32_t *__restrict__ rowid, int32_t *__restrict__ t_row,
+    int32_t *__restrict__ tmp) {
     __shared__ int32_t s_off[kRows + 1];
     __shared__ int32_t s_key[kCap];
+    if (cols_dev) cols = *cols_dev;
     const int64_t ntiles = (cols + ct - 1) / ct, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t tile = nm::xcd_tile(id, npad);
@@ -203,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
                 int rank = 0;
                 for (int q = b; q < e; ++q) rank += s_key[q] < key;
                 t_perm[first + b + rank] = key;
-                t_row[first + b + rank] = rowid[key];
+                if (t_row) t_row[first + b + rank] = rowid[key];
             }
             __syncthreads();
         };
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
             for (int j = threadIdx.x; j < len; j += kBlock) {
                 const int32_t key = src[j];
                 if (src != col) col[j] = key;
-                t_row[first + j] = rowid[key];
+                if (t_row) t_row[first + j] = rowid[key];
             }
             __syncthreads();
             s0 += 1;
@@ -318,8 +322,8 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
         const int ct = tile_rows(cols, nnz);
         grid = xcd_padded(ceil_div(cols, ct));
         if (grid > 65536) grid = 65536;
-        hipLaunchKernelGGL(tp_order_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, ct, plan.t_indptr,
-                           plan.t_perm, rowid, plan.t_row, w.tmp);
+        hipLaunchKernelGGL(tp_order_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, (const int32_t *)nullptr, ct,
+                           plan.t_indptr, plan.t_perm, rowid, plan.t_row, w.tmp);
         NM_LAUNCH_CHECK("tp_order_kernel");
     }
     hipLaunchKernelGGL(symmetry_init_kernel, dim3(1), dim3(64), 0, s, plan.flags, rows == cols ? 1 : 0);
@@ -331,6 +335,19 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
                            plan.c_ptr32, plan.t_row, plan.t_indptr, plan.flags);
     }
     NM_LAUNCH_CHECK("symmetry check");
+    return NM_OK;
+}
+
+int segments_sort_i32(const int32_t *nseg_dev, int64_t nseg_max, int64_t nkeys, const int32_t *seg_ptr,
+                      int32_t *keys, int32_t *tmp, hipStream_t s) {
+    if (nkeys <= 0 || nseg_max <= 0) return NM_OK;
+    // few segments per workgroup: their number is not known here, and they may be long
+    const int ct = 8;
+    int64_t grid = xcd_padded(ceil_div(nseg_max, ct));
+    if (grid > 8192) grid = 8192;
+    hipLaunchKernelGGL(tp_order_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nseg_max, nseg_dev, ct, seg_ptr, keys,
+                       (const int32_t *)nullptr, (int32_t *)nullptr, tmp);
+    NM_LAUNCH_CHECK("tp_order_kernel (segments)");
     return NM_OK;
 }
 

@@ -62,4 +62,10 @@ size_t tplan_work_bytes(int64_t rows, int64_t cols, int64_t nnz);
 int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices, const int64_t *indptr,
                 const TPlan &plan, void *work, size_t work_bytes, int32_t *rowid_out, hipStream_t s);
 
+// Puts the int32 keys of every segment [seg_ptr[j], seg_ptr[j + 1]) into ascending order, in
+// place (keys inside a segment are distinct).  The number of segments is read from the device
+// (`nseg_dev`, at most nseg_max); `tmp` holds nkeys int32 of scratch.
+int segments_sort_i32(const int32_t *nseg_dev, int64_t nseg_max, int64_t nkeys, const int32_t *seg_ptr,
+                      int32_t *keys, int32_t *tmp, hipStream_t s);
+
 }  // namespace nm

@@ -813,7 +813,15 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
     C_indptr = index_tensor(C_indptr, "C_indptr");
     c10::hip::HIPGuard guard(dev.index());
     Tensor grad_A = torch::empty_like(A_data), grad_B = torch::empty_like(B_data);
-    if (auto plan = backward_plan(A_indices, A_indptr, A_rows, A_cols, dev)) {
+    // The plan-based kernel looks every column of a row of B up in a staged row of C per entry of
+    // A, the stateless one stages a row of C once and looks the rows of B up in it: with rows of C
+    // many times longer than rows of B the stateless kernel is the faster one, and the default mode
+    // takes it ("eager" asks for the deterministic sums whatever they cost).
+    const int mode = backward_mode_now();
+    const double mean_c = A_rows > 0 ? (double)grad_C.numel() / A_rows : 0.;
+    const double mean_b = B_rows > 0 ? (double)B_data.numel() / B_rows : 0.;
+    const bool on_plan = mode == kEager || (mode == kPlanned && mean_c <= 4. * std::max(mean_b, 1.));
+    if (auto plan = on_plan ? backward_plan(A_indices, A_indptr, A_rows, A_cols, dev) : nullptr) {
         check(nm_spgemm_backward_planned(dtype_of(A_data), A_rows, A_cols, A_data.numel(), B_data.numel(),
                                          grad_C.numel(), grad_C.data_ptr(), C_indices.data_ptr<int64_t>(),
                                          C_indptr.data_ptr<int64_t>(), A_data.data_ptr(), plan->mem.data_ptr(),

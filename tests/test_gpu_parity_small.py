@@ -272,3 +272,35 @@ def test_fp32_long_rows_against_a_double_evaluation(dev):
             err_cpu = np.abs(cpu.astype(np.float64) - exact)
             bound = 4 * err_cpu + rtol * np.abs(exact).max()
             assert np.all(err_gpu <= bound), f"{name} {what}: worst excess {float((err_gpu - bound).max()):.3e}"
+
+
+def test_sptrsv_signalling_equals_barriers_and_gives_up_instead_of_waiting_forever(dev):
+    """The single-workgroup solve kernels can keep their wavefronts in step by neighbour-to-neighbour
+    signals where the triangle allows it (a stencil's does) instead of a barrier per level.  Same
+    bits either way; and with the poll limit forced from the host every wavefront leaves at once,
+    the call returns, and x is NaN throughout instead of wrong."""
+    import ctypes
+    from numml_amd import _lib
+    L = _lib.lib()
+    d, i, p, (n, _) = G.poisson2d_lower(300, np.float64, diag_seed=2)      # 599 levels, up to 300 rows wide
+    b = randn(3, n, np.float64)
+    D, I, P, Bv = to_dev(dev, d, i, p, b)
+    x_ref = oracle.sptrsv_forward(n, n, d, i, p, True, False, b)
+    g = randn(4, n, np.float64)
+    gA_ref, gb_ref = oracle.sptrsv_backward(g, x_ref, n, n, d, i, p, True, False)
+    try:
+        for signalling in (1, 0):
+            assert L.nm_sptrsv_configure(0, signalling) == 0
+            x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
+            assert_same(host(x), x_ref, f"x (signalling={signalling})")
+            gA, gb = ext.sptrsv_backward(to_dev(dev, g)[0], x, n, n, D, I, P, True, False, Bv)
+            assert_same(host(gb), gb_ref, f"grad_b (signalling={signalling})")
+            assert_same(host(gA), gA_ref, f"grad_A (signalling={signalling})")
+        assert L.nm_sptrsv_configure(-1, 1) == 0                           # give up at once
+        x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
+        torch.cuda.synchronize()
+        assert bool(torch.isnan(x).all())
+    finally:
+        assert L.nm_sptrsv_configure(0, 0) == 0
+    x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
+    assert_same(host(x), x_ref, "x after the defaults were restored")
