@@ -163,7 +163,11 @@ int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
  * C between them:
  *
  *   nm_spgemm_workspace_bytes  -> bytes of device scratch both phases need
- *   nm_spgemm_symbolic         -> fills C_indptr (A_rows + 1 entries)
+ *   nm_spgemm_symbolic         -> fills C_indptr (A_rows + 1 entries).  With
+ *                                 host_landing (see below; may be NULL) the call
+ *                                 waits for its first kernel, learns how many
+ *                                 rows need the hash path and, when none does,
+ *                                 leaves the hash path's launches out
  *   nm_spgemm_symbolic_result  -> waits for the symbolic phase and hands the
  *                                 host nnz(C) = C_indptr[A_rows], with which
  *                                 the caller allocates, and the number of rows
@@ -200,7 +204,7 @@ int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols,
                        const int64_t *A_indices, const int64_t *A_indptr,
                        const int64_t *B_indices, const int64_t *B_indptr,
                        int64_t *C_indptr, void *workspace, size_t workspace_bytes,
-                       nm_stream stream);
+                       void *host_landing, nm_stream stream);
 
 int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const void *workspace,
                               size_t workspace_bytes, int64_t *nnz_C, int64_t *hash_rows,

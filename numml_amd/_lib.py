@@ -40,7 +40,7 @@ _SIGNATURES = {
                           _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "nm_spgemm_workspace_bytes": [_c_i64, _c_i64, ctypes.POINTER(_c_size)],
     "nm_spgemm_symbolic": [_c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                           _c_size, _c_ptr],
+                           _c_size, _c_ptr, _c_ptr],
     "nm_spgemm_symbolic_result": [_c_i64, _c_i64, _c_ptr, _c_size, ctypes.POINTER(_c_i64),
                                   ctypes.POINTER(_c_i64), _c_ptr, _c_ptr],
     "nm_spgemm_numeric": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,

@@ -209,7 +209,8 @@ __device__ __forceinline__ void merge_stage(int64_t bb, int len, const int64_t *
 __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     int64_t rows, int64_t nbatch_padded, const int64_t *__restrict__ A_indices,
     const int64_t *__restrict__ A_indptr, const int64_t *__restrict__ B_indices,
-    const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key, int64_t *__restrict__ C_count) {
+    const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key, int64_t *__restrict__ C_count,
+    unsigned long long *__restrict__ hash_rows) {
     __shared__ int32_t s_col[(kMergeCap + 1) * kMergeStride];
     __shared__ int64_t s_bb[kBlock];
     __shared__ int32_t s_len[kBlock];
@@ -235,6 +236,10 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     const int32_t ubc = merge_sum((int32_t)(ub > 0x0fffffff ? 0x0fffffff : ub));
     const bool merge = live && (ae - ab) <= kMergeCap && merge_max(mx) <= kMergeCap;
     if (live && !merge && gl == 0) key[row] = ubc;
+    {   // rows left to the hash path are counted (a product of stencil matrices has none: no atomic at all)
+        const unsigned long long left = __ballot(live && !merge && gl == 0);
+        if (left != 0 && (threadIdx.x & 63) == 0) atomicAdd(hash_rows, (unsigned long long)__popcll(left));
+    }
     merge_stage<float, false>(my_bb, merge ? my_len : 0, B_indices, nullptr, A_indptr, s_bb, s_len, s_col, nullptr);
     const int32_t *pc = s_col + threadIdx.x;
     int32_t cur = *pc;
@@ -459,12 +464,9 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
 }
 
 // What the host needs between the phases, in one place: nnz(C) and the rows the hash path took.
-__global__ void summary_kernel(const int64_t *__restrict__ nnz_c, const int32_t *__restrict__ bins,
-                               int64_t *__restrict__ summary) {
-    if (threadIdx.x == 0) {
-        summary[0] = *nnz_c;
-        summary[1] = bins[kBinStart + kBins];
-    }
+// summary[1] already holds the number of rows on the hash path (counted by the first kernel).
+__global__ void summary_kernel(const int64_t *__restrict__ nnz_c, int64_t *__restrict__ summary) {
+    if (threadIdx.x == 0) summary[0] = *nnz_c;
 }
 
 // host_pinned[0..1] = summary, then host_pinned[2] = ticket: the host polls the ticket.
@@ -1247,7 +1249,7 @@ extern "C" int nm_spgemm_workspace_bytes(int64_t A_rows, int64_t B_cols, size_t 
 extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t *A_indices,
                                   const int64_t *A_indptr, const int64_t *B_indices, const int64_t *B_indptr,
                                   int64_t *C_indptr, void *workspace, size_t workspace_bytes,
-                                  nm_stream stream) {
+                                  void *host_landing, nm_stream stream) {
     if (int rc = check_common(A_rows, B_cols)) return rc;
     NM_REQUIRE(A_cols >= 0, "negative size");
     NM_REQUIRE(A_indptr && B_indptr && C_indptr && workspace, "null pointer argument");
@@ -1258,10 +1260,30 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     hipStream_t s = nm::as_stream(stream);
     if (A_rows == 0) return nm::fill_async(C_indptr, 1, (int64_t)0, s);
 
+    if (int rc = nm::fill_async(w.summary, 2, (int64_t)0, s)) return rc;
     const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
     hipLaunchKernelGGL(symbolic_front_kernel, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
-                       A_indices, A_indptr, B_indices, B_indptr, w.key, C_indptr);
+                       A_indices, A_indptr, B_indices, B_indptr, w.key, C_indptr,
+                       reinterpret_cast<unsigned long long *>(w.summary + 1));
     NM_LAUNCH_CHECK("symbolic_front_kernel");
+    // With a landing place in pinned host memory the host learns here how many rows the first
+    // kernel left to the hash path; with none (a product of stencil or aggregation matrices) the
+    // binning and the nine launches of the hash path, which would find nothing to do, are left out.
+    bool hashed = true;
+    if (host_landing) {
+        volatile int64_t *both = (volatile int64_t *)host_landing;
+        const int64_t ticket = both[2] + 1;
+        hipLaunchKernelGGL(summary_out_kernel, dim3(1), dim3(64), 0, s, w.summary, both, ticket);
+        NM_LAUNCH_CHECK("summary_out_kernel");
+        bool arrived = false;
+        for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = both[2] == ticket;
+        if (!arrived) {
+            NM_HIP_TRY(hipStreamSynchronize(s));
+            NM_REQUIRE(both[2] == ticket, "the count of hash-path rows did not arrive");
+        }
+        hashed = both[1] != 0;
+    }
+    if (hashed) {
     if (int rc = bin_rows(A_rows, kSymLimit, w, s)) return rc;
 
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup0, kSymTable0>), dim3(kPersistGrid), dim3(kBlock), 0, s, 0, w.bins,
@@ -1282,9 +1304,10 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     hipLaunchKernelGGL(symbolic_spill_kernel, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm, B_cols,
                        A_indices, A_indptr, B_indices, B_indptr, w.mark, C_indptr);
     NM_LAUNCH_CHECK("symbolic_spill_kernel");
+    }
     // counts sit in C_indptr[0, rows), C_indptr[rows] = 0: the exclusive scan is the row pointer
     if (int rc = nm::scan_exclusive_i64(C_indptr, A_rows + 1, w.scan, s)) return rc;
-    hipLaunchKernelGGL(summary_kernel, dim3(1), dim3(64), 0, s, C_indptr + A_rows, w.bins, w.summary);
+    hipLaunchKernelGGL(summary_kernel, dim3(1), dim3(64), 0, s, C_indptr + A_rows, w.summary);
     NM_LAUNCH_CHECK("summary_kernel");
     return NM_OK;
 }

@@ -773,7 +773,7 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     nm_stream st = current_stream(dev);
     check(nm_spgemm_symbolic(A_rows, A_cols, B_cols, A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
                              B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
-                             C_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, st),
+                             C_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, host_landing(), st),
           "nm_spgemm_symbolic");
     // the one device->host read the interface makes inherent: C is returned exactly sized
     int64_t nnz_c = 0, hash_rows = 0;

@@ -498,7 +498,7 @@ def spgemm_forward(A_rows, A_cols, A_data, A_indices, A_indptr,
         st = _stream(dev)
         _lib.check(L.nm_spgemm_symbolic(
             A_rows, A_cols, B_cols, _ptr(A_indices), _ptr(A_indptr), _ptr(B_indices), _ptr(B_indptr),
-            _ptr(C_indptr), _ptr(work), nbytes.value, st), "nm_spgemm_symbolic")
+            _ptr(C_indptr), _ptr(work), nbytes.value, _ptr(_host_landing()), st), "nm_spgemm_symbolic")
         nnz_c, hash_rows = ctypes.c_int64(0), ctypes.c_int64(0)
         _lib.check(L.nm_spgemm_symbolic_result(A_rows, B_cols, _ptr(work), nbytes.value, ctypes.byref(nnz_c),
                                                ctypes.byref(hash_rows), _ptr(_host_landing()), st),

@@ -266,10 +266,11 @@ def test_spgemm_through_the_c_abi_with_and_without_the_hash_row_count(dev, hint)
         _lib.check(L.nm_spgemm_workspace_bytes(r, c, ctypes.byref(nbytes)), "bytes")
         work = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
         Cp = torch.empty(r + 1, dtype=torch.int64, device=dev)
-        _lib.check(L.nm_spgemm_symbolic(r, c, c, ptr(I), ptr(P), ptr(I), ptr(P), ptr(Cp), ptr(work), nbytes.value, st), "symbolic")
-        nnz_c, hash_rows = ctypes.c_int64(-7), ctypes.c_int64(-7)
         # with a pinned landing place for the device to write into (hint "given"), and without one
         landing = torch.zeros(3, dtype=torch.int64).pin_memory() if hint == "given" else None
+        _lib.check(L.nm_spgemm_symbolic(r, c, c, ptr(I), ptr(P), ptr(I), ptr(P), ptr(Cp), ptr(work), nbytes.value,
+                                        ptr(landing) if landing is not None else None, st), "symbolic")
+        nnz_c, hash_rows = ctypes.c_int64(-7), ctypes.c_int64(-7)
         _lib.check(L.nm_spgemm_symbolic_result(r, c, ptr(work), nbytes.value, ctypes.byref(nnz_c), ctypes.byref(hash_rows),
                                                ptr(landing) if landing is not None else None, st), "result")
         Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(r, c, d, i, p, r, c, d, i, p)
