@@ -244,6 +244,44 @@ int nm_spgemm_backward_planned(nm_dtype dt, int64_t A_rows, int64_t A_cols, int6
                                const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
                                void *grad_A, void *grad_B, nm_stream stream);
 
+/* Product plan of C = A B: per stored entry of A, where its row of B and its row of
+ * C start and, for each of the (at most eight) entries of that row of B, the
+ * position of its column inside the row of C.  Built once for a pair of patterns
+ * and their product's pattern; afterwards the numeric product and both gradients
+ * need no merge, hash table or search (the reference repeats the symbolic work in
+ * every call, cpp/sparse_csr_gemm_cuda.cu:10-302, and searches C in every backward
+ * pass, cpp/sparse_csr_cpu.cpp:246-303).  Results are bit-identical to
+ * nm_spgemm_numeric / nm_spgemm_backward_planned: sums run in the serial loops' order.
+ *
+ *   nm_spgemm_plan_build    C_indices / C_indptr must be the pattern of A B as
+ *                           nm_spgemm_numeric returns it (complete, rows ascending).
+ *                           A_plan_mem: the transposed-structure plan of A
+ *                           (nm_csr_transpose_plan_build).  *usable = 1 when every
+ *                           row of A, every row of B that A names and every row of C
+ *                           stays within 8 / 8 / 64 entries, no column of A holds
+ *                           more than 4096 and all positions fit 31 bits; otherwise
+ *                           0 and the plan must not be used.  Waits for the stream
+ *                           (through host_landing, 24 bytes of pinned host memory,
+ *                           when given; NULL: a copy and a synchronisation).
+ *   nm_spgemm_numeric_planned   C_data of the product, C_indptr as built from.
+ *   nm_spgemm_backward_mapped   grad_A and / or grad_B (either may be NULL) of
+ *                           gC laid out on the plan's pattern of C. */
+int nm_spgemm_plan_bytes(int64_t A_nnz, size_t *plan_bytes);
+int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                         const int64_t *A_indices, const int64_t *A_indptr,
+                         const int64_t *B_indices, const int64_t *B_indptr,
+                         const int64_t *C_indices, const int64_t *C_indptr,
+                         const void *A_plan_mem, void *plan_mem, size_t plan_bytes,
+                         void *host_landing, int *usable, nm_stream stream);
+int nm_spgemm_numeric_planned(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                              const void *A_data, const int64_t *A_indptr, const void *B_data,
+                              const void *plan_mem, const int64_t *C_indptr, void *C_data,
+                              nm_stream stream);
+int nm_spgemm_backward_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t A_nnz,
+                              int64_t B_nnz, int64_t C_nnz, const void *gC, const void *A_data,
+                              const void *A_plan_mem, const void *B_data, const int64_t *B_indptr,
+                              const void *plan_mem, void *grad_A, void *grad_B, nm_stream stream);
+
 /* ---------------------------------------------------------------- SpTRSV
  * Level-scheduled triangular solve.  Stands in for sptrsv_forward /
  * sptrsv_backward (cpp/sparse_csr.hpp:94-105, cpp/sparse_csr_cpu.cpp:652-759).

@@ -100,6 +100,11 @@ __device__ __forceinline__ double dpp_move_zero(double v) {
     return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 
+template <int CTRL>
+__device__ __forceinline__ int dpp_move_zero(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+
 __device__ __forceinline__ float read_lane(float v, int l) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
 }

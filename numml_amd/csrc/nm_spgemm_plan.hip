@@ -1,0 +1,400 @@
+// Product plan of a sparse product C = A B: what the numeric work needs to know about
+// the three patterns, computed once per pair of patterns and reused for as long as only the
+// VALUES of A and B change (a training loop over a fixed hierarchy, the reference's own use).
+// The reference redoes the symbolic work on every call (cpp/sparse_csr_gemm_cuda.cu:10-302 on
+// the device, the std::map rows of cpp/sparse_csr_cpu.cpp:177-214 on the host) and searches C
+// again in every backward pass (cpp/sparse_csr_cpu.cpp:246-303); with a plan neither happens.
+//
+// Per stored entry e = (i, j) of A the plan holds
+//
+//   bstart[e]   where row j of B starts                                   (int32)
+//   cstart[e]   where row i of C starts                                   (int32)
+//   dest[e]     eight bytes: byte k is the position inside row i of C of the column of the
+//               k-th entry of row j of B, 0xFF when that row has no k-th entry
+//
+// so that the product a_e * b_(j,k) is known to belong to C[cstart[e] + dest[e][k]] without a
+// merge, a hash table or a search.  The plan exists for products whose rows all stay inside the
+// merge path's limits: at most kCap entries per row of A and per row of B that A names, and
+// rows of C of at most kRowCap entries; nm_spgemm_plan_build reports whether they hold.
+//
+//   forward    eight lanes per row of C; the products of the row's entries of A are added to
+//              the row's accumulators in LDS one entry of A after the other, i.e. every C entry
+//              receives its products in the order of A's row starting from +0.0 -- the order of
+//              the serial loop (cpp/sparse_csr_cpu.cpp:193-200), bit for bit;
+//   grad_A[e]  = sum_k gC[cstart[e] + dest[e][k]] * b_(j,k), k ascending (the merge of
+//              cpp/sparse_csr_cpu.cpp:261-274 meets the columns in that order);
+//   grad_B[(j,k)] = sum over the entries e of column j of A, rows ascending (the order of
+//              cpp/sparse_csr_cpu.cpp:291-303), of a_e * gC[cstart[e] + dest[e][k]], walked on
+//              the transposed-structure plan of A.
+//
+// No atomics, nothing to clear, every gradient entry written once by one lane.
+#include "nm_common.hpp"
+#include "nm_transpose.hpp"
+
+namespace {
+
+using nm::kWave;
+
+constexpr int kBlock = 256;
+constexpr int kCap = 8;                  // entries per row of A and per named row of B
+constexpr int kRowCap = kCap * kCap;     // entries per row of C
+constexpr int kGroupsPerBlock = kBlock / kCap;
+constexpr int32_t kMaxColumn = 4096;     // entries per column of A: one group of lanes walks a column
+constexpr uint8_t kNone = 0xFF;
+
+struct PPlan {
+    int32_t *flag;     // [0] != 0: a limit does not hold, the plan must not be used
+    int32_t *bstart;   // [A_nnz]
+    int32_t *cstart;   // [A_nnz]
+    uint8_t *dest;     // [A_nnz * 8]
+};
+
+size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += nm::align256(bytes);
+        return q;
+    };
+    int32_t *flag = (int32_t *)take(64);
+    int32_t *bs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
+    int32_t *cs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
+    uint8_t *d = (uint8_t *)take((size_t)(A_nnz + 1) * 8);
+    if (p) *p = PPlan{flag, bs, cs, d};
+    return off;
+}
+
+__device__ __forceinline__ void group_fence() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); }
+
+// ---- build -----------------------------------------------------------------------
+
+// Eight lanes per row of A: lane k takes the k-th entry of each B row the row names and finds
+// its column in row i of C.
+__global__ __launch_bounds__(kBlock) void plan_map_kernel(
+    int64_t rows, const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
+    const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
+    const int64_t *__restrict__ C_indices, const int64_t *__restrict__ C_indptr, PPlan p) {
+    const int k = threadIdx.x & (kCap - 1);
+    const int64_t stride = (int64_t)gridDim.x * kGroupsPerBlock;
+    bool bad = false;
+    for (int64_t row = (int64_t)blockIdx.x * kGroupsPerBlock + threadIdx.x / kCap; row < rows; row += stride) {
+        const int64_t ab = A_indptr[row], ae = A_indptr[row + 1];
+        const int64_t cs = C_indptr[row], ce = C_indptr[row + 1];
+        if (ae - ab > kCap || ce - cs > kRowCap) {
+            bad = true;
+            continue;
+        }
+        for (int64_t e = ab; e < ae; ++e) {
+            const int64_t j = A_indices[e];
+            const int64_t bb = B_indptr[j], blen = B_indptr[j + 1] - bb;
+            if (blen > kCap) {
+                bad = true;
+                break;
+            }
+            uint8_t d = kNone;
+            if (k < blen) {
+                const int64_t col = B_indices[bb + k];
+                int64_t lo = cs, hi = ce;
+                while (lo < hi) {
+                    const int64_t mid = (lo + hi) >> 1;
+                    if (C_indices[mid] < col) lo = mid + 1;
+                    else hi = mid;
+                }
+                if (lo < ce && C_indices[lo] == col) d = (uint8_t)(lo - cs);
+                else bad = true;   // C is not the pattern of A B
+            }
+            p.dest[e * kCap + k] = d;
+            if (k == 0) {
+                p.bstart[e] = (int32_t)bb;
+                p.cstart[e] = (int32_t)cs;
+            }
+        }
+    }
+    if (bad) p.flag[0] = 1;
+}
+
+__global__ __launch_bounds__(kBlock) void plan_columns_kernel(int64_t cols, const int32_t *__restrict__ t_indptr,
+                                                              int32_t *flag) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    bool bad = false;
+    for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < cols; j += stride)
+        bad |= t_indptr[j + 1] - t_indptr[j] > kMaxColumn;
+    if (bad) flag[0] = 1;
+}
+
+__global__ void plan_flag_out_kernel(const int32_t *flag, volatile int64_t *host_pinned, int64_t ticket) {
+    if (threadIdx.x == 0) {
+        host_pinned[0] = flag[0];
+        __threadfence_system();
+        host_pinned[2] = ticket;
+    }
+}
+
+// ---- forward -----------------------------------------------------------------------
+
+// Row stride of the accumulators: one more than the row capacity, so that the eight rows of a
+// wavefront start in different LDS banks.
+constexpr int kAccStride = kRowCap + 1;
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
+    int64_t rows, int64_t ntiles_padded, const T *__restrict__ A_data, const int64_t *__restrict__ A_indptr,
+    const T *__restrict__ B_data, const int32_t *__restrict__ bstart, const uint8_t *__restrict__ dest,
+    const int64_t *__restrict__ C_indptr, T *__restrict__ C_data) {
+    __shared__ T s_acc[kGroupsPerBlock * kAccStride];
+    const int k = threadIdx.x & (kCap - 1), g = threadIdx.x / kCap;
+    const int64_t row = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + g;
+    const bool live = row < rows;
+    const int64_t *pa = A_indptr + (live ? row : 0), *pc = C_indptr + (live ? row : 0);
+    const int64_t ab = pa[0], ae = live ? pa[1] : ab;
+    const int64_t cs = pc[0];
+    const int clen = live ? (int)(pc[1] - cs) : 0;
+    T *acc = s_acc + g * kAccStride;
+#pragma unroll
+    for (int q = 0; q < kCap; ++q) acc[k + kCap * q] = T(0);
+    // everything the row needs is requested before anything is used: two round trips
+    T av[kCap], bv[kCap];
+    int32_t bs[kCap];
+    uint8_t db[kCap];
+#pragma unroll
+    for (int a = 0; a < kCap; ++a) {
+        const int64_t e = ab + a < ae ? ab + a : 0;   // entry 0: readable whenever a row has entries
+        av[a] = A_data[e];
+        bs[a] = bstart[e];
+        db[a] = ab + a < ae ? dest[e * kCap + k] : kNone;
+    }
+#pragma unroll
+    for (int a = 0; a < kCap; ++a) bv[a] = B_data[db[a] != kNone ? (int64_t)bs[a] + k : 0];
+    group_fence();
+#pragma unroll
+    for (int a = 0; a < kCap; ++a) {
+        // the lanes of a group hold different entries of one B row: different columns, different
+        // accumulators; the entries of A take their turns one after the other
+        if (db[a] != kNone) acc[db[a]] = acc[db[a]] + av[a] * bv[a];
+        group_fence();
+    }
+#pragma unroll
+    for (int q = 0; q < kCap; ++q)
+        if (k + kCap * q < clen) C_data[cs + k + kCap * q] = acc[k + kCap * q];
+}
+
+// ---- backward ------------------------------------------------------------------------
+
+// grad_A.  A wavefront takes 64 consecutive entries of A, eight at a time with eight lanes per
+// entry (coalesced reads of the B rows); the terms change places through LDS so that lane e
+// then adds the eight terms of entry e in ascending k.
+constexpr int kTermStride = kCap + 1;
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void grad_a_mapped_kernel(
+    int64_t A_nnz, const T *__restrict__ gC, const T *__restrict__ B_data, const int32_t *__restrict__ bstart,
+    const int32_t *__restrict__ cstart, const uint8_t *__restrict__ dest, T *__restrict__ grad_A) {
+    __shared__ T s_term[(kBlock / kWave) * kWave * kTermStride];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int k = lane & (kCap - 1), g = lane / kCap;
+    T *term = s_term + wave * kWave * kTermStride;
+    const int64_t base = ((int64_t)blockIdx.x * (kBlock / kWave) + wave) * kWave;
+    int32_t bs[kCap], cs[kCap];
+    uint8_t db[kCap];
+#pragma unroll
+    for (int p = 0; p < kCap; ++p) {
+        const int64_t e = base + p * kCap + g;
+        const int64_t es = e < A_nnz ? e : 0;
+        bs[p] = bstart[es];
+        cs[p] = cstart[es];
+        db[p] = e < A_nnz ? dest[es * kCap + k] : kNone;
+    }
+#pragma unroll
+    for (int p = 0; p < kCap; ++p) {
+        const bool have = db[p] != kNone;
+        const T gv = gC[have ? (int64_t)cs[p] + db[p] : 0];
+        const T bv = B_data[have ? (int64_t)bs[p] + k : 0];
+        term[(p * kCap + g) * kTermStride + k] = have ? gv * bv : T(0);
+    }
+    group_fence();
+    T acc = T(0);
+#pragma unroll
+    for (int q = 0; q < kCap; ++q) acc += term[lane * kTermStride + q];
+    if (base + lane < A_nnz) grad_A[base + lane] = acc;
+}
+
+// grad_B.  Eight lanes per row j of B, lane k its k-th entry; the group walks column j of A on
+// the transposed-structure plan (rows ascending), eight entries per round trip.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
+    int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
+    const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm, const int64_t *__restrict__ B_indptr,
+    const int32_t *__restrict__ cstart, const uint8_t *__restrict__ dest, T *__restrict__ grad_B) {
+    const int k = threadIdx.x & (kCap - 1);
+    const int64_t j = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + threadIdx.x / kCap;
+    if (j >= B_rows) return;
+    const int64_t bb = B_indptr[j], blen = B_indptr[j + 1] - bb;
+    const int32_t pb = t_indptr[j], pe = t_indptr[j + 1];
+    if (pb == pe) {   // no entry of A in this column: the row's gradient is zero, however long the row
+        for (int64_t q = k; q < blen; q += kCap) grad_B[bb + q] = T(0);
+        return;
+    }
+    // a named row: at most kCap entries (the plan's build checked it)
+    const bool mine = k < blen;
+    T acc = T(0);
+    for (int32_t t0 = pb; t0 < pe; t0 += kCap) {
+        int32_t e[kCap];
+#pragma unroll
+        for (int u = 0; u < kCap; ++u) e[u] = t_perm[t0 + u < pe ? t0 + u : pb];
+        T a[kCap];
+        int32_t cs[kCap];
+        uint8_t db[kCap];
+#pragma unroll
+        for (int u = 0; u < kCap; ++u) {
+            a[u] = A_data[e[u]];
+            cs[u] = cstart[e[u]];
+            db[u] = mine ? dest[(int64_t)e[u] * kCap + k] : kNone;
+        }
+        T gv[kCap];
+#pragma unroll
+        for (int u = 0; u < kCap; ++u) gv[u] = gC[db[u] != kNone ? (int64_t)cs[u] + db[u] : 0];
+#pragma unroll
+        for (int u = 0; u < kCap; ++u)
+            if (t0 + u < pe && db[u] != kNone) acc += a[u] * gv[u];
+    }
+    if (mine) grad_B[bb + k] = acc;
+}
+
+template <typename T>
+int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A_data, const nm::TPlan &t,
+                    const void *B_data, const int64_t *B_indptr, const PPlan &p, void *grad_A, void *grad_B,
+                    hipStream_t s) {
+    if (grad_A && A_nnz > 0) {
+        const int64_t grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
+        NM_REQUIRE(grid < nm::kMaxGrid, "too many entries");
+        hipLaunchKernelGGL(grad_a_mapped_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, (const T *)gC,
+                           (const T *)B_data, p.bstart, p.cstart, p.dest, (T *)grad_A);
+        NM_LAUNCH_CHECK("grad_a_mapped_kernel");
+    }
+    if (grad_B && A_cols > 0) {
+        const int64_t grid = nm::xcd_padded(nm::ceil_div(A_cols, (int64_t)kGroupsPerBlock));
+        NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+        hipLaunchKernelGGL(grad_b_mapped_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, grid,
+                           (const T *)gC, (const T *)A_data, t.t_indptr, t.t_perm, B_indptr, p.cstart, p.dest,
+                           (T *)grad_B);
+        NM_LAUNCH_CHECK("grad_b_mapped_kernel");
+    }
+    return NM_OK;
+}
+
+}  // namespace
+
+extern "C" int nm_spgemm_plan_bytes(int64_t A_nnz, size_t *plan_bytes) {
+    NM_REQUIRE(plan_bytes != nullptr && A_nnz >= 0, "bad arguments");
+    *plan_bytes = pplan_layout(A_nnz, nullptr, nullptr);
+    return NM_OK;
+}
+
+extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                                    const int64_t *A_indices, const int64_t *A_indptr, const int64_t *B_indices,
+                                    const int64_t *B_indptr, const int64_t *C_indices, const int64_t *C_indptr,
+                                    const void *A_plan_mem, void *plan_mem, size_t plan_bytes, void *host_landing,
+                                    int *usable, nm_stream stream) {
+    NM_REQUIRE(A_rows >= 0 && A_cols >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
+    NM_REQUIRE(usable && plan_mem && A_plan_mem && A_indptr && B_indptr && C_indptr, "null pointer argument");
+    NM_REQUIRE((A_nnz == 0 || A_indices) && (B_nnz == 0 || B_indices) && (C_nnz == 0 || C_indices),
+               "null pointer argument");
+    const size_t need = pplan_layout(A_nnz, nullptr, nullptr);
+    if (plan_bytes < need) return nm::fail(NM_ERR_WORKSPACE, "plan of %zu bytes, %zu needed", plan_bytes, need);
+    *usable = 0;
+    // positions are kept in 32 bits
+    const int64_t lim = (int64_t)1 << 31;
+    if (A_nnz >= lim || B_nnz >= lim || C_nnz >= lim || A_rows == 0 || A_nnz == 0) return NM_OK;
+    hipStream_t s = nm::as_stream(stream);
+    PPlan p;
+    pplan_layout(A_nnz, plan_mem, &p);
+    nm::TPlan t;
+    nm::tplan_layout(A_rows, A_cols, A_nnz, const_cast<void *>(A_plan_mem), &t);
+    if (int rc = nm::fill_async(p.flag, 16, (int32_t)0, s)) return rc;
+    int64_t grid = nm::ceil_div(A_rows, (int64_t)kGroupsPerBlock);
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(plan_map_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_indices, A_indptr,
+                       B_indices, B_indptr, C_indices, C_indptr, p);
+    NM_LAUNCH_CHECK("plan_map_kernel");
+    grid = nm::ceil_div(A_cols > 0 ? A_cols : 1, (int64_t)kBlock);
+    if (grid > 4096) grid = 4096;
+    hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, p.flag);
+    NM_LAUNCH_CHECK("plan_columns_kernel");
+    int32_t flag = 1;
+    if (host_landing) {
+        volatile int64_t *land = (volatile int64_t *)host_landing;
+        const int64_t ticket = land[2] + 1;
+        hipLaunchKernelGGL(plan_flag_out_kernel, dim3(1), dim3(64), 0, s, p.flag, land, ticket);
+        NM_LAUNCH_CHECK("plan_flag_out_kernel");
+        bool arrived = false;
+        for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = land[2] == ticket;
+        if (!arrived) {
+            NM_HIP_TRY(hipStreamSynchronize(s));
+            NM_REQUIRE(land[2] == ticket, "the plan's verdict did not arrive");
+        }
+        flag = (int32_t)land[0];
+    } else {
+        NM_HIP_TRY(hipMemcpyAsync(&flag, p.flag, sizeof(flag), hipMemcpyDeviceToHost, s));
+        NM_HIP_TRY(hipStreamSynchronize(s));
+    }
+    *usable = flag == 0 ? 1 : 0;
+    return NM_OK;
+}
+
+extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                                         const void *A_data, const int64_t *A_indptr, const void *B_data,
+                                         const void *plan_mem, const int64_t *C_indptr, void *C_data,
+                                         nm_stream stream) {
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(A_rows >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
+    if (A_rows == 0 || A_nnz == 0 || B_nnz == 0 || C_nnz == 0) return NM_OK;   // C has no entries
+    NM_REQUIRE(A_data && A_indptr && B_data && plan_mem && C_indptr && C_data, "null pointer argument");
+    PPlan p;
+    pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p);
+    hipStream_t s = nm::as_stream(stream);
+    const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)kGroupsPerBlock));
+    NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+    if (dt == NM_F32)
+        hipLaunchKernelGGL(numeric_planned_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, grid,
+                           (const float *)A_data, A_indptr, (const float *)B_data, p.bstart, p.dest, C_indptr,
+                           (float *)C_data);
+    else
+        hipLaunchKernelGGL(numeric_planned_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, grid,
+                           (const double *)A_data, A_indptr, (const double *)B_data, p.bstart, p.dest, C_indptr,
+                           (double *)C_data);
+    NM_LAUNCH_CHECK("numeric_planned_kernel");
+    return NM_OK;
+}
+
+extern "C" int nm_spgemm_backward_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz,
+                                         int64_t C_nnz, const void *gC, const void *A_data,
+                                         const void *A_plan_mem, const void *B_data, const int64_t *B_indptr,
+                                         const void *plan_mem, void *grad_A, void *grad_B, nm_stream stream) {
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(A_rows >= 0 && A_cols >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
+    NM_REQUIRE(A_nnz > 0 && A_rows > 0, "a product plan exists only for a matrix with entries");
+    if (!grad_A && !grad_B) return NM_OK;
+    hipStream_t s = nm::as_stream(stream);
+    if (B_nnz == 0 || C_nnz == 0) {
+        // no product reaches a stored entry of C: both gradients are zero
+        if (grad_A) {
+            int rc = dt == NM_F32 ? nm::fill_async((float *)grad_A, A_nnz, 0.0f, s)
+                                  : nm::fill_async((double *)grad_A, A_nnz, 0.0, s);
+            if (rc) return rc;
+        }
+        if (grad_B && B_nnz > 0) {
+            int rc = dt == NM_F32 ? nm::fill_async((float *)grad_B, B_nnz, 0.0f, s)
+                                  : nm::fill_async((double *)grad_B, B_nnz, 0.0, s);
+            if (rc) return rc;
+        }
+        return NM_OK;
+    }
+    NM_REQUIRE(gC && A_data && A_plan_mem && B_data && B_indptr && plan_mem, "null pointer argument");
+    PPlan p;
+    pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p);
+    nm::TPlan t;
+    nm::tplan_layout(A_rows, A_cols, A_nnz, const_cast<void *>(A_plan_mem), &t);
+    if (dt == NM_F32)
+        return launch_backward<float>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s);
+    return launch_backward<double>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s);
+}

@@ -169,13 +169,17 @@ struct Alias {
 };
 
 struct Plan {
-    char kind;  // 'T' transposed structure, 'L' level schedule, 'U' filled pattern of the LU factors
-    Key key;
+    // 'T' transposed structure, 'L' level schedule, 'U' filled pattern of the LU factors,
+    // 'P' product plan of A B (key: A's pattern, key2: B's)
+    char kind;
+    Key key, key2;
     int64_t a, b;
     Tensor mem;
     size_t bytes = 0;
-    std::vector<Tensor> derived;             // 'U': structure tensors handed out to callers
+    std::vector<Tensor> derived;             // 'U', 'P': structure tensors handed out to callers
     std::vector<uint32_t> derived_versions;  //      and their version counters when built
+    bool usable = true;                      // 'P': false when the product is beyond the plan's limits
+    std::shared_ptr<Plan> parent;            // 'P': the transposed-structure plan of A it walks
     nm_sptrsv_plan *handle = nullptr;
     // the stream the plan was built on and the event that marks its completion there
     c10::StreamId build_stream = 0;
@@ -187,7 +191,7 @@ struct Plan {
 
 struct Sighting {
     char kind;
-    Key key;
+    Key key, key2;
     int64_t a, b;
 };
 
@@ -276,10 +280,10 @@ void join_plan(const Plan &plan, const c10::Device &dev) {
         c10::hip::HIPCachingAllocator::recordStream(plan.mem.storage().data_ptr(), stream.hip_stream());
 }
 
-std::shared_ptr<Plan> find_plan_locked(char kind, const Key &key, int64_t a, int64_t b) {
+std::shared_ptr<Plan> find_plan_locked(char kind, const Key &key, int64_t a, int64_t b, const Key &key2 = Key()) {
     for (auto it = g_plans.begin(); it != g_plans.end(); ++it) {
         Plan &p = **it;
-        if (p.kind == kind && p.key == key && p.a == a && p.b == b) {
+        if (p.kind == kind && p.key == key && p.key2 == key2 && p.a == a && p.b == b) {
             if (it != g_plans.begin()) g_plans.splice(g_plans.begin(), g_plans, it);
             return g_plans.front();
         }
@@ -319,13 +323,13 @@ std::shared_ptr<Plan> cached(char kind, const Tensor &indices, const Tensor &ind
         if (second_sighting) {
             bool seen = false;
             for (auto it = g_sightings.begin(); it != g_sightings.end(); ++it)
-                if (it->kind == kind && it->key == key && it->a == a && it->b == b) {
+                if (it->kind == kind && it->key == key && it->key2 == Key() && it->a == a && it->b == b) {
                     g_sightings.erase(it);
                     seen = true;
                     break;
                 }
             if (!seen) {
-                g_sightings.push_front(Sighting{kind, key, a, b});
+                g_sightings.push_front(Sighting{kind, key, Key(), a, b});
                 while (g_sightings.size() > kSightingTableSize) g_sightings.pop_back();
                 return nullptr;
             }
@@ -396,6 +400,123 @@ std::shared_ptr<Plan> level_plan(const Tensor &indices, const Tensor &indptr, in
                                 current_stream(dev)),
               "nm_sptrsv_analyse");  // synchronises its stream
     });
+}
+
+// ---- product plans ---------------------------------------------------------------
+//
+// A product A B whose rows all stay on the merge path (nm_spgemm_symbolic_result reports no row
+// on the hash path) can be given a product plan: the pattern of C and, per entry of A, where its
+// products go.  With it a forward pass is one numeric kernel and a backward pass two gather
+// kernels; the values are the ones the stateless kernels give, bit for bit.  The plan is keyed
+// on the content of both patterns and follows the policy of the transposed-structure plans:
+// built the second time the pair is seen ("planned"), at once ("eager"), never ("atomic").
+// Results of planned forward passes SHARE the plan's C_indices / C_indptr tensors (the pattern
+// is the same by construction); a plan whose tensors have been written to in place is dropped.
+
+void drop_plan(const std::shared_ptr<Plan> &plan) {
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    for (auto it = g_plans.begin(); it != g_plans.end(); ++it)
+        if (*it == plan) {
+            g_plan_bytes -= plan->bytes;
+            g_plans.erase(it);
+            return;
+        }
+}
+
+// The product plan of the pair; nullptr when there is none or its pattern tensors were edited.
+// With `compute` false the pair is looked up through the alias table only (no key is computed:
+// what a call may do before it knows whether the product is eligible at all).
+std::shared_ptr<Plan> peek_product_plan(const Tensor &A_indices, const Tensor &A_indptr, const Tensor &B_indices,
+                                        const Tensor &B_indptr, int64_t A_rows, int64_t B_cols,
+                                        const c10::Device &dev, bool compute = false) {
+    Key ka, kb;
+    if (!structure_key(A_indices, A_indptr, compute, &ka) || !structure_key(B_indices, B_indptr, compute, &kb))
+        return nullptr;
+    std::shared_ptr<Plan> plan;
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        plan = find_plan_locked('P', ka, A_rows, B_cols, kb);
+    }
+    if (!plan) return nullptr;
+    for (size_t i = 0; i < plan->derived.size(); ++i)
+        if (plan->derived[i]._version() != plan->derived_versions[i]) {
+            drop_plan(plan);
+            return nullptr;
+        }
+    join_plan(*plan, dev);
+    if (plan->parent) join_plan(*plan->parent, dev);
+    return plan;
+}
+
+// After a stateless forward pass of a product without hash-path rows: notes the pair, or builds
+// its plan around the pattern of C that the pass has just produced.
+void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, const Tensor &B_indices,
+                           const Tensor &B_indptr, const Tensor &C_indices, const Tensor &C_indptr,
+                           int64_t A_rows, int64_t A_cols, int64_t B_cols, const c10::Device &dev) {
+    const int mode = backward_mode_now();
+    if (mode == kAtomic || A_indices.numel() == 0 || C_indices.numel() == 0) return;
+    Key ka, kb;
+    structure_key(A_indices, A_indptr, true, &ka);
+    structure_key(B_indices, B_indptr, true, &kb);
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        if (find_plan_locked('P', ka, A_rows, B_cols, kb)) return;   // e.g. one that turned out unusable
+        if (mode == kPlanned) {
+            bool seen = false;
+            for (auto it = g_sightings.begin(); it != g_sightings.end(); ++it)
+                if (it->kind == 'P' && it->key == ka && it->key2 == kb && it->a == A_rows && it->b == B_cols) {
+                    g_sightings.erase(it);
+                    seen = true;
+                    break;
+                }
+            if (!seen) {
+                g_sightings.push_front(Sighting{'P', ka, kb, A_rows, B_cols});
+                while (g_sightings.size() > kSightingTableSize) g_sightings.pop_back();
+                return;
+            }
+        }
+    }
+    auto plan = std::make_shared<Plan>();
+    plan->kind = 'P';
+    plan->key = ka;
+    plan->key2 = kb;
+    plan->a = A_rows;
+    plan->b = B_cols;
+    plan->parent = transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev);
+    size_t pbytes = 0;
+    check(nm_spgemm_plan_bytes(A_indices.numel(), &pbytes), "nm_spgemm_plan_bytes");
+    plan->mem = scratch(pbytes, dev);
+    int usable = 0;
+    check(nm_spgemm_plan_build(A_rows, A_cols, A_indices.numel(), B_indices.numel(), C_indices.numel(),
+                               A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                               B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                               C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(),
+                               plan->parent->mem.data_ptr(), plan->mem.data_ptr(), pbytes, host_landing(), &usable,
+                               current_stream(dev)),
+          "nm_spgemm_plan_build");
+    plan->usable = usable != 0;
+    if (plan->usable) {
+        plan->derived = {C_indices, C_indptr};
+        for (const Tensor &t : plan->derived) plan->derived_versions.push_back(t._version());
+    } else {
+        plan->mem = Tensor();   // remembered as unusable, so that the pair is not analysed again
+        plan->parent.reset();
+    }
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev.index());
+    plan->build_stream = stream.id();
+    plan->ready = std::make_unique<at::cuda::CUDAEvent>();
+    plan->ready->record(stream);
+    plan->bytes = plan->mem.defined() ? (size_t)plan->mem.nbytes() : 0;
+    for (const Tensor &t : plan->derived) plan->bytes += (size_t)t.nbytes();
+    g_plans_built.fetch_add(1, std::memory_order_relaxed);
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    g_plans.push_front(plan);
+    g_plan_bytes += plan->bytes;
+    const size_t limit = g_plan_bytes_limit.load(std::memory_order_relaxed);
+    while (g_plans.size() > 1 && g_plan_bytes > limit) {
+        g_plan_bytes -= g_plans.back()->bytes;
+        g_plans.pop_back();
+    }
 }
 
 Tensor solve(const Plan &plan, bool transposed, const Tensor &A_data, bool unit, const Tensor &b, int64_t rows,
@@ -765,6 +886,21 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     B_indices = index_tensor(B_indices, "B_indices");
     B_indptr = index_tensor(B_indptr, "B_indptr");
     c10::hip::HIPGuard guard(dev.index());
+    const bool plans = backward_mode_now() != kAtomic;
+    auto on_plan = [&](const Plan &plan) -> std::vector<Tensor> {
+        const Tensor &C_indices = plan.derived[0], &C_indptr = plan.derived[1];
+        Tensor C_data = torch::empty({C_indices.numel()}, A_data.options());
+        check(nm_spgemm_numeric_planned(dtype_of(A_data), A_rows, A_data.numel(), B_data.numel(), C_indices.numel(),
+                                        A_data.data_ptr(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
+                                        plan.mem.data_ptr(), C_indptr.data_ptr<int64_t>(), C_data.data_ptr(),
+                                        current_stream(dev)),
+              "nm_spgemm_numeric_planned");
+        return {C_data, C_indices, C_indptr};
+    };
+    if (plans) {
+        auto plan = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, A_rows, B_cols, dev);
+        if (plan && plan->usable) return on_plan(*plan);
+    }
     size_t bytes = 0;
     check(nm_spgemm_workspace_bytes(A_rows, B_cols, &bytes), "nm_spgemm_workspace_bytes");
     Tensor work = scratch(bytes, dev);
@@ -780,6 +916,12 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     check(nm_spgemm_symbolic_result(A_rows, B_cols, work.data_ptr(), bytes, &nnz_c, &hash_rows, host_landing(),
                                     st),
           "nm_spgemm_symbolic_result");
+    if (plans && hash_rows == 0 && nnz_c > 0) {
+        // eligible for a product plan: worth a content key per pattern that arrives in tensors not
+        // seen before (a clone, a product computed again), which may find the pair's plan
+        auto plan = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, A_rows, B_cols, dev, true);
+        if (plan && plan->usable) return on_plan(*plan);
+    }
     Tensor C_indices = torch::empty({nnz_c}, iopt);
     Tensor C_data = torch::empty({nnz_c}, A_data.options());
     check(nm_spgemm_numeric(dtype_of(A_data), A_rows, A_cols, B_cols, A_data.data_ptr(),
@@ -788,6 +930,9 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
                             C_indptr.data_ptr<int64_t>(), C_indices.data_ptr<int64_t>(), C_data.data_ptr(),
                             work.data_ptr(), bytes, hash_rows, st),
           "nm_spgemm_numeric");
+    if (hash_rows == 0)
+        consider_product_plan(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr, A_rows, A_cols, B_cols,
+                              dev);
     return {C_data, C_indices, C_indptr};
 }
 
@@ -813,6 +958,20 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
     C_indptr = index_tensor(C_indptr, "C_indptr");
     c10::hip::HIPGuard guard(dev.index());
     Tensor grad_A = torch::empty_like(A_data), grad_B = torch::empty_like(B_data);
+    if (backward_mode_now() != kAtomic) {
+        // the product plan applies when grad_C lies on the very pattern tensors the plan handed out
+        auto pp = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, A_rows, B_cols, dev);
+        if (pp && pp->usable && pp->derived[0].data_ptr() == C_indices.data_ptr() &&
+            pp->derived[1].data_ptr() == C_indptr.data_ptr() && pp->derived[0].numel() == C_indices.numel()) {
+            check(nm_spgemm_backward_mapped(dtype_of(A_data), A_rows, A_cols, A_data.numel(), B_data.numel(),
+                                            grad_C.numel(), grad_C.data_ptr(), A_data.data_ptr(),
+                                            pp->parent->mem.data_ptr(), B_data.data_ptr(),
+                                            B_indptr.data_ptr<int64_t>(), pp->mem.data_ptr(), grad_A.data_ptr(),
+                                            grad_B.data_ptr(), current_stream(dev)),
+                  "nm_spgemm_backward_mapped");
+            return {grad_A, grad_B};
+        }
+    }
     // The plan-based kernel looks every column of a row of B up in a staged row of C per entry of
     // A, the stateless one stages a row of C once and looks the rows of B up in it: with rows of C
     // many times longer than rows of B the stateless kernel is the faster one, and the default mode

@@ -547,6 +547,60 @@ def spgemm_backward(grad_C, C_indices, C_indptr,
     return [grad_A, grad_B]
 
 
+class ProductPlan:
+    """Product plan of C = A B (nm_spgemm_plan_build): numeric product and gradients of a product
+    whose three patterns are known, without the symbolic phase and without searches.
+
+    ``usable`` is False when a row is longer than the plan's limits; then neither method may be
+    called.  The plan keeps the structure tensors it was built from alive.
+    """
+
+    def __init__(self, A_rows, A_cols, A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr):
+        dev = _need_device(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr)
+        L = _lib.lib()
+        self.dev, self.A_rows, self.A_cols = dev, A_rows, A_cols
+        self.A_nnz, self.B_nnz, self.C_nnz = A_indices.shape[0], B_indices.shape[0], C_indices.shape[0]
+        self.A_indptr, self.B_indptr, self.C_indptr, self.C_indices = A_indptr, B_indptr, C_indptr, C_indices
+        with torch.cuda.device(dev):
+            self.transposed = _transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev)
+            nbytes = ctypes.c_size_t(0)
+            _lib.check(L.nm_spgemm_plan_bytes(self.A_nnz, ctypes.byref(nbytes)), "nm_spgemm_plan_bytes")
+            self.mem = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+            usable = ctypes.c_int(0)
+            _lib.check(L.nm_spgemm_plan_build(
+                A_rows, A_cols, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(A_indices), _ptr(A_indptr),
+                _ptr(B_indices), _ptr(B_indptr), _ptr(C_indices), _ptr(C_indptr), _ptr(self.transposed.mem),
+                _ptr(self.mem), nbytes.value, _ptr(_host_landing()), ctypes.byref(usable), _stream(dev)),
+                "nm_spgemm_plan_build")
+            self.usable = bool(usable.value)
+
+    def numeric(self, A_data, B_data):
+        """C_data of the product (the pattern is the one the plan was built from)."""
+        if not self.usable:
+            raise RuntimeError("this product has rows beyond the plan's limits")
+        A_data, B_data = A_data.contiguous(), B_data.contiguous()
+        with torch.cuda.device(self.dev):
+            C_data = torch.empty(self.C_nnz, dtype=A_data.dtype, device=self.dev)
+            _lib.check(_lib.lib().nm_spgemm_numeric_planned(
+                _dt(A_data), self.A_rows, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(A_data), _ptr(self.A_indptr),
+                _ptr(B_data), _ptr(self.mem), _ptr(self.C_indptr), _ptr(C_data), _stream(self.dev)),
+                "nm_spgemm_numeric_planned")
+        return C_data
+
+    def backward(self, grad_C, A_data, B_data):
+        """[grad_A, grad_B] of grad_C laid out on the plan's pattern of C."""
+        if not self.usable:
+            raise RuntimeError("this product has rows beyond the plan's limits")
+        A_data, B_data, grad_C = A_data.contiguous(), B_data.contiguous(), grad_C.contiguous()
+        with torch.cuda.device(self.dev):
+            grad_A, grad_B = torch.empty_like(A_data), torch.empty_like(B_data)
+            _lib.check(_lib.lib().nm_spgemm_backward_mapped(
+                _dt(A_data), self.A_rows, self.A_cols, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(grad_C),
+                _ptr(A_data), _ptr(self.transposed.mem), _ptr(B_data), _ptr(self.B_indptr), _ptr(self.mem),
+                _ptr(grad_A), _ptr(grad_B), _stream(self.dev)), "nm_spgemm_backward_mapped")
+        return [grad_A, grad_B]
+
+
 # ------------------------------------------------------------------- SpTRSV
 
 class _Plan:

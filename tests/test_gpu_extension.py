@@ -230,10 +230,96 @@ def test_loop_of_fresh_products_builds_one_plan_per_pattern(dev, cpp):
         (C @ X).sum().backward()
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
-    # C's pattern for the SpMV backward, and at most A's own for the product's backward
-    assert cpp.plan_cache_stats()[0] - built0 <= 2 and cpp.plan_cache_size() <= 2
+    # C's pattern for the SpMV backward, A's own for the product's backward, and the product plan of A A
+    assert cpp.plan_cache_stats()[0] - built0 <= 3 and cpp.plan_cache_size() <= 3
     steady = sorted(times[3:])[len(times[3:]) // 2]
     assert max(times[3:]) <= 2.0 * steady, times
+    cpp.clear_plan_cache()
+
+
+def test_product_plan_policy(dev, cpp):
+    """A product without hash-path rows: the first call runs the stateless kernels and builds
+    nothing, the second builds the product plan around its own result, later calls run on the plan
+    and hand out the plan's pattern tensors; values and gradients stay bit-identical to the oracle's
+    for new values on the same patterns.  An in-place edit of a handed-out pattern tensor drops the
+    plan; "atomic" never plans; a product beyond the plan's limits is remembered as such."""
+    dtype = np.float64
+    d, i, p, (n, _) = G.laplace3d(10, dtype, 2)
+    I, P = to_dev(dev, i, p)
+
+    def check(call, seed):
+        a, b = randn(seed, d.shape[0], dtype), randn(seed + 1, d.shape[0], dtype)
+        A, B = to_dev(dev, a, b)
+        C_data, C_indices, C_indptr = cpp.spgemm_forward(n, n, A, I, P, n, n, B, I, P)
+        cd, ci, cp = oracle.spgemm_forward(n, n, a, i, p, n, n, b, i, p)
+        assert_same(host(C_indptr), cp, f"{call}: C_indptr")
+        assert_same(host(C_indices), ci, f"{call}: C_indices")
+        assert_same(host(C_data), cd, f"{call}: C_data")
+        g = randn(seed + 2, cd.shape[0], dtype)
+        gA, gB = cpp.spgemm_backward(to_dev(dev, g)[0], C_indices, C_indptr, n, n, A, I, P, n, n, B, I, P)
+        rA, rB = oracle.spgemm_backward(g, ci, cp, n, n, a, i, p, n, n, b, i, p)
+        assert_same(host(gA), rA, f"{call}: grad_A")
+        return C_indices, C_indptr, host(gB), rB
+
+    cpp.clear_plan_cache()
+    cpp.set_backward_mode("planned")
+    built0 = cpp.plan_cache_stats()[0]
+    check("first call", 1)                                   # stateless forward; backward: first sighting of A
+    assert cpp.plan_cache_stats()[0] == built0
+    ci2, cp2, gB, rB = check("second call", 4)               # builds A's transposed plan and the product plan
+    assert cpp.plan_cache_stats()[0] == built0 + 2 and cpp.plan_cache_size() == 2
+    assert_same(gB, rB, "second call: grad_B (mapped, bitwise)")
+    ci3, cp3, gB, rB = check("third call", 7)                # numeric kernel only, on the plan
+    assert ci3.data_ptr() == ci2.data_ptr() and cp3.data_ptr() == cp2.data_ptr(), "the plan's pattern tensors"
+    assert cpp.plan_cache_stats()[0] == built0 + 2
+    assert_same(gB, rB, "third call: grad_B (mapped, bitwise)")
+    # a gradient laid out on OTHER tensors of the same pattern takes the search-based kernels
+    ci4, cp4 = ci3.clone(), cp3.clone()
+    a, b = randn(20, d.shape[0], dtype), randn(21, d.shape[0], dtype)
+    g = randn(22, ci4.shape[0], dtype)
+    A, B = to_dev(dev, a, b)
+    gA, gB = cpp.spgemm_backward(to_dev(dev, g)[0], ci4, cp4, n, n, A, I, P, n, n, B, I, P)
+    rA, rB = oracle.spgemm_backward(g, host(ci4), host(cp4), n, n, a, i, p, n, n, b, i, p)
+    assert_same(host(gA), rA, "grad_A on foreign pattern tensors")
+    assert_same(host(gB), rB, "grad_B on foreign pattern tensors")
+    # an in-place edit of a handed-out pattern tensor: the plan is dropped, results stay right
+    ci3.add_(0)
+    ci5, _, _, _ = check("after an in-place edit", 10)
+    assert ci5.data_ptr() != ci3.data_ptr()
+    # "atomic": no plan is looked for or built
+    cpp.clear_plan_cache()
+    cpp.set_backward_mode("atomic")
+    for seed in (30, 33, 36):
+        check("atomic mode", seed)
+    assert cpp.plan_cache_size() == 0
+    # "eager": the plan is built by the first call; the pattern in fresh tensors finds it
+    cpp.set_backward_mode("eager")
+    built1 = cpp.plan_cache_stats()[0]
+    ci6, _, _, _ = check("eager, first call", 40)
+    assert cpp.plan_cache_stats()[0] == built1 + 2
+    I_saved, P_saved = I, P
+    I, P = I.clone(), P.clone()
+    ci7, _, gB, rB = check("eager, cloned patterns", 43)
+    assert ci7.data_ptr() == ci6.data_ptr() and cpp.plan_cache_stats()[0] == built1 + 2
+    assert_same(gB, rB, "grad_B through cloned patterns")
+    I, P = I_saved, P_saved
+    # a product with a row of nine entries has no hash-path row only if ... it has one: not eligible;
+    # one whose rows of B are too long for the plan but short enough for the merge path does not exist
+    # either (both limits are eight), so "unusable" arises from long columns of A only
+    cpp.clear_plan_cache()
+    rows = 5000
+    ai = np.zeros(rows, dtype=np.int64)                      # every row of A names column 0
+    ap = np.arange(rows + 1, dtype=np.int64)
+    ad = randn(50, rows, dtype)
+    bd, bi, bp, _ = G.ragged_csr(3, 40, 4, 51, dtype, min_len=2)
+    AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+    for _ in range(3):
+        C_data, C_indices, C_indptr = cpp.spgemm_forward(rows, 3, AD, AI, AP, 3, 40, BD, BI, BP)
+        cd, ci, cp = oracle.spgemm_forward(rows, 3, ad, ai, ap, 3, 40, bd, bi, bp)
+        assert_same(host(C_data), cd, "long column of A: C_data")
+        assert_same(host(C_indices), ci, "long column of A: C_indices")
+    assert cpp.plan_cache_stats()[0] == built1 + 2 + 2       # A's transposed plan and the (unusable) product plan, once
+    cpp.set_backward_mode("planned")
     cpp.clear_plan_cache()
 
 

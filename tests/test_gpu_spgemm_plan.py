@@ -1,0 +1,125 @@
+"""Product plan of a sparse product (nm_spgemm_plan_build and the kernels that run on it).
+
+The planned numeric product and the mapped gradients must reproduce, bit for bit, what the
+stateless SpGEMM kernels and the CPU oracle give (whose sums run in the order of
+cpp/sparse_csr_cpu.cpp:177-303): structure is exact, values are compared with assert_same.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as mirror
+from util import assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+
+def _short_rows(rows, cols, max_len, seed, dtype, min_len=0):
+    return G.ragged_csr(rows, cols, max_len, seed, dtype, min_len=min_len)
+
+
+def _cases(dtype):
+    yield "poisson2d x poisson2d", G.poisson2d(23, dtype, jitter_seed=1), G.poisson2d(23, dtype, jitter_seed=2)
+    yield "laplace3d x laplace3d", G.laplace3d(9, dtype, jitter_seed=3), G.laplace3d(9, dtype, jitter_seed=4)
+    yield "tridiag x tridiag", G.tridiag(300, dtype), G.tridiag(300, dtype)
+    a = _short_rows(500, 300, 8, 5, dtype)
+    b = _short_rows(300, 700, 8, 6, dtype)
+    yield "ragged rectangular, empty rows", a, b
+    a = _short_rows(64, 40, 8, 7, dtype, min_len=8)
+    b = _short_rows(40, 4000, 8, 8, dtype, min_len=8)
+    yield "every row full: 64 entries per row of C", a, b
+    a = _short_rows(1, 1, 1, 9, dtype, min_len=1)
+    yield "one by one", a, a
+
+
+def _unpack(m):
+    d, i, p = m[0], m[1], m[2]
+    shape = m[3] if len(m) > 3 else None
+    return d, i, p, shape
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_planned_product_and_gradients_match_the_stateless_kernels_and_the_oracle(dev, dtype):
+    for name, A, B in _cases(dtype):
+        ad, ai, ap, ashape = _unpack(A)
+        bd, bi, bp, bshape = _unpack(B)
+        A_rows, A_cols = ashape
+        B_rows, B_cols = bshape
+        assert A_cols == B_rows, name
+        AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+        C_data, C_indices, C_indptr = mirror.spgemm_forward(A_rows, A_cols, AD, AI, AP, B_rows, B_cols, BD, BI, BP)
+        plan = mirror.ProductPlan(A_rows, A_cols, AI, AP, BI, BP, C_indices, C_indptr)
+        assert plan.usable, name
+        # new values on the same patterns: the plan knows nothing of the values it was built beside
+        ad2, bd2 = randn(11, ad.shape[0], dtype), randn(12, bd.shape[0], dtype)
+        AD2, BD2 = to_dev(dev, ad2, bd2)
+        ref_data, ref_indices, ref_indptr = mirror.spgemm_forward(A_rows, A_cols, AD2, AI, AP, B_rows, B_cols, BD2,
+                                                                  BI, BP)
+        assert_same(host(ref_indices), host(C_indices), f"{name}: pattern")
+        got = plan.numeric(AD2, BD2)
+        assert_same(host(got), host(ref_data), f"{name}: C_data vs stateless kernels")
+        cd, ci, cp = oracle.spgemm_forward(A_rows, A_cols, ad2, ai, ap, B_rows, B_cols, bd2, bi, bp)
+        assert_same(host(got), cd, f"{name}: C_data vs oracle")
+        g = randn(13, cd.shape[0], dtype)
+        Gz, = to_dev(dev, g)
+        gA, gB = plan.backward(Gz, AD2, BD2)
+        rA, rB = oracle.spgemm_backward(g, ci, cp, A_rows, A_cols, ad2, ai, ap, B_rows, B_cols, bd2, bi, bp)
+        assert_same(host(gA), rA, f"{name}: grad_A vs oracle")
+        assert_same(host(gB), rB, f"{name}: grad_B vs oracle")
+        old = mirror.BACKWARD_MODE
+        mirror.BACKWARD_MODE = "eager"
+        try:
+            sA, sB = mirror.spgemm_backward(Gz, C_indices, C_indptr, A_rows, A_cols, AD2, AI, AP, B_rows, B_cols,
+                                            BD2, BI, BP)
+        finally:
+            mirror.BACKWARD_MODE = old
+        assert_same(host(gA), host(sA), f"{name}: grad_A vs the search-based kernel")
+        assert_same(host(gB), host(sB), f"{name}: grad_B vs the search-based kernel")
+
+
+def test_signed_zeros_and_explicit_zeros_keep_the_serial_result(dev):
+    dtype = np.float64
+    ad, ai, ap, ashape = _unpack(G.poisson2d(12, dtype))
+    bd, bi, bp, bshape = _unpack(G.poisson2d(12, dtype))
+    ad = ad.copy()
+    bd = bd.copy()
+    ad[::3] = 0.0
+    ad[1::7] = -0.0
+    bd[::4] = -1.0
+    bd[2::5] = 0.0
+    n = ashape[0]
+    AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+    C_data, C_indices, C_indptr = mirror.spgemm_forward(n, n, AD, AI, AP, n, n, BD, BI, BP)
+    plan = mirror.ProductPlan(n, n, AI, AP, BI, BP, C_indices, C_indptr)
+    assert plan.usable
+    got = plan.numeric(AD, BD)
+    cd, ci, cp = oracle.spgemm_forward(n, n, ad, ai, ap, n, n, bd, bi, bp)
+    assert np.array_equal(np.signbit(host(got)), np.signbit(cd)), "signs of zeros"
+    assert_same(host(got), cd, "C_data")
+
+
+def test_rows_beyond_the_limits_are_refused(dev):
+    dtype = np.float64
+    # a row of A with nine entries
+    ad, ai, ap, ashape = _unpack(_short_rows(50, 60, 9, 21, dtype, min_len=9))
+    bd, bi, bp, bshape = _unpack(_short_rows(60, 80, 4, 22, dtype))
+    AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+    _, C_indices, C_indptr = mirror.spgemm_forward(50, 60, AD, AI, AP, 60, 80, BD, BI, BP)
+    assert not mirror.ProductPlan(50, 60, AI, AP, BI, BP, C_indices, C_indptr).usable
+    # a named row of B with nine entries
+    ad, ai, ap, ashape = _unpack(_short_rows(50, 60, 4, 23, dtype, min_len=1))
+    bd, bi, bp, bshape = _unpack(_short_rows(60, 80, 9, 24, dtype, min_len=9))
+    AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+    _, C_indices, C_indptr = mirror.spgemm_forward(50, 60, AD, AI, AP, 60, 80, BD, BI, BP)
+    plan = mirror.ProductPlan(50, 60, AI, AP, BI, BP, C_indices, C_indptr)
+    assert not plan.usable
+    with pytest.raises(RuntimeError):
+        plan.numeric(AD, BD)
+    # a pattern of C that is not the product's
+    ad, ai, ap, ashape = _unpack(G.tridiag(40, dtype))
+    AD, AI, AP = to_dev(dev, ad, ai, ap)
+    assert not mirror.ProductPlan(40, 40, AI, AP, AI, AP, AI, AP).usable
