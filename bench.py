@@ -341,9 +341,30 @@ class SpGEMM(Workload):
             L, self.hostL = R, self.hostR
         self.L, self.R = L, R
         self.rows, self.cols, self.nnz = rows, cols, int(L[0].shape[0])
+        # The first steps on a new pair of patterns are timed one by one: in the default mode the
+        # second one builds the product plan (and the transposed-structure plan under it) when no
+        # row of the product needs the hash path.
+        # (one step in the stateless mode first, which notes and plans nothing: it takes the
+        # one-time costs of a process -- code objects loaded, allocator pools grown -- out of the way)
+        mode = _binding.backward_mode()
+        _binding.set_backward_mode("atomic")
         C = ext.spgemm_forward(rows, cols, *L, rows, cols, *R)
         self.nnzC = C[0].shape[0]
         self.gC = torch.from_numpy(np.random.default_rng(1).standard_normal(self.nnzC)).to(dev)
+        ext.spgemm_backward(self.gC, C[1], C[2], rows, cols, *L, rows, cols, *R)
+        _binding.set_backward_mode(mode)
+        ext.clear_plan_cache()
+        firsts = []
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            C = ext.spgemm_forward(rows, cols, *L, rows, cols, *R)
+            ext.spgemm_backward(self.gC, C[1], C[2], rows, cols, *L, rows, cols, *R)
+            torch.cuda.synchronize()
+            firsts.append(round((time.perf_counter() - t0) * 1e3, 3))
+        self.first_steps_ms = firsts
+        self.planned = (_binding.backward_mode() != "atomic" and _binding.name == "compiled"
+                        and self.left == "A")
         self.C = C
         lens = np.diff(p)
         self.products = int(lens[self.hostL[1]].sum())
@@ -355,12 +376,25 @@ class SpGEMM(Workload):
         # read again for every product) is an upper bound and is reported apart; most of those
         # reads are served by the caches.
         self.bytes_per_step = self.nnz * (s + 8) + nnzR * (s + 8) + self.nnzC * (s + 8) + 2 * rows * 8
+        self.stateless_forward_bytes = self.bytes_per_step
         self.dominant_bytes = self.bytes_per_step
         self.dominant_name = "spgemm forward (symbolic + numeric launches, host read of nnz(C) included)"
+        if self.planned:
+            # forward on the product plan: values of both operands, 12 bytes of plan per entry of
+            # the left operand (row start in B, eight destination bytes), both row pointer arrays,
+            # the values of C; the pattern of C is the plan's and is not written again
+            self.bytes_per_step = self.nnz * (s + 12) + nnzR * s + self.nnzC * s + 2 * rows * 8
+            self.dominant_bytes = self.bytes_per_step
+            self.dominant_name = "numeric_planned_kernel (the whole forward on the product plan)"
         self.config = {"workload": f"spgemm_{self.left}xA_fwd_bwd_f64_laplace3d_{n}", "rows": rows,
                        "nnz_left": self.nnz, "nnz_right": nnzR,
                        "nnz_C": self.nnzC, "products": self.products, "index_bytes": 8,
-                       "forward_compulsory_bytes": self.bytes_per_step,
+                       "mode": ("product plan (pattern of C and the destination of every product kept per pair of "
+                                "patterns; values, and both gradients, recomputed every step)"
+                                if self.planned else "stateless (symbolic + numeric every step)"),
+                       "first_three_steps_ms": firsts,
+                       "forward_bytes": self.bytes_per_step,
+                       "forward_compulsory_bytes": self.stateless_forward_bytes,
                        "forward_gather_inclusive_bytes": (self.nnz * (s + 8) + rows * 8
                                                           + self.products * (s + 8)
                                                           + self.nnzC * (s + 8) + rows * 8)}
@@ -370,6 +404,48 @@ class SpGEMM(Workload):
         g = self.ext.spgemm_backward(self.gC, C[1], C[2], self.rows, self.cols, *self.L,
                                      self.rows, self.cols, *self.R)
         return C, g
+
+    def after(self, rec, steps):
+        """The same step with no plan of any kind (symbolic + numeric forward, search-free atomic
+        backward), the cost of building the plans, and the steps after which they have paid off."""
+        import torch
+        from numml_amd import _binding
+        if not self.planned:
+            return
+        mode = _binding.backward_mode()
+        _binding.set_backward_mode("atomic")
+        self.ext.clear_plan_cache()
+        try:
+            for _ in range(3):
+                self.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                self.step()
+            torch.cuda.synchronize()
+            stateless = (time.perf_counter() - t0) / steps * 1e3
+            evs = []
+            for _ in range(steps):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                self.dominant()
+                e1.record()
+                evs.append((e0, e1))
+            torch.cuda.synchronize()
+            fwd = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+        finally:
+            _binding.set_backward_mode(mode)
+        build = max(self.first_steps_ms) - stateless
+        gain = stateless - rec["ms_per_step"]
+        c = rec["config"]
+        c["stateless_ms_per_step"] = round(stateless, 5)
+        c["stateless_GFLOPs"] = round(self.flops / (stateless * 1e-3) / 1e9, 3)
+        c["stateless_forward_ms"] = round(fwd, 5)
+        c["stateless_forward_frac_of_hbm_peak_on_compulsory_bytes"] = round(
+            self.stateless_forward_bytes / (fwd * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        c["plan_build_ms"] = round(build, 3)
+        c["plan_break_even_steps"] = int(np.ceil(build / gain)) if gain > 0 else None
+        c["amortised_ms_per_step_over_100_steps"] = round(rec["ms_per_step"] + build / 100, 5)
 
     def dominant(self):
         return self.ext.spgemm_forward(self.rows, self.cols, *self.L, self.rows, self.cols, *self.R)

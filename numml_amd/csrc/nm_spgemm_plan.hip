@@ -131,6 +131,13 @@ __global__ void plan_flag_out_kernel(const int32_t *flag, volatile int64_t *host
 }
 
 // ---- forward -----------------------------------------------------------------------
+//
+// A vector memory instruction costs the address unit the same sixteen or so cycles whether its
+// 64 lanes fetch 512 bytes or eight lanes' worth, and these kernels are bound by the number of such
+// instructions, not by bytes.  So whatever belongs to an ENTRY (its value, where its rows start,
+// its destination bytes) is loaded once, by the lane whose number the entry has -- one coalesced
+// instruction per array -- and handed to the lanes that need it through LDS, where a read of
+// one address by eight lanes is a broadcast.
 
 // Row stride of the accumulators: one more than the row capacity, so that the eight rows of a
 // wavefront start in different LDS banks.
@@ -142,6 +149,9 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     const T *__restrict__ B_data, const int32_t *__restrict__ bstart, const uint8_t *__restrict__ dest,
     const int64_t *__restrict__ C_indptr, T *__restrict__ C_data) {
     __shared__ T s_acc[kGroupsPerBlock * kAccStride];
+    __shared__ T s_av[kBlock];                       // per group: the row's entries of A ...
+    __shared__ int32_t s_bs[kBlock];                 // ... where their rows of B start ...
+    __shared__ __align__(8) uint8_t s_db[kBlock * kCap];   // ... and their destination bytes
     const int k = threadIdx.x & (kCap - 1), g = threadIdx.x / kCap;
     const int64_t row = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + g;
     const bool live = row < rows;
@@ -149,28 +159,34 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     const int64_t ab = pa[0], ae = live ? pa[1] : ab;
     const int64_t cs = pc[0];
     const int clen = live ? (int)(pc[1] - cs) : 0;
+    const int alen = (int)(ae - ab);
     T *acc = s_acc + g * kAccStride;
 #pragma unroll
-    for (int q = 0; q < kCap; ++q) acc[k + kCap * q] = T(0);
-    // everything the row needs is requested before anything is used: two round trips
-    T av[kCap], bv[kCap];
-    int32_t bs[kCap];
+    for (int q = 0; q < kCap; ++q)
+        if (k + kCap * q < clen) acc[k + kCap * q] = T(0);
+    {   // lane k of the group fetches entry k of the row
+        const int64_t e = k < alen ? ab + k : 0;   // entry 0: readable whenever the matrix has entries
+        const T av = A_data[e];
+        const int32_t bs = bstart[e];
+        const uint64_t db = *reinterpret_cast<const uint64_t *>(dest + e * kCap);
+        s_av[threadIdx.x] = av;
+        s_bs[threadIdx.x] = bs;
+        *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) = k < alen ? db : ~uint64_t(0);
+    }
+    group_fence();
+    const int slot = g * kCap;
     uint8_t db[kCap];
+    T bv[kCap];
 #pragma unroll
     for (int a = 0; a < kCap; ++a) {
-        const int64_t e = ab + a < ae ? ab + a : 0;   // entry 0: readable whenever a row has entries
-        av[a] = A_data[e];
-        bs[a] = bstart[e];
-        db[a] = ab + a < ae ? dest[e * kCap + k] : kNone;
+        db[a] = s_db[(slot + a) * kCap + k];
+        bv[a] = B_data[db[a] != kNone ? (int64_t)s_bs[slot + a] + k : 0];
     }
-#pragma unroll
-    for (int a = 0; a < kCap; ++a) bv[a] = B_data[db[a] != kNone ? (int64_t)bs[a] + k : 0];
-    group_fence();
 #pragma unroll
     for (int a = 0; a < kCap; ++a) {
         // the lanes of a group hold different entries of one B row: different columns, different
         // accumulators; the entries of A take their turns one after the other
-        if (db[a] != kNone) acc[db[a]] = acc[db[a]] + av[a] * bv[a];
+        if (db[a] != kNone) acc[db[a]] = acc[db[a]] + s_av[slot + a] * bv[a];
         group_fence();
     }
 #pragma unroll
@@ -194,6 +210,8 @@ __global__ __launch_bounds__(kBlock) void grad_a_mapped_kernel(
     const int k = lane & (kCap - 1), g = lane / kCap;
     T *term = s_term + wave * kWave * kTermStride;
     const int64_t base = ((int64_t)blockIdx.x * (kBlock / kWave) + wave) * kWave;
+    // (here the eight lanes of an entry fetch its starts themselves: handing them round through
+    // LDS, as the other kernels do, measured slower -- the two gathers below dominate)
     int32_t bs[kCap], cs[kCap];
     uint8_t db[kCap];
 #pragma unroll
@@ -219,43 +237,51 @@ __global__ __launch_bounds__(kBlock) void grad_a_mapped_kernel(
 }
 
 // grad_B.  Eight lanes per row j of B, lane k its k-th entry; the group walks column j of A on
-// the transposed-structure plan (rows ascending), eight entries per round trip.
+// the transposed-structure plan (rows ascending), eight entries per round trip: lane u fetches
+// what belongs to the u-th of them, LDS hands it round.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
     const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm, const int64_t *__restrict__ B_indptr,
     const int32_t *__restrict__ cstart, const uint8_t *__restrict__ dest, T *__restrict__ grad_B) {
-    const int k = threadIdx.x & (kCap - 1);
+    __shared__ T s_a[kBlock];
+    __shared__ int32_t s_cs[kBlock];
+    __shared__ __align__(8) uint8_t s_db[kBlock * kCap];
+    const int k = threadIdx.x & (kCap - 1), slot = threadIdx.x & ~(kCap - 1);
     const int64_t j = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + threadIdx.x / kCap;
-    if (j >= B_rows) return;
-    const int64_t bb = B_indptr[j], blen = B_indptr[j + 1] - bb;
-    const int32_t pb = t_indptr[j], pe = t_indptr[j + 1];
+    const bool live = j < B_rows;
+    const int64_t *pb_ = B_indptr + (live ? j : 0);
+    const int64_t bb = pb_[0], blen = live ? pb_[1] - bb : 0;
+    const int32_t *pt = t_indptr + (live ? j : 0);
+    const int32_t pb = pt[0], pe = live ? pt[1] : pb;
     if (pb == pe) {   // no entry of A in this column: the row's gradient is zero, however long the row
         for (int64_t q = k; q < blen; q += kCap) grad_B[bb + q] = T(0);
-        return;
+        return;       // (no workgroup barrier anywhere in this kernel)
     }
     // a named row: at most kCap entries (the plan's build checked it)
     const bool mine = k < blen;
     T acc = T(0);
     for (int32_t t0 = pb; t0 < pe; t0 += kCap) {
-        int32_t e[kCap];
-#pragma unroll
-        for (int u = 0; u < kCap; ++u) e[u] = t_perm[t0 + u < pe ? t0 + u : pb];
-        T a[kCap];
-        int32_t cs[kCap];
-        uint8_t db[kCap];
-#pragma unroll
-        for (int u = 0; u < kCap; ++u) {
-            a[u] = A_data[e[u]];
-            cs[u] = cstart[e[u]];
-            db[u] = mine ? dest[(int64_t)e[u] * kCap + k] : kNone;
+        {
+            const bool have = t0 + k < pe;
+            const int32_t e = t_perm[have ? t0 + k : pb];
+            s_a[threadIdx.x] = A_data[e];
+            s_cs[threadIdx.x] = cstart[e];
+            *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) =
+                have ? *reinterpret_cast<const uint64_t *>(dest + (int64_t)e * kCap) : ~uint64_t(0);
         }
+        group_fence();
+        uint8_t db[kCap];
         T gv[kCap];
 #pragma unroll
-        for (int u = 0; u < kCap; ++u) gv[u] = gC[db[u] != kNone ? (int64_t)cs[u] + db[u] : 0];
+        for (int u = 0; u < kCap; ++u) {
+            db[u] = mine ? s_db[(slot + u) * kCap + k] : kNone;
+            gv[u] = gC[db[u] != kNone ? (int64_t)s_cs[slot + u] + db[u] : 0];
+        }
 #pragma unroll
         for (int u = 0; u < kCap; ++u)
-            if (t0 + u < pe && db[u] != kNone) acc += a[u] * gv[u];
+            if (db[u] != kNone) acc += s_a[slot + u] * gv[u];
+        group_fence();   // the exchange slots are written again in the next round
     }
     if (mine) grad_B[bb + k] = acc;
 }
