@@ -102,6 +102,29 @@ class Workload:
         raise NotImplementedError
 
 
+def _first_calls(ext, call, n=3):
+    """Wall time of the first `n` calls on a new sparsity pattern, one by one, in ms.  One call
+    in the stateless mode comes first -- it notes and plans nothing and takes the one-time costs
+    of a process (code objects loaded, allocator pools grown) out of the way -- then the plan
+    cache is emptied, so that what is timed is: first sighting, the call that builds the plan
+    (the second in the default mode), a steady call."""
+    import torch
+    from numml_amd import _binding
+    mode = _binding.backward_mode()
+    _binding.set_backward_mode("atomic")
+    call()
+    _binding.set_backward_mode(mode)
+    ext.clear_plan_cache()
+    firsts = []
+    for _ in range(n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        call()
+        torch.cuda.synchronize()
+        firsts.append(round((time.perf_counter() - t0) * 1e3, 3))
+    return firsts
+
+
 def _spmv_bytes(rows, cols, nnz, s, i_fwd=8):
     """Algorithmic bytes of one forward and one backward.  i_fwd: index bytes the forward reads
     per entry and per row pointer (8 as the interface delivers them, 4 when the kernel reads
@@ -151,13 +174,7 @@ class SpMV(Workload):
         # Structure analysis is timed apart from the steps.  The first backward calls on a new
         # sparsity pattern are timed one by one: the transposed-structure plan of the default
         # backward is built (and cached) during one of them.
-        firsts = []
-        for _ in range(3):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            ext.spgemv_backward(self.Gv, rows, cols, self.D, self.I, self.P, self.X)
-            torch.cuda.synchronize()
-            firsts.append(round((time.perf_counter() - t0) * 1e3, 3))
+        firsts = _first_calls(ext, lambda: ext.spgemv_backward(self.Gv, rows, cols, self.D, self.I, self.P, self.X))
         self.first_backward_ms = firsts
         self.config = {"workload": f"spmv_fwd_bwd_{self.dtype}_{self.label}", "rows": rows,
                        "first_three_backward_calls_ms": firsts,
@@ -191,6 +208,9 @@ class SpMV(Workload):
             _binding.set_backward_mode(mode)
         build = max(self.first_backward_ms) - rec["roofline"]["avg_ms"]
         gain = stateless - rec["ms_per_step"]
+        i8 = rec["config"]["bytes_per_step_with_int64_forward"] / (rec["ms_per_step"] * 1e-3) / 1e9
+        rec["config"]["GBps_on_int64_forward_model"] = round(i8, 1)
+        rec["config"]["pct_of_hbm_peak_on_int64_forward_model"] = round(100.0 * i8 / HBM_PEAK_GBS, 2)
         rec["config"]["stateless_ms_per_step"] = round(stateless, 5)
         rec["config"]["stateless_GBps_int64_structure"] = round(
             rec["config"]["bytes_per_step_with_int64_forward"] / (stateless * 1e-3) / 1e9, 1)
@@ -259,13 +279,8 @@ class SpMM(Workload):
         self.dominant_name = ("spdmm_bwd_kernel (grad_A) + spdmm_fwd_flat_kernel on the transposed plan (grad_B)"
                               if _binding.backward_mode() != "atomic"
                               else "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)")
-        firsts = []          # the plan of the default backward is built during one of these
-        for _ in range(3):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            ext.spdmm_backward(rows, cols, self.D, self.I, self.P, self.B, self.Gv)
-            torch.cuda.synchronize()
-            firsts.append(round((time.perf_counter() - t0) * 1e3, 3))
+        # the plan of the default backward is built during one of these
+        firsts = _first_calls(ext, lambda: ext.spdmm_backward(rows, cols, self.D, self.I, self.P, self.B, self.Gv))
         self.config = {"workload": "spmm_fwd_bwd_f32_poisson2d_1024_n64" if self.banded
                        else "spmm_fwd_bwd_f32_powerlaw_1M_n64", "rows": rows, "nnz": nnz,
                        "first_three_backward_calls_ms": firsts, "backward": _binding.backward_mode(),
@@ -346,22 +361,15 @@ class SpGEMM(Workload):
         # row of the product needs the hash path.
         # (one step in the stateless mode first, which notes and plans nothing: it takes the
         # one-time costs of a process -- code objects loaded, allocator pools grown -- out of the way)
-        mode = _binding.backward_mode()
-        _binding.set_backward_mode("atomic")
-        C = ext.spgemm_forward(rows, cols, *L, rows, cols, *R)
-        self.nnzC = C[0].shape[0]
-        self.gC = torch.from_numpy(np.random.default_rng(1).standard_normal(self.nnzC)).to(dev)
-        ext.spgemm_backward(self.gC, C[1], C[2], rows, cols, *L, rows, cols, *R)
-        _binding.set_backward_mode(mode)
-        ext.clear_plan_cache()
-        firsts = []
-        for _ in range(3):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
+        def one_step():
             C = ext.spgemm_forward(rows, cols, *L, rows, cols, *R)
+            if not hasattr(self, "gC"):
+                self.nnzC = C[0].shape[0]
+                self.gC = torch.from_numpy(np.random.default_rng(1).standard_normal(self.nnzC)).to(dev)
             ext.spgemm_backward(self.gC, C[1], C[2], rows, cols, *L, rows, cols, *R)
-            torch.cuda.synchronize()
-            firsts.append(round((time.perf_counter() - t0) * 1e3, 3))
+            self.C = C
+        firsts = _first_calls(ext, one_step)
+        C = self.C
         self.first_steps_ms = firsts
         self.planned = (_binding.backward_mode() != "atomic" and _binding.name == "compiled"
                         and self.left == "A")

@@ -236,10 +236,10 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     const int32_t ubc = merge_sum((int32_t)(ub > 0x0fffffff ? 0x0fffffff : ub));
     const bool merge = live && (ae - ab) <= kMergeCap && merge_max(mx) <= kMergeCap;
     if (live && !merge && gl == 0) key[row] = ubc;
-    {   // rows left to the hash path are counted (a product of stencil matrices has none: no atomic at all)
-        const unsigned long long left = __ballot(live && !merge && gl == 0);
-        if (left != 0 && (threadIdx.x & 63) == 0) atomicAdd(hash_rows, (unsigned long long)__popcll(left));
-    }
+    // A row left to the hash path raises a flag (a plain store of the same value by whoever finds one:
+    // a counter that every wavefront of a product of long rows adds to would be a quarter of a
+    // million atomics on one address); the exact count comes from the binning, if it runs.
+    if (live && !merge && gl == 0) *hash_rows = 1;
     merge_stage<float, false>(my_bb, merge ? my_len : 0, B_indices, nullptr, A_indptr, s_bb, s_len, s_col, nullptr);
     const int32_t *pc = s_col + threadIdx.x;
     int32_t cur = *pc;
@@ -464,9 +464,13 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
 }
 
 // What the host needs between the phases, in one place: nnz(C) and the rows the hash path took.
-// summary[1] already holds the number of rows on the hash path (counted by the first kernel).
-__global__ void summary_kernel(const int64_t *__restrict__ nnz_c, int64_t *__restrict__ summary) {
-    if (threadIdx.x == 0) summary[0] = *nnz_c;
+// `bins` is null when no row went to the hash path (summary[1] is then 0 already).
+__global__ void summary_kernel(const int64_t *__restrict__ nnz_c, const int32_t *__restrict__ bins,
+                               int64_t *__restrict__ summary) {
+    if (threadIdx.x == 0) {
+        summary[0] = *nnz_c;
+        if (bins) summary[1] = bins[kBinStart + kBins];
+    }
 }
 
 // host_pinned[0..1] = summary, then host_pinned[2] = ticket: the host polls the ticket.
@@ -1266,8 +1270,8 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
                        A_indices, A_indptr, B_indices, B_indptr, w.key, C_indptr,
                        reinterpret_cast<unsigned long long *>(w.summary + 1));
     NM_LAUNCH_CHECK("symbolic_front_kernel");
-    // With a landing place in pinned host memory the host learns here how many rows the first
-    // kernel left to the hash path; with none (a product of stencil or aggregation matrices) the
+    // With a landing place in pinned host memory the host learns here whether the first kernel
+    // left any row to the hash path; with none (a product of stencil or aggregation matrices) the
     // binning and the nine launches of the hash path, which would find nothing to do, are left out.
     bool hashed = true;
     if (host_landing) {
@@ -1307,7 +1311,8 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     }
     // counts sit in C_indptr[0, rows), C_indptr[rows] = 0: the exclusive scan is the row pointer
     if (int rc = nm::scan_exclusive_i64(C_indptr, A_rows + 1, w.scan, s)) return rc;
-    hipLaunchKernelGGL(summary_kernel, dim3(1), dim3(64), 0, s, C_indptr + A_rows, w.summary);
+    hipLaunchKernelGGL(summary_kernel, dim3(1), dim3(64), 0, s, C_indptr + A_rows,
+                       hashed ? w.bins : (const int32_t *)nullptr, w.summary);
     NM_LAUNCH_CHECK("summary_kernel");
     return NM_OK;
 }
