@@ -1,10 +1,11 @@
 // Level-scheduled sparse triangular solve for gfx950.
 //
 // Analysis (once per sparsity pattern).  The strictly-triangular entries of A
-// define a dependency DAG.  The transposed-structure plan (stable radix sort by
-// column) gives every row's dependents; a Kahn sweep run by one workgroup peels
-// the DAG level by level and leaves the rows in level order: row order[q] sits
-// in "slot" q, level l owns slots [level_ptr[l], level_ptr[l+1]).  The plan
+// define a dependency DAG.  The transposed-structure plan (counting sort by
+// column, rows ascending inside a column) gives every row's dependents; a Kahn
+// sweep run by one workgroup peels the DAG level by level, the rows of each level
+// are then put into ascending order, and row order[q] sits in "slot" q, level l
+// owning slots [level_ptr[l], level_ptr[l+1]).  The plan
 // then stores, for both solve directions (A and A^T), a level-major packed copy
 // of the triangle: per slot the range of its dependencies, per dependency the
 // SLOT of the row it refers to and the position of its coefficient in A's

@@ -124,6 +124,16 @@ def test_cfg4_spgemm_fp64_laplace128(dev):
     gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], C.indices, C.indptr, rows, cols, D, I, P, rows, cols, D, I, P)
     assert_same(host(gA), gA_ref, "grad_A")
     assert_same(host(gB), gB_ref, "grad_B")
+    # the first product built the product plan (the tests run in "eager" mode): a second one is the
+    # planned numeric kernel alone, on the plan's pattern tensors, and the gradients above were the
+    # mapped kernels'; on copies of the pattern tensors the search-based kernels run instead
+    Cd2, Ci2, Cp2 = ext.spgemm_forward(rows, cols, D, I, P, rows, cols, D, I, P)
+    assert Ci2.data_ptr() == C.indices.data_ptr() and Cp2.data_ptr() == C.indptr.data_ptr()
+    assert_same(host(Cd2), Cd_ref, "C_data on the product plan")
+    gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], C.indices.clone(), C.indptr.clone(), rows, cols, D, I, P,
+                                 rows, cols, D, I, P)
+    assert_same(host(gA), gA_ref, "grad_A (search-based, on A's transposed plan)")
+    assert_same(host(gB), gB_ref, "grad_B (search-based, on A's transposed plan)")
     _binding.set_backward_mode("atomic")      # the stateless kernels: grad_B by atomics, tolerance
     gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], C.indices, C.indptr, rows, cols, D, I, P, rows, cols, D, I, P)
     assert_same(host(gA), gA_ref, "grad_A (stateless)")
@@ -202,6 +212,9 @@ def test_cfg4_matrix_in_fp32(dev):
     gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, rows, cols, d, i, p, rows, cols, d, i, p)
     assert_same(host(gA), gA_ref, "grad_A")
     assert_same(host(gB), gB_ref, "grad_B")
+    Cd2, Ci2, Cp2 = ext.spgemm_forward(rows, cols, D, I, P, rows, cols, D, I, P)
+    assert Ci2.data_ptr() == Ci.data_ptr()
+    assert_same(host(Cd2), Cd_ref, "C_data on the product plan")
 
 
 def test_cfg5_matrix_in_fp32(dev):
