@@ -63,3 +63,42 @@ def test_triangular_solve_in_a_graph_and_on_a_side_stream(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert_same(host(x), oracle.sptrsv_forward(n, n, d, i, p, True, False, b_h), "replayed solve")
+
+
+def test_sparse_product_on_its_plan_in_a_graph(dev):
+    """Once a pair of patterns has its product plan, the forward is one kernel and the backward
+    two, none of which allocates outside torch's allocator, waits or clears memory: they can be
+    captured and replayed with new values in the same buffers."""
+    d, i, p, (n, _) = G.laplace3d(8, np.float64, 1)
+    D, I, P = to_dev(dev, d, i, p)
+    E = to_dev(dev, randn(1, d.shape[0], np.float64))[0]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # builds the plans (the suite runs in "eager" mode)
+        C0 = ops.spgemm_forward(n, n, D, I, P, n, n, E, I, P)
+        Gc = torch.zeros_like(C0[0])
+        ops.spgemm_backward(Gc, C0[1], C0[2], n, n, D, I, P, n, n, E, I, P)
+    torch.cuda.current_stream().wait_stream(side)
+    built = ops.plan_cache_stats()[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        Cd, Ci, Cp = ops.spgemm_forward(n, n, D, I, P, n, n, E, I, P)
+        gA, gB = ops.spgemm_backward(Gc, Ci, Cp, n, n, D, I, P, n, n, E, I, P)
+    assert ops.plan_cache_stats()[0] == built, "nothing is analysed during capture"
+    assert Ci.data_ptr() == C0[1].data_ptr()
+    ci, cp = host(Ci), host(Cp)
+    for seed in (3, 4, 5):          # replays with new values, eager work and syncs in between
+        a_h, b_h, g_h = randn(seed, d.shape[0], np.float64), randn(seed + 10, d.shape[0], np.float64), randn(seed + 20, ci.shape[0], np.float64)
+        D.copy_(torch.from_numpy(a_h))
+        E.copy_(torch.from_numpy(b_h))
+        Gc.copy_(torch.from_numpy(g_h))
+        graph.replay()
+        torch.cuda.synchronize()
+        cd_ref, ci_ref, cp_ref = oracle.spgemm_forward(n, n, a_h, i, p, n, n, b_h, i, p)
+        assert_same(ci, ci_ref, "pattern")
+        assert_same(host(Cd), cd_ref, "replayed C_data")
+        gA_ref, gB_ref = oracle.spgemm_backward(g_h, ci_ref, cp_ref, n, n, a_h, i, p, n, n, b_h, i, p)
+        assert_same(host(gA), gA_ref, "replayed grad_A")
+        assert_same(host(gB), gB_ref, "replayed grad_B")
+        eager = ops.spgemm_forward(n, n, D, I, P, n, n, E, I, P)
+        assert torch.equal(eager[0], Cd)

@@ -123,3 +123,32 @@ def test_rows_beyond_the_limits_are_refused(dev):
     ad, ai, ap, ashape = _unpack(G.tridiag(40, dtype))
     AD, AI, AP = to_dev(dev, ad, ai, ap)
     assert not mirror.ProductPlan(40, 40, AI, AP, AI, AP, AI, AP).usable
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_random_short_row_products(dev, seed, dtype):
+    """Shapes, fill and row lengths drawn at random inside the plan's limits (rows of 0..8 entries in
+    both operands, rectangular, columns never named, rows never named)."""
+    rng = np.random.default_rng(100 + seed)
+    m, kdim, n = (int(rng.integers(1, 3000)) for _ in range(3))
+    la, lb = int(rng.integers(1, 9)), int(rng.integers(1, 9))
+    ad, ai, ap, _ = G.ragged_csr(m, kdim, min(la, kdim), 200 + seed, dtype)
+    bd, bi, bp, _ = G.ragged_csr(kdim, n, min(lb, n), 300 + seed, dtype)
+    AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+    C_data, C_indices, C_indptr = mirror.spgemm_forward(m, kdim, AD, AI, AP, kdim, n, BD, BI, BP)
+    plan = mirror.ProductPlan(m, kdim, AI, AP, BI, BP, C_indices, C_indptr)
+    if ai.shape[0] == 0:
+        assert not plan.usable          # nothing to plan for a matrix without entries
+        return
+    assert plan.usable
+    ad2, bd2 = randn(seed, ad.shape[0], dtype), randn(seed + 50, bd.shape[0], dtype)
+    AD2, BD2 = to_dev(dev, ad2, bd2)
+    cd, ci, cp = oracle.spgemm_forward(m, kdim, ad2, ai, ap, kdim, n, bd2, bi, bp)
+    assert_same(host(C_indices), ci, "pattern")
+    assert_same(host(plan.numeric(AD2, BD2)), cd, "C_data")
+    g = randn(seed + 70, cd.shape[0], dtype)
+    gA, gB = plan.backward(to_dev(dev, g)[0], AD2, BD2)
+    rA, rB = oracle.spgemm_backward(g, ci, cp, m, kdim, ad2, ai, ap, kdim, n, bd2, bi, bp)
+    assert_same(host(gA), rA, "grad_A")
+    assert_same(host(gB), rB, "grad_B")
