@@ -50,6 +50,7 @@ struct Packed {        // one solve direction, level-major (all int32, device)
     int32_t *dsrc;     // [nnz]    position of its coefficient in A's data
     int32_t *diag;     // [rows]   position of the diagonal coefficient, -1 when not stored
     int32_t *ell_ds;   // [ell_capacity] fixed-width dependency entries, `pre` per row (ring byte offset | far bit)
+    int32_t *lvl_sig;  // [levels] which neighbouring wavefronts the rows of a level wait for (kSigLower | kSigHigher)
 };
 // Entries of the fixed-width (ELLPACK) arrays; the layout is used when (rows + kEllPad) * pre
 // fits.  kEllPad slots of padding follow the last row in every array the fixed-width kernel
@@ -88,8 +89,11 @@ constexpr int kBlock = 256;
 constexpr int kRing = 8192;            // LDS ring of recent solutions (doubles, power of two)
 // Levels a wavefront of the signalling kernel may run ahead of the slowest one of its
 // workgroup; the ring must keep what the slowest still reads while the fastest writes.
-constexpr int kSkew = 2;
-constexpr int kRingSafe = kRing - (kSkew + 1) * kNarrow;
+constexpr int kSkew = 5;
+constexpr int kRingSafe = kRing - 3 * kNarrow;                 // how far back (in slots) a ring read may reach
+constexpr int kRingSafeSig = kRing - (kSkew + 1) * kNarrow;    // ... when wavefronts run up to kSkew levels apart
+constexpr int32_t kSigLower = 1, kSigHigher = 2;               // bits of lvl_sig
+constexpr int32_t kSigNever = 1000;                            // a reach that rules the signalling kernel out
 // Largest distance, in wavefronts, between a row and the rows it depends on (both counted from
 // the start of their level) for which wavefronts signal each other instead of meeting at a
 // workgroup barrier after every level.
@@ -135,6 +139,7 @@ size_t plan_layout(int64_t rows, int64_t nnz, void *base, Layout *L) {
         l.dir[d].dsrc = take(nnz + 1);
         l.dir[d].diag = take(rows + 1);
         l.dir[d].ell_ds = take(ell_capacity(rows, nnz));
+        l.dir[d].lvl_sig = take(rows + 1);
     }
     if (L) *L = l;
     return off;
@@ -601,7 +606,8 @@ __device__ __forceinline__ int32_t level_of_slot(const int32_t *__restrict__ lev
 __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict__ dptr,
                                 const int32_t *__restrict__ dslot, const int32_t *__restrict__ level_ptr,
                                 int32_t nlevels, const int32_t *__restrict__ level_launch,
-                                int32_t *__restrict__ ell_ds, int32_t *__restrict__ reach) {
+                                int32_t *__restrict__ ell_ds, int32_t *__restrict__ reach,
+                                int32_t *__restrict__ lvl_sig) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     // the padding slots behind the last row get "absent" entries: lanes that read them must find a valid offset
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (rows + kEllPad) * pre; i += stride) {
@@ -619,8 +625,13 @@ __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict
             if (near) {
                 // wavefront of the row and of the row it waits for, each inside its own level
                 const int32_t wq = ((int32_t)q - level_ptr[lq]) >> 6, wd = (ds - level_ptr[ld]) >> 6;
-                const int32_t far = wq > wd ? wq - wd : wd - wq;
+                int32_t far = wq > wd ? wq - wd : wd - wq;
+                if (dist >= kRingSafeSig) far = kSigNever;   // too far back for wavefronts that run apart
                 if (far > *reach) atomicMax(reach, far);
+                // which neighbour the rows of this level wait for: with dependencies on one side only,
+                // the wavefronts form a pipeline instead of moving in step
+                const int32_t bit = wd < wq ? kSigLower : (wd > wq ? kSigHigher : 0);
+                if (bit && (lvl_sig[lq] & bit) == 0) atomicOr(lvl_sig + lq, bit);
             }
         }
         ell_ds[i] = out;
@@ -650,7 +661,7 @@ __global__ void gather_ell_kernel(int64_t rows, int pre, const T *__restrict__ d
 }
 
 struct EllArgs {
-    const int32_t *level_ptr, *ell_ds, *dptr, *dslot;
+    const int32_t *level_ptr, *ell_ds, *dptr, *dslot, *lvl_sig;
     const double *ell_coef, *rb;
     double *xs;
     int unit;
@@ -666,6 +677,18 @@ template <int PRE> struct EllVals {
     double v[PRE];
     double bv, dv;
 };
+
+// Makes the compiler have the operands of a stage in registers HERE (an empty instruction that
+// claims to read and write them): used to keep copies between stages in front of the next request.
+template <int PRE> __device__ __forceinline__ void settle(EllVals<PRE> &v) {
+#pragma unroll
+    for (int e = 0; e < PRE; ++e) {
+        asm volatile("" : "+v"(v.ds[e]));
+        asm volatile("" : "+v"(v.v[e]));
+    }
+    asm volatile("" : "+v"(v.bv));
+    asm volatile("" : "+v"(v.dv));
+}
 
 __device__ __forceinline__ Bounds load_bounds_uniform(const int32_t *s_lp, int it, int count, int l0, int step,
                                                       int lmin) {
@@ -714,17 +737,66 @@ template <int PRE> __device__ __forceinline__ EllVals<PRE> load_ell(const EllArg
 // wavefront only ever waits for lower levels, so the waits end; as a backstop a wavefront
 // that has polled `poll_limit` times without success raises a flag that makes every wavefront
 // leave, and the solve's status word tells the last kernel of the solve to hand out NaN.
+// Byte offset of a __shared__ object inside the workgroup's LDS.
+__device__ __forceinline__ uint32_t lds_offset(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
+}
+
+// Polls the LDS word at `at` until, in every lane, it is at least `need`, at most `limit` times;
+// `seen` is what the last poll read, `left` the polls that were left (0: gave up).  `nap`: sleep
+// between polls (0 none, 1 short, 2 long).  All 64 lanes must be active.
+__device__ __forceinline__ void sig_wait(uint32_t at, int32_t need, int32_t limit, int nap, int32_t &seen,
+                                         int32_t &left) {
+    if (nap == 0)
+        asm volatile("s_mov_b32 %1, %4\n"
+                     "1:\n\t"
+                     "ds_read_b32 %0, %2\n\t"
+                     "s_waitcnt lgkmcnt(0)\n\t"
+                     "v_cmp_lt_i32 vcc, %0, %3\n\t"
+                     "s_cmp_eq_u64 vcc, 0\n\t"
+                     "s_cbranch_scc1 2f\n\t"
+                     "s_sub_u32 %1, %1, 1\n\t"
+                     "s_cmp_eq_u32 %1, 0\n\t"
+                     "s_cbranch_scc1 2f\n\t"
+                     "s_branch 1b\n"
+                     "2:\n"
+                     : "=&v"(seen), "=&s"(left)
+                     : "v"(at), "v"(need), "s"(limit)
+                     : "vcc", "scc", "memory");
+    else
+        asm volatile("s_mov_b32 %1, %4\n"
+                     "1:\n\t"
+                     "ds_read_b32 %0, %2\n\t"
+                     "s_waitcnt lgkmcnt(0)\n\t"
+                     "v_cmp_lt_i32 vcc, %0, %3\n\t"
+                     "s_cmp_eq_u64 vcc, 0\n\t"
+                     "s_cbranch_scc1 2f\n\t"
+                     "s_sub_u32 %1, %1, 1\n\t"
+                     "s_cmp_eq_u32 %1, 0\n\t"
+                     "s_cbranch_scc1 2f\n\t"
+                     "s_sleep 1\n\t"
+                     "s_branch 1b\n"
+                     "2:\n"
+                     : "=&v"(seen), "=&s"(left)
+                     : "v"(at), "v"(need), "s"(limit)
+                     : "vcc", "scc", "memory");
+}
+
 template <int PRE, int DEPTH, bool SIG = false>
 __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step,
-                                                             int64_t poll_limit = 0, int32_t *status = nullptr) {
+                                                             int64_t poll_limit = 0, int32_t *status = nullptr,
+                                                             int tune_sleep = 1, int tune_skew = kSkew) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
     __shared__ int32_t s_lp[kMaxLevels + 1];
     __shared__ int32_t s_done[kNarrow / 64];   // SIG: levels each wavefront has finished
     __shared__ int32_t s_abort;
+    __shared__ uint8_t s_sig[SIG ? kMaxLevels : 1];   // SIG: the neighbours a level's rows wait for
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
     for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
+    if (SIG)
+        for (int i = threadIdx.x; i < count; i += blockDim.x) s_sig[i] = (uint8_t)a.lvl_sig[lmin + i];
     if (threadIdx.x == 0) ring[kRing] = 0.;
-    if (SIG && threadIdx.x < kNarrow / 64) s_done[threadIdx.x] = 0;
+    if (SIG && threadIdx.x < kNarrow / 64) s_done[threadIdx.x] = poll_limit < 0 ? 0x7fffffff : 0;
     if (SIG && threadIdx.x == 0) s_abort = poll_limit < 0 ? 1 : 0;   // a negative limit: give up at once (tests)
     __syncthreads();
     const int sig_lane = threadIdx.x & 63, sig_wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -740,83 +812,140 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
     // early, before the barrier, so that the request does not start with an LDS round trip.
     Bounds ahead = load_bounds_uniform(s_lp, DEPTH, count, l0, step, lmin);
 
-    for (int it0 = 0; it0 < count; it0 += DEPTH) {
+    // one level: `cur` holds its operands
+    auto level = [&](int it, const EllVals<PRE> &cur) {
+        // all ring reads go out together, unconditionally
+        double xj[PRE];
+        int32_t any = 0;
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            const int it = it0 + d;
-            if (it >= count) break;   // uniform over the workgroup
-            if (SIG && gave_up) break;
-            if (SIG) {
-                // lane w looks at wavefront w's count of finished levels
-                int64_t polls = 0;
-                for (;;) {
-                    // (relaxed atomic accesses of the LDS words themselves: a pointer to them would be
-                    // taken for a pointer to any memory, and its loads would wait for the global ones)
-                    const int32_t mine_done =
-                        __hip_atomic_load(&s_done[sig_lane & (kNarrow / 64 - 1)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    const int32_t seen = sig_lane < sig_waves ? mine_done : 0x7fffffff;
-                    const bool near = sig_lane + kSigReach >= sig_wave && sig_lane <= sig_wave + kSigReach;
-                    if (__ballot(seen >= (near ? it : it - kSkew)) == ~0ull) break;
-                    if (__hip_atomic_load(&s_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0 ||
-                        ++polls > poll_limit) {
-                        __hip_atomic_store(&s_abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                        gave_up = true;
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(1);
-                }
-                if (gave_up) break;
-            }
-            const EllVals<PRE> cur = qv[d];
-            qv[d] = load_ell<PRE>(a, ahead);
+        for (int e = 0; e < PRE; ++e) {
+            xj[e] = *reinterpret_cast<const double *>(ring_bytes + (cur.ds[e] & kEllOffsetMask));
+            any |= cur.ds[e];
+        }
+        ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
+        double acc = 0.;
+#pragma unroll
+        for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
+        const bool live = (int)threadIdx.x < cur.qe - cur.qb;
+        if ((any & kEllFar) && live) {
+            // a dependency the ring does not hold: redo the sum in the same order from global memory
+            // (slots and then solutions are requested together; entries past the row's own
+            //  name a valid slot and are not added)
+            const int q = cur.qb + (int)threadIdx.x;
+            const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
+            int32_t sl[PRE];
+            double xg[PRE];
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
+            acc = 0.;
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) acc += e < n ? cur.v[e] * xg[e] : 0.;
+        }
+        double xi = cur.bv - acc;
+        if (!a.unit) xi /= cur.dv;
+        if (live) {
+            const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
+            *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
+            *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
+        }
+    };
+    if (!SIG) {
+        // (the level body is written out here rather than shared with the signalling loop below:
+        // shared through a lambda it compiled to a few more scalar instructions per level)
+        for (int it0 = 0; it0 < count; it0 += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                const int it = it0 + d;
+                if (it >= count) break;   // uniform over the workgroup
+                const EllVals<PRE> cur = qv[d];
+                qv[d] = load_ell<PRE>(a, ahead);
 
-            // all ring reads go out together, unconditionally
-            double xj[PRE];
-            int32_t any = 0;
+                // all ring reads go out together, unconditionally
+                double xj[PRE];
+                int32_t any = 0;
 #pragma unroll
-            for (int e = 0; e < PRE; ++e) {
-                xj[e] = *reinterpret_cast<const double *>(ring_bytes + (cur.ds[e] & kEllOffsetMask));
-                any |= cur.ds[e];
-            }
-            ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
-            double acc = 0.;
+                for (int e = 0; e < PRE; ++e) {
+                    xj[e] = *reinterpret_cast<const double *>(ring_bytes + (cur.ds[e] & kEllOffsetMask));
+                    any |= cur.ds[e];
+                }
+                ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
+                double acc = 0.;
 #pragma unroll
-            for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
-            const bool live = (int)threadIdx.x < cur.qe - cur.qb;
-            if ((any & kEllFar) && live) {
-                // a dependency the ring does not hold: redo the sum in the same order from global memory
-                // (slots and then solutions are requested together; entries past the row's own
-                //  name a valid slot and are not added)
-                const int q = cur.qb + (int)threadIdx.x;
-                const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
-                int32_t sl[PRE];
-                double xg[PRE];
+                for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
+                const bool live = (int)threadIdx.x < cur.qe - cur.qb;
+                if ((any & kEllFar) && live) {
+                    // a dependency the ring does not hold: redo the sum in the same order from global memory
+                    // (slots and then solutions are requested together; entries past the row's own
+                    //  name a valid slot and are not added)
+                    const int q = cur.qb + (int)threadIdx.x;
+                    const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
+                    int32_t sl[PRE];
+                    double xg[PRE];
 #pragma unroll
-                for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
+                    for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
 #pragma unroll
-                for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
-                acc = 0.;
+                    for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
+                    acc = 0.;
 #pragma unroll
-                for (int e = 0; e < PRE; ++e) acc += e < n ? cur.v[e] * xg[e] : 0.;
-            }
-            double xi = cur.bv - acc;
-            if (!a.unit) xi /= cur.dv;
-            if (live) {
-                const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
-                *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
-                *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
-            }
-            if (SIG) {
-                // the ring write above is in LDS before the count moves (one wavefront's LDS
-                // accesses are served in the order it issued them)
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                if (sig_lane == 0)
-                    __hip_atomic_store(&s_done[sig_wave], it + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            } else {
+                    for (int e = 0; e < PRE; ++e) acc += e < n ? cur.v[e] * xg[e] : 0.;
+                }
+                double xi = cur.bv - acc;
+                if (!a.unit) xi /= cur.dv;
+                if (live) {
+                    const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
+                    *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
+                    *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
+                }
                 __syncthreads();
             }
         }
-        if (SIG && gave_up) break;
+    } else {
+        // Stages are refilled in place, as above.  The wait for the neighbours is written in
+        // assembly (sig_wait): with a polling LOOP among the level's statements the compiler hands
+        // the operand stages from level to level through register copies, and the copy of the
+        // stage just requested waits for that request -- a memory round trip per level, far more
+        // than any rendezvous costs.  As one opaque instruction the wait leaves the loop as
+        // straight as the barrier version's.
+        //   lane w < waves polls s_done[w]; lane 63 reads the abort word along with them.
+        const uint32_t poll_at = lds_offset(sig_lane < sig_waves ? (const void *)&s_done[sig_lane] : (const void *)&s_abort);
+        const int32_t limit32 = poll_limit > 0x7fffffff ? 0x7fffffff : (poll_limit < 1 ? 1 : (int32_t)poll_limit);
+        for (int it0 = 0; it0 < count; it0 += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                const int it = it0 + d;
+                if (it >= count) break;   // uniform over the workgroup
+                // the wavefronts this one waits for at this level: the lower and / or the higher
+                // neighbour must have finished the level before; nobody may be kSkew levels behind
+                const int32_t sides = s_sig[l0 + it * step - lmin];
+                const bool near = (sig_lane + 1 == sig_wave && (sides & kSigLower)) ||
+                                  (sig_lane == sig_wave + 1 && (sides & kSigHigher));
+                const int32_t need = sig_lane < sig_waves ? (near ? it : it - tune_skew) : (int32_t)0x80000000;
+                int32_t seen, left;
+                sig_wait(poll_at, need, limit32, tune_sleep, seen, left);
+                int32_t aborted = __builtin_amdgcn_readlane(seen, 63);
+                if (__builtin_expect(left == 0, 0)) {
+                    // out of polls: every counter jumps to the end, so that nobody waits for anybody
+                    // any more, and the abort word makes the solve hand out NaN
+                    if (sig_lane < kNarrow / 64)
+                        __hip_atomic_store(&s_done[sig_lane], 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    if (sig_lane == 0) __hip_atomic_store(&s_abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    aborted = 1;
+                }
+                const EllVals<PRE> cur = qv[d];
+                qv[d] = load_ell<PRE>(a, ahead);
+                level(it, cur);
+                // the ring write above is in LDS before the count moves (one wavefront's LDS
+                // accesses are served in the order it issued them); after an abort the count stays
+                // at the end
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                if (sig_lane == 0)
+                    __hip_atomic_store(&s_done[sig_wave], aborted ? 0x7fffffff : it + 1, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+        gave_up = __hip_atomic_load(&s_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0;
     }
     if (SIG && gave_up && sig_lane == 0 && status) status[0] = 1;
 }
@@ -905,7 +1034,7 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     }
     const int dirn = transposed ? 1 : 0;
     const int pre = p->ell_pre[dirn];
-    EllArgs ea{p->level_ptr, P.ell_ds, P.dptr, P.dslot, a.w.ell_coef, a.w.rb, a.w.xs, unit};
+    EllArgs ea{p->level_ptr, P.ell_ds, P.dptr, P.dslot, P.lvl_sig, a.w.ell_coef, a.w.rb, a.w.xs, unit};
     if (pre > 0) {
         int64_t grid = nm::ceil_div(p->rows * pre, kBlock);
         if (grid > 65536) grid = 65536;
@@ -939,15 +1068,21 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
             // (and there is more than one wavefront); else they meet at a barrier after every level
             const bool sig = pre > 0 && L.block > 64 && p->reach[dirn] <= kSigReach && g_sig_enabled.load();
             const int64_t limit = g_sig_poll_limit.load();
+            static const int tune_sleep = [] { const char *e = std::getenv("NUMML_AMD_SIG_SLEEP"); return e ? atoi(e) : 1; }();
+            static const int tune_skew = [] {
+                const char *e = std::getenv("NUMML_AMD_SIG_SKEW");
+                const int v = e ? atoi(e) : kSkew;
+                return v < 0 ? 0 : (v > kSkew ? kSkew : v);
+            }();
             if (pre == 2 && sig)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4, true>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
-                                   limit, a.w.status);
+                                   limit, a.w.status, tune_sleep, tune_skew);
             else if (pre == 4 && sig)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3, true>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
-                                   limit, a.w.status);
+                                   limit, a.w.status, tune_sleep, tune_skew);
             else if (pre == 8 && sig)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2, true>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
-                                   limit, a.w.status);
+                                   limit, a.w.status, tune_sleep, tune_skew);
             else if (pre == 2)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
                                    (int64_t)0, (int32_t *)nullptr);
@@ -1198,9 +1333,10 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             p->ell_pre[d] = pre;
             int64_t grid = nm::ceil_div(rows * pre, kBlock);
             if (grid > 65536) grid = 65536;
+            if (int rc = nm::fill_async(p->dir[d].lvl_sig, (int64_t)p->nlevels + 1, (int32_t)0, s)) return bail(rc);
             hipLaunchKernelGGL(ell_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, pre, p->dir[d].dptr,
                                p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, p->dir[d].ell_ds,
-                               L.meta + 4 + d);
+                               L.meta + 4 + d, p->dir[d].lvl_sig);
             if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
         }
     }
