@@ -265,7 +265,40 @@ int nm_spgemm_backward_planned(nm_dtype dt, int64_t A_rows, int64_t A_cols, int6
  *                           when given; NULL: a copy and a synchronisation).
  *   nm_spgemm_numeric_planned   C_data of the product, C_indptr as built from.
  *   nm_spgemm_backward_mapped   grad_A and / or grad_B (either may be NULL) of
- *                           gC laid out on the plan's pattern of C. */
+ *                           gC laid out on the plan's pattern of C.
+ *
+ * The plan can also be had as a by-product of the product's first computation:
+ *   nm_spgemm_symbolic_mapped   nm_spgemm_symbolic that, while it merges the rows to
+ *                           count them, records in plan_mem where every product of a
+ *                           merge-path row goes (the plan's destination bytes and B
+ *                           row starts).  A and B must have fewer than 2^31 entries.
+ *   nm_spgemm_numeric_mapped    nm_spgemm_numeric that, when hash_rows is 0 (every row
+ *                           on the merge path, from nm_spgemm_symbolic_result) and
+ *                           C_nnz < 2^31, adds the products up on those records
+ *                           instead of merging the rows a second time, and fills in
+ *                           the plan's C row starts; otherwise it is nm_spgemm_numeric
+ *                           and plan_mem holds nothing usable.  Same results, bit
+ *                           for bit.
+ *   nm_spgemm_plan_adopt    checks what such a plan still needs before the kernels
+ *                           above may run on it (no column of A with more than 4096
+ *                           entries: A_plan_mem is A's transposed-structure plan;
+ *                           sizes below 2^31; hash_rows == 0) and reports `usable`
+ *                           like nm_spgemm_plan_build.  Waits for the stream. */
+int nm_spgemm_symbolic_mapped(int64_t A_rows, int64_t A_cols, int64_t B_cols, int64_t A_nnz, int64_t B_nnz,
+                              const int64_t *A_indices, const int64_t *A_indptr,
+                              const int64_t *B_indices, const int64_t *B_indptr,
+                              int64_t *C_indptr, void *workspace, size_t workspace_bytes,
+                              void *plan_mem, size_t plan_bytes, void *host_landing, nm_stream stream);
+int nm_spgemm_numeric_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t B_cols,
+                             int64_t A_nnz, int64_t C_nnz,
+                             const void *A_data, const int64_t *A_indices, const int64_t *A_indptr,
+                             const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
+                             const int64_t *C_indptr, int64_t *C_indices, void *C_data,
+                             void *workspace, size_t workspace_bytes, int64_t hash_rows,
+                             void *plan_mem, size_t plan_bytes, nm_stream stream);
+int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                         int64_t hash_rows, const void *A_plan_mem, void *plan_mem, size_t plan_bytes,
+                         void *host_landing, int *usable, nm_stream stream);
 int nm_spgemm_plan_bytes(int64_t A_nnz, size_t *plan_bytes);
 int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
                          const int64_t *A_indices, const int64_t *A_indptr,

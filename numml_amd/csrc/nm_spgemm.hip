@@ -32,6 +32,7 @@
 //   + nnzC*(s+8) + rowsA*8
 #include "nm_common.hpp"
 #include "nm_scan.hpp"
+#include "nm_spgemm_plan.hpp"
 
 namespace {
 
@@ -210,7 +211,7 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     int64_t rows, int64_t nbatch_padded, const int64_t *__restrict__ A_indices,
     const int64_t *__restrict__ A_indptr, const int64_t *__restrict__ B_indices,
     const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key, int64_t *__restrict__ C_count,
-    unsigned long long *__restrict__ hash_rows) {
+    unsigned long long *__restrict__ hash_rows, uint64_t *__restrict__ dest, int32_t *__restrict__ bstart) {
     __shared__ int32_t s_col[(kMergeCap + 1) * kMergeStride];
     __shared__ int64_t s_bb[kBlock];
     __shared__ int32_t s_len[kBlock];
@@ -244,20 +245,32 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     const int32_t *pc = s_col + threadIdx.x;
     int32_t cur = *pc;
     int cnt = 0, it = 0;
+    // With `dest` given the merge also leaves behind WHERE every product goes: byte k of a lane's
+    // word is the pass in which the k-th entry of its B row was taken, i.e. the position of that
+    // entry's column in the row of C (0xFF: no such entry).  The numeric phase can then add the
+    // products up without merging again, and the words are what a product plan is made of.
+    uint64_t where = ~uint64_t(0);
+    int shift = 0;
     for (;;) {
         const int32_t m = merge_min(cur);
         const bool open = m != kColEnd;
         if (__ballot(open) == 0) break;
-        ++it;
-        if (open) cnt = it;   // an open group emits one column per pass
         if (cur == m && open) {
+            where ^= (uint64_t)(0xFF ^ it) << shift;
+            shift += 8;
             pc += kMergeStride;
             cur = *pc;
         }
+        ++it;
+        if (open) cnt = it;   // an open group emits one column per pass
     }
     if (merge && gl == 0) {
         C_count[row] = cnt;
         key[row] = kMergedKey;
+    }
+    if (dest && merge && ab + gl < ae) {
+        dest[ab + gl] = where;
+        bstart[ab + gl] = (int32_t)my_bb;
     }
 }
 
@@ -1250,10 +1263,14 @@ extern "C" int nm_spgemm_workspace_bytes(int64_t A_rows, int64_t B_cols, size_t 
     return NM_OK;
 }
 
-extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t *A_indices,
-                                  const int64_t *A_indptr, const int64_t *B_indices, const int64_t *B_indptr,
-                                  int64_t *C_indptr, void *workspace, size_t workspace_bytes,
-                                  void *host_landing, nm_stream stream) {
+namespace {
+
+// The symbolic phase; with `map` its first kernel also records where every product of a
+// merge-path row goes (the destination bytes and B row starts of a product plan).
+int symbolic_phase(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t *A_indices,
+                   const int64_t *A_indptr, const int64_t *B_indices, const int64_t *B_indptr, int64_t *C_indptr,
+                   void *workspace, size_t workspace_bytes, void *host_landing, const nm::PPlan *map,
+                   nm_stream stream) {
     if (int rc = check_common(A_rows, B_cols)) return rc;
     NM_REQUIRE(A_cols >= 0, "negative size");
     NM_REQUIRE(A_indptr && B_indptr && C_indptr && workspace, "null pointer argument");
@@ -1268,7 +1285,9 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
     const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
     hipLaunchKernelGGL(symbolic_front_kernel, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
                        A_indices, A_indptr, B_indices, B_indptr, w.key, C_indptr,
-                       reinterpret_cast<unsigned long long *>(w.summary + 1));
+                       reinterpret_cast<unsigned long long *>(w.summary + 1),
+                       map ? reinterpret_cast<uint64_t *>(map->dest) : (uint64_t *)nullptr,
+                       map ? map->bstart : (int32_t *)nullptr);
     NM_LAUNCH_CHECK("symbolic_front_kernel");
     // With a landing place in pinned host memory the host learns here whether the first kernel
     // left any row to the hash path; with none (a product of stencil or aggregation matrices) the
@@ -1315,6 +1334,31 @@ extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols
                        hashed ? w.bins : (const int32_t *)nullptr, w.summary);
     NM_LAUNCH_CHECK("summary_kernel");
     return NM_OK;
+}
+
+}  // namespace
+
+extern "C" int nm_spgemm_symbolic(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t *A_indices,
+                                  const int64_t *A_indptr, const int64_t *B_indices, const int64_t *B_indptr,
+                                  int64_t *C_indptr, void *workspace, size_t workspace_bytes,
+                                  void *host_landing, nm_stream stream) {
+    return symbolic_phase(A_rows, A_cols, B_cols, A_indices, A_indptr, B_indices, B_indptr, C_indptr, workspace,
+                          workspace_bytes, host_landing, nullptr, stream);
+}
+
+extern "C" int nm_spgemm_symbolic_mapped(int64_t A_rows, int64_t A_cols, int64_t B_cols, int64_t A_nnz,
+                                         int64_t B_nnz, const int64_t *A_indices, const int64_t *A_indptr,
+                                         const int64_t *B_indices, const int64_t *B_indptr, int64_t *C_indptr,
+                                         void *workspace, size_t workspace_bytes, void *plan_mem,
+                                         size_t plan_bytes, void *host_landing, nm_stream stream) {
+    NM_REQUIRE(A_nnz >= 0 && B_nnz >= 0 && plan_mem, "bad arguments");
+    NM_REQUIRE(A_nnz < ((int64_t)1 << 31) && B_nnz < ((int64_t)1 << 31), "the plan keeps positions in 31 bits");
+    const size_t need = nm::pplan_layout(A_nnz, nullptr, nullptr);
+    if (plan_bytes < need) return nm::fail(NM_ERR_WORKSPACE, "plan of %zu bytes, %zu needed", plan_bytes, need);
+    nm::PPlan map;
+    nm::pplan_layout(A_nnz, plan_mem, &map);
+    return symbolic_phase(A_rows, A_cols, B_cols, A_indices, A_indptr, B_indices, B_indptr, C_indptr, workspace,
+                          workspace_bytes, host_landing, &map, stream);
 }
 
 extern "C" int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const void *workspace,
@@ -1398,6 +1442,28 @@ extern "C" int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, in
                                      C_indptr, C_indices, C_data, s);
     return launch_numeric<double>(w, B_cols, A_data, A_indices, A_indptr, B_data, B_indices, B_indptr, C_indptr,
                                   C_indices, C_data, s);
+}
+
+extern "C" int nm_spgemm_numeric_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t B_cols, int64_t A_nnz,
+                                        int64_t C_nnz, const void *A_data, const int64_t *A_indices,
+                                        const int64_t *A_indptr, const void *B_data, const int64_t *B_indices,
+                                        const int64_t *B_indptr, const int64_t *C_indptr, int64_t *C_indices,
+                                        void *C_data, void *workspace, size_t workspace_bytes, int64_t hash_rows,
+                                        void *plan_mem, size_t plan_bytes, nm_stream stream) {
+    // rows on the hash path (or an unknown number of them), or positions beyond 31 bits: the map
+    // the symbolic phase left is incomplete or unusable, the ordinary numeric phase runs
+    if (hash_rows != 0 || !plan_mem || A_nnz <= 0 || C_nnz <= 0 || C_nnz >= ((int64_t)1 << 31))
+        return nm_spgemm_numeric(dt, A_rows, A_cols, B_cols, A_data, A_indices, A_indptr, B_data, B_indices, B_indptr,
+                                 C_indptr, C_indices, C_data, workspace, workspace_bytes, hash_rows, stream);
+    if (int rc = check_common(A_rows, B_cols)) return rc;
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(A_data && A_indptr && B_data && B_indices && C_indptr && C_indices && C_data, "null pointer argument");
+    const size_t need = nm::pplan_layout(A_nnz, nullptr, nullptr);
+    if (plan_bytes < need) return nm::fail(NM_ERR_WORKSPACE, "plan of %zu bytes, %zu needed", plan_bytes, need);
+    nm::PPlan map;
+    nm::pplan_layout(A_nnz, plan_mem, &map);
+    return nm::spgemm_numeric_on_map(dt, A_rows, A_nnz, A_data, A_indptr, B_data, B_indices, map, C_indptr, C_indices,
+                                     C_data, nm::as_stream(stream));
 }
 
 extern "C" int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, const void *gC,

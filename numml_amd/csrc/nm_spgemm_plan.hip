@@ -28,41 +28,20 @@
 //              the transposed-structure plan of A.
 //
 // No atomics, nothing to clear, every gradient entry written once by one lane.
-#include "nm_common.hpp"
-#include "nm_transpose.hpp"
+#include "nm_spgemm_plan.hpp"
 
 namespace {
 
 using nm::kWave;
+using nm::PPlan;
+using nm::pplan_layout;
 
 constexpr int kBlock = 256;
-constexpr int kCap = 8;                  // entries per row of A and per named row of B
-constexpr int kRowCap = kCap * kCap;     // entries per row of C
+constexpr int kCap = nm::kPlanCap;            // entries per row of A and per named row of B
+constexpr int kRowCap = nm::kPlanRowCap;      // entries per row of C
 constexpr int kGroupsPerBlock = kBlock / kCap;
-constexpr int32_t kMaxColumn = 4096;     // entries per column of A: one group of lanes walks a column
-constexpr uint8_t kNone = 0xFF;
-
-struct PPlan {
-    int32_t *flag;     // [0] != 0: a limit does not hold, the plan must not be used
-    int32_t *bstart;   // [A_nnz]
-    int32_t *cstart;   // [A_nnz]
-    uint8_t *dest;     // [A_nnz * 8]
-};
-
-size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p) {
-    size_t off = 0;
-    auto take = [&](size_t bytes) {
-        void *q = base ? static_cast<char *>(base) + off : nullptr;
-        off += nm::align256(bytes);
-        return q;
-    };
-    int32_t *flag = (int32_t *)take(64);
-    int32_t *bs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
-    int32_t *cs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
-    uint8_t *d = (uint8_t *)take((size_t)(A_nnz + 1) * 8);
-    if (p) *p = PPlan{flag, bs, cs, d};
-    return off;
-}
+constexpr int32_t kMaxColumn = 4096;          // entries per column of A: one group of lanes walks a column
+constexpr uint8_t kNone = nm::kPlanNone;
 
 __device__ __forceinline__ void group_fence() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); }
 
@@ -143,12 +122,17 @@ __global__ void plan_flag_out_kernel(const int32_t *flag, volatile int64_t *host
 // wavefront start in different LDS banks.
 constexpr int kAccStride = kRowCap + 1;
 
-template <typename T>
+// COLS: the pattern of C is not there yet (the product is being computed for the first time, on the
+// destination bytes the symbolic phase left behind): every product also drops its column beside its
+// accumulator, the columns are written out with the values, and cstart is filled in.
+template <typename T, bool COLS>
 __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     int64_t rows, int64_t ntiles_padded, const T *__restrict__ A_data, const int64_t *__restrict__ A_indptr,
-    const T *__restrict__ B_data, const int32_t *__restrict__ bstart, const uint8_t *__restrict__ dest,
-    const int64_t *__restrict__ C_indptr, T *__restrict__ C_data) {
+    const T *__restrict__ B_data, const int64_t *__restrict__ B_indices, const int32_t *__restrict__ bstart,
+    const uint8_t *__restrict__ dest, const int64_t *__restrict__ C_indptr, T *__restrict__ C_data,
+    int64_t *__restrict__ C_indices, int32_t *__restrict__ cstart) {
     __shared__ T s_acc[kGroupsPerBlock * kAccStride];
+    __shared__ int32_t s_ccol[COLS ? kGroupsPerBlock * kAccStride : 1];
     __shared__ T s_av[kBlock];                       // per group: the row's entries of A ...
     __shared__ int32_t s_bs[kBlock];                 // ... where their rows of B start ...
     __shared__ __align__(8) uint8_t s_db[kBlock * kCap];   // ... and their destination bytes
@@ -172,26 +156,37 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
         s_av[threadIdx.x] = av;
         s_bs[threadIdx.x] = bs;
         *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) = k < alen ? db : ~uint64_t(0);
+        if (COLS && k < alen) cstart[e] = (int32_t)cs;
     }
     group_fence();
     const int slot = g * kCap;
     uint8_t db[kCap];
     T bv[kCap];
+    int32_t bc[kCap];
 #pragma unroll
     for (int a = 0; a < kCap; ++a) {
         db[a] = s_db[(slot + a) * kCap + k];
-        bv[a] = B_data[db[a] != kNone ? (int64_t)s_bs[slot + a] + k : 0];
+        const int64_t at = db[a] != kNone ? (int64_t)s_bs[slot + a] + k : 0;
+        bv[a] = B_data[at];
+        if (COLS) bc[a] = *reinterpret_cast<const int32_t *>(B_indices + at);   // columns fit 31 bits
     }
+    int32_t *ccol = s_ccol + (COLS ? g * kAccStride : 0);
 #pragma unroll
     for (int a = 0; a < kCap; ++a) {
         // the lanes of a group hold different entries of one B row: different columns, different
         // accumulators; the entries of A take their turns one after the other
-        if (db[a] != kNone) acc[db[a]] = acc[db[a]] + s_av[slot + a] * bv[a];
+        if (db[a] != kNone) {
+            acc[db[a]] = acc[db[a]] + s_av[slot + a] * bv[a];
+            if (COLS) ccol[db[a]] = bc[a];   // every product of an entry of C brings the same column
+        }
         group_fence();
     }
 #pragma unroll
     for (int q = 0; q < kCap; ++q)
-        if (k + kCap * q < clen) C_data[cs + k + kCap * q] = acc[k + kCap * q];
+        if (k + kCap * q < clen) {
+            C_data[cs + k + kCap * q] = acc[k + kCap * q];
+            if (COLS) C_indices[cs + k + kCap * q] = (int64_t)ccol[k + kCap * q];
+        }
 }
 
 // ---- backward ------------------------------------------------------------------------
@@ -367,6 +362,50 @@ extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nn
     return NM_OK;
 }
 
+extern "C" int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                                    int64_t hash_rows, const void *A_plan_mem, void *plan_mem, size_t plan_bytes,
+                                    void *host_landing, int *usable, nm_stream stream) {
+    NM_REQUIRE(A_rows >= 0 && A_cols >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
+    NM_REQUIRE(usable && plan_mem && A_plan_mem, "null pointer argument");
+    const size_t need = pplan_layout(A_nnz, nullptr, nullptr);
+    if (plan_bytes < need) return nm::fail(NM_ERR_WORKSPACE, "plan of %zu bytes, %zu needed", plan_bytes, need);
+    *usable = 0;
+    const int64_t lim = (int64_t)1 << 31;
+    // what the forward pass that filled the plan has established: every row on the merge path
+    // (hence the limits on rows of A, B and C); what is left is the length of A's columns
+    if (hash_rows != 0 || A_nnz >= lim || B_nnz >= lim || C_nnz >= lim || A_rows == 0 || A_nnz == 0 || C_nnz == 0)
+        return NM_OK;
+    hipStream_t s = nm::as_stream(stream);
+    PPlan p;
+    pplan_layout(A_nnz, plan_mem, &p);
+    nm::TPlan t;
+    nm::tplan_layout(A_rows, A_cols, A_nnz, const_cast<void *>(A_plan_mem), &t);
+    if (int rc = nm::fill_async(p.flag, 16, (int32_t)0, s)) return rc;
+    int64_t grid = nm::ceil_div(A_cols > 0 ? A_cols : 1, (int64_t)kBlock);
+    if (grid > 4096) grid = 4096;
+    hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, p.flag);
+    NM_LAUNCH_CHECK("plan_columns_kernel");
+    int32_t flag = 1;
+    if (host_landing) {
+        volatile int64_t *land = (volatile int64_t *)host_landing;
+        const int64_t ticket = land[2] + 1;
+        hipLaunchKernelGGL(plan_flag_out_kernel, dim3(1), dim3(64), 0, s, p.flag, land, ticket);
+        NM_LAUNCH_CHECK("plan_flag_out_kernel");
+        bool arrived = false;
+        for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = land[2] == ticket;
+        if (!arrived) {
+            NM_HIP_TRY(hipStreamSynchronize(s));
+            NM_REQUIRE(land[2] == ticket, "the plan's verdict did not arrive");
+        }
+        flag = (int32_t)land[0];
+    } else {
+        NM_HIP_TRY(hipMemcpyAsync(&flag, p.flag, sizeof(flag), hipMemcpyDeviceToHost, s));
+        NM_HIP_TRY(hipStreamSynchronize(s));
+    }
+    *usable = flag == 0 ? 1 : 0;
+    return NM_OK;
+}
+
 extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
                                          const void *A_data, const int64_t *A_indptr, const void *B_data,
                                          const void *plan_mem, const int64_t *C_indptr, void *C_data,
@@ -381,13 +420,31 @@ extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int64_t A_rows, int64_t A_
     const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)kGroupsPerBlock));
     NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
     if (dt == NM_F32)
-        hipLaunchKernelGGL(numeric_planned_kernel<float>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, grid,
-                           (const float *)A_data, A_indptr, (const float *)B_data, p.bstart, p.dest, C_indptr,
-                           (float *)C_data);
+        hipLaunchKernelGGL((numeric_planned_kernel<float, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
+                           grid, (const float *)A_data, A_indptr, (const float *)B_data, (const int64_t *)nullptr,
+                           p.bstart, p.dest, C_indptr, (float *)C_data, (int64_t *)nullptr, (int32_t *)nullptr);
     else
-        hipLaunchKernelGGL(numeric_planned_kernel<double>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, grid,
-                           (const double *)A_data, A_indptr, (const double *)B_data, p.bstart, p.dest, C_indptr,
-                           (double *)C_data);
+        hipLaunchKernelGGL((numeric_planned_kernel<double, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
+                           grid, (const double *)A_data, A_indptr, (const double *)B_data, (const int64_t *)nullptr,
+                           p.bstart, p.dest, C_indptr, (double *)C_data, (int64_t *)nullptr, (int32_t *)nullptr);
+    NM_LAUNCH_CHECK("numeric_planned_kernel");
+    return NM_OK;
+}
+
+int nm::spgemm_numeric_on_map(nm_dtype dt, int64_t A_rows, int64_t A_nnz, const void *A_data,
+                              const int64_t *A_indptr, const void *B_data, const int64_t *B_indices, const PPlan &p,
+                              const int64_t *C_indptr, int64_t *C_indices, void *C_data, hipStream_t s) {
+    if (A_rows == 0 || A_nnz == 0) return NM_OK;
+    const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)kGroupsPerBlock));
+    NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+    if (dt == NM_F32)
+        hipLaunchKernelGGL((numeric_planned_kernel<float, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
+                           grid, (const float *)A_data, A_indptr, (const float *)B_data, B_indices, p.bstart, p.dest,
+                           C_indptr, (float *)C_data, C_indices, p.cstart);
+    else
+        hipLaunchKernelGGL((numeric_planned_kernel<double, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
+                           grid, (const double *)A_data, A_indptr, (const double *)B_data, B_indices, p.bstart, p.dest,
+                           C_indptr, (double *)C_data, C_indices, p.cstart);
     NM_LAUNCH_CHECK("numeric_planned_kernel");
     return NM_OK;
 }

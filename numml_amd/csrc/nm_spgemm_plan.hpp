@@ -1,0 +1,45 @@
+// Product plan of a sparse product C = A B (see nm_spgemm_plan.hip for what it is and what runs
+// on it).  Shared between the file that builds and uses the plan and the SpGEMM forward, whose
+// symbolic phase can leave the plan's destination bytes behind as a by-product of its merge and
+// whose numeric phase can then run on them.
+#pragma once
+
+#include "nm_common.hpp"
+#include "nm_transpose.hpp"
+
+namespace nm {
+
+constexpr int kPlanCap = 8;                      // entries per row of A and per named row of B
+constexpr int kPlanRowCap = kPlanCap * kPlanCap; // entries per row of C
+constexpr uint8_t kPlanNone = 0xFF;              // destination byte of an entry a B row does not have
+
+struct PPlan {
+    int32_t *flag;     // [0] != 0: a limit does not hold, the plan must not be used
+    int32_t *bstart;   // [A_nnz] where the row of B that entry e of A names starts
+    int32_t *cstart;   // [A_nnz] where the row of C that entry e of A lies in starts
+    uint8_t *dest;     // [A_nnz * 8] byte k: position in that row of C of the k-th entry of that row of B
+};
+
+inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += align256(bytes);
+        return q;
+    };
+    int32_t *flag = (int32_t *)take(64);
+    int32_t *bs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
+    int32_t *cs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
+    uint8_t *d = (uint8_t *)take((size_t)(A_nnz + 1) * 8);
+    if (p) *p = PPlan{flag, bs, cs, d};
+    return off;
+}
+
+// C_data AND C_indices of the product from the destination bytes and row starts of B that the
+// symbolic phase left in `p` (every row on the merge path); also writes p.cstart, which completes
+// the plan.  C_indptr is the scanned row pointer.
+int spgemm_numeric_on_map(nm_dtype dt, int64_t A_rows, int64_t A_nnz, const void *A_data, const int64_t *A_indptr,
+                          const void *B_data, const int64_t *B_indices, const PPlan &p, const int64_t *C_indptr,
+                          int64_t *C_indices, void *C_data, hipStream_t s);
+
+}  // namespace nm

@@ -448,11 +448,14 @@ std::shared_ptr<Plan> peek_product_plan(const Tensor &A_indices, const Tensor &A
     return plan;
 }
 
-// After a stateless forward pass of a product without hash-path rows: notes the pair, or builds
-// its plan around the pattern of C that the pass has just produced.
+// After a stateless forward pass of a product without hash-path rows: notes the pair, or makes
+// its plan around the pattern of C that the pass has just produced.  `filled`: plan memory that
+// the pass filled as it went (nm_spgemm_symbolic_mapped / nm_spgemm_numeric_mapped), which only
+// has to be checked; without it the plan is built from the three patterns.
 void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, const Tensor &B_indices,
                            const Tensor &B_indptr, const Tensor &C_indices, const Tensor &C_indptr,
-                           int64_t A_rows, int64_t A_cols, int64_t B_cols, const c10::Device &dev) {
+                           int64_t A_rows, int64_t A_cols, int64_t B_cols, const c10::Device &dev,
+                           const Tensor &filled = Tensor()) {
     const int mode = backward_mode_now();
     if (mode == kAtomic || A_indices.numel() == 0 || C_indices.numel() == 0) return;
     Key ka, kb;
@@ -485,15 +488,23 @@ void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, cons
     plan->parent = transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev);
     size_t pbytes = 0;
     check(nm_spgemm_plan_bytes(A_indices.numel(), &pbytes), "nm_spgemm_plan_bytes");
-    plan->mem = scratch(pbytes, dev);
     int usable = 0;
-    check(nm_spgemm_plan_build(A_rows, A_cols, A_indices.numel(), B_indices.numel(), C_indices.numel(),
-                               A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
-                               B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
-                               C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(),
-                               plan->parent->mem.data_ptr(), plan->mem.data_ptr(), pbytes, host_landing(), &usable,
-                               current_stream(dev)),
-          "nm_spgemm_plan_build");
+    if (filled.defined()) {
+        plan->mem = filled;
+        check(nm_spgemm_plan_adopt(A_rows, A_cols, A_indices.numel(), B_indices.numel(), C_indices.numel(), 0,
+                                   plan->parent->mem.data_ptr(), plan->mem.data_ptr(), pbytes, host_landing(),
+                                   &usable, current_stream(dev)),
+              "nm_spgemm_plan_adopt");
+    } else {
+        plan->mem = scratch(pbytes, dev);
+        check(nm_spgemm_plan_build(A_rows, A_cols, A_indices.numel(), B_indices.numel(), C_indices.numel(),
+                                   A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                   B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                                   C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(),
+                                   plan->parent->mem.data_ptr(), plan->mem.data_ptr(), pbytes, host_landing(),
+                                   &usable, current_stream(dev)),
+              "nm_spgemm_plan_build");
+    }
     plan->usable = usable != 0;
     if (plan->usable) {
         plan->derived = {C_indices, C_indptr};
@@ -907,10 +918,28 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
     Tensor C_indptr = torch::empty({(int64_t)A_rows + 1}, iopt);
     nm_stream st = current_stream(dev);
-    check(nm_spgemm_symbolic(A_rows, A_cols, B_cols, A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
-                             B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
-                             C_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes, host_landing(), st),
-          "nm_spgemm_symbolic");
+    // Unless plans are switched off, the symbolic merge records where every product goes (16 bytes
+    // per entry of A): with no row on the hash path the numeric phase then adds the products up on
+    // those records instead of merging the rows again, and the records are a product plan's.
+    const int64_t A_nnz = A_data.numel(), B_nnz = B_data.numel();
+    const int64_t lim31 = (int64_t)1 << 31;
+    Tensor filled;
+    size_t pbytes = 0;
+    if (plans && A_nnz > 0 && A_nnz < lim31 && B_nnz < lim31) {
+        check(nm_spgemm_plan_bytes(A_nnz, &pbytes), "nm_spgemm_plan_bytes");
+        filled = scratch(pbytes, dev);
+        check(nm_spgemm_symbolic_mapped(A_rows, A_cols, B_cols, A_nnz, B_nnz, A_indices.data_ptr<int64_t>(),
+                                        A_indptr.data_ptr<int64_t>(), B_indices.data_ptr<int64_t>(),
+                                        B_indptr.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(), work.data_ptr(),
+                                        bytes, filled.data_ptr(), pbytes, host_landing(), st),
+              "nm_spgemm_symbolic_mapped");
+    } else {
+        check(nm_spgemm_symbolic(A_rows, A_cols, B_cols, A_indices.data_ptr<int64_t>(),
+                                 A_indptr.data_ptr<int64_t>(), B_indices.data_ptr<int64_t>(),
+                                 B_indptr.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(), work.data_ptr(), bytes,
+                                 host_landing(), st),
+              "nm_spgemm_symbolic");
+    }
     // the one device->host read the interface makes inherent: C is returned exactly sized
     int64_t nnz_c = 0, hash_rows = 0;
     check(nm_spgemm_symbolic_result(A_rows, B_cols, work.data_ptr(), bytes, &nnz_c, &hash_rows, host_landing(),
@@ -924,15 +953,17 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     }
     Tensor C_indices = torch::empty({nnz_c}, iopt);
     Tensor C_data = torch::empty({nnz_c}, A_data.options());
-    check(nm_spgemm_numeric(dtype_of(A_data), A_rows, A_cols, B_cols, A_data.data_ptr(),
-                            A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
-                            B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
-                            C_indptr.data_ptr<int64_t>(), C_indices.data_ptr<int64_t>(), C_data.data_ptr(),
-                            work.data_ptr(), bytes, hash_rows, st),
-          "nm_spgemm_numeric");
-    if (hash_rows == 0)
+    const bool on_map = filled.defined() && hash_rows == 0 && nnz_c > 0 && nnz_c < lim31;
+    check(nm_spgemm_numeric_mapped(dtype_of(A_data), A_rows, A_cols, B_cols, A_nnz, nnz_c, A_data.data_ptr(),
+                                   A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
+                                   B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                                   C_indptr.data_ptr<int64_t>(), C_indices.data_ptr<int64_t>(), C_data.data_ptr(),
+                                   work.data_ptr(), bytes, hash_rows, on_map ? filled.data_ptr() : nullptr, pbytes,
+                                   st),
+          "nm_spgemm_numeric_mapped");
+    if (on_map)
         consider_product_plan(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr, A_rows, A_cols, B_cols,
-                              dev);
+                              dev, filled);
     return {C_data, C_indices, C_indptr};
 }
 

@@ -547,15 +547,63 @@ def spgemm_backward(grad_C, C_indices, C_indptr,
     return [grad_A, grad_B]
 
 
+def spgemm_forward_mapped(A_rows, A_cols, A_data, A_indices, A_indptr,
+                          B_rows, B_cols, B_data, B_indices, B_indptr):
+    """[C_data, C_indices, C_indptr, plan]: spgemm_forward through nm_spgemm_symbolic_mapped /
+    nm_spgemm_numeric_mapped, which compute the product on the destination records that the
+    symbolic merge leaves behind, and the ProductPlan those records make (its ``usable`` is False
+    when the product has rows on the hash path or the plan's limits do not hold)."""
+    _check_csr("spgemm_forward", A_rows, A_cols, A_data, A_indices, A_indptr)
+    _check_csr("spgemm_forward", B_rows, B_cols, B_data, B_indices, B_indptr)
+    if A_cols != B_rows:
+        raise RuntimeError(f"spgemm_forward: A has {A_cols} columns but B has {B_rows} rows")
+    dev = _need_device(A_data, A_indices, A_indptr, B_data, B_indices, B_indptr)
+    _same_dtype(A_data, B_data, "B_data")
+    A_data, B_data = A_data.contiguous(), B_data.contiguous()
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    B_indices, B_indptr = _idx(B_indices, "B_indices"), _idx(B_indptr, "B_indptr")
+    L = _lib.lib()
+    A_nnz, B_nnz = A_indices.shape[0], B_indices.shape[0]
+    with torch.cuda.device(dev):
+        nbytes, pbytes = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _lib.check(L.nm_spgemm_workspace_bytes(A_rows, B_cols, ctypes.byref(nbytes)),
+                   "nm_spgemm_workspace_bytes")
+        _lib.check(L.nm_spgemm_plan_bytes(A_nnz, ctypes.byref(pbytes)), "nm_spgemm_plan_bytes")
+        work = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+        mem = torch.empty(max(pbytes.value, 8), dtype=torch.uint8, device=dev)
+        C_indptr = torch.empty(A_rows + 1, dtype=torch.int64, device=dev)
+        st = _stream(dev)
+        _lib.check(L.nm_spgemm_symbolic_mapped(
+            A_rows, A_cols, B_cols, A_nnz, B_nnz, _ptr(A_indices), _ptr(A_indptr), _ptr(B_indices),
+            _ptr(B_indptr), _ptr(C_indptr), _ptr(work), nbytes.value, _ptr(mem), pbytes.value,
+            _ptr(_host_landing()), st), "nm_spgemm_symbolic_mapped")
+        nnz_c, hash_rows = ctypes.c_int64(0), ctypes.c_int64(0)
+        _lib.check(L.nm_spgemm_symbolic_result(A_rows, B_cols, _ptr(work), nbytes.value, ctypes.byref(nnz_c),
+                                               ctypes.byref(hash_rows), _ptr(_host_landing()), st),
+                   "nm_spgemm_symbolic_result")
+        C_indices = torch.empty(nnz_c.value, dtype=torch.int64, device=dev)
+        C_data = torch.empty(nnz_c.value, dtype=A_data.dtype, device=dev)
+        _lib.check(L.nm_spgemm_numeric_mapped(
+            _dt(A_data), A_rows, A_cols, B_cols, A_nnz, nnz_c.value, _ptr(A_data), _ptr(A_indices),
+            _ptr(A_indptr), _ptr(B_data), _ptr(B_indices), _ptr(B_indptr), _ptr(C_indptr), _ptr(C_indices),
+            _ptr(C_data), _ptr(work), nbytes.value, hash_rows.value, _ptr(mem), pbytes.value, st),
+            "nm_spgemm_numeric_mapped")
+        plan = ProductPlan(A_rows, A_cols, A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr,
+                           adopt=(mem, hash_rows.value))
+    return [C_data, C_indices, C_indptr, plan]
+
+
 class ProductPlan:
     """Product plan of C = A B (nm_spgemm_plan_build): numeric product and gradients of a product
     whose three patterns are known, without the symbolic phase and without searches.
 
     ``usable`` is False when a row is longer than the plan's limits; then neither method may be
-    called.  The plan keeps the structure tensors it was built from alive.
+    called.  The plan keeps the structure tensors it was built from alive.  With ``adopt`` =
+    (plan memory filled by a mapped forward pass, its hash_rows) nothing is built: the memory is
+    checked (nm_spgemm_plan_adopt) and taken over.
     """
 
-    def __init__(self, A_rows, A_cols, A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr):
+    def __init__(self, A_rows, A_cols, A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr, adopt=None):
         dev = _need_device(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr)
         L = _lib.lib()
         self.dev, self.A_rows, self.A_cols = dev, A_rows, A_cols
@@ -565,8 +613,16 @@ class ProductPlan:
             self.transposed = _transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev)
             nbytes = ctypes.c_size_t(0)
             _lib.check(L.nm_spgemm_plan_bytes(self.A_nnz, ctypes.byref(nbytes)), "nm_spgemm_plan_bytes")
-            self.mem = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
             usable = ctypes.c_int(0)
+            if adopt is not None:
+                self.mem, hash_rows = adopt
+                _lib.check(L.nm_spgemm_plan_adopt(
+                    A_rows, A_cols, self.A_nnz, self.B_nnz, self.C_nnz, hash_rows, _ptr(self.transposed.mem),
+                    _ptr(self.mem), nbytes.value, _ptr(_host_landing()), ctypes.byref(usable), _stream(dev)),
+                    "nm_spgemm_plan_adopt")
+                self.usable = bool(usable.value)
+                return
+            self.mem = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
             _lib.check(L.nm_spgemm_plan_build(
                 A_rows, A_cols, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(A_indices), _ptr(A_indptr),
                 _ptr(B_indices), _ptr(B_indptr), _ptr(C_indices), _ptr(C_indptr), _ptr(self.transposed.mem),

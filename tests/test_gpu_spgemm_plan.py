@@ -70,6 +70,17 @@ def test_planned_product_and_gradients_match_the_stateless_kernels_and_the_oracl
         rA, rB = oracle.spgemm_backward(g, ci, cp, A_rows, A_cols, ad2, ai, ap, B_rows, B_cols, bd2, bi, bp)
         assert_same(host(gA), rA, f"{name}: grad_A vs oracle")
         assert_same(host(gB), rB, f"{name}: grad_B vs oracle")
+        # the same product computed on the records its own symbolic phase leaves behind, and the plan
+        # those records make
+        md, mi, mp, mplan = mirror.spgemm_forward_mapped(A_rows, A_cols, AD2, AI, AP, B_rows, B_cols, BD2, BI, BP)
+        assert_same(host(mp), cp, f"{name}: C_indptr (mapped forward)")
+        assert_same(host(mi), ci, f"{name}: C_indices (mapped forward)")
+        assert_same(host(md), cd, f"{name}: C_data (mapped forward)")
+        assert mplan.usable, name
+        assert_same(host(mplan.numeric(AD, BD)), host(C_data), f"{name}: C_data on the adopted plan")
+        mA, mB = mplan.backward(Gz, AD2, BD2)
+        assert_same(host(mA), rA, f"{name}: grad_A on the adopted plan")
+        assert_same(host(mB), rB, f"{name}: grad_B on the adopted plan")
         old = mirror.BACKWARD_MODE
         mirror.BACKWARD_MODE = "eager"
         try:
@@ -142,6 +153,16 @@ def test_random_short_row_products(dev, seed, dtype):
         assert not plan.usable          # nothing to plan for a matrix without entries
         return
     assert plan.usable
+    md, mi, mp, mplan = mirror.spgemm_forward_mapped(m, kdim, AD, AI, AP, kdim, n, BD, BI, BP)
+    assert_same(host(mi), host(C_indices), "pattern (mapped forward)")
+    assert_same(host(md), host(C_data), "C_data (mapped forward)")
+    assert mplan.usable
+    # the adopted plan is the built one, array for array (flag word, then bstart, cstart, dest,
+    # each starting on a multiple of 256 bytes)
+    nnz_a, off = ai.shape[0], 256
+    for name, width in (("bstart", 4), ("cstart", 4), ("dest", 8)):
+        assert torch.equal(mplan.mem[off:off + nnz_a * width], plan.mem[off:off + nnz_a * width]), name
+        off += ((nnz_a + 1) * width + 255) // 256 * 256
     ad2, bd2 = randn(seed, ad.shape[0], dtype), randn(seed + 50, bd.shape[0], dtype)
     AD2, BD2 = to_dev(dev, ad2, bd2)
     cd, ci, cp = oracle.spgemm_forward(m, kdim, ad2, ai, ap, kdim, n, bd2, bi, bp)
