@@ -101,6 +101,19 @@ __global__ __launch_bounds__(kBlock) void plan_columns_kernel(int64_t cols, cons
     if (bad) flag[0] = 1;
 }
 
+// The column-major copies of cstart and dest (entry t of the transposed plan is entry t_perm[t]).
+__global__ __launch_bounds__(kBlock) void plan_by_column_kernel(int64_t A_nnz, const int32_t *__restrict__ t_perm,
+                                                               PPlan p) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    const uint64_t *dest64 = reinterpret_cast<const uint64_t *>(p.dest);
+    uint64_t *t_dest64 = reinterpret_cast<uint64_t *>(p.t_dest);
+    for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < A_nnz; t += stride) {
+        const int32_t e = t_perm[t];
+        p.t_cstart[t] = p.cstart[e];
+        t_dest64[t] = dest64[e];
+    }
+}
+
 __global__ void plan_flag_out_kernel(const int32_t *flag, volatile int64_t *host_pinned, int64_t ticket) {
     if (threadIdx.x == 0) {
         host_pinned[0] = flag[0];
@@ -238,7 +251,7 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
     const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm, const int64_t *__restrict__ B_indptr,
-    const int32_t *__restrict__ cstart, const uint8_t *__restrict__ dest, T *__restrict__ grad_B) {
+    const int32_t *__restrict__ t_cstart, const uint8_t *__restrict__ t_dest, T *__restrict__ grad_B) {
     __shared__ T s_a[kBlock];
     __shared__ int32_t s_cs[kBlock];
     __shared__ __align__(8) uint8_t s_db[kBlock * kCap];
@@ -259,11 +272,11 @@ __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     for (int32_t t0 = pb; t0 < pe; t0 += kCap) {
         {
             const bool have = t0 + k < pe;
-            const int32_t e = t_perm[have ? t0 + k : pb];
-            s_a[threadIdx.x] = A_data[e];
-            s_cs[threadIdx.x] = cstart[e];
+            const int32_t t = have ? t0 + k : pb;
+            s_a[threadIdx.x] = A_data[t_perm[t]];
+            s_cs[threadIdx.x] = t_cstart[t];
             *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) =
-                have ? *reinterpret_cast<const uint64_t *>(dest + (int64_t)e * kCap) : ~uint64_t(0);
+                have ? *reinterpret_cast<const uint64_t *>(t_dest + (int64_t)t * kCap) : ~uint64_t(0);
         }
         group_fence();
         uint8_t db[kCap];
@@ -296,7 +309,7 @@ int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A
         const int64_t grid = nm::xcd_padded(nm::ceil_div(A_cols, (int64_t)kGroupsPerBlock));
         NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
         hipLaunchKernelGGL(grad_b_mapped_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, grid,
-                           (const T *)gC, (const T *)A_data, t.t_indptr, t.t_perm, B_indptr, p.cstart, p.dest,
+                           (const T *)gC, (const T *)A_data, t.t_indptr, t.t_perm, B_indptr, p.t_cstart, p.t_dest,
                            (T *)grad_B);
         NM_LAUNCH_CHECK("grad_b_mapped_kernel");
     }
@@ -341,6 +354,10 @@ extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nn
     if (grid > 4096) grid = 4096;
     hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, p.flag);
     NM_LAUNCH_CHECK("plan_columns_kernel");
+    grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p);
+    NM_LAUNCH_CHECK("plan_by_column_kernel");
     int32_t flag = 1;
     if (host_landing) {
         volatile int64_t *land = (volatile int64_t *)host_landing;
@@ -385,6 +402,10 @@ extern "C" int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nn
     if (grid > 4096) grid = 4096;
     hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, p.flag);
     NM_LAUNCH_CHECK("plan_columns_kernel");
+    grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p);
+    NM_LAUNCH_CHECK("plan_by_column_kernel");
     int32_t flag = 1;
     if (host_landing) {
         volatile int64_t *land = (volatile int64_t *)host_landing;

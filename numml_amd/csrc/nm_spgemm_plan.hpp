@@ -18,6 +18,11 @@ struct PPlan {
     int32_t *bstart;   // [A_nnz] where the row of B that entry e of A names starts
     int32_t *cstart;   // [A_nnz] where the row of C that entry e of A lies in starts
     uint8_t *dest;     // [A_nnz * 8] byte k: position in that row of C of the k-th entry of that row of B
+    // cstart and dest once more in COLUMN-major order of A (entry t of the transposed-structure
+    // plan): the kernel that walks A by column streams them instead of gathering 12 bytes from a
+    // different line for every entry.  Filled when the plan is built or adopted.
+    int32_t *t_cstart; // [A_nnz]
+    uint8_t *t_dest;   // [A_nnz * 8]
 };
 
 inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p) {
@@ -31,7 +36,9 @@ inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p) {
     int32_t *bs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
     int32_t *cs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
     uint8_t *d = (uint8_t *)take((size_t)(A_nnz + 1) * 8);
-    if (p) *p = PPlan{flag, bs, cs, d};
+    int32_t *tcs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
+    uint8_t *td = (uint8_t *)take((size_t)(A_nnz + 1) * 8);
+    if (p) *p = PPlan{flag, bs, cs, d, tcs, td};
     return off;
 }
 

@@ -1264,6 +1264,10 @@ std::string backward_mode() {
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "numml_torch_cpp on AMD gfx950: differentiable CSR SpMV / SpMM / SpGEMM / SpTRSV";
+    // The plan cache holds device tensors and events.  They are given back while the interpreter,
+    // torch's allocator and the HIP runtime are still there: left to this library's static
+    // destructors they would be freed after those have gone.
+    pybind11::module_::import("atexit").attr("register")(pybind11::cpp_function([] { clear_plan_cache(); }));
     m.def("spgemv_forward", &spgemv_forward, "SPGEMV forward");
     m.def("spgemv_backward", &spgemv_backward, "SPGEMV backward");
     m.def("spgemm_forward", &spgemm_forward, "SPGEMM forward");

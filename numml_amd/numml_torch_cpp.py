@@ -9,6 +9,7 @@ from its caching allocator) and for the current stream, nothing else.
 Unlike the reference there is no CPU implementation behind these functions:
 tensors that are not on a HIP device raise ``RuntimeError``.
 """
+import atexit
 import collections
 import ctypes
 import os
@@ -134,6 +135,10 @@ BACKWARD_MODE = os.environ.get("NUMML_AMD_BACKWARD", "planned")
 def clear_plan_cache():
     with _plans_lock:
         _plans.clear()
+
+
+# plans hold device tensors and events: given back while torch is still whole
+atexit.register(clear_plan_cache)
 
 
 def _cached(kind, indices, indptr, extra, make):
