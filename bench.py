@@ -371,8 +371,7 @@ class SpGEMM(Workload):
         firsts = _first_calls(ext, one_step)
         C = self.C
         self.first_steps_ms = firsts
-        self.planned = (_binding.backward_mode() != "atomic" and _binding.name == "compiled"
-                        and self.left == "A")
+        self.planned = _binding.backward_mode() != "atomic" and _binding.name == "compiled"
         self.C = C
         lens = np.diff(p)
         self.products = int(lens[self.hostL[1]].sum())

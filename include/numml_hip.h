@@ -256,14 +256,17 @@ int nm_spgemm_backward_planned(nm_dtype dt, int64_t A_rows, int64_t A_cols, int6
  *   nm_spgemm_plan_build    C_indices / C_indptr must be the pattern of A B as
  *                           nm_spgemm_numeric returns it (complete, rows ascending).
  *                           A_plan_mem: the transposed-structure plan of A
- *                           (nm_csr_transpose_plan_build).  *usable = 1 when every
- *                           row of A, every row of B that A names and every row of C
- *                           stays within 8 / 8 / 64 entries, no column of A holds
- *                           more than 4096 and all positions fit 31 bits; otherwise
- *                           0 and the plan must not be used.  Waits for the stream
- *                           (through host_landing, 24 bytes of pinned host memory,
- *                           when given; NULL: a copy and a synchronisation).
- *   nm_spgemm_numeric_planned   C_data of the product, C_indptr as built from.
+ *                           (nm_csr_transpose_plan_build).  *usable = 0: the plan
+ *                           must not be used (a row of B that A names has more than
+ *                           8 entries, a row of C more than 254, a column of A more
+ *                           than 4096, or a position does not fit 31 bits).
+ *                           Otherwise the product's class: 1 -- rows of A of at most
+ *                           8 and rows of C of at most 64 entries, 2 -- longer rows of
+ *                           A, 3 -- also rows of C of 65..254 entries.  Waits for the
+ *                           stream (through host_landing, 24 bytes of pinned host
+ *                           memory, when given; NULL: a copy and a synchronisation).
+ *   nm_spgemm_numeric_planned   C_data of the product, C_indptr as built from;
+ *                           plan_class as reported when the plan was built.
  *   nm_spgemm_backward_mapped   grad_A and / or grad_B (either may be NULL) of
  *                           gC laid out on the plan's pattern of C.
  *
@@ -306,8 +309,8 @@ int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t 
                          const int64_t *C_indices, const int64_t *C_indptr,
                          const void *A_plan_mem, void *plan_mem, size_t plan_bytes,
                          void *host_landing, int *usable, nm_stream stream);
-int nm_spgemm_numeric_planned(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
-                              const void *A_data, const int64_t *A_indptr, const void *B_data,
+int nm_spgemm_numeric_planned(nm_dtype dt, int plan_class, int64_t A_rows, int64_t A_nnz, int64_t B_nnz,
+                              int64_t C_nnz, const void *A_data, const int64_t *A_indptr, const void *B_data,
                               const void *plan_mem, const int64_t *C_indptr, void *C_data,
                               nm_stream stream);
 int nm_spgemm_backward_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_t A_nnz,

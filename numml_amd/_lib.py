@@ -59,8 +59,8 @@ _SIGNATURES = {
     "nm_spgemm_plan_bytes": [_c_i64, ctypes.POINTER(_c_size)],
     "nm_spgemm_plan_build": [_c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                              _c_ptr, _c_ptr, _c_size, _c_ptr, ctypes.POINTER(_c_int), _c_ptr],
-    "nm_spgemm_numeric_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                                  _c_ptr, _c_ptr],
+    "nm_spgemm_numeric_planned": [_c_int, _c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                  _c_ptr, _c_ptr, _c_ptr],
     "nm_spgemm_backward_mapped": [_c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_sptrsv_plan_bytes": [_c_i64, _c_i64, ctypes.POINTER(_c_size), ctypes.POINTER(_c_size)],

@@ -13,9 +13,13 @@
 //               k-th entry of row j of B, 0xFF when that row has no k-th entry
 //
 // so that the product a_e * b_(j,k) is known to belong to C[cstart[e] + dest[e][k]] without a
-// merge, a hash table or a search.  The plan exists for products whose rows all stay inside the
-// merge path's limits: at most kCap entries per row of A and per row of B that A names, and
-// rows of C of at most kRowCap entries; nm_spgemm_plan_build reports whether they hold.
+// merge, a hash table or a search.  The plan exists for products in which every row of B that A
+// names has at most kCap entries and every row of C at most kWideCap; rows of A may be of any
+// length.  nm_spgemm_plan_build reports whether that holds and which of three classes the product
+// is in: 1 -- rows of A of at most kCap entries and rows of C of at most kRowCap (everything the
+// SpGEMM merge path takes; such a plan is also a by-product of the mapped forward pass), 2 -- longer
+// rows of A, 3 -- also rows of C of up to kWideCap entries.  The class picks the forward kernel;
+// the gradient kernels are the same for all.
 //
 //   forward    eight lanes per row of C; the products of the row's entries of A are added to
 //              the row's accumulators in LDS one entry of A after the other, i.e. every C entry
@@ -40,6 +44,7 @@ constexpr int kBlock = 256;
 constexpr int kCap = nm::kPlanCap;            // entries per row of A and per named row of B
 constexpr int kRowCap = nm::kPlanRowCap;      // entries per row of C
 constexpr int kGroupsPerBlock = kBlock / kCap;
+constexpr int kWideCap = 254;                 // entries per row of C in class 3 (a destination is a byte, 0xFF is taken)
 constexpr int32_t kMaxColumn = 4096;          // entries per column of A: one group of lanes walks a column
 constexpr uint8_t kNone = nm::kPlanNone;
 
@@ -55,14 +60,16 @@ __global__ __launch_bounds__(kBlock) void plan_map_kernel(
     const int64_t *__restrict__ C_indices, const int64_t *__restrict__ C_indptr, PPlan p) {
     const int k = threadIdx.x & (kCap - 1);
     const int64_t stride = (int64_t)gridDim.x * kGroupsPerBlock;
-    bool bad = false;
+    bool bad = false, long_a = false, wide_c = false;
     for (int64_t row = (int64_t)blockIdx.x * kGroupsPerBlock + threadIdx.x / kCap; row < rows; row += stride) {
         const int64_t ab = A_indptr[row], ae = A_indptr[row + 1];
         const int64_t cs = C_indptr[row], ce = C_indptr[row + 1];
-        if (ae - ab > kCap || ce - cs > kRowCap) {
+        if (ce - cs > kWideCap) {
             bad = true;
             continue;
         }
+        if (ae - ab > kCap) long_a = true;
+        if (ce - cs > kRowCap) wide_c = true;
         for (int64_t e = ab; e < ae; ++e) {
             const int64_t j = A_indices[e];
             const int64_t bb = B_indptr[j], blen = B_indptr[j + 1] - bb;
@@ -90,6 +97,8 @@ __global__ __launch_bounds__(kBlock) void plan_map_kernel(
         }
     }
     if (bad) p.flag[0] = 1;
+    if (long_a) p.flag[1] = 1;
+    if (wide_c) p.flag[2] = 1;
 }
 
 __global__ __launch_bounds__(kBlock) void plan_columns_kernel(int64_t cols, const int32_t *__restrict__ t_indptr,
@@ -117,6 +126,7 @@ __global__ __launch_bounds__(kBlock) void plan_by_column_kernel(int64_t A_nnz, c
 __global__ void plan_flag_out_kernel(const int32_t *flag, volatile int64_t *host_pinned, int64_t ticket) {
     if (threadIdx.x == 0) {
         host_pinned[0] = flag[0];
+        host_pinned[1] = flag[2] ? 3 : (flag[1] ? 2 : 1);   // the product's class
         __threadfence_system();
         host_pinned[2] = ticket;
     }
@@ -200,6 +210,63 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
             C_data[cs + k + kCap * q] = acc[k + kCap * q];
             if (COLS) C_indices[cs + k + kCap * q] = (int64_t)ccol[k + kCap * q];
         }
+}
+
+// The same for rows of A of any length (taken eight entries at a time) and rows of C of up to CAP
+// entries: classes 2 and 3.  A workgroup has as many groups of eight lanes as accumulator rows
+// fit some 16 KB of LDS.
+template <int CAP> struct LongShape {
+    static constexpr int kGroups = CAP <= kRowCap ? 32 : 8;
+    static constexpr int kThreads = kGroups * kCap;
+    static constexpr int kStride = CAP + 1;
+};
+
+template <typename T, int CAP>
+__global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_long_kernel(
+    int64_t rows, int64_t ntiles_padded, const T *__restrict__ A_data, const int64_t *__restrict__ A_indptr,
+    const T *__restrict__ B_data, const int32_t *__restrict__ bstart, const uint8_t *__restrict__ dest,
+    const int64_t *__restrict__ C_indptr, T *__restrict__ C_data) {
+    using S = LongShape<CAP>;
+    __shared__ T s_acc[S::kGroups * S::kStride];
+    __shared__ T s_av[S::kThreads];
+    __shared__ int32_t s_bs[S::kThreads];
+    __shared__ __align__(8) uint8_t s_db[S::kThreads * kCap];
+    const int k = threadIdx.x & (kCap - 1), g = threadIdx.x / kCap;
+    const int64_t row = nm::xcd_tile(blockIdx.x, ntiles_padded) * S::kGroups + g;
+    const bool live = row < rows;
+    const int64_t *pa = A_indptr + (live ? row : 0), *pc = C_indptr + (live ? row : 0);
+    const int64_t ab = pa[0], ae = live ? pa[1] : ab;
+    const int64_t cs = pc[0];
+    const int clen = live ? (int)(pc[1] - cs) : 0;
+    T *acc = s_acc + g * S::kStride;
+    for (int d = k; d < clen; d += kCap) acc[d] = T(0);
+    const int slot = g * kCap;
+    for (int64_t base = ab; base < ae; base += kCap) {
+        {   // lane k of the group fetches entry base + k of the row
+            const bool have = base + k < ae;
+            const int64_t e = have ? base + k : base;
+            const T av = A_data[e];
+            const int32_t bs = bstart[e];
+            const uint64_t db = *reinterpret_cast<const uint64_t *>(dest + e * kCap);
+            s_av[threadIdx.x] = av;
+            s_bs[threadIdx.x] = bs;
+            *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) = have ? db : ~uint64_t(0);
+        }
+        group_fence();
+        uint8_t db[kCap];
+        T bv[kCap];
+#pragma unroll
+        for (int a = 0; a < kCap; ++a) {
+            db[a] = s_db[(slot + a) * kCap + k];
+            bv[a] = B_data[db[a] != kNone ? (int64_t)s_bs[slot + a] + k : 0];
+        }
+#pragma unroll
+        for (int a = 0; a < kCap; ++a) {
+            if (db[a] != kNone) acc[db[a]] = acc[db[a]] + s_av[slot + a] * bv[a];
+            group_fence();
+        }
+    }
+    for (int d = k; d < clen; d += kCap) C_data[cs + d] = acc[d];
 }
 
 // ---- backward ------------------------------------------------------------------------
@@ -294,6 +361,29 @@ __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     if (mine) grad_B[bb + k] = acc;
 }
 
+// Brings the plan's flags to the host: *usable = 0, or the product's class (1, 2, 3).
+int read_verdict(const PPlan &p, void *host_landing, int *usable, hipStream_t s) {
+    int32_t flags[3] = {1, 0, 0};
+    if (host_landing) {
+        volatile int64_t *land = (volatile int64_t *)host_landing;
+        const int64_t ticket = land[2] + 1;
+        hipLaunchKernelGGL(plan_flag_out_kernel, dim3(1), dim3(64), 0, s, p.flag, land, ticket);
+        NM_LAUNCH_CHECK("plan_flag_out_kernel");
+        bool arrived = false;
+        for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = land[2] == ticket;
+        if (!arrived) {
+            NM_HIP_TRY(hipStreamSynchronize(s));
+            NM_REQUIRE(land[2] == ticket, "the plan's verdict did not arrive");
+        }
+        *usable = land[0] != 0 ? 0 : (int)land[1];
+        return NM_OK;
+    }
+    NM_HIP_TRY(hipMemcpyAsync(flags, p.flag, sizeof(flags), hipMemcpyDeviceToHost, s));
+    NM_HIP_TRY(hipStreamSynchronize(s));
+    *usable = flags[0] != 0 ? 0 : (flags[2] ? 3 : (flags[1] ? 2 : 1));
+    return NM_OK;
+}
+
 template <typename T>
 int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A_data, const nm::TPlan &t,
                     const void *B_data, const int64_t *B_indptr, const PPlan &p, void *grad_A, void *grad_B,
@@ -358,25 +448,7 @@ extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nn
     if (grid > 65536) grid = 65536;
     hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p);
     NM_LAUNCH_CHECK("plan_by_column_kernel");
-    int32_t flag = 1;
-    if (host_landing) {
-        volatile int64_t *land = (volatile int64_t *)host_landing;
-        const int64_t ticket = land[2] + 1;
-        hipLaunchKernelGGL(plan_flag_out_kernel, dim3(1), dim3(64), 0, s, p.flag, land, ticket);
-        NM_LAUNCH_CHECK("plan_flag_out_kernel");
-        bool arrived = false;
-        for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = land[2] == ticket;
-        if (!arrived) {
-            NM_HIP_TRY(hipStreamSynchronize(s));
-            NM_REQUIRE(land[2] == ticket, "the plan's verdict did not arrive");
-        }
-        flag = (int32_t)land[0];
-    } else {
-        NM_HIP_TRY(hipMemcpyAsync(&flag, p.flag, sizeof(flag), hipMemcpyDeviceToHost, s));
-        NM_HIP_TRY(hipStreamSynchronize(s));
-    }
-    *usable = flag == 0 ? 1 : 0;
-    return NM_OK;
+    return read_verdict(p, host_landing, usable, s);
 }
 
 extern "C" int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
@@ -406,38 +478,39 @@ extern "C" int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nn
     if (grid > 65536) grid = 65536;
     hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p);
     NM_LAUNCH_CHECK("plan_by_column_kernel");
-    int32_t flag = 1;
-    if (host_landing) {
-        volatile int64_t *land = (volatile int64_t *)host_landing;
-        const int64_t ticket = land[2] + 1;
-        hipLaunchKernelGGL(plan_flag_out_kernel, dim3(1), dim3(64), 0, s, p.flag, land, ticket);
-        NM_LAUNCH_CHECK("plan_flag_out_kernel");
-        bool arrived = false;
-        for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = land[2] == ticket;
-        if (!arrived) {
-            NM_HIP_TRY(hipStreamSynchronize(s));
-            NM_REQUIRE(land[2] == ticket, "the plan's verdict did not arrive");
-        }
-        flag = (int32_t)land[0];
-    } else {
-        NM_HIP_TRY(hipMemcpyAsync(&flag, p.flag, sizeof(flag), hipMemcpyDeviceToHost, s));
-        NM_HIP_TRY(hipStreamSynchronize(s));
-    }
-    *usable = flag == 0 ? 1 : 0;
+    return read_verdict(p, host_landing, usable, s);
+}
+
+template <typename T, int CAP>
+int launch_long(int64_t A_rows, const void *A_data, const int64_t *A_indptr, const void *B_data, const PPlan &p,
+                const int64_t *C_indptr, void *C_data, hipStream_t s) {
+    using S = LongShape<CAP>;
+    const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)S::kGroups));
+    NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+    hipLaunchKernelGGL((numeric_planned_long_kernel<T, CAP>), dim3((unsigned)grid), dim3(S::kThreads), 0, s, A_rows, grid,
+                       (const T *)A_data, A_indptr, (const T *)B_data, p.bstart, p.dest, C_indptr, (T *)C_data);
+    NM_LAUNCH_CHECK("numeric_planned_long_kernel");
     return NM_OK;
 }
 
-extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
-                                         const void *A_data, const int64_t *A_indptr, const void *B_data,
-                                         const void *plan_mem, const int64_t *C_indptr, void *C_data,
-                                         nm_stream stream) {
+extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int plan_class, int64_t A_rows, int64_t A_nnz, int64_t B_nnz,
+                                         int64_t C_nnz, const void *A_data, const int64_t *A_indptr,
+                                         const void *B_data, const void *plan_mem, const int64_t *C_indptr,
+                                         void *C_data, nm_stream stream) {
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
+    NM_REQUIRE(plan_class >= 1 && plan_class <= 3, "plan class %d (nm_spgemm_plan_build reports 1, 2 or 3)", plan_class);
     NM_REQUIRE(A_rows >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
     if (A_rows == 0 || A_nnz == 0 || B_nnz == 0 || C_nnz == 0) return NM_OK;   // C has no entries
     NM_REQUIRE(A_data && A_indptr && B_data && plan_mem && C_indptr && C_data, "null pointer argument");
     PPlan p;
     pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p);
     hipStream_t s = nm::as_stream(stream);
+    if (plan_class == 2)
+        return dt == NM_F32 ? launch_long<float, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s)
+                            : launch_long<double, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
+    if (plan_class == 3)
+        return dt == NM_F32 ? launch_long<float, 256>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s)
+                            : launch_long<double, 256>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
     const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)kGroupsPerBlock));
     NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
     if (dt == NM_F32)

@@ -179,6 +179,7 @@ struct Plan {
     std::vector<Tensor> derived;             // 'U', 'P': structure tensors handed out to callers
     std::vector<uint32_t> derived_versions;  //      and their version counters when built
     bool usable = true;                      // 'P': false when the product is beyond the plan's limits
+    int plan_class = 1;                      // 'P': which forward kernel the product takes (nm_spgemm_plan_build)
     std::shared_ptr<Plan> parent;            // 'P': the transposed-structure plan of A it walks
     nm_sptrsv_plan *handle = nullptr;
     // the stream the plan was built on and the event that marks its completion there
@@ -506,6 +507,7 @@ void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, cons
               "nm_spgemm_plan_build");
     }
     plan->usable = usable != 0;
+    plan->plan_class = usable;
     if (plan->usable) {
         plan->derived = {C_indices, C_indptr};
         for (const Tensor &t : plan->derived) plan->derived_versions.push_back(t._version());
@@ -901,7 +903,8 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     auto on_plan = [&](const Plan &plan) -> std::vector<Tensor> {
         const Tensor &C_indices = plan.derived[0], &C_indptr = plan.derived[1];
         Tensor C_data = torch::empty({C_indices.numel()}, A_data.options());
-        check(nm_spgemm_numeric_planned(dtype_of(A_data), A_rows, A_data.numel(), B_data.numel(), C_indices.numel(),
+        check(nm_spgemm_numeric_planned(dtype_of(A_data), plan.plan_class, A_rows, A_data.numel(), B_data.numel(),
+                                        C_indices.numel(),
                                         A_data.data_ptr(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
                                         plan.mem.data_ptr(), C_indptr.data_ptr<int64_t>(), C_data.data_ptr(),
                                         current_stream(dev)),
@@ -945,8 +948,8 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     check(nm_spgemm_symbolic_result(A_rows, B_cols, work.data_ptr(), bytes, &nnz_c, &hash_rows, host_landing(),
                                     st),
           "nm_spgemm_symbolic_result");
-    if (plans && hash_rows == 0 && nnz_c > 0) {
-        // eligible for a product plan: worth a content key per pattern that arrives in tensors not
+    if (plans && nnz_c > 0) {
+        // a product plan may exist: worth a content key per pattern that arrives in tensors not
         // seen before (a clone, a product computed again), which may find the pair's plan
         auto plan = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, A_rows, B_cols, dev, true);
         if (plan && plan->usable) return on_plan(*plan);
@@ -961,9 +964,14 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
                                    work.data_ptr(), bytes, hash_rows, on_map ? filled.data_ptr() : nullptr, pbytes,
                                    st),
           "nm_spgemm_numeric_mapped");
+    // note the pair, or make its plan: from the memory this pass filled, or (rows on the hash
+    // path: the plan's own analysis says whether the product is within its limits) from the patterns
     if (on_map)
         consider_product_plan(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr, A_rows, A_cols, B_cols,
                               dev, filled);
+    else if (plans && nnz_c > 0)
+        consider_product_plan(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr, A_rows, A_cols, B_cols,
+                              dev);
     return {C_data, C_indices, C_indptr};
 }
 

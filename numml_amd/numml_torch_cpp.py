@@ -625,7 +625,7 @@ class ProductPlan:
                     A_rows, A_cols, self.A_nnz, self.B_nnz, self.C_nnz, hash_rows, _ptr(self.transposed.mem),
                     _ptr(self.mem), nbytes.value, _ptr(_host_landing()), ctypes.byref(usable), _stream(dev)),
                     "nm_spgemm_plan_adopt")
-                self.usable = bool(usable.value)
+                self.usable, self.plan_class = bool(usable.value), usable.value
                 return
             self.mem = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
             _lib.check(L.nm_spgemm_plan_build(
@@ -633,7 +633,7 @@ class ProductPlan:
                 _ptr(B_indices), _ptr(B_indptr), _ptr(C_indices), _ptr(C_indptr), _ptr(self.transposed.mem),
                 _ptr(self.mem), nbytes.value, _ptr(_host_landing()), ctypes.byref(usable), _stream(dev)),
                 "nm_spgemm_plan_build")
-            self.usable = bool(usable.value)
+            self.usable, self.plan_class = bool(usable.value), usable.value
 
     def numeric(self, A_data, B_data):
         """C_data of the product (the pattern is the one the plan was built from)."""
@@ -643,7 +643,8 @@ class ProductPlan:
         with torch.cuda.device(self.dev):
             C_data = torch.empty(self.C_nnz, dtype=A_data.dtype, device=self.dev)
             _lib.check(_lib.lib().nm_spgemm_numeric_planned(
-                _dt(A_data), self.A_rows, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(A_data), _ptr(self.A_indptr),
+                _dt(A_data), self.plan_class, self.A_rows, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(A_data),
+                _ptr(self.A_indptr),
                 _ptr(B_data), _ptr(self.mem), _ptr(self.C_indptr), _ptr(C_data), _stream(self.dev)),
                 "nm_spgemm_numeric_planned")
         return C_data

@@ -113,13 +113,52 @@ def test_signed_zeros_and_explicit_zeros_keep_the_serial_result(dev):
     assert_same(host(got), cd, "C_data")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_rows_of_the_left_operand_and_wide_rows_of_the_product(dev, dtype):
+    """Classes 2 and 3 of the plan: rows of A of any length (products that take the hash path), rows
+    of C of up to 254 entries; B's named rows stay within eight entries."""
+    cases = [
+        ("(A A) A on a 3D grid: 25-entry rows of A, 62-entry rows of C", 2, None),
+        ("ragged rows of up to 30 entries times rows of up to 8: wide rows of C", 3,
+         (G.ragged_csr(700, 500, 30, 61, dtype), G.ragged_csr(500, 90000, 8, 62, dtype, min_len=4))),
+        ("ragged rows of up to 30 entries times rows of up to 2", 2,
+         (G.ragged_csr(900, 800, 30, 63, dtype, min_len=9), G.ragged_csr(800, 50, 2, 64, dtype))),
+    ]
+    for name, want_class, mats in cases:
+        if mats is None:
+            d, i, p, (n, _) = G.laplace3d(12, dtype, jitter_seed=5)
+            D, I, P = to_dev(dev, d, i, p)
+            Ld, Li, Lp = mirror.spgemm_forward(n, n, D, I, P, n, n, D, I, P)
+            A = (host(Ld), host(Li), host(Lp), (n, n))
+            B = (d, i, p, (n, n))
+        else:
+            A, B = mats
+        ad, ai, ap, (m, kdim) = A
+        bd, bi, bp, (_, ncols) = B
+        AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+        C_data, C_indices, C_indptr = mirror.spgemm_forward(m, kdim, AD, AI, AP, kdim, ncols, BD, BI, BP)
+        plan = mirror.ProductPlan(m, kdim, AI, AP, BI, BP, C_indices, C_indptr)
+        assert plan.usable and plan.plan_class == want_class, (name, plan.plan_class)
+        ad2, bd2 = randn(71, ad.shape[0], dtype), randn(72, bd.shape[0], dtype)
+        AD2, BD2 = to_dev(dev, ad2, bd2)
+        cd, ci, cp = oracle.spgemm_forward(m, kdim, ad2, ai, ap, kdim, ncols, bd2, bi, bp)
+        assert_same(host(C_indices), ci, f"{name}: pattern")
+        assert_same(host(plan.numeric(AD2, BD2)), cd, f"{name}: C_data")
+        g = randn(73, cd.shape[0], dtype)
+        gA, gB = plan.backward(to_dev(dev, g)[0], AD2, BD2)
+        rA, rB = oracle.spgemm_backward(g, ci, cp, m, kdim, ad2, ai, ap, kdim, ncols, bd2, bi, bp)
+        assert_same(host(gA), rA, f"{name}: grad_A")
+        assert_same(host(gB), rB, f"{name}: grad_B")
+
+
 def test_rows_beyond_the_limits_are_refused(dev):
     dtype = np.float64
-    # a row of A with nine entries
-    ad, ai, ap, ashape = _unpack(_short_rows(50, 60, 9, 21, dtype, min_len=9))
-    bd, bi, bp, bshape = _unpack(_short_rows(60, 80, 4, 22, dtype))
+    # a row of C with more than 254 entries
+    ad, ai, ap, ashape = _unpack(_short_rows(50, 60, 40, 21, dtype, min_len=40))
+    bd, bi, bp, bshape = _unpack(_short_rows(60, 80000, 8, 22, dtype, min_len=8))
     AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
-    _, C_indices, C_indptr = mirror.spgemm_forward(50, 60, AD, AI, AP, 60, 80, BD, BI, BP)
+    _, C_indices, C_indptr = mirror.spgemm_forward(50, 60, AD, AI, AP, 60, 80000, BD, BI, BP)
+    assert int((C_indptr[1:] - C_indptr[:-1]).max()) > 254
     assert not mirror.ProductPlan(50, 60, AI, AP, BI, BP, C_indices, C_indptr).usable
     # a named row of B with nine entries
     ad, ai, ap, ashape = _unpack(_short_rows(50, 60, 4, 23, dtype, min_len=1))
