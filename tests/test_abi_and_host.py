@@ -50,6 +50,19 @@ def test_argument_checks_report_through_nm_last_error():
     assert L.nm_spgemm_workspace_bytes(1000, 1000, ctypes.byref(nbytes)) == 0 and nbytes.value > 0
     with pytest.raises(_lib.NummlHipError, match="status 1"):
         _lib.check(L.nm_spgemv_forward(7, 1, 1, 1, None, None, None, None, None, None), "nm_spgemv_forward")
+    # product plans: a class nm_spgemm_plan_build never reports, a plan memory that is too small, and
+    # sizes beyond what a plan's 32-bit positions hold -- all refused on the host, nothing launched
+    assert L.nm_spgemm_numeric_planned(1, 0, 4, 4, 4, 4, None, None, None, None, None, None, None) == 1
+    assert b"plan class" in L.nm_last_error()
+    pbytes = ctypes.c_size_t(0)
+    assert L.nm_spgemm_plan_bytes(1000, ctypes.byref(pbytes)) == 0 and pbytes.value >= 28 * 1000
+    usable = ctypes.c_int(7)
+    assert L.nm_spgemm_plan_adopt(4, 4, 1000, 10, 10, 0, ctypes.c_void_p(8), ctypes.c_void_p(8), 16, None,
+                                  ctypes.byref(usable), None) == 3                  # NM_ERR_WORKSPACE
+    assert L.nm_spgemm_plan_adopt(4, 4, 2 ** 31, 10, 10, 0, ctypes.c_void_p(8), ctypes.c_void_p(8), 2 ** 40, None,
+                                  ctypes.byref(usable), None) == 0 and usable.value == 0
+    assert L.nm_spgemm_plan_adopt(4, 4, 1000, 10, 10, 5, ctypes.c_void_p(8), ctypes.c_void_p(8), 2 ** 40, None,
+                                  ctypes.byref(usable), None) == 0 and usable.value == 0    # rows on the hash path
 
 
 def test_mirror_has_the_reference_signatures():
