@@ -348,6 +348,10 @@ int nm_sptrsv_analyse(int64_t rows, int64_t nnz,
 /* Number of dependency levels / of kernel launches one solve issues. */
 int64_t nm_sptrsv_plan_levels(const nm_sptrsv_plan *plan);
 int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan);
+/* Levels of the solve with A (transposed = 0) or with A^T (1) that sit in runs of one-row levels
+ * which a single wavefront walks with the newest solution in a register (banded factors,
+ * bidiagonal and tridiagonal triangles); diagnostics. */
+int64_t nm_sptrsv_plan_chain_levels(const nm_sptrsv_plan *plan, int transposed);
 
 void nm_sptrsv_plan_destroy(nm_sptrsv_plan *plan);
 

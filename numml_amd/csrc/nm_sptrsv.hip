@@ -58,6 +58,13 @@ struct Packed {        // one solve direction, level-major (all int32, device)
 // the level's width, so the slots behind a level's end must be readable.
 constexpr int64_t kEllPad = 1024;   // == kNarrow, the widest single-workgroup launch
 inline int64_t ell_capacity(int64_t rows, int64_t nnz) { return 2 * nnz + 2 * rows + 8 + 8 * kEllPad; }
+// Doubles of the per-call coefficient area: the fixed-width layout, or the coefficient rows of
+// the chain kernels (64 per chain row, whatever the band's width: room for chains of up to
+// 65536 rows in all; longer ones take what fits).
+inline int64_t coef_capacity(int64_t rows, int64_t nnz) {
+    const int64_t chains = 66 * (rows < 65536 ? rows : 65536) + 8 * kEllPad;
+    return ell_capacity(rows, nnz) > chains ? ell_capacity(rows, nnz) : chains;
+}
 }  // namespace
 
 struct nm_sptrsv_plan {
@@ -77,6 +84,12 @@ struct nm_sptrsv_plan {
         int32_t block;   // lanes of the single-workgroup launch (narrow runs)
         int32_t width = 0;          // rows of its widest level
         int32_t group[2] = {0, 0};  // per direction: lanes that share a row (0: one lane per row)
+        // per direction: 0, or how a run of one-row levels is solved by a single wavefront that
+        // keeps the newest solution in a register (1: every row waits for the row before it only;
+        // 64: rows wait for up to the 64 rows before them), and where its coefficients go
+        int32_t chain[2] = {0, 0};
+        int64_t chain_at[2] = {0, 0};
+        bool chain_candidate = false;
     };
     std::vector<Launch> launches;
 };
@@ -295,7 +308,7 @@ inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork
     w.dg = take(rows + 1);
     w.rhs = take(rows + 1);
     w.coef = take(nnz + 1);
-    w.ell_coef = take(ell_capacity(rows, nnz));
+    w.ell_coef = take(coef_capacity(rows, nnz));
     w.rb = take(2 * (rows + kEllPad) + 2);
     w.status = (int32_t *)take(2);
     if (W) *W = w;
@@ -998,6 +1011,240 @@ __global__ __launch_bounds__(kBlock) void sptrsv_level_group_kernel(SolveArgs a,
     }
 }
 
+// ---- chains: runs of levels of one row each -----------------------------------
+//
+// A banded factor, a bidiagonal or a tridiagonal triangle is one long chain: every level has
+// one row, and that row waits for the row of the level before it.  The workgroup kernels
+// above pay a barrier, an LDS round trip and a division of ~30 dependent instructions per
+// level for it.  Here ONE wavefront walks the chain and hands the newest solution from step
+// to step in a scalar register pair:
+//   * lane l owns the rows at chain positions t = l (mod 64); 64 rows are in flight, and at
+//     step k every lane adds (its coefficient on row k-1) x (solution k-1) to the sum of the row
+//     it owns -- the solutions arrive in the order in which the serial loop visits them
+//     (cpp/sparse_csr_cpu.cpp:672-718 walks a row from its farthest dependency to its nearest),
+//     so each row's sum is formed in exactly that order;
+//   * what a row needs from outside its launch (rows solved by earlier launches) comes first in
+//     that order and is summed ahead of time, for all rows at once, by chain_prepare_kernel;
+//   * the division is three operations with a reciprocal that chain_prepare_kernel formed with
+//     a true division: q0 = n y, r = n - d q0 (exact), q = q0 + r y.  After every 64 steps each
+//     lane checks its own row's quotient against a true division, bit for bit; a block that
+//     fails (a zero, infinite or NaN operand, a range the shortcut does not cover) is solved
+//     again, and the rest of the launch with it, by the plain loop with true divisions.
+// The 64 steps of a block are unrolled; a block's coefficient rows are registers that are
+// refilled in place, right after use, with the rows of the block after it.
+constexpr int kChainMin = 64;                       // levels; shorter runs stay with the workgroup kernels
+constexpr int32_t kChainBad = 1, kChainWide = 2;    // verdict bits of chain_check_kernel
+// doubles a chain launch of m rows takes in the coefficient area: wide chains one row of 64 per
+// position (+ one row before the first, + 64 rows that the last block requests ahead), and a
+// word of presence bits per position; narrow chains one coefficient per position
+inline int64_t chain_doubles(int64_t m, int kind) {
+    const int64_t m64 = (m + 63) / 64 * 64;
+    return kind == 64 ? (m64 + 64) * 64 + m64 + 64 : m64 + 64;
+}
+
+struct ChainArgs {
+    const int32_t *dptr, *dslot;   // this direction's packed dependencies, in accumulation order
+    const double *coef, *dg, *rhs; // level-major values of this call (gather_values_kernel)
+    double *xs;                    // running solution by slot
+    double *sum0, *recip;          // by slot: sum over the dependencies outside the launch; 1 / diagonal
+    double *band;                  // wide chains: [position + 1][64] coefficients on the row before that
+                                   // position, lane = owner; narrow chains: [position] the one coefficient
+    unsigned long long *has;       // wide chains: [position + 1] which lanes have a coefficient there
+    int32_t q0, q1, m, step;       // slots [q0, q1), m = q1 - q0 rows, walked upwards (+1) or downwards (-1)
+    int unit;
+};
+
+__device__ __forceinline__ int32_t chain_slot(const ChainArgs &c, int32_t t) {
+    return c.step > 0 ? c.q0 + t : c.q1 - 1 - t;
+}
+__device__ __forceinline__ int32_t chain_pos(const ChainArgs &c, int32_t q) {
+    return c.step > 0 ? q - c.q0 : c.q1 - 1 - q;
+}
+
+// Plan time: may the chain kernels take this run of one-row levels in this direction?  In a
+// row's accumulation order the dependencies outside the launch must all come before those
+// inside it, the ones inside must be at most 64 positions back and in ascending position.
+__global__ void chain_check_kernel(int32_t nlevels, int dirn, const int32_t *__restrict__ level_ptr,
+                                   const int32_t *__restrict__ cand_of_level, const int32_t *__restrict__ cq,
+                                   const int32_t *__restrict__ dptr, const int32_t *__restrict__ dslot,
+                                   int32_t *__restrict__ verdict) {
+    const int32_t stride = (int32_t)(gridDim.x * blockDim.x);
+    for (int32_t l = (int32_t)(blockIdx.x * blockDim.x + threadIdx.x); l < nlevels; l += stride) {
+        const int32_t ci = cand_of_level[l];
+        if (ci < 0) continue;
+        const int32_t q = level_ptr[l], q0 = cq[2 * ci], q1 = cq[2 * ci + 1];
+        const int32_t t = dirn == 0 ? q - q0 : q1 - 1 - q;
+        int32_t bits = 0, inside = 0, last = -1;
+        for (int32_t at = dptr[q]; at < dptr[q + 1]; ++at) {
+            const int32_t ds = dslot[at];
+            if (ds >= q0 && ds < q1) {
+                const int32_t k = dirn == 0 ? ds - q0 : q1 - 1 - ds;
+                if (t - k < 1 || t - k > 64 || k <= last) bits |= kChainBad;
+                if (t - k != 1) bits |= kChainWide;
+                last = k;
+                ++inside;
+            } else if (inside > 0) {
+                bits |= kChainBad;
+            }
+        }
+        if (inside > 1) bits |= kChainWide;
+        if (t > 0 && inside == 0) bits |= kChainBad;
+        if (bits) atomicOr(verdict + 2 * ci + dirn, bits);
+    }
+}
+
+// Per call and launch, one lane per row of the chain: the part of the row's sum that does not
+// wait for the chain, the reciprocal of its diagonal, and its coefficients on the chain in
+// the layout the chain kernel streams (the wide layout is cleared before this runs).
+template <bool BAND>
+__global__ void chain_prepare_kernel(ChainArgs c) {
+    const int32_t t = (int32_t)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (t >= c.m) return;
+    const int32_t q = chain_slot(c, t);
+    double acc = 0., only = 0.;
+    for (int32_t at = c.dptr[q]; at < c.dptr[q + 1]; ++at) {
+        const int32_t ds = c.dslot[at];
+        const double v = c.coef[at];
+        if (ds < c.q0 || ds >= c.q1) {
+            acc += v * c.xs[ds];
+        } else if (BAND) {
+            const int32_t k = chain_pos(c, ds);
+            c.band[(size_t)(k + 1) * 64 + (t & 63)] = v;
+            atomicOr(c.has + k + 1, 1ull << (t & 63));
+        } else {
+            only = v;
+        }
+    }
+    c.sum0[q] = acc;
+    c.recip[q] = c.unit ? 1. : 1. / c.dg[q];
+    if (!BAND) c.band[t] = only;
+}
+
+__device__ __forceinline__ double lane_value(double v, int lane) {   // `lane` is uniform
+    const int lo = __builtin_amdgcn_readlane(__double2loint(v), lane);
+    const int hi = __builtin_amdgcn_readlane(__double2hiint(v), lane);
+    return __hiloint2double(hi, lo);
+}
+
+__device__ __forceinline__ bool same_bits(double a, double b) {
+    return __double_as_longlong(a) == __double_as_longlong(b);
+}
+
+template <bool BAND, bool UNIT>
+__global__ __launch_bounds__(64) void sptrsv_chain_kernel(ChainArgs c) {
+    const int lane = (int)threadIdx.x;
+    const int32_t m = c.m;
+    const double *__restrict__ band = c.band;
+    // what the lanes computed at the 64 steps of a block: the quotient, and for wide chains with a
+    // division the numerator beside it
+    constexpr bool kPair = BAND && !UNIT;
+    __shared__ double s_keep[(kPair ? 2 : 1) * 64 * 64];
+    double X = 0.;            // the newest solution (uniform)
+    double row[BAND ? 64 : 1];
+    double acc = 0.;          // wide chains: the sum of the row this lane owns
+    int32_t k0 = 0;
+    // operands of the block's rows (lane l: position k0 + l), requested one block ahead
+    auto at_slot = [&](int32_t t) { return chain_slot(c, t < m ? t : m - 1); };
+    double bv = c.rhs[at_slot(lane)], dv = c.dg[at_slot(lane)], yv = c.recip[at_slot(lane)];
+    double s0 = c.sum0[at_slot(lane)], cv = 0.;
+    if (BAND) {
+#pragma unroll
+        for (int s = 0; s < 64; ++s) row[s] = band[(size_t)s * 64 + lane];
+        acc = s0;
+    } else {
+        cv = band[lane];
+    }
+    bool fast = true;
+    for (; k0 < m; k0 += 64) {
+        const int32_t t = k0 + lane;
+        const int32_t qn = at_slot(t + 64);
+        const double bvN = c.rhs[qn], dvN = c.dg[qn], yvN = c.recip[qn], s0N = c.sum0[qn];
+        const double cvN = BAND ? 0. : band[t + 64];   // padded: 64 entries behind the last row
+        const double Xin = X, acc_in = acc;
+        // "is this step's row mine" is compared afresh at every step: 64 masks kept from block to
+        // block would not fit the scalar registers
+        int32_t t_mark = t;
+        asm volatile("" : "+v"(t_mark));
+        const double *__restrict__ ahead = band + (size_t)(k0 + 64) * 64;   // padded: 64 rows behind the last
+#pragma unroll
+        for (int s = 0; s < 64; ++s) {
+            if (BAND) {
+                acc = acc + row[s] * X;
+                row[s] = ahead[s * 64 + lane];
+            } else {
+                acc = s0 + cv * X;
+            }
+            const double n = bv - acc;
+            double q = n;
+            if (!UNIT) {
+                const double q0 = n * yv;
+                const double r = __builtin_fma(-dv, q0, n);
+                q = __builtin_fma(r, yv, q0);
+            }
+            // every lane files what it computed; only lane s's entry of step s means anything
+            if (kPair) reinterpret_cast<double2 *>(s_keep)[s * 64 + lane] = make_double2(n, q);
+            else s_keep[s * 64 + lane] = q;
+            if (BAND) acc = (t_mark == k0 + s) ? s0N : acc;
+            X = lane_value(q, s);
+        }
+        double n_keep = 0., q_keep;
+        if (kPair) {
+            const double2 nq = reinterpret_cast<const double2 *>(s_keep)[lane * 64 + lane];
+            n_keep = nq.x;
+            q_keep = nq.y;
+        } else {
+            q_keep = s_keep[lane * 64 + lane];
+        }
+        // every lane checks the row it finished in this block
+        bool ok = true;
+        if (t < m) {
+            if (BAND) {
+                // a skipped coefficient was multiplied as 0.0: exact only for finite solutions
+                ok = (UNIT || same_bits(n_keep / dv, q_keep)) && __builtin_isfinite(q_keep);
+            } else {
+                double before = __shfl_up(q_keep, 1);
+                if (lane == 0) before = Xin;
+                const double n = bv - (s0 + cv * before);
+                ok = same_bits(UNIT ? n : n / dv, q_keep);
+            }
+        }
+        if (!__all(ok) || !__builtin_isfinite(Xin)) {
+            X = Xin;
+            acc = acc_in;
+            fast = false;
+            break;
+        }
+        if (t < m) c.xs[chain_slot(c, t)] = q_keep;
+        bv = bvN; dv = dvN; yv = yvN; s0 = s0N; cv = cvN;
+    }
+    if (fast) return;
+    // the plain loop: true divisions, coefficients that are absent are skipped
+    for (; k0 < m; k0 += 64) {
+        const int32_t t = k0 + lane;
+        const int32_t qs = at_slot(t), qn = at_slot(t + 64);
+        bv = c.rhs[qs]; dv = c.dg[qs]; s0 = c.sum0[qs];
+        const double s0N = c.sum0[qn];
+        if (!BAND) cv = band[t];
+        double q_keep = 0.;
+        for (int s = 0; s < 64; ++s) {
+            if (BAND) {
+                const double v = band[(size_t)(k0 + s) * 64 + lane];
+                if ((c.has[k0 + s] >> lane) & 1ull) acc = acc + v * X;
+            } else {
+                acc = s0 + cv * X;   // position 0 has no coefficient (0.0) and meets X = 0.0
+            }
+            const double n = bv - acc;
+            const double q = UNIT ? n : n / dv;
+            if (lane == s) {
+                q_keep = q;
+                if (BAND) acc = s0N;
+            }
+            X = lane_value(q, s);
+        }
+        if (t < m) c.xs[chain_slot(c, t)] = q_keep;
+    }
+}
+
 // x[order[q]] = xs[q], rounded once to the value type (cpp/sparse_csr_cpu.cpp:722).
 // `status` (may be null): nonzero when a kernel of this solve gave up waiting; x is then NaN throughout.
 template <typename T>
@@ -1046,7 +1293,41 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     const int n = (int)p->launches.size();
     for (int li = 0; li < n; ++li) {
         const auto &L = p->launches[transposed ? n - 1 - li : li];
-        if (L.wide) {
+        if (L.chain[dirn] != 0) {
+            // one wavefront walks the run of one-row levels; `ell_coef` and `rb` are free for it
+            // (a direction that has chains does not use the fixed-width layout)
+            ChainArgs c;
+            c.dptr = P.dptr;
+            c.dslot = P.dslot;
+            c.coef = a.w.coef;
+            c.dg = a.w.dg;
+            c.rhs = a.w.rhs;
+            c.xs = a.w.xs;
+            c.sum0 = a.w.rb;
+            c.recip = a.w.rb + (p->rows + kEllPad);
+            c.band = a.w.ell_coef + L.chain_at[dirn];
+            c.q0 = L.q0;
+            c.q1 = L.q1;
+            c.m = L.q1 - L.q0;
+            c.step = transposed ? -1 : 1;
+            c.unit = unit;
+            const int64_t m64 = (int64_t)nm::ceil_div((int64_t)c.m, 64) * 64;
+            const bool wide_chain = L.chain[dirn] == 64;
+            c.has = reinterpret_cast<unsigned long long *>(c.band + (m64 + 64) * 64);
+            const unsigned pgrid = (unsigned)nm::ceil_div((int64_t)c.m, kBlock);
+            if (wide_chain) {
+                if (int rc = nm::fill_async(c.band, chain_doubles(c.m, 64), 0., s)) return rc;
+                hipLaunchKernelGGL(chain_prepare_kernel<true>, dim3(pgrid), dim3(kBlock), 0, s, c);
+                if (unit) hipLaunchKernelGGL((sptrsv_chain_kernel<true, true>), dim3(1), dim3(64), 0, s, c);
+                else hipLaunchKernelGGL((sptrsv_chain_kernel<true, false>), dim3(1), dim3(64), 0, s, c);
+            } else {
+                if (int rc = nm::fill_async(c.band + c.m, m64 + 64 - c.m, 0., s)) return rc;
+                hipLaunchKernelGGL(chain_prepare_kernel<false>, dim3(pgrid), dim3(kBlock), 0, s, c);
+                if (unit) hipLaunchKernelGGL((sptrsv_chain_kernel<false, true>), dim3(1), dim3(64), 0, s, c);
+                else hipLaunchKernelGGL((sptrsv_chain_kernel<false, false>), dim3(1), dim3(64), 0, s, c);
+            }
+            NM_LAUNCH_CHECK("sptrsv_chain_kernel");
+        } else if (L.wide) {
             const int G = L.group[dirn] > 0 ? L.group[dirn] : 1;
             const unsigned grid = (unsigned)nm::ceil_div((int64_t)(L.q1 - L.q0) * G, kBlock);
             if (G == 16)
@@ -1243,7 +1524,7 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         return b;
     };
     constexpr int32_t kMinSegment = 32;   // levels; shorter segments are not worth a launch
-    auto push_narrow = [&](int32_t a0, int32_t a1) {
+    auto push_plain = [&](int32_t a0, int32_t a1) {
         int32_t s0 = a0, block = lanes_for(a0);
         auto flush = [&](int32_t end) {
             for (int32_t c0 = s0; c0 < end; c0 += kMaxLevels) {
@@ -1272,6 +1553,28 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             }
         }
         flush(a1);
+    };
+    // Runs of at least kChainMin one-row levels inside a narrow run become launches of their own
+    // (candidates for the single-wavefront chain kernels; a direction that cannot use those runs
+    // them like any other narrow launch).
+    auto push_narrow = [&](int32_t a0, int32_t a1) {
+        int32_t plain0 = a0;
+        for (int32_t l = a0; l < a1;) {
+            if (lp[l + 1] - lp[l] != 1) { ++l; continue; }
+            int32_t e = l;
+            while (e < a1 && lp[e + 1] - lp[e] == 1) ++e;
+            if (e - l >= kChainMin) {
+                if (l > plain0) push_plain(plain0, l);
+                for (int32_t c0 = l; c0 < e; c0 += kMaxLevels) {
+                    const int32_t c1 = c0 + kMaxLevels < e ? c0 + kMaxLevels : e;
+                    p->launches.push_back({c0, c1, lp[c0], lp[c1], false, 64});
+                    p->launches.back().chain_candidate = true;
+                }
+                plain0 = e;
+            }
+            l = e;
+        }
+        if (a1 > plain0) push_plain(plain0, a1);
     };
     // dependency ranges of both directions: a level is also given a launch of its own when it
     // has enough entries to be worth the chip (one CU takes ~10 us over a level of a few
@@ -1326,9 +1629,71 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     if (hipMemcpyAsync(L.level_launch, level_launch.data(), level_launch.size() * 4, hipMemcpyHostToDevice, s) !=
         hipSuccess)
         return bail(nm::fail(NM_ERR_HIP, "uploading the launch table failed"));
+    // Which runs of one-row levels the chain kernels take, per direction (W.count64 and W.deg
+    // are free by now: candidate of every level, the candidates' slot ranges, the verdicts).
+    bool chains[2] = {false, false};
+    {
+        std::vector<int32_t> cand((size_t)p->nlevels + 1, -1), cq;
+        std::vector<size_t> cand_launch;
+        for (size_t li = 0; li < p->launches.size(); ++li) {
+            const auto &C = p->launches[li];
+            if (!C.chain_candidate) continue;
+            for (int32_t l = C.l0; l < C.l1; ++l) cand[l] = (int32_t)cand_launch.size();
+            cq.push_back(C.q0);
+            cq.push_back(C.q1);
+            cand_launch.push_back(li);
+        }
+        if (!cand_launch.empty()) {
+            int32_t *d_cand = reinterpret_cast<int32_t *>(W.count64), *d_cq = d_cand + (rows + 1);
+            std::vector<int32_t> verdict(cq.size(), 0);
+            if (hipMemcpyAsync(d_cand, cand.data(), cand.size() * 4, hipMemcpyHostToDevice, s) != hipSuccess ||
+                hipMemcpyAsync(d_cq, cq.data(), cq.size() * 4, hipMemcpyHostToDevice, s) != hipSuccess)
+                return bail(nm::fail(NM_ERR_HIP, "uploading the chain candidates failed"));
+            if (int rc = nm::fill_async(W.deg, (int64_t)cq.size(), (int32_t)0, s)) return bail(rc);
+            int64_t lgrid = nm::ceil_div((int64_t)p->nlevels, kBlock);
+            if (lgrid > 65536) lgrid = 65536;
+            for (int d = 0; d < 2; ++d) {
+                hipLaunchKernelGGL(chain_check_kernel, dim3((unsigned)lgrid), dim3(kBlock), 0, s, p->nlevels, d,
+                                   p->level_ptr, d_cand, d_cq, p->dir[d].dptr, p->dir[d].dslot, W.deg);
+                if (hipGetLastError() != hipSuccess)
+                    return bail(nm::fail(NM_ERR_HIP, "chain_check_kernel launch failed"));
+            }
+            if (hipMemcpyAsync(verdict.data(), W.deg, verdict.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
+                hipStreamSynchronize(s) != hipSuccess)
+                return bail(nm::fail(NM_ERR_HIP, "reading the chain verdicts back failed"));
+            for (int d = 0; d < 2; ++d) {
+                // the coefficient area is shared with the fixed-width layout: a direction takes its
+                // chains when they hold at least half of its levels, or when it has no such layout
+                const int32_t md = p->max_deps[d];
+                const bool ell_possible = md <= 8 && rows < (1 << 30);
+                int64_t at = 0, levels = 0;
+                std::vector<std::pair<size_t, int>> taken;
+                for (size_t ci = 0; ci < cand_launch.size(); ++ci) {
+                    const int32_t v = verdict[2 * ci + d];
+                    if (v & kChainBad) continue;
+                    const auto &C = p->launches[cand_launch[ci]];
+                    const int kind = (v & kChainWide) ? 64 : 1;
+                    const int64_t need = chain_doubles(C.q1 - C.q0, kind);
+                    if (at + need > coef_capacity(rows, nnz)) continue;
+                    taken.push_back({cand_launch[ci], kind});
+                    at += need;
+                    levels += C.l1 - C.l0;
+                }
+                if (taken.empty() || (ell_possible && 2 * levels < p->nlevels)) continue;
+                chains[d] = true;
+                at = 0;
+                for (const auto &tk : taken) {
+                    auto &C = p->launches[tk.first];
+                    C.chain[d] = tk.second;
+                    C.chain_at[d] = at;
+                    at += chain_doubles(C.q1 - C.q0, tk.second);
+                }
+            }
+        }
+    }
     for (int d = 0; d < 2; ++d) {
         const int32_t md = p->max_deps[d];
-        const int pre = md <= 2 ? 2 : (md <= 4 ? 4 : (md <= 8 ? 8 : 0));
+        const int pre = chains[d] ? 0 : (md <= 2 ? 2 : (md <= 4 ? 4 : (md <= 8 ? 8 : 0)));
         if (pre > 0 && rows < (1 << 30) && (rows + kEllPad) * pre <= ell_capacity(rows, nnz)) {
             p->ell_pre[d] = pre;
             int64_t grid = nm::ceil_div(rows * pre, kBlock);
@@ -1354,6 +1719,14 @@ extern "C" int64_t nm_sptrsv_plan_levels(const nm_sptrsv_plan *plan) { return pl
 
 extern "C" int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan) {
     return plan ? (int64_t)plan->launches.size() : -1;
+}
+
+extern "C" int64_t nm_sptrsv_plan_chain_levels(const nm_sptrsv_plan *plan, int transposed) {
+    if (!plan) return -1;
+    int64_t n = 0;
+    for (const auto &L : plan->launches)
+        if (L.chain[transposed ? 1 : 0] != 0) n += L.l1 - L.l0;
+    return n;
 }
 
 extern "C" void nm_sptrsv_plan_destroy(nm_sptrsv_plan *plan) { delete plan; }

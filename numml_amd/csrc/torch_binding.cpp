@@ -1229,6 +1229,17 @@ std::tuple<int64_t, int64_t> sptrsv_schedule(int A_rows, Tensor A_indices, Tenso
     return {nm_sptrsv_plan_levels(plan->handle), nm_sptrsv_plan_launches(plan->handle)};
 }
 
+std::tuple<int64_t, int64_t> sptrsv_chain_levels(int A_rows, Tensor A_indices, Tensor A_indptr, bool lower) {
+    TORCH_CHECK(A_indptr.dim() == 1 && A_indptr.numel() == (int64_t)A_rows + 1 && A_indices.dim() == 1,
+                "sptrsv_chain_levels: expected ", A_rows + 1, " row pointers, got shape ", A_indptr.sizes());
+    const auto dev = need_device({&A_indices, &A_indptr});
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    auto plan = level_plan(A_indices, A_indptr, A_rows, lower, dev);
+    return {nm_sptrsv_plan_chain_levels(plan->handle, 0), nm_sptrsv_plan_chain_levels(plan->handle, 1)};
+}
+
 void clear_plan_cache() {
     std::lock_guard<std::mutex> lock(g_plans_mutex);
     g_plans.clear();
@@ -1297,6 +1308,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("csr_extract_diagonal_forward", &csr_extract_diagonal_forward, "CSR extract diagonal forward");
     m.def("csr_extract_diagonal_backward", &csr_extract_diagonal_backward, "CSR extract diagonal backward");
     m.def("sptrsv_schedule", &sptrsv_schedule, "(levels, launches per solve) of a triangular pattern");
+    m.def("sptrsv_chain_levels", &sptrsv_chain_levels,
+          "levels of the solves with A and with A^T that the single-wavefront chain kernels take");
     m.def("clear_plan_cache", &clear_plan_cache, "Drop every cached structure plan");
     m.def("plan_cache_size", &plan_cache_size, "Number of cached structure plans");
     m.def("plan_cache_bytes", &plan_cache_bytes, "Device memory held by the cached structure plans");

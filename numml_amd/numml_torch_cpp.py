@@ -25,7 +25,7 @@ __all__ = [
     "csr_transpose_forward", "csr_transpose_backward", "splincomb_forward", "splincomb_backward",
     "csr_to_dense_forward", "csr_to_dense_backward", "csr_row_sum_forward", "csr_row_sum_backward",
     "csr_extract_diagonal_forward", "csr_extract_diagonal_backward",
-    "clear_plan_cache", "plan_cache_size", "sptrsv_schedule",
+    "clear_plan_cache", "plan_cache_size", "sptrsv_schedule", "sptrsv_chain_levels",
 ]
 
 
@@ -685,6 +685,8 @@ class _Plan:
         self.handle = handle
         self.levels = int(L.nm_sptrsv_plan_levels(handle))
         self.launches = int(L.nm_sptrsv_plan_launches(handle))
+        self.chain_levels = (int(L.nm_sptrsv_plan_chain_levels(handle, 0)),
+                             int(L.nm_sptrsv_plan_chain_levels(handle, 1)))
         # nm_sptrsv_analyse synchronised its stream, so the plan is complete for every stream
 
     def __del__(self):
@@ -810,6 +812,18 @@ def sptrsv_schedule(A_rows, A_indices, A_indptr, lower):
     with torch.cuda.device(dev):
         plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
     return plan.levels, plan.launches
+
+
+def sptrsv_chain_levels(A_rows, A_indices, A_indptr, lower):
+    """Levels of the solve with A and of the solve with A^T that the single-wavefront chain
+    kernels take (runs of one-row levels); diagnostics, no counterpart in the reference."""
+    if A_indptr.dim() != 1 or A_indptr.shape[0] != A_rows + 1 or A_indices.dim() != 1:
+        raise RuntimeError(f"sptrsv_chain_levels: expected {A_rows + 1} row pointers, got shape {list(A_indptr.shape)}")
+    dev = _need_device(A_indices, A_indptr)
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
+    return plan.chain_levels
 
 
 def plan_cache_size():
