@@ -500,7 +500,7 @@ class SpTRSV(Workload):
         s = 8
         self.bytes_per_step = 2 * (self.nnz * (s + 8) + (rows + 1) * 8 + 2 * rows * s) + self.nnz * s
         self.dominant_bytes = self.nnz * (s + 8) + (rows + 1) * 8 + 2 * rows * s
-        self.dominant_name = "forward solve: gather_values_kernel + sptrsv_ring_kernel + unslot_kernel"
+        self.dominant_name = "forward solve: gather_ell_kernel + sptrsv_ell_kernel + unslot_kernel"
         self.config = {"workload": "sptrsv_fwd_bwd_f64_tril_poisson2d_1024", "rows": rows, "nnz": self.nnz,
                        "levels": 2 * n - 1, "analysis_plus_first_solve_ms": round(self.analysis_ms, 3)}
 
