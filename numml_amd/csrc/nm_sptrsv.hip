@@ -1565,8 +1565,12 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             while (e < a1 && lp[e + 1] - lp[e] == 1) ++e;
             if (e - l >= kChainMin) {
                 if (l > plain0) push_plain(plain0, l);
-                for (int32_t c0 = l; c0 < e; c0 += kMaxLevels) {
-                    const int32_t c1 = c0 + kMaxLevels < e ? c0 + kMaxLevels : e;
+                // at most kMaxLevels levels each (a direction that cannot use the chain kernels runs
+                // them like any other narrow launch), in pieces of equal length
+                const int32_t pieces = (e - l + kMaxLevels - 1) / kMaxLevels;
+                const int32_t each = (e - l + pieces - 1) / pieces;
+                for (int32_t c0 = l; c0 < e; c0 += each) {
+                    const int32_t c1 = c0 + each < e ? c0 + each : e;
                     p->launches.push_back({c0, c1, lp[c0], lp[c1], false, 64});
                     p->launches.back().chain_candidate = true;
                 }
