@@ -276,7 +276,7 @@ class SpMM(Workload):
                           + cols * n * s)
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
-        self.dominant_name = ("spdmm_bwd_kernel (grad_A) + spdmm_fwd_flat_kernel on the transposed plan (grad_B)"
+        self.dominant_name = ("spdmm_bwd_fused_kernel: both gradients from one walk over A by column (transposed plan)"
                               if _binding.backward_mode() != "atomic"
                               else "spdmm_bwd_kernel (+ fill_kernel clearing grad_B)")
         # the plan of the default backward is built during one of these
@@ -287,9 +287,11 @@ class SpMM(Workload):
                        "dense_cols": n, "index_bytes": 8,
                        "algorithmic_bytes_per_step": self.bytes_per_step,
                        "gather_bytes_fwd": nnz * n * s}
-        # every entry of A fetches one row of the dense operand in each of the three products
-        # (forward: B; dot products of the backward: B; transposed product: the gradient of C)
-        self.gather_inclusive_bytes = self.bytes_per_step + 3 * nnz * n * s - 3 * cols * n * s
+        # every entry of A fetches one row of a dense operand in each walk over A: the forward (B) and
+        # the backward on the plan (the gradient of C, which serves both gradients); the stateless
+        # backward makes a third (rows of B for the dot products)
+        walks = 3 if _binding.backward_mode() == "atomic" else 2
+        self.gather_inclusive_bytes = self.bytes_per_step + walks * nnz * n * s - walks * cols * n * s
 
     def after(self, rec, steps):
         """The same step priced on the bytes that are gathered, not on the operands' sizes: what the

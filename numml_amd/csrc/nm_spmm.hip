@@ -251,6 +251,28 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
     }
 }
 
+// Sums over the wavefront of kBatch (= 8) lane-wise products at once.  Three folding steps
+// halve the number of vectors while pairing lanes 1, 2 and 4 apart, after which lane l holds
+// the partial sum of vector l & 7 over its group of 8 lanes; three more steps add the eight
+// groups.  27 instructions instead of 8 full reductions; the result for vector u is in every
+// lane with (l & 7) == u.
+template <typename T> __device__ __forceinline__ T fold8(const T (&p)[kBatch], int lane) {
+    static_assert(kBatch == 8, "fold8 folds eight vectors");
+    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
+    T q[4], r[2];
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+        q[m] = (b0 ? p[2 * m + 1] : p[2 * m]) + nm::dpp_move<0xB1>(b0 ? p[2 * m] : p[2 * m + 1]);
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+        r[m] = (b1 ? q[2 * m + 1] : q[2 * m]) + nm::dpp_move<0x4E>(b1 ? q[2 * m] : q[2 * m + 1]);
+    T t = (b2 ? r[1] : r[0]) + __shfl_xor(b2 ? r[0] : r[1], 4, kWave);
+    t += nm::dpp_move<0x128>(t);          // row_ror 8: the other group of the 16-lane row
+    t += __shfl_xor(t, 16, kWave);
+    t += __shfl_xor(t, 32, kWave);
+    return t;
+}
+
 // grad_A[k] = <gC[row(k),:], B[col(k),:]> (SDDMM) and, when grad_B is given, the
 // atomic scatter grad_B[col,:] += data[k] * gC[row,:].  Entry-balanced: a
 // wavefront owns 64 consecutive stored entries whatever rows they belong to
@@ -334,27 +356,7 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
                 bv[u] = grad_A ? brow[live ? c : 0] : T(0);
             }
         };
-        // Sums over the wavefront of kBatch (= 8) lane-wise products at once.  Three
-        // folding steps halve the number of vectors while pairing lanes 1, 2 and 4 apart,
-        // after which lane l holds the partial sum of vector l & 7 over its group of 8
-        // lanes; three more steps add the eight groups.  27 instructions instead of
-        // 8 full reductions; the result for vector u is in every lane with (l & 7) == u.
-        auto reduce8 = [&](const T (&p)[kBatch]) {
-            static_assert(kBatch == 8, "reduce8 folds eight vectors");
-            const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
-            T q[4], r[2];
-#pragma unroll
-            for (int m = 0; m < 4; ++m)
-                q[m] = (b0 ? p[2 * m + 1] : p[2 * m]) + nm::dpp_move<0xB1>(b0 ? p[2 * m] : p[2 * m + 1]);
-#pragma unroll
-            for (int m = 0; m < 2; ++m)
-                r[m] = (b1 ? q[2 * m + 1] : q[2 * m]) + nm::dpp_move<0x4E>(b1 ? q[2 * m] : q[2 * m + 1]);
-            T t = (b2 ? r[1] : r[0]) + __shfl_xor(b2 ? r[0] : r[1], 4, kWave);
-            t += nm::dpp_move<0x128>(t);          // row_ror 8: the other group of the 16-lane row
-            t += __shfl_xor(t, 16, kWave);
-            t += __shfl_xor(t, 32, kWave);
-            return t;
-        };
+        auto reduce8 = [&](const T (&p)[kBatch]) { return fold8<T>(p, lane); };
         auto consume = [&](int j0, const int64_t (&col)[kBatch], int64_t c, bool live, const T (&gv)[kBatch],
                            const T (&bv)[kBatch]) {
             if (grad_B) {
@@ -418,6 +420,196 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
         }
         if (grad_A && lane < cnt) grad_A[k] = mydot;
     }
+}
+
+// ---- both gradients in one walk over A by column ---------------------------------
+//
+// grad_B = A^T gC walks A by column on the transposed-structure plan and gathers, per stored
+// entry, the row of gC it names.  The dot product grad_A[k] = <gC[row,:], B[col,:]> needs that
+// same row of gC and the column's own row of B, which a wavefront that owns the column can
+// keep at hand.  So one walk serves both gradients and the second pass of gathers (rows of B
+// per entry, as the row-major kernel above makes them) falls away: half the gathered bytes of
+// the backward.  grad_B is added in the same order as by spdmm_fwd_flat_kernel on the plan
+// and the dot products are folded exactly like spdmm_bwd_kernel's, so both gradients keep
+// their bits.  At most 64 dense columns (one column tile).
+template <typename T>
+__device__ __forceinline__ void fused_long_columns(int64_t cols, const T *__restrict__ data,
+                                                   const int32_t *__restrict__ t_row,
+                                                   const int32_t *__restrict__ t_indptr,
+                                                   const int32_t *__restrict__ t_perm, const T *__restrict__ gC,
+                                                   int64_t ldg, const T *__restrict__ B, int64_t ldb, int64_t n,
+                                                   T *__restrict__ grad_B, int64_t ldgb, T *__restrict__ grad_A,
+                                                   int lane, int wave) {
+    __shared__ T s_part[kWavesPerBlock][kWave];
+    __shared__ int s_long[kScoutRows];
+    __shared__ int s_nlong;
+    const int64_t g0 = (int64_t)blockIdx.x * kScoutRows;
+    if (threadIdx.x == 0) s_nlong = 0;
+    __syncthreads();
+    for (int t = threadIdx.x; t < kScoutRows && g0 + t < cols; t += kBlock)
+        if (t_indptr[g0 + t + 1] - t_indptr[g0 + t] > kSplitRow) s_long[atomicAdd(&s_nlong, 1)] = t;
+    __syncthreads();
+    const int nl = s_nlong;
+    const bool live = lane < n;
+    for (int li = 0; li < nl; ++li) {   // uniform over the workgroup
+        const int64_t col = g0 + s_long[li];
+        const int64_t rb = t_indptr[col], re = t_indptr[col + 1];
+        int64_t chunk = (re - rb + kWavesPerBlock - 1) / kWavesPerBlock;
+        chunk = (chunk + kWave - 1) / kWave * kWave;
+        const int64_t kb0 = rb + wave * chunk;
+        const int64_t ke0 = kb0 + chunk < re ? kb0 + chunk : re;
+        const T bj = live ? B[col * ldb + lane] : T(0);
+        T acc = T(0);
+        for (int64_t kb = kb0; kb < ke0; kb += kWave) {
+            const int64_t k = kb + lane;
+            const int64_t myrow = k < ke0 ? (int64_t)t_row[k] : 0;
+            const int32_t myperm = k < ke0 ? t_perm[k] : 0;
+            const T myval = k < ke0 ? data[myperm] : T(0);
+            const int cnt = (int)(ke0 - kb < kWave ? ke0 - kb : kWave);
+            T mydot = T(0);
+            for (int j = 0; j < cnt; ++j) {
+                const T gv = gC[__shfl(myrow, j, kWave) * ldg + (live ? lane : 0)];
+                acc += __shfl(myval, j, kWave) * gv;
+                const T t = nm::wave_sum(live ? gv * bj : T(0));
+                if (lane == j) mydot = t;
+            }
+            if (lane < cnt) grad_A[myperm] = mydot;
+        }
+        s_part[wave][lane] = acc;
+        __syncthreads();
+        if (wave == 0 && live) {
+            T sum = s_part[0][lane];
+            for (int w = 1; w < kWavesPerBlock; ++w) sum += s_part[w][lane];
+            grad_B[col * ldgb + lane] = sum;
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void spdmm_bwd_fused_kernel(
+    int64_t cols, const T *__restrict__ data, const int32_t *__restrict__ t_row,
+    const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm, const T *__restrict__ gC,
+    int64_t ldg, const T *__restrict__ B, int64_t ldb, int64_t n, T *__restrict__ grad_B, int64_t ldgb,
+    T *__restrict__ grad_A) {
+    __shared__ T s_b[kWavesPerBlock][kFlatRows][kWave];   // rows of B of the columns a wavefront owns
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int64_t long_blocks = (cols + kScoutRows - 1) / kScoutRows;
+    if ((int64_t)blockIdx.x < long_blocks) {
+        fused_long_columns<T>(cols, data, t_row, t_indptr, t_perm, gC, ldg, B, ldb, n, grad_B, ldgb, grad_A, lane,
+                              wave);
+        return;
+    }
+    const int64_t r0 = (((int64_t)blockIdx.x - long_blocks) * kWavesPerBlock + wave) * kFlatRows;
+    if (r0 >= cols) return;
+    const int nr = (int)(cols - r0 < kFlatRows ? cols - r0 : kFlatRows);
+    const bool live = lane < n;
+    for (int r = 0; r < nr; ++r) s_b[wave][r][lane] = live ? B[(r0 + r) * ldb + lane] : T(0);
+    const int64_t my_ptr = (int64_t)t_indptr[r0 + (lane <= nr ? lane : nr)];
+    auto ptr_of = [&](int l) {
+        const long long lo = __builtin_amdgcn_readlane((int)(my_ptr & 0xffffffffll), l);
+        const long long hi = __builtin_amdgcn_readlane((int)(my_ptr >> 32), l);
+        return (int64_t)((hi << 32) | (lo & 0xffffffffll));
+    };
+    const int64_t begin = ptr_of(0), end = ptr_of(nr);
+    const int64_t row_bytes = ldg * (int64_t)sizeof(T);
+    const char *__restrict__ Gc = reinterpret_cast<const char *>(gC + (live ? lane : 0));
+    int r = 0;   // current column (relative), its range, whether it is computed here
+    int64_t row_begin = begin, row_end = ptr_of(1);
+    bool mine = row_end - row_begin <= kSplitRow;
+    T acc = T(0);
+    T cur_b = s_b[wave][0][lane];
+    auto next_row = [&]() {
+        if (mine && live) grad_B[(r0 + r) * ldgb + lane] = acc;
+        acc = T(0);
+        ++r;
+        row_begin = row_end;
+        row_end = ptr_of(r + 1 <= nr ? r + 1 : nr);
+        mine = row_end - row_begin <= kSplitRow;
+        cur_b = s_b[wave][r < nr ? r : nr - 1][lane];
+    };
+    auto close_row = [&]() {
+        next_row();
+        while (r < nr && row_end == row_begin) next_row();
+    };
+    while (r < nr && row_end == row_begin) next_row();   // empty columns at the head
+    int64_t kb = begin;
+    auto fetch = [&](int64_t at, int64_t &row, T &val, int32_t &pos) {
+        const int64_t k = at + lane < end ? at + lane : (end > begin ? end - 1 : 0);
+        row = end > begin ? (int64_t)t_row[k] : 0;
+        pos = end > begin ? t_perm[k] : 0;
+        val = end > begin ? data[pos] : T(0);
+    };
+    int64_t myrow, nextrow;
+    T myval, nextval;
+    int32_t mypos, nextpos;
+    fetch(kb, myrow, myval, mypos);
+    while (kb < end) {   // entry kb belongs to column r
+        if (!mine) {     // a long column is not computed here: jump over what is left of it
+            kb = row_end;
+            close_row();
+            if (kb >= end) break;
+            fetch(kb, myrow, myval, mypos);
+            continue;
+        }
+        const int cnt = (int)(end - kb < kWave ? end - kb : kWave);
+        fetch(kb + kWave, nextrow, nextval, nextpos);   // in flight while this chunk is used
+        const int64_t k = kb + lane;
+        const int64_t myoff = myrow * row_bytes;
+        int rid = 0;
+        for (int l = 1; l < nr; ++l) rid += k >= ptr_of(l) ? 1 : 0;
+        const int64_t my_row_end = __shfl(my_ptr, rid + 1, kWave);
+        const unsigned long long ends = __ballot(lane < cnt && k + 1 == my_row_end);
+        // entries of a long column inside this chunk are not computed here: their dot products
+        // are written by the workgroup that takes the column
+        const int64_t my_row_begin = __shfl(my_ptr, rid, kWave);
+        const bool here = lane < cnt && my_row_end - my_row_begin <= kSplitRow;
+        T mydot = T(0);
+        auto gather = [&](int j0, T (&gv)[kBatch]) {
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int j = __builtin_amdgcn_readfirstlane(j0 + u < cnt ? j0 + u : cnt - 1);
+                const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(myoff & 0xffffffffll), j);
+                const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(myoff >> 32), j);
+                gv[u] = *reinterpret_cast<const T *>(Gc + (int64_t)(((unsigned long long)hi << 32) | lo));
+            }
+        };
+        // Returns true when the walk met a long column inside the batch (the rest of the chunk is
+        // then abandoned and taken up again behind that column).
+        auto add_up = [&](int j0, const T (&gv)[kBatch]) {
+            const int m = cnt - j0 < kBatch ? cnt - j0 : kBatch;
+            T p[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) p[u] = T(0);
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                if (u >= m) break;
+                const int j = __builtin_amdgcn_readfirstlane(j0 + u);
+                acc += nm::read_lane(myval, j) * gv[u];
+                p[u] = live ? gv[u] * cur_b : T(0);
+                if ((ends >> j) & 1ull) close_row();
+            }
+            const T t = fold8<T>(p, lane);
+            if ((lane >> 3) == (j0 >> 3)) mydot += t;   // lane j0 + u takes vector u
+        };
+        T gva[kBatch], gvb[kBatch];
+        gather(0, gva);
+        for (int j0 = 0;; j0 += 2 * kBatch) {
+            if (j0 + kBatch < cnt) gather(j0 + kBatch, gvb);
+            add_up(j0, gva);
+            if (j0 + kBatch >= cnt) break;
+            if (j0 + 2 * kBatch < cnt) gather(j0 + 2 * kBatch, gva);
+            add_up(j0 + kBatch, gvb);
+            if (j0 + 2 * kBatch >= cnt) break;
+        }
+        if (here) grad_A[mypos] = mydot;
+        kb += cnt;
+        myrow = nextrow;
+        myval = nextval;
+        mypos = nextpos;
+    }
+    while (r < nr) next_row();   // columns of a wavefront whose entries ran out before them
 }
 
 // ---- narrow dense operands (n <= 32) -----------------------------------------------
@@ -644,6 +836,23 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
     NM_REQUIRE(plan_mem != nullptr, "plan is null");
     nm::TPlan t;
     nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
+    if (grad_A && grad_B && rows > 0 && cols > 0 && nnz > 0 && n > 32 && n <= kWave) {
+        // one column tile: both gradients from a single walk over A by column
+        NM_REQUIRE(B != nullptr && gC != nullptr, "B or gC is null");
+        NM_REQUIRE(ldb >= n && ldg >= n && ldgb >= n, "row stride smaller than the row");
+        hipStream_t s = nm::as_stream(stream);
+        const unsigned grid = flat_grid_for(cols);
+        if (dt == NM_F32)
+            hipLaunchKernelGGL(spdmm_bwd_fused_kernel<float>, dim3(grid), dim3(kBlock), 0, s, cols, (const float *)data,
+                               t.t_row, t.t_indptr, t.t_perm, (const float *)gC, ldg, (const float *)B, ldb, n,
+                               (float *)grad_B, ldgb, (float *)grad_A);
+        else
+            hipLaunchKernelGGL(spdmm_bwd_fused_kernel<double>, dim3(grid), dim3(kBlock), 0, s, cols,
+                               (const double *)data, t.t_row, t.t_indptr, t.t_perm, (const double *)gC, ldg,
+                               (const double *)B, ldb, n, (double *)grad_B, ldgb, (double *)grad_A);
+        NM_LAUNCH_CHECK("spdmm_bwd_fused_kernel");
+        return NM_OK;
+    }
     if (grad_A) {
         if (int rc = backward_impl(dt, rows, cols, nnz, data, indices, indptr, B, ldb, gC, ldg, n, grad_A, nullptr, 0,
                                    t.chunk_row, stream))

@@ -91,6 +91,68 @@ def test_spmm_forward_backward(dev, dtype, n, backward_mode):
             assert_same(host(gB), gB_ref, f"{name} grad_B (bitwise)")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_spmm_backward_on_one_walk(dev, dtype):
+    """With 33-64 dense columns the backward on a plan forms both gradients in one walk over A by
+    column.  Against the oracle, and bit for bit against the two separate walks it replaces (the C
+    ABI computes one gradient alone the old way), on patterns with columns of more than 512
+    entries (shared by a workgroup), empty columns and rows, and a single long chunk."""
+    import ctypes
+    import scipy.sparse as sps
+    from numml_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(5)
+
+    def with_dense_columns(rows, cols, density, dense_cols):
+        M = sps.random(rows, cols, density=density, random_state=7, format="lil", dtype=np.float64)
+        for c in dense_cols:
+            M[:, c] = rng.standard_normal((rows, 1))
+        M = M.tocsr().astype(dtype)
+        M.sort_indices()
+        return M.data.copy(), M.indices.astype(np.int64), M.indptr.astype(np.int64), (rows, cols)
+
+    cases = [("ragged", G.random_csr(700, 300, 0.02, 5, dtype)),
+             ("long_columns", with_dense_columns(1500, 200, 0.01, (3, 77, 199))),
+             ("one_column", with_dense_columns(900, 1, 0.0, (0,))),
+             ("powerlaw_T", G.powerlaw(3000, 3000, target_nnz=60000, max_deg=2500, seed=7, dtype=dtype)),
+             ("poisson64", G.poisson2d(64, dtype, jitter_seed=3))]
+    # the power-law matrix transposed: its long rows become long columns
+    d, i, p, (r, c) = cases[3][1]
+    T = sps.csr_matrix((d, i, p), shape=(r, c)).T.tocsr()
+    T.sort_indices()
+    cases[3] = ("powerlaw_T", (T.data.astype(dtype), T.indices.astype(np.int64), T.indptr.astype(np.int64), (c, r)))
+    old = ext.BACKWARD_MODE
+    ext.BACKWARD_MODE = "eager"
+    try:
+        for name, (d, i, p, (rows, cols)) in cases:
+            for n in (33, 48, 64):
+                B, gC = randn(1, (cols, n), dtype), randn(2, (rows, n), dtype)
+                gA_ref, gB_ref = oracle.spdmm_backward(rows, cols, d, i, p, B, gC)
+                D, I, P, Bd, gCd = to_dev(dev, d, i, p, B, gC)
+                gA, gB = ext.spdmm_backward(rows, cols, D, I, P, Bd, gCd)
+                assert_close(host(gA), gA_ref, f"{name} n={n} grad_A")
+                assert_close(host(gB), gB_ref, f"{name} n={n} grad_B")
+                longest = int(np.bincount(i, minlength=1).max()) if i.size else 0
+                if longest <= 512:
+                    assert_same(host(gB), gB_ref, f"{name} n={n} grad_B (bitwise)")
+                # one gradient at a time goes the old way: the row-major dot products, the product on the plan
+                plan = ext._transpose_plan(I, P, rows, cols, dev)
+                gA2, gB2 = torch.empty_like(D), torch.empty_like(gB)
+                args = (ext._dt(D), rows, cols, D.shape[0], D.data_ptr(), I.data_ptr(), P.data_ptr(),
+                        plan.mem.data_ptr(), Bd.data_ptr(), n, gCd.data_ptr(), n, n)
+                assert L.nm_spdmm_backward_planned(*args, gA2.data_ptr(), None, n, None) == 0
+                assert L.nm_spdmm_backward_planned(*args, None, gB2.data_ptr(), n, None) == 0
+                torch.cuda.synchronize()
+                if longest <= 512:
+                    assert_same(host(gA), host(gA2), f"{name} n={n} grad_A: one walk vs two")
+                    assert_same(host(gB), host(gB2), f"{name} n={n} grad_B: one walk vs two")
+                else:       # columns shared by a workgroup sum their dot products in another order
+                    assert_close(host(gA), host(gA2), f"{name} n={n} grad_A: one walk vs two")
+                    assert_same(host(gB), host(gB2), f"{name} n={n} grad_B: one walk vs two")
+    finally:
+        ext.BACKWARD_MODE = old
+
+
 def test_spmm_strided_operand(dev):
     d, i, p, (rows, cols) = G.random_csr(200, 150, 0.05, 11, np.float64)
     wide = randn(3, (cols, 40), np.float64)
