@@ -361,6 +361,70 @@ __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     if (mine) grad_B[bb + k] = acc;
 }
 
+// Both gradients from the walk by column.  The eight lanes of row j of B gather, for every entry
+// e of column j of A, the eight entries of gC that e's products went to -- which is also all
+// that grad_A[e] = sum_k gC[..] * B[j][k] needs besides the row of B the lanes own.  So the terms
+// of grad_A are formed from the values just gathered and change places through LDS exactly as
+// in grad_a_mapped_kernel (lane u adds the eight terms of the round's u-th entry in ascending
+// k: the same bits), and the row-major walk with its own gathers of gC falls away.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void grad_ab_mapped_kernel(
+    int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
+    const T *__restrict__ B_data, const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm,
+    const int64_t *__restrict__ B_indptr, const int32_t *__restrict__ t_cstart, const uint8_t *__restrict__ t_dest,
+    T *__restrict__ grad_A, T *__restrict__ grad_B) {
+    __shared__ T s_a[kBlock];
+    __shared__ int32_t s_cs[kBlock];
+    __shared__ __align__(8) uint8_t s_db[kBlock * kCap];
+    __shared__ T s_term[kBlock * kTermStride];
+    const int k = threadIdx.x & (kCap - 1), slot = threadIdx.x & ~(kCap - 1);
+    const int64_t j = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + threadIdx.x / kCap;
+    const bool live = j < B_rows;
+    const int64_t *pb_ = B_indptr + (live ? j : 0);
+    const int64_t bb = pb_[0], blen = live ? pb_[1] - bb : 0;
+    const int32_t *pt = t_indptr + (live ? j : 0);
+    const int32_t pb = pt[0], pe = live ? pt[1] : pb;
+    if (pb == pe) {   // no entry of A in this column: the row's gradient is zero, however long the row
+        for (int64_t q = k; q < blen; q += kCap) grad_B[bb + q] = T(0);
+        return;       // (no workgroup barrier anywhere in this kernel)
+    }
+    const bool mine = k < blen;
+    const T bk = mine ? B_data[bb + k] : T(0);
+    T acc = T(0);
+    for (int32_t t0 = pb; t0 < pe; t0 += kCap) {
+        const bool have = t0 + k < pe;
+        const int32_t pos = t_perm[have ? t0 + k : pb];
+        {
+            const int32_t t = have ? t0 + k : pb;
+            s_a[threadIdx.x] = A_data[pos];
+            s_cs[threadIdx.x] = t_cstart[t];
+            *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) =
+                have ? *reinterpret_cast<const uint64_t *>(t_dest + (int64_t)t * kCap) : ~uint64_t(0);
+        }
+        group_fence();
+        uint8_t db[kCap];
+        T gv[kCap];
+#pragma unroll
+        for (int u = 0; u < kCap; ++u) {
+            db[u] = mine ? s_db[(slot + u) * kCap + k] : kNone;
+            gv[u] = gC[db[u] != kNone ? (int64_t)s_cs[slot + u] + db[u] : 0];
+        }
+#pragma unroll
+        for (int u = 0; u < kCap; ++u) {
+            const bool on = db[u] != kNone;
+            if (on) acc += s_a[slot + u] * gv[u];
+            s_term[(slot + u) * kTermStride + k] = on ? gv[u] * bk : T(0);
+        }
+        group_fence();
+        T dot = T(0);
+#pragma unroll
+        for (int q = 0; q < kCap; ++q) dot += s_term[(slot + k) * kTermStride + q];
+        if (have) grad_A[pos] = dot;
+        group_fence();   // the exchange slots are written again in the next round
+    }
+    if (mine) grad_B[bb + k] = acc;
+}
+
 // Brings the plan's flags to the host: *usable = 0, or the product's class (1, 2, 3).
 int read_verdict(const PPlan &p, void *host_landing, int *usable, hipStream_t s) {
     int32_t flags[3] = {1, 0, 0};
@@ -388,6 +452,15 @@ template <typename T>
 int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A_data, const nm::TPlan &t,
                     const void *B_data, const int64_t *B_indptr, const PPlan &p, void *grad_A, void *grad_B,
                     hipStream_t s) {
+    if (grad_A && grad_B && A_nnz > 0 && A_cols > 0) {
+        const int64_t grid = nm::xcd_padded(nm::ceil_div(A_cols, (int64_t)kGroupsPerBlock));
+        NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+        hipLaunchKernelGGL(grad_ab_mapped_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, grid,
+                           (const T *)gC, (const T *)A_data, (const T *)B_data, t.t_indptr, t.t_perm, B_indptr,
+                           p.t_cstart, p.t_dest, (T *)grad_A, (T *)grad_B);
+        NM_LAUNCH_CHECK("grad_ab_mapped_kernel");
+        return NM_OK;
+    }
     if (grad_A && A_nnz > 0) {
         const int64_t grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
         NM_REQUIRE(grid < nm::kMaxGrid, "too many entries");
