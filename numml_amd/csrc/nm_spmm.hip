@@ -431,7 +431,8 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
 // per entry, as the row-major kernel above makes them) falls away: half the gathered bytes of
 // the backward.  grad_B is added in the same order as by spdmm_fwd_flat_kernel on the plan
 // and the dot products are folded exactly like spdmm_bwd_kernel's, so both gradients keep
-// their bits.  At most 64 dense columns (one column tile).
+// their bits.  Dense operands wider than 64 columns are taken 64 columns at a time, as by the
+// forward kernel; the dot products add up over the tiles in grad_A.
 template <typename T>
 __device__ __forceinline__ void fused_long_columns(int64_t cols, const T *__restrict__ data,
                                                    const int32_t *__restrict__ t_row,
@@ -450,7 +451,6 @@ __device__ __forceinline__ void fused_long_columns(int64_t cols, const T *__rest
         if (t_indptr[g0 + t + 1] - t_indptr[g0 + t] > kSplitRow) s_long[atomicAdd(&s_nlong, 1)] = t;
     __syncthreads();
     const int nl = s_nlong;
-    const bool live = lane < n;
     for (int li = 0; li < nl; ++li) {   // uniform over the workgroup
         const int64_t col = g0 + s_long[li];
         const int64_t rb = t_indptr[col], re = t_indptr[col + 1];
@@ -458,31 +458,35 @@ __device__ __forceinline__ void fused_long_columns(int64_t cols, const T *__rest
         chunk = (chunk + kWave - 1) / kWave * kWave;
         const int64_t kb0 = rb + wave * chunk;
         const int64_t ke0 = kb0 + chunk < re ? kb0 + chunk : re;
-        const T bj = live ? B[col * ldb + lane] : T(0);
-        T acc = T(0);
-        for (int64_t kb = kb0; kb < ke0; kb += kWave) {
-            const int64_t k = kb + lane;
-            const int64_t myrow = k < ke0 ? (int64_t)t_row[k] : 0;
-            const int32_t myperm = k < ke0 ? t_perm[k] : 0;
-            const T myval = k < ke0 ? data[myperm] : T(0);
-            const int cnt = (int)(ke0 - kb < kWave ? ke0 - kb : kWave);
-            T mydot = T(0);
-            for (int j = 0; j < cnt; ++j) {
-                const T gv = gC[__shfl(myrow, j, kWave) * ldg + (live ? lane : 0)];
-                acc += __shfl(myval, j, kWave) * gv;
-                const T t = nm::wave_sum(live ? gv * bj : T(0));
-                if (lane == j) mydot = t;
+        for (int64_t c0 = 0; c0 < n; c0 += kWave) {   // 64 dense columns at a time
+            const int64_t c = c0 + lane;
+            const bool live = c < n;
+            const T bj = live ? B[col * ldb + c] : T(0);
+            T acc = T(0);
+            for (int64_t kb = kb0; kb < ke0; kb += kWave) {
+                const int64_t k = kb + lane;
+                const int64_t myrow = k < ke0 ? (int64_t)t_row[k] : 0;
+                const int32_t myperm = k < ke0 ? t_perm[k] : 0;
+                const T myval = k < ke0 ? data[myperm] : T(0);
+                const int cnt = (int)(ke0 - kb < kWave ? ke0 - kb : kWave);
+                T mydot = T(0);
+                for (int j = 0; j < cnt; ++j) {
+                    const T gv = gC[__shfl(myrow, j, kWave) * ldg + (live ? c : 0)];
+                    acc += __shfl(myval, j, kWave) * gv;
+                    const T t = nm::wave_sum(live ? gv * bj : T(0));
+                    if (lane == j) mydot = t;
+                }
+                if (lane < cnt) grad_A[myperm] = c0 == 0 ? mydot : grad_A[myperm] + mydot;
             }
-            if (lane < cnt) grad_A[myperm] = mydot;
+            s_part[wave][lane] = acc;
+            __syncthreads();
+            if (wave == 0 && live) {
+                T sum = s_part[0][lane];
+                for (int w = 1; w < kWavesPerBlock; ++w) sum += s_part[w][lane];
+                grad_B[col * ldgb + c] = sum;
+            }
+            __syncthreads();
         }
-        s_part[wave][lane] = acc;
-        __syncthreads();
-        if (wave == 0 && live) {
-            T sum = s_part[0][lane];
-            for (int w = 1; w < kWavesPerBlock; ++w) sum += s_part[w][lane];
-            grad_B[col * ldgb + lane] = sum;
-        }
-        __syncthreads();
     }
 }
 
@@ -504,8 +508,6 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_fused_kernel(
     const int64_t r0 = (((int64_t)blockIdx.x - long_blocks) * kWavesPerBlock + wave) * kFlatRows;
     if (r0 >= cols) return;
     const int nr = (int)(cols - r0 < kFlatRows ? cols - r0 : kFlatRows);
-    const bool live = lane < n;
-    for (int r = 0; r < nr; ++r) s_b[wave][r][lane] = live ? B[(r0 + r) * ldb + lane] : T(0);
     const int64_t my_ptr = (int64_t)t_indptr[r0 + (lane <= nr ? lane : nr)];
     auto ptr_of = [&](int l) {
         const long long lo = __builtin_amdgcn_readlane((int)(my_ptr & 0xffffffffll), l);
@@ -514,102 +516,106 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_fused_kernel(
     };
     const int64_t begin = ptr_of(0), end = ptr_of(nr);
     const int64_t row_bytes = ldg * (int64_t)sizeof(T);
-    const char *__restrict__ Gc = reinterpret_cast<const char *>(gC + (live ? lane : 0));
-    int r = 0;   // current column (relative), its range, whether it is computed here
-    int64_t row_begin = begin, row_end = ptr_of(1);
-    bool mine = row_end - row_begin <= kSplitRow;
-    T acc = T(0);
-    T cur_b = s_b[wave][0][lane];
-    auto next_row = [&]() {
-        if (mine && live) grad_B[(r0 + r) * ldgb + lane] = acc;
-        acc = T(0);
-        ++r;
-        row_begin = row_end;
-        row_end = ptr_of(r + 1 <= nr ? r + 1 : nr);
-        mine = row_end - row_begin <= kSplitRow;
-        cur_b = s_b[wave][r < nr ? r : nr - 1][lane];
-    };
-    auto close_row = [&]() {
-        next_row();
-        while (r < nr && row_end == row_begin) next_row();
-    };
-    while (r < nr && row_end == row_begin) next_row();   // empty columns at the head
-    int64_t kb = begin;
-    auto fetch = [&](int64_t at, int64_t &row, T &val, int32_t &pos) {
-        const int64_t k = at + lane < end ? at + lane : (end > begin ? end - 1 : 0);
-        row = end > begin ? (int64_t)t_row[k] : 0;
-        pos = end > begin ? t_perm[k] : 0;
-        val = end > begin ? data[pos] : T(0);
-    };
-    int64_t myrow, nextrow;
-    T myval, nextval;
-    int32_t mypos, nextpos;
-    fetch(kb, myrow, myval, mypos);
-    while (kb < end) {   // entry kb belongs to column r
-        if (!mine) {     // a long column is not computed here: jump over what is left of it
-            kb = row_end;
-            close_row();
-            if (kb >= end) break;
-            fetch(kb, myrow, myval, mypos);
-            continue;
-        }
-        const int cnt = (int)(end - kb < kWave ? end - kb : kWave);
-        fetch(kb + kWave, nextrow, nextval, nextpos);   // in flight while this chunk is used
-        const int64_t k = kb + lane;
-        const int64_t myoff = myrow * row_bytes;
-        int rid = 0;
-        for (int l = 1; l < nr; ++l) rid += k >= ptr_of(l) ? 1 : 0;
-        const int64_t my_row_end = __shfl(my_ptr, rid + 1, kWave);
-        const unsigned long long ends = __ballot(lane < cnt && k + 1 == my_row_end);
-        // entries of a long column inside this chunk are not computed here: their dot products
-        // are written by the workgroup that takes the column
-        const int64_t my_row_begin = __shfl(my_ptr, rid, kWave);
-        const bool here = lane < cnt && my_row_end - my_row_begin <= kSplitRow;
-        T mydot = T(0);
-        auto gather = [&](int j0, T (&gv)[kBatch]) {
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const int j = __builtin_amdgcn_readfirstlane(j0 + u < cnt ? j0 + u : cnt - 1);
-                const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(myoff & 0xffffffffll), j);
-                const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(myoff >> 32), j);
-                gv[u] = *reinterpret_cast<const T *>(Gc + (int64_t)(((unsigned long long)hi << 32) | lo));
-            }
+    for (int64_t c0 = 0; c0 < n; c0 += kWave) {   // 64 dense columns at a time; the dot products add up over the tiles
+        const int64_t c = c0 + lane;
+        const bool live = c < n;
+        const bool first_tile = c0 == 0;
+        for (int r = 0; r < nr; ++r) s_b[wave][r][lane] = live ? B[(r0 + r) * ldb + c] : T(0);
+        const char *__restrict__ Gc = reinterpret_cast<const char *>(gC + (live ? c : 0));
+        int r = 0;   // current column (relative), its range, whether it is computed here
+        int64_t row_begin = begin, row_end = ptr_of(1);
+        bool mine = row_end - row_begin <= kSplitRow;
+        T acc = T(0);
+        T cur_b = s_b[wave][0][lane];
+        auto next_row = [&]() {
+            if (mine && live) grad_B[(r0 + r) * ldgb + c] = acc;
+            acc = T(0);
+            ++r;
+            row_begin = row_end;
+            row_end = ptr_of(r + 1 <= nr ? r + 1 : nr);
+            mine = row_end - row_begin <= kSplitRow;
+            cur_b = s_b[wave][r < nr ? r : nr - 1][lane];
         };
-        // Returns true when the walk met a long column inside the batch (the rest of the chunk is
-        // then abandoned and taken up again behind that column).
-        auto add_up = [&](int j0, const T (&gv)[kBatch]) {
-            const int m = cnt - j0 < kBatch ? cnt - j0 : kBatch;
-            T p[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) p[u] = T(0);
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                if (u >= m) break;
-                const int j = __builtin_amdgcn_readfirstlane(j0 + u);
-                acc += nm::read_lane(myval, j) * gv[u];
-                p[u] = live ? gv[u] * cur_b : T(0);
-                if ((ends >> j) & 1ull) close_row();
-            }
-            const T t = fold8<T>(p, lane);
-            if ((lane >> 3) == (j0 >> 3)) mydot += t;   // lane j0 + u takes vector u
+        auto close_row = [&]() {
+            next_row();
+            while (r < nr && row_end == row_begin) next_row();
         };
-        T gva[kBatch], gvb[kBatch];
-        gather(0, gva);
-        for (int j0 = 0;; j0 += 2 * kBatch) {
-            if (j0 + kBatch < cnt) gather(j0 + kBatch, gvb);
-            add_up(j0, gva);
-            if (j0 + kBatch >= cnt) break;
-            if (j0 + 2 * kBatch < cnt) gather(j0 + 2 * kBatch, gva);
-            add_up(j0 + kBatch, gvb);
-            if (j0 + 2 * kBatch >= cnt) break;
+        while (r < nr && row_end == row_begin) next_row();   // empty columns at the head
+        int64_t kb = begin;
+        auto fetch = [&](int64_t at, int64_t &row, T &val, int32_t &pos) {
+            const int64_t k = at + lane < end ? at + lane : (end > begin ? end - 1 : 0);
+            row = end > begin ? (int64_t)t_row[k] : 0;
+            pos = end > begin ? t_perm[k] : 0;
+            val = end > begin ? data[pos] : T(0);
+        };
+        int64_t myrow, nextrow;
+        T myval, nextval;
+        int32_t mypos, nextpos;
+        fetch(kb, myrow, myval, mypos);
+        while (kb < end) {   // entry kb belongs to column r
+            if (!mine) {     // a long column is not computed here: jump over what is left of it
+                kb = row_end;
+                close_row();
+                if (kb >= end) break;
+                fetch(kb, myrow, myval, mypos);
+                continue;
+            }
+            const int cnt = (int)(end - kb < kWave ? end - kb : kWave);
+            fetch(kb + kWave, nextrow, nextval, nextpos);   // in flight while this chunk is used
+            const int64_t k = kb + lane;
+            const int64_t myoff = myrow * row_bytes;
+            int rid = 0;
+            for (int l = 1; l < nr; ++l) rid += k >= ptr_of(l) ? 1 : 0;
+            const int64_t my_row_end = __shfl(my_ptr, rid + 1, kWave);
+            const unsigned long long ends = __ballot(lane < cnt && k + 1 == my_row_end);
+            // entries of a long column inside this chunk are not computed here: their dot products
+            // are written by the workgroup that takes the column
+            const int64_t my_row_begin = __shfl(my_ptr, rid, kWave);
+            const bool here = lane < cnt && my_row_end - my_row_begin <= kSplitRow;
+            T mydot = T(0);
+            auto gather = [&](int j0, T (&gv)[kBatch]) {
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const int j = __builtin_amdgcn_readfirstlane(j0 + u < cnt ? j0 + u : cnt - 1);
+                    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(myoff & 0xffffffffll), j);
+                    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(myoff >> 32), j);
+                    gv[u] = *reinterpret_cast<const T *>(Gc + (int64_t)(((unsigned long long)hi << 32) | lo));
+                }
+            };
+            auto add_up = [&](int j0, const T (&gv)[kBatch]) {
+                const int m = cnt - j0 < kBatch ? cnt - j0 : kBatch;
+                T p[kBatch];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) p[u] = T(0);
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    if (u >= m) break;
+                    const int j = __builtin_amdgcn_readfirstlane(j0 + u);
+                    acc += nm::read_lane(myval, j) * gv[u];
+                    p[u] = live ? gv[u] * cur_b : T(0);
+                    if ((ends >> j) & 1ull) close_row();
+                }
+                const T t = fold8<T>(p, lane);
+                if ((lane >> 3) == (j0 >> 3)) mydot += t;   // lane j0 + u takes vector u
+            };
+            T gva[kBatch], gvb[kBatch];
+            gather(0, gva);
+            for (int j0 = 0;; j0 += 2 * kBatch) {
+                if (j0 + kBatch < cnt) gather(j0 + kBatch, gvb);
+                add_up(j0, gva);
+                if (j0 + kBatch >= cnt) break;
+                if (j0 + 2 * kBatch < cnt) gather(j0 + 2 * kBatch, gva);
+                add_up(j0 + kBatch, gvb);
+                if (j0 + 2 * kBatch >= cnt) break;
+            }
+            if (here) grad_A[mypos] = first_tile ? mydot : grad_A[mypos] + mydot;
+            kb += cnt;
+            myrow = nextrow;
+            myval = nextval;
+            mypos = nextpos;
         }
-        if (here) grad_A[mypos] = mydot;
-        kb += cnt;
-        myrow = nextrow;
-        myval = nextval;
-        mypos = nextpos;
+        while (r < nr) next_row();   // columns of a wavefront whose entries ran out before them
     }
-    while (r < nr) next_row();   // columns of a wavefront whose entries ran out before them
 }
 
 // ---- narrow dense operands (n <= 32) -----------------------------------------------
@@ -836,8 +842,11 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
     NM_REQUIRE(plan_mem != nullptr, "plan is null");
     nm::TPlan t;
     nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
-    if (grad_A && grad_B && rows > 0 && cols > 0 && nnz > 0 && n > 32 && n <= kWave) {
-        // one column tile: both gradients from a single walk over A by column
+    if (grad_A && grad_B && rows > 0 && cols > 0 && nnz > 0 && n > 32) {
+        // both gradients from a single walk over A by column (measured on the 16 M-entry power-law
+        // matrix: 1.02 against 1.29 ms at 64 dense columns, 2.18 against 2.80 ms at 128, even at 32;
+        // with 16 or fewer the narrow dot-product kernel below and a separate product are faster,
+        // 0.70-0.74 against 0.81-0.82 ms)
         NM_REQUIRE(B != nullptr && gC != nullptr, "B or gC is null");
         NM_REQUIRE(ldb >= n && ldg >= n && ldgb >= n, "row stride smaller than the row");
         hipStream_t s = nm::as_stream(stream);

@@ -93,8 +93,7 @@ def test_spmm_forward_backward(dev, dtype, n, backward_mode):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_spmm_backward_on_one_walk(dev, dtype):
-    """With 33-64 dense columns the backward on a plan forms both gradients in one walk over A by
-    column.  Against the oracle, and bit for bit against the two separate walks it replaces (the C
+    """The backward on a plan forms both gradients in one walk over A by column.  Against the oracle, and bit for bit against the two separate walks it replaces (the C
     ABI computes one gradient alone the old way), on patterns with columns of more than 512
     entries (shared by a workgroup), empty columns and rows, and a single long chunk."""
     import ctypes
@@ -125,7 +124,7 @@ def test_spmm_backward_on_one_walk(dev, dtype):
     ext.BACKWARD_MODE = "eager"
     try:
         for name, (d, i, p, (rows, cols)) in cases:
-            for n in (33, 48, 64):
+            for n in (5, 33, 64, 100):
                 B, gC = randn(1, (cols, n), dtype), randn(2, (rows, n), dtype)
                 gA_ref, gB_ref = oracle.spdmm_backward(rows, cols, d, i, p, B, gC)
                 D, I, P, Bd, gCd = to_dev(dev, d, i, p, B, gC)
@@ -143,8 +142,11 @@ def test_spmm_backward_on_one_walk(dev, dtype):
                 assert L.nm_spdmm_backward_planned(*args, gA2.data_ptr(), None, n, None) == 0
                 assert L.nm_spdmm_backward_planned(*args, None, gB2.data_ptr(), n, None) == 0
                 torch.cuda.synchronize()
-                if longest <= 512:
+                if longest <= 512 and n > 32:
                     assert_same(host(gA), host(gA2), f"{name} n={n} grad_A: one walk vs two")
+                    assert_same(host(gB), host(gB2), f"{name} n={n} grad_B: one walk vs two")
+                elif longest <= 512:    # up to 32 columns the separate dot products fold 8-32 lanes, not 64
+                    assert_close(host(gA), host(gA2), f"{name} n={n} grad_A: one walk vs two")
                     assert_same(host(gB), host(gB2), f"{name} n={n} grad_B: one walk vs two")
                 else:       # columns shared by a workgroup sum their dot products in another order
                     assert_close(host(gA), host(gA2), f"{name} n={n} grad_A: one walk vs two")
