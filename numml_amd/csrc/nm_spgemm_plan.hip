@@ -101,13 +101,29 @@ __global__ __launch_bounds__(kBlock) void plan_map_kernel(
     if (wide_c) p.flag[2] = 1;
 }
 
+// Checks the length of A's columns and notes in flag[3] how far from the diagonal A reaches
+// (the largest |row - column| of a stored entry: rows ascend inside a column, so its first and
+// last entry decide), which the backward uses to order its tiles.
 __global__ __launch_bounds__(kBlock) void plan_columns_kernel(int64_t cols, const int32_t *__restrict__ t_indptr,
-                                                              int32_t *flag) {
+                                                              const int32_t *__restrict__ t_row, int32_t *flag) {
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     bool bad = false;
-    for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < cols; j += stride)
-        bad |= t_indptr[j + 1] - t_indptr[j] > kMaxColumn;
+    int32_t far = 0;
+    for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < cols; j += stride) {
+        const int32_t pb = t_indptr[j], pe = t_indptr[j + 1];
+        bad |= pe - pb > kMaxColumn;
+        if (pe > pb) {
+            const int32_t lo = (int32_t)j - t_row[pb], hi = t_row[pe - 1] - (int32_t)j;
+            far = far > lo ? far : lo;
+            far = far > hi ? far : hi;
+        }
+    }
     if (bad) flag[0] = 1;
+    for (int off = 32; off > 0; off >>= 1) {
+        const int32_t other = __shfl_xor(far, off, kWave);
+        far = far > other ? far : other;
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0 && far > 0) atomicMax(flag + 3, far);
 }
 
 // The column-major copies of cstart and dest (entry t of the transposed plan is entry t_perm[t]).
@@ -275,6 +291,8 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_long
 // entry (coalesced reads of the B rows); the terms change places through LDS so that lane e
 // then adds the eight terms of entry e in ascending k.
 constexpr int kTermStride = kCap + 1;
+constexpr int kStripTiles = 32;        // tiles (of kGroupsPerBlock rows of B) per strip of the backward's walk
+constexpr int kStripFrom = 8192;       // rows: columns that reach less far keep the plain order
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void grad_a_mapped_kernel(
@@ -372,13 +390,35 @@ __global__ __launch_bounds__(kBlock) void grad_ab_mapped_kernel(
     int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
     const T *__restrict__ B_data, const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm,
     const int64_t *__restrict__ B_indptr, const int32_t *__restrict__ t_cstart, const uint8_t *__restrict__ t_dest,
-    T *__restrict__ grad_A, T *__restrict__ grad_B) {
+    T *__restrict__ grad_A, T *__restrict__ grad_B, const int32_t *__restrict__ flag) {
     __shared__ T s_a[kBlock];
     __shared__ int32_t s_cs[kBlock];
     __shared__ __align__(8) uint8_t s_db[kBlock * kCap];
     __shared__ T s_term[kBlock * kTermStride];
     const int k = threadIdx.x & (kCap - 1), slot = threadIdx.x & ~(kCap - 1);
-    const int64_t j = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + threadIdx.x / kCap;
+    // Every XCD walks one contiguous eighth of the rows of B.  A column of A reaches `far` rows
+    // from the diagonal (a 3D stencil: one grid plane), and the rows of gC it names there are
+    // wanted again one plane of rows later: when a plane's worth of work is more than an L2
+    // holds, the eighth is walked in strips instead -- rows [q S, (q + 1) S) of plane 0, of
+    // plane 1, ..., then the next strip -- so that what is wanted again was fetched a strip ago.
+    // (cfg4: 0.39 -> 0.35 ms; strips of 1024 rows; 256 and 4096 rows were slower.)
+    int64_t tile;
+    {
+        const int64_t per = ntiles_padded / nm::kXcds, x = blockIdx.x % nm::kXcds;
+        int64_t u = blockIdx.x / nm::kXcds;
+        const int64_t far = flag[3];
+        const int64_t plane = far / kGroupsPerBlock / kStripTiles * kStripTiles;   // in tiles, whole strips
+        if (far >= kStripFrom && plane > 0) {
+            const int64_t planes = per / plane;
+            if (u < planes * plane) {
+                const int64_t o = u % kStripTiles, zq = u / kStripTiles;
+                const int64_t z = zq % planes, q = zq / planes;
+                u = z * plane + q * kStripTiles + o;
+            }
+        }
+        tile = x * per + u;
+    }
+    const int64_t j = tile * kGroupsPerBlock + threadIdx.x / kCap;
     const bool live = j < B_rows;
     const int64_t *pb_ = B_indptr + (live ? j : 0);
     const int64_t bb = pb_[0], blen = live ? pb_[1] - bb : 0;
@@ -457,7 +497,7 @@ int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A
         NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
         hipLaunchKernelGGL(grad_ab_mapped_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, grid,
                            (const T *)gC, (const T *)A_data, (const T *)B_data, t.t_indptr, t.t_perm, B_indptr,
-                           p.t_cstart, p.t_dest, (T *)grad_A, (T *)grad_B);
+                           p.t_cstart, p.t_dest, (T *)grad_A, (T *)grad_B, p.flag);
         NM_LAUNCH_CHECK("grad_ab_mapped_kernel");
         return NM_OK;
     }
@@ -515,7 +555,8 @@ extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nn
     NM_LAUNCH_CHECK("plan_map_kernel");
     grid = nm::ceil_div(A_cols > 0 ? A_cols : 1, (int64_t)kBlock);
     if (grid > 4096) grid = 4096;
-    hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, p.flag);
+    hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, t.t_row,
+                       p.flag);
     NM_LAUNCH_CHECK("plan_columns_kernel");
     grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
     if (grid > 65536) grid = 65536;
@@ -545,7 +586,8 @@ extern "C" int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nn
     if (int rc = nm::fill_async(p.flag, 16, (int32_t)0, s)) return rc;
     int64_t grid = nm::ceil_div(A_cols > 0 ? A_cols : 1, (int64_t)kBlock);
     if (grid > 4096) grid = 4096;
-    hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, p.flag);
+    hipLaunchKernelGGL(plan_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, t.t_indptr, t.t_row,
+                       p.flag);
     NM_LAUNCH_CHECK("plan_columns_kernel");
     grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
     if (grid > 65536) grid = 65536;

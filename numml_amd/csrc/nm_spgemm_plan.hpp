@@ -14,7 +14,8 @@ constexpr int kPlanRowCap = kPlanCap * kPlanCap; // entries per row of C
 constexpr uint8_t kPlanNone = 0xFF;              // destination byte of an entry a B row does not have
 
 struct PPlan {
-    int32_t *flag;     // [0] != 0: a limit does not hold, the plan must not be used
+    int32_t *flag;     // [0] != 0: a limit does not hold, the plan must not be used; [1], [2]: the product's
+                       // class; [3]: the largest |row - column| of an entry of A
     int32_t *bstart;   // [A_nnz] where the row of B that entry e of A names starts
     int32_t *cstart;   // [A_nnz] where the row of C that entry e of A lies in starts
     uint8_t *dest;     // [A_nnz * 8] byte k: position in that row of C of the k-th entry of that row of B
