@@ -92,6 +92,33 @@ def test_planned_product_and_gradients_match_the_stateless_kernels_and_the_oracl
         assert_same(host(gB), host(sB), f"{name}: grad_B vs the search-based kernel")
 
 
+def test_backward_walks_far_reaching_patterns_in_strips(dev):
+    """When A reaches 8192 rows or more from its diagonal, the kernel that forms both gradients walks
+    each XCD's share of the rows in strips.  The order is only a schedule: every row must still be
+    taken exactly once.  A band at +-9000 on 300 000 rows leaves a tail that the strips do not cover
+    (walked in plain order), and one gradient alone still goes through the two separate kernels."""
+    import scipy.sparse as sps
+    n, far = 300_000, 9000
+    rng = np.random.default_rng(3)
+    diags = [rng.standard_normal(n - abs(o)) for o in (-far, -1, 0, 1, far)]
+    A = sps.diags(diags, (-far, -1, 0, 1, far), shape=(n, n), format="csr")
+    A.sort_indices()
+    ad, ai, ap = A.data.copy(), A.indices.astype(np.int64), A.indptr.astype(np.int64)
+    bd = rng.standard_normal(ad.shape[0])
+    AD, AI, AP, BD = to_dev(dev, ad, ai, ap, bd)
+    C_data, C_indices, C_indptr = mirror.spgemm_forward(n, n, AD, AI, AP, n, n, BD, AI, AP)
+    plan = mirror.ProductPlan(n, n, AI, AP, AI, AP, C_indices, C_indptr)
+    assert plan.usable
+    cd, ci, cp = oracle.spgemm_forward(n, n, ad, ai, ap, n, n, bd, ai, ap)
+    assert_same(host(plan.numeric(AD, BD)), cd, "C_data")
+    g = randn(5, cd.shape[0], np.float64)
+    Gz, = to_dev(dev, g)
+    rA, rB = oracle.spgemm_backward(g, ci, cp, n, n, ad, ai, ap, n, n, bd, ai, ap)
+    gA, gB = plan.backward(Gz, AD, BD)
+    assert_same(host(gA), rA, "grad_A (both gradients in one walk, in strips)")
+    assert_same(host(gB), rB, "grad_B (both gradients in one walk, in strips)")
+
+
 def test_signed_zeros_and_explicit_zeros_keep_the_serial_result(dev):
     dtype = np.float64
     ad, ai, ap, ashape = _unpack(G.poisson2d(12, dtype))
