@@ -125,14 +125,38 @@ def _first_calls(ext, call, n=3):
     return firsts
 
 
-def _spmv_bytes(rows, cols, nnz, s, i_fwd=8):
-    """Algorithmic bytes of one forward and one backward.  i_fwd: index bytes the forward reads
-    per entry and per row pointer (8 as the interface delivers them, 4 when the kernel reads
-    the 32-bit copies a transposed-structure plan holds).  The planned backward reads two
-    int32 per entry (row and position in the plan), i.e. the same 8 index bytes per entry as
-    the int64 row-major formula, and 4-byte column pointers."""
-    fwd = nnz * (s + i_fwd) + (rows + 1) * i_fwd + cols * s + rows * s
-    bwd = nnz * (s + 8) + (rows + 1) * 8 + rows * s + cols * s + nnz * s + cols * s
+def _spmv_bytes(rows, cols, nnz, s, i_fwd=8, i_bwd=8, planned=None):
+    """Algorithmic bytes of one forward and one backward, every array counted once at the width
+    the kernel reads.  i_fwd: index bytes the forward reads per entry (8 as the interface delivers
+    them, 4 for the 32-bit copies a transposed-structure plan holds, 2 for the plan's 16-bit
+    column offsets of a banded pattern).  i_bwd: structure bytes the backward reads per entry
+    (8: int64 columns without a plan, or row and position as two int32 of the plan; 4: the
+    plan's packed word of a banded pattern).  Row and column pointers are 8 bytes wide as the
+    interface delivers them and 4 in a plan (`planned`; by default a plan is assumed whenever
+    an index width below 8 is given)."""
+    if planned is None:
+        planned = i_fwd < 8 or i_bwd < 8
+    ptr = 4 if planned else 8
+    fwd = nnz * (s + i_fwd) + (rows + 1) * ptr + cols * s + rows * s
+    bwd = nnz * (s + i_bwd) + (cols + 1) * ptr + rows * s + cols * s + nnz * s + cols * s
+    return fwd, bwd
+
+
+def _spmv_plan_widths(indices, indptr, rows, cols):
+    """(index bytes per entry of the planned forward, structure bytes per entry of the planned
+    backward) for this pattern, by the rules the plan build applies on the device: 16-bit column
+    offsets from the first row of a block of 512 rows where all of them fit (and rows are short
+    enough for 512-row blocks), one packed word per entry where the row offset from the first
+    column of a block of 256 columns and the distance to the mirror position both fit 16 bits."""
+    nnz = indices.shape[0]
+    row_of = np.repeat(np.arange(rows, dtype=np.int64), np.diff(indptr))
+    off = indices - (row_of & ~np.int64(511))
+    mean = -(-nnz // rows) if rows else 1
+    fwd = 2 if nnz and off.min() >= -32768 and off.max() <= 32767 and 4096 // max(mean, 1) >= 512 else 4
+    perm = np.argsort(indices, kind="stable")
+    dr = row_of[perm] - (indices[perm] & ~np.int64(255))
+    dk = perm - np.arange(nnz, dtype=np.int64)
+    bwd = 4 if nnz and min(dr.min(), dk.min()) >= -32768 and max(dr.max(), dk.max()) <= 32767 else 8
     return fwd, bwd
 
 
@@ -166,7 +190,10 @@ class SpMV(Workload):
         # with a plan in the cache (every step after the second backward) the forward reads the
         # plan's 32-bit structure
         planned = _binding.backward_mode() != "atomic" and _binding.name == "compiled"
-        self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s, 4 if planned else 8)
+        i_fwd, i_bwd = _spmv_plan_widths(i, p, rows, cols) if planned else (8, 8)
+        if _binding.backward_mode() != "atomic" and not planned:    # ctypes mirror: planned backward only
+            i_bwd = _spmv_plan_widths(i, p, rows, cols)[1]
+        self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s, i_fwd, i_bwd, planned=_binding.backward_mode() != "atomic")
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
         self.dominant_name = ("spmv_bwd_planned_kernel" if _binding.backward_mode() != "atomic"
@@ -178,10 +205,11 @@ class SpMV(Workload):
         self.first_backward_ms = firsts
         self.config = {"workload": f"spmv_fwd_bwd_{self.dtype}_{self.label}", "rows": rows,
                        "first_three_backward_calls_ms": firsts,
-                       "nnz": self.nnz, "index_bytes_forward": 4 if planned else 8,
-                       "index_bytes_backward": 8, "backward": _binding.backward_mode(),
+                       "nnz": self.nnz, "index_bytes_forward": i_fwd,
+                       "index_bytes_backward": i_bwd, "backward": _binding.backward_mode(),
                        "forward_bytes": self.fwd_bytes, "backward_bytes": self.bwd_bytes,
-                       "bytes_per_step_with_int64_forward": sum(_spmv_bytes(rows, cols, self.nnz, s, 8)),
+                       "bytes_per_step_with_int64_structure": sum(_spmv_bytes(rows, cols, self.nnz, s, 8, 8)),
+                       "bytes_per_step_with_int32_structure": sum(_spmv_bytes(rows, cols, self.nnz, s, 4, 8, planned=True)),
                        "binding": _binding.name,
                        "algorithmic_bytes_per_step": self.bytes_per_step}
 
@@ -208,12 +236,16 @@ class SpMV(Workload):
             _binding.set_backward_mode(mode)
         build = max(self.first_backward_ms) - rec["roofline"]["avg_ms"]
         gain = stateless - rec["ms_per_step"]
-        i8 = rec["config"]["bytes_per_step_with_int64_forward"] / (rec["ms_per_step"] * 1e-3) / 1e9
-        rec["config"]["GBps_on_int64_forward_model"] = round(i8, 1)
-        rec["config"]["pct_of_hbm_peak_on_int64_forward_model"] = round(100.0 * i8 / HBM_PEAK_GBS, 2)
+        # the same steps priced on the structure as the interface delivers it (int64) and on the
+        # plan's plain 32-bit structure (int32 columns forward, two int32 per entry backward: the
+        # model of earlier records); `value` prices every array at the width the kernels read
+        for key in ("int64", "int32"):
+            gbs = rec["config"][f"bytes_per_step_with_{key}_structure"] / (rec["ms_per_step"] * 1e-3) / 1e9
+            rec["config"][f"GBps_on_{key}_structure_model"] = round(gbs, 1)
+            rec["config"][f"pct_of_hbm_peak_on_{key}_structure_model"] = round(100.0 * gbs / HBM_PEAK_GBS, 2)
         rec["config"]["stateless_ms_per_step"] = round(stateless, 5)
         rec["config"]["stateless_GBps_int64_structure"] = round(
-            rec["config"]["bytes_per_step_with_int64_forward"] / (stateless * 1e-3) / 1e9, 1)
+            rec["config"]["bytes_per_step_with_int64_structure"] / (stateless * 1e-3) / 1e9, 1)
         rec["config"]["plan_build_ms"] = round(build, 3)
         rec["config"]["plan_break_even_steps"] = int(np.ceil(build / gain)) if gain > 0 else None
         rec["config"]["amortised_ms_per_step_over_100_steps"] = round(rec["ms_per_step"] + build / 100, 5)

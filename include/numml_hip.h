@@ -116,7 +116,9 @@ int nm_csr_transpose_backward(nm_dtype dt, int64_t nnz, const void *grad_At,
 /* nm_spgemv_forward for a pattern whose transposed-structure plan has been
  * built: the kernel reads the plan's 32-bit copies of A's column indices and
  * row pointers instead of the int64 arrays (4 instead of 8 index bytes per
- * entry); same sums in the same order, so y is bit-identical. */
+ * entry), and where every entry lies within 32 767 columns of its block of 512
+ * rows (banded matrices) the plan's 16-bit column offsets (2 bytes per entry);
+ * same sums in the same order, so y is bit-identical. */
 int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
                               const void *data, const void *plan_mem,
                               const void *x, void *y, nm_stream stream);
@@ -124,11 +126,19 @@ int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
 /* nm_spgemv_backward on a transposed-structure plan: walks A by column, so
  * grad_x needs neither clearing nor atomics, is summed in ascending row order
  * (the order of cpp/sparse_csr_cpu.cpp:68-73) and is identical on every run.
- * Either output may be NULL. */
+ * Either output may be NULL.  Banded patterns are walked on one packed word
+ * per entry (the plan's t_pack) in place of two 32-bit indices; arrays below
+ * 4 GiB are addressed with 32-bit offsets. */
 int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
                                const void *data, const void *plan_mem,
                                const void *x, const void *g,
                                void *grad_A, void *grad_x, nm_stream stream);
+
+/* Test hook (no counterpart in the reference): `wide_offsets` = 1 makes
+ * nm_spgemv_backward_planned address its arrays with 64-bit offsets whatever
+ * their size -- the variant that arrays of 4 GiB and more take -- so that it
+ * can be run on small inputs; 0 restores the choice by size.  Process-wide. */
+int nm_spgemv_configure(int wide_offsets);
 
 /* ------------------------------------------------------------------ SpMM
  * C = A B with dense row-major B (cols x n, row stride ldb elements) and

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "nm_sptrsv_solve_bytes": [_c_i64, _c_i64, ctypes.POINTER(_c_size)],
     "nm_sptrsv_solve": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr],
     "nm_sptrsv_configure": [_c_i64, _c_int],
+    "nm_spgemv_configure": [_c_int],
     "nm_sptrsv_solve_static_capacity": [ctypes.POINTER(_c_size)],
     "nm_sptrsv_solve_static": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "nm_csr_transpose_forward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,

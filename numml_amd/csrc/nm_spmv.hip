@@ -13,6 +13,8 @@
 // Algorithmic HBM bytes, s = sizeof(value):
 //   forward : nnz*(s+8) + (rows+1)*8 + cols*s + rows*s
 //   backward: nnz*(s+8) + (rows+1)*8 + rows*s + cols*s + nnz*s + cols*s
+#include <algorithm>
+#include <atomic>
 #include <type_traits>
 
 #include "nm_common.hpp"
@@ -97,7 +99,7 @@ inline int block_rows(int64_t rows, int64_t nnz, int most, int cap) {
 // largest e in [s0, nr] with at most cap entries in rows [s0, e); e == s0 when row s0
 // alone is longer.
 __device__ __forceinline__ int run_end(const int32_t *s_off, int s0, int nr, int cap) {
-    const int32_t limit = s_off[s0] + cap;
+    const int64_t limit = (int64_t)s_off[s0] + cap;
     if (s_off[nr] <= limit) return nr;
     int lo = s0, hi = nr;
     while (hi - lo > 1) {
@@ -107,6 +109,17 @@ __device__ __forceinline__ int run_end(const int32_t *s_off, int s0, int nr, int
     return lo;
 }
 
+// Element idx of an array.  O32: the array is smaller than 4 GiB, so the address is the base (in
+// scalar registers) plus a 32-bit byte offset (one vector register instead of two per access).
+template <bool O32, typename X>
+__device__ __forceinline__ X *at(X *base, int32_t idx) {
+    if (O32) {
+        using C = std::conditional_t<std::is_const<X>::value, const char, char>;
+        return reinterpret_cast<X *>(reinterpret_cast<C *>(base) + (uint32_t)idx * (uint32_t)sizeof(X));
+    }
+    return base + idx;
+}
+
 // UNIT: x is taken as all ones and not read, which makes y the row sums
 // (cpp/sparse_csr_cpu.cpp:1121-1127); a * 1 == a exactly, so the summation is
 // the same storage-order sum.
@@ -114,14 +127,18 @@ __device__ __forceinline__ int run_end(const int32_t *s_off, int s0, int nr, int
 // IDX: int64_t for the structure arrays as the interface delivers them, int32_t for the
 // 32-bit copies a transposed-structure plan of the same pattern holds.
 template <typename T, int BLOCK, int R, int CAP, bool UNIT = false, typename IDX = int64_t>
-__global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_num_sgpr(72))) void spmv_fwd_kernel(
     int64_t rows, int rt, const T *__restrict__ data, const IDX *__restrict__ indices,
-    const IDX *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y) {
+    const IDX *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y,
+    const int16_t *__restrict__ off16 = nullptr, const int32_t *__restrict__ flags = nullptr) {
     // rt <= R: rows per block of this launch (block_rows)
     __shared__ int32_t s_off[R + 1];
     __shared__ T s_prod[CAP];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // off16: columns as 16-bit offsets from the first row of a block of nm::kPackRows rows (a plan's
+    // c_off16, valid when its flags[2] is set); read when a workgroup's rows are exactly such a block
+    const bool packed = sizeof(IDX) == 4 && !UNIT && off16 != nullptr && rt == nm::kPackRows && flags[2] != 0;
 
     const int64_t ntiles = (rows + rt - 1) / rt, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
@@ -140,31 +157,43 @@ __global__ __launch_bounds__(BLOCK) void spmv_fwd_kernel(
             // does), two requests in flight
             typedef T TV __attribute__((ext_vector_type(4), aligned(sizeof(T))));
             typedef IDX IV __attribute__((ext_vector_type(4), aligned(sizeof(IDX))));
+            typedef int16_t SV __attribute__((ext_vector_type(4), aligned(2)));
             const T *__restrict__ d = data + base;
             const IDX *__restrict__ ci = indices + base;
+            const int16_t *__restrict__ co = off16 ? off16 + base : nullptr;
             const int n4 = n & ~3;
             constexpr int U = NM_FWD32_VEC_U;
-            for (int k0 = threadIdx.x * 4; k0 < n4; k0 += U * 4 * BLOCK) {
-                TV aa[U];
-                IV cc[U];
-                T xx[U][4];
+            auto walk = [&](auto pk) {
+                constexpr bool PACKED = decltype(pk)::value;
+                for (int k0 = threadIdx.x * 4; k0 < n4; k0 += U * 4 * BLOCK) {
+                    TV aa[U];
+                    IV cc[U];
+                    T xx[U][4];
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int kc = k0 + u * 4 * BLOCK < n4 ? k0 + u * 4 * BLOCK : n4 - 4;
-                    aa[u] = __builtin_nontemporal_load(reinterpret_cast<const TV *>(d + kc));
-                    cc[u] = __builtin_nontemporal_load(reinterpret_cast<const IV *>(ci + kc));
-                }
+                    for (int u = 0; u < U; ++u) {
+                        const int kc = k0 + u * 4 * BLOCK < n4 ? k0 + u * 4 * BLOCK : n4 - 4;
+                        aa[u] = __builtin_nontemporal_load(reinterpret_cast<const TV *>(d + kc));
+                        if (PACKED) {
+                            const SV o = __builtin_nontemporal_load(reinterpret_cast<const SV *>(co + kc));
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) xx[u][q] = x[cc[u][q]];
-#pragma unroll
-                for (int u = 0; u < U; ++u)
-                    if (k0 + u * 4 * BLOCK < n4) {
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) s_prod[k0 + u * 4 * BLOCK + q] = aa[u][q] * xx[u][q];
+                            for (int q = 0; q < 4; ++q) cc[u][q] = (IDX)r0 + o[q];
+                        } else {
+                            cc[u] = __builtin_nontemporal_load(reinterpret_cast<const IV *>(ci + kc));
+                        }
                     }
-            }
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) xx[u][q] = x[cc[u][q]];
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        if (k0 + u * 4 * BLOCK < n4) {
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) s_prod[k0 + u * 4 * BLOCK + q] = aa[u][q] * xx[u][q];
+                        }
+                }
+            };
+            if (packed) walk(std::true_type{}); else walk(std::false_type{});
             for (int k = n4 + threadIdx.x; k < n; k += BLOCK) s_prod[k] = d[k] * x[ci[k]];
             __syncthreads();
             for (int t = threadIdx.x; t < nr; t += BLOCK) {
@@ -425,41 +454,62 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
 // pattern is symmetric (plan flag) the column-major entry p is the mirror of the
 // row-major entry p = (row c, column r), so the lane writes
 // grad_A[p] = g[c] * x[r] instead: a coalesced store, every entry once.
-template <typename T, int R, int CAP>
+template <typename T, int R, int CAP, bool O32>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 8 : 7))) void spmv_bwd_planned_kernel(
     int64_t cols, const T *__restrict__ data, const int32_t *__restrict__ t_indptr,
-    const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm,
+    const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm, const int32_t *__restrict__ t_pack,
     const int32_t *__restrict__ flags, const T *__restrict__ x, const T *__restrict__ g,
     T *__restrict__ grad_A, T *__restrict__ grad_x) {
+    static_assert(R == nm::kPackCols, "t_pack holds rows relative to the first column of a workgroup's block");
     __shared__ int32_t s_off[R + 1];
     __shared__ __align__(16) T s_v[CAP];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const bool mirror = flags[0] != 0;
+    // one packed word per entry in place of (t_row, t_perm): patterns near the diagonal
+    const bool packed = flags[1] != 0;
+    static_assert(R == kBlock, "lane t of a workgroup stages column t of its block");
     const int64_t ntiles = (cols + R - 1) / R, npad = nm::xcd_padded(ntiles);
+    const bool fused = mirror && grad_A && grad_x;
+    // the factor a column's entries share: g[column] (symmetric pattern: the lane writes the mirror
+    // entry) or x[column]
+    const T *__restrict__ own_of = grad_A ? (mirror ? g : x) : nullptr;
+    const int tid = threadIdx.x;
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
         const int64_t tile = nm::xcd_tile_reversed(id, npad);
         if (tile >= ntiles) continue;
         const int64_t c0 = tile * R;
         const int nc = (int)(cols - c0 < R ? cols - c0 : R);
-        const int32_t base = t_indptr[c0];
-        for (int t = threadIdx.x; t <= nc; t += kBlock) {
-            const int32_t d = t_indptr[c0 + t] - base;
-            s_off[t] = d > kHuge ? kHuge : d;
-        }
+        // Lane t holds the bounds of column c0 + t and its own factor; all three loads leave
+        // together (one memory round trip before the tile's entries can be read).
+        const int32_t my_a = *at<O32>(t_indptr, (int32_t)c0 + (tid < nc ? tid : nc));
+        const int32_t my_b = *at<O32>(t_indptr, (int32_t)c0 + (tid + 1 < nc ? tid + 1 : nc));
+        const T my_own = own_of ? *at<O32>(own_of, (int32_t)c0 + (tid < nc ? tid : nc - 1)) : T(0);
+        // s_off[t] = first entry of column c0 + t in the plan (an absolute position), t = 0 .. nc
+        s_off[tid] = my_a;
+        if (tid == nc - 1) s_off[nc] = my_b;
         __syncthreads();
-        const int n = s_off[nc];
-        const bool fused = mirror && grad_A && grad_x;
+        const int32_t base = s_off[0];
+        const int n = s_off[nc] - base;
 
         // s_v[j] = own[column] for the entries j of columns [s0, e0); o0 = offset of column s0.
         // WHOLE (the tile fits): one lane per column.  Otherwise columns of kLongRow entries
         // or more are spread by a wavefront.
-        auto spread = [&](auto whole, const T *__restrict__ own, const int s0, const int e0, const int o0) {
+        auto spread = [&](auto whole, const T *__restrict__ own, const int s0, const int e0, const int32_t o0) {
             constexpr bool WHOLE = decltype(whole)::value;
             for (int tb = s0; tb < e0; tb += kBlock) {
                 const int t = tb + threadIdx.x;
-                const int jb = t < e0 ? s_off[t] - o0 : 0, je = t < e0 ? s_off[t + 1] - o0 : 0;
-                const T v = t < e0 ? own[c0 + t] : T(0);
+                int jb, je;
+                T v;
+                if (WHOLE) {    // s0 == 0, e0 == nc <= kBlock: one pass, lane = column, all in registers
+                    jb = t < e0 ? my_a - o0 : 0;
+                    je = t < e0 ? my_b - o0 : 0;
+                    v = my_own;
+                } else {
+                    jb = t < e0 ? s_off[t] - o0 : 0;
+                    je = t < e0 ? s_off[t + 1] - o0 : 0;
+                    v = t < e0 ? own[c0 + t] : T(0);
+                }
                 const bool wide = !WHOLE && je - jb >= kLongRow;
                 if (!wide)
                     for (int j = jb; j < je; ++j) s_v[j] = v;
@@ -474,11 +524,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
         };
         // grad_x[column] = sum of the column's slice of s_v: in storage order by one lane, or
         // (not WHOLE, kLongRow entries or more) lane l of a wavefront adds entries l, l + 64, ...
-        auto sums = [&](auto whole, const int s0, const int e0, const int o0) {
+        auto sums = [&](auto whole, const int s0, const int e0, const int32_t o0) {
             constexpr bool WHOLE = decltype(whole)::value;
             for (int tb = s0; tb < e0; tb += kBlock) {
                 const int t = tb + threadIdx.x;
-                const int jb = t < e0 ? s_off[t] - o0 : 0, je = t < e0 ? s_off[t + 1] - o0 : 0;
+                const int jb = t < e0 ? (WHOLE ? my_a : s_off[t]) - o0 : 0;
+                const int je = t < e0 ? (WHOLE ? my_b : s_off[t + 1]) - o0 : 0;
                 const bool wide = !WHOLE && je - jb >= kLongRow;
                 if (t < e0 && !wide) {
                     T acc = 0;
@@ -553,27 +604,38 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
                 }
                 return;
             }
-            constexpr int K = NM_BWD_K;
+            // (one entry fewer where every address takes a register pair, or the lanes spill)
+            constexpr int K = O32 ? NM_BWD_K : NM_BWD_K - 1;
             for (int p0 = threadIdx.x; p0 < cnt; p0 += K * kBlock) {
                 int32_t kk[K], rr[K];
                 T gg[K], xx[K], dd[K];
+                if (packed) {
 #pragma unroll
-                for (int u = 0; u < K; ++u) {
-                    const int pc = p0 + u * kBlock < cnt ? p0 + u * kBlock : cnt - 1;
-                    kk[u] = nm::stream_load(tp + pc);
-                    rr[u] = nm::stream_load(tr + pc);
+                    for (int u = 0; u < K; ++u) {
+                        const int pc = p0 + u * kBlock < cnt ? p0 + u * kBlock : cnt - 1;
+                        const int32_t w = nm::stream_load(at<O32>(t_pack, first + pc));
+                        kk[u] = first + pc + (w >> 16);
+                        rr[u] = (int32_t)c0 + (int16_t)w;
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < K; ++u) {
+                        const int pc = p0 + u * kBlock < cnt ? p0 + u * kBlock : cnt - 1;
+                        kk[u] = nm::stream_load(at<O32>(t_perm, first + pc));
+                        rr[u] = nm::stream_load(at<O32>(t_row, first + pc));
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < K; ++u) {
-                    gg[u] = g[rr[u]];
-                    xx[u] = x[rr[u]];
-                    dd[u] = data[kk[u]];
+                    gg[u] = *at<O32>(g, rr[u]);
+                    xx[u] = *at<O32>(x, rr[u]);
+                    dd[u] = *at<O32>(data, kk[u]);
                 }
                 if (p0 + (K - 1) * kBlock < cnt) {
 #pragma unroll
                     for (int u = 0; u < K; ++u) {
                         const int p = p0 + u * kBlock;
-                        ga[p] = s_v[p] * xx[u];
+                        *at<O32>(grad_A, first + p) = s_v[p] * xx[u];
                         s_v[p] = gg[u] * dd[u];
                     }
                 } else {
@@ -581,7 +643,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
                     for (int u = 0; u < K; ++u) {
                         const int p = p0 + u * kBlock;
                         if (p < cnt) {
-                            ga[p] = s_v[p] * xx[u];
+                            *at<O32>(grad_A, first + p) = s_v[p] * xx[u];
                             s_v[p] = gg[u] * dd[u];
                         }
                     }
@@ -593,8 +655,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
             const int32_t *__restrict__ tr = t_row + first;
             const int32_t *__restrict__ tp = t_perm + first;
             for (int p = threadIdx.x; p < cnt; p += kBlock) {
-                const int32_t k = nm::stream_load(tp + p);
-                const int32_t r = nm::stream_load(tr + p);
+                int32_t k, r;
+                if (packed) {
+                    const int32_t w = nm::stream_load(t_pack + first + p);
+                    k = first + p + (w >> 16);
+                    r = (int32_t)c0 + (int16_t)w;
+                } else {
+                    k = nm::stream_load(tp + p);
+                    r = nm::stream_load(tr + p);
+                }
                 const T gr = g[r];
                 if (grad_A) {
                     if (mirror) grad_A[first + p] = s_v[p] * x[r];
@@ -606,18 +675,18 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
         // columns [s0, e0) through LDS
         auto run = [&](auto whole, const int s0, const int e0) {
             constexpr bool WHOLE = decltype(whole)::value;
-            const int o0 = WHOLE ? 0 : s_off[s0];
+            const int32_t o0 = WHOLE ? base : s_off[s0];
             const int cnt = s_off[e0] - o0;
             if (fused) {
                 spread(whole, g, s0, e0, o0);
                 __syncthreads();
-                entries_fused(base + o0, cnt);
+                entries_fused(o0, cnt);
             } else {
                 if (grad_A) {
-                    spread(whole, mirror ? g : x, s0, e0, o0);
+                    spread(whole, own_of, s0, e0, o0);
                     __syncthreads();
                 }
-                entries_any(base + o0, cnt);
+                entries_any(o0, cnt);
             }
             if (grad_x) {
                 __syncthreads();
@@ -638,9 +707,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
                 }
                 // a column longer than the tile, CAP entries at a time; wavefront 0 keeps the
                 // lanes' partial sums (CAP is a multiple of 64: entry p stays with lane p % 64)
-                const int32_t first = base + s_off[s0];
+                const int32_t first = s_off[s0];
                 const int len = s_off[s0 + 1] - s_off[s0];
-                const T own = grad_A ? (mirror ? g : x)[c0 + s0] : T(0);
+                const T own = grad_A ? own_of[c0 + s0] : T(0);
                 T acc = 0;
                 for (int q0 = 0; q0 < len; q0 += CAP) {
                     const int cnt = len - q0 < CAP ? len - q0 : CAP;
@@ -695,6 +764,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
     }
 }
 
+// set by nm_spgemv_configure: 64-bit offsets in the planned backward whatever the sizes (tests)
+std::atomic<bool> g_wide_offsets{false};
+
 int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const int64_t *indices,
               const int64_t *indptr) {
     NM_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0, "negative size (rows=%lld cols=%lld nnz=%lld)",
@@ -706,13 +778,13 @@ int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const i
 
 template <typename T, typename IDX>
 int launch_fwd(int64_t rows, int64_t nnz, const T *data, const IDX *indices, const IDX *indptr, const T *x,
-               T *y, hipStream_t s) {
+               T *y, hipStream_t s, const int16_t *off16 = nullptr, const int32_t *flags = nullptr) {
     constexpr int R = kFwdR, CAP = kFwdCap;
     const int rt = block_rows(rows, nnz, R, CAP);
     int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, false, IDX>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s,
-                       rows, rt, data, indices, indptr, x, y);
+                       rows, rt, data, indices, indptr, x, y, off16, flags);
     NM_LAUNCH_CHECK("spmv_fwd_kernel");
     return NM_OK;
 }
@@ -724,7 +796,8 @@ int launch_row_sum(int64_t rows, int64_t nnz, const T *data, const int64_t *indp
     int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, true>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows,
-                       rt, data, (const int64_t *)nullptr, indptr, (const T *)nullptr, y);
+                       rt, data, (const int64_t *)nullptr, indptr, (const T *)nullptr, y, (const int16_t *)nullptr,
+                       (const int32_t *)nullptr);
     NM_LAUNCH_CHECK("spmv_fwd_kernel<unit>");
     return NM_OK;
 }
@@ -775,9 +848,9 @@ extern "C" int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
         return launch_fwd<float, int32_t>(rows, nnz, (const float *)data, t.c_idx32, t.c_ptr32, (const float *)x,
-                                          (float *)y, s);
+                                          (float *)y, s, t.c_off16, t.flags);
     return launch_fwd<double, int32_t>(rows, nnz, (const double *)data, t.c_idx32, t.c_ptr32, (const double *)x,
-                                       (double *)y, s);
+                                       (double *)y, s, t.c_off16, t.flags);
 }
 
 extern "C" int nm_csr_row_sum_forward(nm_dtype dt, int64_t rows, int64_t nnz, const void *data,
@@ -826,6 +899,11 @@ extern "C" int nm_masked_outer(nm_dtype dt, int64_t rows, int64_t nnz, const int
                               (double *)out, nullptr, s);
 }
 
+extern "C" int nm_spgemv_configure(int wide_offsets) {
+    g_wide_offsets.store(wide_offsets != 0, std::memory_order_relaxed);
+    return NM_OK;
+}
+
 extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
                                           const void *plan_mem, const void *x, const void *g, void *grad_A,
                                           void *grad_x, nm_stream stream) {
@@ -836,20 +914,33 @@ extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t col
     nm::TPlan t;
     nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
     hipStream_t s = nm::as_stream(stream);
+    // every array the kernel indexes stays below 4 GiB: 32-bit byte offsets
+    const int64_t longest = std::max(std::max(rows, cols) + 2, nnz + 1);
+    const bool o32 = !g_wide_offsets.load(std::memory_order_relaxed) && longest * (dt == NM_F32 ? 4 : 8) < (int64_t(1) << 32);
     if (dt == NM_F32) {
         constexpr int R = kPlannedR, CAP = kPlannedCap;
         int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
         if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-        hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                           (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.flags, (const float *)x, (const float *)g,
-                           (float *)grad_A, (float *)grad_x);
+        if (o32)
+            hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
+                               (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const float *)x,
+                               (const float *)g, (float *)grad_A, (float *)grad_x);
+        else
+            hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
+                               (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const float *)x,
+                               (const float *)g, (float *)grad_A, (float *)grad_x);
     } else {
         constexpr int R = kPlannedR, CAP = kPlannedCap;
         int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
         if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-        hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                           (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.flags, (const double *)x,
-                           (const double *)g, (double *)grad_A, (double *)grad_x);
+        if (o32)
+            hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
+                               (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const double *)x,
+                               (const double *)g, (double *)grad_A, (double *)grad_x);
+        else
+            hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
+                               (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const double *)x,
+                               (const double *)g, (double *)grad_A, (double *)grad_x);
     }
     NM_LAUNCH_CHECK("spmv_bwd_planned_kernel");
     return NM_OK;

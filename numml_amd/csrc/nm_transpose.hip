@@ -257,7 +257,44 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
 }
 
 __global__ void symmetry_init_kernel(int32_t *flags, int square) {
-    if (threadIdx.x == 0) flags[0] = square;
+    if (threadIdx.x == 0) {
+        flags[0] = square;
+        flags[1] = 1;
+        flags[2] = 1;
+    }
+}
+
+// t_pack and c_off16 of the plan; clears flags[1] / flags[2] when a difference does not fit 16 bits.
+// A workgroup takes blocks of kPackCols columns, then blocks of kPackRows rows, lane = entry.
+__global__ __launch_bounds__(kBlock) void tp_pack_kernel(
+    int64_t rows, int64_t cols, const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_row,
+    const int32_t *__restrict__ t_perm, const int32_t *__restrict__ c_ptr32, const int32_t *__restrict__ c_idx32,
+    int32_t *__restrict__ t_pack, int16_t *__restrict__ c_off16, int32_t *flags) {
+    bool fits_t = true, fits_c = true;
+    const int64_t cblocks = (cols + nm::kPackCols - 1) / nm::kPackCols;
+    for (int64_t b = blockIdx.x; b < cblocks; b += gridDim.x) {
+        const int64_t c0 = b * nm::kPackCols;
+        const int64_t c1 = c0 + nm::kPackCols < cols ? c0 + nm::kPackCols : cols;
+        const int32_t pe = t_indptr[c1];
+        for (int32_t p = t_indptr[c0] + (int32_t)threadIdx.x; p < pe; p += kBlock) {
+            const int64_t dr = (int64_t)t_row[p] - c0, dk = (int64_t)t_perm[p] - p;
+            fits_t &= dr >= -32768 && dr <= 32767 && dk >= -32768 && dk <= 32767;
+            t_pack[p] = (int32_t)(((uint32_t)dr & 0xffffu) | ((uint32_t)dk << 16));
+        }
+    }
+    const int64_t rblocks = (rows + nm::kPackRows - 1) / nm::kPackRows;
+    for (int64_t b = blockIdx.x; b < rblocks; b += gridDim.x) {
+        const int64_t r0 = b * nm::kPackRows;
+        const int64_t r1 = r0 + nm::kPackRows < rows ? r0 + nm::kPackRows : rows;
+        const int32_t ke = c_ptr32[r1];
+        for (int32_t k = c_ptr32[r0] + (int32_t)threadIdx.x; k < ke; k += kBlock) {
+            const int64_t dc = (int64_t)c_idx32[k] - r0;
+            fits_c &= dc >= -32768 && dc <= 32767;
+            c_off16[k] = (int16_t)dc;
+        }
+    }
+    if (!fits_t) flags[1] = 0;
+    if (!fits_c) flags[2] = 0;
 }
 
 // Clears flags[0] unless A^T has exactly A's structure.
@@ -335,6 +372,13 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
                            plan.c_ptr32, plan.t_row, plan.t_indptr, plan.flags);
     }
     NM_LAUNCH_CHECK("symmetry check");
+    if (nnz > 0) {
+        int64_t grid = ceil_div(cols > rows ? cols : rows, (int64_t)kPackCols);
+        if (grid > 65536) grid = 65536;
+        hipLaunchKernelGGL(tp_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, cols, plan.t_indptr,
+                           plan.t_row, plan.t_perm, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.flags);
+        NM_LAUNCH_CHECK("tp_pack_kernel");
+    }
     return NM_OK;
 }
 

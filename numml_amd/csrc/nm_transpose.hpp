@@ -13,6 +13,14 @@
 //   c_ptr32[i]   row pointers of A in 32 bits                                   (rows + 1)
 //                (kernels that find a plan read these instead of the int64
 //                arrays the interface delivers: half the index traffic)
+//   t_pack[p]    t_row and t_perm of entry p in one word, for patterns whose entries lie near
+//                the diagonal: low 16 bits = t_row[p] minus the first column of the entry's
+//                block of kPackCols columns, high 16 bits = t_perm[p] - p, both signed.
+//                Valid when flags[1] != 0 (every difference fits)                (nnz)
+//   c_off16[k]   c_idx32[k] minus the first row of the entry's block of kPackRows rows, signed
+//                16 bits.  Valid when flags[2] != 0                              (nnz)
+//                (the SpMV kernels read these instead of the 32-bit arrays: half the index
+//                traffic again on banded matrices)
 //
 // Inside a column the entries keep A's row-major order (the sort is stable), so
 // rows ascend, exactly like the counting-sort transpose of the reference
@@ -31,7 +39,13 @@ struct TPlan {
     int32_t *flags;
     int32_t *c_idx32;
     int32_t *c_ptr32;
+    int32_t *t_pack;
+    int16_t *c_off16;
 };
+
+// Blocks the packed offsets are relative to: the columns one workgroup of the planned SpMV
+// backward owns, and the rows one workgroup of the forward owns when rows are short.
+constexpr int kPackCols = 256, kPackRows = 512;
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
@@ -50,7 +64,9 @@ inline size_t tplan_layout(int64_t rows, int64_t cols, int64_t nnz, void *base, 
     int32_t *f = (int32_t *)take(16 * 4);
     int32_t *ci = (int32_t *)take((size_t)(nnz + 1) * 4);
     int32_t *cp = (int32_t *)take((size_t)(rows + 2) * 4);
-    if (p) *p = TPlan{a, b, c, h, f, ci, cp};
+    int32_t *tw = (int32_t *)take((size_t)(nnz + 1) * 4);
+    int16_t *co = (int16_t *)take((size_t)(nnz + 8) * 2);
+    if (p) *p = TPlan{a, b, c, h, f, ci, cp, tw, co};
     return off;
 }
 

@@ -1,0 +1,122 @@
+"""SpMV on a transposed-structure plan, through the C ABI: the packed structure of banded
+patterns (one word per entry in the backward, 16-bit column offsets in the forward), patterns
+whose offsets do not fit it, and both ways of addressing (32-bit offsets for arrays below
+4 GiB, 64-bit ones beyond, forced here on small inputs).  Against the serial loops of
+cpp/sparse_csr_cpu.cpp:29-35 and :60-73.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import scipy.sparse as sps
+import torch
+
+import oracle
+from numml_amd import _lib
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as ext
+from util import assert_close, assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+
+def _csr(M, dtype):
+    M = sps.csr_matrix(M).astype(dtype)
+    M.sort_indices()
+    return M.data.copy(), M.indices.astype(np.int64), M.indptr.astype(np.int64), M.shape
+
+
+def _symmetric_band(n, offsets, seed, dtype):
+    rng = np.random.default_rng(seed)
+    diags = [rng.uniform(0.5, 1.5, n - abs(o)) for o in offsets]
+    return _csr(sps.diags(diags, offsets, shape=(n, n)), dtype)
+
+
+def _wide_rows(n, per_row, reach, seed, dtype):
+    """Symmetric pattern, about 2 * per_row entries in every row within `reach` of the diagonal."""
+    rng = np.random.default_rng(seed)
+    r = np.repeat(np.arange(n), per_row)
+    c = np.clip(r + rng.integers(-reach, reach + 1, r.size), 0, n - 1)
+    M = sps.coo_matrix((np.ones(r.size), (r, c)), shape=(n, n)).tocsr()
+    M = ((M + M.T) > 0).astype(np.float64)
+    M.data = rng.uniform(0.5, 1.5, M.nnz)
+    return _csr(M, dtype)
+
+
+def _cross(n, seed, dtype):
+    """A band plus one full row and one full column: a column (and a row) longer than a tile."""
+    rng = np.random.default_rng(seed)
+    M = sps.diags([np.ones(n - 1), np.ones(n), np.ones(n - 1)], [-1, 0, 1], shape=(n, n)).tolil()
+    M[n // 3, :] = 1.0
+    M[:, n // 3] = 1.0
+    M = M.tocsr()
+    M.data = rng.uniform(0.5, 1.5, M.nnz)
+    return _csr(M, dtype)
+
+
+def _cases(dtype):
+    # name, matrix, (backward packed, forward packed), sums in storage order throughout
+    yield "poisson64", G.poisson2d(64, dtype, jitter_seed=3), (1, 1), True
+    yield "tridiag5000", G.tridiag(5000, dtype), (1, 1), True
+    # an entry 40 000 columns from the diagonal: no 16-bit offset holds it
+    yield "far_band", _symmetric_band(50000, [-40000, -1, 0, 1, 40000], 4, dtype), (0, 0), True
+    # near the diagonal, but a row's mirror entries lie more than 32 767 positions away
+    yield "thick_band", _wide_rows(3000, 20, 1500, 5, dtype), (0, 1), False
+    yield "rectangular", G.random_csr(700, 300, 0.02, 5, dtype), (1, 1), True
+    yield "cross", _cross(6000, 6, dtype), (1, 1), False
+    yield "empty", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(6, np.int64), (5, 4)), None, True
+
+
+def _plan_flags(plan, rows, cols, nnz):
+    a = lambda v: (v + 255) & ~255
+    off = a((cols + 1) * 4) + 2 * a((nnz + 1) * 4) + a(((nnz + 63) // 64 + 1) * 4)
+    return plan.mem[off:off + 12].cpu().view(torch.int32).tolist()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_planned_spmv_packed_and_plain_structure(dev, dtype):
+    L = _lib.lib()
+    dt = 0 if dtype == np.float32 else 1
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    try:
+        for name, (d, i, p, (rows, cols)), packed, exact in _cases(dtype):
+            nnz = d.shape[0]
+            x, g = randn(1, cols, dtype), randn(2, rows, dtype)
+            y_ref = oracle.spgemv_forward(rows, cols, d, i, p, x)
+            gA_ref, gx_ref = oracle.spgemv_backward(g, rows, cols, d, i, p, x)
+            D, I, P, X, Gd = to_dev(dev, d, i, p, x, g)
+            plan = ext._TransposePlan(I, P, rows, cols, dev)
+            if packed is not None:
+                flags = _plan_flags(plan, rows, cols, nnz)
+                assert (flags[1], flags[2]) == packed, f"{name}: plan flags {flags}"
+            results = []
+            for wide in (0, 1):
+                assert L.nm_spgemv_configure(wide) == 0
+                y = torch.full((rows,), 7.0, dtype=D.dtype, device=dev)
+                gA = torch.full((nnz,), 7.0, dtype=D.dtype, device=dev)
+                gx = torch.full((cols,), 7.0, dtype=D.dtype, device=dev)
+                _lib.check(L.nm_spgemv_forward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(y),
+                                                       stream), "nm_spgemv_forward_planned")
+                _lib.check(L.nm_spgemv_backward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
+                                                        ptr(gA), ptr(gx), stream), "nm_spgemv_backward_planned")
+                same = assert_same if exact else assert_close
+                same(host(y), y_ref, f"{name} y (wide={wide})")
+                assert_same(host(gA), gA_ref, f"{name} grad_A (wide={wide})")
+                same(host(gx), gx_ref, f"{name} grad_x (wide={wide})")
+                # one gradient at a time: the walk that does not fuse the two
+                gA1 = torch.full((nnz,), 7.0, dtype=D.dtype, device=dev)
+                gx1 = torch.full((cols,), 7.0, dtype=D.dtype, device=dev)
+                _lib.check(L.nm_spgemv_backward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
+                                                        ptr(gA1), None, stream), "nm_spgemv_backward_planned")
+                _lib.check(L.nm_spgemv_backward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
+                                                        None, ptr(gx1), stream), "nm_spgemv_backward_planned")
+                assert_same(host(gA1), host(gA), f"{name} grad_A alone (wide={wide})")
+                assert_same(host(gx1), host(gx), f"{name} grad_x alone (wide={wide})")
+                results.append((host(y), host(gA), host(gx)))
+            for a, b, what in zip(results[0], results[1], ("y", "grad_A", "grad_x")):
+                assert_same(a, b, f"{name} {what}: 32-bit against 64-bit offsets")
+    finally:
+        assert L.nm_spgemv_configure(0) == 0
