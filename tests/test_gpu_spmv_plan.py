@@ -66,6 +66,11 @@ def _cases(dtype):
     yield "thick_band", _wide_rows(3000, 20, 1500, 5, dtype), (0, 1), False
     yield "rectangular", G.random_csr(700, 300, 0.02, 5, dtype), (1, 1), True
     yield "cross", _cross(6000, 6, dtype), (1, 1), False
+    # rows and columns of thousands of entries spread over 50 000 columns: the plain 32-bit arrays
+    # on every path of the kernels (runs of columns, columns longer than a tile)
+    yield "powerlaw50k", G.powerlaw(50000, 50000, target_nnz=400000, max_deg=6000, seed=9, dtype=dtype), (0, 0), False
+    yield "powerlaw50k_T", _csr(sps.csr_matrix(G.powerlaw(50000, 50000, target_nnz=400000, max_deg=6000, seed=10,
+                                                          dtype=dtype)[:3], shape=(50000, 50000)).T, dtype), (0, 0), False
     yield "empty", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(6, np.int64), (5, 4)), None, True
 
 
