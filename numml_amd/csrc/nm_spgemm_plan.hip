@@ -123,7 +123,9 @@ __global__ __launch_bounds__(kBlock) void plan_columns_kernel(int64_t cols, cons
         const int32_t other = __shfl_xor(far, off, kWave);
         far = far > other ? far : other;
     }
-    if ((threadIdx.x & (kWave - 1)) == 0 && far > 0) atomicMax(flag + 3, far);
+    // (only a wavefront that has something new to say: thousands of atomics on one word cost more
+    // than the rest of the kernel)
+    if ((threadIdx.x & (kWave - 1)) == 0 && far > *(volatile int32_t *)(flag + 3)) atomicMax(flag + 3, far);
 }
 
 // The column-major copies of cstart and dest (entry t of the transposed plan is entry t_perm[t]).
