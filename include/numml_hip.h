@@ -493,6 +493,33 @@ int nm_splincomb_backward(nm_dtype dt, int64_t rows,
                           const void *grad_C, const int64_t *C_indices, const int64_t *C_indptr,
                           void *grad_A, void *grad_B, nm_stream stream);
 
+/* The linear combination of two patterns that stay the same while the values
+ * change (no counterpart in the reference, which merges the rows again on every
+ * call).  nm_splincomb_plan_build records, for the pattern of C that
+ * nm_splincomb_numeric produced, which entry of A and of B lies at every entry
+ * of C and where every entry of A and of B lies in C (int32; patterns of 2^31
+ * entries or more are refused with NM_ERR_UNSUPPORTED).  On these maps
+ * nm_splincomb_numeric_planned fills C_data in one pass -- no symbolic phase, no
+ * read of nnz(C) by the host -- and nm_splincomb_backward_planned gathers the
+ * gradients; both produce the bits of the calls they replace.  The caller keeps
+ * C's pattern (it is the same for every call).  Either gradient may be NULL. */
+int nm_splincomb_plan_bytes(int64_t A_nnz, int64_t B_nnz, int64_t C_nnz, size_t *plan_bytes);
+
+int nm_splincomb_plan_build(int64_t rows, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                            const int64_t *A_indices, const int64_t *A_indptr,
+                            const int64_t *B_indices, const int64_t *B_indptr,
+                            const int64_t *C_indices, const int64_t *C_indptr,
+                            void *plan_mem, size_t plan_bytes, nm_stream stream);
+
+int nm_splincomb_numeric_planned(nm_dtype dt, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                                 double alpha, const void *A_data, double beta, const void *B_data,
+                                 const void *plan_mem, void *C_data, nm_stream stream);
+
+int nm_splincomb_backward_planned(nm_dtype dt, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                                  double alpha, double beta, const void *grad_C,
+                                  const void *plan_mem, void *grad_A, void *grad_B,
+                                  nm_stream stream);
+
 /* ------------------------------------------ dense copy, row sums, diagonal
  * dense[i, j] = data[k] on a zero background (row stride ld >= cols); stands in for
  * csr_to_dense_forward (cpp/sparse_csr_cpu.cpp:1052-1076).  The backward gathers

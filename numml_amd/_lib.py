@@ -81,6 +81,13 @@ _SIGNATURES = {
                              _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_splincomb_backward": [_c_int, _c_i64, _c_dbl, _c_ptr, _c_ptr, _c_dbl, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                               _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_splincomb_plan_bytes": [_c_i64, _c_i64, _c_i64, ctypes.POINTER(_c_size)],
+    "nm_splincomb_plan_build": [_c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                _c_size, _c_ptr],
+    "nm_splincomb_numeric_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_dbl, _c_ptr, _c_dbl, _c_ptr, _c_ptr, _c_ptr,
+                                     _c_ptr],
+    "nm_splincomb_backward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_dbl, _c_dbl, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                      _c_ptr],
     "nm_csr_to_dense_forward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "nm_csr_to_dense_backward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_csr_row_sum_forward": [_c_int, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr],

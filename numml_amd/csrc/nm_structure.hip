@@ -776,3 +776,200 @@ extern "C" int nm_splincomb_backward(nm_dtype dt, int64_t rows, double alpha, co
     }
     return NM_OK;
 }
+
+// ---- the linear combination on cached maps ---------------------------------------
+//
+// For two patterns that stay the same while the values change (A - B in every iteration of a
+// loop) the merge of the two rows is done once: the plan holds, all int32,
+//
+//   srcA[o], srcB[o]   the entry of A / of B at the coordinate of the o-th entry of C, -1 for none
+//   posA[k], posB[k]   the entry of C at the coordinate of the k-th entry of A / of B
+//
+// after which the forward is one pass over C (two map streams, two gathers that run forward
+// through the operands, one store) and each gradient one gather -- no symbolic phase, no read of
+// nnz(C) by the host, no search.  The values are formed as the merge forms them
+// (cpp/sparse_csr_cpu.cpp:431-468): alpha * a, beta * b, or the sum of the two.
+
+namespace {
+
+struct LcPlan {
+    int32_t *srcA, *srcB, *posA, *posB;
+};
+
+size_t lcplan_layout(int64_t A_nnz, int64_t B_nnz, int64_t C_nnz, void *base, LcPlan *p) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        void *q = base ? static_cast<char *>(base) + off : nullptr;
+        off += nm::align256(bytes);
+        return (int32_t *)q;
+    };
+    int32_t *sa = take((size_t)(C_nnz + 1) * 4), *sb = take((size_t)(C_nnz + 1) * 4);
+    int32_t *pa = take((size_t)(A_nnz + 1) * 4), *pb = take((size_t)(B_nnz + 1) * 4);
+    if (p) *p = LcPlan{sa, sb, pa, pb};
+    return off;
+}
+
+constexpr int kMapLanes = 8;   // lanes per row of the map build
+
+// Eight lanes per row: lane k takes entries k, k + 8, ... of the row of X and finds each one's
+// column in the row of C by bisection.
+__global__ __launch_bounds__(kBlock) void lincomb_map_kernel(int64_t rows, const int64_t *__restrict__ X_indices,
+                                                             const int64_t *__restrict__ X_indptr,
+                                                             const int64_t *__restrict__ C_indices,
+                                                             const int64_t *__restrict__ C_indptr,
+                                                             int32_t *__restrict__ src, int32_t *__restrict__ pos) {
+    const int k = threadIdx.x & (kMapLanes - 1);
+    const int64_t stride = (int64_t)gridDim.x * (kBlock / kMapLanes);
+    for (int64_t row = (int64_t)blockIdx.x * (kBlock / kMapLanes) + threadIdx.x / kMapLanes; row < rows;
+         row += stride) {
+        const int64_t xb = X_indptr[row], xe = X_indptr[row + 1];
+        const int64_t cs = C_indptr[row], ce = C_indptr[row + 1];
+        for (int64_t e = xb + k; e < xe; e += kMapLanes) {
+            const int64_t col = X_indices[e];
+            int64_t lo = cs, hi = ce;
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) >> 1;
+                if (C_indices[mid] < col) lo = mid + 1; else hi = mid;
+            }
+            const bool found = lo < ce && C_indices[lo] == col;   // always, when C is the union of the patterns
+            pos[e] = (int32_t)(found ? lo : (cs < ce ? cs : 0));
+            if (found) src[lo] = (int32_t)e;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lincomb_planned_kernel(int64_t C_nnz, T alpha, const T *__restrict__ A_data,
+                                                                 T beta, const T *__restrict__ B_data,
+                                                                 const int32_t *__restrict__ srcA,
+                                                                 const int32_t *__restrict__ srcB,
+                                                                 T *__restrict__ C_data) {
+    constexpr int K = 4;
+    const int64_t stride = (int64_t)gridDim.x * kBlock * K;
+    for (int64_t o0 = (int64_t)blockIdx.x * kBlock * K + threadIdx.x; o0 < C_nnz; o0 += stride) {
+        int32_t ia[K], ib[K];
+        T va[K], vb[K];
+#pragma unroll
+        for (int u = 0; u < K; ++u) {
+            const int64_t o = o0 + u * kBlock < C_nnz ? o0 + u * kBlock : C_nnz - 1;
+            ia[u] = nm::stream_load(srcA + o);
+            ib[u] = nm::stream_load(srcB + o);
+        }
+#pragma unroll
+        for (int u = 0; u < K; ++u) {
+            va[u] = ia[u] >= 0 ? A_data[ia[u]] : T(0);
+            vb[u] = ib[u] >= 0 ? B_data[ib[u]] : T(0);
+        }
+#pragma unroll
+        for (int u = 0; u < K; ++u) {
+            const int64_t o = o0 + u * kBlock;
+            if (o >= C_nnz) break;
+            const T pa = alpha * va[u], pb = beta * vb[u];
+            nm::stream_store(C_data + o, ib[u] < 0 ? pa : (ia[u] < 0 ? pb : pa + pb));
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lincomb_back_planned_kernel(int64_t X_nnz, T coef, const T *__restrict__ gC,
+                                                                      const int32_t *__restrict__ pos,
+                                                                      T *__restrict__ grad_X) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x; k < X_nnz; k += stride)
+        nm::stream_store(grad_X + k, coef * gC[nm::stream_load(pos + k)]);
+}
+
+unsigned flat_grid(int64_t n, int per_block) {
+    int64_t g = nm::ceil_div(n, (int64_t)per_block);
+    return (unsigned)(g > 65536 ? 65536 : (g < 1 ? 1 : g));
+}
+
+}  // namespace
+
+extern "C" int nm_splincomb_plan_bytes(int64_t A_nnz, int64_t B_nnz, int64_t C_nnz, size_t *plan_bytes) {
+    NM_REQUIRE(plan_bytes && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "bad argument");
+    *plan_bytes = lcplan_layout(A_nnz, B_nnz, C_nnz, nullptr, nullptr);
+    return NM_OK;
+}
+
+extern "C" int nm_splincomb_plan_build(int64_t rows, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                                       const int64_t *A_indices, const int64_t *A_indptr, const int64_t *B_indices,
+                                       const int64_t *B_indptr, const int64_t *C_indices, const int64_t *C_indptr,
+                                       void *plan_mem, size_t plan_bytes, nm_stream stream) {
+    NM_REQUIRE(rows >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
+    const int64_t lim = (int64_t)1 << 31;
+    if (A_nnz >= lim || B_nnz >= lim || C_nnz >= lim)
+        return nm::fail(NM_ERR_UNSUPPORTED, "the maps of a linear combination hold positions in 32 bits");
+    NM_REQUIRE(plan_mem && A_indptr && B_indptr && C_indptr, "null pointer argument");
+    NM_REQUIRE((A_nnz == 0 || A_indices) && (B_nnz == 0 || B_indices) && (C_nnz == 0 || C_indices),
+               "null pointer argument");
+    const size_t need = lcplan_layout(A_nnz, B_nnz, C_nnz, nullptr, nullptr);
+    if (plan_bytes < need) return nm::fail(NM_ERR_WORKSPACE, "plan of %zu bytes, %zu needed", plan_bytes, need);
+    LcPlan p;
+    lcplan_layout(A_nnz, B_nnz, C_nnz, plan_mem, &p);
+    hipStream_t s = nm::as_stream(stream);
+    if (int rc = nm::fill_async(p.srcA, C_nnz, (int32_t)-1, s)) return rc;
+    if (int rc = nm::fill_async(p.srcB, C_nnz, (int32_t)-1, s)) return rc;
+    if (rows == 0) return NM_OK;
+    const unsigned grid = flat_grid(rows, kBlock / kMapLanes);
+    if (A_nnz > 0) {
+        hipLaunchKernelGGL(lincomb_map_kernel, dim3(grid), dim3(kBlock), 0, s, rows, A_indices, A_indptr, C_indices,
+                           C_indptr, p.srcA, p.posA);
+        NM_LAUNCH_CHECK("lincomb_map_kernel");
+    }
+    if (B_nnz > 0) {
+        hipLaunchKernelGGL(lincomb_map_kernel, dim3(grid), dim3(kBlock), 0, s, rows, B_indices, B_indptr, C_indices,
+                           C_indptr, p.srcB, p.posB);
+        NM_LAUNCH_CHECK("lincomb_map_kernel");
+    }
+    return NM_OK;
+}
+
+extern "C" int nm_splincomb_numeric_planned(nm_dtype dt, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz, double alpha,
+                                            const void *A_data, double beta, const void *B_data,
+                                            const void *plan_mem, void *C_data, nm_stream stream) {
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "bad dtype %d", (int)dt);
+    NM_REQUIRE(A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
+    if (C_nnz == 0) return NM_OK;
+    NM_REQUIRE(plan_mem && C_data && (A_nnz == 0 || A_data) && (B_nnz == 0 || B_data), "null pointer argument");
+    LcPlan p;
+    lcplan_layout(A_nnz, B_nnz, C_nnz, const_cast<void *>(plan_mem), &p);
+    hipStream_t s = nm::as_stream(stream);
+    const unsigned grid = flat_grid(C_nnz, kBlock * 4);
+    if (dt == NM_F32)
+        hipLaunchKernelGGL(lincomb_planned_kernel<float>, dim3(grid), dim3(kBlock), 0, s, C_nnz, (float)alpha,
+                           (const float *)A_data, (float)beta, (const float *)B_data, p.srcA, p.srcB, (float *)C_data);
+    else
+        hipLaunchKernelGGL(lincomb_planned_kernel<double>, dim3(grid), dim3(kBlock), 0, s, C_nnz, alpha,
+                           (const double *)A_data, beta, (const double *)B_data, p.srcA, p.srcB, (double *)C_data);
+    NM_LAUNCH_CHECK("lincomb_planned_kernel");
+    return NM_OK;
+}
+
+extern "C" int nm_splincomb_backward_planned(nm_dtype dt, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz, double alpha,
+                                             double beta, const void *grad_C, const void *plan_mem, void *grad_A,
+                                             void *grad_B, nm_stream stream) {
+    NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "bad dtype %d", (int)dt);
+    NM_REQUIRE(A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
+    NM_REQUIRE(plan_mem != nullptr, "null plan");
+    LcPlan p;
+    lcplan_layout(A_nnz, B_nnz, C_nnz, const_cast<void *>(plan_mem), &p);
+    hipStream_t s = nm::as_stream(stream);
+    for (int side = 0; side < 2; ++side) {
+        void *out = side == 0 ? grad_A : grad_B;
+        const int64_t n = side == 0 ? A_nnz : B_nnz;
+        if (!out || n == 0) continue;
+        NM_REQUIRE(grad_C != nullptr, "grad_C is null");   // an operand with entries: C has entries
+        const int32_t *pos = side == 0 ? p.posA : p.posB;
+        const double coef = side == 0 ? alpha : beta;
+        const unsigned grid = flat_grid(n, kBlock);
+        if (dt == NM_F32)
+            hipLaunchKernelGGL(lincomb_back_planned_kernel<float>, dim3(grid), dim3(kBlock), 0, s, n, (float)coef,
+                               (const float *)grad_C, pos, (float *)out);
+        else
+            hipLaunchKernelGGL(lincomb_back_planned_kernel<double>, dim3(grid), dim3(kBlock), 0, s, n, coef,
+                               (const double *)grad_C, pos, (double *)out);
+        NM_LAUNCH_CHECK("lincomb_back_planned_kernel");
+    }
+    return NM_OK;
+}

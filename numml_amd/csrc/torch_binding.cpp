@@ -170,7 +170,8 @@ struct Alias {
 
 struct Plan {
     // 'T' transposed structure, 'L' level schedule, 'U' filled pattern of the LU factors,
-    // 'P' product plan of A B (key: A's pattern, key2: B's)
+    // 'P' product plan of A B (key: A's pattern, key2: B's), 'S' maps of a linear combination
+    // alpha A + beta B (key: A's pattern, key2: B's)
     char kind;
     Key key, key2;
     int64_t a, b;
@@ -429,14 +430,14 @@ void drop_plan(const std::shared_ptr<Plan> &plan) {
 // what a call may do before it knows whether the product is eligible at all).
 std::shared_ptr<Plan> peek_product_plan(const Tensor &A_indices, const Tensor &A_indptr, const Tensor &B_indices,
                                         const Tensor &B_indptr, int64_t A_rows, int64_t B_cols,
-                                        const c10::Device &dev, bool compute = false) {
+                                        const c10::Device &dev, bool compute = false, char kind = 'P') {
     Key ka, kb;
     if (!structure_key(A_indices, A_indptr, compute, &ka) || !structure_key(B_indices, B_indptr, compute, &kb))
         return nullptr;
     std::shared_ptr<Plan> plan;
     {
         std::lock_guard<std::mutex> lock(g_plans_mutex);
-        plan = find_plan_locked('P', ka, A_rows, B_cols, kb);
+        plan = find_plan_locked(kind, ka, A_rows, B_cols, kb);
     }
     if (!plan) return nullptr;
     for (size_t i = 0; i < plan->derived.size(); ++i)
@@ -520,6 +521,72 @@ void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, cons
     plan->ready = std::make_unique<at::cuda::CUDAEvent>();
     plan->ready->record(stream);
     plan->bytes = plan->mem.defined() ? (size_t)plan->mem.nbytes() : 0;
+    for (const Tensor &t : plan->derived) plan->bytes += (size_t)t.nbytes();
+    g_plans_built.fetch_add(1, std::memory_order_relaxed);
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    g_plans.push_front(plan);
+    g_plan_bytes += plan->bytes;
+    const size_t limit = g_plan_bytes_limit.load(std::memory_order_relaxed);
+    while (g_plans.size() > 1 && g_plan_bytes > limit) {
+        g_plan_bytes -= g_plans.back()->bytes;
+        g_plans.pop_back();
+    }
+}
+
+// After a stateless linear combination: notes the pair of patterns, or (second sighting; first in
+// eager mode) records the maps of the combination around the pattern of C just produced.
+void consider_sum_plan(const Tensor &A_indices, const Tensor &A_indptr, const Tensor &B_indices,
+                       const Tensor &B_indptr, const Tensor &C_indices, const Tensor &C_indptr, int64_t rows,
+                       int64_t cols, const c10::Device &dev) {
+    const int mode = backward_mode_now();
+    const int64_t lim = (int64_t)1 << 31;
+    if (mode == kAtomic || C_indices.numel() == 0 || A_indices.numel() >= lim || B_indices.numel() >= lim ||
+        C_indices.numel() >= lim)
+        return;
+    Key ka, kb;
+    structure_key(A_indices, A_indptr, true, &ka);
+    structure_key(B_indices, B_indptr, true, &kb);
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        if (find_plan_locked('S', ka, rows, cols, kb)) return;
+        if (mode == kPlanned) {
+            bool seen = false;
+            for (auto it = g_sightings.begin(); it != g_sightings.end(); ++it)
+                if (it->kind == 'S' && it->key == ka && it->key2 == kb && it->a == rows && it->b == cols) {
+                    g_sightings.erase(it);
+                    seen = true;
+                    break;
+                }
+            if (!seen) {
+                g_sightings.push_front(Sighting{'S', ka, kb, rows, cols});
+                while (g_sightings.size() > kSightingTableSize) g_sightings.pop_back();
+                return;
+            }
+        }
+    }
+    auto plan = std::make_shared<Plan>();
+    plan->kind = 'S';
+    plan->key = ka;
+    plan->key2 = kb;
+    plan->a = rows;
+    plan->b = cols;
+    size_t pbytes = 0;
+    check(nm_splincomb_plan_bytes(A_indices.numel(), B_indices.numel(), C_indices.numel(), &pbytes),
+          "nm_splincomb_plan_bytes");
+    plan->mem = scratch(pbytes, dev);
+    check(nm_splincomb_plan_build(rows, A_indices.numel(), B_indices.numel(), C_indices.numel(),
+                                  A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                  B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                                  C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(), plan->mem.data_ptr(),
+                                  pbytes, current_stream(dev)),
+          "nm_splincomb_plan_build");
+    plan->derived = {C_indices, C_indptr};
+    for (const Tensor &t : plan->derived) plan->derived_versions.push_back(t._version());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev.index());
+    plan->build_stream = stream.id();
+    plan->ready = std::make_unique<at::cuda::CUDAEvent>();
+    plan->ready->record(stream);
+    plan->bytes = (size_t)plan->mem.nbytes();
     for (const Tensor &t : plan->derived) plan->bytes += (size_t)t.nbytes();
     g_plans_built.fetch_add(1, std::memory_order_relaxed);
     std::lock_guard<std::mutex> lock(g_plans_mutex);
@@ -665,6 +732,18 @@ std::vector<Tensor> splincomb_forward(int rows, int cols, Tensor alpha, Tensor A
     // cpp/sparse_csr_cpu.cpp:413-414); they usually are host tensors already
     const double a = alpha.item<double>(), b = beta.item<double>();
     c10::hip::HIPGuard guard(dev.index());
+    if (backward_mode_now() != kAtomic) {
+        // patterns seen before (alias lookup only): one pass over the cached maps; the result shares
+        // the plan's pattern tensors, as a planned product does
+        if (auto plan = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, rows, cols, dev, false, 'S')) {
+            Tensor C_data = torch::empty({plan->derived[0].numel()}, A_data.options());
+            check(nm_splincomb_numeric_planned(dtype_of(A_data), A_indices.numel(), B_indices.numel(), C_data.numel(),
+                                               a, A_data.data_ptr(), b, B_data.data_ptr(), plan->mem.data_ptr(),
+                                               C_data.data_ptr(), current_stream(dev)),
+                  "nm_splincomb_numeric_planned");
+            return {C_data, plan->derived[0], plan->derived[1]};
+        }
+    }
     size_t bytes = 0;
     check(nm_splincomb_workspace_bytes(rows, &bytes), "nm_splincomb_workspace_bytes");
     Tensor work = scratch(bytes, dev);
@@ -683,6 +762,7 @@ std::vector<Tensor> splincomb_forward(int rows, int cols, Tensor alpha, Tensor A
                                B_indptr.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(),
                                C_indices.data_ptr<int64_t>(), C_data.data_ptr(), st),
           "nm_splincomb_numeric");
+    consider_sum_plan(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr, rows, cols, dev);
     return {C_data, C_indices, C_indptr};
 }
 
@@ -707,6 +787,18 @@ std::vector<Tensor> splincomb_backward(int rows, int cols, Tensor alpha, Tensor 
     c10::hip::HIPGuard guard(dev.index());
     Tensor grad_A = torch::empty_like(A_data, at::MemoryFormat::Contiguous);
     Tensor grad_B = torch::empty_like(B_data, at::MemoryFormat::Contiguous);
+    if (backward_mode_now() != kAtomic) {
+        // the maps belong to the pattern tensors the planned forward handed out: those very tensors
+        auto plan = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, rows, cols, dev, false, 'S');
+        if (plan && plan->derived[0].data_ptr() == C_indices.data_ptr() &&
+            plan->derived[1].data_ptr() == C_indptr.data_ptr() && plan->derived[0].numel() == C_indices.numel()) {
+            check(nm_splincomb_backward_planned(dtype_of(A_data), A_indices.numel(), B_indices.numel(),
+                                                C_indices.numel(), a, b, grad_C_data.data_ptr(), plan->mem.data_ptr(),
+                                                grad_A.data_ptr(), grad_B.data_ptr(), current_stream(dev)),
+                  "nm_splincomb_backward_planned");
+            return {grad_A, grad_B};
+        }
+    }
     check(nm_splincomb_backward(dtype_of(A_data), rows, a, A_indices.data_ptr<int64_t>(),
                                 A_indptr.data_ptr<int64_t>(), b, B_indices.data_ptr<int64_t>(),
                                 B_indptr.data_ptr<int64_t>(), grad_C_data.data_ptr(), C_indices.data_ptr<int64_t>(),

@@ -68,6 +68,58 @@ def test_splincomb_forward_backward(dev, ext, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mode", ["planned", "eager"])
+def test_splincomb_on_cached_maps(dev, dtype, mode):
+    # The same two patterns with new values and new coefficients in every call, as in a loop over
+    # A - B: the compiled binding records the maps of the combination (at the second sighting of the
+    # pair, at the first in eager mode) and then fills C in one pass and gathers the gradients; every
+    # call must give the bits of the serial merge (cpp/sparse_csr_cpu.cpp:387-560).
+    ext = numml_amd.load_compiled()
+    old = ext.backward_mode()
+    ext.set_backward_mode(mode)
+    try:
+        for name, (ad, ai, ap, (r, c)), (bd, bi, bp, _) in _pairs(dtype):
+            ext.clear_plan_cache()
+            ai, ap, bi, bp = (np.asarray(v, np.int64) for v in (ai, ap, bi, bp))
+            AI, AP, BI, BP = to_dev(dev, ai, ap, bi, bp)
+            shared = None
+            built0 = ext.plan_cache_stats()[0]
+            for it, (alpha, beta) in enumerate(((1.0, 1.0), (1.0, -1.0), (0.75, -2.5), (-0.5, 3.0))):
+                a_vals = (ad * (1 + it)).astype(dtype) + randn(20 + it, ad.shape[0], dtype)
+                b_vals = (bd * (2 - it)).astype(dtype) + randn(30 + it, bd.shape[0], dtype)
+                Cd_ref, Ci_ref, Cp_ref = oracle.splincomb_forward(r, c, alpha, a_vals, ai, ap, beta, b_vals, bi, bp)
+                AD, BD = to_dev(dev, a_vals, b_vals)
+                Cd, Ci, Cp = ext.splincomb_forward(r, c, torch.tensor(alpha), AD, AI, AP, torch.tensor(beta), BD, BI, BP)
+                assert_same(host(Cp), Cp_ref, f"{name} call {it} C_indptr")
+                assert_same(host(Ci), Ci_ref, f"{name} call {it} C_indices")
+                assert_same(host(Cd), Cd_ref, f"{name} call {it} C_data")
+                g = randn(3 + it, Cd_ref.shape[0], dtype)
+                gA, gB = ext.splincomb_backward(r, c, torch.tensor(alpha), AD, AI, AP, torch.tensor(beta), BD, BI, BP,
+                                                to_dev(dev, g)[0], Ci, Cp)
+                gA_ref, gB_ref = oracle.splincomb_backward(r, c, alpha, a_vals, ai, ap, beta, b_vals, bi, bp, g,
+                                                           Ci_ref, Cp_ref)
+                assert_same(host(gA), gA_ref, f"{name} call {it} grad_A")
+                assert_same(host(gB), gB_ref, f"{name} call {it} grad_B")
+                # a backward given a copy of the pattern (not the tensors the plan handed out) must
+                # not trust the maps' positions blindly: it searches, with the same result
+                gA2, gB2 = ext.splincomb_backward(r, c, torch.tensor(alpha), AD, AI, AP, torch.tensor(beta), BD, BI,
+                                                  BP, to_dev(dev, g)[0], Ci.clone(), Cp.clone())
+                assert_same(host(gA2), gA_ref, f"{name} call {it} grad_A on a copied pattern")
+                assert_same(host(gB2), gB_ref, f"{name} call {it} grad_B on a copied pattern")
+                first_planned = 2 if mode == "planned" else 1
+                if Cd_ref.shape[0] > 0 and it >= first_planned:
+                    # results on the maps share the plan's pattern tensors
+                    if shared is not None:
+                        assert Ci.data_ptr() == shared[0] and Cp.data_ptr() == shared[1], f"{name} call {it}"
+                    shared = (Ci.data_ptr(), Cp.data_ptr())
+            if Cd_ref.shape[0] > 0:
+                assert ext.plan_cache_stats()[0] - built0 == 1, f"{name}: one set of maps for the pair"
+    finally:
+        ext.set_backward_mode(old)
+        ext.clear_plan_cache()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_dense_rowsum_diagonal(dev, ext, dtype):
     cases = [("poisson", G.poisson2d(24, dtype, 1)), ("random", G.random_csr(130, 170, 0.07, 2, dtype)),
              ("tall", G.random_csr(400, 9, 0.3, 3, dtype)), ("one_dense_row", G.random_csr(3, 6000, 0.9, 4, dtype, empty_rows=False)),
