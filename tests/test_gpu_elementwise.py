@@ -119,6 +119,37 @@ def test_splincomb_on_cached_maps(dev, dtype, mode):
         ext.clear_plan_cache()
 
 
+def test_splincomb_maps_at_full_size(dev):
+    # the 2048 x 2048 Poisson pattern (4.2 M rows) against a shifted copy of itself: the pass over the
+    # cached maps and the gathering backward give the bits of the merging forward and the searching
+    # backward, and (A - B) + B has A's pattern again with values equal to rounding
+    ext = numml_amd.load_compiled()
+    old = ext.backward_mode()
+    d, i, p, (r, c) = G.poisson2d(2048, np.float32, jitter_seed=0)
+    d2 = G.poisson2d(2048, np.float32, jitter_seed=1)[0]
+    AD, BD, I, P = to_dev(dev, d, d2, i, p)
+    BI, BP = I.clone(), P.clone()
+    g = to_dev(dev, randn(4, d.shape[0], np.float32))[0]
+    one, mone = torch.tensor(1.0), torch.tensor(-1.0)
+    try:
+        ext.set_backward_mode("atomic")
+        ref = ext.splincomb_forward(r, c, one, AD, I, P, mone, BD, BI, BP)
+        gref = ext.splincomb_backward(r, c, one, AD, I, P, mone, BD, BI, BP, g, ref[1], ref[2])
+        ext.set_backward_mode("eager")
+        ext.clear_plan_cache()
+        ext.splincomb_forward(r, c, one, AD, I, P, mone, BD, BI, BP)          # records the maps
+        out = ext.splincomb_forward(r, c, one, AD, I, P, mone, BD, BI, BP)    # runs on them
+        gout = ext.splincomb_backward(r, c, one, AD, I, P, mone, BD, BI, BP, g, out[1], out[2])
+        for a, b, what in zip(out + gout, ref + gref, ("C_data", "C_indices", "C_indptr", "grad_A", "grad_B")):
+            assert torch.equal(a, b), what
+        back = ext.splincomb_forward(r, c, one, out[0], out[1], out[2], one, BD, BI, BP)
+        assert torch.equal(back[1], I) and torch.equal(back[2], P)
+        assert_close(host(back[0]), d, "(A - B) + B")
+    finally:
+        ext.set_backward_mode(old)
+        ext.clear_plan_cache()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_dense_rowsum_diagonal(dev, ext, dtype):
     cases = [("poisson", G.poisson2d(24, dtype, 1)), ("random", G.random_csr(130, 170, 0.07, 2, dtype)),
