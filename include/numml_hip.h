@@ -328,6 +328,29 @@ int nm_spgemm_backward_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64
                               const void *A_plan_mem, const void *B_data, const int64_t *B_indptr,
                               const void *plan_mem, void *grad_A, void *grad_B, nm_stream stream);
 
+/* Product plans for named rows of B of up to 16 or 32 entries (no counterpart in
+ * the reference): `octets` = 2 or 4 destination octets per entry of A instead of
+ * one.  nm_spgemm_plan_build reports in `usable` a NEGATIVE number -L when the
+ * only limit its one-octet plan misses is that the longest row of B that A names
+ * has L entries, 9 <= L <= 32: the caller then allocates
+ * nm_spgemm_plan_bytes_wide(A_nnz, L <= 16 ? 2 : 4) and calls
+ * nm_spgemm_plan_build_wide with that number of octets, which reports class 4
+ * (two octets) or 5 (four), to be handed to nm_spgemm_numeric_planned and
+ * nm_spgemm_backward_mapped_wide; with octets = 1 and classes 1 to 3 these are
+ * the calls above.  Same sums in the same order, bit for bit. */
+int nm_spgemm_plan_bytes_wide(int64_t A_nnz, int octets, size_t *plan_bytes);
+int nm_spgemm_plan_build_wide(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
+                              const int64_t *A_indices, const int64_t *A_indptr,
+                              const int64_t *B_indices, const int64_t *B_indptr,
+                              const int64_t *C_indices, const int64_t *C_indptr,
+                              const void *A_plan_mem, void *plan_mem, size_t plan_bytes, int octets,
+                              void *host_landing, int *usable, nm_stream stream);
+int nm_spgemm_backward_mapped_wide(nm_dtype dt, int plan_class, int64_t A_rows, int64_t A_cols,
+                                   int64_t A_nnz, int64_t B_nnz, int64_t C_nnz, const void *gC,
+                                   const void *A_data, const void *A_plan_mem, const void *B_data,
+                                   const int64_t *B_indptr, const void *plan_mem,
+                                   void *grad_A, void *grad_B, nm_stream stream);
+
 /* ---------------------------------------------------------------- SpTRSV
  * Level-scheduled triangular solve.  Stands in for sptrsv_forward /
  * sptrsv_backward (cpp/sparse_csr.hpp:94-105, cpp/sparse_csr_cpu.cpp:652-759).

@@ -63,6 +63,11 @@ _SIGNATURES = {
                                   _c_ptr, _c_ptr, _c_ptr],
     "nm_spgemm_backward_mapped": [_c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_spgemm_plan_bytes_wide": [_c_i64, _c_int, ctypes.POINTER(_c_size)],
+    "nm_spgemm_plan_build_wide": [_c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                  _c_ptr, _c_ptr, _c_ptr, _c_size, _c_int, _c_ptr, ctypes.POINTER(_c_int), _c_ptr],
+    "nm_spgemm_backward_mapped_wide": [_c_int, _c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr,
+                                       _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_sptrsv_plan_bytes": [_c_i64, _c_i64, ctypes.POINTER(_c_size), ctypes.POINTER(_c_size)],
     "nm_sptrsv_analyse": [_c_i64, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_size, _c_ptr, _c_size,
                           ctypes.POINTER(_c_ptr), _c_ptr],

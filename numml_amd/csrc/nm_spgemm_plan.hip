@@ -57,15 +57,16 @@ __device__ __forceinline__ void group_fence() { __builtin_amdgcn_fence(__ATOMIC_
 __global__ __launch_bounds__(kBlock) void plan_map_kernel(
     int64_t rows, const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
     const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
-    const int64_t *__restrict__ C_indices, const int64_t *__restrict__ C_indptr, PPlan p) {
+    const int64_t *__restrict__ C_indices, const int64_t *__restrict__ C_indptr, PPlan p, int octets) {
     const int k = threadIdx.x & (kCap - 1);
     const int64_t stride = (int64_t)gridDim.x * kGroupsPerBlock;
-    bool bad = false, long_a = false, wide_c = false;
+    bool bad = false, other = false, long_a = false, wide_c = false;
+    int32_t longest = 0;
     for (int64_t row = (int64_t)blockIdx.x * kGroupsPerBlock + threadIdx.x / kCap; row < rows; row += stride) {
         const int64_t ab = A_indptr[row], ae = A_indptr[row + 1];
         const int64_t cs = C_indptr[row], ce = C_indptr[row + 1];
         if (ce - cs > kWideCap) {
-            bad = true;
+            bad = other = true;
             continue;
         }
         if (ae - ab > kCap) long_a = true;
@@ -73,23 +74,26 @@ __global__ __launch_bounds__(kBlock) void plan_map_kernel(
         for (int64_t e = ab; e < ae; ++e) {
             const int64_t j = A_indices[e];
             const int64_t bb = B_indptr[j], blen = B_indptr[j + 1] - bb;
-            if (blen > kCap) {
+            longest = blen > longest ? (int32_t)(blen < 0x7fffffff ? blen : 0x7fffffff) : longest;
+            if (blen > kCap * octets) {
                 bad = true;
-                break;
+                continue;   // (the other rows are still looked at: the caller learns the longest)
             }
-            uint8_t d = kNone;
-            if (k < blen) {
-                const int64_t col = B_indices[bb + k];
-                int64_t lo = cs, hi = ce;
-                while (lo < hi) {
-                    const int64_t mid = (lo + hi) >> 1;
-                    if (C_indices[mid] < col) lo = mid + 1;
-                    else hi = mid;
+            for (int o = 0; o < octets; ++o) {
+                uint8_t d = kNone;
+                if (kCap * o + k < blen) {
+                    const int64_t col = B_indices[bb + kCap * o + k];
+                    int64_t lo = cs, hi = ce;
+                    while (lo < hi) {
+                        const int64_t mid = (lo + hi) >> 1;
+                        if (C_indices[mid] < col) lo = mid + 1;
+                        else hi = mid;
+                    }
+                    if (lo < ce && C_indices[lo] == col) d = (uint8_t)(lo - cs);
+                    else bad = other = true;   // C is not the pattern of A B
                 }
-                if (lo < ce && C_indices[lo] == col) d = (uint8_t)(lo - cs);
-                else bad = true;   // C is not the pattern of A B
+                p.dest[(e * octets + o) * kCap + k] = d;
             }
-            p.dest[e * kCap + k] = d;
             if (k == 0) {
                 p.bstart[e] = (int32_t)bb;
                 p.cstart[e] = (int32_t)cs;
@@ -99,6 +103,8 @@ __global__ __launch_bounds__(kBlock) void plan_map_kernel(
     if (bad) p.flag[0] = 1;
     if (long_a) p.flag[1] = 1;
     if (wide_c) p.flag[2] = 1;
+    if (other) p.flag[5] = 1;
+    if (longest > *(volatile int32_t *)(p.flag + 4)) atomicMax(p.flag + 4, longest);
 }
 
 // Checks the length of A's columns and notes in flag[3] how far from the diagonal A reaches
@@ -118,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void plan_columns_kernel(int64_t cols, cons
             far = far > hi ? far : hi;
         }
     }
-    if (bad) flag[0] = 1;
+    if (bad) flag[0] = flag[5] = 1;
     for (int off = 32; off > 0; off >>= 1) {
         const int32_t other = __shfl_xor(far, off, kWave);
         far = far > other ? far : other;
@@ -130,20 +136,21 @@ __global__ __launch_bounds__(kBlock) void plan_columns_kernel(int64_t cols, cons
 
 // The column-major copies of cstart and dest (entry t of the transposed plan is entry t_perm[t]).
 __global__ __launch_bounds__(kBlock) void plan_by_column_kernel(int64_t A_nnz, const int32_t *__restrict__ t_perm,
-                                                               PPlan p) {
+                                                               PPlan p, int octets) {
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     const uint64_t *dest64 = reinterpret_cast<const uint64_t *>(p.dest);
     uint64_t *t_dest64 = reinterpret_cast<uint64_t *>(p.t_dest);
     for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < A_nnz; t += stride) {
-        const int32_t e = t_perm[t];
+        const int64_t e = t_perm[t];
         p.t_cstart[t] = p.cstart[e];
-        t_dest64[t] = dest64[e];
+        for (int o = 0; o < octets; ++o) t_dest64[t * octets + o] = dest64[e * octets + o];
     }
 }
 
 __global__ void plan_flag_out_kernel(const int32_t *flag, volatile int64_t *host_pinned, int64_t ticket) {
     if (threadIdx.x == 0) {
-        host_pinned[0] = flag[0];
+        // 0: usable; 1: not usable; 2: not usable for the length of B's rows only (bits 8..: the longest)
+        host_pinned[0] = flag[0] == 0 ? 0 : (flag[5] == 0 ? 2 + ((int64_t)flag[4] << 8) : 1);
         host_pinned[1] = flag[2] ? 3 : (flag[1] ? 2 : 1);   // the product's class
         __threadfence_system();
         host_pinned[2] = ticket;
@@ -287,6 +294,64 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_long
     for (int d = k; d < clen; d += kCap) C_data[cs + d] = acc[d];
 }
 
+// The same for products whose named rows of B have up to 8 * OCT entries (classes 4 and 5): an entry
+// of A has OCT octets of destination bytes, lane k of the group takes entry 8 o + k of the row of B
+// in octet o.  The entries of A still take their turns one after the other (the octets of one entry
+// go to different columns of C), so every entry of C receives its products in the order of A's row.
+template <typename T, int OCT>
+__global__ __launch_bounds__(LongShape<256>::kThreads) void numeric_planned_wide_kernel(
+    int64_t rows, int64_t ntiles_padded, const T *__restrict__ A_data, const int64_t *__restrict__ A_indptr,
+    const T *__restrict__ B_data, const int32_t *__restrict__ bstart, const uint8_t *__restrict__ dest,
+    const int64_t *__restrict__ C_indptr, T *__restrict__ C_data) {
+    using S = LongShape<256>;
+    __shared__ T s_acc[S::kGroups * S::kStride];
+    __shared__ T s_av[S::kThreads];
+    __shared__ int32_t s_bs[S::kThreads];
+    __shared__ __align__(8) uint8_t s_db[S::kThreads * kCap * OCT];
+    const int k = threadIdx.x & (kCap - 1), g = threadIdx.x / kCap;
+    const int64_t row = nm::xcd_tile(blockIdx.x, ntiles_padded) * S::kGroups + g;
+    const bool live = row < rows;
+    const int64_t *pa = A_indptr + (live ? row : 0), *pc = C_indptr + (live ? row : 0);
+    const int64_t ab = pa[0], ae = live ? pa[1] : ab;
+    const int64_t cs = pc[0];
+    const int clen = live ? (int)(pc[1] - cs) : 0;
+    T *acc = s_acc + g * S::kStride;
+    for (int d = k; d < clen; d += kCap) acc[d] = T(0);
+    const int slot = g * kCap;
+    constexpr int kPer = kCap / OCT;   // entries of A whose octets are fetched together (8 gathers in flight)
+    for (int64_t base = ab; base < ae; base += kCap) {
+        {   // lane k of the group fetches entry base + k of the row
+            const bool have = base + k < ae;
+            const int64_t e = have ? base + k : base;
+            s_av[threadIdx.x] = A_data[e];
+            s_bs[threadIdx.x] = bstart[e];
+#pragma unroll
+            for (int o = 0; o < OCT; ++o)
+                *reinterpret_cast<uint64_t *>(s_db + (threadIdx.x * OCT + o) * kCap) =
+                    have ? *reinterpret_cast<const uint64_t *>(dest + (e * OCT + o) * kCap) : ~uint64_t(0);
+        }
+        group_fence();
+#pragma unroll
+        for (int a0 = 0; a0 < kCap; a0 += kPer) {
+            uint8_t db[kCap];
+            T bv[kCap];
+#pragma unroll
+            for (int u = 0; u < kCap; ++u) {
+                const int a = a0 + u / OCT, o = u % OCT;
+                db[u] = s_db[((slot + a) * OCT + o) * kCap + k];
+                bv[u] = B_data[db[u] != kNone ? (int64_t)s_bs[slot + a] + kCap * o + k : 0];
+            }
+#pragma unroll
+            for (int u = 0; u < kCap; ++u) {
+                const int a = a0 + u / OCT;
+                if (db[u] != kNone) acc[db[u]] = acc[db[u]] + s_av[slot + a] * bv[u];
+                if (u % OCT == OCT - 1) group_fence();   // the next entry of A may meet the same columns
+            }
+        }
+    }
+    for (int d = k; d < clen; d += kCap) C_data[cs + d] = acc[d];
+}
+
 // ---- backward ------------------------------------------------------------------------
 
 // grad_A.  A wavefront takes 64 consecutive entries of A, eight at a time with eight lanes per
@@ -381,6 +446,103 @@ __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     if (mine) grad_B[bb + k] = acc;
 }
 
+// grad_A and grad_B for named rows of B of up to 8 * OCT entries.  grad_A: the octets of an entry
+// are worked off one after the other by the entry's eight lanes, and the lane that adds the terms
+// goes on adding where the octet before left off: ascending k over the whole row.  grad_B: a group
+// of eight lanes per OCTET of a row of B.
+template <typename T, int OCT>
+__global__ __launch_bounds__(kBlock) void grad_a_wide_kernel(
+    int64_t A_nnz, const T *__restrict__ gC, const T *__restrict__ B_data, const int32_t *__restrict__ bstart,
+    const int32_t *__restrict__ cstart, const uint8_t *__restrict__ dest, T *__restrict__ grad_A) {
+    __shared__ T s_term[(kBlock / kWave) * kWave * kTermStride];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int k = lane & (kCap - 1), g = lane / kCap;
+    T *term = s_term + wave * kWave * kTermStride;
+    const int64_t base = ((int64_t)blockIdx.x * (kBlock / kWave) + wave) * kWave;
+    int32_t bs[kCap], cs[kCap];
+#pragma unroll
+    for (int p = 0; p < kCap; ++p) {
+        const int64_t e = base + p * kCap + g;
+        const int64_t es = e < A_nnz ? e : 0;
+        bs[p] = bstart[es];
+        cs[p] = cstart[es];
+    }
+    T acc = T(0);
+    for (int o = 0; o < OCT; ++o) {
+        uint8_t db[kCap];
+#pragma unroll
+        for (int p = 0; p < kCap; ++p) {
+            const int64_t e = base + p * kCap + g;
+            db[p] = e < A_nnz ? dest[(e * OCT + o) * kCap + k] : kNone;
+        }
+#pragma unroll
+        for (int p = 0; p < kCap; ++p) {
+            const bool have = db[p] != kNone;
+            const T gv = gC[have ? (int64_t)cs[p] + db[p] : 0];
+            const T bv = B_data[have ? (int64_t)bs[p] + kCap * o + k : 0];
+            term[(p * kCap + g) * kTermStride + k] = have ? gv * bv : T(0);
+        }
+        group_fence();
+        // (an absent entry of the row of B has the term +0.0: x + 0.0 == x for every x the sum can
+        // hold at that point except -0.0, which a sum that started from +0.0 never is)
+#pragma unroll
+        for (int q = 0; q < kCap; ++q) acc += term[lane * kTermStride + q];
+        group_fence();   // the exchange slots are written again for the next octet
+    }
+    if (base + lane < A_nnz) grad_A[base + lane] = acc;
+}
+
+template <typename T, int OCT>
+__global__ __launch_bounds__(kBlock) void grad_b_wide_kernel(
+    int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
+    const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm, const int64_t *__restrict__ B_indptr,
+    const int32_t *__restrict__ t_cstart, const uint8_t *__restrict__ t_dest, T *__restrict__ grad_B) {
+    __shared__ T s_a[kBlock];
+    __shared__ int32_t s_cs[kBlock];
+    __shared__ __align__(8) uint8_t s_db[kBlock * kCap];
+    const int k = threadIdx.x & (kCap - 1), slot = threadIdx.x & ~(kCap - 1);
+    const int64_t gid = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + threadIdx.x / kCap;
+    const int64_t j = gid / OCT;
+    const int o = (int)(gid % OCT);
+    const bool live = j < B_rows;
+    const int64_t *pb_ = B_indptr + (live ? j : 0);
+    const int64_t bb = pb_[0], blen = live ? pb_[1] - bb : 0;
+    const int32_t *pt = t_indptr + (live ? j : 0);
+    const int32_t pb = pt[0], pe = live ? pt[1] : pb;
+    if (pb == pe) {   // no entry of A in this column: the row's gradient is zero, however long the row
+        if (kCap * o + k < blen) grad_B[bb + kCap * o + k] = T(0);
+        if (o == 0)
+            for (int64_t q = kCap * OCT + k; q < blen; q += kCap) grad_B[bb + q] = T(0);
+        return;       // (no workgroup barrier anywhere in this kernel)
+    }
+    // a named row: at most kCap * OCT entries (the plan's build checked it)
+    const bool mine = kCap * o + k < blen;
+    T acc = T(0);
+    for (int32_t t0 = pb; t0 < pe; t0 += kCap) {
+        {
+            const bool have = t0 + k < pe;
+            const int32_t t = have ? t0 + k : pb;
+            s_a[threadIdx.x] = A_data[t_perm[t]];
+            s_cs[threadIdx.x] = t_cstart[t];
+            *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) =
+                have ? *reinterpret_cast<const uint64_t *>(t_dest + ((int64_t)t * OCT + o) * kCap) : ~uint64_t(0);
+        }
+        group_fence();
+        uint8_t db[kCap];
+        T gv[kCap];
+#pragma unroll
+        for (int u = 0; u < kCap; ++u) {
+            db[u] = mine ? s_db[(slot + u) * kCap + k] : kNone;
+            gv[u] = gC[db[u] != kNone ? (int64_t)s_cs[slot + u] + db[u] : 0];
+        }
+#pragma unroll
+        for (int u = 0; u < kCap; ++u)
+            if (db[u] != kNone) acc += s_a[slot + u] * gv[u];
+        group_fence();   // the exchange slots are written again in the next round
+    }
+    if (mine) grad_B[bb + kCap * o + k] = acc;
+}
+
 // Both gradients from the walk by column.  The eight lanes of row j of B gather, for every entry
 // e of column j of A, the eight entries of gC that e's products went to -- which is also all
 // that grad_A[e] = sum_k gC[..] * B[j][k] needs besides the row of B the lanes own.  So the terms
@@ -467,9 +629,15 @@ __global__ __launch_bounds__(kBlock) void grad_ab_mapped_kernel(
     if (mine) grad_B[bb + k] = acc;
 }
 
-// Brings the plan's flags to the host: *usable = 0, or the product's class (1, 2, 3).
-int read_verdict(const PPlan &p, void *host_landing, int *usable, hipStream_t s) {
-    int32_t flags[3] = {1, 0, 0};
+// Brings the plan's flags to the host.  *usable = the product's class when the plan can be used
+// (1, 2, 3 with one octet per named row of B; 4 with two octets, 5 with four: always the kernels
+// for rows of any length); 0 when it cannot; -L when the only obstacle is that the longest row of
+// B that A names has L entries, more than this plan's octets hold but no more than 32 -- a plan
+// with more octets would do.
+int class_of(int octets, int by_rows) { return octets == 1 ? by_rows : (octets == 2 ? 4 : 5); }
+
+int read_verdict(const PPlan &p, void *host_landing, int *usable, hipStream_t s, int octets) {
+    int64_t state, by_rows;
     if (host_landing) {
         volatile int64_t *land = (volatile int64_t *)host_landing;
         const int64_t ticket = land[2] + 1;
@@ -481,19 +649,61 @@ int read_verdict(const PPlan &p, void *host_landing, int *usable, hipStream_t s)
             NM_HIP_TRY(hipStreamSynchronize(s));
             NM_REQUIRE(land[2] == ticket, "the plan's verdict did not arrive");
         }
-        *usable = land[0] != 0 ? 0 : (int)land[1];
-        return NM_OK;
+        state = land[0];
+        by_rows = land[1];
+    } else {
+        int32_t flags[6] = {1, 0, 0, 0, 0, 1};
+        NM_HIP_TRY(hipMemcpyAsync(flags, p.flag, sizeof(flags), hipMemcpyDeviceToHost, s));
+        NM_HIP_TRY(hipStreamSynchronize(s));
+        state = flags[0] == 0 ? 0 : (flags[5] == 0 ? 2 + ((int64_t)flags[4] << 8) : 1);
+        by_rows = flags[2] ? 3 : (flags[1] ? 2 : 1);
     }
-    NM_HIP_TRY(hipMemcpyAsync(flags, p.flag, sizeof(flags), hipMemcpyDeviceToHost, s));
-    NM_HIP_TRY(hipStreamSynchronize(s));
-    *usable = flags[0] != 0 ? 0 : (flags[2] ? 3 : (flags[1] ? 2 : 1));
+    if (state == 0) {
+        *usable = class_of(octets, (int)by_rows);
+    } else if ((state & 0xff) == 2) {
+        const int64_t longest = state >> 8;
+        *usable = longest > kCap * octets && longest <= kCap * nm::kPlanMaxOctets ? -(int)longest : 0;
+    } else {
+        *usable = 0;
+    }
+    return NM_OK;
+}
+
+// octets of a plan of this class (0: no such class)
+int octets_of(int plan_class) {
+    return plan_class >= 1 && plan_class <= 3 ? 1 : (plan_class == 4 ? 2 : (plan_class == 5 ? 4 : 0));
+}
+
+template <typename T, int OCT>
+int launch_backward_wide(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A_data, const nm::TPlan &t,
+                         const void *B_data, const int64_t *B_indptr, const PPlan &p, void *grad_A, void *grad_B,
+                         hipStream_t s) {
+    if (grad_A && A_nnz > 0) {
+        const int64_t grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
+        NM_REQUIRE(grid < nm::kMaxGrid, "too many entries");
+        hipLaunchKernelGGL((grad_a_wide_kernel<T, OCT>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz,
+                           (const T *)gC, (const T *)B_data, p.bstart, p.cstart, p.dest, (T *)grad_A);
+        NM_LAUNCH_CHECK("grad_a_wide_kernel");
+    }
+    if (grad_B && A_cols > 0) {
+        const int64_t grid = nm::xcd_padded(nm::ceil_div(A_cols * OCT, (int64_t)kGroupsPerBlock));
+        NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+        hipLaunchKernelGGL((grad_b_wide_kernel<T, OCT>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, grid,
+                           (const T *)gC, (const T *)A_data, t.t_indptr, t.t_perm, B_indptr, p.t_cstart, p.t_dest,
+                           (T *)grad_B);
+        NM_LAUNCH_CHECK("grad_b_wide_kernel");
+    }
     return NM_OK;
 }
 
 template <typename T>
 int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A_data, const nm::TPlan &t,
                     const void *B_data, const int64_t *B_indptr, const PPlan &p, void *grad_A, void *grad_B,
-                    hipStream_t s) {
+                    hipStream_t s, int octets = 1) {
+    if (octets == 2)
+        return launch_backward_wide<T, 2>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s);
+    if (octets == 4)
+        return launch_backward_wide<T, 4>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s);
     if (grad_A && grad_B && A_nnz > 0 && A_cols > 0) {
         const int64_t grid = nm::xcd_padded(nm::ceil_div(A_cols, (int64_t)kGroupsPerBlock));
         NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
@@ -529,16 +739,35 @@ extern "C" int nm_spgemm_plan_bytes(int64_t A_nnz, size_t *plan_bytes) {
     return NM_OK;
 }
 
+extern "C" int nm_spgemm_plan_bytes_wide(int64_t A_nnz, int octets, size_t *plan_bytes) {
+    NM_REQUIRE(plan_bytes != nullptr && A_nnz >= 0, "bad arguments");
+    NM_REQUIRE(octets == 1 || octets == 2 || octets == 4, "octets %d (1, 2 or 4)", octets);
+    *plan_bytes = pplan_layout(A_nnz, nullptr, nullptr, octets);
+    return NM_OK;
+}
+
 extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
                                     const int64_t *A_indices, const int64_t *A_indptr, const int64_t *B_indices,
                                     const int64_t *B_indptr, const int64_t *C_indices, const int64_t *C_indptr,
                                     const void *A_plan_mem, void *plan_mem, size_t plan_bytes, void *host_landing,
                                     int *usable, nm_stream stream) {
+    return nm_spgemm_plan_build_wide(A_rows, A_cols, A_nnz, B_nnz, C_nnz, A_indices, A_indptr, B_indices, B_indptr,
+                                     C_indices, C_indptr, A_plan_mem, plan_mem, plan_bytes, 1, host_landing, usable,
+                                     stream);
+}
+
+extern "C" int nm_spgemm_plan_build_wide(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz,
+                                         int64_t C_nnz, const int64_t *A_indices, const int64_t *A_indptr,
+                                         const int64_t *B_indices, const int64_t *B_indptr,
+                                         const int64_t *C_indices, const int64_t *C_indptr, const void *A_plan_mem,
+                                         void *plan_mem, size_t plan_bytes, int octets, void *host_landing,
+                                         int *usable, nm_stream stream) {
+    NM_REQUIRE(octets == 1 || octets == 2 || octets == 4, "octets %d (1, 2 or 4)", octets);
     NM_REQUIRE(A_rows >= 0 && A_cols >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
     NM_REQUIRE(usable && plan_mem && A_plan_mem && A_indptr && B_indptr && C_indptr, "null pointer argument");
     NM_REQUIRE((A_nnz == 0 || A_indices) && (B_nnz == 0 || B_indices) && (C_nnz == 0 || C_indices),
                "null pointer argument");
-    const size_t need = pplan_layout(A_nnz, nullptr, nullptr);
+    const size_t need = pplan_layout(A_nnz, nullptr, nullptr, octets);
     if (plan_bytes < need) return nm::fail(NM_ERR_WORKSPACE, "plan of %zu bytes, %zu needed", plan_bytes, need);
     *usable = 0;
     // positions are kept in 32 bits
@@ -546,14 +775,14 @@ extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nn
     if (A_nnz >= lim || B_nnz >= lim || C_nnz >= lim || A_rows == 0 || A_nnz == 0) return NM_OK;
     hipStream_t s = nm::as_stream(stream);
     PPlan p;
-    pplan_layout(A_nnz, plan_mem, &p);
+    pplan_layout(A_nnz, plan_mem, &p, octets);
     nm::TPlan t;
     nm::tplan_layout(A_rows, A_cols, A_nnz, const_cast<void *>(A_plan_mem), &t);
     if (int rc = nm::fill_async(p.flag, 16, (int32_t)0, s)) return rc;
     int64_t grid = nm::ceil_div(A_rows, (int64_t)kGroupsPerBlock);
     if (grid > 65536) grid = 65536;
     hipLaunchKernelGGL(plan_map_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows, A_indices, A_indptr,
-                       B_indices, B_indptr, C_indices, C_indptr, p);
+                       B_indices, B_indptr, C_indices, C_indptr, p, octets);
     NM_LAUNCH_CHECK("plan_map_kernel");
     grid = nm::ceil_div(A_cols > 0 ? A_cols : 1, (int64_t)kBlock);
     if (grid > 4096) grid = 4096;
@@ -562,9 +791,9 @@ extern "C" int nm_spgemm_plan_build(int64_t A_rows, int64_t A_cols, int64_t A_nn
     NM_LAUNCH_CHECK("plan_columns_kernel");
     grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
     if (grid > 65536) grid = 65536;
-    hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p);
+    hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p, octets);
     NM_LAUNCH_CHECK("plan_by_column_kernel");
-    return read_verdict(p, host_landing, usable, s);
+    return read_verdict(p, host_landing, usable, s, octets);
 }
 
 extern "C" int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
@@ -593,9 +822,9 @@ extern "C" int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nn
     NM_LAUNCH_CHECK("plan_columns_kernel");
     grid = nm::ceil_div(A_nnz, (int64_t)kBlock);
     if (grid > 65536) grid = 65536;
-    hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p);
+    hipLaunchKernelGGL(plan_by_column_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, A_nnz, t.t_perm, p, 1);
     NM_LAUNCH_CHECK("plan_by_column_kernel");
-    return read_verdict(p, host_landing, usable, s);
+    return read_verdict(p, host_landing, usable, s, 1);
 }
 
 template <typename T, int CAP>
@@ -615,13 +844,36 @@ extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int plan_class, int64_t A_
                                          const void *B_data, const void *plan_mem, const int64_t *C_indptr,
                                          void *C_data, nm_stream stream) {
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
-    NM_REQUIRE(plan_class >= 1 && plan_class <= 3, "plan class %d (nm_spgemm_plan_build reports 1, 2 or 3)", plan_class);
+    NM_REQUIRE(octets_of(plan_class) != 0, "plan class %d (nm_spgemm_plan_build reports 1 to 5)", plan_class);
     NM_REQUIRE(A_rows >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
     if (A_rows == 0 || A_nnz == 0 || B_nnz == 0 || C_nnz == 0) return NM_OK;   // C has no entries
     NM_REQUIRE(A_data && A_indptr && B_data && plan_mem && C_indptr && C_data, "null pointer argument");
     PPlan p;
-    pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p);
+    pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p, octets_of(plan_class));
     hipStream_t s = nm::as_stream(stream);
+    if (plan_class >= 4) {
+        using S = LongShape<256>;
+        const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)S::kGroups));
+        NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+        if (plan_class == 4 && dt == NM_F32)
+            hipLaunchKernelGGL((numeric_planned_wide_kernel<float, 2>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
+                               A_rows, grid, (const float *)A_data, A_indptr, (const float *)B_data, p.bstart, p.dest,
+                               C_indptr, (float *)C_data);
+        else if (plan_class == 4)
+            hipLaunchKernelGGL((numeric_planned_wide_kernel<double, 2>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
+                               A_rows, grid, (const double *)A_data, A_indptr, (const double *)B_data, p.bstart,
+                               p.dest, C_indptr, (double *)C_data);
+        else if (dt == NM_F32)
+            hipLaunchKernelGGL((numeric_planned_wide_kernel<float, 4>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
+                               A_rows, grid, (const float *)A_data, A_indptr, (const float *)B_data, p.bstart, p.dest,
+                               C_indptr, (float *)C_data);
+        else
+            hipLaunchKernelGGL((numeric_planned_wide_kernel<double, 4>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
+                               A_rows, grid, (const double *)A_data, A_indptr, (const double *)B_data, p.bstart,
+                               p.dest, C_indptr, (double *)C_data);
+        NM_LAUNCH_CHECK("numeric_planned_wide_kernel");
+        return NM_OK;
+    }
     if (plan_class == 2)
         return dt == NM_F32 ? launch_long<float, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s)
                             : launch_long<double, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
@@ -664,6 +916,17 @@ extern "C" int nm_spgemm_backward_mapped(nm_dtype dt, int64_t A_rows, int64_t A_
                                          int64_t C_nnz, const void *gC, const void *A_data,
                                          const void *A_plan_mem, const void *B_data, const int64_t *B_indptr,
                                          const void *plan_mem, void *grad_A, void *grad_B, nm_stream stream) {
+    return nm_spgemm_backward_mapped_wide(dt, 1, A_rows, A_cols, A_nnz, B_nnz, C_nnz, gC, A_data, A_plan_mem, B_data,
+                                          B_indptr, plan_mem, grad_A, grad_B, stream);
+}
+
+extern "C" int nm_spgemm_backward_mapped_wide(nm_dtype dt, int plan_class, int64_t A_rows, int64_t A_cols,
+                                              int64_t A_nnz, int64_t B_nnz, int64_t C_nnz, const void *gC,
+                                              const void *A_data, const void *A_plan_mem, const void *B_data,
+                                              const int64_t *B_indptr, const void *plan_mem, void *grad_A,
+                                              void *grad_B, nm_stream stream) {
+    const int octets = octets_of(plan_class);
+    NM_REQUIRE(octets != 0, "plan class %d (nm_spgemm_plan_build reports 1 to 5)", plan_class);
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
     NM_REQUIRE(A_rows >= 0 && A_cols >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
     NM_REQUIRE(A_nnz > 0 && A_rows > 0, "a product plan exists only for a matrix with entries");
@@ -685,10 +948,10 @@ extern "C" int nm_spgemm_backward_mapped(nm_dtype dt, int64_t A_rows, int64_t A_
     }
     NM_REQUIRE(gC && A_data && A_plan_mem && B_data && B_indptr && plan_mem, "null pointer argument");
     PPlan p;
-    pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p);
+    pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p, octets);
     nm::TPlan t;
     nm::tplan_layout(A_rows, A_cols, A_nnz, const_cast<void *>(A_plan_mem), &t);
     if (dt == NM_F32)
-        return launch_backward<float>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s);
-    return launch_backward<double>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s);
+        return launch_backward<float>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s, octets);
+    return launch_backward<double>(A_cols, A_nnz, gC, A_data, t, B_data, B_indptr, p, grad_A, grad_B, s, octets);
 }

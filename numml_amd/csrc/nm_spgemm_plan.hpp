@@ -9,24 +9,28 @@
 
 namespace nm {
 
-constexpr int kPlanCap = 8;                      // entries per row of A and per named row of B
+constexpr int kPlanCap = 8;                      // entries per row of A (class 1) and per octet of a row of B
+constexpr int kPlanMaxOctets = 4;                // octets of a named row of B at most (rows of up to 32 entries)
 constexpr int kPlanRowCap = kPlanCap * kPlanCap; // entries per row of C
 constexpr uint8_t kPlanNone = 0xFF;              // destination byte of an entry a B row does not have
 
 struct PPlan {
     int32_t *flag;     // [0] != 0: a limit does not hold, the plan must not be used; [1], [2]: the product's
-                       // class; [3]: the largest |row - column| of an entry of A
+                       // class; [3]: the largest |row - column| of an entry of A; [4]: the longest row of
+                       // B that A names; [5] != 0: a limit other than that length does not hold
     int32_t *bstart;   // [A_nnz] where the row of B that entry e of A names starts
     int32_t *cstart;   // [A_nnz] where the row of C that entry e of A lies in starts
-    uint8_t *dest;     // [A_nnz * 8] byte k: position in that row of C of the k-th entry of that row of B
+    uint8_t *dest;     // [A_nnz * 8 * octets] byte k of octet o: position in that row of C of entry 8 o + k of
+                       // that row of B
     // cstart and dest once more in COLUMN-major order of A (entry t of the transposed-structure
     // plan): the kernel that walks A by column streams them instead of gathering 12 bytes from a
     // different line for every entry.  Filled when the plan is built or adopted.
     int32_t *t_cstart; // [A_nnz]
-    uint8_t *t_dest;   // [A_nnz * 8]
+    uint8_t *t_dest;   // [A_nnz * 8 * octets]
 };
 
-inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p) {
+// octets: 1 for products whose named rows of B have at most 8 entries, 2 for up to 16, 4 for up to 32
+inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p, int octets = 1) {
     size_t off = 0;
     auto take = [&](size_t bytes) {
         void *q = base ? static_cast<char *>(base) + off : nullptr;
@@ -36,9 +40,9 @@ inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p) {
     int32_t *flag = (int32_t *)take(64);
     int32_t *bs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
     int32_t *cs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
-    uint8_t *d = (uint8_t *)take((size_t)(A_nnz + 1) * 8);
+    uint8_t *d = (uint8_t *)take((size_t)(A_nnz + 1) * 8 * octets);
     int32_t *tcs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
-    uint8_t *td = (uint8_t *)take((size_t)(A_nnz + 1) * 8);
+    uint8_t *td = (uint8_t *)take((size_t)(A_nnz + 1) * 8 * octets);
     if (p) *p = PPlan{flag, bs, cs, d, tcs, td};
     return off;
 }

@@ -506,9 +506,23 @@ void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, cons
                                    plan->parent->mem.data_ptr(), plan->mem.data_ptr(), pbytes, host_landing(),
                                    &usable, current_stream(dev)),
               "nm_spgemm_plan_build");
+        if (usable < 0) {
+            // the only obstacle is the length of the rows of B that A names (9 to 32 entries): a plan
+            // with two or four destination octets per entry of A
+            const int octets = -usable <= 16 ? 2 : 4;
+            check(nm_spgemm_plan_bytes_wide(A_indices.numel(), octets, &pbytes), "nm_spgemm_plan_bytes_wide");
+            plan->mem = scratch(pbytes, dev);
+            check(nm_spgemm_plan_build_wide(A_rows, A_cols, A_indices.numel(), B_indices.numel(), C_indices.numel(),
+                                            A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
+                                            B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
+                                            C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(),
+                                            plan->parent->mem.data_ptr(), plan->mem.data_ptr(), pbytes, octets,
+                                            host_landing(), &usable, current_stream(dev)),
+                  "nm_spgemm_plan_build_wide");
+        }
     }
-    plan->usable = usable != 0;
-    plan->plan_class = usable;
+    plan->usable = usable > 0;
+    plan->plan_class = usable > 0 ? usable : 0;
     if (plan->usable) {
         plan->derived = {C_indices, C_indptr};
         for (const Tensor &t : plan->derived) plan->derived_versions.push_back(t._version());
@@ -1094,12 +1108,12 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
         auto pp = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, A_rows, B_cols, dev);
         if (pp && pp->usable && pp->derived[0].data_ptr() == C_indices.data_ptr() &&
             pp->derived[1].data_ptr() == C_indptr.data_ptr() && pp->derived[0].numel() == C_indices.numel()) {
-            check(nm_spgemm_backward_mapped(dtype_of(A_data), A_rows, A_cols, A_data.numel(), B_data.numel(),
-                                            grad_C.numel(), grad_C.data_ptr(), A_data.data_ptr(),
-                                            pp->parent->mem.data_ptr(), B_data.data_ptr(),
-                                            B_indptr.data_ptr<int64_t>(), pp->mem.data_ptr(), grad_A.data_ptr(),
-                                            grad_B.data_ptr(), current_stream(dev)),
-                  "nm_spgemm_backward_mapped");
+            check(nm_spgemm_backward_mapped_wide(dtype_of(A_data), pp->plan_class, A_rows, A_cols, A_data.numel(),
+                                                 B_data.numel(), grad_C.numel(), grad_C.data_ptr(),
+                                                 A_data.data_ptr(), pp->parent->mem.data_ptr(), B_data.data_ptr(),
+                                                 B_indptr.data_ptr<int64_t>(), pp->mem.data_ptr(),
+                                                 grad_A.data_ptr(), grad_B.data_ptr(), current_stream(dev)),
+                  "nm_spgemm_backward_mapped_wide");
             return {grad_A, grad_B};
         }
     }

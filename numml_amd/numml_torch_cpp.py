@@ -625,7 +625,7 @@ class ProductPlan:
                     A_rows, A_cols, self.A_nnz, self.B_nnz, self.C_nnz, hash_rows, _ptr(self.transposed.mem),
                     _ptr(self.mem), nbytes.value, _ptr(_host_landing()), ctypes.byref(usable), _stream(dev)),
                     "nm_spgemm_plan_adopt")
-                self.usable, self.plan_class = bool(usable.value), usable.value
+                self.usable, self.plan_class = usable.value > 0, usable.value
                 return
             self.mem = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
             _lib.check(L.nm_spgemm_plan_build(
@@ -633,7 +633,19 @@ class ProductPlan:
                 _ptr(B_indices), _ptr(B_indptr), _ptr(C_indices), _ptr(C_indptr), _ptr(self.transposed.mem),
                 _ptr(self.mem), nbytes.value, _ptr(_host_landing()), ctypes.byref(usable), _stream(dev)),
                 "nm_spgemm_plan_build")
-            self.usable, self.plan_class = bool(usable.value), usable.value
+            if usable.value < 0:
+                # the only obstacle is the length of the rows of B that A names (9 to 32 entries):
+                # a plan with two or four destination octets per entry of A
+                octets = 2 if -usable.value <= 16 else 4
+                _lib.check(L.nm_spgemm_plan_bytes_wide(self.A_nnz, octets, ctypes.byref(nbytes)),
+                           "nm_spgemm_plan_bytes_wide")
+                self.mem = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=dev)
+                _lib.check(L.nm_spgemm_plan_build_wide(
+                    A_rows, A_cols, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(A_indices), _ptr(A_indptr),
+                    _ptr(B_indices), _ptr(B_indptr), _ptr(C_indices), _ptr(C_indptr), _ptr(self.transposed.mem),
+                    _ptr(self.mem), nbytes.value, octets, _ptr(_host_landing()), ctypes.byref(usable), _stream(dev)),
+                    "nm_spgemm_plan_build_wide")
+            self.usable, self.plan_class = usable.value > 0, usable.value
 
     def numeric(self, A_data, B_data):
         """C_data of the product (the pattern is the one the plan was built from)."""
@@ -656,10 +668,10 @@ class ProductPlan:
         A_data, B_data, grad_C = A_data.contiguous(), B_data.contiguous(), grad_C.contiguous()
         with torch.cuda.device(self.dev):
             grad_A, grad_B = torch.empty_like(A_data), torch.empty_like(B_data)
-            _lib.check(_lib.lib().nm_spgemm_backward_mapped(
-                _dt(A_data), self.A_rows, self.A_cols, self.A_nnz, self.B_nnz, self.C_nnz, _ptr(grad_C),
-                _ptr(A_data), _ptr(self.transposed.mem), _ptr(B_data), _ptr(self.B_indptr), _ptr(self.mem),
-                _ptr(grad_A), _ptr(grad_B), _stream(self.dev)), "nm_spgemm_backward_mapped")
+            _lib.check(_lib.lib().nm_spgemm_backward_mapped_wide(
+                _dt(A_data), self.plan_class, self.A_rows, self.A_cols, self.A_nnz, self.B_nnz, self.C_nnz,
+                _ptr(grad_C), _ptr(A_data), _ptr(self.transposed.mem), _ptr(B_data), _ptr(self.B_indptr),
+                _ptr(self.mem), _ptr(grad_A), _ptr(grad_B), _stream(self.dev)), "nm_spgemm_backward_mapped_wide")
         return [grad_A, grad_B]
 
 

@@ -323,6 +323,45 @@ def test_product_plan_policy(dev, cpp):
     cpp.clear_plan_cache()
 
 
+def test_product_plan_for_rows_of_the_right_operand_of_up_to_32_entries(dev, cpp):
+    """A (A A) on a 3D grid -- the right operand has 25-entry rows, so the product takes the hash path --
+    in a loop with new values: the first call is stateless, the second leaves a product plan with four
+    destination octets per entry behind, later calls run the numeric kernel and both gradients on it;
+    every call gives the oracle's bits."""
+    dtype = np.float64
+    d, i, p, (n, _) = G.laplace3d(9, dtype, 3)
+    D, I, P = to_dev(dev, d, i, p)
+    Sd, SI, SP = cpp.spgemm_forward(n, n, D, I, P, n, n, D, I, P)
+    si, sp = host(SI), host(SP)
+    cpp.clear_plan_cache()
+    cpp.set_backward_mode("planned")
+    try:
+        built0 = cpp.plan_cache_stats()[0]
+        shared = None
+        for call in range(4):
+            a, b = randn(60 + call, d.shape[0], dtype), randn(70 + call, si.shape[0], dtype)
+            A, B = to_dev(dev, a, b)
+            C_data, C_indices, C_indptr = cpp.spgemm_forward(n, n, A, I, P, n, n, B, SI, SP)
+            cd, ci, cp = oracle.spgemm_forward(n, n, a, i, p, n, n, b, si, sp)
+            assert_same(host(C_indptr), cp, f"call {call}: C_indptr")
+            assert_same(host(C_indices), ci, f"call {call}: C_indices")
+            assert_same(host(C_data), cd, f"call {call}: C_data")
+            g = randn(80 + call, cd.shape[0], dtype)
+            gA, gB = cpp.spgemm_backward(to_dev(dev, g)[0], C_indices, C_indptr, n, n, A, I, P, n, n, B, SI, SP)
+            rA, rB = oracle.spgemm_backward(g, ci, cp, n, n, a, i, p, n, n, b, si, sp)
+            assert_same(host(gA), rA, f"call {call}: grad_A")
+            if call >= 1:                   # on the plan: rows ascending, the serial order
+                assert_same(host(gB), rB, f"call {call}: grad_B")
+            if call >= 2:
+                if shared is not None:
+                    assert C_indices.data_ptr() == shared, "the plan's pattern tensors"
+                shared = C_indices.data_ptr()
+        assert cpp.plan_cache_stats()[0] == built0 + 2      # A's transposed plan and the product plan
+    finally:
+        cpp.set_backward_mode("planned")
+        cpp.clear_plan_cache()
+
+
 def test_install_registers_the_reference_module_name(cpp):
     import sys
     saved = sys.modules.pop("numml_torch_cpp", None)

@@ -178,6 +178,62 @@ def test_long_rows_of_the_left_operand_and_wide_rows_of_the_product(dev, dtype):
         assert_same(host(gB), rB, f"{name}: grad_B")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_named_rows_of_the_right_operand_of_up_to_32_entries(dev, dtype):
+    """Classes 4 and 5 of the plan: two or four destination octets per entry of A, for products whose
+    rows of B have up to 16 or 32 entries (a 3D stencil times its own square, a 27-point matrix
+    squared).  Product and both gradients bit for bit, as for the one-octet plans."""
+    def stencil27(n):
+        import scipy.sparse as sps
+        one = sps.diags([np.ones(n - 1), np.ones(n), np.ones(n - 1)], [-1, 0, 1])
+        M = sps.kron(sps.kron(one, one), one).tocsr()
+        M.sort_indices()
+        rng = np.random.default_rng(7)
+        return (rng.standard_normal(M.nnz).astype(dtype), M.indices.astype(np.int64), M.indptr.astype(np.int64), M.shape)
+
+    d, i, p, (n, _) = G.laplace3d(10, dtype, jitter_seed=5)
+    D, I, P = to_dev(dev, d, i, p)
+    Sd, Si, Sp = mirror.spgemm_forward(n, n, D, I, P, n, n, D, I, P)
+    square = (host(Sd), host(Si), host(Sp), (n, n))
+    cases = [
+        ("rows of up to 6 entries times rows of 9 to 16", 4,
+         G.ragged_csr(600, 500, 6, 81, dtype, min_len=1), G.ragged_csr(500, 3000, 16, 82, dtype, min_len=9)),
+        ("rows of up to 7 entries times rows of 17 to 32", 5,
+         G.ragged_csr(400, 300, 7, 83, dtype), G.ragged_csr(300, 9000, 32, 84, dtype, min_len=17)),
+        ("rows of up to 12 entries times rows of up to 20", 5,
+         G.ragged_csr(700, 500, 12, 85, dtype, min_len=5), G.ragged_csr(500, 600, 20, 86, dtype, min_len=3)),
+        ("A (A A) on a 3D grid: 25-entry rows of B, 63-entry rows of C", 5, (d, i, p, (n, n)), square),
+        ("27-point matrix squared: 27-entry rows of B, 125-entry rows of C", 5, stencil27(9), stencil27(9)),
+    ]
+    for name, want_class, A, B in cases:
+        ad, ai, ap, (m, kdim) = A
+        bd, bi, bp, (_, ncols) = B
+        AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+        C_data, C_indices, C_indptr = mirror.spgemm_forward(m, kdim, AD, AI, AP, kdim, ncols, BD, BI, BP)
+        plan = mirror.ProductPlan(m, kdim, AI, AP, BI, BP, C_indices, C_indptr)
+        assert plan.usable and plan.plan_class == want_class, (name, plan.plan_class)
+        ad2, bd2 = randn(91, ad.shape[0], dtype), randn(92, bd.shape[0], dtype)
+        AD2, BD2 = to_dev(dev, ad2, bd2)
+        cd, ci, cp = oracle.spgemm_forward(m, kdim, ad2, ai, ap, kdim, ncols, bd2, bi, bp)
+        assert_same(host(C_indices), ci, f"{name}: pattern")
+        assert_same(host(plan.numeric(AD2, BD2)), cd, f"{name}: C_data")
+        g = randn(93, cd.shape[0], dtype)
+        gA, gB = plan.backward(to_dev(dev, g)[0], AD2, BD2)
+        rA, rB = oracle.spgemm_backward(g, ci, cp, m, kdim, ad2, ai, ap, kdim, ncols, bd2, bi, bp)
+        assert_same(host(gA), rA, f"{name}: grad_A")
+        assert_same(host(gB), rB, f"{name}: grad_B")
+        # one gradient at a time
+        L = mirror._lib.lib()
+        for which in (0, 1):
+            out = torch.full_like(AD2 if which == 0 else BD2, 7.0)
+            mirror._lib.check(L.nm_spgemm_backward_mapped_wide(
+                mirror._dt(AD2), plan.plan_class, m, kdim, ad.shape[0], bd.shape[0], cd.shape[0],
+                mirror._ptr(to_dev(dev, g)[0]), mirror._ptr(AD2), mirror._ptr(plan.transposed.mem), mirror._ptr(BD2),
+                mirror._ptr(BP), mirror._ptr(plan.mem), mirror._ptr(out) if which == 0 else None,
+                mirror._ptr(out) if which == 1 else None, mirror._stream(dev)), "nm_spgemm_backward_mapped_wide")
+            assert_same(host(out), rA if which == 0 else rB, f"{name}: gradient {which} alone")
+
+
 def test_rows_beyond_the_limits_are_refused(dev):
     dtype = np.float64
     # a row of C with more than 254 entries
@@ -187,11 +243,11 @@ def test_rows_beyond_the_limits_are_refused(dev):
     _, C_indices, C_indptr = mirror.spgemm_forward(50, 60, AD, AI, AP, 60, 80000, BD, BI, BP)
     assert int((C_indptr[1:] - C_indptr[:-1]).max()) > 254
     assert not mirror.ProductPlan(50, 60, AI, AP, BI, BP, C_indices, C_indptr).usable
-    # a named row of B with nine entries
+    # a named row of B with 33 entries (up to 32 there are plans with two or four octets per entry)
     ad, ai, ap, ashape = _unpack(_short_rows(50, 60, 4, 23, dtype, min_len=1))
-    bd, bi, bp, bshape = _unpack(_short_rows(60, 80, 9, 24, dtype, min_len=9))
+    bd, bi, bp, bshape = _unpack(_short_rows(60, 800, 33, 24, dtype, min_len=33))
     AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
-    _, C_indices, C_indptr = mirror.spgemm_forward(50, 60, AD, AI, AP, 60, 80, BD, BI, BP)
+    _, C_indices, C_indptr = mirror.spgemm_forward(50, 60, AD, AI, AP, 60, 800, BD, BI, BP)
     plan = mirror.ProductPlan(50, 60, AI, AP, BI, BP, C_indices, C_indptr)
     assert not plan.usable
     with pytest.raises(RuntimeError):
