@@ -268,8 +268,10 @@ int nm_spgemm_backward_planned(nm_dtype dt, int64_t A_rows, int64_t A_cols, int6
  *                           A_plan_mem: the transposed-structure plan of A
  *                           (nm_csr_transpose_plan_build).  *usable = 0: the plan
  *                           must not be used (a row of B that A names has more than
- *                           8 entries, a row of C more than 254, a column of A more
- *                           than 4096, or a position does not fit 31 bits).
+ *                           32 entries, a row of C more than 254, a column of A more
+ *                           than 4096, or a position does not fit 31 bits); negative:
+ *                           it must not be used either, but a plan with more octets
+ *                           can be (nm_spgemm_plan_build_wide, below).
  *                           Otherwise the product's class: 1 -- rows of A of at most
  *                           8 and rows of C of at most 64 entries, 2 -- longer rows of
  *                           A, 3 -- also rows of C of 65..254 entries.  Waits for the
