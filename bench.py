@@ -27,6 +27,7 @@ on):
   sptrsv  fp64 triangular solve fwd+bwd, tril(Poisson 1024^2), 2047 levels
   spsolve fp64 direct solve fwd+bwd (LU without pivoting + four triangular solves), Poisson 64^2
   lincomb    fp32 A - B (splincomb) + its backward, both on the spmv matrix pattern
+  spgemm_wide  fp64 A (A A) forward + backward on the 3D matrix: 25-entry rows of the right operand
   transpose  fp32 explicit CSR transpose + its backward on the spmv matrix
   copy    256 MiB device copy (counter calibration / practical bandwidth ceiling)
   ref_timing  the shapes the reference's own timing script uses (demos/timing.py:177-217,
@@ -368,9 +369,9 @@ class SpGEMM(Workload):
     unit = "GFLOP/s"
     dtype = "f64"
 
-    def __init__(self, left="A"):
-        self.left = left
-        self.name = "spgemm" if left == "A" else "spgemm_hash"
+    def __init__(self, left="A", right="A"):
+        self.left, self.right = left, right
+        self.name = "spgemm_wide" if right == "AA" else ("spgemm" if left == "A" else "spgemm_hash")
 
     def setup(self, dev):
         import torch
@@ -381,13 +382,13 @@ class SpGEMM(Workload):
         n = int(os.environ.get("NM_BENCH_SPGEMM_N", "128"))
         d, i, p, (rows, cols) = G.laplace3d(n, np.float64, jitter_seed=0)
         t = lambda a: torch.from_numpy(a).to(dev)
-        R = (t(d), t(i), t(p))
-        self.hostR = (d, i, p)
-        if self.left == "AA":
-            L = tuple(ext.spgemm_forward(rows, cols, *R, rows, cols, *R))
-            self.hostL = tuple(v.cpu().numpy() for v in L)
-        else:
-            L, self.hostL = R, self.hostR
+        base = (t(d), t(i), t(p))
+        host_base = (d, i, p)
+        if "AA" in (self.left, self.right):
+            square = tuple(ext.spgemm_forward(rows, cols, *base, rows, cols, *base))
+            host_square = tuple(v.cpu().numpy() for v in square)
+        L, self.hostL = (square, host_square) if self.left == "AA" else (base, host_base)
+        R, self.hostR = (square, host_square) if self.right == "AA" else (base, host_base)
         self.L, self.R = L, R
         self.rows, self.cols, self.nnz = rows, cols, int(L[0].shape[0])
         # The first steps on a new pair of patterns are timed one by one: in the default mode the
@@ -407,11 +408,11 @@ class SpGEMM(Workload):
         self.first_steps_ms = firsts
         self.planned = _binding.backward_mode() != "atomic" and _binding.name == "compiled"
         self.C = C
-        lens = np.diff(p)
+        lens = np.diff(self.hostR[2])
         self.products = int(lens[self.hostL[1]].sum())
         self.flops = 2 * self.products
         s = 8
-        nnzR = int(d.shape[0])
+        nnzR = int(self.hostR[0].shape[0])
         # Compulsory traffic of the forward: both operands and the result once, the two row
         # pointer arrays.  The gather-inclusive figure (every referenced row of the right operand
         # read again for every product) is an upper bound and is reported apart; most of those
@@ -424,10 +425,14 @@ class SpGEMM(Workload):
             # forward on the product plan: values of both operands, 12 bytes of plan per entry of
             # the left operand (row start in B, eight destination bytes), both row pointer arrays,
             # the values of C; the pattern of C is the plan's and is not written again
-            self.bytes_per_step = self.nnz * (s + 12) + nnzR * s + self.nnzC * s + 2 * rows * 8
+            # (rows of the right operand of 17 to 32 entries: four octets of destination bytes)
+            plan_bytes = 4 + 8 * (4 if self.right == "AA" else 1)
+            self.bytes_per_step = self.nnz * (s + plan_bytes) + nnzR * s + self.nnzC * s + 2 * rows * 8
             self.dominant_bytes = self.bytes_per_step
-            self.dominant_name = "numeric_planned_kernel (the whole forward on the product plan)"
-        self.config = {"workload": f"spgemm_{self.left}xA_fwd_bwd_f64_laplace3d_{n}", "rows": rows,
+            self.dominant_name = ("numeric_planned_wide_kernel (the whole forward on the product plan)"
+                                  if self.right == "AA" else
+                                  "numeric_planned_kernel (the whole forward on the product plan)")
+        self.config = {"workload": f"spgemm_{self.left}x{self.right}_fwd_bwd_f64_laplace3d_{n}", "rows": rows,
                        "nnz_left": self.nnz, "nnz_right": nnzR,
                        "nnz_C": self.nnzC, "products": self.products, "index_bytes": 8,
                        "mode": ("product plan (pattern of C and the destination of every product kept per pair of "
@@ -815,6 +820,7 @@ WORKLOADS = {
     "spgemm": SpGEMM,
     # off the reference's configurations: rows of 25 entries instead of 5-7
     "spgemm_hash": lambda: SpGEMM("AA"),
+    "spgemm_wide": lambda: SpGEMM("A", "AA"),
     "spmv_rows25": lambda: SpMV(128, np.float32, 0, "laplace3d_128_squared", squared3d=True),
     "sptrsv": SpTRSV,
     "spsolve": SpSolve,
