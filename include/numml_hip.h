@@ -337,7 +337,8 @@ int nm_spgemm_backward_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64
  * has L entries, 9 <= L <= 32: the caller then allocates
  * nm_spgemm_plan_bytes_wide(A_nnz, L <= 16 ? 2 : 4) and calls
  * nm_spgemm_plan_build_wide with that number of octets, which reports class 4
- * (two octets) or 5 (four), to be handed to nm_spgemm_numeric_planned and
+ * (two octets) or 5 (four), 6 or 7 when rows of C have 65 to 254 entries as
+ * well, to be handed to nm_spgemm_numeric_planned and
  * nm_spgemm_backward_mapped_wide; with octets = 1 and classes 1 to 3 these are
  * the calls above.  Same sums in the same order, bit for bit. */
 int nm_spgemm_plan_bytes_wide(int64_t A_nnz, int octets, size_t *plan_bytes);

@@ -298,12 +298,12 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_long
 // of A has OCT octets of destination bytes, lane k of the group takes entry 8 o + k of the row of B
 // in octet o.  The entries of A still take their turns one after the other (the octets of one entry
 // go to different columns of C), so every entry of C receives its products in the order of A's row.
-template <typename T, int OCT>
-__global__ __launch_bounds__(LongShape<256>::kThreads) void numeric_planned_wide_kernel(
+template <typename T, int OCT, int CAP>
+__global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_wide_kernel(
     int64_t rows, int64_t ntiles_padded, const T *__restrict__ A_data, const int64_t *__restrict__ A_indptr,
     const T *__restrict__ B_data, const int32_t *__restrict__ bstart, const uint8_t *__restrict__ dest,
     const int64_t *__restrict__ C_indptr, T *__restrict__ C_data) {
-    using S = LongShape<256>;
+    using S = LongShape<CAP>;
     __shared__ T s_acc[S::kGroups * S::kStride];
     __shared__ T s_av[S::kThreads];
     __shared__ int32_t s_bs[S::kThreads];
@@ -630,11 +630,13 @@ __global__ __launch_bounds__(kBlock) void grad_ab_mapped_kernel(
 }
 
 // Brings the plan's flags to the host.  *usable = the product's class when the plan can be used
-// (1, 2, 3 with one octet per named row of B; 4 with two octets, 5 with four: always the kernels
-// for rows of any length); 0 when it cannot; -L when the only obstacle is that the longest row of
+// (1, 2, 3 with one octet per named row of B; 4 with two octets, 5 with four, 6 and 7 the same with
+// rows of C of 65-254 entries: always the kernels for rows of A of any length); 0 when it cannot; -L when the only obstacle is that the longest row of
 // B that A names has L entries, more than this plan's octets hold but no more than 32 -- a plan
 // with more octets would do.
-int class_of(int octets, int by_rows) { return octets == 1 ? by_rows : (octets == 2 ? 4 : 5); }
+int class_of(int octets, int by_rows) {
+    return octets == 1 ? by_rows : (octets == 2 ? 4 : 5) + (by_rows == 3 ? 2 : 0);
+}
 
 int read_verdict(const PPlan &p, void *host_landing, int *usable, hipStream_t s, int octets) {
     int64_t state, by_rows;
@@ -671,7 +673,8 @@ int read_verdict(const PPlan &p, void *host_landing, int *usable, hipStream_t s,
 
 // octets of a plan of this class (0: no such class)
 int octets_of(int plan_class) {
-    return plan_class >= 1 && plan_class <= 3 ? 1 : (plan_class == 4 ? 2 : (plan_class == 5 ? 4 : 0));
+    return plan_class >= 1 && plan_class <= 3 ? 1
+           : (plan_class == 4 || plan_class == 6 ? 2 : (plan_class == 5 || plan_class == 7 ? 4 : 0));
 }
 
 template <typename T, int OCT>
@@ -839,41 +842,48 @@ int launch_long(int64_t A_rows, const void *A_data, const int64_t *A_indptr, con
     return NM_OK;
 }
 
+template <typename T, int OCT, int CAP>
+int launch_wide_typed(int64_t A_rows, const void *A_data, const int64_t *A_indptr, const void *B_data, const PPlan &p,
+                      const int64_t *C_indptr, void *C_data, hipStream_t s) {
+    using S = LongShape<CAP>;
+    const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)S::kGroups));
+    NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
+    hipLaunchKernelGGL((numeric_planned_wide_kernel<T, OCT, CAP>), dim3((unsigned)grid), dim3(S::kThreads), 0, s, A_rows,
+                       grid, (const T *)A_data, A_indptr, (const T *)B_data, p.bstart, p.dest, C_indptr, (T *)C_data);
+    NM_LAUNCH_CHECK("numeric_planned_wide_kernel");
+    return NM_OK;
+}
+
+template <typename T>
+int launch_wide_of(int plan_class, int64_t A_rows, const void *A_data, const int64_t *A_indptr, const void *B_data,
+                   const PPlan &p, const int64_t *C_indptr, void *C_data, hipStream_t s) {
+    switch (plan_class) {
+        case 4: return launch_wide_typed<T, 2, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
+        case 5: return launch_wide_typed<T, 4, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
+        case 6: return launch_wide_typed<T, 2, 256>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
+        default: return launch_wide_typed<T, 4, 256>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
+    }
+}
+
+static int launch_wide(nm_dtype dt, int plan_class, int64_t A_rows, const void *A_data, const int64_t *A_indptr,
+                const void *B_data, const PPlan &p, const int64_t *C_indptr, void *C_data, hipStream_t s) {
+    return dt == NM_F32 ? launch_wide_of<float>(plan_class, A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s)
+                        : launch_wide_of<double>(plan_class, A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
+}
+
 extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int plan_class, int64_t A_rows, int64_t A_nnz, int64_t B_nnz,
                                          int64_t C_nnz, const void *A_data, const int64_t *A_indptr,
                                          const void *B_data, const void *plan_mem, const int64_t *C_indptr,
                                          void *C_data, nm_stream stream) {
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
-    NM_REQUIRE(octets_of(plan_class) != 0, "plan class %d (nm_spgemm_plan_build reports 1 to 5)", plan_class);
+    NM_REQUIRE(octets_of(plan_class) != 0, "plan class %d (nm_spgemm_plan_build reports 1 to 7)", plan_class);
     NM_REQUIRE(A_rows >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
     if (A_rows == 0 || A_nnz == 0 || B_nnz == 0 || C_nnz == 0) return NM_OK;   // C has no entries
     NM_REQUIRE(A_data && A_indptr && B_data && plan_mem && C_indptr && C_data, "null pointer argument");
     PPlan p;
     pplan_layout(A_nnz, const_cast<void *>(plan_mem), &p, octets_of(plan_class));
     hipStream_t s = nm::as_stream(stream);
-    if (plan_class >= 4) {
-        using S = LongShape<256>;
-        const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)S::kGroups));
-        NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
-        if (plan_class == 4 && dt == NM_F32)
-            hipLaunchKernelGGL((numeric_planned_wide_kernel<float, 2>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
-                               A_rows, grid, (const float *)A_data, A_indptr, (const float *)B_data, p.bstart, p.dest,
-                               C_indptr, (float *)C_data);
-        else if (plan_class == 4)
-            hipLaunchKernelGGL((numeric_planned_wide_kernel<double, 2>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
-                               A_rows, grid, (const double *)A_data, A_indptr, (const double *)B_data, p.bstart,
-                               p.dest, C_indptr, (double *)C_data);
-        else if (dt == NM_F32)
-            hipLaunchKernelGGL((numeric_planned_wide_kernel<float, 4>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
-                               A_rows, grid, (const float *)A_data, A_indptr, (const float *)B_data, p.bstart, p.dest,
-                               C_indptr, (float *)C_data);
-        else
-            hipLaunchKernelGGL((numeric_planned_wide_kernel<double, 4>), dim3((unsigned)grid), dim3(S::kThreads), 0, s,
-                               A_rows, grid, (const double *)A_data, A_indptr, (const double *)B_data, p.bstart,
-                               p.dest, C_indptr, (double *)C_data);
-        NM_LAUNCH_CHECK("numeric_planned_wide_kernel");
-        return NM_OK;
-    }
+    if (plan_class >= 4) return launch_wide(dt, plan_class, A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
     if (plan_class == 2)
         return dt == NM_F32 ? launch_long<float, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s)
                             : launch_long<double, kRowCap>(A_rows, A_data, A_indptr, B_data, p, C_indptr, C_data, s);
@@ -926,7 +936,7 @@ extern "C" int nm_spgemm_backward_mapped_wide(nm_dtype dt, int plan_class, int64
                                               const int64_t *B_indptr, const void *plan_mem, void *grad_A,
                                               void *grad_B, nm_stream stream) {
     const int octets = octets_of(plan_class);
-    NM_REQUIRE(octets != 0, "plan class %d (nm_spgemm_plan_build reports 1 to 5)", plan_class);
+    NM_REQUIRE(octets != 0, "plan class %d (nm_spgemm_plan_build reports 1 to 7)", plan_class);
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
     NM_REQUIRE(A_rows >= 0 && A_cols >= 0 && A_nnz >= 0 && B_nnz >= 0 && C_nnz >= 0, "negative size");
     NM_REQUIRE(A_nnz > 0 && A_rows > 0, "a product plan exists only for a matrix with entries");
