@@ -244,6 +244,13 @@ class SpMV(Workload):
             gbs = rec["config"][f"bytes_per_step_with_{key}_structure"] / (rec["ms_per_step"] * 1e-3) / 1e9
             rec["config"][f"GBps_on_{key}_structure_model"] = round(gbs, 1)
             rec["config"][f"pct_of_hbm_peak_on_{key}_structure_model"] = round(100.0 * gbs / HBM_PEAK_GBS, 2)
+        rec["value_note"] = (
+            f"value prices every array at the width the kernels read ({rec['config']['algorithmic_bytes_per_step'] / 1e6:.1f} MB "
+            f"per step); the same step is {rec['config']['GBps_on_int64_structure_model']:.0f} GB/s = "
+            f"{rec['config']['pct_of_hbm_peak_on_int64_structure_model']:.1f} % of peak on the arrays as the interface "
+            f"delivers them ({rec['config']['bytes_per_step_with_int64_structure'] / 1e6:.1f} MB, the model of the first "
+            f"record) and {rec['config']['GBps_on_int32_structure_model']:.0f} GB/s = "
+            f"{rec['config']['pct_of_hbm_peak_on_int32_structure_model']:.1f} % on the plan's 32-bit structure")
         rec["config"]["stateless_ms_per_step"] = round(stateless, 5)
         rec["config"]["stateless_GBps_int64_structure"] = round(
             rec["config"]["bytes_per_step_with_int64_structure"] / (stateless * 1e-3) / 1e9, 1)
@@ -1028,7 +1035,7 @@ def main():
     if args.workload == "spmv" and not args.no_extras:
         from numml_amd import _binding
         keep = ("value", "unit", "ms_per_step", "steps", "warmup", "higher_is_better", "dtype", "config",
-                "roofline", "roofline_gather_inclusive", "cpu_baseline", "pct_of_hbm_peak")
+                "roofline", "roofline_gather_inclusive", "cpu_baseline", "pct_of_hbm_peak", "value_note")
         out["workloads"] = {}
         for name in EXTRAS:
             _binding.ops.clear_plan_cache()
