@@ -189,7 +189,7 @@ def test_product_path_does_not_touch_the_oracle():
 
 
 def test_integration_snippet_runs():
-    # the "keep the reference's CPU path" block of INTEGRATION.md, executed as written against a
+    # the integration guide's "keep the reference's CPU path" block, executed as written against a
     # stand-in for the reference's compiled module
     import sys
     import types
