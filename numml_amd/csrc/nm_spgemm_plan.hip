@@ -50,6 +50,21 @@ constexpr uint8_t kNone = nm::kPlanNone;
 
 __device__ __forceinline__ void group_fence() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); }
 
+// p[i] and p[i + 1] with one request (these kernels are bound by the number of vector memory
+// instructions a wavefront issues, and a row's two pointers sit side by side).
+struct Pair64 { int64_t lo, hi; };
+struct Pair32 { int32_t lo, hi; };
+__device__ __forceinline__ Pair64 load_pair(const int64_t *p) {
+    typedef int64_t V __attribute__((ext_vector_type(2), aligned(8)));
+    const V v = *reinterpret_cast<const V *>(p);
+    return Pair64{v[0], v[1]};
+}
+__device__ __forceinline__ Pair32 load_pair(const int32_t *p) {
+    typedef int32_t V __attribute__((ext_vector_type(2), aligned(4)));
+    const V v = *reinterpret_cast<const V *>(p);
+    return Pair32{v[0], v[1]};
+}
+
 // ---- build -----------------------------------------------------------------------
 
 // Eight lanes per row of A: lane k takes the k-th entry of each B row the row names and finds
@@ -187,10 +202,10 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     const int k = threadIdx.x & (kCap - 1), g = threadIdx.x / kCap;
     const int64_t row = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + g;
     const bool live = row < rows;
-    const int64_t *pa = A_indptr + (live ? row : 0), *pc = C_indptr + (live ? row : 0);
-    const int64_t ab = pa[0], ae = live ? pa[1] : ab;
-    const int64_t cs = pc[0];
-    const int clen = live ? (int)(pc[1] - cs) : 0;
+    const Pair64 pa = load_pair(A_indptr + (live ? row : 0)), pc = load_pair(C_indptr + (live ? row : 0));
+    const int64_t ab = pa.lo, ae = live ? pa.hi : ab;
+    const int64_t cs = pc.lo;
+    const int clen = live ? (int)(pc.hi - cs) : 0;
     const int alen = (int)(ae - ab);
     T *acc = s_acc + g * kAccStride;
 #pragma unroll
@@ -229,12 +244,53 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
         }
         group_fence();
     }
+    if (COLS) {
 #pragma unroll
-    for (int q = 0; q < kCap; ++q)
-        if (k + kCap * q < clen) {
-            C_data[cs + k + kCap * q] = acc[k + kCap * q];
-            if (COLS) C_indices[cs + k + kCap * q] = (int64_t)ccol[k + kCap * q];
+        for (int q = 0; q < kCap; ++q)
+            if (k + kCap * q < clen) {
+                C_data[cs + k + kCap * q] = acc[k + kCap * q];
+                C_indices[cs + k + kCap * q] = (int64_t)ccol[k + kCap * q];
+            }
+    } else {
+        // W consecutive entries (16 bytes) per lane and request: a half or a quarter of the store
+        // instructions (256 -> 276 us without at cfg4)
+        constexpr int W = 16 / (int)sizeof(T);
+        typedef T VW __attribute__((ext_vector_type(W), aligned(sizeof(T))));
+#pragma unroll
+        for (int q = 0; q < kRowCap / (kCap * W); ++q) {
+            const int at = W * k + W * kCap * q;
+            if (at + W <= clen) {
+                VW v;
+#pragma unroll
+                for (int w = 0; w < W; ++w) v[w] = acc[at + w];
+                *reinterpret_cast<VW *>(C_data + cs + at) = v;
+            } else {
+#pragma unroll
+                for (int w = 0; w < W; ++w)
+                    if (at + w < clen) C_data[cs + at + w] = acc[at + w];
+            }
         }
+    }
+}
+
+// A row of C from its accumulators in LDS, by the eight lanes of its group: 16 bytes per lane and
+// request (a half or a quarter of the store instructions of one entry per lane).
+template <typename T>
+__device__ __forceinline__ void store_row(T *__restrict__ out, const T *acc, int clen, int k) {
+    constexpr int W = 16 / (int)sizeof(T);
+    typedef T VW __attribute__((ext_vector_type(W), aligned(sizeof(T))));
+    for (int at = W * k; at < clen; at += W * kCap) {
+        if (at + W <= clen) {
+            VW v;
+#pragma unroll
+            for (int w = 0; w < W; ++w) v[w] = acc[at + w];
+            *reinterpret_cast<VW *>(out + at) = v;
+        } else {
+#pragma unroll
+            for (int w = 0; w < W; ++w)
+                if (at + w < clen) out[at + w] = acc[at + w];
+        }
+    }
 }
 
 // The same for rows of A of any length (taken eight entries at a time) and rows of C of up to CAP
@@ -259,10 +315,10 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_long
     const int k = threadIdx.x & (kCap - 1), g = threadIdx.x / kCap;
     const int64_t row = nm::xcd_tile(blockIdx.x, ntiles_padded) * S::kGroups + g;
     const bool live = row < rows;
-    const int64_t *pa = A_indptr + (live ? row : 0), *pc = C_indptr + (live ? row : 0);
-    const int64_t ab = pa[0], ae = live ? pa[1] : ab;
-    const int64_t cs = pc[0];
-    const int clen = live ? (int)(pc[1] - cs) : 0;
+    const Pair64 pa = load_pair(A_indptr + (live ? row : 0)), pc = load_pair(C_indptr + (live ? row : 0));
+    const int64_t ab = pa.lo, ae = live ? pa.hi : ab;
+    const int64_t cs = pc.lo;
+    const int clen = live ? (int)(pc.hi - cs) : 0;
     T *acc = s_acc + g * S::kStride;
     for (int d = k; d < clen; d += kCap) acc[d] = T(0);
     const int slot = g * kCap;
@@ -291,7 +347,7 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_long
             group_fence();
         }
     }
-    for (int d = k; d < clen; d += kCap) C_data[cs + d] = acc[d];
+    store_row(C_data + cs, acc, clen, k);
 }
 
 // The same for products whose named rows of B have up to 8 * OCT entries (classes 4 and 5): an entry
@@ -311,10 +367,10 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_wide
     const int k = threadIdx.x & (kCap - 1), g = threadIdx.x / kCap;
     const int64_t row = nm::xcd_tile(blockIdx.x, ntiles_padded) * S::kGroups + g;
     const bool live = row < rows;
-    const int64_t *pa = A_indptr + (live ? row : 0), *pc = C_indptr + (live ? row : 0);
-    const int64_t ab = pa[0], ae = live ? pa[1] : ab;
-    const int64_t cs = pc[0];
-    const int clen = live ? (int)(pc[1] - cs) : 0;
+    const Pair64 pa = load_pair(A_indptr + (live ? row : 0)), pc = load_pair(C_indptr + (live ? row : 0));
+    const int64_t ab = pa.lo, ae = live ? pa.hi : ab;
+    const int64_t cs = pc.lo;
+    const int clen = live ? (int)(pc.hi - cs) : 0;
     T *acc = s_acc + g * S::kStride;
     for (int d = k; d < clen; d += kCap) acc[d] = T(0);
     const int slot = g * kCap;
@@ -349,7 +405,7 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_wide
             }
         }
     }
-    for (int d = k; d < clen; d += kCap) C_data[cs + d] = acc[d];
+    store_row(C_data + cs, acc, clen, k);
 }
 
 // ---- backward ------------------------------------------------------------------------
@@ -410,10 +466,10 @@ __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     const int k = threadIdx.x & (kCap - 1), slot = threadIdx.x & ~(kCap - 1);
     const int64_t j = nm::xcd_tile(blockIdx.x, ntiles_padded) * kGroupsPerBlock + threadIdx.x / kCap;
     const bool live = j < B_rows;
-    const int64_t *pb_ = B_indptr + (live ? j : 0);
-    const int64_t bb = pb_[0], blen = live ? pb_[1] - bb : 0;
-    const int32_t *pt = t_indptr + (live ? j : 0);
-    const int32_t pb = pt[0], pe = live ? pt[1] : pb;
+    const Pair64 pb_ = load_pair(B_indptr + (live ? j : 0));
+    const int64_t bb = pb_.lo, blen = live ? pb_.hi - bb : 0;
+    const Pair32 pt = load_pair(t_indptr + (live ? j : 0));
+    const int32_t pb = pt.lo, pe = live ? pt.hi : pb;
     if (pb == pe) {   // no entry of A in this column: the row's gradient is zero, however long the row
         for (int64_t q = k; q < blen; q += kCap) grad_B[bb + q] = T(0);
         return;       // (no workgroup barrier anywhere in this kernel)
@@ -505,10 +561,10 @@ __global__ __launch_bounds__(kBlock) void grad_b_wide_kernel(
     const int64_t j = gid / OCT;
     const int o = (int)(gid % OCT);
     const bool live = j < B_rows;
-    const int64_t *pb_ = B_indptr + (live ? j : 0);
-    const int64_t bb = pb_[0], blen = live ? pb_[1] - bb : 0;
-    const int32_t *pt = t_indptr + (live ? j : 0);
-    const int32_t pb = pt[0], pe = live ? pt[1] : pb;
+    const Pair64 pb_ = load_pair(B_indptr + (live ? j : 0));
+    const int64_t bb = pb_.lo, blen = live ? pb_.hi - bb : 0;
+    const Pair32 pt = load_pair(t_indptr + (live ? j : 0));
+    const int32_t pb = pt.lo, pe = live ? pt.hi : pb;
     if (pb == pe) {   // no entry of A in this column: the row's gradient is zero, however long the row
         if (kCap * o + k < blen) grad_B[bb + kCap * o + k] = T(0);
         if (o == 0)
@@ -584,10 +640,10 @@ __global__ __launch_bounds__(kBlock) void grad_ab_mapped_kernel(
     }
     const int64_t j = tile * kGroupsPerBlock + threadIdx.x / kCap;
     const bool live = j < B_rows;
-    const int64_t *pb_ = B_indptr + (live ? j : 0);
-    const int64_t bb = pb_[0], blen = live ? pb_[1] - bb : 0;
-    const int32_t *pt = t_indptr + (live ? j : 0);
-    const int32_t pb = pt[0], pe = live ? pt[1] : pb;
+    const Pair64 pb_ = load_pair(B_indptr + (live ? j : 0));
+    const int64_t bb = pb_.lo, blen = live ? pb_.hi - bb : 0;
+    const Pair32 pt = load_pair(t_indptr + (live ? j : 0));
+    const int32_t pb = pt.lo, pe = live ? pt.hi : pb;
     if (pb == pe) {   // no entry of A in this column: the row's gradient is zero, however long the row
         for (int64_t q = k; q < blen; q += kCap) grad_B[bb + q] = T(0);
         return;       // (no workgroup barrier anywhere in this kernel)
