@@ -52,6 +52,7 @@ __device__ __forceinline__ void group_fence() { __builtin_amdgcn_fence(__ATOMIC_
 
 // p[i] and p[i + 1] with one request (these kernels are bound by the number of vector memory
 // instructions a wavefront issues, and a row's two pointers sit side by side).
+typedef uint32_t U4 __attribute__((ext_vector_type(4)));
 struct Pair64 { int64_t lo, hi; };
 struct Pair32 { int32_t lo, hi; };
 __device__ __forceinline__ Pair64 load_pair(const int64_t *p) {
@@ -157,8 +158,18 @@ __global__ __launch_bounds__(kBlock) void plan_by_column_kernel(int64_t A_nnz, c
     uint64_t *t_dest64 = reinterpret_cast<uint64_t *>(p.t_dest);
     for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < A_nnz; t += stride) {
         const int64_t e = t_perm[t];
-        p.t_cstart[t] = p.cstart[e];
+        const int32_t cs = p.cstart[e];
+        p.t_cstart[t] = cs;
         for (int o = 0; o < octets; ++o) t_dest64[t * octets + o] = dest64[e * octets + o];
+        if (octets == 1) {
+            const uint64_t d = dest64[e];
+            U4 r;
+            r[0] = (uint32_t)e;
+            r[1] = (uint32_t)cs;
+            r[2] = (uint32_t)d;
+            r[3] = (uint32_t)(d >> 32);
+            reinterpret_cast<U4 *>(p.t_rec)[t] = r;
+        }
     }
 }
 
@@ -458,8 +469,8 @@ __global__ __launch_bounds__(kBlock) void grad_a_mapped_kernel(
 template <typename T>
 __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
     int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
-    const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm, const int64_t *__restrict__ B_indptr,
-    const int32_t *__restrict__ t_cstart, const uint8_t *__restrict__ t_dest, T *__restrict__ grad_B) {
+    const int32_t *__restrict__ t_indptr, const int64_t *__restrict__ B_indptr,
+    const uint32_t *__restrict__ t_rec, T *__restrict__ grad_B) {
     __shared__ T s_a[kBlock];
     __shared__ int32_t s_cs[kBlock];
     __shared__ __align__(8) uint8_t s_db[kBlock * kCap];
@@ -481,10 +492,11 @@ __global__ __launch_bounds__(kBlock) void grad_b_mapped_kernel(
         {
             const bool have = t0 + k < pe;
             const int32_t t = have ? t0 + k : pb;
-            s_a[threadIdx.x] = A_data[t_perm[t]];
-            s_cs[threadIdx.x] = t_cstart[t];
+            const U4 rec = reinterpret_cast<const U4 *>(t_rec)[t];   // position, row start of C, destinations
+            s_a[threadIdx.x] = A_data[rec[0]];
+            s_cs[threadIdx.x] = (int32_t)rec[1];
             *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) =
-                have ? *reinterpret_cast<const uint64_t *>(t_dest + (int64_t)t * kCap) : ~uint64_t(0);
+                have ? ((uint64_t)rec[3] << 32) | rec[2] : ~uint64_t(0);
         }
         group_fence();
         uint8_t db[kCap];
@@ -608,9 +620,9 @@ __global__ __launch_bounds__(kBlock) void grad_b_wide_kernel(
 template <typename T>
 __global__ __launch_bounds__(kBlock) void grad_ab_mapped_kernel(
     int64_t B_rows, int64_t ntiles_padded, const T *__restrict__ gC, const T *__restrict__ A_data,
-    const T *__restrict__ B_data, const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_perm,
-    const int64_t *__restrict__ B_indptr, const int32_t *__restrict__ t_cstart, const uint8_t *__restrict__ t_dest,
-    T *__restrict__ grad_A, T *__restrict__ grad_B, const int32_t *__restrict__ flag) {
+    const T *__restrict__ B_data, const int32_t *__restrict__ t_indptr, const int64_t *__restrict__ B_indptr,
+    const uint32_t *__restrict__ t_rec, T *__restrict__ grad_A, T *__restrict__ grad_B,
+    const int32_t *__restrict__ flag) {
     __shared__ T s_a[kBlock];
     __shared__ int32_t s_cs[kBlock];
     __shared__ __align__(8) uint8_t s_db[kBlock * kCap];
@@ -653,13 +665,14 @@ __global__ __launch_bounds__(kBlock) void grad_ab_mapped_kernel(
     T acc = T(0);
     for (int32_t t0 = pb; t0 < pe; t0 += kCap) {
         const bool have = t0 + k < pe;
-        const int32_t pos = t_perm[have ? t0 + k : pb];
+        // position in A's arrays, row start of C and destination bytes of the entry: one request
+        const U4 rec = reinterpret_cast<const U4 *>(t_rec)[have ? t0 + k : pb];
+        const int32_t pos = (int32_t)rec[0];
         {
-            const int32_t t = have ? t0 + k : pb;
             s_a[threadIdx.x] = A_data[pos];
-            s_cs[threadIdx.x] = t_cstart[t];
+            s_cs[threadIdx.x] = (int32_t)rec[1];
             *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) =
-                have ? *reinterpret_cast<const uint64_t *>(t_dest + (int64_t)t * kCap) : ~uint64_t(0);
+                have ? ((uint64_t)rec[3] << 32) | rec[2] : ~uint64_t(0);
         }
         group_fence();
         uint8_t db[kCap];
@@ -767,8 +780,8 @@ int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A
         const int64_t grid = nm::xcd_padded(nm::ceil_div(A_cols, (int64_t)kGroupsPerBlock));
         NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
         hipLaunchKernelGGL(grad_ab_mapped_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, grid,
-                           (const T *)gC, (const T *)A_data, (const T *)B_data, t.t_indptr, t.t_perm, B_indptr,
-                           p.t_cstart, p.t_dest, (T *)grad_A, (T *)grad_B, p.flag);
+                           (const T *)gC, (const T *)A_data, (const T *)B_data, t.t_indptr, B_indptr, p.t_rec,
+                           (T *)grad_A, (T *)grad_B, p.flag);
         NM_LAUNCH_CHECK("grad_ab_mapped_kernel");
         return NM_OK;
     }
@@ -783,8 +796,7 @@ int launch_backward(int64_t A_cols, int64_t A_nnz, const void *gC, const void *A
         const int64_t grid = nm::xcd_padded(nm::ceil_div(A_cols, (int64_t)kGroupsPerBlock));
         NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
         hipLaunchKernelGGL(grad_b_mapped_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, A_cols, grid,
-                           (const T *)gC, (const T *)A_data, t.t_indptr, t.t_perm, B_indptr, p.t_cstart, p.t_dest,
-                           (T *)grad_B);
+                           (const T *)gC, (const T *)A_data, t.t_indptr, B_indptr, p.t_rec, (T *)grad_B);
         NM_LAUNCH_CHECK("grad_b_mapped_kernel");
     }
     return NM_OK;
