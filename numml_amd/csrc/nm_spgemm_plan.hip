@@ -159,9 +159,10 @@ __global__ __launch_bounds__(kBlock) void plan_by_column_kernel(int64_t A_nnz, c
     for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < A_nnz; t += stride) {
         const int64_t e = t_perm[t];
         const int32_t cs = p.cstart[e];
-        p.t_cstart[t] = cs;
-        for (int o = 0; o < octets; ++o) t_dest64[t * octets + o] = dest64[e * octets + o];
-        if (octets == 1) {
+        if (octets > 1) {
+            p.t_cstart[t] = cs;
+            for (int o = 0; o < octets; ++o) t_dest64[t * octets + o] = dest64[e * octets + o];
+        } else {
             const uint64_t d = dest64[e];
             U4 r;
             r[0] = (uint32_t)e;
@@ -169,6 +170,14 @@ __global__ __launch_bounds__(kBlock) void plan_by_column_kernel(int64_t A_nnz, c
             r[2] = (uint32_t)d;
             r[3] = (uint32_t)(d >> 32);
             reinterpret_cast<U4 *>(p.t_rec)[t] = r;
+            // (entry t of this loop as a row-major entry: every entry is some t)
+            const uint64_t dr = dest64[t];
+            U4 q;
+            q[0] = (uint32_t)p.bstart[t];
+            q[1] = (uint32_t)p.cstart[t];
+            q[2] = (uint32_t)dr;
+            q[3] = (uint32_t)(dr >> 32);
+            reinterpret_cast<U4 *>(p.rec)[t] = q;
         }
     }
 }
@@ -204,7 +213,7 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     int64_t rows, int64_t ntiles_padded, const T *__restrict__ A_data, const int64_t *__restrict__ A_indptr,
     const T *__restrict__ B_data, const int64_t *__restrict__ B_indices, const int32_t *__restrict__ bstart,
     const uint8_t *__restrict__ dest, const int64_t *__restrict__ C_indptr, T *__restrict__ C_data,
-    int64_t *__restrict__ C_indices, int32_t *__restrict__ cstart) {
+    int64_t *__restrict__ C_indices, int32_t *__restrict__ cstart, const uint32_t *__restrict__ rec) {
     __shared__ T s_acc[kGroupsPerBlock * kAccStride];
     __shared__ int32_t s_ccol[COLS ? kGroupsPerBlock * kAccStride : 1];
     __shared__ T s_av[kBlock];                       // per group: the row's entries of A ...
@@ -225,8 +234,16 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     {   // lane k of the group fetches entry k of the row
         const int64_t e = k < alen ? ab + k : 0;   // entry 0: readable whenever the matrix has entries
         const T av = A_data[e];
-        const int32_t bs = bstart[e];
-        const uint64_t db = *reinterpret_cast<const uint64_t *>(dest + e * kCap);
+        int32_t bs;
+        uint64_t db;
+        if (COLS) {   // the plan is still being filled: its separate arrays
+            bs = bstart[e];
+            db = *reinterpret_cast<const uint64_t *>(dest + e * kCap);
+        } else {      // a finished plan: row start of B and destination bytes in one request
+            const U4 r = reinterpret_cast<const U4 *>(rec)[e];
+            bs = (int32_t)r[0];
+            db = ((uint64_t)r[3] << 32) | r[2];
+        }
         s_av[threadIdx.x] = av;
         s_bs[threadIdx.x] = bs;
         *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) = k < alen ? db : ~uint64_t(0);
@@ -963,11 +980,11 @@ extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int plan_class, int64_t A_
     if (dt == NM_F32)
         hipLaunchKernelGGL((numeric_planned_kernel<float, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            grid, (const float *)A_data, A_indptr, (const float *)B_data, (const int64_t *)nullptr,
-                           p.bstart, p.dest, C_indptr, (float *)C_data, (int64_t *)nullptr, (int32_t *)nullptr);
+                           p.bstart, p.dest, C_indptr, (float *)C_data, (int64_t *)nullptr, (int32_t *)nullptr, p.rec);
     else
         hipLaunchKernelGGL((numeric_planned_kernel<double, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            grid, (const double *)A_data, A_indptr, (const double *)B_data, (const int64_t *)nullptr,
-                           p.bstart, p.dest, C_indptr, (double *)C_data, (int64_t *)nullptr, (int32_t *)nullptr);
+                           p.bstart, p.dest, C_indptr, (double *)C_data, (int64_t *)nullptr, (int32_t *)nullptr, p.rec);
     NM_LAUNCH_CHECK("numeric_planned_kernel");
     return NM_OK;
 }
@@ -981,11 +998,11 @@ int nm::spgemm_numeric_on_map(nm_dtype dt, int64_t A_rows, int64_t A_nnz, const 
     if (dt == NM_F32)
         hipLaunchKernelGGL((numeric_planned_kernel<float, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            grid, (const float *)A_data, A_indptr, (const float *)B_data, B_indices, p.bstart, p.dest,
-                           C_indptr, (float *)C_data, C_indices, p.cstart);
+                           C_indptr, (float *)C_data, C_indices, p.cstart, (const uint32_t *)nullptr);
     else
         hipLaunchKernelGGL((numeric_planned_kernel<double, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            grid, (const double *)A_data, A_indptr, (const double *)B_data, B_indices, p.bstart, p.dest,
-                           C_indptr, (double *)C_data, C_indices, p.cstart);
+                           C_indptr, (double *)C_data, C_indices, p.cstart, (const uint32_t *)nullptr);
     NM_LAUNCH_CHECK("numeric_planned_kernel");
     return NM_OK;
 }

@@ -24,13 +24,16 @@ struct PPlan {
                        // that row of B
     // cstart and dest once more in COLUMN-major order of A (entry t of the transposed-structure
     // plan): the kernel that walks A by column streams them instead of gathering 12 bytes from a
-    // different line for every entry.  Filled when the plan is built or adopted.
+    // different line for every entry.  Filled when the plan is built or adopted.  Plans of two and
+    // four octets only (one-octet plans have t_rec instead).
     int32_t *t_cstart; // [A_nnz]
     uint8_t *t_dest;   // [A_nnz * 8 * octets]
     // one-octet plans: what the walk by column wants of entry t in ONE 16-byte record --
     // {position in A's arrays (t_perm), t_cstart, the eight destination bytes} -- so that a lane
     // fetches it with one request instead of three
     uint32_t *t_rec;   // [A_nnz * 4]
+    // the same for the walk by row: {bstart, cstart, the eight destination bytes} of entry e
+    uint32_t *rec;     // [A_nnz * 4]
 };
 
 // octets: 1 for products whose named rows of B have at most 8 entries, 2 for up to 16, 4 for up to 32
@@ -45,10 +48,11 @@ inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p, int octets = 1) 
     int32_t *bs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
     int32_t *cs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
     uint8_t *d = (uint8_t *)take((size_t)(A_nnz + 1) * 8 * octets);
-    int32_t *tcs = (int32_t *)take((size_t)(A_nnz + 1) * 4);
-    uint8_t *td = (uint8_t *)take((size_t)(A_nnz + 1) * 8 * octets);
+    int32_t *tcs = octets > 1 ? (int32_t *)take((size_t)(A_nnz + 1) * 4) : nullptr;
+    uint8_t *td = octets > 1 ? (uint8_t *)take((size_t)(A_nnz + 1) * 8 * octets) : nullptr;
     uint32_t *tr = octets == 1 ? (uint32_t *)take((size_t)(A_nnz + 1) * 16) : nullptr;
-    if (p) *p = PPlan{flag, bs, cs, d, tcs, td, tr};
+    uint32_t *rr = octets == 1 ? (uint32_t *)take((size_t)(A_nnz + 1) * 16) : nullptr;
+    if (p) *p = PPlan{flag, bs, cs, d, tcs, td, tr, rr};
     return off;
 }
 
