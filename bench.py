@@ -429,11 +429,13 @@ class SpGEMM(Workload):
         self.dominant_bytes = self.bytes_per_step
         self.dominant_name = "spgemm forward (symbolic + numeric launches, host read of nnz(C) included)"
         if self.planned:
-            # forward on the product plan: values of both operands, 12 bytes of plan per entry of
-            # the left operand (row start in B, eight destination bytes), both row pointer arrays,
-            # the values of C; the pattern of C is the plan's and is not written again
-            # (rows of the right operand of 17 to 32 entries: four octets of destination bytes)
-            plan_bytes = 4 + 8 * (4 if self.right == "AA" else 1)
+            # forward on the product plan: values of both operands, one 16-byte record of plan per
+            # entry of the left operand (row start in B, row start in C, eight destination bytes),
+            # both row pointer arrays, the values of C; the pattern of C is the plan's and is not
+            # written again
+            # (rows of the right operand of 17 to 32 entries: row start and four octets of
+            # destination bytes from separate arrays)
+            plan_bytes = 4 + 8 * 4 if self.right == "AA" else 16
             self.bytes_per_step = self.nnz * (s + plan_bytes) + nnzR * s + self.nnzC * s + 2 * rows * 8
             self.dominant_bytes = self.bytes_per_step
             self.dominant_name = ("numeric_planned_wide_kernel (the whole forward on the product plan)"
