@@ -217,6 +217,31 @@ def test_cfg4_matrix_in_fp32(dev):
     assert_same(host(Cd2), Cd_ref, "C_data on the product plan")
 
 
+def test_cfg4_pattern_times_its_square(dev):
+    """A (A A) on a 64^3 grid: named rows of B of 25 entries, rows of C of 63 -- the four-octet product
+    plan on a few thousand workgroups (the small cases cover a handful)."""
+    d, i, p, (rows, cols) = G.laplace3d(64, np.float64, jitter_seed=3)
+    D, I, P = to_dev(dev, d, i, p)
+    Sd, Si, Sp = ext.spgemm_forward(rows, cols, D, I, P, rows, cols, D, I, P)
+    sd, si, sp_ = host(Sd), host(Si), host(Sp)
+    assert int(np.diff(sp_).max()) == 25
+    Cd, Ci, Cp = ext.spgemm_forward(rows, cols, D, I, P, rows, cols, Sd, Si, Sp)
+    Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(rows, cols, d, i, p, rows, cols, sd, si, sp_)
+    assert int(np.diff(Cp_ref).max()) == 63
+    assert_same(host(Cp), Cp_ref, "C_indptr")
+    assert_same(host(Ci), Ci_ref, "C_indices")
+    assert_same(host(Cd), Cd_ref, "C_data")
+    # again: the planned numeric kernel alone, on the plan's pattern tensors
+    Cd2, Ci2, Cp2 = ext.spgemm_forward(rows, cols, D, I, P, rows, cols, Sd, Si, Sp)
+    assert Ci2.data_ptr() == Ci.data_ptr() and Cp2.data_ptr() == Cp.data_ptr()
+    assert_same(host(Cd2), Cd_ref, "C_data on the product plan")
+    gC = randn(4, Cd_ref.shape[0], np.float64)
+    gA, gB = ext.spgemm_backward(to_dev(dev, gC)[0], Ci, Cp, rows, cols, D, I, P, rows, cols, Sd, Si, Sp)
+    gA_ref, gB_ref = oracle.spgemm_backward(gC, Ci_ref, Cp_ref, rows, cols, d, i, p, rows, cols, sd, si, sp_)
+    assert_same(host(gA), gA_ref, "grad_A")
+    assert_same(host(gB), gB_ref, "grad_B")
+
+
 def test_cfg5_matrix_in_fp32(dev):
     d, i, p, (n, _) = G.poisson2d_lower(1024, np.float32, diag_seed=0)
     b, g = randn(1, n, np.float32), randn(2, n, np.float32)
