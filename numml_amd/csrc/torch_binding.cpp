@@ -380,12 +380,20 @@ std::shared_ptr<Plan> transpose_plan(const Tensor &indices, const Tensor &indptr
     });
 }
 
+// A transposed-structure plan keeps rows, columns and positions in 32 bits
+// (nm_csr_transpose_plan_bytes refuses more); larger matrices run the stateless kernels, which
+// take 64-bit offsets throughout.
+bool fits_a_plan(int64_t rows, int64_t cols, int64_t nnz) {
+    const int64_t lim = 0x7ffffffe;
+    return rows < lim && cols < lim && nnz < lim;
+}
+
 // The transposed-structure plan a backward pass should use under the current mode, or nullptr
 // for the stateless kernels.
 std::shared_ptr<Plan> backward_plan(const Tensor &indices, const Tensor &indptr, int64_t rows, int64_t cols,
                                     const c10::Device &dev) {
     const int mode = backward_mode_now();
-    if (mode == kAtomic) return nullptr;
+    if (mode == kAtomic || !fits_a_plan(rows, cols, indices.numel())) return nullptr;
     return transpose_plan(indices, indptr, rows, cols, dev, mode == kPlanned);
 }
 
@@ -460,6 +468,9 @@ void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, cons
                            const Tensor &filled = Tensor()) {
     const int mode = backward_mode_now();
     if (mode == kAtomic || A_indices.numel() == 0 || C_indices.numel() == 0) return;
+    if (!fits_a_plan(A_rows, A_cols, A_indices.numel()) || !fits_a_plan(A_cols, B_cols, B_indices.numel()) ||
+        !fits_a_plan(A_rows, B_cols, C_indices.numel()))
+        return;
     Key ka, kb;
     structure_key(A_indices, A_indptr, true, &ka);
     structure_key(B_indices, B_indptr, true, &kb);

@@ -178,6 +178,13 @@ class _TransposePlan:
         # work enqueued later on this same stream
 
 
+def _fits_a_plan(rows, cols, nnz):
+    """A transposed-structure plan keeps rows, columns and positions in 32 bits; larger matrices
+    run the stateless kernels, which take 64-bit offsets throughout."""
+    lim = 0x7ffffffe
+    return rows < lim and cols < lim and nnz < lim
+
+
 def _transpose_plan(indices, indptr, rows, cols, dev):
     plan = _cached("T", indices, indptr, (rows, cols),
                    lambda: _TransposePlan(indices, indptr, rows, cols, dev))
@@ -219,7 +226,7 @@ def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_x = torch.empty_like(x)
-        if BACKWARD_MODE != "atomic":
+        if BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, x.shape[0], A_data.shape[0]):
             plan = _transpose_plan(A_col_ind, A_rowptr, A_rows, x.shape[0], dev)
             _lib.check(_lib.lib().nm_spgemv_backward_planned(
                 _dt(A_data), A_rows, x.shape[0], A_data.shape[0], _ptr(A_data), _ptr(plan.mem), _ptr(x),
@@ -449,7 +456,7 @@ def spdmm_backward(A_rows, A_cols, A_data, A_indices, A_indptr, B, grad_C):
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_B = torch.empty((B.shape[0], n), dtype=B.dtype, device=dev)
-        if BACKWARD_MODE != "atomic":
+        if BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, B.shape[0], A_data.shape[0]):
             plan = _transpose_plan(A_indices, A_indptr, A_rows, B.shape[0], dev)
             _lib.check(_lib.lib().nm_spdmm_backward_planned(
                 _dt(A_data), A_rows, B.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_indices),
@@ -537,7 +544,7 @@ def spgemm_backward(grad_C, C_indices, C_indptr,
     with torch.cuda.device(dev):
         grad_A = torch.empty_like(A_data)
         grad_B = torch.empty_like(B_data)
-        if BACKWARD_MODE != "atomic":
+        if BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, A_cols, A_data.shape[0]):
             plan = _transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev)
             _lib.check(_lib.lib().nm_spgemm_backward_planned(
                 _dt(A_data), A_rows, A_cols, A_data.shape[0], B_data.shape[0], grad_C.shape[0], _ptr(grad_C),
