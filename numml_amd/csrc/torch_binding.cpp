@@ -1135,7 +1135,13 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
     const int mode = backward_mode_now();
     const double mean_c = A_rows > 0 ? (double)grad_C.numel() / A_rows : 0.;
     const double mean_b = B_rows > 0 ? (double)B_data.numel() / B_rows : 0.;
-    const bool on_plan = mode == kEager || (mode == kPlanned && mean_c <= 4. * std::max(mean_b, 1.));
+    // It also shares the work out by row of B and hands a row whose products (its entries times the
+    // entries of A's column) run into the thousands to a single workgroup: where that is the average
+    // row, the stateless kernel is many times faster (2 M rows of A naming 16 rows of B: 8 ms against
+    // seconds).
+    const double mean_col = A_cols > 0 ? (double)A_data.numel() / A_cols : 0.;
+    const bool on_plan = mode == kEager ||
+                         (mode == kPlanned && mean_c <= 4. * std::max(mean_b, 1.) && mean_b * mean_col <= 4096.);
     if (auto plan = on_plan ? backward_plan(A_indices, A_indptr, A_rows, A_cols, dev) : nullptr) {
         check(nm_spgemm_backward_planned(dtype_of(A_data), A_rows, A_cols, A_data.numel(), B_data.numel(),
                                          grad_C.numel(), grad_C.data_ptr(), C_indices.data_ptr<int64_t>(),

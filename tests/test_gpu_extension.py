@@ -323,6 +323,40 @@ def test_product_plan_policy(dev, cpp):
     cpp.clear_plan_cache()
 
 
+def test_default_mode_keeps_heavy_rows_of_the_right_operand_off_the_planned_backward(dev, cpp):
+    """The plan-based backward gives a row of B to a group of lanes, a heavy one (its entries times
+    the entries of A's column in the thousands) to one workgroup: where the AVERAGE row is that
+    heavy the default mode stays with the stateless kernels, however often the pattern is seen;
+    "eager" still takes the plan."""
+    dtype = np.float32
+    rows = 6000
+    ai = (np.arange(rows) % 2).astype(np.int64)               # 3000 entries in each of A's two columns
+    ap = np.arange(rows + 1, dtype=np.int64)
+    ad = randn(80, rows, dtype)
+    bd, bi, bp, _ = G.ragged_csr(2, 300, 40, 81, dtype, min_len=40)
+    AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+    cd, ci, cp = oracle.spgemm_forward(rows, 2, ad, ai, ap, 2, 300, bd, bi, bp)
+    g = randn(82, cd.shape[0], dtype)
+    rA, rB = oracle.spgemm_backward(g, ci, cp, rows, 2, ad, ai, ap, 2, 300, bd, bi, bp)
+    Gd, CI, CP = to_dev(dev, g, ci, cp)
+    cpp.clear_plan_cache()
+    try:
+        cpp.set_backward_mode("planned")
+        for _ in range(3):
+            gA, gB = cpp.spgemm_backward(Gd, CI, CP, rows, 2, AD, AI, AP, 2, 300, BD, BI, BP)
+            assert_same(host(gA), rA, "grad_A")
+            assert_close(host(gB), rB, "grad_B (atomics)")
+        assert cpp.plan_cache_size() == 0
+        cpp.set_backward_mode("eager")
+        gA, gB = cpp.spgemm_backward(Gd, CI, CP, rows, 2, AD, AI, AP, 2, 300, BD, BI, BP)
+        assert cpp.plan_cache_size() == 1
+        assert_same(host(gA), rA, "grad_A on the plan")
+        assert_close(host(gB), rB, "grad_B on the plan (heavy rows: tree order)")
+    finally:
+        cpp.set_backward_mode("planned")
+        cpp.clear_plan_cache()
+
+
 def test_product_plan_for_rows_of_the_right_operand_of_up_to_32_entries(dev, cpp):
     """A (A A) on a 3D grid -- the right operand has 25-entry rows, so the product takes the hash path --
     in a loop with new values: the first call is stateless, the second leaves a product plan with four
