@@ -35,6 +35,19 @@ def _with_dense_columns(dtype):
     return data, rc[:, 1].astype(np.int64), indptr, (rows, cols)
 
 
+def _arrowhead(dtype, n=200_003):
+    """Diagonal, dense first row, dense first column: one column of n entries (some fifty pieces of
+    LDS keys and six merge passes in the ordering kernel, by a workgroup of its own)."""
+    r = np.concatenate([np.arange(n), np.zeros(n - 1, np.int64), np.arange(1, n)])
+    c = np.concatenate([np.arange(n), np.arange(1, n), np.zeros(n - 1, np.int64)])
+    order = np.lexsort((c, r))
+    r, c = r[order], c[order]
+    indptr = np.zeros(n + 1, np.int64)
+    np.cumsum(np.bincount(r, minlength=n), out=indptr[1:])
+    data = np.random.default_rng(12).standard_normal(r.shape[0]).astype(dtype)
+    return data, c.astype(np.int64), indptr, (n, n)
+
+
 def _with_duplicates(dtype):
     """Stored entries with equal coordinates (the container keeps them, numml/sparse/_csr.py:78-99):
     the transpose must keep their storage order."""
@@ -52,6 +65,7 @@ def _cases(dtype):
     yield "empty_rows_cols", G.random_csr(120, 130, 0.01, 3, dtype)
     yield "powerlaw", G.powerlaw(3000, 2500, 40000, max_deg=1200, seed=4, dtype=dtype)
     yield "dense_columns", _with_dense_columns(dtype)
+    yield "arrowhead", _arrowhead(dtype)
     yield "duplicates", _with_duplicates(dtype)
     yield "no_entries", (np.zeros(0, dtype), np.zeros(0, np.int64), np.zeros(6, np.int64), (5, 7))
     yield "one", (np.ones(1, dtype), np.zeros(1, np.int64), np.array([0, 1], np.int64), (1, 1))
