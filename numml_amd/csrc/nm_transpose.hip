@@ -35,7 +35,7 @@ using nm::kWave;
 constexpr int kBlock = 256;
 constexpr int kRows = 512;      // rows (columns) a workgroup stages offsets for
 constexpr int kCap = 4096;      // LDS keys of the ordering kernel
-constexpr int kSlice = 16;      // consecutive outputs one lane produces in a merge pass
+constexpr int kSlice = 8;       // consecutive outputs one lane produces in a merge pass
 
 struct WorkT {
     int64_t *count;        // [cols + 1] per-column counters, then column pointers
@@ -184,14 +184,17 @@ __device__ void merge_pass(const int32_t *__restrict__ src, int32_t *__restrict_
 // Step 4.  A workgroup owns `ct` consecutive columns.  `cols_dev`, when given, holds the number of
 // columns on the device (a caller that does not know it on the host yet); rowid / t_row may be null
 // (keys are then only put in order).
+// LONG: only the columns longer than the LDS keys (their code needs twice the registers, which would
+// halve the wavefronts of every launch; a pattern without such columns passes through this
+// instantiation on its column pointers alone); otherwise only the others.
+template <bool LONG>
 __global__ __launch_bounds__(kBlock) void tp_order_kernel(
     int64_t cols, const int32_t *__restrict__ cols_dev, int ct, const int32_t *__restrict__ t_indptr,
     int32_t *__restrict__ t_perm, const int32_t *__restrict__ rowid, int32_t *__restrict__ t_row,
     int32_t *__restrict__ tmp) {
     __shared__ int32_t s_off[kRows + 1];
     __shared__ __align__(16) int32_t s_key[kCap];
-    __shared__ int32_t s_alt[kCap];   // second run of a merge pass
-    static_assert(kSlice * kBlock == kCap, "a lane's kSlice candidates of either run fit the LDS keys");
+    static_assert(2 * kSlice * kBlock == kCap, "a lane's kSlice candidates of both runs fit the LDS keys");
     if (cols_dev) cols = *cols_dev;
     const int64_t ntiles = (cols + ct - 1) / ct, npad = nm::xcd_padded(ntiles);
     for (int64_t id = blockIdx.x; id < npad; id += gridDim.x) {
@@ -228,8 +231,12 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
         for (int s0 = 0; s0 < nc;) {
             const int e0 = run_end(s_off, s0, nc, kCap);
             if (e0 > s0) {
-                ranked(s0, e0);
+                if (!LONG) ranked(s0, e0);
                 s0 = e0;
+                continue;
+            }
+            if (!LONG) {
+                s0 += 1;
                 continue;
             }
             // One column longer than the LDS keys.  Pieces of kCap keys are ranked in LDS and
@@ -245,7 +252,7 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
                 // a lane ranks its kCap / kBlock keys together: every staged key is read once
                 // (four to an LDS read) and compared with all of them -- independent additions,
                 // where one key at a time waited for LDS at every step (ordering a column of 2^20
-                // entries: 866 -> 108 ms together with the merge passes' LDS staging)
+                // entries: 866 ms -> about 0.1 s together with the merge passes' LDS staging)
                 constexpr int KPL = kCap / kBlock;
                 typedef int32_t I4 __attribute__((ext_vector_type(4)));
                 int32_t key[KPL];
@@ -270,7 +277,7 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
             }
             int32_t *src = alt, *dst = col;
             for (int width = kCap; width < len; width *= 2) {
-                merge_pass(src, dst, len, width, s_key, s_alt);
+                merge_pass(src, dst, len, width, s_key, s_key + kSlice * kBlock);
                 __syncthreads();
                 int32_t *sw = src; src = dst; dst = sw;
             }
@@ -392,9 +399,12 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
         const int ct = tile_rows(cols, nnz, 1);
         grid = xcd_padded(ceil_div(cols, ct));
         if (grid > 65536) grid = 65536;
-        hipLaunchKernelGGL(tp_order_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, (const int32_t *)nullptr, ct,
-                           plan.t_indptr, plan.t_perm, rowid, plan.t_row, w.tmp);
+        hipLaunchKernelGGL(tp_order_kernel<false>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, (const int32_t *)nullptr,
+                           ct, plan.t_indptr, plan.t_perm, rowid, plan.t_row, w.tmp);
         NM_LAUNCH_CHECK("tp_order_kernel");
+        hipLaunchKernelGGL(tp_order_kernel<true>, dim3((unsigned)grid), dim3(kBlock), 0, s, cols, (const int32_t *)nullptr,
+                           ct, plan.t_indptr, plan.t_perm, rowid, plan.t_row, w.tmp);
+        NM_LAUNCH_CHECK("tp_order_kernel<long>");
     }
     hipLaunchKernelGGL(symmetry_init_kernel, dim3(1), dim3(64), 0, s, plan.flags, rows == cols ? 1 : 0);
     if (rows == cols) {
@@ -422,9 +432,12 @@ int segments_sort_i32(const int32_t *nseg_dev, int64_t nseg_max, int64_t nkeys, 
     const int ct = 8;
     int64_t grid = xcd_padded(ceil_div(nseg_max, ct));
     if (grid > 8192) grid = 8192;
-    hipLaunchKernelGGL(tp_order_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, nseg_max, nseg_dev, ct, seg_ptr, keys,
-                       (const int32_t *)nullptr, (int32_t *)nullptr, tmp);
+    hipLaunchKernelGGL(tp_order_kernel<false>, dim3((unsigned)grid), dim3(kBlock), 0, s, nseg_max, nseg_dev, ct, seg_ptr,
+                       keys, (const int32_t *)nullptr, (int32_t *)nullptr, tmp);
     NM_LAUNCH_CHECK("tp_order_kernel (segments)");
+    hipLaunchKernelGGL(tp_order_kernel<true>, dim3((unsigned)grid), dim3(kBlock), 0, s, nseg_max, nseg_dev, ct, seg_ptr,
+                       keys, (const int32_t *)nullptr, (int32_t *)nullptr, tmp);
+    NM_LAUNCH_CHECK("tp_order_kernel<long> (segments)");
     return NM_OK;
 }
 
