@@ -818,22 +818,35 @@ __global__ __launch_bounds__(kBlock) void lincomb_map_kernel(int64_t rows, const
                                                              const int64_t *__restrict__ C_indices,
                                                              const int64_t *__restrict__ C_indptr,
                                                              int32_t *__restrict__ src, int32_t *__restrict__ pos) {
-    const int k = threadIdx.x & (kMapLanes - 1);
-    const int64_t stride = (int64_t)gridDim.x * (kBlock / kMapLanes);
-    for (int64_t row = (int64_t)blockIdx.x * (kBlock / kMapLanes) + threadIdx.x / kMapLanes; row < rows;
-         row += stride) {
-        const int64_t xb = X_indptr[row], xe = X_indptr[row + 1];
-        const int64_t cs = C_indptr[row], ce = C_indptr[row + 1];
-        for (int64_t e = xb + k; e < xe; e += kMapLanes) {
-            const int64_t col = X_indices[e];
-            int64_t lo = cs, hi = ce;
-            while (lo < hi) {
-                const int64_t mid = (lo + hi) >> 1;
-                if (C_indices[mid] < col) lo = mid + 1; else hi = mid;
+    constexpr int kGroups = kBlock / kMapLanes;
+    constexpr int64_t kLongMapRow = 2048;   // rows of X from here on are shared by the whole workgroup
+    const int k = threadIdx.x & (kMapLanes - 1), g = threadIdx.x / kMapLanes;
+    auto place = [&](const int64_t e, const int64_t cs, const int64_t ce) {
+        const int64_t col = X_indices[e];
+        int64_t lo = cs, hi = ce;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (C_indices[mid] < col) lo = mid + 1; else hi = mid;
+        }
+        const bool found = lo < ce && C_indices[lo] == col;   // always, when C is the union of the patterns
+        pos[e] = (int32_t)(found ? lo : (cs < ce ? cs : 0));
+        if (found) src[lo] = (int32_t)e;
+    };
+    for (int64_t row0 = (int64_t)blockIdx.x * kGroups; row0 < rows; row0 += (int64_t)gridDim.x * kGroups) {
+        const int64_t row = row0 + g;
+        if (row < rows) {
+            const int64_t xb = X_indptr[row], xe = X_indptr[row + 1];
+            if (xe - xb < kLongMapRow) {
+                const int64_t cs = C_indptr[row], ce = C_indptr[row + 1];
+                for (int64_t e = xb + k; e < xe; e += kMapLanes) place(e, cs, ce);
             }
-            const bool found = lo < ce && C_indices[lo] == col;   // always, when C is the union of the patterns
-            pos[e] = (int32_t)(found ? lo : (cs < ce ? cs : 0));
-            if (found) src[lo] = (int32_t)e;
+        }
+        // the long rows among these (eight lanes took 0.3 s over a row of 2^19 entries)
+        for (int g2 = 0; g2 < kGroups && row0 + g2 < rows; ++g2) {
+            const int64_t xb = X_indptr[row0 + g2], xe = X_indptr[row0 + g2 + 1];
+            if (xe - xb < kLongMapRow) continue;
+            const int64_t cs = C_indptr[row0 + g2], ce = C_indptr[row0 + g2 + 1];
+            for (int64_t e = xb + threadIdx.x; e < xe; e += kBlock) place(e, cs, ce);
         }
     }
 }
