@@ -256,25 +256,64 @@ __global__ void pack_kernel(int64_t rows, int eff_lower, int fill, const int32_t
                             int64_t *__restrict__ count64, const int32_t *__restrict__ dptr,
                             int32_t *__restrict__ dslot, int32_t *__restrict__ dsrc, int32_t *__restrict__ diag,
                             int32_t *max_deps) {
+    // rows of this many entries and more are walked by the wavefront, 64 entries at a time (one
+    // lane took a quarter of a second over a row of 2^19 entries)
+    constexpr int64_t kLongPackRow = 1024;
+    const int lane = threadIdx.x & 63;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < rows; q += stride) {
-        const int64_t i = order[q];
-        const int64_t kb = TR ? (int64_t)t_indptr[i] : indptr[i];
-        const int64_t ke = TR ? (int64_t)t_indptr[i + 1] : indptr[i + 1];
-        int64_t n = 0;
-        int32_t dpos = -1;
-        int32_t out = fill ? dptr[q] : 0;
-        for (int64_t e = 0; e < ke - kb; ++e) {
-            const int64_t k = eff_lower ? kb + e : ke - 1 - e;
-            const int64_t j = TR ? (int64_t)t_row[k] : indices[k];
-            const int32_t src = TR ? t_perm[k] : (int32_t)k;
-            if (j == i) { dpos = src; continue; }
-            if (eff_lower ? j > i : j < i) continue;   // other side of the diagonal: not part of the solve
-            if (fill) { dslot[out] = slot_of[j]; dsrc[out] = src; ++out; }
-            ++n;
+    // (q0 is the same for the lanes of a wavefront: they stay in the loop together)
+    for (int64_t q0 = (int64_t)blockIdx.x * blockDim.x + (threadIdx.x & ~63); q0 < rows; q0 += stride) {
+        const int64_t q = q0 + lane;
+        const bool live = q < rows;
+        const int64_t i = live ? order[q] : 0;
+        const int64_t kb = !live ? 0 : TR ? (int64_t)t_indptr[i] : indptr[i];
+        const int64_t ke = !live ? 0 : TR ? (int64_t)t_indptr[i + 1] : indptr[i + 1];
+        const int32_t out0 = live && fill ? dptr[q] : 0;
+        const bool shared = ke - kb >= kLongPackRow;
+        if (live && !shared) {
+            int64_t n = 0;
+            int32_t dpos = -1;
+            int32_t out = out0;
+            for (int64_t e = 0; e < ke - kb; ++e) {
+                const int64_t k = eff_lower ? kb + e : ke - 1 - e;
+                const int64_t j = TR ? (int64_t)t_row[k] : indices[k];
+                const int32_t src = TR ? t_perm[k] : (int32_t)k;
+                if (j == i) { dpos = src; continue; }
+                if (eff_lower ? j > i : j < i) continue;   // other side of the diagonal: not part of the solve
+                if (fill) { dslot[out] = slot_of[j]; dsrc[out] = src; ++out; }
+                ++n;
+            }
+            if (fill) { diag[q] = dpos; if (n > *max_deps) atomicMax(max_deps, (int32_t)(n > 0x7fffffff ? 0x7fffffff : n)); }
+            else count64[q] = n;
         }
-        if (fill) { diag[q] = dpos; if (n > *max_deps) atomicMax(max_deps, (int32_t)(n > 0x7fffffff ? 0x7fffffff : n)); }
-        else count64[q] = n;
+        for (unsigned long long todo = __ballot(shared); todo; todo &= todo - 1) {
+            const int owner = __builtin_ctzll(todo);
+            const int64_t wi = __shfl(i, owner, 64), wkb = __shfl(kb, owner, 64), wke = __shfl(ke, owner, 64);
+            const int32_t wout = __shfl(out0, owner, 64);
+            int64_t n = 0;
+            int32_t dpos = -1;
+            for (int64_t e0 = 0; e0 < wke - wkb; e0 += 64) {
+                const int64_t e = e0 + lane;
+                const bool valid = e < wke - wkb;
+                const int64_t k = !valid ? wkb : eff_lower ? wkb + e : wke - 1 - e;
+                const int64_t j = TR ? (int64_t)t_row[k] : indices[k];
+                const int32_t src = TR ? t_perm[k] : (int32_t)k;
+                const bool on_diag = valid && j == wi;
+                const bool keep = valid && !on_diag && !(eff_lower ? j > wi : j < wi);
+                const unsigned long long kept = __ballot(keep), diags = __ballot(on_diag);
+                if (fill && keep) {
+                    const int64_t at = (int64_t)wout + n + __popcll(kept & ((1ull << lane) - 1));
+                    dslot[at] = slot_of[j];
+                    dsrc[at] = src;
+                }
+                n += __popcll(kept);
+                if (diags) dpos = __shfl(src, 63 - __builtin_clzll(diags), 64);   // the last one met, as in the serial walk
+            }
+            if (lane == owner) {
+                if (fill) { diag[q] = dpos; if (n > *max_deps) atomicMax(max_deps, (int32_t)(n > 0x7fffffff ? 0x7fffffff : n)); }
+                else count64[q] = n;
+            }
+        }
     }
 }
 

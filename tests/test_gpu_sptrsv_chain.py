@@ -163,3 +163,27 @@ def test_values_the_division_shortcut_does_not_cover(dev, dtype):
         b3[::7] *= big
         b3[3::7] *= float(np.finfo(dtype).tiny)
         solve_and_compare(dev, M, True, False, dtype, f"extreme magnitudes, band {width}", b=b3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("lower", [True, False])
+def test_a_dense_row_and_a_dense_column(dev, dtype, lower):
+    # arrowhead triangles of 5000 rows: one row (and, in the other triangle, one column) of 5000
+    # entries, which the level analysis packs by a wavefront instead of a lane (the order of a row's
+    # dependencies is the one of the serial walk, cpp/sparse_csr_cpu.cpp:672-718; rows this long are
+    # added across lanes, hence the tolerance)
+    n = 5000
+    rng = np.random.default_rng(31)
+    for dense_row in (True, False):
+        L = sps.lil_matrix((n, n))
+        L.setdiag(rng.uniform(2.0, 3.0, n))
+        if dense_row:
+            L[n - 1, :n - 1] = rng.uniform(-1, 1, n - 1) / n
+        else:
+            L[1:, 0] = (rng.uniform(-1, 1, n - 1) / n).reshape(-1, 1)
+        for k in range(5, n, 7):
+            L[k, k - 3] = 0.1
+        M = L.tocsr() if lower else L.tocsr().T
+        solve_and_compare(dev, M, lower, False, dtype, f"arrowhead, dense {'row' if dense_row else 'column'}", exact=False)
+        solve_and_compare(dev, M, lower, True, dtype, f"unit arrowhead, dense {'row' if dense_row else 'column'}",
+                          exact=False)
