@@ -15,6 +15,7 @@
 //   backward: nnz*(s+8) + (rows+1)*8 + rows*s + cols*s + nnz*s + cols*s
 #include <algorithm>
 #include <atomic>
+#include <cstdint>
 #include <type_traits>
 
 #include "nm_common.hpp"
@@ -130,6 +131,113 @@ __device__ __forceinline__ X *at(X *base, int32_t idx) {
     return base + idx;
 }
 
+// 1: kernels that find a staging list in the plan load the listed segments of x (and, in the
+// backward, of g) into LDS with coalesced requests and look the factors of the entries up there,
+// instead of one gather instruction per entry and operand.  A gather of 64 scattered words keeps
+// the address unit of a compute unit busy for as long as a 1 KB coalesced request, and it was these
+// instructions, not bytes, that the kernels waited for (2048 x 2048 Poisson matrix, fp32: forward
+// 37.9 -> 31 us in a lab kernel).
+#ifndef NM_STAGE_FWD
+#define NM_STAGE_FWD 1
+#endif
+#ifndef NM_STAGE_BWD
+#define NM_STAGE_BWD 1
+#endif
+
+// quads of staged x per lane of the forward
+template <int BLOCK> constexpr int kFwdXQ = nm::kStageFwd * nm::kStageSeg / (4 * BLOCK);
+
+// One tile of the forward whose block of rows has a staging list (see nm_transpose.hpp): n entries,
+// 4 <= n <= NQ * 4 * BLOCK <= CAP, starting at `base`.  Written to issue
+// as few vector memory instructions as the tile's bytes allow, all of them before the first wait:
+// the list arrives in scalar registers with the tile's ends, x comes a quad per lane, a lane owns two
+// neighbouring rows and fetches their three pointers with one request, their sums leave as a pair.
+template <typename T, int BLOCK, int R, int CAP, int NQ>
+__device__ __forceinline__ void fwd_tile_staged(const int64_t r0, const int nr, const int32_t base, const int n,
+                                                const T *__restrict__ data, const int16_t *__restrict__ off16,
+                                                const int32_t *__restrict__ indptr, const int32_t lo0,
+                                                const int32_t hi0, const int32_t lo1, const int32_t hi1,
+                                                const T *__restrict__ x,
+                                                T *__restrict__ y, T *s_prod, T *s_x) {
+    typedef T TV __attribute__((ext_vector_type(4), aligned(sizeof(T))));
+    typedef T T2 __attribute__((ext_vector_type(2), aligned(sizeof(T))));
+    typedef uint32_t SV __attribute__((ext_vector_type(2), aligned(2)));    // four 16-bit places
+    typedef int32_t I3 __attribute__((ext_vector_type(3), aligned(4)));
+    constexpr int XQ = kFwdXQ<BLOCK>;                                       // quads of x per lane
+    static_assert(NQ * 4 * BLOCK <= CAP && XQ * 4 * BLOCK == nm::kStageFwd * nm::kStageSeg, "whole quads per lane");
+    static_assert(R == 2 * BLOCK && nm::kStageSeg == 128, "two rows per lane, two segments per wavefront and request");
+    const int tid = threadIdx.x;
+    // The wavefront's two segments per request (lo/hi = places 2 * wave + 8 u and the next one of
+    // the list, in scalar registers); an unused place loads segment 0.
+    TV xs[XQ];
+#pragma unroll
+    for (int u = 0; u < XQ; ++u) {
+        int32_t seg = u == 0 ? ((tid & 32) ? hi0 : lo0) : ((tid & 32) ? hi1 : lo1);
+        seg = seg < 0 ? 0 : seg;
+        xs[u] = *reinterpret_cast<const TV *>(x + (int64_t)seg * nm::kStageSeg + 4 * (tid & 31));
+    }
+    // pointers of rows 2 tid, 2 tid + 1 and the end of the second one
+    int32_t p0, p1, p2;
+    if (nr == R) {
+        const I3 pp = *reinterpret_cast<const I3 *>(indptr + r0 + 2 * tid);
+        p0 = pp[0], p1 = pp[1], p2 = pp[2];
+    } else {
+        const int t = 2 * tid;
+        p0 = indptr[r0 + (t < nr ? t : nr)];
+        p1 = indptr[r0 + (t + 1 < nr ? t + 1 : nr)];
+        p2 = indptr[r0 + (t + 2 < nr ? t + 2 : nr)];
+    }
+    // the entries: values and places in the staged segments, every quad of the tile at once; the
+    // last quad is moved back to end with the tile and overlaps the one before it
+    const T *__restrict__ d = data + base;
+    const int16_t *__restrict__ co = off16 + base;
+    TV aa[NQ];
+    SV oo[NQ];
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+        int kc = tid * 4 + u * 4 * BLOCK;
+        kc = kc < n - 4 ? kc : n - 4;
+        aa[u] = __builtin_nontemporal_load(reinterpret_cast<const TV *>(d + kc));
+        oo[u] = __builtin_nontemporal_load(reinterpret_cast<const SV *>(co + kc));
+    }
+#pragma unroll
+    for (int u = 0; u < XQ; ++u) *reinterpret_cast<TV *>(s_x + 4 * (tid + u * BLOCK)) = xs[u];
+    __syncthreads();
+    // (the entries are pinned here: left alone, the compiler moves the requests of a quad that only
+    // some lanes use down into the branch that uses it, behind the barrier)
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(aa[u][q]));
+        asm volatile("" : "+v"(oo[u][0]), "+v"(oo[u][1]));
+    }
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+        int k = tid * 4 + u * 4 * BLOCK;
+        if (k < n) {
+            k = k < n - 4 ? k : n - 4;
+            TV p;
+            p[0] = aa[u][0] * s_x[oo[u][0] & 0xffffu];
+            p[1] = aa[u][1] * s_x[oo[u][0] >> 16];
+            p[2] = aa[u][2] * s_x[oo[u][1] & 0xffffu];
+            p[3] = aa[u][3] * s_x[oo[u][1] >> 16];
+            *reinterpret_cast<TV *>(s_prod + k) = p;
+        }
+    }
+    __syncthreads();
+    // storage-order sums of the lane's two rows
+    T acc0 = 0, acc1 = 0;
+    for (int j = p0 - base; j < p1 - base; ++j) acc0 += s_prod[j];
+    for (int j = p1 - base; j < p2 - base; ++j) acc1 += s_prod[j];
+    if (2 * tid + 1 < nr) {
+        T2 out;
+        out[0] = acc0, out[1] = acc1;
+        __builtin_nontemporal_store(out, reinterpret_cast<T2 *>(y + r0 + 2 * tid));
+    } else if (2 * tid < nr) {
+        nm::stream_store(y + r0 + 2 * tid, acc0);
+    }
+}
+
 // UNIT: x is taken as all ones and not read, which makes y the row sums
 // (cpp/sparse_csr_cpu.cpp:1121-1127); a * 1 == a exactly, so the summation is
 // the same storage-order sum.
@@ -140,10 +248,13 @@ template <typename T, int BLOCK, int R, int CAP, bool UNIT = false, typename IDX
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_num_sgpr(72))) void spmv_fwd_kernel(
     int64_t rows, int rt, const T *__restrict__ data, const IDX *__restrict__ indices,
     const IDX *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y,
-    const int16_t *__restrict__ off16 = nullptr, const int32_t *__restrict__ flags = nullptr) {
+    const int16_t *__restrict__ off16 = nullptr, const int32_t *__restrict__ flags = nullptr,
+    const int32_t *__restrict__ f_desc = nullptr) {
     // rt <= R: rows per block of this launch (block_rows)
+    constexpr bool STAGE = NM_STAGE_FWD && NM_FWD32_VEC && sizeof(IDX) == 4 && !UNIT && R == nm::kPackRows;
     __shared__ int32_t s_off[R + 1];
-    __shared__ T s_prod[CAP];
+    __shared__ __align__(16) T s_prod[CAP];
+    __shared__ __align__(16) T s_x[STAGE ? nm::kStageFwd * nm::kStageSeg : 4];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     // off16: columns as 16-bit offsets from the first row of a block of nm::kPackRows rows (a plan's
@@ -158,6 +269,36 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_num_sgpr(72))) void sp
         int nr = (int)(rows - r0 < rt ? rows - r0 : rt);
         nr = nr < R ? nr : R;   // rt <= R
         const int64_t base = indptr[r0];
+        bool packed_here = packed;
+        if constexpr (STAGE) if (f_desc != nullptr && rt == nm::kPackRows) {
+            // A block of rows with a staging list keeps places in that list where other blocks
+            // keep column offsets.  The tile's end, the head of its list and the wavefront's
+            // four places of the list are requested together (scalar loads, one round trip);
+            // `live` is always true and only keeps those requests in front of the branch.
+            const int32_t *__restrict__ desc = f_desc + tile * nm::kStageDesc;
+            const int64_t span = (int64_t)indptr[r0 + nr] - base;
+            const int32_t d0 = desc[0];
+            static_assert(kFwdXQ<BLOCK> == 2, "two requests per lane cover the list");
+            const int32_t lo0 = desc[2 * wave], hi0 = desc[2 * wave + 1];
+            const int32_t lo1 = desc[BLOCK / 32 + 2 * wave], hi1 = desc[BLOCK / 32 + 2 * wave + 1];
+            const bool live = (lo0 & hi0 & lo1 & hi1) != INT32_MIN;
+            if ((span >= 4) & (d0 >= 0) & live) {
+                if (span <= CAP) {
+                    // as many quads per lane as the tile has (a 5-point row block: three of four)
+                    constexpr int NQ = CAP / (4 * BLOCK);
+                    const int32_t *__restrict__ ip = reinterpret_cast<const int32_t *>(indptr);
+                    if (span <= (NQ - 1) * 4 * BLOCK)
+                        fwd_tile_staged<T, BLOCK, R, CAP, NQ - 1>(r0, nr, (int32_t)base, (int)span, data, off16, ip,
+                                                                  lo0, hi0, lo1, hi1, x, y, s_prod, s_x);
+                    else
+                        fwd_tile_staged<T, BLOCK, R, CAP, NQ>(r0, nr, (int32_t)base, (int)span, data, off16, ip, lo0, hi0,
+                                                              lo1, hi1, x, y, s_prod, s_x);
+                    __syncthreads();
+                    continue;
+                }
+                packed_here = false;
+            }
+        }
         // Both ends of the tile are the same for every lane (scalar loads), so the entry streams
         // can be requested without waiting for the row pointers to pass through LDS: those stay
         // in registers until the products are on their way.
@@ -223,7 +364,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_num_sgpr(72))) void sp
                         }
                 }
             };
-            if (packed) walk(std::true_type{}); else walk(std::false_type{});
+            if (packed_here) walk(std::true_type{}); else walk(std::false_type{});
             for (int k = n4 + threadIdx.x; k < n; k += BLOCK) s_prod[k] = d[k] * x[ci[k]];
             if (early) {
 #pragma unroll
@@ -478,6 +619,121 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
     }
 }
 
+// quads of staged g (and x) per lane of the planned backward
+template <int BLOCK> constexpr int kBwdXQ = (nm::kStageBwd * nm::kStageSeg / 4 + BLOCK - 1) / BLOCK;
+
+// One tile of the planned backward, both gradients of a symmetric pattern, for a block of columns
+// with a staging list and valid packed words: n entries, 1 <= n <= CAP, the first one at position
+// `base` of the plan.  Like fwd_tile_staged it issues every request of the tile before its first
+// wait, unconditionally (a request inside a branch makes the compiler's wait counts pessimistic:
+// it then waits for nearly everything in flight), in the order in which the answers are needed
+// (requests are answered in order), and as few vector memory instructions as the bytes allow: the
+// listed segments of g and x a quad per lane, a column's two bounds with one request, the packed
+// words of the first 1024 entries four consecutive entries per lane (QUAD; grad_A then leaves 16
+// bytes per lane as well) and the rest in ER rounds of one entry per lane; only the values of A
+// are gathered entry by entry.  SEG2: the list has more than eight places.
+template <typename T, int R, int CAP, bool O32, bool QUAD, int ER, bool SEG2>
+__device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, const int32_t base, const int n,
+                                                const int32_t lo0, const int32_t hi0, const int32_t lo1,
+                                                const int32_t hi1, const T *__restrict__ data,
+                                                const int32_t *__restrict__ t_indptr,
+                                                const int32_t *__restrict__ t_pack, const T *__restrict__ x,
+                                                const T *__restrict__ g, T *__restrict__ grad_A,
+                                                T *__restrict__ grad_x, T *s_v, T *s_g, T *s_x) {
+    typedef T TV __attribute__((ext_vector_type(4), aligned(sizeof(T))));
+    typedef int32_t I4 __attribute__((ext_vector_type(4), aligned(4)));
+    typedef int32_t I2 __attribute__((ext_vector_type(2), aligned(4)));
+    constexpr int XQ = SEG2 ? kBwdXQ<kBlock> : 1;
+    constexpr int kQuads = QUAD ? 4 * kBlock : 0;       // entries of the quad phase
+    static_assert(R == kBlock && nm::kStageSeg == 128, "lane = column, two segments per wavefront and request");
+    static_assert(kBwdXQ<kBlock> == 2, "a list of at most sixteen places");
+    const int tid = threadIdx.x;
+    // packed words
+    I4 wq;
+    if (QUAD) wq = __builtin_nontemporal_load(reinterpret_cast<const I4 *>(at<O32>(t_pack, base + tid * 4)));
+    int32_t we[ER > 0 ? ER : 1];
+#pragma unroll
+    for (int r = 0; r < ER; ++r) {
+        const int k = kQuads + r * kBlock + tid;
+        we[r] = nm::stream_load(at<O32>(t_pack, base + (k < n ? k : n - 1)));
+    }
+    // the wavefront's two segments per request (an unused place of the list loads segment 0)
+    TV gs[XQ], xs[XQ];
+#pragma unroll
+    for (int u = 0; u < XQ; ++u) {
+        // (separate scalars, not an array: the compiler turns a choice between array elements into
+        // an indexed read of a copy of the array in scratch memory)
+        int32_t seg = u == 0 ? ((tid & 32) ? hi0 : lo0) : ((tid & 32) ? hi1 : lo1);
+        seg = seg < 0 ? 0 : seg;
+        const int64_t at0 = (int64_t)seg * nm::kStageSeg + 4 * (tid & 31);
+        gs[u] = *reinterpret_cast<const TV *>(g + at0);
+        xs[u] = *reinterpret_cast<const TV *>(x + at0);
+    }
+    // bounds of column c0 + tid and the factor its entries share (the lane writes the mirror entry)
+    int32_t pa, pb;
+    if (nc == R) {
+        const I2 pp = *reinterpret_cast<const I2 *>(t_indptr + c0 + tid);
+        pa = pp[0], pb = pp[1];
+    } else {
+        pa = t_indptr[c0 + (tid < nc ? tid : nc)];
+        pb = t_indptr[c0 + (tid + 1 < nc ? tid + 1 : nc)];
+    }
+    T own = g[c0 + (tid < nc ? tid : nc - 1)];
+    // the values of A at the positions the packed words name
+    T dq[4], de[ER > 0 ? ER : 1];
+    if (QUAD) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dq[q] = *at<O32>(data, base + tid * 4 + q + (wq[q] >> 16));
+    }
+#pragma unroll
+    for (int r = 0; r < ER; ++r) {
+        const int k = kQuads + r * kBlock + tid;
+        const int kc = k < n ? k : n - 1;
+        de[r] = *at<O32>(data, base + kc + (we[r] >> 16));
+    }
+#pragma unroll
+    for (int u = 0; u < XQ; ++u)
+        if (4 * (tid + u * kBlock) < nm::kStageBwd * nm::kStageSeg) {      // (the list's last places: half a workgroup)
+            *reinterpret_cast<TV *>(s_g + 4 * (tid + u * kBlock)) = gs[u];
+            *reinterpret_cast<TV *>(s_x + 4 * (tid + u * kBlock)) = xs[u];
+        }
+    // (pinned: left alone, the compiler moves the request for `own` down into the branch that
+    // uses it, behind the gathers)
+    asm volatile("" : "+v"(own));
+    if (tid < nc)
+        for (int j = pa - base; j < pb - base; ++j) s_v[j] = own;
+    __syncthreads();
+    if (QUAD) {
+        const int k = tid * 4;
+        const TV sv = *reinterpret_cast<const TV *>(s_v + k);
+        TV out, nv;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int li = wq[q] & 0xffff;
+            out[q] = sv[q] * s_x[li];
+            nv[q] = s_g[li] * dq[q];
+        }
+        *reinterpret_cast<TV *>(s_v + k) = nv;
+        *reinterpret_cast<TV *>(at<O32>(grad_A, base + k)) = out;
+    }
+#pragma unroll
+    for (int r = 0; r < ER; ++r) {
+        const int k = kQuads + r * kBlock + tid;
+        if (k < n) {
+            const int li = we[r] & 0xffff;
+            *at<O32>(grad_A, base + k) = s_v[k] * s_x[li];
+            s_v[k] = s_g[li] * de[r];
+        }
+    }
+    __syncthreads();
+    // grad_x[column] = sum of the column's slice in ascending row order
+    if (tid < nc) {
+        T acc = 0;
+        for (int j = pa - base; j < pb - base; ++j) acc += s_v[j];
+        grad_x[c0 + tid] = acc;
+    }
+}
+
 // Backward over the transposed-structure plan (columns of A as rows of A^T):
 // no atomics and no clearing of grad_x.  A workgroup owns R consecutive
 // columns; lane p of the entry-parallel phase reads (row, position) of the
@@ -492,14 +748,20 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_kernel(
 // row-major entry p = (row c, column r), so the lane writes
 // grad_A[p] = g[c] * x[r] instead: a coalesced store, every entry once.
 template <typename T, int R, int CAP, bool O32>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 8 : 7))) void spmv_bwd_planned_kernel(
+__global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
     int64_t cols, const T *__restrict__ data, const int32_t *__restrict__ t_indptr,
     const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm, const int32_t *__restrict__ t_pack,
     const int32_t *__restrict__ flags, const T *__restrict__ x, const T *__restrict__ g,
-    T *__restrict__ grad_A, T *__restrict__ grad_x) {
+    T *__restrict__ grad_A, T *__restrict__ grad_x, const int32_t *__restrict__ b_desc) {
     static_assert(R == nm::kPackCols, "t_pack holds rows relative to the first column of a workgroup's block");
+    static_assert(nm::kStageBwdCap <= CAP, "a block with a staging list fits the tile");
+    constexpr bool STAGE = NM_STAGE_BWD != 0;
+    constexpr int kStaged = nm::kStageBwd * nm::kStageSeg;
     __shared__ int32_t s_off[R + 1];
     __shared__ __align__(16) T s_v[CAP];
+    // the segments of g and of x that a block with a staging list names
+    __shared__ __align__(16) T s_g[STAGE ? kStaged : 4];
+    __shared__ __align__(16) T s_x[STAGE ? kStaged : 4];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const bool mirror = flags[0] != 0;
@@ -517,11 +779,68 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
         if (tile >= ntiles) continue;
         const int64_t c0 = tile * R;
         const int nc = (int)(cols - c0 < R ? cols - c0 : R);
+        if constexpr (STAGE) if (fused && packed && b_desc != nullptr) {
+            // a block of columns with a staging list, both gradients: the tile's ends, the head of
+            // its list and the wavefront's four places of the list come together (scalar loads);
+            // `live` is always true and only keeps those requests in front of the branch
+            const int32_t *__restrict__ desc = b_desc + tile * nm::kStageDesc;
+            const int32_t first = t_indptr[c0], n_all = t_indptr[c0 + nc] - first, d0 = desc[0];
+            static_assert(kBwdXQ<kBlock> == 2, "two requests per lane cover the list");
+            const int32_t lo0 = desc[2 * wave], hi0 = desc[2 * wave + 1];
+            const int32_t lo1 = desc[kBlock / 32 + 2 * wave], hi1 = desc[kBlock / 32 + 2 * wave + 1];
+            const bool live = (lo0 & hi0 & lo1 & hi1) != INT32_MIN;
+            if ((d0 >= 0) & (n_all >= 1) & (n_all <= CAP) & live) {
+                const bool seg2 = desc[8] >= 0;
+#define NM_BWD_TILE(QUAD, ER, SEG2)                                                                                \
+    bwd_tile_staged<T, R, CAP, O32, QUAD, ER, SEG2>(c0, nc, first, n_all, lo0, hi0, lo1, hi1, data, t_indptr, t_pack, x, g, grad_A, \
+                                                    grad_x, s_v, s_g, s_x)
+                // (the five-point block: 1024 entries in quads and one round, eight segments)
+                if (n_all >= 4 * kBlock && n_all <= 5 * kBlock && !seg2) NM_BWD_TILE(true, 1, false);
+                else if (n_all >= 4 * kBlock) NM_BWD_TILE(true, (CAP - 4 * kBlock) / kBlock, true);
+                else NM_BWD_TILE(false, 4, true);
+#undef NM_BWD_TILE
+                __syncthreads();
+                continue;
+            }
+        }
         // Lane t holds the bounds of column c0 + t and its own factor; all three loads leave
         // together (one memory round trip before the tile's entries can be read).
         const int32_t my_a = *at<O32>(t_indptr, (int32_t)c0 + (tid < nc ? tid : nc));
         const int32_t my_b = *at<O32>(t_indptr, (int32_t)c0 + (tid + 1 < nc ? tid + 1 : nc));
         const T my_own = own_of ? *at<O32>(own_of, (int32_t)c0 + (tid < nc ? tid : nc - 1)) : T(0);
+        // A block of columns with a staging list (only made where the packed words are valid) keeps
+        // in the low half of a packed word the place of the entry's row in the listed segments:
+        // those segments of g (and of x, where the mirror entry is written) go to LDS, a quad per
+        // lane and request.
+        bool staged = false;
+        if constexpr (STAGE) {
+            typedef T TV __attribute__((ext_vector_type(4), aligned(sizeof(T))));
+            constexpr int XQ = (kStaged / 4 + kBlock - 1) / kBlock;
+            const int32_t *__restrict__ desc = b_desc + tile * nm::kStageDesc;
+            // (both gradients of such a block were taken by bwd_tile_staged above)
+            staged = !fused && packed && b_desc != nullptr && desc[0] >= 0;
+            if (staged) {
+                const bool want_x = mirror && grad_A != nullptr;
+                TV gs[XQ], xs[XQ];
+#pragma unroll
+                for (int u = 0; u < XQ; ++u) {
+                    const int f = tid + u * kBlock;
+                    int32_t seg = desc[f < kStaged / 4 ? f / (nm::kStageSeg / 4) : 0];
+                    seg = seg < 0 ? 0 : seg;
+                    const int64_t at0 = (int64_t)seg * nm::kStageSeg + 4 * (f % (nm::kStageSeg / 4));
+                    gs[u] = *reinterpret_cast<const TV *>(g + at0);
+                    xs[u] = *reinterpret_cast<const TV *>((want_x ? x : g) + at0);
+                }
+#pragma unroll
+                for (int u = 0; u < XQ; ++u) {
+                    const int f = tid + u * kBlock;
+                    if (f < kStaged / 4) {
+                        *reinterpret_cast<TV *>(s_g + 4 * f) = gs[u];
+                        *reinterpret_cast<TV *>(s_x + 4 * f) = xs[u];
+                    }
+                }
+            }
+        }
         // s_off[t] = first entry of column c0 + t in the plan (an absolute position), t = 0 .. nc
         s_off[tid] = my_a;
         if (tid == nc - 1) s_off[nc] = my_b;
@@ -696,14 +1015,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
                 if (packed) {
                     const int32_t w = nm::stream_load(t_pack + first + p);
                     k = first + p + (w >> 16);
-                    r = (int32_t)c0 + (int16_t)w;
+                    r = (STAGE && staged) ? (w & 0xffff) : (int32_t)c0 + (int16_t)w;
                 } else {
                     k = nm::stream_load(tp + p);
                     r = nm::stream_load(tr + p);
                 }
-                const T gr = g[r];
+                const T gr = (STAGE && staged) ? s_g[r] : g[r];
                 if (grad_A) {
-                    if (mirror) grad_A[first + p] = s_v[p] * x[r];
+                    if (mirror) grad_A[first + p] = s_v[p] * ((STAGE && staged) ? s_x[r] : x[r]);
                     else grad_A[k] = gr * s_v[p];
                 }
                 if (grad_x) s_v[p] = gr * data[k];
@@ -815,13 +1134,14 @@ int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const i
 
 template <typename T, typename IDX>
 int launch_fwd(int64_t rows, int64_t nnz, const T *data, const IDX *indices, const IDX *indptr, const T *x,
-               T *y, hipStream_t s, const int16_t *off16 = nullptr, const int32_t *flags = nullptr) {
+               T *y, hipStream_t s, const int16_t *off16 = nullptr, const int32_t *flags = nullptr,
+               const int32_t *f_desc = nullptr) {
     constexpr int R = kFwdR, CAP = kFwdCap<T>;
     const int rt = block_rows(rows, nnz, R, CAP);
     int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, false, IDX>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s,
-                       rows, rt, data, indices, indptr, x, y, off16, flags);
+                       rows, rt, data, indices, indptr, x, y, off16, flags, f_desc);
     NM_LAUNCH_CHECK("spmv_fwd_kernel");
     return NM_OK;
 }
@@ -834,7 +1154,7 @@ int launch_row_sum(int64_t rows, int64_t nnz, const T *data, const int64_t *indp
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
     hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, true>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s, rows,
                        rt, data, (const int64_t *)nullptr, indptr, (const T *)nullptr, y, (const int16_t *)nullptr,
-                       (const int32_t *)nullptr);
+                       (const int32_t *)nullptr, (const int32_t *)nullptr);
     NM_LAUNCH_CHECK("spmv_fwd_kernel<unit>");
     return NM_OK;
 }
@@ -885,9 +1205,9 @@ extern "C" int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
         return launch_fwd<float, int32_t>(rows, nnz, (const float *)data, t.c_idx32, t.c_ptr32, (const float *)x,
-                                          (float *)y, s, t.c_off16, t.flags);
+                                          (float *)y, s, t.c_off16, t.flags, nnz > 0 ? t.f_desc : nullptr);
     return launch_fwd<double, int32_t>(rows, nnz, (const double *)data, t.c_idx32, t.c_ptr32, (const double *)x,
-                                       (double *)y, s, t.c_off16, t.flags);
+                                       (double *)y, s, t.c_off16, t.flags, nnz > 0 ? t.f_desc : nullptr);
 }
 
 extern "C" int nm_csr_row_sum_forward(nm_dtype dt, int64_t rows, int64_t nnz, const void *data,
@@ -961,11 +1281,11 @@ extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t col
         if (o32)
             hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
                                (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const float *)x,
-                               (const float *)g, (float *)grad_A, (float *)grad_x);
+                               (const float *)g, (float *)grad_A, (float *)grad_x, nnz > 0 ? t.b_desc : nullptr);
         else
             hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
                                (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const float *)x,
-                               (const float *)g, (float *)grad_A, (float *)grad_x);
+                               (const float *)g, (float *)grad_A, (float *)grad_x, nnz > 0 ? t.b_desc : nullptr);
     } else {
         constexpr int R = kPlannedR, CAP = kPlannedCap;
         int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
@@ -973,11 +1293,11 @@ extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t col
         if (o32)
             hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
                                (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const double *)x,
-                               (const double *)g, (double *)grad_A, (double *)grad_x);
+                               (const double *)g, (double *)grad_A, (double *)grad_x, nnz > 0 ? t.b_desc : nullptr);
         else
             hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
                                (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const double *)x,
-                               (const double *)g, (double *)grad_A, (double *)grad_x);
+                               (const double *)g, (double *)grad_A, (double *)grad_x, nnz > 0 ? t.b_desc : nullptr);
     }
     NM_LAUNCH_CHECK("spmv_bwd_planned_kernel");
     return NM_OK;

@@ -335,6 +335,92 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
     if (!fits_c) flags[2] = 0;
 }
 
+// Staging lists (f_desc / b_desc of the plan).  A workgroup takes one block of kPackRows rows
+// (FWD) or of kPackCols columns; `key` of an entry is its column (FWD: c_idx32) or its row
+// (t_row).  The segments the block's keys fall into are collected in a small LDS hash set; when
+// there are at most MOST of them, all of them whole (a segment cut off by the end of the vector
+// the kernels will load it from would be read past that end), they are ranked and every entry
+// gets 128 * rank + offset inside the segment: written over c_off16[k] (FWD) or over the low half
+// of t_pack[p].  Runs after tp_pack_kernel.
+template <bool FWD, int MOST>
+__global__ __launch_bounds__(kBlock) void tp_stage_kernel(
+    int64_t nblocks, int64_t nlines, int64_t veclen, const int32_t *__restrict__ ptr, const int32_t *__restrict__ key,
+    int32_t *__restrict__ t_pack, int16_t *__restrict__ c_off16, int32_t *__restrict__ desc,
+    const int32_t *__restrict__ flags) {
+    constexpr int kSlots = 64, kBlockLines = FWD ? nm::kPackRows : nm::kPackCols;
+    constexpr int kMostEntries = FWD ? nm::kStageFwdCap : nm::kStageBwdCap;
+    __shared__ int32_t s_tab[kSlots], s_rank[kSlots], s_count, s_bad;
+    const bool enabled = FWD || flags[1] != 0;   // the backward only reads t_pack when it is valid
+    for (int64_t b = blockIdx.x; b < nblocks; b += gridDim.x) {
+        const int64_t l0 = b * kBlockLines;
+        const int64_t l1 = l0 + kBlockLines < nlines ? l0 + kBlockLines : nlines;
+        const int32_t pb = ptr[l0], pe = ptr[l1];
+        if (threadIdx.x < kSlots) {
+            s_tab[threadIdx.x] = -1;
+            s_rank[threadIdx.x] = 0;
+        }
+        if (threadIdx.x == 0) {
+            s_count = 0;
+            s_bad = (!enabled || pe - pb > kMostEntries || pe == pb) ? 1 : 0;
+        }
+        __syncthreads();
+        // the slot of a segment in the table; inserts it when `insert`.  -1: table full or given up
+        auto slot_of = [&](int32_t seg, bool insert) -> int {
+            int h = (int)(((uint32_t)seg * 0x9E3779B1u) >> 26);
+            for (int step = 0; step < kSlots; ++step, h = (h + 1) & (kSlots - 1)) {
+                int32_t seen = s_tab[h];
+                if (seen == -1 && insert) {
+                    seen = atomicCAS(&s_tab[h], -1, seg);
+                    if (seen == -1) {
+                        atomicAdd(&s_count, 1);
+                        return h;
+                    }
+                }
+                if (seen == seg) return h;
+                if (seen == -1) return -1;
+            }
+            return -1;
+        };
+        if (s_bad == 0) {
+            for (int32_t p = pb + (int32_t)threadIdx.x; p < pe; p += kBlock) {
+                const int32_t seg = key[p] / nm::kStageSeg;
+                if ((int64_t)(seg + 1) * nm::kStageSeg > veclen || slot_of(seg, true) < 0) s_bad = 1;
+                if (s_count > MOST) break;
+            }
+        }
+        __syncthreads();
+        const bool staged = s_bad == 0 && s_count <= MOST;
+        if (staged && threadIdx.x < kSlots) {
+            const int32_t mine = s_tab[threadIdx.x];
+            if (mine >= 0) {
+                int r = 0;
+                for (int j = 0; j < kSlots; ++j) {
+                    const int32_t other = s_tab[j];
+                    r += other >= 0 && other < mine;
+                }
+                s_rank[threadIdx.x] = r;
+                desc[b * nm::kStageDesc + r] = mine;
+            }
+        }
+        if (threadIdx.x < nm::kStageDesc) {
+            // places the ranked segments do not fill (written above by other lanes: different places)
+            if (!staged) desc[b * nm::kStageDesc + threadIdx.x] = -2;
+            else if ((int)threadIdx.x >= s_count) desc[b * nm::kStageDesc + threadIdx.x] = -1;
+        }
+        __syncthreads();
+        if (staged) {
+            for (int32_t p = pb + (int32_t)threadIdx.x; p < pe; p += kBlock) {
+                const int32_t k = key[p];
+                const int h = slot_of(k / nm::kStageSeg, false);
+                const int32_t where = s_rank[h < 0 ? 0 : h] * nm::kStageSeg + k % nm::kStageSeg;
+                if (FWD) c_off16[p] = (int16_t)where;
+                else t_pack[p] = (int32_t)(((uint32_t)t_pack[p] & 0xffff0000u) | (uint32_t)where);
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // Clears flags[0] unless A^T has exactly A's structure.
 __global__ void symmetry_check_kernel(int64_t nnz, int64_t cols, const int32_t *__restrict__ col32,
                                       const int32_t *__restrict__ ptr32, const int32_t *__restrict__ t_row,
@@ -421,6 +507,15 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
         hipLaunchKernelGGL(tp_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, cols, plan.t_indptr,
                            plan.t_row, plan.t_perm, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.flags);
         NM_LAUNCH_CHECK("tp_pack_kernel");
+        const int64_t rblocks = ceil_div(rows, (int64_t)kPackRows), cblocks = ceil_div(cols, (int64_t)kPackCols);
+        grid = rblocks > 65536 ? 65536 : rblocks;
+        hipLaunchKernelGGL((tp_stage_kernel<true, kStageFwd>), dim3((unsigned)grid), dim3(kBlock), 0, s, rblocks, rows,
+                           cols, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.f_desc, plan.flags);
+        NM_LAUNCH_CHECK("tp_stage_kernel<rows>");
+        grid = cblocks > 65536 ? 65536 : cblocks;
+        hipLaunchKernelGGL((tp_stage_kernel<false, kStageBwd>), dim3((unsigned)grid), dim3(kBlock), 0, s, cblocks, cols,
+                           rows, plan.t_indptr, plan.t_row, plan.t_pack, plan.c_off16, plan.b_desc, plan.flags);
+        NM_LAUNCH_CHECK("tp_stage_kernel<columns>");
     }
     return NM_OK;
 }

@@ -21,6 +21,17 @@
 //                16 bits.  Valid when flags[2] != 0                              (nnz)
 //                (the SpMV kernels read these instead of the 32-bit arrays: half the index
 //                traffic again on banded matrices)
+//   f_desc[b]    staging list of the b-th block of kPackRows rows: the up to kStageFwd segments of
+//                kStageSeg consecutive columns that the block's entries name, ascending, -1 for
+//                unused places (kStageDesc ints per block).  A block that has one keeps, in
+//                c_off16[k], the place of entry k's column in that list times kStageSeg plus the
+//                column's offset inside its segment: the forward loads the listed segments of x
+//                into LDS with coalesced requests and looks every entry's factor up there.
+//                f_desc[b][0] == -2: no list (more segments than fit, a segment that is cut off
+//                by the end of x, more entries than a tile holds); c_off16 is as described above
+//   b_desc[b]    the same for the b-th block of kPackCols columns and the ROWS its entries lie
+//                in (up to kStageBwd segments); such a block keeps the place in the list in the
+//                low half of t_pack[p].  Only made when flags[1] != 0
 //
 // Inside a column the entries keep A's row-major order (the sort is stable), so
 // rows ascend, exactly like the counting-sort transpose of the reference
@@ -41,11 +52,18 @@ struct TPlan {
     int32_t *c_ptr32;
     int32_t *t_pack;
     int16_t *c_off16;
+    int32_t *f_desc;
+    int32_t *b_desc;
 };
 
 // Blocks the packed offsets are relative to: the columns one workgroup of the planned SpMV
 // backward owns, and the rows one workgroup of the forward owns when rows are short.
 constexpr int kPackCols = 256, kPackRows = 512;
+// Segments of a vector that a block's entries name: length, most per block of rows (forward) and
+// per block of columns (backward), ints per list.
+constexpr int kStageSeg = 128, kStageFwd = 16, kStageBwd = 12, kStageDesc = 16;
+// Entries a block may hold to get a list: the LDS tiles of the kernels that use it.
+constexpr int kStageFwdCap = 4096, kStageBwdCap = 2048;
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
@@ -66,7 +84,9 @@ inline size_t tplan_layout(int64_t rows, int64_t cols, int64_t nnz, void *base, 
     int32_t *cp = (int32_t *)take((size_t)(rows + 2) * 4);
     int32_t *tw = (int32_t *)take((size_t)(nnz + 1) * 4);
     int16_t *co = (int16_t *)take((size_t)(nnz + 8) * 2);
-    if (p) *p = TPlan{a, b, c, h, f, ci, cp, tw, co};
+    int32_t *fd = (int32_t *)take((size_t)((rows + kPackRows - 1) / kPackRows + 1) * kStageDesc * 4);
+    int32_t *bd = (int32_t *)take((size_t)((cols + kPackCols - 1) / kPackCols + 1) * kStageDesc * 4);
+    if (p) *p = TPlan{a, b, c, h, f, ci, cp, tw, co, fd, bd};
     return off;
 }
 
