@@ -117,6 +117,22 @@ void check_matrix(const char *who, const char *name, const Tensor &t, int64_t ro
                 t.sizes());
 }
 
+// Which of its two gradients a backward pass computes.  The reference's GPU path computes a
+// gradient only for an operand that requires one (cpp/sparse_csr_cuda.cu:662, :682) and leaves
+// the other tensor undefined, its CPU path always computes both.  Here: both when neither
+// operand requires a gradient (a direct call outside autograd, what the CPU path would give),
+// otherwise those that are required; a gradient that is left out comes back undefined (None in
+// Python), which autograd treats like the value it would have thrown away.
+struct Wanted {
+    bool first, second;
+};
+Wanted wanted(const Tensor &a, const Tensor &b) {
+    const bool ra = a.requires_grad(), rb = b.requires_grad();
+    if (!ra && !rb) return {true, true};
+    return {ra, rb};
+}
+void *ptr_or_null(const Tensor &t) { return t.defined() ? t.data_ptr() : nullptr; }
+
 // How SpMV / SpMM backward compute grad_x / grad_B:
 //   "planned" (default)  on a cached transposed-structure plan (deterministic, no atomics) from
 //                        the SECOND time a sparsity pattern is seen; the first sighting runs the
@@ -219,6 +235,14 @@ void *host_landing() {
     return landing.data_ptr();
 }
 
+// Tensors made under torch.inference_mode() carry no version counter (asking for it throws).
+// A pair of such structure tensors gets no entry in the alias table -- an edit in place could
+// not be noticed -- so a call that needs a plan computes their content key every time and one
+// that only peeks runs its stateless kernels; pattern tensors of this kind that a plan hands
+// out count as version 0.
+bool tracked(const Tensor &t) { return !t.is_inference(); }
+uint32_t version_of(const Tensor &t) { return tracked(t) ? t._version() : 0; }
+
 bool alias_matches(const Alias &al, const Tensor &indices, const Tensor &indptr) {
     return al.idx_impl == indices.unsafeGetTensorImpl() && al.ptr_impl == indptr.unsafeGetTensorImpl() &&
            al.idx_ptr == indices.data_ptr() && al.ptr_ptr == indptr.data_ptr() &&
@@ -230,7 +254,8 @@ bool alias_matches(const Alias &al, const Tensor &indices, const Tensor &indptr)
 // The content key of (indices, indptr): from the alias table, or computed (waits for the stream).
 // With `compute` false a pair of tensors that has not been seen yields false instead.
 bool structure_key(const Tensor &indices, const Tensor &indptr, bool compute, Key *out) {
-    {
+    const bool aliased = tracked(indices) && tracked(indptr);
+    if (aliased) {
         std::lock_guard<std::mutex> lock(g_plans_mutex);
         for (auto it = g_aliases.begin(); it != g_aliases.end(); ++it) {
             if (alias_matches(*it, indices, indptr)) {
@@ -251,6 +276,10 @@ bool structure_key(const Tensor &indices, const Tensor &indptr, bool compute, Ke
                             current_stream(dev)),
           "nm_structure_hash");
     g_keys_computed.fetch_add(1, std::memory_order_relaxed);
+    if (!aliased) {
+        *out = Key{h[0], h[1], indices.numel(), indptr.numel(), dev.index()};
+        return true;
+    }
     Alias al{indices.unsafeGetTensorImpl(),
              indptr.unsafeGetTensorImpl(),
              WeakImpl(indices.getIntrusivePtr()),
@@ -449,7 +478,7 @@ std::shared_ptr<Plan> peek_product_plan(const Tensor &A_indices, const Tensor &A
     }
     if (!plan) return nullptr;
     for (size_t i = 0; i < plan->derived.size(); ++i)
-        if (plan->derived[i]._version() != plan->derived_versions[i]) {
+        if (version_of(plan->derived[i]) != plan->derived_versions[i]) {
             drop_plan(plan);
             return nullptr;
         }
@@ -536,7 +565,7 @@ void consider_product_plan(const Tensor &A_indices, const Tensor &A_indptr, cons
     plan->plan_class = usable > 0 ? usable : 0;
     if (plan->usable) {
         plan->derived = {C_indices, C_indptr};
-        for (const Tensor &t : plan->derived) plan->derived_versions.push_back(t._version());
+        for (const Tensor &t : plan->derived) plan->derived_versions.push_back(version_of(t));
     } else {
         plan->mem = Tensor();   // remembered as unusable, so that the pair is not analysed again
         plan->parent.reset();
@@ -606,7 +635,7 @@ void consider_sum_plan(const Tensor &A_indices, const Tensor &A_indptr, const Te
                                   pbytes, current_stream(dev)),
           "nm_splincomb_plan_build");
     plan->derived = {C_indices, C_indptr};
-    for (const Tensor &t : plan->derived) plan->derived_versions.push_back(t._version());
+    for (const Tensor &t : plan->derived) plan->derived_versions.push_back(version_of(t));
     auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev.index());
     plan->build_stream = stream.id();
     plan->ready = std::make_unique<at::cuda::CUDAEvent>();
@@ -678,22 +707,25 @@ std::vector<Tensor> spgemv_backward(Tensor grad_z, int A_rows, int A_cols, Tenso
     const auto dev = need_device({&grad_z, &A_data, &A_col_ind, &A_rowptr, &x});
     same_dtype(A_data, x, "x");
     same_dtype(A_data, grad_z, "grad_z");
+    const Wanted want = wanted(A_data, x);
     A_data = A_data.contiguous();
     x = x.contiguous();
     grad_z = grad_z.contiguous();
     A_col_ind = index_tensor(A_col_ind, "A_col_ind");
     A_rowptr = index_tensor(A_rowptr, "A_rowptr");
     c10::hip::HIPGuard guard(dev.index());
-    Tensor grad_A = torch::empty_like(A_data), grad_x = torch::empty_like(x);
+    Tensor grad_A, grad_x;
+    if (want.first) grad_A = torch::empty_like(A_data);
+    if (want.second) grad_x = torch::empty_like(x);
     if (auto plan = backward_plan(A_col_ind, A_rowptr, A_rows, x.size(0), dev)) {
         check(nm_spgemv_backward_planned(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
                                          plan->mem.data_ptr(), x.data_ptr(), grad_z.data_ptr(),
-                                         grad_A.data_ptr(), grad_x.data_ptr(), current_stream(dev)),
+                                         ptr_or_null(grad_A), ptr_or_null(grad_x), current_stream(dev)),
               "nm_spgemv_backward_planned");
     } else {
         check(nm_spgemv_backward(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
                                  A_col_ind.data_ptr<int64_t>(), A_rowptr.data_ptr<int64_t>(), x.data_ptr(),
-                                 grad_z.data_ptr(), grad_A.data_ptr(), grad_x.data_ptr(), current_stream(dev)),
+                                 grad_z.data_ptr(), ptr_or_null(grad_A), ptr_or_null(grad_x), current_stream(dev)),
               "nm_spgemv_backward");
     }
     return {grad_A, grad_x};
@@ -810,8 +842,10 @@ std::vector<Tensor> splincomb_backward(int rows, int cols, Tensor alpha, Tensor 
     C_indptr = index_tensor(C_indptr, "C_indptr");
     const double a = alpha.item<double>(), b = beta.item<double>();
     c10::hip::HIPGuard guard(dev.index());
-    Tensor grad_A = torch::empty_like(A_data, at::MemoryFormat::Contiguous);
-    Tensor grad_B = torch::empty_like(B_data, at::MemoryFormat::Contiguous);
+    const Wanted want = wanted(A_data, B_data);
+    Tensor grad_A, grad_B;
+    if (want.first) grad_A = torch::empty_like(A_data, at::MemoryFormat::Contiguous);
+    if (want.second) grad_B = torch::empty_like(B_data, at::MemoryFormat::Contiguous);
     if (backward_mode_now() != kAtomic) {
         // the maps belong to the pattern tensors the planned forward handed out: those very tensors
         auto plan = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, rows, cols, dev, false, 'S');
@@ -819,7 +853,7 @@ std::vector<Tensor> splincomb_backward(int rows, int cols, Tensor alpha, Tensor 
             plan->derived[1].data_ptr() == C_indptr.data_ptr() && plan->derived[0].numel() == C_indices.numel()) {
             check(nm_splincomb_backward_planned(dtype_of(A_data), A_indices.numel(), B_indices.numel(),
                                                 C_indices.numel(), a, b, grad_C_data.data_ptr(), plan->mem.data_ptr(),
-                                                grad_A.data_ptr(), grad_B.data_ptr(), current_stream(dev)),
+                                                ptr_or_null(grad_A), ptr_or_null(grad_B), current_stream(dev)),
                   "nm_splincomb_backward_planned");
             return {grad_A, grad_B};
         }
@@ -827,7 +861,7 @@ std::vector<Tensor> splincomb_backward(int rows, int cols, Tensor alpha, Tensor 
     check(nm_splincomb_backward(dtype_of(A_data), rows, a, A_indices.data_ptr<int64_t>(),
                                 A_indptr.data_ptr<int64_t>(), b, B_indices.data_ptr<int64_t>(),
                                 B_indptr.data_ptr<int64_t>(), grad_C_data.data_ptr(), C_indices.data_ptr<int64_t>(),
-                                C_indptr.data_ptr<int64_t>(), grad_A.data_ptr(), grad_B.data_ptr(),
+                                C_indptr.data_ptr<int64_t>(), ptr_or_null(grad_A), ptr_or_null(grad_B),
                                 current_stream(dev)),
           "nm_splincomb_backward");
     return {grad_A, grad_B};
@@ -973,6 +1007,7 @@ std::vector<Tensor> spdmm_backward(int A_rows, int A_cols, Tensor A_data, Tensor
     const auto dev = need_device({&A_data, &A_indices, &A_indptr, &B, &grad_C});
     same_dtype(A_data, B, "B");
     same_dtype(A_data, grad_C, "grad_C");
+    const Wanted want = wanted(A_data, B);
     A_data = A_data.contiguous();
     A_indices = index_tensor(A_indices, "A_indices");
     A_indptr = index_tensor(A_indptr, "A_indptr");
@@ -981,19 +1016,21 @@ std::vector<Tensor> spdmm_backward(int A_rows, int A_cols, Tensor A_data, Tensor
     grad_C = row_major(grad_C, &ldg);
     const int64_t n = B.size(1);
     c10::hip::HIPGuard guard(dev.index());
-    Tensor grad_A = torch::empty_like(A_data);
-    Tensor grad_B = torch::empty({B.size(0), n}, B.options());
-    if (auto plan = backward_plan(A_indices, A_indptr, A_rows, B.size(0), dev)) {
+    Tensor grad_A, grad_B;
+    if (want.first) grad_A = torch::empty_like(A_data);
+    if (want.second) grad_B = torch::empty({B.size(0), n}, B.options());
+    // (the dot products alone walk A by row and need no plan)
+    if (auto plan = want.second ? backward_plan(A_indices, A_indptr, A_rows, B.size(0), dev) : nullptr) {
         check(nm_spdmm_backward_planned(dtype_of(A_data), A_rows, B.size(0), A_data.numel(), A_data.data_ptr(),
                                         A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
                                         plan->mem.data_ptr(), B.data_ptr(), ldb, grad_C.data_ptr(), ldg, n,
-                                        grad_A.data_ptr(), grad_B.data_ptr(), std::max<int64_t>(n, 1),
+                                        ptr_or_null(grad_A), ptr_or_null(grad_B), std::max<int64_t>(n, 1),
                                         current_stream(dev)),
               "nm_spdmm_backward_planned");
     } else {
         check(nm_spdmm_backward(dtype_of(A_data), A_rows, B.size(0), A_data.numel(), A_data.data_ptr(),
                                 A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B.data_ptr(), ldb,
-                                grad_C.data_ptr(), ldg, n, grad_A.data_ptr(), grad_B.data_ptr(),
+                                grad_C.data_ptr(), ldg, n, ptr_or_null(grad_A), ptr_or_null(grad_B),
                                 std::max<int64_t>(n, 1), current_stream(dev)),
               "nm_spdmm_backward");
     }
@@ -1103,6 +1140,7 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
                                   &B_indices, &B_indptr});
     same_dtype(A_data, B_data, "B_data");
     same_dtype(A_data, grad_C, "grad_C");
+    const Wanted want = wanted(A_data, B_data);
     A_data = A_data.contiguous();
     B_data = B_data.contiguous();
     grad_C = grad_C.contiguous();
@@ -1113,7 +1151,9 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
     C_indices = index_tensor(C_indices, "C_indices");
     C_indptr = index_tensor(C_indptr, "C_indptr");
     c10::hip::HIPGuard guard(dev.index());
-    Tensor grad_A = torch::empty_like(A_data), grad_B = torch::empty_like(B_data);
+    Tensor grad_A, grad_B;
+    if (want.first) grad_A = torch::empty_like(A_data);
+    if (want.second) grad_B = torch::empty_like(B_data);
     if (backward_mode_now() != kAtomic) {
         // the product plan applies when grad_C lies on the very pattern tensors the plan handed out
         auto pp = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, A_rows, B_cols, dev);
@@ -1123,7 +1163,7 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
                                                  B_data.numel(), grad_C.numel(), grad_C.data_ptr(),
                                                  A_data.data_ptr(), pp->parent->mem.data_ptr(), B_data.data_ptr(),
                                                  B_indptr.data_ptr<int64_t>(), pp->mem.data_ptr(),
-                                                 grad_A.data_ptr(), grad_B.data_ptr(), current_stream(dev)),
+                                                 ptr_or_null(grad_A), ptr_or_null(grad_B), current_stream(dev)),
                   "nm_spgemm_backward_mapped_wide");
             return {grad_A, grad_B};
         }
@@ -1147,7 +1187,7 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
                                          grad_C.numel(), grad_C.data_ptr(), C_indices.data_ptr<int64_t>(),
                                          C_indptr.data_ptr<int64_t>(), A_data.data_ptr(), plan->mem.data_ptr(),
                                          B_data.data_ptr(), B_indices.data_ptr<int64_t>(),
-                                         B_indptr.data_ptr<int64_t>(), grad_A.data_ptr(), grad_B.data_ptr(),
+                                         B_indptr.data_ptr<int64_t>(), ptr_or_null(grad_A), ptr_or_null(grad_B),
                                          current_stream(dev)),
               "nm_spgemm_backward_planned");
         return {grad_A, grad_B};
@@ -1155,8 +1195,8 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
     check(nm_spgemm_backward(dtype_of(A_data), A_rows, A_data.numel(), B_data.numel(), grad_C.data_ptr(),
                              C_indices.data_ptr<int64_t>(), C_indptr.data_ptr<int64_t>(), A_data.data_ptr(),
                              A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(), B_data.data_ptr(),
-                             B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(), grad_A.data_ptr(),
-                             grad_B.data_ptr(), current_stream(dev)),
+                             B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(), ptr_or_null(grad_A),
+                             ptr_or_null(grad_B), current_stream(dev)),
           "nm_spgemm_backward");
     return {grad_A, grad_B};
 }
@@ -1188,6 +1228,8 @@ std::vector<Tensor> sptrsv_backward(Tensor grad_x, Tensor x, int A_rows, int A_c
     const auto dev = need_device({&grad_x, &x, &A_data, &A_indices, &A_indptr});
     same_dtype(A_data, grad_x, "grad_x");
     same_dtype(A_data, x, "x");
+    // (grad_A is formed from grad_b, so the transposed solve runs whichever gradient is wanted)
+    const Wanted want = wanted(A_data, b);
     A_data = A_data.contiguous();
     grad_x = grad_x.contiguous();
     x = x.contiguous();
@@ -1196,11 +1238,13 @@ std::vector<Tensor> sptrsv_backward(Tensor grad_x, Tensor x, int A_rows, int A_c
     c10::hip::HIPGuard guard(dev.index());
     auto plan = level_plan(A_indices, A_indptr, A_rows, lower, dev);
     Tensor grad_b = solve(*plan, true, A_data, unit, grad_x, A_rows, dev);
+    if (!want.first) return {Tensor(), grad_b};
     Tensor grad_A = torch::empty_like(A_data);
     check(nm_masked_outer(dtype_of(A_data), A_rows, A_data.numel(), A_indices.data_ptr<int64_t>(),
                           A_indptr.data_ptr<int64_t>(), -1.0, grad_b.data_ptr(), x.data_ptr(), grad_A.data_ptr(),
                           current_stream(dev)),
           "nm_masked_outer");
+    if (!want.second) return {grad_A, Tensor()};
     return {grad_A, grad_b};
 }
 
@@ -1243,11 +1287,11 @@ std::shared_ptr<Plan> lu_pattern(const Tensor &A_indices, const Tensor &A_indptr
                                            Mt_indptr.data_ptr<int64_t>(), Mt_to_M.data_ptr<int64_t>(), stream),
                   "nm_csr_transpose_forward");
             p.derived = {M_indices, M_indptr, Mt_indices, Mt_indptr, Mt_to_M};
-            for (const Tensor &t : p.derived) p.derived_versions.push_back(t._version());
+            for (const Tensor &t : p.derived) p.derived_versions.push_back(version_of(t));
         });
         bool intact = true;   // a caller may have edited the tensors it was handed
         for (size_t i = 0; i < plan->derived.size(); ++i)
-            intact = intact && plan->derived[i]._version() == plan->derived_versions[i];
+            intact = intact && version_of(plan->derived[i]) == plan->derived_versions[i];
         if (intact || attempt > 0) {
             TORCH_CHECK(intact, "the cached factor pattern was modified in place");
             return plan;

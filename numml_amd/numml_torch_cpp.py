@@ -63,6 +63,15 @@ def _same_dtype(a, b, what):
         raise RuntimeError(f"expected {what} of type {a.dtype} but found {b.dtype}")
 
 
+def _wanted(a, b):
+    """Which of its two gradients a backward pass computes: both when neither operand requires a
+    gradient (a direct call outside autograd; what the reference's CPU path gives), otherwise
+    those that are required -- the reference's GPU path computes a gradient only for an operand
+    that requires one (cpp/sparse_csr_cuda.cu:662, :682).  A gradient left out is returned as None."""
+    ra, rb = bool(a.requires_grad), bool(getattr(b, "requires_grad", False))
+    return (True, True) if not (ra or rb) else (ra, rb)
+
+
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
@@ -221,11 +230,12 @@ def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
     dev = _need_device(grad_z, A_data, A_col_ind, A_rowptr, x)
     _same_dtype(A_data, x, "x")
     _same_dtype(A_data, grad_z, "grad_z")
+    want_A, want_x = _wanted(A_data, x)
     A_data, x, grad_z = A_data.contiguous(), x.contiguous(), grad_z.contiguous()
     A_col_ind, A_rowptr = _idx(A_col_ind, "A_col_ind"), _idx(A_rowptr, "A_rowptr")
     with torch.cuda.device(dev):
-        grad_A = torch.empty_like(A_data)
-        grad_x = torch.empty_like(x)
+        grad_A = torch.empty_like(A_data) if want_A else None
+        grad_x = torch.empty_like(x) if want_x else None
         if BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, x.shape[0], A_data.shape[0]):
             plan = _transpose_plan(A_col_ind, A_rowptr, A_rows, x.shape[0], dev)
             _lib.check(_lib.lib().nm_spgemv_backward_planned(
@@ -323,9 +333,10 @@ def splincomb_backward(rows, cols, alpha, A_data, A_indices, A_indptr, beta, B_d
     B_indices, B_indptr = _idx(B_indices, "B_indices"), _idx(B_indptr, "B_indptr")
     C_indices, C_indptr = _idx(C_indices, "C_indices"), _idx(C_indptr, "C_indptr")
     a, b = _scalar(alpha), _scalar(beta)
+    want_A, want_B = _wanted(A_data, B_data)
     with torch.cuda.device(dev):
-        grad_A = torch.empty(A_data.shape[0], dtype=A_data.dtype, device=dev)
-        grad_B = torch.empty(B_data.shape[0], dtype=B_data.dtype, device=dev)
+        grad_A = torch.empty(A_data.shape[0], dtype=A_data.dtype, device=dev) if want_A else None
+        grad_B = torch.empty(B_data.shape[0], dtype=B_data.dtype, device=dev) if want_B else None
         _lib.check(_lib.lib().nm_splincomb_backward(
             _dt(A_data), rows, a, _ptr(A_indices), _ptr(A_indptr), b, _ptr(B_indices), _ptr(B_indptr),
             _ptr(grad_C_data), _ptr(C_indices), _ptr(C_indptr), _ptr(grad_A), _ptr(grad_B), _stream(dev)),
@@ -448,15 +459,16 @@ def spdmm_backward(A_rows, A_cols, A_data, A_indices, A_indptr, B, grad_C):
     dev = _need_device(A_data, A_indices, A_indptr, B, grad_C)
     _same_dtype(A_data, B, "B")
     _same_dtype(A_data, grad_C, "grad_C")
+    want_A, want_B = _wanted(A_data, B)
     A_data = A_data.contiguous()
     A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
     B, ldb = _rowmajor(B)
     grad_C, ldg = _rowmajor(grad_C)
     n = B.shape[1]
     with torch.cuda.device(dev):
-        grad_A = torch.empty_like(A_data)
-        grad_B = torch.empty((B.shape[0], n), dtype=B.dtype, device=dev)
-        if BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, B.shape[0], A_data.shape[0]):
+        grad_A = torch.empty_like(A_data) if want_A else None
+        grad_B = torch.empty((B.shape[0], n), dtype=B.dtype, device=dev) if want_B else None
+        if want_B and BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, B.shape[0], A_data.shape[0]):
             plan = _transpose_plan(A_indices, A_indptr, A_rows, B.shape[0], dev)
             _lib.check(_lib.lib().nm_spdmm_backward_planned(
                 _dt(A_data), A_rows, B.shape[0], A_data.shape[0], _ptr(A_data), _ptr(A_indices),
@@ -537,13 +549,14 @@ def spgemm_backward(grad_C, C_indices, C_indptr,
                        B_data, B_indices, B_indptr)
     _same_dtype(A_data, B_data, "B_data")
     _same_dtype(A_data, grad_C, "grad_C")
+    want_A, want_B = _wanted(A_data, B_data)
     A_data, B_data, grad_C = A_data.contiguous(), B_data.contiguous(), grad_C.contiguous()
     A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
     B_indices, B_indptr = _idx(B_indices, "B_indices"), _idx(B_indptr, "B_indptr")
     C_indices, C_indptr = _idx(C_indices, "C_indices"), _idx(C_indptr, "C_indptr")
     with torch.cuda.device(dev):
-        grad_A = torch.empty_like(A_data)
-        grad_B = torch.empty_like(B_data)
+        grad_A = torch.empty_like(A_data) if want_A else None
+        grad_B = torch.empty_like(B_data) if want_B else None
         if BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, A_cols, A_data.shape[0]):
             plan = _transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev)
             _lib.check(_lib.lib().nm_spgemm_backward_planned(
@@ -885,13 +898,17 @@ def sptrsv_backward(grad_x, x, A_rows, A_cols, A_data, A_indices, A_indptr, lowe
     dev = _need_device(grad_x, x, A_data, A_indices, A_indptr)
     _same_dtype(A_data, grad_x, "grad_x")
     _same_dtype(A_data, x, "x")
+    want_A, want_b = _wanted(A_data, b)
     A_data, grad_x, x = A_data.contiguous(), grad_x.contiguous(), x.contiguous()
     A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
     with torch.cuda.device(dev):
         plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
+        # (grad_A is formed from grad_b, so the transposed solve runs whichever gradient is wanted)
         grad_b = _solve(plan, True, A_data, A_indices, A_indptr, unit, grad_x, A_rows, dev)
+        if not want_A:
+            return [None, grad_b]
         grad_A = torch.empty_like(A_data)
         _lib.check(_lib.lib().nm_masked_outer(
             _dt(A_data), A_rows, A_data.shape[0], _ptr(A_indices), _ptr(A_indptr), -1.0,
             _ptr(grad_b), _ptr(x), _ptr(grad_A), _stream(dev)), "nm_masked_outer")
-    return [grad_A, grad_b]
+    return [grad_A, grad_b if want_b else None]

@@ -502,7 +502,10 @@ class SparseCSRTensor(object):
 
     @property
     def grad(self):
-        return SparseCSRTensor((self.data.grad, self.indices, self.indptr), self.shape, clone=False)
+        # a copy of the values, as in the reference (numml/sparse/_csr.py:620-637 clones what it
+        # wraps): editing A.grad in place must not change the gradient autograd accumulates into.
+        # The pattern tensors are shared with A.
+        return SparseCSRTensor((self.data.grad.clone(), self.indices, self.indptr), self.shape, clone=False)
 
     @property
     def grad_fn(self):

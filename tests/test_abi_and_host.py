@@ -172,6 +172,11 @@ def test_container_from_dense_scipy_and_moves():
     assert A.requires_grad and A.data.requires_grad
     (A.data * torch.tensor([2., 4., 6.])).sum().backward()           # gradients live on A.data
     assert A.grad.data.tolist() == [2., 4., 6.]
+    # A.grad wraps a COPY of the values, like the reference's constructor (numml/sparse/_csr.py:620-637):
+    # an in-place edit of it leaves the gradient autograd accumulates into alone
+    A.grad.data.zero_()
+    assert A.data.grad.tolist() == [2., 4., 6.]
+    assert A.grad.indices.data_ptr() == A.indices.data_ptr()          # the pattern is shared
     E = sp.eye(4, k=-1)
     assert E.indptr.tolist() == [0, 0, 1, 2, 3] and E.indices.tolist() == [0, 1, 2]
     assert "sparse matrix tensor" in repr(A)

@@ -62,7 +62,10 @@ def test_cfg2_spmv_fp32_poisson2048(dev, mode):
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
 
 
-def test_cfg3_spmm_fp32_powerlaw(dev):
+@pytest.mark.parametrize("mode", ["eager", "atomic"])
+def test_cfg3_spmm_fp32_powerlaw(dev, mode):
+    """eager: the fused kernel on the plan (what the benchmark times); atomic: the stateless
+    kernels, which the default mode runs on the first backward of a pattern."""
     rows = cols = 1_000_000
     n = 64
     d, i, p, _ = G.powerlaw(rows, cols, target_nnz=16_000_000, seed=0, dtype=np.float32)
@@ -70,6 +73,8 @@ def test_cfg3_spmm_fp32_powerlaw(dev):
     assert lens.max() == 10_000 and lens.min() >= 1 and 14e6 < d.shape[0] < 17e6
     B, gC = randn(1, (cols, n), np.float32), randn(2, (rows, n), np.float32)
     D, I, P, Bd, Gd = to_dev(dev, d, i, p, B, gC)
+    ext.clear_plan_cache()
+    _binding.set_backward_mode(mode)
     C = ext.spdmm_forward(rows, cols, D, I, P, Bd)
     gA, gB = ext.spdmm_backward(rows, cols, D, I, P, Bd, Gd)
     C, gA, gB = host(C), host(gA), host(gB)
@@ -78,6 +83,14 @@ def test_cfg3_spmm_fp32_powerlaw(dev):
     C64 = A64 @ B.astype(np.float64)
     assert np.all(np.abs(C - C64) <= 1e-5 * np.abs(C64) + 1e-5 * np.abs(C64).max()), "C (all rows, vs double)"
     del C64
+    # grad_A[k] = <gC[row(k)], B[col(k)]> (cpp/sparse_csr_cpu.cpp:625-636), EVERY stored entry, in
+    # double, a million entries at a time
+    row_of = np.repeat(np.arange(rows, dtype=np.int64), lens)
+    want = np.empty(d.shape[0], np.float64)
+    for k0 in range(0, d.shape[0], 1 << 20):
+        k1 = min(k0 + (1 << 20), d.shape[0])
+        want[k0:k1] = np.einsum("kn,kn->k", gC[row_of[k0:k1]].astype(np.float64), B[i[k0:k1]].astype(np.float64))
+    assert np.all(np.abs(gA - want) <= 1e-5 * np.abs(want) + 1e-5 * np.abs(want).max()), "grad_A (all entries, vs double)"
     # oracle on the first 30k rows (its row->column->entry loop is slow): C and grad_A are row-local
     sub = 30_000
     nz = int(p[sub])
@@ -92,7 +105,7 @@ def test_cfg3_spmm_fp32_powerlaw(dev):
     sl = slice(int(p[r]), int(p[r + 1]))
     one = np.array([0, lens[r]], dtype=np.int64)
     assert_close(C[r:r + 1], oracle.spdmm_forward(1, cols, d[sl], i[sl], one, B), "C (longest row)")
-    # grad_B = A^T gC against SciPy in double, all rows
+    # grad_B = A^T gC against SciPy in double, all rows (cpp/sparse_csr_cpu.cpp:639-646)
     At = A64.T.tocsr()
     gB_ref = (At @ gC.astype(np.float64))
     scale = np.abs(gB_ref).max()
@@ -101,6 +114,18 @@ def test_cfg3_spmm_fp32_powerlaw(dev):
     lhs = float(np.sum(C.astype(np.float64) * gC))
     rhs = float(np.sum(gB.astype(np.float64) * B))
     assert abs(lhs - rhs) <= 1e-4 * abs(lhs)
+    # the gradient somebody asked for alone: the transposed product without the dot products
+    # (the fixed adjacency of a GNN layer), and the dot products without the transposed product
+    Breq = Bd.clone().requires_grad_(True)
+    none_A, gB1 = ext.spdmm_backward(rows, cols, D, I, P, Breq, Gd)
+    assert none_A is None
+    if mode == "eager":
+        assert_same(host(gB1), gB, "grad_B alone")
+    else:
+        assert np.all(np.abs(host(gB1) - gB_ref) <= 1e-5 * np.abs(gB_ref) + 1e-5 * scale), "grad_B alone"
+    gA1, none_B = ext.spdmm_backward(rows, cols, D.clone().requires_grad_(True), I, P, Bd, Gd)
+    assert none_B is None
+    assert np.all(np.abs(host(gA1) - want) <= 1e-5 * np.abs(want) + 1e-5 * np.abs(want).max()), "grad_A alone"
 
 
 def test_cfg4_spgemm_fp64_laplace128(dev):
