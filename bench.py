@@ -29,7 +29,10 @@ on):
   lincomb    fp32 A - B (splincomb) + its backward, both on the spmv matrix pattern
   spgemm_wide  fp64 A (A A) forward + backward on the 3D matrix: 25-entry rows of the right operand
   transpose  fp32 explicit CSR transpose + its backward on the spmv matrix
-  copy    256 MiB device copy (counter calibration / practical bandwidth ceiling)
+  copy    256 MiB device copy (counter calibration)
+  stream  a plain streaming kernel at several mixes of bytes read and written (the part's practical
+          ceiling; the spmv line carries it at the SpMV kernels' own mixes as `stream_ceiling`)
+  spgemm_hash  fp64 (A A) A forward + backward: 25-entry rows of the left operand, the hash kernels
   ref_timing  the shapes the reference's own timing script uses (demos/timing.py:177-217,
           264-348, 520-558): tridiagonal SpMV N = 32 768, tridiagonal SpSpMM and SpDMM
           N = 16 384, bidiagonal SpTRSV N = 32 768, through the Python surface, us per call
@@ -62,17 +65,22 @@ def _source_sha(files):
     return h.hexdigest()[:16]
 
 
-def _traffic(workload):
-    """Measured HBM bytes per launch of the dominant kernel, from the committed
-    rocprofv3 counter summaries (profiles/traffic.json; a separate counter run, not
-    this one), or None.  An entry records the hash of the kernel sources it was
-    measured on; when those have changed since, the figure is stale and None is
-    reported instead."""
+def _traffic(workload, kernel=None):
+    """Measured HBM bytes per launch, from the committed rocprofv3 counter summaries
+    (profiles/traffic.json; a separate counter run, not this one), or None: of the workload's
+    dominant kernel or, with `kernel`, of the kernel whose name contains that string.  An entry
+    records the hash of the kernel sources it was measured on; when those have changed since,
+    the figure is stale and None is reported instead."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
             entry = json.load(f).get(workload, {})
         if "sources" in entry and _source_sha(entry["sources"]) != entry.get("sources_sha16"):
+            return None
+        if kernel is not None:
+            for name, rec in entry.get("per_kernel", {}).items():
+                if kernel in name:
+                    return rec.get("traffic_bytes")
             return None
         return entry.get("traffic_bytes")
     except (OSError, ValueError):
@@ -96,11 +104,61 @@ class Workload:
         """Runs the dominant launch once (events are recorded around this call)."""
         raise NotImplementedError
 
+    def ops(self):
+        """The launches of a step that are timed one by one with events: a list of
+        (kernel name, callable, algorithmic bytes, name in the profiler's tables).  The longest of
+        them is the step's dominant kernel.  Default: the one `dominant` launch."""
+        return [(self.dominant_name, self.dominant, self.dominant_bytes, None)]
+
     def value(self, ms_per_step):
         return self.bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
     def cpu_baseline(self, budget_s):
         raise NotImplementedError
+
+
+def _event_ms(call, reps):
+    """Mean time of one `call` in ms, events recorded around each of `reps` calls on torch's
+    current stream (the stream the extension hands to the C ABI)."""
+    import torch
+    call()
+    evs = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        call()
+        e1.record()
+        evs.append((e0, e1))
+    torch.cuda.synchronize()
+    return float(np.mean([a.elapsed_time(b) for a, b in evs]))
+
+
+def stream_ceiling(dev, mixes):
+    """What this part streams with a plain kernel (nm_stream_probe: 16-byte nontemporal requests,
+    grid stride) at given mixes of bytes read and written: `mixes` maps a label to (read bytes,
+    written bytes).  Every launch starts somewhere else in a 1 GiB source, so that what the
+    memory-side cache keeps of one launch is of no use to the next.  GB/s per label."""
+    import torch
+    from numml_amd import _binding
+    ext = _binding.ops
+    if not hasattr(ext, "stream_probe"):
+        return None
+    span = 1 << 30
+    src = torch.empty(span // 4, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty((256 << 20) // 4, dtype=torch.float32, device=dev)
+    out = {}
+    for label, (rd, wr) in mixes.items():
+        rd, wr = int(rd) // 16 * 16, min(int(wr), int(rd), 256 << 20) // 16 * 16
+        starts = [(k * (160 << 20)) % (span - rd) // 16 * 16 for k in range(8)] if rd < span else [0]
+        state = {"k": 0}
+        def one():
+            off = starts[state["k"] % len(starts)] // 4
+            state["k"] += 1
+            ext.stream_probe(src[off:], rd, dst, wr)
+        ms = _event_ms(one, 24)
+        out[label] = {"read_bytes": rd, "write_bytes": wr, "ms": round(ms, 5),
+                      "GBps": round((rd + wr) / (ms * 1e-3) / 1e9, 1)}
+    return out
 
 
 def _first_calls(ext, call, n=3):
@@ -195,6 +253,22 @@ class SpMV(Workload):
         if _binding.backward_mode() != "atomic" and not planned:    # ctypes mirror: planned backward only
             i_bwd = _spmv_plan_widths(i, p, rows, cols)[1]
         self.fwd_bytes, self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s, i_fwd, i_bwd, planned=_binding.backward_mode() != "atomic")
+        # What the plan build found (compiled binding): blocks of 512 rows / 256 columns whose
+        # entries name few enough 128-element segments of x / g get a staging list (64 bytes a
+        # block, read by the kernels) and 16-bit places in it instead of column offsets.
+        self.plan_info = None
+        if planned and hasattr(ext, "transpose_plan_info") and self.nnz:
+            sym, pk_b, pk_f, st_r, n_r, st_c, n_c = ext.transpose_plan_info(rows, cols, self.I, self.P)
+            self.plan_info = {"symmetric": bool(sym), "packed_backward": bool(pk_b), "packed_forward": bool(pk_f),
+                              "row_blocks_with_staging_list": st_r, "row_blocks": n_r,
+                              "column_blocks_with_staging_list": st_c, "column_blocks": n_c}
+            mean = -(-self.nnz // rows)
+            if st_r == n_r and 4096 // max(mean, 1) >= 512 and i_fwd > 2:
+                i_fwd = 2               # every block has a list: 16-bit places whatever the offsets are
+                self.fwd_bytes = _spmv_bytes(rows, cols, self.nnz, s, i_fwd, i_bwd, planned=True)[0]
+            if 4096 // max(mean, 1) >= 512:
+                self.fwd_bytes += 64 * st_r
+            self.bwd_bytes += 64 * st_c
         self.bytes_per_step = self.fwd_bytes + self.bwd_bytes
         self.dominant_bytes = self.bwd_bytes
         self.dominant_name = ("spmv_bwd_planned_kernel" if _binding.backward_mode() != "atomic"
@@ -213,6 +287,17 @@ class SpMV(Workload):
                        "bytes_per_step_with_int32_structure": sum(_spmv_bytes(rows, cols, self.nnz, s, 4, 8, planned=True)),
                        "binding": _binding.name,
                        "algorithmic_bytes_per_step": self.bytes_per_step}
+        if self.plan_info:
+            self.config["plan"] = self.plan_info
+
+    def ops(self):
+        from numml_amd import _binding
+        planned = _binding.backward_mode() != "atomic"
+        return [("spmv_fwd_kernel" + (" (on the plan's structure)" if planned else ""),
+                 lambda: self.ext.spgemv_forward(self.rows, self.cols, self.D, self.I, self.P, self.X),
+                 self.fwd_bytes, "spmv_fwd_kernel"),
+                (self.dominant_name, self.dominant, self.bwd_bytes,
+                 "spmv_bwd_planned_kernel" if planned else "spmv_bwd_kernel")]
 
     def after(self, rec, steps):
         """The same step without a plan (stateless backward with atomics), the cost of building
@@ -235,7 +320,8 @@ class SpMV(Workload):
             stateless = (time.perf_counter() - t0) / steps * 1e3
         finally:
             _binding.set_backward_mode(mode)
-        build = max(self.first_backward_ms) - rec["roofline"]["avg_ms"]
+        bwd_ms = next(k["avg_ms"] for k in rec["kernels"] if "bwd" in k["name"])
+        build = max(self.first_backward_ms) - bwd_ms
         gain = stateless - rec["ms_per_step"]
         # the same steps priced on the structure as the interface delivers it (int64) and on the
         # plan's plain 32-bit structure (int32 columns forward, two int32 per entry backward: the
@@ -333,9 +419,38 @@ class SpMM(Workload):
         walks = 3 if _binding.backward_mode() == "atomic" else 2
         self.gather_inclusive_bytes = self.bytes_per_step + walks * nnz * n * s - walks * cols * n * s
 
+    def ops(self):
+        from numml_amd import _binding
+        planned = _binding.backward_mode() != "atomic"
+        return [("spdmm_fwd_flat_kernel",
+                 lambda: self.ext.spdmm_forward(self.rows, self.cols, self.D, self.I, self.P, self.B),
+                 self.fwd_bytes, "spdmm_fwd_flat_kernel"),
+                (self.dominant_name, self.dominant, self.bwd_bytes,
+                 "spdmm_bwd_fused_kernel" if planned else "spdmm_bwd_kernel")]
+
     def after(self, rec, steps):
         """The same step priced on the bytes that are gathered, not on the operands' sizes: what the
-        caches have to deliver when no two entries share a row of the dense operand."""
+        caches have to deliver when no two entries share a row of the dense operand.  And the step
+        of a layer whose matrix is fixed (a GNN's adjacency): only the dense operand requires a
+        gradient, so the backward is the transposed product alone."""
+        import torch
+        Breq = self.B.detach().clone().requires_grad_(True)
+        def step_b_only():
+            self.ext.spdmm_forward(self.rows, self.cols, self.D, self.I, self.P, Breq)
+            gA, gB = self.ext.spdmm_backward(self.rows, self.cols, self.D, self.I, self.P, Breq, self.Gv)
+            assert gA is None and gB is not None
+        for _ in range(3):
+            step_b_only()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step_b_only()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        s, n, nnz = 4, self.n, self.nnz
+        b_only = self.fwd_bytes + nnz * (s + 8) + (self.cols + 1) * 4 + self.rows * n * s + self.cols * n * s
+        rec["config"]["ms_per_step_grad_B_only"] = round(ms, 5)
+        rec["config"]["GBps_grad_B_only"] = round(b_only / (ms * 1e-3) / 1e9, 1)
         gi = self.gather_inclusive_bytes
         rec["roofline_gather_inclusive"] = {
             "bytes_per_step": int(gi), "achieved": round(gi / (rec["ms_per_step"] * 1e-3) / 1e9, 1),
@@ -420,6 +535,9 @@ class SpGEMM(Workload):
         self.flops = 2 * self.products
         s = 8
         nnzR = int(self.hostR[0].shape[0])
+        # plan bytes per entry of the left operand: one 16-byte record, or (rows of the right operand
+        # of 17 to 32 entries) a row start and four octets of destination bytes
+        plan_bytes_of = lambda right: 4 + 8 * 4 if right == "AA" else 16
         # Compulsory traffic of the forward: both operands and the result once, the two row
         # pointer arrays.  The gather-inclusive figure (every referenced row of the right operand
         # read again for every product) is an upper bound and is reported apart; most of those
@@ -435,12 +553,21 @@ class SpGEMM(Workload):
             # written again
             # (rows of the right operand of 17 to 32 entries: row start and four octets of
             # destination bytes from separate arrays)
-            plan_bytes = 4 + 8 * 4 if self.right == "AA" else 16
+            plan_bytes = plan_bytes_of(self.right)
             self.bytes_per_step = self.nnz * (s + plan_bytes) + nnzR * s + self.nnzC * s + 2 * rows * 8
             self.dominant_bytes = self.bytes_per_step
             self.dominant_name = ("numeric_planned_wide_kernel (the whole forward on the product plan)"
                                   if self.right == "AA" else
                                   "numeric_planned_kernel (the whole forward on the product plan)")
+        # Backward on the product plan (grad_ab_mapped_kernel: both gradients from one walk over A by
+        # column): the gradient of C, the values of both operands, the plan's column-major record of
+        # every entry of A, the column pointers of A and the row pointers of B in; both gradients out.
+        # Stateless (spgemm_bwd_kernel): the pattern of C and both operands' patterns as well, and
+        # grad_B is cleared first.
+        self.bwd_bytes_planned = (self.nnzC * s + self.nnz * s + nnzR * s + self.nnz * plan_bytes_of(self.right)
+                                  + (cols + 1) * 4 + (rows + 1) * 8 + self.nnz * s + nnzR * s)
+        self.bwd_bytes_stateless = (self.nnzC * (s + 8) + (rows + 1) * 8 + self.nnz * (s + 8) + nnzR * (s + 8)
+                                    + 2 * (rows + 1) * 8 + self.nnz * s + 2 * nnzR * s)
         self.config = {"workload": f"spgemm_{self.left}x{self.right}_fwd_bwd_f64_laplace3d_{n}", "rows": rows,
                        "nnz_left": self.nnz, "nnz_right": nnzR,
                        "nnz_C": self.nnzC, "products": self.products, "index_bytes": 8,
@@ -459,6 +586,24 @@ class SpGEMM(Workload):
         g = self.ext.spgemm_backward(self.gC, C[1], C[2], self.rows, self.cols, *self.L,
                                      self.rows, self.cols, *self.R)
         return C, g
+
+    def backward(self):
+        C = self.C
+        return self.ext.spgemm_backward(self.gC, C[1], C[2], self.rows, self.cols, *self.L,
+                                        self.rows, self.cols, *self.R)
+
+    def ops(self):
+        self.C = self.dominant()            # the pattern tensors a backward on the plan has to be given
+        if self.planned:
+            wide = self.right == "AA"
+            return [(self.dominant_name, self.dominant, self.dominant_bytes,
+                     "numeric_planned_wide_kernel" if wide else "numeric_planned_kernel"),
+                    ("grad_a_wide_kernel + grad_b_wide_kernel (both gradients on the product plan)" if wide else
+                     "grad_ab_mapped_kernel (both gradients from one walk over A by column, on the product plan)",
+                     self.backward, self.bwd_bytes_planned, "grad_b_wide_kernel" if wide else "grad_ab_mapped_kernel")]
+        return [(self.dominant_name, self.dominant, self.dominant_bytes, "numeric_front_kernel"),
+                ("spgemm_bwd_kernel (+ fill_kernel clearing grad_B)", self.backward, self.bwd_bytes_stateless,
+                 "spgemm_bwd_kernel")]
 
     def after(self, rec, steps):
         """The same step with no plan of any kind (symbolic + numeric forward, search-free atomic
@@ -488,8 +633,26 @@ class SpGEMM(Workload):
                 evs.append((e0, e1))
             torch.cuda.synchronize()
             fwd = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+            self.C = self.dominant()
+            bwd = _event_ms(self.backward, steps)
         finally:
             _binding.set_backward_mode(mode)
+        # the path every first product on a pair of patterns takes (and the only one for rows
+        # beyond a plan's limits): merge kernels where every row is short, the hash kernels otherwise
+        hashed = self.left == "AA" or self.right == "AA"
+        fwd_name = ("symbolic_hash_kernel + numeric_hash_kernel (row-binned LDS hash tables) + scans, host read of nnz(C)"
+                    if hashed else "symbolic_front_kernel + numeric_front_kernel (merge path) + scans, host read of nnz(C)")
+        rec["roofline_stateless"] = {
+            "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "kernels": [
+                {"name": fwd_name, "avg_ms": round(fwd, 5), "algorithmic_bytes": int(self.stateless_forward_bytes),
+                 "achieved": round(self.stateless_forward_bytes / (fwd * 1e-3) / 1e9, 1),
+                 "frac": round(self.stateless_forward_bytes / (fwd * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                 "GFLOPs": round(self.flops / (fwd * 1e-3) / 1e9, 1)},
+                {"name": "spgemm_bwd_kernel (+ fill_kernel clearing grad_B)", "avg_ms": round(bwd, 5),
+                 "algorithmic_bytes": int(self.bwd_bytes_stateless),
+                 "achieved": round(self.bwd_bytes_stateless / (bwd * 1e-3) / 1e9, 1),
+                 "frac": round(self.bwd_bytes_stateless / (bwd * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}]}
         build = max(self.first_steps_ms) - stateless
         gain = stateless - rec["ms_per_step"]
         c = rec["config"]
@@ -511,13 +674,22 @@ class SpGEMM(Workload):
     def cpu_baseline(self, budget_s):
         import oracle
         rows, cols = self.rows, self.cols
+        # the full product of the metric's configuration (3.5 s); of a larger one the first rows of
+        # the left operand (the product is row-local), scaled by the products they make
+        sub = rows if self.products <= 150_000_000 else max(1, int(rows * 40_000_000 / self.products))
+        Ld, Li, Lp = self.hostL
+        nz = int(Lp[sub])
+        L = (Ld[:nz], Li[:nz], Lp[:sub + 1])
+        done = int(np.diff(self.hostR[2])[Li[:nz]].sum())
         t0 = time.perf_counter()
-        C = oracle.spgemm_forward(rows, cols, *self.hostL, rows, cols, *self.hostR)
+        C = oracle.spgemm_forward(sub, cols, *L, rows, cols, *self.hostR)
         gC = np.random.default_rng(1).standard_normal(C[0].shape[0])
-        oracle.spgemm_backward(gC, C[1], C[2], rows, cols, *self.hostL, rows, cols, *self.hostR)
+        oracle.spgemm_backward(gC, C[1], C[2], sub, cols, *L, rows, cols, *self.hostR)
         el = time.perf_counter() - t0
-        return {"value": self.flops / el / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
-                "sample": "1 x (spgemm_forward + spgemm_backward) of the full workload, serial C oracle "
+        what = ("the full workload" if sub == rows else
+                f"the first {sub} rows of the left operand ({done} of {self.products} products), scaled by products")
+        return {"value": 2 * done / el / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+                "sample": f"1 x (spgemm_forward + spgemm_backward) of {what}, serial C oracle "
                           "(bisection instead of the reference's std::map lookup)"}
 
 
@@ -565,6 +737,14 @@ class SpTRSV(Workload):
 
     def dominant(self):
         return self.ext.sptrsv_forward(self.rows, self.rows, self.D, self.I, self.P, True, False, self.Bv)
+
+    def ops(self):
+        x = self.dominant()
+        s = 8
+        return [(self.dominant_name, self.dominant, self.dominant_bytes, "sptrsv_ell_kernel"),
+                ("backward: transposed solve (the same three kernels on the packed A^T) + spmv_bwd_kernel as the masked outer product",
+                 lambda: self.ext.sptrsv_backward(self.Gv, x, self.rows, self.rows, self.D, self.I, self.P, True, False, self.Bv),
+                 self.dominant_bytes + self.nnz * (s + 8) + 2 * self.rows * s, None)]
 
     def value(self, ms_per_step):
         return ms_per_step
@@ -947,7 +1127,9 @@ def ref_timing(dev, cpu_seconds):
 
 
 # The other configurations the metric names, measured beside the headline in the default run.
-EXTRAS = ("spmm", "spgemm", "sptrsv", "spmv64")
+# (`spgemm_hash`, off those configurations, is the product that takes the row-binned hash kernels;
+# the 7-point matrix squared never leaves the merge path.)
+EXTRAS = ("spmm", "spgemm", "spgemm_hash", "sptrsv", "spmv64")
 
 
 def measure(w, dev, steps, warmup, cpu_seconds):
@@ -967,22 +1149,22 @@ def measure(w, dev, steps, warmup, cpu_seconds):
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / steps * 1e3
 
-    # Kernel-level timing for the roofline: the same launches, events around each one on the
-    # stream they run on (torch's current stream is the one handed to the C ABI).
-    evs = []
-    for _ in range(steps):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        w.dominant()
-        e1.record()
-        evs.append((e0, e1))
-    torch.cuda.synchronize()
-    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
-    achieved = w.dominant_bytes / (kernel_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": w.dominant_name, "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "algorithmic_bytes": int(w.dominant_bytes), "avg_ms": round(kernel_ms, 5),
-                "traffic": _traffic(w.name)}
+    # Kernel-level timing for the roofline: the launches of a step one by one, events around each
+    # on the stream they run on (torch's current stream is the one handed to the C ABI).  The
+    # roofline object is that of the LONGEST of them, the step's dominant kernel.
+    kernels = []
+    for name, call, nbytes, prof_name in w.ops():
+        ms = _event_ms(call, steps)
+        achieved = nbytes / (ms * 1e-3) / 1e9
+        kernels.append({"name": name, "avg_ms": round(ms, 5), "algorithmic_bytes": int(nbytes),
+                        "achieved": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBS, 4),
+                        "traffic": _traffic(w.name, prof_name) if prof_name else None})
+    top = max(kernels, key=lambda k: k["avg_ms"])
+    roofline = {"bound": "hbm", "kernel": top["name"], "achieved": top["achieved"],
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": top["frac"],
+                "algorithmic_bytes": top["algorithmic_bytes"], "avg_ms": top["avg_ms"],
+                "traffic": top["traffic"] if top["traffic"] is not None else
+                (_traffic(w.name) if top["name"] == getattr(w, "dominant_name", None) else None)}
 
     cpu = None
     if cpu_seconds > 0:
@@ -996,7 +1178,7 @@ def measure(w, dev, steps, warmup, cpu_seconds):
         "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": w.higher_is_better, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic", "config": w.config,
-        "roofline": roofline, "cpu_baseline": cpu,
+        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
     }
     if w.unit == "GB/s":
         rec["pct_of_hbm_peak"] = round(100.0 * value / HBM_PEAK_GBS, 2)
@@ -1010,7 +1192,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="spmv", choices=sorted(WORKLOADS) + ["ref_timing"])
+    ap.add_argument("--workload", default="spmv", choices=sorted(WORKLOADS) + ["ref_timing", "stream"])
     ap.add_argument("--cpu-seconds", type=float, default=10.0,
                     help="CPU time budget of the cpu_baseline leg (0 skips it)")
     ap.add_argument("--no-extras", action="store_true",
@@ -1032,12 +1214,38 @@ def main():
     if args.workload == "ref_timing":
         print(json.dumps(ref_timing(dev, args.cpu_seconds)))
         return
+    if args.workload == "stream":
+        mib = 1 << 20
+        print(json.dumps({"metric": "plain streaming kernel, GB/s by mix of reads and writes", "unit": "GB/s",
+                          "n_gpus": 1, "data": "synthetic", "config": {"workload": "stream"},
+                          "mixes": stream_ceiling(dev, {"read_only_256MiB": (256 * mib, 0),
+                                                        "copy_256MiB": (256 * mib, 256 * mib),
+                                                        "2_reads_1_write": (256 * mib, 128 * mib),
+                                                        "9_reads_1_write": (180 * mib, 20 * mib)})}))
+        return
 
-    out = measure(WORKLOADS[args.workload](), dev, args.steps, args.warmup, args.cpu_seconds)
+    w = WORKLOADS[args.workload]()
+    out = measure(w, dev, args.steps, args.warmup, args.cpu_seconds)
+    if args.workload in ("spmv", "spmv64", "spmv_rows25"):
+        # The same part's plain streaming rate at each kernel's own mix of bytes read and written
+        # (and the step's), next to the kernels' fractions of the 8 TB/s peak.
+        s = w.D.element_size()
+        fwd_w, bwd_w = w.rows * s, w.nnz * s + w.cols * s
+        mixes = stream_ceiling(dev, {"forward_mix": (w.fwd_bytes - fwd_w, fwd_w),
+                                     "backward_mix": (w.bwd_bytes - bwd_w, bwd_w),
+                                     "step_mix": (w.bytes_per_step - fwd_w - bwd_w, fwd_w + bwd_w),
+                                     "read_only_256MiB": (256 << 20, 0), "copy_256MiB": (256 << 20, 256 << 20)})
+        if mixes:
+            out["stream_ceiling"] = mixes
+            for k in out["kernels"]:
+                mix = mixes["forward_mix" if "fwd" in k["name"] else "backward_mix"]
+                k["frac_of_stream_ceiling"] = round(k["achieved"] / mix["GBps"], 4)
+            out["frac_of_stream_ceiling"] = round(out["value"] / mixes["step_mix"]["GBps"], 4)
     if args.workload == "spmv" and not args.no_extras:
         from numml_amd import _binding
         keep = ("value", "unit", "ms_per_step", "steps", "warmup", "higher_is_better", "dtype", "config",
-                "roofline", "roofline_gather_inclusive", "cpu_baseline", "pct_of_hbm_peak", "value_note")
+                "roofline", "roofline_stateless", "kernels", "roofline_gather_inclusive", "cpu_baseline",
+                "pct_of_hbm_peak", "value_note")
         out["workloads"] = {}
         for name in EXTRAS:
             _binding.ops.clear_plan_cache()
@@ -1045,6 +1253,12 @@ def main():
             rec = measure(WORKLOADS[name](), dev, args.extra_steps, min(args.warmup, 3),
                           min(args.cpu_seconds, args.extra_cpu_seconds))
             out["workloads"][name] = {k: rec[k] for k in keep if k in rec}
+        # the shapes the reference's own timing script uses, through the Python surface
+        _binding.ops.clear_plan_cache()
+        torch.cuda.empty_cache()
+        rt = ref_timing(dev, min(args.cpu_seconds, args.extra_cpu_seconds))
+        out["workloads"]["ref_timing"] = {"unit": "us", "config": rt["config"], "cpu_baseline": rt["cpu_baseline"],
+                                          "rows": rt["rows"]}
     print(json.dumps(out))
 
 

@@ -42,6 +42,13 @@ int nm_version(void);
 /* Message of the last failure on the calling thread ("" if none). */
 const char *nm_last_error(void);
 
+/* Calibration of the bandwidth figures, no counterpart in the reference: one
+ * plain kernel that reads `read_bytes` from src and writes `write_bytes` to dst
+ * (both multiples of 16, write_bytes <= read_bytes; 16-byte requests, grid
+ * stride), i.e. what this part streams at a given mix of reads and writes.  The
+ * SpMV kernels' mixes are measured with it next to their own rates. */
+int nm_stream_probe(const void *src, size_t read_bytes, void *dst, size_t write_bytes, nm_stream stream);
+
 /* ------------------------------------------------------------------ SpMV
  * y = A x.  Stands in for spgemv_forward (cpp/sparse_csr.hpp:32-36,
  * cpp/sparse_csr_cpu.cpp:11-39; CUDA launch site cpp/sparse_csr_cuda.cu:42-67).
@@ -96,6 +103,16 @@ int nm_csr_transpose_plan_build(int64_t rows, int64_t cols, int64_t nnz,
                                 const int64_t *indices, const int64_t *indptr,
                                 void *plan_mem, size_t plan_bytes,
                                 void *work, size_t work_bytes, nm_stream stream);
+
+/* What a built plan found out about the pattern, copied to the host: info[0]
+ * pattern symmetric, info[1] / info[2] the packed words of the backward / the
+ * 16-bit column offsets of the forward are valid, info[4] blocks of 512 rows
+ * with a staging list (the SpMV forward loads the segments of x such a block
+ * names into LDS), info[5] blocks of 256 columns with one (the same for the
+ * backward); the other entries are 0.  Waits for `stream`.  Diagnostics: no
+ * counterpart in the reference. */
+int nm_csr_transpose_plan_info(int64_t rows, int64_t cols, int64_t nnz, const void *plan_mem,
+                               int32_t info[16], nm_stream stream);
 
 /* The explicit transpose.  Stands in for csr_transpose_forward
  * (cpp/sparse_csr.hpp:57-61, cpp/sparse_csr_cpu.cpp:311-367): widens a built

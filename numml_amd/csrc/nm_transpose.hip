@@ -296,6 +296,7 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
 
 __global__ void symmetry_init_kernel(int32_t *flags, int square) {
     if (threadIdx.x == 0) {
+        for (int k = 0; k < 16; ++k) flags[k] = 0;
         flags[0] = square;
         flags[1] = 1;
         flags[2] = 1;
@@ -346,7 +347,7 @@ template <bool FWD, int MOST>
 __global__ __launch_bounds__(kBlock) void tp_stage_kernel(
     int64_t nblocks, int64_t nlines, int64_t veclen, const int32_t *__restrict__ ptr, const int32_t *__restrict__ key,
     int32_t *__restrict__ t_pack, int16_t *__restrict__ c_off16, int32_t *__restrict__ desc,
-    const int32_t *__restrict__ flags) {
+    int32_t *__restrict__ flags) {
     constexpr int kSlots = 64, kBlockLines = FWD ? nm::kPackRows : nm::kPackCols;
     constexpr int kMostEntries = FWD ? nm::kStageFwdCap : nm::kStageBwdCap;
     __shared__ int32_t s_tab[kSlots], s_rank[kSlots], s_count, s_bad;
@@ -390,6 +391,7 @@ __global__ __launch_bounds__(kBlock) void tp_stage_kernel(
         }
         __syncthreads();
         const bool staged = s_bad == 0 && s_count <= MOST;
+        if (staged && threadIdx.x == 0) atomicAdd(&flags[FWD ? 4 : 5], 1);    // (nm_csr_transpose_plan_info)
         if (staged && threadIdx.x < kSlots) {
             const int32_t mine = s_tab[threadIdx.x];
             if (mine >= 0) {
@@ -558,4 +560,17 @@ extern "C" int nm_csr_transpose_plan_build(int64_t rows, int64_t cols, int64_t n
         return nm::fail(NM_ERR_WORKSPACE, "plan memory of %zu bytes, %zu needed", plan_bytes, need);
     return nm::tplan_build(rows, cols, nnz, indices, indptr, plan, work, work_bytes, nullptr,
                            nm::as_stream(stream));
+}
+
+extern "C" int nm_csr_transpose_plan_info(int64_t rows, int64_t cols, int64_t nnz, const void *plan_mem,
+                                          int32_t info[16], nm_stream stream) {
+    if (int rc = check_sizes(rows, cols, nnz)) return rc;
+    NM_REQUIRE(plan_mem != nullptr && info != nullptr, "null pointer argument");
+    nm::TPlan plan;
+    nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &plan);
+    hipStream_t s = nm::as_stream(stream);
+    NM_HIP_TRY(hipMemcpyAsync(info, plan.flags, 16 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    NM_HIP_TRY(hipStreamSynchronize(s));
+    if (nnz == 0) info[1] = info[2] = info[4] = info[5] = 0;     // (nothing was packed or listed)
+    return NM_OK;
 }

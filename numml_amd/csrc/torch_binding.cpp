@@ -1407,6 +1407,36 @@ std::tuple<int64_t, int64_t> sptrsv_chain_levels(int A_rows, Tensor A_indices, T
     return {nm_sptrsv_plan_chain_levels(plan->handle, 0), nm_sptrsv_plan_chain_levels(plan->handle, 1)};
 }
 
+// What the transposed-structure plan of a pattern (the cached one, or one built now) found out:
+// (symmetric, packed words of the backward valid, 16-bit column offsets of the forward valid,
+// row blocks with a staging list, row blocks, column blocks with one, column blocks).
+// Diagnostics; waits for the stream.
+std::vector<int64_t> transpose_plan_info(int A_rows, int A_cols, Tensor A_indices, Tensor A_indptr) {
+    TORCH_CHECK(A_indptr.dim() == 1 && A_indptr.numel() == (int64_t)A_rows + 1 && A_indices.dim() == 1,
+                "transpose_plan_info: expected ", A_rows + 1, " row pointers, got shape ", A_indptr.sizes());
+    const auto dev = need_device({&A_indices, &A_indptr});
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    auto plan = transpose_plan(A_indices, A_indptr, A_rows, A_cols, dev);
+    int32_t info[16];
+    check(nm_csr_transpose_plan_info(A_rows, A_cols, A_indices.numel(), plan->mem.data_ptr(), info,
+                                     current_stream(dev)),
+          "nm_csr_transpose_plan_info");
+    return {info[0], info[1], info[2], info[4], ((int64_t)A_rows + 511) / 512, info[5], ((int64_t)A_cols + 255) / 256};
+}
+
+// Time-free helper of the bandwidth calibration: enqueues one nm_stream_probe launch.
+void stream_probe(Tensor src, int64_t read_bytes, Tensor dst, int64_t write_bytes) {
+    const auto dev = need_device({&src, &dst});
+    TORCH_CHECK(src.is_contiguous() && dst.is_contiguous() && read_bytes <= (int64_t)src.nbytes() &&
+                    write_bytes <= (int64_t)dst.nbytes(),
+                "stream_probe: buffers smaller than the byte counts");
+    c10::hip::HIPGuard guard(dev.index());
+    check(nm_stream_probe(src.data_ptr(), (size_t)read_bytes, dst.data_ptr(), (size_t)write_bytes, current_stream(dev)),
+          "nm_stream_probe");
+}
+
 void clear_plan_cache() {
     std::lock_guard<std::mutex> lock(g_plans_mutex);
     g_plans.clear();
@@ -1477,6 +1507,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sptrsv_schedule", &sptrsv_schedule, "(levels, launches per solve) of a triangular pattern");
     m.def("sptrsv_chain_levels", &sptrsv_chain_levels,
           "levels of the solves with A and with A^T that the single-wavefront chain kernels take");
+    m.def("transpose_plan_info", &transpose_plan_info,
+          "(symmetric, packed backward, packed forward, staged row blocks, row blocks, staged column blocks, "
+          "column blocks) of a pattern's transposed-structure plan");
+    m.def("stream_probe", &stream_probe, "one launch of the streaming calibration kernel (read_bytes in, write_bytes out)");
     m.def("clear_plan_cache", &clear_plan_cache, "Drop every cached structure plan");
     m.def("plan_cache_size", &plan_cache_size, "Number of cached structure plans");
     m.def("plan_cache_bytes", &plan_cache_bytes, "Device memory held by the cached structure plans");

@@ -38,7 +38,7 @@ def test_ctypes_table_covers_the_header():
                                      "nm_sptrsv_plan_launches", "nm_sptrsv_plan_chain_levels",
                                      "nm_sptrsv_plan_destroy"}
     assert set(_declared()) == table
-    assert L.nm_version() == 1000
+    assert L.nm_version() == 1001
     assert L.nm_last_error() == b""
 
 
