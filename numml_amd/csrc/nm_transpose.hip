@@ -303,124 +303,122 @@ __global__ void symmetry_init_kernel(int32_t *flags, int square) {
     }
 }
 
-// t_pack and c_off16 of the plan; clears flags[1] / flags[2] when a difference does not fit 16 bits.
+// Staging list of one block of rows (keys = columns of its entries) or of columns (keys = rows of
+// its entries), entries [pb, pe) of `key`; line0 = the block's first row / column.  The segments of
+// kStageSeg consecutive keys that the block names are marked in a bitmap over the segments within
+// 32768 keys of line0 (what a 16-bit offset reaches; a block that names a key further away gets no
+// list).  When at most MOST segments are marked, all of them whole (a segment cut off by the end
+// of the vector the kernels will load it from would be read past that end), they are written to
+// desc in ascending order (kStageDesc ints, unused places -1) and true is returned:
+// stage_place(key) then gives kStageSeg * (rank of the key's segment) + offset inside the segment.
+// Otherwise desc[0] = -2.  Called by a whole workgroup.
+struct StageTable {
+    static constexpr int kReach = 32768 / nm::kStageSeg;        // segments either side of line0's
+    static constexpr int kWords = (2 * kReach + 8 + 31) / 32;   // (+ the block's own segments)
+    uint32_t bits[kWords];
+    int32_t before[kWords];     // marked segments in the words before this one
+    int32_t seg0, count, bad;
+};
+
+template <int MOST>
+__device__ __forceinline__ bool stage_block(StageTable &t, int64_t line0, int32_t pb, int32_t pe, int most_entries,
+                                            int64_t veclen, const int32_t *__restrict__ key,
+                                            int32_t *__restrict__ desc) {
+    if (threadIdx.x < StageTable::kWords) t.bits[threadIdx.x] = 0;
+    const int32_t seg0 = (int32_t)(line0 / nm::kStageSeg) - StageTable::kReach;
+    if (threadIdx.x == 0) {
+        t.seg0 = seg0;
+        t.bad = (pe - pb > most_entries || pe == pb) ? 1 : 0;
+    }
+    __syncthreads();
+    if (t.bad == 0) {
+        bool bad = false;
+        for (int32_t p = pb + (int32_t)threadIdx.x; p < pe; p += kBlock) {
+            const int32_t seg = key[p] / nm::kStageSeg, rel = seg - seg0;
+            if (rel < 0 || rel >= StageTable::kWords * 32 || (int64_t)(seg + 1) * nm::kStageSeg > veclen) bad = true;
+            else atomicOr(&t.bits[rel >> 5], 1u << (rel & 31));
+        }
+        if (bad) t.bad = 1;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int n = 0;
+        for (int w = 0; w < StageTable::kWords; ++w) {
+            t.before[w] = n;
+            n += __builtin_popcount(t.bits[w]);
+        }
+        t.count = n;
+    }
+    __syncthreads();
+    const bool staged = t.bad == 0 && t.count <= MOST;
+    if (threadIdx.x < nm::kStageDesc) desc[threadIdx.x] = staged ? -1 : -2;
+    __syncthreads();
+    if (staged && threadIdx.x < StageTable::kWords) {
+        // the marked segments of this word, to their ranks' places of the list
+        uint32_t word = t.bits[threadIdx.x];
+        for (int r = t.before[threadIdx.x]; word; word &= word - 1, ++r)
+            desc[r] = seg0 + (int32_t)threadIdx.x * 32 + __builtin_ctz(word);
+    }
+    return staged;
+}
+
+__device__ __forceinline__ int32_t stage_place(const StageTable &t, int32_t k) {
+    const int32_t rel = k / nm::kStageSeg - t.seg0;
+    const int rank = t.before[rel >> 5] + __builtin_popcount(t.bits[rel >> 5] & ((1u << (rel & 31)) - 1u));
+    return rank * nm::kStageSeg + k % nm::kStageSeg;
+}
+
+// t_pack, c_off16 and the staging lists of the plan; clears flags[1] / flags[2] when a difference
+// does not fit 16 bits and counts the blocks that got a list in flags[4] (rows) / flags[5] (columns).
 // A workgroup takes blocks of kPackCols columns, then blocks of kPackRows rows, lane = entry.
 __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
     int64_t rows, int64_t cols, const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_row,
     const int32_t *__restrict__ t_perm, const int32_t *__restrict__ c_ptr32, const int32_t *__restrict__ c_idx32,
-    int32_t *__restrict__ t_pack, int16_t *__restrict__ c_off16, int32_t *flags) {
+    int32_t *__restrict__ t_pack, int16_t *__restrict__ c_off16, int32_t *__restrict__ f_desc,
+    int32_t *__restrict__ b_desc, int32_t *flags) {
+    __shared__ StageTable table;
     bool fits_t = true, fits_c = true;
     const int64_t cblocks = (cols + nm::kPackCols - 1) / nm::kPackCols;
     for (int64_t b = blockIdx.x; b < cblocks; b += gridDim.x) {
         const int64_t c0 = b * nm::kPackCols;
         const int64_t c1 = c0 + nm::kPackCols < cols ? c0 + nm::kPackCols : cols;
-        const int32_t pe = t_indptr[c1];
-        for (int32_t p = t_indptr[c0] + (int32_t)threadIdx.x; p < pe; p += kBlock) {
-            const int64_t dr = (int64_t)t_row[p] - c0, dk = (int64_t)t_perm[p] - p;
-            fits_t &= dr >= -32768 && dr <= 32767 && dk >= -32768 && dk <= 32767;
-            t_pack[p] = (int32_t)(((uint32_t)dr & 0xffffu) | ((uint32_t)dk << 16));
+        const int32_t pb = t_indptr[c0], pe = t_indptr[c1];
+        // (a list made here is only read when every packed word of the plan turns out valid)
+        const bool staged = stage_block<nm::kStageBwd>(table, c0, pb, pe, nm::kStageBwdCap, rows, t_row,
+                                                       b_desc + b * nm::kStageDesc);
+        if (staged && threadIdx.x == 0) atomicAdd(&flags[5], 1);
+        for (int32_t p0 = pb; p0 < pe; p0 += kBlock) {
+            const int32_t p = p0 + (int32_t)threadIdx.x;
+            const bool active = p < pe;
+            const int32_t r = active ? t_row[p] : 0;
+            const int64_t dr = (int64_t)r - c0, dk = active ? (int64_t)t_perm[p] - p : 0;
+            fits_t &= !active || (dr >= -32768 && dr <= 32767 && dk >= -32768 && dk <= 32767);
+            const uint32_t low = staged && active ? (uint32_t)stage_place(table, r) : ((uint32_t)dr & 0xffffu);
+            if (active) t_pack[p] = (int32_t)(low | ((uint32_t)dk << 16));
         }
+        __syncthreads();
     }
     const int64_t rblocks = (rows + nm::kPackRows - 1) / nm::kPackRows;
     for (int64_t b = blockIdx.x; b < rblocks; b += gridDim.x) {
         const int64_t r0 = b * nm::kPackRows;
         const int64_t r1 = r0 + nm::kPackRows < rows ? r0 + nm::kPackRows : rows;
-        const int32_t ke = c_ptr32[r1];
-        for (int32_t k = c_ptr32[r0] + (int32_t)threadIdx.x; k < ke; k += kBlock) {
-            const int64_t dc = (int64_t)c_idx32[k] - r0;
-            fits_c &= dc >= -32768 && dc <= 32767;
-            c_off16[k] = (int16_t)dc;
+        const int32_t kb = c_ptr32[r0], ke = c_ptr32[r1];
+        const bool staged = stage_block<nm::kStageFwd>(table, r0, kb, ke, nm::kStageFwdCap, cols, c_idx32,
+                                                       f_desc + b * nm::kStageDesc);
+        if (staged && threadIdx.x == 0) atomicAdd(&flags[4], 1);
+        for (int32_t k0 = kb; k0 < ke; k0 += kBlock) {
+            const int32_t k = k0 + (int32_t)threadIdx.x;
+            const bool active = k < ke;
+            const int32_t c = active ? c_idx32[k] : 0;
+            const int64_t dc = (int64_t)c - r0;
+            fits_c &= !active || (dc >= -32768 && dc <= 32767);
+            const int32_t v = staged && active ? stage_place(table, c) : (int32_t)dc;
+            if (active) c_off16[k] = (int16_t)v;
         }
+        __syncthreads();
     }
     if (!fits_t) flags[1] = 0;
     if (!fits_c) flags[2] = 0;
-}
-
-// Staging lists (f_desc / b_desc of the plan).  A workgroup takes one block of kPackRows rows
-// (FWD) or of kPackCols columns; `key` of an entry is its column (FWD: c_idx32) or its row
-// (t_row).  The segments the block's keys fall into are collected in a small LDS hash set; when
-// there are at most MOST of them, all of them whole (a segment cut off by the end of the vector
-// the kernels will load it from would be read past that end), they are ranked and every entry
-// gets 128 * rank + offset inside the segment: written over c_off16[k] (FWD) or over the low half
-// of t_pack[p].  Runs after tp_pack_kernel.
-template <bool FWD, int MOST>
-__global__ __launch_bounds__(kBlock) void tp_stage_kernel(
-    int64_t nblocks, int64_t nlines, int64_t veclen, const int32_t *__restrict__ ptr, const int32_t *__restrict__ key,
-    int32_t *__restrict__ t_pack, int16_t *__restrict__ c_off16, int32_t *__restrict__ desc,
-    int32_t *__restrict__ flags) {
-    constexpr int kSlots = 64, kBlockLines = FWD ? nm::kPackRows : nm::kPackCols;
-    constexpr int kMostEntries = FWD ? nm::kStageFwdCap : nm::kStageBwdCap;
-    __shared__ int32_t s_tab[kSlots], s_rank[kSlots], s_count, s_bad;
-    const bool enabled = FWD || flags[1] != 0;   // the backward only reads t_pack when it is valid
-    for (int64_t b = blockIdx.x; b < nblocks; b += gridDim.x) {
-        const int64_t l0 = b * kBlockLines;
-        const int64_t l1 = l0 + kBlockLines < nlines ? l0 + kBlockLines : nlines;
-        const int32_t pb = ptr[l0], pe = ptr[l1];
-        if (threadIdx.x < kSlots) {
-            s_tab[threadIdx.x] = -1;
-            s_rank[threadIdx.x] = 0;
-        }
-        if (threadIdx.x == 0) {
-            s_count = 0;
-            s_bad = (!enabled || pe - pb > kMostEntries || pe == pb) ? 1 : 0;
-        }
-        __syncthreads();
-        // the slot of a segment in the table; inserts it when `insert`.  -1: table full or given up
-        auto slot_of = [&](int32_t seg, bool insert) -> int {
-            int h = (int)(((uint32_t)seg * 0x9E3779B1u) >> 26);
-            for (int step = 0; step < kSlots; ++step, h = (h + 1) & (kSlots - 1)) {
-                int32_t seen = s_tab[h];
-                if (seen == -1 && insert) {
-                    seen = atomicCAS(&s_tab[h], -1, seg);
-                    if (seen == -1) {
-                        atomicAdd(&s_count, 1);
-                        return h;
-                    }
-                }
-                if (seen == seg) return h;
-                if (seen == -1) return -1;
-            }
-            return -1;
-        };
-        if (s_bad == 0) {
-            for (int32_t p = pb + (int32_t)threadIdx.x; p < pe; p += kBlock) {
-                const int32_t seg = key[p] / nm::kStageSeg;
-                if ((int64_t)(seg + 1) * nm::kStageSeg > veclen || slot_of(seg, true) < 0) s_bad = 1;
-                if (s_count > MOST) break;
-            }
-        }
-        __syncthreads();
-        const bool staged = s_bad == 0 && s_count <= MOST;
-        if (staged && threadIdx.x == 0) atomicAdd(&flags[FWD ? 4 : 5], 1);    // (nm_csr_transpose_plan_info)
-        if (staged && threadIdx.x < kSlots) {
-            const int32_t mine = s_tab[threadIdx.x];
-            if (mine >= 0) {
-                int r = 0;
-                for (int j = 0; j < kSlots; ++j) {
-                    const int32_t other = s_tab[j];
-                    r += other >= 0 && other < mine;
-                }
-                s_rank[threadIdx.x] = r;
-                desc[b * nm::kStageDesc + r] = mine;
-            }
-        }
-        if (threadIdx.x < nm::kStageDesc) {
-            // places the ranked segments do not fill (written above by other lanes: different places)
-            if (!staged) desc[b * nm::kStageDesc + threadIdx.x] = -2;
-            else if ((int)threadIdx.x >= s_count) desc[b * nm::kStageDesc + threadIdx.x] = -1;
-        }
-        __syncthreads();
-        if (staged) {
-            for (int32_t p = pb + (int32_t)threadIdx.x; p < pe; p += kBlock) {
-                const int32_t k = key[p];
-                const int h = slot_of(k / nm::kStageSeg, false);
-                const int32_t where = s_rank[h < 0 ? 0 : h] * nm::kStageSeg + k % nm::kStageSeg;
-                if (FWD) c_off16[p] = (int16_t)where;
-                else t_pack[p] = (int32_t)(((uint32_t)t_pack[p] & 0xffff0000u) | (uint32_t)where);
-            }
-        }
-        __syncthreads();
-    }
 }
 
 // Clears flags[0] unless A^T has exactly A's structure.
@@ -507,17 +505,9 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
         int64_t grid = ceil_div(cols > rows ? cols : rows, (int64_t)kPackCols);
         if (grid > 65536) grid = 65536;
         hipLaunchKernelGGL(tp_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, cols, plan.t_indptr,
-                           plan.t_row, plan.t_perm, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.flags);
+                           plan.t_row, plan.t_perm, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.f_desc,
+                           plan.b_desc, plan.flags);
         NM_LAUNCH_CHECK("tp_pack_kernel");
-        const int64_t rblocks = ceil_div(rows, (int64_t)kPackRows), cblocks = ceil_div(cols, (int64_t)kPackCols);
-        grid = rblocks > 65536 ? 65536 : rblocks;
-        hipLaunchKernelGGL((tp_stage_kernel<true, kStageFwd>), dim3((unsigned)grid), dim3(kBlock), 0, s, rblocks, rows,
-                           cols, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.f_desc, plan.flags);
-        NM_LAUNCH_CHECK("tp_stage_kernel<rows>");
-        grid = cblocks > 65536 ? 65536 : cblocks;
-        hipLaunchKernelGGL((tp_stage_kernel<false, kStageBwd>), dim3((unsigned)grid), dim3(kBlock), 0, s, cblocks, cols,
-                           rows, plan.t_indptr, plan.t_row, plan.t_pack, plan.c_off16, plan.b_desc, plan.flags);
-        NM_LAUNCH_CHECK("tp_stage_kernel<columns>");
     }
     return NM_OK;
 }
