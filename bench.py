@@ -258,7 +258,7 @@ class SpMV(Workload):
         # block, read by the kernels) and 16-bit places in it instead of column offsets.
         self.plan_info = None
         if planned and hasattr(ext, "transpose_plan_info") and self.nnz:
-            sym, pk_b, pk_f, st_r, n_r, st_c, n_c = ext.transpose_plan_info(rows, cols, self.I, self.P)
+            sym, pk_b, pk_f, st_r, n_r, st_c, n_c = ext.transpose_plan_info(rows, cols, self.I, self.P)[:7]
             self.plan_info = {"symmetric": bool(sym), "packed_backward": bool(pk_b), "packed_forward": bool(pk_f),
                               "row_blocks_with_staging_list": st_r, "row_blocks": n_r,
                               "column_blocks_with_staging_list": st_c, "column_blocks": n_c}

@@ -86,6 +86,14 @@ int nm_structure_hash(int64_t nnz, int64_t nptr, const int64_t *indices, const i
                       void *work, size_t work_bytes, void *host_landing, uint64_t *key,
                       nm_stream stream);
 
+/* Entries of the longest row of a pattern (one pass over indptr), delivered to the
+ * host like the key above: `work` holds 8 bytes of device scratch, `host_landing`
+ * as for nm_structure_hash (or NULL).  Waits for the result.  No counterpart in
+ * the reference; callers that choose between kernels by how the work is spread
+ * ask for it once per pattern. */
+int nm_csr_longest_row(int64_t rows, const int64_t *indptr, void *work, size_t work_bytes,
+                       void *host_landing, int64_t *longest, nm_stream stream);
+
 /* ---------------------------------------------- transposed-structure plan
  * The pattern of A^T as 32-bit arrays (column pointers, row of each entry and
  * its position in A's arrays, rows ascending inside a column) together with
@@ -109,8 +117,12 @@ int nm_csr_transpose_plan_build(int64_t rows, int64_t cols, int64_t nnz,
  * 16-bit column offsets of the forward are valid, info[4] blocks of 512 rows
  * with a staging list (the SpMV forward loads the segments of x such a block
  * names into LDS), info[5] blocks of 256 columns with one (the same for the
- * backward); the other entries are 0.  Waits for `stream`.  Diagnostics: no
- * counterpart in the reference. */
+ * backward), info[6] / info[7] entries of the longest column / row, info[8] the
+ * most entries that columns of more than 512 entries hold inside one aligned
+ * group of 64 columns (such a group is one workgroup's in the SpMM kernels);
+ * the other entries are 0.  Waits for `stream`.  No counterpart in the
+ * reference; a caller's choice between the kernels on a plan and the stateless
+ * ones can be based on it. */
 int nm_csr_transpose_plan_info(int64_t rows, int64_t cols, int64_t nnz, const void *plan_mem,
                                int32_t info[16], nm_stream stream);
 

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "nm_csr_transpose_plan_bytes": [_c_i64, _c_i64, _c_i64, ctypes.POINTER(_c_size), ctypes.POINTER(_c_size)],
     "nm_csr_transpose_plan_build": [_c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr, _c_size,
                                     _c_ptr],
+    "nm_csr_longest_row": [_c_i64, _c_ptr, _c_ptr, _c_size, _c_ptr, ctypes.POINTER(_c_i64), _c_ptr],
     "nm_csr_transpose_plan_info": [_c_i64, _c_i64, _c_i64, _c_ptr, ctypes.POINTER(ctypes.c_int32), _c_ptr],
     "nm_stream_probe": [_c_ptr, _c_size, _c_ptr, _c_size, _c_ptr],
     "nm_spgemv_forward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],

@@ -149,3 +149,64 @@ extern "C" int nm_structure_hash(int64_t nnz, int64_t nptr, const int64_t *indic
     NM_HIP_TRY(hipStreamSynchronize(s));
     return NM_OK;
 }
+
+namespace {
+
+__global__ __launch_bounds__(kBlock) void longest_row_kernel(int64_t rows, const int64_t *__restrict__ indptr,
+                                                             unsigned long long *__restrict__ out) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    long long len = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < rows; i += stride) {
+        const long long d = indptr[i + 1] - indptr[i];
+        len = d > len ? d : len;
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const long long o = __shfl_xor(len, off, kWave);
+        len = o > len ? o : len;
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0 && len > 0) atomicMax(out, (unsigned long long)len);
+}
+
+__global__ void land_word_kernel(const unsigned long long *__restrict__ word, volatile uint64_t *host_landing,
+                                 uint64_t ticket) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        host_landing[0] = *word;
+        __threadfence_system();
+        host_landing[2] = ticket;
+    }
+}
+
+}  // namespace
+
+extern "C" int nm_csr_longest_row(int64_t rows, const int64_t *indptr, void *work, size_t work_bytes,
+                                  void *host_landing, int64_t *longest, nm_stream stream) {
+    NM_REQUIRE(rows >= 0 && longest != nullptr && work != nullptr && work_bytes >= 8, "bad arguments");
+    NM_REQUIRE(rows == 0 || indptr != nullptr, "indptr is null");
+    hipStream_t s = nm::as_stream(stream);
+    unsigned long long *out = (unsigned long long *)work;
+    if (int rc = nm::fill_async(out, (int64_t)1, 0ull, s)) return rc;
+    if (rows > 0) {
+        hipLaunchKernelGGL(longest_row_kernel, dim3(blocks_for(rows)), dim3(kBlock), 0, s, rows, indptr, out);
+        NM_LAUNCH_CHECK("longest_row_kernel");
+    }
+    volatile uint64_t *land = (volatile uint64_t *)host_landing;
+    if (land) {
+        const uint64_t ticket = land[2] + 1;
+        hipLaunchKernelGGL(land_word_kernel, dim3(1), dim3(64), 0, s, out, land, ticket);
+        NM_LAUNCH_CHECK("land_word_kernel");
+        bool arrived = false;
+        for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = land[2] == ticket;
+        if (!arrived) {
+            NM_HIP_TRY(hipStreamSynchronize(s));
+            NM_REQUIRE(land[2] == ticket, "the result did not arrive");
+        }
+        *longest = (int64_t)land[0];
+        return NM_OK;
+    }
+    unsigned long long host = 0;
+    NM_HIP_TRY(hipMemcpyAsync(&host, out, sizeof(host), hipMemcpyDeviceToHost, s));
+    NM_HIP_TRY(hipStreamSynchronize(s));
+    *longest = (int64_t)host;
+    return NM_OK;
+}

@@ -383,6 +383,24 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
         const int64_t c0 = b * nm::kPackCols;
         const int64_t c1 = c0 + nm::kPackCols < cols ? c0 + nm::kPackCols : cols;
         const int32_t pb = t_indptr[c0], pe = t_indptr[c1];
+        {
+            // statistics the caller's policy reads (nm_csr_transpose_plan_info): the longest column,
+            // and the most entries that columns of more than 512 entries hold inside one group of 64
+            // columns -- the SpMM kernels give such a group to one workgroup, which takes those
+            // columns one after the other
+            const int64_t c = c0 + threadIdx.x;
+            int len = c < c1 ? t_indptr[c + 1] - t_indptr[c] : 0;
+            int heavy = len > 512 ? len : 0;
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) {
+                len = max(len, __shfl_xor(len, off, kWave));
+                heavy += __shfl_xor(heavy, off, kWave);
+            }
+            if ((threadIdx.x & (kWave - 1)) == 0) {
+                atomicMax(&flags[6], len);
+                if (heavy) atomicMax(&flags[8], heavy);
+            }
+        }
         // (a list made here is only read when every packed word of the plan turns out valid)
         const bool staged = stage_block<nm::kStageBwd>(table, c0, pb, pe, nm::kStageBwdCap, rows, t_row,
                                                        b_desc + b * nm::kStageDesc);
@@ -403,6 +421,13 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
         const int64_t r0 = b * nm::kPackRows;
         const int64_t r1 = r0 + nm::kPackRows < rows ? r0 + nm::kPackRows : rows;
         const int32_t kb = c_ptr32[r0], ke = c_ptr32[r1];
+        {
+            int len = 0;    // the longest row
+            for (int64_t r = r0 + threadIdx.x; r < r1; r += kBlock) len = max(len, c_ptr32[r + 1] - c_ptr32[r]);
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) len = max(len, __shfl_xor(len, off, kWave));
+            if ((threadIdx.x & (kWave - 1)) == 0) atomicMax(&flags[7], len);
+        }
         const bool staged = stage_block<nm::kStageFwd>(table, r0, kb, ke, nm::kStageFwdCap, cols, c_idx32,
                                                        f_desc + b * nm::kStageDesc);
         if (staged && threadIdx.x == 0) atomicAdd(&flags[4], 1);

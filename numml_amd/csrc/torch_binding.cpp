@@ -22,7 +22,9 @@
 #include <c10/hip/HIPGuard.h>
 #include <c10/hip/HIPStream.h>
 
+#include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <cstdlib>
 #include <list>
 #include <memory>
@@ -182,6 +184,7 @@ struct Alias {
     const void *idx_ptr, *ptr_ptr;
     uint32_t idx_version, ptr_version;
     Key key;
+    int64_t longest_row = -1;    // entries of the pattern's longest row, once somebody has asked
 };
 
 struct Plan {
@@ -199,6 +202,10 @@ struct Plan {
     int plan_class = 1;                      // 'P': which forward kernel the product takes (nm_spgemm_plan_build)
     std::shared_ptr<Plan> parent;            // 'P': the transposed-structure plan of A it walks
     nm_sptrsv_plan *handle = nullptr;
+    // 'T': what the build found out about the pattern (nm_csr_transpose_plan_info), read back
+    // the first time a policy asks for it
+    int32_t info[16] = {0};
+    std::atomic<bool> info_loaded{false};
     // the stream the plan was built on and the event that marks its completion there
     c10::StreamId build_stream = 0;
     std::unique_ptr<at::cuda::CUDAEvent> ready;
@@ -299,6 +306,28 @@ bool structure_key(const Tensor &indices, const Tensor &indptr, bool compute, Ke
     g_aliases.push_front(std::move(al));
     while (g_aliases.size() > kAliasTableSize) g_aliases.pop_back();
     return true;
+}
+
+// Entries of the longest row of a pattern: remembered with the pair of tensors' entry in the alias
+// table (a pair that has none is measured every time).
+int64_t longest_row(const Tensor &indices, const Tensor &indptr, int64_t rows, const c10::Device &dev) {
+    const bool aliased = tracked(indices) && tracked(indptr);
+    if (aliased) {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        for (const Alias &al : g_aliases)
+            if (alias_matches(al, indices, indptr) && al.longest_row >= 0) return al.longest_row;
+    }
+    Tensor work = scratch(8, dev);
+    int64_t longest = 0;
+    check(nm_csr_longest_row(rows, indptr.data_ptr<int64_t>(), work.data_ptr(), 8, host_landing(), &longest,
+                             current_stream(dev)),
+          "nm_csr_longest_row");
+    if (aliased) {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        for (Alias &al : g_aliases)
+            if (alias_matches(al, indices, indptr)) al.longest_row = longest;
+    }
+    return longest;
 }
 
 // Makes `plan` usable on the current stream: work enqueued there from now on runs after the
@@ -408,6 +437,23 @@ std::shared_ptr<Plan> transpose_plan(const Tensor &indices, const Tensor &indptr
               "nm_csr_transpose_plan_build");
     });
 }
+
+// Statistics of a transposed-structure plan's pattern (one wait for the stream per plan).
+const int32_t *plan_info(Plan &plan, int64_t rows, int64_t cols, int64_t nnz, const c10::Device &dev) {
+    if (!plan.info_loaded.load(std::memory_order_acquire)) {
+        int32_t info[16];
+        check(nm_csr_transpose_plan_info(rows, cols, nnz, plan.mem.data_ptr(), info, current_stream(dev)),
+              "nm_csr_transpose_plan_info");
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        std::copy(info, info + 16, plan.info);
+        plan.info_loaded.store(true, std::memory_order_release);
+    }
+    return plan.info;
+}
+
+// Which kernels the last backward pass of each kind ran (diagnostics and tests of the policy).
+std::atomic<int> g_last_spdmm_backward{-1}, g_last_spgemm_backward{-1};
+enum Path : int { kStateless = 0, kOnTransposedPlan = 1, kOnProductPlan = 2 };
 
 // A transposed-structure plan keeps rows, columns and positions in 32 bits
 // (nm_csr_transpose_plan_bytes refuses more); larger matrices run the stateless kernels, which
@@ -1020,7 +1066,19 @@ std::vector<Tensor> spdmm_backward(int A_rows, int A_cols, Tensor A_data, Tensor
     if (want.first) grad_A = torch::empty_like(A_data);
     if (want.second) grad_B = torch::empty({B.size(0), n}, B.options());
     // (the dot products alone walk A by row and need no plan)
-    if (auto plan = want.second ? backward_plan(A_indices, A_indptr, A_rows, B.size(0), dev) : nullptr) {
+    auto plan = want.second ? backward_plan(A_indices, A_indptr, A_rows, B.size(0), dev) : nullptr;
+    if (plan && backward_mode_now() == kPlanned) {
+        // The kernels on the plan give every aligned group of 64 columns to one workgroup, which
+        // takes the group's columns of more than 512 entries one after the other (~0.12 us an entry
+        // with both gradients, ~0.02 us for the transposed product alone), while the stateless
+        // kernels spread every entry over the chip at ~0.2 ns: where one group holds more than a
+        // thousandth (a hundredth) of the matrix in such columns, the stateless kernels are the
+        // faster ones.  ("eager" asks for the deterministic sums whatever they cost.)
+        const int64_t heavy = plan_info(*plan, A_rows, B.size(0), A_data.numel(), dev)[8];
+        if (heavy * (want.first ? 1000 : 100) > A_data.numel()) plan = nullptr;
+    }
+    g_last_spdmm_backward.store(plan ? kOnTransposedPlan : kStateless, std::memory_order_relaxed);
+    if (plan) {
         check(nm_spdmm_backward_planned(dtype_of(A_data), A_rows, B.size(0), A_data.numel(), A_data.data_ptr(),
                                         A_indices.data_ptr<int64_t>(), A_indptr.data_ptr<int64_t>(),
                                         plan->mem.data_ptr(), B.data_ptr(), ldb, grad_C.data_ptr(), ldg, n,
@@ -1159,6 +1217,7 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
         auto pp = peek_product_plan(A_indices, A_indptr, B_indices, B_indptr, A_rows, B_cols, dev);
         if (pp && pp->usable && pp->derived[0].data_ptr() == C_indices.data_ptr() &&
             pp->derived[1].data_ptr() == C_indptr.data_ptr() && pp->derived[0].numel() == C_indices.numel()) {
+            g_last_spgemm_backward.store(kOnProductPlan, std::memory_order_relaxed);
             check(nm_spgemm_backward_mapped_wide(dtype_of(A_data), pp->plan_class, A_rows, A_cols, A_data.numel(),
                                                  B_data.numel(), grad_C.numel(), grad_C.data_ptr(),
                                                  A_data.data_ptr(), pp->parent->mem.data_ptr(), B_data.data_ptr(),
@@ -1182,7 +1241,18 @@ std::vector<Tensor> spgemm_backward(Tensor grad_C, Tensor C_indices, Tensor C_in
     const double mean_col = A_cols > 0 ? (double)A_data.numel() / A_cols : 0.;
     const bool on_plan = mode == kEager ||
                          (mode == kPlanned && mean_c <= 4. * std::max(mean_b, 1.) && mean_b * mean_col <= 4096.);
-    if (auto plan = on_plan ? backward_plan(A_indices, A_indptr, A_rows, A_cols, dev) : nullptr) {
+    auto plan = on_plan ? backward_plan(A_indices, A_indptr, A_rows, A_cols, dev) : nullptr;
+    if (plan && mode == kPlanned) {
+        // Means hide a few heavy rows among many light ones: the longest column of A (from the plan)
+        // times the longest row of B (measured once per pair of B's structure tensors) bounds the
+        // products the busiest workgroup makes.
+        const int64_t longest_col = plan_info(*plan, A_rows, A_cols, A_data.numel(), dev)[6];
+        Key kb;
+        structure_key(B_indices, B_indptr, true, &kb);      // (an alias entry to remember the length with)
+        if (longest_col * longest_row(B_indices, B_indptr, B_rows, dev) > 65536) plan = nullptr;
+    }
+    g_last_spgemm_backward.store(plan ? kOnTransposedPlan : kStateless, std::memory_order_relaxed);
+    if (plan) {
         check(nm_spgemm_backward_planned(dtype_of(A_data), A_rows, A_cols, A_data.numel(), B_data.numel(),
                                          grad_C.numel(), grad_C.data_ptr(), C_indices.data_ptr<int64_t>(),
                                          C_indptr.data_ptr<int64_t>(), A_data.data_ptr(), plan->mem.data_ptr(),
@@ -1409,8 +1479,8 @@ std::tuple<int64_t, int64_t> sptrsv_chain_levels(int A_rows, Tensor A_indices, T
 
 // What the transposed-structure plan of a pattern (the cached one, or one built now) found out:
 // (symmetric, packed words of the backward valid, 16-bit column offsets of the forward valid,
-// row blocks with a staging list, row blocks, column blocks with one, column blocks).
-// Diagnostics; waits for the stream.
+// row blocks with a staging list, row blocks, column blocks with one, column blocks, longest column,
+// longest row, most entries of long columns in one group of 64 columns).  Diagnostics; waits for the stream.
 std::vector<int64_t> transpose_plan_info(int A_rows, int A_cols, Tensor A_indices, Tensor A_indptr) {
     TORCH_CHECK(A_indptr.dim() == 1 && A_indptr.numel() == (int64_t)A_rows + 1 && A_indices.dim() == 1,
                 "transpose_plan_info: expected ", A_rows + 1, " row pointers, got shape ", A_indptr.sizes());
@@ -1423,7 +1493,8 @@ std::vector<int64_t> transpose_plan_info(int A_rows, int A_cols, Tensor A_indice
     check(nm_csr_transpose_plan_info(A_rows, A_cols, A_indices.numel(), plan->mem.data_ptr(), info,
                                      current_stream(dev)),
           "nm_csr_transpose_plan_info");
-    return {info[0], info[1], info[2], info[4], ((int64_t)A_rows + 511) / 512, info[5], ((int64_t)A_cols + 255) / 256};
+    return {info[0], info[1], info[2], info[4], ((int64_t)A_rows + 511) / 512, info[5], ((int64_t)A_cols + 255) / 256,
+            info[6], info[7], info[8]};
 }
 
 // Time-free helper of the bandwidth calibration: enqueues one nm_stream_probe launch.
@@ -1435,6 +1506,17 @@ void stream_probe(Tensor src, int64_t read_bytes, Tensor dst, int64_t write_byte
     c10::hip::HIPGuard guard(dev.index());
     check(nm_stream_probe(src.data_ptr(), (size_t)read_bytes, dst.data_ptr(), (size_t)write_bytes, current_stream(dev)),
           "nm_stream_probe");
+}
+
+// ("stateless" | "transposed plan" | "product plan" | "none yet") for the last spdmm_backward and
+// the last spgemm_backward of this process.
+std::tuple<std::string, std::string> last_backward_paths() {
+    auto name = [](int p) -> std::string {
+        return p == kStateless ? "stateless" : p == kOnTransposedPlan ? "transposed plan"
+               : p == kOnProductPlan ? "product plan" : "none yet";
+    };
+    return {name(g_last_spdmm_backward.load(std::memory_order_relaxed)),
+            name(g_last_spgemm_backward.load(std::memory_order_relaxed))};
 }
 
 void clear_plan_cache() {
@@ -1511,6 +1593,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           "(symmetric, packed backward, packed forward, staged row blocks, row blocks, staged column blocks, "
           "column blocks) of a pattern's transposed-structure plan");
     m.def("stream_probe", &stream_probe, "one launch of the streaming calibration kernel (read_bytes in, write_bytes out)");
+    m.def("last_backward_paths", &last_backward_paths,
+          "which kernels the last spdmm_backward and the last spgemm_backward ran");
     m.def("clear_plan_cache", &clear_plan_cache, "Drop every cached structure plan");
     m.def("plan_cache_size", &plan_cache_size, "Number of cached structure plans");
     m.def("plan_cache_bytes", &plan_cache_bytes, "Device memory held by the cached structure plans");

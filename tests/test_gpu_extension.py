@@ -357,6 +357,83 @@ def test_default_mode_keeps_heavy_rows_of_the_right_operand_off_the_planned_back
         cpp.clear_plan_cache()
 
 
+def test_default_mode_judges_by_the_heaviest_rows_and_columns_not_by_means(dev, cpp):
+    """Means hide a few heavy rows or columns among many light ones.  (a) SpGEMM backward: two rows
+    of B with 512 entries, named by two columns of A with 2000 entries, in matrices that are
+    diagonal otherwise: every mean is about one, yet the plan-based kernel would hand each heavy
+    row (a million products) to a single workgroup.  (b) SpMM backward: a matrix with one dense
+    column; the kernels on the plan take a column of more than 512 entries serially.  The default
+    mode takes the stateless kernels for both however often it sees the pattern; "eager" takes the
+    plans; both match the oracle."""
+    import scipy.sparse as sps
+    dtype = np.float64
+    rng = np.random.default_rng(90)
+    n = 1_000_000
+
+    def csr(m):
+        m = m.tocsr()
+        m.sum_duplicates()
+        m.sort_indices()
+        return m.data.astype(dtype), m.indices.astype(np.int64), m.indptr.astype(np.int64)
+
+    # ---- (a)
+    heavy = (1000, 300_000)
+    ar = np.concatenate([np.arange(n)] + [rng.choice(n, 2000, replace=False) for _ in heavy])
+    ac = np.concatenate([np.arange(n)] + [np.full(2000, k) for k in heavy])
+    A = csr(sps.coo_matrix((rng.standard_normal(ar.size), (ar, ac)), shape=(n, n)))
+    br = np.concatenate([np.arange(n)] + [np.full(512, k) for k in heavy])
+    bc = np.concatenate([np.arange(n)] + [rng.choice(n, 512, replace=False) for _ in heavy])
+    B = csr(sps.coo_matrix((rng.standard_normal(br.size), (br, bc)), shape=(n, n)))
+    cd, ci, cp = oracle.spgemm_forward(n, n, *A, n, n, *B)
+    assert cd.shape[0] / n <= 4 * B[0].shape[0] / n          # the means would let the plan through
+    g = randn(91, cd.shape[0], dtype)
+    rA, rB = oracle.spgemm_backward(g, ci, cp, n, n, *A, n, n, *B)
+    dA, dB = to_dev(dev, *A), to_dev(dev, *B)
+    Gd, CI, CP = to_dev(dev, g, ci, cp)
+    cpp.clear_plan_cache()
+    try:
+        cpp.set_backward_mode("planned")
+        for _ in range(3):
+            gA, gB = cpp.spgemm_backward(Gd, CI, CP, n, n, *dA, n, n, *dB)
+            assert cpp.last_backward_paths()[1] == "stateless"
+            assert_same(host(gA), rA, "grad_A")
+            assert_close(host(gB), rB, "grad_B (atomics)")
+        cpp.set_backward_mode("eager")
+        gA, gB = cpp.spgemm_backward(Gd, CI, CP, n, n, *dA, n, n, *dB)
+        assert cpp.last_backward_paths()[1] == "transposed plan"
+        assert_same(host(gA), rA, "grad_A on the plan")
+        assert_close(host(gB), rB, "grad_B on the plan")
+        # ---- (b)
+        n = 60_000
+        mr = np.concatenate([np.arange(n), np.arange(1, 30_001)])
+        mc = np.concatenate([np.arange(n), np.zeros(30_000, dtype=np.int64)])
+        M = csr(sps.coo_matrix((rng.standard_normal(mr.size), (mr, mc)), shape=(n, n)))
+        band = csr(sps.diags([rng.standard_normal(n - 1), rng.standard_normal(n), rng.standard_normal(n - 1)], [-1, 0, 1]))
+        Bd, Gc = randn(92, (n, 40), dtype), randn(93, (n, 40), dtype)
+        dM, dBand = to_dev(dev, *M), to_dev(dev, *band)
+        dBd, dGc = to_dev(dev, Bd, Gc)
+        for mat, dmat, want in ((M, dM, "stateless"), (band, dBand, "transposed plan")):
+            ref = oracle.spdmm_backward(n, n, *mat, Bd, Gc)
+            cpp.set_backward_mode("planned")
+            cpp.clear_plan_cache()
+            for call in range(3):
+                gA, gB = cpp.spdmm_backward(n, n, *dmat, dBd, dGc)
+                if call:                                    # (the first sighting is stateless for every pattern)
+                    assert cpp.last_backward_paths()[0] == want
+                assert_close(host(gA), ref[0], "spdmm grad_A")
+                assert_close(host(gB), ref[1], "spdmm grad_B")
+            cpp.set_backward_mode("eager")
+            gA, gB = cpp.spdmm_backward(n, n, *dmat, dBd, dGc)
+            assert cpp.last_backward_paths()[0] == "transposed plan"
+            assert_close(host(gA), ref[0], "spdmm grad_A on the plan")
+            assert_close(host(gB), ref[1], "spdmm grad_B on the plan")
+        info = cpp.transpose_plan_info(n, n, dM[1], dM[2])
+        assert info[7] == 30_001 and info[9] == 30_001       # longest column; entries of long columns in its group
+    finally:
+        cpp.set_backward_mode("planned")
+        cpp.clear_plan_cache()
+
+
 def test_product_plan_for_rows_of_the_right_operand_of_up_to_32_entries(dev, cpp):
     """A (A A) on a 3D grid -- the right operand has 25-entry rows, so the product takes the hash path --
     in a loop with new values: the first call is stateless, the second leaves a product plan with four
