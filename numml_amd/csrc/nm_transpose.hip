@@ -375,7 +375,7 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
     int64_t rows, int64_t cols, const int32_t *__restrict__ t_indptr, const int32_t *__restrict__ t_row,
     const int32_t *__restrict__ t_perm, const int32_t *__restrict__ c_ptr32, const int32_t *__restrict__ c_idx32,
     int32_t *__restrict__ t_pack, int16_t *__restrict__ c_off16, int32_t *__restrict__ f_desc,
-    int32_t *__restrict__ b_desc, int32_t *flags) {
+    int32_t *__restrict__ b_desc, int32_t *__restrict__ stats, int32_t *flags) {
     __shared__ StageTable table;
     bool fits_t = true, fits_c = true;
     const int64_t cblocks = (cols + nm::kPackCols - 1) / nm::kPackCols;
@@ -396,15 +396,16 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
                 len = max(len, __shfl_xor(len, off, kWave));
                 heavy += __shfl_xor(heavy, off, kWave);
             }
+            // (left per wavefront and reduced by tp_stats_kernel: thousands of workgroups raising the
+            // same word with atomics took longer than all the rest of the build)
             if ((threadIdx.x & (kWave - 1)) == 0) {
-                atomicMax(&flags[6], len);
-                if (heavy) atomicMax(&flags[8], heavy);
+                stats[b * 8 + threadIdx.x / kWave] = len;
+                stats[b * 8 + 4 + threadIdx.x / kWave] = heavy;
             }
         }
         // (a list made here is only read when every packed word of the plan turns out valid)
         const bool staged = stage_block<nm::kStageBwd>(table, c0, pb, pe, nm::kStageBwdCap, rows, t_row,
                                                        b_desc + b * nm::kStageDesc);
-        if (staged && threadIdx.x == 0) atomicAdd(&flags[5], 1);
         for (int32_t p0 = pb; p0 < pe; p0 += kBlock) {
             const int32_t p = p0 + (int32_t)threadIdx.x;
             const bool active = p < pe;
@@ -426,11 +427,10 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
             for (int64_t r = r0 + threadIdx.x; r < r1; r += kBlock) len = max(len, c_ptr32[r + 1] - c_ptr32[r]);
 #pragma unroll
             for (int off = kWave / 2; off > 0; off >>= 1) len = max(len, __shfl_xor(len, off, kWave));
-            if ((threadIdx.x & (kWave - 1)) == 0) atomicMax(&flags[7], len);
+            if ((threadIdx.x & (kWave - 1)) == 0) stats[cblocks * 8 + b * 4 + threadIdx.x / kWave] = len;
         }
         const bool staged = stage_block<nm::kStageFwd>(table, r0, kb, ke, nm::kStageFwdCap, cols, c_idx32,
                                                        f_desc + b * nm::kStageDesc);
-        if (staged && threadIdx.x == 0) atomicAdd(&flags[4], 1);
         for (int32_t k0 = kb; k0 < ke; k0 += kBlock) {
             const int32_t k = k0 + (int32_t)threadIdx.x;
             const bool active = k < ke;
@@ -444,6 +444,43 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
     }
     if (!fits_t) flags[1] = 0;
     if (!fits_c) flags[2] = 0;
+}
+
+// flags[4] / flags[5]: blocks of rows / columns with a staging list; flags[6] / flags[7]: the longest
+// column / row; flags[8]: the most entries that columns of more than 512 entries hold inside one
+// aligned group of 64 columns.  From what tp_pack_kernel left per block and per wavefront.
+__global__ __launch_bounds__(kBlock) void tp_stats_kernel(int64_t rblocks, int64_t cblocks,
+                                                          const int32_t *__restrict__ f_desc,
+                                                          const int32_t *__restrict__ b_desc,
+                                                          const int32_t *__restrict__ stats, int32_t *flags) {
+    __shared__ int32_t s_red[5][kBlock / kWave];
+    const int64_t stride = (int64_t)gridDim.x * kBlock, tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    int v[5] = {0, 0, 0, 0, 0};     // staged row blocks, staged column blocks, longest column, longest row, heavy
+    for (int64_t b = tid; b < rblocks; b += stride) v[0] += f_desc[b * nm::kStageDesc] >= 0;
+    for (int64_t b = tid; b < cblocks; b += stride) v[1] += b_desc[b * nm::kStageDesc] >= 0;
+    for (int64_t i = tid; i < cblocks * 8; i += stride) {
+        if ((i & 4) == 0) v[2] = max(v[2], stats[i]);
+        else v[4] = max(v[4], stats[i]);
+    }
+    for (int64_t i = tid; i < rblocks * 4; i += stride) v[3] = max(v[3], stats[cblocks * 8 + i]);
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1)
+#pragma unroll
+        for (int k = 0; k < 5; ++k) {
+            const int o = __shfl_xor(v[k], off, kWave);
+            v[k] = k < 2 ? v[k] + o : max(v[k], o);
+        }
+    if ((threadIdx.x & (kWave - 1)) == 0)
+        for (int k = 0; k < 5; ++k) s_red[k][threadIdx.x / kWave] = v[k];
+    __syncthreads();
+    if (threadIdx.x < 5) {
+        const int k = threadIdx.x;
+        int r = 0;
+        for (int w = 0; w < kBlock / kWave; ++w) r = k < 2 ? r + s_red[k][w] : max(r, s_red[k][w]);
+        const int slot = k == 0 ? 4 : k == 1 ? 5 : k == 2 ? 6 : k == 3 ? 7 : 8;
+        if (k < 2) { if (r) atomicAdd(&flags[slot], r); }
+        else if (r) atomicMax(&flags[slot], r);
+    }
 }
 
 // Clears flags[0] unless A^T has exactly A's structure.
@@ -531,8 +568,11 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
         if (grid > 65536) grid = 65536;
         hipLaunchKernelGGL(tp_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, cols, plan.t_indptr,
                            plan.t_row, plan.t_perm, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.f_desc,
-                           plan.b_desc, plan.flags);
+                           plan.b_desc, plan.stats, plan.flags);
         NM_LAUNCH_CHECK("tp_pack_kernel");
+        hipLaunchKernelGGL(tp_stats_kernel, dim3(32), dim3(kBlock), 0, s, ceil_div(rows, (int64_t)kPackRows),
+                           ceil_div(cols, (int64_t)kPackCols), plan.f_desc, plan.b_desc, plan.stats, plan.flags);
+        NM_LAUNCH_CHECK("tp_stats_kernel");
     }
     return NM_OK;
 }

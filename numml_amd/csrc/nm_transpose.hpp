@@ -54,6 +54,7 @@ struct TPlan {
     int16_t *c_off16;
     int32_t *f_desc;
     int32_t *b_desc;
+    int32_t *stats;     // per wavefront of the packing kernel: lengths it saw (reduced into flags[6..8])
 };
 
 // Blocks the packed offsets are relative to: the columns one workgroup of the planned SpMV
@@ -86,7 +87,8 @@ inline size_t tplan_layout(int64_t rows, int64_t cols, int64_t nnz, void *base, 
     int16_t *co = (int16_t *)take((size_t)(nnz + 8) * 2);
     int32_t *fd = (int32_t *)take((size_t)((rows + kPackRows - 1) / kPackRows + 1) * kStageDesc * 4);
     int32_t *bd = (int32_t *)take((size_t)((cols + kPackCols - 1) / kPackCols + 1) * kStageDesc * 4);
-    if (p) *p = TPlan{a, b, c, h, f, ci, cp, tw, co, fd, bd};
+    int32_t *st = (int32_t *)take((size_t)(((cols + kPackCols - 1) / kPackCols) * 8 + ((rows + kPackRows - 1) / kPackRows) * 4 + 8) * 4);
+    if (p) *p = TPlan{a, b, c, h, f, ci, cp, tw, co, fd, bd, st};
     return off;
 }
 
