@@ -33,6 +33,7 @@ _SIGNATURES = {
     "nm_csr_transpose_plan_info": [_c_i64, _c_i64, _c_i64, _c_ptr, ctypes.POINTER(ctypes.c_int32), _c_ptr],
     "nm_stream_probe": [_c_ptr, _c_size, _c_ptr, _c_size, _c_ptr],
     "nm_spgemv_forward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "nm_spgemv_forward_planned_lists": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_spgemv_backward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                    _c_ptr, _c_ptr],
     "nm_spdmm_backward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64,

@@ -244,14 +244,21 @@ __device__ __forceinline__ void fwd_tile_staged(const int64_t r0, const int nr, 
 //
 // IDX: int64_t for the structure arrays as the interface delivers them, int32_t for the
 // 32-bit copies a transposed-structure plan of the same pattern holds.
-template <typename T, int BLOCK, int R, int CAP, bool UNIT = false, typename IDX = int64_t>
+//
+// LISTS: the instantiation that takes the tiles with a staging list through fwd_tile_staged.  It
+// keeps LDS for the staged segments of x, which costs resident workgroups on patterns without
+// lists (fp64: 43 instead of 26 KB), so it is a separate instantiation that the caller asks for;
+// without it a tile with a list is read through the plan's 32-bit columns (its 16-bit words hold
+// places in the list, not offsets).
+template <typename T, int BLOCK, int R, int CAP, bool UNIT = false, typename IDX = int64_t, bool LISTS = false>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_num_sgpr(72))) void spmv_fwd_kernel(
     int64_t rows, int rt, const T *__restrict__ data, const IDX *__restrict__ indices,
     const IDX *__restrict__ indptr, const T *__restrict__ x, T *__restrict__ y,
     const int16_t *__restrict__ off16 = nullptr, const int32_t *__restrict__ flags = nullptr,
     const int32_t *__restrict__ f_desc = nullptr) {
     // rt <= R: rows per block of this launch (block_rows)
-    constexpr bool STAGE = NM_STAGE_FWD && NM_FWD32_VEC && sizeof(IDX) == 4 && !UNIT && R == nm::kPackRows;
+    constexpr bool STAGE = LISTS && NM_STAGE_FWD && NM_FWD32_VEC && sizeof(IDX) == 4 && !UNIT && R == nm::kPackRows;
+    constexpr bool HAS_LISTS = NM_STAGE_FWD && sizeof(IDX) == 4 && !UNIT && R == nm::kPackRows;
     __shared__ int32_t s_off[R + 1];
     __shared__ __align__(16) T s_prod[CAP];
     __shared__ __align__(16) T s_x[STAGE ? nm::kStageFwd * nm::kStageSeg : 4];
@@ -270,6 +277,9 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_num_sgpr(72))) void sp
         nr = nr < R ? nr : R;   // rt <= R
         const int64_t base = indptr[r0];
         bool packed_here = packed;
+        if constexpr (HAS_LISTS && !STAGE) {
+            if (packed && f_desc != nullptr && f_desc[tile * nm::kStageDesc] >= 0) packed_here = false;
+        }
         if constexpr (STAGE) if (f_desc != nullptr && rt == nm::kPackRows) {
             // A block of rows with a staging list keeps places in that list where other blocks
             // keep column offsets.  The tile's end, the head of its list and the wavefront's
@@ -631,11 +641,11 @@ template <int BLOCK> constexpr int kBwdXQ = (nm::kStageBwd * nm::kStageSeg / 4 +
 // listed segments of g and x a quad per lane, a column's two bounds with one request, the packed
 // words of the first 1024 entries four consecutive entries per lane (QUAD; grad_A then leaves 16
 // bytes per lane as well) and the rest in ER rounds of one entry per lane; only the values of A
-// are gathered entry by entry.  SEG2: the list has more than eight places.
-template <typename T, int R, int CAP, bool O32, bool QUAD, int ER, bool SEG2>
+// are gathered entry by entry.
+template <typename T, int R, int CAP, bool O32, bool QUAD, int ER>
 __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, const int32_t base, const int n,
                                                 const int32_t lo0, const int32_t hi0, const int32_t lo1,
-                                                const int32_t hi1, const T *__restrict__ data,
+                                                const int32_t hi1, const bool seg2, const T *__restrict__ data,
                                                 const int32_t *__restrict__ t_indptr,
                                                 const int32_t *__restrict__ t_pack, const T *__restrict__ x,
                                                 const T *__restrict__ g, T *__restrict__ grad_A,
@@ -643,11 +653,22 @@ __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, 
     typedef T TV __attribute__((ext_vector_type(4), aligned(sizeof(T))));
     typedef int32_t I4 __attribute__((ext_vector_type(4), aligned(4)));
     typedef int32_t I2 __attribute__((ext_vector_type(2), aligned(4)));
-    constexpr int XQ = SEG2 ? kBwdXQ<kBlock> : 1;
     constexpr int kQuads = QUAD ? 4 * kBlock : 0;       // entries of the quad phase
     static_assert(R == kBlock && nm::kStageSeg == 128, "lane = column, two segments per wavefront and request");
     static_assert(kBwdXQ<kBlock> == 2, "a list of at most sixteen places");
     const int tid = threadIdx.x;
+    // Places eight and up of the list (seg2: the list has that many): the one request of the tile
+    // that is not made every time.  It goes first: a request that may or may not have been made
+    // only spoils the compiler's count of what is still in flight for the requests BEHIND it.
+    TV gs1, xs1;
+    const bool second = seg2 && 4 * (tid + kBlock) < nm::kStageBwd * nm::kStageSeg;
+    if (seg2) {
+        int32_t seg = (tid & 32) ? hi1 : lo1;
+        seg = seg < 0 ? 0 : seg;
+        const int64_t at0 = (int64_t)seg * nm::kStageSeg + 4 * (tid & 31);
+        gs1 = *reinterpret_cast<const TV *>(g + at0);
+        xs1 = *reinterpret_cast<const TV *>(x + at0);
+    }
     // packed words
     I4 wq;
     if (QUAD) wq = __builtin_nontemporal_load(reinterpret_cast<const I4 *>(at<O32>(t_pack, base + tid * 4)));
@@ -657,17 +678,16 @@ __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, 
         const int k = kQuads + r * kBlock + tid;
         we[r] = nm::stream_load(at<O32>(t_pack, base + (k < n ? k : n - 1)));
     }
-    // the wavefront's two segments per request (an unused place of the list loads segment 0)
-    TV gs[XQ], xs[XQ];
-#pragma unroll
-    for (int u = 0; u < XQ; ++u) {
+    // the wavefront's two segments of places 0-7 (an unused place of the list loads segment 0)
+    TV gs0, xs0;
+    {
         // (separate scalars, not an array: the compiler turns a choice between array elements into
         // an indexed read of a copy of the array in scratch memory)
-        int32_t seg = u == 0 ? ((tid & 32) ? hi0 : lo0) : ((tid & 32) ? hi1 : lo1);
+        int32_t seg = (tid & 32) ? hi0 : lo0;
         seg = seg < 0 ? 0 : seg;
         const int64_t at0 = (int64_t)seg * nm::kStageSeg + 4 * (tid & 31);
-        gs[u] = *reinterpret_cast<const TV *>(g + at0);
-        xs[u] = *reinterpret_cast<const TV *>(x + at0);
+        gs0 = *reinterpret_cast<const TV *>(g + at0);
+        xs0 = *reinterpret_cast<const TV *>(x + at0);
     }
     // bounds of column c0 + tid and the factor its entries share (the lane writes the mirror entry)
     int32_t pa, pb;
@@ -691,12 +711,12 @@ __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, 
         const int kc = k < n ? k : n - 1;
         de[r] = *at<O32>(data, base + kc + (we[r] >> 16));
     }
-#pragma unroll
-    for (int u = 0; u < XQ; ++u)
-        if (4 * (tid + u * kBlock) < nm::kStageBwd * nm::kStageSeg) {      // (the list's last places: half a workgroup)
-            *reinterpret_cast<TV *>(s_g + 4 * (tid + u * kBlock)) = gs[u];
-            *reinterpret_cast<TV *>(s_x + 4 * (tid + u * kBlock)) = xs[u];
-        }
+    *reinterpret_cast<TV *>(s_g + 4 * tid) = gs0;
+    *reinterpret_cast<TV *>(s_x + 4 * tid) = xs0;
+    if (second) {       // (the list's last places: half a workgroup)
+        *reinterpret_cast<TV *>(s_g + 4 * (tid + kBlock)) = gs1;
+        *reinterpret_cast<TV *>(s_x + 4 * (tid + kBlock)) = xs1;
+    }
     // (pinned: left alone, the compiler moves the request for `own` down into the branch that
     // uses it, behind the gathers)
     asm volatile("" : "+v"(own));
@@ -789,15 +809,22 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
             const int32_t lo0 = desc[2 * wave], hi0 = desc[2 * wave + 1];
             const int32_t lo1 = desc[kBlock / 32 + 2 * wave], hi1 = desc[kBlock / 32 + 2 * wave + 1];
             const bool live = (lo0 & hi0 & lo1 & hi1) != INT32_MIN;
-            if ((d0 >= 0) & (n_all >= 1) & (n_all <= CAP) & live) {
+            if ((d0 >= 0) & (n_all >= 4 * kBlock) & (n_all <= CAP) & live) {
                 const bool seg2 = desc[8] >= 0;
-#define NM_BWD_TILE(QUAD, ER, SEG2)                                                                                \
-    bwd_tile_staged<T, R, CAP, O32, QUAD, ER, SEG2>(c0, nc, first, n_all, lo0, hi0, lo1, hi1, data, t_indptr, t_pack, x, g, grad_A, \
-                                                    grad_x, s_v, s_g, s_x)
-                // (the five-point block: 1024 entries in quads and one round, eight segments)
-                if (n_all >= 4 * kBlock && n_all <= 5 * kBlock && !seg2) NM_BWD_TILE(true, 1, false);
-                else if (n_all >= 4 * kBlock) NM_BWD_TILE(true, (CAP - 4 * kBlock) / kBlock, true);
-                else NM_BWD_TILE(false, 4, true);
+#define NM_BWD_TILE(QUAD, ER)                                                                                       \
+    bwd_tile_staged<T, R, CAP, O32, QUAD, ER>(c0, nc, first, n_all, lo0, hi0, lo1, hi1, seg2, data, t_indptr, t_pack, \
+                                              x, g, grad_A, grad_x, s_v, s_g, s_x)
+                // the first 1024 entries in quads where there are as many, the rest in rounds of 256
+                // (the five-point block: quads and one round)
+                static_assert(CAP == 8 * kBlock, "up to four rounds behind the quads");
+                static_assert(nm::kStageBwdMin == 4 * kBlock, "a block with a list fills the quads");
+                switch ((n_all - 4 * kBlock + kBlock - 1) / kBlock) {
+                    case 0: NM_BWD_TILE(true, 0); break;
+                    case 1: NM_BWD_TILE(true, 1); break;
+                    case 2: NM_BWD_TILE(true, 2); break;
+                    case 3: NM_BWD_TILE(true, 3); break;
+                    default: NM_BWD_TILE(true, 4); break;
+                }
 #undef NM_BWD_TILE
                 __syncthreads();
                 continue;
@@ -1132,7 +1159,7 @@ int check_csr(int64_t rows, int64_t cols, int64_t nnz, const void *data, const i
     return NM_OK;
 }
 
-template <typename T, typename IDX>
+template <typename T, typename IDX, bool LISTS = false>
 int launch_fwd(int64_t rows, int64_t nnz, const T *data, const IDX *indices, const IDX *indptr, const T *x,
                T *y, hipStream_t s, const int16_t *off16 = nullptr, const int32_t *flags = nullptr,
                const int32_t *f_desc = nullptr) {
@@ -1140,7 +1167,7 @@ int launch_fwd(int64_t rows, int64_t nnz, const T *data, const IDX *indices, con
     const int rt = block_rows(rows, nnz, R, CAP);
     int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, false, IDX>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s,
+    hipLaunchKernelGGL((spmv_fwd_kernel<T, kFwdBlock, R, CAP, false, IDX, LISTS>), dim3((unsigned)grid), dim3(kFwdBlock), 0, s,
                        rows, rt, data, indices, indptr, x, y, off16, flags, f_desc);
     NM_LAUNCH_CHECK("spmv_fwd_kernel");
     return NM_OK;
@@ -1193,8 +1220,10 @@ extern "C" int nm_spgemv_forward(nm_dtype dt, int64_t rows, int64_t cols, int64_
     return nm::fail(NM_ERR_INVALID, "unknown dtype %d", (int)dt);
 }
 
-extern "C" int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
-                                         const void *plan_mem, const void *x, void *y, nm_stream stream) {
+namespace {
+template <bool LISTS>
+int forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data, const void *plan_mem,
+                    const void *x, void *y, nm_stream stream) {
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
     NM_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0 && plan_mem != nullptr, "bad sizes or null plan");
     if (rows == 0) return NM_OK;
@@ -1204,10 +1233,21 @@ extern "C" int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols
     nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
     hipStream_t s = nm::as_stream(stream);
     if (dt == NM_F32)
-        return launch_fwd<float, int32_t>(rows, nnz, (const float *)data, t.c_idx32, t.c_ptr32, (const float *)x,
-                                          (float *)y, s, t.c_off16, t.flags, nnz > 0 ? t.f_desc : nullptr);
-    return launch_fwd<double, int32_t>(rows, nnz, (const double *)data, t.c_idx32, t.c_ptr32, (const double *)x,
-                                       (double *)y, s, t.c_off16, t.flags, nnz > 0 ? t.f_desc : nullptr);
+        return launch_fwd<float, int32_t, LISTS>(rows, nnz, (const float *)data, t.c_idx32, t.c_ptr32, (const float *)x,
+                                                 (float *)y, s, t.c_off16, t.flags, nnz > 0 ? t.f_desc : nullptr);
+    return launch_fwd<double, int32_t, LISTS>(rows, nnz, (const double *)data, t.c_idx32, t.c_ptr32, (const double *)x,
+                                              (double *)y, s, t.c_off16, t.flags, nnz > 0 ? t.f_desc : nullptr);
+}
+}  // namespace
+
+extern "C" int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                         const void *plan_mem, const void *x, void *y, nm_stream stream) {
+    return forward_planned<false>(dt, rows, cols, nnz, data, plan_mem, x, y, stream);
+}
+
+extern "C" int nm_spgemv_forward_planned_lists(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                               const void *plan_mem, const void *x, void *y, nm_stream stream) {
+    return forward_planned<true>(dt, rows, cols, nnz, data, plan_mem, x, y, stream);
 }
 
 extern "C" int nm_csr_row_sum_forward(nm_dtype dt, int64_t rows, int64_t nnz, const void *data,

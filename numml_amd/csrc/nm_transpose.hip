@@ -321,14 +321,14 @@ struct StageTable {
 };
 
 template <int MOST>
-__device__ __forceinline__ bool stage_block(StageTable &t, int64_t line0, int32_t pb, int32_t pe, int most_entries,
-                                            int64_t veclen, const int32_t *__restrict__ key,
+__device__ __forceinline__ bool stage_block(StageTable &t, int64_t line0, int32_t pb, int32_t pe, int least_entries,
+                                            int most_entries, int64_t veclen, const int32_t *__restrict__ key,
                                             int32_t *__restrict__ desc) {
     if (threadIdx.x < StageTable::kWords) t.bits[threadIdx.x] = 0;
     const int32_t seg0 = (int32_t)(line0 / nm::kStageSeg) - StageTable::kReach;
     if (threadIdx.x == 0) {
         t.seg0 = seg0;
-        t.bad = (pe - pb > most_entries || pe == pb) ? 1 : 0;
+        t.bad = (pe - pb > most_entries || pe - pb < least_entries || pe == pb) ? 1 : 0;
     }
     __syncthreads();
     if (t.bad == 0) {
@@ -404,8 +404,10 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
             }
         }
         // (a list made here is only read when every packed word of the plan turns out valid)
-        const bool staged = stage_block<nm::kStageBwd>(table, c0, pb, pe, nm::kStageBwdCap, rows, t_row,
-                                                       b_desc + b * nm::kStageDesc);
+        // (a block of fewer than 1024 entries -- under four a column -- is a tile so small that the
+        // backward is bound by the round trips of a tile, and the kernel without lists makes one fewer)
+        const bool staged = stage_block<nm::kStageBwd>(table, c0, pb, pe, nm::kStageBwdMin, nm::kStageBwdCap, rows,
+                                                       t_row, b_desc + b * nm::kStageDesc);
         for (int32_t p0 = pb; p0 < pe; p0 += kBlock) {
             const int32_t p = p0 + (int32_t)threadIdx.x;
             const bool active = p < pe;
@@ -429,7 +431,7 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
             for (int off = kWave / 2; off > 0; off >>= 1) len = max(len, __shfl_xor(len, off, kWave));
             if ((threadIdx.x & (kWave - 1)) == 0) stats[cblocks * 8 + b * 4 + threadIdx.x / kWave] = len;
         }
-        const bool staged = stage_block<nm::kStageFwd>(table, r0, kb, ke, nm::kStageFwdCap, cols, c_idx32,
+        const bool staged = stage_block<nm::kStageFwd>(table, r0, kb, ke, 4, nm::kStageFwdCap, cols, c_idx32,
                                                        f_desc + b * nm::kStageDesc);
         for (int32_t k0 = kb; k0 < ke; k0 += kBlock) {
             const int32_t k = k0 + (int32_t)threadIdx.x;
@@ -448,15 +450,24 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
 
 // flags[4] / flags[5]: blocks of rows / columns with a staging list; flags[6] / flags[7]: the longest
 // column / row; flags[8]: the most entries that columns of more than 512 entries hold inside one
-// aligned group of 64 columns.  From what tp_pack_kernel left per block and per wavefront.
-__global__ __launch_bounds__(kBlock) void tp_stats_kernel(int64_t rblocks, int64_t cblocks,
+// aligned group of 64 columns; flags[9]: blocks of rows with a list and at most 3072 entries.  From what
+// tp_pack_kernel left per block and per wavefront.
+__global__ __launch_bounds__(kBlock) void tp_stats_kernel(int64_t rows, int64_t rblocks, int64_t cblocks,
+                                                          const int32_t *__restrict__ c_ptr32,
                                                           const int32_t *__restrict__ f_desc,
                                                           const int32_t *__restrict__ b_desc,
                                                           const int32_t *__restrict__ stats, int32_t *flags) {
-    __shared__ int32_t s_red[5][kBlock / kWave];
+    __shared__ int32_t s_red[6][kBlock / kWave];
     const int64_t stride = (int64_t)gridDim.x * kBlock, tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    int v[5] = {0, 0, 0, 0, 0};     // staged row blocks, staged column blocks, longest column, longest row, heavy
-    for (int64_t b = tid; b < rblocks; b += stride) v[0] += f_desc[b * nm::kStageDesc] >= 0;
+    // staged row blocks, staged column blocks, longest column, longest row, heavy, staged row blocks of
+    // at most 3072 entries (what the forward's fp64 tile holds)
+    int v[6] = {0, 0, 0, 0, 0, 0};
+    for (int64_t b = tid; b < rblocks; b += stride) {
+        const bool staged = f_desc[b * nm::kStageDesc] >= 0;
+        const int64_t r1 = (b + 1) * nm::kPackRows < rows ? (b + 1) * nm::kPackRows : rows;
+        v[0] += staged;
+        v[5] += staged && c_ptr32[r1] - c_ptr32[b * nm::kPackRows] <= 3072;
+    }
     for (int64_t b = tid; b < cblocks; b += stride) v[1] += b_desc[b * nm::kStageDesc] >= 0;
     for (int64_t i = tid; i < cblocks * 8; i += stride) {
         if ((i & 4) == 0) v[2] = max(v[2], stats[i]);
@@ -466,19 +477,20 @@ __global__ __launch_bounds__(kBlock) void tp_stats_kernel(int64_t rblocks, int64
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1)
 #pragma unroll
-        for (int k = 0; k < 5; ++k) {
+        for (int k = 0; k < 6; ++k) {
             const int o = __shfl_xor(v[k], off, kWave);
-            v[k] = k < 2 ? v[k] + o : max(v[k], o);
+            v[k] = (k < 2 || k == 5) ? v[k] + o : max(v[k], o);
         }
     if ((threadIdx.x & (kWave - 1)) == 0)
-        for (int k = 0; k < 5; ++k) s_red[k][threadIdx.x / kWave] = v[k];
+        for (int k = 0; k < 6; ++k) s_red[k][threadIdx.x / kWave] = v[k];
     __syncthreads();
-    if (threadIdx.x < 5) {
+    if (threadIdx.x < 6) {
         const int k = threadIdx.x;
+        const bool sum = k < 2 || k == 5;
         int r = 0;
-        for (int w = 0; w < kBlock / kWave; ++w) r = k < 2 ? r + s_red[k][w] : max(r, s_red[k][w]);
-        const int slot = k == 0 ? 4 : k == 1 ? 5 : k == 2 ? 6 : k == 3 ? 7 : 8;
-        if (k < 2) { if (r) atomicAdd(&flags[slot], r); }
+        for (int w = 0; w < kBlock / kWave; ++w) r = sum ? r + s_red[k][w] : max(r, s_red[k][w]);
+        const int slot = k == 0 ? 4 : k == 1 ? 5 : k == 2 ? 6 : k == 3 ? 7 : k == 4 ? 8 : 9;
+        if (sum) { if (r) atomicAdd(&flags[slot], r); }
         else if (r) atomicMax(&flags[slot], r);
     }
 }
@@ -570,8 +582,9 @@ int tplan_build(int64_t rows, int64_t cols, int64_t nnz, const int64_t *indices,
                            plan.t_row, plan.t_perm, plan.c_ptr32, plan.c_idx32, plan.t_pack, plan.c_off16, plan.f_desc,
                            plan.b_desc, plan.stats, plan.flags);
         NM_LAUNCH_CHECK("tp_pack_kernel");
-        hipLaunchKernelGGL(tp_stats_kernel, dim3(32), dim3(kBlock), 0, s, ceil_div(rows, (int64_t)kPackRows),
-                           ceil_div(cols, (int64_t)kPackCols), plan.f_desc, plan.b_desc, plan.stats, plan.flags);
+        hipLaunchKernelGGL(tp_stats_kernel, dim3(32), dim3(kBlock), 0, s, rows, ceil_div(rows, (int64_t)kPackRows),
+                           ceil_div(cols, (int64_t)kPackCols), plan.c_ptr32, plan.f_desc, plan.b_desc, plan.stats,
+                           plan.flags);
         NM_LAUNCH_CHECK("tp_stats_kernel");
     }
     return NM_OK;
@@ -626,6 +639,6 @@ extern "C" int nm_csr_transpose_plan_info(int64_t rows, int64_t cols, int64_t nn
     hipStream_t s = nm::as_stream(stream);
     NM_HIP_TRY(hipMemcpyAsync(info, plan.flags, 16 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
     NM_HIP_TRY(hipStreamSynchronize(s));
-    if (nnz == 0) info[1] = info[2] = info[4] = info[5] = 0;     // (nothing was packed or listed)
+    if (nnz == 0) info[1] = info[2] = info[4] = info[5] = info[9] = 0;     // (nothing was packed or listed)
     return NM_OK;
 }

@@ -31,7 +31,8 @@
 //                by the end of x, more entries than a tile holds); c_off16 is as described above
 //   b_desc[b]    the same for the b-th block of kPackCols columns and the ROWS its entries lie
 //                in (up to kStageBwd segments); such a block keeps the place in the list in the
-//                low half of t_pack[p].  Only made when flags[1] != 0
+//                low half of t_pack[p].  Only read when flags[1] != 0; blocks of fewer than
+//                kStageBwdMin entries get none
 //
 // Inside a column the entries keep A's row-major order (the sort is stable), so
 // rows ascend, exactly like the counting-sort transpose of the reference
@@ -64,7 +65,7 @@ constexpr int kPackCols = 256, kPackRows = 512;
 // per block of columns (backward), ints per list.
 constexpr int kStageSeg = 128, kStageFwd = 16, kStageBwd = 12, kStageDesc = 16;
 // Entries a block may hold to get a list: the LDS tiles of the kernels that use it.
-constexpr int kStageFwdCap = 4096, kStageBwdCap = 2048;
+constexpr int kStageFwdCap = 4096, kStageBwdCap = 2048, kStageBwdMin = 1024;
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 

@@ -105,6 +105,11 @@ def test_planned_spmv_packed_and_plain_structure(dev, dtype):
                 gx = torch.full((cols,), 7.0, dtype=D.dtype, device=dev)
                 _lib.check(L.nm_spgemv_forward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(y),
                                                        stream), "nm_spgemv_forward_planned")
+                # the instantiation that takes blocks with a staging list through LDS: the same bits
+                y_l = torch.full((rows,), 7.0, dtype=D.dtype, device=dev)
+                _lib.check(L.nm_spgemv_forward_planned_lists(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X),
+                                                             ptr(y_l), stream), "nm_spgemv_forward_planned_lists")
+                assert torch.equal(y, y_l), f"{name}: forward with and without staging lists"
                 _lib.check(L.nm_spgemv_backward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
                                                         ptr(gA), ptr(gx), stream), "nm_spgemv_backward_planned")
                 same = assert_same if exact else assert_close
