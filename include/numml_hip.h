@@ -177,8 +177,21 @@ int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t 
                                const void *x, const void *g,
                                void *grad_A, void *grad_x, nm_stream stream);
 
+/* The same gradients by the instantiation that takes blocks of 256 columns with
+ * a staging list (nm_csr_transpose_plan_info: info[5]) through LDS: the listed
+ * segments of g and x are loaded with coalesced requests and the entries'
+ * factors looked up there; nm_spgemv_backward_planned walks such a block on
+ * the plan's unpacked row and position arrays instead.  The LDS it reserves
+ * costs resident workgroups and the list one more dependent load per block:
+ * for plans most of whose column blocks have a list (same bits either way).  No
+ * counterpart in the reference. */
+int nm_spgemv_backward_planned_lists(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                                     const void *data, const void *plan_mem,
+                                     const void *x, const void *g,
+                                     void *grad_A, void *grad_x, nm_stream stream);
+
 /* Test hook (no counterpart in the reference): `wide_offsets` = 1 makes
- * nm_spgemv_backward_planned address its arrays with 64-bit offsets whatever
+ * nm_spgemv_backward_planned(_lists) address its arrays with 64-bit offsets whatever
  * their size -- the variant that arrays of 4 GiB and more take -- so that it
  * can be run on small inputs; 0 restores the choice by size.  Process-wide. */
 int nm_spgemv_configure(int wide_offsets);

@@ -36,6 +36,8 @@ _SIGNATURES = {
     "nm_spgemv_forward_planned_lists": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "nm_spgemv_backward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                    _c_ptr, _c_ptr],
+    "nm_spgemv_backward_planned_lists": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                   _c_ptr, _c_ptr],
     "nm_spdmm_backward_planned": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64,
                                   _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "nm_spdmm_forward": [_c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64,

@@ -767,15 +767,22 @@ __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, 
 // pattern is symmetric (plan flag) the column-major entry p is the mirror of the
 // row-major entry p = (row c, column r), so the lane writes
 // grad_A[p] = g[c] * x[r] instead: a coalesced store, every entry once.
-template <typename T, int R, int CAP, bool O32>
-__global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
+// LISTS: the build for plans most of whose column blocks have a staging list (it keeps the listed
+// segments of g and x in LDS).  The other build takes a block with a list through the plan's
+// unpacked arrays (t_row, t_perm), which every plan holds, and needs no LDS for segments.
+// (The resident wavefronts asked for are what each build reaches anyway; stating them changes the
+// schedule the compiler picks, measured 4 M-row tridiagonal fp32 47.6 -> 40.8 us, 2048^2 five-point
+// 61.4 -> 59.9 us.)
+template <typename T, int R, int CAP, bool O32, bool LISTS>
+__global__ __launch_bounds__(kBlock)
+__attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? (LISTS ? 6 : 8) : (LISTS ? 3 : 7)))) void spmv_bwd_planned_kernel(
     int64_t cols, const T *__restrict__ data, const int32_t *__restrict__ t_indptr,
     const int32_t *__restrict__ t_row, const int32_t *__restrict__ t_perm, const int32_t *__restrict__ t_pack,
     const int32_t *__restrict__ flags, const T *__restrict__ x, const T *__restrict__ g,
     T *__restrict__ grad_A, T *__restrict__ grad_x, const int32_t *__restrict__ b_desc) {
     static_assert(R == nm::kPackCols, "t_pack holds rows relative to the first column of a workgroup's block");
     static_assert(nm::kStageBwdCap <= CAP, "a block with a staging list fits the tile");
-    constexpr bool STAGE = NM_STAGE_BWD != 0;
+    constexpr bool STAGE = LISTS && NM_STAGE_BWD != 0;
     constexpr int kStaged = nm::kStageBwd * nm::kStageSeg;
     __shared__ int32_t s_off[R + 1];
     __shared__ __align__(16) T s_v[CAP];
@@ -786,7 +793,7 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const bool mirror = flags[0] != 0;
     // one packed word per entry in place of (t_row, t_perm): patterns near the diagonal
-    const bool packed = flags[1] != 0;
+    const bool packed_plan = flags[1] != 0;
     static_assert(R == kBlock, "lane t of a workgroup stages column t of its block");
     const int64_t ntiles = (cols + R - 1) / R, npad = nm::xcd_padded(ntiles);
     const bool fused = mirror && grad_A && grad_x;
@@ -799,6 +806,9 @@ __global__ __launch_bounds__(kBlock) void spmv_bwd_planned_kernel(
         if (tile >= ntiles) continue;
         const int64_t c0 = tile * R;
         const int nc = (int)(cols - c0 < R ? cols - c0 : R);
+        bool packed = packed_plan;
+        // (the low half of a packed word of a block with a list is a place in the listed segments)
+        if constexpr (!STAGE) if (packed_plan && b_desc != nullptr) packed = b_desc[tile * nm::kStageDesc] < 0;
         if constexpr (STAGE) if (fused && packed && b_desc != nullptr) {
             // a block of columns with a staging list, both gradients: the tile's ends, the head of
             // its list and the wavefront's four places of the list come together (scalar loads);
@@ -1301,9 +1311,27 @@ extern "C" int nm_spgemv_configure(int wide_offsets) {
     return NM_OK;
 }
 
-extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
-                                          const void *plan_mem, const void *x, const void *g, void *grad_A,
-                                          void *grad_x, nm_stream stream) {
+namespace {
+template <typename T, bool LISTS>
+void launch_bwd_planned(int64_t cols, int64_t nnz, const nm::TPlan &t, bool o32, const void *data, const void *x,
+                        const void *g, void *grad_A, void *grad_x, hipStream_t s) {
+    constexpr int R = kPlannedR, CAP = kPlannedCap;
+    int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
+    if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
+    const int32_t *desc = nnz > 0 ? t.b_desc : nullptr;
+    if (o32)
+        hipLaunchKernelGGL((spmv_bwd_planned_kernel<T, R, CAP, true, LISTS>), dim3((unsigned)grid), dim3(kBlock), 0, s,
+                           cols, (const T *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const T *)x,
+                           (const T *)g, (T *)grad_A, (T *)grad_x, desc);
+    else
+        hipLaunchKernelGGL((spmv_bwd_planned_kernel<T, R, CAP, false, LISTS>), dim3((unsigned)grid), dim3(kBlock), 0, s,
+                           cols, (const T *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const T *)x,
+                           (const T *)g, (T *)grad_A, (T *)grad_x, desc);
+}
+
+template <bool LISTS>
+int backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data, const void *plan_mem,
+                     const void *x, const void *g, void *grad_A, void *grad_x, nm_stream stream) {
     NM_REQUIRE(dt == NM_F32 || dt == NM_F64, "unknown dtype %d", (int)dt);
     NM_REQUIRE(rows >= 0 && cols >= 0 && nnz >= 0 && plan_mem != nullptr, "bad sizes or null plan");
     if (cols == 0 || (!grad_A && !grad_x)) return NM_OK;
@@ -1314,31 +1342,21 @@ extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t col
     // every array the kernel indexes stays below 4 GiB: 32-bit byte offsets
     const int64_t longest = std::max(std::max(rows, cols) + 2, nnz + 1);
     const bool o32 = !g_wide_offsets.load(std::memory_order_relaxed) && longest * (dt == NM_F32 ? 4 : 8) < (int64_t(1) << 32);
-    if (dt == NM_F32) {
-        constexpr int R = kPlannedR, CAP = kPlannedCap;
-        int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
-        if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-        if (o32)
-            hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                               (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const float *)x,
-                               (const float *)g, (float *)grad_A, (float *)grad_x, nnz > 0 ? t.b_desc : nullptr);
-        else
-            hipLaunchKernelGGL((spmv_bwd_planned_kernel<float, R, CAP, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                               (const float *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const float *)x,
-                               (const float *)g, (float *)grad_A, (float *)grad_x, nnz > 0 ? t.b_desc : nullptr);
-    } else {
-        constexpr int R = kPlannedR, CAP = kPlannedCap;
-        int64_t grid = nm::xcd_padded(nm::ceil_div(cols, R));
-        if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;
-        if (o32)
-            hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                               (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const double *)x,
-                               (const double *)g, (double *)grad_A, (double *)grad_x, nnz > 0 ? t.b_desc : nullptr);
-        else
-            hipLaunchKernelGGL((spmv_bwd_planned_kernel<double, R, CAP, false>), dim3((unsigned)grid), dim3(kBlock), 0, s, cols,
-                               (const double *)data, t.t_indptr, t.t_row, t.t_perm, t.t_pack, t.flags, (const double *)x,
-                               (const double *)g, (double *)grad_A, (double *)grad_x, nnz > 0 ? t.b_desc : nullptr);
-    }
+    if (dt == NM_F32) launch_bwd_planned<float, LISTS>(cols, nnz, t, o32, data, x, g, grad_A, grad_x, s);
+    else launch_bwd_planned<double, LISTS>(cols, nnz, t, o32, data, x, g, grad_A, grad_x, s);
     NM_LAUNCH_CHECK("spmv_bwd_planned_kernel");
     return NM_OK;
+}
+}  // namespace
+
+extern "C" int nm_spgemv_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
+                                          const void *plan_mem, const void *x, const void *g, void *grad_A,
+                                          void *grad_x, nm_stream stream) {
+    return backward_planned<false>(dt, rows, cols, nnz, data, plan_mem, x, g, grad_A, grad_x, stream);
+}
+
+extern "C" int nm_spgemv_backward_planned_lists(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
+                                                const void *data, const void *plan_mem, const void *x,
+                                                const void *g, void *grad_A, void *grad_x, nm_stream stream) {
+    return backward_planned<true>(dt, rows, cols, nnz, data, plan_mem, x, g, grad_A, grad_x, stream);
 }

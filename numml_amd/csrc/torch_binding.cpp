@@ -770,9 +770,12 @@ std::vector<Tensor> spgemv_backward(Tensor grad_z, int A_rows, int A_cols, Tenso
     if (want.first) grad_A = torch::empty_like(A_data);
     if (want.second) grad_x = torch::empty_like(x);
     if (auto plan = backward_plan(A_col_ind, A_rowptr, A_rows, x.size(0), dev)) {
-        check(nm_spgemv_backward_planned(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),
-                                         plan->mem.data_ptr(), x.data_ptr(), grad_z.data_ptr(),
-                                         ptr_or_null(grad_A), ptr_or_null(grad_x), current_stream(dev)),
+        // most blocks of 256 columns have a staging list: the instantiation that stages g and x in LDS
+        const int32_t *info = plan_info(*plan, A_rows, x.size(0), A_data.numel(), dev);
+        const bool lists = 2 * (int64_t)info[5] >= ((int64_t)x.size(0) + 255) / 256;
+        check((lists ? nm_spgemv_backward_planned_lists : nm_spgemv_backward_planned)(
+                  dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(), plan->mem.data_ptr(),
+                  x.data_ptr(), grad_z.data_ptr(), ptr_or_null(grad_A), ptr_or_null(grad_x), current_stream(dev)),
               "nm_spgemv_backward_planned");
     } else {
         check(nm_spgemv_backward(dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(),

@@ -185,6 +185,18 @@ class _TransposePlan:
         self.ready.record(torch.cuda.current_stream(dev))
         # `work` returns to torch's caching allocator, which hands it out again only to
         # work enqueued later on this same stream
+        self._shape, self._info = (rows, cols, nnz), None
+
+    def info(self, dev):
+        """The plan's figures (nm_csr_transpose_plan_info), fetched once: the call waits for the
+        stream."""
+        if self._info is None:
+            buf = (ctypes.c_int32 * 16)()
+            rows, cols, nnz = self._shape
+            _lib.check(_lib.lib().nm_csr_transpose_plan_info(rows, cols, nnz, _ptr(self.mem), buf, _stream(dev)),
+                       "nm_csr_transpose_plan_info")
+            self._info = list(buf)
+        return self._info
 
 
 def _fits_a_plan(rows, cols, nnz):
@@ -238,7 +250,10 @@ def spgemv_backward(grad_z, A_rows, A_cols, A_data, A_col_ind, A_rowptr, x):
         grad_x = torch.empty_like(x) if want_x else None
         if BACKWARD_MODE != "atomic" and _fits_a_plan(A_rows, x.shape[0], A_data.shape[0]):
             plan = _transpose_plan(A_col_ind, A_rowptr, A_rows, x.shape[0], dev)
-            _lib.check(_lib.lib().nm_spgemv_backward_planned(
+            # most blocks of 256 columns have a staging list: the build that stages g and x in LDS
+            lists = 2 * plan.info(dev)[5] >= (x.shape[0] + 255) // 256
+            entry = _lib.lib().nm_spgemv_backward_planned_lists if lists else _lib.lib().nm_spgemv_backward_planned
+            _lib.check(entry(
                 _dt(A_data), A_rows, x.shape[0], A_data.shape[0], _ptr(A_data), _ptr(plan.mem), _ptr(x),
                 _ptr(grad_z), _ptr(grad_A), _ptr(grad_x), _stream(dev)), "nm_spgemv_backward_planned")
             return [grad_A, grad_x]

@@ -112,6 +112,24 @@ def test_planned_spmv_packed_and_plain_structure(dev, dtype):
                 assert torch.equal(y, y_l), f"{name}: forward with and without staging lists"
                 _lib.check(L.nm_spgemv_backward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
                                                         ptr(gA), ptr(gx), stream), "nm_spgemv_backward_planned")
+                # the same for the backward: both builds, both gradients and each alone
+                for gA_want, gx_want in ((True, True), (True, False), (False, True)):
+                    gA_l = torch.full((nnz,), 7.0, dtype=D.dtype, device=dev) if gA_want else None
+                    gx_l = torch.full((cols,), 7.0, dtype=D.dtype, device=dev) if gx_want else None
+                    gA_p = torch.full((nnz,), 7.0, dtype=D.dtype, device=dev) if gA_want else None
+                    gx_p = torch.full((cols,), 7.0, dtype=D.dtype, device=dev) if gx_want else None
+                    _lib.check(L.nm_spgemv_backward_planned_lists(
+                        dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
+                        ptr(gA_l) if gA_want else None, ptr(gx_l) if gx_want else None, stream),
+                        "nm_spgemv_backward_planned_lists")
+                    _lib.check(L.nm_spgemv_backward_planned(
+                        dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
+                        ptr(gA_p) if gA_want else None, ptr(gx_p) if gx_want else None, stream),
+                        "nm_spgemv_backward_planned")
+                    if gA_want:
+                        assert torch.equal(gA_l, gA_p), f"{name}: grad_A with and without staging lists"
+                    if gx_want:
+                        assert torch.equal(gx_l, gx_p), f"{name}: grad_x with and without staging lists"
                 same = assert_same if exact else assert_close
                 same(host(y), y_ref, f"{name} y (wide={wide})")
                 assert_same(host(gA), gA_ref, f"{name} grad_A (wide={wide})")
