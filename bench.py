@@ -601,7 +601,8 @@ class SpGEMM(Workload):
                     ("grad_a_wide_kernel + grad_b_wide_kernel (both gradients on the product plan)" if wide else
                      "grad_ab_mapped_kernel (both gradients from one walk over A by column, on the product plan)",
                      self.backward, self.bwd_bytes_planned, "grad_b_wide_kernel" if wide else "grad_ab_mapped_kernel")]
-        return [(self.dominant_name, self.dominant, self.dominant_bytes, "numeric_front_kernel"),
+        return [(self.dominant_name, self.dominant, self.dominant_bytes,
+                 "numeric_hash_kernel" if self.left == "AA" or self.right == "AA" else "numeric_planned_kernel"),
                 ("spgemm_bwd_kernel (+ fill_kernel clearing grad_B)", self.backward, self.bwd_bytes_stateless,
                  "spgemm_bwd_kernel")]
 
@@ -641,7 +642,8 @@ class SpGEMM(Workload):
         # beyond a plan's limits): merge kernels where every row is short, the hash kernels otherwise
         hashed = self.left == "AA" or self.right == "AA"
         fwd_name = ("symbolic_hash_kernel + numeric_hash_kernel (row-binned LDS hash tables) + scans, host read of nnz(C)"
-                    if hashed else "symbolic_front_kernel + numeric_front_kernel (merge path) + scans, host read of nnz(C)")
+                    if hashed else "symbolic_front_kernel (merge path, recording where each product goes in scratch of the call) "
+                    "+ numeric_planned_kernel<COLS> (products added on those records) + scans, host read of nnz(C)")
         rec["roofline_stateless"] = {
             "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "kernels": [

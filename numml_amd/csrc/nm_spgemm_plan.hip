@@ -201,21 +201,82 @@ __global__ void plan_flag_out_kernel(const int32_t *flag, volatile int64_t *host
 // instruction per array -- and handed to the lanes that need it through LDS, where a read of
 // one address by eight lanes is a broadcast.
 
-// Row stride of the accumulators: one more than the row capacity, so that the eight rows of a
-// wavefront start in different LDS banks.
-constexpr int kAccStride = kRowCap + 1;
+// LDS per wavefront: its eight rows at kAccShort entries apart when none has more than half the
+// capacity, else four rows at a time, twice as far apart (see numeric_planned_kernel).
+constexpr int kAccShort = kRowCap / 2 + 1;
+
+// The rows of C that the groups of a wavefront have accumulated lie one behind the other in C
+// (consecutive rows), so the wavefront writes them as ONE span: lane l takes entries 2 l and
+// 2 l + 1 of the span (then + 128 ...), 16 bytes per lane and array, whole kilobytes per request.
+// Written row by row instead, every request is eight separate pieces of a row each; the stores of
+// the column indices alone were 140 us of the 519 us this kernel took on the 128^3 seven-point
+// product that way.  `clen`: entries of the lane's row, 0 for a row that is not part of this span
+// (past the end of the matrix, or of the other half of the wavefront); `first`: where the span
+// starts in C; the row of group q has its entries at acc + slot(q) (and its columns at ccol +
+// slot(q)), slot(q) = q * kAccShort, or (q % 4) * 2 * kAccShort when the halves take turns.
+template <typename T, bool COLS>
+__device__ __forceinline__ void store_wave_rows(const T *acc, const int32_t *ccol, int clen, int64_t first,
+                                                bool halves, T *__restrict__ C_data,
+                                                int64_t *__restrict__ C_indices) {
+    typedef T T2 __attribute__((ext_vector_type(2), aligned(sizeof(T))));
+    typedef int64_t L2 __attribute__((ext_vector_type(2), aligned(8)));
+    constexpr int kGroups = kWave / kCap;
+    // off[q]: entries in front of group q's row in the span; at[q] + j is where entry j of the span
+    // sits in LDS when it belongs to group q.  All wavefront-uniform.
+    int off[kGroups + 1], at[kGroups];
+    off[0] = 0;
+#pragma unroll
+    for (int q = 0; q < kGroups; ++q) {
+        off[q + 1] = off[q] + __builtin_amdgcn_readlane(clen, q * kCap);
+        at[q] = (halves ? (q & 3) * 2 * kAccShort : q * kAccShort) - off[q];
+    }
+    const int total = off[kGroups];
+    const int lane = threadIdx.x & (kWave - 1);
+    T *out = C_data + first;
+    int64_t *outc = COLS ? C_indices + first : nullptr;
+    for (int j = 2 * lane; j < total; j += 2 * kWave) {
+        int a0 = at[0], a1 = at[0];
+#pragma unroll
+        for (int q = 1; q < kGroups; ++q) {   // the last group that starts at or before the entry
+            a0 = j >= off[q] ? at[q] : a0;
+            a1 = j + 1 >= off[q] ? at[q] : a1;
+        }
+        if (j + 1 < total) {
+            T2 v;
+            v[0] = acc[a0 + j];
+            v[1] = acc[a1 + j + 1];
+            *reinterpret_cast<T2 *>(out + j) = v;
+            if (COLS) {
+                L2 c;
+                c[0] = (int64_t)ccol[a0 + j];
+                c[1] = (int64_t)ccol[a1 + j + 1];
+                *reinterpret_cast<L2 *>(outc + j) = c;
+            }
+        } else {
+            out[j] = acc[a0 + j];
+            if (COLS) outc[j] = (int64_t)ccol[a0 + j];
+        }
+    }
+}
 
 // COLS: the pattern of C is not there yet (the product is being computed for the first time, on the
 // destination bytes the symbolic phase left behind): every product also drops its column beside its
 // accumulator, the columns are written out with the values, and cstart is filled in.
+//
+// The kernel waits on memory (row pointers, then the row's entries of A and their records, then the
+// rows of B: three round trips a wavefront), so what decides its speed is how many wavefronts a CU
+// holds, and that is decided by the accumulators in LDS.  They are sized for rows of C of at most
+// kRowCap / 2 entries; a wavefront that has a longer row (wavefronts synchronise with nobody) takes
+// its eight rows four at a time, each with room for kRowCap entries.
 template <typename T, bool COLS>
 __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     int64_t rows, int64_t ntiles_padded, const T *__restrict__ A_data, const int64_t *__restrict__ A_indptr,
     const T *__restrict__ B_data, const int64_t *__restrict__ B_indices, const int32_t *__restrict__ bstart,
     const uint8_t *__restrict__ dest, const int64_t *__restrict__ C_indptr, T *__restrict__ C_data,
     int64_t *__restrict__ C_indices, int32_t *__restrict__ cstart, const uint32_t *__restrict__ rec) {
-    __shared__ T s_acc[kGroupsPerBlock * kAccStride];
-    __shared__ int32_t s_ccol[COLS ? kGroupsPerBlock * kAccStride : 1];
+    static_assert(2 * kAccShort >= kRowCap + 1 && (kWave / kCap) % 2 == 0, "half the rows at twice the stride");
+    __shared__ T s_acc[kGroupsPerBlock * kAccShort];
+    __shared__ int32_t s_ccol[COLS ? kGroupsPerBlock * kAccShort : 1];
     __shared__ T s_av[kBlock];                       // per group: the row's entries of A ...
     __shared__ int32_t s_bs[kBlock];                 // ... where their rows of B start ...
     __shared__ __align__(8) uint8_t s_db[kBlock * kCap];   // ... and their destination bytes
@@ -227,10 +288,6 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
     const int64_t cs = pc.lo;
     const int clen = live ? (int)(pc.hi - cs) : 0;
     const int alen = (int)(ae - ab);
-    T *acc = s_acc + g * kAccStride;
-#pragma unroll
-    for (int q = 0; q < kCap; ++q)
-        if (k + kCap * q < clen) acc[k + kCap * q] = T(0);
     {   // lane k of the group fetches entry k of the row
         const int64_t e = k < alen ? ab + k : 0;   // entry 0: readable whenever the matrix has entries
         const T av = A_data[e];
@@ -261,43 +318,39 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
         bv[a] = B_data[at];
         if (COLS) bc[a] = *reinterpret_cast<const int32_t *>(B_indices + at);   // columns fit 31 bits
     }
-    int32_t *ccol = s_ccol + (COLS ? g * kAccStride : 0);
+    constexpr int kWaveGroups = kWave / kCap;
+    const int wave_first = (threadIdx.x / kWave) * kWaveGroups;   // the wavefront's first group
+    const int gq = g - wave_first;
+    const bool halves = __ballot(clen > kRowCap / 2) != 0;        // wavefront-uniform
+    T *wave_acc = s_acc + wave_first * kAccShort;
+    int32_t *wave_ccol = s_ccol + (COLS ? wave_first * kAccShort : 0);
+    const int mine = halves ? (gq & 3) * 2 * kAccShort : gq * kAccShort;
+    T *acc = wave_acc + mine;
+    int32_t *ccol = wave_ccol + (COLS ? mine : 0);
+    for (int pass = 0; pass < (halves ? 2 : 1); ++pass) {
+        const bool on = !halves || (gq >> 2) == pass;
+        if (on) {
 #pragma unroll
-    for (int a = 0; a < kCap; ++a) {
-        // the lanes of a group hold different entries of one B row: different columns, different
-        // accumulators; the entries of A take their turns one after the other
-        if (db[a] != kNone) {
-            acc[db[a]] = acc[db[a]] + s_av[slot + a] * bv[a];
-            if (COLS) ccol[db[a]] = bc[a];   // every product of an entry of C brings the same column
+            for (int q = 0; q < kCap; ++q)
+                if (k + kCap * q < clen) acc[k + kCap * q] = T(0);
         }
         group_fence();
-    }
-    if (COLS) {
 #pragma unroll
-        for (int q = 0; q < kCap; ++q)
-            if (k + kCap * q < clen) {
-                C_data[cs + k + kCap * q] = acc[k + kCap * q];
-                C_indices[cs + k + kCap * q] = (int64_t)ccol[k + kCap * q];
+        for (int a = 0; a < kCap; ++a) {
+            // the lanes of a group hold different entries of one B row: different columns, different
+            // accumulators; the entries of A take their turns one after the other
+            if (on && db[a] != kNone) {
+                acc[db[a]] = acc[db[a]] + s_av[slot + a] * bv[a];
+                if (COLS) ccol[db[a]] = bc[a];   // every product of an entry of C brings the same column
             }
-    } else {
-        // W consecutive entries (16 bytes) per lane and request: a half or a quarter of the store
-        // instructions (256 -> 276 us without at cfg4)
-        constexpr int W = 16 / (int)sizeof(T);
-        typedef T VW __attribute__((ext_vector_type(W), aligned(sizeof(T))));
-#pragma unroll
-        for (int q = 0; q < kRowCap / (kCap * W); ++q) {
-            const int at = W * k + W * kCap * q;
-            if (at + W <= clen) {
-                VW v;
-#pragma unroll
-                for (int w = 0; w < W; ++w) v[w] = acc[at + w];
-                *reinterpret_cast<VW *>(C_data + cs + at) = v;
-            } else {
-#pragma unroll
-                for (int w = 0; w < W; ++w)
-                    if (at + w < clen) C_data[cs + at + w] = acc[at + w];
-            }
+            group_fence();
         }
+        // (the last fence above has made every group's sums visible to the whole wavefront)
+        const int from = halves && pass == 1 ? kWave / 2 : 0;   // the lane whose row starts the span
+        const int64_t first = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)cs, from) |
+                              ((int64_t)__builtin_amdgcn_readlane((int)(cs >> 32), from) << 32);
+        store_wave_rows<T, COLS>(wave_acc, wave_ccol, on ? clen : 0, first, halves, C_data, C_indices);
+        group_fence();   // the other half's turn overwrites these accumulators
     }
 }
 

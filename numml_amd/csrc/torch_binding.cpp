@@ -1142,14 +1142,15 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
     const auto iopt = torch::TensorOptions().dtype(torch::kInt64).device(dev);
     Tensor C_indptr = torch::empty({(int64_t)A_rows + 1}, iopt);
     nm_stream st = current_stream(dev);
-    // Unless plans are switched off, the symbolic merge records where every product goes (16 bytes
-    // per entry of A): with no row on the hash path the numeric phase then adds the products up on
-    // those records instead of merging the rows again, and the records are a product plan's.
+    // The symbolic merge records where every product goes (16 bytes per entry of A, scratch of this
+    // call): with no row on the hash path the numeric phase then adds the products up on those
+    // records instead of merging the rows again (cheaper than the second merge whether or not
+    // anything is kept), and unless plans are switched off the records become a product plan's.
     const int64_t A_nnz = A_data.numel(), B_nnz = B_data.numel();
     const int64_t lim31 = (int64_t)1 << 31;
     Tensor filled;
     size_t pbytes = 0;
-    if (plans && A_nnz > 0 && A_nnz < lim31 && B_nnz < lim31) {
+    if (A_nnz > 0 && A_nnz < lim31 && B_nnz < lim31) {
         check(nm_spgemm_plan_bytes(A_nnz, &pbytes), "nm_spgemm_plan_bytes");
         filled = scratch(pbytes, dev);
         check(nm_spgemm_symbolic_mapped(A_rows, A_cols, B_cols, A_nnz, B_nnz, A_indices.data_ptr<int64_t>(),
@@ -1187,7 +1188,7 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
           "nm_spgemm_numeric_mapped");
     // note the pair, or make its plan: from the memory this pass filled, or (rows on the hash
     // path: the plan's own analysis says whether the product is within its limits) from the patterns
-    if (on_map)
+    if (on_map && plans)
         consider_product_plan(A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr, A_rows, A_cols, B_cols,
                               dev, filled);
     else if (plans && nnz_c > 0)
