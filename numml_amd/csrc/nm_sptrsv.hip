@@ -49,7 +49,7 @@ struct Packed {        // one solve direction, level-major (all int32, device)
     int32_t *dslot;    // [nnz]    slot of the row a dependency refers to
     int32_t *dsrc;     // [nnz]    position of its coefficient in A's data
     int32_t *diag;     // [rows]   position of the diagonal coefficient, -1 when not stored
-    int32_t *ell_ds;   // [ell_capacity] fixed-width dependency entries, `pre` per row (ring byte offset | far bit)
+    int32_t *ell_ds;   // [ell_capacity] room for the fixed-width dependency entries: 16 bits each, `pre` per row
     int32_t *lvl_sig;  // [levels] which neighbouring wavefronts the rows of a level wait for (kSigLower | kSigHigher)
 };
 // Entries of the fixed-width (ELLPACK) arrays; the layout is used when (rows + kEllPad) * pre
@@ -636,15 +636,22 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_group_kernel(SolveArgs a, int 
 // which matters because the workgroup's wavefronts share one CU and the level time
 // is the time to issue their instructions.
 
-// An entry of the fixed-width dependency array is what the level needs and nothing else: the
-// BYTE offset of the dependency's solution in the LDS ring (bits 0..16), and bit 20 when the
-// ring of this launch cannot serve it (the row was solved by another launch, or too many slots
-// ago; the rare slow path then finds the slot in the range-based arrays).  An absent dependency
-// points at ring entry kRing, which holds 0.0 for ever, and its coefficient is 0.0: it adds
-// +0.0 to the sum, so the level needs no "is there a dependency" test at all.  Deciding all
-// this once, at plan time, keeps a dozen instructions per dependency out of every level.
-constexpr int32_t kEllFar = 1 << 20;
-constexpr int32_t kEllOffsetMask = (1 << 17) - 1;
+// An entry of the fixed-width dependency array is what the level needs and nothing else, in 16
+// bits: twice the number of the dependency's entry in the LDS ring (four times that is its byte
+// offset there), plus 1 when the ring of this launch cannot serve it (the row was solved by
+// another launch, or too many slots ago; the rare slow path then finds the slot in the
+// range-based arrays).  An absent dependency points at ring entry kRing, which holds 0.0 for
+// ever, and its coefficient is 0.0: it adds +0.0 to the sum, so the level needs no "is there a
+// dependency" test at all.  Deciding all this once, at plan time, keeps a dozen instructions per
+// dependency out of every level.  (Two bytes, not four: everything a row needs passes through
+// the ONE compute unit the workgroup lives on, at the ~110 GB/s that unit can stream -- 44
+// instead of 48 bytes a row were 0.97 -> 0.88 ms per solve on the 1024^2 triangle.)
+constexpr uint32_t kEllFarPair = 0x00010001u;       // the "not in the ring" bits of a pair of entries
+constexpr uint32_t kEllByteMask = 0x3fff8u;         // byte offset in the ring, once the entry is shifted in place
+static_assert(kRing * 2 + 1 < 65536 && (kRing * 8 & ~kEllByteMask) == 0, "a ring entry number fits 15 bits");
+__device__ __forceinline__ uint32_t ell_ring_bytes(uint32_t pair, int e) {
+    return (e & 1) ? (pair >> 14) & kEllByteMask : (pair << 2) & kEllByteMask;
+}
 
 __device__ __forceinline__ int32_t level_of_slot(const int32_t *__restrict__ level_ptr, int32_t nlevels, int32_t q) {
     int32_t lo = 0, hi = nlevels;   // last l with level_ptr[l] <= q
@@ -658,7 +665,7 @@ __device__ __forceinline__ int32_t level_of_slot(const int32_t *__restrict__ lev
 __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict__ dptr,
                                 const int32_t *__restrict__ dslot, const int32_t *__restrict__ level_ptr,
                                 int32_t nlevels, const int32_t *__restrict__ level_launch,
-                                int32_t *__restrict__ ell_ds, int32_t *__restrict__ reach,
+                                uint16_t *__restrict__ ell_ds, int32_t *__restrict__ reach,
                                 int32_t *__restrict__ lvl_sig) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     // the padding slots behind the last row get "absent" entries: lanes that read them must find a valid offset
@@ -666,14 +673,14 @@ __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict
         const int64_t q = i / pre;
         const int e = (int)(i - q * pre);
         const int32_t lo = q < rows ? dptr[q] : 0, n = q < rows ? dptr[q + 1] - lo : 0;
-        int32_t out = kRing * 8;   // absent: the ring entry that is always 0.0
+        uint32_t out = kRing * 2;   // absent: the ring entry that is always 0.0
         if (e < n) {
             const int32_t ds = dslot[lo + e];
             const int32_t dist = ds > (int32_t)q ? ds - (int32_t)q : (int32_t)q - ds;
             const int32_t lq = level_of_slot(level_ptr, nlevels, (int32_t)q), ld = level_of_slot(level_ptr, nlevels, ds);
             const bool same = level_launch[lq] == level_launch[ld];
             const bool near = same && dist < kRingSafe;
-            out = ((ds & (kRing - 1)) * 8) | (near ? 0 : kEllFar);
+            out = ((uint32_t)(ds & (kRing - 1)) * 2) | (near ? 0u : 1u);
             if (near) {
                 // wavefront of the row and of the row it waits for, each inside its own level
                 const int32_t wq = ((int32_t)q - level_ptr[lq]) >> 6, wd = (ds - level_ptr[ld]) >> 6;
@@ -686,7 +693,7 @@ __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict
                 if (bit && (lvl_sig[lq] & bit) == 0) atomicOr(lvl_sig + lq, bit);
             }
         }
-        ell_ds[i] = out;
+        ell_ds[i] = (uint16_t)out;
     }
 }
 
@@ -713,7 +720,8 @@ __global__ void gather_ell_kernel(int64_t rows, int pre, const T *__restrict__ d
 }
 
 struct EllArgs {
-    const int32_t *level_ptr, *ell_ds, *dptr, *dslot, *lvl_sig;
+    const int32_t *level_ptr, *dptr, *dslot, *lvl_sig;
+    const uint16_t *ell_ds;
     const double *ell_coef, *rb;
     double *xs;
     int unit;
@@ -725,7 +733,7 @@ struct EllArgs {
 // compute a value that is never stored.
 template <int PRE> struct EllVals {
     int qb, qe;
-    int32_t ds[PRE];
+    uint32_t ds[PRE / 2];   // pairs of 16-bit dependency entries
     double v[PRE];
     double bv, dv;
 };
@@ -734,10 +742,9 @@ template <int PRE> struct EllVals {
 // claims to read and write them): used to keep copies between stages in front of the next request.
 template <int PRE> __device__ __forceinline__ void settle(EllVals<PRE> &v) {
 #pragma unroll
-    for (int e = 0; e < PRE; ++e) {
-        asm volatile("" : "+v"(v.ds[e]));
-        asm volatile("" : "+v"(v.v[e]));
-    }
+    for (int e = 0; e < PRE / 2; ++e) asm volatile("" : "+v"(v.ds[e]));
+#pragma unroll
+    for (int e = 0; e < PRE; ++e) asm volatile("" : "+v"(v.v[e]));
     asm volatile("" : "+v"(v.bv));
     asm volatile("" : "+v"(v.dv));
 }
@@ -749,26 +756,26 @@ __device__ __forceinline__ Bounds load_bounds_uniform(const int32_t *s_lp, int i
 }
 
 template <int PRE> __device__ __forceinline__ EllVals<PRE> load_ell(const EllArgs &a, const Bounds &b) {
-    typedef int32_t IV __attribute__((ext_vector_type(PRE)));
+    static_assert(PRE % 2 == 0, "dependency entries come in pairs");
+    typedef uint32_t IV __attribute__((ext_vector_type(PRE / 2)));
     typedef double DV __attribute__((ext_vector_type(PRE)));
     typedef double D2 __attribute__((ext_vector_type(2)));
     EllVals<PRE> v;
     v.qb = b.qb;
     v.qe = b.qe;
-    const uint32_t lane_ds = threadIdx.x * (uint32_t)(sizeof(int32_t) * PRE);
+    const uint32_t lane_ds = threadIdx.x * (uint32_t)(sizeof(uint16_t) * PRE);
     const uint32_t lane_cf = threadIdx.x * (uint32_t)(sizeof(double) * PRE);
     const uint32_t lane_rb = threadIdx.x * (uint32_t)(sizeof(double) * 2);
-    const char *pd = reinterpret_cast<const char *>(a.ell_ds) + (int64_t)b.qb * (int64_t)(sizeof(int32_t) * PRE);
+    const char *pd = reinterpret_cast<const char *>(a.ell_ds) + (int64_t)b.qb * (int64_t)(sizeof(uint16_t) * PRE);
     const char *pc = reinterpret_cast<const char *>(a.ell_coef) + (int64_t)b.qb * (int64_t)(sizeof(double) * PRE);
     const char *pr = reinterpret_cast<const char *>(a.rb) + (int64_t)b.qb * (int64_t)(sizeof(double) * 2);
     const IV dsv = *reinterpret_cast<const IV *>(pd + lane_ds);
     const DV cv = *reinterpret_cast<const DV *>(pc + lane_cf);
     const D2 r = *reinterpret_cast<const D2 *>(pr + lane_rb);
 #pragma unroll
-    for (int e = 0; e < PRE; ++e) {
-        v.ds[e] = dsv[e];
-        v.v[e] = cv[e];
-    }
+    for (int e = 0; e < PRE / 2; ++e) v.ds[e] = dsv[e];
+#pragma unroll
+    for (int e = 0; e < PRE; ++e) v.v[e] = cv[e];
     v.bv = r[0];
     v.dv = r[1];
     return v;
@@ -868,18 +875,18 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
     auto level = [&](int it, const EllVals<PRE> &cur) {
         // all ring reads go out together, unconditionally
         double xj[PRE];
-        int32_t any = 0;
+        uint32_t any = 0;
 #pragma unroll
         for (int e = 0; e < PRE; ++e) {
-            xj[e] = *reinterpret_cast<const double *>(ring_bytes + (cur.ds[e] & kEllOffsetMask));
-            any |= cur.ds[e];
+            xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
+            any |= cur.ds[e / 2];
         }
         ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
         double acc = 0.;
 #pragma unroll
         for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
         const bool live = (int)threadIdx.x < cur.qe - cur.qb;
-        if ((any & kEllFar) && live) {
+        if ((any & kEllFarPair) && live) {
             // a dependency the ring does not hold: redo the sum in the same order from global memory
             // (slots and then solutions are requested together; entries past the row's own
             //  name a valid slot and are not added)
@@ -915,19 +922,22 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
                 qv[d] = load_ell<PRE>(a, ahead);
 
                 // all ring reads go out together, unconditionally
+                // (unpacking the offsets one level early, in the shadow of that level's ring reads,
+                // was slower, 0.92 -> 1.12 ms: state carried from level to level makes the compiler
+                // wait for the operand request just issued)
                 double xj[PRE];
-                int32_t any = 0;
+                uint32_t any = 0;
 #pragma unroll
                 for (int e = 0; e < PRE; ++e) {
-                    xj[e] = *reinterpret_cast<const double *>(ring_bytes + (cur.ds[e] & kEllOffsetMask));
-                    any |= cur.ds[e];
+                    xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
+                    any |= cur.ds[e / 2];
                 }
                 ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
                 double acc = 0.;
 #pragma unroll
                 for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
                 const bool live = (int)threadIdx.x < cur.qe - cur.qb;
-                if ((any & kEllFar) && live) {
+                if ((any & kEllFarPair) && live) {
                     // a dependency the ring does not hold: redo the sum in the same order from global memory
                     // (slots and then solutions are requested together; entries past the row's own
                     //  name a valid slot and are not added)
@@ -1320,7 +1330,8 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     }
     const int dirn = transposed ? 1 : 0;
     const int pre = p->ell_pre[dirn];
-    EllArgs ea{p->level_ptr, P.ell_ds, P.dptr, P.dslot, P.lvl_sig, a.w.ell_coef, a.w.rb, a.w.xs, unit};
+    EllArgs ea{p->level_ptr, P.dptr, P.dslot, P.lvl_sig, reinterpret_cast<const uint16_t *>(P.ell_ds), a.w.ell_coef,
+               a.w.rb, a.w.xs, unit};
     if (pre > 0) {
         int64_t grid = nm::ceil_div(p->rows * pre, kBlock);
         if (grid > 65536) grid = 65536;
@@ -1743,7 +1754,8 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             if (grid > 65536) grid = 65536;
             if (int rc = nm::fill_async(p->dir[d].lvl_sig, (int64_t)p->nlevels + 1, (int32_t)0, s)) return bail(rc);
             hipLaunchKernelGGL(ell_pack_kernel, dim3((unsigned)grid), dim3(kBlock), 0, s, rows, pre, p->dir[d].dptr,
-                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, p->dir[d].ell_ds,
+                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch,
+                               reinterpret_cast<uint16_t *>(p->dir[d].ell_ds),
                                L.meta + 4 + d, p->dir[d].lvl_sig);
             if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
         }
