@@ -1074,6 +1074,21 @@ def ref_timing(dev, cpu_seconds):
         cpu_op(lambda: (oracle.spgemv_forward(N, N, d, i, p, x_h),
                         oracle.spgemv_backward(ones, N, N, d, i, p, x_h)), 1000))
 
+    # What torch itself takes for the same protocol around a custom Function that does nothing (one
+    # autograd node, `.sum().backward()`, gradient accumulated into a leaf): the floor under every
+    # "Backward" row here, whatever the kernels cost.
+    class _Twice(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, v):
+            return v * 2
+
+        @staticmethod
+        def backward(ctx, gv):
+            return gv * 2
+
+    add("autograd floor (identity-like Function, .sum().backward(), no sparse kernel)", N, 1000,
+        time_op(lambda: _Twice.apply(x).sum().backward(), 1000), 0.0)
+
     # SpSpMM and SpDMM, tridiagonal A, B = -A, N = 16 384, 2 iterations (:264-348)
     N = 16_384
     A, (d, i, p) = csr(G.tridiag(N, f32))

@@ -36,7 +36,7 @@ def test_cfg1_spmv_fp64_poisson256_autograd(dev):
     assert A.grad.shape == (rows, cols) and A.grad.nnz == d.shape[0]
 
 
-@pytest.mark.parametrize("mode", ["eager", "atomic"])
+@pytest.mark.parametrize("mode", ["eager", "atomic", "planned"])
 def test_cfg2_spmv_fp32_poisson2048(dev, mode):
     d, i, p, (rows, cols) = G.poisson2d(2048, np.float32, jitter_seed=0)
     assert rows == 4194304 and d.shape[0] == 20963328
@@ -56,16 +56,24 @@ def test_cfg2_spmv_fp32_poisson2048(dev, mode):
     if mode == "eager":
         assert_same(host(gx), gx_ref, "grad_x (bitwise)")
         assert torch.equal(gx, gx2) and torch.equal(gA, gA2)       # run-to-run identical
+    if mode == "planned":
+        # the default mode: the first backward on the pattern ran the stateless kernels (atomic
+        # sums, tolerance above); the second sighting built the plan and is the CPU loop's sum
+        assert_same(host(gx2), gx_ref, "grad_x of the second backward (bitwise)")
+        assert_same(host(gA2), gA_ref, "grad_A of the second backward")
+        gA3, gx3 = ext.spgemv_backward(Gv, rows, cols, D, I, P, X)
+        assert torch.equal(gx3, gx2) and torch.equal(gA3, gA2)
     # adjoint identity <A x, g> = <x, A^T g> in double
     lhs = float(host(y).astype(np.float64) @ g.astype(np.float64))
     rhs = float(host(gx).astype(np.float64) @ x.astype(np.float64))
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
 
 
-@pytest.mark.parametrize("mode", ["eager", "atomic"])
+@pytest.mark.parametrize("mode", ["eager", "atomic", "planned"])
 def test_cfg3_spmm_fp32_powerlaw(dev, mode):
     """eager: the fused kernel on the plan (what the benchmark times); atomic: the stateless
-    kernels, which the default mode runs on the first backward of a pattern."""
+    kernels; planned (the default): stateless on the first backward of the pattern, on the plan from
+    the second (the single-gradient calls at the end)."""
     rows = cols = 1_000_000
     n = 64
     d, i, p, _ = G.powerlaw(rows, cols, target_nnz=16_000_000, seed=0, dtype=np.float32)
