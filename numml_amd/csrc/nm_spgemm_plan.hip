@@ -213,10 +213,10 @@ constexpr int kAccShort = kRowCap / 2 + 1;
 // product that way.  `clen`: entries of the lane's row, 0 for a row that is not part of this span
 // (past the end of the matrix, or of the other half of the wavefront); `first`: where the span
 // starts in C; the row of group q has its entries at acc + slot(q) (and its columns at ccol +
-// slot(q)), slot(q) = q * kAccShort, or (q % 4) * 2 * kAccShort when the halves take turns.
+// slot(q)), slot(q) = q * stride, or (q % 4) * 2 * stride when the halves take turns.
 template <typename T, bool COLS>
 __device__ __forceinline__ void store_wave_rows(const T *acc, const int32_t *ccol, int clen, int64_t first,
-                                                bool halves, T *__restrict__ C_data,
+                                                int stride, bool halves, T *__restrict__ C_data,
                                                 int64_t *__restrict__ C_indices) {
     typedef T T2 __attribute__((ext_vector_type(2), aligned(sizeof(T))));
     typedef int64_t L2 __attribute__((ext_vector_type(2), aligned(8)));
@@ -228,7 +228,7 @@ __device__ __forceinline__ void store_wave_rows(const T *acc, const int32_t *cco
 #pragma unroll
     for (int q = 0; q < kGroups; ++q) {
         off[q + 1] = off[q] + __builtin_amdgcn_readlane(clen, q * kCap);
-        at[q] = (halves ? (q & 3) * 2 * kAccShort : q * kAccShort) - off[q];
+        at[q] = (halves ? (q & 3) * 2 * stride : q * stride) - off[q];
     }
     const int total = off[kGroups];
     const int lane = threadIdx.x & (kWave - 1);
@@ -257,6 +257,17 @@ __device__ __forceinline__ void store_wave_rows(const T *acc, const int32_t *cco
             if (COLS) outc[j] = (int64_t)ccol[a0 + j];
         }
     }
+}
+
+// The rows of the wavefront's groups, `stride` apart from `wave_acc` on, as one span (every lane of
+// the wavefront must get here; cs: where the lane's row starts in C).
+template <typename T>
+__device__ __forceinline__ void store_wave_span(const T *wave_acc, int stride, int clen, int64_t cs,
+                                                T *__restrict__ C_data) {
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    const int64_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)cs) |
+                          ((int64_t)__builtin_amdgcn_readfirstlane((int)(cs >> 32)) << 32);
+    store_wave_rows<T, false>(wave_acc, nullptr, clen, first, stride, false, C_data, nullptr);
 }
 
 // COLS: the pattern of C is not there yet (the product is being computed for the first time, on the
@@ -349,28 +360,8 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
         const int from = halves && pass == 1 ? kWave / 2 : 0;   // the lane whose row starts the span
         const int64_t first = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)cs, from) |
                               ((int64_t)__builtin_amdgcn_readlane((int)(cs >> 32), from) << 32);
-        store_wave_rows<T, COLS>(wave_acc, wave_ccol, on ? clen : 0, first, halves, C_data, C_indices);
+        store_wave_rows<T, COLS>(wave_acc, wave_ccol, on ? clen : 0, first, kAccShort, halves, C_data, C_indices);
         group_fence();   // the other half's turn overwrites these accumulators
-    }
-}
-
-// A row of C from its accumulators in LDS, by the eight lanes of its group: 16 bytes per lane and
-// request (a half or a quarter of the store instructions of one entry per lane).
-template <typename T>
-__device__ __forceinline__ void store_row(T *__restrict__ out, const T *acc, int clen, int k) {
-    constexpr int W = 16 / (int)sizeof(T);
-    typedef T VW __attribute__((ext_vector_type(W), aligned(sizeof(T))));
-    for (int at = W * k; at < clen; at += W * kCap) {
-        if (at + W <= clen) {
-            VW v;
-#pragma unroll
-            for (int w = 0; w < W; ++w) v[w] = acc[at + w];
-            *reinterpret_cast<VW *>(out + at) = v;
-        } else {
-#pragma unroll
-            for (int w = 0; w < W; ++w)
-                if (at + w < clen) out[at + w] = acc[at + w];
-        }
     }
 }
 
@@ -428,7 +419,7 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_long
             group_fence();
         }
     }
-    store_row(C_data + cs, acc, clen, k);
+    store_wave_span(s_acc + (threadIdx.x / kWave) * (kWave / kCap) * S::kStride, S::kStride, clen, cs, C_data);
 }
 
 // The same for products whose named rows of B have up to 8 * OCT entries (classes 4 and 5): an entry
@@ -486,7 +477,7 @@ __global__ __launch_bounds__(LongShape<CAP>::kThreads) void numeric_planned_wide
             }
         }
     }
-    store_row(C_data + cs, acc, clen, k);
+    store_wave_span(s_acc + (threadIdx.x / kWave) * (kWave / kCap) * S::kStride, S::kStride, clen, cs, C_data);
 }
 
 // ---- backward ------------------------------------------------------------------------
