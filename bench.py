@@ -266,6 +266,9 @@ class SpMV(Workload):
             if st_r == n_r and 4096 // max(mean, 1) >= 512 and i_fwd > 2:
                 i_fwd = 2               # every block has a list: 16-bit places whatever the offsets are
                 self.fwd_bytes = _spmv_bytes(rows, cols, self.nnz, s, i_fwd, i_bwd, planned=True)[0]
+            if pk_b and i_bwd > 4:
+                i_bwd = 4               # blocks with a list keep 21 bits of distance in the packed word
+                self.bwd_bytes = _spmv_bytes(rows, cols, self.nnz, s, i_fwd, i_bwd, planned=True)[1]
             if 4096 // max(mean, 1) >= 512:
                 self.fwd_bytes += 64 * st_r
             self.bwd_bytes += 64 * st_c

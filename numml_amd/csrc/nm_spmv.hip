@@ -703,13 +703,13 @@ __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, 
     T dq[4], de[ER > 0 ? ER : 1];
     if (QUAD) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) dq[q] = *at<O32>(data, base + tid * 4 + q + (wq[q] >> 16));
+        for (int q = 0; q < 4; ++q) dq[q] = *at<O32>(data, base + tid * 4 + q + (wq[q] >> nm::kStagePlaceBits));
     }
 #pragma unroll
     for (int r = 0; r < ER; ++r) {
         const int k = kQuads + r * kBlock + tid;
         const int kc = k < n ? k : n - 1;
-        de[r] = *at<O32>(data, base + kc + (we[r] >> 16));
+        de[r] = *at<O32>(data, base + kc + (we[r] >> nm::kStagePlaceBits));
     }
     *reinterpret_cast<TV *>(s_g + 4 * tid) = gs0;
     *reinterpret_cast<TV *>(s_x + 4 * tid) = xs0;
@@ -729,7 +729,7 @@ __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, 
         TV out, nv;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int li = wq[q] & 0xffff;
+            const int li = wq[q] & ((1 << nm::kStagePlaceBits) - 1);
             out[q] = sv[q] * s_x[li];
             nv[q] = s_g[li] * dq[q];
         }
@@ -740,7 +740,7 @@ __device__ __forceinline__ void bwd_tile_staged(const int64_t c0, const int nc, 
     for (int r = 0; r < ER; ++r) {
         const int k = kQuads + r * kBlock + tid;
         if (k < n) {
-            const int li = we[r] & 0xffff;
+            const int li = we[r] & ((1 << nm::kStagePlaceBits) - 1);
             *at<O32>(grad_A, base + k) = s_v[k] * s_x[li];
             s_v[k] = s_g[li] * de[r];
         }
@@ -839,6 +839,9 @@ __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? (LISTS ? 6 : 8) : (LISTS ? 3
                 __syncthreads();
                 continue;
             }
+            // (a block with a list always has the entries that test asks for; were it ever not so,
+            // its words must not be read as row offsets)
+            if (d0 >= 0) packed = false;
         }
         // Lane t holds the bounds of column c0 + t and its own factor; all three loads leave
         // together (one memory round trip before the tile's entries can be read).
@@ -1051,8 +1054,8 @@ __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? (LISTS ? 6 : 8) : (LISTS ? 3
                 int32_t k, r;
                 if (packed) {
                     const int32_t w = nm::stream_load(t_pack + first + p);
-                    k = first + p + (w >> 16);
-                    r = (STAGE && staged) ? (w & 0xffff) : (int32_t)c0 + (int16_t)w;
+                    k = first + p + ((STAGE && staged) ? w >> nm::kStagePlaceBits : w >> 16);
+                    r = (STAGE && staged) ? (w & ((1 << nm::kStagePlaceBits) - 1)) : (int32_t)c0 + (int16_t)w;
                 } else {
                     k = nm::stream_load(tp + p);
                     r = nm::stream_load(tr + p);

@@ -413,9 +413,15 @@ __global__ __launch_bounds__(kBlock) void tp_pack_kernel(
             const bool active = p < pe;
             const int32_t r = active ? t_row[p] : 0;
             const int64_t dr = (int64_t)r - c0, dk = active ? (int64_t)t_perm[p] - p : 0;
-            fits_t &= !active || (dr >= -32768 && dr <= 32767 && dk >= -32768 && dk <= 32767);
-            const uint32_t low = staged && active ? (uint32_t)stage_place(table, r) : ((uint32_t)dr & 0xffffu);
-            if (active) t_pack[p] = (int32_t)(low | ((uint32_t)dk << 16));
+            constexpr int64_t kFar = int64_t(1) << (31 - nm::kStagePlaceBits);
+            if (staged) {   // place | distance, see kStagePlaceBits
+                fits_t &= !active || (dk >= -kFar && dk < kFar);
+                if (active)
+                    t_pack[p] = (int32_t)((uint32_t)stage_place(table, r) | ((uint32_t)dk << nm::kStagePlaceBits));
+            } else {
+                fits_t &= !active || (dr >= -32768 && dr <= 32767 && dk >= -32768 && dk <= 32767);
+                if (active) t_pack[p] = (int32_t)(((uint32_t)dr & 0xffffu) | ((uint32_t)dk << 16));
+            }
         }
         __syncthreads();
     }

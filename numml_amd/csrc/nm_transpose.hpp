@@ -15,8 +15,10 @@
 //                arrays the interface delivers: half the index traffic)
 //   t_pack[p]    t_row and t_perm of entry p in one word, for patterns whose entries lie near
 //                the diagonal: low 16 bits = t_row[p] minus the first column of the entry's
-//                block of kPackCols columns, high 16 bits = t_perm[p] - p, both signed.
-//                Valid when flags[1] != 0 (every difference fits)                (nnz)
+//                block of kPackCols columns, high 16 bits = t_perm[p] - p, both signed.  In a
+//                block of columns that has a staging list (b_desc): low kStagePlaceBits bits =
+//                the entry's place among the listed segments, the bits above = t_perm[p] - p.
+//                Valid when flags[1] != 0 (every difference fits its block's layout)  (nnz)
 //   c_off16[k]   c_idx32[k] minus the first row of the entry's block of kPackRows rows, signed
 //                16 bits.  Valid when flags[2] != 0                              (nnz)
 //                (the SpMV kernels read these instead of the 32-bit arrays: half the index
@@ -31,8 +33,8 @@
 //                by the end of x, more entries than a tile holds); c_off16 is as described above
 //   b_desc[b]    the same for the b-th block of kPackCols columns and the ROWS its entries lie
 //                in (up to kStageBwd segments); such a block keeps the place in the list in the
-//                low half of t_pack[p].  Only read when flags[1] != 0; blocks of fewer than
-//                kStageBwdMin entries get none
+//                low bits of t_pack[p] (above).  Only read when flags[1] != 0; blocks of fewer
+//                than kStageBwdMin entries get none
 //
 // Inside a column the entries keep A's row-major order (the sort is stable), so
 // rows ascend, exactly like the counting-sort transpose of the reference
@@ -66,6 +68,12 @@ constexpr int kPackCols = 256, kPackRows = 512;
 constexpr int kStageSeg = 128, kStageFwd = 16, kStageBwd = 12, kStageDesc = 16;
 // Entries a block may hold to get a list: the LDS tiles of the kernels that use it.
 constexpr int kStageFwdCap = 4096, kStageBwdCap = 2048, kStageBwdMin = 1024;
+// A packed word of a block of columns WITH a list: the entry's place among the listed segments in
+// the low kStagePlaceBits bits, t_perm[p] - p in the 32 - kStagePlaceBits above (a place needs
+// fewer bits than a row offset, and the distance may then be sixteen times as far: the mirror
+// entries of a 128^3 seven-point pattern lie 115 000 positions apart).
+constexpr int kStagePlaceBits = 11;
+static_assert(kStageBwd * kStageSeg <= (1 << kStagePlaceBits), "a place fits its field");
 
 inline size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 

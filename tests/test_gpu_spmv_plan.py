@@ -64,6 +64,17 @@ def _cases(dtype):
     yield "far_band", _symmetric_band(50000, [-40000, -1, 0, 1, 40000], 4, dtype), (0, 0), True
     # near the diagonal, but a row's mirror entries lie more than 32 767 positions away
     yield "thick_band", _wide_rows(3000, 20, 1500, 5, dtype), (0, 1), False
+    # 3D seven-point pattern on 72^3: a column's entries one grid plane away lie 36 000 positions
+    # from their mirror entries -- beyond the 16 bits of a plain packed word, inside the field a
+    # block WITH a staging list has for the distance; every block of columns has a list
+    yield "stencil3d_72", G.laplace3d(72, dtype, jitter_seed=7), (1, 1), True
+    # the same followed by a tridiagonal block (three entries a column: no list, plain packed
+    # words): both layouts of the word in one plan
+    d3, i3, p3, (n3, _) = G.laplace3d(72, dtype, jitter_seed=8)
+    dt_, it_, pt_, (nt_, _) = G.tridiag(5000, dtype)
+    yield "stencil3d_then_tridiag", _csr(sps.block_diag([sps.csr_matrix((d3, i3, p3), shape=(n3, n3)),
+                                                         sps.csr_matrix((dt_, it_, pt_), shape=(nt_, nt_))]),
+                                         dtype), (1, 1), True
     yield "rectangular", G.random_csr(700, 300, 0.02, 5, dtype), (1, 1), True
     yield "cross", _cross(6000, 6, dtype), (1, 1), False
     # rows and columns of thousands of entries spread over 50 000 columns: the plain 32-bit arrays
