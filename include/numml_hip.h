@@ -120,8 +120,9 @@ int nm_csr_transpose_plan_build(int64_t rows, int64_t cols, int64_t nnz,
  * backward), info[6] / info[7] entries of the longest column / row, info[8] the
  * most entries that columns of more than 512 entries hold inside one aligned
  * group of 64 columns (such a group is one workgroup's in the SpMM kernels),
- * info[9] the blocks counted in info[4] that hold at most 3072 entries (the
- * forward's tile in fp64; 4096 in fp32, which every block with a list fits);
+ * info[9] the blocks counted in info[4] that hold at most 3072 entries (a
+ * figure for callers that size tiles of their own; the forward build with lists
+ * takes 4096 entries in both value types, which every block with a list fits);
  * the other entries are 0.  Waits for `stream`.  No counterpart in the
  * reference; a caller's choice between the kernels on a plan and the stateless
  * ones can be based on it. */
@@ -155,13 +156,16 @@ int nm_spgemv_forward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
                               const void *x, void *y, nm_stream stream);
 
 /* The same product by the instantiation that takes blocks of 512 rows with a
- * staging list (nm_csr_transpose_plan_info: info[4], info[9]) through LDS: the
+ * staging list (nm_csr_transpose_plan_info: info[4]) through LDS: the
  * segments of x such a block names are loaded with coalesced requests and the
  * entries' factors looked up there, where nm_spgemv_forward_planned gathers them
  * one by one through the plan's 32-bit columns.  It reserves LDS for those
  * segments, which costs resident workgroups on blocks without a list: for plans
- * most of whose blocks have one (same bits either way).  No counterpart in the
- * reference. */
+ * most of whose blocks have one.  Rows of fewer than 32 entries are summed by one
+ * lane in storage order in both, the same bits; a longer row is shared by a
+ * wavefront where its block exceeds the tile, and in fp64 this build's tile
+ * holds 4096 products against 3072, so such rows can differ in rounding between
+ * the two.  No counterpart in the reference. */
 int nm_spgemv_forward_planned_lists(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz,
                                     const void *data, const void *plan_mem,
                                     const void *x, void *y, nm_stream stream);

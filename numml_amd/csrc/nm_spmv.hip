@@ -1176,7 +1176,10 @@ template <typename T, typename IDX, bool LISTS = false>
 int launch_fwd(int64_t rows, int64_t nnz, const T *data, const IDX *indices, const IDX *indptr, const T *x,
                T *y, hipStream_t s, const int16_t *off16 = nullptr, const int32_t *flags = nullptr,
                const int32_t *f_desc = nullptr) {
-    constexpr int R = kFwdR, CAP = kFwdCap<T>;
+    // (the build with lists reserves LDS for the listed segments anyway, which holds a CU to three
+    // workgroups in fp64 whether the tile has 3072 or 4096 products: it takes the whole 4096, so
+    // that blocks of 512 rows with seven entries a row stay blocks of 512 rows)
+    constexpr int R = kFwdR, CAP = LISTS ? NM_FWD_CAP : kFwdCap<T>;
     const int rt = block_rows(rows, nnz, R, CAP);
     int64_t grid = nm::xcd_padded(nm::ceil_div(rows, rt));
     if (grid > nm::kMaxGrid) grid = nm::kMaxGrid;

@@ -733,11 +733,10 @@ Tensor spgemv_forward(int A_rows, int A_cols, Tensor A_data, Tensor A_col_ind, T
     // a pattern whose transposed-structure plan exists is read through the plan's 32-bit
     // copies of the structure (half the index bytes); looking for it costs no device work
     if (auto plan = peek_plan('T', A_col_ind, A_rowptr, A_rows, x.size(0), dev)) {
-        // most blocks of 512 rows have a staging list that this value type's tile can take: the
-        // instantiation that stages x in LDS (it gives up resident workgroups for that)
+        // most blocks of 512 rows have a staging list: the instantiation that stages x in LDS (it
+        // gives up resident workgroups for that)
         const int32_t *info = plan_info(*plan, A_rows, x.size(0), A_data.numel(), dev);
-        const int64_t listed = info[A_data.scalar_type() == torch::kFloat32 ? 4 : 9];
-        const bool lists = 2 * listed >= ((int64_t)A_rows + 511) / 512;
+        const bool lists = 2 * (int64_t)info[4] >= ((int64_t)A_rows + 511) / 512;
         check((lists ? nm_spgemv_forward_planned_lists : nm_spgemv_forward_planned)(
                   dtype_of(A_data), A_rows, x.size(0), A_data.numel(), A_data.data_ptr(), plan->mem.data_ptr(),
                   x.data_ptr(), y.data_ptr(), current_stream(dev)),

@@ -120,7 +120,13 @@ def test_planned_spmv_packed_and_plain_structure(dev, dtype):
                 y_l = torch.full((rows,), 7.0, dtype=D.dtype, device=dev)
                 _lib.check(L.nm_spgemv_forward_planned_lists(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X),
                                                              ptr(y_l), stream), "nm_spgemv_forward_planned_lists")
-                assert torch.equal(y, y_l), f"{name}: forward with and without staging lists"
+                # (rows that one lane sums in storage order -- fewer than 32 entries -- come out the
+                # same bit for bit; a longer row is shared by a wavefront where its block does not fit
+                # the tile, and the two builds have different tiles in fp64)
+                if exact:
+                    assert torch.equal(y, y_l), f"{name}: forward with and without staging lists"
+                else:
+                    assert_close(host(y_l), host(y), f"{name}: forward with and without staging lists")
                 _lib.check(L.nm_spgemv_backward_planned(dt, rows, cols, nnz, ptr(D), ptr(plan.mem), ptr(X), ptr(Gd),
                                                         ptr(gA), ptr(gx), stream), "nm_spgemv_backward_planned")
                 # the same for the backward: both builds, both gradients and each alone
