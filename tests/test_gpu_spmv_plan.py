@@ -75,6 +75,11 @@ def _cases(dtype):
     yield "stencil3d_then_tridiag", _csr(sps.block_diag([sps.csr_matrix((d3, i3, p3), shape=(n3, n3)),
                                                          sps.csr_matrix((dt_, it_, pt_), shape=(nt_, nt_))]),
                                          dtype), (1, 1), True
+    # 4, 6 and 8 entries a column: blocks of 256 columns with exactly 1024, 1536 and 2048 entries,
+    # i.e. the backward's tile with a list and no, two and four rounds behind its quads
+    for per in (4, 6, 8):
+        offs = [o for o in range(-per // 2, per // 2 + 1) if o != 0]
+        yield f"band{per}", _symmetric_band(6000, offs, 10 + per, dtype), (1, 1), True
     yield "rectangular", G.random_csr(700, 300, 0.02, 5, dtype), (1, 1), True
     yield "cross", _cross(6000, 6, dtype), (1, 1), False
     # rows and columns of thousands of entries spread over 50 000 columns: the plain 32-bit arrays
