@@ -618,7 +618,12 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
             // a wavefront gives each of its wavefronts its own 64 entries of A's row (the
             // order of insertion does not matter for the count).
             constexpr int S = G < kWave ? G : kWave;
+            // A group of 16 lanes takes TWO rows of B per step, eight lanes each: the rows these bins
+            // see are mostly shorter than eight entries (stencil powers), and insertion into a set
+            // has no order to keep, so the second half of the group need not idle.
+            constexpr int W = G == 16 ? 8 : S, NSUB = S / W;
             const int sl = gl & (S - 1), sub = G > kWave ? __builtin_amdgcn_readfirstlane(gl / S) : 0;
+            const int hl = sl & (W - 1), half = sl / W;
             const int gbase = (threadIdx.x & (kWave - 1)) & ~(S - 1);
             row = live ? perm[idx] : 0;
             const int64_t ab = live ? A_indptr[row] : 0, ae = live ? A_indptr[row + 1] : 0;
@@ -628,22 +633,26 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
                 const int64_t my_j = mine ? A_indices[my_ai] : 0;
                 const int64_t my_bb = mine ? B_indptr[my_j] : 0, my_be = mine ? B_indptr[my_j + 1] : 0;
                 const int nb = (int)(ae - a0 < S ? ae - a0 : S);
-                for (int e0 = 0; e0 < nb; e0 += kAhead) {
+                for (int e0 = 0; e0 < nb; e0 += kAhead * NSUB) {
                     int32_t pk[kAhead];
                     int64_t bbs[kAhead], bes[kAhead];
+                    bool has[kAhead];
 #pragma unroll
                     for (int u = 0; u < kAhead; ++u) {
-                        const int src = gbase + (e0 + u < nb ? e0 + u : e0);
+                        const int e = e0 + u * NSUB + half;
+                        has[u] = e < nb;
+                        const int src = gbase + (has[u] ? e : e0);
                         bbs[u] = __shfl(my_bb, src, kWave);
                         bes[u] = __shfl(my_be, src, kWave);
-                        const int64_t kk = bbs[u] + sl;
-                        pk[u] = (e0 + u < nb && kk < bes[u]) ? (int32_t)B_indices[kk] : kEmpty;
+                        const int64_t kk = bbs[u] + hl;
+                        pk[u] = (has[u] && kk < bes[u]) ? (int32_t)B_indices[kk] : kEmpty;
                     }
 #pragma unroll
                     for (int u = 0; u < kAhead; ++u) {
-                        if (e0 + u >= nb) break;
+                        if (e0 + u * NSUB >= nb) break;
                         if (pk[u] != kEmpty) insert(pk[u]);
-                        for (int64_t kk = bbs[u] + S + sl; kk < bes[u]; kk += S) insert((int32_t)B_indices[kk]);
+                        if (has[u])
+                            for (int64_t kk = bbs[u] + W + hl; kk < bes[u]; kk += W) insert((int32_t)B_indices[kk]);
                     }
                 }
             }
