@@ -179,3 +179,29 @@ def test_conjugate_gradients_and_training_through_the_solver(dev):
     rows = np.repeat(np.arange(n), np.diff(p))
     gA = Ad.grad.numpy()[rows, i]
     assert np.allclose(host(A.grad.data), gA, rtol=1e-8, atol=1e-10 * np.abs(gA).max())
+
+
+def test_stream_probe_and_longest_row_through_the_c_abi(dev):
+    """The two helper entry points callers use beside the operators: the plain streaming kernel
+    (copies the first write_bytes of what it reads, leaves the rest of the destination alone,
+    refuses sizes that are not multiples of 16) and the longest row of a pattern."""
+    import ctypes
+    from numml_amd import _lib
+    L = _lib.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    src = torch.arange(1 << 16, dtype=torch.float32, device=dev)
+    dst = torch.full((1 << 16,), -1.0, device=dev)
+    half = src.numel() * 4 // 2
+    _lib.check(L.nm_stream_probe(ptr(src), src.numel() * 4, ptr(dst), half, stream), "nm_stream_probe")
+    assert torch.equal(dst[:1 << 15], src[:1 << 15]) and bool((dst[1 << 15:] == -1).all())
+    _lib.check(L.nm_stream_probe(ptr(src), src.numel() * 4, None, 0, stream), "nm_stream_probe (read only)")
+    assert L.nm_stream_probe(ptr(src), 24, ptr(dst), 16, stream) != 0          # not a multiple of 16
+    assert L.nm_stream_probe(ptr(src), 64, ptr(dst), 128, stream) != 0         # writes more than it reads
+    for lens in ([3, 0, 7, 2], [0, 0, 0], [5], list(np.random.default_rng(3).integers(0, 900, 5000))):
+        indptr = torch.tensor(np.concatenate([[0], np.cumsum(lens)]).astype(np.int64), device=dev)
+        work = torch.empty(4096, dtype=torch.uint8, device=dev)
+        longest = ctypes.c_int64(-1)
+        _lib.check(L.nm_csr_longest_row(len(lens), ptr(indptr), ptr(work), work.numel(), None,
+                                        ctypes.byref(longest), stream), "nm_csr_longest_row")
+        assert longest.value == max(lens)
