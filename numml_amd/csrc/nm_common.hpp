@@ -105,6 +105,22 @@ __device__ __forceinline__ int dpp_move_zero(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
 }
 
+// Lane N of every aligned row of 16 lanes, handed to all lanes of that row (v_mov_b32_dpp
+// row_newbcast: one vector instruction per 32 bits, where a shuffle by lane number goes through
+// the LDS crossbar and waits for it).
+template <int N> __device__ __forceinline__ int row_lane(int v) {
+    static_assert(N >= 0 && N < 16, "a lane of a row of 16");
+    return __builtin_amdgcn_update_dpp(0, v, 0x150 + N, 0xf, 0xf, false);
+}
+template <int N> __device__ __forceinline__ int64_t row_lane(int64_t v) {
+    const int lo = row_lane<N>((int)(v & 0xffffffffll)), hi = row_lane<N>((int)(v >> 32));
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+template <int N> __device__ __forceinline__ float row_lane(float v) { return __int_as_float(row_lane<N>(__float_as_int(v))); }
+template <int N> __device__ __forceinline__ double row_lane(double v) {
+    return __longlong_as_double(row_lane<N>((int64_t)__double_as_longlong(v)));
+}
+
 __device__ __forceinline__ float read_lane(float v, int l) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
 }

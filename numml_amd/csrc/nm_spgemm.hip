@@ -716,10 +716,15 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
     const int gl = threadIdx.x % G, gi = G >= kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x / G) : threadIdx.x / G;
     int32_t *tab = s_keys + gi * STRIDE;
     T *val = s_vals + gi * STRIDE;
-    // compacted (column, slot) lists used to order the row on the way out
+    // compacted (column, slot) lists used to order the row on the way out.  The groups that share
+    // a wavefront keep them where the key table was (its keys are in registers by then): LDS per
+    // row is what decides how many rows a CU has in flight.
     constexpr int CSTRIDE = TABLE / 2 + 4;
-    int32_t *ck = s_keys + GPB * STRIDE + gi * 2 * CSTRIDE;
+    constexpr bool ALIAS = G <= kWave;
+    static_assert(!ALIAS || (CSTRIDE + TABLE / 4 <= TABLE && TABLE <= 65536), "the lists fit the key table");
+    int32_t *ck = ALIAS ? tab : s_keys + GPB * STRIDE + gi * 2 * CSTRIDE;
     int32_t *cs = ck + CSTRIDE;
+    uint16_t *cs16 = reinterpret_cast<uint16_t *>(cs);
     const int32_t b0 = bins[kBinStart + bin], b1 = bins[kBinStart + bin + 1];
     for (int32_t idx0 = b0 + blockIdx.x * GPB; idx0 < b1; idx0 += gridDim.x * GPB) {
         const int32_t idx = idx0 + gi;
@@ -754,21 +759,11 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
                 const T my_a = mine ? A_data[my_ai] : T(0);
                 const int64_t my_bb = mine ? B_indptr[my_j] : 0, my_be = mine ? B_indptr[my_j + 1] : 0;
                 const int nb = (int)(ae - a0 < G ? ae - a0 : G);
-                for (int e0 = 0; e0 < nb; e0 += kAhead) {
-                    int32_t pk[kAhead];
-                    T pv[kAhead], as[kAhead];
-                    int64_t bbs[kAhead], bes[kAhead];
-#pragma unroll
-                    for (int u = 0; u < kAhead; ++u) {
-                        const int src = gbase + (e0 + u < nb ? e0 + u : e0);
-                        bbs[u] = __shfl(my_bb, src, kWave);
-                        bes[u] = __shfl(my_be, src, kWave);
-                        as[u] = __shfl(my_a, src, kWave);
-                        const int64_t kk = bbs[u] + gl;
-                        const bool ok = e0 + u < nb && kk < bes[u];
-                        pk[u] = ok ? (int32_t)B_indices[kk] : kEmpty;
-                        pv[u] = ok ? B_data[kk] : T(0);
-                    }
+                int32_t pk[kAhead];
+                T pv[kAhead], as[kAhead];
+                int64_t bbs[kAhead], bes[kAhead];
+                // the entries of A's row held by lanes e0 .. e0 + kAhead - 1 of the group, applied in turn
+                auto apply = [&](int e0) {
 #pragma unroll
                     for (int u = 0; u < kAhead; ++u) {
                         if (e0 + u >= nb) break;
@@ -776,6 +771,63 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
                         for (int64_t kk = bbs[u] + G + gl; kk < bes[u]; kk += G)
                             add((int32_t)B_indices[kk], as[u] * B_data[kk]);
                         group_sync<G>();  // the next entry of A's row adds after this one
+                    }
+                };
+                if constexpr (G == 16) {
+                    // A group is one 16-lane DPP row: what lane e of the group holds reaches the others
+                    // by a row broadcast (one vector move per 32 bits) instead of a shuffle by lane
+                    // number through the LDS crossbar.  That is cheap enough to fetch an entry's value
+                    // and the bounds of its row of B again when they are used, so only the columns and
+                    // values requested ahead stay in registers (116 -> fewer registers: more wavefronts).
+                    static_assert(2 * kAhead == G, "two batches cover the group");
+                    const int my_len = (int)(my_be - my_bb);
+                    using std::integral_constant;
+                    auto batch = [&](auto first) {
+                        constexpr int E0 = decltype(first)::value;
+                        auto fetch = [&](auto uc) {
+                            constexpr int U = decltype(uc)::value;
+                            const int64_t kk = nm::row_lane<E0 + U>(my_bb) + gl;
+                            const bool ok = E0 + U < nb && gl < nm::row_lane<E0 + U>(my_len);
+                            pk[U] = ok ? (int32_t)B_indices[kk] : kEmpty;
+                            pv[U] = ok ? B_data[kk] : T(0);
+                        };
+                        auto apply_one = [&](auto uc) {
+                            constexpr int U = decltype(uc)::value;
+                            if (E0 + U >= nb) return;
+                            const T a = nm::row_lane<E0 + U>(my_a);
+                            if (pk[U] != kEmpty) add(pk[U], a * pv[U]);
+                            if (nm::row_lane<E0 + U>(my_len) > G) {   // the rest of a row of B longer than the group
+                                const int64_t bb = nm::row_lane<E0 + U>(my_bb), be = nm::row_lane<E0 + U>(my_be);
+                                for (int64_t kk = bb + G + gl; kk < be; kk += G) add((int32_t)B_indices[kk], a * B_data[kk]);
+                            }
+                            group_sync<G>();  // the next entry of A's row adds after this one
+                        };
+                        static_assert(kAhead == 8, "eight rows of B ahead");
+                        fetch(integral_constant<int, 0>{}); fetch(integral_constant<int, 1>{});
+                        fetch(integral_constant<int, 2>{}); fetch(integral_constant<int, 3>{});
+                        fetch(integral_constant<int, 4>{}); fetch(integral_constant<int, 5>{});
+                        fetch(integral_constant<int, 6>{}); fetch(integral_constant<int, 7>{});
+                        apply_one(integral_constant<int, 0>{}); apply_one(integral_constant<int, 1>{});
+                        apply_one(integral_constant<int, 2>{}); apply_one(integral_constant<int, 3>{});
+                        apply_one(integral_constant<int, 4>{}); apply_one(integral_constant<int, 5>{});
+                        apply_one(integral_constant<int, 6>{}); apply_one(integral_constant<int, 7>{});
+                    };
+                    batch(integral_constant<int, 0>{});
+                    if (nb > kAhead) batch(integral_constant<int, kAhead>{});
+                } else {
+                    for (int e0 = 0; e0 < nb; e0 += kAhead) {
+#pragma unroll
+                        for (int u = 0; u < kAhead; ++u) {
+                            const int src = gbase + (e0 + u < nb ? e0 + u : e0);
+                            bbs[u] = __shfl(my_bb, src, kWave);
+                            bes[u] = __shfl(my_be, src, kWave);
+                            as[u] = __shfl(my_a, src, kWave);
+                            const int64_t kk = bbs[u] + gl;
+                            const bool ok = e0 + u < nb && kk < bes[u];
+                            pk[u] = ok ? (int32_t)B_indices[kk] : kEmpty;
+                            pv[u] = ok ? B_data[kk] : T(0);
+                        }
+                        apply(e0);
                     }
                 }
             }
@@ -878,8 +930,14 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
             // half of their table, so this is a fraction of the compares a rank over the whole
             // table would take.
             const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);
+            constexpr int K = TABLE / G;
+            int32_t keys[K];
             int mine = 0;
-            for (int t = gl; t < TABLE; t += G) mine += tab[t] != kEmpty;
+#pragma unroll
+            for (int q = 0; q < K; ++q) {
+                keys[q] = tab[gl + q * G];
+                mine += keys[q] != kEmpty;
+            }
             int incl = mine;
 #pragma unroll
             for (int off = 1; off < G; off <<= 1) {
@@ -888,10 +946,14 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
             }
             const int c = __shfl(incl, gbase + G - 1, kWave);
             int pos = incl - mine;
-            for (int t = gl; t < TABLE; t += G) {
-                const int32_t key = tab[t];
-                if (key != kEmpty) { ck[pos] = key; cs[pos] = t; ++pos; }
-            }
+            group_sync<G>();   // every lane holds its part of the table: the lists may take its place
+#pragma unroll
+            for (int q = 0; q < K; ++q)
+                if (keys[q] != kEmpty) {
+                    ck[pos] = keys[q];
+                    cs16[pos] = (uint16_t)(gl + q * G);
+                    ++pos;
+                }
             if (gl < 4) ck[c + gl] = kEmpty;   // pad the list to a multiple of four keys
             group_sync<G>();
             if (live) {
@@ -906,7 +968,7 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
                         rank += (q.x < key) + (q.y < key) + (q.z < key) + (q.w < key);
                     }
                     C_indices[base + rank] = (int64_t)key;
-                    C_data[base + rank] = val[cs[e]];
+                    C_data[base + rank] = val[cs16[e]];
                 }
             }
         }
@@ -1239,7 +1301,8 @@ int launch_numeric(const Work &w, int64_t B_cols, const void *A_data, const int6
         constexpr int G = decltype(group)::value, TABLE = decltype(table)::value;
         auto k = numeric_hash_kernel<T, G, TABLE>;
         // tables (values + keys), padded apart when groups share a workgroup, and the two compaction lists
-        const size_t lds = (kBlock / G) * (per * (TABLE + (G < kBlock ? kTablePad : 0)) + 4 * (TABLE + 8));
+        // (narrow groups keep the lists where the key table was)
+        const size_t lds = (kBlock / G) * (per * (TABLE + (G < kBlock ? kTablePad : 0)) + (G > kWave ? 4 * (TABLE + 8) : 0));
         if (lds > 64 * 1024)
             NM_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
