@@ -1,5 +1,6 @@
 // Shared host/device helpers of libnumml_hip.so (gfx950 only).
 #pragma once
+#include <utility>
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -103,6 +104,16 @@ __device__ __forceinline__ double dpp_move_zero(double v) {
 template <int CTRL>
 __device__ __forceinline__ int dpp_move_zero(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose index is a
+// compile-time constant in the body (DPP controls, register arrays).
+template <int N, typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl<N>(f, std::make_integer_sequence<int, N>{});
 }
 
 // Lane N of every aligned row of 16 lanes, handed to all lanes of that row (v_mov_b32_dpp

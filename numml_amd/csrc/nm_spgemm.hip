@@ -52,6 +52,9 @@ inline int spill_groups(int64_t B_cols) {
 constexpr int kSpillBlock = 1024;
 constexpr int kTablePad = 4;         // entries between the hash tables of neighbouring groups (16 bytes)
 constexpr int kAhead = 8;            // B rows whose first columns a group requests before inserting any
+#ifndef NM_HASH_BATCH
+#define NM_HASH_BATCH 8
+#endif
 
 // bin upper limits (inclusive); the last bin takes the rest and spills
 constexpr int32_t kSymLimit[7] = {64, 128, 256, 512, 1024, 2048, 8192};     // on the product bound
@@ -779,41 +782,35 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
                     // number through the LDS crossbar.  That is cheap enough to fetch an entry's value
                     // and the bounds of its row of B again when they are used, so only the columns and
                     // values requested ahead stay in registers (116 -> fewer registers: more wavefronts).
-                    static_assert(2 * kAhead == G, "two batches cover the group");
+                    constexpr int BATCH = NM_HASH_BATCH;   // rows of B requested ahead: 8 or 16
+                    static_assert(G % BATCH == 0, "whole batches cover the group");
                     const int my_len = (int)(my_be - my_bb);
-                    using std::integral_constant;
+                    int32_t qk[BATCH];
+                    T qv[BATCH];
                     auto batch = [&](auto first) {
                         constexpr int E0 = decltype(first)::value;
-                        auto fetch = [&](auto uc) {
+                        nm::static_for<BATCH>([&](auto uc) {
                             constexpr int U = decltype(uc)::value;
                             const int64_t kk = nm::row_lane<E0 + U>(my_bb) + gl;
                             const bool ok = E0 + U < nb && gl < nm::row_lane<E0 + U>(my_len);
-                            pk[U] = ok ? (int32_t)B_indices[kk] : kEmpty;
-                            pv[U] = ok ? B_data[kk] : T(0);
-                        };
-                        auto apply_one = [&](auto uc) {
+                            qk[U] = ok ? (int32_t)B_indices[kk] : kEmpty;
+                            qv[U] = ok ? B_data[kk] : T(0);
+                        });
+                        nm::static_for<BATCH>([&](auto uc) {
                             constexpr int U = decltype(uc)::value;
                             if (E0 + U >= nb) return;
                             const T a = nm::row_lane<E0 + U>(my_a);
-                            if (pk[U] != kEmpty) add(pk[U], a * pv[U]);
+                            if (qk[U] != kEmpty) add(qk[U], a * qv[U]);
                             if (nm::row_lane<E0 + U>(my_len) > G) {   // the rest of a row of B longer than the group
                                 const int64_t bb = nm::row_lane<E0 + U>(my_bb), be = nm::row_lane<E0 + U>(my_be);
                                 for (int64_t kk = bb + G + gl; kk < be; kk += G) add((int32_t)B_indices[kk], a * B_data[kk]);
                             }
                             group_sync<G>();  // the next entry of A's row adds after this one
-                        };
-                        static_assert(kAhead == 8, "eight rows of B ahead");
-                        fetch(integral_constant<int, 0>{}); fetch(integral_constant<int, 1>{});
-                        fetch(integral_constant<int, 2>{}); fetch(integral_constant<int, 3>{});
-                        fetch(integral_constant<int, 4>{}); fetch(integral_constant<int, 5>{});
-                        fetch(integral_constant<int, 6>{}); fetch(integral_constant<int, 7>{});
-                        apply_one(integral_constant<int, 0>{}); apply_one(integral_constant<int, 1>{});
-                        apply_one(integral_constant<int, 2>{}); apply_one(integral_constant<int, 3>{});
-                        apply_one(integral_constant<int, 4>{}); apply_one(integral_constant<int, 5>{});
-                        apply_one(integral_constant<int, 6>{}); apply_one(integral_constant<int, 7>{});
+                        });
                     };
-                    batch(integral_constant<int, 0>{});
-                    if (nb > kAhead) batch(integral_constant<int, kAhead>{});
+                    batch(std::integral_constant<int, 0>{});
+                    if constexpr (BATCH < G)
+                        if (nb > BATCH) batch(std::integral_constant<int, BATCH < G ? BATCH : 0>{});
                 } else {
                     for (int e0 = 0; e0 < nb; e0 += kAhead) {
 #pragma unroll
