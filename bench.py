@@ -87,6 +87,21 @@ def _traffic(workload, kernel=None):
         return None
 
 
+def _traffic_of(workload, names):
+    """`names`: a kernel name, "*" for the figure of the workload's entry as a whole (an operation
+    made of several launches: their sum), or a tuple of those to be added up; None when any is
+    missing."""
+    if not names:
+        return None
+    total = 0
+    for n in (names if isinstance(names, tuple) else (names,)):
+        t = _traffic(workload) if n == "*" else _traffic(workload, n)
+        if t is None:
+            return None
+        total += t
+    return total
+
+
 class Workload:
     name = ""
     metric = "SpMV/SpMM eff. HBM GB/s (% of peak); SpGEMM GFLOP/s; tri-solve ms"
@@ -746,10 +761,10 @@ class SpTRSV(Workload):
     def ops(self):
         x = self.dominant()
         s = 8
-        return [(self.dominant_name, self.dominant, self.dominant_bytes, "sptrsv_ell_kernel"),
+        return [(self.dominant_name, self.dominant, self.dominant_bytes, "*"),
                 ("backward: transposed solve (the same three kernels on the packed A^T) + spmv_bwd_kernel as the masked outer product",
                  lambda: self.ext.sptrsv_backward(self.Gv, x, self.rows, self.rows, self.D, self.I, self.P, True, False, self.Bv),
-                 self.dominant_bytes + self.nnz * (s + 8) + 2 * self.rows * s, None)]
+                 self.dominant_bytes + self.nnz * (s + 8) + 2 * self.rows * s, ("*", "spmv_bwd_kernel"))]
 
     def value(self, ms_per_step):
         return ms_per_step
@@ -1210,7 +1225,7 @@ def measure(w, dev, steps, warmup, cpu_seconds):
         achieved = nbytes / (ms * 1e-3) / 1e9
         kernels.append({"name": name, "avg_ms": round(ms, 5), "algorithmic_bytes": int(nbytes),
                         "achieved": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBS, 4),
-                        "traffic": _traffic(w.name, prof_name) if prof_name else None})
+                        "traffic": _traffic_of(w.name, prof_name)})
     top = max(kernels, key=lambda k: k["avg_ms"])
     roofline = {"bound": "hbm", "kernel": top["name"], "achieved": top["achieved"],
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": top["frac"],
