@@ -128,6 +128,17 @@ template <int N> __device__ __forceinline__ int64_t row_lane(int64_t v) {
     return ((int64_t)hi << 32) | (uint32_t)lo;
 }
 template <int N> __device__ __forceinline__ float row_lane(float v) { return __int_as_float(row_lane<N>(__float_as_int(v))); }
+// Lane LO of the row to its lanes 0-7 and lane HI to its lanes 8-15 (two moves, each writing two
+// of the row's four banks).
+template <int LO, int HI> __device__ __forceinline__ int row_lane_halves(int v) {
+    static_assert(LO >= 0 && LO < 16 && HI >= 0 && HI < 16, "lanes of a row of 16");
+    const int r = __builtin_amdgcn_update_dpp(0, v, 0x150 + LO, 0xf, 0x3, false);
+    return __builtin_amdgcn_update_dpp(r, v, 0x150 + HI, 0xf, 0xc, false);
+}
+template <int LO, int HI> __device__ __forceinline__ int64_t row_lane_halves(int64_t v) {
+    const int lo = row_lane_halves<LO, HI>((int)(v & 0xffffffffll)), hi = row_lane_halves<LO, HI>((int)(v >> 32));
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
 template <int N> __device__ __forceinline__ double row_lane(double v) {
     return __longlong_as_double(row_lane<N>((int64_t)__double_as_longlong(v)));
 }

@@ -659,6 +659,36 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
                 const int64_t my_j = mine ? A_indices[my_ai] : 0;
                 const int64_t my_bb = mine ? B_indptr[my_j] : 0, my_be = mine ? B_indptr[my_j + 1] : 0;
                 const int nb = (int)(ae - a0 < S ? ae - a0 : S);
+                if constexpr (G == 16) {
+                    // the group is one DPP row: entries 2 u and 2 u + 1 of A's row reach the two halves
+                    // by row broadcasts instead of shuffles through the LDS crossbar, and the bounds of a
+                    // row of B longer than eight entries are fetched again where its rest is walked
+                    static_assert(kAhead * NSUB == G && W == 8, "one batch of pairs covers the group");
+                    const int my_len = (int)(my_be - my_bb);
+                    int32_t qk[kAhead];
+                    nm::static_for<kAhead>([&](auto uc) {
+                        constexpr int U = decltype(uc)::value;
+                        // (broadcasts first, with all sixteen lanes active; then the lane's own tests)
+                        const int64_t kk = nm::row_lane_halves<2 * U, 2 * U + 1>(my_bb) + hl;
+                        const int len = nm::row_lane_halves<2 * U, 2 * U + 1>(my_len);
+                        const bool ok = (2 * U + half < nb) & (hl < len);
+                        qk[U] = ok ? (int32_t)B_indices[kk] : kEmpty;
+                    });
+                    nm::static_for<kAhead>([&](auto uc) {
+                        constexpr int U = decltype(uc)::value;
+                        if (2 * U >= nb) return;
+                        if (qk[U] != kEmpty) insert(qk[U]);
+                        // (the test is the same in all sixteen lanes, so that the broadcasts behind it
+                        // find their source lanes active)
+                        const int len_lo = nm::row_lane<2 * U>(my_len), len_hi = nm::row_lane<2 * U + 1>(my_len);
+                        if ((len_lo > W) | (len_hi > W)) {   // (lanes past the row's end hold a length of 0)
+                            const int64_t bb = nm::row_lane_halves<2 * U, 2 * U + 1>(my_bb);
+                            const int64_t be_row = nm::row_lane_halves<2 * U, 2 * U + 1>(my_be);
+                            const int64_t be = 2 * U + half < nb ? be_row : bb;
+                            for (int64_t kk = bb + W + hl; kk < be; kk += W) insert((int32_t)B_indices[kk]);
+                        }
+                    });
+                } else
                 for (int e0 = 0; e0 < nb; e0 += kAhead * NSUB) {
                     int32_t pk[kAhead];
                     int64_t bbs[kAhead], bes[kAhead];
@@ -815,7 +845,8 @@ __global__ __launch_bounds__(kBlock) void numeric_hash_kernel(
                         nm::static_for<BATCH>([&](auto uc) {
                             constexpr int U = decltype(uc)::value;
                             const int64_t kk = nm::row_lane<E0 + U>(my_bb) + gl;
-                            const bool ok = E0 + U < nb && gl < nm::row_lane<E0 + U>(my_len);
+                            const int len = nm::row_lane<E0 + U>(my_len);
+                            const bool ok = (E0 + U < nb) & (gl < len);
                             qk[U] = ok ? (int32_t)B_indices[kk] : kEmpty;
                             qv[U] = ok ? B_data[kk] : T(0);
                         });
