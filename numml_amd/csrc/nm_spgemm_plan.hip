@@ -245,12 +245,14 @@ __device__ __forceinline__ void store_wave_rows(const T *acc, const int32_t *cco
             T2 v;
             v[0] = acc[a0 + j];
             v[1] = acc[a1 + j + 1];
-            *reinterpret_cast<T2 *>(out + j) = v;
+            // (written once and not read again by this kernel: nontemporal, which leaves L2 to the
+            // rows of B -- 0.209 -> 0.190 ms on the 128^3 seven-point product)
+            __builtin_nontemporal_store(v, reinterpret_cast<T2 *>(out + j));
             if (COLS) {
                 L2 c;
                 c[0] = (int64_t)ccol[a0 + j];
                 c[1] = (int64_t)ccol[a1 + j + 1];
-                *reinterpret_cast<L2 *>(outc + j) = c;
+                __builtin_nontemporal_store(c, reinterpret_cast<L2 *>(outc + j));
             }
         } else {
             out[j] = acc[a0 + j];
