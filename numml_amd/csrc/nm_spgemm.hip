@@ -271,9 +271,9 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
         C_count[row] = cnt;
         key[row] = kMergedKey;
     }
-    if (dest && merge && ab + gl < ae) {
-        dest[ab + gl] = where;
-        bstart[ab + gl] = (int32_t)my_bb;
+    if (dest && merge && ab + gl < ae) {   // (read once, by another kernel: nontemporal)
+        __builtin_nontemporal_store(where, dest + ab + gl);
+        __builtin_nontemporal_store((int32_t)my_bb, bstart + ab + gl);
     }
 }
 

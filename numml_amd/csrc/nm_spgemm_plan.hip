@@ -317,7 +317,7 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
         s_av[threadIdx.x] = av;
         s_bs[threadIdx.x] = bs;
         *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) = k < alen ? db : ~uint64_t(0);
-        if (COLS && k < alen) cstart[e] = (int32_t)cs;
+        if (COLS && k < alen) __builtin_nontemporal_store((int32_t)cs, cstart + e);
     }
     group_fence();
     const int slot = g * kCap;
