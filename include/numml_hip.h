@@ -448,6 +448,10 @@ int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan);
  * which a single wavefront walks with the newest solution in a register (banded factors,
  * bidiagonal and tridiagonal triangles); diagnostics. */
 int64_t nm_sptrsv_plan_chain_levels(const nm_sptrsv_plan *plan, int transposed);
+/* Launches of the solve with A (transposed = 0) or with A^T (1) whose levels are each shared by
+ * several workgroups (levels of more than 256 rows whose dependencies cross between the
+ * workgroups' parts in a way that can be pipelined: triangles of grid stencils); diagnostics. */
+int64_t nm_sptrsv_plan_shared_launches(const nm_sptrsv_plan *plan, int transposed);
 
 void nm_sptrsv_plan_destroy(nm_sptrsv_plan *plan);
 
@@ -463,18 +467,25 @@ int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
                     const void *data, int unit, const void *b, void *x,
                     void *work, size_t work_bytes, nm_stream stream);
 
-/* How the single-workgroup kernels of the solve keep their wavefronts in step
- * (no counterpart in the reference).  By default every wavefront meets at a
- * workgroup barrier after every level.  With `signalling` = 1, where no row of
- * a triangle depends on a row more than one wavefront away inside the level
- * before it (stencil and banded matrices), a wavefront instead publishes the
- * levels it has finished in LDS and waits only for its neighbours.  (Measured
- * slower than the barrier on MI355X, hence off by default; results are the same
- * bits.)  All wavefronts of a workgroup are resident and only wait for lower
- * levels, so the waits end; `poll_limit` bounds the polls of one wait all the
- * same (0: the default of 2^22; negative: give up at once, for tests): when it
- * is exceeded every wavefront of the launch leaves and x comes back as NaN
- * throughout.  Process-wide; takes effect with the next solve. */
+/* How the level kernels of the solve synchronise (no counterpart in the reference).
+ * `signalling` is a set of bits.
+ * Bit 0 (default off): inside a single-workgroup launch every wavefront meets at a
+ * workgroup barrier after every level; with the bit set, where no row of a triangle
+ * depends on a row more than one wavefront away inside the level before it (stencil
+ * and banded matrices), a wavefront instead publishes the levels it has finished in
+ * LDS and waits only for its neighbours.  (Measured slower than the barrier on
+ * MI355X, hence off; results are the same bits.)
+ * Bit 1 (default off): launches that the plan would share among up to four
+ * workgroups (nm_sptrsv_plan_shared_launches; each takes 256 rows of every level and
+ * receives the few values it needs from the others through device memory, running a
+ * few levels behind the workgroup it receives from) are taken by one workgroup
+ * instead.  Results are the same bits either way.
+ * All waiting is for rows of lower levels, by wavefronts of workgroups that are all
+ * resident (a shared launch needs as many free compute units as it has workgroups),
+ * so the waits end; `poll_limit` bounds the polls of one wait all the same (0: the
+ * default of 2^22, seconds; negative: give up at once, for tests): when it is
+ * exceeded the waiting stops for good and x comes back as NaN throughout.
+ * Process-wide; takes effect with the next solve. */
 int nm_sptrsv_configure(int64_t poll_limit, int signalling);
 
 /* nm_sptrsv_solve without the `work` argument, for callers that cannot allocate

@@ -143,6 +143,8 @@ def lib():
     L.nm_sptrsv_plan_launches.restype = _c_i64
     L.nm_sptrsv_plan_chain_levels.argtypes = [_c_ptr, _c_int]
     L.nm_sptrsv_plan_chain_levels.restype = _c_i64
+    L.nm_sptrsv_plan_shared_launches.argtypes = [_c_ptr, _c_int]
+    L.nm_sptrsv_plan_shared_launches.restype = _c_i64
     L.nm_sptrsv_plan_destroy.argtypes = [_c_ptr]
     L.nm_sptrsv_plan_destroy.restype = None
     _lib = L

@@ -21,8 +21,11 @@
 // this call's coefficients, diagonal and right-hand side into level-major
 // order (as doubles), so the workgroup reads contiguous streams only, two and
 // one level ahead through a register pipeline.  A level wider than 1024 rows gets a grid launch of its own.
-// Stream order is the only synchronisation between launches: no kernel ever
-// waits on another workgroup, so nothing can hang.
+// Where the plan finds it possible, a run of levels wider than 256 rows is shared by up
+// to four workgroups that pass the few values they need from each other through device
+// memory (sptrsv_team_kernel).  Stream order is the only synchronisation between launches;
+// inside a shared launch a workgroup waits for values of lower levels only, all its
+// workgroups are resident, and every wait is bounded (a solve that gives up returns NaN).
 //
 // A row is one lane; sums run in double, in the walk order of the serial
 // CPU loop (cpp/sparse_csr_cpu.cpp:672-718: ascending for a lower triangle,
@@ -37,6 +40,7 @@
 #include "nm_scan.hpp"
 #include "nm_transpose.hpp"
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <mutex>
@@ -51,6 +55,7 @@ struct Packed {        // one solve direction, level-major (all int32, device)
     int32_t *diag;     // [rows]   position of the diagonal coefficient, -1 when not stored
     int32_t *ell_ds;   // [ell_capacity] room for the fixed-width dependency entries: 16 bits each, `pre` per row
     int32_t *lvl_sig;  // [levels] which neighbouring wavefronts the rows of a level wait for (kSigLower | kSigHigher)
+    int32_t *team;     // [team_capacity] exchange tables of the launches that several workgroups share
 };
 // Entries of the fixed-width (ELLPACK) arrays; the layout is used when (rows + kEllPad) * pre
 // fits.  kEllPad slots of padding follow the last row in every array the fixed-width kernel
@@ -65,6 +70,12 @@ inline int64_t coef_capacity(int64_t rows, int64_t nnz) {
     const int64_t chains = 66 * (rows < 65536 ? rows : 65536) + 8 * kEllPad;
     return ell_capacity(rows, nnz) > chains ? ell_capacity(rows, nnz) : chains;
 }
+// Launches that several workgroups share (see sptrsv_team_kernel): most workgroups, values that
+// may pass between workgroups in one solve direction, ints of the tables that say which.
+constexpr int kTeamMax = 4;
+inline int64_t team_cells_capacity(int64_t rows) { return rows / 16 + 2048; }
+constexpr int64_t kTeamCellPadding = 64;   // readable cells past the last one (a poll reads 64 at a time)
+inline int64_t team_capacity(int64_t rows) { return 3 * team_cells_capacity(rows) + rows / 16 + 16384; }
 }  // namespace
 
 struct nm_sptrsv_plan {
@@ -90,8 +101,16 @@ struct nm_sptrsv_plan {
         int32_t chain[2] = {0, 0};
         int64_t chain_at[2] = {0, 0};
         bool chain_candidate = false;
+        // per direction: the workgroups that share every level of the launch (0: one workgroup
+        // takes it), where the tables of their exchange start in Packed::team, the first of their
+        // mailbox cells, and each workgroup's part of the import and export lists
+        struct Team {
+            int32_t P = 0, at = 0, cell0 = 0, n_imp = 0;
+            int32_t imp_off[kTeamMax + 1] = {}, exp_off[kTeamMax + 1] = {};
+        } team[2];
     };
     std::vector<Launch> launches;
+    int32_t team_cells[2] = {0, 0};   // mailbox cells one solve clears, per direction
 };
 
 namespace {
@@ -121,6 +140,11 @@ std::atomic<int64_t> g_sig_poll_limit{int64_t(1) << 22};
 // Off by default: on the 1024 x 1024 Poisson triangle (2047 levels, up to 16 wavefronts) a solve
 // takes 0.97 ms with a barrier per level and 1.30 ms with signals -- the two dependent LDS round
 // trips of a poll cost more than the barrier's wait for the slowest wavefront saves.
+// Launches shared by several workgroups (sptrsv_team_kernel), where the plan has found them possible.
+std::atomic<bool> g_team_enabled{[] {
+    const char *e = std::getenv("NUMML_AMD_SPTRSV_TEAMS");   // "0": one workgroup per launch
+    return !(e && e[0] == '0');
+}()};
 std::atomic<bool> g_sig_enabled{[] {
     const char *e = std::getenv("NUMML_AMD_SPTRSV_SIGNALLING");   // "1": neighbours signal
     return e && e[0] == '1';
@@ -153,6 +177,7 @@ size_t plan_layout(int64_t rows, int64_t nnz, void *base, Layout *L) {
         l.dir[d].diag = take(rows + 1);
         l.dir[d].ell_ds = take(ell_capacity(rows, nnz));
         l.dir[d].lvl_sig = take(rows + 1);
+        l.dir[d].team = take(team_capacity(rows));
     }
     if (L) *L = l;
     return off;
@@ -333,6 +358,7 @@ struct SolveWork {
     double *ell_coef;  // fixed-width copy of coef (0 padded), `pre` per slot
     double *rb;        // (right-hand side, diagonal) pairs per slot
     int32_t *status;   // [2]: nonzero when a kernel of this solve gave up waiting
+    unsigned long long *cells;   // mailbox of values that pass between the workgroups of a shared launch, two words each
 };
 
 inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork *W) {
@@ -350,6 +376,7 @@ inline size_t solve_work_layout(int64_t rows, int64_t nnz, void *base, SolveWork
     w.ell_coef = take(coef_capacity(rows, nnz));
     w.rb = take(2 * (rows + kEllPad) + 2);
     w.status = (int32_t *)take(2);
+    w.cells = (unsigned long long *)take(2 * (team_cells_capacity(rows) + kTeamCellPadding) + 2);
     if (W) *W = w;
     return off;
 }
@@ -702,10 +729,13 @@ __global__ void gather_ell_kernel(int64_t rows, int pre, const T *__restrict__ d
                                   const int32_t *__restrict__ order, const int32_t *__restrict__ dptr,
                                   const int32_t *__restrict__ dsrc, const int32_t *__restrict__ diag,
                                   double *__restrict__ ell_coef, double *__restrict__ rb,
-                                  int32_t *__restrict__ status) {
+                                  int32_t *__restrict__ status, unsigned long long *__restrict__ cells,
+                                  int64_t cell_words) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (tid == 0) status[0] = 0;   // first kernel of the solve
+    // the mailbox of the launches that several workgroups share: empty before the solve starts
+    for (int64_t i = tid; i < cell_words; i += stride) cells[i] = 0ull;
     for (int64_t i = tid; i < rows * pre; i += stride) {
         const int64_t q = i / pre;
         const int e = (int)(i - q * pre);
@@ -1012,6 +1042,270 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
     if (SIG && gave_up && sig_lane == 0 && status) status[0] = 1;
 }
 
+// ---- several workgroups per level ---------------------------------------------------------
+//
+// One workgroup streams a level's operands through the one compute unit it lives on, and at a
+// thousand rows a level that is what a level costs (44 bytes a row at the ~110 GB/s one unit
+// streams).  Here P workgroups share every level of a launch: workgroup k takes the rows
+// [k * kTeamChunk, (k + 1) * kTeamChunk) of each level, so each unit streams a quarter.  What
+// keeps that from costing a hand-over between compute units per level (0.6-0.75 us through
+// device memory, more than a whole level takes) is that the workgroups do NOT move in step:
+//
+//  * a workgroup keeps its own LDS ring and its own barrier per level, exactly as the
+//    single-workgroup kernel does, with one more wavefront that computes nothing;
+//  * a value that a row of ANOTHER workgroup needs (the plan lists them: `exports`, by the level
+//    that produces them) is read from the ring by that service wavefront one level after it was
+//    computed and stored to a mailbox cell in device memory: two 64-bit words, each half of the
+//    double next to a tag, so that a reader that finds both tags set has the whole value
+//    (a naturally aligned 64-bit access is never torn; no fence, no second flag);
+//  * the service wavefront of the consumer polls the cells of its `imports` (listed by the level
+//    that first needs them) S levels ahead of use and writes what has arrived into its ring;
+//    only when a value is still missing at the barrier before the level that needs it does it
+//    wait, and with it the workgroup.
+//
+// On a triangle whose dependencies cross the cut in one direction (the tril of a grid: a row
+// depends on its left and lower neighbours of the previous level) the consumers simply fall a few
+// levels behind their producers and nobody waits again until the direction changes.  The plan
+// only makes a launch shared when that is possible: per level, "workgroup a needs a value that
+// workgroup b computes at the level before" must not form a cycle (such a level would need the
+// hand-over inside the level; see build_team).  Every workgroup of the grid is resident (P <= 4 of
+// the chip's 256 units) and a workgroup only waits for values of lower levels, so the waits end;
+// as a backstop a service wavefront that has polled `poll_limit` times for one level stops
+// waiting for good and the solve hands out NaN, as for the signalling kernel above.
+constexpr int kTeamChunk = 256;            // rows of a level that one workgroup takes
+constexpr int kTeamStages = 6;             // polls in flight
+constexpr int kTeamAhead = kRing - kRingSafe;   // slots ahead of its own level a workgroup may import
+constexpr int kTeamExports = 4096;         // values one workgroup may hand out in one launch (their list lives in LDS)
+static_assert((kTeamExports & (kTeamExports - 1)) == 0, "a power of two");
+constexpr int kTeamNeedBits = 18;          // a workgroup's imports in one launch are counted in these
+static_assert(kTeamExports < (1 << (31 - kTeamNeedBits)), "exports and imports share a word");
+static_assert(kTeamCellPadding >= 64, "a poll reads 64 cells from any import on");
+
+struct TeamArgs {
+    const int32_t *tab;          // [P][count+1] imports needed up to a level, [P][count+1] exports before a level,
+                                 // [n_imp] slot of an import (not read by the kernel: the cell names it),
+                                 // [n_imp] slot of an export, [n_imp] its cell
+    unsigned long long *cells;   // this launch's mailbox cells
+    int32_t P, n_imp;
+    int32_t quiet;               // first of the padding cells, counted from `cells`
+    int32_t imp_off[kTeamMax + 1], exp_off[kTeamMax + 1];
+};
+
+struct TeamPoll { int cs; unsigned long long w0, w1; };
+
+template <int PRE, int DEPTH>
+__global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a, TeamArgs t, int l0, int count, int step,
+                                                                       int64_t poll_limit, int32_t *status) {
+    __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
+    __shared__ int32_t s_lp[kMaxLevels + 1];
+    // what the service wavefront needs at a level, in one LDS read: x = the limit an imported
+    // slot is held against (times `step`), y = imports the NEXT level needs (low kTeamNeedBits
+    // bits) and exports of the levels before this one (the bits above)
+    __shared__ int2 s_sv[kMaxLevels + 1];
+    __shared__ int2 s_exl[kTeamExports];   // (slot, cell) of this workgroup's exports
+    const int k = blockIdx.x;
+    const int lmin = step > 0 ? l0 : l0 - (count - 1);
+    for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
+    for (int i = threadIdx.x; i <= count; i += blockDim.x) {
+        const int l = l0 + (i < count ? i : count - 1) * step - lmin;
+        const int qnow = step > 0 ? a.level_ptr[lmin + l] : a.level_ptr[lmin + l + 1];
+        const int need = t.tab[k * (count + 1) + (i + 1 < count ? i + 1 : count)];
+        const int before = t.tab[(t.P + k) * (count + 1) + i];
+        s_sv[i] = make_int2(step * qnow + kTeamAhead, need | (before << kTeamNeedBits));
+    }
+    {
+        const int32_t *lists = t.tab + 2 * t.P * (count + 1);
+        const int32_t *exp_ds = lists + t.n_imp + t.exp_off[k], *exp_cell = lists + 2 * t.n_imp + t.exp_off[k];
+        const int n_exp = t.exp_off[k + 1] - t.exp_off[k];
+        for (int i = threadIdx.x; i < n_exp; i += blockDim.x) s_exl[i] = make_int2(exp_ds[i], exp_cell[i]);
+    }
+    if (threadIdx.x == 0) ring[kRing] = 0.;
+    __syncthreads();
+    const char *ring_bytes = reinterpret_cast<const char *>(ring);
+    if (threadIdx.x < kTeamChunk) {
+        // the rows: the single-workgroup kernel's level loop on this workgroup's part of a level
+        const uint32_t lane8 = threadIdx.x * 8u;
+        const int shift = k * kTeamChunk;
+        auto part = [&](int it) {
+            Bounds b = load_bounds_uniform(s_lp, it, count, l0, step, lmin);
+            b.qb += shift;
+            return b;
+        };
+        EllVals<PRE> qv[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, part(d));
+        Bounds ahead = part(DEPTH);
+        for (int it0 = 0; it0 < count; it0 += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                const int it = it0 + d;
+                if (it >= count) break;   // uniform over the workgroup
+                const EllVals<PRE> cur = qv[d];
+                qv[d] = load_ell<PRE>(a, ahead);
+                double xj[PRE];
+                uint32_t any = 0;
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) {
+                    xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
+                    any |= cur.ds[e / 2];
+                }
+                ahead = part(it + DEPTH + 1);
+                double acc = 0.;
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
+                const bool live = (int)threadIdx.x < cur.qe - cur.qb;
+                if ((any & kEllFarPair) && live) {
+                    // a row solved by an earlier launch: that value from global memory, the sum in
+                    // the same order.  (Only that value: what this launch computes is taken from
+                    // the ring as ever -- in global memory a value of another workgroup of this
+                    // launch is not ordered before this read.)
+                    const int q = cur.qb + (int)threadIdx.x;
+                    const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
+                    int32_t sl[PRE];
+                    double xg[PRE];
+#pragma unroll
+                    for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
+#pragma unroll
+                    for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
+                    acc = 0.;
+#pragma unroll
+                    for (int e = 0; e < PRE; ++e) {
+                        const bool far = (cur.ds[e / 2] >> ((e & 1) * 16)) & 1u;
+                        acc += e < n ? cur.v[e] * (far ? xg[e] : xj[e]) : 0.;
+                    }
+                }
+                double xi = cur.bv - acc;
+                if (!a.unit) xi /= cur.dv;
+                if (live) {
+                    const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
+                    *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
+                    *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
+                }
+                __syncthreads();
+            }
+        }
+        return;
+    }
+
+    // the two service wavefronts: one hands out, one takes in (as one wavefront they had as many
+    // instructions to issue per level as a row's wavefront, and the barrier waited for them)
+    const int lane = threadIdx.x & 63;
+    if (threadIdx.x < kTeamChunk + 64) {
+        // the values of the level before, now in the ring, that other workgroups wait for; what
+        // a level needs from the tables in LDS is read one level early (a level's chain of
+        // dependent LDS round trips is what the whole workgroup waits for at the barrier)
+        int e0 = 0;
+        int svy = s_sv[0].y;
+        int2 xl = s_exl[lane];
+        for (int it = 0; it < count; ++it) {
+            const int e1 = __builtin_amdgcn_readfirstlane(svy >> kTeamNeedBits);
+            const int2 mine = xl;
+            svy = s_sv[it + 1].y;
+            xl = s_exl[(e1 + lane) & (kTeamExports - 1)];
+            auto hand_out = [&](int2 x) {
+                const double v = ring[x.x & (kRing - 1)];
+                const unsigned long long tag = (unsigned long long)(uint32_t)(x.x + 1) << 32;
+                unsigned long long *cell = t.cells + 2 * (int64_t)x.y;
+                __hip_atomic_store(cell, tag | (uint32_t)__double2loint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(cell + 1, tag | (uint32_t)__double2hiint(v), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            };
+            if (e1 > e0) {
+                if (e0 + lane < e1) hand_out(mine);
+                for (int e = e0 + 64 + lane; e < e1; e += 64) hand_out(s_exl[e]);
+            }
+            e0 = e1;
+            __syncthreads();
+        }
+        return;
+    }
+    const int n_imp = t.imp_off[k + 1] - t.imp_off[k];
+    // this lane's cell of a poll that starts at import 0 (a poll reads 64 cells whatever the
+    // list's length: the mailbox ends with kTeamCellPadding cells that nobody writes)
+    const unsigned long long *cells_lane = t.cells + 2 * ((int64_t)t.imp_off[k] + lane);
+    const unsigned long long *quiet_lane = t.cells + 2 * ((int64_t)t.quiet + lane);
+    int c = 0;   // imports [0, c) are in the ring
+    // A poll reads the two words of 64 cells, from import `cs` on.  Nothing else the loop below
+    // needs comes from device memory: the hardware hands loads back in the order they were
+    // issued, so one fresh load that a level waits for would wait for every poll in flight.
+    auto issue = [&](int cs) {
+        TeamPoll p;
+        p.cs = cs;
+        // (with nothing left to import, the cells that nobody writes: polling cells that another
+        // workgroup is waiting on slows the polls down, and with them this workgroup)
+        const unsigned long long *at = cs < n_imp ? cells_lane + 2 * (int64_t)cs : quiet_lane;
+        p.w0 = __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        p.w1 = __hip_atomic_load(at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return p;
+    };
+    // What a poll found goes into the ring.  A cell's words carry the slot + 1 next to the halves
+    // of the value, 0 while empty.  (A slot too far ahead of this workgroup's own level would land
+    // on a ring entry that its rows still read: it is taken by a later poll.  An import below `c`
+    // is in the ring already: a poll made many levels ago must not write it again, its ring
+    // entry may belong to a newer slot by now.)
+    auto take = [&](const TeamPoll &p, int lim) {
+        const uint32_t tag = (uint32_t)(p.w0 >> 32);
+        const int32_t ds = (int32_t)tag - 1;
+        const int j = p.cs + lane;
+        const bool have = j < n_imp && tag != 0u && (uint32_t)(p.w1 >> 32) == tag;
+        const bool ok = have && j >= c && (step > 0 ? ds : -ds) <= lim;
+        if (ok) ring[ds & (kRing - 1)] = __hiloint2double((int)(uint32_t)p.w1, (int)(uint32_t)p.w0);
+        const unsigned long long m = __ballot(ok || j < c);
+        const int lead = m == ~0ull ? 64 : __builtin_ctzll(~m);
+        c = c > p.cs + lead ? c : p.cs + lead;
+    };
+    const int32_t limit32 = poll_limit > 0x7fffffff ? 0x7fffffff : (poll_limit < 1 ? 1 : (int32_t)poll_limit);
+    if (poll_limit < 0) {   // give up at once (tests)
+        c = 0x3fffffff;
+        if (lane == 0) status[0] = 1;
+    }
+    TeamPoll st[kTeamStages];
+#pragma unroll
+    for (int d = 0; d < kTeamStages; ++d) st[d] = issue(c);
+    // one level: what poll `p` found comes in, and the poll is made again (the level's entry of
+    // the table in LDS is read one level early)
+    int2 cur = s_sv[0];
+    auto serve = [&](int it, TeamPoll &p) {
+        const int need = __builtin_amdgcn_readfirstlane(cur.y & ((1 << kTeamNeedBits) - 1));
+        const int lim = __builtin_amdgcn_readfirstlane(cur.x);
+        cur = s_sv[it + 1];
+        take(p, lim);
+        // everything the next level reads must be in the ring before this level's barrier
+        if (__builtin_expect(c < need, 0)) {
+            int32_t polls = 0;
+            while (c < need) {
+                take(issue(c), lim);
+                if (c >= need) break;
+                if (++polls >= limit32) {
+                    c = 0x3fffffff;   // never waits again; the solve hands out NaN
+                    if (lane == 0) status[0] = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            // (leaves this branch with no load in flight, so that the straight path's wait
+            // counts are those of the polls alone)
+            __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+        }
+        p = issue(c);
+        __syncthreads();
+    };
+    // Whole rounds of kTeamStages levels, then the rest without a way back to the loop's head: on
+    // a path from the middle of a round to the head the polls would have been issued in another
+    // order, and the compiler, which must count for every path, would wait for all of them at
+    // every level.
+    int it = 0;
+    for (; it + kTeamStages <= count; it += kTeamStages) {
+#pragma unroll
+        for (int d = 0; d < kTeamStages; ++d) serve(it + d, st[d]);
+    }
+#pragma unroll
+    for (int d = 0; d < kTeamStages; ++d) {
+        if (it + d >= count) return;
+        serve(it + d, st[d]);
+    }
+}
+
 // One wide level: slots [q0, q1), one lane per row.
 __global__ __launch_bounds__(kBlock) void sptrsv_level_kernel(SolveArgs a, int q0, int q1) {
     const int q = q0 + (int)(blockIdx.x * blockDim.x + threadIdx.x);
@@ -1296,6 +1590,114 @@ __global__ __launch_bounds__(64) void sptrsv_chain_kernel(ChainArgs c) {
 
 // x[order[q]] = xs[q], rounded once to the value type (cpp/sparse_csr_cpu.cpp:722).
 // `status` (may be null): nonzero when a kernel of this solve gave up waiting; x is then NaN throughout.
+// Exchange tables of a launch that P = ceil(width / kTeamChunk) workgroups share, for one solve
+// direction (`dptr`, `dslot`: that direction's packed dependencies on the host; `level_of`: the
+// level of every slot).  Appends to `tab` what TeamArgs::tab describes and fills `T`; returns false
+// (and leaves both alone) when the launch is better left to one workgroup:
+//   * a row reads, through global memory, a row of the same launch (too many slots back for the
+//     ring): between workgroups nothing orders that read after the write;
+//   * at some level the waits "a needs what b computes at the level before" form a cycle: those
+//     workgroups would have to exchange values inside every such level;
+//   * more values cross than a service wavefront polls in passing (16 per workgroup and level
+//     on average), or than the mailbox, the tables or a workgroup's LDS list of exports hold.
+bool build_team(const nm_sptrsv_plan::Launch &L, int d, const std::vector<int32_t> &lp,
+                const std::vector<int32_t> &dptr, const std::vector<int32_t> &dslot,
+                const std::vector<int32_t> &level_of, int64_t cells_left, int64_t ints_left,
+                std::vector<int32_t> &tab, nm_sptrsv_plan::Launch::Team &T) {
+    const int32_t count = L.l1 - L.l0;
+    const int32_t P = (L.width + kTeamChunk - 1) / kTeamChunk;
+    if (P < 2 || P > kTeamMax || count < 16) return false;
+    auto iter_of = [&](int32_t l) { return d == 0 ? l - L.l0 : (L.l1 - 1) - l; };
+    struct Cross { int32_t k, ds, it, kd, itd; };
+    std::vector<Cross> cross;
+    for (int32_t l = L.l0; l < L.l1; ++l)
+        for (int32_t q = lp[l]; q < lp[l + 1]; ++q) {
+            const int32_t k = (q - lp[l]) / kTeamChunk;
+            for (int32_t e = dptr[q]; e < dptr[q + 1]; ++e) {
+                const int32_t ds = dslot[e], ld = level_of[ds];
+                if (ld < L.l0 || ld >= L.l1) continue;   // an earlier launch: ordered by the stream
+                if ((ds > q ? ds - q : q - ds) >= kRingSafe) return false;
+                const int32_t kd = (ds - lp[ld]) / kTeamChunk;
+                if (kd != k) cross.push_back({k, ds, iter_of(l), kd, iter_of(ld)});
+            }
+            if ((int64_t)cross.size() > 4 * cells_left + 1024) return false;
+        }
+    // one import per (workgroup, slot): the first level that needs it
+    std::sort(cross.begin(), cross.end(), [](const Cross &x, const Cross &y) {
+        return x.k != y.k ? x.k < y.k : (x.ds != y.ds ? x.ds < y.ds : x.it < y.it);
+    });
+    cross.erase(std::unique(cross.begin(), cross.end(),
+                            [](const Cross &x, const Cross &y) { return x.k == y.k && x.ds == y.ds; }),
+                cross.end());
+    const int64_t n = (int64_t)cross.size();
+    const int64_t ints = (int64_t)2 * P * (count + 1) + 3 * n;
+    if (n > cells_left || ints > ints_left || n > (int64_t)16 * count * P || n >= (int64_t(1) << kTeamNeedBits))
+        return false;
+    // waits on the level just before, per level: a cycle among them cannot be pipelined away
+    {
+        std::vector<uint16_t> adj((size_t)count, 0);
+        for (const Cross &x : cross)
+            if (x.itd == x.it - 1) adj[x.it] |= (uint16_t)(1u << (x.k * kTeamMax + x.kd));
+        for (int32_t j = 0; j < count; ++j) {
+            if (!adj[j]) continue;
+            bool r[kTeamMax][kTeamMax];
+            for (int u = 0; u < kTeamMax; ++u)
+                for (int v = 0; v < kTeamMax; ++v) r[u][v] = (adj[j] >> (u * kTeamMax + v)) & 1;
+            for (int m = 0; m < kTeamMax; ++m)
+                for (int u = 0; u < kTeamMax; ++u)
+                    for (int v = 0; v < kTeamMax; ++v) r[u][v] = r[u][v] || (r[u][m] && r[m][v]);
+            for (int u = 0; u < kTeamMax; ++u)
+                if (r[u][u]) return false;
+        }
+    }
+    {   // a workgroup's list of exports lives in LDS
+        int64_t out[kTeamMax] = {};
+        for (const Cross &x : cross)
+            if (++out[x.kd] > kTeamExports) return false;
+    }
+    // imports by (workgroup, first level that reads them); an import's place in that order is its cell
+    std::stable_sort(cross.begin(), cross.end(),
+                     [](const Cross &x, const Cross &y) { return x.k != y.k ? x.k < y.k : x.it < y.it; });
+    T.P = P;
+    T.at = (int32_t)tab.size();
+    T.n_imp = (int32_t)n;
+    tab.resize(tab.size() + (size_t)ints, 0);
+    int32_t *need = tab.data() + T.at, *before = need + (size_t)P * (count + 1);
+    int32_t *imp_ds = before + (size_t)P * (count + 1), *exp_ds = imp_ds + n, *exp_cell = exp_ds + n;
+    for (int k = 0; k <= kTeamMax; ++k) T.imp_off[k] = T.exp_off[k] = 0;
+    for (const Cross &x : cross) {
+        ++T.imp_off[x.k + 1];
+        ++T.exp_off[x.kd + 1];
+    }
+    for (int k = 0; k < kTeamMax; ++k) {
+        T.imp_off[k + 1] += T.imp_off[k];
+        T.exp_off[k + 1] += T.exp_off[k];
+    }
+    // need[k][j]: imports of workgroup k that levels up to its j-th read
+    for (int64_t i = 0; i < n; ++i) {
+        imp_ds[i] = cross[i].ds;
+        ++need[(size_t)cross[i].k * (count + 1) + cross[i].it];
+    }
+    for (int k = 0; k < P; ++k)
+        for (int32_t j = 1; j <= count; ++j) need[(size_t)k * (count + 1) + j] += need[(size_t)k * (count + 1) + j - 1];
+    // exports by (workgroup, level that computes them); before[k][j]: those of levels before its j-th
+    std::vector<int64_t> by((size_t)n);
+    for (int64_t i = 0; i < n; ++i) by[i] = i;
+    std::stable_sort(by.begin(), by.end(), [&](int64_t x, int64_t y) {
+        return cross[x].kd != cross[y].kd ? cross[x].kd < cross[y].kd : cross[x].itd < cross[y].itd;
+    });
+    for (int64_t i = 0; i < n; ++i) {
+        const Cross &x = cross[by[i]];
+        exp_ds[i] = x.ds;
+        exp_cell[i] = (int32_t)by[i];
+        if (x.itd + 1 <= count) ++before[(size_t)x.kd * (count + 1) + x.itd + 1];
+    }
+    for (int k = 0; k < P; ++k)
+        for (int32_t j = 1; j <= count; ++j)
+            before[(size_t)k * (count + 1) + j] += before[(size_t)k * (count + 1) + j - 1];
+    return true;
+}
+
 template <typename T>
 __global__ void unslot_kernel(int64_t n, const int32_t *__restrict__ order, const double *__restrict__ xs,
                               T *__restrict__ x, const int32_t *__restrict__ status) {
@@ -1337,7 +1739,8 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
         if (grid > 65536) grid = 65536;
         const T *dat = p->nnz > 0 ? (const T *)data : (const T *)b;
         hipLaunchKernelGGL(gather_ell_kernel<T>, dim3((unsigned)grid), dim3(kBlock), 0, s, p->rows, pre, dat,
-                           (const T *)b, p->order, P.dptr, P.dsrc, P.diag, a.w.ell_coef, a.w.rb, a.w.status);
+                           (const T *)b, p->order, P.dptr, P.dsrc, P.diag, a.w.ell_coef, a.w.rb, a.w.status,
+                           a.w.cells, (int64_t)2 * p->team_cells[dirn]);
         NM_LAUNCH_CHECK("gather_ell_kernel");
     }
     const int n = (int)p->launches.size();
@@ -1405,6 +1808,29 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
                 const int v = e ? atoi(e) : kSkew;
                 return v < 0 ? 0 : (v > kSkew ? kSkew : v);
             }();
+            const auto &TM = L.team[dirn];
+            if (pre > 0 && TM.P > 1 && g_team_enabled.load()) {
+                // several workgroups share every level
+                TeamArgs ta;
+                ta.tab = P.team + TM.at;
+                ta.cells = a.w.cells + 2 * (int64_t)TM.cell0;
+                ta.P = TM.P;
+                ta.n_imp = TM.n_imp;
+                ta.quiet = (int32_t)(team_cells_capacity(p->rows) - TM.cell0);
+                for (int k = 0; k <= kTeamMax; ++k) {
+                    ta.imp_off[k] = TM.imp_off[k];
+                    ta.exp_off[k] = TM.exp_off[k];
+                }
+                const dim3 tg((unsigned)TM.P), tb(kTeamChunk + 128);
+                if (pre == 2)
+                    hipLaunchKernelGGL((sptrsv_team_kernel<2, 4>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status);
+                else if (pre == 4)
+                    hipLaunchKernelGGL((sptrsv_team_kernel<4, 3>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status);
+                else
+                    hipLaunchKernelGGL((sptrsv_team_kernel<8, 2>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status);
+                NM_LAUNCH_CHECK("sptrsv_team_kernel");
+                continue;
+            }
             if (pre == 2 && sig)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4, true>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
                                    limit, a.w.status, tune_sleep, tune_skew);
@@ -1760,9 +2186,46 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
         }
     }
+    // Launches wider than one workgroup's share of a level, in directions with the fixed-width
+    // layout: the tables of what passes between their workgroups, where that can be pipelined.
+    std::vector<int32_t> team_tab[2];
+    {
+        bool any = false;
+        for (const auto &C : p->launches) any = any || (!C.wide && C.width > kTeamChunk);
+        std::vector<int32_t> level_of, dslot_h;
+        if (any && (p->ell_pre[0] > 0 || p->ell_pre[1] > 0)) {
+            level_of.resize((size_t)rows);
+            for (int32_t l = 0; l < p->nlevels; ++l)
+                for (int32_t q = lp[l]; q < lp[l + 1]; ++q) level_of[q] = l;
+        }
+        for (int d = 0; d < 2 && any; ++d) {
+            if (p->ell_pre[d] == 0 || nnz == 0) continue;
+            dslot_h.resize((size_t)nnz);
+            if (hipMemcpyAsync(dslot_h.data(), p->dir[d].dslot, dslot_h.size() * 4, hipMemcpyDeviceToHost, s) !=
+                    hipSuccess ||
+                hipStreamSynchronize(s) != hipSuccess)
+                return bail(nm::fail(NM_ERR_HIP, "reading the dependency slots back failed"));
+            int64_t cells = 0;
+            for (auto &C : p->launches) {
+                if (C.wide || C.chain[d] != 0 || C.width <= kTeamChunk) continue;
+                nm_sptrsv_plan::Launch::Team T;
+                if (!build_team(C, d, lp, dptr_h[d], dslot_h, level_of, team_cells_capacity(rows) - cells,
+                                team_capacity(rows) - (int64_t)team_tab[d].size(), team_tab[d], T))
+                    continue;
+                T.cell0 = (int32_t)cells;
+                cells += T.n_imp;
+                C.team[d] = T;
+            }
+            p->team_cells[d] = (int32_t)cells;
+            if (!team_tab[d].empty() &&
+                hipMemcpyAsync(p->dir[d].team, team_tab[d].data(), team_tab[d].size() * 4, hipMemcpyHostToDevice, s) !=
+                    hipSuccess)
+                return bail(nm::fail(NM_ERR_HIP, "uploading the exchange tables failed"));
+        }
+    }
     int32_t reach_h[2] = {0, 0};
     if (hipMemcpyAsync(reach_h, L.meta + 4, sizeof(reach_h), hipMemcpyDeviceToHost, s) != hipSuccess ||
-        hipStreamSynchronize(s) != hipSuccess)   // also keeps `level_launch` alive until its copy is done
+        hipStreamSynchronize(s) != hipSuccess)   // also keeps `level_launch` and `team_tab` alive until their copies are done
         return bail(nm::fail(NM_ERR_HIP, "waiting for the plan to complete failed"));
     p->reach[0] = reach_h[0];
     p->reach[1] = reach_h[1];
@@ -1781,6 +2244,14 @@ extern "C" int64_t nm_sptrsv_plan_chain_levels(const nm_sptrsv_plan *plan, int t
     int64_t n = 0;
     for (const auto &L : plan->launches)
         if (L.chain[transposed ? 1 : 0] != 0) n += L.l1 - L.l0;
+    return n;
+}
+
+extern "C" int64_t nm_sptrsv_plan_shared_launches(const nm_sptrsv_plan *plan, int transposed) {
+    if (!plan) return -1;
+    int64_t n = 0;
+    for (const auto &L : plan->launches)
+        if (L.team[transposed ? 1 : 0].P > 1) ++n;
     return n;
 }
 
@@ -1869,14 +2340,17 @@ extern "C" int nm_sptrsv_solve_static(const nm_sptrsv_plan *plan, nm_dtype dt, i
     return solve_typed<float>(plan, transposed, data, unit, b, x, work, s);
 }
 
-// Test and diagnostics hooks of the triangular solve's single-workgroup kernels.
-//   poll_limit   polls one wavefront makes at one level before every wavefront of the launch
-//                leaves and the solve hands out NaN (0 restores the default, a negative value
-//                makes the kernels give up at once);
-//   signalling   0 (default): wavefronts meet at a workgroup barrier after every level;
-//                1: neighbours signal, where no row depends on a row more than one wavefront away.
+// Test and diagnostics hooks of the triangular solve's level kernels.
+//   poll_limit   polls one wavefront makes at one level (for its neighbours, or for the values of
+//                another workgroup) before it stops waiting and the solve hands out NaN (0 restores
+//                the default, a negative value makes the kernels give up at once);
+//   signalling   bit 0: wavefronts of a workgroup signal their neighbours, where no row depends on
+//                a row more than one wavefront away, instead of meeting at a barrier after every
+//                level (default off); bit 1: launches that the plan would share among several
+//                workgroups are taken by one (default: shared).
 extern "C" int nm_sptrsv_configure(int64_t poll_limit, int signalling) {
     g_sig_poll_limit.store(poll_limit == 0 ? int64_t(1) << 22 : poll_limit);
-    g_sig_enabled.store(signalling != 0);
+    g_sig_enabled.store((signalling & 1) != 0);
+    g_team_enabled.store((signalling & 2) == 0);
     return NM_OK;
 }

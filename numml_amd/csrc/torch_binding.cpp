@@ -1486,6 +1486,17 @@ std::tuple<int64_t, int64_t> sptrsv_chain_levels(int A_rows, Tensor A_indices, T
     return {nm_sptrsv_plan_chain_levels(plan->handle, 0), nm_sptrsv_plan_chain_levels(plan->handle, 1)};
 }
 
+std::tuple<int64_t, int64_t> sptrsv_shared_launches(int A_rows, Tensor A_indices, Tensor A_indptr, bool lower) {
+    TORCH_CHECK(A_indptr.dim() == 1 && A_indptr.numel() == (int64_t)A_rows + 1 && A_indices.dim() == 1,
+                "sptrsv_shared_launches: expected ", A_rows + 1, " row pointers, got shape ", A_indptr.sizes());
+    const auto dev = need_device({&A_indices, &A_indptr});
+    A_indices = index_tensor(A_indices, "A_indices");
+    A_indptr = index_tensor(A_indptr, "A_indptr");
+    c10::hip::HIPGuard guard(dev.index());
+    auto plan = level_plan(A_indices, A_indptr, A_rows, lower, dev);
+    return {nm_sptrsv_plan_shared_launches(plan->handle, 0), nm_sptrsv_plan_shared_launches(plan->handle, 1)};
+}
+
 // What the transposed-structure plan of a pattern (the cached one, or one built now) found out:
 // (symmetric, packed words of the backward valid, 16-bit column offsets of the forward valid,
 // row blocks with a staging list, row blocks, column blocks with one, column blocks, longest column,
@@ -1598,6 +1609,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sptrsv_schedule", &sptrsv_schedule, "(levels, launches per solve) of a triangular pattern");
     m.def("sptrsv_chain_levels", &sptrsv_chain_levels,
           "levels of the solves with A and with A^T that the single-wavefront chain kernels take");
+    m.def("sptrsv_shared_launches", &sptrsv_shared_launches,
+          "launches of the solves with A and with A^T whose levels several workgroups share");
     m.def("transpose_plan_info", &transpose_plan_info,
           "(symmetric, packed backward, packed forward, staged row blocks, row blocks, staged column blocks, "
           "column blocks) of a pattern's transposed-structure plan");

@@ -25,7 +25,7 @@ __all__ = [
     "csr_transpose_forward", "csr_transpose_backward", "splincomb_forward", "splincomb_backward",
     "csr_to_dense_forward", "csr_to_dense_backward", "csr_row_sum_forward", "csr_row_sum_backward",
     "csr_extract_diagonal_forward", "csr_extract_diagonal_backward",
-    "clear_plan_cache", "plan_cache_size", "sptrsv_schedule", "sptrsv_chain_levels",
+    "clear_plan_cache", "plan_cache_size", "sptrsv_schedule", "sptrsv_chain_levels", "sptrsv_shared_launches",
 ]
 
 
@@ -734,6 +734,8 @@ class _Plan:
         self.launches = int(L.nm_sptrsv_plan_launches(handle))
         self.chain_levels = (int(L.nm_sptrsv_plan_chain_levels(handle, 0)),
                              int(L.nm_sptrsv_plan_chain_levels(handle, 1)))
+        self.shared_launches = (int(L.nm_sptrsv_plan_shared_launches(handle, 0)),
+                                int(L.nm_sptrsv_plan_shared_launches(handle, 1)))
         # nm_sptrsv_analyse synchronised its stream, so the plan is complete for every stream
 
     def __del__(self):
@@ -871,6 +873,18 @@ def sptrsv_chain_levels(A_rows, A_indices, A_indptr, lower):
     with torch.cuda.device(dev):
         plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
     return plan.chain_levels
+
+
+def sptrsv_shared_launches(A_rows, A_indices, A_indptr, lower):
+    """Launches of the solve with A and of the solve with A^T whose levels several workgroups
+    share; diagnostics, no counterpart in the reference."""
+    if A_indptr.dim() != 1 or A_indptr.shape[0] != A_rows + 1 or A_indices.dim() != 1:
+        raise RuntimeError(f"sptrsv_shared_launches: expected {A_rows + 1} row pointers, got shape {list(A_indptr.shape)}")
+    dev = _need_device(A_indices, A_indptr)
+    A_indices, A_indptr = _idx(A_indices, "A_indices"), _idx(A_indptr, "A_indptr")
+    with torch.cuda.device(dev):
+        plan = _plan_for(A_indices, A_indptr, A_rows, lower, dev)
+    return plan.shared_launches
 
 
 def plan_cache_size():

@@ -36,7 +36,7 @@ def test_ctypes_table_covers_the_header():
     L = _lib.lib()
     table = set(_lib._SIGNATURES) | {"nm_version", "nm_last_error", "nm_sptrsv_plan_levels",
                                      "nm_sptrsv_plan_launches", "nm_sptrsv_plan_chain_levels",
-                                     "nm_sptrsv_plan_destroy"}
+                                     "nm_sptrsv_plan_shared_launches", "nm_sptrsv_plan_destroy"}
     assert set(_declared()) == table
     assert L.nm_version() == 1001
     assert L.nm_last_error() == b""

@@ -1,0 +1,130 @@
+"""Triangular solves whose wide levels are shared by several workgroups: each takes 256 rows of
+every level, and the few values a workgroup needs from the others pass through a mailbox in
+device memory while the consumer runs a few levels behind.  The plan shares a launch only
+where that can be pipelined; every case is solved both ways (shared, and by one workgroup) and
+compared bit for bit with the other and with the serial loops of
+cpp/sparse_csr_cpu.cpp:652-759.
+"""
+import numpy as np
+import pytest
+import scipy.sparse as sps
+import torch
+
+import oracle
+from numml_amd import _lib
+from numml_amd import generators as G
+from numml_amd import numml_torch_cpp as ext
+from util import assert_same, host, randn, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _csr(M, dtype):
+    M = sps.csr_matrix(M).astype(dtype)
+    M.sort_indices()
+    return M.data.copy(), M.indices.astype(np.int64), M.indptr.astype(np.int64), M.shape[0]
+
+
+def _generations(gens, width, offsets, seed):
+    """Row j of generation g depends on rows j + o (o in `offsets`) of generation g - 1: every
+    generation is one level of `width` rows."""
+    rng = np.random.default_rng(seed)
+    n = gens * width
+    rows, cols = [np.arange(n)], [np.arange(n)]
+    g, j = np.divmod(np.arange(width, n), width)
+    for o in offsets:
+        ok = (j + o >= 0) & (j + o < width)
+        rows.append((g * width + j)[ok])
+        cols.append(((g - 1) * width + j + o)[ok])
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    vals = np.where(rows == cols, rng.uniform(1.0, 1.5, rows.size), rng.uniform(-0.3, 0.3, rows.size))
+    return sps.csr_matrix((vals, (rows, cols)), shape=(n, n))
+
+
+def _stencil9_lower(n, seed):
+    """Lower triangle of the 2D nine-point stencil on an n x n grid."""
+    rng = np.random.default_rng(seed)
+    idx = np.arange(n * n).reshape(n, n)
+    rows, cols = [idx.ravel()], [idx.ravel()]
+    for di, dj in ((-1, -1), (-1, 0), (-1, 1), (0, -1)):
+        i0, i1 = max(0, -di), n - max(0, di)
+        j0, j1 = max(0, -dj), n - max(0, dj)
+        rows.append(idx[i0:i1, j0:j1].ravel())
+        cols.append(idx[i0 + di:i1 + di, j0 + dj:j1 + dj].ravel())
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    vals = np.where(rows == cols, rng.uniform(1.0, 1.5, rows.size), rng.uniform(-0.2, 0.2, rows.size))
+    return sps.csr_matrix((vals, (rows, cols)), shape=(n * n, n * n))
+
+
+def _cases():
+    # name, matrix, lower, unit, dtype, shared launches expected (forward solve, transposed solve)
+    d, i, p, (n, _) = G.poisson2d_lower(300, np.float64, diag_seed=5)
+    tril = sps.csr_matrix((d, i, p), shape=(n, n))
+    yield "tril of the 300^2 five-point matrix", tril, True, False, np.float64, (True, True)
+    # (off-diagonal row sums below one, so that the unit-diagonal solve stays bounded)
+    damped = sps.tril(tril, -1) * 0.3 + sps.diags(tril.diagonal())
+    yield "the same, unit diagonal, fp32", damped.tocsr(), True, True, np.float32, (True, True)
+    d, i, p, (n, _) = G.poisson2d_lower(560, np.float64, diag_seed=6)
+    triu = sps.csr_matrix((d, i, p), shape=(n, n)).T.tocsr()
+    yield "triu of the 560^2 five-point matrix (three workgroups)", triu, False, False, np.float64, (True, True)
+    yield "tril of the 640^2 nine-point matrix", _stencil9_lower(640, 7), True, False, np.float64, (True, True)
+    # dependencies on one side only: the consumer falls behind its producer once
+    yield "levels of 700 rows, neighbours below", _generations(40, 700, (-2, -1, 0), 8), True, False, np.float64, (True, None)
+    # both neighbours: two workgroups would wait for each other at every level
+    yield "levels of 700 rows, neighbours on both sides", _generations(40, 700, (-1, 0, 1), 9), True, False, \
+        np.float64, (False, False)
+    # far more values would cross than a wavefront polls in passing
+    rng = np.random.default_rng(10)
+    scattered = _generations(30, 600, (0,), 10).tolil()
+    for g in range(1, 30):
+        for j in range(0, 600, 2):
+            scattered[g * 600 + j, (g - 1) * 600 + int(rng.integers(0, 600))] = 0.1
+    yield "levels of 600 rows, scattered dependencies", scattered.tocsr(), True, False, np.float64, (False, None)
+
+
+def test_shared_launches_match_one_workgroup_and_the_serial_loop(dev):
+    L = _lib.lib()
+    try:
+        for name, M, lower, unit, dtype, expect in _cases():
+            d, i, p, n = _csr(M, dtype)
+            b, g = randn(21, n, dtype), randn(22, n, dtype)
+            x_ref = oracle.sptrsv_forward(n, n, d, i, p, lower, unit, b)
+            gA_ref, gb_ref = oracle.sptrsv_backward(g, x_ref, n, n, d, i, p, lower, unit)
+            D, I, P, Bv, Gv = to_dev(dev, d, i, p, b, g)
+            shared = ext.sptrsv_shared_launches(n, I, P, lower)
+            for dirn, want in enumerate(expect):
+                if want is not None:
+                    assert (shared[dirn] > 0) == want, f"{name}: shared launches {shared}"
+            got = {}
+            for one_workgroup in (0, 2):
+                assert L.nm_sptrsv_configure(0, one_workgroup) == 0
+                x = ext.sptrsv_forward(n, n, D, I, P, lower, unit, Bv)
+                gA, gb = ext.sptrsv_backward(Gv, x, n, n, D, I, P, lower, unit, Bv)
+                got[one_workgroup] = (host(x), host(gA), host(gb))
+            for a, c, what in zip(got[0], got[2], ("x", "grad_A", "grad_b")):
+                assert_same(a, c, f"{name}: {what}, shared against one workgroup")
+            assert_same(got[0][0], x_ref, f"{name}: x")
+            assert_same(got[0][1], gA_ref, f"{name}: grad_A")
+            assert_same(got[0][2], gb_ref, f"{name}: grad_b")
+    finally:
+        assert L.nm_sptrsv_configure(0, 0) == 0
+
+
+def test_shared_launch_gives_up_instead_of_waiting_forever(dev):
+    """With the poll limit forced from the host no workgroup waits for another: the call returns
+    and x is NaN throughout instead of wrong."""
+    L = _lib.lib()
+    d, i, p, (n, _) = G.poisson2d_lower(300, np.float64, diag_seed=2)
+    b = randn(3, n, np.float64)
+    D, I, P, Bv = to_dev(dev, d, i, p, b)
+    assert ext.sptrsv_shared_launches(n, I, P, True)[0] > 0
+    x_ref = oracle.sptrsv_forward(n, n, d, i, p, True, False, b)
+    try:
+        assert L.nm_sptrsv_configure(-1, 0) == 0
+        x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
+        torch.cuda.synchronize()
+        assert bool(torch.isnan(x).all())
+    finally:
+        assert L.nm_sptrsv_configure(0, 0) == 0
+    x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
+    assert_same(host(x), x_ref, "x after the defaults were restored")
