@@ -72,7 +72,7 @@ inline int64_t coef_capacity(int64_t rows, int64_t nnz) {
 }
 // Launches that several workgroups share (see sptrsv_team_kernel): most workgroups, values that
 // may pass between workgroups in one solve direction, ints of the tables that say which.
-constexpr int kTeamMax = 4;
+constexpr int kTeamMax = 16;
 inline int64_t team_cells_capacity(int64_t rows) { return rows / 16 + 2048; }
 constexpr int64_t kTeamCellPadding = 64;   // readable cells past the last one (a poll reads 64 at a time)
 inline int64_t team_capacity(int64_t rows) { return 3 * team_cells_capacity(rows) + rows / 16 + 16384; }
@@ -101,6 +101,9 @@ struct nm_sptrsv_plan {
         int32_t chain[2] = {0, 0};
         int64_t chain_at[2] = {0, 0};
         bool chain_candidate = false;
+        // a stretch of levels wider than one workgroup takes, none wider than a team takes: shared
+        // by a team in the directions that have one, else launched level by level like `wide` ones
+        bool run = false;
         // per direction: the workgroups that share every level of the launch (0: one workgroup
         // takes it), where the tables of their exchange start in Packed::team, the first of their
         // mailbox cells, and each workgroup's part of the import and export lists
@@ -111,6 +114,7 @@ struct nm_sptrsv_plan {
     };
     std::vector<Launch> launches;
     int32_t team_cells[2] = {0, 0};   // mailbox cells one solve clears, per direction
+    std::vector<int32_t> lp_host;     // level_ptr on the host (the level-by-level launches of a run)
 };
 
 namespace {
@@ -1098,8 +1102,8 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
                                                                        int64_t poll_limit, int32_t *status) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
     __shared__ int32_t s_lp[kMaxLevels + 1];
-    // what the service wavefront needs at a level, in one LDS read: x = the limit an imported
-    // slot is held against (times `step`), y = imports the NEXT level needs (low kTeamNeedBits
+    // what the service wavefronts need at a level, in one LDS read: x = the limit an imported
+    // slot (times `step`) is held against, y = imports the NEXT level needs (low kTeamNeedBits
     // bits) and exports of the levels before this one (the bits above)
     __shared__ int2 s_sv[kMaxLevels + 1];
     __shared__ int2 s_exl[kTeamExports];   // (slot, cell) of this workgroup's exports
@@ -1107,11 +1111,16 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
     for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
     for (int i = threadIdx.x; i <= count; i += blockDim.x) {
+        // An imported slot lands on the ring entry of the slot kRing before it, which this
+        // workgroup's rows read as long as it is less than kRingSafe behind them: a slot may come
+        // in once it is at most kTeamAhead past the first of the workgroup's rows of the level
+        // (solving A^T the slots descend: at most kTeamAhead below the last of them).
         const int l = l0 + (i < count ? i : count - 1) * step - lmin;
-        const int qnow = step > 0 ? a.level_ptr[lmin + l] : a.level_ptr[lmin + l + 1];
+        const int mine = a.level_ptr[lmin + l] + k * kTeamChunk;
+        const int lim = step > 0 ? mine + kTeamAhead : -(mine + kTeamChunk - 1) + kTeamAhead;
         const int need = t.tab[k * (count + 1) + (i + 1 < count ? i + 1 : count)];
         const int before = t.tab[(t.P + k) * (count + 1) + i];
-        s_sv[i] = make_int2(step * qnow + kTeamAhead, need | (before << kTeamNeedBits));
+        s_sv[i] = make_int2(lim, need | (before << kTeamNeedBits));
     }
     {
         const int32_t *lists = t.tab + 2 * t.P * (count + 1);
@@ -1126,9 +1135,11 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
         // the rows: the single-workgroup kernel's level loop on this workgroup's part of a level
         const uint32_t lane8 = threadIdx.x * 8u;
         const int shift = k * kTeamChunk;
+        // (a workgroup without rows in a level starts at the level's end: its lanes load the
+        // operands of the kTeamChunk slots from there on, and those are readable)
         auto part = [&](int it) {
             Bounds b = load_bounds_uniform(s_lp, it, count, l0, step, lmin);
-            b.qb += shift;
+            b.qb = b.qb + shift < b.qe ? b.qb + shift : b.qe;
             return b;
         };
         EllVals<PRE> qv[DEPTH];
@@ -1598,6 +1609,8 @@ __global__ __launch_bounds__(64) void sptrsv_chain_kernel(ChainArgs c) {
 //     ring): between workgroups nothing orders that read after the write;
 //   * at some level the waits "a needs what b computes at the level before" form a cycle: those
 //     workgroups would have to exchange values inside every such level;
+//   * the direction in which values cross between two workgroups changes more than once in 32
+//     levels: every change costs a hand-over's latency;
 //   * more values cross than a service wavefront polls in passing (16 per workgroup and level
 //     on average), or than the mailbox, the tables or a workgroup's LDS list of exports hold.
 bool build_team(const nm_sptrsv_plan::Launch &L, int d, const std::vector<int32_t> &lp,
@@ -1635,20 +1648,42 @@ bool build_team(const nm_sptrsv_plan::Launch &L, int d, const std::vector<int32_
         return false;
     // waits on the level just before, per level: a cycle among them cannot be pipelined away
     {
-        std::vector<uint16_t> adj((size_t)count, 0);
+        std::vector<uint16_t> adj((size_t)count * kTeamMax, 0);   // [level][consumer]: its producers
+        std::vector<uint8_t> any_edge((size_t)count, 0);
         for (const Cross &x : cross)
-            if (x.itd == x.it - 1) adj[x.it] |= (uint16_t)(1u << (x.k * kTeamMax + x.kd));
+            if (x.itd == x.it - 1) {
+                adj[(size_t)x.it * kTeamMax + x.k] |= (uint16_t)(1u << x.kd);
+                any_edge[x.it] = 1;
+            }
+        static_assert(kTeamMax <= 16, "a workgroup's producers fit sixteen bits");
         for (int32_t j = 0; j < count; ++j) {
-            if (!adj[j]) continue;
-            bool r[kTeamMax][kTeamMax];
-            for (int u = 0; u < kTeamMax; ++u)
-                for (int v = 0; v < kTeamMax; ++v) r[u][v] = (adj[j] >> (u * kTeamMax + v)) & 1;
+            if (!any_edge[j]) continue;
+            uint16_t r[kTeamMax];
+            for (int u = 0; u < kTeamMax; ++u) r[u] = adj[(size_t)j * kTeamMax + u];
             for (int m = 0; m < kTeamMax; ++m)
                 for (int u = 0; u < kTeamMax; ++u)
-                    for (int v = 0; v < kTeamMax; ++v) r[u][v] = r[u][v] || (r[u][m] && r[m][v]);
+                    if ((r[u] >> m) & 1) r[u] |= r[m];
             for (int u = 0; u < kTeamMax; ++u)
-                if (r[u][u]) return false;
+                if ((r[u] >> u) & 1) return false;
         }
+    }
+    // A consumer runs a few levels behind its producer, and the hand-over's latency is paid once.
+    // Where the direction between two workgroups changes, it is paid again (the workgroup that
+    // was ahead must now wait for the one that was behind): a triangle whose dependencies cross
+    // the cut now this way, now that (the nine-point stencil's alternate from level to level) is
+    // faster on one workgroup.  One change per 32 levels is what a shared level's gain pays for.
+    {
+        std::vector<Cross> byit(cross);
+        std::stable_sort(byit.begin(), byit.end(), [](const Cross &x, const Cross &y) { return x.it < y.it; });
+        int8_t last[kTeamMax][kTeamMax] = {};
+        int64_t changes = 0;
+        for (const Cross &x : byit) {
+            const int lo = x.k < x.kd ? x.k : x.kd, hi = x.k < x.kd ? x.kd : x.k;
+            const int8_t dirn = x.k < x.kd ? 1 : 2;
+            if (last[lo][hi] != 0 && last[lo][hi] != dirn) ++changes;
+            last[lo][hi] = dirn;
+        }
+        if (changes * 32 > count) return false;
     }
     {   // a workgroup's list of exports lives in LDS
         int64_t out[kTeamMax] = {};
@@ -1719,7 +1754,10 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
     a.dslot = P.dslot;
     a.unit = unit;
     bool any_wide = false;
-    for (const auto &L : p->launches) any_wide = any_wide || L.wide;
+    const bool teams = g_team_enabled.load();
+    for (const auto &L : p->launches)
+        any_wide = any_wide || L.wide ||
+                   (L.run && !(teams && p->ell_pre[transposed ? 1 : 0] > 0 && L.team[transposed ? 1 : 0].P > 1));
     if (any_wide || p->ell_pre[transposed ? 1 : 0] == 0) {   // the range-based arrays have readers
         int64_t m = p->nnz > p->rows ? p->nnz : p->rows;
         int64_t grid = nm::ceil_div(m, kBlock);
@@ -1780,18 +1818,24 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
                 else hipLaunchKernelGGL((sptrsv_chain_kernel<false, false>), dim3(1), dim3(64), 0, s, c);
             }
             NM_LAUNCH_CHECK("sptrsv_chain_kernel");
-        } else if (L.wide) {
+        } else if (L.wide || (L.run && !(teams && pre > 0 && L.team[dirn].P > 1))) {
+            // a grid launch per level (a run without a team: its levels one after the other)
             const int G = L.group[dirn] > 0 ? L.group[dirn] : 1;
-            const unsigned grid = (unsigned)nm::ceil_div((int64_t)(L.q1 - L.q0) * G, kBlock);
-            if (G == 16)
-                hipLaunchKernelGGL(sptrsv_level_group_kernel<16>, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
-            else if (G == 8)
-                hipLaunchKernelGGL(sptrsv_level_group_kernel<8>, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
-            else if (G == 4)
-                hipLaunchKernelGGL(sptrsv_level_group_kernel<4>, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
-            else
-                hipLaunchKernelGGL(sptrsv_level_kernel, dim3(grid), dim3(kBlock), 0, s, a, L.q0, L.q1);
-            NM_LAUNCH_CHECK("sptrsv_level_kernel");
+            const int nl = L.l1 - L.l0;
+            for (int j = 0; j < nl; ++j) {
+                const int l = transposed ? L.l1 - 1 - j : L.l0 + j;
+                const int q0 = L.wide ? L.q0 : p->lp_host[l], q1 = L.wide ? L.q1 : p->lp_host[l + 1];
+                const unsigned grid = (unsigned)nm::ceil_div((int64_t)(q1 - q0) * G, kBlock);
+                if (G == 16)
+                    hipLaunchKernelGGL(sptrsv_level_group_kernel<16>, dim3(grid), dim3(kBlock), 0, s, a, q0, q1);
+                else if (G == 8)
+                    hipLaunchKernelGGL(sptrsv_level_group_kernel<8>, dim3(grid), dim3(kBlock), 0, s, a, q0, q1);
+                else if (G == 4)
+                    hipLaunchKernelGGL(sptrsv_level_group_kernel<4>, dim3(grid), dim3(kBlock), 0, s, a, q0, q1);
+                else
+                    hipLaunchKernelGGL(sptrsv_level_kernel, dim3(grid), dim3(kBlock), 0, s, a, q0, q1);
+                NM_LAUNCH_CHECK("sptrsv_level_kernel");
+            }
         } else {
             const int count = L.l1 - L.l0;
             const int l0 = transposed ? L.l1 - 1 : L.l0, step = transposed ? -1 : 1;
@@ -1809,7 +1853,7 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
                 return v < 0 ? 0 : (v > kSkew ? kSkew : v);
             }();
             const auto &TM = L.team[dirn];
-            if (pre > 0 && TM.P > 1 && g_team_enabled.load()) {
+            if (pre > 0 && TM.P > 1 && teams) {
                 // several workgroups share every level
                 TeamArgs ta;
                 ta.tab = P.team + TM.at;
@@ -2068,19 +2112,42 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
             return bail(nm::fail(NM_ERR_HIP, "reading the dependency counts back failed"));
     }
     auto level_entries = [&](int d, int32_t l) { return dptr_h[d][lp[l + 1]] - dptr_h[d][lp[l]]; };
-    int32_t run0 = -1;
-    for (int32_t l = 0; l < p->nlevels; ++l) {
+    auto is_wide = [&](int32_t l) {
         const int32_t width = lp[l + 1] - lp[l];
         const int32_t entries = level_entries(0, l) > level_entries(1, l) ? level_entries(0, l) : level_entries(1, l);
-        const bool wide = width > kNarrow || (width >= kWideRows && entries >= kWideEntries);
-        if (!wide) {
+        return width > kNarrow || (width >= kWideRows && entries >= kWideEntries);
+    };
+    // levels wider than one workgroup takes but not than a team of them: a stretch of at least
+    // kRunMin becomes one launch that a team may share (build_team decides per direction)
+    constexpr int32_t kRunMin = 16;
+    auto team_width = [&](int32_t l) {
+        const int32_t width = lp[l + 1] - lp[l];
+        return width > kNarrow && width <= kTeamMax * kTeamChunk;
+    };
+    int32_t run0 = -1;
+    for (int32_t l = 0; l < p->nlevels; ++l) {
+        if (!is_wide(l)) {
             if (run0 < 0) run0 = l;
             continue;
         }
         if (run0 >= 0) { push_narrow(run0, l); run0 = -1; }
+        int32_t e = l;
+        while (e < p->nlevels && team_width(e)) ++e;
+        if (e - l >= kRunMin) {
+            const int32_t pieces = (e - l + kMaxLevels - 1) / kMaxLevels;
+            const int32_t each = (e - l + pieces - 1) / pieces;
+            for (int32_t c0 = l; c0 < e; c0 += each) {
+                const int32_t c1 = c0 + each < e ? c0 + each : e;
+                p->launches.push_back({c0, c1, lp[c0], lp[c1], false, kBlock});
+                p->launches.back().run = true;
+            }
+            l = e - 1;
+            continue;
+        }
         p->launches.push_back({l, l + 1, lp[l], lp[l + 1], true, kBlock});
     }
     if (run0 >= 0) push_narrow(run0, p->nlevels);
+    p->lp_host = lp;
     // Rows long enough to be shared by several lanes: decided per launch and direction from the
     // mean number of dependencies of its rows, where no fixed-width layout serves the direction.
     for (auto &L : p->launches) {
@@ -2091,7 +2158,7 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         for (auto &L : p->launches) {
             if (L.q1 <= L.q0) continue;
             const double mean = double(dptr_h[d][L.q1] - dptr_h[d][L.q0]) / double(L.q1 - L.q0);
-            if (L.wide) {
+            if (L.wide || L.run) {
                 // a level of its own: lanes per row by its mean row length
                 L.group[d] = mean >= 10. ? 16 : (mean >= 5. ? 8 : (mean >= 2.5 ? 4 : 0));
                 continue;

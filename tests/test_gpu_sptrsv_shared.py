@@ -67,11 +67,20 @@ def _cases():
     d, i, p, (n, _) = G.poisson2d_lower(560, np.float64, diag_seed=6)
     triu = sps.csr_matrix((d, i, p), shape=(n, n)).T.tocsr()
     yield "triu of the 560^2 five-point matrix (three workgroups)", triu, False, False, np.float64, (True, True)
-    yield "tril of the 640^2 nine-point matrix", _stencil9_lower(640, 7), True, False, np.float64, (True, True)
+    # the nine-point stencil's dependencies cross the cut in alternating directions from level to
+    # level once the levels shrink: the launches of the growing half are shared, the others not
+    yield "tril of the 640^2 nine-point matrix", _stencil9_lower(640, 7), True, False, np.float64, (None, None)
     # dependencies on one side only: the consumer falls behind its producer once
     yield "levels of 700 rows, neighbours below", _generations(40, 700, (-2, -1, 0), 8), True, False, np.float64, (True, None)
     # both neighbours: two workgroups would wait for each other at every level
     yield "levels of 700 rows, neighbours on both sides", _generations(40, 700, (-1, 0, 1), 9), True, False, \
+        np.float64, (False, False)
+    # levels wider than one workgroup takes (1024 rows): a team of up to sixteen shares them ...
+    d, i, p, (n, _) = G.poisson2d_lower(1300, np.float64, diag_seed=11)
+    yield "tril of the 1300^2 five-point matrix (levels of up to 1300 rows)", sps.csr_matrix((d, i, p), shape=(n, n)), \
+        True, False, np.float64, (True, True)
+    # ... and where no team can, such a stretch of levels is launched level by level
+    yield "levels of 1500 rows, neighbours on both sides", _generations(24, 1500, (-1, 0, 1), 12), True, False, \
         np.float64, (False, False)
     # far more values would cross than a wavefront polls in passing
     rng = np.random.default_rng(10)
