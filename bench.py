@@ -745,7 +745,7 @@ class SpTRSV(Workload):
         s = 8
         self.bytes_per_step = 2 * (self.nnz * (s + 8) + (rows + 1) * 8 + 2 * rows * s) + self.nnz * s
         self.dominant_bytes = self.nnz * (s + 8) + (rows + 1) * 8 + 2 * rows * s
-        self.dominant_name = "forward solve: gather_ell_kernel + sptrsv_ell_kernel + unslot_kernel"
+        self.dominant_name = "forward solve: gather_ell_kernel + sptrsv_ell_kernel / sptrsv_team_kernel + unslot_kernel"
         self.config = {"workload": "sptrsv_fwd_bwd_f64_tril_poisson2d_1024", "rows": rows, "nnz": self.nnz,
                        "levels": 2 * n - 1, "analysis_plus_first_solve_ms": round(self.analysis_ms, 3)}
 
@@ -762,7 +762,7 @@ class SpTRSV(Workload):
         x = self.dominant()
         s = 8
         return [(self.dominant_name, self.dominant, self.dominant_bytes, "*"),
-                ("backward: transposed solve (the same three kernels on the packed A^T) + spmv_bwd_kernel as the masked outer product",
+                ("backward: transposed solve (the same kernels on the packed A^T) + spmv_bwd_kernel as the masked outer product",
                  lambda: self.ext.sptrsv_backward(self.Gv, x, self.rows, self.rows, self.D, self.I, self.P, True, False, self.Bv),
                  self.dominant_bytes + self.nnz * (s + 8) + 2 * self.rows * s, ("*", "spmv_bwd_kernel"))]
 
