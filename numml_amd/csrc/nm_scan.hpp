@@ -40,14 +40,32 @@ __device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t *s_wa
     return before + inc - v;
 }
 
+// Whether this workgroup's tile lies inside a[0, n) whole and a's 16-byte pairs are aligned
+// (uniform over the workgroup).
+typedef int64_t I64x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ bool scan_tile_whole(const int64_t *a, int64_t n) {
+    static_assert(kScanItems % 2 == 0, "items are loaded in pairs");
+    return ((int64_t)blockIdx.x + 1) * kScanTile <= n && (reinterpret_cast<uintptr_t>(a) & 15) == 0;
+}
+
 static __global__ __launch_bounds__(kScanBlock) void scan_tile_sums_kernel(const int64_t *__restrict__ a, int64_t n,
                                                                     int64_t *__restrict__ sums) {
     __shared__ int64_t s_wave[kScanBlock / kWave];
     const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
     int64_t v = 0;
+    if (scan_tile_whole(a, n)) {
+        // a whole tile: the lane's 64 bytes in four 16-byte loads, no test per item
+        const I64x2 *p = reinterpret_cast<const I64x2 *>(a + base);
 #pragma unroll
-    for (int i = 0; i < kScanItems; ++i)
-        if (base + i < n) v += a[base + i];
+        for (int i = 0; i < kScanItems / 2; ++i) {
+            const I64x2 w = p[i];
+            v += w[0] + w[1];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kScanItems; ++i)
+            if (base + i < n) v += a[base + i];
+    }
     int64_t total;
     block_exclusive_scan(v, s_wave, total);
     if (threadIdx.x == 0) sums[blockIdx.x] = total;
@@ -74,17 +92,41 @@ static __global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(int64_t *
     const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
     int64_t item[kScanItems];
     int64_t v = 0;
+    const bool whole = scan_tile_whole(a, n);
+    if (whole) {
+        const I64x2 *p = reinterpret_cast<const I64x2 *>(a + base);
 #pragma unroll
-    for (int i = 0; i < kScanItems; ++i) {
-        item[i] = base + i < n ? a[base + i] : 0;
-        v += item[i];
+        for (int i = 0; i < kScanItems / 2; ++i) {
+            const I64x2 w = p[i];
+            item[2 * i] = w[0];
+            item[2 * i + 1] = w[1];
+            v += w[0] + w[1];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kScanItems; ++i) {
+            item[i] = base + i < n ? a[base + i] : 0;
+            v += item[i];
+        }
     }
     int64_t total;
     int64_t run = sums[blockIdx.x] + block_exclusive_scan(v, s_wave, total);
+    if (whole) {
+        I64x2 *p = reinterpret_cast<I64x2 *>(a + base);
 #pragma unroll
-    for (int i = 0; i < kScanItems; ++i) {
-        if (base + i < n) a[base + i] = run;
-        run += item[i];
+        for (int i = 0; i < kScanItems / 2; ++i) {
+            I64x2 w;
+            w[0] = run;
+            w[1] = run + item[2 * i];
+            run = w[1] + item[2 * i + 1];
+            p[i] = w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kScanItems; ++i) {
+            if (base + i < n) a[base + i] = run;
+            run += item[i];
+        }
     }
 }
 
