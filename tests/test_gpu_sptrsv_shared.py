@@ -143,3 +143,29 @@ def test_shared_launch_gives_up_instead_of_waiting_forever(dev):
         assert L.nm_sptrsv_configure(0, 0) == 0
     x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
     assert_same(host(x), x_ref, "x after the defaults were restored")
+
+
+def test_shared_launch_in_a_graph(dev):
+    """A captured solve with shared launches, replayed with eager solves of another right-hand side
+    in between: every replay empties the mailbox again (the gathering kernel does, inside the
+    graph) and gives the serial loop's bits."""
+    from numml_amd._binding import ops
+    d, i, p, (n, _) = G.poisson2d_lower(300, np.float64, diag_seed=4)
+    D, I, P = to_dev(dev, d, i, p)
+    B = to_dev(dev, randn(1, n, np.float64))[0]
+    other = to_dev(dev, randn(9, n, np.float64))[0]
+    x0 = ops.sptrsv_forward(n, n, D, I, P, True, False, B)      # analysis happens here, once
+    torch.cuda.synchronize()
+    assert ext.sptrsv_shared_launches(n, I, P, True)[0] > 0
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        x = ops.sptrsv_forward(n, n, D, I, P, True, False, B)
+    for seed in (2, 3, 4):
+        b_h = randn(seed, n, np.float64)
+        B.copy_(torch.from_numpy(b_h))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_same(host(x), oracle.sptrsv_forward(n, n, d, i, p, True, False, b_h), f"replayed solve {seed}")
+        eager = ops.sptrsv_forward(n, n, D, I, P, True, False, other)
+        torch.cuda.synchronize()
+        assert_same(host(eager), oracle.sptrsv_forward(n, n, d, i, p, True, False, host(other)), "eager solve between replays")
