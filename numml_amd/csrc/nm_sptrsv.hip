@@ -1601,40 +1601,63 @@ __global__ __launch_bounds__(64) void sptrsv_chain_kernel(ChainArgs c) {
 
 // x[order[q]] = xs[q], rounded once to the value type (cpp/sparse_csr_cpu.cpp:722).
 // `status` (may be null): nonzero when a kernel of this solve gave up waiting; x is then NaN throughout.
+// The dependencies of one solve direction that cross between the 256-row parts of the levels of
+// a launch that a team may share: (launch, consumer's part, dependency's slot, consumer's level,
+// dependency's level) per crossing, appended in no particular order; `bad[launch]` is raised when
+// a row of the launch depends on a row of the same launch too many slots back for the ring.
+// `cand_l0[launch]` is the launch's first level, -1 when it is no candidate in this direction.
+constexpr int kCrossInts = 5;
+__global__ void team_cross_kernel(int64_t rows, const int32_t *__restrict__ dptr, const int32_t *__restrict__ dslot,
+                                  const int32_t *__restrict__ level_ptr, int32_t nlevels,
+                                  const int32_t *__restrict__ level_launch, const int32_t *__restrict__ cand_l0,
+                                  const int32_t *__restrict__ cand_l1, int32_t *__restrict__ out, int32_t capacity,
+                                  int32_t *__restrict__ count, int32_t *__restrict__ bad) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < rows; q += stride) {
+        const int32_t l = level_of_slot(level_ptr, nlevels, (int32_t)q);
+        const int32_t li = level_launch[l];
+        if (li < 0) continue;
+        const int32_t l0 = cand_l0[li], l1 = cand_l1[li];
+        if (l0 < 0) continue;
+        const int32_t k = ((int32_t)q - level_ptr[l]) / kTeamChunk;
+        for (int32_t e = dptr[q]; e < dptr[q + 1]; ++e) {
+            const int32_t ds = dslot[e];
+            const int32_t ld = level_of_slot(level_ptr, nlevels, ds);
+            if (ld < l0 || ld >= l1) continue;   // an earlier launch: ordered by the stream
+            if ((ds > (int32_t)q ? ds - (int32_t)q : (int32_t)q - ds) >= kRingSafe) {
+                bad[li] = 1;
+                continue;
+            }
+            const int32_t kd = (ds - level_ptr[ld]) / kTeamChunk;
+            if (kd == k) continue;
+            const int32_t at = atomicAdd(count, 1);
+            if (at < capacity) {
+                int32_t *r = out + (int64_t)at * kCrossInts;
+                r[0] = li; r[1] = k; r[2] = ds; r[3] = l; r[4] = ld;
+            }
+        }
+    }
+}
+
 // Exchange tables of a launch that P = ceil(width / kTeamChunk) workgroups share, for one solve
-// direction (`dptr`, `dslot`: that direction's packed dependencies on the host; `level_of`: the
-// level of every slot).  Appends to `tab` what TeamArgs::tab describes and fills `T`; returns false
-// (and leaves both alone) when the launch is better left to one workgroup:
-//   * a row reads, through global memory, a row of the same launch (too many slots back for the
-//     ring): between workgroups nothing orders that read after the write;
+// direction, from the dependencies that cross between the workgroups' parts of its levels
+// (`cross`, collected on the device by team_cross_kernel, which also rules out a launch in which
+// a row reads, through global memory, a row of the same launch -- too many slots back for the
+// ring: between workgroups nothing orders that read after the write).  Appends to `tab` what
+// TeamArgs::tab describes and fills `T`; returns false (and leaves both alone) when the launch is
+// better left to one workgroup:
 //   * at some level the waits "a needs what b computes at the level before" form a cycle: those
 //     workgroups would have to exchange values inside every such level;
 //   * the direction in which values cross between two workgroups changes more than once in 32
 //     levels: every change costs a hand-over's latency;
 //   * more values cross than a service wavefront polls in passing (16 per workgroup and level
 //     on average), or than the mailbox, the tables or a workgroup's LDS list of exports hold.
-bool build_team(const nm_sptrsv_plan::Launch &L, int d, const std::vector<int32_t> &lp,
-                const std::vector<int32_t> &dptr, const std::vector<int32_t> &dslot,
-                const std::vector<int32_t> &level_of, int64_t cells_left, int64_t ints_left,
+struct Cross { int32_t k, ds, it, kd, itd; };   // workgroup k needs slot ds at its level `it`; kd computes it at `itd`
+bool build_team(const nm_sptrsv_plan::Launch &L, std::vector<Cross> &cross, int64_t cells_left, int64_t ints_left,
                 std::vector<int32_t> &tab, nm_sptrsv_plan::Launch::Team &T) {
     const int32_t count = L.l1 - L.l0;
     const int32_t P = (L.width + kTeamChunk - 1) / kTeamChunk;
     if (P < 2 || P > kTeamMax || count < 16) return false;
-    auto iter_of = [&](int32_t l) { return d == 0 ? l - L.l0 : (L.l1 - 1) - l; };
-    struct Cross { int32_t k, ds, it, kd, itd; };
-    std::vector<Cross> cross;
-    for (int32_t l = L.l0; l < L.l1; ++l)
-        for (int32_t q = lp[l]; q < lp[l + 1]; ++q) {
-            const int32_t k = (q - lp[l]) / kTeamChunk;
-            for (int32_t e = dptr[q]; e < dptr[q + 1]; ++e) {
-                const int32_t ds = dslot[e], ld = level_of[ds];
-                if (ld < L.l0 || ld >= L.l1) continue;   // an earlier launch: ordered by the stream
-                if ((ds > q ? ds - q : q - ds) >= kRingSafe) return false;
-                const int32_t kd = (ds - lp[ld]) / kTeamChunk;
-                if (kd != k) cross.push_back({k, ds, iter_of(l), kd, iter_of(ld)});
-            }
-            if ((int64_t)cross.size() > 4 * cells_left + 1024) return false;
-        }
     // one import per (workgroup, slot): the first level that needs it
     std::sort(cross.begin(), cross.end(), [](const Cross &x, const Cross &y) {
         return x.k != y.k ? x.k < y.k : (x.ds != y.ds ? x.ds < y.ds : x.it < y.it);
@@ -2258,25 +2281,61 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     std::vector<int32_t> team_tab[2];
     {
         bool any = false;
-        for (const auto &C : p->launches) any = any || (!C.wide && C.width > kTeamChunk);
-        std::vector<int32_t> level_of, dslot_h;
-        if (any && (p->ell_pre[0] > 0 || p->ell_pre[1] > 0)) {
-            level_of.resize((size_t)rows);
-            for (int32_t l = 0; l < p->nlevels; ++l)
-                for (int32_t q = lp[l]; q < lp[l + 1]; ++q) level_of[q] = l;
-        }
+        if (g_team_enabled.load())   // (switched off: no tables, the plan's launches stay with one workgroup)
+            for (const auto &C : p->launches) any = any || (!C.wide && C.width > kTeamChunk);
+        const int32_t nl = (int32_t)p->launches.size();
+        // device scratch that is free by now: W.deg = [count][bad per launch], W.count64 = first and
+        // last level of the candidates, W.rowid = the crossings
+        int32_t *d_count = W.deg, *d_bad = W.deg + 1;
+        int32_t *d_l0 = reinterpret_cast<int32_t *>(W.count64), *d_l1 = d_l0 + nl;
+        const int64_t cap64 = (nnz + 1) / kCrossInts < 4 * team_cells_capacity(rows) + 1024
+                                  ? (nnz + 1) / kCrossInts : 4 * team_cells_capacity(rows) + 1024;
+        const int32_t capacity = (int32_t)cap64;
+        std::vector<int32_t> cand_l0((size_t)nl), cand_l1((size_t)nl), recs, head((size_t)nl + 1);
         for (int d = 0; d < 2 && any; ++d) {
-            if (p->ell_pre[d] == 0 || nnz == 0) continue;
-            dslot_h.resize((size_t)nnz);
-            if (hipMemcpyAsync(dslot_h.data(), p->dir[d].dslot, dslot_h.size() * 4, hipMemcpyDeviceToHost, s) !=
-                    hipSuccess ||
+            if (p->ell_pre[d] == 0 || nnz == 0 || nl > rows) continue;
+            bool some = false;
+            for (int32_t li = 0; li < nl; ++li) {
+                const auto &C = p->launches[li];
+                const bool cand = !C.wide && C.chain[d] == 0 && C.width > kTeamChunk;
+                cand_l0[li] = cand ? C.l0 : -1;
+                cand_l1[li] = C.l1;
+                some = some || cand;
+            }
+            if (!some) continue;
+            if (int rc = nm::fill_async(W.deg, (int64_t)nl + 1, (int32_t)0, s)) return bail(rc);
+            if (hipMemcpyAsync(d_l0, cand_l0.data(), (size_t)nl * 4, hipMemcpyHostToDevice, s) != hipSuccess ||
+                hipMemcpyAsync(d_l1, cand_l1.data(), (size_t)nl * 4, hipMemcpyHostToDevice, s) != hipSuccess)
+                return bail(nm::fail(NM_ERR_HIP, "uploading the candidate launches failed"));
+            hipLaunchKernelGGL(team_cross_kernel, dim3((unsigned)rgrid), dim3(kBlock), 0, s, rows, p->dir[d].dptr,
+                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, d_l0, d_l1, W.rowid,
+                               capacity, d_count, d_bad);
+            if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "team_cross_kernel launch failed"));
+            head.assign((size_t)nl + 1, 0);   // [0]: crossings found, [1 + li]: launch li ruled out
+            if (hipMemcpyAsync(head.data(), W.deg, head.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
                 hipStreamSynchronize(s) != hipSuccess)
-                return bail(nm::fail(NM_ERR_HIP, "reading the dependency slots back failed"));
+                return bail(nm::fail(NM_ERR_HIP, "reading the crossings' count back failed"));
+            if (head[0] > capacity) continue;   // far more cross than any team exchanges
+            recs.resize((size_t)head[0] * kCrossInts);
+            if (!recs.empty() &&
+                (hipMemcpyAsync(recs.data(), W.rowid, recs.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
+                 hipStreamSynchronize(s) != hipSuccess))
+                return bail(nm::fail(NM_ERR_HIP, "reading the crossings back failed"));
+            std::vector<std::vector<Cross>> per((size_t)nl);
+            for (size_t r = 0; r + kCrossInts <= recs.size(); r += kCrossInts) {
+                const int32_t li = recs[r];
+                const auto &C = p->launches[li];
+                auto iter_of = [&](int32_t l) { return d == 0 ? l - C.l0 : (C.l1 - 1) - l; };
+                per[li].push_back({recs[r + 1], recs[r + 2], iter_of(recs[r + 3]), 0, iter_of(recs[r + 4])});
+                // the producer's part of its level
+                per[li].back().kd = (recs[r + 2] - lp[recs[r + 4]]) / kTeamChunk;
+            }
             int64_t cells = 0;
-            for (auto &C : p->launches) {
-                if (C.wide || C.chain[d] != 0 || C.width <= kTeamChunk) continue;
+            for (int32_t li = 0; li < nl; ++li) {
+                auto &C = p->launches[li];
+                if (cand_l0[li] < 0 || head[1 + li] != 0) continue;
                 nm_sptrsv_plan::Launch::Team T;
-                if (!build_team(C, d, lp, dptr_h[d], dslot_h, level_of, team_cells_capacity(rows) - cells,
+                if (!build_team(C, per[li], team_cells_capacity(rows) - cells,
                                 team_capacity(rows) - (int64_t)team_tab[d].size(), team_tab[d], T))
                     continue;
                 T.cell0 = (int32_t)cells;
