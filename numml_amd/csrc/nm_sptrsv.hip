@@ -75,7 +75,7 @@ inline int64_t coef_capacity(int64_t rows, int64_t nnz) {
 constexpr int kTeamMax = 16;
 inline int64_t team_cells_capacity(int64_t rows) { return rows / 16 + 2048; }
 constexpr int64_t kTeamCellPadding = 64;   // readable cells past the last one (a poll reads 64 at a time)
-inline int64_t team_capacity(int64_t rows) { return 3 * team_cells_capacity(rows) + rows / 16 + 16384; }
+inline int64_t team_capacity(int64_t rows) { return 3 * team_cells_capacity(rows) + rows / 4 + 65536; }
 }  // namespace
 
 struct nm_sptrsv_plan {
@@ -1050,36 +1050,37 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
 //
 // One workgroup streams a level's operands through the one compute unit it lives on, and at a
 // thousand rows a level that is what a level costs (44 bytes a row at the ~110 GB/s one unit
-// streams).  Here P workgroups share every level of a launch: workgroup k takes the rows
-// [k * kTeamChunk, (k + 1) * kTeamChunk) of each level, so each unit streams a quarter.  What
-// keeps that from costing a hand-over between compute units per level (0.6-0.75 us through
-// device memory, more than a whole level takes) is that the workgroups do NOT move in step:
+// streams).  Here P workgroups share every level of a launch: workgroup k takes a part of at
+// most kTeamChunk rows of each level (the plan's table says which: see team_parts_kernel), so
+// each unit streams a fraction.  What keeps that from costing a hand-over between compute units
+// per level (0.6-0.75 us through device memory, more than a whole level takes) is that the
+// workgroups do NOT move in step:
 //
 //  * a workgroup keeps its own LDS ring and its own barrier per level, exactly as the
-//    single-workgroup kernel does, with one more wavefront that computes nothing;
+//    single-workgroup kernel does, with two more wavefronts that compute nothing;
 //  * a value that a row of ANOTHER workgroup needs (the plan lists them: `exports`, by the level
-//    that produces them) is read from the ring by that service wavefront one level after it was
-//    computed and stored to a mailbox cell in device memory: two 64-bit words, each half of the
-//    double next to a tag, so that a reader that finds both tags set has the whole value
+//    that produces them) is read from the ring by the first service wavefront one level after
+//    it was computed and stored to a mailbox cell in device memory: two 64-bit words, each half
+//    of the double next to a tag, so that a reader that finds both tags set has the whole value
 //    (a naturally aligned 64-bit access is never torn; no fence, no second flag);
-//  * the service wavefront of the consumer polls the cells of its `imports` (listed by the level
-//    that first needs them) S levels ahead of use and writes what has arrived into its ring;
-//    only when a value is still missing at the barrier before the level that needs it does it
-//    wait, and with it the workgroup.
+//  * the second service wavefront polls the cells of the workgroup's `imports` (listed by the
+//    level that first needs them) several levels ahead of use and writes what has arrived into
+//    the ring; only when a value is still missing at the barrier before the level that needs it
+//    does it wait, and with it the workgroup.
 //
-// On a triangle whose dependencies cross the cut in one direction (the tril of a grid: a row
-// depends on its left and lower neighbours of the previous level) the consumers simply fall a few
-// levels behind their producers and nobody waits again until the direction changes.  The plan
-// only makes a launch shared when that is possible: per level, "workgroup a needs a value that
-// workgroup b computes at the level before" must not form a cycle (such a level would need the
-// hand-over inside the level; see build_team).  Every workgroup of the grid is resident (P <= 4 of
-// the chip's 256 units) and a workgroup only waits for values of lower levels, so the waits end;
-// as a backstop a service wavefront that has polled `poll_limit` times for one level stops
-// waiting for good and the solve hands out NaN, as for the signalling kernel above.
-constexpr int kTeamChunk = 256;            // rows of a level that one workgroup takes
+// Where values cross between two workgroups in one direction (parts by row number: always; the
+// tril of a grid cut by position: a row depends on its left and lower neighbours of the previous
+// level) the consumers simply fall a few levels behind their producers and nobody waits again.
+// The plan only makes a launch shared when that is possible: per level, "workgroup a needs a
+// value that workgroup b computes at the level before" must not form a cycle (such a level would
+// need the hand-over inside the level; see build_team).  Every workgroup of the grid is resident
+// (P <= 16 of the chip's 256 units) and a workgroup only waits for values of lower levels, so the
+// waits end; as a backstop a service wavefront that has polled `poll_limit` times for one level
+// stops waiting for good and the solve hands out NaN, as for the signalling kernel above.
+constexpr int kTeamChunk = 256;            // most rows of a level that one workgroup takes
 constexpr int kTeamStages = 6;             // polls in flight
 constexpr int kTeamAhead = kRing - kRingSafe;   // slots ahead of its own level a workgroup may import
-constexpr int kTeamExports = 4096;         // values one workgroup may hand out in one launch (their list lives in LDS)
+constexpr int kTeamExports = 2048;         // values one workgroup may hand out in one launch (their list lives in LDS)
 static_assert((kTeamExports & (kTeamExports - 1)) == 0, "a power of two");
 constexpr int kTeamNeedBits = 18;          // a workgroup's imports in one launch are counted in these
 static_assert(kTeamExports < (1 << (31 - kTeamNeedBits)), "exports and imports share a word");
@@ -1090,6 +1091,7 @@ struct TeamArgs {
                                  // [n_imp] slot of an import (not read by the kernel: the cell names it),
                                  // [n_imp] slot of an export, [n_imp] its cell
     unsigned long long *cells;   // this launch's mailbox cells
+                                 // [count][P+1] the slots at which the workgroups' parts of a level start
     int32_t P, n_imp;
     int32_t quiet;               // first of the padding cells, counted from `cells`
     int32_t imp_off[kTeamMax + 1], exp_off[kTeamMax + 1];
@@ -1101,7 +1103,7 @@ template <int PRE, int DEPTH>
 __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a, TeamArgs t, int l0, int count, int step,
                                                                        int64_t poll_limit, int32_t *status) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
-    __shared__ int32_t s_lp[kMaxLevels + 1];
+    __shared__ int2 s_mine[kMaxLevels + 1];   // this workgroup's part of every level: first slot, end
     // what the service wavefronts need at a level, in one LDS read: x = the limit an imported
     // slot (times `step`) is held against, y = imports the NEXT level needs (low kTeamNeedBits
     // bits) and exports of the levels before this one (the bits above)
@@ -1109,15 +1111,17 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
     __shared__ int2 s_exl[kTeamExports];   // (slot, cell) of this workgroup's exports
     const int k = blockIdx.x;
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
-    for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
+    const int32_t *parts = t.tab + 2 * t.P * (count + 1) + 3 * t.n_imp;   // [level - lmin][P + 1]
+    for (int i = threadIdx.x; i <= count; i += blockDim.x)
+        s_mine[i] = i < count ? make_int2(parts[i * (t.P + 1) + k], parts[i * (t.P + 1) + k + 1]) : make_int2(0, 0);
     for (int i = threadIdx.x; i <= count; i += blockDim.x) {
         // An imported slot lands on the ring entry of the slot kRing before it, which this
         // workgroup's rows read as long as it is less than kRingSafe behind them: a slot may come
         // in once it is at most kTeamAhead past the first of the workgroup's rows of the level
         // (solving A^T the slots descend: at most kTeamAhead below the last of them).
         const int l = l0 + (i < count ? i : count - 1) * step - lmin;
-        const int mine = a.level_ptr[lmin + l] + k * kTeamChunk;
-        const int lim = step > 0 ? mine + kTeamAhead : -(mine + kTeamChunk - 1) + kTeamAhead;
+        const int first = parts[l * (t.P + 1) + k], end = parts[l * (t.P + 1) + k + 1];
+        const int lim = step > 0 ? first + kTeamAhead : -(end - 1) + kTeamAhead;
         const int need = t.tab[k * (count + 1) + (i + 1 < count ? i + 1 : count)];
         const int before = t.tab[(t.P + k) * (count + 1) + i];
         s_sv[i] = make_int2(lim, need | (before << kTeamNeedBits));
@@ -1134,13 +1138,12 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
     if (threadIdx.x < kTeamChunk) {
         // the rows: the single-workgroup kernel's level loop on this workgroup's part of a level
         const uint32_t lane8 = threadIdx.x * 8u;
-        const int shift = k * kTeamChunk;
-        // (a workgroup without rows in a level starts at the level's end: its lanes load the
-        // operands of the kTeamChunk slots from there on, and those are readable)
+        // (lanes past the end of the part load the operands of the slots that follow it: readable,
+        // whatever the part's length)
         auto part = [&](int it) {
-            Bounds b = load_bounds_uniform(s_lp, it, count, l0, step, lmin);
-            b.qb = b.qb + shift < b.qe ? b.qb + shift : b.qe;
-            return b;
+            int2 m = make_int2(0, 0);
+            if (it < count) m = s_mine[l0 + it * step - lmin];
+            return Bounds{__builtin_amdgcn_readfirstlane(m.x), __builtin_amdgcn_readfirstlane(m.y)};
         };
         EllVals<PRE> qv[DEPTH];
 #pragma unroll
@@ -1601,16 +1604,84 @@ __global__ __launch_bounds__(64) void sptrsv_chain_kernel(ChainArgs c) {
 
 // x[order[q]] = xs[q], rounded once to the value type (cpp/sparse_csr_cpu.cpp:722).
 // `status` (may be null): nonzero when a kernel of this solve gave up waiting; x is then NaN throughout.
-// The dependencies of one solve direction that cross between the 256-row parts of the levels of
-// a launch that a team may share: (launch, consumer's part, dependency's slot, consumer's level,
-// dependency's level) per crossing, appended in no particular order; `bad[launch]` is raised when
-// a row of the launch depends on a row of the same launch too many slots back for the ring.
-// `cand_l0[launch]` is the launch's first level, -1 when it is no candidate in this direction.
-constexpr int kCrossInts = 5;
+// ---- which rows of a level a workgroup of a team takes ---------------------------------------
+//
+// By ROW NUMBER where that works: the rows of a launch are cut into P ranges of row numbers and
+// workgroup k takes, of every level, the rows of range k (inside a level rows ascend, so that is
+// a stretch of the level's slots).  A lower triangle's row depends on rows with smaller numbers
+// only, a value therefore never crosses from a higher range to a lower one (solving A^T: never
+// from a lower to a higher): consumers run behind their producers for good, whatever the
+// stencil.  It works when no range holds more than kTeamChunk rows of one level -- triangles of
+// grid stencils, whose levels run across the grid.  Otherwise by POSITION: workgroup k takes
+// the slots [kTeamChunk k, kTeamChunk (k + 1)) of a level, and build_team checks whether the
+// crossings that come of it can be pipelined.
+constexpr int kPartStride = kTeamMax + 1;   // starts of the parts of one level, then the level's end
+
+// Smallest and largest row number of every candidate launch (span[2 li], span[2 li + 1]; the
+// host presets them): rows ascend inside a level, so a level's first and last slot are enough.
+__global__ void team_span_kernel(int32_t nlevels, const int32_t *__restrict__ order,
+                                 const int32_t *__restrict__ level_ptr, const int32_t *__restrict__ level_launch,
+                                 const int32_t *__restrict__ cand_l0, int32_t *__restrict__ span) {
+    const int32_t l = blockIdx.x * blockDim.x + threadIdx.x;
+    if (l >= nlevels || level_ptr[l + 1] <= level_ptr[l]) return;
+    const int32_t li = level_launch[l];
+    if (li < 0 || cand_l0[li] < 0) return;
+    atomicMin(span + 2 * li, order[level_ptr[l]]);
+    atomicMax(span + 2 * li + 1, order[level_ptr[l + 1] - 1]);
+}
+
+// part[l][k] = first slot of workgroup k's part of level l, for k = 0 .. P (P: the level's end);
+// most[li] = the longest part of launch li.  parts[li] > 0: P ranges of row numbers that start at
+// split[li][k]; parts[li] < 0: -P parts by position.
+__global__ void team_parts_kernel(int32_t nlevels, const int32_t *__restrict__ order,
+                                  const int32_t *__restrict__ level_ptr, const int32_t *__restrict__ level_launch,
+                                  const int32_t *__restrict__ cand_l0, const int32_t *__restrict__ parts,
+                                  const int32_t *__restrict__ split, int32_t *__restrict__ part,
+                                  int32_t *__restrict__ most) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)nlevels * kPartStride) return;
+    const int32_t l = (int32_t)(idx / kPartStride), k = (int32_t)(idx % kPartStride);
+    const int32_t li = level_launch[l];
+    if (li < 0 || cand_l0[li] < 0) return;
+    const int32_t P = parts[li] < 0 ? -parts[li] : parts[li];
+    if (k > P) return;
+    const int32_t q0 = level_ptr[l], q1 = level_ptr[l + 1];
+    auto start_of = [&](int32_t kk) {
+        if (kk <= 0) return q0;
+        if (kk >= P) return q1;
+        if (parts[li] < 0) return q0 + kk * kTeamChunk < q1 ? q0 + kk * kTeamChunk : q1;
+        const int32_t from = split[li * kPartStride + kk];
+        int32_t lo = q0, hi = q1;   // first slot of the level whose row number is >= from
+        while (lo < hi) {
+            const int32_t mid = (lo + hi) >> 1;
+            if (order[mid] < from) lo = mid + 1; else hi = mid;
+        }
+        return lo;
+    };
+    const int32_t mine = start_of(k);
+    part[idx] = mine;
+    if (k < P) atomicMax(most + li, start_of(k + 1) - mine);
+}
+
+// The workgroup that takes slot q of level l.
+__device__ __forceinline__ int32_t part_of(const int32_t *__restrict__ part, int32_t l, int32_t P, int32_t q) {
+    int32_t k = 0;
+    while (k + 1 < P && part[(int64_t)l * kPartStride + k + 1] <= q) ++k;
+    return k;
+}
+
+// The dependencies of one solve direction that cross between the parts of the levels of a
+// launch that a team may share: (launch, consumer's workgroup, producer's workgroup, the
+// dependency's slot, consumer's level, dependency's level) per crossing, appended in no particular
+// order; `bad[launch]` is raised when a row of the launch depends on a row of the same launch
+// too many slots back for the ring.  `cand_l0[launch]` is the launch's first level, -1 when it
+// is no candidate in this direction.
+constexpr int kCrossInts = 6;
 __global__ void team_cross_kernel(int64_t rows, const int32_t *__restrict__ dptr, const int32_t *__restrict__ dslot,
                                   const int32_t *__restrict__ level_ptr, int32_t nlevels,
                                   const int32_t *__restrict__ level_launch, const int32_t *__restrict__ cand_l0,
-                                  const int32_t *__restrict__ cand_l1, int32_t *__restrict__ out, int32_t capacity,
+                                  const int32_t *__restrict__ cand_l1, const int32_t *__restrict__ parts,
+                                  const int32_t *__restrict__ part, int32_t *__restrict__ out, int32_t capacity,
                                   int32_t *__restrict__ count, int32_t *__restrict__ bad) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < rows; q += stride) {
@@ -1619,7 +1690,8 @@ __global__ void team_cross_kernel(int64_t rows, const int32_t *__restrict__ dptr
         if (li < 0) continue;
         const int32_t l0 = cand_l0[li], l1 = cand_l1[li];
         if (l0 < 0) continue;
-        const int32_t k = ((int32_t)q - level_ptr[l]) / kTeamChunk;
+        const int32_t P = parts[li] < 0 ? -parts[li] : parts[li];
+        const int32_t k = part_of(part, l, P, (int32_t)q);
         for (int32_t e = dptr[q]; e < dptr[q + 1]; ++e) {
             const int32_t ds = dslot[e];
             const int32_t ld = level_of_slot(level_ptr, nlevels, ds);
@@ -1628,19 +1700,20 @@ __global__ void team_cross_kernel(int64_t rows, const int32_t *__restrict__ dptr
                 bad[li] = 1;
                 continue;
             }
-            const int32_t kd = (ds - level_ptr[ld]) / kTeamChunk;
+            const int32_t kd = part_of(part, ld, P, ds);
             if (kd == k) continue;
             const int32_t at = atomicAdd(count, 1);
             if (at < capacity) {
                 int32_t *r = out + (int64_t)at * kCrossInts;
-                r[0] = li; r[1] = k; r[2] = ds; r[3] = l; r[4] = ld;
+                r[0] = li; r[1] = k; r[2] = kd; r[3] = ds; r[4] = l; r[5] = ld;
             }
         }
     }
 }
 
-// Exchange tables of a launch that P = ceil(width / kTeamChunk) workgroups share, for one solve
-// direction, from the dependencies that cross between the workgroups' parts of its levels
+// Exchange tables of a launch that P workgroups share, for one solve direction (d = 0: with A),
+// from the dependencies that cross between the workgroups' parts of its levels (`part`: where
+// the parts of every level start)
 // (`cross`, collected on the device by team_cross_kernel, which also rules out a launch in which
 // a row reads, through global memory, a row of the same launch -- too many slots back for the
 // ring: between workgroups nothing orders that read after the write).  Appends to `tab` what
@@ -1653,11 +1726,19 @@ __global__ void team_cross_kernel(int64_t rows, const int32_t *__restrict__ dptr
 //   * more values cross than a service wavefront polls in passing (16 per workgroup and level
 //     on average), or than the mailbox, the tables or a workgroup's LDS list of exports hold.
 struct Cross { int32_t k, ds, it, kd, itd; };   // workgroup k needs slot ds at its level `it`; kd computes it at `itd`
-bool build_team(const nm_sptrsv_plan::Launch &L, std::vector<Cross> &cross, int64_t cells_left, int64_t ints_left,
-                std::vector<int32_t> &tab, nm_sptrsv_plan::Launch::Team &T) {
+bool build_team(const nm_sptrsv_plan::Launch &L, int d, int32_t P, const int32_t *part, std::vector<Cross> &cross,
+                int64_t cells_left, int64_t ints_left, std::vector<int32_t> &tab, nm_sptrsv_plan::Launch::Team &T) {
     const int32_t count = L.l1 - L.l0;
-    const int32_t P = (L.width + kTeamChunk - 1) / kTeamChunk;
     if (P < 2 || P > kTeamMax || count < 16) return false;
+    // A value is taken in at the latest during the level before the one that reads it, and it may
+    // only be taken in once it lies no further than kTeamAhead ahead of the workgroup's own rows
+    // (sptrsv_team_kernel: its ring entry is in use until then).  One that never would, would be
+    // waited for until the solve gives up.
+    for (const Cross &x : cross) {
+        const int32_t before = d == 0 ? L.l0 + x.it - 1 : L.l1 - x.it;   // the level of the workgroup's x.it - 1
+        const int32_t first = part[(int64_t)before * kPartStride + x.k], end = part[(int64_t)before * kPartStride + x.k + 1];
+        if (d == 0 ? x.ds > first + kTeamAhead : x.ds < end - 1 - kTeamAhead) return false;
+    }
     // one import per (workgroup, slot): the first level that needs it
     std::sort(cross.begin(), cross.end(), [](const Cross &x, const Cross &y) {
         return x.k != y.k ? x.k < y.k : (x.ds != y.ds ? x.ds < y.ds : x.it < y.it);
@@ -1666,7 +1747,7 @@ bool build_team(const nm_sptrsv_plan::Launch &L, std::vector<Cross> &cross, int6
                             [](const Cross &x, const Cross &y) { return x.k == y.k && x.ds == y.ds; }),
                 cross.end());
     const int64_t n = (int64_t)cross.size();
-    const int64_t ints = (int64_t)2 * P * (count + 1) + 3 * n;
+    const int64_t ints = (int64_t)2 * P * (count + 1) + 3 * n + (int64_t)count * (P + 1);
     if (n > cells_left || ints > ints_left || n > (int64_t)16 * count * P || n >= (int64_t(1) << kTeamNeedBits))
         return false;
     // waits on the level just before, per level: a cycle among them cannot be pipelined away
@@ -1753,6 +1834,10 @@ bool build_team(const nm_sptrsv_plan::Launch &L, std::vector<Cross> &cross, int6
     for (int k = 0; k < P; ++k)
         for (int32_t j = 1; j <= count; ++j)
             before[(size_t)k * (count + 1) + j] += before[(size_t)k * (count + 1) + j - 1];
+    // the parts of the launch's levels
+    int32_t *parts_out = exp_cell + n;
+    for (int32_t l = 0; l < count; ++l)
+        for (int k = 0; k <= P; ++k) parts_out[(size_t)l * (P + 1) + k] = part[(int64_t)(L.l0 + l) * kPartStride + k];
     return true;
 }
 
@@ -2284,59 +2369,111 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         if (g_team_enabled.load())   // (switched off: no tables, the plan's launches stay with one workgroup)
             for (const auto &C : p->launches) any = any || (!C.wide && C.width > kTeamChunk);
         const int32_t nl = (int32_t)p->launches.size();
-        // device scratch that is free by now: W.deg = [count][bad per launch], W.count64 = first and
-        // last level of the candidates, W.rowid = the crossings
+        // Device scratch that is free by now.  W.count64 (ints): first and last level of the
+        // candidates, their number of parts, span of row numbers, longest part, where the ranges of
+        // row numbers start.  W.deg: [crossings][ruled out, per launch].  W.rowid: where the parts of
+        // every level start, then the crossings.
+        constexpr int kPerLaunch = 2 + 1 + 2 + 1 + kPartStride;
+        const int64_t part_ints = (int64_t)p->nlevels * kPartStride;
+        any = any && nnz > 0 && nl <= rows && (int64_t)nl * kPerLaunch <= 2 * (rows + 1) &&
+              part_ints + 1024 * kCrossInts <= nnz + 1 && (p->ell_pre[0] > 0 || p->ell_pre[1] > 0);
+        int32_t *d_l0 = reinterpret_cast<int32_t *>(W.count64), *d_l1 = d_l0 + nl, *d_parts = d_l1 + nl;
+        int32_t *d_span = d_parts + nl, *d_most = d_span + 2 * nl, *d_split = d_most + nl;
         int32_t *d_count = W.deg, *d_bad = W.deg + 1;
-        int32_t *d_l0 = reinterpret_cast<int32_t *>(W.count64), *d_l1 = d_l0 + nl;
-        const int64_t cap64 = (nnz + 1) / kCrossInts < 4 * team_cells_capacity(rows) + 1024
-                                  ? (nnz + 1) / kCrossInts : 4 * team_cells_capacity(rows) + 1024;
-        const int32_t capacity = (int32_t)cap64;
-        std::vector<int32_t> cand_l0((size_t)nl), cand_l1((size_t)nl), recs, head((size_t)nl + 1);
-        for (int d = 0; d < 2 && any; ++d) {
-            if (p->ell_pre[d] == 0 || nnz == 0 || nl > rows) continue;
-            bool some = false;
+        int32_t *d_part = W.rowid, *d_recs = W.rowid + part_ints;
+        int64_t cap64 = (nnz + 1 - part_ints) / kCrossInts;
+        if (cap64 > 4 * team_cells_capacity(rows) + 1024) cap64 = 4 * team_cells_capacity(rows) + 1024;
+        const int32_t capacity = any ? (int32_t)cap64 : 0;
+        std::vector<int32_t> cand_l0((size_t)nl, -1), cand_l1((size_t)nl, 0), parts((size_t)nl, 0), recs,
+            head((size_t)nl + 1), span((size_t)2 * nl), most((size_t)nl), split((size_t)nl * kPartStride, 0), part_h;
+        auto up = [&](int32_t *dst, const std::vector<int32_t> &src) {
+            return src.empty() || hipMemcpyAsync(dst, src.data(), src.size() * 4, hipMemcpyHostToDevice, s) == hipSuccess;
+        };
+        auto down = [&](std::vector<int32_t> &dst, const int32_t *src) {
+            return dst.empty() || (hipMemcpyAsync(dst.data(), src, dst.size() * 4, hipMemcpyDeviceToHost, s) == hipSuccess &&
+                                   hipStreamSynchronize(s) == hipSuccess);
+        };
+        const unsigned lgrid = (unsigned)nm::ceil_div((int64_t)p->nlevels, kBlock);
+        const unsigned pgrid = (unsigned)nm::ceil_div(part_ints > 0 ? part_ints : 1, (int64_t)kBlock);
+        if (any) {
+            // the parts of every level of every launch that is a candidate in either direction
             for (int32_t li = 0; li < nl; ++li) {
                 const auto &C = p->launches[li];
-                const bool cand = !C.wide && C.chain[d] == 0 && C.width > kTeamChunk;
+                const bool cand = !C.wide && C.width > kTeamChunk && C.width <= kTeamMax * kTeamChunk &&
+                                  ((p->ell_pre[0] > 0 && C.chain[0] == 0) || (p->ell_pre[1] > 0 && C.chain[1] == 0));
                 cand_l0[li] = cand ? C.l0 : -1;
                 cand_l1[li] = C.l1;
-                some = some || cand;
+                parts[li] = cand ? (C.width + kTeamChunk - 1) / kTeamChunk : 0;
+                span[2 * li] = 0x7fffffff;
+                span[2 * li + 1] = -1;
+            }
+            if (!up(d_l0, cand_l0) || !up(d_l1, cand_l1) || !up(d_span, span))
+                return bail(nm::fail(NM_ERR_HIP, "uploading the candidate launches failed"));
+            hipLaunchKernelGGL(team_span_kernel, dim3(lgrid), dim3(kBlock), 0, s, p->nlevels, p->order, p->level_ptr,
+                               L.level_launch, d_l0, d_span);
+            if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "team_span_kernel launch failed"));
+            if (!down(span, d_span)) return bail(nm::fail(NM_ERR_HIP, "reading the launches' row numbers back failed"));
+            // by row number, with as few workgroups as keep every part within kTeamChunk rows; by
+            // position where not even kTeamMax ranges do
+            for (bool again = true; again;) {
+                for (int32_t li = 0; li < nl; ++li) {
+                    if (parts[li] <= 0) continue;
+                    const int64_t lo = span[2 * li], n = (int64_t)span[2 * li + 1] - lo + 1;
+                    for (int k = 0; k <= parts[li]; ++k) split[(size_t)li * kPartStride + k] = (int32_t)(lo + n * k / parts[li]);
+                }
+                if (!up(d_parts, parts) || !up(d_split, split))
+                    return bail(nm::fail(NM_ERR_HIP, "uploading the ranges of row numbers failed"));
+                if (int rc = nm::fill_async(d_most, (int64_t)nl, (int32_t)0, s)) return bail(rc);
+                hipLaunchKernelGGL(team_parts_kernel, dim3(pgrid), dim3(kBlock), 0, s, p->nlevels, p->order, p->level_ptr,
+                                   L.level_launch, d_l0, d_parts, d_split, d_part, d_most);
+                if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "team_parts_kernel launch failed"));
+                if (!down(most, d_most)) return bail(nm::fail(NM_ERR_HIP, "reading the longest parts back failed"));
+                again = false;
+                for (int32_t li = 0; li < nl; ++li) {
+                    if (parts[li] <= 0 || most[li] <= kTeamChunk) continue;
+                    const int32_t by_position = (p->launches[li].width + kTeamChunk - 1) / kTeamChunk;
+                    parts[li] = parts[li] < kTeamMax ? parts[li] + 1 : -by_position;
+                    again = true;
+                }
+            }
+            part_h.resize((size_t)part_ints);
+            if (!down(part_h, d_part)) return bail(nm::fail(NM_ERR_HIP, "reading the parts back failed"));
+        }
+        for (int d = 0; d < 2 && any; ++d) {
+            if (p->ell_pre[d] == 0) continue;
+            bool some = false;
+            std::vector<int32_t> mine(cand_l0);   // the candidates of this direction
+            for (int32_t li = 0; li < nl; ++li) {
+                if (p->launches[li].chain[d] != 0) mine[li] = -1;
+                some = some || mine[li] >= 0;
             }
             if (!some) continue;
             if (int rc = nm::fill_async(W.deg, (int64_t)nl + 1, (int32_t)0, s)) return bail(rc);
-            if (hipMemcpyAsync(d_l0, cand_l0.data(), (size_t)nl * 4, hipMemcpyHostToDevice, s) != hipSuccess ||
-                hipMemcpyAsync(d_l1, cand_l1.data(), (size_t)nl * 4, hipMemcpyHostToDevice, s) != hipSuccess)
-                return bail(nm::fail(NM_ERR_HIP, "uploading the candidate launches failed"));
+            if (!up(d_l0, mine)) return bail(nm::fail(NM_ERR_HIP, "uploading the candidate launches failed"));
             hipLaunchKernelGGL(team_cross_kernel, dim3((unsigned)rgrid), dim3(kBlock), 0, s, rows, p->dir[d].dptr,
-                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, d_l0, d_l1, W.rowid,
-                               capacity, d_count, d_bad);
+                               p->dir[d].dslot, p->level_ptr, p->nlevels, L.level_launch, d_l0, d_l1, d_parts, d_part,
+                               d_recs, capacity, d_count, d_bad);
             if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "team_cross_kernel launch failed"));
             head.assign((size_t)nl + 1, 0);   // [0]: crossings found, [1 + li]: launch li ruled out
-            if (hipMemcpyAsync(head.data(), W.deg, head.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
-                hipStreamSynchronize(s) != hipSuccess)
-                return bail(nm::fail(NM_ERR_HIP, "reading the crossings' count back failed"));
+            if (!down(head, W.deg)) return bail(nm::fail(NM_ERR_HIP, "reading the crossings' count back failed"));
             if (head[0] > capacity) continue;   // far more cross than any team exchanges
             recs.resize((size_t)head[0] * kCrossInts);
-            if (!recs.empty() &&
-                (hipMemcpyAsync(recs.data(), W.rowid, recs.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
-                 hipStreamSynchronize(s) != hipSuccess))
-                return bail(nm::fail(NM_ERR_HIP, "reading the crossings back failed"));
+            if (!down(recs, d_recs)) return bail(nm::fail(NM_ERR_HIP, "reading the crossings back failed"));
             std::vector<std::vector<Cross>> per((size_t)nl);
             for (size_t r = 0; r + kCrossInts <= recs.size(); r += kCrossInts) {
                 const int32_t li = recs[r];
                 const auto &C = p->launches[li];
                 auto iter_of = [&](int32_t l) { return d == 0 ? l - C.l0 : (C.l1 - 1) - l; };
-                per[li].push_back({recs[r + 1], recs[r + 2], iter_of(recs[r + 3]), 0, iter_of(recs[r + 4])});
-                // the producer's part of its level
-                per[li].back().kd = (recs[r + 2] - lp[recs[r + 4]]) / kTeamChunk;
+                per[li].push_back({recs[r + 1], recs[r + 3], iter_of(recs[r + 4]), recs[r + 2], iter_of(recs[r + 5])});
             }
             int64_t cells = 0;
             for (int32_t li = 0; li < nl; ++li) {
                 auto &C = p->launches[li];
-                if (cand_l0[li] < 0 || head[1 + li] != 0) continue;
+                if (mine[li] < 0 || head[1 + li] != 0) continue;
                 nm_sptrsv_plan::Launch::Team T;
-                if (!build_team(C, per[li], team_cells_capacity(rows) - cells,
-                                team_capacity(rows) - (int64_t)team_tab[d].size(), team_tab[d], T))
+                if (!build_team(C, d, parts[li] < 0 ? -parts[li] : parts[li], part_h.data(), per[li],
+                                team_cells_capacity(rows) - cells, team_capacity(rows) - (int64_t)team_tab[d].size(),
+                                team_tab[d], T))
                     continue;
                 T.cell0 = (int32_t)cells;
                 cells += T.n_imp;

@@ -1,6 +1,7 @@
-"""Triangular solves whose wide levels are shared by several workgroups: each takes 256 rows of
-every level, and the few values a workgroup needs from the others pass through a mailbox in
-device memory while the consumer runs a few levels behind.  The plan shares a launch only
+"""Triangular solves whose wide levels are shared by several workgroups: each takes up to 256
+rows of every level (a range of row numbers where that works, else of positions in the level),
+and the few values a workgroup needs from the others pass through a mailbox in device memory
+while the consumer runs a few levels behind.  The plan shares a launch only
 where that can be pipelined; every case is solved both ways (shared, and by one workgroup) and
 compared bit for bit with the other and with the serial loops of
 cpp/sparse_csr_cpu.cpp:652-759.
@@ -67,9 +68,9 @@ def _cases():
     d, i, p, (n, _) = G.poisson2d_lower(560, np.float64, diag_seed=6)
     triu = sps.csr_matrix((d, i, p), shape=(n, n)).T.tocsr()
     yield "triu of the 560^2 five-point matrix (three workgroups)", triu, False, False, np.float64, (True, True)
-    # the nine-point stencil's dependencies cross the cut in alternating directions from level to
-    # level once the levels shrink: the launches of the growing half are shared, the others not
-    yield "tril of the 640^2 nine-point matrix", _stencil9_lower(640, 7), True, False, np.float64, (None, None)
+    # the nine-point stencil: cut by position, its dependencies would cross in alternating
+    # directions from level to level once the levels shrink; cut by row number they cannot
+    yield "tril of the 640^2 nine-point matrix", _stencil9_lower(640, 7), True, False, np.float64, (True, True)
     # dependencies on one side only: the consumer falls behind its producer once
     yield "levels of 700 rows, neighbours below", _generations(40, 700, (-2, -1, 0), 8), True, False, np.float64, (True, None)
     # both neighbours: two workgroups would wait for each other at every level
