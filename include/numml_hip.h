@@ -475,8 +475,8 @@ int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
  * and banded matrices), a wavefront instead publishes the levels it has finished in
  * LDS and waits only for its neighbours.  (Measured slower than the barrier on
  * MI355X, hence off; results are the same bits.)
- * Bit 1 (default off): launches that the plan would share among up to four
- * workgroups (nm_sptrsv_plan_shared_launches; each takes 256 rows of every level and
+ * Bit 1 (default off): launches that the plan would share among up to sixteen
+ * workgroups (nm_sptrsv_plan_shared_launches; each takes up to 256 rows of every level and
  * receives the few values it needs from the others through device memory, running a
  * few levels behind the workgroup it receives from) are taken by one workgroup
  * instead (and a pattern analysed while the bit is set gets no such launches at all, whatever
