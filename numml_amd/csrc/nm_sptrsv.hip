@@ -1082,6 +1082,7 @@ constexpr int kTeamStages = 6;             // polls in flight
 constexpr int kTeamAhead = kRing - kRingSafe;   // slots ahead of its own level a workgroup may import
 constexpr int kTeamExports = 2048;         // values one workgroup may hand out in one launch (their list lives in LDS)
 static_assert((kTeamExports & (kTeamExports - 1)) == 0, "a power of two");
+constexpr int kTeamLevels = kTeamExports;  // most levels of a launch that a team may share
 constexpr int kTeamNeedBits = 18;          // a workgroup's imports in one launch are counted in these
 static_assert(kTeamExports < (1 << (31 - kTeamNeedBits)), "exports and imports share a word");
 static_assert(kTeamCellPadding >= 64, "a poll reads 64 cells from any import on");
@@ -2155,8 +2156,11 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     auto push_plain = [&](int32_t a0, int32_t a1) {
         int32_t s0 = a0, block = lanes_for(a0);
         auto flush = [&](int32_t end) {
-            for (int32_t c0 = s0; c0 < end; c0 += kMaxLevels) {
-                const int32_t c1 = c0 + kMaxLevels < end ? c0 + kMaxLevels : end;
+            // (a launch that a team may share hands out, per workgroup, about a value per level:
+            // kTeamLevels of them keep the list of those within what the team kernel holds)
+            const int32_t most = block > kTeamChunk ? kTeamLevels : kMaxLevels;
+            for (int32_t c0 = s0; c0 < end; c0 += most) {
+                const int32_t c1 = c0 + most < end ? c0 + most : end;
                 p->launches.push_back({c0, c1, lp[c0], lp[c1], false, block});
             }
         };
@@ -2242,7 +2246,7 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
         int32_t e = l;
         while (e < p->nlevels && team_width(e)) ++e;
         if (e - l >= kRunMin) {
-            const int32_t pieces = (e - l + kMaxLevels - 1) / kMaxLevels;
+            const int32_t pieces = (e - l + kTeamLevels - 1) / kTeamLevels;
             const int32_t each = (e - l + pieces - 1) / pieces;
             for (int32_t c0 = l; c0 < e; c0 += each) {
                 const int32_t c1 = c0 + each < e ? c0 + each : e;
