@@ -45,6 +45,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 namespace {
@@ -101,6 +102,10 @@ struct nm_sptrsv_plan {
         int32_t chain[2] = {0, 0};
         int64_t chain_at[2] = {0, 0};
         bool chain_candidate = false;
+        // per direction: the launch's first levels, up to the last one in which a row reads a row that
+        // its LDS ring cannot serve (a row of an earlier launch); the levels after them take the level
+        // loop that does not look for such rows
+        int32_t far_levels[2] = {0x7fffffff, 0x7fffffff};
         // a stretch of levels wider than one workgroup takes, none wider than a team takes: shared
         // by a team in the directions that have one, else launched level by level like `wide` ones
         bool run = false;
@@ -129,6 +134,7 @@ constexpr int kSkew = 5;
 constexpr int kRingSafe = kRing - 3 * kNarrow;                 // how far back (in slots) a ring read may reach
 constexpr int kRingSafeSig = kRing - (kSkew + 1) * kNarrow;    // ... when wavefronts run up to kSkew levels apart
 constexpr int32_t kSigLower = 1, kSigHigher = 2;               // bits of lvl_sig
+constexpr int32_t kSigFar = 4;                                 // ... a row of the level reads a row that the ring cannot serve
 constexpr int32_t kSigNever = 1000;                            // a reach that rules the signalling kernel out
 // Largest distance, in wavefronts, between a row and the rows it depends on (both counted from
 // the start of their level) for which wavefronts signal each other instead of meeting at a
@@ -712,6 +718,7 @@ __global__ void ell_pack_kernel(int64_t rows, int pre, const int32_t *__restrict
             const bool same = level_launch[lq] == level_launch[ld];
             const bool near = same && dist < kRingSafe;
             out = ((uint32_t)(ds & (kRing - 1)) * 2) | (near ? 0u : 1u);
+            if (!near && (lvl_sig[lq] & kSigFar) == 0) atomicOr(lvl_sig + lq, kSigFar);
             if (near) {
                 // wavefront of the row and of the row it waits for, each inside its own level
                 const int32_t wq = ((int32_t)q - level_ptr[lq]) >> 6, wd = (ds - level_ptr[ld]) >> 6;
@@ -878,7 +885,8 @@ __device__ __forceinline__ void sig_wait(uint32_t at, int32_t need, int32_t limi
 template <int PRE, int DEPTH, bool SIG = false>
 __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, int count, int step,
                                                              int64_t poll_limit = 0, int32_t *status = nullptr,
-                                                             int tune_sleep = 1, int tune_skew = kSkew) {
+                                                             int tune_sleep = 1, int tune_skew = kSkew,
+                                                             int far_levels = 0x7fffffff) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
     __shared__ int32_t s_lp[kMaxLevels + 1];
     __shared__ int32_t s_done[kNarrow / 64];   // SIG: levels each wavefront has finished
@@ -946,55 +954,74 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
     };
     if (!SIG) {
         // (the level body is written out here rather than shared with the signalling loop below:
-        // shared through a lambda it compiled to a few more scalar instructions per level)
-        for (int it0 = 0; it0 < count; it0 += DEPTH) {
+        // shared through that loop's lambda it compiled to a few more scalar instructions per level)
+        //
+        // LEAN: the levels behind the launch's first `far_levels`, in which no row reads a row that
+        // the ring cannot serve (the plan knows), of a solve that divides by the diagonal.  Their
+        // body has no test for such rows and none for the unit diagonal: a level lasts as long as it
+        // takes one wavefront to issue its ~70 instructions, and these are eleven of them
+        // (0.92 -> 0.88 ms per solve on the 1024^2 triangle).
+        auto one_level = [&](auto lean, int it, EllVals<PRE> &stage) {
+            constexpr bool LEAN = decltype(lean)::value;
+            const EllVals<PRE> cur = stage;
+            stage = load_ell<PRE>(a, ahead);
+
+            // all ring reads go out together, unconditionally
+            // (unpacking the offsets one level early, in the shadow of that level's ring reads,
+            // was slower, 0.92 -> 1.12 ms: state carried from level to level makes the compiler
+            // wait for the operand request just issued)
+            double xj[PRE];
+            uint32_t any = 0;
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) {
+                xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
+                any |= cur.ds[e / 2];
+            }
+            ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
+            double acc = 0.;
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
+            const bool live = (int)threadIdx.x < cur.qe - cur.qb;
+            if (!LEAN && (any & kEllFarPair) && live) {
+                // a dependency the ring does not hold: redo the sum in the same order from global memory
+                // (slots and then solutions are requested together; entries past the row's own
+                //  name a valid slot and are not added)
+                const int q = cur.qb + (int)threadIdx.x;
+                const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
+                int32_t sl[PRE];
+                double xg[PRE];
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
+                acc = 0.;
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) acc += e < n ? cur.v[e] * xg[e] : 0.;
+            }
+            double xi = cur.bv - acc;
+            if (LEAN || !a.unit) xi /= cur.dv;
+            if (live) {
+                const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
+                *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
+                *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
+            }
+            __syncthreads();
+        };
+        // whole rounds of DEPTH levels with the tests, the rest without
+        const int tested = a.unit || far_levels >= count ? count : (far_levels + DEPTH - 1) / DEPTH * DEPTH;
+        int it0 = 0;
+        for (; it0 < tested; it0 += DEPTH) {
 #pragma unroll
             for (int d = 0; d < DEPTH; ++d) {
-                const int it = it0 + d;
-                if (it >= count) break;   // uniform over the workgroup
-                const EllVals<PRE> cur = qv[d];
-                qv[d] = load_ell<PRE>(a, ahead);
-
-                // all ring reads go out together, unconditionally
-                // (unpacking the offsets one level early, in the shadow of that level's ring reads,
-                // was slower, 0.92 -> 1.12 ms: state carried from level to level makes the compiler
-                // wait for the operand request just issued)
-                double xj[PRE];
-                uint32_t any = 0;
+                if (it0 + d >= count) break;   // uniform over the workgroup
+                one_level(std::false_type{}, it0 + d, qv[d]);
+            }
+        }
+        for (; it0 < count; it0 += DEPTH) {
 #pragma unroll
-                for (int e = 0; e < PRE; ++e) {
-                    xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
-                    any |= cur.ds[e / 2];
-                }
-                ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
-                double acc = 0.;
-#pragma unroll
-                for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
-                const bool live = (int)threadIdx.x < cur.qe - cur.qb;
-                if ((any & kEllFarPair) && live) {
-                    // a dependency the ring does not hold: redo the sum in the same order from global memory
-                    // (slots and then solutions are requested together; entries past the row's own
-                    //  name a valid slot and are not added)
-                    const int q = cur.qb + (int)threadIdx.x;
-                    const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
-                    int32_t sl[PRE];
-                    double xg[PRE];
-#pragma unroll
-                    for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
-#pragma unroll
-                    for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
-                    acc = 0.;
-#pragma unroll
-                    for (int e = 0; e < PRE; ++e) acc += e < n ? cur.v[e] * xg[e] : 0.;
-                }
-                double xi = cur.bv - acc;
-                if (!a.unit) xi /= cur.dv;
-                if (live) {
-                    const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
-                    *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
-                    *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
-                }
-                __syncthreads();
+            for (int d = 0; d < DEPTH; ++d) {
+                if (it0 + d >= count) break;
+                one_level(std::true_type{}, it0 + d, qv[d]);
             }
         }
     } else {
@@ -1102,7 +1129,7 @@ struct TeamPoll { int cs; unsigned long long w0, w1; };
 
 template <int PRE, int DEPTH>
 __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a, TeamArgs t, int l0, int count, int step,
-                                                                       int64_t poll_limit, int32_t *status) {
+                                                                       int64_t poll_limit, int32_t *status, int far_levels) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
     __shared__ int2 s_mine[kMaxLevels + 1];   // this workgroup's part of every level: first slot, end
     // what the service wavefronts need at a level, in one LDS read: x = the limit an imported
@@ -1150,53 +1177,66 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, part(d));
         Bounds ahead = part(DEPTH);
-        for (int it0 = 0; it0 < count; it0 += DEPTH) {
+        // (LEAN: as in sptrsv_ell_kernel)
+        auto one_level = [&](auto lean, int it, EllVals<PRE> &stage) {
+            constexpr bool LEAN = decltype(lean)::value;
+            const EllVals<PRE> cur = stage;
+            stage = load_ell<PRE>(a, ahead);
+            double xj[PRE];
+            uint32_t any = 0;
 #pragma unroll
-            for (int d = 0; d < DEPTH; ++d) {
-                const int it = it0 + d;
-                if (it >= count) break;   // uniform over the workgroup
-                const EllVals<PRE> cur = qv[d];
-                qv[d] = load_ell<PRE>(a, ahead);
-                double xj[PRE];
-                uint32_t any = 0;
+            for (int e = 0; e < PRE; ++e) {
+                xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
+                any |= cur.ds[e / 2];
+            }
+            ahead = part(it + DEPTH + 1);
+            double acc = 0.;
+#pragma unroll
+            for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
+            const bool live = (int)threadIdx.x < cur.qe - cur.qb;
+            if (!LEAN && (any & kEllFarPair) && live) {
+                // a row solved by an earlier launch: that value from global memory, the sum in
+                // the same order.  (Only that value: what this launch computes is taken from
+                // the ring as ever -- in global memory a value of another workgroup of this
+                // launch is not ordered before this read.)
+                const int q = cur.qb + (int)threadIdx.x;
+                const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
+                int32_t sl[PRE];
+                double xg[PRE];
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
+#pragma unroll
+                for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
+                acc = 0.;
 #pragma unroll
                 for (int e = 0; e < PRE; ++e) {
-                    xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
-                    any |= cur.ds[e / 2];
+                    const bool far = (cur.ds[e / 2] >> ((e & 1) * 16)) & 1u;
+                    acc += e < n ? cur.v[e] * (far ? xg[e] : xj[e]) : 0.;
                 }
-                ahead = part(it + DEPTH + 1);
-                double acc = 0.;
+            }
+            double xi = cur.bv - acc;
+            if (LEAN || !a.unit) xi /= cur.dv;
+            if (live) {
+                const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
+                *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
+                *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
+            }
+            __syncthreads();
+        };
+        const int tested = a.unit || far_levels >= count ? count : (far_levels + DEPTH - 1) / DEPTH * DEPTH;
+        int it0 = 0;
+        for (; it0 < tested; it0 += DEPTH) {
 #pragma unroll
-                for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
-                const bool live = (int)threadIdx.x < cur.qe - cur.qb;
-                if ((any & kEllFarPair) && live) {
-                    // a row solved by an earlier launch: that value from global memory, the sum in
-                    // the same order.  (Only that value: what this launch computes is taken from
-                    // the ring as ever -- in global memory a value of another workgroup of this
-                    // launch is not ordered before this read.)
-                    const int q = cur.qb + (int)threadIdx.x;
-                    const int32_t dlo = a.dptr[q], n = a.dptr[q + 1] - dlo;
-                    int32_t sl[PRE];
-                    double xg[PRE];
+            for (int d = 0; d < DEPTH; ++d) {
+                if (it0 + d >= count) break;   // uniform over the workgroup
+                one_level(std::false_type{}, it0 + d, qv[d]);
+            }
+        }
+        for (; it0 < count; it0 += DEPTH) {
 #pragma unroll
-                    for (int e = 0; e < PRE; ++e) sl[e] = a.dslot[dlo + (e < n ? e : 0)];
-#pragma unroll
-                    for (int e = 0; e < PRE; ++e) xg[e] = a.xs[sl[e]];
-                    acc = 0.;
-#pragma unroll
-                    for (int e = 0; e < PRE; ++e) {
-                        const bool far = (cur.ds[e / 2] >> ((e & 1) * 16)) & 1u;
-                        acc += e < n ? cur.v[e] * (far ? xg[e] : xj[e]) : 0.;
-                    }
-                }
-                double xi = cur.bv - acc;
-                if (!a.unit) xi /= cur.dv;
-                if (live) {
-                    const uint32_t at = (uint32_t)cur.qb * 8u + lane8;
-                    *reinterpret_cast<double *>(const_cast<char *>(ring_bytes) + (at & (kRing * 8 - 1))) = xi;
-                    *reinterpret_cast<double *>(reinterpret_cast<char *>(a.xs) + (int64_t)cur.qb * 8 + lane8) = xi;
-                }
-                __syncthreads();
+            for (int d = 0; d < DEPTH; ++d) {
+                if (it0 + d >= count) break;
+                one_level(std::true_type{}, it0 + d, qv[d]);
             }
         }
         return;
@@ -1976,11 +2016,14 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
                 }
                 const dim3 tg((unsigned)TM.P), tb(kTeamChunk + 128);
                 if (pre == 2)
-                    hipLaunchKernelGGL((sptrsv_team_kernel<2, 4>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status);
+                    hipLaunchKernelGGL((sptrsv_team_kernel<2, 4>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status,
+                                       L.far_levels[dirn]);
                 else if (pre == 4)
-                    hipLaunchKernelGGL((sptrsv_team_kernel<4, 3>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status);
+                    hipLaunchKernelGGL((sptrsv_team_kernel<4, 3>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status,
+                                       L.far_levels[dirn]);
                 else
-                    hipLaunchKernelGGL((sptrsv_team_kernel<8, 2>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status);
+                    hipLaunchKernelGGL((sptrsv_team_kernel<8, 2>), tg, tb, 0, s, ea, ta, l0, count, step, limit, a.w.status,
+                                       L.far_levels[dirn]);
                 NM_LAUNCH_CHECK("sptrsv_team_kernel");
                 continue;
             }
@@ -1995,13 +2038,13 @@ int solve_typed(const nm_sptrsv_plan *p, int transposed, const void *data, int u
                                    limit, a.w.status, tune_sleep, tune_skew);
             else if (pre == 2)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<2, 4>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
-                                   (int64_t)0, (int32_t *)nullptr);
+                                   (int64_t)0, (int32_t *)nullptr, 1, kSkew, L.far_levels[dirn]);
             else if (pre == 4)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<4, 3>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
-                                   (int64_t)0, (int32_t *)nullptr);
+                                   (int64_t)0, (int32_t *)nullptr, 1, kSkew, L.far_levels[dirn]);
             else if (pre == 8)
                 hipLaunchKernelGGL((sptrsv_ell_kernel<8, 2>), dim3(1), dim3(L.block), 0, s, ea, l0, count, step,
-                                   (int64_t)0, (int32_t *)nullptr);
+                                   (int64_t)0, (int32_t *)nullptr, 1, kSkew, L.far_levels[dirn]);
             else if (L.group[dirn] > 0) {
                 // several lanes per row: as many groups as the widest level has rows, within one workgroup
                 const int G = L.group[dirn];
@@ -2363,6 +2406,23 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
                                reinterpret_cast<uint16_t *>(p->dir[d].ell_ds),
                                L.meta + 4 + d, p->dir[d].lvl_sig);
             if (hipGetLastError() != hipSuccess) return bail(nm::fail(NM_ERR_HIP, "ell_pack_kernel launch failed"));
+        }
+    }
+    // per launch and direction: the first levels, up to the last one with a row that reads outside the ring
+    for (int d = 0; d < 2; ++d) {
+        if (p->ell_pre[d] == 0) continue;
+        std::vector<int32_t> sig((size_t)p->nlevels);
+        if (hipMemcpyAsync(sig.data(), p->dir[d].lvl_sig, sig.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
+            hipStreamSynchronize(s) != hipSuccess)
+            return bail(nm::fail(NM_ERR_HIP, "reading the levels' marks back failed"));
+        for (auto &C : p->launches) {
+            int32_t last = 0;   // levels of the launch, in the direction's order, that must be tested
+            for (int32_t l = C.l0; l < C.l1; ++l)
+                if (sig[l] & kSigFar) {
+                    const int32_t it = d == 0 ? l - C.l0 : (C.l1 - 1) - l;
+                    last = last > it + 1 ? last : it + 1;
+                }
+            C.far_levels[d] = last;
         }
     }
     // Launches wider than one workgroup's share of a level, in directions with the fixed-width
