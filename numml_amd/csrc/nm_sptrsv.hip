@@ -790,6 +790,15 @@ template <int PRE> __device__ __forceinline__ void settle(EllVals<PRE> &v) {
     asm volatile("" : "+v"(v.dv));
 }
 
+// The same from a copy of the launch's level bounds with kBoundsPad more entries at either end
+// (repeats of the first and of the last bound): the levels behind the launch's last one, whose
+// operands the pipeline requests all the same, are empty ones there, and the read needs no test.
+constexpr int kBoundsPad = 8;
+__device__ __forceinline__ Bounds load_bounds_padded(const int32_t *s_lpp, int it, int l0, int step, int lmin) {
+    const int l = l0 + it * step - lmin + kBoundsPad;
+    return Bounds{__builtin_amdgcn_readfirstlane(s_lpp[l]), __builtin_amdgcn_readfirstlane(s_lpp[l + 1])};
+}
+
 __device__ __forceinline__ Bounds load_bounds_uniform(const int32_t *s_lp, int it, int count, int l0, int step,
                                                       int lmin) {
     const Bounds b = load_bounds(s_lp, it, count, l0, step, lmin);
@@ -888,12 +897,16 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
                                                              int tune_sleep = 1, int tune_skew = kSkew,
                                                              int far_levels = 0x7fffffff) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
-    __shared__ int32_t s_lp[kMaxLevels + 1];
+    __shared__ int32_t s_lp[kMaxLevels + 1 + 2 * kBoundsPad];   // padded: see load_bounds_padded
+    static_assert(DEPTH + 2 <= kBoundsPad, "the pipeline looks DEPTH + 1 levels past the last");
     __shared__ int32_t s_done[kNarrow / 64];   // SIG: levels each wavefront has finished
     __shared__ int32_t s_abort;
     __shared__ uint8_t s_sig[SIG ? kMaxLevels : 1];   // SIG: the neighbours a level's rows wait for
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
-    for (int i = threadIdx.x; i <= count; i += blockDim.x) s_lp[i] = a.level_ptr[lmin + i];
+    for (int i = threadIdx.x; i <= count + 2 * kBoundsPad; i += blockDim.x) {
+        const int at = i - kBoundsPad;
+        s_lp[i] = a.level_ptr[lmin + (at < 0 ? 0 : (at > count ? count : at))];
+    }
     if (SIG)
         for (int i = threadIdx.x; i < count; i += blockDim.x) s_sig[i] = (uint8_t)a.lvl_sig[lmin + i];
     if (threadIdx.x == 0) ring[kRing] = 0.;
@@ -908,10 +921,10 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
 
     EllVals<PRE> qv[DEPTH];   // operands of levels it .. it + DEPTH - 1, each refilled in place
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, load_bounds_uniform(s_lp, d, count, l0, step, lmin));
+    for (int d = 0; d < DEPTH; ++d) qv[d] = load_ell<PRE>(a, load_bounds_padded(s_lp, d, l0, step, lmin));
     // The bounds of the level whose operands are requested next are read from LDS one level
     // early, before the barrier, so that the request does not start with an LDS round trip.
-    Bounds ahead = load_bounds_uniform(s_lp, DEPTH, count, l0, step, lmin);
+    Bounds ahead = load_bounds_padded(s_lp, DEPTH, l0, step, lmin);
 
     // one level: `cur` holds its operands
     auto level = [&](int it, const EllVals<PRE> &cur) {
@@ -923,7 +936,7 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
             xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
             any |= cur.ds[e / 2];
         }
-        ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
+        ahead = load_bounds_padded(s_lp, it + DEPTH + 1, l0, step, lmin);
         double acc = 0.;
 #pragma unroll
         for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
@@ -977,7 +990,7 @@ __global__ __launch_bounds__(kNarrow) void sptrsv_ell_kernel(EllArgs a, int l0, 
                 xj[e] = *reinterpret_cast<const double *>(ring_bytes + ell_ring_bytes(cur.ds[e / 2], e));
                 any |= cur.ds[e / 2];
             }
-            ahead = load_bounds_uniform(s_lp, it + DEPTH + 1, count, l0, step, lmin);
+            ahead = load_bounds_padded(s_lp, it + DEPTH + 1, l0, step, lmin);
             double acc = 0.;
 #pragma unroll
             for (int e = 0; e < PRE; ++e) acc += cur.v[e] * xj[e];   // absent: 0.0 * 0.0
@@ -1131,7 +1144,10 @@ template <int PRE, int DEPTH>
 __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a, TeamArgs t, int l0, int count, int step,
                                                                        int64_t poll_limit, int32_t *status, int far_levels) {
     __shared__ double ring[kRing + 1];   // [kRing] stays 0.0: what an absent dependency reads
-    __shared__ int2 s_mine[kMaxLevels + 1];   // this workgroup's part of every level: first slot, end
+    // this workgroup's part of every level: first slot, end; kBoundsPad empty parts at either end
+    // for the levels behind the launch's last one, whose operands the pipeline requests all the same
+    __shared__ int2 s_mine[kMaxLevels + 1 + 2 * kBoundsPad];
+    static_assert(DEPTH + 2 <= kBoundsPad, "the pipeline looks DEPTH + 1 levels past the last");
     // what the service wavefronts need at a level, in one LDS read: x = the limit an imported
     // slot (times `step`) is held against, y = imports the NEXT level needs (low kTeamNeedBits
     // bits) and exports of the levels before this one (the bits above)
@@ -1140,8 +1156,11 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
     const int k = blockIdx.x;
     const int lmin = step > 0 ? l0 : l0 - (count - 1);
     const int32_t *parts = t.tab + 2 * t.P * (count + 1) + 3 * t.n_imp;   // [level - lmin][P + 1]
-    for (int i = threadIdx.x; i <= count; i += blockDim.x)
-        s_mine[i] = i < count ? make_int2(parts[i * (t.P + 1) + k], parts[i * (t.P + 1) + k + 1]) : make_int2(0, 0);
+    for (int i = threadIdx.x; i < count + 2 * kBoundsPad; i += blockDim.x) {
+        const int at = i - kBoundsPad, in = at < 0 ? 0 : (at < count ? at : count - 1);
+        const int first = parts[in * (t.P + 1) + k];
+        s_mine[i] = make_int2(first, at == in ? parts[in * (t.P + 1) + k + 1] : first);
+    }
     for (int i = threadIdx.x; i <= count; i += blockDim.x) {
         // An imported slot lands on the ring entry of the slot kRing before it, which this
         // workgroup's rows read as long as it is less than kRingSafe behind them: a slot may come
@@ -1169,8 +1188,7 @@ __global__ __launch_bounds__(kTeamChunk + 128) void sptrsv_team_kernel(EllArgs a
         // (lanes past the end of the part load the operands of the slots that follow it: readable,
         // whatever the part's length)
         auto part = [&](int it) {
-            int2 m = make_int2(0, 0);
-            if (it < count) m = s_mine[l0 + it * step - lmin];
+            const int2 m = s_mine[l0 + it * step - lmin + kBoundsPad];
             return Bounds{__builtin_amdgcn_readfirstlane(m.x), __builtin_amdgcn_readfirstlane(m.y)};
         };
         EllVals<PRE> qv[DEPTH];
