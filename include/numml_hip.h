@@ -479,8 +479,7 @@ int nm_sptrsv_solve(const nm_sptrsv_plan *plan, nm_dtype dt, int transposed,
  * workgroups (nm_sptrsv_plan_shared_launches; each takes up to 256 rows of every level and
  * receives the few values it needs from the others through device memory, running a
  * few levels behind the workgroup it receives from) are taken by one workgroup
- * instead (and a pattern analysed while the bit is set gets no such launches at all, whatever
- * the bit says later).  Results are the same bits either way.
+ * instead.  Results are the same bits either way.
  * All waiting is for rows of lower levels, by wavefronts of workgroups that are all
  * resident (a shared launch needs as many free compute units as it has workgroups),
  * so the waits end; `poll_limit` bounds the polls of one wait all the same (0: the

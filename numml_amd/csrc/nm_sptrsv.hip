@@ -2448,7 +2448,13 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
     std::vector<int32_t> team_tab[2];
     {
         bool any = false;
-        if (g_team_enabled.load())   // (switched off: no tables, the plan's launches stay with one workgroup)
+        // (NUMML_AMD_SPTRSV_TEAMS=0: no tables at all; nm_sptrsv_configure only decides whether a
+        // solve uses them)
+        static const bool build_tables = [] {
+            const char *e = std::getenv("NUMML_AMD_SPTRSV_TEAMS");
+            return !(e && e[0] == '0');
+        }();
+        if (build_tables)
             for (const auto &C : p->launches) any = any || (!C.wide && C.width > kTeamChunk);
         const int32_t nl = (int32_t)p->launches.size();
         // Device scratch that is free by now.  W.count64 (ints): first and last level of the

@@ -110,7 +110,6 @@ def test_shared_launches_match_one_workgroup_and_the_serial_loop(dev):
                 if want is not None:
                     assert (shared[dirn] > 0) == want, f"{name}: shared launches {shared}"
             got = {}
-            # (shared last: a pattern analysed while sharing is switched off gets no exchange tables)
             for one_workgroup in (2, 0):
                 assert L.nm_sptrsv_configure(0, one_workgroup) == 0
                 x = ext.sptrsv_forward(n, n, D, I, P, lower, unit, Bv)
