@@ -170,3 +170,56 @@ def test_shared_launch_in_a_graph(dev):
         eager = ops.sptrsv_forward(n, n, D, I, P, True, False, other)
         torch.cuda.synchronize()
         assert_same(host(eager), oracle.sptrsv_forward(n, n, d, i, p, True, False, host(other)), "eager solve between replays")
+
+
+def _random_generations(rng, gens, width, reach, keep, shuffle):
+    """Levels of `width` rows; a row depends on each of the rows within `reach` positions of its own
+    in the level before with probability `keep` (its own position always, so that every generation
+    is one level).  `shuffle`: rows of a level are numbered in a random order, so that ranges of row
+    numbers and positions in the level have nothing to do with each other."""
+    n = gens * width
+    number = np.arange(n).reshape(gens, width)
+    if shuffle:
+        for g in range(gens):
+            number[g] = number[g][rng.permutation(width)]
+    rows, cols = [np.arange(n)], [np.arange(n)]
+    for o in range(-reach[0], reach[1] + 1):
+        j = np.arange(max(0, -o), min(width, width - o))
+        for g in range(1, gens):
+            on = j[(rng.random(j.size) < keep) | (o == 0)]
+            rows.append(number[g][on])
+            cols.append(number[g - 1][on + o])
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    vals = np.where(rows == cols, rng.uniform(1.0, 1.5, rows.size), rng.uniform(-0.25, 0.25, rows.size))
+    M = sps.csr_matrix((vals, (rows, cols)), shape=(n, n))
+    assert (sps.triu(M, 1)).nnz == 0
+    return M
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_wide_levels_shared_or_not(dev, seed):
+    """Random triangles with levels of several hundred to a few thousand rows: whatever the plan
+    decides for them (ranges of row numbers, positions, one workgroup, a launch per level), both
+    solves and both gradients are the serial loop's, bit for bit."""
+    rng = np.random.default_rng(100 + seed)
+    gens = int(rng.integers(18, 40))
+    width = int(rng.integers(300, 2600))
+    reach = [(2, 0), (0, 2), (1, 1), (3, 0), (0, 1), (2, 2), (1, 0), (0, 1)][seed]
+    M = _random_generations(rng, gens, width, reach, float(rng.uniform(0.3, 1.0)), shuffle=seed >= 6)
+    L = _lib.lib()
+    d, i, p, n = _csr(M, np.float64)
+    b, g = randn(31 + seed, n, np.float64), randn(41 + seed, n, np.float64)
+    x_ref = oracle.sptrsv_forward(n, n, d, i, p, True, False, b)
+    gA_ref, gb_ref = oracle.sptrsv_backward(g, x_ref, n, n, d, i, p, True, False)
+    D, I, P, Bv, Gv = to_dev(dev, d, i, p, b, g)
+    try:
+        for one_workgroup in (2, 0):
+            assert L.nm_sptrsv_configure(0, one_workgroup) == 0
+            x = ext.sptrsv_forward(n, n, D, I, P, True, False, Bv)
+            gA, gb = ext.sptrsv_backward(Gv, x, n, n, D, I, P, True, False, Bv)
+            what = f"{gens} levels of {width} rows, reach {reach}, one_workgroup={one_workgroup}"
+            assert_same(host(x), x_ref, f"x: {what}")
+            assert_same(host(gA), gA_ref, f"grad_A: {what}")
+            assert_same(host(gb), gb_ref, f"grad_b: {what}")
+    finally:
+        assert L.nm_sptrsv_configure(0, 0) == 0
