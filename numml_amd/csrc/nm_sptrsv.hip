@@ -1130,9 +1130,9 @@ static_assert(kTeamCellPadding >= 64, "a poll reads 64 cells from any import on"
 struct TeamArgs {
     const int32_t *tab;          // [P][count+1] imports needed up to a level, [P][count+1] exports before a level,
                                  // [n_imp] slot of an import (not read by the kernel: the cell names it),
-                                 // [n_imp] slot of an export, [n_imp] its cell
-    unsigned long long *cells;   // this launch's mailbox cells
+                                 // [n_imp] slot of an export, [n_imp] its cell,
                                  // [count][P+1] the slots at which the workgroups' parts of a level start
+    unsigned long long *cells;   // this launch's mailbox cells
     int32_t P, n_imp;
     int32_t quiet;               // first of the padding cells, counted from `cells`
     int32_t imp_off[kTeamMax + 1], exp_off[kTeamMax + 1];
