@@ -36,6 +36,7 @@ constexpr int kBlock = 256;
 constexpr int kRows = 512;      // rows (columns) a workgroup stages offsets for
 constexpr int kCap = 4096;      // LDS keys of the ordering kernel
 constexpr int kSlice = 8;       // consecutive outputs one lane produces in a merge pass
+constexpr int kSortMin = 128;   // keys from which a column is sorted by a network instead of ranked key by key
 
 struct WorkT {
     int64_t *count;        // [cols + 1] per-column counters, then column pointers
@@ -228,9 +229,52 @@ __global__ __launch_bounds__(kBlock) void tp_order_kernel(
             __syncthreads();
         };
 
+        // one column of kSortMin..kCap keys: a bitonic sort in LDS (ranking compares every key
+        // with every other one of its column: fine for the handful of entries of a matrix column,
+        // quadratic for the thousand rows of a level of a triangular solve's schedule)
+        auto sorted = [&](const int c) {
+            const int o0 = s_off[c], cnt = s_off[c + 1] - o0;
+            const int32_t first = base + o0;
+            int n = 2;
+            while (n < cnt) n <<= 1;
+            for (int j = threadIdx.x; j < n; j += kBlock) s_key[j] = j < cnt ? t_perm[first + j] : kPastAll;
+            __syncthreads();
+            for (int k = 2; k <= n; k <<= 1)
+                for (int j = k >> 1; j > 0; j >>= 1) {
+                    for (int t = threadIdx.x; t < n / 2; t += kBlock) {
+                        const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1)), p = i | j;   // a pair at distance j
+                        const int32_t a = s_key[i], b = s_key[p];
+                        if ((a > b) == ((i & k) == 0)) {
+                            s_key[i] = b;
+                            s_key[p] = a;
+                        }
+                    }
+                    __syncthreads();
+                }
+            for (int j = threadIdx.x; j < cnt; j += kBlock) {
+                const int32_t key = s_key[j];
+                t_perm[first + j] = key;
+                if (t_row) t_row[first + j] = rowid[key];
+            }
+            __syncthreads();
+        };
+
         for (int s0 = 0; s0 < nc;) {
-            const int e0 = run_end(s_off, s0, nc, kCap);
+            int e0 = run_end(s_off, s0, nc, kCap);
             if (e0 > s0) {
+                // a column worth sorting on its own ends the run before it
+                bool mine = false;
+                for (int c = s0 + threadIdx.x; c < e0; c += kBlock) mine = mine || s_off[c + 1] - s_off[c] >= kSortMin;
+                if (__syncthreads_or(mine)) {
+                    int c = s0;
+                    while (c < e0 && s_off[c + 1] - s_off[c] < kSortMin) ++c;   // c < e0: there is one
+                    if (c == s0) {
+                        if (!LONG) sorted(s0);
+                        s0 += 1;
+                        continue;
+                    }
+                    e0 = c;
+                }
                 if (!LONG) ranked(s0, e0);
                 s0 = e0;
                 continue;
