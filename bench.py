@@ -576,6 +576,8 @@ class SpGEMM(Workload):
             self.dominant_bytes = self.bytes_per_step
             self.dominant_name = ("numeric_planned_wide_kernel (the whole forward on the product plan)"
                                   if self.right == "AA" else
+                                  "numeric_planned_long_kernel (the whole forward on the product plan; rows of the "
+                                  "left operand of more than eight entries)" if self.left == "AA" else
                                   "numeric_planned_kernel (the whole forward on the product plan)")
         # Backward on the product plan (grad_ab_mapped_kernel: both gradients from one walk over A by
         # column): the gradient of C, the values of both operands, the plan's column-major record of
@@ -615,7 +617,8 @@ class SpGEMM(Workload):
         if self.planned:
             wide = self.right == "AA"
             return [(self.dominant_name, self.dominant, self.dominant_bytes,
-                     "numeric_planned_wide_kernel" if wide else "numeric_planned_kernel"),
+                     "numeric_planned_wide_kernel" if wide else
+                     ("numeric_planned_long_kernel" if self.left == "AA" else "numeric_planned_kernel")),
                     ("grad_a_wide_kernel + grad_b_wide_kernel (both gradients on the product plan)" if wide else
                      "grad_ab_mapped_kernel (both gradients from one walk over A by column, on the product plan)",
                      self.backward, self.bwd_bytes_planned, "grad_b_wide_kernel" if wide else "grad_ab_mapped_kernel")]
