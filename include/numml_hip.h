@@ -441,7 +441,7 @@ int nm_sptrsv_analyse(int64_t rows, int64_t nnz,
                       void *plan_mem, size_t plan_bytes, void *work, size_t work_bytes,
                       nm_sptrsv_plan **plan, nm_stream stream);
 
-/* Number of dependency levels / of kernel launches one solve issues. */
+/* Number of dependency levels / of level-kernel launches one solve with A issues. */
 int64_t nm_sptrsv_plan_levels(const nm_sptrsv_plan *plan);
 int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan);
 /* Levels of the solve with A (transposed = 0) or with A^T (1) that sit in runs of one-row levels

@@ -2587,7 +2587,12 @@ extern "C" int nm_sptrsv_analyse(int64_t rows, int64_t nnz, const int64_t *indic
 extern "C" int64_t nm_sptrsv_plan_levels(const nm_sptrsv_plan *plan) { return plan ? plan->nlevels : -1; }
 
 extern "C" int64_t nm_sptrsv_plan_launches(const nm_sptrsv_plan *plan) {
-    return plan ? (int64_t)plan->launches.size() : -1;
+    if (!plan) return -1;
+    // (of the solve with A; a stretch of wide levels that no team shares is launched level by level)
+    int64_t n = 0;
+    for (const auto &L : plan->launches)
+        n += L.run && !(plan->ell_pre[0] > 0 && L.team[0].P > 1) ? L.l1 - L.l0 : 1;
+    return n;
 }
 
 extern "C" int64_t nm_sptrsv_plan_chain_levels(const nm_sptrsv_plan *plan, int transposed) {
