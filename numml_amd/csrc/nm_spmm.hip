@@ -78,6 +78,7 @@ __device__ __forceinline__ T row_times_dense(T acc, int64_t kb0, int64_t ke0, co
 // of the grid.
 constexpr int kFlatRows = 8;
 constexpr int kScoutRows = 64;   // rows a scout workgroup inspects for long ones
+constexpr int kColsPerSlice = 1024;   // dense columns one workgroup walks (wider operands: more workgroups)
 
 // The work of a "scout" workgroup (the first ceil(rows / kScoutRows) of the grid): look for
 // long rows among kScoutRows rows and share every one found among the workgroup's
@@ -134,6 +135,16 @@ __global__ __launch_bounds__(kBlock) void spdmm_fwd_flat_kernel(
     // derived from it -- row ranges, loop bounds, addresses -- in scalar registers and the
     // control flow free of execution-mask bookkeeping)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // A dense operand of thousands of columns is cut into slices of kColsPerSlice (the grid's
+    // second dimension): a wavefront that walked all of them one after the other had 256
+    // dependent rounds of loads at 16 384 columns, and a 16 384-row matrix fills the chip with
+    // only eight such wavefronts per compute unit.
+    {
+        const int64_t first = (int64_t)blockIdx.y * kColsPerSlice;
+        B += first;
+        C += first;
+        n = n - first < kColsPerSlice ? n - first : kColsPerSlice;
+    }
     // The first `long_blocks` workgroups look for long rows, kScoutRows rows each, and
     // share every one they find among their wavefronts (contiguous parts, partial sums added
     // in wavefront order: deterministic, equal to the serial sum to rounding).  They come
@@ -286,8 +297,15 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
     const T *__restrict__ gC, int64_t ldg, int64_t n, T *__restrict__ grad_A,
     T *__restrict__ grad_B, int64_t ldgb, const int32_t *__restrict__ chunk_row) {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // WIDE: dot products alone over thousands of dense columns.  The wavefronts of a workgroup then
+    // share a chunk of entries and take every fourth tile of columns each (their sums meet in LDS,
+    // in wavefront order): a matrix of a few ten thousand entries has too few chunks to fill the
+    // chip with one wavefront per chunk, and each would walk hundreds of tiles on its own.
+    const bool wide = !grad_B && n > 4 * kColsPerSlice;
+    __shared__ T s_dot[kWavesPerBlock][kWave];
+    const int64_t wave0 = wide ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * kWavesPerBlock + wave;
+    const int64_t nwaves = wide ? (int64_t)gridDim.x : (int64_t)gridDim.x * kWavesPerBlock;
     const int64_t nchunks = (nnz + kWave - 1) / kWave;
     for (int64_t ch = wave0; ch < nchunks; ch += nwaves) {
         const int64_t kb = ch * kWave;
@@ -409,6 +427,28 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
             for (int j0 = 0; j0 < cnt; j0 += kBatch) {
                 int64_t col[kBatch], rw[kBatch];
                 locate(j0, col, rw);
+                if (wide) {
+                    // (with fewer columns: the tile-by-tile sums below, which are the one-walk kernel's,
+                    // bit for bit)  A lane keeps its
+                    // columns' share of the eight sums and the lanes are added up once, behind the
+                    // last tile (a reduction per tile is 27 instructions for 16 loads; at 16 384 dense
+                    // columns that was most of the kernel)
+                    T part[kBatch];
+#pragma unroll
+                    for (int u = 0; u < kBatch; ++u) part[u] = T(0);
+#pragma unroll 2
+                    for (int64_t c0 = (int64_t)wave * kWave; c0 < n; c0 += kWavesPerBlock * kWave) {
+                        const int64_t c = c0 + lane;
+                        const bool live = c < n;
+                        T bv[kBatch], gv[kBatch];
+                        fetch(col, rw, c, live, gv, bv);
+#pragma unroll
+                        for (int u = 0; u < kBatch; ++u) part[u] += live ? gv[u] * bv[u] : T(0);
+                    }
+                    const T t = reduce8(part);
+                    if ((lane >> 3) == (j0 >> 3)) mydot += t;
+                    continue;
+                }
                 for (int64_t c0 = 0; c0 < n; c0 += kWave) {
                     const int64_t c = c0 + lane;
                     const bool live = c < n;
@@ -417,6 +457,15 @@ __global__ __launch_bounds__(kBlock) void spdmm_bwd_kernel(
                     consume(j0, col, c, live, gv, bv);
                 }
             }
+        }
+        if (wide) {
+            s_dot[wave][lane] = mydot;
+            __syncthreads();
+            mydot = s_dot[0][lane];
+            for (int w = 1; w < kWavesPerBlock; ++w) mydot += s_dot[w][lane];
+            if (wave == 0 && lane < cnt) grad_A[k] = mydot;
+            __syncthreads();   // the sums are written again for the workgroup's next chunk
+            continue;
         }
         if (grad_A && lane < cnt) grad_A[k] = mydot;
     }
@@ -721,8 +770,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_narrow_kernel(
 template <typename T, typename IDX, bool PERM>
 void launch_product(unsigned grid, hipStream_t s, int64_t rows, const T *data, const IDX *indices, const IDX *indptr,
                     const int32_t *perm, const T *B, int64_t ldb, int64_t n, T *C, int64_t ldc) {
-    hipLaunchKernelGGL((spdmm_fwd_flat_kernel<T, IDX, PERM>), dim3(grid), dim3(kBlock), 0, s, rows, data, indices,
-                       indptr, perm, B, ldb, n, C, ldc);
+    hipLaunchKernelGGL((spdmm_fwd_flat_kernel<T, IDX, PERM>), dim3(grid, (unsigned)nm::ceil_div(n, (int64_t)kColsPerSlice)),
+                       dim3(kBlock), 0, s, rows, data, indices, indptr, perm, B, ldb, n, C, ldc);
 }
 
 int check_args(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const void *data,
@@ -793,7 +842,8 @@ int backward_impl(nm_dtype dt, int64_t rows, int64_t cols, int64_t nnz, const vo
     if (rows == 0 || nnz == 0 || n == 0 || (!grad_A && !grad_B)) return NM_OK;
     NM_REQUIRE(B != nullptr && gC != nullptr, "B or gC is null");
     NM_REQUIRE(ldb >= n && ldg >= n, "row stride smaller than the row");
-    const dim3 grid(wave_grid(nm::ceil_div(nnz, kWave), kWavesPerBlock));
+    // (dot products alone over thousands of dense columns: a workgroup per chunk of 64 entries)
+    const dim3 grid(wave_grid(nm::ceil_div(nnz, kWave), grad_A && !grad_B && n > 4 * kColsPerSlice ? 1 : kWavesPerBlock));
     if (grad_A && !grad_B && n <= 32) {
 #define NM_NARROW(T, W)                                                                                          \
     hipLaunchKernelGGL((sddmm_narrow_kernel<T, W>), grid, dim3(kBlock), 0, s, rows, nnz, indices, indptr,          \
@@ -842,7 +892,9 @@ extern "C" int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols
     NM_REQUIRE(plan_mem != nullptr, "plan is null");
     nm::TPlan t;
     nm::tplan_layout(rows, cols, nnz, const_cast<void *>(plan_mem), &t);
-    if (grad_A && grad_B && rows > 0 && cols > 0 && nnz > 0 && n > 32) {
+    // (a dense operand of thousands of columns: the fused walk takes its column tiles one after the
+    // other, the product below is cut into slices of kColsPerSlice over the grid)
+    if (grad_A && grad_B && rows > 0 && cols > 0 && nnz > 0 && n > 32 && n <= 4 * kColsPerSlice) {
         // both gradients from a single walk over A by column (measured on the 16 M-entry power-law
         // matrix: 1.02 against 1.29 ms at 64 dense columns, 2.18 against 2.80 ms at 128, even at 32;
         // with 16 or fewer the narrow dot-product kernel below and a separate product are faster,

@@ -165,6 +165,26 @@ def test_spmm_strided_operand(dev):
     assert_same(host(Ct), oracle.spdmm_forward(rows, cols, d, i, p, wide[:, ::2]), "strided columns")
 
 
+def test_spmm_thousands_of_dense_columns(dev, backward_mode):
+    """A dense operand wider than one workgroup's slice of columns (1024) and than the widest the
+    one-walk backward takes (4096): the forward and the product of the backward are cut into
+    slices over the grid, the dot products of grad_A are shared by a workgroup's wavefronts.
+    Against cpp/sparse_csr_cpu.cpp:599-646."""
+    mode = backward_mode
+    dtype, n = np.float64, 4200
+    d, i, p, (rows, cols) = G.random_csr(150, 90, 0.08, 21, dtype)
+    B, gC = randn(5, (cols, n), dtype), randn(6, (rows, n), dtype)
+    C_ref = oracle.spdmm_forward(rows, cols, d, i, p, B)
+    gA_ref, gB_ref = oracle.spdmm_backward(rows, cols, d, i, p, B, gC)
+    D, I, P, Bd, gCd = to_dev(dev, d, i, p, B, gC)
+    for sighting in range(2):   # (a plan is built at a pattern's second sighting)
+        C = ext.spdmm_forward(rows, cols, D, I, P, Bd)
+        gA, gB = ext.spdmm_backward(rows, cols, D, I, P, Bd, gCd)
+        assert_same(host(C), C_ref, f"C ({mode}, call {sighting})")
+        assert_close(host(gA), gA_ref, f"grad_A ({mode}, call {sighting})")
+        assert_close(host(gB), gB_ref, f"grad_B ({mode}, call {sighting})")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_spgemm_forward_backward(dev, dtype):
     cases = [
