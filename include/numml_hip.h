@@ -235,9 +235,14 @@ int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
  *   nm_spgemm_workspace_bytes  -> bytes of device scratch both phases need
  *   nm_spgemm_symbolic         -> fills C_indptr (A_rows + 1 entries).  With
  *                                 host_landing (see below; may be NULL) the call
- *                                 waits for its first kernel, learns how many
- *                                 rows need the hash path and, when none does,
- *                                 leaves the hash path's launches out
+ *                                 makes the row pointer as soon as its first
+ *                                 kernel has counted the short rows, waits for
+ *                                 nnz(C) and the news whether any row needs
+ *                                 the hash path and, when none does, leaves
+ *                                 the hash path's launches out; the
+ *                                 nm_spgemm_symbolic_result that follows on the
+ *                                 same workspace and landing place then returns
+ *                                 at once
  *   nm_spgemm_symbolic_result  -> waits for the symbolic phase and hands the
  *                                 host nnz(C) = C_indptr[A_rows], with which
  *                                 the caller allocates, and the number of rows
@@ -246,7 +251,7 @@ int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
  *                                 cpp/sparse_csr_cpu.cpp:166, is this
  *                                 synchronisation point); a caller may read
  *                                 C_indptr[A_rows] itself instead.
- *                                 host_landing: 24 bytes of pinned host memory
+ *                                 host_landing: 32 bytes of pinned host memory
  *                                 the device can write (hipHostMalloc with
  *                                 hipHostMallocCoherent, or a pinned torch
  *                                 tensor), zeroed once by the caller when it is
@@ -254,8 +259,13 @@ int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
  *                                 call, which has a one-lane kernel write the
  *                                 two numbers and a ticket there and polls the
  *                                 ticket (a few us instead of the ~30 us of a
- *                                 stream wait).  One landing place serves one
- *                                 call at a time (one per host thread).  NULL:
+ *                                 stream wait); the fourth word is the host's
+ *                                 own note that nm_spgemm_symbolic has had the
+ *                                 numbers landed already.  One landing place
+ *                                 serves one call at a time (one per host
+ *                                 thread), and the landing place given to
+ *                                 nm_spgemm_symbolic is the one to give to the
+ *                                 nm_spgemm_symbolic_result after it.  NULL:
  *                                 a plain copy and hipStreamSynchronize.  The
  *                                 library itself allocates nothing here.
  *   nm_spgemm_numeric          -> fills C_indices (ascending in each row) and
@@ -335,7 +345,7 @@ int nm_spgemm_backward_planned(nm_dtype dt, int64_t A_rows, int64_t A_cols, int6
  *                           Otherwise the product's class: 1 -- rows of A of at most
  *                           8 and rows of C of at most 64 entries, 2 -- longer rows of
  *                           A, 3 -- also rows of C of 65..254 entries.  Waits for the
- *                           stream (through host_landing, 24 bytes of pinned host
+ *                           stream (through host_landing, 32 bytes of pinned host
  *                           memory, when given; NULL: a copy and a synchronisation).
  *   nm_spgemm_numeric_planned   C_data of the product, C_indptr as built from;
  *                           plan_class as reported when the plan was built.

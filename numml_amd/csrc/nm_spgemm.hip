@@ -76,7 +76,8 @@ struct Work {
     int32_t *key;      // [rows] binning key (product bound, then exact length)
     int32_t *perm;     // [rows] rows grouped by bin
     int32_t *bins;     // [kBinInts]: rows per bin [0, kBins), first row of bin b at kBinStart + b (end at + b + 1), cursor at kBinCursor + b
-    int64_t *scan;     // scan scratch
+    int64_t *count;    // [rows + 1] entries per row of C, before the row pointer is made of them
+    int64_t *scan;     // [tiles + 1] sums of the counts by tile of the row pointer's scan
     int32_t *mark;     // [spill_groups(B_cols) * B_cols]
     double *acc;       // [spill_groups(B_cols) * B_cols]
     int64_t *summary;  // [2]: nnz(C) and the number of rows on the hash path, for the host
@@ -94,11 +95,12 @@ size_t work_layout(int64_t rows, int64_t B_cols, void *base, Work *w) {
     int32_t *key = (int32_t *)take((rows + 1) * 4);
     int32_t *perm = (int32_t *)take((rows + 1) * 4);
     int32_t *bins = (int32_t *)take(kBinInts * 4);
+    int64_t *count = (int64_t *)take((size_t)(rows + 1) * 8);
     int64_t *scan = (int64_t *)take(nm::scan_scratch_bytes(rows + 1));
+    int64_t *summary = (int64_t *)take(2 * 8);
     int32_t *mark = (int32_t *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 4);
     double *acc = (double *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 8);
-    int64_t *summary = (int64_t *)take(2 * 8);
-    if (w) *w = Work{key, perm, bins, scan, mark, acc, summary};
+    if (w) *w = Work{key, perm, bins, count, scan, mark, acc, summary};
     return off;
 }
 
@@ -214,7 +216,8 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     int64_t rows, int64_t nbatch_padded, const int64_t *__restrict__ A_indices,
     const int64_t *__restrict__ A_indptr, const int64_t *__restrict__ B_indices,
     const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key, int64_t *__restrict__ C_count,
-    unsigned long long *__restrict__ hash_rows, uint64_t *__restrict__ dest, int32_t *__restrict__ bstart) {
+    unsigned long long *__restrict__ hash_rows, unsigned long long token, uint64_t *__restrict__ dest,
+    int32_t *__restrict__ bstart) {
     __shared__ int32_t s_col[(kMergeCap + 1) * kMergeStride];
     __shared__ int64_t s_bb[kBlock];
     __shared__ int32_t s_len[kBlock];
@@ -242,8 +245,10 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     if (live && !merge && gl == 0) key[row] = ubc;
     // A row left to the hash path raises a flag (a plain store of the same value by whoever finds one:
     // a counter that every wavefront of a product of long rows adds to would be a quarter of a
-    // million atomics on one address); the exact count comes from the binning, if it runs.
-    if (live && !merge && gl == 0) *hash_rows = 1;
+    // million atomics on one address); the exact count comes from the binning, if it runs.  The flag
+    // is raised by writing the call's token, so that nobody need lower it first: whatever the word
+    // held before is not this call's token, or at worst makes the hash path run over no rows.
+    if (live && !merge && gl == 0) *hash_rows = token;
     merge_stage<float, false>(my_bb, merge ? my_len : 0, B_indices, nullptr, A_indptr, s_bb, s_len, s_col, nullptr);
     const int32_t *pc = s_col + threadIdx.x;
     int32_t cur = *pc;
@@ -501,13 +506,87 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
     }
 }
 
-// What the host needs between the phases, in one place: nnz(C) and the rows the hash path took.
-// `bins` is null when no row went to the hash path (summary[1] is then 0 already).
-__global__ void summary_kernel(const int64_t *__restrict__ nnz_c, const int32_t *__restrict__ bins,
-                               int64_t *__restrict__ summary) {
-    if (threadIdx.x == 0) {
-        summary[0] = *nnz_c;
-        if (bins) summary[1] = bins[kBinStart + kBins];
+// Row pointer of C from the rows' counts, and what the host needs between the phases: nnz(C) and
+// the rows the hash path took.  count[0, n) with count[n - 1] == 0 -> C_indptr[0, n) (its exclusive
+// scan, not in place: the counts of the merge path's rows survive a pass made before the hash
+// path's rows are counted).  `sums` holds the sum of every tile of kScanTile counts; with
+// `scanned` == 0 a workgroup adds up the sums before its own (a few thousand numbers out of L2
+// against one more launch), otherwise they have been scanned already (their total behind them).
+// The first workgroup, with nothing before it, adds up all tiles instead: nnz(C), which it leaves
+// in summary[0], with the number of hash-path rows in summary[1] (from `bins`; where bins is null,
+// 1 if the first kernel has left `token` there).  With `host_pinned` it also drops both into the
+// host's landing place, followed by the ticket the host polls for: the host needs the numbers,
+// not the row pointer, so it is told first and sizes C while the row pointer is being written.
+constexpr int kInlineTiles = 4096;
+__global__ __launch_bounds__(nm::kScanBlock) void row_pointer_kernel(
+    const int64_t *__restrict__ count, int64_t n, const int64_t *__restrict__ sums, int scanned,
+    int64_t *__restrict__ C_indptr, const int32_t *__restrict__ bins, int64_t *__restrict__ summary,
+    int64_t token, volatile int64_t *host_pinned, int64_t ticket) {
+    using nm::kScanItems;
+    __shared__ int64_t s_wave[nm::kScanBlock / kWave];
+    const int64_t base = (int64_t)blockIdx.x * nm::kScanTile + (int64_t)threadIdx.x * kScanItems;
+    int64_t item[kScanItems];
+    int64_t v = 0;
+    const bool whole = nm::scan_tile_whole(count, n) && (reinterpret_cast<uintptr_t>(C_indptr) & 15) == 0;
+    if (whole) {
+        const nm::I64x2 *p = reinterpret_cast<const nm::I64x2 *>(count + base);
+#pragma unroll
+        for (int i = 0; i < kScanItems / 2; ++i) {
+            const nm::I64x2 w = p[i];
+            item[2 * i] = w[0];
+            item[2 * i + 1] = w[1];
+            v += w[0] + w[1];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kScanItems; ++i) {
+            item[i] = base + i < n ? count[base + i] : 0;
+            v += item[i];
+        }
+    }
+    // (the first workgroup, which has nothing before it, adds up all tiles instead: nnz(C), for the host)
+    int64_t before;
+    if (scanned) {
+        before = sums[blockIdx.x == 0 ? gridDim.x : blockIdx.x];
+    } else {
+        const int upto = blockIdx.x == 0 ? (int)gridDim.x : (int)blockIdx.x;
+        int64_t part = 0;
+        for (int t = threadIdx.x; t < upto; t += nm::kScanBlock) part += sums[t];
+        nm::block_exclusive_scan(part, s_wave, before);
+    }
+    if (blockIdx.x == 0) {
+        if (threadIdx.x == 0) {
+            const int64_t nnz = before;
+            const int64_t hashed = bins ? (int64_t)bins[kBinStart + kBins] : (summary[1] == token ? 1 : 0);
+            summary[0] = nnz;
+            summary[1] = hashed;
+            if (host_pinned) {
+                host_pinned[0] = nnz;
+                host_pinned[1] = hashed;
+                __threadfence_system();
+                host_pinned[2] = ticket;
+            }
+        }
+        before = 0;
+    }
+    int64_t total;
+    int64_t run = before + nm::block_exclusive_scan(v, s_wave, total);
+    if (whole) {
+        nm::I64x2 *p = reinterpret_cast<nm::I64x2 *>(C_indptr + base);
+#pragma unroll
+        for (int i = 0; i < kScanItems / 2; ++i) {
+            nm::I64x2 w;
+            w[0] = run;
+            w[1] = run + item[2 * i];
+            run = w[1] + item[2 * i + 1];
+            p[i] = w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kScanItems; ++i) {
+            if (base + i < n) C_indptr[base + i] = run;
+            run += item[i];
+        }
     }
 }
 
@@ -1404,59 +1483,79 @@ int symbolic_phase(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t
     hipStream_t s = nm::as_stream(stream);
     if (A_rows == 0) return nm::fill_async(C_indptr, 1, (int64_t)0, s);
 
-    if (int rc = nm::fill_async(w.summary, 2, (int64_t)0, s)) return rc;
+    const int64_t tiles = nm::ceil_div(A_rows + 1, nm::kScanTile);
+    if (tiles > nm::kMaxGrid) return nm::fail(NM_ERR_UNSUPPORTED, "%lld rows are too many", (long long)A_rows);
+    // What the first kernel writes over summary[1] where it leaves a row to the hash path: not a
+    // count of rows (the word's content at the end of every call) and not an earlier call's token.
+    volatile int64_t *both = (volatile int64_t *)host_landing;
+    const int64_t ticket = both ? both[2] + 1 : 1;
+    const int64_t token = ticket | ((int64_t)1 << 62);
     const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
     hipLaunchKernelGGL(symbolic_front_kernel, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
-                       A_indices, A_indptr, B_indices, B_indptr, w.key, C_indptr,
-                       reinterpret_cast<unsigned long long *>(w.summary + 1),
+                       A_indices, A_indptr, B_indices, B_indptr, w.key, w.count,
+                       reinterpret_cast<unsigned long long *>(w.summary + 1), (unsigned long long)token,
                        map ? reinterpret_cast<uint64_t *>(map->dest) : (uint64_t *)nullptr,
                        map ? map->bstart : (int32_t *)nullptr);
     NM_LAUNCH_CHECK("symbolic_front_kernel");
-    // With a landing place in pinned host memory the host learns here whether the first kernel
-    // left any row to the hash path; with none (a product of stencil or aggregation matrices) the
-    // binning and the nine launches of the hash path, which would find nothing to do, are left out.
-    bool hashed = true;
-    if (host_landing) {
-        volatile int64_t *both = (volatile int64_t *)host_landing;
-        const int64_t ticket = both[2] + 1;
-        hipLaunchKernelGGL(summary_out_kernel, dim3(1), dim3(64), 0, s, w.summary, both, ticket);
-        NM_LAUNCH_CHECK("summary_out_kernel");
+    // The row pointer from the counts: their sums by tile, then the pass that writes it.
+    auto row_pointer = [&](const int32_t *bins, volatile int64_t *landing) -> int {
+        hipLaunchKernelGGL(nm::scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(nm::kScanBlock), 0, s, w.count,
+                           A_rows + 1, w.scan);
+        NM_LAUNCH_CHECK("scan_tile_sums_kernel");
+        const bool scanned = tiles > kInlineTiles;
+        if (scanned) {
+            hipLaunchKernelGGL(nm::scan_sums_kernel, dim3(1), dim3(1024), 0, s, w.scan, tiles);
+            NM_LAUNCH_CHECK("scan_sums_kernel");
+        }
+        hipLaunchKernelGGL(row_pointer_kernel, dim3((unsigned)tiles), dim3(nm::kScanBlock), 0, s, w.count, A_rows + 1,
+                           w.scan, scanned ? 1 : 0, C_indptr, bins, w.summary, token, landing, ticket);
+        NM_LAUNCH_CHECK("row_pointer_kernel");
+        return NM_OK;
+    };
+    // With a landing place in pinned host memory the row pointer is made at once, as if the first
+    // kernel had taken every row (it has, for a product of stencil or aggregation matrices), and its
+    // last workgroup tells the host nnz(C) and whether a row was left to the hash path.  If none was,
+    // that was the symbolic phase: the binning and the nine launches of the hash path, which would
+    // find nothing to do, are left out, and nm_spgemm_symbolic_result finds its answer landed (the
+    // workspace's address in the landing place's fourth word says so).  Otherwise the pass was for
+    // nothing (30 us against the milliseconds of a hash path) and is made again below.
+    if (both) {
+        both[3] = 0;
+        if (int rc = row_pointer(nullptr, both)) return rc;
         bool arrived = false;
         for (int spin = 0; spin < (1 << 22) && !arrived; ++spin) arrived = both[2] == ticket;
         if (!arrived) {
             NM_HIP_TRY(hipStreamSynchronize(s));
             NM_REQUIRE(both[2] == ticket, "the count of hash-path rows did not arrive");
         }
-        hashed = both[1] != 0;
+        if (both[1] == 0) {
+            both[3] = (int64_t)reinterpret_cast<intptr_t>(workspace);
+            return NM_OK;
+        }
     }
-    if (hashed) {
+    {
     if (int rc = bin_rows(A_rows, kSymLimit, w, s)) return rc;
 
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup0, kSymTable0>), dim3(kPersistGrid), dim3(kBlock), 0, s, 0, w.bins,
-                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, w.count);
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup1, kSymTable1>), dim3(kPersistGrid), dim3(kBlock), 0, s, 1, w.bins,
-                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, w.count);
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup2, kSymTable2>), dim3(kPersistGrid), dim3(kBlock), 0, s, 2, w.bins,
-                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, w.count);
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup3, kSymTable3>), dim3(kPersistGrid), dim3(kBlock), 0, s, 3, w.bins,
-                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, w.count);
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup4, kSymTable4>), dim3(kPersistGrid), dim3(kBlock), 0, s, 4, w.bins,
-                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, w.count);
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup5, kSymTable5>), dim3(kPersistGrid), dim3(kBlock), 0, s, 5, w.bins,
-                       w.perm, A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+                       w.perm, A_indices, A_indptr, B_indices, B_indptr, w.count);
     hipLaunchKernelGGL((symbolic_hash_kernel<kGroup6, kSymTable6>), dim3(1024), dim3(kBlock), 0, s, 6, w.bins, w.perm,
-                       A_indices, A_indptr, B_indices, B_indptr, C_indptr);
+                       A_indices, A_indptr, B_indices, B_indptr, w.count);
     NM_LAUNCH_CHECK("symbolic_hash_kernel");
     hipLaunchKernelGGL(symbolic_spill_kernel, dim3(spill_groups(B_cols)), dim3(kSpillBlock), 0, s, w.bins, w.perm, B_cols,
-                       A_indices, A_indptr, B_indices, B_indptr, w.mark, C_indptr);
+                       A_indices, A_indptr, B_indices, B_indptr, w.mark, w.count);
     NM_LAUNCH_CHECK("symbolic_spill_kernel");
     }
-    // counts sit in C_indptr[0, rows), C_indptr[rows] = 0: the exclusive scan is the row pointer
-    if (int rc = nm::scan_exclusive_i64(C_indptr, A_rows + 1, w.scan, s)) return rc;
-    hipLaunchKernelGGL(summary_kernel, dim3(1), dim3(64), 0, s, C_indptr + A_rows,
-                       hashed ? w.bins : (const int32_t *)nullptr, w.summary);
-    NM_LAUNCH_CHECK("summary_kernel");
-    return NM_OK;
+    return row_pointer(w.bins, nullptr);
 }
 
 }  // namespace
@@ -1511,6 +1610,13 @@ extern "C" int nm_spgemm_symbolic_result(int64_t A_rows, int64_t B_cols, const v
     // copy-engine transfer of 16 bytes, takes ~30 us, several times what the kernels of a small
     // product take together.  The ticket is one more than the last one this landing place saw.
     volatile int64_t *both = (volatile int64_t *)host_landing;
+    if (both[3] != 0 && both[3] == (int64_t)reinterpret_cast<intptr_t>(workspace)) {
+        // nm_spgemm_symbolic on this workspace has had the numbers dropped here already
+        both[3] = 0;
+        *nnz_C = both[0];
+        *hash_rows = both[1];
+        return NM_OK;
+    }
     const int64_t ticket = both[2] + 1;
     hipLaunchKernelGGL(summary_out_kernel, dim3(1), dim3(64), 0, s, w.summary, both, ticket);
     NM_LAUNCH_CHECK("summary_out_kernel");

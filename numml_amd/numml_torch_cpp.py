@@ -503,11 +503,11 @@ _landing = threading.local()
 
 
 def _host_landing():
-    """24 bytes of pinned host memory per host thread: where nm_spgemm_symbolic_result has the
+    """32 bytes of pinned host memory per host thread: where nm_spgemm_symbolic_result has the
     device drop nnz(C) (torch's pinned-memory allocator owns it)."""
     t = getattr(_landing, "t", None)
     if t is None:
-        t = _landing.t = torch.zeros(3, dtype=torch.int64).pin_memory()
+        t = _landing.t = torch.zeros(4, dtype=torch.int64).pin_memory()
     return t
 
 

@@ -486,10 +486,14 @@ def test_install_registers_the_reference_module_name(cpp):
             sys.modules["numml_torch_cpp"] = saved
 
 
-@pytest.mark.parametrize("hint", ["given", "unknown"])
+@pytest.mark.parametrize("hint", ["given", "unknown", "landing for the first call only",
+                                  "landing for the second call only"])
 def test_spgemm_through_the_c_abi_with_and_without_the_hash_row_count(dev, hint):
     """The numeric phase takes the number of hash-path rows that nm_spgemm_symbolic_result reports
-    (0 lets it leave the hash launches out), or -1 from a caller that read nnz(C) itself."""
+    (0 lets it leave the hash launches out), or -1 from a caller that read nnz(C) itself.  With a
+    landing place nm_spgemm_symbolic has the numbers landed itself where no row needs the hash
+    path, and the result call after it only reads them; a caller may also give the landing place
+    to one of the two calls only."""
     import ctypes
     from numml_amd import _lib
     L = _lib.lib()
@@ -503,12 +507,17 @@ def test_spgemm_through_the_c_abi_with_and_without_the_hash_row_count(dev, hint)
         work = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
         Cp = torch.empty(r + 1, dtype=torch.int64, device=dev)
         # with a pinned landing place for the device to write into (hint "given"), and without one
-        landing = torch.zeros(3, dtype=torch.int64).pin_memory() if hint == "given" else None
+        landing = torch.zeros(4, dtype=torch.int64).pin_memory() if hint != "unknown" else None
+        first = landing if hint in ("given", "landing for the first call only") else None
+        second = landing if hint in ("given", "landing for the second call only") else None
         _lib.check(L.nm_spgemm_symbolic(r, c, c, ptr(I), ptr(P), ptr(I), ptr(P), ptr(Cp), ptr(work), nbytes.value,
-                                        ptr(landing) if landing is not None else None, st), "symbolic")
+                                        ptr(first) if first is not None else None, st), "symbolic")
         nnz_c, hash_rows = ctypes.c_int64(-7), ctypes.c_int64(-7)
         _lib.check(L.nm_spgemm_symbolic_result(r, c, ptr(work), nbytes.value, ctypes.byref(nnz_c), ctypes.byref(hash_rows),
-                                               ptr(landing) if landing is not None else None, st), "result")
+                                               ptr(second) if second is not None else None, st), "result")
+        if hint == "given":
+            # the note that the numbers had landed is taken back by the call that read them
+            assert int(landing[3]) == 0, name
         Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(r, c, d, i, p, r, c, d, i, p)
         assert nnz_c.value == Cd_ref.shape[0] == int(Cp[-1].item()), name
         assert (hash_rows.value == 0) == name.startswith("stencil"), (name, hash_rows.value)
