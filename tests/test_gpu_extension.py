@@ -528,3 +528,39 @@ def test_spgemm_through_the_c_abi_with_and_without_the_hash_row_count(dev, hint)
         assert_same(host(Cp), Cp_ref, f"{name} C_indptr")
         assert_same(host(Ci), Ci_ref, f"{name} C_indices")
         assert_same(host(Cd), Cd_ref, f"{name} C_data")
+
+
+@pytest.mark.parametrize("landing_given", [True, False])
+def test_spgemm_row_pointer_of_more_rows_than_the_tile_sums_are_added_up_in_place_for(dev, landing_given):
+    """Past 4096 tiles of 2048 rows the sums of the tiles are scanned by a launch of their own
+    before the row pointer is written, and the first workgroup reads nnz(C) behind them.  A
+    product of two diagonal matrices of 9 000 000 rows has a closed form: the row pointer counts
+    up by one, the columns are the rows, the values the products of the diagonals."""
+    import ctypes
+    from numml_amd import _lib
+    L = _lib.lib()
+    n = 9_000_000
+    D = torch.arange(1, n + 1, dtype=torch.float64, device=dev) * 0.5
+    I = torch.arange(n, dtype=torch.int64, device=dev)
+    P = torch.arange(n + 1, dtype=torch.int64, device=dev)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(L.nm_spgemm_workspace_bytes(n, n, ctypes.byref(nbytes)), "bytes")
+    work = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+    Cp = torch.full((n + 1,), -1, dtype=torch.int64, device=dev)
+    landing = torch.zeros(4, dtype=torch.int64).pin_memory() if landing_given else None
+    where = ptr(landing) if landing_given else None
+    _lib.check(L.nm_spgemm_symbolic(n, n, n, ptr(I), ptr(P), ptr(I), ptr(P), ptr(Cp), ptr(work), nbytes.value,
+                                    where, st), "symbolic")
+    nnz_c, hash_rows = ctypes.c_int64(-7), ctypes.c_int64(-7)
+    _lib.check(L.nm_spgemm_symbolic_result(n, n, ptr(work), nbytes.value, ctypes.byref(nnz_c), ctypes.byref(hash_rows),
+                                           where, st), "result")
+    assert (nnz_c.value, hash_rows.value) == (n, 0)
+    assert torch.equal(Cp, P)
+    Ci = torch.empty(n, dtype=torch.int64, device=dev)
+    Cd = torch.empty(n, dtype=torch.float64, device=dev)
+    _lib.check(L.nm_spgemm_numeric(1, n, n, n, ptr(D), ptr(I), ptr(P), ptr(D), ptr(I), ptr(P), ptr(Cp), ptr(Ci), ptr(Cd),
+                                   ptr(work), nbytes.value, hash_rows.value, st), "numeric")
+    assert torch.equal(Ci, I)
+    assert torch.equal(Cd, D * D)
