@@ -243,10 +243,16 @@ int nm_spdmm_backward_planned(nm_dtype dt, int64_t rows, int64_t cols, int64_t n
  *                                 nm_spgemm_symbolic_result that follows on the
  *                                 same workspace and landing place then returns
  *                                 at once
- *   nm_spgemm_symbolic_result  -> waits for the symbolic phase and hands the
- *                                 host nnz(C) = C_indptr[A_rows], with which
- *                                 the caller allocates, and the number of rows
- *                                 the hash path took (the reference's own
+ *   nm_spgemm_symbolic_result  -> hands the host nnz(C) = C_indptr[A_rows],
+ *                                 with which the caller allocates, and the
+ *                                 number of rows the hash path took.  With a
+ *                                 landing place it returns when the two numbers
+ *                                 are known, which can be before the last
+ *                                 entries of C_indptr are written: C_indptr is
+ *                                 complete for work queued on `stream` after
+ *                                 this call, not for another stream or a host
+ *                                 read without hipStreamSynchronize.  With NULL
+ *                                 it waits for the stream (the reference's own
  *                                 read of the last row pointer,
  *                                 cpp/sparse_csr_cpu.cpp:166, is this
  *                                 synchronisation point); a caller may read
