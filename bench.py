@@ -662,9 +662,9 @@ class SpGEMM(Workload):
         # the path every first product on a pair of patterns takes (and the only one for rows
         # beyond a plan's limits): merge kernels where every row is short, the hash kernels otherwise
         hashed = self.left == "AA" or self.right == "AA"
-        fwd_name = ("symbolic_hash_kernel + numeric_hash_kernel (row-binned LDS hash tables) + scans, host read of nnz(C)"
+        fwd_name = ("symbolic_hash_kernel + numeric_hash_kernel (row-binned LDS hash tables) + row_pointer_kernel, host read of nnz(C)"
                     if hashed else "symbolic_front_kernel (merge path, recording where each product goes in scratch of the call) "
-                    "+ numeric_planned_kernel<COLS> (products added on those records) + scans, host read of nnz(C)")
+                    "+ numeric_planned_kernel<COLS> (products added on those records) + row_pointer_kernel, host read of nnz(C)")
         rec["roofline_stateless"] = {
             "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "kernels": [
