@@ -564,3 +564,37 @@ def test_spgemm_row_pointer_of_more_rows_than_the_tile_sums_are_added_up_in_plac
                                    ptr(work), nbytes.value, hash_rows.value, st), "numeric")
     assert torch.equal(Ci, I)
     assert torch.equal(Cd, D * D)
+
+
+@pytest.mark.parametrize("rows", [1, 2047, 2048, 4095, 4096, 6143, 10_000])
+def test_spgemm_row_pointer_at_tile_boundaries_and_in_unaligned_memory(dev, rows):
+    """The row pointer is written 16 bytes at a time where a tile of 2048 of its entries is whole and
+    the arrays allow it, entry by entry otherwise: row counts around the tile size, into a row
+    pointer that starts 8 bytes off a 16-byte boundary, against the oracle."""
+    import ctypes
+    from numml_amd import _lib
+    L = _lib.lib()
+    d, i, p, (r, c) = G.tridiag(rows, np.float64)
+    D, I, P = to_dev(dev, d, i, p)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(L.nm_spgemm_workspace_bytes(r, c, ctypes.byref(nbytes)), "bytes")
+    Cd_ref, Ci_ref, Cp_ref = oracle.spgemm_forward(r, c, d, i, p, r, c, d, i, p)
+    landing = torch.zeros(4, dtype=torch.int64).pin_memory()
+    for shift in (0, 1):
+        work = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+        room = torch.full((r + 2,), -1, dtype=torch.int64, device=dev)
+        Cp = room[shift:shift + r + 1]
+        assert Cp.data_ptr() % 16 == 8 * shift
+        _lib.check(L.nm_spgemm_symbolic(r, c, c, ptr(I), ptr(P), ptr(I), ptr(P), ptr(Cp), ptr(work), nbytes.value,
+                                        ptr(landing), st), "symbolic")
+        nnz_c, hash_rows = ctypes.c_int64(-7), ctypes.c_int64(-7)
+        _lib.check(L.nm_spgemm_symbolic_result(r, c, ptr(work), nbytes.value, ctypes.byref(nnz_c),
+                                               ctypes.byref(hash_rows), ptr(landing), st), "result")
+        assert (nnz_c.value, hash_rows.value) == (Cd_ref.shape[0], 0), (rows, shift)
+        assert_same(host(Cp), Cp_ref, f"{rows} rows, shift {shift}: C_indptr")
+        if shift:   # the entry before the row pointer is nobody's
+            assert int(room[0].item()) == -1
+        else:
+            assert int(room[r + 1].item()) == -1
