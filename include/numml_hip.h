@@ -366,8 +366,11 @@ int nm_spgemm_backward_planned(nm_dtype dt, int64_t A_rows, int64_t A_cols, int6
  *   nm_spgemm_numeric_mapped    nm_spgemm_numeric that, when hash_rows is 0 (every row
  *                           on the merge path, from nm_spgemm_symbolic_result) and
  *                           C_nnz < 2^31, adds the products up on those records
- *                           instead of merging the rows a second time, and fills in
- *                           the plan's C row starts; otherwise it is nm_spgemm_numeric
+ *                           instead of merging the rows a second time, and, with
+ *                           keep_plan != 0, fills in the plan's C row starts (4 bytes
+ *                           per entry of A that a caller who will not adopt the plan
+ *                           need not have written: keep_plan == 0, plan_mem is then
+ *                           scratch of the call); otherwise it is nm_spgemm_numeric
  *                           and plan_mem holds nothing usable.  Same results, bit
  *                           for bit.
  *   nm_spgemm_plan_adopt    checks what such a plan still needs before the kernels
@@ -386,7 +389,7 @@ int nm_spgemm_numeric_mapped(nm_dtype dt, int64_t A_rows, int64_t A_cols, int64_
                              const void *B_data, const int64_t *B_indices, const int64_t *B_indptr,
                              const int64_t *C_indptr, int64_t *C_indices, void *C_data,
                              void *workspace, size_t workspace_bytes, int64_t hash_rows,
-                             void *plan_mem, size_t plan_bytes, nm_stream stream);
+                             void *plan_mem, size_t plan_bytes, int keep_plan, nm_stream stream);
 int nm_spgemm_plan_adopt(int64_t A_rows, int64_t A_cols, int64_t A_nnz, int64_t B_nnz, int64_t C_nnz,
                          int64_t hash_rows, const void *A_plan_mem, void *plan_mem, size_t plan_bytes,
                          void *host_landing, int *usable, nm_stream stream);

@@ -59,7 +59,7 @@ _SIGNATURES = {
                                   _c_ptr, _c_size, _c_ptr, _c_size, _c_ptr, _c_ptr],
     "nm_spgemm_numeric_mapped": [_c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_i64, _c_ptr, _c_size,
-                                 _c_ptr],
+                                 _c_int, _c_ptr],
     "nm_spgemm_plan_adopt": [_c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_size, _c_ptr,
                              ctypes.POINTER(_c_int), _c_ptr],
     "nm_spgemm_plan_bytes": [_c_i64, ctypes.POINTER(_c_size)],

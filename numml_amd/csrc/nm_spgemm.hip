@@ -76,7 +76,7 @@ struct Work {
     int32_t *key;      // [rows] binning key (product bound, then exact length)
     int32_t *perm;     // [rows] rows grouped by bin
     int32_t *bins;     // [kBinInts]: rows per bin [0, kBins), first row of bin b at kBinStart + b (end at + b + 1), cursor at kBinCursor + b
-    int64_t *count;    // [rows + 1] entries per row of C, before the row pointer is made of them
+    int32_t *count;    // [rows + 1] entries per row of C, before the row pointer is made of them
     int64_t *scan;     // [tiles + 1] sums of the counts by tile of the row pointer's scan
     int32_t *mark;     // [spill_groups(B_cols) * B_cols]
     double *acc;       // [spill_groups(B_cols) * B_cols]
@@ -95,7 +95,7 @@ size_t work_layout(int64_t rows, int64_t B_cols, void *base, Work *w) {
     int32_t *key = (int32_t *)take((rows + 1) * 4);
     int32_t *perm = (int32_t *)take((rows + 1) * 4);
     int32_t *bins = (int32_t *)take(kBinInts * 4);
-    int64_t *count = (int64_t *)take((size_t)(rows + 1) * 8);
+    int32_t *count = (int32_t *)take((size_t)(rows + 1) * 4);
     int64_t *scan = (int64_t *)take(nm::scan_scratch_bytes(rows + 1));
     int64_t *summary = (int64_t *)take(2 * 8);
     int32_t *mark = (int32_t *)take((size_t)spill_groups(B_cols) * (B_cols + 1) * 4);
@@ -215,7 +215,7 @@ __device__ __forceinline__ void merge_stage(int64_t bb, int len, const int64_t *
 __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     int64_t rows, int64_t nbatch_padded, const int64_t *__restrict__ A_indices,
     const int64_t *__restrict__ A_indptr, const int64_t *__restrict__ B_indices,
-    const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key, int64_t *__restrict__ C_count,
+    const int64_t *__restrict__ B_indptr, int32_t *__restrict__ key, int32_t *__restrict__ C_count,
     unsigned long long *__restrict__ hash_rows, unsigned long long token, uint64_t *__restrict__ dest,
     int32_t *__restrict__ bstart) {
     __shared__ int32_t s_col[(kMergeCap + 1) * kMergeStride];
@@ -250,33 +250,43 @@ __global__ __launch_bounds__(kBlock) void symbolic_front_kernel(
     // held before is not this call's token, or at worst makes the hash path run over no rows.
     if (live && !merge && gl == 0) *hash_rows = token;
     merge_stage<float, false>(my_bb, merge ? my_len : 0, B_indices, nullptr, A_indptr, s_bb, s_len, s_col, nullptr);
-    const int32_t *pc = s_col + threadIdx.x;
+    int32_t *pc = s_col + threadIdx.x;
     int32_t cur = *pc;
-    int cnt = 0, it = 0;
-    // With `dest` given the merge also leaves behind WHERE every product goes: byte k of a lane's
-    // word is the pass in which the k-th entry of its B row was taken, i.e. the position of that
-    // entry's column in the row of C (0xFF: no such entry).  The numeric phase can then add the
-    // products up without merging again, and the words are what a product plan is made of.
-    uint64_t where = ~uint64_t(0);
-    int shift = 0;
+    int it = 0, last = -1;
+    // The merge also leaves behind WHERE every product goes: the pass in which the k-th entry of a
+    // lane's B row is taken is the position of that entry's column in the row of C.  A column that
+    // has been taken is not needed again, so the pass is written over it in LDS -- one store, where
+    // shifting it into a 64-bit word cost five vector instructions in a loop that is bound by what
+    // it issues -- and the words the numeric phase adds the products up on (byte k = the pass of
+    // entry k, 0xFF: no such entry; also what a product plan is made of) are put together after the
+    // loop: the low byte of a place never taken is the past-the-end column's, 0xFF.
+    static_assert((kColEnd & 0xFF) == 0xFF, "an entry never taken reads as no entry");
     for (;;) {
         const int32_t m = merge_min(cur);
         const bool open = m != kColEnd;
         if (__ballot(open) == 0) break;
         if (cur == m && open) {
-            where ^= (uint64_t)(0xFF ^ it) << shift;
-            shift += 8;
+            last = it;
+            *pc = it;
             pc += kMergeStride;
             cur = *pc;
         }
         ++it;
-        if (open) cnt = it;   // an open group emits one column per pass
     }
+    const int cnt = merge_max(last) + 1;   // an open group emits one column per pass
     if (merge && gl == 0) {
         C_count[row] = cnt;
         key[row] = kMergedKey;
     }
     if (dest && merge && ab + gl < ae) {   // (read once, by another kernel: nontemporal)
+        const int32_t *mine = s_col + threadIdx.x;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            lo |= ((uint32_t)mine[j * kMergeStride] & 0xFFu) << (8 * j);
+            hi |= ((uint32_t)mine[(4 + j) * kMergeStride] & 0xFFu) << (8 * j);
+        }
+        const uint64_t where = ((uint64_t)hi << 32) | lo;
         __builtin_nontemporal_store(where, dest + ab + gl);
         __builtin_nontemporal_store((int32_t)my_bb, bstart + ab + gl);
     }
@@ -506,6 +516,34 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
     }
 }
 
+// Sums of the rows' counts by tile of kScanTile rows: the first pass of the row pointer's scan.
+typedef int32_t I32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bool count_tile_whole(const int32_t *a, int64_t n) {
+    static_assert(nm::kScanItems % 4 == 0, "counts are loaded four at a time");
+    return ((int64_t)blockIdx.x + 1) * nm::kScanTile <= n && (reinterpret_cast<uintptr_t>(a) & 15) == 0;
+}
+__global__ __launch_bounds__(nm::kScanBlock) void count_tile_sums_kernel(const int32_t *__restrict__ count, int64_t n,
+                                                                       int64_t *__restrict__ sums) {
+    __shared__ int64_t s_wave[nm::kScanBlock / kWave];
+    const int64_t base = (int64_t)blockIdx.x * nm::kScanTile + (int64_t)threadIdx.x * nm::kScanItems;
+    int64_t v = 0;
+    if (count_tile_whole(count, n)) {
+        const I32x4 *p = reinterpret_cast<const I32x4 *>(count + base);
+#pragma unroll
+        for (int i = 0; i < nm::kScanItems / 4; ++i) {
+            const I32x4 w = p[i];
+            v += (int64_t)w[0] + w[1] + w[2] + w[3];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < nm::kScanItems; ++i)
+            if (base + i < n) v += count[base + i];
+    }
+    int64_t total;
+    nm::block_exclusive_scan(v, s_wave, total);
+    if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
 // Row pointer of C from the rows' counts, and what the host needs between the phases: nnz(C) and
 // the rows the hash path took.  count[0, n) with count[n - 1] == 0 -> C_indptr[0, n) (its exclusive
 // scan, not in place: the counts of the merge path's rows survive a pass made before the hash
@@ -519,23 +557,25 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(int64_t rows, const
 // not the row pointer, so it is told first and sizes C while the row pointer is being written.
 constexpr int kInlineTiles = 4096;
 __global__ __launch_bounds__(nm::kScanBlock) void row_pointer_kernel(
-    const int64_t *__restrict__ count, int64_t n, const int64_t *__restrict__ sums, int scanned,
+    const int32_t *__restrict__ count, int64_t n, const int64_t *__restrict__ sums, int scanned,
     int64_t *__restrict__ C_indptr, const int32_t *__restrict__ bins, int64_t *__restrict__ summary,
     int64_t token, volatile int64_t *host_pinned, int64_t ticket) {
     using nm::kScanItems;
     __shared__ int64_t s_wave[nm::kScanBlock / kWave];
     const int64_t base = (int64_t)blockIdx.x * nm::kScanTile + (int64_t)threadIdx.x * kScanItems;
-    int64_t item[kScanItems];
+    int32_t item[kScanItems];
     int64_t v = 0;
-    const bool whole = nm::scan_tile_whole(count, n) && (reinterpret_cast<uintptr_t>(C_indptr) & 15) == 0;
+    const bool whole = count_tile_whole(count, n) && (reinterpret_cast<uintptr_t>(C_indptr) & 15) == 0;
     if (whole) {
-        const nm::I64x2 *p = reinterpret_cast<const nm::I64x2 *>(count + base);
+        const I32x4 *p = reinterpret_cast<const I32x4 *>(count + base);
 #pragma unroll
-        for (int i = 0; i < kScanItems / 2; ++i) {
-            const nm::I64x2 w = p[i];
-            item[2 * i] = w[0];
-            item[2 * i + 1] = w[1];
-            v += w[0] + w[1];
+        for (int i = 0; i < kScanItems / 4; ++i) {
+            const I32x4 w = p[i];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                item[4 * i + u] = w[u];
+                v += w[u];
+            }
         }
     } else {
 #pragma unroll
@@ -690,7 +730,7 @@ __global__ __launch_bounds__(kBlock) void symbolic_hash_kernel(
     int bin, const int32_t *__restrict__ bins, const int32_t *__restrict__ perm,
     const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
     const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr,
-    int64_t *__restrict__ C_count) {
+    int32_t *__restrict__ C_count) {
     constexpr int GPB = kBlock / G;
     // the tables of the groups that share a wavefront start kTablePad entries apart in
     // bank space; without the pad they would all map slot t to the same LDS bank
@@ -803,7 +843,7 @@ __global__ __launch_bounds__(kSpillBlock) void symbolic_spill_kernel(
     const int32_t *__restrict__ bins, const int32_t *__restrict__ perm, int64_t B_cols,
     const int64_t *__restrict__ A_indices, const int64_t *__restrict__ A_indptr,
     const int64_t *__restrict__ B_indices, const int64_t *__restrict__ B_indptr, int32_t *mark_all,
-    int64_t *__restrict__ C_count) {
+    int32_t *__restrict__ C_count) {
     __shared__ int s_red[kSpillBlock / kWave];
     const int32_t b0 = bins[kBinStart + kBins - 1], b1 = bins[kBinStart + kBins];
     if (b0 + (int32_t)blockIdx.x >= b1) return;
@@ -1499,9 +1539,9 @@ int symbolic_phase(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t
     NM_LAUNCH_CHECK("symbolic_front_kernel");
     // The row pointer from the counts: their sums by tile, then the pass that writes it.
     auto row_pointer = [&](const int32_t *bins, volatile int64_t *landing) -> int {
-        hipLaunchKernelGGL(nm::scan_tile_sums_kernel, dim3((unsigned)tiles), dim3(nm::kScanBlock), 0, s, w.count,
+        hipLaunchKernelGGL(count_tile_sums_kernel, dim3((unsigned)tiles), dim3(nm::kScanBlock), 0, s, w.count,
                            A_rows + 1, w.scan);
-        NM_LAUNCH_CHECK("scan_tile_sums_kernel");
+        NM_LAUNCH_CHECK("count_tile_sums_kernel");
         const bool scanned = tiles > kInlineTiles;
         if (scanned) {
             hipLaunchKernelGGL(nm::scan_sums_kernel, dim3(1), dim3(1024), 0, s, w.scan, tiles);
@@ -1514,7 +1554,7 @@ int symbolic_phase(int64_t A_rows, int64_t A_cols, int64_t B_cols, const int64_t
     };
     // With a landing place in pinned host memory the row pointer is made at once, as if the first
     // kernel had taken every row (it has, for a product of stencil or aggregation matrices), and its
-    // last workgroup tells the host nnz(C) and whether a row was left to the hash path.  If none was,
+    // first workgroup tells the host nnz(C) and whether a row was left to the hash path.  If none was,
     // that was the symbolic phase: the binning and the nine launches of the hash path, which would
     // find nothing to do, are left out, and nm_spgemm_symbolic_result finds its answer landed (the
     // workspace's address in the landing place's fourth word says so).  Otherwise the pass was for
@@ -1678,7 +1718,7 @@ extern "C" int nm_spgemm_numeric_mapped(nm_dtype dt, int64_t A_rows, int64_t A_c
                                         const int64_t *A_indptr, const void *B_data, const int64_t *B_indices,
                                         const int64_t *B_indptr, const int64_t *C_indptr, int64_t *C_indices,
                                         void *C_data, void *workspace, size_t workspace_bytes, int64_t hash_rows,
-                                        void *plan_mem, size_t plan_bytes, nm_stream stream) {
+                                        void *plan_mem, size_t plan_bytes, int keep_plan, nm_stream stream) {
     // rows on the hash path (or an unknown number of them), or positions beyond 31 bits: the map
     // the symbolic phase left is incomplete or unusable, the ordinary numeric phase runs
     if (hash_rows != 0 || !plan_mem || A_nnz <= 0 || C_nnz <= 0 || C_nnz >= ((int64_t)1 << 31))
@@ -1692,7 +1732,7 @@ extern "C" int nm_spgemm_numeric_mapped(nm_dtype dt, int64_t A_rows, int64_t A_c
     nm::PPlan map;
     nm::pplan_layout(A_nnz, plan_mem, &map);
     return nm::spgemm_numeric_on_map(dt, A_rows, A_nnz, A_data, A_indptr, B_data, B_indices, map, C_indptr, C_indices,
-                                     C_data, nm::as_stream(stream));
+                                     C_data, keep_plan != 0, nm::as_stream(stream));
 }
 
 extern "C" int nm_spgemm_backward(nm_dtype dt, int64_t A_rows, int64_t A_nnz, int64_t B_nnz, const void *gC,

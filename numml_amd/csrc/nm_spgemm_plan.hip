@@ -317,7 +317,7 @@ __global__ __launch_bounds__(kBlock) void numeric_planned_kernel(
         s_av[threadIdx.x] = av;
         s_bs[threadIdx.x] = bs;
         *reinterpret_cast<uint64_t *>(s_db + threadIdx.x * kCap) = k < alen ? db : ~uint64_t(0);
-        if (COLS && k < alen) __builtin_nontemporal_store((int32_t)cs, cstart + e);
+        if (COLS && cstart && k < alen) __builtin_nontemporal_store((int32_t)cs, cstart + e);
     }
     group_fence();
     const int slot = g * kCap;
@@ -1037,18 +1037,20 @@ extern "C" int nm_spgemm_numeric_planned(nm_dtype dt, int plan_class, int64_t A_
 
 int nm::spgemm_numeric_on_map(nm_dtype dt, int64_t A_rows, int64_t A_nnz, const void *A_data,
                               const int64_t *A_indptr, const void *B_data, const int64_t *B_indices, const PPlan &p,
-                              const int64_t *C_indptr, int64_t *C_indices, void *C_data, hipStream_t s) {
+                              const int64_t *C_indptr, int64_t *C_indices, void *C_data, bool keep, hipStream_t s) {
+    // (the plan's C row starts are written only for a caller that may make a plan of the records)
+    int32_t *cstart = keep ? p.cstart : nullptr;
     if (A_rows == 0 || A_nnz == 0) return NM_OK;
     const int64_t grid = nm::xcd_padded(nm::ceil_div(A_rows, (int64_t)kGroupsPerBlock));
     NM_REQUIRE(grid < nm::kMaxGrid, "too many rows");
     if (dt == NM_F32)
         hipLaunchKernelGGL((numeric_planned_kernel<float, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            grid, (const float *)A_data, A_indptr, (const float *)B_data, B_indices, p.bstart, p.dest,
-                           C_indptr, (float *)C_data, C_indices, p.cstart, (const uint32_t *)nullptr);
+                           C_indptr, (float *)C_data, C_indices, cstart, (const uint32_t *)nullptr);
     else
         hipLaunchKernelGGL((numeric_planned_kernel<double, true>), dim3((unsigned)grid), dim3(kBlock), 0, s, A_rows,
                            grid, (const double *)A_data, A_indptr, (const double *)B_data, B_indices, p.bstart, p.dest,
-                           C_indptr, (double *)C_data, C_indices, p.cstart, (const uint32_t *)nullptr);
+                           C_indptr, (double *)C_data, C_indices, cstart, (const uint32_t *)nullptr);
     NM_LAUNCH_CHECK("numeric_planned_kernel");
     return NM_OK;
 }

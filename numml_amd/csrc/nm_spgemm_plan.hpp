@@ -57,10 +57,10 @@ inline size_t pplan_layout(int64_t A_nnz, void *base, PPlan *p, int octets = 1) 
 }
 
 // C_data AND C_indices of the product from the destination bytes and row starts of B that the
-// symbolic phase left in `p` (every row on the merge path); also writes p.cstart, which completes
-// the plan.  C_indptr is the scanned row pointer.
+// symbolic phase left in `p` (every row on the merge path); with `keep` also writes p.cstart, which
+// completes the plan.  C_indptr is the scanned row pointer.
 int spgemm_numeric_on_map(nm_dtype dt, int64_t A_rows, int64_t A_nnz, const void *A_data, const int64_t *A_indptr,
                           const void *B_data, const int64_t *B_indices, const PPlan &p, const int64_t *C_indptr,
-                          int64_t *C_indices, void *C_data, hipStream_t s);
+                          int64_t *C_indices, void *C_data, bool keep, hipStream_t s);
 
 }  // namespace nm

@@ -1183,7 +1183,7 @@ std::vector<Tensor> spgemm_forward(int A_rows, int A_cols, Tensor A_data, Tensor
                                    B_indices.data_ptr<int64_t>(), B_indptr.data_ptr<int64_t>(),
                                    C_indptr.data_ptr<int64_t>(), C_indices.data_ptr<int64_t>(), C_data.data_ptr(),
                                    work.data_ptr(), bytes, hash_rows, on_map ? filled.data_ptr() : nullptr, pbytes,
-                                   st),
+                                   plans ? 1 : 0, st),
           "nm_spgemm_numeric_mapped");
     // note the pair, or make its plan: from the memory this pass filled, or (rows on the hash
     // path: the plan's own analysis says whether the product is within its limits) from the patterns

@@ -626,7 +626,7 @@ def spgemm_forward_mapped(A_rows, A_cols, A_data, A_indices, A_indptr,
         _lib.check(L.nm_spgemm_numeric_mapped(
             _dt(A_data), A_rows, A_cols, B_cols, A_nnz, nnz_c.value, _ptr(A_data), _ptr(A_indices),
             _ptr(A_indptr), _ptr(B_data), _ptr(B_indices), _ptr(B_indptr), _ptr(C_indptr), _ptr(C_indices),
-            _ptr(C_data), _ptr(work), nbytes.value, hash_rows.value, _ptr(mem), pbytes.value, st),
+            _ptr(C_data), _ptr(work), nbytes.value, hash_rows.value, _ptr(mem), pbytes.value, 1, st),
             "nm_spgemm_numeric_mapped")
         plan = ProductPlan(A_rows, A_cols, A_indices, A_indptr, B_indices, B_indptr, C_indices, C_indptr,
                            adopt=(mem, hash_rows.value))
