@@ -598,3 +598,28 @@ def test_spgemm_row_pointer_at_tile_boundaries_and_in_unaligned_memory(dev, rows
             assert int(room[0].item()) == -1
         else:
             assert int(room[r + 1].item()) == -1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_spgemm_forward_with_plans_switched_off(dev, cpp, dtype):
+    """In the stateless mode the forward still adds the products up on the records of its own
+    symbolic merge where every row is short, but leaves out what only a plan made of those records
+    would read (keep_plan == 0): the same bits as the oracle's, twice in a row, and nothing is kept."""
+    cpp.set_backward_mode("atomic")
+    try:
+        for name, (ad, ai, ap, (m, k)), (bd, bi, bp, (k2, n)) in (
+                ("stencil", G.poisson2d(37, dtype, 3), G.poisson2d(37, dtype, 4)),
+                ("tridiagonal, 5000 rows", G.tridiag(5000, dtype), G.tridiag(5000, dtype, 1.0, -2.0, 1.0)),
+                ("random: rows on both paths", G.random_csr(400, 300, 0.03, 5, dtype),
+                 G.random_csr(300, 500, 0.03, 6, dtype))):
+            cpp.clear_plan_cache()
+            AD, AI, AP, BD, BI, BP = to_dev(dev, ad, ai, ap, bd, bi, bp)
+            rd, ri, rp = oracle.spgemm_forward(m, k, ad, ai, ap, k2, n, bd, bi, bp)
+            for call in range(2):
+                Cd, Ci, Cp = cpp.spgemm_forward(m, k, AD, AI, AP, k2, n, BD, BI, BP)
+                assert_same(host(Cp), rp, f"{name}, call {call}: C_indptr")
+                assert_same(host(Ci), ri, f"{name}, call {call}: C_indices")
+                assert_same(host(Cd), rd, f"{name}, call {call}: C_data")
+            assert cpp.plan_cache_size() == 0, name
+    finally:
+        cpp.set_backward_mode("eager")
