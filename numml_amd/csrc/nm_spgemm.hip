@@ -1251,6 +1251,18 @@ constexpr int kBwdLongChunk = 256;   // rows a workgroup of the long-row kernel 
 constexpr int kBwdWide = 64;         // rows of B longer than this are walked by a whole wavefront ...
 constexpr int kBwdWideCap = 1024;    // ... up to this many per row of A (the rest stay with their group)
 
+// What the last of every eight consecutive lanes holds, handed to all eight (ds_swizzle in bit
+// mode: lane = (lane & 0x18) | 7 inside each half of the wavefront; no address to compute).
+__device__ __forceinline__ float group_last(float v) {
+    return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x00F8));
+}
+__device__ __forceinline__ double group_last(double v) {
+    const long long bits = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_ds_swizzle((int)(bits & 0xffffffffll), 0x00F8);
+    const int hi = __builtin_amdgcn_ds_swizzle((int)(bits >> 32), 0x00F8);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
     int64_t A_rows, const T *__restrict__ gC, const int64_t *__restrict__ C_indices,
@@ -1259,6 +1271,7 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
     const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
     const int64_t *__restrict__ B_indptr, T *__restrict__ grad_A, T *__restrict__ grad_B) {
     constexpr int G = kBwdG, GPB = kBlock / G;
+    static_assert(G == 8 && kBwdStage == 64, "group_last and the six-step search are written for these");
     __shared__ int32_t s_ci[GPB * kBwdStage];
     __shared__ T s_g[GPB * kBwdStage];
     const int gl = threadIdx.x % G, gi = G >= kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x / G) : threadIdx.x / G;
@@ -1271,10 +1284,12 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
         const int64_t cb = live ? C_indptr[i] : 0, ce = live ? C_indptr[i + 1] : 0;
         const int clen = (int)(ce - cb < 0x7fffffff ? ce - cb : 0x7fffffff);
         const bool here = live && clen <= kBwdStage;   // longer rows are left to spgemm_bwd_long_kernel
+        // (places past the row's end hold a column no entry has: the search below takes six steps
+        // whatever the row's length and needs no bound)
         if (here)
-            for (int t = gl; t < clen; t += G) {
-                ci[t] = (int32_t)C_indices[cb + t];
-                cg[t] = gC[cb + t];
+            for (int t = gl; t < kBwdStage; t += G) {
+                ci[t] = t < clen ? (int32_t)C_indices[cb + t] : 0x7fffffff;
+                if (t < clen) cg[t] = gC[cb + t];
             }
         group_sync<G>();
         const int64_t ab = here ? A_indptr[i] : 0, ae = here ? A_indptr[i + 1] : 0;
@@ -1294,24 +1309,25 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
                 for (int64_t kk0 = bb; kk0 < be; kk0 += G) {
                     const int64_t kk = kk0 + gl;
                     const bool have = kk < be;
-                    const int64_t c = have ? B_indices[kk] : -1;
+                    const int32_t c = have ? (int32_t)B_indices[kk] : -1;
                     const T bval = have ? B_data[kk] : T(0);
-                    int l = 0, h = clen;
-                    while (l < h) {
-                        const int mid = (l + h) >> 1;
-                        if ((int64_t)ci[mid] < c) l = mid + 1; else h = mid;
-                    }
-                    const bool hit = have && l < clen && (int64_t)ci[l] == c;
+                    // the number of staged columns below c (at most 63), in six steps without a branch
+                    int l = 0;
+#pragma unroll
+                    for (int step = kBwdStage / 2; step > 0; step >>= 1)
+                        if (ci[l + step - 1] < c) l += step;
+                    const bool hit = have && ci[l] == c;
                     const T g = hit ? cg[l] : T(0);
                     if (hit && grad_B) nm::atomic_add(grad_B + kk, a * g);
-                    const T prod = g * bval;
-                    // ordered sum over the group's lanes = ascending column
-                    const int cnt = (int)(be - kk0 < G ? be - kk0 : G);
-                    for (int l2 = 0; l2 < cnt; ++l2) {
-                        const T pl = __shfl(prod, gbase + l2, kWave);
-                        const int hl = __shfl((int)hit, gbase + l2, kWave);
-                        if (hl) acc += pl;
-                    }
+                    // Ordered sum over the group's lanes = ascending column: the running sum walks up
+                    // the lanes, one DPP shift and one addition a step (every lane adds what its lower
+                    // neighbour held a step ago to its own product; lane s is right after step s and
+                    // is read at step s + 1, what the others hold meanwhile is never used).  A lane
+                    // without a product adds +0.0, which changes no sum that began at +0.0.
+                    T run = acc + (hit ? g * bval : T(0));
+#pragma unroll
+                    for (int step = 1; step < G; ++step) run = nm::dpp_move<0x111>(run) + (hit ? g * bval : T(0));
+                    acc = group_last(run);
                 }
                 if (gl == e) my_acc = acc;
             }
