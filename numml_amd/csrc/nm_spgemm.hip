@@ -1251,16 +1251,21 @@ constexpr int kBwdLongChunk = 256;   // rows a workgroup of the long-row kernel 
 constexpr int kBwdWide = 64;         // rows of B longer than this are walked by a whole wavefront ...
 constexpr int kBwdWideCap = 1024;    // ... up to this many per row of A (the rest stay with their group)
 
-// What the last of every eight consecutive lanes holds, handed to all eight (ds_swizzle in bit
-// mode: lane = (lane & 0x18) | 7 inside each half of the wavefront; no address to compute).
-__device__ __forceinline__ float group_last(float v) {
-    return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x00F8));
+// What lane E of every eight consecutive lanes holds, handed to all eight (ds_swizzle in bit mode:
+// lane = (lane & 0x18) | E inside each half of the wavefront; no address to compute).
+template <int E> __device__ __forceinline__ int group_lane(int v) {
+    static_assert(E >= 0 && E < 8, "a lane of the group");
+    return __builtin_amdgcn_ds_swizzle(v, (E << 5) | 0x18);
 }
-__device__ __forceinline__ double group_last(double v) {
-    const long long bits = __double_as_longlong(v);
-    const int lo = __builtin_amdgcn_ds_swizzle((int)(bits & 0xffffffffll), 0x00F8);
-    const int hi = __builtin_amdgcn_ds_swizzle((int)(bits >> 32), 0x00F8);
-    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+template <int E> __device__ __forceinline__ float group_lane(float v) {
+    return __int_as_float(group_lane<E>(__float_as_int(v)));
+}
+template <int E> __device__ __forceinline__ int64_t group_lane(int64_t v) {
+    const int lo = group_lane<E>((int)(v & 0xffffffffll)), hi = group_lane<E>((int)(v >> 32));
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+template <int E> __device__ __forceinline__ double group_lane(double v) {
+    return __longlong_as_double(group_lane<E>((int64_t)__double_as_longlong(v)));
 }
 
 template <typename T>
@@ -1271,13 +1276,16 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
     const T *__restrict__ B_data, const int64_t *__restrict__ B_indices,
     const int64_t *__restrict__ B_indptr, T *__restrict__ grad_A, T *__restrict__ grad_B) {
     constexpr int G = kBwdG, GPB = kBlock / G;
-    static_assert(G == 8 && kBwdStage == 64, "group_last and the six-step search are written for these");
-    __shared__ int32_t s_ci[GPB * kBwdStage];
-    __shared__ T s_g[GPB * kBwdStage];
+    static_assert(G == 8 && kBwdStage == 64, "group_lane and the six-step search are written for these");
+    // (a group's row starts one bank further on than its neighbour's: the groups of a wavefront
+    // probe the same place of their rows at the same step of the search)
+    constexpr int kStride = kBwdStage + 1;
+    __shared__ int32_t s_ci[GPB * kStride];
+    __shared__ T s_g[GPB * kStride];
     const int gl = threadIdx.x % G, gi = G >= kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x / G) : threadIdx.x / G;
     const int gbase = (threadIdx.x & (kWave - 1)) & ~(G - 1);   // first lane of the group inside its wavefront
-    int32_t *ci = s_ci + gi * kBwdStage;
-    T *cg = s_g + gi * kBwdStage;
+    int32_t *ci = s_ci + gi * kStride;
+    T *cg = s_g + gi * kStride;
     for (int64_t i0 = (int64_t)blockIdx.x * GPB; i0 < A_rows; i0 += (int64_t)gridDim.x * GPB) {
         const int64_t i = i0 + gi;
         const bool live = i < A_rows;
@@ -1301,16 +1309,21 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
             const T my_a = (mine && grad_B) ? A_data[my_ai] : T(0);
             const int64_t my_bb = mine ? B_indptr[my_k] : 0, my_be = mine ? B_indptr[my_k + 1] : 0;
             const int nb = (int)(ae - a0 < G ? ae - a0 : G);
+            const int my_len = (int)(my_be - my_bb);
             T my_acc = 0;
-            for (int e = 0; e < nb; ++e) {
-                const int64_t bb = __shfl(my_bb, gbase + e, kWave), be = __shfl(my_be, gbase + e, kWave);
-                const T a = __shfl(my_a, gbase + e, kWave);
+            // (unrolled: the lane whose entry is applied is then a constant of the instruction that
+            // hands its row start, length and value to the group, with no address to compute)
+            nm::static_for<G>([&](auto ec) {
+                constexpr int e = decltype(ec)::value;
+                if (e >= nb) return;
+                const int64_t bb = group_lane<e>(my_bb), be = bb + group_lane<e>(my_len);
+                const T a = grad_B ? group_lane<e>(my_a) : T(0);
                 T acc = 0;
                 for (int64_t kk0 = bb; kk0 < be; kk0 += G) {
                     const int64_t kk = kk0 + gl;
                     const bool have = kk < be;
                     const int32_t c = have ? (int32_t)B_indices[kk] : -1;
-                    const T bval = have ? B_data[kk] : T(0);
+                    const T bval = have && grad_A ? B_data[kk] : T(0);
                     // the number of staged columns below c (at most 63), in six steps without a branch
                     int l = 0;
 #pragma unroll
@@ -1319,18 +1332,20 @@ __global__ __launch_bounds__(kBlock) void spgemm_bwd_kernel(
                     const bool hit = have && ci[l] == c;
                     const T g = hit ? cg[l] : T(0);
                     if (hit && grad_B) nm::atomic_add(grad_B + kk, a * g);
+                    if (!grad_A) continue;
                     // Ordered sum over the group's lanes = ascending column: the running sum walks up
                     // the lanes, one DPP shift and one addition a step (every lane adds what its lower
                     // neighbour held a step ago to its own product; lane s is right after step s and
                     // is read at step s + 1, what the others hold meanwhile is never used).  A lane
                     // without a product adds +0.0, which changes no sum that began at +0.0.
-                    T run = acc + (hit ? g * bval : T(0));
+                    const T prod = g * bval;   // (g is +0.0 without a hit, bval finite or the lane's own)
+                    T run = acc + (hit ? prod : T(0));
 #pragma unroll
-                    for (int step = 1; step < G; ++step) run = nm::dpp_move<0x111>(run) + (hit ? g * bval : T(0));
-                    acc = group_last(run);
+                    for (int step = 1; step < G; ++step) run = nm::dpp_move<0x111>(run) + (hit ? prod : T(0));
+                    acc = group_lane<G - 1>(run);
                 }
                 if (gl == e) my_acc = acc;
-            }
+            });
             if (mine && grad_A) grad_A[my_ai] = my_acc;
         }
         group_sync<G>();
