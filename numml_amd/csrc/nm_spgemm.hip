@@ -1727,7 +1727,9 @@ extern "C" int nm_spgemm_numeric(nm_dtype dt, int64_t A_rows, int64_t A_cols, in
         if (int rc = bin_rows(A_rows, kNumLimit, w, s)) return rc;
     }
     const int64_t nbatch = nm::xcd_padded(nm::ceil_div(A_rows, kMergeRows));
-    if (dt == NM_F32)
+    // (every row on the hash path: the merge kernel would look at each row's key and leave)
+    if (hash_rows == A_rows) {
+    } else if (dt == NM_F32)
         hipLaunchKernelGGL(numeric_front_kernel<float>, dim3((unsigned)nbatch), dim3(kBlock), 0, s, A_rows, nbatch,
                            w.key, (const float *)A_data, A_indices, A_indptr, (const float *)B_data, B_indices,
                            B_indptr, C_indptr, C_indices, (float *)C_data);
